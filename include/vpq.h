@@ -1,0 +1,201 @@
+/*
+ * vpq.h -- C ABI of the MI355X (gfx950) 4-bit / group-64 affine quantized
+ * linear operator: QMV (decode GEMV, 1..16 rows), QMM (prefill / DiT GEMM with
+ * an optional fused runtime LoRA), the dense expansion of a pack, and the
+ * packer.
+ *
+ * The entry points replace, one for one, the Metal kernels VPIPE's model
+ * families dispatch through their quantized-linear convention
+ * (docs/PLUGINS.md:202-224): the argument ORDER is the Metal buffer-slot order
+ *     0:w  1:scales  2:biases  3:x  4:y  5:K  6:N  [7:M]
+ * so a call site changes one line.  Citations are file:line in the reference
+ * tree (tgo-app-dev/vpipe).
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer (hipMalloc / torch device memory).
+ *   - bf16 values are uint16_t bit patterns.  Element type is bf16 everywhere
+ *     (the reference's `_bf16` metallib twins, -DVPIPE_ELT=bfloat).
+ *   - Packed layout, unchanged from generative-models/quantize:
+ *       w       uint32 [N, K/8]    q[n, 8j+i] = (w[n,j] >> 4i) & 0xF
+ *       scales  bf16   [N, K/64]
+ *       biases  bf16   [N, K/64]   W[n,k] = scales[n,k/64]*q[n,k] + biases[n,k/64]
+ *     `biases` is the quantizer's zero point, NOT the linear layer's additive
+ *     bias; no kernel here has an additive-bias slot, as in the reference
+ *     (generative-models/minimax-h3/metal-minimax-h3-transformer.cc:2250-2256).
+ *   - Calls are asynchronous and ordered on `stream` (a hipStream_t passed as
+ *     void*; NULL is the null stream).  They never synchronise and never
+ *     allocate; scratch is caller-provided.  The caller owns every buffer and
+ *     keeps it alive until the stream has passed the call.
+ *   - Return value: VPQ_OK or a negative vpq_status.  Shape and alignment
+ *     preconditions are checked on the host before anything is launched; a
+ *     failed check launches nothing.  The reference leaves those checks to the
+ *     caller (docs/PLUGINS.md:207-220) and reports GPU faults only at
+ *     Fence::wait_ok (apple-silicon/metal-compute/command-stream.h:92-99); a
+ *     fault here surfaces at the caller's next stream synchronisation.
+ *   - A stream must not run two calls concurrently that share a workspace.
+ */
+#ifndef VPQ_H
+#define VPQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* vpq_stream_t; /* hipStream_t */
+
+typedef enum vpq_status {
+  VPQ_OK = 0,
+  VPQ_ERR_NULL_POINTER = -1,  /* a required buffer is NULL */
+  VPQ_ERR_BAD_SHAPE = -2,     /* K, N, M, r out of the supported domain */
+  VPQ_ERR_MISALIGNED = -3,    /* a pointer is not aligned as required */
+  VPQ_ERR_WORKSPACE = -4,     /* workspace missing or too small */
+  VPQ_ERR_DEVICE = -5,        /* the HIP runtime reported an error */
+  VPQ_ERR_UNSUPPORTED = -6    /* not a gfx950 device */
+} vpq_status;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int vpq_version(void);
+
+/* Human-readable text of a status code; never NULL. */
+const char* vpq_status_string(int status);
+
+/* Text of the last HIP error this thread saw inside the library ("" if none). */
+const char* vpq_last_device_error(void);
+
+/* Checks that the current HIP device is a gfx950 part and caches its
+ * properties.  Optional: every entry point does it on first use.
+ * Stands where MetalCompute::valid() stands
+ * (apple-silicon/metal-compute/metal-compute.h:274-301). */
+int vpq_init(void);
+
+/* Number of compute units of the current device (0 before a successful init). */
+int vpq_device_cu_count(void);
+
+/* ---- a1: dense expansion ------------------------------------------------
+ * Replaces `affine_dequant_w4g64`
+ * (gpu-kernels/metal/quant/affine_dequant.metal:25-58; slots 0:w 1:scales
+ * 2:biases 3:y_deq 4:K 5:N).  w_deq[n,k] = bf16_rne(fp32(s*q + b)), bit-exact
+ * with the reference expression.  Requires K % 64 == 0, K, N > 0; w_deq
+ * 16-byte aligned. */
+int vpq_dequant_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                           const uint16_t* biases, uint16_t* w_deq, int K, int N);
+
+/* ---- a2/a3/a4: QMV, 1 <= M <= 16 ---------------------------------------
+ * Replaces `affine_qmv_w4g64` (gpu-kernels/metal/quant/affine_qmv.metal:286-301;
+ * slots 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N), its `_add` twin (:347-363,
+ * slot 7: residual) and the batched tiles `affine_qmv_batch*_w4g64`
+ * (:1573-1709, 2156-2330; slot 7: m_total): y[M,N] = x[M,K] . W^T with the
+ * QMV arithmetic -- the weight is never rounded to bf16; per (row, group) the
+ * kernel forms sum(x*q) and sum(x) in fp32 and combines them as
+ * scale*sum(x*q) + bias*sum(x) (affine_qmv.metal:151-174), fp32 accumulate,
+ * one bf16 rounding on store.  With `residual` ([M,N] bf16, nullable) the
+ * rounded result is added to it in fp32 and rounded again, as `_add` does
+ * (:264-266).
+ * Requires K % 64 == 0, N > 0, 1 <= M <= 16.
+ * `ws` is scratch for the split-K variant: vpq_qmv_workspace_bytes() bytes,
+ * 256-byte aligned, ZERO-FILLED ONCE by the caller before its first use (the
+ * kernels leave it zero-filled again); it may be NULL, in which case shapes
+ * that would have used split-K run unsplit.
+ * `variant`: 0 = automatic; other values select a specific kernel for
+ * measurement (see VPQ_QMV_* below). */
+int vpq_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                       int K, int N, int M, const uint16_t* residual,
+                       void* ws, size_t ws_bytes, int variant);
+
+/* Same arithmetic, fp32 [M,N] output before the final rounding (measurement of
+ * the accumulation error apart from the bf16 store). */
+int vpq_qmv_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                         const uint16_t* biases, const uint16_t* x, float* y,
+                         int K, int N, int M, void* ws, size_t ws_bytes, int variant);
+
+/* Bytes of split-K scratch the QMV entry points may use for this shape
+ * (an upper bound over variants; a multiple of 256). */
+size_t vpq_qmv_workspace_bytes(int K, int N, int M);
+
+enum {
+  VPQ_QMV_AUTO = 0,
+  VPQ_QMV_SIMPLE = 1,      /* one wavefront per output row, fp32 VALU */
+  VPQ_QMV_MFMA = 2,        /* LDS-staged codes, bf16 MFMA on the integer codes */
+  VPQ_QMV_MFMA_SPLITK = 3  /* as 2, K split across workgroups through `ws` */
+};
+
+/* ---- a6/a7/a8 (+a10): QMM ----------------------------------------------
+ * Replaces `affine_qmm_steel_w4g64[_bm64|_bm128]`
+ * (gpu-kernels/metal/quant/affine_qmm_steel.metal:461-561; slots 0:w 1:scales
+ * 2:biases 3:x 4:y 5:K 6:N 7:M), `affine_qmm_mma_w4g64`
+ * (affine_qmm_mma.metal:50-128) and the dequant-once route
+ * (generative-models/minimax-h3/metal-minimax-h3-transformer.cc:2020-2160):
+ * y[M,N] = bf16_rne( x[M,K] . bf16(W)^T ) -- the weight tile is dequantized in
+ * fp32 and rounded to bf16 once (affine_qmm_steel.metal:78-96), contracted on
+ * bf16 MFMA with fp32 accumulation, one rounding on store.  M and N need not be
+ * tile multiples (affine_qmm_steel.metal:304-317).
+ * With a LoRA (lora_a [r,K], lora_b [N,r], bf16, checkpoint orientation --
+ * generative-models/lora-fusion.h:20-27): t = bf16(alpha * bf16(x . A^T)) is
+ * written to lora_t_ws [M,r] first (the SCALED tile,
+ * gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273), then t . B^T is added
+ * into the same fp32 accumulator before the single store (the fused tile,
+ * dense_gemm_mma.metal:297-348).  lora_a == NULL or alpha == 0 means no adapter,
+ * and the output is then bit-identical to the call without one
+ * (metal-minimax-h3-transformer.cc:2211-2219).
+ * Requires K % 64 == 0, M, N > 0, r % 32 == 0 and 0 < r <= 128 when a LoRA is
+ * given; x, y rows may be of any length (K, N) but the base pointers must be
+ * 16-byte aligned. */
+int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                       int K, int N, int M,
+                       const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
+                       uint16_t* lora_t_ws);
+
+/* The adapter's first GEMM alone: t[M,r] = bf16(alpha * bf16(x . A^T)).
+ * Replaces `lora_gemm_a_` (metal-minimax-h3-transformer.cc:1030-1067). */
+int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t,
+                    int M, int K, int r, float alpha);
+
+/* ---- a5: the size-based entrance ----------------------------------------
+ * Replaces `MetalQwenModel::qmm_auto_`
+ * (generative-models/qwen3/metal-qwen-model.cc:3964-4033): M <= 16 runs the QMV
+ * arithmetic, larger M the QMM arithmetic.  (The reference crosses over at
+ * M = 8; this build's GEMV tile holds 16 rows.) */
+int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                          const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                          int K, int N, int M, void* ws, size_t ws_bytes);
+
+/* ---- a12: the packer ------------------------------------------------------
+ * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:
+ * 243-301; slots 0:x 1:w 2:s 3:b 4:K 5:N 6:clip) driven by
+ * AffineQuantizer::quantize_linear (generative-models/quantize/affine-quantizer.cc:
+ * 52-84): per 64-wide group scale = (max-min)/15, bias = min,
+ * q = clamp(round((v-min)/scale), 0, 15); scales and biases are emitted as IEEE
+ * F16 bit patterns, the on-disk format.  `src` is bf16 [N,K]. */
+int vpq_quantize_w4g64(vpq_stream_t stream, const uint16_t* src, uint32_t* w,
+                       uint16_t* scales_f16, uint16_t* biases_f16, int K, int N, float clip);
+
+/* F16 -> bf16 conversion of scales / biases a bf16 model does once at load
+ * (docs/PLUGINS.md:210-213). */
+int vpq_f16_to_bf16(vpq_stream_t stream, const uint16_t* in_f16, uint16_t* out_bf16, size_t count);
+
+/* ---- measurement aid (no counterpart in the reference's kernels; the
+ * reference times command buffers with Fence::gpu_times(),
+ * apple-silicon/metal-compute/command-stream.h:119-126) -----------------------
+ * vpq_profile_enable(n > 0): from now on each kernel the library launches is
+ * bracketed by its own pair of HIP events (hipExtLaunchKernel start/stop), up to
+ * n launches; n <= 0 switches it off.  vpq_profile_read() waits for the recorded
+ * launches, writes each kernel's duration in milliseconds, in launch order, to
+ * kernel_ms[0..capacity) and returns how many launches were recorded (or a
+ * negative status), then starts over.  Not for use under graph capture; one
+ * thread at a time. */
+int vpq_profile_enable(int max_launches);
+int vpq_profile_read(float* kernel_ms, int capacity);
+
+/* Output byte sizes of the packer (generative-models/quantize/affine-quantizer.h:37-40). */
+size_t vpq_weight_bytes(int N, int K);
+size_t vpq_scale_bytes(int N, int K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VPQ_H */

@@ -1,0 +1,173 @@
+"""ctypes front end of the CPU oracle (oracle/vpq_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
+bench.py's cpu_baseline leg -- never by the shipped package.  Arrays are numpy;
+bf16/f16 values travel as uint16 bit patterns.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libvpq_oracle.so")
+_lib = None
+
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_u32p = ctypes.POINTER(ctypes.c_uint32)
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+
+
+def build(force=False):
+    """Compile the C restatement with the committed Makefile."""
+    if force and os.path.exists(_SO):
+        os.remove(_SO)
+    subprocess.run(["make", "-C", _HERE, "libvpq_oracle.so"], check=True,
+                   stdout=subprocess.DEVNULL)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = ctypes.CDLL(_SO)
+        L.vpo_f32_to_bf16.restype = ctypes.c_uint16
+        L.vpo_f32_to_bf16.argtypes = [ctypes.c_float]
+        L.vpo_bf16_to_f32.restype = ctypes.c_float
+        L.vpo_bf16_to_f32.argtypes = [ctypes.c_uint16]
+        L.vpo_f32_to_f16.restype = ctypes.c_uint16
+        L.vpo_f32_to_f16.argtypes = [ctypes.c_float]
+        L.vpo_f16_to_f32.restype = ctypes.c_float
+        L.vpo_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.vpo_weight_bytes.restype = ctypes.c_size_t
+        L.vpo_scale_bytes.restype = ctypes.c_size_t
+        L.vpo_num_threads.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def _p(a, t):
+    return None if a is None else a.ctypes.data_as(t)
+
+
+def _c(a, dt):
+    if a is None:
+        return None
+    return np.ascontiguousarray(a, dtype=dt)
+
+
+def f32_to_bf16(a):
+    """Element-wise RNE fp32 -> bf16 bits through the C helper."""
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, dtype=np.uint16)
+    lib().vpo_f32_to_bf16_array(_p(a, _f32p), _p(out, _u16p), ctypes.c_size_t(a.size))
+    return out
+
+
+def f32_to_f16(a):
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, dtype=np.uint16)
+    lib().vpo_f32_to_f16_array(_p(a, _f32p), _p(out, _u16p), ctypes.c_size_t(a.size))
+    return out
+
+
+def f16_to_f32(bits):
+    bits = _c(bits, np.uint16)
+    out = np.empty(bits.shape, dtype=np.float32)
+    lib().vpo_f16_to_f32_array(_p(bits, _u16p), _p(out, _f32p), ctypes.c_size_t(bits.size))
+    return out
+
+
+def bf16_to_f32(bits):
+    """Exact widening of bf16 bits (numpy; no rounding involved)."""
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f16_to_bf16(bits):
+    bits = _c(bits, np.uint16)
+    out = np.empty_like(bits)
+    lib().vpo_f16_to_bf16_array(_p(bits, _u16p), _p(out, _u16p), ctypes.c_size_t(bits.size))
+    return out
+
+
+def dequant_bf16(w, s, b, K, N):
+    w, s, b = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16)
+    out = np.empty((N, K), dtype=np.uint16)
+    lib().vpo_dequant_w4g64_bf16(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(out, _u16p), K, N)
+    return out
+
+
+def dequant_f32(w, s, b, K, N):
+    w, s, b = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16)
+    out = np.empty((N, K), dtype=np.float32)
+    lib().vpo_dequant_w4g64_f32(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(out, _f32p), K, N)
+    return out
+
+
+def qmv(w, s, b, x, K, N, M, residual=None):
+    """-> (y64 [M,N] float64, y_bf16 [M,N] uint16); un-rounded-weight semantics."""
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    residual = _c(residual, np.uint16)
+    y64 = np.empty((M, N), dtype=np.float64)
+    yb = np.empty((M, N), dtype=np.uint16)
+    lib().vpo_qmv_w4g64(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p),
+                        _p(y64, _f64p), _p(yb, _u16p), K, N, M, _p(residual, _u16p))
+    return y64, yb
+
+
+def qmv_factored(w, s, b, x, K, N, M):
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    y64 = np.empty((M, N), dtype=np.float64)
+    lib().vpo_qmv_w4g64_factored(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p),
+                                 _p(y64, _f64p), K, N, M)
+    return y64
+
+
+def lora_t(x, A, M, K, r, alpha):
+    x, A = _c(x, np.uint16), _c(A, np.uint16)
+    t = np.empty((M, r), dtype=np.uint16)
+    lib().vpo_lora_t(_p(x, _u16p), _p(A, _u16p), _p(t, _u16p), M, K, r, ctypes.c_float(alpha))
+    return t
+
+
+def qmm(w, s, b, x, K, N, M, t=None, B=None, r=0):
+    """-> (y64, y_bf16); bf16-rounded-weight semantics, optional fused LoRA term."""
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    t, B = _c(t, np.uint16), _c(B, np.uint16)
+    y64 = np.empty((M, N), dtype=np.float64)
+    yb = np.empty((M, N), dtype=np.uint16)
+    lib().vpo_qmm_w4g64(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p),
+                        _p(y64, _f64p), _p(yb, _u16p), K, N, M,
+                        _p(t, _u16p), _p(B, _u16p), r)
+    return y64, yb
+
+
+def quantize(wsrc, K, N, clip=1.0):
+    """fp32 [N,K] -> (codes u32 [N,K/8], scales f16 bits [N,K/64], biases f16 bits)."""
+    wsrc = _c(wsrc, np.float32)
+    codes = np.empty((N, K // 8), dtype=np.uint32)
+    s = np.empty((N, K // 64), dtype=np.uint16)
+    b = np.empty((N, K // 64), dtype=np.uint16)
+    lib().vpo_quantize_w4g64(_p(wsrc, _f32p), _p(codes, _u32p), _p(s, _u16p), _p(b, _u16p),
+                             K, N, ctypes.c_float(clip))
+    return codes, s, b
+
+
+def cpu_dequant_matmul(w, s, b, x, K, N, M, wdeq=None, xf=None):
+    """The timed CPU baseline: dequant to fp32 [N,K] + fp32 dot, bf16 out."""
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    if wdeq is None:
+        wdeq = np.empty((N, K), dtype=np.float32)
+    if xf is None:
+        xf = np.empty((M, K), dtype=np.float32)
+    y = np.empty((M, N), dtype=np.uint16)
+    lib().vpo_cpu_dequant_matmul(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p),
+                                 _p(y, _u16p), _p(wdeq, _f32p), _p(xf, _f32p), K, N, M)
+    return y
+
+
+def num_threads():
+    return int(lib().vpo_num_threads())

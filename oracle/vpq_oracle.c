@@ -1,0 +1,402 @@
+/*
+ * vpq_oracle.c -- CPU restatement of VPIPE's 4-bit / group-64 affine
+ * quantized matmul path.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE.  It is the checker the HIP kernels are
+ * compared against and the timed CPU baseline of the benchmark.  Nothing in
+ * the shipped library links, loads or calls it.
+ *
+ * Every function cites the file:line of the reference (tgo-app-dev/vpipe) it
+ * restates.  Paths are relative to the reference tree.  The reference's own
+ * implementation is Metal Shading Language + Objective-C++ and cannot be built
+ * on Linux, so nothing here is compiled from it; the algorithms are restated.
+ *
+ * What pins each function (checked in tests/test_oracle_*.py):
+ *   bf16/f16 conversions   exhaustive agreement with torch / numpy casts
+ *   dequant                numpy re-derivation from the three independent
+ *                          layout statements in the reference + closed forms
+ *   qmv / qmm              one-hot activations (y == W[n,k]), degenerate
+ *                          quantizers (q=0, b=-8s&q=8, s=0), float64 numpy
+ *                          matmul, linearity, the reference tests' own
+ *                          procedural inputs and asserted tolerances
+ *   lora                   float64 numpy, scale 0 == no adapter, the
+ *                          reference's M=96 test shape (reduced) tolerance
+ *   quantize (packer)      exact recovery of on-grid data, the reference's
+ *                          round-trip error bounds, numpy re-derivation
+ * Parity that only an Apple-GPU run could pin -- the last-bit effect of the
+ * Metal kernels' summation order (simd_sum tree, steel BlockMMA K order,
+ * matmul2d) -- is NOT pinned: the oracle accumulates in double instead, and
+ * kernels are compared to it within the stated tolerance.
+ *
+ * Packed layout (gpu-kernels/metal/quant/affine_dequant.metal:45-52,
+ * affine_qmm_mma.metal:98-99, tests/unit-tests/metal-lm/quant-gemv.cc:245-248):
+ *   w       uint32 [N, K/8]   q[n, 8j+i] = (w[n,j] >> 4i) & 0xF
+ *   scales  elt    [N, K/64]
+ *   biases  elt    [N, K/64]  W[n,k] = scales[n,k/64]*q[n,k] + biases[n,k/64]
+ * Element type is bf16 carried as uint16_t.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define VPO_GROUP 64
+
+/* ---- scalar conversions ------------------------------------------------ */
+
+/* tests/unit-tests/metal-compute-gemm-mma.cc:41-46 (round to nearest even on
+ * the upper 16 bits).  NaN is kept a NaN, which the reference helper does not
+ * guarantee; no test input contains one. */
+uint16_t vpo_f32_to_bf16(float f)
+{
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  if ((x & 0x7fffffffu) > 0x7f800000u) { return (uint16_t)((x >> 16) | 0x40u); }
+  const uint32_t rounding = 0x7fffu + ((x >> 16) & 1u);
+  return (uint16_t)((x + rounding) >> 16);
+}
+
+/* tests/unit-tests/metal-compute-gemm-mma.cc:47-52 */
+float vpo_bf16_to_f32(uint16_t h)
+{
+  const uint32_t x = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &x, 4);
+  return f;
+}
+
+/* IEEE binary16 <-> binary32, round to nearest even.  The packer emits its
+ * scales and biases with Metal's `(half)` cast
+ * (gpu-kernels/metal/quant/affine_dequant.metal:270-271), which is this. */
+uint16_t vpo_f32_to_f16(float f)
+{
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  const uint32_t ax = x & 0x7fffffffu;
+  if (ax > 0x7f800000u) { return (uint16_t)(sign | 0x7e00u); }       /* NaN */
+  if (ax >= 0x47800000u) { return (uint16_t)(sign | 0x7c00u); }      /* >= 65536: inf */
+  if (ax < 0x33000000u) { return (uint16_t)sign; }                   /* < 2^-25 */
+  int e = (int)(ax >> 23) - 127;
+  uint32_t m = (ax & 0x7fffffu) | 0x800000u;                         /* 24-bit */
+  int shift;                                                         /* bits to drop */
+  uint32_t base;
+  if (e < -14) { shift = 13 + (-14 - e); base = 0; }                 /* subnormal */
+  else         { shift = 13; base = (uint32_t)(e + 15) << 10; m &= 0x7fffffu; }
+  const uint32_t keep = m >> shift;
+  const uint32_t rem = m & ((1u << shift) - 1u);
+  const uint32_t half = 1u << (shift - 1);
+  uint32_t h = base + keep;
+  if (rem > half || (rem == half && (keep & 1u))) { h += 1; }        /* carries into exp */
+  return (uint16_t)(sign | h);
+}
+
+float vpo_f16_to_f32(uint16_t h)
+{
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  const uint32_t e = (h >> 10) & 0x1fu;
+  const uint32_t m = h & 0x3ffu;
+  uint32_t x;
+  if (e == 0) {
+    if (m == 0) { x = sign; }
+    else {
+      float v = (float)m * 5.9604644775390625e-8f;                   /* m * 2^-24 */
+      memcpy(&x, &v, 4);
+      x |= sign;
+    }
+  } else if (e == 31) { x = sign | 0x7f800000u | (m << 13); }
+  else { x = sign | ((e + 112u) << 23) | (m << 13); }
+  float f;
+  memcpy(&f, &x, 4);
+  return f;
+}
+
+/* Loaders of bf16 models turn the packer's F16 scales/biases into bf16 once at
+ * load (docs/PLUGINS.md:210-213,
+ * generative-models/minimax-h3/metal-minimax-h3-transformer.cc:766-778). */
+void vpo_f16_to_bf16_array(const uint16_t* in, uint16_t* out, size_t n)
+{
+  for (size_t i = 0; i < n; ++i) { out[i] = vpo_f32_to_bf16(vpo_f16_to_f32(in[i])); }
+}
+
+void vpo_f32_to_bf16_array(const float* in, uint16_t* out, size_t n)
+{
+  for (size_t i = 0; i < n; ++i) { out[i] = vpo_f32_to_bf16(in[i]); }
+}
+
+void vpo_f32_to_f16_array(const float* in, uint16_t* out, size_t n)
+{
+  for (size_t i = 0; i < n; ++i) { out[i] = vpo_f32_to_f16(in[i]); }
+}
+
+void vpo_f16_to_f32_array(const uint16_t* in, float* out, size_t n)
+{
+  for (size_t i = 0; i < n; ++i) { out[i] = vpo_f16_to_f32(in[i]); }
+}
+
+static inline unsigned nibble(const uint32_t* w, size_t n, int Kw, int k)
+{
+  return (w[n * (size_t)Kw + (size_t)(k >> 3)] >> (4 * (k & 7))) & 0xfu;
+}
+
+/* ---- a1: dequant ------------------------------------------------------- */
+
+/* gpu-kernels/metal/quant/affine_dequant.metal:25-58: one u32 word -> eight
+ * outputs, out = (elt)(s * (float)q + b) with s, b widened to fp32.  s*q is
+ * exact in fp32 (8-bit x 4-bit significands) so a fused or unfused multiply-add
+ * gives the same fp32 value; it is written as two operations here and compiled
+ * with -ffp-contract=off. */
+void vpo_dequant_w4g64_f32(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           float* out, int K, int N)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      out[n * (size_t)K + k] = sq + b;
+    }
+  }
+}
+
+void vpo_dequant_w4g64_bf16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            uint16_t* out, int K, int N)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      out[n * (size_t)K + k] = vpo_f32_to_bf16(sq + b);
+    }
+  }
+}
+
+/* ---- a2/a3: QMV -------------------------------------------------------- */
+
+/* The CPU reference loop of the reference's own QMV test,
+ * tests/unit-tests/metal-lm/quant-gemv.cc:255-265:
+ *     acc(double) += (double)x[k] * (s*(float)q + b)        (inner term in fp32)
+ * It is the un-rounded-weight semantics of the Metal QMV kernels
+ * (gpu-kernels/metal/quant/affine_qmv.metal:151-174: scale*sum(x*q) +
+ * bias*sum(x), never rounding the weight to the element type).  y64 receives
+ * the double sums [M,N]; y_bf16 (nullable) their RNE cast, after adding
+ * residual[M,N] (nullable) the way affine_qmv_w4g64_add does
+ * (affine_qmv.metal:264-266: the fp32 result is cast to the element type,
+ * THEN the residual is added in the element type). */
+void vpo_qmv_w4g64(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, double* y64, uint16_t* y_bf16,
+                   int K, int N, int M, const uint16_t* residual)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      wrow[k] = sq + b;
+    }
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      double acc = 0.0;
+      const uint16_t* xr = x + m * (size_t)K;
+      for (int k = 0; k < K; ++k) { acc += (double)vpo_bf16_to_f32(xr[k]) * (double)wrow[k]; }
+      if (y64) { y64[m * (size_t)N + n] = acc; }
+      if (y_bf16) {
+        uint16_t v = vpo_f32_to_bf16((float)acc);
+        if (residual) {
+          v = vpo_f32_to_bf16(vpo_bf16_to_f32(v) + vpo_bf16_to_f32(residual[m * (size_t)N + n]));
+        }
+        y_bf16[m * (size_t)N + n] = v;
+      }
+    }
+  }
+  free(wrow);
+}
+
+/* The kernel's own algebra, gpu-kernels/metal/quant/affine_qmv.metal:151-174
+ * (qdot) and :228-258 (block loop): per (row, group) the two sums sum(x*q) and
+ * sum(x) are formed and combined as scale*accum + sum*bias.  Here both sums and
+ * the running result are kept in double (the reference keeps fp32 and, for
+ * bf16, forms sum(x) in bf16 quad sums -- affine_qmv.metal:60-67 -- which this
+ * restatement deliberately does not copy).  Exists to show that the factored
+ * form and the direct form above are the same number. */
+void vpo_qmv_w4g64_factored(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* x, double* y64, int K, int N, int M)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  for (size_t m = 0; m < (size_t)M; ++m) {
+    const uint16_t* xr = x + m * (size_t)K;
+    for (size_t n = 0; n < (size_t)N; ++n) {
+      double acc = 0.0;
+      for (int g = 0; g < Kg; ++g) {
+        double sxq = 0.0, sx = 0.0;
+        for (int k = g * VPO_GROUP; k < (g + 1) * VPO_GROUP; ++k) {
+          const double xv = (double)vpo_bf16_to_f32(xr[k]);
+          sxq += xv * (double)nibble(w, n, Kw, k);
+          sx += xv;
+        }
+        acc += (double)vpo_bf16_to_f32(scales[n * Kg + g]) * sxq +
+               sx * (double)vpo_bf16_to_f32(biases[n * Kg + g]);
+      }
+      y64[m * (size_t)N + n] = acc;
+    }
+  }
+}
+
+/* ---- a6/a7/a8 (+a10): QMM with optional LoRA --------------------------- */
+
+/* t[M,r] of a runtime LoRA: gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273
+ * (SCALED tile: the fp32 contraction x.A^T lands in an element-typed
+ * cooperative tensor, then `(elt)((float)*it * scale)` -- two roundings) with A
+ * in checkpoint orientation [r,K] (generative-models/lora-fusion.h:20-27).
+ * Contraction in double. */
+void vpo_lora_t(const uint16_t* x, const uint16_t* A, uint16_t* t, int M, int K, int r, float alpha)
+{
+  for (size_t m = 0; m < (size_t)M; ++m) {
+    for (int j = 0; j < r; ++j) {
+      double acc = 0.0;
+      for (int k = 0; k < K; ++k) {
+        acc += (double)vpo_bf16_to_f32(x[m * (size_t)K + k]) *
+               (double)vpo_bf16_to_f32(A[(size_t)j * K + k]);
+      }
+      const float once = vpo_bf16_to_f32(vpo_f32_to_bf16((float)acc));
+      t[m * (size_t)r + j] = vpo_f32_to_bf16(once * alpha);
+    }
+  }
+}
+
+/* Tiled quantized GEMM semantics: every QMM route of the reference rounds the
+ * dequantized weight to the element type BEFORE the contraction
+ * (gpu-kernels/metal/quant/affine_qmm_steel.metal:78-96 with Compute=float,
+ * affine_qmm_mma.metal:96-104, affine_dequant.metal:51), accumulates in fp32
+ * and rounds once on store.  With a LoRA the fused tile adds t.B^T into the
+ * same accumulator before that one store
+ * (gpu-kernels/metal/gemm/dense_gemm_mma.metal:297-348); B is [N,r].  The
+ * contraction here is in double so the result does not depend on an order.
+ * t (nullable with B) is the bf16 [M,r] produced by vpo_lora_t. */
+void vpo_qmm_w4g64(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, double* y64, uint16_t* y_bf16,
+                   int K, int N, int M,
+                   const uint16_t* t, const uint16_t* B, int r)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      wrow[k] = vpo_bf16_to_f32(vpo_f32_to_bf16(sq + b));
+    }
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      double acc = 0.0;
+      const uint16_t* xr = x + m * (size_t)K;
+      for (int k = 0; k < K; ++k) { acc += (double)vpo_bf16_to_f32(xr[k]) * (double)wrow[k]; }
+      if (t && B) {
+        for (int j = 0; j < r; ++j) {
+          acc += (double)vpo_bf16_to_f32(t[m * (size_t)r + j]) *
+                 (double)vpo_bf16_to_f32(B[n * (size_t)r + j]);
+        }
+      }
+      if (y64) { y64[m * (size_t)N + n] = acc; }
+      if (y_bf16) { y_bf16[m * (size_t)N + n] = vpo_f32_to_bf16((float)acc); }
+    }
+  }
+  free(wrow);
+}
+
+/* ---- a12: the packer --------------------------------------------------- */
+
+/* gpu-kernels/metal/quant/affine_dequant.metal:243-285 (affine_quant_impl<4,64>):
+ * per group mn/mx, optional clip toward the midpoint, scale=(mx-mn)/15,
+ * inv = scale>0 ? 1/scale : 0, q = clamp(round((v-mn)*inv), 0, 15) with Metal's
+ * round() = half away from zero (C roundf), scale and mn emitted as F16.
+ * Host twin: generative-models/quantize/model-quantizer.cc:240-264 (lround).
+ * Input is fp32 here (the kernel widens its f16/bf16 input to float first). */
+void vpo_quantize_w4g64(const float* wsrc, uint32_t* codes, uint16_t* scales_f16,
+                        uint16_t* biases_f16, int K, int N, float clip)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int g = 0; g < Kg; ++g) {
+      const float* xp = wsrc + n * (size_t)K + (size_t)g * VPO_GROUP;
+      float mn = INFINITY, mx = -INFINITY;
+      for (int i = 0; i < VPO_GROUP; ++i) {
+        mn = fminf(mn, xp[i]);
+        mx = fmaxf(mx, xp[i]);
+      }
+      if (clip < 1.0f) {
+        const float mid = 0.5f * (mn + mx);
+        mn = mid + (mn - mid) * clip;
+        mx = mid + (mx - mid) * clip;
+      }
+      const float scale = (mx - mn) / 15.0f;
+      const float inv = (scale > 0.0f) ? 1.0f / scale : 0.0f;
+      scales_f16[n * Kg + g] = vpo_f32_to_f16(scale);
+      biases_f16[n * Kg + g] = vpo_f32_to_f16(mn);
+      for (int wi = 0; wi < VPO_GROUP / 8; ++wi) {
+        uint32_t packed = 0;
+        for (int i = 0; i < 8; ++i) {
+          int q = (int)roundf((xp[wi * 8 + i] - mn) * inv);
+          q = q < 0 ? 0 : (q > 15 ? 15 : q);
+          packed |= (uint32_t)q << (4 * i);
+        }
+        codes[n * (size_t)Kw + (size_t)g * (VPO_GROUP / 8) + wi] = packed;
+      }
+    }
+  }
+}
+
+/* Output byte sizes, generative-models/quantize/affine-quantizer.h:37-40. */
+size_t vpo_weight_bytes(int N, int K) { return (size_t)N * (size_t)(K * 4 / 32) * 4; }
+size_t vpo_scale_bytes(int N, int K) { return (size_t)N * (size_t)(K / VPO_GROUP) * 2; }
+
+/* ---- timed CPU baseline ------------------------------------------------ */
+
+/* "quantize-module dequant + fp32 matmul": expand the pack to fp32 [N,K]
+ * (semantics of affine_dequant.metal:25-58 / model-quantizer.cc:257) and run a
+ * plain fp32 dot per output (the float-accumulating oracle loop of
+ * tests/unit-tests/metal-compute-gemm-mma.cc:337-347), bf16 store.  OpenMP over
+ * output rows when built with -fopenmp.  wdeq is caller-provided scratch
+ * [N,K] fp32.  Returns nothing; the benchmark times the call. */
+void vpo_cpu_dequant_matmul(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* x, uint16_t* y, float* wdeq, float* xf,
+                            int K, int N, int M)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  for (size_t i = 0; i < (size_t)M * (size_t)K; ++i) { xf[i] = vpo_bf16_to_f32(x[i]); }
+#pragma omp parallel for schedule(static)
+  for (long n = 0; n < (long)N; ++n) {
+    float* o = wdeq + (size_t)n * K;
+    for (int j = 0; j < Kw; ++j) {
+      const uint32_t p = w[(size_t)n * Kw + j];
+      const float s = vpo_bf16_to_f32(scales[(size_t)n * Kg + j / 8]);
+      const float b = vpo_bf16_to_f32(biases[(size_t)n * Kg + j / 8]);
+      for (int i = 0; i < 8; ++i) {
+        const float sq = s * (float)((p >> (4 * i)) & 0xfu);
+        o[j * 8 + i] = sq + b;
+      }
+    }
+  }
+#pragma omp parallel for schedule(static)
+  for (long n = 0; n < (long)N; ++n) {
+    const float* wr = wdeq + (size_t)n * K;
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      const float* xr = xf + m * (size_t)K;
+      float acc = 0.0f;
+#pragma omp simd reduction(+ : acc)
+      for (int k = 0; k < K; ++k) { acc += xr[k] * wr[k]; }
+      y[m * (size_t)N + (size_t)n] = vpo_f32_to_bf16(acc);
+    }
+  }
+}
+
+#ifdef _OPENMP
+#include <omp.h>
+int vpo_num_threads(void) { return omp_get_max_threads(); }
+#else
+int vpo_num_threads(void) { return 1; }
+#endif

@@ -1,0 +1,74 @@
+"""Shared helpers of the GPU parity tests: tolerance checks and input staging.
+
+Tolerances (written once, used by every GPU test):
+  * dequantized weights: bit-exact.
+  * fp32 result before the store vs the float64 oracle:
+        max |d| / max(|ref|, 1e-2 * rms(ref))  <=  2e-3
+    (relative error with a floor, since zero-mean weights put outputs near 0).
+  * bf16 output vs bf16_rne(oracle): every element within one bf16 ulp (the
+    fp32 sum and the float64 sum may sit on either side of a rounding
+    boundary), and rel-L2 of the bf16 output against the float64 oracle <= 2e-3
+    plus the rounding noise of one bf16 store (2^-9 / sqrt(3) ~ 1.1e-3).
+"""
+import numpy as np
+
+from vpipe_amd import synth
+
+F32_TOL = 2e-3
+REL_L2_TOL = 2e-3 + 1.2e-3
+
+
+def floor_rel_err(got, ref64):
+    ref64 = np.asarray(ref64, dtype=np.float64)
+    rms = np.sqrt((ref64 ** 2).mean())
+    denom = np.maximum(np.abs(ref64), 1e-2 * rms + 1e-30)
+    return (np.abs(np.asarray(got, dtype=np.float64) - ref64) / denom).max()
+
+
+def rel_l2(got, ref64):
+    ref64 = np.asarray(ref64, dtype=np.float64)
+    num = ((np.asarray(got, dtype=np.float64) - ref64) ** 2).sum()
+    den = (ref64 ** 2).sum()
+    return np.sqrt(num / den) if den > 0 else np.sqrt(num)
+
+
+def bf16_ulp_distance(a_bits, b_bits):
+    """Distance in units of bf16 steps on the ordered number line."""
+    def key(x):
+        x = np.asarray(x, dtype=np.uint16).astype(np.int32)
+        return np.where(x & 0x8000, -(x & 0x7FFF), x & 0x7FFF)
+    return np.abs(key(a_bits) - key(b_bits))
+
+
+def check_f32(got_f32, ref64, tol=F32_TOL):
+    e = floor_rel_err(got_f32, ref64)
+    assert e <= tol, "fp32 result off by %.3e (tol %.1e)" % (e, tol)
+    return e
+
+
+def check_bf16(got_bits, ref64, ref_bits=None):
+    if ref_bits is None:
+        ref_bits = synth.f32_to_bf16_bits(np.asarray(ref64, dtype=np.float64).astype(np.float32))
+    d = bf16_ulp_distance(got_bits, ref_bits)
+    assert d.max() <= 1, "bf16 output differs by %d ulp" % d.max()
+    r = rel_l2(synth.bf16_bits_to_f32(got_bits), ref64)
+    assert r <= REL_L2_TOL, "rel-L2 %.3e" % r
+    return float((d != 0).mean()), r
+
+
+class Guarded:
+    """An output buffer with sentinel-filled guard bands on both sides, to catch
+    stores outside [M,N]."""
+
+    def __init__(self, shape, dtype, dev, guard=4096):
+        import torch
+        self.n = int(np.prod(shape))
+        self.guard = guard
+        self.buf = torch.full((self.n + 2 * guard,), -7.0, dtype=dtype, device=dev)
+        self.view = self.buf[guard:guard + self.n].view(shape)
+
+    def assert_intact(self):
+        import torch
+        g = self.guard
+        lo, hi = self.buf[:g].float(), self.buf[g + self.n:].float()
+        assert torch.all(lo == -7.0).item() and torch.all(hi == -7.0).item(), "kernel wrote outside its output"

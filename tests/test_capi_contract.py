@@ -1,0 +1,62 @@
+"""The C-ABI library loads and exports exactly what include/vpq.h declares.
+No GPU: only symbol resolution, argument validation that happens before any
+device call, and the host-side size helpers."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import vpipe_amd
+from vpipe_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "vpq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vpq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = vpipe_amd.load()
+    names = _declared()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(L, n), n
+    assert sorted(n for n, _, _ in capi.SYMBOLS) == names
+
+
+def test_missing_library_is_loud(monkeypatch, tmp_path):
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "_SO", str(tmp_path / "libvpq.so"))
+    with pytest.raises(FileNotFoundError):
+        capi.load()
+
+
+def test_host_side_validation_and_sizes():
+    L = vpipe_amd.load()
+    assert L.vpq_version() >= 100
+    # generative-models/quantize/affine-quantizer.h:37-40
+    assert L.vpq_weight_bytes(96, 256) == 96 * 32 * 4
+    assert L.vpq_scale_bytes(96, 256) == 96 * 4 * 2
+    assert L.vpq_qmv_workspace_bytes(4096, 1024, 1) % 256 == 0
+    assert L.vpq_qmv_workspace_bytes(4096, 1024, 17) == 0
+    one = ctypes.c_void_p(4096)   # never dereferenced: every call below fails validation first
+    null = ctypes.c_void_p(0)
+    # NULL buffers
+    assert L.vpq_dequant_w4g64_bf16(null, null, one, one, one, 64, 1) == -1
+    assert L.vpq_qmv_w4g64_bf16(null, one, one, one, null, one, 64, 8, 1, null, null, 0, 0) == -1
+    # K not a multiple of the group, M out of range, bad rank
+    assert L.vpq_dequant_w4g64_bf16(null, one, one, one, one, 96, 1) == -2
+    assert L.vpq_qmv_w4g64_bf16(null, one, one, one, one, one, 64, 8, 17, null, null, 0, 0) == -2
+    assert L.vpq_qmv_w4g64_bf16(null, one, one, one, one, one, 64, 8, 0, null, null, 0, 0) == -2
+    assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 0, null, null, 0, 0.0, null) == -2
+    assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, one, one, 48, 1.0, one) == -2
+    # misaligned codes / x
+    assert L.vpq_dequant_w4g64_bf16(null, ctypes.c_void_p(4100), one, one, one, 64, 1) == -3
+    assert L.vpq_qmv_w4g64_bf16(null, one, one, one, ctypes.c_void_p(4098), one, 64, 8, 1, null, null, 0, 0) == -3
+    # LoRA without its scratch
+    assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, one, one, 32, 1.0, null) == -4
+    assert b"NULL" in L.vpq_status_string(-1)

@@ -1,0 +1,215 @@
+"""GPU parity: dense expansion (bit-exact) and QMV (every kernel variant) against
+the CPU oracle, through the C ABI.  Cases follow the reference's own tests
+(tests/unit-tests/metal-lm/quant-gemv.cc): K tails, padded/garbage rows, batched
+rows, residual add, and the benchmark's full shapes."""
+import numpy as np
+import pytest
+import torch
+
+from tests import parity
+from tests.golden import refgen
+from vpipe_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+SIMPLE, MFMA, SPLITK, AUTO = capi.VPQ_QMV_SIMPLE, capi.VPQ_QMV_MFMA, capi.VPQ_QMV_MFMA_SPLITK, capi.VPQ_QMV_AUTO
+
+
+def stage(D, dev, w, s, b, x=None):
+    out = [D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev)]
+    if x is not None:
+        out.append(D.bf16(x, dev))
+    return out
+
+
+# ---- a1: dequant is bit-exact -------------------------------------------------
+
+@pytest.mark.parametrize("N,K", [(1, 64), (33, 192), (257, 3840), (4096, 4096)])
+def test_dequant_bit_exact(vpq, oracle, dev, D, N, K):
+    w, s, b = synth.make_weight(N, K, 7 + N)
+    wd, sd, bd = stage(D, dev, w, s, b)
+    out = parity.Guarded((N, K), torch.bfloat16, dev)
+    vpq.dequant_w4g64(wd, sd, bd, K, N, out=out.view)
+    torch.cuda.synchronize()
+    got = D.bits(out.view)
+    assert np.array_equal(got, oracle.dequant_bf16(w, s, b, K, N))
+    out.assert_intact()
+
+
+def test_dequant_every_code_against_every_scale(vpq, oracle, dev, D):
+    # all 16 codes x a sweep of 2^16 (scale, bias) bit patterns: the bf16 rounding
+    # of fp32(s*q+b) must agree everywhere, including ties and cancellation.
+    K = 64
+    N = 1 << 16
+    rng = np.random.default_rng(99)
+    w = np.tile(np.array([0x76543210, 0xFEDCBA98], dtype=np.uint32), (N, K // 16))
+    s = np.arange(N, dtype=np.uint32).astype(np.uint16)[:, None]          # every bf16 pattern once
+    s = np.where((s & 0x7F80) == 0x7F80, np.uint16(0x3C00), s)            # drop inf/nan patterns
+    bvals = synth.f32_to_bf16_bits((-8.0 * synth.bf16_bits_to_f32(s) *
+                                    (1 + 0.05 * rng.standard_normal(s.shape))).astype(np.float32))
+    bvals = np.where((bvals & 0x7F80) == 0x7F80, np.uint16(0), bvals)
+    wd, sd, bd = stage(D, dev, w, s, bvals)
+    got = D.bits(vpq.dequant_w4g64(wd, sd, bd, K, N))
+    want = oracle.dequant_bf16(w, s, bvals, K, N)
+    finite = np.isfinite(synth.bf16_bits_to_f32(want))
+    assert np.array_equal(got[finite], want[finite])
+
+
+# ---- a2/a3/a4: QMV --------------------------------------------------------------
+
+SMALL = [
+    # K, N, M
+    (512, 16, 1), (512, 16, 4), (1024, 48, 2), (1024, 40, 3), (2048, 160, 5),
+    (1536, 33, 7), (512, 95, 8), (2560, 64, 16), (4096, 16, 13),
+]
+
+
+@pytest.mark.parametrize("variant", [SIMPLE, MFMA, AUTO])
+@pytest.mark.parametrize("K,N,M", SMALL)
+def test_qmv_small_shapes(vpq, oracle, dev, D, K, N, M, variant):
+    w, s, b = synth.make_weight(N, K, 1000 + K + N)
+    x = synth.make_act(M, K, 2000 + K + M)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    ws = vpq.qmv_workspace(K, N, M)
+    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, ws=ws, variant=variant, f32out=True)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, ws=ws, variant=variant)
+    torch.cuda.synchronize()
+    parity.check_f32(f.cpu().numpy(), y64)
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    out.assert_intact()
+    assert not ws.any().item()                      # split-K scratch is left zeroed
+
+
+@pytest.mark.parametrize("K,N,M", [(2048, 16, 1), (4096, 64, 4), (1024, 33, 16), (8192, 48, 2)])
+def test_qmv_split_k_matches_oracle_and_is_deterministic(vpq, oracle, dev, D, K, N, M):
+    w, s, b = synth.make_weight(N, K, 31 + K)
+    x = synth.make_act(M, K, 32 + K)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    ws = vpq.qmv_workspace(K, N, M)
+    runs = []
+    for _ in range(3):
+        out = parity.Guarded((M, N), torch.bfloat16, dev)
+        vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, ws=ws, variant=SPLITK)
+        torch.cuda.synchronize()
+        out.assert_intact()
+        runs.append(D.bits(out.view).copy())
+        assert not ws[:256].any().item()            # arrival counters back to zero
+    parity.check_bf16(runs[0], y64, yb)
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, ws=ws, variant=SPLITK, f32out=True)
+    parity.check_f32(f.cpu().numpy(), y64)
+
+
+def test_qmv_one_hot_reads_back_weights_exactly(vpq, oracle, dev, D):
+    # x = e_k: y[n] must be bf16(fp32(s*q+b)) EXACTLY for every kernel -- layout,
+    # nibble order and the un-rounded-weight arithmetic in one known answer.
+    K, N = 1024, 32
+    w, s, b = synth.make_weight(N, K, 5)
+    d32 = oracle.dequant_f32(w, s, b, K, N)
+    wd, sd, bd = stage(D, dev, w, s, b)
+    for variant in (SIMPLE, MFMA):
+        for k in [0, 1, 4, 7, 8, 15, 16, 63, 64, 511, 512, 777, K - 1]:
+            x = np.zeros((1, K), dtype=np.float32)
+            x[0, k] = 1.0
+            y = vpq.qmv_w4g64(wd, sd, bd, D.bf16(synth.f32_to_bf16_bits(x), dev), K, N, 1,
+                              variant=variant, f32out=True)
+            got = y.cpu().numpy()[0]
+            # the MFMA kernel forms s*(128+q) - 128 s ... in fp32: exact for one-hot x
+            assert np.array_equal(got, d32[:, k]), (variant, k)
+
+
+def test_qmv_reference_tail_case(vpq, oracle, dev, D):
+    """metal_lm_smoke.qmv_w4g32_matches_cpu inputs (quant-gemv.cc:215-253) at g64:
+    K = 3840 is not a multiple of 512, x is padded with non-zero values to 4096 and
+    a garbage weight row follows row N-1.  Bar of the reference: max
+    |d|/(|ref|+1e-2) < 0.03."""
+    N, K = 16, 3840
+    c = refgen.knuth_qmv_case(N, K, group=64)
+    s = synth.f32_to_bf16_bits(c["scales"])
+    b = synth.f32_to_bf16_bits(c["biases"])
+    x = synth.f32_to_bf16_bits(c["x"])[None, :]              # 4096 values, only K are used
+    y64, yb = oracle.qmv(c["packed"][:N], s, b, x[:, :K], K, N, 1)
+    wd = D.u32(c["packed"], dev)                             # N+1 rows on the device
+    y = vpq.qmv_w4g64(wd, D.bf16(s, dev), D.bf16(b, dev), D.bf16(x, dev), K, N, 1)
+    got = synth.bf16_bits_to_f32(D.bits(y))[0].astype(np.float64)
+    assert (np.abs(got - y64[0]) / (np.abs(y64[0]) + 1e-2)).max() < 0.03
+    parity.check_bf16(D.bits(y), y64, yb)
+
+
+def test_qmv_batched_rows_are_independent(vpq, oracle, dev, D):
+    # the batched tiles of the reference are bit-identical per row to the M=1 kernel
+    # (affine_qmv.metal:1563-1564); here: row m of an M-row call == the M=1 call on row m.
+    K, N, M = 2048, 64, 7
+    w, s, b = synth.make_weight(N, K, 77)
+    x = synth.make_act(M, K, 78)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    for variant in (SIMPLE, MFMA):
+        full = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=variant))
+        for m in range(M):
+            one = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd[m:m + 1].contiguous(), K, N, 1, variant=variant))
+            assert np.array_equal(full[m], one[0]), (variant, m)
+
+
+def test_qmv_residual_add(vpq, oracle, dev, D):
+    K, N, M = 1024, 48, 2
+    w, s, b = synth.make_weight(N, K, 61)
+    x = synth.make_act(M, K, 62)
+    res = synth.make_act(M, N, 63)
+    _, yr = oracle.qmv(w, s, b, x, K, N, M, residual=res)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    for variant in (SIMPLE, MFMA):
+        y = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, residual=D.bf16(res, dev), variant=variant)
+        assert parity.bf16_ulp_distance(D.bits(y), yr).max() <= 1
+
+
+DECODE_LAYER = [(4096, 4096), (4096, 1024), (4096, 12288), (12288, 4096)]
+
+
+@pytest.mark.parametrize("K,N", DECODE_LAYER)
+def test_qmv_decode_layer_shapes_full(vpq, oracle, dev, D, K, N):
+    w, s, b = synth.make_weight(N, K, 0x5EED0002 + N)
+    x = synth.make_act(1, K, 0x5EED0102 + K)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, 1)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    ws = vpq.qmv_workspace(K, N, 1)
+    for variant in (AUTO, SIMPLE):
+        f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, 1, ws=ws, variant=variant, f32out=True)
+        y = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, 1, ws=ws, variant=variant)
+        parity.check_f32(f.cpu().numpy(), y64)
+        parity.check_bf16(D.bits(y), y64, yb)
+
+
+@pytest.mark.parametrize("K,N", [(5120, 5120), (5120, 17408), (17408, 5120), (5120, 151936)])
+@pytest.mark.parametrize("M", [1, 16])
+def test_qmv_small_batch_shapes_row_sample(vpq, oracle, dev, D, K, N, M):
+    # full-size launch; the oracle evaluates a sample of output rows (first and last
+    # tiles included), since every output row depends on its own weight row only.
+    w, s, b = synth.make_weight(N, K, 0x5EED0003 + N)
+    x = synth.make_act(M, K, 0x5EED0103 + K + M)
+    rng = np.random.default_rng(N + M)
+    rows = np.unique(np.concatenate([np.arange(16), np.arange(N - 16, N), rng.integers(0, N, 224)]))
+    y64, yb = oracle.qmv(w[rows], s[rows], b[rows], x, K, len(rows), M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    ws = vpq.qmv_workspace(K, N, M)
+    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, ws=ws, f32out=True).cpu().numpy()
+    y = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, ws=ws))
+    parity.check_f32(f[:, rows], y64)
+    parity.check_bf16(y[:, rows], y64, yb)
+    # size-independent property over ALL rows: zero activations give exactly zero
+    z = vpq.qmv_w4g64(wd, sd, bd, torch.zeros_like(xd), K, N, M, ws=ws, f32out=True)
+    assert not z.any().item()
+
+
+def test_linear_entrance_routes_by_rows(vpq, oracle, dev, D):
+    # qmm_auto_ (metal-qwen-model.cc:3964-4033): GEMV arithmetic for few rows, GEMM above
+    K, N = 1024, 64
+    w, s, b = synth.make_weight(N, K, 91)
+    wd, sd, bd = stage(D, dev, w, s, b)
+    for M, fn in ((16, oracle.qmv), (17, oracle.qmm)):
+        x = synth.make_act(M, K, 92 + M)
+        y64, yb = fn(w, s, b, x, K, N, M)
+        y = vpq.linear_w4g64(wd, sd, bd, D.bf16(x, dev), K, N, M)
+        parity.check_bf16(D.bits(y), y64, yb)

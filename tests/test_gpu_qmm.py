@@ -1,0 +1,153 @@
+"""GPU parity: QMM (bf16-rounded weight tile, MFMA, fp32 accumulate) and the fused
+runtime LoRA against the CPU oracle, through the C ABI.  Shapes follow the
+reference's qmm tests (tests/unit-tests/metal-compute-gemm-mma.cc:312-498) and
+LoRA test (tests/unit-tests/minimax-h3-blocks.cc:1162-1296), then the
+benchmark's prefill and video-DiT shapes with the oracle on a row/column sample."""
+import numpy as np
+import pytest
+import torch
+
+from tests import parity
+from tests.golden import refgen
+from vpipe_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def stage(D, dev, w, s, b, x):
+    return D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), D.bf16(x, dev)
+
+
+REFERENCE_SHAPES = [
+    # M, N, K  -- qmm_mma.correctness and qmm_mma.ragged_n_matches_reference
+    (64, 64, 64), (96, 128, 128), (130, 320, 256), (512, 256, 2560),
+    (33, 33, 128), (64, 95, 192), (96, 161, 256),
+    (17, 16, 64), (1, 8, 64), (257, 129, 512),
+]
+
+
+@pytest.mark.parametrize("M,N,K", REFERENCE_SHAPES)
+def test_qmm_reference_shapes(vpq, oracle, dev, D, M, N, K):
+    w, s, b = synth.make_weight(N, K, 999 + N + K)
+    x = synth.make_act(M, K, 555 + M + N + K)
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, out=out.view)
+    torch.cuda.synchronize()
+    got = D.bits(out.view)
+    parity.check_bf16(got, y64, yb)
+    out.assert_intact()
+    # the reference's own bar (rel-L2 < 3e-2 against an fp32 CPU loop over the UN-rounded weight)
+    W = oracle.dequant_f32(w, s, b, K, N).astype(np.float64)
+    ref = synth.bf16_bits_to_f32(x).astype(np.float64) @ W.T
+    assert parity.rel_l2(synth.bf16_bits_to_f32(got), ref) < 3e-2
+
+
+def test_qmm_one_hot_reads_back_the_rounded_weight(vpq, oracle, dev, D):
+    # x = e_k  =>  y[m,n] = bf16(fp32(s*q+b)) exactly: the tile's dequant is the a1 arithmetic
+    K, N, M = 256, 144, 20
+    w, s, b = synth.make_weight(N, K, 17)
+    d16 = oracle.dequant_bf16(w, s, b, K, N)
+    x = np.zeros((M, K), dtype=np.float32)
+    ks = [(m * 37 + 5) % K for m in range(M)]
+    for m, k in enumerate(ks):
+        x[m, k] = 1.0
+    wd, sd, bd, xd = stage(D, dev, w, s, b, synth.f32_to_bf16_bits(x))
+    got = D.bits(vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M))
+    for m, k in enumerate(ks):
+        assert np.array_equal(got[m], d16[:, k]), m
+
+
+def test_qmm_reference_lcg_inputs(vpq, oracle, dev, D):
+    """make_act_/make_qw_ inputs of tests/unit-tests/minimax-h3-blocks.cc:121-158
+    (s = 0.01, b = -0.08, LCG bytes); agreement bar of mma_matches_steel: rel-L2 < 3e-2."""
+    M, N, K = 128, 96, 512
+    packed, s0, b0 = refgen.lcg_qweight(N, K, 0xBEEF)
+    s = np.full((N, K // 64), synth.f32_to_bf16_bits(np.float32(s0)), dtype=np.uint16)
+    b = np.full((N, K // 64), synth.f32_to_bf16_bits(np.float32(b0)), dtype=np.uint16)
+    x = synth.f32_to_bf16_bits(refgen.lcg_act(M * K, 21).reshape(M, K))
+    y64, yb = oracle.qmm(packed, s, b, x, K, N, M)
+    got = D.bits(vpq.qmm_w4g64(*stage(D, dev, packed, s, b, x), K, N, M))
+    parity.check_bf16(got, y64, yb)
+
+
+@pytest.mark.parametrize("r,alpha", [(32, 1.0), (64, 0.625), (128, 2.0)])
+def test_qmm_lora_fused(vpq, oracle, dev, D, r, alpha):
+    M, N, K = 96, 160, 512
+    w, s, b = synth.make_weight(N, K, 23)
+    s[:] = synth.f32_to_bf16_bits(np.float32(0.0005))      # small base: the delta is a visible part of y
+    b[:] = synth.f32_to_bf16_bits(np.float32(-0.004))
+    x = synth.f32_to_bf16_bits(refgen.lcg_act(M * K, 21).reshape(M, K))
+    A = synth.f32_to_bf16_bits(refgen.lcg_act(r * K, 29).reshape(r, K))
+    B = synth.f32_to_bf16_bits(refgen.lcg_act(N * r, 31).reshape(N, r))
+    t_ref = oracle.lora_t(x, A, M, K, r, alpha)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    Ad, Bd = D.bf16(A, dev), D.bf16(B, dev)
+    t = vpq.lora_a(xd, Ad, M, K, r, alpha)
+    t_bits = D.bits(t)
+    assert parity.bf16_ulp_distance(t_bits, t_ref).max() <= 1
+    # the fused tile consumes the t the library produced: oracle on that same t
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M, t=t_bits, B=B, r=r)
+    t_ws = torch.empty((M, r), dtype=torch.bfloat16, device=dev)
+    got = D.bits(vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, lora_A=Ad, lora_B=Bd, r=r, alpha=alpha, t_ws=t_ws))
+    assert np.array_equal(D.bits(t_ws), t_bits)
+    parity.check_bf16(got, y64, yb)
+    # float64 end to end: the reference's bar (rel-L2 < 5e-3, delta > 5% of the output)
+    xf = synth.bf16_bits_to_f32(x).astype(np.float64)
+    Wb = synth.bf16_bits_to_f32(oracle.dequant_bf16(w, s, b, K, N)).astype(np.float64)
+    d = alpha * (xf @ synth.bf16_bits_to_f32(A).astype(np.float64).T) @ synth.bf16_bits_to_f32(B).astype(np.float64).T
+    want = xf @ Wb.T + d
+    assert parity.rel_l2(synth.bf16_bits_to_f32(got), want) < 5e-3
+    assert np.sqrt((d ** 2).sum() / (want ** 2).sum()) > 0.05
+
+
+def test_qmm_lora_scale_zero_is_exactly_off(vpq, dev, D):
+    # minimax_h3_lora: strength 0 == no adapter, bit for bit (metal-minimax-h3-transformer.cc:2211-2219)
+    M, N, K, r = 70, 130, 256, 32
+    w, s, b = synth.make_weight(N, K, 3)
+    x = synth.make_act(M, K, 4)
+    A, B = synth.make_lora(N, K, r, 5)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    base = D.bits(vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M))
+    off = D.bits(vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, lora_A=D.bf16(A, dev), lora_B=D.bf16(B, dev),
+                               r=r, alpha=0.0))
+    assert np.array_equal(base, off)
+
+
+def _sampled_check(vpq, oracle, dev, D, M, N, K, seed, lora_r=0, alpha=1.0):
+    """Full-size launch; oracle on a sample of rows of x and rows of W (tile edges included)."""
+    w, s, b = synth.make_weight(N, K, seed)
+    x = synth.make_act(M, K, seed + 1)
+    rng = np.random.default_rng(seed + 2)
+    ms = np.unique(np.concatenate([np.arange(4), np.arange(M - 4, M), rng.integers(0, M, 40)]))
+    ns = np.unique(np.concatenate([np.arange(4), np.arange(N - 4, N), rng.integers(0, N, 56)]))
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    kw = {}
+    t_bits = B = None
+    if lora_r:
+        A, B = synth.make_lora(N, K, lora_r, seed + 3)
+        kw = dict(lora_A=D.bf16(A, dev), lora_B=D.bf16(B, dev), r=lora_r, alpha=alpha,
+                  t_ws=torch.empty((M, lora_r), dtype=torch.bfloat16, device=dev))
+    y = vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, **kw)
+    torch.cuda.synchronize()
+    got = D.bits(y[torch.from_numpy(ms).to(dev)][:, torch.from_numpy(ns).to(dev)])
+    if lora_r:
+        t_all = D.bits(kw["t_ws"])
+        t_ref = oracle.lora_t(x[ms], A, len(ms), K, lora_r, alpha)
+        assert parity.bf16_ulp_distance(t_all[ms], t_ref).max() <= 1
+        t_bits, B = t_all[ms], B[ns]
+    y64, yb = oracle.qmm(w[ns], s[ns], b[ns], x[ms], K, len(ns), len(ms), t=t_bits, B=B, r=lora_r)
+    parity.check_bf16(got, y64, yb)
+    return y
+
+
+@pytest.mark.parametrize("K,N", [(4096, 12288), (12288, 4096), (4096, 4096)])
+def test_qmm_prefill_shapes(vpq, oracle, dev, D, K, N):
+    _sampled_check(vpq, oracle, dev, D, 2048, N, K, 0x5EED0004 + N)
+
+
+@pytest.mark.parametrize("K,N", [(5120, 5120), (5120, 20480), (20480, 5120)])
+def test_qmm_video_dit_shapes_with_lora(vpq, oracle, dev, D, K, N):
+    # M = 16320 = 127*128 + 64: an M tail; y of 5120->20480 is 668 MB: 64-bit addressing
+    _sampled_check(vpq, oracle, dev, D, 16320, N, K, 0x5EED0005 + N, lora_r=32, alpha=1.0)

@@ -1,0 +1,343 @@
+"""Pins for the CPU oracle (oracle/vpq_oracle.c).
+
+The reference holds no golden files for this path and cannot run here, so the
+oracle is pinned by (a) library routines it must reduce to (torch / numpy casts,
+float64 matmul over an independently unpacked weight), (b) closed forms and
+degenerate cases whose answer is fixed by the mathematics, and (c) the reference
+tests' own procedural inputs with the tolerances those tests assert.  Each check
+is chosen so that a plausible mistake -- wrong nibble order, a dropped bias
+term, a transposed operand, a double rounding -- fails it.
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.golden import refgen
+from vpipe_amd import synth
+
+G = 64
+
+
+def np_unpack(w, K):
+    """Independent unpack from the second layout statement of the reference
+    (affine_qmm_mma.metal:98-99 / metal-compute-gemm-mma.cc:276-280): byte b of a
+    row holds k=2b in its low nibble and k=2b+1 in its high nibble."""
+    by = np.ascontiguousarray(w).view(np.uint8).reshape(w.shape[0], -1)
+    q = np.empty((w.shape[0], K), dtype=np.uint8)
+    q[:, 0::2] = by & 0x0F
+    q[:, 1::2] = by >> 4
+    return q
+
+
+def np_dequant64(w, s, b, K):
+    q = np_unpack(w, K).astype(np.float64)
+    sf = synth.bf16_bits_to_f32(s).astype(np.float64)
+    bf = synth.bf16_bits_to_f32(b).astype(np.float64)
+    return np.repeat(sf, G, axis=1) * q + np.repeat(bf, G, axis=1)
+
+
+# ---- conversions ------------------------------------------------------------
+
+def test_bf16_rne_matches_torch_everywhere(oracle):
+    # every bf16 value, its 2 neighbours' midpoints (ties) and points just off them
+    hi = np.arange(0, 1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF], dtype=np.uint32)
+    bits = (hi[:, None] | lows[None, :]).ravel()
+    f = bits.view(np.float32)
+    finite = np.isfinite(f)
+    got = oracle.f32_to_bf16(f[finite])
+    want = torch.from_numpy(f[finite].copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+    # the numpy twin used to generate inputs agrees too
+    assert np.array_equal(synth.f32_to_bf16_bits(f[finite]), want)
+
+
+def test_f16_conversions_match_numpy(oracle):
+    all16 = np.arange(0, 1 << 16, dtype=np.uint16)
+    want = all16.view(np.float16).astype(np.float32)
+    got = oracle.f16_to_f32(all16)
+    ok = np.isfinite(want)
+    assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
+    rng = np.random.default_rng(1)
+    f = np.concatenate([
+        rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-8, 5, 200000),
+        want[ok],                                              # exactly representable
+        (want[ok] * np.float32(1.0 + 2.0 ** -11)),             # near ties
+        np.array([65504.0, 65519.9, 65520.0, 1e-8, 5.96e-8, 2.98e-8, 0.0, -0.0], dtype=np.float32),
+    ]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want16 = f.astype(np.float16).view(np.uint16)
+    assert np.array_equal(oracle.f32_to_f16(f), want16)
+
+
+# ---- layout + dequant -------------------------------------------------------
+
+def test_dequant_matches_independent_numpy(oracle):
+    N, K = 24, 256
+    w, s, b = synth.make_weight(N, K, 11)
+    want = np_dequant64(w, s, b, K)          # exact in float64: s*q has 12 significant bits
+    got32 = oracle.dequant_f32(w, s, b, K, N)
+    assert np.array_equal(got32, want.astype(np.float32))
+    got16 = oracle.dequant_bf16(w, s, b, K, N)
+    want16 = torch.from_numpy(want.astype(np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got16, want16)
+
+
+def test_dequant_layout_known_answer(oracle):
+    # one word 0x76543210 per row: nibble i == i, so W[n, 8j+i] = s*i + b
+    N, K = 2, 64
+    w = np.full((N, K // 8), 0x76543210, dtype=np.uint32)
+    w[1, 3] = 0xFEDCBA98
+    s = synth.f32_to_bf16_bits(np.array([[0.5], [0.25]], dtype=np.float32))
+    b = synth.f32_to_bf16_bits(np.array([[-1.0], [2.0]], dtype=np.float32))
+    d = oracle.dequant_f32(w, s, b, K, N)
+    assert np.array_equal(d[0, :8], 0.5 * np.arange(8) - 1.0)
+    assert np.array_equal(d[1, 24:32], 0.25 * np.arange(8, 16) + 2.0)
+    assert np.array_equal(d[1, :8], 0.25 * np.arange(8) + 2.0)
+
+
+def test_pack_unpack_roundtrip_and_sizes(oracle):
+    rng = np.random.default_rng(5)
+    q = rng.integers(0, 16, size=(7, 128), dtype=np.uint8)
+    w = synth.pack_nibbles(q)
+    assert np.array_equal(synth.unpack_nibbles(w, 128), q)
+    assert np.array_equal(np_unpack(w, 128), q)
+    # generative-models/quantize/affine-quantizer.h:37-40
+    assert oracle.lib().vpo_weight_bytes(96, 256) == 96 * 32 * 4
+    assert oracle.lib().vpo_scale_bytes(96, 256) == 96 * 4 * 2
+
+
+# ---- QMV / QMM: what the mathematics fixes ----------------------------------
+
+@pytest.mark.parametrize("M", [1, 3])
+def test_one_hot_activation_reads_back_the_weight(oracle, M):
+    # x = e_k  =>  y[n] = W[n,k]; pushes layout and dequant through the full matmul
+    N, K = 16, 192
+    w, s, b = synth.make_weight(N, K, 21)
+    d32 = oracle.dequant_f32(w, s, b, K, N)
+    d16 = oracle.dequant_bf16(w, s, b, K, N)
+    for k in [0, 1, 7, 8, 63, 64, 130, K - 1]:
+        x = np.zeros((M, K), dtype=np.float32)
+        x[M - 1, k] = 1.0
+        xb = synth.f32_to_bf16_bits(x)
+        y64, yb = oracle.qmv(w, s, b, xb, K, N, M)
+        assert np.array_equal(y64[M - 1], d32[:, k].astype(np.float64))
+        assert np.array_equal(yb[M - 1], synth.f32_to_bf16_bits(d32[:, k]))
+        assert not y64[: M - 1].any()
+        z64, zb = oracle.qmm(w, s, b, xb, K, N, M)
+        assert np.array_equal(zb[M - 1], d16[:, k])          # QMM sees the bf16-rounded weight
+        assert np.array_equal(z64[M - 1], synth.bf16_bits_to_f32(d16[:, k]).astype(np.float64))
+
+
+def test_degenerate_quantizers(oracle):
+    N, K, M = 8, 256, 2
+    rng = np.random.default_rng(3)
+    x = synth.make_act(M, K, 4)
+    xf = synth.bf16_bits_to_f32(x).astype(np.float64)
+    w, s, b = synth.make_weight(N, K, 5)
+    # all codes zero: y = sum_g b_g * sum_{k in g} x_k
+    w0 = np.zeros_like(w)
+    y64, _ = oracle.qmv(w0, s, b, x, K, N, M)
+    want = xf.reshape(M, K // G, G).sum(axis=2) @ synth.bf16_bits_to_f32(b).astype(np.float64).T
+    assert np.allclose(y64, want, rtol=1e-12, atol=1e-12)
+    # q = 8 everywhere with b = -8 s: every weight is exactly 0
+    w8 = np.full_like(w, 0x88888888)
+    b8 = synth.f32_to_bf16_bits(-8.0 * synth.bf16_bits_to_f32(s))
+    for fn in (oracle.qmv, oracle.qmm):
+        y64, yb = fn(w8, s, b8, x, K, N, M)
+        assert not y64.any() and not yb.any()
+    # scale 0: bias only, whatever the codes
+    s0 = np.zeros_like(s)
+    y64a, _ = oracle.qmv(w, s0, b, x, K, N, M)
+    assert np.allclose(y64a, want, rtol=1e-12, atol=1e-12)
+    del rng
+
+
+@pytest.mark.parametrize("K,N,M", [(64, 5, 1), (512, 33, 4), (4096, 32, 2), (5120, 16, 16)])
+def test_matmul_matches_float64_numpy(oracle, K, N, M):
+    w, s, b = synth.make_weight(N, K, 100 + K)
+    x = synth.make_act(M, K, 200 + K)
+    xf = synth.bf16_bits_to_f32(x).astype(np.float64)
+    W = np_dequant64(w, s, b, K)                              # un-rounded weight, exact
+    W32 = W.astype(np.float32).astype(np.float64)             # the fp32 the QMV path holds
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    assert np.allclose(y64, xf @ W32.T, rtol=1e-11, atol=1e-9)
+    # factored form (scale*sum(x q) + bias*sum(x)) is the same number up to fp32(s*q+b) rounding
+    yf = oracle.qmv_factored(w, s, b, x, K, N, M)
+    assert np.allclose(yf, xf @ W.T, rtol=1e-11, atol=1e-9)
+    scale = np.sqrt((y64 ** 2).mean())
+    assert np.abs(yf - y64).max() < 2e-6 * scale + 1e-6
+    # QMM path: bf16-rounded weight
+    Wb = synth.bf16_bits_to_f32(synth.f32_to_bf16_bits(W.astype(np.float32))).astype(np.float64)
+    z64, zb = oracle.qmm(w, s, b, x, K, N, M)
+    assert np.allclose(z64, xf @ Wb.T, rtol=1e-11, atol=1e-9)
+    assert np.array_equal(zb, synth.f32_to_bf16_bits(z64.astype(np.float32)))
+    assert np.array_equal(yb, synth.f32_to_bf16_bits(y64.astype(np.float32)))
+
+
+def test_linearity_in_x(oracle):
+    K, N = 512, 12
+    w, s, b = synth.make_weight(N, K, 31)
+    # activations on a coarse grid so x1+x2 is exact in bf16
+    rng = np.random.default_rng(32)
+    x1 = (rng.integers(-64, 64, size=(1, K)) / 32.0).astype(np.float32)
+    x2 = (rng.integers(-64, 64, size=(1, K)) / 32.0).astype(np.float32)
+    ya, _ = oracle.qmv(w, s, b, synth.f32_to_bf16_bits(x1), K, N, 1)
+    yb_, _ = oracle.qmv(w, s, b, synth.f32_to_bf16_bits(x2), K, N, 1)
+    yc, _ = oracle.qmv(w, s, b, synth.f32_to_bf16_bits(x1 + x2), K, N, 1)
+    assert np.allclose(ya + yb_, yc, rtol=1e-12, atol=1e-10)
+
+
+def test_residual_add_rounds_twice(oracle):
+    # affine_qmv.metal:264-266: v = (T)result; v += residual  (element-type add)
+    K, N = 128, 9
+    w, s, b = synth.make_weight(N, K, 41)
+    x = synth.make_act(1, K, 42)
+    res = synth.make_act(1, N, 43)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, 1)
+    _, yr = oracle.qmv(w, s, b, x, K, N, 1, residual=res)
+    a = torch.from_numpy(yb.view(np.int16)).view(torch.bfloat16)
+    r = torch.from_numpy(res.view(np.int16)).view(torch.bfloat16)
+    want = (a + r).view(torch.int16).numpy().view(np.uint16)   # torch adds bf16 in fp32 and rounds
+    assert np.array_equal(yr, want)
+
+
+# ---- the reference tests' own inputs and tolerances -------------------------
+
+def test_reference_qmv_case_tail_and_padding(oracle):
+    """metal_lm_smoke.qmv_w4g32_matches_cpu (tests/unit-tests/metal-lm/quant-gemv.cc:207-300)
+    at group 64: N=16, K=3840 (not a multiple of 512), x padded to 4096 with
+    non-zero values, one garbage weight row appended.  The oracle must (a) ignore
+    everything past K and past row N and (b) agree with an independent float64
+    evaluation within the test's own tolerance 0.03 (it agrees to 1e-6)."""
+    N, K = 16, 3840
+    c = refgen.knuth_qmv_case(N, K, group=64)
+    s = synth.f32_to_bf16_bits(c["scales"])
+    b = synth.f32_to_bf16_bits(c["biases"])
+    x = synth.f32_to_bf16_bits(c["x"])[None, :]                 # [1, 4096]
+    w_all = c["packed"]                                          # [17, K/8]
+    assert np.array_equal(np_unpack(w_all[:N], K), c["q"])
+    y64, _ = oracle.qmv(w_all[:N], s, b, x[:, :K], K, N, 1)
+    # CPU loop of the test: acc(double) += x[k] * (s*q + b)
+    W32 = (synth.bf16_bits_to_f32(s).repeat(G, axis=1) * c["q"].astype(np.float32)
+           + synth.bf16_bits_to_f32(b).repeat(G, axis=1)).astype(np.float32)
+    ref = (synth.bf16_bits_to_f32(x[0, :K]).astype(np.float64)[None, :] * W32.astype(np.float64)).sum(axis=1)
+    maxrel = np.abs(y64[0] - ref) / (np.abs(ref) + 1e-2)
+    assert maxrel.max() < 1e-9
+    # poisoned tail: feeding the padded x with K=4096 against garbage gives a different answer
+    assert np.abs(ref).min() > 1.0                              # all-positive x: no cancellation, as the test notes
+
+
+def test_reference_lcg_weight_case(oracle):
+    """make_act_/make_qw_ inputs (tests/unit-tests/minimax-h3-blocks.cc:121-158):
+    s = 0.01, b = -0.08 everywhere, LCG code bytes and activations."""
+    N, K, M = 32, 256, 5
+    packed, s0, b0 = refgen.lcg_qweight(N, K, 0x1234)
+    s = np.full((N, K // G), synth.f32_to_bf16_bits(np.float32(s0)), dtype=np.uint16)
+    b = np.full((N, K // G), synth.f32_to_bf16_bits(np.float32(b0)), dtype=np.uint16)
+    x = synth.f32_to_bf16_bits(refgen.lcg_act(M * K, 21).reshape(M, K))
+    q = np_unpack(packed, K).astype(np.float64)
+    sf = float(synth.bf16_bits_to_f32(s[0, 0]))
+    bf = float(synth.bf16_bits_to_f32(b[0, 0]))
+    Wb = synth.bf16_bits_to_f32(synth.f32_to_bf16_bits((sf * q + bf).astype(np.float32))).astype(np.float64)
+    want = synth.bf16_bits_to_f32(x).astype(np.float64) @ Wb.T
+    z64, zb = oracle.qmm(packed, s, b, x, K, N, M)
+    assert np.allclose(z64, want, rtol=1e-12, atol=1e-12)
+    rel_l2 = np.sqrt(((synth.bf16_bits_to_f32(zb) - want) ** 2).sum() / (want ** 2).sum())
+    assert rel_l2 < 3e-2                                         # metal-compute-gemm-mma.cc:490 bar
+    assert rel_l2 < 3e-3                                         # what one bf16 store actually costs
+
+
+# ---- LoRA --------------------------------------------------------------------
+
+def test_lora_matches_float64_and_reference_tolerance(oracle):
+    """minimax_h3_blocks.lora_accumulate_matches_reference
+    (tests/unit-tests/minimax-h3-blocks.cc:1162-1296) at a reduced shape: same
+    generators (seeds 21/29/31), strength 0.625, rel-L2 < 5e-3 vs float64 and a
+    delta that is a real part of the output."""
+    M, N, K, R = 24, 48, 512, 64
+    scale = 0.625
+    x = synth.f32_to_bf16_bits(refgen.lcg_act(M * K, 21).reshape(M, K))
+    A = synth.f32_to_bf16_bits(refgen.lcg_act(R * K, 29).reshape(R, K))
+    B = synth.f32_to_bf16_bits(refgen.lcg_act(N * R, 31).reshape(N, R))
+    w, s, b = synth.make_weight(N, K, 23)
+    # shrink the base so the adapter is a visible part of the output, as in the reference case
+    s[:] = synth.f32_to_bf16_bits(np.float32(0.0005))
+    b[:] = synth.f32_to_bf16_bits(np.float32(-0.004))
+    t = oracle.lora_t(x, A, M, K, R, scale)
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M, t=t, B=B, r=R)
+    xf = synth.bf16_bits_to_f32(x).astype(np.float64)
+    Wb = synth.bf16_bits_to_f32(oracle.dequant_bf16(w, s, b, K, N)).astype(np.float64)
+    base = xf @ Wb.T
+    d = scale * (xf @ synth.bf16_bits_to_f32(A).astype(np.float64).T) @ synth.bf16_bits_to_f32(B).astype(np.float64).T
+    want = base + d
+    got = synth.bf16_bits_to_f32(yb).astype(np.float64)
+    rl2 = np.sqrt(((got - want) ** 2).sum() / (want ** 2).sum())
+    assert rl2 < 5e-3
+    assert np.sqrt((d ** 2).sum() / (want ** 2).sum()) > 0.05
+    # t itself: two roundings, bf16(scale * bf16(x.A^T))
+    tt = (xf @ synth.bf16_bits_to_f32(A).astype(np.float64).T).astype(np.float32)
+    once = synth.bf16_bits_to_f32(synth.f32_to_bf16_bits(tt))
+    assert np.array_equal(t, synth.f32_to_bf16_bits(once * np.float32(scale)))
+    # an adapter whose t is zero leaves the base untouched, bit for bit
+    _, y0 = oracle.qmm(w, s, b, x, K, N, M)
+    _, y1 = oracle.qmm(w, s, b, x, K, N, M, t=np.zeros_like(t), B=B, r=R)
+    assert np.array_equal(y0, y1)
+
+
+# ---- the packer ----------------------------------------------------------------
+
+def test_quantize_recovers_on_grid_weights_exactly(oracle):
+    # a weight already of the form s*q + b with f16-exact s, b and every group
+    # spanning 0..15 must come back with the same codes, scale and bias
+    N, K = 6, 256
+    rng = np.random.default_rng(7)
+    q = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    q.reshape(N, K // G, G)[:, :, 0] = 0
+    q.reshape(N, K // G, G)[:, :, 1] = 15
+    s = (rng.integers(1, 64, size=(N, K // G)) / 1024.0).astype(np.float32)      # f16-exact
+    b = (-rng.integers(0, 256, size=(N, K // G)) / 256.0).astype(np.float32)
+    W = (np.repeat(s, G, axis=1) * q + np.repeat(b, G, axis=1)).astype(np.float32)
+    codes, sf16, bf16_ = oracle.quantize(W, K, N)
+    assert np.array_equal(synth.unpack_nibbles(codes, K), q)
+    assert np.array_equal(sf16.view(np.float16).astype(np.float32), s)
+    assert np.array_equal(bf16_.view(np.float16).astype(np.float32), b)
+
+
+def test_quantize_roundtrip_bounds_of_the_reference(oracle):
+    """model_quantize_roundtrip.affine_writer_reader_dequant
+    (tests/unit-tests/model-quantize-roundtrip.cc:84-164): N=96, K=256 ramp+ripple
+    source; 4-bit rel-L2 < 0.20; byte sizes."""
+    N, K = 96, 256
+    n = np.arange(N)[:, None]
+    k = np.arange(K)[None, :]
+    v = 0.4 * np.sin(0.05 * k + 0.3 * n) + 0.1 * np.cos(0.7 * k) + 0.002 * (k - K / 2)
+    src = v.astype(np.float16).astype(np.float32)
+    codes, sf16, bf16_ = oracle.quantize(src, K, N)
+    assert codes.nbytes == 96 * 32 * 4 and sf16.nbytes == 96 * 4 * 2
+    sb = oracle.f16_to_bf16(sf16)
+    bb = oracle.f16_to_bf16(bf16_)
+    deq = synth.bf16_bits_to_f32(oracle.dequant_bf16(codes, sb, bb, K, N)).astype(np.float64)
+    err = np.sqrt(((deq - src) ** 2).sum() / (src.astype(np.float64) ** 2).sum())
+    assert err < 0.20
+    # numpy re-derivation of the code assignment (round half away from zero)
+    g = src.reshape(N, K // G, G)
+    mn = g.min(axis=2, keepdims=True)
+    mx = g.max(axis=2, keepdims=True)
+    sc = ((mx - mn) / np.float32(15.0)).astype(np.float32)
+    inv = np.where(sc > 0, np.float32(1.0) / sc, np.float32(0.0)).astype(np.float32)
+    t = ((g - mn) * inv).astype(np.float32)
+    qn = np.clip(np.floor(t + np.float32(0.5)), 0, 15).astype(np.uint8).reshape(N, K)
+    assert np.array_equal(synth.unpack_nibbles(codes, K), qn)
+    assert np.array_equal(sf16, sc.astype(np.float16).view(np.uint16).reshape(N, K // G))
+
+
+def test_cpu_baseline_is_the_same_algorithm(oracle):
+    K, N, M = 512, 40, 3
+    w, s, b = synth.make_weight(N, K, 51)
+    x = synth.make_act(M, K, 52)
+    y = oracle.cpu_dequant_matmul(w, s, b, x, K, N, M)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    got = synth.bf16_bits_to_f32(y).astype(np.float64)
+    assert np.abs(got - y64).max() <= 2.0 ** -7 * np.abs(y64).max()
+    assert (y != yb).mean() < 0.05

@@ -1,0 +1,10 @@
+"""MI355X (gfx950) implementation of VPIPE's 4-bit / group-64 affine quantized
+linear path: QMV, QMM (+ fused runtime LoRA), dense expansion and the packer.
+
+The product is the C-ABI shared library `libvpq.so` (include/vpq.h).  This
+package only loads it and hands it torch device pointers; it contains no CPU
+implementation of any operator and raises if the library is missing.
+"""
+from . import capi  # noqa: F401
+from .capi import (VpqError, dequant_w4g64, f16_to_bf16, lib_path, linear_w4g64, load, lora_a,  # noqa: F401
+                   qmm_w4g64, qmv_w4g64, qmv_workspace, quantize_w4g64)

@@ -1,0 +1,165 @@
+"""ctypes binding of libvpq.so for tests and the benchmark.
+
+torch supplies device memory and the stream; every call goes through the C ABI
+of include/vpq.h with raw device pointers.  There is no fallback: a missing
+library or a non-zero status raises.
+
+Tensor conventions: packed codes are int32 tensors viewed as uint32 words
+[N, K/8]; bf16 data are torch.bfloat16 tensors (or int16 tensors holding the
+bit patterns).
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libvpq.so")
+_lib = None
+
+VPQ_QMV_AUTO, VPQ_QMV_SIMPLE, VPQ_QMV_MFMA, VPQ_QMV_MFMA_SPLITK = 0, 1, 2, 3
+
+# Every symbol include/vpq.h declares: (name, restype, argtypes).
+_vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+SYMBOLS = [
+    ("vpq_version", _i, []),
+    ("vpq_status_string", ctypes.c_char_p, [_i]),
+    ("vpq_last_device_error", ctypes.c_char_p, []),
+    ("vpq_init", _i, []),
+    ("vpq_device_cu_count", _i, []),
+    ("vpq_dequant_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
+    ("vpq_qmv_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _i]),
+    ("vpq_qmv_workspace_bytes", _sz, [_i, _i, _i]),
+    ("vpq_qmm_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _f, _vp]),
+    ("vpq_lora_a_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f]),
+    ("vpq_linear_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz]),
+    ("vpq_quantize_w4g64", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
+    ("vpq_f16_to_bf16", _i, [_vp, _vp, _vp, _sz]),
+    ("vpq_profile_enable", _i, [_i]),
+    ("vpq_profile_read", _i, [_vp, _i]),
+    ("vpq_weight_bytes", _sz, [_i, _i]),
+    ("vpq_scale_bytes", _sz, [_i, _i]),
+]
+
+
+class VpqError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = load().vpq_status_string(status).decode()
+        dev = load().vpq_last_device_error().decode()
+        super().__init__("%s: %s (%d)%s" % (where, msg, status, (" [" + dev + "]") if dev else ""))
+
+
+def lib_path():
+    return _SO
+
+
+def load():
+    """dlopen libvpq.so (built by `python -m vpipe_amd.build`); raises if absent."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            raise FileNotFoundError(
+                "%s is missing: build it with `python -m vpipe_amd.build` (hipcc, gfx950)" % _SO)
+        import torch  # noqa: F401  -- loads the HIP runtime libvpq.so binds to
+        L = ctypes.CDLL(_SO)
+        for name, res, args in SYMBOLS:
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(st, where):
+    if st != 0:
+        raise VpqError(st, where)
+
+
+def qmv_workspace(K, N, M, device="cuda"):
+    """Zero-filled split-K scratch for qmv_w4g64 (reusable across calls on one stream)."""
+    import torch
+    nbytes = load().vpq_qmv_workspace_bytes(K, N, M)
+    return torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)
+
+
+def dequant_w4g64(w, scales, biases, K, N, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((N, K), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_dequant_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out), K, N),
+           "vpq_dequant_w4g64_bf16")
+    return out
+
+
+def qmv_w4g64(w, scales, biases, x, K, N, M, out=None, residual=None, ws=None, variant=0, f32out=False):
+    import torch
+    L = load()
+    ws_bytes = 0 if ws is None else ws.numel() * ws.element_size()
+    if f32out:
+        if out is None:
+            out = torch.empty((M, N), dtype=torch.float32, device=w.device)
+        _check(L.vpq_qmv_w4g64_f32out(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                      K, N, M, _ptr(ws), ws_bytes, variant), "vpq_qmv_w4g64_f32out")
+        return out
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _check(L.vpq_qmv_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                K, N, M, _ptr(residual), _ptr(ws), ws_bytes, variant), "vpq_qmv_w4g64_bf16")
+    return out
+
+
+def lora_a(x, A, M, K, r, alpha, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, r), dtype=torch.bfloat16, device=x.device)
+    _check(load().vpq_lora_a_bf16(_stream(), _ptr(x), _ptr(A), _ptr(out), M, K, r, alpha), "vpq_lora_a_bf16")
+    return out
+
+
+def qmm_w4g64(w, scales, biases, x, K, N, M, out=None, lora_A=None, lora_B=None, r=0, alpha=0.0, t_ws=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    if lora_A is not None and t_ws is None:
+        t_ws = torch.empty((M, r), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                     K, N, M, _ptr(lora_A), _ptr(lora_B), r, alpha, _ptr(t_ws)),
+           "vpq_qmm_w4g64_bf16")
+    return out
+
+
+def linear_w4g64(w, scales, biases, x, K, N, M, out=None, ws=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    ws_bytes = 0 if ws is None else ws.numel() * ws.element_size()
+    _check(load().vpq_linear_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                        K, N, M, _ptr(ws), ws_bytes), "vpq_linear_w4g64_bf16")
+    return out
+
+
+def quantize_w4g64(src, K, N, clip=1.0):
+    """bf16 [N,K] -> (codes int32 [N,K/8], scales f16 bits int16 [N,K/64], biases f16 bits)."""
+    import torch
+    w = torch.empty((N, K // 8), dtype=torch.int32, device=src.device)
+    s = torch.empty((N, K // 64), dtype=torch.int16, device=src.device)
+    b = torch.empty((N, K // 64), dtype=torch.int16, device=src.device)
+    _check(load().vpq_quantize_w4g64(_stream(), _ptr(src), _ptr(w), _ptr(s), _ptr(b), K, N, clip),
+           "vpq_quantize_w4g64")
+    return w, s, b
+
+
+def f16_to_bf16(t):
+    import torch
+    out = torch.empty(t.shape, dtype=torch.int16, device=t.device)
+    _check(load().vpq_f16_to_bf16(_stream(), _ptr(t), _ptr(out), t.numel()), "vpq_f16_to_bf16")
+    return out

@@ -1,0 +1,292 @@
+// The C ABI (include/vpq.h): argument validation, device check and kernel
+// selection.  Nothing here allocates device memory or synchronises.
+#include "../../include/vpq.h"
+
+#include <hip/hip_runtime.h>
+#include <string.h>
+
+#include <atomic>
+#include <mutex>
+
+#include "vpq_internal.h"
+
+namespace vpq {
+ProfileState& profile_state()
+{
+  static ProfileState ps;
+  return ps;
+}
+}  // namespace vpq
+
+namespace {
+
+struct DeviceState {
+  std::atomic<int> status{1};  // 1 = not initialised, 0 = ok, <0 = vpq_status
+  int cu_count = 0;
+};
+
+DeviceState g_dev;
+std::mutex g_init_mutex;
+thread_local char g_last_error[256] = "";
+
+int device_error(hipError_t e)
+{
+  const char* s = hipGetErrorString(e);
+  strncpy(g_last_error, s ? s : "unknown HIP error", sizeof(g_last_error) - 1);
+  g_last_error[sizeof(g_last_error) - 1] = '\0';
+  return VPQ_ERR_DEVICE;
+}
+
+int ensure_init()
+{
+  int st = g_dev.status.load(std::memory_order_acquire);
+  if (st <= 0) { return st; }
+  std::lock_guard<std::mutex> lock(g_init_mutex);
+  st = g_dev.status.load(std::memory_order_acquire);
+  if (st <= 0) { return st; }
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { return device_error(e); }
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) { return device_error(e); }
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    strncpy(g_last_error, "device is not gfx950", sizeof(g_last_error) - 1);
+    g_dev.status.store(VPQ_ERR_UNSUPPORTED, std::memory_order_release);
+    return VPQ_ERR_UNSUPPORTED;
+  }
+  g_dev.cu_count = prop.multiProcessorCount;
+  g_dev.status.store(VPQ_OK, std::memory_order_release);
+  return VPQ_OK;
+}
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+inline int finish(hipError_t e) { return e == hipSuccess ? VPQ_OK : device_error(e); }
+
+int check_pack(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, int K, int N)
+{
+  if (w == nullptr || scales == nullptr || biases == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (K <= 0 || N <= 0 || (K % 64) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  // Rows of codes are K/2 bytes, a multiple of 32: 16-byte alignment of the base
+  // makes every 128-bit load of the kernels aligned.  Scales/biases are read
+  // with 2-byte loads by the general kernels; the vector paths need 16.
+  if (!aligned(w, 16) || !aligned(scales, 2) || !aligned(biases, 2)) { return VPQ_ERR_MISALIGNED; }
+  return VPQ_OK;
+}
+
+int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+               const uint16_t* biases, const uint16_t* x, void* y, bool y_f32, int K, int N, int M,
+               const uint16_t* residual, void* ws, size_t ws_bytes, int variant)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
+  if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
+  if (ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }
+  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_MFMA_SPLITK) { return VPQ_ERR_BAD_SHAPE; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+
+  vpq::QmvArgs a;
+  a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y; a.residual = residual;
+  a.K = K; a.N = N; a.M = M; a.y_f32 = y_f32; a.ws = ws; a.ws_bytes = ws_bytes;
+  a.cu_count = g_dev.cu_count;
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+
+  const bool mfma_ok = vpq::qmv_mfma_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
+  if (variant == VPQ_QMV_SIMPLE) { return finish(vpq::launch_qmv_simple(hs, a)); }
+  if (variant == VPQ_QMV_MFMA || variant == VPQ_QMV_MFMA_SPLITK) {
+    if (!mfma_ok) { return VPQ_ERR_BAD_SHAPE; }
+    if (variant == VPQ_QMV_MFMA_SPLITK) {
+      if (ws == nullptr) { return VPQ_ERR_WORKSPACE; }
+      int splits = K / 512 < 4 ? K / 512 : 4;
+      if (splits < 2) { return VPQ_ERR_BAD_SHAPE; }
+      if (ws_bytes < vpq::qmv_mfma_workspace_bytes(K, N, M)) { return VPQ_ERR_WORKSPACE; }
+      return finish(vpq::launch_qmv_mfma(hs, a, splits));
+    }
+    return finish(vpq::launch_qmv_mfma(hs, a, 1));
+  }
+  if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a, 0)); }
+  return finish(vpq::launch_qmv_simple(hs, a));
+}
+
+}  // namespace
+
+extern "C" {
+
+int vpq_version(void) { return 100; }
+
+const char* vpq_status_string(int status)
+{
+  switch (status) {
+    case VPQ_OK: return "ok";
+    case VPQ_ERR_NULL_POINTER: return "a required buffer is NULL";
+    case VPQ_ERR_BAD_SHAPE: return "shape outside the supported domain";
+    case VPQ_ERR_MISALIGNED: return "pointer not aligned as required";
+    case VPQ_ERR_WORKSPACE: return "workspace missing or too small";
+    case VPQ_ERR_DEVICE: return "HIP runtime error";
+    case VPQ_ERR_UNSUPPORTED: return "device is not gfx950";
+    default: return "unknown status";
+  }
+}
+
+const char* vpq_last_device_error(void) { return g_last_error; }
+
+int vpq_init(void) { return ensure_init(); }
+
+int vpq_device_cu_count(void) { return g_dev.status.load() == VPQ_OK ? g_dev.cu_count : 0; }
+
+int vpq_dequant_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                           const uint16_t* biases, uint16_t* w_deq, int K, int N)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (w_deq == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (!aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_dequant(reinterpret_cast<hipStream_t>(stream), w, scales, biases, w_deq, K, N));
+}
+
+int vpq_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                       const uint16_t* residual, void* ws, size_t ws_bytes, int variant)
+{
+  return qmv_common(stream, w, scales, biases, x, y, false, K, N, M, residual, ws, ws_bytes, variant);
+}
+
+int vpq_qmv_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                         const uint16_t* biases, const uint16_t* x, float* y, int K, int N, int M,
+                         void* ws, size_t ws_bytes, int variant)
+{
+  return qmv_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr, ws, ws_bytes, variant);
+}
+
+size_t vpq_qmv_workspace_bytes(int K, int N, int M)
+{
+  if (K <= 0 || N <= 0 || M < 1 || M > 16) { return 0; }
+  return vpq::qmv_mfma_workspace_bytes(K, N, M);
+}
+
+int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t,
+                    int M, int K, int r, float alpha)
+{
+  if (x == nullptr || lora_a == nullptr || t == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M <= 0 || K <= 0 || (K % 64) != 0 || r <= 0 || r > 128 || (r % 32) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(lora_a, 16) || !aligned(t, 16)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::GemmArgs g{};
+  g.w = nullptr; g.b_dense = lora_a; g.x = x; g.y = t;
+  g.K = K; g.N = r; g.M = M; g.r = 0; g.out_scale = alpha; g.scaled_epilogue = true;
+  g.cu_count = g_dev.cu_count;
+  return finish(vpq::launch_gemm(reinterpret_cast<hipStream_t>(stream), g));
+}
+
+int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                       const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
+                       uint16_t* lora_t_ws)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16)) { return VPQ_ERR_MISALIGNED; }
+  const bool lora = lora_a != nullptr && alpha != 0.0f;
+  if (lora) {
+    if (lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
+    if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
+    if (r <= 0 || r > 128 || (r % 32) != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (!aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) { return VPQ_ERR_MISALIGNED; }
+  }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (lora) {
+    st = vpq_lora_a_bf16(stream, x, lora_a, lora_t_ws, M, K, r, alpha);
+    if (st != VPQ_OK) { return st; }
+  }
+  vpq::GemmArgs g{};
+  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
+  g.K = K; g.N = N; g.M = M;
+  g.lora_t = lora ? lora_t_ws : nullptr;
+  g.lora_b = lora ? lora_b : nullptr;
+  g.r = lora ? r : 0;
+  g.out_scale = 1.0f; g.scaled_epilogue = false;
+  g.cu_count = g_dev.cu_count;
+  return finish(vpq::launch_gemm(hs, g));
+}
+
+int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                          const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                          void* ws, size_t ws_bytes)
+{
+  if (M >= 1 && M <= 16) {
+    return vpq_qmv_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, nullptr, ws, ws_bytes, VPQ_QMV_AUTO);
+  }
+  return vpq_qmm_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, nullptr, nullptr, 0, 0.0f, nullptr);
+}
+
+int vpq_quantize_w4g64(vpq_stream_t stream, const uint16_t* src, uint32_t* w, uint16_t* scales_f16,
+                       uint16_t* biases_f16, int K, int N, float clip)
+{
+  if (src == nullptr || w == nullptr || scales_f16 == nullptr || biases_f16 == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (K <= 0 || N <= 0 || (K % 64) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(src, 16) || !aligned(w, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_quantize(reinterpret_cast<hipStream_t>(stream), src, w, scales_f16, biases_f16, K, N, clip));
+}
+
+int vpq_f16_to_bf16(vpq_stream_t stream, const uint16_t* in_f16, uint16_t* out_bf16, size_t count)
+{
+  if (in_f16 == nullptr || out_bf16 == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_f16_to_bf16(reinterpret_cast<hipStream_t>(stream), in_f16, out_bf16, count));
+}
+
+int vpq_profile_enable(int max_launches)
+{
+  vpq::ProfileState& ps = vpq::profile_state();
+  if (max_launches <= 0) {
+    ps.on = false;
+    return VPQ_OK;
+  }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  while (ps.events.size() < (size_t)max_launches * 2) {
+    hipEvent_t e;
+    const hipError_t err = hipEventCreate(&e);
+    if (err != hipSuccess) { return device_error(err); }
+    ps.events.push_back(e);
+  }
+  ps.used = 0;
+  ps.on = true;
+  return VPQ_OK;
+}
+
+int vpq_profile_read(float* kernel_ms, int capacity)
+{
+  vpq::ProfileState& ps = vpq::profile_state();
+  const int n = (int)(ps.used / 2);
+  for (int i = 0; i < n && i < capacity; ++i) {
+    hipError_t err = hipEventSynchronize(ps.events[2 * i + 1]);
+    if (err != hipSuccess) { return device_error(err); }
+    float ms = 0.0f;
+    err = hipEventElapsedTime(&ms, ps.events[2 * i], ps.events[2 * i + 1]);
+    if (err != hipSuccess) { return device_error(err); }
+    if (kernel_ms != nullptr) { kernel_ms[i] = ms; }
+  }
+  ps.used = 0;
+  return n;
+}
+
+size_t vpq_weight_bytes(int N, int K) { return (size_t)N * (size_t)(K * 4 / 32) * 4; }
+size_t vpq_scale_bytes(int N, int K) { return (size_t)N * (size_t)(K / 64) * 2; }
+
+}  // extern "C"

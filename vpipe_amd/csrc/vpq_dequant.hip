@@ -1,0 +1,134 @@
+// Bandwidth kernels around the packed format: dense expansion, the packer,
+// and the F16 -> bf16 conversion of scales/biases done once at load.
+#include "vpq_device.h"
+#include "vpq_internal.h"
+
+namespace vpq {
+
+// One thread per packed word: 4-byte coalesced loads, 16-byte coalesced
+// stores.  out = bf16_rne(fp32(s*q + b)); s*q is exact in fp32 (8-bit x 4-bit
+// significands), so the fused multiply-add below equals the two-step form of
+// gpu-kernels/metal/quant/affine_dequant.metal:45-52 bit for bit.
+__global__ __launch_bounds__(256) void dequant_w4g64_kernel(
+    const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
+    const uint16_t* __restrict__ biases, uint4* __restrict__ out, int Kw, size_t total_words)
+{
+  const int Kg = Kw >> 3;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total_words;
+       idx += (size_t)gridDim.x * 256) {
+    const size_t n = idx / (size_t)Kw;
+    const int j = (int)(idx - n * (size_t)Kw);
+    const size_t g = n * (size_t)Kg + (size_t)(j >> 3);
+    const float s = bf16_bits_to_f32(scales[g]);
+    const float b = bf16_bits_to_f32(biases[g]);
+    const uint32_t p = w[idx];
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { v[i] = fmaf(s, (float)((p >> (4 * i)) & 0xfu), b); }
+    uint4 o;
+    o.x = pack_bf16x2(v[0], v[1]);
+    o.y = pack_bf16x2(v[2], v[3]);
+    o.z = pack_bf16x2(v[4], v[5]);
+    o.w = pack_bf16x2(v[6], v[7]);
+    out[idx] = o;
+  }
+}
+
+hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* scales,
+                          const uint16_t* biases, uint16_t* out, int K, int N)
+{
+  const int Kw = K / 8;
+  const size_t total = (size_t)N * (size_t)Kw;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536 * 4) { blocks = 65536 * 4; }
+  return launch_kernel(dequant_w4g64_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, scales,
+                       biases, reinterpret_cast<uint4*>(out), Kw, total);
+}
+
+// One thread per 64-wide group, as the reference's packer
+// (gpu-kernels/metal/quant/affine_dequant.metal:243-285): min/max, optional
+// clip toward the midpoint, scale = (mx-mn)/15, q = clamp(round((v-mn)/scale)),
+// round half away from zero, scale and min emitted as IEEE F16.
+__global__ __launch_bounds__(64) void quantize_w4g64_kernel(
+    const uint16_t* __restrict__ src, uint32_t* __restrict__ w, uint16_t* __restrict__ s_f16,
+    uint16_t* __restrict__ b_f16, int K, int N, float clip)
+{
+  const int Kg = K / kGroup;
+  const int grp = blockIdx.x * 64 + threadIdx.x;
+  const int n = blockIdx.y;
+  if (grp >= Kg || n >= N) { return; }
+  const uint16_t* xp = src + (size_t)n * K + (size_t)grp * kGroup;
+  float v[kGroup];
+  float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kGroup / 8; ++i) {
+    const uint4 d = reinterpret_cast<const uint4*>(xp)[i];
+    const uint32_t dd[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[i * 8 + 2 * j] = bf16_lo_to_f32(dd[j]);
+      v[i * 8 + 2 * j + 1] = bf16_hi_to_f32(dd[j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kGroup; ++i) {
+    mn = fminf(mn, v[i]);
+    mx = fmaxf(mx, v[i]);
+  }
+  if (clip < 1.0f) {
+    const float mid = 0.5f * (mn + mx);
+    mn = mid + (mn - mid) * clip;
+    mx = mid + (mx - mid) * clip;
+  }
+  const float scale = (mx - mn) / 15.0f;
+  const float inv = (scale > 0.0f) ? 1.0f / scale : 0.0f;
+  s_f16[(size_t)n * Kg + grp] = __builtin_bit_cast(uint16_t, (_Float16)scale);
+  b_f16[(size_t)n * Kg + grp] = __builtin_bit_cast(uint16_t, (_Float16)mn);
+  uint32_t* wp = w + (size_t)n * (K / 8) + (size_t)grp * (kGroup / 8);
+#pragma unroll
+  for (int wi = 0; wi < kGroup / 8; ++wi) {
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int q = (int)roundf((v[wi * 8 + i] - mn) * inv);
+      q = q < 0 ? 0 : (q > 15 ? 15 : q);
+      packed |= (uint32_t)q << (4 * i);
+    }
+    wp[wi] = packed;
+  }
+}
+
+hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
+                           uint16_t* b_f16, int K, int N, float clip)
+{
+  const int Kg = K / kGroup;
+  // grid.y carries N; rows beyond 65535 are covered by launching in bands.
+  for (int n0 = 0; n0 < N; n0 += 65535) {
+    const int rows = (N - n0 < 65535) ? (N - n0) : 65535;
+    const hipError_t e = launch_kernel(
+        quantize_w4g64_kernel, dim3((unsigned)((Kg + 63) / 64), (unsigned)rows), dim3(64), 0, st,
+        src + (size_t)n0 * K, w + (size_t)n0 * (K / 8), s_f16 + (size_t)n0 * Kg,
+        b_f16 + (size_t)n0 * Kg, K, rows, clip);
+    if (e != hipSuccess) { return e; }
+  }
+  return hipSuccess;
+}
+
+__global__ __launch_bounds__(256) void f16_to_bf16_kernel(const uint16_t* __restrict__ in,
+                                                          uint16_t* __restrict__ out, size_t count)
+{
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count;
+       i += (size_t)gridDim.x * 256) {
+    out[i] = (uint16_t)f32_to_bf16_bits(f16_bits_to_f32(in[i]));
+  }
+}
+
+hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out, size_t count)
+{
+  size_t blocks = (count + 255) / 256;
+  if (blocks > 65536) { blocks = 65536; }
+  if (blocks == 0) { return hipSuccess; }
+  return launch_kernel(f16_to_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, in, out, count);
+}
+
+}  // namespace vpq

@@ -1,0 +1,68 @@
+// Device-side helpers shared by the gfx950 kernels: vector types, bf16
+// conversions, nibble unpacking and the wave64 reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vpq {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
+
+constexpr int kGroup = 64;    // quantization group along K
+constexpr int kWave = 64;     // CDNA wavefront
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16)
+{
+  return __uint_as_float(bits16 << 16);
+}
+
+// Upper half of a dword holding two bf16 values, widened in one AND.
+__device__ __forceinline__ float bf16_hi_to_f32(uint32_t packed)
+{
+  return __uint_as_float(packed & 0xffff0000u);
+}
+
+__device__ __forceinline__ float bf16_lo_to_f32(uint32_t packed)
+{
+  return __uint_as_float(packed << 16);
+}
+
+// fp32 -> bf16 bits, round to nearest even; NaN stays a quiet NaN.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
+{
+  const uint32_t x = __float_as_uint(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) { return (x >> 16) | 0x40u; }
+  return (x + 0x7fffu + ((x >> 16) & 1u)) >> 16;
+}
+
+// Two fp32 -> one dword of two bf16 (lo = a, hi = b) through the hardware
+// converter (v_cvt_pk_bf16_f32, round to nearest even).
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b)
+{
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+  bf16x2 v;
+  v[0] = (__bf16)a;
+  v[1] = (__bf16)b;
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// IEEE binary16 bits -> fp32 (exact).
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
+{
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+// Sum over the 64 lanes of a wavefront; every lane receives the total.
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) { v += __shfl_xor(v, off, kWave); }
+  return v;
+}
+
+}  // namespace vpq

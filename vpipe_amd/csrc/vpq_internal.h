@@ -1,0 +1,83 @@
+// Host-side launch functions behind the C ABI.  Each validates nothing: the
+// C ABI layer (vpq_api.hip) has already checked shapes, alignment and pointers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <vector>
+
+namespace vpq {
+
+// Measurement aid: while `on`, every kernel launch is bracketed by a pair of HIP
+// events handed to hipExtLaunchKernel, which stamps them at the kernel's own
+// start and end (no launch gap included).  One state per process; the
+// benchmark enables it from a single thread.
+struct ProfileState {
+  bool on = false;
+  std::vector<hipEvent_t> events;  // start0, stop0, start1, stop1, ...
+  size_t used = 0;
+};
+ProfileState& profile_state();
+
+template <typename F, typename... Args>
+inline hipError_t launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st,
+                                Args... args)
+{
+  ProfileState& ps = profile_state();
+  if (ps.on && ps.used + 2 <= ps.events.size()) {
+    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, st, ps.events[ps.used],
+                          ps.events[ps.used + 1], 0, args...);
+    ps.used += 2;
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, st, args...);
+  }
+  return hipGetLastError();
+}
+
+struct QmvArgs {
+  const uint32_t* w;
+  const uint16_t* scales;
+  const uint16_t* biases;
+  const uint16_t* x;
+  void* y;                   // bf16 [M,N] or fp32 [M,N]
+  const uint16_t* residual;  // nullable, bf16 [M,N]
+  int K, N, M;
+  bool y_f32;
+  void* ws;                  // split-K scratch (nullable)
+  size_t ws_bytes;
+  int cu_count;
+};
+
+struct GemmArgs {
+  const uint32_t* w;         // packed codes, or nullptr for a dense B
+  const uint16_t* scales;
+  const uint16_t* biases;
+  const uint16_t* b_dense;   // dense bf16 B [N,K] when w == nullptr
+  const uint16_t* x;         // [M,K]
+  uint16_t* y;               // [M,N]
+  int K, N, M;
+  const uint16_t* lora_t;    // nullable, [M,r]
+  const uint16_t* lora_b;    // nullable, [N,r]
+  int r;
+  float out_scale;           // LoRA-A epilogue: y = bf16(out_scale * bf16(acc)); unused otherwise
+  bool scaled_epilogue;
+  int cu_count;
+};
+
+hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* scales,
+                          const uint16_t* biases, uint16_t* out, int K, int N);
+hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a);
+// Returns hipErrorInvalidValue if the shape is outside what the MFMA kernel
+// handles (the caller then falls back to the simple kernel).
+bool qmv_mfma_supports(int K, int N, int M);
+hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits);
+size_t qmv_mfma_workspace_bytes(int K, int N, int M);
+hipError_t launch_gemm(hipStream_t st, const GemmArgs& a);
+hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
+                           uint16_t* b_f16, int K, int N, float clip);
+hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out, size_t count);
+
+}  // namespace vpq

@@ -1,0 +1,343 @@
+// QMV (1 <= M <= 16) as a bandwidth kernel on bf16 MFMA.
+//
+// Work decomposition.  The [N,K] pack is cut into items of 16 weight rows x KS
+// k-values (KS = 512: 8 quantization groups, 4 KB of codes).  A workgroup owns
+// one 16-row tile of N and a K range; its wavefronts take the items of that
+// range round-robin and their partial sums are added through LDS at the end
+// (split-K inside the workgroup).  With split_k > 1 several workgroups share a
+// tile through fp32 partials in a caller-provided workspace and the last one to
+// arrive folds them in a fixed order.
+//
+// Per item and wavefront:
+//   codes   16 rows x KS/2 bytes, fetched with 128-bit direct-to-LDS loads in
+//           which 16 consecutive lanes cover 256 contiguous bytes of one row
+//           (full cache lines), into a wave-private LDS buffer.  The 16-byte
+//           chunks of a row are stored XOR-swizzled so that the later 64-bit
+//           reads (lane = weight row) do not collide on LDS banks.
+//   scales, biases   one 128-bit load per lane (8 groups of the lane's row).
+//   x       each lane loads the 16-byte pieces its MFMA A operand needs
+//           straight from global/L2 (x is tiny and shared by every workgroup).
+//   math    the integer codes are turned into bf16 (128 + q) by one
+//           v_and_or_b32 per nibble pair and contracted with x on
+//           v_mfma_f32_16x16x32_bf16, two MFMAs per group.  The accumulator is
+//           seeded with -128*sum(x) so the MFMA result is exactly the group's
+//           sum(x*q); then y += scale*sum(x*q) + bias*sum(x) in fp32 -- the
+//           factored form of gpu-kernels/metal/quant/affine_qmv.metal:151-174,
+//           with sum(x) in fp32 (the reference forms it in bf16 quad sums,
+//           affine_qmv.metal:60-67, an error source not reproduced here).
+// The weight is never rounded to bf16: q, 128+q and x are exact in bf16, the
+// products are exact in fp32.
+#include "vpq_device.h"
+#include "vpq_internal.h"
+
+namespace vpq {
+
+namespace {
+
+constexpr int kTileN = 16;
+
+struct QmvParams {
+  const uint32_t* w;
+  const uint16_t* scales;
+  const uint16_t* biases;
+  const uint16_t* x;
+  void* y;
+  const uint16_t* residual;
+  float* partial;        // [split_k][M][N] fp32 (split_k > 1)
+  unsigned* counters;    // [tiles_n] arrival counters, zero between calls
+  int K, N, M;
+  int slices;            // K / KS
+  int slices_per_block;  // items of one workgroup's K range
+  int split_k;
+};
+
+// (a & mask) | magic in one VALU op.  VOP3 on gfx9 takes no literal and one
+// scalar operand, so the mask rides in an SGPR and the magic in a VGPR.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic)
+{
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(magic));
+  return d;
+}
+
+// Eight nibbles of one packed word -> eight bf16 values 128+q, element order
+// [k0,k4,k1,k5,k2,k6,k3,k7] (nibbles i and i+4 sit 16 bits apart, which is what
+// one and_or extracts into the two halves of a dword).
+__device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t word, uint32_t magic)
+{
+  u32x4 v;
+  v[0] = and_or(word, 0x000f000fu, magic);
+  v[1] = and_or(word >> 4, 0x000f000fu, magic);
+  v[2] = and_or(word >> 8, 0x000f000fu, magic);
+  v[3] = and_or(word >> 12, 0x000f000fu, magic);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// Eight consecutive bf16 of x -> the element order codes_to_bf16 produces.
+__device__ __forceinline__ bf16x8 permute_x(uint4 d)
+{
+  u32x4 v;
+  v[0] = __builtin_amdgcn_perm(d.z, d.x, 0x05040100u);  // x0,x4
+  v[1] = __builtin_amdgcn_perm(d.z, d.x, 0x07060302u);  // x1,x5
+  v[2] = __builtin_amdgcn_perm(d.w, d.y, 0x05040100u);  // x2,x6
+  v[3] = __builtin_amdgcn_perm(d.w, d.y, 0x07060302u);  // x3,x7
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+}  // namespace
+
+// KS: k-values per item (512).  MR: accumulator registers per lane = ceil(M/4).
+// Row m of x sits in MFMA row 4*(m%4) + m/4, so that output row m is register
+// m/4 of lane group m%4 and M <= 4 needs a single accumulator register.
+template <int KS, int MR, bool F32OUT>
+__global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
+{
+  constexpr int G = KS / kGroup;            // groups per item (8)
+  constexpr int ROW_BYTES = KS / 2;         // code bytes per row per item (256)
+  constexpr int CH = ROW_BYTES / 16;        // 16-byte chunks per row (16)
+  constexpr int ROWS_PER_LOAD = kWave / CH; // rows one load instruction covers (4)
+  constexpr int NLOAD = kTileN / ROWS_PER_LOAD;
+  constexpr int ITEM_BYTES = kTileN * ROW_BYTES;
+  static_assert(KS == 512, "scale/bias vector loads assume 8 groups per item");
+
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int NW = blockDim.x >> 6;
+  uint8_t* wbuf = lds + wave * ITEM_BYTES;
+  float* red = reinterpret_cast<float*>(lds + NW * ITEM_BYTES);
+
+  const int n0 = blockIdx.x * kTileN;
+  const int fr = lane & 15;                 // MFMA row (A) / column (B, D) of this lane
+  const int g = lane >> 4;                  // k sub-block of this lane
+  const int m_real = 4 * (fr & 3) + (fr >> 2);
+  // MFMA rows beyond M produce outputs nobody stores; they read the last live row.
+  const int x_row = m_real < p.M ? m_real : p.M - 1;
+  const int Kg = p.K >> 6;
+  const size_t row_bytes_total = (size_t)p.K >> 1;
+
+  // Per-lane global byte offsets of the NLOAD code loads (item-independent part).
+  size_t code_off[NLOAD];
+#pragma unroll
+  for (int i = 0; i < NLOAD; ++i) {
+    const int row = i * ROWS_PER_LOAD + lane / CH;
+    const int chunk = (lane % CH) ^ (row & (CH - 1));
+    const int grow = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
+    code_off[i] = (size_t)grow * row_bytes_total + (size_t)chunk * 16;
+  }
+  const int srow = (n0 + fr < p.N) ? (n0 + fr) : (p.N - 1);
+  // LDS byte address of this lane's two words of group 0: row fr, chunk g/2 (swizzled), half g%2.
+  const int lds_row = fr * ROW_BYTES;
+  const int lds_half = (g & 1) * 8;
+  const int lds_chunk0 = (g >> 1) ^ fr;
+
+  const uint32_t magic = 0x43004300u;       // bf16 128.0 in both halves
+  u32x4 m128;
+  m128[0] = m128[1] = m128[2] = m128[3] = 0xc300c300u;  // bf16 -128.0
+  const bf16x8 neg128 = __builtin_bit_cast(bf16x8, m128);
+
+  float acc[MR];
+#pragma unroll
+  for (int r = 0; r < MR; ++r) { acc[r] = 0.0f; }
+
+  const int sl_begin = blockIdx.y * p.slices_per_block;
+  int sl_end = sl_begin + p.slices_per_block;
+  if (sl_end > p.slices) { sl_end = p.slices; }
+
+  for (int sl = sl_begin + wave; sl < sl_end; sl += NW) {
+    // 1. codes: global -> LDS, no registers in between.
+    const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.w) + (size_t)sl * ROW_BYTES;
+#pragma unroll
+    for (int i = 0; i < NLOAD; ++i) {
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(wbase + code_off[i]),
+          (__attribute__((address_space(3))) void*)(wbuf + i * (kWave * 16)), 16, 0, 0);
+    }
+    // 2. scales and biases of this lane's row: 8 groups each.
+    const uint4 sv = *reinterpret_cast<const uint4*>(p.scales + (size_t)srow * Kg + (size_t)sl * G);
+    const uint4 bv = *reinterpret_cast<const uint4*>(p.biases + (size_t)srow * Kg + (size_t)sl * G);
+    // 3. x: this lane's A operands, two per group.
+    bf16x8 afrag[2 * G];
+    {
+      const uint16_t* xp = p.x + (size_t)x_row * p.K + (size_t)sl * KS + g * 16;
+#pragma unroll
+      for (int grp = 0; grp < G; ++grp) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          afrag[2 * grp + t] = permute_x(*reinterpret_cast<const uint4*>(xp + grp * kGroup + t * 8));
+        }
+      }
+    }
+    // 4. codes have landed in this wave's buffer.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    const uint32_t sd[4] = {sv.x, sv.y, sv.z, sv.w};
+    const uint32_t bd[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+    for (int grp = 0; grp < G; ++grp) {
+      // -128 * sum(x) of the group, in the accumulator layout (same for every column).
+      floatx4 xneg = {0.f, 0.f, 0.f, 0.f};
+      xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp], neg128, xneg, 0, 0, 0);
+      xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp + 1], neg128, xneg, 0, 0, 0);
+      const int chunk = (2 * grp) ^ lds_chunk0;      // == (2*grp + g/2) ^ fr, CH == 16
+      const uint2 cw = *reinterpret_cast<const uint2*>(wbuf + lds_row + chunk * 16 + lds_half);
+      floatx4 s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp], codes_to_bf16(cw.x, magic),
+                                                            xneg, 0, 0, 0);
+      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp + 1], codes_to_bf16(cw.y, magic),
+                                                   s4, 0, 0, 0);
+      const float s = (grp & 1) ? bf16_hi_to_f32(sd[grp >> 1]) : bf16_lo_to_f32(sd[grp >> 1]);
+      const float b = (grp & 1) ? bf16_hi_to_f32(bd[grp >> 1]) : bf16_lo_to_f32(bd[grp >> 1]);
+      const float b2 = b * -0.0078125f;              // bias * sum(x) = (bias / -128) * xneg
+#pragma unroll
+      for (int r = 0; r < MR; ++r) {
+        acc[r] = fmaf(s, s4[r], acc[r]);
+        acc[r] = fmaf(b2, xneg[r], acc[r]);
+      }
+    }
+  }
+
+  // Sum the wavefronts' partials.  acc[r] of lane l is y[m = 4r + l/16][n0 + l%16].
+#pragma unroll
+  for (int r = 0; r < MR; ++r) { red[(wave * MR + r) * kWave + lane] = acc[r]; }
+  __syncthreads();
+
+  const int t = threadIdx.x;
+  float total = 0.0f;
+  int m = 0, n = 0;
+  const bool owner = t < MR * kWave;
+  if (owner) {
+    const int r = t >> 6, l = t & 63;
+    for (int wv = 0; wv < NW; ++wv) { total += red[(wv * MR + r) * kWave + l]; }
+    m = 4 * r + (l >> 4);
+    n = n0 + (l & 15);
+  }
+  const bool valid = owner && m < p.M && n < p.N;
+
+  if (p.split_k > 1) {
+    // Publish this workgroup's partial, then let the last arrival fold all of
+    // them in index order (deterministic whatever the arrival order).
+    if (valid) { p.partial[((size_t)blockIdx.y * p.M + m) * p.N + n] = total; }
+    __threadfence();
+    __syncthreads();
+    __shared__ unsigned arrived;
+    if (t == 0) { arrived = atomicAdd(&p.counters[blockIdx.x], 1u); }
+    __syncthreads();
+    if (arrived != (unsigned)(p.split_k - 1)) { return; }
+    __threadfence();
+    if (valid) {
+      total = 0.0f;
+      for (int sk = 0; sk < p.split_k; ++sk) {
+        total += __builtin_nontemporal_load(&p.partial[((size_t)sk * p.M + m) * p.N + n]);
+      }
+    }
+    if (t == 0) { p.counters[blockIdx.x] = 0u; }
+  }
+
+  if (valid) {
+    const size_t o = (size_t)m * p.N + n;
+    if (F32OUT) {
+      reinterpret_cast<float*>(p.y)[o] = total;
+    } else {
+      uint32_t v = f32_to_bf16_bits(total);
+      if (p.residual != nullptr) {
+        v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(p.residual[o]));
+      }
+      reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)v;
+    }
+  }
+}
+
+namespace {
+
+constexpr int kKS = 512;
+constexpr int kMaxWaves = 16;
+
+// Number of K ranges (workgroups per 16-row tile) for a shape: split only when
+// the tiles alone leave most of the chip idle.
+int choose_split(int K, int N, int cu_count)
+{
+  const int tiles = (N + kTileN - 1) / kTileN;
+  const int slices = K / kKS;
+  int split = 1;
+  while (tiles * split < cu_count && split * 2 <= slices && split < 8) { split *= 2; }
+  return split;
+}
+
+size_t counters_bytes(int N)
+{
+  const size_t tiles = (size_t)(N + kTileN - 1) / kTileN;
+  return (tiles * sizeof(unsigned) + 255) / 256 * 256;
+}
+
+}  // namespace
+
+bool qmv_mfma_supports(int K, int N, int M)
+{
+  return K % kKS == 0 && N >= 1 && M >= 1 && M <= 16;
+}
+
+size_t qmv_mfma_workspace_bytes(int K, int N, int M)
+{
+  (void)K;
+  const size_t part = (size_t)8 * (size_t)M * (size_t)N * sizeof(float);
+  return counters_bytes(N) + (part + 255) / 256 * 256;
+}
+
+hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
+{
+  QmvParams p;
+  p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
+  p.residual = a.residual;
+  p.K = a.K; p.N = a.N; p.M = a.M;
+  p.slices = a.K / kKS;
+
+  int split = force_splits > 0 ? force_splits : choose_split(a.K, a.N, a.cu_count);
+  if (split > p.slices) { split = p.slices; }
+  if (split > 8) { split = 8; }
+  const size_t need = counters_bytes(a.N) + (size_t)split * a.M * a.N * sizeof(float);
+  if (split > 1 && (a.ws == nullptr || a.ws_bytes < need)) {
+    if (force_splits > 1) { return hipErrorInvalidValue; }
+    split = 1;
+  }
+  p.slices_per_block = (p.slices + split - 1) / split;
+  split = (p.slices + p.slices_per_block - 1) / p.slices_per_block;
+  p.split_k = split;
+  p.counters = reinterpret_cast<unsigned*>(a.ws);
+  p.partial = (a.ws != nullptr)
+                  ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.ws) + counters_bytes(a.N))
+                  : nullptr;
+
+  // Wavefronts per workgroup: every wavefront gets the same number of items
+  // where the slice count allows it.
+  const int per_wave = (p.slices_per_block + kMaxWaves - 1) / kMaxWaves;
+  int nw = (p.slices_per_block + per_wave - 1) / per_wave;
+  int mr = (a.M + 3) / 4;
+  if (mr == 3) { mr = 4; }
+  // The final reduction is done by mr*64 threads.
+  if (nw < mr) { nw = mr; }
+
+  const size_t lds_bytes = (size_t)nw * (kTileN * kKS / 2) + (size_t)nw * mr * kWave * sizeof(float);
+  const dim3 grid((unsigned)((a.N + kTileN - 1) / kTileN), (unsigned)split), block((unsigned)(nw * kWave));
+
+  static bool attr_done[8] = {false, false, false, false, false, false, false, false};
+  auto launch = [&](auto kern, int slot) -> hipError_t {
+    if (!attr_done[slot]) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) { return e; }
+      attr_done[slot] = true;
+    }
+    return launch_kernel(kern, grid, block, lds_bytes, st, p);
+  };
+  const int mr_t = mr;
+  if (a.y_f32) {
+    if (mr_t == 1) { return launch(qmv_mfma_kernel<kKS, 1, true>, 0); }
+    if (mr_t == 2) { return launch(qmv_mfma_kernel<kKS, 2, true>, 1); }
+    return launch(qmv_mfma_kernel<kKS, 4, true>, 2);
+  }
+  if (mr_t == 1) { return launch(qmv_mfma_kernel<kKS, 1, false>, 3); }
+  if (mr_t == 2) { return launch(qmv_mfma_kernel<kKS, 2, false>, 4); }
+  return launch(qmv_mfma_kernel<kKS, 4, false>, 5);
+}
+
+}  // namespace vpq

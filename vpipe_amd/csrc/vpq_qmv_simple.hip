@@ -1,0 +1,88 @@
+// QMV, general-shape kernel: one wavefront per output row, fp32 VALU.
+// Handles every K % 64 == 0, every N and 1 <= M <= 16; used for shapes the
+// MFMA kernel does not take (K not a multiple of 512, N not a multiple of 16)
+// and as an independent second implementation in the tests.
+//
+// Arithmetic: W[n,k] = fma(s, q, b) in fp32 (never rounded to bf16),
+// acc += x * W in fp32, wave reduction, one bf16 rounding on store -- the
+// semantics of gpu-kernels/metal/quant/affine_qmv.metal:151-174, 228-283.
+#include "vpq_device.h"
+#include "vpq_internal.h"
+
+namespace vpq {
+
+template <int MT, bool F32OUT>
+__global__ __launch_bounds__(256) void qmv_simple_kernel(
+    const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
+    const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x, void* __restrict__ y,
+    const uint16_t* __restrict__ residual, int K, int N, int M)
+{
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + wave;
+  if (n >= N) { return; }  // wave-uniform
+  const int Kw = K >> 3, Kg = K >> 6;
+  const uint32_t* wrow = w + (size_t)n * Kw;
+  const uint16_t* srow = scales + (size_t)n * Kg;
+  const uint16_t* brow = biases + (size_t)n * Kg;
+
+  for (int m0 = 0; m0 < M; m0 += MT) {
+    float acc[MT];
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) { acc[mm] = 0.0f; }
+    // Each lane takes 32 consecutive k (one 128-bit load of codes, half a group).
+    for (int k0 = lane * 32; k0 < K; k0 += kWave * 32) {
+      const uint4 c4 = *reinterpret_cast<const uint4*>(wrow + (k0 >> 3));
+      const uint32_t codes[4] = {c4.x, c4.y, c4.z, c4.w};
+      const float s = bf16_bits_to_f32(srow[k0 >> 6]);
+      const float b = bf16_bits_to_f32(brow[k0 >> 6]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float wv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { wv[j] = fmaf(s, (float)((codes[i] >> (4 * j)) & 0xfu), b); }
+#pragma unroll
+        for (int mm = 0; mm < MT; ++mm) {
+          const int row = (m0 + mm < M) ? (m0 + mm) : (M - 1);
+          const uint4 x4 = *reinterpret_cast<const uint4*>(x + (size_t)row * K + k0 + 8 * i);
+          const uint32_t xd[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            acc[mm] = fmaf(bf16_lo_to_f32(xd[j]), wv[2 * j], acc[mm]);
+            acc[mm] = fmaf(bf16_hi_to_f32(xd[j]), wv[2 * j + 1], acc[mm]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) {
+      const float total = wave_sum(acc[mm]);
+      const int row = m0 + mm;
+      if (lane == 0 && row < M) {
+        const size_t o = (size_t)row * N + n;
+        if (F32OUT) {
+          reinterpret_cast<float*>(y)[o] = total;
+        } else {
+          uint32_t v = f32_to_bf16_bits(total);
+          if (residual != nullptr) {
+            v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(residual[o]));
+          }
+          reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)v;
+        }
+      }
+    }
+  }
+}
+
+hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a)
+{
+  const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
+#define VPQ_LAUNCH(MT, F32)                                                                    \
+  launch_kernel(qmv_simple_kernel<MT, F32>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
+                a.residual, a.K, a.N, a.M)
+  if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH(1, true) : VPQ_LAUNCH(1, false); }
+  return a.y_f32 ? VPQ_LAUNCH(4, true) : VPQ_LAUNCH(4, false);
+#undef VPQ_LAUNCH
+}
+
+}  // namespace vpq
