@@ -96,9 +96,10 @@ int vpq_dequant_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_
  * (:264-266).
  * Requires K % 64 == 0, N > 0, 1 <= M <= 16.
  * `ws` is scratch for the split-K variant: vpq_qmv_workspace_bytes() bytes,
- * 256-byte aligned, ZERO-FILLED ONCE by the caller before its first use (the
- * kernels leave it zero-filled again); it may be NULL, in which case shapes
- * that would have used split-K run unsplit.
+ * 256-byte aligned, ZERO-FILLED ONCE by the caller before its first use (it
+ * starts with arrival counters, which every call returns to zero; the rest
+ * holds fp32 partials); it may be NULL, in which case shapes that would have
+ * used split-K run unsplit.
  * `variant`: 0 = automatic; other values select a specific kernel for
  * measurement (see VPQ_QMV_* below). */
 int vpq_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

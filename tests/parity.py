@@ -5,10 +5,12 @@ Tolerances (written once, used by every GPU test):
   * fp32 result before the store vs the float64 oracle:
         max |d| / max(|ref|, 1e-2 * rms(ref))  <=  2e-3
     (relative error with a floor, since zero-mean weights put outputs near 0).
-  * bf16 output vs bf16_rne(oracle): every element within one bf16 ulp (the
-    fp32 sum and the float64 sum may sit on either side of a rounding
-    boundary), and rel-L2 of the bf16 output against the float64 oracle <= 2e-3
-    plus the rounding noise of one bf16 store (2^-9 / sqrt(3) ~ 1.1e-3).
+  * bf16 output: the bound above plus one bf16 step at |ref| (one rounding, and
+    the fp32 and float64 sums may sit on either side of a rounding boundary);
+    every element that is not tiny against the rms within one bf16 ulp of
+    bf16_rne(oracle); at most 2% of elements differing from it at all; rel-L2
+    against the float64 oracle <= 2e-3 plus the noise of one bf16 store
+    (2^-9 / sqrt(3) ~ 1.1e-3).
 """
 import numpy as np
 
@@ -46,14 +48,34 @@ def check_f32(got_f32, ref64, tol=F32_TOL):
     return e
 
 
+def bf16_ulp(v):
+    """Spacing of bf16 numbers at magnitude |v| (8 significant bits)."""
+    v = np.abs(np.asarray(v, dtype=np.float64))
+    e = np.floor(np.log2(np.maximum(v, 2.0 ** -126)))
+    return 2.0 ** (e - 7)
+
+
 def check_bf16(got_bits, ref64, ref_bits=None):
+    """bf16 output = (fp32 result within the floored 2e-3 of the oracle) rounded once:
+    |got - ref| <= 2e-3 * max(|ref|, 1e-2 rms) + one bf16 step at |ref|.  Where the
+    output is not tiny against the rms this is the same as `within one bf16 ulp of
+    bf16(oracle)`; the mismatch rate and rel-L2 are bounded as well."""
+    ref64 = np.asarray(ref64, dtype=np.float64)
     if ref_bits is None:
-        ref_bits = synth.f32_to_bf16_bits(np.asarray(ref64, dtype=np.float64).astype(np.float32))
+        ref_bits = synth.f32_to_bf16_bits(ref64.astype(np.float32))
+    got = synth.bf16_bits_to_f32(got_bits).astype(np.float64)
+    rms = np.sqrt((ref64 ** 2).mean())
+    allowed = F32_TOL * np.maximum(np.abs(ref64), 1e-2 * rms) + bf16_ulp(ref64)
+    worst = (np.abs(got - ref64) / allowed).max()
+    assert worst <= 1.0, "bf16 output off by %.2f x the allowed error" % worst
     d = bf16_ulp_distance(got_bits, ref_bits)
-    assert d.max() <= 1, "bf16 output differs by %d ulp" % d.max()
-    r = rel_l2(synth.bf16_bits_to_f32(got_bits), ref64)
+    big = np.abs(ref64) >= 0.05 * rms
+    assert d[big].max(initial=0) <= 1, "bf16 output differs by %d ulp on a non-tiny element" % d[big].max()
+    mismatch = float((d != 0).mean())
+    assert mismatch <= 0.02, "bf16 output differs from bf16(oracle) on %.2f%% of elements" % (100 * mismatch)
+    r = rel_l2(got, ref64)
     assert r <= REL_L2_TOL, "rel-L2 %.3e" % r
-    return float((d != 0).mean()), r
+    return mismatch, r
 
 
 class Guarded:

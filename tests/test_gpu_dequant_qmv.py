@@ -79,7 +79,7 @@ def test_qmv_small_shapes(vpq, oracle, dev, D, K, N, M, variant):
     parity.check_f32(f.cpu().numpy(), y64)
     parity.check_bf16(D.bits(out.view), y64, yb)
     out.assert_intact()
-    assert not ws.any().item()                      # split-K scratch is left zeroed
+    assert not ws[:256].any().item()                # arrival counters are left zeroed
 
 
 @pytest.mark.parametrize("K,N,M", [(2048, 16, 1), (4096, 64, 4), (1024, 33, 16), (8192, 48, 2)])

@@ -51,25 +51,18 @@ struct QmvParams {
   int split_k;
 };
 
-// (a & mask) | magic in one VALU op.  VOP3 on gfx9 takes no literal and one
-// scalar operand, so the mask rides in an SGPR and the magic in a VGPR.
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic)
-{
-  uint32_t d;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(magic));
-  return d;
-}
-
 // Eight nibbles of one packed word -> eight bf16 values 128+q, element order
 // [k0,k4,k1,k5,k2,k6,k3,k7] (nibbles i and i+4 sit 16 bits apart, which is what
-// one and_or extracts into the two halves of a dword).
-__device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t word, uint32_t magic)
+// one (w >> 4i) & 0x000f000f extracts into the two halves of a dword).  `mask`
+// and `magic` arrive as opaque register values so that each pair costs a single
+// v_and_or_b32 (VOP3 on gfx9 encodes no literal operand).
+__device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t word, uint32_t mask, uint32_t magic)
 {
   u32x4 v;
-  v[0] = and_or(word, 0x000f000fu, magic);
-  v[1] = and_or(word >> 4, 0x000f000fu, magic);
-  v[2] = and_or(word >> 8, 0x000f000fu, magic);
-  v[3] = and_or(word >> 12, 0x000f000fu, magic);
+  v[0] = (word & mask) | magic;
+  v[1] = ((word >> 4) & mask) | magic;
+  v[2] = ((word >> 8) & mask) | magic;
+  v[3] = ((word >> 12) & mask) | magic;
   return __builtin_bit_cast(bf16x8, v);
 }
 
@@ -131,7 +124,10 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
   const int lds_half = (g & 1) * 8;
   const int lds_chunk0 = (g >> 1) ^ fr;
 
-  const uint32_t magic = 0x43004300u;       // bf16 128.0 in both halves
+  uint32_t magic = 0x43004300u;             // bf16 128.0 in both halves
+  uint32_t mask = 0x000f000fu;
+  asm volatile("" : "+v"(magic));           // no instruction: only hides the constants
+  asm volatile("" : "+s"(mask));            // from constant folding (see codes_to_bf16)
   u32x4 m128;
   m128[0] = m128[1] = m128[2] = m128[3] = 0xc300c300u;  // bf16 -128.0
   const bf16x8 neg128 = __builtin_bit_cast(bf16x8, m128);
@@ -181,9 +177,9 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
       xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp + 1], neg128, xneg, 0, 0, 0);
       const int chunk = (2 * grp) ^ lds_chunk0;      // == (2*grp + g/2) ^ fr, CH == 16
       const uint2 cw = *reinterpret_cast<const uint2*>(wbuf + lds_row + chunk * 16 + lds_half);
-      floatx4 s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp], codes_to_bf16(cw.x, magic),
+      floatx4 s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp], codes_to_bf16(cw.x, mask, magic),
                                                             xneg, 0, 0, 0);
-      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp + 1], codes_to_bf16(cw.y, magic),
+      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp + 1], codes_to_bf16(cw.y, mask, magic),
                                                    s4, 0, 0, 0);
       const float s = (grp & 1) ? bf16_hi_to_f32(sd[grp >> 1]) : bf16_lo_to_f32(sd[grp >> 1]);
       const float b = (grp & 1) ? bf16_hi_to_f32(bd[grp >> 1]) : bf16_lo_to_f32(bd[grp >> 1]);
@@ -251,6 +247,9 @@ namespace {
 
 constexpr int kKS = 512;
 constexpr int kMaxWaves = 16;
+// Largest dynamic LDS a launch asks for: 16 wave buffers + 16 x 4 reduction rows
+// (the kernel also holds a few bytes of static LDS, so not the full 160 KB).
+constexpr int kMaxLdsBytes = kMaxWaves * (kTileN * kKS / 2) + kMaxWaves * 4 * kWave * 4;
 
 // Number of K ranges (workgroups per 16-row tile) for a shape: split only when
 // the tiles alone leave most of the chip idle.
@@ -323,7 +322,7 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   auto launch = [&](auto kern, int slot) -> hipError_t {
     if (!attr_done[slot]) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
       if (e != hipSuccess) { return e; }
       attr_done[slot] = true;
     }
