@@ -82,6 +82,34 @@ def test_qmv_small_shapes(vpq, oracle, dev, D, K, N, M, variant):
     assert not ws[:256].any().item()                # arrival counters are left zeroed
 
 
+STREAM_SHAPES = [
+    # K, N, M: one and several slices per wavefront, ragged last tile, more tiles than
+    # workgroups (each workgroup walks several tiles), every M the kernel takes
+    (512, 16, 1), (1024, 33, 2), (4096, 95, 3), (4096, 16 * 800 + 5, 1), (8192, 48, 4),
+    (12288, 160, 1), (12288, 16 * 300, 2), (17408, 64, 1), (17408, 33, 2), (24576, 17, 1),
+]
+
+
+@pytest.mark.parametrize("K,N,M", STREAM_SHAPES)
+def test_qmv_streaming_kernel(vpq, oracle, dev, D, K, N, M):
+    w, s, b = synth.make_weight(N, K, 4000 + K + N)
+    x = synth.make_act(M, K, 5000 + K + M)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=capi.VPQ_QMV_STREAM, f32out=True)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, variant=capi.VPQ_QMV_STREAM)
+    torch.cuda.synchronize()
+    parity.check_f32(f.cpu().numpy(), y64)
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    out.assert_intact()
+    # same inputs through the one-item-per-wavefront kernel: same arithmetic, so the fp32
+    # results agree to accumulation-order noise
+    f2 = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=MFMA, f32out=True)
+    rms = float(np.sqrt((y64 ** 2).mean()))
+    assert (f - f2).abs().max().item() <= 1e-5 * rms + 1e-6
+
+
 @pytest.mark.parametrize("K,N,M", [(2048, 16, 1), (4096, 64, 4), (1024, 33, 16), (8192, 48, 2)])
 def test_qmv_split_k_matches_oracle_and_is_deterministic(vpq, oracle, dev, D, K, N, M):
     w, s, b = synth.make_weight(N, K, 31 + K)
@@ -110,7 +138,7 @@ def test_qmv_one_hot_reads_back_weights_exactly(vpq, oracle, dev, D):
     w, s, b = synth.make_weight(N, K, 5)
     d32 = oracle.dequant_f32(w, s, b, K, N)
     wd, sd, bd = stage(D, dev, w, s, b)
-    for variant in (SIMPLE, MFMA):
+    for variant in (SIMPLE, MFMA, capi.VPQ_QMV_STREAM):
         for k in [0, 1, 4, 7, 8, 15, 16, 63, 64, 511, 512, 777, K - 1]:
             x = np.zeros((1, K), dtype=np.float32)
             x[0, k] = 1.0

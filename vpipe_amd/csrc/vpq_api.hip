@@ -86,7 +86,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
   if (ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }
-  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_MFMA_SPLITK) { return VPQ_ERR_BAD_SHAPE; }
+  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_STREAM) { return VPQ_ERR_BAD_SHAPE; }
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
 
@@ -98,7 +98,9 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
 
   const bool mfma_ok = vpq::qmv_mfma_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
   if (variant == VPQ_QMV_SIMPLE) { return finish(vpq::launch_qmv_simple(hs, a)); }
-  if (variant == VPQ_QMV_MFMA || variant == VPQ_QMV_MFMA_SPLITK) {
+  if (variant == VPQ_QMV_STREAM) {
+    // handled below, after the shape check of the streaming kernel
+  } else if (variant == VPQ_QMV_MFMA || variant == VPQ_QMV_MFMA_SPLITK) {
     if (!mfma_ok) { return VPQ_ERR_BAD_SHAPE; }
     if (variant == VPQ_QMV_MFMA_SPLITK) {
       if (ws == nullptr) { return VPQ_ERR_WORKSPACE; }
@@ -109,7 +111,17 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
     }
     return finish(vpq::launch_qmv_mfma(hs, a, 1));
   }
-  if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a, 0)); }
+  const bool stream_ok = mfma_ok && vpq::qmv_stream_supports(K, N, M);
+  if (variant == VPQ_QMV_STREAM) {
+    if (!stream_ok) { return VPQ_ERR_BAD_SHAPE; }
+    return finish(vpq::launch_qmv_stream(hs, a));
+  }
+  // Measured on MI355X (HBM-cold weights): the streaming kernel wins once a wavefront can walk a
+  // tile's whole K and the launch is long (lm_head-sized packs); below that the
+  // one-item-per-wavefront kernel finishes sooner.
+  const double pack_bytes = (double)N * (double)K * 9.0 / 16.0;
+  if (stream_ok && pack_bytes >= 150e6) { return finish(vpq::launch_qmv_stream(hs, a)); }
+  if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a, 1)); }
   return finish(vpq::launch_qmv_simple(hs, a));
 }
 

@@ -75,6 +75,8 @@ hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a);
 bool qmv_mfma_supports(int K, int N, int M);
 hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits);
 size_t qmv_mfma_workspace_bytes(int K, int N, int M);
+bool qmv_stream_supports(int K, int N, int M);
+hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);
 hipError_t launch_gemm(hipStream_t st, const GemmArgs& a);
 hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
                            uint16_t* b_f16, int K, int N, float clip);

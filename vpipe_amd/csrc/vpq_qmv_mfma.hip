@@ -1,22 +1,24 @@
 // QMV (1 <= M <= 16) as a bandwidth kernel on bf16 MFMA.
 //
-// Work decomposition.  The [N,K] pack is cut into items of 16 weight rows x KS
-// k-values (KS = 512: 8 quantization groups, 4 KB of codes).  A workgroup owns
-// one 16-row tile of N and a K range; its wavefronts take the items of that
-// range round-robin and their partial sums are added through LDS at the end
-// (split-K inside the workgroup).  With split_k > 1 several workgroups share a
-// tile through fp32 partials in a caller-provided workspace and the last one to
+// Work decomposition.  The [N,K] pack is cut into items of 16 weight rows x 512
+// k-values (8 quantization groups, 4 KB of codes).  A workgroup owns one 16-row
+// tile of N and a K range; its wavefronts take the items of that range
+// round-robin and their partial sums are added through LDS at the end (split-K
+// inside the workgroup).  With split_k > 1 several workgroups share a tile
+// through fp32 partials in a caller-provided workspace and the last one to
 // arrive folds them in a fixed order.
 //
 // Per item and wavefront:
-//   codes   16 rows x KS/2 bytes, fetched with 128-bit direct-to-LDS loads in
+//   codes   16 rows x 256 bytes, fetched with 128-bit direct-to-LDS loads in
 //           which 16 consecutive lanes cover 256 contiguous bytes of one row
 //           (full cache lines), into a wave-private LDS buffer.  The 16-byte
 //           chunks of a row are stored XOR-swizzled so that the later 64-bit
 //           reads (lane = weight row) do not collide on LDS banks.
 //   scales, biases   one 128-bit load per lane (8 groups of the lane's row).
-//   x       each lane loads the 16-byte pieces its MFMA A operand needs
-//           straight from global/L2 (x is tiny and shared by every workgroup).
+//   x       M <= 4: the wavefront loads its 512-value slice of each row with
+//           one coalesced 128-bit load per lane, reorders it once and parks it
+//           in wave-private LDS, from where every lane reads its MFMA A
+//           operands.  M > 4: each lane loads its A operands from global/L2.
 //   math    the integer codes are turned into bf16 (128 + q) by one
 //           v_and_or_b32 per nibble pair and contracted with x on
 //           v_mfma_f32_16x16x32_bf16, two MFMAs per group.  The accumulator is
@@ -27,6 +29,11 @@
 //           affine_qmv.metal:60-67, an error source not reproduced here).
 // The weight is never rounded to bf16: q, 128+q and x are exact in bf16, the
 // products are exact in fp32.
+//
+// No inline-assembly VALU instruction may sit near the MFMAs: the compiler's
+// hazard recogniser cannot see what such a statement writes, and a register an
+// MFMA in flight still reads can be overwritten.  Everything here is plain C
+// and builtins.
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -35,6 +42,12 @@ namespace vpq {
 namespace {
 
 constexpr int kTileN = 16;
+constexpr int kKS = 512;                 // k-values per item
+constexpr int kG = kKS / kGroup;         // groups per item (8)
+constexpr int kRowBytes = kKS / 2;       // code bytes per row per item (256)
+constexpr int kItemBytes = kTileN * kRowBytes;
+constexpr int kXRowBytes = kKS * 2 + 16; // LDS stride of one staged x row (bf16) + pad
+constexpr int kMaxWaves = 16;
 
 struct QmvParams {
   const uint32_t* w;
@@ -46,9 +59,10 @@ struct QmvParams {
   float* partial;        // [split_k][M][N] fp32 (split_k > 1)
   unsigned* counters;    // [tiles_n] arrival counters, zero between calls
   int K, N, M;
-  int slices;            // K / KS
+  int slices;            // K / 512
   int slices_per_block;  // items of one workgroup's K range
   int split_k;
+  int wave_lds_bytes;    // codes buffer + staged x rows of one wavefront
 };
 
 // Eight nibbles of one packed word -> eight bf16 values 128+q, element order
@@ -67,38 +81,36 @@ __device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t word, uint32_t mask, ui
 }
 
 // Eight consecutive bf16 of x -> the element order codes_to_bf16 produces.
-__device__ __forceinline__ bf16x8 permute_x(uint4 d)
+__device__ __forceinline__ uint4 permute_x(uint4 d)
 {
-  u32x4 v;
-  v[0] = __builtin_amdgcn_perm(d.z, d.x, 0x05040100u);  // x0,x4
-  v[1] = __builtin_amdgcn_perm(d.z, d.x, 0x07060302u);  // x1,x5
-  v[2] = __builtin_amdgcn_perm(d.w, d.y, 0x05040100u);  // x2,x6
-  v[3] = __builtin_amdgcn_perm(d.w, d.y, 0x07060302u);  // x3,x7
-  return __builtin_bit_cast(bf16x8, v);
+  uint4 v;
+  v.x = __builtin_amdgcn_perm(d.z, d.x, 0x05040100u);  // x0,x4
+  v.y = __builtin_amdgcn_perm(d.z, d.x, 0x07060302u);  // x1,x5
+  v.z = __builtin_amdgcn_perm(d.w, d.y, 0x05040100u);  // x2,x6
+  v.w = __builtin_amdgcn_perm(d.w, d.y, 0x07060302u);  // x3,x7
+  return v;
 }
 
 }  // namespace
 
-// KS: k-values per item (512).  MR: accumulator registers per lane = ceil(M/4).
-// Row m of x sits in MFMA row 4*(m%4) + m/4, so that output row m is register
-// m/4 of lane group m%4 and M <= 4 needs a single accumulator register.
-template <int KS, int MR, bool F32OUT>
+// MR: accumulator registers per lane = ceil(M/4).  Row m of x sits in MFMA row
+// 4*(m%4) + m/4, so that output row m is register m/4 of lane group m%4 and
+// M <= 4 needs a single accumulator register.
+// XLDS: x is staged through wave-private LDS (M <= 4).
+template <int MR, bool XLDS, bool F32OUT>
 __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
 {
-  constexpr int G = KS / kGroup;            // groups per item (8)
-  constexpr int ROW_BYTES = KS / 2;         // code bytes per row per item (256)
-  constexpr int CH = ROW_BYTES / 16;        // 16-byte chunks per row (16)
-  constexpr int ROWS_PER_LOAD = kWave / CH; // rows one load instruction covers (4)
+  constexpr int CH = kRowBytes / 16;          // 16-byte chunks per row (16)
+  constexpr int ROWS_PER_LOAD = kWave / CH;   // rows one load instruction covers (4)
   constexpr int NLOAD = kTileN / ROWS_PER_LOAD;
-  constexpr int ITEM_BYTES = kTileN * ROW_BYTES;
-  static_assert(KS == 512, "scale/bias vector loads assume 8 groups per item");
 
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int NW = blockDim.x >> 6;
-  uint8_t* wbuf = lds + wave * ITEM_BYTES;
-  float* red = reinterpret_cast<float*>(lds + NW * ITEM_BYTES);
+  uint8_t* wbuf = lds + wave * p.wave_lds_bytes;
+  uint8_t* xbuf = wbuf + kItemBytes;
+  float* red = reinterpret_cast<float*>(lds + NW * p.wave_lds_bytes);
 
   const int n0 = blockIdx.x * kTileN;
   const int fr = lane & 15;                 // MFMA row (A) / column (B, D) of this lane
@@ -107,22 +119,26 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
   // MFMA rows beyond M produce outputs nobody stores; they read the last live row.
   const int x_row = m_real < p.M ? m_real : p.M - 1;
   const int Kg = p.K >> 6;
-  const size_t row_bytes_total = (size_t)p.K >> 1;
+  const uint32_t row_bytes_total = (uint32_t)p.K >> 1;
 
-  // Per-lane global byte offsets of the NLOAD code loads (item-independent part).
-  size_t code_off[NLOAD];
+  // Wave-uniform bases (tile origin) + 32-bit per-lane offsets.
+  const uint8_t* wtile = reinterpret_cast<const uint8_t*>(p.w) + (size_t)n0 * row_bytes_total;
+  uint32_t code_off[NLOAD];
 #pragma unroll
   for (int i = 0; i < NLOAD; ++i) {
     const int row = i * ROWS_PER_LOAD + lane / CH;
     const int chunk = (lane % CH) ^ (row & (CH - 1));
-    const int grow = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
-    code_off[i] = (size_t)grow * row_bytes_total + (size_t)chunk * 16;
+    const int rrow = (n0 + row < p.N) ? row : (p.N - 1 - n0);
+    code_off[i] = (uint32_t)rrow * row_bytes_total + (uint32_t)chunk * 16;
   }
-  const int srow = (n0 + fr < p.N) ? (n0 + fr) : (p.N - 1);
+  const int srow = (n0 + fr < p.N) ? fr : (p.N - 1 - n0);
+  const uint16_t* stile = p.scales + (size_t)n0 * Kg;
+  const uint16_t* btile = p.biases + (size_t)n0 * Kg;
+  const uint32_t sb_off = (uint32_t)srow * (uint32_t)Kg;
   // LDS byte address of this lane's two words of group 0: row fr, chunk g/2 (swizzled), half g%2.
-  const int lds_row = fr * ROW_BYTES;
-  const int lds_half = (g & 1) * 8;
+  const int lds_code0 = fr * kRowBytes + (g & 1) * 8;
   const int lds_chunk0 = (g >> 1) ^ fr;
+  const int lds_x0 = x_row * kXRowBytes + g * 32;
 
   uint32_t magic = 0x43004300u;             // bf16 128.0 in both halves
   uint32_t mask = 0x000f000fu;
@@ -142,7 +158,7 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
 
   for (int sl = sl_begin + wave; sl < sl_end; sl += NW) {
     // 1. codes: global -> LDS, no registers in between.
-    const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.w) + (size_t)sl * ROW_BYTES;
+    const uint8_t* wbase = wtile + (size_t)sl * kRowBytes;
 #pragma unroll
     for (int i = 0; i < NLOAD; ++i) {
       __builtin_amdgcn_global_load_lds(
@@ -150,17 +166,25 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
           (__attribute__((address_space(3))) void*)(wbuf + i * (kWave * 16)), 16, 0, 0);
     }
     // 2. scales and biases of this lane's row: 8 groups each.
-    const uint4 sv = *reinterpret_cast<const uint4*>(p.scales + (size_t)srow * Kg + (size_t)sl * G);
-    const uint4 bv = *reinterpret_cast<const uint4*>(p.biases + (size_t)srow * Kg + (size_t)sl * G);
-    // 3. x: this lane's A operands, two per group.
-    bf16x8 afrag[2 * G];
-    {
-      const uint16_t* xp = p.x + (size_t)x_row * p.K + (size_t)sl * KS + g * 16;
+    const uint4 sv = *reinterpret_cast<const uint4*>(stile + (size_t)sl * kG + sb_off);
+    const uint4 bv = *reinterpret_cast<const uint4*>(btile + (size_t)sl * kG + sb_off);
+    // 3. x.
+    bf16x8 afrag[XLDS ? 1 : 2 * kG];
+    if (XLDS) {
+      // Lane l takes k = 8l..8l+7 of each row: one coalesced 1 KB load per row.
+      const uint16_t* xs = p.x + (size_t)sl * kKS + lane * 8;
+      for (int m = 0; m < p.M; ++m) {
+        const uint4 d = *reinterpret_cast<const uint4*>(xs + (size_t)m * p.K);
+        *reinterpret_cast<uint4*>(xbuf + m * kXRowBytes + lane * 16) = permute_x(d);
+      }
+    } else {
+      const uint16_t* xp = p.x + (size_t)x_row * p.K + (size_t)sl * kKS + g * 16;
 #pragma unroll
-      for (int grp = 0; grp < G; ++grp) {
+      for (int grp = 0; grp < kG; ++grp) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          afrag[2 * grp + t] = permute_x(*reinterpret_cast<const uint4*>(xp + grp * kGroup + t * 8));
+          afrag[2 * grp + t] = __builtin_bit_cast(
+              bf16x8, permute_x(*reinterpret_cast<const uint4*>(xp + grp * kGroup + t * 8)));
         }
       }
     }
@@ -170,17 +194,23 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
     const uint32_t sd[4] = {sv.x, sv.y, sv.z, sv.w};
     const uint32_t bd[4] = {bv.x, bv.y, bv.z, bv.w};
 #pragma unroll
-    for (int grp = 0; grp < G; ++grp) {
+    for (int grp = 0; grp < kG; ++grp) {
+      bf16x8 a0, a1;
+      if (XLDS) {
+        a0 = *reinterpret_cast<const bf16x8*>(xbuf + lds_x0 + grp * 128);
+        a1 = *reinterpret_cast<const bf16x8*>(xbuf + lds_x0 + grp * 128 + 16);
+      } else {
+        a0 = afrag[2 * grp];
+        a1 = afrag[2 * grp + 1];
+      }
       // -128 * sum(x) of the group, in the accumulator layout (same for every column).
       floatx4 xneg = {0.f, 0.f, 0.f, 0.f};
-      xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp], neg128, xneg, 0, 0, 0);
-      xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp + 1], neg128, xneg, 0, 0, 0);
-      const int chunk = (2 * grp) ^ lds_chunk0;      // == (2*grp + g/2) ^ fr, CH == 16
-      const uint2 cw = *reinterpret_cast<const uint2*>(wbuf + lds_row + chunk * 16 + lds_half);
-      floatx4 s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp], codes_to_bf16(cw.x, mask, magic),
-                                                            xneg, 0, 0, 0);
-      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag[2 * grp + 1], codes_to_bf16(cw.y, mask, magic),
-                                                   s4, 0, 0, 0);
+      xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, neg128, xneg, 0, 0, 0);
+      xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, neg128, xneg, 0, 0, 0);
+      const int chunk = (2 * grp) ^ lds_chunk0;      // == (2*grp + g/2) ^ fr
+      const uint2 cw = *reinterpret_cast<const uint2*>(wbuf + lds_code0 + chunk * 16);
+      floatx4 s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, codes_to_bf16(cw.x, mask, magic), xneg, 0, 0, 0);
+      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, codes_to_bf16(cw.y, mask, magic), s4, 0, 0, 0);
       const float s = (grp & 1) ? bf16_hi_to_f32(sd[grp >> 1]) : bf16_lo_to_f32(sd[grp >> 1]);
       const float b = (grp & 1) ? bf16_hi_to_f32(bd[grp >> 1]) : bf16_lo_to_f32(bd[grp >> 1]);
       const float b2 = b * -0.0078125f;              // bias * sum(x) = (bias / -128) * xneg
@@ -245,11 +275,10 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
 
 namespace {
 
-constexpr int kKS = 512;
-constexpr int kMaxWaves = 16;
-// Largest dynamic LDS a launch asks for: 16 wave buffers + 16 x 4 reduction rows
-// (the kernel also holds a few bytes of static LDS, so not the full 160 KB).
-constexpr int kMaxLdsBytes = kMaxWaves * (kTileN * kKS / 2) + kMaxWaves * 4 * kWave * 4;
+// Largest dynamic LDS a launch asks for: 16 wave buffers (codes + 4 staged x
+// rows) + 16 x 4 reduction rows.  The kernel also holds a few bytes of static
+// LDS, so this stays below the 160 KB of a CU.
+constexpr int kMaxLdsBytes = kMaxWaves * (kItemBytes + 4 * kXRowBytes) + kMaxWaves * 4 * kWave * 4;
 
 // Number of K ranges (workgroups per 16-row tile) for a shape: split only when
 // the tiles alone leave most of the chip idle.
@@ -315,7 +344,9 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   // The final reduction is done by mr*64 threads.
   if (nw < mr) { nw = mr; }
 
-  const size_t lds_bytes = (size_t)nw * (kTileN * kKS / 2) + (size_t)nw * mr * kWave * sizeof(float);
+  const bool xlds = a.M <= 4;
+  p.wave_lds_bytes = kItemBytes + (xlds ? a.M * kXRowBytes : 0);
+  const size_t lds_bytes = (size_t)nw * p.wave_lds_bytes + (size_t)nw * mr * kWave * sizeof(float);
   const dim3 grid((unsigned)((a.N + kTileN - 1) / kTileN), (unsigned)split), block((unsigned)(nw * kWave));
 
   static bool attr_done[8] = {false, false, false, false, false, false, false, false};
@@ -328,15 +359,14 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
     }
     return launch_kernel(kern, grid, block, lds_bytes, st, p);
   };
-  const int mr_t = mr;
   if (a.y_f32) {
-    if (mr_t == 1) { return launch(qmv_mfma_kernel<kKS, 1, true>, 0); }
-    if (mr_t == 2) { return launch(qmv_mfma_kernel<kKS, 2, true>, 1); }
-    return launch(qmv_mfma_kernel<kKS, 4, true>, 2);
+    if (mr == 1) { return launch(qmv_mfma_kernel<1, true, true>, 0); }
+    if (mr == 2) { return launch(qmv_mfma_kernel<2, false, true>, 1); }
+    return launch(qmv_mfma_kernel<4, false, true>, 2);
   }
-  if (mr_t == 1) { return launch(qmv_mfma_kernel<kKS, 1, false>, 3); }
-  if (mr_t == 2) { return launch(qmv_mfma_kernel<kKS, 2, false>, 4); }
-  return launch(qmv_mfma_kernel<kKS, 4, false>, 5);
+  if (mr == 1) { return launch(qmv_mfma_kernel<1, true, false>, 3); }
+  if (mr == 2) { return launch(qmv_mfma_kernel<2, false, false>, 4); }
+  return launch(qmv_mfma_kernel<4, false, false>, 5);
 }
 
 }  // namespace vpq
