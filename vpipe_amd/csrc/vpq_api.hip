@@ -230,7 +230,7 @@ int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
   g.r = lora ? r : 0;
   g.out_scale = 1.0f; g.scaled_epilogue = false;
   g.cu_count = g_dev.cu_count;
-  return finish(vpq::launch_gemm(hs, g));
+  return finish(vpq::launch_qmm_tile(hs, g));
 }
 
 int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

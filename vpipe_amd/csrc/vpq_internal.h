@@ -78,6 +78,8 @@ size_t qmv_mfma_workspace_bytes(int K, int N, int M);
 bool qmv_stream_supports(int K, int N, int M);
 hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);
 hipError_t launch_gemm(hipStream_t st, const GemmArgs& a);
+// 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.
+hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a);
 hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
                            uint16_t* b_f16, int K, int N, float clip);
 hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out, size_t count);
