@@ -1,25 +1,41 @@
 // QMM main kernel: y[M,N] = x[M,K] . bf16(W)^T (+ t[M,r] . B[N,r]^T) on
 // v_mfma_f32_32x32x16_bf16 with fp32 accumulation.
 //
-// One workgroup (4 wavefronts, 2x2) owns a 256(M) x 128(N) tile of y; each
-// wavefront accumulates 128 x 64 of it in 128 registers.  Per 64-wide K step (one
-// quantization group, so one scale/bias per weight row per step):
-//   x tile [256,64] bf16   global -> LDS by 128-bit direct-to-LDS loads (no
-//                          registers, no VALU), 8 rows x 128 contiguous bytes per
-//                          load instruction;
-//   W tile [128,64]        32 codes per thread: global -> registers ->
-//                          fp32 fma(s,q,b) -> bf16 RNE -> LDS.  The value is
-//                          bf16_rne(fp32(s*q+b)), the tile arithmetic of
-//                          gpu-kernels/metal/quant/affine_qmm_steel.metal:78-96
-//                          (Compute=float) and affine_qmm_mma.metal:96-104.
+// One workgroup owns a 256(M) x 128(N) tile of y and runs 12 wavefronts in two
+// roles, both present on every SIMD, so that the matrix pipe and the vector ALU
+// work at the same time without relying on instruction scheduling inside a
+// wavefront:
+//   * 8 consumer wavefronts (4x2) only read operand fragments from LDS and issue
+//     MFMAs; each accumulates 64 x 64 of the tile in 64 registers.  Two of them
+//     share a SIMD: while one waits for its fragments the other feeds the matrix
+//     pipe;
+//   * 4 producer wavefronts bring the next tiles in.  Per 64-wide K step (one
+//     quantization group, so one scale/bias per weight row per step):
+//       x tile [256,64] bf16   global -> LDS by 128-bit direct-to-LDS loads (no
+//                              registers, no VALU), 8 rows x 128 contiguous bytes
+//                              per load instruction;
+//       W tile [128,64]        32 codes per thread: global -> registers ->
+//                              fp32 fma(s,q,b) -> bf16 RNE -> LDS.  The value is
+//                              bf16_rne(fp32(s*q+b)), the tile arithmetic of
+//                              gpu-kernels/metal/quant/affine_qmm_steel.metal:78-96
+//                              (Compute=float) and affine_qmm_mma.metal:96-104.
+// Three LDS stages: while the consumers work on step s the producers fill the
+// stage of step s+2, so a global load has two steps to land; one s_barrier per
+// step.  Keeping loads in flight across a barrier needs exact waits on the load
+// counter, which the compiler cannot provide for values carried around a loop
+// (it waits for everything).  So in the steady state the producers request
+// their codes and scales with load instructions written out by hand and wait
+// for them with explicit counts, and the x tiles and W tiles live in two
+// separate LDS arrays, so that a store of dequantized weights is not ordered
+// after the x tile still in flight.
 // LDS rows are 128 bytes (64 bf16) with the eight 16-byte chunks of a row stored
 // at position chunk ^ ((row >> 1) & 7): the 128-bit operand reads of the MFMAs
-// (lane = row) then spread over all 64 banks.  Two LDS stages: while the MFMAs
-// consume stage s, the loads of stage s+1 are in flight and its W tile is
-// dequantized into the other stage; one barrier per step.
+// (lane = row) then spread over all 64 banks.
 // With a LoRA the same accumulators take r more values of K from t[M,r] and
 // B[N,r] (dense, both through direct-to-LDS loads) before the single store
 // (gpu-kernels/metal/gemm/dense_gemm_mma.metal:297-348).
+#include <type_traits>
+
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -28,10 +44,15 @@ namespace vpq {
 namespace {
 
 constexpr int TM = 256, TN = 128, TK = 64;
-constexpr int kThreads = 256;
+constexpr int kConsumers = 8;                        // consumer wavefronts: kConsumers/2 along M, 2 along N
+constexpr int kProducers = 4;
+constexpr int kThreads = (kConsumers + kProducers) * 64;
+constexpr int kWaveM = TM / (kConsumers / 2);       // x rows per consumer wavefront
+constexpr int kIT = kWaveM / 32;                    // 32-row x fragments per consumer wavefront
+constexpr int kStages = 3;
 constexpr int kRowB = TK * 2;                       // 128 bytes per LDS row
-constexpr int kStageBytes = (TM + TN) * kRowB;      // 48 KB
-constexpr int kLds = 2 * kStageBytes;               // 96 KB
+constexpr int kXStage = TM * kRowB;                 // 32 KB
+constexpr int kWStage = TN * kRowB;                 // 16 KB
 
 struct TileParams {
   const uint32_t* w;
@@ -72,17 +93,50 @@ __device__ __forceinline__ uint4 dequant_word(uint32_t word, float s, float b)
   return o;
 }
 
+// Workgroup barrier without a memory fence: the callers wait on the counters they need.
+// The empty statements keep the compiler from moving LDS accesses across it.
+__device__ __forceinline__ void wg_barrier()
+{
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// One step's codes (32 nibbles), scale and bias of a producer thread, requested by load
+// instructions the compiler does not track: the owner waits for them with wait_codes().
+struct CodeRegs {
+  u32x4 codes;
+  uint32_t s_bits, b_bits;
+};
+
+__device__ __forceinline__ void request_codes(CodeRegs& r, const uint8_t* codes, const uint16_t* s,
+                                              const uint16_t* b)
+{
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.codes) : "v"(codes) : "memory");
+  asm volatile("global_load_ushort %0, %1, off" : "=v"(r.s_bits) : "v"(s) : "memory");
+  asm volatile("global_load_ushort %0, %1, off" : "=v"(r.b_bits) : "v"(b) : "memory");
+}
+
+// Waits until at most YOUNGER vector-memory requests issued after r's are outstanding; the
+// registers pass through the statement so that no use of them can be moved above the wait.
+template <int YOUNGER>
+__device__ __forceinline__ void wait_codes(CodeRegs& r)
+{
+  asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r.codes), "+v"(r.s_bits), "+v"(r.b_bits) : "n"(YOUNGER) : "memory");
+}
+
 }  // namespace
 
 template <bool LORA>
 __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
 {
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  __shared__ __attribute__((aligned(16))) uint8_t x_lds[kStages * kXStage];   // 96 KB
+  __shared__ __attribute__((aligned(16))) uint8_t w_lds[kStages * kWStage];   // 48 KB
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const bool producer = wave >= kConsumers;
 
   // Consecutive workgroups walk M first: they share one weight tile.
   const int tile = blockIdx.x;
@@ -91,74 +145,182 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   const int m0 = tm * TM, n0 = tn * TN;
   const int KT = p.K / TK;
 
-  // ---- x tile: 32 direct-to-LDS loads per step, 8 per wavefront.  Load i of wave w covers
-  //      tile rows (8w + i)*8 .. +8; lane l takes row l/8, LDS position l%8.
-  const uint8_t* xblk = reinterpret_cast<const uint8_t*>(p.x) + (size_t)m0 * p.K * 2;
-  uint32_t a_off[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = (wave * 8 + i) * 8 + (lane >> 3);
-    const int chunk = swz(row, lane & 7);
-    const int rg = (m0 + row < p.M) ? row : (p.M - 1 - m0);
-    a_off[i] = (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u;
-  }
-  // ---- W tile: thread t dequantizes 32 codes of row t/2 (k half t%2) per step.
-  const int qrow = tid >> 1, qhalf = tid & 1;
-  const int qrg = (n0 + qrow < p.N) ? (n0 + qrow) : (p.N - 1);
-  const uint8_t* wrow = reinterpret_cast<const uint8_t*>(p.w) + (size_t)qrg * (p.K >> 1) + qhalf * 16;
-  const uint16_t* srow = p.scales + (size_t)qrg * (p.K >> 6);
-  const uint16_t* brow = p.biases + (size_t)qrg * (p.K >> 6);
-  int b_dst[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) { b_dst[i] = TM * kRowB + qrow * kRowB + swz(qrow, qhalf * 4 + i) * 16; }
-
-  auto issue_x = [&](int step, int stage) {
-    const uint8_t* src = xblk + (size_t)step * (TK * 2);
-    uint8_t* dst = lds + stage * kStageBytes + wave * (64 * kRowB);
+  if (producer) {
+    // ======================= producers =======================
+    const int pw = wave - kConsumers;     // 0..3
+    const int pt = tid - kConsumers * 64; // 0..255
+    // x tile: 32 direct-to-LDS loads per step, 8 per wavefront.  Load i of wave pw covers tile
+    // rows (8 pw + i)*8 .. +8; lane l takes row l/8, LDS position l%8.
+    const uint8_t* xblk = reinterpret_cast<const uint8_t*>(p.x) + (size_t)m0 * p.K * 2;
+    uint32_t a_off[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + a_off[i]),
-                                       (__attribute__((address_space(3))) void*)(dst + i * (8 * kRowB)), 16, 0, 0);
+      const int row = (pw * 8 + i) * 8 + (lane >> 3);
+      const int chunk = swz(row, lane & 7);
+      const int rg = (m0 + row < p.M) ? row : (p.M - 1 - m0);
+      a_off[i] = (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u;
     }
-  };
+    // W tile: thread pt dequantizes 32 codes of row pt/2 (k half pt%2) per step.
+    const int qrow = pt >> 1, qhalf = pt & 1;
+    const int qrg = (n0 + qrow < p.N) ? (n0 + qrow) : (p.N - 1);
+    const uint8_t* wrow = reinterpret_cast<const uint8_t*>(p.w) + (size_t)qrg * (p.K >> 1) + qhalf * 16;
+    const uint16_t* srow = p.scales + (size_t)qrg * (p.K >> 6);
+    const uint16_t* brow = p.biases + (size_t)qrg * (p.K >> 6);
+    int b_dst[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { b_dst[i] = qrow * kRowB + swz(qrow, qhalf * 4 + i) * 16; }
 
-  floatx16 acc[2][4];   // [jt: 32 weight rows][it: 32 x rows]
+    auto issue_x = [&](int step, int stage) {
+      const uint8_t* src = xblk + (size_t)step * (TK * 2);
+      uint8_t* dst = x_lds + stage * kXStage + pw * (64 * kRowB);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + a_off[i]),
+                                         (__attribute__((address_space(3))) void*)(dst + i * (8 * kRowB)), 16, 0, 0);
+      }
+    };
+    auto dequant_to = [&](int stage, const CodeRegs& r) {
+      const float sc = bf16_bits_to_f32(r.s_bits), bi = bf16_bits_to_f32(r.b_bits);
+      uint8_t* nb = w_lds + stage * kWStage;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word(r.codes[i], sc, bi); }
+    };
+    auto request = [&](CodeRegs& r, int step) {
+      request_codes(r, wrow + (size_t)step * (TK / 2), srow + step, brow + step);
+    };
+
+    // Prologue: steps 0 and 1 complete in stages 0 and 1; codes of steps 2 and 3 requested.
+    CodeRegs ra, rb;                       // codes of even / odd steps
+    request(ra, 0);
+    request(rb, KT > 1 ? 1 : 0);
+    issue_x(0, 0);
+    if (KT > 1) { issue_x(1, 1); }
+    wait_codes<0>(ra);
+    wait_codes<0>(rb);
+    dequant_to(0, ra);
+    if (KT > 1) { dequant_to(1, rb); }
+    request(ra, KT > 2 ? 2 : 0);
+    request(rb, KT > 3 ? 3 : 0);
+    asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");   // all but the 6 code requests
+    wg_barrier();
+
+    // Steady state, step s fills the stage of step t = s+2.  Requests in issue order:
+    //   ..., x(t-1) [8], codes(t+1) [3], x(t) [8], codes(t+2) [3]
+    // x(t) goes out first so that it has two whole steps to land.  codes(t) were requested two
+    // steps ago: 8 + 3 + 8 = 19 younger requests may stay in flight while they are awaited.
+    // Before the barrier x(t-1), the tile of step s+1, must have landed: 14 younger requests.
+    // The first fill follows the prologue, where only codes(3) [3] and x(2) [8] are younger.
+    auto fill = [&](auto younger, int t, int stage, CodeRegs& r) {
+      issue_x(t, stage);
+      wait_codes<decltype(younger)::value>(r);
+      dequant_to(stage, r);
+      request(r, t + 2 < KT ? t + 2 : t);           // the last two requests are never used
+      asm volatile("s_waitcnt vmcnt(14) lgkmcnt(0)" ::: "memory");
+    };
+    auto next_stage = [](int stage) { return stage == kStages - 1 ? 0 : stage + 1; };
+    auto odd_fill = [&](int t, int stage) {
+      if (t < KT) {
+        fill(std::integral_constant<int, 19>(), t, stage, rb);
+      } else {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      }
+    };
+    int tstage = 2;                        // stage of step s+2
+    int s = 0;
+    if (KT > 2) {
+      fill(std::integral_constant<int, 11>(), 2, tstage, ra);
+      wg_barrier();
+      tstage = next_stage(tstage);
+      odd_fill(3, tstage);
+      wg_barrier();
+      tstage = next_stage(tstage);
+      s = 2;
+    }
+    for (; s + 2 < KT; s += 2) {
+      fill(std::integral_constant<int, 19>(), s + 2, tstage, ra);   // even step: codes in ra
+      wg_barrier();
+      tstage = next_stage(tstage);
+      odd_fill(s + 3, tstage);
+      wg_barrier();
+      tstage = next_stage(tstage);
+    }
+    for (; s < KT; ++s) {                  // the last one or two steps fill nothing
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      wg_barrier();
+    }
+
+    if (LORA) {
+      const int steps = (p.r + TK - 1) / TK;
+      for (int st = 0; st < steps; ++st) {
+        const int kleft = p.r - st * TK;                 // >= 32, a multiple of 32
+        const int chunks = kleft >= TK ? 8 : (kleft >> 3);
+        // t tile: 256 rows, as the x tile; B tile: 128 rows, 4 loads per wavefront.  Stage 0.
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int row = (pw * 8 + i) * 8 + (lane >> 3);
+          const int chunk = swz(row, lane & 7);
+          const int rg = (m0 + row < p.M) ? (m0 + row) : (p.M - 1);
+          if (chunk < chunks) {
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(p.lora_t + (size_t)rg * p.r + st * TK + chunk * 8),
+                (__attribute__((address_space(3))) void*)(x_lds + pw * (64 * kRowB) + i * (8 * kRowB)), 16, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = (pw * 4 + i) * 8 + (lane >> 3);
+          const int chunk = swz(row, lane & 7);
+          const int rg = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
+          if (chunk < chunks) {
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(p.lora_b + (size_t)rg * p.r + st * TK + chunk * 8),
+                (__attribute__((address_space(3))) void*)(w_lds + pw * (32 * kRowB) + i * (8 * kRowB)), 16, 0, 0);
+          }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wg_barrier();                                    // tiles ready
+        wg_barrier();                                    // consumers done with them
+      }
+    }
+    return;
+  }
+
+  // ======================= consumers =======================
+  const int wm = wave >> 1, wn = wave & 1;
+  floatx16 acc[2][kIT];   // [jt: 32 weight rows][it: 32 x rows]
 #pragma unroll
   for (int jt = 0; jt < 2; ++jt) {
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
+    for (int it = 0; it < kIT; ++it) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) { acc[jt][it][e] = 0.0f; }
     }
   }
-
   const int frow = lane & 31;      // row of a 32-row operand fragment
   const int fkh = lane >> 5;       // which 8 of the 16 k
-  // Operand read addresses (stage-relative) for k-step 0; k-step ks adds chunk 2*ks.
-  int w_rd[2], x_rd[4];
+  int w_rd[2], x_rd[kIT];          // stage-relative operand rows
 #pragma unroll
-  for (int jt = 0; jt < 2; ++jt) { w_rd[jt] = TM * kRowB + (wn * 64 + jt * 32 + frow) * kRowB; }
+  for (int jt = 0; jt < 2; ++jt) { w_rd[jt] = (wn * 64 + jt * 32 + frow) * kRowB; }
 #pragma unroll
-  for (int it = 0; it < 4; ++it) { x_rd[it] = (wm * 128 + it * 32 + frow) * kRowB; }
-  const int w_sw = ((wn * 64 + frow) >> 1) & 7;   // jt*32 does not change (row >> 1) & 7
-  const int x_sw = ((wm * 128 + frow) >> 1) & 7;
+  for (int it = 0; it < kIT; ++it) { x_rd[it] = (wm * kWaveM + it * 32 + frow) * kRowB; }
+  const int f_sw = (frow >> 1) & 7;   // the tile offsets are multiples of 16 rows: same swizzle for all
 
   auto mma_stage = [&](int stage, int ksteps) {
-    const uint8_t* base = lds + stage * kStageBytes;
+    const uint8_t* xb = x_lds + stage * kXStage;
+    const uint8_t* wb = w_lds + stage * kWStage;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       if (ks < ksteps) {
-        const int cw = ((2 * ks + fkh) ^ w_sw) * 16;
-        const int cx = ((2 * ks + fkh) ^ x_sw) * 16;
-        bf16x8 wf[2], xf[4];
+        const int c = ((2 * ks + fkh) ^ f_sw) * 16;
+        bf16x8 wf[2], xf[kIT];
 #pragma unroll
-        for (int jt = 0; jt < 2; ++jt) { wf[jt] = *reinterpret_cast<const bf16x8*>(base + w_rd[jt] + cw); }
+        for (int jt = 0; jt < 2; ++jt) { wf[jt] = *reinterpret_cast<const bf16x8*>(wb + w_rd[jt] + c); }
 #pragma unroll
-        for (int it = 0; it < 4; ++it) { xf[it] = *reinterpret_cast<const bf16x8*>(base + x_rd[it] + cx); }
+        for (int it = 0; it < kIT; ++it) { xf[it] = *reinterpret_cast<const bf16x8*>(xb + x_rd[it] + c); }
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt) {
 #pragma unroll
-          for (int it = 0; it < 4; ++it) {
+          for (int it = 0; it < kIT; ++it) {
             acc[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[jt], xf[it], acc[jt][it], 0, 0, 0);
           }
         }
@@ -166,83 +328,31 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     }
   };
 
-  // ---- prologue: stage 0 ----
-  uint4 codes = *reinterpret_cast<const uint4*>(wrow);
-  float sc = bf16_bits_to_f32(srow[0]), bi = bf16_bits_to_f32(brow[0]);
-  issue_x(0, 0);
-  {
-    const uint32_t cw4[4] = {codes.x, codes.y, codes.z, codes.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { *reinterpret_cast<uint4*>(lds + b_dst[i]) = dequant_word(cw4[i], sc, bi); }
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-
+  wg_barrier();                          // stages 0 and 1 are ready
+  int cstage = 0;
   for (int s = 0; s < KT; ++s) {
-    const int stage = s & 1;
-    const bool more = s + 1 < KT;
-    if (more) {
-      // codes and scales first, then the x tile: the dequant below then waits for its own
-      // loads only, with the eight direct-to-LDS loads still in flight.
-      codes = *reinterpret_cast<const uint4*>(wrow + (size_t)(s + 1) * (TK / 2));
-      sc = bf16_bits_to_f32(srow[s + 1]);
-      bi = bf16_bits_to_f32(brow[s + 1]);
-      issue_x(s + 1, stage ^ 1);
-    }
-    mma_stage(stage, 4);
-    if (more) {
-      const uint32_t cw4[4] = {codes.x, codes.y, codes.z, codes.w};
-      uint8_t* nb = lds + (stage ^ 1) * kStageBytes;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) { *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word(cw4[i], sc, bi); }
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    mma_stage(cstage, 4);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // every operand read of this stage is done
+    wg_barrier();
+    cstage = (cstage == kStages - 1) ? 0 : cstage + 1;
   }
-
   if (LORA) {
-    // r more values of K: t[M,r] against B[N,r], 64 per step, both tiles by direct-to-LDS loads.
     const int steps = (p.r + TK - 1) / TK;
     for (int st = 0; st < steps; ++st) {
-      const int kleft = p.r - st * TK;                 // >= 32, a multiple of 32
+      const int kleft = p.r - st * TK;
       const int chunks = kleft >= TK ? 8 : (kleft >> 3);
-      uint8_t* sbase = lds;                            // stage 0 is free after the last barrier
-      // t tile: 256 rows, as the x tile.
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int row = (wave * 8 + i) * 8 + (lane >> 3);
-        const int chunk = swz(row, lane & 7);
-        const int rg = (m0 + row < p.M) ? (m0 + row) : (p.M - 1);
-        if (chunk < chunks) {
-          __builtin_amdgcn_global_load_lds(
-              (const __attribute__((address_space(1))) void*)(p.lora_t + (size_t)rg * p.r + st * TK + chunk * 8),
-              (__attribute__((address_space(3))) void*)(sbase + wave * (64 * kRowB) + i * (8 * kRowB)), 16, 0, 0);
-        }
-      }
-      // B tile: 128 rows, 4 loads per wavefront.
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = (wave * 4 + i) * 8 + (lane >> 3);
-        const int chunk = swz(row, lane & 7);
-        const int rg = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
-        if (chunk < chunks) {
-          __builtin_amdgcn_global_load_lds(
-              (const __attribute__((address_space(1))) void*)(p.lora_b + (size_t)rg * p.r + st * TK + chunk * 8),
-              (__attribute__((address_space(3))) void*)(sbase + TM * kRowB + wave * (32 * kRowB) + i * (8 * kRowB)), 16, 0, 0);
-        }
-      }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
+      wg_barrier();
       mma_stage(0, chunks >> 1);
-      __syncthreads();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wg_barrier();
     }
   }
 
   // ---- store: lane holds, for x row m = lane%32 of each it, 4 consecutive n per register quad ----
   const bool vec_ok = (p.N & 3) == 0;
 #pragma unroll
-  for (int it = 0; it < 4; ++it) {
-    const int m = m0 + wm * 128 + it * 32 + frow;
+  for (int it = 0; it < kIT; ++it) {
+    const int m = m0 + wm * kWaveM + it * 32 + frow;
     if (m >= p.M) { continue; }
     uint16_t* yrow = p.y + (size_t)m * p.N;
 #pragma unroll
@@ -279,17 +389,8 @@ hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a)
   p.tiles_m = (a.M + TM - 1) / TM;
   p.tiles_n = (a.N + TN - 1) / TN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
-  static bool attr_done[2] = {false, false};
-  auto launch = [&](auto kern, int slot) -> hipError_t {
-    if (!attr_done[slot]) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-      if (e != hipSuccess) { return e; }
-      attr_done[slot] = true;
-    }
-    return launch_kernel(kern, grid, block, (size_t)kLds, st, p);
-  };
-  return a.lora_t != nullptr ? launch(qmm_tile_kernel<true>, 0) : launch(qmm_tile_kernel<false>, 1);
+  return a.lora_t != nullptr ? launch_kernel(qmm_tile_kernel<true>, grid, block, 0, st, p)
+                             : launch_kernel(qmm_tile_kernel<false>, grid, block, 0, st, p);
 }
 
 }  // namespace vpq
