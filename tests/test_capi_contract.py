@@ -60,3 +60,17 @@ def test_host_side_validation_and_sizes():
     # LoRA without its scratch
     assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, one, one, 32, 1.0, null) == -4
     assert b"NULL" in L.vpq_status_string(-1)
+
+
+def test_host_layer_and_its_test_driver_load():
+    # the C++ host layer links against the C ABI; its C test driver exports the encoder protocol
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    host = os.path.join(root, "vpipe_amd", "libvpq_host.so")
+    drv = os.path.join(root, "tests", "host", "libhost_driver.so")
+    assert os.path.exists(host) and os.path.exists(drv), "run python -m vpipe_amd.build"
+    vpipe_amd.load()
+    ctypes.CDLL(host, mode=ctypes.RTLD_GLOBAL)
+    D = ctypes.CDLL(drv)
+    for name in ("hd_open", "hd_close", "hd_set_function", "hd_set_buffer", "hd_set_constant_i32", "hd_dispatch",
+                 "hd_scope_begin", "hd_scope_end", "hd_dispatch_count", "hd_wait_ok", "hd_reason", "hd_quant_linear"):
+        assert hasattr(D, name), name

@@ -1,0 +1,273 @@
+"""GPU parity through the C++ host layer: the quantized-linear call sites are written in the
+reference's encoder protocol (library/function by name, buffers in slots 0-4, K/N[/M] as
+constants 5-7, dispatch with the reference's grid expressions, errors at the fence) -- the
+form of llama3/metal-llama-model.cc:354-366, qwen3/metal-qwen-model.cc:3981-3991 and
+minimax-h3/metal-minimax-h3-transformer.cc:1813-1828 -- and checked against the CPU oracle."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests import parity
+from vpipe_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+class Driver:
+    def __init__(self):
+        path = os.path.join(HERE, "host", "libhost_driver.so")
+        assert os.path.exists(path), "tests/host/libhost_driver.so is not built (python -m vpipe_amd.build)"
+        L = ctypes.CDLL(path)
+        L.hd_open.restype = ctypes.c_void_p
+        L.hd_close.argtypes = [ctypes.c_void_p]
+        L.hd_set_function.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_char_p]
+        L.hd_set_buffer.argtypes = [ctypes.c_void_p, ctypes.c_uint, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t]
+        L.hd_set_constant_i32.argtypes = [ctypes.c_void_p, ctypes.c_uint, ctypes.c_int]
+        L.hd_dispatch.argtypes = [ctypes.c_void_p] + [ctypes.c_uint] * 6
+        L.hd_scope_begin.argtypes = [ctypes.c_void_p]
+        L.hd_scope_end.argtypes = [ctypes.c_void_p]
+        L.hd_dispatch_count.argtypes = [ctypes.c_void_p]
+        L.hd_dispatch_count.restype = ctypes.c_long
+        L.hd_wait_ok.argtypes = [ctypes.c_void_p]
+        L.hd_reason.argtypes = [ctypes.c_void_p]
+        L.hd_reason.restype = ctypes.c_char_p
+        L.hd_quant_linear.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                      ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p,
+                                      ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_void_p]
+        self.L = L
+        self.h = L.hd_open()
+        assert self.h, "CommandStream::create failed"
+
+    def close(self):
+        self.L.hd_close(self.h)
+        self.h = None
+
+    def set_function(self, lib, fn):
+        return self.L.hd_set_function(self.h, lib.encode(), fn.encode())
+
+    def set_buffer(self, index, t, byte_offset=0):
+        if t is None:
+            self.L.hd_set_buffer(self.h, index, None, 0, 0)
+        else:
+            self.L.hd_set_buffer(self.h, index, t.data_ptr(), t.numel() * t.element_size(), byte_offset)
+
+    def set_constant(self, index, v):
+        self.L.hd_set_constant_i32(self.h, index, int(v))
+
+    def dispatch(self, grid, tg):
+        torch.cuda.synchronize()   # the tests stage their tensors on torch's stream
+        self.L.hd_dispatch(self.h, *grid, *tg)
+
+    def wait_ok(self):
+        ok = self.L.hd_wait_ok(self.h)
+        return bool(ok), self.L.hd_reason(self.h).decode()
+
+
+@pytest.fixture()
+def enc(vpq, dev):
+    torch.cuda.synchronize()
+    d = Driver()
+    yield d
+    d.close()
+
+
+def stage(D, dev, w, s, b, x):
+    return D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), D.bf16(x, dev)
+
+
+def encode_linear(enc, lib, fn, wd, sd, bd, xd, yd, K, N, M=None, grid=(32, 1, 1), tg=(32, 2, 1), x_off=0, y_off=0):
+    assert enc.set_function(lib, fn) == 1
+    enc.set_buffer(0, wd)
+    enc.set_buffer(1, sd)
+    enc.set_buffer(2, bd)
+    enc.set_buffer(3, xd, x_off)
+    enc.set_buffer(4, yd, y_off)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    if M is not None:
+        enc.set_constant(7, M)
+    enc.dispatch(grid, tg)
+
+
+def test_qmv_call_site(enc, oracle, dev, D):
+    # llama decode projection: dispatch {32, N/4, 1}, threadgroup {32, 2, 1}
+    K, N = 1024, 512
+    w, s, b = synth.make_weight(N, K, 3)
+    x = synth.make_act(1, K, 4)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    yd = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_w4g64", wd, sd, bd, xd, yd, K, N, grid=(32, N // 4, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    y64, yb = oracle.qmv(w, s, b, x, K, N, 1)
+    parity.check_bf16(D.bits(yd), y64, yb)
+
+
+def test_qmv_add_and_batch_call_sites(enc, oracle, dev, D):
+    K, N, M = 512, 256, 4
+    w, s, b = synth.make_weight(N, K, 5)
+    x = synth.make_act(M, K, 6)
+    res = synth.make_act(1, N, 7)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    # _add: slot 7 holds the residual; one x row
+    yd = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    resd = D.bf16(res, dev)
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_w4g64_add") == 1
+    for i, t in enumerate((wd, sd, bd, xd, yd)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.set_buffer(7, resd)
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    # batch: slot 7 = m_total, rows tiled on grid.z
+    yb_d = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_batch_w4g64", wd, sd, bd, xd, yb_d, K, N, M=M,
+                  grid=(32, N // 4, (M + 1) // 2))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    _, yr = oracle.qmv(w, s, b, x[:1], K, N, 1, residual=res)   # the fp64 value is the one before the add
+    assert parity.bf16_ulp_distance(D.bits(yd), yr).max() <= 1
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    parity.check_bf16(D.bits(yb_d), y64, yb)
+
+
+@pytest.mark.parametrize("lib,fn", [("affine_qmm_steel_bf16", "affine_qmm_steel_w4g64"),
+                                    ("affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm64"),
+                                    ("affine_qmm_mma_bf16", "affine_qmm_mma_w4g64")])
+def test_qmm_call_site_with_byte_offsets(enc, oracle, dev, D, lib, fn):
+    # minimax-h3 qmm_dispatch_: x and y bound with byte offsets (element offset * 2)
+    K, N, M = 256, 192, 70
+    w, s, b = synth.make_weight(N, K, 8)
+    x = synth.make_act(M, K, 9)
+    wd, sd, bd, _ = stage(D, dev, w, s, b, x)
+    xpad = torch.zeros((M + 3) * K, dtype=torch.bfloat16, device=dev)
+    xpad[3 * K:] = D.bf16(x, dev).reshape(-1)
+    ypad = torch.zeros((M + 2) * N, dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, lib, fn, wd, sd, bd, xpad, ypad, K, N, M=M, grid=(((N + 31) // 32) * 32, ((M + 63) // 64) * 2, 2),
+                  tg=(32, 2, 2), x_off=3 * K * 2, y_off=2 * N * 2)
+    ok, why = enc.wait_ok()
+    assert ok, why
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M)
+    got = D.bits(ypad)
+    assert not got[:2 * N].any(), "rows before the offset were written"
+    parity.check_bf16(got[2 * N:].reshape(M, N), y64, yb)
+
+
+def test_dequant_call_site(enc, oracle, dev, D):
+    K, N = 320, 48
+    w, s, b = synth.make_weight(N, K, 10)
+    wd, sd, bd = D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev)
+    out = torch.zeros((N, K), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_dequant_bf16", "affine_dequant_w4g64") == 1
+    for i, t in enumerate((wd, sd, bd, out)):
+        enc.set_buffer(i, t)
+    enc.set_constant(4, K)
+    enc.set_constant(5, N)
+    enc.dispatch((K // 8, N, 1), (64, 1, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert np.array_equal(D.bits(out), oracle.dequant_bf16(w, s, b, K, N))
+
+
+def test_concurrent_scope_qkv(enc, oracle, dev, D):
+    # unfused q|k|v inside a concurrent scope, then a dependent projection on the joined stream
+    K, Nq, Nkv = 1024, 1024, 256
+    ws = [synth.make_weight(n, K, 20 + i) for i, n in enumerate((Nq, Nkv, Nkv))]
+    x = synth.make_act(1, K, 30)
+    xd = D.bf16(x, dev)
+    outs = [torch.zeros((1, n), dtype=torch.bfloat16, device=dev) for n in (Nq, Nkv, Nkv)]
+    staged = [(D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev)) for (w, s, b) in ws]
+    wo, so, bo = synth.make_weight(K, Nq, 40)
+    wod, sod, bod = D.u32(wo, dev), D.bf16(so, dev), D.bf16(bo, dev)
+    yo = torch.zeros((1, K), dtype=torch.bfloat16, device=dev)
+    for rep in range(3):
+        enc.L.hd_scope_begin(enc.h)
+        for (wd, sd, bd), yd, n in zip(staged, outs, (Nq, Nkv, Nkv)):
+            encode_linear(enc, "affine_qmv_bf16", "affine_qmv_w4g64", wd, sd, bd, xd, yd, K, n, grid=(32, n // 4, 1))
+        enc.L.hd_scope_end(enc.h)
+        # depends on q: must see the finished q projection
+        encode_linear(enc, "affine_qmv_bf16", "affine_qmv_w4g64", wod, sod, bod, outs[0], yo, Nq, K, grid=(32, K // 4, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert enc.L.hd_dispatch_count(enc.h) == 12
+    for (w, s, b), yd, n in zip(ws, outs, (Nq, Nkv, Nkv)):
+        y64, yb = oracle.qmv(w, s, b, x, K, n, 1)
+        parity.check_bf16(D.bits(yd), y64, yb)
+    q_bits = D.bits(outs[0])
+    y64, yb = oracle.qmv(wo, so, bo, q_bits, Nq, K, 1)
+    parity.check_bf16(D.bits(yo), y64, yb)
+
+
+def test_errors_surface_at_the_fence(enc, dev, D):
+    K, N = 128, 64
+    w, s, b = synth.make_weight(N, K, 11)
+    x = synth.make_act(1, K, 12)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    yd = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    # an unknown function name gives an invalid function; dispatching it is an error at the fence
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_w3g64") == 0
+    enc.dispatch((32, 1, 1), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert not ok and "function" in why
+    # a missing slot (set_buffer of an empty buffer is a no-op) is reported, nothing is launched
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_w4g64") == 1
+    enc.set_buffer(0, wd)
+    enc.set_buffer(1, sd)
+    enc.set_buffer(2, None)
+    enc.set_buffer(3, xd)
+    enc.set_buffer(4, yd)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert not ok and "affine_qmv_w4g64" in why
+    assert not D.bits(yd).any()
+    # a bad shape (K not a multiple of the group) is the library's own status text
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_w4g64", wd, sd, bd, xd, yd, 100, N, grid=(32, N // 4, 1))
+    ok, why = enc.wait_ok()
+    assert not ok
+    # the stream is usable again after the error was reported
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_w4g64", wd, sd, bd, xd, yd, K, N, grid=(32, N // 4, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert D.bits(yd).any()
+
+
+@pytest.mark.parametrize("M", [1, 8, 40])
+def test_quant_linear_forward_routes_by_m(enc, oracle, dev, D, M):
+    K, N = 512, 320
+    w, s, b = synth.make_weight(N, K, 13)
+    x = synth.make_act(M, K, 14 + M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    yd = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+    enc.L.hd_quant_linear(enc.h, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), K, N, xd.data_ptr(), yd.data_ptr(), M,
+                          None, None, 0, 0.0, None)
+    ok, why = enc.wait_ok()
+    assert ok, why
+    y64, yb = (oracle.qmv if M <= 16 else oracle.qmm)(w, s, b, x, K, N, M)
+    parity.check_bf16(D.bits(yd), y64, yb)
+
+
+def test_quant_linear_forward_with_lora(enc, oracle, dev, D):
+    K, N, M, r, strength = 512, 256, 48, 32, 0.625
+    w, s, b = synth.make_weight(N, K, 15)
+    x = synth.make_act(M, K, 16)
+    A, B = synth.make_lora(N, K, r, 17, std=0.05)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    Ad, Bd = D.bf16(A, dev), D.bf16(B, dev)
+    td = torch.zeros((M, r), dtype=torch.bfloat16, device=dev)
+    yd = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+    enc.L.hd_quant_linear(enc.h, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), K, N, xd.data_ptr(), yd.data_ptr(), M,
+                          Ad.data_ptr(), Bd.data_ptr(), r, strength, td.data_ptr())
+    ok, why = enc.wait_ok()
+    assert ok, why
+    t = oracle.lora_t(x, A, M, K, r, strength)
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M, t=t, B=B, r=r)
+    parity.check_bf16(D.bits(yd), y64, yb)

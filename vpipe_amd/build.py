@@ -44,7 +44,32 @@ def build(verbose=False):
                        capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
+    build_host()
     return OUT
+
+
+HOST_OUT = os.path.join(HERE, "libvpq_host.so")
+ROOT = os.path.dirname(HERE)
+DRIVER_SRC = os.path.join(ROOT, "tests", "host", "host_driver.cc")
+DRIVER_OUT = os.path.join(ROOT, "tests", "host", "libhost_driver.so")
+
+
+def _host_cc(args):
+    r = subprocess.run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-Wall", "-shared", "-D__HIP_PLATFORM_AMD__"] + args,
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("host build failed:\n" + r.stderr)
+
+
+def build_host():
+    """The C++ host layer (no device code) and, when the tests are present, their C driver over it."""
+    inc = ["-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(HERE, "host")]
+    _host_cc(inc + [os.path.join(HERE, "host", "vpq_host.cc"), "-o", HOST_OUT, "-L" + HERE, "-lvpq",
+                    "-Wl,-rpath,$ORIGIN"])
+    if os.path.exists(DRIVER_SRC):
+        _host_cc(inc + [DRIVER_SRC, "-o", DRIVER_OUT, "-L" + HERE, "-lvpq_host", "-lvpq",
+                        "-Wl,-rpath,$ORIGIN/../../vpipe_amd"])
+    return HOST_OUT
 
 
 if __name__ == "__main__":

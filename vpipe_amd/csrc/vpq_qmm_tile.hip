@@ -1,14 +1,14 @@
 // QMM main kernel: y[M,N] = x[M,K] . bf16(W)^T (+ t[M,r] . B[N,r]^T) on
 // v_mfma_f32_32x32x16_bf16 with fp32 accumulation.
 //
-// One workgroup owns a 256(M) x 128(N) tile of y and runs 12 wavefronts in two
-// roles, both present on every SIMD, so that the matrix pipe and the vector ALU
+// One workgroup owns a 256(M) x 128(N) tile of y and runs 8 wavefronts in two
+// roles, one of each on every SIMD, so that the matrix pipe and the vector ALU
 // work at the same time without relying on instruction scheduling inside a
 // wavefront:
-//   * 8 consumer wavefronts (4x2) only read operand fragments from LDS and issue
-//     MFMAs; each accumulates 64 x 64 of the tile in 64 registers.  Two of them
-//     share a SIMD: while one waits for its fragments the other feeds the matrix
-//     pipe;
+//   * 4 consumer wavefronts (2x2) only read operand fragments from LDS and issue
+//     MFMAs; each accumulates 128 x 64 of the tile in 128 registers (0.75 KB of
+//     LDS reads per MFMA; on this part sustained MFMA throughput on real data is
+//     bounded by power, so bytes moved per MFMA matter as much as issue slots);
 //   * 4 producer wavefronts bring the next tiles in.  Per 64-wide K step (one
 //     quantization group, so one scale/bias per weight row per step):
 //       x tile [256,64] bf16   global -> LDS by 128-bit direct-to-LDS loads (no
@@ -44,7 +44,7 @@ namespace vpq {
 namespace {
 
 constexpr int TM = 256, TN = 128, TK = 64;
-constexpr int kConsumers = 8;                        // consumer wavefronts: kConsumers/2 along M, 2 along N
+constexpr int kConsumers = 4;                        // consumer wavefronts: kConsumers/2 along M, 2 along N
 constexpr int kProducers = 4;
 constexpr int kThreads = (kConsumers + kProducers) * 64;
 constexpr int kWaveM = TM / (kConsumers / 2);       // x rows per consumer wavefront

@@ -1,0 +1,442 @@
+// Implementation of the C++ host layer over the C ABI (see vpq_host.h).
+#include "vpq_host.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+#include <utility>
+
+#include "vpq.h"
+
+namespace vpipe_amd {
+
+// ---------------------------------------------------------------- DeviceBuffer
+DeviceBuffer::DeviceBuffer(DeviceBuffer&& o) noexcept : _ptr(o._ptr), _bytes(o._bytes), _owned(o._owned)
+{
+  o._ptr = nullptr; o._bytes = 0; o._owned = false;
+}
+
+DeviceBuffer& DeviceBuffer::operator=(DeviceBuffer&& o) noexcept
+{
+  if (this != &o) {
+    if (_owned && _ptr) { (void)hipFree(_ptr); }
+    _ptr = o._ptr; _bytes = o._bytes; _owned = o._owned;
+    o._ptr = nullptr; o._bytes = 0; o._owned = false;
+  }
+  return *this;
+}
+
+DeviceBuffer::~DeviceBuffer()
+{
+  if (_owned && _ptr) { (void)hipFree(_ptr); }
+}
+
+DeviceBuffer DeviceBuffer::allocate(std::size_t bytes)
+{
+  DeviceBuffer b;
+  void* p = nullptr;
+  if (bytes > 0 && hipMalloc(&p, bytes) == hipSuccess) {
+    b._ptr = p; b._bytes = bytes; b._owned = true;
+  } else {
+    (void)hipGetLastError();
+  }
+  return b;
+}
+
+DeviceBuffer DeviceBuffer::wrap(void* device_ptr, std::size_t bytes) noexcept
+{
+  DeviceBuffer b;
+  b._ptr = device_ptr; b._bytes = device_ptr ? bytes : 0; b._owned = false;
+  return b;
+}
+
+bool DeviceBuffer::upload(const void* host, std::size_t bytes, std::size_t byte_offset) const
+{
+  if (empty() || byte_offset + bytes > _bytes) { return false; }
+  return hipMemcpy(static_cast<char*>(_ptr) + byte_offset, host, bytes, hipMemcpyHostToDevice) == hipSuccess;
+}
+
+bool DeviceBuffer::download(void* host, std::size_t bytes, std::size_t byte_offset) const
+{
+  if (empty() || byte_offset + bytes > _bytes) { return false; }
+  return hipMemcpy(host, static_cast<const char*>(_ptr) + byte_offset, bytes, hipMemcpyDeviceToHost) == hipSuccess;
+}
+
+// ---------------------------------------------------------------- QuantLibrary
+namespace {
+
+struct FnEntry {
+  const char* library;
+  const char* function;
+  QuantKernel kind;
+};
+
+// Function names of the reference's bf16 metallibs that this path serves.
+const FnEntry kFunctions[] = {
+    {"affine_dequant_bf16", "affine_dequant_w4g64", QuantKernel::Dequant},
+    {"affine_qmv_bf16", "affine_qmv_w4g64", QuantKernel::Qmv},
+    {"affine_qmv_bf16", "affine_qmv_w4g64_add", QuantKernel::QmvAdd},
+    {"affine_qmv_bf16", "affine_qmv_batch_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch4_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch4_xp_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch8_xp_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch8_xp2_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64", QuantKernel::Qmm},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm64", QuantKernel::Qmm},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm128", QuantKernel::Qmm},
+    {"affine_qmm_mma_bf16", "affine_qmm_mma_w4g64", QuantKernel::Qmm},
+};
+
+}  // namespace
+
+QuantLibrary QuantLibrary::load(const std::string& name)
+{
+  QuantLibrary lib;
+  for (const FnEntry& e : kFunctions) {
+    if (name == e.library) { lib._name = name; break; }
+  }
+  return lib;
+}
+
+QuantFunction QuantLibrary::function(const std::string& fn_name) const
+{
+  QuantFunction fn;
+  for (const FnEntry& e : kFunctions) {
+    if (_name == e.library && fn_name == e.function) {
+      fn._kind = e.kind;
+      fn._name = fn_name;
+      break;
+    }
+  }
+  return fn;
+}
+
+// ---------------------------------------------------------------- CommandStream
+CommandStream::CommandStream(CommandStream&& o) noexcept { *this = std::move(o); }
+
+CommandStream& CommandStream::operator=(CommandStream&& o) noexcept
+{
+  if (this != &o) {
+    release();
+    _main = o._main; _owns_main = o._owns_main; _valid = o._valid;
+    _fork_event = o._fork_event;
+    for (int i = 0; i < kSideStreams; ++i) { _side[i] = o._side[i]; _join_event[i] = o._join_event[i]; }
+    _ws = std::move(o._ws);
+    _error = std::move(o._error);
+    o._main = nullptr; o._owns_main = false; o._valid = false; o._fork_event = nullptr;
+    for (int i = 0; i < kSideStreams; ++i) { o._side[i] = nullptr; o._join_event[i] = nullptr; }
+  }
+  return *this;
+}
+
+CommandStream::~CommandStream() { release(); }
+
+void CommandStream::release()
+{
+  if (!_valid) { return; }
+  (void)hipStreamSynchronize(static_cast<hipStream_t>(_main));
+  for (int i = 0; i < kSideStreams; ++i) {
+    if (_side[i]) { (void)hipStreamDestroy(static_cast<hipStream_t>(_side[i])); _side[i] = nullptr; }
+    if (_join_event[i]) { (void)hipEventDestroy(static_cast<hipEvent_t>(_join_event[i])); _join_event[i] = nullptr; }
+  }
+  if (_fork_event) { (void)hipEventDestroy(static_cast<hipEvent_t>(_fork_event)); _fork_event = nullptr; }
+  if (_owns_main && _main) { (void)hipStreamDestroy(static_cast<hipStream_t>(_main)); }
+  _main = nullptr;
+  _valid = false;
+}
+
+CommandStream CommandStream::create()
+{
+  CommandStream s;
+  if (vpq_init() != VPQ_OK) { return s; }
+  hipStream_t st = nullptr;
+  if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) {
+    (void)hipGetLastError();
+    return s;
+  }
+  s._main = st; s._owns_main = true; s._valid = true;
+  return s;
+}
+
+CommandStream CommandStream::adopt(void* hip_stream)
+{
+  CommandStream s;
+  if (vpq_init() != VPQ_OK) { return s; }
+  s._main = hip_stream; s._owns_main = false; s._valid = true;
+  return s;
+}
+
+bool CommandStream::ensure_side_streams()
+{
+  if (_fork_event) { return true; }
+  hipEvent_t ev = nullptr;
+  if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) { return false; }
+  _fork_event = ev;
+  for (int i = 0; i < kSideStreams; ++i) {
+    hipStream_t st = nullptr;
+    hipEvent_t je = nullptr;
+    if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&je, hipEventDisableTiming) != hipSuccess) {
+      return false;
+    }
+    _side[i] = st;
+    _join_event[i] = je;
+  }
+  return true;
+}
+
+void* CommandStream::qmv_workspace(std::size_t bytes)
+{
+  if (bytes == 0) { return nullptr; }
+  if (_ws.size() < bytes) {
+    // Work already queued may still use the old scratch: drain before replacing it.
+    (void)hipStreamSynchronize(static_cast<hipStream_t>(_main));
+    _ws = DeviceBuffer::allocate(bytes);
+    if (_ws.empty()) { return nullptr; }
+    if (hipMemset(_ws.data(), 0, bytes) != hipSuccess) { _ws = DeviceBuffer(); return nullptr; }
+  }
+  return _ws.data();
+}
+
+void CommandStream::record_error(int status, const std::string& what)
+{
+  if (_error.empty()) {
+    _error = what + ": " + vpq_status_string(status);
+    if (status == VPQ_ERR_DEVICE) { _error += std::string(" (") + vpq_last_device_error() + ")"; }
+  }
+}
+
+Fence CommandStream::commit()
+{
+  Fence f;
+  f._stream = _valid ? this : nullptr;
+  return f;
+}
+
+bool Fence::wait_ok(std::string* reason)
+{
+  if (_stream == nullptr) {
+    if (reason) { *reason = "empty fence"; }
+    return false;
+  }
+  const hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(_stream->_main));
+  if (e != hipSuccess && _stream->_error.empty()) { _stream->_error = std::string("device: ") + hipGetErrorString(e); }
+  if (!_stream->_error.empty()) {
+    if (reason) { *reason = _stream->_error; }
+    _stream->_error.clear();
+    return false;
+  }
+  return true;
+}
+
+// ---------------------------------------------------------------- ComputeEncoder
+ComputeEncoder::ComputeEncoder(ComputeEncoder&& o) noexcept { *this = std::move(o); }
+
+ComputeEncoder& ComputeEncoder::operator=(ComputeEncoder&& o) noexcept
+{
+  if (this != &o) {
+    end();
+    _stream = o._stream; _fn = o._fn; _n_dispatch = o._n_dispatch;
+    _scope_depth = o._scope_depth; _scope_next = o._scope_next; _scope_used = o._scope_used;
+    for (unsigned i = 0; i < kSlots; ++i) { _slots[i] = o._slots[i]; }
+    o._stream = nullptr;
+  }
+  return *this;
+}
+
+ComputeEncoder::~ComputeEncoder() { end(); }
+
+void ComputeEncoder::end() { _stream = nullptr; }
+
+void ComputeEncoder::set_function(const QuantFunction& fn)
+{
+  if (!valid()) { return; }
+  _fn = fn;
+  for (unsigned i = 0; i < kSlots; ++i) { _slots[i] = Slot(); }
+}
+
+void ComputeEncoder::set_buffer(unsigned index, const DeviceBuffer& buf, std::size_t byte_offset)
+{
+  if (!valid() || index >= kSlots || buf.empty()) { return; }
+  if (byte_offset > buf.size()) {
+    _stream->record_error(VPQ_ERR_BAD_SHAPE, "set_buffer offset beyond the buffer");
+    return;
+  }
+  _slots[index].ptr = static_cast<char*>(buf.data()) + byte_offset;
+  _slots[index].is_buffer = true;
+  _slots[index].is_const = false;
+}
+
+void ComputeEncoder::set_constant_bytes(unsigned index, const void* bytes, std::size_t size)
+{
+  if (!valid() || index >= kSlots || bytes == nullptr) { return; }
+  Slot& s = _slots[index];
+  s = Slot();
+  s.is_const = true;
+  if (size == 4) {
+    std::int32_t v; std::memcpy(&v, bytes, 4); s.ivalue = v;
+    std::memcpy(&s.fvalue, bytes, 4);
+  } else if (size == 8) {
+    std::int64_t v; std::memcpy(&v, bytes, 8); s.ivalue = v;
+  } else {
+    s.is_const = false;   // the kernels of this path take only int / float scalars
+  }
+}
+
+ComputeEncoder::ConcurrentScope::ConcurrentScope(ComputeEncoder* e, bool active) noexcept
+{
+  if (e == nullptr || !e->valid() || !active) { return; }
+  if (e->_scope_depth == 0) {
+    CommandStream* s = e->_stream;
+    if (!s->ensure_side_streams()) {
+      (void)hipGetLastError();
+      return;   // stays serial
+    }
+    (void)hipEventRecord(static_cast<hipEvent_t>(s->_fork_event), static_cast<hipStream_t>(s->_main));
+    e->_scope_next = 0;
+    e->_scope_used = 0;
+  }
+  ++e->_scope_depth;
+  _e = e;
+}
+
+ComputeEncoder::ConcurrentScope::~ConcurrentScope()
+{
+  if (_e == nullptr || !_e->valid()) { return; }
+  if (--_e->_scope_depth == 0) {
+    CommandStream* s = _e->_stream;
+    for (int i = 0; i < _e->_scope_used; ++i) {
+      (void)hipEventRecord(static_cast<hipEvent_t>(s->_join_event[i]), static_cast<hipStream_t>(s->_side[i]));
+      (void)hipStreamWaitEvent(static_cast<hipStream_t>(s->_main), static_cast<hipEvent_t>(s->_join_event[i]), 0);
+    }
+    _e->_scope_used = 0;
+  }
+}
+
+void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgroup*/)
+{
+  if (!valid()) { return; }
+  CommandStream* s = _stream;
+  if (!_fn.valid()) {
+    s->record_error(VPQ_ERR_NULL_POINTER, "dispatch without a function");
+    return;
+  }
+  auto buf = [&](unsigned i) -> void* { return _slots[i].is_buffer ? _slots[i].ptr : nullptr; };
+  auto has_int = [&](unsigned i) { return _slots[i].is_const; };
+  auto ival = [&](unsigned i) { return static_cast<int>(_slots[i].ivalue); };
+
+  // Inside a concurrent scope the first dispatch stays on the main stream, the following ones
+  // go to side streams that start after everything queued before the scope.
+  hipStream_t st = static_cast<hipStream_t>(s->_main);
+  const bool in_scope = _scope_depth > 0;
+  if (in_scope && _scope_next > 0) {
+    const int side = (_scope_next - 1) % CommandStream::kSideStreams;
+    st = static_cast<hipStream_t>(s->_side[side]);
+    if (side >= _scope_used) {
+      (void)hipStreamWaitEvent(st, static_cast<hipEvent_t>(s->_fork_event), 0);
+      _scope_used = side + 1;
+    }
+  }
+  if (in_scope) { ++_scope_next; }
+
+  int status = VPQ_OK;
+  const QuantKernel kind = _fn.kind();
+  if (kind == QuantKernel::Dequant) {
+    // slots 0:w 1:scales 2:biases 3:w_deq 4:K 5:N
+    if (!buf(0) || !buf(1) || !buf(2) || !buf(3) || !has_int(4) || !has_int(5)) {
+      status = VPQ_ERR_NULL_POINTER;
+    } else {
+      status = vpq_dequant_w4g64_bf16(st, static_cast<const uint32_t*>(buf(0)), static_cast<const uint16_t*>(buf(1)),
+                                      static_cast<const uint16_t*>(buf(2)), static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
+    }
+  } else {
+    // slots 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N, 7: residual | m_total | M
+    if (!buf(0) || !buf(1) || !buf(2) || !buf(3) || !buf(4) || !has_int(5) || !has_int(6)) {
+      status = VPQ_ERR_NULL_POINTER;
+    } else {
+      const uint32_t* w = static_cast<const uint32_t*>(buf(0));
+      const uint16_t* sc = static_cast<const uint16_t*>(buf(1));
+      const uint16_t* bi = static_cast<const uint16_t*>(buf(2));
+      const uint16_t* x = static_cast<const uint16_t*>(buf(3));
+      uint16_t* y = static_cast<uint16_t*>(buf(4));
+      const int K = ival(5), N = ival(6);
+      if (kind == QuantKernel::Qmm) {
+        if (!has_int(7)) {
+          status = VPQ_ERR_NULL_POINTER;
+        } else {
+          status = vpq_qmm_w4g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), nullptr, nullptr, 0, 0.f, nullptr);
+        }
+      } else {
+        int M = 1;
+        const uint16_t* residual = nullptr;
+        if (kind == QuantKernel::Qmv) {
+          M = grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1;
+        } else if (kind == QuantKernel::QmvAdd) {
+          M = grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1;
+          residual = static_cast<const uint16_t*>(buf(7));
+          if (residual == nullptr) { status = VPQ_ERR_NULL_POINTER; }
+        } else {
+          if (!has_int(7)) { status = VPQ_ERR_NULL_POINTER; }
+          M = ival(7);
+        }
+        if (status == VPQ_OK) {
+          // The split-K scratch is shared by the stream, so concurrent dispatches go without it.
+          void* ws = nullptr;
+          std::size_t ws_bytes = 0;
+          if (!in_scope && K > 0 && N > 0 && M > 0 && M <= 16) {
+            ws_bytes = vpq_qmv_workspace_bytes(K, N, M);
+            ws = s->qmv_workspace(ws_bytes);
+            if (ws == nullptr) { ws_bytes = 0; }
+          }
+          status = vpq_qmv_w4g64_bf16(st, w, sc, bi, x, y, K, N, M, residual, ws, ws_bytes, VPQ_QMV_AUTO);
+        }
+      }
+    }
+  }
+  if (status != VPQ_OK) { s->record_error(status, _fn.name()); }
+  ++_n_dispatch;
+}
+
+// ---------------------------------------------------------------- QuantLinear
+void quant_linear_forward(CommandStream& stream, const Linear& lin, const DeviceBuffer& x, std::size_t x_off,
+                          const DeviceBuffer& y, std::size_t y_off, int M, const LoraFactors* lora,
+                          const DeviceBuffer* lora_t)
+{
+  if (!stream.valid()) { return; }
+  if (lin.codes == nullptr || lin.scales == nullptr || lin.qbias == nullptr || lin.codes->empty() ||
+      lin.scales->empty() || lin.qbias->empty() || x.empty() || y.empty()) {
+    stream.record_error(VPQ_ERR_NULL_POINTER, "quant_linear_forward");
+    return;
+  }
+  const uint32_t* w = reinterpret_cast<const uint32_t*>(static_cast<const char*>(lin.codes->data()) + lin.codes_off);
+  const uint16_t* sc = reinterpret_cast<const uint16_t*>(static_cast<const char*>(lin.scales->data()) + lin.scales_off);
+  const uint16_t* bi = reinterpret_cast<const uint16_t*>(static_cast<const char*>(lin.qbias->data()) + lin.qbias_off);
+  const uint16_t* xp = reinterpret_cast<const uint16_t*>(static_cast<const char*>(x.data()) + x_off);
+  uint16_t* yp = reinterpret_cast<uint16_t*>(static_cast<char*>(y.data()) + y_off);
+  hipStream_t st = static_cast<hipStream_t>(stream.native());
+  int status;
+  const bool with_lora = lora != nullptr && lora->a != nullptr && lora->b != nullptr && lora->rank > 0 &&
+                         lora->strength != 0.f && !lora->a->empty() && !lora->b->empty();
+  if (with_lora) {
+    // An adapter always takes the GEMM route: its second factor is folded into the tile's accumulator.
+    if (lora_t == nullptr || lora_t->size() < static_cast<std::size_t>(M) * lora->rank * 2) {
+      stream.record_error(VPQ_ERR_WORKSPACE, "quant_linear_forward: lora_t scratch too small");
+      return;
+    }
+    status = vpq_qmm_w4g64_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M, static_cast<const uint16_t*>(lora->a->data()),
+                                static_cast<const uint16_t*>(lora->b->data()), lora->rank, lora->strength,
+                                static_cast<uint16_t*>(lora_t->data()));
+  } else {
+    void* ws = nullptr;
+    std::size_t ws_bytes = 0;
+    if (M <= 16 && M > 0 && lin.K > 0 && lin.N > 0) {
+      ws_bytes = vpq_qmv_workspace_bytes(lin.K, lin.N, M);
+      ws = stream.qmv_workspace(ws_bytes);
+      if (ws == nullptr) { ws_bytes = 0; }
+    }
+    status = vpq_linear_w4g64_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M, ws, ws_bytes);
+  }
+  if (status != VPQ_OK) { stream.record_error(status, "quant_linear_forward"); }
+}
+
+}  // namespace vpipe_amd
