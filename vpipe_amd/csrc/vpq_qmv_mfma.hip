@@ -47,6 +47,7 @@ constexpr int kG = kKS / kGroup;         // groups per item (8)
 constexpr int kRowBytes = kKS / 2;       // code bytes per row per item (256)
 constexpr int kItemBytes = kTileN * kRowBytes;
 constexpr int kXRowBytes = kKS * 2 + 16; // LDS stride of one staged x row (bf16) + pad
+constexpr int kXsumBytes = 4 * kG * 4;   // -128*sum(x) per staged row and group (fp32)
 constexpr int kMaxWaves = 16;
 
 struct QmvParams {
@@ -91,6 +92,20 @@ __device__ __forceinline__ uint4 permute_x(uint4 d)
   return v;
 }
 
+// Sum over each aligned run of 8 lanes (one quantization group of the staged x slice);
+// every lane of the run receives it.  Three DPP steps: lane^1, lane^2, then the mirror
+// image inside the run, which exchanges its two quads.
+__device__ __forceinline__ float sum_over_8_lanes(float v)
+{
+  int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false);       // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, t);
+  t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false);      // row_half_mirror
+  v += __builtin_bit_cast(float, t);
+  return v;
+}
+
 }  // namespace
 
 // MR: accumulator registers per lane = ceil(M/4).  Row m of x sits in MFMA row
@@ -110,6 +125,8 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
   const int NW = blockDim.x >> 6;
   uint8_t* wbuf = lds + wave * p.wave_lds_bytes;
   uint8_t* xbuf = wbuf + kItemBytes;
+  float* xsum = reinterpret_cast<float*>(xbuf + p.M * kXRowBytes);   // [M][8 groups], XLDS only
+  const int xsum_row = (lane >> 4) < p.M ? (lane >> 4) : p.M - 1;
   float* red = reinterpret_cast<float*>(lds + NW * p.wave_lds_bytes);
 
   const int n0 = blockIdx.x * kTileN;
@@ -173,9 +190,14 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
     if (XLDS) {
       // Lane l takes k = 8l..8l+7 of each row: one coalesced 1 KB load per row.
       const uint16_t* xs = p.x + (size_t)sl * kKS + lane * 8;
+      // The 8 lanes that hold one group also form -128 * sum(x) of that group on the way.
       for (int m = 0; m < p.M; ++m) {
         const uint4 d = *reinterpret_cast<const uint4*>(xs + (size_t)m * p.K);
         *reinterpret_cast<uint4*>(xbuf + m * kXRowBytes + lane * 16) = permute_x(d);
+        float s8 = (bf16_lo_to_f32(d.x) + bf16_hi_to_f32(d.x)) + (bf16_lo_to_f32(d.y) + bf16_hi_to_f32(d.y)) +
+                   (bf16_lo_to_f32(d.z) + bf16_hi_to_f32(d.z)) + (bf16_lo_to_f32(d.w) + bf16_hi_to_f32(d.w));
+        s8 = sum_over_8_lanes(s8);
+        if ((lane & 7) == 0) { xsum[m * kG + (lane >> 3)] = -128.0f * s8; }
       }
     } else {
       const uint16_t* xp = p.x + (size_t)x_row * p.K + (size_t)sl * kKS + g * 16;
@@ -193,6 +215,13 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
 
     const uint32_t sd[4] = {sv.x, sv.y, sv.z, sv.w};
     const uint32_t bd[4] = {bv.x, bv.y, bv.z, bv.w};
+    float xn[kG];                               // XLDS: -128 * sum(x) per group, row lane/16
+    if (XLDS) {
+      const floatx4 lo = *reinterpret_cast<const floatx4*>(xsum + xsum_row * kG);
+      const floatx4 hi = *reinterpret_cast<const floatx4*>(xsum + xsum_row * kG + 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { xn[i] = lo[i]; xn[4 + i] = hi[i]; }
+    }
 #pragma unroll
     for (int grp = 0; grp < kG; ++grp) {
       bf16x8 a0, a1;
@@ -203,10 +232,15 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
         a0 = afrag[2 * grp];
         a1 = afrag[2 * grp + 1];
       }
-      // -128 * sum(x) of the group, in the accumulator layout (same for every column).
+      // -128 * sum(x) of the group, in the accumulator layout (same for every column): from the
+      // staging pass when x went through LDS (only register 0 is a live row then), else by MFMA.
       floatx4 xneg = {0.f, 0.f, 0.f, 0.f};
-      xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, neg128, xneg, 0, 0, 0);
-      xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, neg128, xneg, 0, 0, 0);
+      if (XLDS) {
+        xneg[0] = xn[grp];
+      } else {
+        xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, neg128, xneg, 0, 0, 0);
+        xneg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, neg128, xneg, 0, 0, 0);
+      }
       const int chunk = (2 * grp) ^ lds_chunk0;      // == (2*grp + g/2) ^ fr
       const uint2 cw = *reinterpret_cast<const uint2*>(wbuf + lds_code0 + chunk * 16);
       floatx4 s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, codes_to_bf16(cw.x, mask, magic), xneg, 0, 0, 0);
@@ -278,7 +312,7 @@ namespace {
 // Largest dynamic LDS a launch asks for: 16 wave buffers (codes + 4 staged x
 // rows) + 16 x 4 reduction rows.  The kernel also holds a few bytes of static
 // LDS, so this stays below the 160 KB of a CU.
-constexpr int kMaxLdsBytes = kMaxWaves * (kItemBytes + 4 * kXRowBytes) + kMaxWaves * 4 * kWave * 4;
+constexpr int kMaxLdsBytes = kMaxWaves * (kItemBytes + 4 * kXRowBytes + kXsumBytes) + kMaxWaves * 4 * kWave * 4;
 
 // Number of K ranges (workgroups per 16-row tile) for a shape: split only when
 // the tiles alone leave most of the chip idle.
@@ -345,7 +379,7 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   if (nw < mr) { nw = mr; }
 
   const bool xlds = a.M <= 4;
-  p.wave_lds_bytes = kItemBytes + (xlds ? a.M * kXRowBytes : 0);
+  p.wave_lds_bytes = kItemBytes + (xlds ? a.M * kXRowBytes + kXsumBytes : 0);
   const size_t lds_bytes = (size_t)nw * p.wave_lds_bytes + (size_t)nw * mr * kWave * sizeof(float);
   const dim3 grid((unsigned)((a.N + kTileN - 1) / kTileN), (unsigned)split), block((unsigned)(nw * kWave));
 
