@@ -28,6 +28,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16
+# HBM-side bytes per QMV launch of the default workload (average over a layer's seven launches),
+# from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE per dispatch).  FETCH_SIZE reads half
+# the bytes of a 256 MiB device-to-device copy on this part, so it is scaled by 2.0; WRITE_SIZE
+# by 1.0.  109.68 MB fetched per layer, writes below the counter's resolution.
+TRAFFIC_PER_LAUNCH = 15.67e6
 
 DECODE_LAYER = [("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024), ("o", 4096, 4096),
                 ("gate", 4096, 12288), ("up", 4096, 12288), ("down", 12288, 4096)]
@@ -56,6 +61,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the QMM section")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 256 MiB device-to-device copies (a kernel of known traffic, to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--concurrent", action="store_true",
                     help="capture q|k|v and gate|up as concurrent graph branches (measured slower than one "
                          "stream on MI355X: 55.7 vs 42.5 us per layer)")
@@ -178,8 +186,9 @@ def main():
     kernel_us_per_layer = float(dur.sum(axis=1).mean())
     avg_launch_us = kernel_us_per_layer / len(DECODE_LAYER)
     achieved = layer_bytes / (kernel_us_per_layer * 1e-6) / 1e9
+    default_workload = args.variant == 0
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_PER_LAUNCH if default_workload else None,
                 "kernel": "qmv_mfma_kernel (all seven launches of a layer)", "avg_launch_us": round(avg_launch_us, 3),
                 "bytes_per_launch": layer_bytes / len(DECODE_LAYER),
                 "launches_timed": n_launch}
@@ -259,6 +268,14 @@ def main():
                                "sample": "%d passes of the same decode-layer set (one layer's weights), "
                                          "dequant to fp32 [N,K] + fp32 dot, OpenMP over N" % n_pass,
                                "ms_per_step": round(el / n_pass * 1e3, 3)}
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(generator=gen)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["copy_calibration"] = {"bytes_read": 256 << 20, "bytes_written": 256 << 20, "copies": 3}
 
     print(json.dumps(out))
 
