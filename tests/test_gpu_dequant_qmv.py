@@ -90,6 +90,32 @@ STREAM_SHAPES = [
 ]
 
 
+RING_SHAPES = STREAM_SHAPES + [
+    # every M (1, 2 and 4 accumulator registers), ragged N, several tiles per workgroup,
+    # one to five slices per wavefront
+    (512, 16, 16), (1024, 40, 5), (2048, 33, 8), (4096, 16 * 1030 + 7, 4), (5120, 16 * 600, 9), (20480, 72, 16),
+    (4096, 16 * 2100 + 3, 1), (12288, 16 * 700 + 9, 3),
+]
+
+
+@pytest.mark.parametrize("K,N,M", RING_SHAPES)
+def test_qmv_ring_kernel(vpq, oracle, dev, D, K, N, M):
+    w, s, b = synth.make_weight(N, K, 6000 + K + N)
+    x = synth.make_act(M, K, 7000 + K + M)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=capi.VPQ_QMV_RING, f32out=True)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, variant=capi.VPQ_QMV_RING)
+    torch.cuda.synchronize()
+    parity.check_f32(f.cpu().numpy(), y64)
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    out.assert_intact()
+    # bit-reproducible: a second launch gives the same bits
+    f2 = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=capi.VPQ_QMV_RING, f32out=True)
+    assert torch.equal(f, f2)
+
+
 @pytest.mark.parametrize("K,N,M", STREAM_SHAPES)
 def test_qmv_streaming_kernel(vpq, oracle, dev, D, K, N, M):
     w, s, b = synth.make_weight(N, K, 4000 + K + N)

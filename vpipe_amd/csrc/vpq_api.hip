@@ -86,7 +86,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
   if (ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }
-  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_STREAM) { return VPQ_ERR_BAD_SHAPE; }
+  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_RING) { return VPQ_ERR_BAD_SHAPE; }
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
 
@@ -98,6 +98,10 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
 
   const bool mfma_ok = vpq::qmv_mfma_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
   if (variant == VPQ_QMV_SIMPLE) { return finish(vpq::launch_qmv_simple(hs, a)); }
+  if (variant == VPQ_QMV_RING) {
+    if (!mfma_ok || !vpq::qmv_ring_supports(K, N, M)) { return VPQ_ERR_BAD_SHAPE; }
+    return finish(vpq::launch_qmv_ring(hs, a, 0, 0));
+  }
   if (variant == VPQ_QMV_STREAM) {
     // handled below, after the shape check of the streaming kernel
   } else if (variant == VPQ_QMV_MFMA || variant == VPQ_QMV_MFMA_SPLITK) {
@@ -121,6 +125,14 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   // one-item-per-wavefront kernel finishes sooner.
   const double pack_bytes = (double)N * (double)K * 9.0 / 16.0;
   if (stream_ok && pack_bytes >= 150e6) { return finish(vpq::launch_qmv_stream(hs, a)); }
+  // Several rows of x: the ring kernel keeps x in registers for all the tiles of a workgroup, so
+  // its time does not grow with M up to 8 rows (measured 8.8 vs 12.0 us at 4096->12288, M=4;
+  // 23 vs 35 us at 17408->5120, M=8).  Its workgroups have 8 wavefronts: with 2 rows it only
+  // pays where the k-slices fill them evenly; at 9..16 rows the per-item kernel is ahead again.
+  if (mfma_ok && vpq::qmv_ring_supports(K, N, M) && M >= 2 && M <= 8) {
+    const bool even = ((K / 512) % 8) == 0;
+    if (M >= 3 || even) { return finish(vpq::launch_qmv_ring(hs, a, 0, 0)); }
+  }
   if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a, 1)); }
   return finish(vpq::launch_qmv_simple(hs, a));
 }

@@ -77,6 +77,9 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits);
 size_t qmv_mfma_workspace_bytes(int K, int N, int M);
 bool qmv_stream_supports(int K, int N, int M);
 hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);
+bool qmv_ring_supports(int K, int N, int M);
+// tc_hint / nw_hint > 0 force the tiles / wavefronts per workgroup (measurement only).
+hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint);
 hipError_t launch_gemm(hipStream_t st, const GemmArgs& a);
 // 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.
 hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a);

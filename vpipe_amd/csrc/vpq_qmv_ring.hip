@@ -1,0 +1,436 @@
+// QMV (1 <= M <= 16) for K % 512 == 0: x in registers, everything else through a two-slot
+// LDS ring of direct-to-LDS loads per wavefront.
+//
+// The [N,K] pack is cut into items of 16 weight rows x 512 k (8 quantization groups, 4 KB
+// of codes).  A workgroup of NW wavefronts owns TC consecutive 16-row tiles; wavefront w
+// owns the k-slices w, w+NW, ... and walks, slice by slice, over the workgroup's tiles.
+//   x       The wavefront's slice of x (every row, 512 values) is brought in ONCE per slice
+//           and stays in 64 registers in the MFMA A-operand layout; so does -128 * sum(x) per
+//           group (two MFMAs against a constant -128 operand).  Nothing about x is repeated
+//           per item, whatever M is.
+//   items   One item is five 128-bit direct-to-LDS loads into a wave-private slot: four for
+//           the codes (16 rows x 256 bytes, chunks XOR-swizzled so that the 64-bit reads,
+//           lane = weight row, do not collide on banks) and one for the 16 rows' scales and
+//           biases (8 groups each).  Two slots per wavefront; a slot's content is copied to
+//           registers first, the slot is re-requested for the item after next, and only then
+//           the copy is contracted: two items are in flight during the arithmetic.
+//   waits   Every request in flight is a direct-to-LDS load, so the load counter retires
+//           them in issue order and `s_waitcnt vmcnt(n)` with n = requests issued after the
+//           item is exact.  This is deliberate: register loads and direct-to-LDS loads do
+//           NOT retire in order with respect to each other on this part (measured: waiting
+//           with counts that mix the two read slots before their last load had landed), so a
+//           count over a mixed queue proves nothing.  For M <= 4 the slices of x come through
+//           LDS the same way (four loads, requested a whole slice ahead); for M > 4 they are
+//           plain register loads and the queue is drained (vmcnt(0)) at each change of slice.
+//           The LDS reads of what those loads wrote are written as asm so that the compiler,
+//           which cannot see the counts, does not add its own wait for everything.
+//   math    codes -> bf16 (128 + q) by one v_and_or_b32 per nibble pair, contracted with x
+//           on v_mfma_f32_16x16x32_bf16 seeded with -128*sum(x): the result is the group's
+//           sum(x*q) exactly; then y += scale*sum(x*q) + bias*sum(x) in fp32 -- the factored
+//           form of gpu-kernels/metal/quant/affine_qmv.metal:151-174.  The weight is never
+//           rounded to bf16.
+//   sums    per item the 16 x M partial results of a wavefront go to its own row of an LDS
+//           table (added to what an earlier slice left there); after the last item one
+//           barrier, and the first TC*MR*64 threads add the rows in wavefront order and
+//           store y.  The order is fixed, so results are bit-reproducible.
+//
+// No inline-assembly VALU instruction may sit near the MFMAs (the compiler's hazard
+// recogniser cannot see what such a statement writes); the asm here is loads and waits only.
+#include <type_traits>
+
+#include "vpq_device.h"
+#include "vpq_internal.h"
+
+namespace vpq {
+
+namespace {
+
+constexpr int kTileN = 16;
+constexpr int kKS = 512;                 // k-values per item
+constexpr int kG = kKS / kGroup;         // groups per item (8)
+constexpr int kRowBytes = kKS / 2;       // code bytes per row per item (256)
+constexpr int kCodeBytes = kTileN * kRowBytes;   // 4096
+constexpr int kSlotBytes = kCodeBytes + 1024;    // + one 64-lane load of scales | biases (twice)
+constexpr int kItemLoads = 5;            // direct-to-LDS loads per item
+constexpr int kXLoads = 4;               // direct-to-LDS loads per slice of x (M <= 4)
+constexpr int kXBytes = kXLoads * 1024;  // staged rows of one slice of x
+constexpr int kMaxTcMr = 4;              // TC * MR <= 4 bounds the LDS table of partial sums
+
+struct RingParams {
+  const uint32_t* w;
+  const uint16_t* scales;
+  const uint16_t* biases;
+  const uint16_t* x;
+  void* y;
+  const uint16_t* residual;
+  int K, N, M;
+  int slices;   // K / 512
+  int tiles;    // ceil(N / 16)
+  int tc;       // tiles per workgroup
+};
+
+// Eight nibbles of one packed word -> eight bf16 values 128+q, element order
+// [k0,k4,k1,k5,k2,k6,k3,k7].  `mask` and `magic` arrive as opaque register values so that
+// each pair costs a single v_and_or_b32.
+__device__ __forceinline__ bf16x8 ring_codes_to_bf16(uint32_t word, uint32_t mask, uint32_t magic)
+{
+  u32x4 v;
+  v[0] = (word & mask) | magic;
+  v[1] = ((word >> 4) & mask) | magic;
+  v[2] = ((word >> 8) & mask) | magic;
+  v[3] = ((word >> 12) & mask) | magic;
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// Eight consecutive bf16 of x -> the element order ring_codes_to_bf16 produces.
+__device__ __forceinline__ u32x4 ring_permute_x(u32x4 d)
+{
+  u32x4 v;
+  v[0] = __builtin_amdgcn_perm(d[2], d[0], 0x05040100u);  // x0,x4
+  v[1] = __builtin_amdgcn_perm(d[2], d[0], 0x07060302u);  // x1,x5
+  v[2] = __builtin_amdgcn_perm(d[3], d[1], 0x05040100u);  // x2,x6
+  v[3] = __builtin_amdgcn_perm(d[3], d[1], 0x07060302u);  // x3,x7
+  return v;
+}
+
+__device__ __forceinline__ uint32_t lds_address(const void* p)
+{
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+
+// LDS reads the compiler does not order against the direct-to-LDS loads in flight (it would
+// wait for all of them); the caller has waited for the loads that filled the address.
+__device__ __forceinline__ u32x2 lds_read_b64(uint32_t addr)
+{
+  u32x2 v;
+  asm volatile("ds_read_b64 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr)
+{
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+
+__device__ __forceinline__ void load_to_lds(const void* src, void* lds_dst)
+{
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_loads()
+{
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// An item taken out of its slot: the lane's codes (8 groups x 2 words), scales and biases.
+struct Taken {
+  u32x2 cws[kG];
+  u32x4 s, b;
+};
+
+}  // namespace
+
+// MR: accumulator registers per lane = ceil(M/4).  Row m of x sits in MFMA row 4*(m%4) + m/4,
+// so that output row m is register m/4 of lane group m%4.  MR == 1 (M <= 4) stages x through LDS.
+template <int NW, int MR, bool F32OUT>
+__global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(const RingParams p)
+{
+  constexpr bool XDMA = (MR == 1);
+  __shared__ __attribute__((aligned(16))) uint8_t ring0[NW * kSlotBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t ring1[NW * kSlotBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t xstage[XDMA ? NW * kXBytes : 16];
+  __shared__ float sums[kMaxTcMr * NW * kWave];      // [tile][wave][register][lane]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int fr = lane & 15;                 // MFMA row (A) / column (B, D) of this lane
+  const int g = lane >> 4;                  // k sub-block of this lane
+  const int m_real = 4 * (fr & 3) + (fr >> 2);
+  // MFMA rows beyond M produce outputs nobody stores; they read the last live row.
+  const int x_row = m_real < p.M ? m_real : p.M - 1;
+  const int Kg = p.K >> 6;
+  const uint32_t row_bytes = (uint32_t)p.K >> 1;
+  const int tile0 = blockIdx.x * p.tc;
+  const int TC = p.tc;
+
+  uint8_t* slot0 = ring0 + wave * kSlotBytes;
+  uint8_t* slot1 = ring1 + wave * kSlotBytes;
+  uint8_t* xbuf = xstage + (XDMA ? wave * kXBytes : 0);
+  // Code words of the lane, relative to a slot: row fr, chunk (2*grp + g/2) ^ fr, half g%2.
+  const uint32_t code_rel = (uint32_t)(fr * kRowBytes + (g & 1) * 8);
+  const int lds_chunk0 = (g >> 1) ^ fr;
+  // Load j of an item covers rows 4j..4j+3: lane l takes row 4j + l/16, LDS position l%16.
+  const int ld_row = lane >> 4;
+  const int ld_pos = lane & 15;
+
+  uint32_t magic = 0x43004300u;             // bf16 128.0 in both halves
+  uint32_t mask = 0x000f000fu;
+  asm volatile("" : "+v"(magic));           // no instruction: only hides the constants
+  asm volatile("" : "+s"(mask));            // from constant folding
+  u32x4 m128;
+  m128[0] = m128[1] = m128[2] = m128[3] = 0xc300c300u;  // bf16 -128.0
+  const bf16x8 neg128 = __builtin_bit_cast(bf16x8, m128);
+
+  // This wavefront's items: slices wave, wave+NW, ... (rounds) x the workgroup's tiles.
+  const int rounds = (p.slices - wave + NW - 1) / NW;     // <= 0 for an idle wavefront
+  const int n_items = rounds > 0 ? rounds * TC : 0;
+
+  // Requests item i into a slot (i is clamped to the last item, so that the loop can request
+  // without a condition; a tile beyond the last one re-reads the last tile and its results
+  // are dropped at the store).
+  auto request = [&](int i, uint8_t* slot) {
+    const int ii = i < n_items ? i : n_items - 1;
+    const int r = ii / TC;
+    const int t = ii - r * TC;
+    const int sl = wave + r * NW;
+    int tile = tile0 + t;
+    if (tile >= p.tiles) { tile = p.tiles - 1; }
+    const int n0 = tile * kTileN;
+    const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.w) + (size_t)n0 * row_bytes + (size_t)sl * kRowBytes;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = 4 * j + ld_row;
+      const int rrow = (n0 + row < p.N) ? row : (p.N - 1 - n0);
+      const uint32_t off = (uint32_t)rrow * row_bytes + (uint32_t)((ld_pos ^ row) & 15) * 16u;
+      load_to_lds(wbase + off, slot + j * (kWave * 16));
+    }
+    // Lanes 0-15: the 8 scales of rows 0-15; lanes 16-31: their biases; lanes 32-63 repeat.
+    const int srow = (n0 + fr < p.N) ? (n0 + fr) : (p.N - 1);
+    const uint16_t* sb = ((lane & 16) ? p.biases : p.scales) + (size_t)srow * Kg + (size_t)sl * kG;
+    load_to_lds(sb, slot + kCodeBytes);
+  };
+
+  // Waits until only the loads issued after the slot's item can be in flight and copies the
+  // lane's part of the item out of the slot.
+  auto take = [&](const uint8_t* slot, bool x_behind, Taken& it) {
+    if (XDMA && x_behind) {
+      wait_loads<kItemLoads + kXLoads>();
+    } else {
+      wait_loads<kItemLoads>();
+    }
+    const uint32_t base = lds_address(slot);
+#pragma unroll
+    for (int grp = 0; grp < kG; ++grp) {
+      it.cws[grp] = lds_read_b64(base + code_rel + (uint32_t)(((2 * grp) ^ lds_chunk0) * 16));
+    }
+    it.s = lds_read_b128(base + kCodeBytes + (uint32_t)fr * 16);
+    it.b = lds_read_b128(base + kCodeBytes + 256 + (uint32_t)fr * 16);
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(it.cws[0]), "+v"(it.cws[1]), "+v"(it.cws[2]), "+v"(it.cws[3]), "+v"(it.cws[4]), "+v"(it.cws[5]),
+                   "+v"(it.cws[6]), "+v"(it.cws[7]), "+v"(it.s), "+v"(it.b)
+                 :
+                 : "memory");
+  };
+
+  u32x4 xq[2 * kG];         // the slice of x as A operands
+  float xneg[kG][MR];       // -128 * sum(x) per group, accumulator layout
+
+  // M <= 4: requests slice r of x, rows 0..3 (rows beyond M repeat the last one), 1 KB each.
+  auto request_x = [&](int r) {
+    const int sl = wave + r * NW;
+#pragma unroll
+    for (int m = 0; m < kXLoads; ++m) {
+      const int mm = m < p.M ? m : p.M - 1;
+      load_to_lds(p.x + (size_t)mm * p.K + (size_t)sl * kKS + lane * 8, xbuf + m * 1024);
+    }
+  };
+  // Brings slice r of x into xq and forms xneg.  `younger`: loads issued after the slice's
+  // request that may stay in flight (M <= 4); for M > 4 the queue is drained.
+  auto fetch_x = [&](int r, auto younger) {
+    if (XDMA) {
+      wait_loads<decltype(younger)::value>();
+      // fragment (grp, t) of lane (fr, g): k = grp*64 + g*16 + t*8 of row x_row
+      const uint32_t xa = lds_address(xbuf) + (uint32_t)(x_row * 1024 + g * 32);
+#pragma unroll
+      for (int grp = 0; grp < kG; ++grp) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { xq[2 * grp + t] = lds_read_b128(xa + (uint32_t)(grp * 128 + t * 16)); }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(xq[0]), "+v"(xq[1]), "+v"(xq[2]), "+v"(xq[3]), "+v"(xq[4]), "+v"(xq[5]), "+v"(xq[6]),
+                     "+v"(xq[7]), "+v"(xq[8]), "+v"(xq[9]), "+v"(xq[10]), "+v"(xq[11]), "+v"(xq[12]), "+v"(xq[13]),
+                     "+v"(xq[14]), "+v"(xq[15])
+                   :
+                   : "memory");
+    } else {
+      const int sl = wave + r * NW;
+      const uint16_t* xp = p.x + (size_t)x_row * p.K + (size_t)sl * kKS + g * 16;
+#pragma unroll
+      for (int grp = 0; grp < kG; ++grp) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xq[2 * grp + t]) : "v"(xp + grp * kGroup + t * 8) : "memory");
+        }
+      }
+      asm volatile("s_waitcnt vmcnt(0)"
+                   : "+v"(xq[0]), "+v"(xq[1]), "+v"(xq[2]), "+v"(xq[3]), "+v"(xq[4]), "+v"(xq[5]), "+v"(xq[6]),
+                     "+v"(xq[7]), "+v"(xq[8]), "+v"(xq[9]), "+v"(xq[10]), "+v"(xq[11]), "+v"(xq[12]), "+v"(xq[13]),
+                     "+v"(xq[14]), "+v"(xq[15])
+                   :
+                   : "memory");
+    }
+#pragma unroll
+    for (int i = 0; i < 2 * kG; ++i) { xq[i] = ring_permute_x(xq[i]); }
+#pragma unroll
+    for (int grp = 0; grp < kG; ++grp) {
+      floatx4 xn = {0.f, 0.f, 0.f, 0.f};
+      xn = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xq[2 * grp]), neg128, xn, 0, 0, 0);
+      xn = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xq[2 * grp + 1]), neg128, xn, 0, 0, 0);
+#pragma unroll
+      for (int q = 0; q < MR; ++q) { xneg[grp][q] = xn[q]; }
+    }
+  };
+
+  // Contracts a taken item i and adds its partial sums to this wavefront's row of `sums`.
+  auto compute = [&](int i, const Taken& it) {
+    const int r = i / TC;
+    const int t = i - r * TC;
+    const uint32_t sd[4] = {it.s[0], it.s[1], it.s[2], it.s[3]};
+    const uint32_t bd[4] = {it.b[0], it.b[1], it.b[2], it.b[3]};
+    float acc[MR];
+#pragma unroll
+    for (int q = 0; q < MR; ++q) { acc[q] = 0.0f; }
+#pragma unroll
+    for (int grp = 0; grp < kG; ++grp) {
+      const u32x2 cw = it.cws[grp];
+      floatx4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int q = 0; q < MR; ++q) { s4[q] = xneg[grp][q]; }
+      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xq[2 * grp]),
+                                                    ring_codes_to_bf16(cw[0], mask, magic), s4, 0, 0, 0);
+      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xq[2 * grp + 1]),
+                                                    ring_codes_to_bf16(cw[1], mask, magic), s4, 0, 0, 0);
+      const float s = (grp & 1) ? bf16_hi_to_f32(sd[grp >> 1]) : bf16_lo_to_f32(sd[grp >> 1]);
+      const float b = (grp & 1) ? bf16_hi_to_f32(bd[grp >> 1]) : bf16_lo_to_f32(bd[grp >> 1]);
+      const float b2 = b * -0.0078125f;              // bias * sum(x) = (bias / -128) * xneg
+#pragma unroll
+      for (int q = 0; q < MR; ++q) {
+        acc[q] = fmaf(s, s4[q], acc[q]);
+        acc[q] = fmaf(b2, xneg[grp][q], acc[q]);
+      }
+    }
+    float* mine = sums + ((t * NW + wave) * MR) * kWave + lane;
+#pragma unroll
+    for (int q = 0; q < MR; ++q) {
+      if (r == 0) {
+        mine[q * kWave] = acc[q];
+      } else {
+        mine[q * kWave] += acc[q];
+      }
+    }
+  };
+
+  if (n_items > 0) {
+    int r = 0;                          // slice (round) of the item being computed
+    int left = TC;                      // items left in it
+    int x_behind = 0;                   // takes whose item still has a request of x behind it
+    bool fresh = false;                 // the next compute starts a new slice
+    if (XDMA) { request_x(0); }
+    request(0, slot0);
+    request(1, slot1);
+    fetch_x(0, std::integral_constant<int, 2 * kItemLoads>());
+    if (XDMA && rounds > 1) { request_x(1); x_behind = 2; }
+    Taken it;
+    // One item: take it out of its slot, re-request the slot for the item after next, bring
+    // in the next slice of x if the item starts one (and request the slice after that, a
+    // whole slice ahead), contract.
+    auto step = [&](int i, uint8_t* slot) {
+      take(slot, x_behind > 0, it);
+      if (x_behind > 0) { --x_behind; }
+      request(i + 2, slot);
+      if (fresh) {
+        fetch_x(r, std::integral_constant<int, kItemLoads>());
+        fresh = false;
+        if (XDMA && r + 1 < rounds) { request_x(r + 1); x_behind = 2; }
+      }
+      compute(i, it);
+      if (--left == 0) { ++r; left = TC; fresh = true; }
+    };
+    for (int i = 0; i < n_items; i += 2) {
+      step(i, slot0);
+      if (i + 1 < n_items) { step(i + 1, slot1); }
+    }
+    // The requests past the end are still writing this wavefront's slots.
+    wait_loads<0>();
+  }
+  __syncthreads();
+
+  // Thread t of the first TC*MR*64 adds, in wavefront order, the partial sums of one
+  // (tile, register, lane) and stores y[m = 4*register + lane/16][tile*16 + lane%16].
+  const int tid = threadIdx.x;
+  if (tid < TC * MR * kWave) {
+    const int t = tid / (MR * kWave);
+    const int q = (tid / kWave) % MR;
+    const int l = tid & 63;
+    const int live = p.slices < NW ? p.slices : NW;
+    float total = 0.0f;
+    for (int wv = 0; wv < live; ++wv) { total += sums[((t * NW + wv) * MR + q) * kWave + l]; }
+    const int m = 4 * q + (l >> 4);
+    const int tile = tile0 + t;
+    const int n = tile * kTileN + (l & 15);
+    if (tile < p.tiles && m < p.M && n < p.N) {
+      const size_t o = (size_t)m * p.N + n;
+      if (F32OUT) {
+        reinterpret_cast<float*>(p.y)[o] = total;
+      } else {
+        uint32_t v = f32_to_bf16_bits(total);
+        if (p.residual != nullptr) {
+          v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(p.residual[o]));
+        }
+        reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)v;
+      }
+    }
+  }
+}
+
+bool qmv_ring_supports(int K, int N, int M)
+{
+  return K % kKS == 0 && N >= 1 && M >= 1 && M <= 16;
+}
+
+namespace {
+
+template <int NW>
+hipError_t launch_nw(hipStream_t st, const RingParams& p, int mr, bool f32)
+{
+  const dim3 grid((unsigned)((p.tiles + p.tc - 1) / p.tc)), block((unsigned)(NW * kWave));
+  if (f32) {
+    if (mr == 1) { return launch_kernel(qmv_ring_kernel<NW, 1, true>, grid, block, 0, st, p); }
+    if (mr == 2) { return launch_kernel(qmv_ring_kernel<NW, 2, true>, grid, block, 0, st, p); }
+    return launch_kernel(qmv_ring_kernel<NW, 4, true>, grid, block, 0, st, p);
+  }
+  if (mr == 1) { return launch_kernel(qmv_ring_kernel<NW, 1, false>, grid, block, 0, st, p); }
+  if (mr == 2) { return launch_kernel(qmv_ring_kernel<NW, 2, false>, grid, block, 0, st, p); }
+  return launch_kernel(qmv_ring_kernel<NW, 4, false>, grid, block, 0, st, p);
+}
+
+}  // namespace
+
+// tc_hint > 0 forces the tiles per workgroup (measurement).
+hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint)
+{
+  (void)nw_hint;
+  RingParams p;
+  p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
+  p.residual = a.residual;
+  p.K = a.K; p.N = a.N; p.M = a.M;
+  p.slices = a.K / kKS;
+  p.tiles = (a.N + kTileN - 1) / kTileN;
+  int mr = (a.M + 3) / 4;
+  if (mr == 3) { mr = 4; }
+  const int tc_max = kMaxTcMr / mr;
+  // Enough tiles per workgroup that one workgroup per CU covers the matrix in one pass.
+  const int cus = a.cu_count > 0 ? a.cu_count : 256;
+  int tc = (p.tiles + cus - 1) / cus;
+  if (tc_hint > 0) { tc = tc_hint; }
+  if (tc > tc_max) { tc = tc_max; }
+  if (tc < 1) { tc = 1; }
+  p.tc = tc;
+  return launch_nw<8>(st, p, mr, a.y_f32);
+}
+
+}  // namespace vpq
