@@ -7,6 +7,9 @@ down 12288->4096), in GB/s of ALGORITHMIC bytes (packed codes + scales + biases
 + x + y, each once).  A step is one pass over the seven projections of one
 layer; consecutive steps use different layers' weights (8 layers, 868 MB in
 rotation) so that no pass finds its weights in the 256 MB last-level cache.
+By default q|k|v go out as one grouped launch and so do gate|up (the reference's
+fused-QKV dispatch: same seven results, four launches); `--launch separate`
+times seven launches, and the other mode's time is reported beside `value`.
 The timed region is one HIP graph of `steps` passes, replayed between two
 events on the launch stream with inputs already resident in HBM.
 
@@ -28,11 +31,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16
-# HBM-side bytes per QMV launch of the default workload (average over a layer's seven launches),
+# HBM-side bytes per decode layer of the default workload (all its QMV launches together),
 # from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE per dispatch).  FETCH_SIZE reads half
 # the bytes of a 256 MiB device-to-device copy on this part, so it is scaled by 2.0; WRITE_SIZE
 # by 1.0.  109.68 MB fetched per layer, writes below the counter's resolution.
-TRAFFIC_PER_LAUNCH = 15.67e6
+TRAFFIC_PER_LAYER = 109.68e6
 
 DECODE_LAYER = [("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024), ("o", 4096, 4096),
                 ("gate", 4096, 12288), ("up", 4096, 12288), ("down", 12288, 4096)]
@@ -64,9 +67,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device-to-device copies (a kernel of known traffic, to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
-    ap.add_argument("--concurrent", action="store_true",
-                    help="capture q|k|v and gate|up as concurrent graph branches (measured slower than one "
-                         "stream on MI355X: 55.7 vs 42.5 us per layer)")
+    ap.add_argument("--launch", choices=["grouped", "separate", "concurrent"], default="grouped",
+                    help="how a layer's seven projections are launched (default: q|k|v and gate|up grouped)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
@@ -102,16 +104,31 @@ def main():
         w, s, b = layers[li][j]
         vpipe_amd.qmv_w4g64(w, s, b, xs[K], K, N, 1, out=ys[j], ws=wss[j], variant=args.variant)
 
-    def layer_pass(li):
+    def group(li, js):
+        K = DECODE_LAYER[js[0]][1]
+        packs = [layers[li][j] + (DECODE_LAYER[j][2],) for j in js]
+        vpipe_amd.qmv_group_w4g64(packs, xs[K], K, 1, outs=[ys[j] for j in js])
+
+    def pass_separate(li):
+        """Seven launches, one per projection."""
         for j in range(len(DECODE_LAYER)):
             project(li, j)
 
+    def pass_grouped(li):
+        """Four launches: q|k|v read the same x and go out as ONE grouped launch, so do gate|up
+        (the reference's fused-QKV dispatch, gpu-kernels/metal/quant/affine_qmv.metal:405-516);
+        o and down are single launches.  Same seven results, bit for bit."""
+        group(li, (0, 1, 2))
+        project(li, 3)
+        group(li, (4, 5))
+        project(li, 6)
+
     side = [torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)]
 
-    def layer_pass_concurrent(li):
-        """The layer's dataflow: q|k|v are independent of each other, so are gate|up (the reference
-        encodes them in a concurrent scope, apple-silicon/metal-compute/compute-encoder.h,
-        ConcurrentScope); o follows the attention, down follows gate|up."""
+    def pass_concurrent(li):
+        """Seven launches with q|k|v and gate|up as concurrent graph branches (the reference's
+        ConcurrentScope, apple-silicon/metal-compute/compute-encoder.h).  Measured slower than one
+        stream on MI355X (55.7 vs 42.5 us per layer); kept for reproduction."""
         main = torch.cuda.current_stream()
         side[0].wait_stream(main)
         side[1].wait_stream(main)
@@ -130,68 +147,84 @@ def main():
         main.wait_stream(side[0])
         project(li, 6)
 
+    def time_steps(layer_pass, steps, use_graph):
+        """ms per step of `steps` passes: one HIP graph replayed between two events (or eager)."""
+        graph = None
+        if use_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for i in range(steps):
+                    layer_pass(i % args.layers)
+            graph.replay()                      # untimed: first replay uploads the graph
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(steps):
+                layer_pass(i % args.layers)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    def kernel_durations(layer_pass, launches_per_pass):
+        """Per-kernel durations (hipExtLaunchKernel events: kernel start -> end), us [pass, launch]."""
+        passes = max(4 * args.layers, 32)
+        n_launch = passes * launches_per_pass
+        st = L.vpq_profile_enable(n_launch)
+        if st != 0:
+            raise vpipe_amd.VpqError(st, "vpq_profile_enable")
+        for i in range(passes):
+            layer_pass(i % args.layers)
+        buf = (ctypes.c_float * n_launch)()
+        got = L.vpq_profile_read(buf, n_launch)
+        L.vpq_profile_enable(0)
+        assert got == n_launch, got
+        return np.array(buf[:], dtype=np.float64).reshape(passes, launches_per_pass) * 1e3
+
+    modes = {"grouped": (pass_grouped, 4, "q|k|v and gate|up as grouped launches (4 launches per layer)"),
+             "separate": (pass_separate, 7, "one launch per projection (7 launches per layer)"),
+             "concurrent": (pass_concurrent, 7, "7 launches, q|k|v and gate|up as concurrent graph branches")}
+    if args.variant != 0 and args.launch == "grouped":
+        args.launch = "separate"                # a forced kernel variant only exists per projection
+    layer_pass, launches_per_layer, launch_text = modes[args.launch]
+    use_graph = not args.no_graph
+
     for i in range(args.warmup):
+        pass_separate(i % args.layers)
         layer_pass(i % args.layers)
     torch.cuda.synchronize()
 
     # ---- timed region ---------------------------------------------------------------
-    concurrent = args.concurrent and not args.no_graph
-    launch = "hipgraph, q|k|v and gate|up as concurrent branches" if concurrent else "hipgraph, one stream"
-    graph = None
-    if not args.no_graph:
-        try:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                for i in range(args.steps):
-                    (layer_pass_concurrent if concurrent else layer_pass)(i % args.layers)
-            graph.replay()                      # untimed: first replay uploads the graph
-            torch.cuda.synchronize()
-        except Exception as e:                  # capture unsupported: fall back to eager, say so
-            print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
-            graph = None
-    if graph is None:
-        launch = "eager"
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    e0.record()
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(args.steps):
-            layer_pass(i % args.layers)
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1)
-    ms_per_step = ms / args.steps
+    ms_per_step = time_steps(layer_pass, args.steps, use_graph)
     value = layer_bytes / (ms_per_step * 1e-3) / 1e9
+    launch = ("hipgraph, " if use_graph else "eager, ") + launch_text
+    other = "separate" if args.launch != "separate" else "grouped"
+    ms_other = time_steps(modes[other][0], args.steps, use_graph) if args.variant == 0 else None
 
-    # ---- per-kernel durations (hipExtLaunchKernel events: kernel start -> end) --------
-    passes = max(4 * args.layers, 32)
-    n_launch = passes * len(DECODE_LAYER)
-    st = L.vpq_profile_enable(n_launch)
-    if st != 0:
-        raise vpipe_amd.VpqError(st, "vpq_profile_enable")
-    for i in range(passes):
-        layer_pass(i % args.layers)
-    buf = (ctypes.c_float * n_launch)()
-    got = L.vpq_profile_read(buf, n_launch)
-    L.vpq_profile_enable(0)
-    assert got == n_launch, got
-    dur = np.array(buf[:], dtype=np.float64).reshape(passes, len(DECODE_LAYER)) * 1e3   # us
+    # ---- per-kernel durations ---------------------------------------------------------
+    dur = kernel_durations(layer_pass, launches_per_layer)
+    kernel_us_per_layer = float(dur.sum(axis=1).mean())
+    avg_launch_us = kernel_us_per_layer / launches_per_layer
+    achieved = layer_bytes / (kernel_us_per_layer * 1e-6) / 1e9
+    dur7 = dur if launches_per_layer == 7 else kernel_durations(pass_separate, 7)
     per_shape = {}
     for j, (name, K, N) in enumerate(DECODE_LAYER):
-        us = float(dur[:, j].mean())
+        us = float(dur7[:, j].mean())
         per_shape[name] = {"K": K, "N": N, "us": round(us, 3),
                            "GBps": round(alg_bytes(K, N, 1) / (us * 1e-6) / 1e9, 1)}
-    kernel_us_per_layer = float(dur.sum(axis=1).mean())
-    avg_launch_us = kernel_us_per_layer / len(DECODE_LAYER)
-    achieved = layer_bytes / (kernel_us_per_layer * 1e-6) / 1e9
     default_workload = args.variant == 0
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_PER_LAUNCH if default_workload else None,
-                "kernel": "qmv_mfma_kernel (all seven launches of a layer)", "avg_launch_us": round(avg_launch_us, 3),
-                "bytes_per_launch": layer_bytes / len(DECODE_LAYER),
-                "launches_timed": n_launch}
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": TRAFFIC_PER_LAYER / launches_per_layer if default_workload else None,
+                "kernel": "qmv_mfma_kernel (all %d launches of a layer)" % launches_per_layer,
+                "avg_launch_us": round(avg_launch_us, 3),
+                "bytes_per_launch": layer_bytes / launches_per_layer,
+                "launches_timed": int(dur.size)}
+    if launches_per_layer == 4:
+        roofline["launch_us"] = {n: round(float(dur[:, i].mean()), 3) for i, n in enumerate(("q|k|v", "o", "gate|up", "down"))}
 
     out = {
         "metric": "4-bit QMV HBM GB/s at batch 1 (decode-layer projection set)",
@@ -208,6 +241,8 @@ def main():
         "per_shape": per_shape,
         "roofline": roofline,
     }
+    if ms_other is not None:
+        out["us_per_layer_" + other] = round(ms_other * 1e3, 3)
 
     # ---- QMM at M = 2048 ---------------------------------------------------------------
     if not args.no_qmm:

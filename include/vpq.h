@@ -167,6 +167,23 @@ int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t
                           const uint16_t* biases, const uint16_t* x, uint16_t* y,
                           int K, int N, int M, void* ws, size_t ws_bytes);
 
+/* ---- several projections of one x in one launch ------------------------
+ * Replaces `affine_qmv_qkv_w4g64` (gpu-kernels/metal/quant/affine_qmv.metal:
+ * 405-516; slots 0:w 1:scales 2:biases 3:x 4:q_out 5:k_out 6:v_out 7:K
+ * 8:q_rows 9:k_rows 10:v_rows), the reference's answer to separate small
+ * GEMVs that under-occupy the GPU: `count` (1..4) packs [N_i, K] that share
+ * x [M,K], K and M are contracted by ONE kernel launch, each into its own
+ * y_i [M,N_i].  The row-concatenated q|k|v weight of the reference is the
+ * case w[1] = w[0] + q_rows*K/8 words (scales, biases alike); gate|up of an
+ * MLP is count = 2.  Arithmetic and requirements are those of
+ * vpq_qmv_w4g64_bf16 per pack (no residual); results are bit-identical to
+ * `count` separate calls of its VPQ_QMV_MFMA kernel.  The pointer tables are
+ * host arrays, read before the call returns.  Shapes the grouped kernel does
+ * not take (K % 512 != 0) run as separate launches. */
+int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,
+                             const uint16_t* const* scales, const uint16_t* const* biases,
+                             const uint16_t* x, uint16_t* const* y, int K, const int* N, int M);
+
 /* ---- a12: the packer ------------------------------------------------------
  * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:
  * 243-301; slots 0:x 1:w 2:s 3:b 4:K 5:N 6:clip) driven by

@@ -267,3 +267,44 @@ def test_linear_entrance_routes_by_rows(vpq, oracle, dev, D):
         y64, yb = fn(w, s, b, x, K, N, M)
         y = vpq.linear_w4g64(wd, sd, bd, D.bf16(x, dev), K, N, M)
         parity.check_bf16(D.bits(y), y64, yb)
+
+
+@pytest.mark.parametrize("K,Ns,M", [(4096, (4096, 1024, 1024), 1), (4096, (12288, 12288), 1), (1024, (48, 33, 16, 95), 3),
+                                    (2048, (64,), 2), (12288, (160, 4096), 16), (3840, (64, 32), 1)])
+def test_qmv_grouped_launch_equals_separate_launches(vpq, oracle, dev, D, K, Ns, M):
+    # q|k|v and gate|up in one launch (the reference's fused QKV GEMV, affine_qmv.metal:405-516):
+    # bit-identical to separate launches, and within tolerance of the oracle
+    packs, refs = [], []
+    x = synth.make_act(M, K, 9000 + K + M)
+    xd = D.bf16(x, dev)
+    for i, N in enumerate(Ns):
+        w, s, b = synth.make_weight(N, K, 8000 + 7 * i + N)
+        packs.append((D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), N))
+        refs.append(oracle.qmv(w, s, b, x, K, N, M))
+    outs = [parity.Guarded((M, N), torch.bfloat16, dev) for N in Ns]
+    vpq.qmv_group_w4g64(packs, xd, K, M, outs=[o.view for o in outs])
+    torch.cuda.synchronize()
+    variant = MFMA if K % 512 == 0 else AUTO
+    for (wd, sd, bd, N), (y64, yb), out in zip(packs, refs, outs):
+        got = D.bits(out.view)
+        parity.check_bf16(got, y64, yb)
+        out.assert_intact()
+        single = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=variant))
+        assert np.array_equal(got, single)
+
+
+def test_qmv_grouped_row_concatenated_qkv(vpq, oracle, dev, D):
+    # the reference's layout: one row-concatenated q|k|v pack, three outputs
+    K, rows, M = 2048, (256, 64, 64), 1
+    N = sum(rows)
+    w, s, b = synth.make_weight(N, K, 31)
+    x = synth.make_act(M, K, 32)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    packs, r0 = [], 0
+    for r in rows:
+        packs.append((wd[r0:r0 + r], sd[r0:r0 + r], bd[r0:r0 + r], r))
+        r0 += r
+    outs = vpq.qmv_group_w4g64(packs, xd, K, M)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    got = np.concatenate([D.bits(o) for o in outs], axis=1)
+    parity.check_bf16(got, y64, yb)

@@ -32,6 +32,7 @@ SYMBOLS = [
     ("vpq_qmm_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _f, _vp]),
     ("vpq_lora_a_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f]),
     ("vpq_linear_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz]),
+    ("vpq_qmv_group_w4g64_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
     ("vpq_quantize_w4g64", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
     ("vpq_f16_to_bf16", _i, [_vp, _vp, _vp, _sz]),
     ("vpq_profile_enable", _i, [_i]),
@@ -145,6 +146,22 @@ def linear_w4g64(w, scales, biases, x, K, N, M, out=None, ws=None):
     _check(load().vpq_linear_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
                                         K, N, M, _ptr(ws), ws_bytes), "vpq_linear_w4g64_bf16")
     return out
+
+
+def qmv_group_w4g64(packs, x, K, M, outs=None):
+    """packs: list of (w, scales, biases, N), 1..4 of them sharing x [M,K]; one launch."""
+    import torch
+    n = len(packs)
+    if outs is None:
+        outs = [torch.empty((M, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
+    PA = ctypes.c_void_p * n
+    wa = PA(*[p[0].data_ptr() for p in packs])
+    sa = PA(*[p[1].data_ptr() for p in packs])
+    ba = PA(*[p[2].data_ptr() for p in packs])
+    ya = PA(*[o.data_ptr() for o in outs])
+    na = (ctypes.c_int * n)(*[int(p[3]) for p in packs])
+    _check(load().vpq_qmv_group_w4g64_bf16(_stream(), n, wa, sa, ba, _ptr(x), ya, K, na, M), "vpq_qmv_group_w4g64_bf16")
+    return outs
 
 
 def quantize_w4g64(src, K, N, clip=1.0):

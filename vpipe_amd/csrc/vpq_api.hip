@@ -255,6 +255,41 @@ int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t
   return vpq_qmm_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, nullptr, nullptr, 0, 0.0f, nullptr);
 }
 
+int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,
+                             const uint16_t* const* scales, const uint16_t* const* biases,
+                             const uint16_t* x, uint16_t* const* y, int K, const int* N, int M)
+{
+  if (w == nullptr || scales == nullptr || biases == nullptr || y == nullptr || N == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (count < 1 || count > 4) { return VPQ_ERR_BAD_SHAPE; }
+  bool grouped = vpq::qmv_mfma_supports(K, 1, M) && x != nullptr && aligned(x, 16);
+  for (int i = 0; i < count; ++i) {
+    int st = check_pack(w[i], scales[i], biases[i], K, N[i]);
+    if (st != VPQ_OK) { return st; }
+    if (y[i] == nullptr) { return VPQ_ERR_NULL_POINTER; }
+    if (!aligned(y[i], 2)) { return VPQ_ERR_MISALIGNED; }
+    grouped = grouped && aligned(scales[i], 16) && aligned(biases[i], 16);
+  }
+  if (x == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16)) { return VPQ_ERR_MISALIGNED; }
+  if (!grouped) {
+    for (int i = 0; i < count; ++i) {
+      const int st = vpq_qmv_w4g64_bf16(stream, w[i], scales[i], biases[i], x, y[i], K, N[i], M, nullptr, nullptr, 0,
+                                        VPQ_QMV_AUTO);
+      if (st != VPQ_OK) { return st; }
+    }
+    return VPQ_OK;
+  }
+  int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.x = x; a.K = K; a.M = M; a.y_f32 = false; a.cu_count = g_dev.cu_count;
+  vpq::QmvGroup g;
+  g.count = count;
+  for (int i = 0; i < count; ++i) { g.seg[i] = vpq::QmvSeg{w[i], scales[i], biases[i], y[i], N[i]}; }
+  return finish(vpq::launch_qmv_mfma_group(reinterpret_cast<hipStream_t>(stream), a, g));
+}
+
 int vpq_quantize_w4g64(vpq_stream_t stream, const uint16_t* src, uint32_t* w, uint16_t* scales_f16,
                        uint16_t* biases_f16, int K, int N, float clip)
 {

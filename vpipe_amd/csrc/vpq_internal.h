@@ -74,6 +74,20 @@ hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a);
 // handles (the caller then falls back to the simple kernel).
 bool qmv_mfma_supports(int K, int N, int M);
 hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits);
+// Up to four projections that share x, K and M in ONE launch (q|k|v, gate|up): a.w/scales/
+// biases/y/N/residual/ws are ignored, the segments give them.
+struct QmvSeg {
+  const uint32_t* w;
+  const uint16_t* scales;
+  const uint16_t* biases;
+  void* y;
+  int N;
+};
+struct QmvGroup {
+  int count;
+  QmvSeg seg[4];
+};
+hipError_t launch_qmv_mfma_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g);
 size_t qmv_mfma_workspace_bytes(int K, int N, int M);
 bool qmv_stream_supports(int K, int N, int M);
 hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);

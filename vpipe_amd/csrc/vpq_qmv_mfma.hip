@@ -64,6 +64,11 @@ struct QmvParams {
   int slices_per_block;  // items of one workgroup's K range
   int split_k;
   int wave_lds_bytes;    // codes buffer + staged x rows of one wavefront
+  // Grouped launch (nseg > 1): workgroup blockIdx.x belongs to the segment whose tile range
+  // holds it; each segment is its own [N_i, K] pack and output.
+  int nseg;
+  QmvSeg seg[4];
+  int seg_tile_end[4];
 };
 
 // Eight nibbles of one packed word -> eight bf16 values 128+q, element order
@@ -129,7 +134,20 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
   const int xsum_row = (lane >> 4) < p.M ? (lane >> 4) : p.M - 1;
   float* red = reinterpret_cast<float*>(lds + NW * p.wave_lds_bytes);
 
-  const int n0 = blockIdx.x * kTileN;
+  // The pack this workgroup works on: the single one, or its segment of a grouped launch.
+  const uint32_t* w_ = p.w;
+  const uint16_t* scales_ = p.scales;
+  const uint16_t* biases_ = p.biases;
+  void* y_ = p.y;
+  int N_ = p.N;
+  int tile = blockIdx.x;
+  if (p.nseg > 1) {
+    int s = 0;
+    while (s + 1 < p.nseg && tile >= p.seg_tile_end[s]) { ++s; }
+    if (s > 0) { tile -= p.seg_tile_end[s - 1]; }
+    w_ = p.seg[s].w; scales_ = p.seg[s].scales; biases_ = p.seg[s].biases; y_ = p.seg[s].y; N_ = p.seg[s].N;
+  }
+  const int n0 = tile * kTileN;
   const int fr = lane & 15;                 // MFMA row (A) / column (B, D) of this lane
   const int g = lane >> 4;                  // k sub-block of this lane
   const int m_real = 4 * (fr & 3) + (fr >> 2);
@@ -139,18 +157,18 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
   const uint32_t row_bytes_total = (uint32_t)p.K >> 1;
 
   // Wave-uniform bases (tile origin) + 32-bit per-lane offsets.
-  const uint8_t* wtile = reinterpret_cast<const uint8_t*>(p.w) + (size_t)n0 * row_bytes_total;
+  const uint8_t* wtile = reinterpret_cast<const uint8_t*>(w_) + (size_t)n0 * row_bytes_total;
   uint32_t code_off[NLOAD];
 #pragma unroll
   for (int i = 0; i < NLOAD; ++i) {
     const int row = i * ROWS_PER_LOAD + lane / CH;
     const int chunk = (lane % CH) ^ (row & (CH - 1));
-    const int rrow = (n0 + row < p.N) ? row : (p.N - 1 - n0);
+    const int rrow = (n0 + row < N_) ? row : (N_ - 1 - n0);
     code_off[i] = (uint32_t)rrow * row_bytes_total + (uint32_t)chunk * 16;
   }
-  const int srow = (n0 + fr < p.N) ? fr : (p.N - 1 - n0);
-  const uint16_t* stile = p.scales + (size_t)n0 * Kg;
-  const uint16_t* btile = p.biases + (size_t)n0 * Kg;
+  const int srow = (n0 + fr < N_) ? fr : (N_ - 1 - n0);
+  const uint16_t* stile = scales_ + (size_t)n0 * Kg;
+  const uint16_t* btile = biases_ + (size_t)n0 * Kg;
   const uint32_t sb_off = (uint32_t)srow * (uint32_t)Kg;
   // LDS byte address of this lane's two words of group 0: row fr, chunk g/2 (swizzled), half g%2.
   const int lds_code0 = fr * kRowBytes + (g & 1) * 8;
@@ -271,7 +289,7 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
     m = 4 * r + (l >> 4);
     n = n0 + (l & 15);
   }
-  const bool valid = owner && m < p.M && n < p.N;
+  const bool valid = owner && m < p.M && n < N_;
 
   if (p.split_k > 1) {
     // Publish this workgroup's partial, then let the last arrival fold all of
@@ -294,15 +312,15 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
   }
 
   if (valid) {
-    const size_t o = (size_t)m * p.N + n;
+    const size_t o = (size_t)m * N_ + n;
     if (F32OUT) {
-      reinterpret_cast<float*>(p.y)[o] = total;
+      reinterpret_cast<float*>(y_)[o] = total;
     } else {
       uint32_t v = f32_to_bf16_bits(total);
       if (p.residual != nullptr) {
         v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(p.residual[o]));
       }
-      reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)v;
+      reinterpret_cast<uint16_t*>(y_)[o] = (uint16_t)v;
     }
   }
 }
@@ -351,6 +369,7 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
   p.residual = a.residual;
   p.K = a.K; p.N = a.N; p.M = a.M;
+  p.nseg = 1;
   p.slices = a.K / kKS;
 
   int split = force_splits > 0 ? force_splits : choose_split(a.K, a.N, a.cu_count);
@@ -401,6 +420,55 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   if (mr == 1) { return launch(qmv_mfma_kernel<1, true, false>, 3); }
   if (mr == 2) { return launch(qmv_mfma_kernel<2, false, false>, 4); }
   return launch(qmv_mfma_kernel<4, false, false>, 5);
+}
+
+hipError_t launch_qmv_mfma_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g)
+{
+  QmvParams p;
+  p.w = nullptr; p.scales = nullptr; p.biases = nullptr; p.x = a.x; p.y = nullptr;
+  p.residual = nullptr;
+  p.K = a.K; p.N = 0; p.M = a.M;
+  p.slices = a.K / kKS;
+  p.slices_per_block = p.slices;
+  p.split_k = 1;
+  p.counters = nullptr;
+  p.partial = nullptr;
+  p.nseg = g.count;
+  int tiles = 0;
+  for (int i = 0; i < 4; ++i) {
+    if (i < g.count) {
+      p.seg[i] = g.seg[i];
+      tiles += (g.seg[i].N + kTileN - 1) / kTileN;
+    } else {
+      p.seg[i] = g.seg[g.count - 1];
+    }
+    p.seg_tile_end[i] = tiles;
+  }
+  if (g.count == 1) {          // the kernel's single-pack path reads p.w etc.
+    p.w = g.seg[0].w; p.scales = g.seg[0].scales; p.biases = g.seg[0].biases; p.y = g.seg[0].y; p.N = g.seg[0].N;
+  }
+  const int per_wave = (p.slices + kMaxWaves - 1) / kMaxWaves;
+  int nw = (p.slices + per_wave - 1) / per_wave;
+  int mr = (a.M + 3) / 4;
+  if (mr == 3) { mr = 4; }
+  if (nw < mr) { nw = mr; }
+  const bool xlds = a.M <= 4;
+  p.wave_lds_bytes = kItemBytes + (xlds ? a.M * kXRowBytes + kXsumBytes : 0);
+  const size_t lds_bytes = (size_t)nw * p.wave_lds_bytes + (size_t)nw * mr * kWave * sizeof(float);
+  const dim3 grid((unsigned)tiles, 1u), block((unsigned)(nw * kWave));
+  static bool attr_done[3] = {false, false, false};
+  auto launch = [&](auto kern, int slot) -> hipError_t {
+    if (!attr_done[slot]) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
+      if (e != hipSuccess) { return e; }
+      attr_done[slot] = true;
+    }
+    return launch_kernel(kern, grid, block, lds_bytes, st, p);
+  };
+  if (mr == 1) { return launch(qmv_mfma_kernel<1, true, false>, 0); }
+  if (mr == 2) { return launch(qmv_mfma_kernel<2, false, false>, 1); }
+  return launch(qmv_mfma_kernel<4, false, false>, 2);
 }
 
 }  // namespace vpq

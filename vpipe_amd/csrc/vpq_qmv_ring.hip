@@ -14,14 +14,12 @@
 //           biases (8 groups each).  Two slots per wavefront; a slot's content is copied to
 //           registers first, the slot is re-requested for the item after next, and only then
 //           the copy is contracted: two items are in flight during the arithmetic.
-//   waits   Every request in flight is a direct-to-LDS load, so the load counter retires
-//           them in issue order and `s_waitcnt vmcnt(n)` with n = requests issued after the
-//           item is exact.  This is deliberate: register loads and direct-to-LDS loads do
-//           NOT retire in order with respect to each other on this part (measured: waiting
-//           with counts that mix the two read slots before their last load had landed), so a
-//           count over a mixed queue proves nothing.  For M <= 4 the slices of x come through
-//           LDS the same way (four loads, requested a whole slice ahead); for M > 4 they are
-//           plain register loads and the queue is drained (vmcnt(0)) at each change of slice.
+//   waits   The load counter retires requests in issue order, so `s_waitcnt vmcnt(n)` with
+//           n = requests issued after the item is exact.  Everything in flight during the
+//           steady state is a direct-to-LDS load (for M <= 4 the slices of x come through LDS
+//           the same way: four loads, requested a whole slice ahead), which keeps the counts
+//           to one rule: 5 per item, 4 per slice of x.  For M > 4 the slices of x are plain
+//           register loads and the queue is drained (vmcnt(0)) at each change of slice.
 //           The LDS reads of what those loads wrote are written as asm so that the compiler,
 //           which cannot see the counts, does not add its own wait for everything.
 //   math    codes -> bf16 (128 + q) by one v_and_or_b32 per nibble pair, contracted with x
