@@ -271,3 +271,26 @@ def test_quant_linear_forward_with_lora(enc, oracle, dev, D):
     t = oracle.lora_t(x, A, M, K, r, strength)
     y64, yb = oracle.qmm(w, s, b, x, K, N, M, t=t, B=B, r=r)
     parity.check_bf16(D.bits(yd), y64, yb)
+
+
+def test_fused_qkv_call_site(enc, oracle, dev, D):
+    # llama decode: one dispatch over the row-concatenated q|k|v pack, three output buffers
+    # (gpu-kernels/metal/quant/affine_qmv.metal:405-516)
+    K, rows = 1024, (512, 128, 128)
+    N = sum(rows)
+    w, s, b = synth.make_weight(N, K, 50)
+    x = synth.make_act(1, K, 51)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    outs = [torch.zeros((1, r), dtype=torch.bfloat16, device=dev) for r in rows]
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_qkv_w4g64") == 1
+    for i, t in enumerate((wd, sd, bd, xd, outs[0], outs[1], outs[2])):
+        enc.set_buffer(i, t)
+    enc.set_constant(7, K)
+    for i, r in enumerate(rows):
+        enc.set_constant(8 + i, r)
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    y64, yb = oracle.qmv(w, s, b, x, K, N, 1)
+    got = np.concatenate([D.bits(o) for o in outs], axis=1)
+    parity.check_bf16(got, y64, yb)

@@ -81,6 +81,7 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_batch4_xp_w4g64", QuantKernel::QmvBatch},
     {"affine_qmv_bf16", "affine_qmv_batch8_xp_w4g64", QuantKernel::QmvBatch},
     {"affine_qmv_bf16", "affine_qmv_batch8_xp2_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_qkv_w4g64", QuantKernel::QmvQkv},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64", QuantKernel::Qmm},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm64", QuantKernel::Qmm},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm128", QuantKernel::Qmm},
@@ -348,6 +349,31 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
     } else {
       status = vpq_dequant_w4g64_bf16(st, static_cast<const uint32_t*>(buf(0)), static_cast<const uint16_t*>(buf(1)),
                                       static_cast<const uint16_t*>(buf(2)), static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
+    }
+  } else if (kind == QuantKernel::QmvQkv) {
+    // gpu-kernels/metal/quant/affine_qmv.metal:497-516: slots 0:w 1:scales 2:biases 3:x 4:q_out
+    // 5:k_out 6:v_out 7:K 8:q_rows 9:k_rows 10:v_rows; the pack is the row-concatenated q|k|v.
+    if (!buf(0) || !buf(1) || !buf(2) || !buf(3) || !buf(4) || !buf(5) || !has_int(7) || !has_int(8) || !has_int(9) ||
+        !has_int(10) || (ival(10) > 0 && !buf(6))) {
+      status = VPQ_ERR_NULL_POINTER;
+    } else if (ival(7) <= 0 || ival(7) % 64 != 0 || ival(8) <= 0 || ival(9) <= 0 || ival(10) < 0) {
+      status = VPQ_ERR_BAD_SHAPE;
+    } else {
+      const int K = ival(7);
+      const int rows[3] = {ival(8), ival(9), ival(10)};
+      const uint32_t* w[3];
+      const uint16_t* sc[3];
+      const uint16_t* bi[3];
+      uint16_t* y[3] = {static_cast<uint16_t*>(buf(4)), static_cast<uint16_t*>(buf(5)), static_cast<uint16_t*>(buf(6))};
+      size_t r0 = 0;
+      for (int i = 0; i < 3; ++i) {
+        w[i] = static_cast<const uint32_t*>(buf(0)) + r0 * (size_t)(K / 8);
+        sc[i] = static_cast<const uint16_t*>(buf(1)) + r0 * (size_t)(K / 64);
+        bi[i] = static_cast<const uint16_t*>(buf(2)) + r0 * (size_t)(K / 64);
+        r0 += (size_t)rows[i];
+      }
+      status = vpq_qmv_group_w4g64_bf16(st, rows[2] > 0 ? 3 : 2, w, sc, bi, static_cast<const uint16_t*>(buf(3)), y, K,
+                                        rows, 1);
     }
   } else {
     // slots 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N, 7: residual | m_total | M

@@ -73,6 +73,8 @@ enum class QuantKernel : std::uint8_t {
   QmvAdd,         // affine_qmv_w4g64_add          slot 7 = residual buffer
   QmvBatch,       // affine_qmv_batch*_w4g64       slot 7 = m_total
   Qmm,            // affine_qmm_steel_w4g64[_bm64|_bm128], affine_qmm_mma_w4g64    slot 7 = M
+  QmvQkv,         // affine_qmv_qkv_w4g64: row-concatenated q|k|v pack, slots 4,5,6 = q,k,v outputs,
+                  //   7 = K, 8,9,10 = q_rows, k_rows, v_rows (v_rows == 0: q|k only); one launch
 };
 
 class QuantFunction {
