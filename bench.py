@@ -40,6 +40,8 @@ TRAFFIC_PER_LAYER = 109.68e6
 DECODE_LAYER = [("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024), ("o", 4096, 4096),
                 ("gate", 4096, 12288), ("up", 4096, 12288), ("down", 12288, 4096)]
 PREFILL = [("gate_up", 4096, 12288), ("down", 12288, 4096), ("attn", 4096, 4096)]
+SMALL_BATCH = [(5120, 5120), (5120, 17408), (17408, 5120), (5120, 151936)]
+DIT = [(5120, 5120), (5120, 20480), (20480, 5120)]
 
 
 def alg_bytes(K, N, M):
@@ -63,6 +65,7 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="QMV kernel variant (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the QMM section")
+    ap.add_argument("--no-extras", action="store_true", help="skip the small-batch QMV and video-DiT QMM sections")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 256 MiB device-to-device copies (a kernel of known traffic, to scale "
@@ -104,10 +107,14 @@ def main():
         w, s, b = layers[li][j]
         vpipe_amd.qmv_w4g64(w, s, b, xs[K], K, N, 1, out=ys[j], ws=wss[j], variant=args.variant)
 
+    groups = {}
+
     def group(li, js):
-        K = DECODE_LAYER[js[0]][1]
-        packs = [layers[li][j] + (DECODE_LAYER[j][2],) for j in js]
-        vpipe_amd.qmv_group_w4g64(packs, xs[K], K, 1, outs=[ys[j] for j in js])
+        if (li, js) not in groups:
+            K = DECODE_LAYER[js[0]][1]
+            packs = [layers[li][j] + (DECODE_LAYER[j][2],) for j in js]
+            groups[(li, js)] = vpipe_amd.capi.QmvGroup(packs, xs[K], K, 1, [ys[j] for j in js])
+        groups[(li, js)].launch()
 
     def pass_separate(li):
         """Seven launches, one per projection."""
@@ -274,6 +281,59 @@ def main():
         out["roofline_qmm"] = {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TF,
                                "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TF, 4), "traffic": None,
                                "kernel": "qmm_tile_kernel<false>"}
+
+    # ---- the other configurations, as context (not part of `value`) -----------------------
+    if not args.no_extras:
+        def kernel_us(fn, iters):
+            for _ in range(2):
+                fn(0)
+            torch.cuda.synchronize()
+            L.vpq_profile_enable(4 * iters)
+            for i in range(iters):
+                fn(i)
+            kb = (ctypes.c_float * (4 * iters))()
+            n = L.vpq_profile_read(kb, 4 * iters)
+            L.vpq_profile_enable(0)
+            return float(np.sum(kb[:n])) * 1e3 / iters     # all kernels of a call (LoRA: two)
+
+        # small-batch QMV of a 5120-hidden model, weights rotated so that they come from HBM
+        small = {}
+        for K, N in SMALL_BATCH:
+            copies = max(2, min(8, int(600e6 // (N * K * 9 // 16))))
+            packs = [make_weight(torch, N, K, dev, gen) for _ in range(copies)]
+            row = {}
+            for M in (1, 2, 4, 8, 16):
+                x = torch.randn((M, K), device=dev, generator=gen).bfloat16()
+                y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+
+                def call(i, x=x, y=y, M=M):
+                    w, s, b = packs[i % copies]
+                    vpipe_amd.qmv_w4g64(w, s, b, x, K, N, M, out=y)
+                us = kernel_us(call, 2 * copies)
+                row["M=%d" % M] = {"us": round(us, 2), "GBps": round(alg_bytes(K, N, M) / (us * 1e-6) / 1e9, 1)}
+            small["%d->%d" % (K, N)] = row
+            del packs
+        out["qmv_small_batch"] = small
+
+        # video-DiT QMM with the fused rank-32 LoRA (flops of the base contraction only)
+        M, r, alpha = 16320, 32, 1.0
+        dit = {}
+        for K, N in DIT:
+            w, s, b = make_weight(torch, N, K, dev, gen)
+            x = torch.randn((M, K), device=dev, generator=gen).bfloat16()
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            A = (torch.randn((r, K), device=dev, generator=gen) * 0.02).bfloat16()
+            B = (torch.randn((N, r), device=dev, generator=gen) * 0.02).bfloat16()
+            t = torch.empty((M, r), dtype=torch.bfloat16, device=dev)
+            us0 = kernel_us(lambda i: vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y), 3)
+            us1 = kernel_us(lambda i: vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y, lora_A=A, lora_B=B, r=r,
+                                                         alpha=alpha, t_ws=t), 3)
+            flops = 2.0 * M * N * K
+            dit["%d->%d" % (K, N)] = {"us": round(us0, 1), "TFLOPs": round(flops / (us0 * 1e-6) / 1e12, 1),
+                                      "us_with_lora": round(us1, 1),
+                                      "TFLOPs_with_lora": round(flops / (us1 * 1e-6) / 1e12, 1)}
+            del w, s, b, x, y, A, B, t
+        out["qmm_dit_m16320_lora_r32"] = dit
 
     # ---- CPU baseline: the oracle's dequant + fp32 matmul on the host cores ------------
     if not args.no_cpu:

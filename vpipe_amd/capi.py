@@ -148,20 +148,35 @@ def linear_w4g64(w, scales, biases, x, K, N, M, out=None, ws=None):
     return out
 
 
+class QmvGroup:
+    """The pointer tables of a grouped launch, built once for a fixed set of tensors so that a
+    launch costs one foreign call (a decode loop launches the same groups every token)."""
+
+    def __init__(self, packs, x, K, M, outs):
+        n = len(packs)
+        PA = ctypes.c_void_p * n
+        self.keep = (packs, x, outs)       # the tables hold raw pointers: keep the tensors alive
+        self.n, self.K, self.M = n, K, M
+        self.w = PA(*[p[0].data_ptr() for p in packs])
+        self.s = PA(*[p[1].data_ptr() for p in packs])
+        self.b = PA(*[p[2].data_ptr() for p in packs])
+        self.y = PA(*[o.data_ptr() for o in outs])
+        self.N = (ctypes.c_int * n)(*[int(p[3]) for p in packs])
+        self.x = _ptr(x)
+        self.outs = outs
+
+    def launch(self):
+        _check(load().vpq_qmv_group_w4g64_bf16(_stream(), self.n, self.w, self.s, self.b, self.x, self.y, self.K,
+                                               self.N, self.M), "vpq_qmv_group_w4g64_bf16")
+        return self.outs
+
+
 def qmv_group_w4g64(packs, x, K, M, outs=None):
     """packs: list of (w, scales, biases, N), 1..4 of them sharing x [M,K]; one launch."""
     import torch
-    n = len(packs)
     if outs is None:
         outs = [torch.empty((M, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
-    PA = ctypes.c_void_p * n
-    wa = PA(*[p[0].data_ptr() for p in packs])
-    sa = PA(*[p[1].data_ptr() for p in packs])
-    ba = PA(*[p[2].data_ptr() for p in packs])
-    ya = PA(*[o.data_ptr() for o in outs])
-    na = (ctypes.c_int * n)(*[int(p[3]) for p in packs])
-    _check(load().vpq_qmv_group_w4g64_bf16(_stream(), n, wa, sa, ba, _ptr(x), ya, K, na, M), "vpq_qmv_group_w4g64_bf16")
-    return outs
+    return QmvGroup(packs, x, K, M, outs).launch()
 
 
 def quantize_w4g64(src, K, N, clip=1.0):
