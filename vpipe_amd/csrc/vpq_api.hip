@@ -203,11 +203,7 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
   if (!aligned(x, 16) || !aligned(lora_a, 16) || !aligned(t, 16)) { return VPQ_ERR_MISALIGNED; }
   const int st = ensure_init();
   if (st != VPQ_OK) { return st; }
-  vpq::GemmArgs g{};
-  g.w = nullptr; g.b_dense = lora_a; g.x = x; g.y = t;
-  g.K = K; g.N = r; g.M = M; g.r = 0; g.out_scale = alpha; g.scaled_epilogue = true;
-  g.cu_count = g_dev.cu_count;
-  return finish(vpq::launch_gemm(reinterpret_cast<hipStream_t>(stream), g));
+  return finish(vpq::launch_lora_a(reinterpret_cast<hipStream_t>(stream), x, lora_a, t, M, K, r, alpha));
 }
 
 int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
@@ -240,7 +236,6 @@ int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
   g.lora_t = lora ? lora_t_ws : nullptr;
   g.lora_b = lora ? lora_b : nullptr;
   g.r = lora ? r : 0;
-  g.out_scale = 1.0f; g.scaled_epilogue = false;
   g.cu_count = g_dev.cu_count;
   return finish(vpq::launch_qmm_tile(hs, g));
 }

@@ -52,18 +52,15 @@ struct QmvArgs {
 };
 
 struct GemmArgs {
-  const uint32_t* w;         // packed codes, or nullptr for a dense B
+  const uint32_t* w;         // packed codes
   const uint16_t* scales;
   const uint16_t* biases;
-  const uint16_t* b_dense;   // dense bf16 B [N,K] when w == nullptr
   const uint16_t* x;         // [M,K]
   uint16_t* y;               // [M,N]
   int K, N, M;
   const uint16_t* lora_t;    // nullable, [M,r]
   const uint16_t* lora_b;    // nullable, [N,r]
   int r;
-  float out_scale;           // LoRA-A epilogue: y = bf16(out_scale * bf16(acc)); unused otherwise
-  bool scaled_epilogue;
   int cu_count;
 };
 
@@ -94,7 +91,9 @@ hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);
 bool qmv_ring_supports(int K, int N, int M);
 // tc_hint / nw_hint > 0 force the tiles / wavefronts per workgroup (measurement only).
 hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint);
-hipError_t launch_gemm(hipStream_t st, const GemmArgs& a);
+// t[M,r] = bf16(alpha * bf16(x . A^T)), r in {32, 64, 96, 128}.
+hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
+                         float alpha);
 // 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.
 hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a);
 hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
