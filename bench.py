@@ -13,8 +13,9 @@ times seven launches, and the other mode's time is reported beside `value`.
 The timed region is one HIP graph of `steps` passes, replayed between two
 events on the launch stream with inputs already resident in HBM.
 
-Also reported on the same JSON line: the per-kernel roofline fraction (kernel
-durations from hipExtLaunchKernel events, no launch gaps), per-shape numbers,
+Also reported on the same JSON line: the roofline fraction of the QMV kernel
+(timed region / launches), per-shape kernel durations of eager launches
+(hipExtLaunchKernel events), the small-batch and video-DiT configurations,
 QMM at M = 2048 in TFLOP/s, and the CPU baseline (the oracle's dequant + fp32
 matmul on the host cores) on a bounded sample.
 """
@@ -65,6 +66,9 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="QMV kernel variant (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the QMM section")
+    ap.add_argument("--only", action="store_true",
+                    help="run nothing but the selected launch mode of the decode-layer set (for a profiler: every "
+                         "QMV launch in the trace then belongs to the timed workload)")
     ap.add_argument("--no-extras", action="store_true", help="skip the small-batch QMV and video-DiT QMM sections")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -199,8 +203,11 @@ def main():
     layer_pass, launches_per_layer, launch_text = modes[args.launch]
     use_graph = not args.no_graph
 
+    if args.only:
+        args.no_qmm = args.no_extras = args.no_cpu = True
     for i in range(args.warmup):
-        pass_separate(i % args.layers)
+        if not args.only:
+            pass_separate(i % args.layers)
         layer_pass(i % args.layers)
     torch.cuda.synchronize()
 
@@ -209,19 +216,25 @@ def main():
     value = layer_bytes / (ms_per_step * 1e-3) / 1e9
     launch = ("hipgraph, " if use_graph else "eager, ") + launch_text
     other = "separate" if args.launch != "separate" else "grouped"
-    ms_other = time_steps(modes[other][0], args.steps, use_graph) if args.variant == 0 else None
+    ms_other = time_steps(modes[other][0], args.steps, use_graph) if args.variant == 0 and not args.only else None
 
-    # ---- per-kernel durations ---------------------------------------------------------
+    # ---- roofline of the dominant kernel ------------------------------------------------
+    # Every launch of the timed region is the same kernel (qmv_mfma_kernel); its average launch
+    # duration is the timed region (events on the launch stream around the graph replay) divided
+    # by the launches in it -- back-to-back kernels of one stream, so launch gaps are included.
+    avg_launch_us = ms_per_step * 1e3 / launches_per_layer
+    achieved = (layer_bytes / launches_per_layer) / (avg_launch_us * 1e-6) / 1e9
+    # Per-launch detail from hipExtLaunchKernel start/stop events of eager launches (these run
+    # slower than the same kernels inside the graph when the host cannot keep the queue full).
     dur = kernel_durations(layer_pass, launches_per_layer)
     kernel_us_per_layer = float(dur.sum(axis=1).mean())
-    avg_launch_us = kernel_us_per_layer / launches_per_layer
-    achieved = layer_bytes / (kernel_us_per_layer * 1e-6) / 1e9
-    dur7 = dur if launches_per_layer == 7 else kernel_durations(pass_separate, 7)
     per_shape = {}
-    for j, (name, K, N) in enumerate(DECODE_LAYER):
-        us = float(dur7[:, j].mean())
-        per_shape[name] = {"K": K, "N": N, "us": round(us, 3),
-                           "GBps": round(alg_bytes(K, N, 1) / (us * 1e-6) / 1e9, 1)}
+    if launches_per_layer == 7 or not args.only:
+        dur7 = dur if launches_per_layer == 7 else kernel_durations(pass_separate, 7)
+        for j, (name, K, N) in enumerate(DECODE_LAYER):
+            us = float(dur7[:, j].mean())
+            per_shape[name] = {"K": K, "N": N, "us": round(us, 3),
+                               "GBps": round(alg_bytes(K, N, 1) / (us * 1e-6) / 1e9, 1)}
     default_workload = args.variant == 0
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
@@ -229,9 +242,10 @@ def main():
                 "kernel": "qmv_mfma_kernel (all %d launches of a layer)" % launches_per_layer,
                 "avg_launch_us": round(avg_launch_us, 3),
                 "bytes_per_launch": layer_bytes / launches_per_layer,
-                "launches_timed": int(dur.size)}
+                "launches_timed": args.steps * launches_per_layer}
     if launches_per_layer == 4:
-        roofline["launch_us"] = {n: round(float(dur[:, i].mean()), 3) for i, n in enumerate(("q|k|v", "o", "gate|up", "down"))}
+        roofline["eager_launch_us"] = {n: round(float(dur[:, i].mean()), 3)
+                                       for i, n in enumerate(("q|k|v", "o", "gate|up", "down"))}
 
     out = {
         "metric": "4-bit QMV HBM GB/s at batch 1 (decode-layer projection set)",
@@ -244,7 +258,7 @@ def main():
                    "algorithmic_bytes_per_step": layer_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "us_per_layer": round(ms_per_step * 1e3, 3),
-        "kernel_us_per_layer": round(kernel_us_per_layer, 3),
+        "eager_kernel_us_per_layer": round(kernel_us_per_layer, 3),
         "per_shape": per_shape,
         "roofline": roofline,
     }
