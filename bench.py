@@ -265,6 +265,40 @@ def main():
     if ms_other is not None:
         out["us_per_layer_" + other] = round(ms_other * 1e3, 3)
 
+    def dense_gemm_us(w, s, b, x, y, K, N, iters=10):
+        """Yardstick, not product: the vendor library's dense bf16 GEMM (torch.matmul) on the SAME
+        operands with the weight expanded to bf16 beforehand -- what a GEMM with no dequantization
+        at all reaches on this box with these (non-trivial) values."""
+        wdeq = vpipe_amd.dequant_w4g64(w, s, b, K, N)
+        for _ in range(3):
+            torch.matmul(x, wdeq.t(), out=y)
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(iters):
+            torch.matmul(x, wdeq.t(), out=y)
+        t1.record()
+        torch.cuda.synchronize()
+        return t0.elapsed_time(t1) * 1e3 / iters
+
+    def dense_route_us(w, s, b, x, y, K, N, M, iters):
+        """The library's own dequant-once route: (expansion + vendor GEMM per call, vendor GEMM alone
+        when the expansion is kept), us per call from events on the stream."""
+        wdeq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+        res = []
+        for expand in (True, False):
+            for _ in range(2):
+                vpipe_amd.qmm_dense_route_w4g64(w, s, b, x, K, N, M, wdeq, expand=expand, out=y)
+            torch.cuda.synchronize()
+            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0.record()
+            for _ in range(iters):
+                vpipe_amd.qmm_dense_route_w4g64(w, s, b, x, K, N, M, wdeq, expand=expand, out=y)
+            t1.record()
+            torch.cuda.synchronize()
+            res.append(t0.elapsed_time(t1) * 1e3 / iters)
+        return res
+
     # ---- QMM at M = 2048 ---------------------------------------------------------------
     if not args.no_qmm:
         M = 2048
@@ -286,7 +320,11 @@ def main():
             L.vpq_profile_enable(0)
             us = float(np.mean(kb[:n])) * 1e3
             flops = 2.0 * M * N * K
-            qmm[name] = {"K": K, "N": N, "M": M, "us": round(us, 2), "TFLOPs": round(flops / (us * 1e-6) / 1e12, 1)}
+            qmm[name] = {"K": K, "N": N, "M": M, "us": round(us, 2), "TFLOPs": round(flops / (us * 1e-6) / 1e12, 1),
+                         "vendor_dense_bf16_TFLOPs": round(flops / (dense_gemm_us(w, s, b, x, y, K, N) * 1e-6) / 1e12, 1)}
+            dr = dense_route_us(w, s, b, x, y, K, N, M, 10)
+            qmm[name]["dense_route_TFLOPs"] = round(flops / (dr[0] * 1e-6) / 1e12, 1)
+            qmm[name]["dense_route_kept_expansion_TFLOPs"] = round(flops / (dr[1] * 1e-6) / 1e12, 1)
             tot_flops += flops
             tot_us += us
             del w, s, b, x, y
@@ -294,7 +332,9 @@ def main():
         out["qmm_m2048"] = qmm
         out["roofline_qmm"] = {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TF,
                                "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TF, 4), "traffic": None,
-                               "kernel": "qmm_tile_kernel<false>"}
+                               "kernel": "qmm_tile_kernel<false>",
+                               "note": "vendor_dense_bf16_TFLOPs in qmm_m2048 = torch.matmul on the expanded "
+                                       "weight, same operands: the dense-GEMM rate this box sustains on real data"}
 
     # ---- the other configurations, as context (not part of `value`) -----------------------
     if not args.no_extras:
@@ -345,7 +385,12 @@ def main():
             flops = 2.0 * M * N * K
             dit["%d->%d" % (K, N)] = {"us": round(us0, 1), "TFLOPs": round(flops / (us0 * 1e-6) / 1e12, 1),
                                       "us_with_lora": round(us1, 1),
-                                      "TFLOPs_with_lora": round(flops / (us1 * 1e-6) / 1e12, 1)}
+                                      "TFLOPs_with_lora": round(flops / (us1 * 1e-6) / 1e12, 1),
+                                      "vendor_dense_bf16_TFLOPs": round(
+                                          flops / (dense_gemm_us(w, s, b, x, y, K, N, iters=3) * 1e-6) / 1e12, 1)}
+            dr = dense_route_us(w, s, b, x, y, K, N, M, 3)
+            dit["%d->%d" % (K, N)]["dense_route_TFLOPs"] = round(flops / (dr[0] * 1e-6) / 1e12, 1)
+            dit["%d->%d" % (K, N)]["dense_route_kept_expansion_TFLOPs"] = round(flops / (dr[1] * 1e-6) / 1e12, 1)
             del w, s, b, x, y, A, B, t
         out["qmm_dit_m16320_lora_r32"] = dit
 

@@ -153,6 +153,25 @@ int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
                        const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
                        uint16_t* lora_t_ws);
 
+/* ---- a8: the dequant-once route -------------------------------------------
+ * Replaces `gemm_mma_` (generative-models/minimax-h3/metal-minimax-h3-transformer.cc:
+ * 2020-2160: `affine_dequant_w4g64` into a scratch, then a dense matrix-unit GEMM,
+ * gpu-kernels/metal/gemm/dense_gemm_mma.metal:44-93): the pack is expanded into
+ * `w_deq` (bf16 [N,K], caller-owned, 2*N*K bytes, 16-byte aligned) and
+ * y = bf16( x . w_deq^T ) is computed by the vendor BLAS (rocBLAS gemm_ex, bf16
+ * operands, fp32 accumulation).  Same arithmetic as vpq_qmm_w4g64_bf16 up to the
+ * order of the fp32 additions.  `expand` != 0 runs the expansion first; 0 says
+ * that `w_deq` already holds this pack's expansion (a weight is immutable after
+ * load, so a caller with the room expands each Linear once).  No adapter on this
+ * route.  rocBLAS is opened at first use (that call allocates its handle);
+ * VPQ_ERR_UNSUPPORTED with the reason in vpq_last_device_error() if it is not
+ * there.  On MI355X this route is the faster one where M is large (measured
+ * 1.5 PFLOP/s at M = 16320 against 0.9 fused) and the fused kernel where the
+ * 2*N*K bytes are not available. */
+int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                                   int K, int N, int M, uint16_t* w_deq, int expand);
+
 /* The adapter's first GEMM alone: t[M,r] = bf16(alpha * bf16(x . A^T)).
  * Replaces `lora_gemm_a_` (metal-minimax-h3-transformer.cc:1030-1067). */
 int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t,

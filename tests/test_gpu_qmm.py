@@ -151,3 +151,22 @@ def test_qmm_prefill_shapes(vpq, oracle, dev, D, K, N):
 def test_qmm_video_dit_shapes_with_lora(vpq, oracle, dev, D, K, N):
     # M = 16320 = 127*128 + 64: an M tail; y of 5120->20480 is 668 MB: 64-bit addressing
     _sampled_check(vpq, oracle, dev, D, 16320, N, K, 0x5EED0005 + N, lora_r=32, alpha=1.0)
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (130, 320, 256), (33, 33, 128), (257, 129, 512), (1, 8, 64)])
+def test_qmm_dense_route_matches_oracle(vpq, oracle, dev, D, M, N, K):
+    # the dequant-once route (expansion + vendor dense GEMM): same arithmetic as the fused kernel
+    w, s, b = synth.make_weight(N, K, 4200 + N + K)
+    x = synth.make_act(M, K, 4300 + M)
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    w_deq = torch.zeros((N, K), dtype=torch.bfloat16, device=dev)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq, expand=True, out=out.view)
+    torch.cuda.synchronize()
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    out.assert_intact()
+    assert np.array_equal(D.bits(w_deq), oracle.dequant_bf16(w, s, b, K, N))
+    # with the kept expansion: no expansion pass, same bits
+    again = vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq, expand=False)
+    assert torch.equal(again, out.view)

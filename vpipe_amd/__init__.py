@@ -7,4 +7,4 @@ implementation of any operator and raises if the library is missing.
 """
 from . import capi  # noqa: F401
 from .capi import (VpqError, dequant_w4g64, f16_to_bf16, lib_path, linear_w4g64, load, lora_a,  # noqa: F401
-                   qmm_w4g64, qmv_group_w4g64, qmv_w4g64, qmv_workspace, quantize_w4g64)
+                   qmm_dense_route_w4g64, qmm_w4g64, qmv_group_w4g64, qmv_w4g64, qmv_workspace, quantize_w4g64)

@@ -240,6 +240,33 @@ int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
   return finish(vpq::launch_qmm_tile(hs, g));
 }
 
+int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                   uint16_t* w_deq, int expand)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (w_deq == nullptr) { return VPQ_ERR_WORKSPACE; }
+  if (M <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (expand != 0) {
+    st = finish(vpq::launch_dequant(hs, w, scales, biases, w_deq, K, N));
+    if (st != VPQ_OK) { return st; }
+  }
+  std::string why;
+  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, &why);
+  if (rc != 0) {
+    strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
+    g_last_error[sizeof(g_last_error) - 1] = '\0';
+    return rc == -1 ? VPQ_ERR_UNSUPPORTED : VPQ_ERR_DEVICE;
+  }
+  return VPQ_OK;
+}
+
 int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                           void* ws, size_t ws_bytes)

@@ -7,6 +7,7 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <string>
 #include <vector>
 
 namespace vpq {
@@ -96,6 +97,10 @@ hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, u
                          float alpha);
 // 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.
 hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a);
+// y[M,N] = x[M,K] . b[N,K]^T on the vendor BLAS (bf16 in, fp32 accumulate, bf16 out).
+// 0, or -1 (rocBLAS unavailable) / -2 (the call failed) with *why set.
+int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,
+                    std::string* why);
 hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
                            uint16_t* b_f16, int K, int N, float clip);
 hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out, size_t count);

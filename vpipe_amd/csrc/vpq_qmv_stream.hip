@@ -274,11 +274,9 @@ hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a)
 
   // K ranges (wavefronts) per tile: the fewest of 1, 2, 4, 8 that still put ~12 wavefronts
   // per CU in the launch; a workgroup is 8 wavefronts = 8 / wpt whole tiles.
-  static const int tune_wpt = getenv("VPQ_TUNE_STREAM_WPT") ? atoi(getenv("VPQ_TUNE_STREAM_WPT")) : 0;
   const long want_units = (long)cus * 12;
   int wpt = 1;
   while (wpt < 8 && wpt < p.slices && (long)p.tiles * wpt < want_units) { wpt *= 2; }
-  if (tune_wpt > 0) { wpt = tune_wpt; }
   if (wpt > p.slices) { wpt = p.slices; }
   if (wpt > 8) { wpt = 8; }
   p.R = (p.slices + wpt - 1) / wpt;
