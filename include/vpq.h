@@ -203,6 +203,51 @@ int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* con
                              const uint16_t* const* scales, const uint16_t* const* biases,
                              const uint16_t* x, uint16_t* const* y, int K, const int* N, int M);
 
+/* ---- fused gate|up projection + SwiGLU -----------------------------------
+ * The MLP of every LM family stores gate and up as ONE pack [N = 2*ffn, K] with
+ * the rows interleaved by output feature (row 2g = gate row g, row 2g+1 = up
+ * row g), built once at load
+ * (generative-models/llama3/metal-llama-model.cc:151-188), so that the
+ * activation fuses into the store and y is the HALVED [M, ffn]:
+ *     y[m, g] = bf16( silu(gate) * up ),  silu(v) = v / (1 + exp(-v)),
+ * evaluated in fp32 on the un-rounded sums, one rounding.
+ *
+ * vpq_interleave_rows builds the interleaved arrays on the device: out row 2i =
+ * a row i, out row 2i+1 = b row i, `rows` rows of `row_bytes` (even) bytes each;
+ * call it for the codes (row_bytes = K/2), the scales and the biases (K/32). */
+int vpq_interleave_rows(vpq_stream_t stream, const void* a, const void* b, void* out,
+                        size_t row_bytes, size_t rows);
+
+/* Replaces `affine_qmv_swiglu_w4g64` (gpu-kernels/metal/quant/affine_qmv.metal:
+ * 816-906; slots 0:w 1:scales 2:biases 3:x 4:y[M,N/2] 5:K 6:N=2*ffn), QMV
+ * arithmetic, 1 <= M <= 16, N even.  `variant` as in vpq_qmv_w4g64_bf16
+ * (VPQ_QMV_STREAM has no such epilogue). */
+int vpq_qmv_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                              int K, int N, int M, int variant);
+
+/* Same, fp32 [M,N/2] output before the final rounding (measurement). */
+int vpq_qmv_swiglu_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, const uint16_t* x, float* y,
+                                int K, int N, int M, int variant);
+
+/* Replaces `affine_qmm_swiglu_w4g64` and its strided twin
+ * (gpu-kernels/metal/quant/affine_qmm_steel.metal:663-768: qmm_t_swiglu_rs_impl;
+ * slots 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N=2*ffn 7:M [8:out_stride 9:out_off]),
+ * QMM arithmetic, any M:  y[m*out_rs + out_off + g] = bf16(silu(gate)*up) with
+ * out_rs = out_stride if > 0, else N/2 (then out_off must be 0). */
+int vpq_qmm_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                              int K, int N, int M, int out_stride, int out_off);
+
+/* The size-based entrance of the fused MLP first half, as the reference's call
+ * sites choose between the two (generative-models/llama3/metal-llama-model.cc:
+ * 466-477 decode, 634-650 and 800-812 prefill): M <= 16 QMV arithmetic, larger
+ * M QMM arithmetic. */
+int vpq_linear_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                 const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                                 int K, int N, int M);
+
 /* ---- a12: the packer ------------------------------------------------------
  * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:
  * 243-301; slots 0:x 1:w 2:s 3:b 4:K 5:N 6:clip) driven by

@@ -145,6 +145,28 @@ def qmm(w, s, b, x, K, N, M, t=None, B=None, r=0):
     return y64, yb
 
 
+def interleave(a, b):
+    """Rows of a and b (same shape, same dtype) alternating: out[2g] = a[g], out[2g+1] = b[g]."""
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    assert a.shape == b.shape and a.dtype == b.dtype
+    out = np.empty((2 * a.shape[0],) + a.shape[1:], dtype=a.dtype)
+    row_bytes = a.strides[0]
+    lib().vpo_interleave_rows(a.ctypes.data_as(ctypes.c_void_p), b.ctypes.data_as(ctypes.c_void_p),
+                              out.ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(row_bytes),
+                              ctypes.c_size_t(a.shape[0]))
+    return out
+
+
+def swiglu(y64):
+    """[M,N] sums of an interleaved gate|up pack -> (out64 [M,N/2], out_bf16 [M,N/2])."""
+    y64 = _c(y64, np.float64)
+    M, N = y64.shape
+    o64 = np.empty((M, N // 2), dtype=np.float64)
+    ob = np.empty((M, N // 2), dtype=np.uint16)
+    lib().vpo_swiglu_pairs(_p(y64, _f64p), _p(o64, _f64p), _p(ob, _u16p), M, N)
+    return o64, ob
+
+
 def quantize(wsrc, K, N, clip=1.0):
     """fp32 [N,K] -> (codes u32 [N,K/8], scales f16 bits [N,K/64], biases f16 bits)."""
     wsrc = _c(wsrc, np.float32)

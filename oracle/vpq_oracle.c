@@ -21,6 +21,9 @@
  *                          procedural inputs and asserted tolerances
  *   lora                   float64 numpy, scale 0 == no adapter, the
  *                          reference's M=96 test shape (reduced) tolerance
+ *   swiglu / interleave    x*expit(x) of scipy, silu(v) - silu(-v) == v, limits;
+ *                          numpy stacking; fused pack == silu(qmv(gate)) * qmv(up)
+ *                          from two separate packs
  *   quantize (packer)      exact recovery of on-grid data, the reference's
  *                          round-trip error bounds, numpy re-derivation
  * Parity that only an Apple-GPU run could pin -- the last-bit effect of the
@@ -306,6 +309,39 @@ void vpo_qmm_w4g64(const uint32_t* w, const uint16_t* scales, const uint16_t* bi
     }
   }
   free(wrow);
+}
+
+/* ---- fused gate|up + SwiGLU --------------------------------------------- */
+
+/* The load-time interleave of two row-major arrays with equal rows,
+ * generative-models/llama3/metal-llama-model.cc:151-188: out row 2g = a row g
+ * (gate), out row 2g+1 = b row g (up); applied alike to codes, scales, biases. */
+void vpo_interleave_rows(const void* a, const void* b, void* out, size_t row_bytes, size_t rows)
+{
+  for (size_t g = 0; g < rows; ++g) {
+    memcpy((char*)out + (2 * g) * row_bytes, (const char*)a + g * row_bytes, row_bytes);
+    memcpy((char*)out + (2 * g + 1) * row_bytes, (const char*)b + g * row_bytes, row_bytes);
+  }
+}
+
+/* The SwiGLU store of the fused gate|up kernels: the sums of an interleaved
+ * [N = 2*ffn, K] pack arrive as y[m, 2g] = gate, y[m, 2g+1] = up and leave as
+ * out[m, g] = T( (gate / (1 + exp(-gate))) * up ), evaluated on the un-rounded
+ * accumulators (gpu-kernels/metal/quant/affine_qmv.metal:882-888 for the GEMV,
+ * affine_qmm_steel.metal:755-766 for the GEMM; the kernels hold fp32 sums, the
+ * oracle applies the same expression to its double sums).  out64 [M,N/2]
+ * double; out_bf16 (nullable) its RNE cast. */
+void vpo_swiglu_pairs(const double* y, double* out64, uint16_t* out_bf16, int M, int N)
+{
+  const int F = N / 2;
+  for (size_t m = 0; m < (size_t)M; ++m) {
+    for (int g = 0; g < F; ++g) {
+      const double ga = y[m * (size_t)N + 2 * g], up = y[m * (size_t)N + 2 * g + 1];
+      const double v = (ga / (1.0 + exp(-ga))) * up;
+      if (out64) { out64[m * (size_t)F + g] = v; }
+      if (out_bf16) { out_bf16[m * (size_t)F + g] = vpo_f32_to_bf16((float)v); }
+    }
+  }
 }
 
 /* ---- a12: the packer --------------------------------------------------- */

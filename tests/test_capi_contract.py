@@ -59,6 +59,14 @@ def test_host_side_validation_and_sizes():
     assert L.vpq_qmv_w4g64_bf16(null, one, one, one, ctypes.c_void_p(4098), one, 64, 8, 1, null, null, 0, 0) == -3
     # LoRA without its scratch
     assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, one, one, 32, 1.0, null) == -4
+    # fused gate|up: odd N, a residual-free epilogue the streaming kernel lacks, a column window
+    # that does not fit its stride, odd row bytes
+    assert L.vpq_qmv_swiglu_w4g64_bf16(null, one, one, one, one, one, 64, 7, 1, 0) == -2
+    assert L.vpq_qmv_swiglu_w4g64_bf16(null, one, one, one, one, one, 64, 8, 1, capi.VPQ_QMV_STREAM) == -2
+    assert L.vpq_qmm_swiglu_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, 6, 4) == -2
+    assert L.vpq_qmm_swiglu_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, 0, 2) == -2
+    assert L.vpq_interleave_rows(null, one, one, one, 3, 4) == -2
+    assert L.vpq_interleave_rows(null, one, null, one, 4, 4) == -1
     assert b"NULL" in L.vpq_status_string(-1)
 
 

@@ -294,3 +294,35 @@ def test_fused_qkv_call_site(enc, oracle, dev, D):
     y64, yb = oracle.qmv(w, s, b, x, K, N, 1)
     got = np.concatenate([D.bits(o) for o in outs], axis=1)
     parity.check_bf16(got, y64, yb)
+
+
+def test_fused_mlp_call_sites(enc, oracle, dev, D):
+    # llama decode (generative-models/llama3/metal-llama-model.cc:466-477): the interleaved gate|up
+    # pack, dispatch {32, ffn/2, 1}; prefill (:634-650): the same pack through affine_qmm_swiglu
+    # with M in slot 7; FLUX.2's strided twin adds out_stride / out_off in slots 8 and 9
+    K, F = 1024, 192
+    gate, up = synth.make_weight(F, K, 60), synth.make_weight(F, K, 61)
+    w, s, b = (oracle.interleave(a, c) for a, c in zip(gate, up))
+    x = synth.make_act(40, K, 62)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    y1 = torch.zeros((1, F), dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_swiglu_w4g64", wd, sd, bd, xd, y1, K, 2 * F,
+                  grid=(32, F // 2, 1))
+    y40 = torch.zeros((40, F), dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, "affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64", wd, sd, bd, xd, y40, K, 2 * F, M=40,
+                  grid=(((2 * F + 31) // 32) * 32, ((40 + 31) // 32) * 2, 2), tg=(32, 2, 2))
+    wide = torch.full((40, 2 * F + 8), 3.0, dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64_rs") == 1
+    for i, t in enumerate((wd, sd, bd, xd, wide)):
+        enc.set_buffer(i, t)
+    for i, v in enumerate((K, 2 * F, 40, 2 * F + 8, F)):
+        enc.set_constant(5 + i, v)
+    enc.dispatch((((2 * F + 31) // 32) * 32, ((40 + 63) // 64) * 2, 2), (32, 2, 2))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    o1, ob1 = oracle.swiglu(oracle.qmv(w, s, b, x[:1], K, 2 * F, 1)[0])
+    parity.check_bf16(D.bits(y1), o1, ob1)
+    o40, ob40 = oracle.swiglu(oracle.qmm(w, s, b, x, K, 2 * F, 40)[0])
+    parity.check_bf16(D.bits(y40), o40, ob40)
+    assert torch.equal(wide[:, F:2 * F], y40)
+    assert (wide[:, :F] == 3.0).all().item() and (wide[:, 2 * F:] == 3.0).all().item()

@@ -341,3 +341,54 @@ def test_cpu_baseline_is_the_same_algorithm(oracle):
     got = synth.bf16_bits_to_f32(y).astype(np.float64)
     assert np.abs(got - y64).max() <= 2.0 ** -7 * np.abs(y64).max()
     assert (y != yb).mean() < 0.05
+
+
+# ---- fused gate|up + SwiGLU -------------------------------------------------------
+
+def test_swiglu_expression_against_scipy_and_identities(oracle):
+    from scipy.special import expit
+    rng = np.random.default_rng(5)
+    y = rng.normal(size=(4, 64)) * 4.0
+    y[0, :8] = [0.0, 3.0, 50.0, 2.0, -50.0, 2.0, 1.0, 0.0]     # gate 0, +large, -large; up 0
+    o64, ob = oracle.swiglu(y)
+    gate, up = y[:, 0::2], y[:, 1::2]
+    assert np.allclose(o64, gate * expit(gate) * up, rtol=1e-14, atol=1e-300)
+    # silu(0) = 0; silu(v) -> v for large v; silu(-large) -> 0; up = 0 -> 0
+    assert o64[0, 0] == 0.0 and abs(o64[0, 1] - 100.0) < 1e-12 and abs(o64[0, 2]) < 1e-18 and o64[0, 3] == 0.0
+    # silu(v) - silu(-v) == v: pairs (v, 1) and (-v, 1)
+    v = rng.normal(size=32) * 3
+    pair = np.stack([np.stack([v, np.ones_like(v)], 1).ravel(), np.stack([-v, np.ones_like(v)], 1).ravel()])
+    o2, _ = oracle.swiglu(pair)
+    assert np.allclose(o2[0] - o2[1], v, rtol=0, atol=1e-15)
+    # gate and up are not interchangeable: the even column is the gate
+    swapped = y.reshape(4, 32, 2)[:, :, ::-1].reshape(4, 64)
+    assert not np.allclose(oracle.swiglu(swapped)[0], o64)
+    assert np.array_equal(ob, oracle.f32_to_bf16(o64.astype(np.float32)))
+
+
+def test_interleave_is_row_alternation(oracle):
+    rng = np.random.default_rng(6)
+    for dt, cols in ((np.uint32, 24), (np.uint16, 3), (np.uint16, 1)):
+        a = rng.integers(0, 60000, size=(7, cols)).astype(dt)
+        b = rng.integers(0, 60000, size=(7, cols)).astype(dt)
+        out = oracle.interleave(a, b)
+        assert np.array_equal(out, np.stack([a, b], axis=1).reshape(14, cols))
+        assert np.array_equal(out[0::2], a) and np.array_equal(out[1::2], b)
+
+
+def test_fused_pack_equals_two_separate_packs(oracle):
+    # the interleave is a permutation, not a different computation
+    # (tests/unit-tests/minimax-h3-blocks.cc:807-846): the fused pack's sums are the two packs' sums
+    K, F, M = 512, 24, 3
+    gw, gs, gb = synth.make_weight(F, K, 41)
+    uw, us, ub = synth.make_weight(F, K, 42)
+    x = synth.make_act(M, K, 43)
+    w, s, b = oracle.interleave(gw, uw), oracle.interleave(gs, us), oracle.interleave(gb, ub)
+    for fn in (oracle.qmv, oracle.qmm):
+        y, _ = fn(w, s, b, x, K, 2 * F, M)
+        g, _ = fn(gw, gs, gb, x, K, F, M)
+        u, _ = fn(uw, us, ub, x, K, F, M)
+        assert np.array_equal(y[:, 0::2], g) and np.array_equal(y[:, 1::2], u)
+        o64, _ = oracle.swiglu(y)
+        assert np.allclose(o64, g / (1.0 + np.exp(-g)) * u, rtol=1e-14)
+

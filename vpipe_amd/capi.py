@@ -34,6 +34,11 @@ SYMBOLS = [
     ("vpq_lora_a_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f]),
     ("vpq_linear_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz]),
     ("vpq_qmv_group_w4g64_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
+    ("vpq_interleave_rows", _i, [_vp, _vp, _vp, _vp, _sz, _sz]),
+    ("vpq_qmv_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_qmv_swiglu_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_qmm_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
+    ("vpq_linear_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     ("vpq_quantize_w4g64", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
     ("vpq_f16_to_bf16", _i, [_vp, _vp, _vp, _sz]),
     ("vpq_profile_enable", _i, [_i]),
@@ -116,6 +121,55 @@ def qmv_w4g64(w, scales, biases, x, K, N, M, out=None, residual=None, ws=None, v
         out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
     _check(L.vpq_qmv_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
                                 K, N, M, _ptr(residual), _ptr(ws), ws_bytes, variant), "vpq_qmv_w4g64_bf16")
+    return out
+
+
+def interleave_gate_up(gate, up):
+    """(w, scales, biases) of gate and of up, each [ffn, ...] -> the interleaved pack [2*ffn, ...]."""
+    import torch
+    outs = []
+    for a, b in zip(gate, up):
+        assert a.shape == b.shape and a.dtype == b.dtype and a.is_contiguous() and b.is_contiguous()
+        out = torch.empty((2 * a.shape[0],) + tuple(a.shape[1:]), dtype=a.dtype, device=a.device)
+        row_bytes = a.stride(0) * a.element_size()
+        _check(load().vpq_interleave_rows(_stream(), _ptr(a), _ptr(b), _ptr(out), row_bytes, a.shape[0]),
+               "vpq_interleave_rows")
+        outs.append(out)
+    return tuple(outs)
+
+
+def qmv_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None, variant=0, f32out=False):
+    """y [M, N/2] = silu(gate) * up over an interleaved gate|up pack [N, K]."""
+    import torch
+    L = load()
+    if f32out:
+        if out is None:
+            out = torch.empty((M, N // 2), dtype=torch.float32, device=w.device)
+        _check(L.vpq_qmv_swiglu_w4g64_f32out(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                             K, N, M, variant), "vpq_qmv_swiglu_w4g64_f32out")
+        return out
+    if out is None:
+        out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=w.device)
+    _check(L.vpq_qmv_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                       K, N, M, variant), "vpq_qmv_swiglu_w4g64_bf16")
+    return out
+
+
+def qmm_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None, out_stride=0, out_off=0):
+    import torch
+    if out is None:
+        out = torch.empty((M, out_stride if out_stride > 0 else N // 2), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                            K, N, M, out_stride, out_off), "vpq_qmm_swiglu_w4g64_bf16")
+    return out
+
+
+def linear_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_linear_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                               K, N, M), "vpq_linear_swiglu_w4g64_bf16")
     return out
 
 

@@ -131,4 +131,40 @@ hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out,
   return launch_kernel(f16_to_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, in, out, count);
 }
 
+// The load-time gate|up interleave of generative-models/llama3/metal-llama-model.cc:151-188 (done
+// there by memcpy on unified memory): out row 2i = a row i, out row 2i+1 = b row i.  One unit
+// (a dword, or a halfword where a scale row is not a multiple of 4 bytes) per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void interleave_rows_kernel(const T* __restrict__ a, const T* __restrict__ b,
+                                                              T* __restrict__ out, size_t row_units,
+                                                              size_t total_units)
+{
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total_units; i += (size_t)gridDim.x * 256) {
+    const size_t orow = i / row_units, col = i - orow * row_units;
+    const T* src = (orow & 1) ? b : a;
+    out[i] = src[(orow >> 1) * row_units + col];
+  }
+}
+
+template <typename T>
+static hipError_t interleave_as(hipStream_t st, const void* a, const void* b, void* out, size_t row_bytes, size_t rows)
+{
+  const size_t row_units = row_bytes / sizeof(T), total = 2 * rows * row_units;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) { blocks = 65536; }
+  if (blocks == 0) { return hipSuccess; }
+  return launch_kernel(interleave_rows_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, st,
+                       reinterpret_cast<const T*>(a), reinterpret_cast<const T*>(b), reinterpret_cast<T*>(out),
+                       row_units, total);
+}
+
+hipError_t launch_interleave_rows(hipStream_t st, const void* a, const void* b, void* out, size_t row_bytes,
+                                  size_t rows)
+{
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+                         reinterpret_cast<uintptr_t>(out) | row_bytes;
+  return (bits & 3) == 0 ? interleave_as<uint32_t>(st, a, b, out, row_bytes, rows)
+                         : interleave_as<uint16_t>(st, a, b, out, row_bytes, rows);
+}
+
 }  // namespace vpq

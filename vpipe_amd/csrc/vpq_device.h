@@ -57,6 +57,20 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
   return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
 
+// SwiGLU of one (gate, up) pair of fp32 sums: silu(gate) * up with silu(g) = g / (1 + exp(-g)),
+// the store expression of gpu-kernels/metal/quant/affine_qmv.metal:882-888 and
+// affine_qmm_steel.metal:755-766.
+__device__ __forceinline__ float swiglu_f32(float gate, float up)
+{
+  return (gate / (1.0f + __expf(-gate))) * up;
+}
+
+// The value lane^1 holds (quad_perm [1,0,3,2]).
+__device__ __forceinline__ float from_neighbour_lane(float v)
+{
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
+}
+
 // Sum over the 64 lanes of a wavefront; every lane receives the total.
 __device__ __forceinline__ float wave_sum(float v)
 {

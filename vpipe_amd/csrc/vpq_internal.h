@@ -50,6 +50,9 @@ struct QmvArgs {
   void* ws;                  // split-K scratch (nullable)
   size_t ws_bytes;
   int cu_count;
+  // The pack is an interleaved gate|up matrix (row 2g gate, 2g+1 up; N even) and y is
+  // [M, N/2] = silu(gate) * up.  No residual with it.
+  bool swiglu = false;
 };
 
 struct GemmArgs {
@@ -63,6 +66,10 @@ struct GemmArgs {
   const uint16_t* lora_b;    // nullable, [N,r]
   int r;
   int cu_count;
+  // Interleaved gate|up pack, y[m * out_stride + out_off + g] = silu(gate) * up, g < N/2.
+  bool swiglu = false;
+  int out_stride = 0;
+  int out_off = 0;
 };
 
 hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* scales,
@@ -104,5 +111,8 @@ int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16
 hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
                            uint16_t* b_f16, int K, int N, float clip);
 hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out, size_t count);
+// out row 2i = a row i, out row 2i+1 = b row i; rows of row_bytes (a multiple of 2) bytes.
+hipError_t launch_interleave_rows(hipStream_t st, const void* a, const void* b, void* out, size_t row_bytes,
+                                  size_t rows);
 
 }  // namespace vpq

@@ -6,6 +6,9 @@
 // Arithmetic: W[n,k] = fma(s, q, b) in fp32 (never rounded to bf16),
 // acc += x * W in fp32, wave reduction, one bf16 rounding on store -- the
 // semantics of gpu-kernels/metal/quant/affine_qmv.metal:151-174, 228-283.
+// With `swiglu` the rows are an interleaved gate|up pack: wavefronts 2j and 2j+1 of a
+// workgroup hold a feature's gate and up sums, the odd one hands its sum over through LDS and
+// the even one stores silu(gate) * up into y[M, N/2] (affine_qmv.metal:816-906).
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -15,12 +18,14 @@ template <int MT, bool F32OUT>
 __global__ __launch_bounds__(256) void qmv_simple_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x, void* __restrict__ y,
-    const uint16_t* __restrict__ residual, int K, int N, int M)
+    const uint16_t* __restrict__ residual, int K, int N, int M, int swiglu)
 {
+  __shared__ float up_sum[4][MT];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
-  const int n = blockIdx.x * 4 + wave;
-  if (n >= N) { return; }  // wave-uniform
+  const int n_raw = blockIdx.x * 4 + wave;
+  const bool live = n_raw < N;            // wave-uniform
+  const int n = live ? n_raw : N - 1;     // idle wavefronts redo the last row and store nothing
   const int Kw = K >> 3, Kg = K >> 6;
   const uint32_t* wrow = w + (size_t)n * Kw;
   const uint16_t* srow = scales + (size_t)n * Kg;
@@ -54,11 +59,38 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
         }
       }
     }
+    if (swiglu) {
+      float total[MT];
+#pragma unroll
+      for (int mm = 0; mm < MT; ++mm) { total[mm] = wave_sum(acc[mm]); }
+      if ((wave & 1) && lane == 0) {
+#pragma unroll
+        for (int mm = 0; mm < MT; ++mm) { up_sum[wave][mm] = total[mm]; }
+      }
+      __syncthreads();
+      if (!(wave & 1) && lane == 0 && live) {
+#pragma unroll
+        for (int mm = 0; mm < MT; ++mm) {
+          const int row = m0 + mm;
+          if (row < M) {
+            const float v = swiglu_f32(total[mm], up_sum[wave + 1][mm]);
+            const size_t o = (size_t)row * (N >> 1) + (n >> 1);
+            if (F32OUT) {
+              reinterpret_cast<float*>(y)[o] = v;
+            } else {
+              reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)f32_to_bf16_bits(v);
+            }
+          }
+        }
+      }
+      __syncthreads();   // up_sum is rewritten by the next batch of rows
+      continue;
+    }
 #pragma unroll
     for (int mm = 0; mm < MT; ++mm) {
       const float total = wave_sum(acc[mm]);
       const int row = m0 + mm;
-      if (lane == 0 && row < M) {
+      if (lane == 0 && row < M && live) {
         const size_t o = (size_t)row * N + n;
         if (F32OUT) {
           reinterpret_cast<float*>(y)[o] = total;
@@ -79,7 +111,7 @@ hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a)
   const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
 #define VPQ_LAUNCH(MT, F32)                                                                    \
   launch_kernel(qmv_simple_kernel<MT, F32>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
-                a.residual, a.K, a.N, a.M)
+                a.residual, a.K, a.N, a.M, a.swiglu ? 1 : 0)
   if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH(1, true) : VPQ_LAUNCH(1, false); }
   return a.y_f32 ? VPQ_LAUNCH(4, true) : VPQ_LAUNCH(4, false);
 #undef VPQ_LAUNCH

@@ -75,6 +75,8 @@ enum class QuantKernel : std::uint8_t {
   Qmm,            // affine_qmm_steel_w4g64[_bm64|_bm128], affine_qmm_mma_w4g64    slot 7 = M
   QmvQkv,         // affine_qmv_qkv_w4g64: row-concatenated q|k|v pack, slots 4,5,6 = q,k,v outputs,
                   //   7 = K, 8,9,10 = q_rows, k_rows, v_rows (v_rows == 0: q|k only); one launch
+  QmvSwiglu,      // affine_qmv_swiglu_w4g64: interleaved gate|up pack, N = 2*ffn, y [M, ffn]; M from grid.x / 32
+  QmmSwiglu,      // affine_qmm_swiglu_w4g64[_bm64|_bm128|_bm64_rs]: slot 7 = M, 8 = out_stride, 9 = out_off (_rs)
 };
 
 class QuantFunction {
