@@ -394,6 +394,46 @@ def main():
             del w, s, b, x, y, A, B, t
         out["qmm_dit_m16320_lora_r32"] = dit
 
+    # ---- fused gate|up + SwiGLU (interleaved pack), as context ------------------------------
+    if not args.no_extras:
+        fused = []
+        for li in range(args.layers):
+            fused.append(vpipe_amd.interleave_gate_up(layers[li][4], layers[li][5]))
+        y_mlp = torch.empty((1, 12288), dtype=torch.bfloat16, device=dev)
+
+        def pass_fused_mlp(li):
+            """q|k|v grouped, o, gate|up + SwiGLU as one launch over the interleaved pack, down."""
+            group(li, (0, 1, 2))
+            project(li, 3)
+            w, s, b = fused[li]
+            vpipe_amd.qmv_swiglu_w4g64(w, s, b, xs[4096], 4096, 24576, 1, out=y_mlp)
+            project(li, 6)
+
+        for i in range(args.layers):
+            pass_fused_mlp(i)
+        torch.cuda.synchronize()
+        ms_f = time_steps(pass_fused_mlp, args.steps, use_graph)
+        fm = {"us_per_layer": round(ms_f * 1e3, 3), "GBps": round((layer_bytes - 2 * 12288) / (ms_f * 1e-3) / 1e9, 1),
+              "launches_per_layer": 4}
+        M = 2048
+        w, s, b = fused[0]
+        x = torch.randn((M, 4096), device=dev, generator=gen).bfloat16()
+        y = torch.empty((M, 12288), dtype=torch.bfloat16, device=dev)
+        for _ in range(3):
+            vpipe_amd.qmm_swiglu_w4g64(w, s, b, x, 4096, 24576, M, out=y)
+        torch.cuda.synchronize()
+        L.vpq_profile_enable(10)
+        for _ in range(10):
+            vpipe_amd.qmm_swiglu_w4g64(w, s, b, x, 4096, 24576, M, out=y)
+        kb = (ctypes.c_float * 10)()
+        n = L.vpq_profile_read(kb, 10)
+        L.vpq_profile_enable(0)
+        us = float(np.mean(kb[:n])) * 1e3
+        fm["qmm_swiglu_m2048_4096->2x12288"] = {"us": round(us, 2),
+                                               "TFLOPs": round(2.0 * M * 24576 * 4096 / (us * 1e-6) / 1e12, 1)}
+        out["fused_mlp_swiglu"] = fm
+        del fused, x, y
+
     # ---- CPU baseline: the oracle's dequant + fp32 matmul on the host cores ------------
     if not args.no_cpu:
         from oracle import oracle
