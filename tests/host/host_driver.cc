@@ -2,11 +2,14 @@
 // the Python tests can write quantized-linear call sites in the reference's encoder protocol
 // (set_function / set_buffer / set_constant / dispatch / fence) and check them against the oracle.
 // Not part of the product; built next to this file.
+#include <algorithm>
 #include <cstring>
+#include <optional>
 #include <string>
 #include <vector>
 
 #include "vpq_host.h"
+#include "vpq_weights.h"
 
 using namespace vpipe_amd;
 
@@ -112,6 +115,100 @@ void hd_quant_linear(void* h, void* codes, void* scales, void* qbias, int K, int
   } else {
     quant_linear_forward(s->stream, lin, bx, 0, by, 0, M);
   }
+}
+
+// ---- checkpoint container (vpq_weights.h) ---------------------------------------------------
+
+void* hw_open(const char* dir, unsigned long long shard_max_bytes)
+{
+  return new PackWriter(dir, shard_max_bytes);
+}
+
+int hw_add(void* h, const char* name, const char* dtype, const long long* shape, int ndim, const void* data,
+           unsigned long long nbytes)
+{
+  std::vector<std::int64_t> shp(shape, shape + ndim);
+  return static_cast<PackWriter*>(h)->add(name, dtype, shp, data, nbytes) ? 1 : 0;
+}
+
+// Closes and frees the writer; 1 if every shard and the index were written.
+int hw_close(void* h)
+{
+  PackWriter* w = static_cast<PackWriter*>(h);
+  const bool ok = w->close();
+  delete w;
+  return ok ? 1 : 0;
+}
+
+static std::string g_why;
+const char* hr_why(void) { return g_why.c_str(); }
+
+void* hr_open(const char* path, int model_dir)
+{
+  g_why.clear();
+  std::optional<PackFile> f = model_dir ? PackFile::open_model(path, &g_why) : PackFile::open(path, &g_why);
+  if (!f) { return nullptr; }
+  return new PackFile(std::move(*f));
+}
+
+void hr_close(void* h) { delete static_cast<PackFile*>(h); }
+
+int hr_count(void* h) { return (int)static_cast<PackFile*>(h)->tensor_names().size(); }
+
+// Name of the i-th tensor (sorted) into buf.
+int hr_name(void* h, int i, char* buf, int cap)
+{
+  std::vector<std::string> names = static_cast<PackFile*>(h)->tensor_names();
+  std::sort(names.begin(), names.end());
+  if (i < 0 || i >= (int)names.size() || (int)names[i].size() + 1 > cap) { return 0; }
+  std::memcpy(buf, names[i].c_str(), names[i].size() + 1);
+  return 1;
+}
+
+// dtype into dtype_buf (16 bytes), up to 8 dims into shape; out = {ndim, nbytes, offset, shard}.
+int hr_info(void* h, const char* name, char* dtype_buf, long long* shape, unsigned long long* out)
+{
+  const TensorInfo* ti = static_cast<PackFile*>(h)->info(name);
+  if (ti == nullptr || ti->shape.size() > 8 || ti->dtype.size() > 15) { return 0; }
+  std::memcpy(dtype_buf, ti->dtype.c_str(), ti->dtype.size() + 1);
+  for (std::size_t i = 0; i < ti->shape.size(); ++i) { shape[i] = ti->shape[i]; }
+  out[0] = ti->shape.size(); out[1] = ti->nbytes; out[2] = ti->offset; out[3] = (unsigned long long)ti->shard;
+  return 1;
+}
+
+int hr_read(void* h, const char* name, void* dst, unsigned long long cap)
+{
+  return static_cast<PackFile*>(h)->read_into(name, dst, cap) ? 1 : 0;
+}
+
+void hr_alignment(void* h, long long* out4)
+{
+  const PackFile::Alignment a = static_cast<PackFile*>(h)->alignment();
+  out4[0] = (long long)a.tensors; out4[1] = (long long)a.misaligned; out4[2] = a.shards; out4[3] = a.bad_shards;
+}
+
+int hr_bits(void* h, const char* prefix, int K) { return static_cast<PackFile*>(h)->affine_bits(prefix, K); }
+int hr_group(void* h, const char* prefix, int K) { return static_cast<PackFile*>(h)->affine_group(prefix, K); }
+
+// Quantizes a bf16 [N,K] device tensor and appends `<prefix>.weight/.scales/.biases` to the writer.
+int hd_quantize_and_add(void* session, void* writer, const char* prefix, void* src_bf16, int K, int N, float clip)
+{
+  Session* s = static_cast<Session*>(session);
+  DeviceBuffer src = DeviceBuffer::wrap(src_bf16, (size_t)N * K * 2);
+  return quantize_and_add(s->stream, *static_cast<PackWriter*>(writer), prefix, src, K, N, clip, &g_why) ? 1 : 0;
+}
+
+// Loads one Linear from the reader and runs y[M,N] = x . W^T through quant_linear_forward.
+// out_kn receives {K, N}.  The loaded buffers live until the call returns (it waits).
+int hd_load_and_run(void* session, void* reader, const char* prefix, int K, void* x, void* y, int M, int* out_kn)
+{
+  Session* s = static_cast<Session*>(session);
+  LoadedLinear lin;
+  if (!static_cast<PackFile*>(reader)->load_linear(s->stream, prefix, K, &lin, &g_why)) { return 0; }
+  out_kn[0] = lin.K; out_kn[1] = lin.N;
+  DeviceBuffer bx = DeviceBuffer::wrap(x, (size_t)M * lin.K * 2), by = DeviceBuffer::wrap(y, (size_t)M * lin.N * 2);
+  quant_linear_forward(s->stream, lin.view(), bx, 0, by, 0, M);
+  return s->stream.commit().wait_ok(&g_why) ? 1 : 0;
 }
 
 }  // extern "C"

@@ -326,3 +326,52 @@ def test_fused_mlp_call_sites(enc, oracle, dev, D):
     parity.check_bf16(D.bits(y40), o40, ob40)
     assert torch.equal(wide[:, F:2 * F], y40)
     assert (wide[:, :F] == 3.0).all().item() and (wide[:, 2 * F:] == 3.0).all().item()
+
+
+@pytest.mark.parametrize("M", [1, 40])
+def test_quantize_write_read_load_run(enc, oracle, dev, D, tmp_path, M):
+    # the producer and the consumer of the on-disk pack: a bf16 weight is quantized on the device and
+    # written as `<prefix>.weight/.scales/.biases` (U32 / F16 / F16), the directory is opened again,
+    # the Linear is loaded (scales and zero points converted F16 -> bf16 on the device, once) and run
+    import safetensors.numpy as stnp
+    L = enc.L
+    L.hw_open.restype = ctypes.c_void_p
+    L.hw_open.argtypes = [ctypes.c_char_p, ctypes.c_ulonglong]
+    L.hw_close.argtypes = [ctypes.c_void_p]
+    L.hr_open.restype = ctypes.c_void_p
+    L.hr_open.argtypes = [ctypes.c_char_p, ctypes.c_int]
+    L.hr_close.argtypes = [ctypes.c_void_p]
+    L.hr_why.restype = ctypes.c_char_p
+    L.hd_quantize_and_add.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_int,
+                                      ctypes.c_int, ctypes.c_float]
+    L.hd_load_and_run.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_void_p,
+                                  ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]
+    K, N = 1024, 96
+    rng = np.random.default_rng(70 + M)
+    src_bits = synth.f32_to_bf16_bits((rng.standard_normal((N, K)) * 0.05).astype(np.float32))
+    src = D.bf16(src_bits, dev)
+    x = synth.make_act(M, K, 71)
+    xd = D.bf16(x, dev)
+    torch.cuda.synchronize()
+    w = L.hw_open(str(tmp_path).encode(), 1 << 30)
+    prefix = b"model.layers.0.mlp.down_proj"
+    assert L.hd_quantize_and_add(enc.h, w, prefix, src.data_ptr(), K, N, 1.0) == 1, L.hr_why()
+    assert L.hw_close(w) == 1
+    # what is on disk is the oracle's packer output, bit for bit, readable by the format's own library
+    codes, s16, b16 = oracle.quantize(synth.bf16_bits_to_f32(src_bits), K, N)
+    disk = stnp.load_file(str(tmp_path / "model-00001-of-00001.safetensors"))
+    assert np.array_equal(disk[prefix.decode() + ".weight"], codes)
+    assert np.array_equal(disk[prefix.decode() + ".scales"].view(np.uint16), s16)
+    assert np.array_equal(disk[prefix.decode() + ".biases"].view(np.uint16), b16)
+    r = L.hr_open(str(tmp_path).encode(), 1)
+    assert r, L.hr_why()
+    yd = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    kn = (ctypes.c_int * 2)()
+    assert L.hd_load_and_run(enc.h, r, prefix, 0, xd.data_ptr(), yd.data_ptr(), M, kn) == 1, L.hr_why()
+    assert tuple(kn) == (K, N)
+    assert L.hd_load_and_run(enc.h, r, b"model.layers.1.mlp.down_proj", 0, xd.data_ptr(), yd.data_ptr(), M, kn) == 0
+    assert L.hd_load_and_run(enc.h, r, prefix, 2048, xd.data_ptr(), yd.data_ptr(), M, kn) == 0    # a 2-bit reading
+    L.hr_close(r)
+    sb, bb = oracle.f16_to_bf16(s16), oracle.f16_to_bf16(b16)
+    y64, yb = (oracle.qmv if M <= 16 else oracle.qmm)(codes, sb, bb, x, K, N, M)
+    parity.check_bf16(D.bits(yd), y64, yb)

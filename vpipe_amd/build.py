@@ -64,7 +64,7 @@ def _host_cc(args):
 def build_host():
     """The C++ host layer (no device code) and, when the tests are present, their C driver over it."""
     inc = ["-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(HERE, "host")]
-    _host_cc(inc + [os.path.join(HERE, "host", "vpq_host.cc"), "-o", HOST_OUT, "-L" + HERE, "-lvpq",
+    _host_cc(inc + [os.path.join(HERE, "host", "vpq_host.cc"), os.path.join(HERE, "host", "vpq_weights.cc"), "-o", HOST_OUT, "-L" + HERE, "-lvpq",
                     "-Wl,-rpath,$ORIGIN"])
     if os.path.exists(DRIVER_SRC):
         _host_cc(inc + [DRIVER_SRC, "-o", DRIVER_OUT, "-L" + HERE, "-lvpq_host", "-lvpq",
