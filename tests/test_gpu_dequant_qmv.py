@@ -95,6 +95,8 @@ RING_SHAPES = STREAM_SHAPES + [
     # one to five slices per wavefront
     (512, 16, 16), (1024, 40, 5), (2048, 33, 8), (4096, 16 * 1030 + 7, 4), (5120, 16 * 600, 9), (20480, 72, 16),
     (4096, 16 * 2100 + 3, 1), (12288, 16 * 700 + 9, 3),
+    # many tiles per workgroup with x in registers: 12 at 6 rows, the cap of 8 at 12 rows
+    (1024, 16 * 3000, 6), (512, 16 * 2100 + 5, 12),
 ]
 
 

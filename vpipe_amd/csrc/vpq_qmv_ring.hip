@@ -52,7 +52,9 @@ constexpr int kSlotBytes = kCodeBytes + 1024;    // + one 64-lane load of scales
 constexpr int kItemLoads = 5;            // direct-to-LDS loads per item
 constexpr int kXLoads = 4;               // direct-to-LDS loads per slice of x (M <= 4)
 constexpr int kXBytes = kXLoads * 1024;  // staged rows of one slice of x
-constexpr int kMaxTcMr = 4;              // TC * MR <= 4 bounds the LDS table of partial sums
+// TC * MR is bounded by the LDS table of partial sums: 8 KB beside the staged x of M <= 4,
+// 64 KB where x lives in registers (more tiles per workgroup = fewer reloads of x).
+constexpr int max_tc_mr(int mr) { return mr == 1 ? 4 : 32; }
 
 struct RingParams {
   const uint32_t* w;
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(const RingParams p)
   __shared__ __attribute__((aligned(16))) uint8_t ring0[NW * kSlotBytes];
   __shared__ __attribute__((aligned(16))) uint8_t ring1[NW * kSlotBytes];
   __shared__ __attribute__((aligned(16))) uint8_t xstage[XDMA ? NW * kXBytes : 16];
-  __shared__ float sums[kMaxTcMr * NW * kWave];      // [tile][wave][register][lane]
+  __shared__ float sums[max_tc_mr(MR) * NW * kWave];  // [tile][wave][register][lane]
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -358,13 +360,13 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(const RingParams p)
   }
   __syncthreads();
 
-  // Thread t of the first TC*MR*64 adds, in wavefront order, the partial sums of one
-  // (tile, register, lane) and stores y[m = 4*register + lane/16][tile*16 + lane%16].
-  const int tid = threadIdx.x;
-  if (tid < TC * MR * kWave) {
-    const int t = tid / (MR * kWave);
-    const int q = (tid / kWave) % MR;
-    const int l = tid & 63;
+  // The TC*MR*64 outputs are dealt to the threads one wavefront's worth at a time: each adds, in
+  // wavefront order, the partial sums of one (tile, register, lane) and stores
+  // y[m = 4*register + lane/16][tile*16 + lane%16].
+  for (int o_idx = threadIdx.x; o_idx < TC * MR * kWave; o_idx += NW * kWave) {
+    const int t = o_idx / (MR * kWave);
+    const int q = (o_idx / kWave) % MR;
+    const int l = o_idx & 63;
     const int live = p.slices < NW ? p.slices : NW;
     float total = 0.0f;
     for (int wv = 0; wv < live; ++wv) { total += sums[((t * NW + wv) * MR + q) * kWave + l]; }
@@ -434,7 +436,7 @@ hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw
   p.tiles = (a.N + kTileN - 1) / kTileN;
   int mr = (a.M + 3) / 4;
   if (mr == 3) { mr = 4; }
-  const int tc_max = kMaxTcMr / mr;
+  const int tc_max = max_tc_mr(mr) / mr;
   // Enough tiles per workgroup that one workgroup per CU covers the matrix in one pass.
   const int cus = a.cu_count > 0 ? a.cu_count : 256;
   int tc = (p.tiles + cus - 1) / cus;
