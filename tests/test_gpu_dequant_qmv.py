@@ -97,6 +97,8 @@ RING_SHAPES = STREAM_SHAPES + [
     (4096, 16 * 2100 + 3, 1), (12288, 16 * 700 + 9, 3),
     # many tiles per workgroup with x in registers: 12 at 6 rows, the cap of 8 at 12 rows
     (1024, 16 * 3000, 6), (512, 16 * 2100 + 5, 12),
+    # 3 and 4 rows over a wide matrix take the two-register form
+    (1024, 16 * 1400 + 2, 3), (512, 16 * 1300, 4),
 ]
 
 

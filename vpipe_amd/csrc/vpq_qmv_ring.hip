@@ -436,10 +436,13 @@ hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw
   p.tiles = (a.N + kTileN - 1) / kTileN;
   int mr = (a.M + 3) / 4;
   if (mr == 3) { mr = 4; }
-  const int tc_max = max_tc_mr(mr) / mr;
   // Enough tiles per workgroup that one workgroup per CU covers the matrix in one pass.
   const int cus = a.cu_count > 0 ? a.cu_count : 256;
   int tc = (p.tiles + cus - 1) / cus;
+  // 3 or 4 rows over a wide matrix: the two-register form takes more tiles per workgroup than
+  // the staged-x form has room for, which is worth more than its idle accumulator register.
+  if (mr == 1 && a.M >= 3 && tc > max_tc_mr(1)) { mr = 2; }
+  const int tc_max = max_tc_mr(mr) / mr;
   if (tc_hint > 0) { tc = tc_hint; }
   if (tc > tc_max) { tc = tc_max; }
   if (tc < 1) { tc = 1; }
