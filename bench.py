@@ -69,6 +69,9 @@ def main():
     ap.add_argument("--only", action="store_true",
                     help="run nothing but the selected launch mode of the decode-layer set (for a profiler: every "
                          "QMV launch in the trace then belongs to the timed workload)")
+    ap.add_argument("--only-qmm", action="store_true",
+                    help="run nothing but the fused QMM kernel on the three M=2048 projections and print their "
+                         "timings (for a profiler: every qmm_tile_kernel dispatch then belongs to that workload)")
     ap.add_argument("--no-extras", action="store_true", help="skip the small-batch QMV and video-DiT QMM sections")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -96,6 +99,27 @@ def main():
     st = L.vpq_init()
     if st != 0:
         raise vpipe_amd.VpqError(st, "vpq_init")
+
+    if args.only_qmm:
+        M, res = 2048, {}
+        for name, K, N in PREFILL:
+            w, s, b = make_weight(torch, N, K, dev, gen)
+            x = torch.randn((M, K), device=dev, generator=gen).bfloat16()
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            for _ in range(3):
+                vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y)
+            torch.cuda.synchronize()
+            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0.record()
+            for _ in range(10):
+                vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y)
+            t1.record()
+            torch.cuda.synchronize()
+            us = t0.elapsed_time(t1) * 1e3 / 10
+            res[name] = {"K": K, "N": N, "M": M, "us": round(us, 2),
+                         "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 1)}
+        print(json.dumps({"qmm_m2048_fused_kernel_only": res}))
+        return
 
     # ---- inputs, resident in HBM ------------------------------------------------
     layers = []
