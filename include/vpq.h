@@ -123,7 +123,7 @@ enum {
   VPQ_QMV_MFMA = 2,        /* LDS-staged codes, bf16 MFMA on the integer codes */
   VPQ_QMV_MFMA_SPLITK = 3, /* as 2, K split across workgroups through `ws` */
   VPQ_QMV_STREAM = 4,      /* M <= 4: persistent workgroups, x staged in LDS, prefetched items */
-  VPQ_QMV_RING = 5         /* x in registers, codes through a two-slot LDS ring per wavefront */
+  VPQ_QMV_RING = 5         /* x in registers across a workgroup's tiles, codes through a two-slot LDS ring per wavefront */
 };
 
 /* ---- a6/a7/a8 (+a10): QMM ----------------------------------------------
