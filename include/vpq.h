@@ -83,6 +83,18 @@ int vpq_device_cu_count(void);
 int vpq_dequant_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                            const uint16_t* biases, uint16_t* w_deq, int K, int N);
 
+/* Dequantizing embedding gather over the same pack (a tied lm_head / embedding
+ * table).  Replaces `dequant_embed_gather_f16`
+ * (gpu-kernels/metal/ops/llm_elementwise.metal:1676-1701; slots 0:ids 1:w 2:scales
+ * 3:biases 4:out 5:H, grid (H, T, 1)): out[t, :] = bf16_rne(fp32(s*q + b)) of table
+ * row ids[t], bit-identical to that row of vpq_dequant_w4g64_bf16.  `ids` is a
+ * device array of T int32; the table is [vocab, H].  A row whose id is outside
+ * [0, vocab) is filled with zeros (the reference reads out of bounds there).
+ * Requires H % 64 == 0, T > 0; out 16-byte aligned. */
+int vpq_embed_gather_w4g64_bf16(vpq_stream_t stream, const int32_t* ids, const uint32_t* w,
+                                const uint16_t* scales, const uint16_t* biases, uint16_t* out,
+                                int H, int T, int vocab);
+
 /* ---- a2/a3/a4: QMV, 1 <= M <= 16 ---------------------------------------
  * Replaces `affine_qmv_w4g64` (gpu-kernels/metal/quant/affine_qmv.metal:286-301;
  * slots 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N), its `_add` twin (:347-363,

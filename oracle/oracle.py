@@ -107,6 +107,16 @@ def dequant_f32(w, s, b, K, N):
     return out
 
 
+def embed_gather(ids, w, s, b, H, vocab):
+    """ids int32 [T] -> bf16 bits [T, H]: dequantized rows of the [vocab, H] table."""
+    ids = _c(ids, np.int32)
+    w, s, b = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16)
+    out = np.empty((ids.size, H), dtype=np.uint16)
+    lib().vpo_embed_gather_w4g64_bf16(ids.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), _p(w, _u32p), _p(s, _u16p),
+                                      _p(b, _u16p), _p(out, _u16p), H, ids.size, vocab)
+    return out
+
+
 def qmv(w, s, b, x, K, N, M, residual=None):
     """-> (y64 [M,N] float64, y_bf16 [M,N] uint16); un-rounded-weight semantics."""
     w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)

@@ -177,6 +177,29 @@ void vpo_dequant_w4g64_bf16(const uint32_t* w, const uint16_t* scales, const uin
   }
 }
 
+/* Dequantizing embedding gather, gpu-kernels/metal/ops/llm_elementwise.metal:1676-1701:
+ * out[t, h] = T(s * q + b) of table row ids[t] -- the dequant expression above applied
+ * to the selected rows.  Rows with an id outside [0, vocab) are zero-filled here
+ * (the reference does not check). */
+void vpo_embed_gather_w4g64_bf16(const int32_t* ids, const uint32_t* w, const uint16_t* scales,
+                                 const uint16_t* biases, uint16_t* out, int H, int T, int vocab)
+{
+  const int Hw = H / 8, Hg = H / VPO_GROUP;
+  for (size_t t = 0; t < (size_t)T; ++t) {
+    const int id = ids[t];
+    for (int h = 0; h < H; ++h) {
+      uint16_t v = 0;
+      if (id >= 0 && id < vocab) {
+        const float s = vpo_bf16_to_f32(scales[(size_t)id * Hg + h / VPO_GROUP]);
+        const float b = vpo_bf16_to_f32(biases[(size_t)id * Hg + h / VPO_GROUP]);
+        const float sq = s * (float)nibble(w, (size_t)id, Hw, h);
+        v = vpo_f32_to_bf16(sq + b);
+      }
+      out[t * (size_t)H + h] = v;
+    }
+  }
+}
+
 /* ---- a2/a3: QMV -------------------------------------------------------- */
 
 /* The CPU reference loop of the reference's own QMV test,

@@ -67,6 +67,8 @@ def test_host_side_validation_and_sizes():
     assert L.vpq_qmm_swiglu_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, 0, 2) == -2
     assert L.vpq_interleave_rows(null, one, one, one, 3, 4) == -2
     assert L.vpq_interleave_rows(null, one, null, one, 4, 4) == -1
+    assert L.vpq_embed_gather_w4g64_bf16(null, null, one, one, one, one, 64, 1, 8) == -1
+    assert L.vpq_embed_gather_w4g64_bf16(null, one, one, one, one, one, 64, 0, 8) == -2
     assert b"NULL" in L.vpq_status_string(-1)
 
 

@@ -55,6 +55,24 @@ def test_dequant_every_code_against_every_scale(vpq, oracle, dev, D):
     assert np.array_equal(got[finite], want[finite])
 
 
+@pytest.mark.parametrize("vocab,H,T", [(37, 192, 8), (1000, 4096, 1), (151936, 1024, 300)])
+def test_embed_gather_rows_are_bit_exact(vpq, oracle, dev, D, vocab, H, T):
+    # dequant_embed_gather (gpu-kernels/metal/ops/llm_elementwise.metal:1676-1701): a gathered row
+    # is that row of the dense table, bit for bit; ids outside the table give zero rows
+    w, s, b = synth.make_weight(vocab, H, 400 + H)
+    rng = np.random.default_rng(T)
+    ids = rng.integers(0, vocab, size=T).astype(np.int32)
+    ids[0], ids[-1] = vocab - 1, 0
+    if T >= 8:
+        ids[3], ids[4] = -1, vocab
+    wd, sd, bd = stage(D, dev, w, s, b)
+    out = parity.Guarded((T, H), torch.bfloat16, dev)
+    vpq.embed_gather_w4g64(torch.from_numpy(ids).to(dev), wd, sd, bd, H, vocab, out=out.view)
+    torch.cuda.synchronize()
+    assert np.array_equal(D.bits(out.view), oracle.embed_gather(ids, w, s, b, H, vocab))
+    out.assert_intact()
+
+
 # ---- a2/a3/a4: QMV --------------------------------------------------------------
 
 SMALL = [

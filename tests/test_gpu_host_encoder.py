@@ -375,3 +375,23 @@ def test_quantize_write_read_load_run(enc, oracle, dev, D, tmp_path, M):
     sb, bb = oracle.f16_to_bf16(s16), oracle.f16_to_bf16(b16)
     y64, yb = (oracle.qmv if M <= 16 else oracle.qmm)(codes, sb, bb, x, K, N, M)
     parity.check_bf16(D.bits(yd), y64, yb)
+
+
+def test_embedding_gather_call_site(enc, oracle, dev, D):
+    # llama decode (generative-models/llama3/metal-llama-model.cc:82): slots 0:ids 1:w 2:scales 3:biases
+    # 4:out 5:H, grid (H, T, 1); the table is the (tied) lm_head pack
+    vocab, H, T = 500, 1024, 6
+    w, s, b = synth.make_weight(vocab, H, 80)
+    ids = np.array([3, 499, 0, 77, 77, 250], dtype=np.int32)
+    idd = torch.from_numpy(ids).to(dev)
+    wd, sd, bd = D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev)
+    out = torch.zeros((T, H), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("llm_elementwise_bf16", "dequant_embed_gather_f16") == 1
+    for i, t in enumerate((idd, wd, sd, bd, out)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, H)
+    enc.dispatch((H, T, 1), (256, 1, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert np.array_equal(D.bits(out), oracle.embed_gather(ids, w, s, b, H, vocab))
+

@@ -392,3 +392,14 @@ def test_fused_pack_equals_two_separate_packs(oracle):
         o64, _ = oracle.swiglu(y)
         assert np.allclose(o64, g / (1.0 + np.exp(-g)) * u, rtol=1e-14)
 
+
+def test_embed_gather_is_row_selection_of_the_dense_table(oracle):
+    vocab, H = 37, 192
+    w, s, b = synth.make_weight(vocab, H, 90)
+    dense = oracle.dequant_bf16(w, s, b, H, vocab)
+    ids = np.array([0, 36, 5, 5, 17, -1, 37, 2], dtype=np.int32)
+    got = oracle.embed_gather(ids, w, s, b, H, vocab)
+    ok = (ids >= 0) & (ids < vocab)
+    assert np.array_equal(got[ok], dense[ids[ok]])
+    assert not got[~ok].any()
+

@@ -26,6 +26,7 @@ SYMBOLS = [
     ("vpq_init", _i, []),
     ("vpq_device_cu_count", _i, []),
     ("vpq_dequant_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_embed_gather_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
     ("vpq_qmv_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _i]),
     ("vpq_qmv_workspace_bytes", _sz, [_i, _i, _i]),
@@ -104,6 +105,17 @@ def dequant_w4g64(w, scales, biases, K, N, out=None):
         out = torch.empty((N, K), dtype=torch.bfloat16, device=w.device)
     _check(load().vpq_dequant_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out), K, N),
            "vpq_dequant_w4g64_bf16")
+    return out
+
+
+def embed_gather_w4g64(ids, w, scales, biases, H, vocab, out=None):
+    """ids: int32 device tensor [T] -> bf16 [T, H], rows of the dequantized table."""
+    import torch
+    T = ids.numel()
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_embed_gather_w4g64_bf16(_stream(), _ptr(ids), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out),
+                                              H, T, vocab), "vpq_embed_gather_w4g64_bf16")
     return out
 
 

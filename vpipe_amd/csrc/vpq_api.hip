@@ -179,6 +179,19 @@ int vpq_dequant_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_
   return finish(vpq::launch_dequant(reinterpret_cast<hipStream_t>(stream), w, scales, biases, w_deq, K, N));
 }
 
+int vpq_embed_gather_w4g64_bf16(vpq_stream_t stream, const int32_t* ids, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, uint16_t* out, int H, int T, int vocab)
+{
+  int st = check_pack(w, scales, biases, H, vocab);
+  if (st != VPQ_OK) { return st; }
+  if (ids == nullptr || out == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (T <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(ids, 4) || !aligned(out, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_embed_gather(reinterpret_cast<hipStream_t>(stream), ids, w, scales, biases, out, H, T, vocab));
+}
+
 int vpq_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                        const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                        const uint16_t* residual, void* ws, size_t ws_bytes, int variant)

@@ -45,6 +45,49 @@ hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* sca
                        biases, reinterpret_cast<uint4*>(out), Kw, total);
 }
 
+// Dequantizing embedding gather (gpu-kernels/metal/ops/llm_elementwise.metal:1676-1701): out row t
+// is the dense expansion of table row ids[t]; the arithmetic is the dequant kernel's, so a
+// gathered row is bit-identical to that row of the dense table.  One thread per packed word.
+// A row whose id is outside [0, vocab) is filled with zeros.
+__global__ __launch_bounds__(256) void embed_gather_w4g64_kernel(
+    const int* __restrict__ ids, const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
+    const uint16_t* __restrict__ biases, uint4* __restrict__ out, int Hw, int vocab, size_t total_words)
+{
+  const int Hg = Hw >> 3;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total_words; idx += (size_t)gridDim.x * 256) {
+    const size_t t = idx / (size_t)Hw;
+    const int j = (int)(idx - t * (size_t)Hw);
+    const int id = ids[t];
+    uint4 o = make_uint4(0, 0, 0, 0);
+    if (id >= 0 && id < vocab) {
+      const size_t g = (size_t)id * (size_t)Hg + (size_t)(j >> 3);
+      const float s = bf16_bits_to_f32(scales[g]);
+      const float b = bf16_bits_to_f32(biases[g]);
+      const uint32_t p = w[(size_t)id * (size_t)Hw + (size_t)j];
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { v[i] = fmaf(s, (float)((p >> (4 * i)) & 0xfu), b); }
+      o.x = pack_bf16x2(v[0], v[1]);
+      o.y = pack_bf16x2(v[2], v[3]);
+      o.z = pack_bf16x2(v[4], v[5]);
+      o.w = pack_bf16x2(v[6], v[7]);
+    }
+    out[idx] = o;
+  }
+}
+
+hipError_t launch_embed_gather(hipStream_t st, const int* ids, const uint32_t* w, const uint16_t* scales,
+                               const uint16_t* biases, uint16_t* out, int H, int T, int vocab)
+{
+  const int Hw = H / 8;
+  const size_t total = (size_t)T * (size_t)Hw;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536 * 4) { blocks = 65536 * 4; }
+  if (blocks == 0) { return hipSuccess; }
+  return launch_kernel(embed_gather_w4g64_kernel, dim3((unsigned)blocks), dim3(256), 0, st, ids, w, scales, biases,
+                       reinterpret_cast<uint4*>(out), Hw, vocab, total);
+}
+
 // One thread per 64-wide group, as the reference's packer
 // (gpu-kernels/metal/quant/affine_dequant.metal:243-285): min/max, optional
 // clip toward the midpoint, scale = (mx-mn)/15, q = clamp(round((v-mn)/scale)),

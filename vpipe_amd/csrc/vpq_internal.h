@@ -74,6 +74,9 @@ struct GemmArgs {
 
 hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, uint16_t* out, int K, int N);
+// out[t, :] = dense expansion of table row ids[t] (zeros for an id outside [0, vocab)).
+hipError_t launch_embed_gather(hipStream_t st, const int* ids, const uint32_t* w, const uint16_t* scales,
+                               const uint16_t* biases, uint16_t* out, int H, int T, int vocab);
 hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a);
 // Returns hipErrorInvalidValue if the shape is outside what the MFMA kernel
 // handles (the caller then falls back to the simple kernel).

@@ -87,6 +87,7 @@ const FnEntry kFunctions[] = {
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm128", QuantKernel::Qmm},
     {"affine_qmm_mma_bf16", "affine_qmm_mma_w4g64", QuantKernel::Qmm},
     {"affine_qmv_bf16", "affine_qmv_swiglu_w4g64", QuantKernel::QmvSwiglu},
+    {"llm_elementwise_bf16", "dequant_embed_gather_f16", QuantKernel::EmbedGather},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm128", QuantKernel::QmmSwiglu},
@@ -269,6 +270,7 @@ void ComputeEncoder::set_buffer(unsigned index, const DeviceBuffer& buf, std::si
     return;
   }
   _slots[index].ptr = static_cast<char*>(buf.data()) + byte_offset;
+  _slots[index].bytes = buf.size() - byte_offset;
   _slots[index].is_buffer = true;
   _slots[index].is_const = false;
 }
@@ -354,6 +356,21 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
     } else {
       status = vpq_dequant_w4g64_bf16(st, static_cast<const uint32_t*>(buf(0)), static_cast<const uint16_t*>(buf(1)),
                                       static_cast<const uint16_t*>(buf(2)), static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
+    }
+  } else if (kind == QuantKernel::EmbedGather) {
+    // gpu-kernels/metal/ops/llm_elementwise.metal:1676-1701: slots 0:ids 1:w 2:scales 3:biases 4:out 5:H,
+    // grid (H, T, 1).  The table's row count is not a slot: it is what the code buffer holds.
+    if (!buf(0) || !buf(1) || !buf(2) || !buf(3) || !buf(4) || !has_int(5)) {
+      status = VPQ_ERR_NULL_POINTER;
+    } else if (ival(5) <= 0 || ival(5) % 64 != 0) {
+      status = VPQ_ERR_BAD_SHAPE;
+    } else {
+      const int H = ival(5);
+      const std::size_t rows = _slots[1].bytes / (static_cast<std::size_t>(H) / 2);
+      const int vocab = rows > 0x7fffffffu ? 0x7fffffff : static_cast<int>(rows);
+      status = vpq_embed_gather_w4g64_bf16(st, static_cast<const int32_t*>(buf(0)), static_cast<const uint32_t*>(buf(1)),
+                                           static_cast<const uint16_t*>(buf(2)), static_cast<const uint16_t*>(buf(3)),
+                                           static_cast<uint16_t*>(buf(4)), H, static_cast<int>(grid.y), vocab);
     }
   } else if (kind == QuantKernel::QmvQkv) {
     // gpu-kernels/metal/quant/affine_qmv.metal:497-516: slots 0:w 1:scales 2:biases 3:x 4:q_out

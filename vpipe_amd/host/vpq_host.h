@@ -77,6 +77,8 @@ enum class QuantKernel : std::uint8_t {
                   //   7 = K, 8,9,10 = q_rows, k_rows, v_rows (v_rows == 0: q|k only); one launch
   QmvSwiglu,      // affine_qmv_swiglu_w4g64: interleaved gate|up pack, N = 2*ffn, y [M, ffn]; M from grid.x / 32
   QmmSwiglu,      // affine_qmm_swiglu_w4g64[_bm64|_bm128|_bm64_rs]: slot 7 = M, 8 = out_stride, 9 = out_off (_rs)
+  EmbedGather,    // dequant_embed_gather_f16: slots 0:ids 1:w 2:scales 3:biases 4:out 5:H; T = grid.y,
+                  //   the vocabulary size is what the bound code buffer holds
 };
 
 class QuantFunction {
@@ -94,7 +96,8 @@ private:
 
 // The reference groups its kernels in metallibs loaded by name; the bf16 twins
 // are the ones this path implements ("affine_qmv_bf16", "affine_qmm_steel_bf16",
-// "affine_qmm_mma_bf16", "affine_dequant_bf16").  Any other name gives an empty library.
+// "affine_qmm_mma_bf16", "affine_dequant_bf16", and "llm_elementwise_bf16" for the dequantizing
+// embedding gather).  Any other name gives an empty library.
 class QuantLibrary {
 public:
   QuantLibrary() noexcept = default;
@@ -167,6 +170,7 @@ private:
   static constexpr unsigned kSlots = 12;
   struct Slot {
     void* ptr = nullptr;
+    std::size_t bytes = 0;       // bytes from ptr to the end of the bound buffer
     bool is_buffer = false;
     bool is_const = false;
     std::int64_t ivalue = 0;
