@@ -260,6 +260,27 @@ int vpq_linear_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const u
                                  const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                  int K, int N, int M);
 
+/* The same fused stores with the activation chosen by the caller: VPQ_GATE_SWIGLU
+ * as above, VPQ_GATE_GEGLU = gelu_tanh(gate) * up with
+ * gelu_tanh(g) = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), which replaces
+ * `affine_qmv_geglu_w4g64` (gpu-kernels/metal/quant/affine_qmv.metal:1352-1447)
+ * and `affine_qmm_geglu_w4g64` (affine_qmm_steel.metal:1460-1572); pack layout,
+ * shapes and requirements as for the SwiGLU entries, which are these with
+ * activation = VPQ_GATE_SWIGLU. */
+enum { VPQ_GATE_SWIGLU = 1, VPQ_GATE_GEGLU = 2 };
+int vpq_qmv_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                             int K, int N, int M, int variant, int activation);
+int vpq_qmv_gated_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                               const uint16_t* biases, const uint16_t* x, float* y,
+                               int K, int N, int M, int variant, int activation);
+int vpq_qmm_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                             int K, int N, int M, int out_stride, int out_off, int activation);
+int vpq_linear_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                                int K, int N, int M, int activation);
+
 /* ---- a12: the packer ------------------------------------------------------
  * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:
  * 243-301; slots 0:x 1:w 2:s 3:b 4:K 5:N 6:clip) driven by

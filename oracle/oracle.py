@@ -177,6 +177,16 @@ def swiglu(y64):
     return o64, ob
 
 
+def geglu(y64):
+    """[M,N] sums of an interleaved gate|up pack -> (out64 [M,N/2], out_bf16): gelu_tanh(gate) * up."""
+    y64 = _c(y64, np.float64)
+    M, N = y64.shape
+    o64 = np.empty((M, N // 2), dtype=np.float64)
+    ob = np.empty((M, N // 2), dtype=np.uint16)
+    lib().vpo_geglu_pairs(_p(y64, _f64p), _p(o64, _f64p), _p(ob, _u16p), M, N)
+    return o64, ob
+
+
 def quantize(wsrc, K, N, clip=1.0):
     """fp32 [N,K] -> (codes u32 [N,K/8], scales f16 bits [N,K/64], biases f16 bits)."""
     wsrc = _c(wsrc, np.float32)

@@ -367,6 +367,25 @@ void vpo_swiglu_pairs(const double* y, double* out64, uint16_t* out_bf16, int M,
   }
 }
 
+/* The GEGLU twin of vpo_swiglu_pairs: out[m, g] = T(0.5 * gate * (1 + tanh(k0 * (gate +
+ * 0.044715 * gate^3))) * up), k0 = sqrt(2/pi) as the reference writes it
+ * (gpu-kernels/metal/quant/affine_qmv.metal:1423-1429, affine_qmm_steel.metal:1541-1544);
+ * evaluated in double on the double sums. */
+void vpo_geglu_pairs(const double* y, double* out64, uint16_t* out_bf16, int M, int N)
+{
+  const int F = N / 2;
+  const double k0 = 0.7978845608028654;
+  for (size_t m = 0; m < (size_t)M; ++m) {
+    for (int g = 0; g < F; ++g) {
+      const double ga = y[m * (size_t)N + 2 * g], up = y[m * (size_t)N + 2 * g + 1];
+      const double t = tanh(k0 * (ga + 0.044715 * ga * ga * ga));
+      const double v = 0.5 * ga * (1.0 + t) * up;
+      if (out64) { out64[m * (size_t)F + g] = v; }
+      if (out_bf16) { out_bf16[m * (size_t)F + g] = vpo_f32_to_bf16((float)v); }
+    }
+  }
+}
+
 /* ---- a12: the packer --------------------------------------------------- */
 
 /* gpu-kernels/metal/quant/affine_dequant.metal:243-285 (affine_quant_impl<4,64>):

@@ -55,7 +55,7 @@ def bf16_ulp(v):
     return 2.0 ** (e - 7)
 
 
-def check_bf16(got_bits, ref64, ref_bits=None):
+def check_bf16(got_bits, ref64, ref_bits=None, mismatch_over_all=True):
     """bf16 output = (fp32 result within the floored 2e-3 of the oracle) rounded once:
     |got - ref| <= 2e-3 * max(|ref|, 1e-2 rms) + one bf16 step at |ref|.  Where the
     output is not tiny against the rms this is the same as `within one bf16 ulp of
@@ -71,7 +71,10 @@ def check_bf16(got_bits, ref64, ref_bits=None):
     d = bf16_ulp_distance(got_bits, ref_bits)
     big = np.abs(ref64) >= 0.05 * rms
     assert d[big].max(initial=0) <= 1, "bf16 output differs by %d ulp on a non-tiny element" % d[big].max()
-    mismatch = float((d != 0).mean())
+    # mismatch_over_all=False: the rate is taken over the non-tiny elements only (for outputs whose
+    # near-zero values are fp32 noise by construction)
+    counted = d if mismatch_over_all else d[big]
+    mismatch = float((counted != 0).mean()) if counted.size else 0.0
     assert mismatch <= 0.02, "bf16 output differs from bf16(oracle) on %.2f%% of elements" % (100 * mismatch)
     r = rel_l2(got, ref64)
     assert r <= REL_L2_TOL, "rel-L2 %.3e" % r

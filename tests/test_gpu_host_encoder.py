@@ -326,6 +326,18 @@ def test_fused_mlp_call_sites(enc, oracle, dev, D):
     parity.check_bf16(D.bits(y40), o40, ob40)
     assert torch.equal(wide[:, F:2 * F], y40)
     assert (wide[:, :F] == 3.0).all().item() and (wide[:, 2 * F:] == 3.0).all().item()
+    # Gemma's twin of the same call site: gelu_tanh(gate) * up
+    yg = torch.zeros((1, F), dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_geglu_w4g64", wd, sd, bd, xd, yg, K, 2 * F, grid=(32, F // 2, 1))
+    yg40 = torch.zeros((40, F), dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, "affine_qmm_steel_bf16", "affine_qmm_geglu_w4g64", wd, sd, bd, xd, yg40, K, 2 * F, M=40,
+                  grid=(((2 * F + 31) // 32) * 32, ((40 + 31) // 32) * 2, 2), tg=(32, 2, 2))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    g1, gb1 = oracle.geglu(oracle.qmv(w, s, b, x[:1], K, 2 * F, 1)[0])
+    parity.check_bf16(D.bits(yg), g1, gb1, mismatch_over_all=False)
+    g40, gb40 = oracle.geglu(oracle.qmm(w, s, b, x, K, 2 * F, 40)[0])
+    parity.check_bf16(D.bits(yg40), g40, gb40, mismatch_over_all=False)
 
 
 @pytest.mark.parametrize("M", [1, 40])

@@ -190,3 +190,48 @@ def test_qmm_swiglu_prefill_shape_sampled(vpq, oracle, dev, D):
     o64, ob = oracle.swiglu(oracle.qmm(w[sel], s[sel], b[sel], x[rows], K, len(sel), len(rows))[0])
     got = D.bits(out.view[torch.from_numpy(rows).to(dev)][:, torch.from_numpy(feats).to(dev)])
     parity.check_bf16(got, o64, ob)
+
+
+# 1 + tanh(z) cancels for gates below about -3: evaluated in fp32, as the reference writes it, the
+# product there is noise around a value of order 1e-6 of the rms (the float64 oracle gives the true
+# tiny value), so which side of a bf16 boundary it lands on is arbitrary.  Those outputs are bounded by
+# the absolute-error check; the mismatch rate is taken over the outputs that are not tiny.
+
+
+@pytest.mark.parametrize("variant", [SIMPLE, MFMA, RING, AUTO])
+@pytest.mark.parametrize("K,F,M", [(512, 17, 4), (2048, 80, 5), (4096, 47, 8), (2560, 32, 16), (8192, 264, 1)])
+def test_qmv_geglu(vpq, oracle, dev, D, K, F, M, variant):
+    # affine_qmv_geglu_w4g64 (gpu-kernels/metal/quant/affine_qmv.metal:1352-1447): the same fused pack,
+    # gelu_tanh(gate) * up
+    _, _, pack = fused_pack(oracle, F, K, 2500 + K + F)
+    x = synth.make_act(M, K, 2600 + K + M)
+    o64, ob = oracle.geglu(oracle.qmv(*pack, x, K, 2 * F, M)[0])
+    wd, sd, bd, xd = stage(D, dev, pack, x)
+    f = vpq.qmv_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, variant=variant, f32out=True, activation=capi.VPQ_GATE_GEGLU)
+    out = parity.Guarded((M, F), torch.bfloat16, dev)
+    vpq.qmv_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, out=out.view, variant=variant, activation=capi.VPQ_GATE_GEGLU)
+    torch.cuda.synchronize()
+    parity.check_f32(f.cpu().numpy(), o64)
+    parity.check_bf16(D.bits(out.view), o64, ob, mismatch_over_all=False)
+    out.assert_intact()
+
+
+@pytest.mark.parametrize("M,F,K", [(64, 64, 64), (130, 160, 256), (257, 65, 512), (300, 192, 2048), (9, 48, 1024)])
+def test_qmm_and_linear_geglu(vpq, oracle, dev, D, M, F, K):
+    _, _, pack = fused_pack(oracle, F, K, 2700 + M + F)
+    x = synth.make_act(M, K, 2800 + M + K)
+    wd, sd, bd, xd = stage(D, dev, pack, x)
+    o64, ob = oracle.geglu(oracle.qmm(*pack, x, K, 2 * F, M)[0])
+    out = parity.Guarded((M, F), torch.bfloat16, dev)
+    vpq.qmm_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, out=out.view, activation=capi.VPQ_GATE_GEGLU)
+    torch.cuda.synchronize()
+    parity.check_bf16(D.bits(out.view), o64, ob, mismatch_over_all=False)
+    out.assert_intact()
+    # the size-based entrance takes the GEMV arithmetic up to 16 rows
+    arith = oracle.qmv if M <= 16 else oracle.qmm
+    l64, lb = oracle.geglu(arith(*pack, x, K, 2 * F, M)[0])
+    got = vpq.linear_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, activation=capi.VPQ_GATE_GEGLU)
+    parity.check_bf16(D.bits(got), l64, lb, mismatch_over_all=False)
+    with pytest.raises(capi.VpqError):
+        vpq.qmm_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, activation=3)
+

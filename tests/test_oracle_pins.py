@@ -403,3 +403,17 @@ def test_embed_gather_is_row_selection_of_the_dense_table(oracle):
     assert np.array_equal(got[ok], dense[ids[ok]])
     assert not got[~ok].any()
 
+
+def test_geglu_expression_against_torch_gelu_tanh(oracle):
+    rng = np.random.default_rng(8)
+    y = rng.normal(size=(3, 40)) * 3.0
+    y[0, :6] = [0.0, 2.0, 30.0, 2.0, -30.0, 2.0]
+    o64, ob = oracle.geglu(y)
+    gate, up = torch.from_numpy(y[:, 0::2].copy()), torch.from_numpy(y[:, 1::2].copy())
+    want = (torch.nn.functional.gelu(gate, approximate="tanh") * up).numpy()
+    assert np.allclose(o64, want, rtol=1e-12, atol=1e-300)
+    assert o64[0, 0] == 0.0 and abs(o64[0, 1] - 60.0) < 1e-9 and abs(o64[0, 2]) < 1e-12
+    # not the sigmoid gate: the two activations differ by a few percent at |g| ~ 1
+    assert not np.allclose(o64, oracle.swiglu(y)[0], rtol=1e-2)
+    assert np.array_equal(ob, oracle.f32_to_bf16(o64.astype(np.float32)))
+

@@ -15,6 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libvpq.so")
 _lib = None
 
+VPQ_GATE_SWIGLU, VPQ_GATE_GEGLU = 1, 2
 VPQ_QMV_AUTO, VPQ_QMV_SIMPLE, VPQ_QMV_MFMA, VPQ_QMV_MFMA_SPLITK, VPQ_QMV_STREAM, VPQ_QMV_RING = 0, 1, 2, 3, 4, 5
 
 # Every symbol include/vpq.h declares: (name, restype, argtypes).
@@ -40,6 +41,10 @@ SYMBOLS = [
     ("vpq_qmv_swiglu_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     ("vpq_linear_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_qmv_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
+    ("vpq_qmv_gated_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
+    ("vpq_qmm_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
+    ("vpq_linear_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_quantize_w4g64", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
     ("vpq_f16_to_bf16", _i, [_vp, _vp, _vp, _sz]),
     ("vpq_profile_enable", _i, [_i]),
@@ -150,38 +155,55 @@ def interleave_gate_up(gate, up):
     return tuple(outs)
 
 
-def qmv_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None, variant=0, f32out=False):
-    """y [M, N/2] = silu(gate) * up over an interleaved gate|up pack [N, K]."""
+def qmv_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None, variant=0, f32out=False, activation=VPQ_GATE_SWIGLU):
+    """y [M, N/2] = act(gate) * up over an interleaved gate|up pack [N, K] (SwiGLU unless `activation` says GEGLU)."""
     import torch
     L = load()
     if f32out:
         if out is None:
             out = torch.empty((M, N // 2), dtype=torch.float32, device=w.device)
-        _check(L.vpq_qmv_swiglu_w4g64_f32out(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
-                                             K, N, M, variant), "vpq_qmv_swiglu_w4g64_f32out")
+        if activation == VPQ_GATE_SWIGLU:
+            st = L.vpq_qmv_swiglu_w4g64_f32out(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M, variant)
+        else:
+            st = L.vpq_qmv_gated_w4g64_f32out(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                              variant, activation)
+        _check(st, "vpq_qmv_gated_w4g64_f32out")
         return out
     if out is None:
         out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=w.device)
-    _check(L.vpq_qmv_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
-                                       K, N, M, variant), "vpq_qmv_swiglu_w4g64_bf16")
+    if activation == VPQ_GATE_SWIGLU:
+        st = L.vpq_qmv_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M, variant)
+    else:
+        st = L.vpq_qmv_gated_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M, variant,
+                                        activation)
+    _check(st, "vpq_qmv_gated_w4g64_bf16")
     return out
 
 
-def qmm_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None, out_stride=0, out_off=0):
+def qmm_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None, out_stride=0, out_off=0, activation=VPQ_GATE_SWIGLU):
     import torch
     if out is None:
         out = torch.empty((M, out_stride if out_stride > 0 else N // 2), dtype=torch.bfloat16, device=w.device)
-    _check(load().vpq_qmm_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
-                                            K, N, M, out_stride, out_off), "vpq_qmm_swiglu_w4g64_bf16")
+    if activation == VPQ_GATE_SWIGLU:
+        st = load().vpq_qmm_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                              out_stride, out_off)
+    else:
+        st = load().vpq_qmm_gated_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                             out_stride, out_off, activation)
+    _check(st, "vpq_qmm_gated_w4g64_bf16")
     return out
 
 
-def linear_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None):
+def linear_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None, activation=VPQ_GATE_SWIGLU):
     import torch
     if out is None:
         out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=w.device)
-    _check(load().vpq_linear_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
-                                               K, N, M), "vpq_linear_swiglu_w4g64_bf16")
+    if activation == VPQ_GATE_SWIGLU:
+        st = load().vpq_linear_swiglu_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M)
+    else:
+        st = load().vpq_linear_gated_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                                activation)
+    _check(st, "vpq_linear_gated_w4g64_bf16")
     return out
 
 

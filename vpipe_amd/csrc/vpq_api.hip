@@ -77,13 +77,14 @@ int check_pack(const uint32_t* w, const uint16_t* scales, const uint16_t* biases
 
 int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                const uint16_t* biases, const uint16_t* x, void* y, bool y_f32, int K, int N, int M,
-               const uint16_t* residual, void* ws, size_t ws_bytes, int variant, bool swiglu = false)
+               const uint16_t* residual, void* ws, size_t ws_bytes, int variant, int gate_act = 0)
 {
   int st = check_pack(w, scales, biases, K, N);
   if (st != VPQ_OK) { return st; }
   if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
   if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
-  if (swiglu && ((N & 1) != 0 || residual != nullptr || variant == VPQ_QMV_STREAM)) { return VPQ_ERR_BAD_SHAPE; }
+  if (gate_act != 0 && gate_act != VPQ_GATE_SWIGLU && gate_act != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (gate_act != 0 && ((N & 1) != 0 || residual != nullptr || variant == VPQ_QMV_STREAM)) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
   if (ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }
@@ -95,7 +96,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y; a.residual = residual;
   a.K = K; a.N = N; a.M = M; a.y_f32 = y_f32; a.ws = ws; a.ws_bytes = ws_bytes;
   a.cu_count = g_dev.cu_count;
-  a.swiglu = swiglu;
+  a.gate_act = gate_act;
   hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
 
   const bool mfma_ok = vpq::qmv_mfma_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
@@ -117,7 +118,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
     }
     return finish(vpq::launch_qmv_mfma(hs, a, 1));
   }
-  const bool stream_ok = mfma_ok && !swiglu && vpq::qmv_stream_supports(K, N, M);
+  const bool stream_ok = mfma_ok && gate_act == 0 && vpq::qmv_stream_supports(K, N, M);
   if (variant == VPQ_QMV_STREAM) {
     if (!stream_ok) { return VPQ_ERR_BAD_SHAPE; }
     return finish(vpq::launch_qmv_stream(hs, a));
@@ -304,27 +305,30 @@ int vpq_interleave_rows(vpq_stream_t stream, const void* a, const void* b, void*
   return finish(vpq::launch_interleave_rows(reinterpret_cast<hipStream_t>(stream), a, b, out, row_bytes, rows));
 }
 
-int vpq_qmv_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
-                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
-                              int variant)
+int vpq_qmv_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                             int variant, int activation)
 {
-  return qmv_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, nullptr, 0, variant, true);
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return qmv_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, nullptr, 0, variant, activation);
 }
 
-int vpq_qmv_swiglu_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
-                                const uint16_t* biases, const uint16_t* x, float* y, int K, int N, int M,
-                                int variant)
+int vpq_qmv_gated_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                               const uint16_t* biases, const uint16_t* x, float* y, int K, int N, int M,
+                               int variant, int activation)
 {
-  return qmv_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr, nullptr, 0, variant, true);
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return qmv_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr, nullptr, 0, variant, activation);
 }
 
-int vpq_qmm_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
-                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
-                              int out_stride, int out_off)
+int vpq_qmm_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                             int out_stride, int out_off, int activation)
 {
   int st = check_pack(w, scales, biases, K, N);
   if (st != VPQ_OK) { return st; }
   if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
   if (M <= 0 || (N & 1) != 0 || out_off < 0) { return VPQ_ERR_BAD_SHAPE; }
   if (out_stride > 0 && out_off + N / 2 > out_stride) { return VPQ_ERR_BAD_SHAPE; }
   if (out_stride <= 0 && out_off != 0) { return VPQ_ERR_BAD_SHAPE; }
@@ -335,17 +339,47 @@ int vpq_qmm_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint
   g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
   g.K = K; g.N = N; g.M = M;
   g.cu_count = g_dev.cu_count;
-  g.swiglu = true;
+  g.gate_act = activation;
   g.out_stride = out_stride;
   g.out_off = out_off;
   return finish(vpq::launch_qmm_tile(reinterpret_cast<hipStream_t>(stream), g));
 }
 
+int vpq_linear_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                int activation)
+{
+  if (M >= 1 && M <= 16) {
+    return vpq_qmv_gated_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, VPQ_QMV_AUTO, activation);
+  }
+  return vpq_qmm_gated_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, 0, 0, activation);
+}
+
+int vpq_qmv_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                              int variant)
+{
+  return vpq_qmv_gated_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, variant, VPQ_GATE_SWIGLU);
+}
+
+int vpq_qmv_swiglu_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, const uint16_t* x, float* y, int K, int N, int M,
+                                int variant)
+{
+  return vpq_qmv_gated_w4g64_f32out(stream, w, scales, biases, x, y, K, N, M, variant, VPQ_GATE_SWIGLU);
+}
+
+int vpq_qmm_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                              int out_stride, int out_off)
+{
+  return vpq_qmm_gated_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, out_stride, out_off, VPQ_GATE_SWIGLU);
+}
+
 int vpq_linear_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                  const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M)
 {
-  if (M >= 1 && M <= 16) { return vpq_qmv_swiglu_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, VPQ_QMV_AUTO); }
-  return vpq_qmm_swiglu_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, 0, 0);
+  return vpq_linear_gated_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, VPQ_GATE_SWIGLU);
 }
 
 int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,

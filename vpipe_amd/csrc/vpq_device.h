@@ -57,11 +57,19 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
   return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
 
-// SwiGLU of one (gate, up) pair of fp32 sums: silu(gate) * up with silu(g) = g / (1 + exp(-g)),
-// the store expression of gpu-kernels/metal/quant/affine_qmv.metal:882-888 and
-// affine_qmm_steel.metal:755-766.
-__device__ __forceinline__ float swiglu_f32(float gate, float up)
+// Gated activation of one (gate, up) pair of fp32 sums, the store expressions of the fused
+// gate|up kernels:
+//   kGateSwiglu  silu(gate) * up, silu(g) = g / (1 + exp(-g))
+//                (gpu-kernels/metal/quant/affine_qmv.metal:882-888, affine_qmm_steel.metal:755-766)
+//   kGateGeglu   gelu_tanh(gate) * up = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * up
+//                (affine_qmv.metal:1423-1429, affine_qmm_steel.metal:1541-1544)
+constexpr int kGateNone = 0, kGateSwiglu = 1, kGateGeglu = 2;
+__device__ __forceinline__ float gated_f32(int act, float gate, float up)
 {
+  if (act == kGateGeglu) {
+    const float t = tanhf(0.7978845608028654f * (gate + 0.044715f * gate * gate * gate));
+    return 0.5f * gate * (1.0f + t) * up;
+  }
   return (gate / (1.0f + __expf(-gate))) * up;
 }
 

@@ -50,9 +50,9 @@ struct QmvArgs {
   void* ws;                  // split-K scratch (nullable)
   size_t ws_bytes;
   int cu_count;
-  // The pack is an interleaved gate|up matrix (row 2g gate, 2g+1 up; N even) and y is
-  // [M, N/2] = silu(gate) * up.  No residual with it.
-  bool swiglu = false;
+  // Non-zero (1 SwiGLU, 2 GEGLU): the pack is an interleaved gate|up matrix (row 2g gate, 2g+1 up;
+  // N even) and y is [M, N/2] = act(gate) * up.  No residual with it.
+  int gate_act = 0;
 };
 
 struct GemmArgs {
@@ -66,8 +66,9 @@ struct GemmArgs {
   const uint16_t* lora_b;    // nullable, [N,r]
   int r;
   int cu_count;
-  // Interleaved gate|up pack, y[m * out_stride + out_off + g] = silu(gate) * up, g < N/2.
-  bool swiglu = false;
+  // Non-zero (1 SwiGLU, 2 GEGLU): interleaved gate|up pack,
+  // y[m * out_stride + out_off + g] = act(gate) * up, g < N/2.
+  int gate_act = 0;
   int out_stride = 0;
   int out_off = 0;
 };

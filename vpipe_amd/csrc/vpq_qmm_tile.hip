@@ -66,7 +66,7 @@ struct TileParams {
   int tiles_m, tiles_n;
   // SwiGLU store (gpu-kernels/metal/quant/affine_qmm_steel.metal:663-768): the pack is an
   // interleaved gate|up matrix and y[m * out_stride + out_off + g] = silu(gate_g) * up_g.
-  int swiglu, out_stride, out_off;
+  int gate_act, out_stride, out_off;
 };
 
 __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
@@ -352,7 +352,7 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   }
 
   // ---- store: lane holds, for x row m = lane%32 of each it, 4 consecutive n per register quad ----
-  if (p.swiglu) {
+  if (p.gate_act) {
     // A register quad is (gate, up, gate, up) of features n/2 and n/2 + 1 (n is a multiple of 4):
     // the activation is register-local and a quad becomes one dword of two bf16.
     const bool pair_ok = ((p.out_stride | p.out_off) & 1) == 0;
@@ -367,8 +367,8 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
         for (int rq = 0; rq < 4; ++rq) {
           const int n = n0 + wn * 64 + jt * 32 + rq * 8 + fkh * 4;
           if (n >= p.N) { continue; }
-          const float f0 = swiglu_f32(acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
-          const float f1 = swiglu_f32(acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
+          const float f0 = gated_f32(p.gate_act, acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
+          const float f1 = gated_f32(p.gate_act, acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
           if (pair_ok && n + 3 < p.N) {
             *reinterpret_cast<uint32_t*>(yrow + (n >> 1)) = pack_bf16x2(f0, f1);
           } else {
@@ -417,7 +417,7 @@ hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a)
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
   p.lora_t = a.lora_t; p.lora_b = a.lora_b;
   p.K = a.K; p.N = a.N; p.M = a.M; p.r = a.r;
-  p.swiglu = a.swiglu ? 1 : 0;
+  p.gate_act = a.gate_act;
   p.out_stride = a.out_stride > 0 ? a.out_stride : a.N / 2;
   p.out_off = a.out_off;
   p.tiles_m = (a.M + TM - 1) / TM;

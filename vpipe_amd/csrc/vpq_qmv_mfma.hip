@@ -66,7 +66,7 @@ struct QmvParams {
   int wave_lds_bytes;    // codes buffer + staged x rows of one wavefront
   // Grouped launch (nseg > 1): workgroup blockIdx.x belongs to the segment whose tile range
   // holds it; each segment is its own [N_i, K] pack and output.
-  int swiglu;            // rows are interleaved gate|up; y is [M, N/2] = silu(gate) * up
+  int gate_act;          // rows are interleaved gate|up; y is [M, N/2] = act(gate) * up (1 SwiGLU, 2 GEGLU)
   int nseg;
   QmvSeg seg[4];
   int seg_tile_end[4];
@@ -312,12 +312,12 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
     if (t == 0) { p.counters[blockIdx.x] = 0u; }
   }
 
-  if (p.swiglu) {
+  if (p.gate_act) {
     // Lanes 2j and 2j+1 hold the gate and the up sum of feature (n0 + 2j) / 2; N is even, so both
     // are valid or neither.
     const float up = from_neighbour_lane(total);
     if (valid && (t & 1) == 0) {
-      const float v = swiglu_f32(total, up);
+      const float v = gated_f32(p.gate_act, total, up);
       const size_t o = (size_t)m * (N_ >> 1) + (n >> 1);
       if (F32OUT) {
         reinterpret_cast<float*>(y_)[o] = v;
@@ -385,7 +385,7 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
   p.residual = a.residual;
   p.K = a.K; p.N = a.N; p.M = a.M;
-  p.swiglu = a.swiglu ? 1 : 0;
+  p.gate_act = a.gate_act;
   p.nseg = 1;
   p.slices = a.K / kKS;
 
@@ -445,7 +445,7 @@ hipError_t launch_qmv_mfma_group(hipStream_t st, const QmvArgs& a, const QmvGrou
   p.w = nullptr; p.scales = nullptr; p.biases = nullptr; p.x = a.x; p.y = nullptr;
   p.residual = nullptr;
   p.K = a.K; p.N = 0; p.M = a.M;
-  p.swiglu = 0;
+  p.gate_act = 0;
   p.slices = a.K / kKS;
   p.slices_per_block = p.slices;
   p.split_k = 1;

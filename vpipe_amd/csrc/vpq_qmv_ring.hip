@@ -67,7 +67,7 @@ struct RingParams {
   int slices;   // K / 512
   int tiles;    // ceil(N / 16)
   int tc;       // tiles per workgroup
-  int swiglu;   // rows are interleaved gate|up; y is [M, N/2] = silu(gate) * up
+  int gate_act; // rows are interleaved gate|up; y is [M, N/2] = act(gate) * up (1 SwiGLU, 2 GEGLU)
 };
 
 // Eight nibbles of one packed word -> eight bf16 values 128+q, element order
@@ -373,11 +373,11 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(const RingParams p)
     const int m = 4 * q + (l >> 4);
     const int tile = tile0 + t;
     const int n = tile * kTileN + (l & 15);
-    if (p.swiglu) {
+    if (p.gate_act) {
       // Lanes 2j and 2j+1 hold the gate and the up sum of one feature (N is even).
       const float up = from_neighbour_lane(total);
       if (tile < p.tiles && m < p.M && n < p.N && (l & 1) == 0) {
-        const float v = swiglu_f32(total, up);
+        const float v = gated_f32(p.gate_act, total, up);
         const size_t o = (size_t)m * (p.N >> 1) + (n >> 1);
         if (F32OUT) {
           reinterpret_cast<float*>(p.y)[o] = v;
@@ -431,7 +431,7 @@ hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
   p.residual = a.residual;
   p.K = a.K; p.N = a.N; p.M = a.M;
-  p.swiglu = a.swiglu ? 1 : 0;
+  p.gate_act = a.gate_act;
   p.slices = a.K / kKS;
   p.tiles = (a.N + kTileN - 1) / kTileN;
   int mr = (a.M + 3) / 4;

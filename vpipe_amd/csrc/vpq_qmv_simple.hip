@@ -6,9 +6,9 @@
 // Arithmetic: W[n,k] = fma(s, q, b) in fp32 (never rounded to bf16),
 // acc += x * W in fp32, wave reduction, one bf16 rounding on store -- the
 // semantics of gpu-kernels/metal/quant/affine_qmv.metal:151-174, 228-283.
-// With `swiglu` the rows are an interleaved gate|up pack: wavefronts 2j and 2j+1 of a
+// With `gate_act` (1 SwiGLU, 2 GEGLU) the rows are an interleaved gate|up pack: wavefronts 2j and 2j+1 of a
 // workgroup hold a feature's gate and up sums, the odd one hands its sum over through LDS and
-// the even one stores silu(gate) * up into y[M, N/2] (affine_qmv.metal:816-906).
+// the even one stores act(gate) * up into y[M, N/2] (affine_qmv.metal:816-906, 1356-1430).
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -18,7 +18,7 @@ template <int MT, bool F32OUT>
 __global__ __launch_bounds__(256) void qmv_simple_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x, void* __restrict__ y,
-    const uint16_t* __restrict__ residual, int K, int N, int M, int swiglu)
+    const uint16_t* __restrict__ residual, int K, int N, int M, int gate_act)
 {
   __shared__ float up_sum[4][MT];
   const int wave = threadIdx.x >> 6;
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
         }
       }
     }
-    if (swiglu) {
+    if (gate_act) {
       float total[MT];
 #pragma unroll
       for (int mm = 0; mm < MT; ++mm) { total[mm] = wave_sum(acc[mm]); }
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
         for (int mm = 0; mm < MT; ++mm) {
           const int row = m0 + mm;
           if (row < M) {
-            const float v = swiglu_f32(total[mm], up_sum[wave + 1][mm]);
+            const float v = gated_f32(gate_act, total[mm], up_sum[wave + 1][mm]);
             const size_t o = (size_t)row * (N >> 1) + (n >> 1);
             if (F32OUT) {
               reinterpret_cast<float*>(y)[o] = v;
@@ -111,7 +111,7 @@ hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a)
   const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
 #define VPQ_LAUNCH(MT, F32)                                                                    \
   launch_kernel(qmv_simple_kernel<MT, F32>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
-                a.residual, a.K, a.N, a.M, a.swiglu ? 1 : 0)
+                a.residual, a.K, a.N, a.M, a.gate_act)
   if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH(1, true) : VPQ_LAUNCH(1, false); }
   return a.y_f32 ? VPQ_LAUNCH(4, true) : VPQ_LAUNCH(4, false);
 #undef VPQ_LAUNCH

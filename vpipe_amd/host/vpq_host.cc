@@ -87,6 +87,8 @@ const FnEntry kFunctions[] = {
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm128", QuantKernel::Qmm},
     {"affine_qmm_mma_bf16", "affine_qmm_mma_w4g64", QuantKernel::Qmm},
     {"affine_qmv_bf16", "affine_qmv_swiglu_w4g64", QuantKernel::QmvSwiglu},
+    {"affine_qmv_bf16", "affine_qmv_geglu_w4g64", QuantKernel::QmvGeglu},
+    {"affine_qmm_steel_bf16", "affine_qmm_geglu_w4g64", QuantKernel::QmmGeglu},
     {"llm_elementwise_bf16", "dequant_embed_gather_f16", QuantKernel::EmbedGather},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64", QuantKernel::QmmSwiglu},
@@ -414,7 +416,7 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
         } else {
           status = vpq_qmm_w4g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), nullptr, nullptr, 0, 0.f, nullptr);
         }
-      } else if (kind == QuantKernel::QmmSwiglu) {
+      } else if (kind == QuantKernel::QmmSwiglu || kind == QuantKernel::QmmGeglu) {
         // gpu-kernels/metal/quant/affine_qmm_steel.metal:801-947: slot 7 = M; the strided twin adds
         // 8 = out_stride, 9 = out_off.  Rows go to the GEMV arithmetic when there are at most 16,
         // the choice the reference makes at its call sites.
@@ -422,12 +424,14 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
           status = VPQ_ERR_NULL_POINTER;
         } else {
           const int stride = has_int(8) ? ival(8) : 0, off = has_int(9) ? ival(9) : 0;
-          status = vpq_qmm_swiglu_w4g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), stride, off);
+          status = vpq_qmm_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), stride, off,
+                                            kind == QuantKernel::QmmGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
         }
-      } else if (kind == QuantKernel::QmvSwiglu) {
+      } else if (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu) {
         // gpu-kernels/metal/quant/affine_qmv.metal:891-906: N = 2*ffn, rows from grid.x
         const int M = grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1;
-        status = vpq_qmv_swiglu_w4g64_bf16(st, w, sc, bi, x, y, K, N, M, VPQ_QMV_AUTO);
+        status = vpq_qmv_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, M, VPQ_QMV_AUTO,
+                                          kind == QuantKernel::QmvGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
       } else {
         int M = 1;
         const uint16_t* residual = nullptr;

@@ -77,6 +77,8 @@ enum class QuantKernel : std::uint8_t {
                   //   7 = K, 8,9,10 = q_rows, k_rows, v_rows (v_rows == 0: q|k only); one launch
   QmvSwiglu,      // affine_qmv_swiglu_w4g64: interleaved gate|up pack, N = 2*ffn, y [M, ffn]; M from grid.x / 32
   QmmSwiglu,      // affine_qmm_swiglu_w4g64[_bm64|_bm128|_bm64_rs]: slot 7 = M, 8 = out_stride, 9 = out_off (_rs)
+  QmvGeglu,       // affine_qmv_geglu_w4g64: as QmvSwiglu with gelu_tanh(gate) * up
+  QmmGeglu,       // affine_qmm_geglu_w4g64: as QmmSwiglu
   EmbedGather,    // dequant_embed_gather_f16: slots 0:ids 1:w 2:scales 3:biases 4:out 5:H; T = grid.y,
                   //   the vocabulary size is what the bound code buffer holds
 };
