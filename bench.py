@@ -458,6 +458,17 @@ def main():
         out["fused_mlp_swiglu"] = fm
         del fused, x, y
 
+        # dense expansion (the a1 kernel): 9/16 B read and 2 B written per weight
+        dq = {}
+        for K, N in ((4096, 4096), (4096, 12288), (5120, 20480)):
+            w, s, b = make_weight(torch, N, K, dev, gen)
+            wdeq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+            us = kernel_us(lambda i: vpipe_amd.dequant_w4g64(w, s, b, K, N, out=wdeq), 6)
+            nbytes = N * K * 9 // 16 + 2 * N * K
+            dq["%dx%d" % (N, K)] = {"us": round(us, 2), "GBps": round(nbytes / (us * 1e-6) / 1e9, 1)}
+            del w, s, b, wdeq
+        out["dequant_w4g64"] = dq
+
     # ---- CPU baseline: the oracle's dequant + fp32 matmul on the host cores ------------
     if not args.no_cpu:
         from oracle import oracle
