@@ -191,9 +191,12 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
 
 /* ---- a5: the size-based entrance ----------------------------------------
  * Replaces `MetalQwenModel::qmm_auto_`
- * (generative-models/qwen3/metal-qwen-model.cc:3964-4033): M <= 16 runs the QMV
- * arithmetic, larger M the QMM arithmetic.  (The reference crosses over at
- * M = 8; this build's GEMV tile holds 16 rows.) */
+ * (generative-models/qwen3/metal-qwen-model.cc:3964-4033) with its ladder
+ * (:3839-3962: GEMV, a batched plan that walks M in slabs, the tiled GEMM): up
+ * to 64 rows run the QMV arithmetic in slabs of at most 16 rows (one launch per
+ * slab), larger M the QMM arithmetic.  (The reference crosses over to the GEMM at
+ * M = 8; here the 256-row GEMM tile does not pay below ~64 rows: measured 57 us at
+ * 4096->4096 for any M <= 256 against ~10 us per slab.) */
 int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y,
                           int K, int N, int M, void* ws, size_t ws_bytes);
@@ -254,8 +257,8 @@ int vpq_qmm_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint
 
 /* The size-based entrance of the fused MLP first half, as the reference's call
  * sites choose between the two (generative-models/llama3/metal-llama-model.cc:
- * 466-477 decode, 634-650 and 800-812 prefill): M <= 16 QMV arithmetic, larger
- * M QMM arithmetic. */
+ * 466-477 decode, 634-650 and 800-812 prefill): up to 64 rows the QMV arithmetic
+ * in slabs of 16 rows, larger M the QMM arithmetic (as vpq_linear_w4g64_bf16). */
 int vpq_linear_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                  const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                  int K, int N, int M);

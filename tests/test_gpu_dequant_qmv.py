@@ -280,15 +280,24 @@ def test_qmv_small_batch_shapes_row_sample(vpq, oracle, dev, D, K, N, M):
 
 
 def test_linear_entrance_routes_by_rows(vpq, oracle, dev, D):
-    # qmm_auto_ (metal-qwen-model.cc:3964-4033): GEMV arithmetic for few rows, GEMM above
-    K, N = 1024, 64
+    # qmm_auto_ and its ladder (metal-qwen-model.cc:3839-4033): GEMV arithmetic for few rows -- one
+    # launch up to 16, slabs of 16 rows up to 64 -- and the GEMM above
+    K, N = 1024, 80
     w, s, b = synth.make_weight(N, K, 91)
     wd, sd, bd = stage(D, dev, w, s, b)
-    for M, fn in ((16, oracle.qmv), (17, oracle.qmm)):
+    for M, fn in ((16, oracle.qmv), (17, oracle.qmv), (41, oracle.qmv), (64, oracle.qmv), (65, oracle.qmm)):
         x = synth.make_act(M, K, 92 + M)
         y64, yb = fn(w, s, b, x, K, N, M)
-        y = vpq.linear_w4g64(wd, sd, bd, D.bf16(x, dev), K, N, M)
-        parity.check_bf16(D.bits(y), y64, yb)
+        out = parity.Guarded((M, N), torch.bfloat16, dev)
+        vpq.linear_w4g64(wd, sd, bd, D.bf16(x, dev), K, N, M, out=out.view)
+        torch.cuda.synchronize()
+        parity.check_bf16(D.bits(out.view), y64, yb)
+        out.assert_intact()
+        if fn is oracle.qmv:
+            # a slab is the plain QMV call on its rows: same bits
+            ref = torch.cat([vpq.qmv_w4g64(wd, sd, bd, D.bf16(x[m0:m0 + 16], dev), K, N, min(16, M - m0))
+                             for m0 in range(0, M, 16)])
+            assert torch.equal(out.view, ref)
 
 
 @pytest.mark.parametrize("K,Ns,M", [(4096, (4096, 1024, 1024), 1), (4096, (12288, 12288), 1), (1024, (48, 33, 16, 95), 3),

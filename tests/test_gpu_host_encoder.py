@@ -238,7 +238,7 @@ def test_errors_surface_at_the_fence(enc, dev, D):
     assert D.bits(yd).any()
 
 
-@pytest.mark.parametrize("M", [1, 8, 40])
+@pytest.mark.parametrize("M", [1, 8, 40, 100])
 def test_quant_linear_forward_routes_by_m(enc, oracle, dev, D, M):
     K, N = 512, 320
     w, s, b = synth.make_weight(N, K, 13)
@@ -250,7 +250,7 @@ def test_quant_linear_forward_routes_by_m(enc, oracle, dev, D, M):
                           None, None, 0, 0.0, None)
     ok, why = enc.wait_ok()
     assert ok, why
-    y64, yb = (oracle.qmv if M <= 16 else oracle.qmm)(w, s, b, x, K, N, M)
+    y64, yb = (oracle.qmv if M <= 64 else oracle.qmm)(w, s, b, x, K, N, M)
     parity.check_bf16(D.bits(yd), y64, yb)
 
 
@@ -385,7 +385,7 @@ def test_quantize_write_read_load_run(enc, oracle, dev, D, tmp_path, M):
     assert L.hd_load_and_run(enc.h, r, prefix, 2048, xd.data_ptr(), yd.data_ptr(), M, kn) == 0    # a 2-bit reading
     L.hr_close(r)
     sb, bb = oracle.f16_to_bf16(s16), oracle.f16_to_bf16(b16)
-    y64, yb = (oracle.qmv if M <= 16 else oracle.qmm)(codes, sb, bb, x, K, N, M)
+    y64, yb = (oracle.qmv if M <= 64 else oracle.qmm)(codes, sb, bb, x, K, N, M)
     parity.check_bf16(D.bits(yd), y64, yb)
 
 

@@ -227,8 +227,8 @@ def test_qmm_and_linear_geglu(vpq, oracle, dev, D, M, F, K):
     torch.cuda.synchronize()
     parity.check_bf16(D.bits(out.view), o64, ob, mismatch_over_all=False)
     out.assert_intact()
-    # the size-based entrance takes the GEMV arithmetic up to 16 rows
-    arith = oracle.qmv if M <= 16 else oracle.qmm
+    # the size-based entrance takes the GEMV arithmetic (in slabs of 16 rows) up to 64 rows
+    arith = oracle.qmv if M <= 64 else oracle.qmm
     l64, lb = oracle.geglu(arith(*pack, x, K, 2 * F, M)[0])
     got = vpq.linear_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, activation=capi.VPQ_GATE_GEGLU)
     parity.check_bf16(D.bits(got), l64, lb, mismatch_over_all=False)

@@ -285,12 +285,23 @@ int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
   return VPQ_OK;
 }
 
+// Rows up to which the size-based entrances run the GEMV arithmetic in slabs of 16 rows instead of
+// the 256-row GEMM tile: below it the tile kernel has one row of tiles and N/128 workgroups, and
+// its time is its K loop's latency (57 us at 4096->4096 for any M <= 256) against ~10 us per slab.
+constexpr int kSlabPlanMaxRows = 64;
+
 int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                           void* ws, size_t ws_bytes)
 {
-  if (M >= 1 && M <= 16) {
-    return vpq_qmv_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, nullptr, ws, ws_bytes, VPQ_QMV_AUTO);
+  if (M >= 1 && M <= kSlabPlanMaxRows && x != nullptr && y != nullptr && K > 0 && N > 0) {
+    for (int m0 = 0; m0 < M; m0 += 16) {
+      const int rows = M - m0 < 16 ? M - m0 : 16;
+      const int st = vpq_qmv_w4g64_bf16(stream, w, scales, biases, x + (size_t)m0 * K, y + (size_t)m0 * N, K, N, rows,
+                                        nullptr, ws, ws_bytes, VPQ_QMV_AUTO);
+      if (st != VPQ_OK) { return st; }
+    }
+    return VPQ_OK;
   }
   return vpq_qmm_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, nullptr, nullptr, 0, 0.0f, nullptr);
 }
@@ -349,8 +360,14 @@ int vpq_linear_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const ui
                                 const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                                 int activation)
 {
-  if (M >= 1 && M <= 16) {
-    return vpq_qmv_gated_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, VPQ_QMV_AUTO, activation);
+  if (M >= 1 && M <= kSlabPlanMaxRows && x != nullptr && y != nullptr && K > 0 && N > 0) {
+    for (int m0 = 0; m0 < M; m0 += 16) {
+      const int rows = M - m0 < 16 ? M - m0 : 16;
+      const int st = vpq_qmv_gated_w4g64_bf16(stream, w, scales, biases, x + (size_t)m0 * K, y + (size_t)m0 * (N / 2), K, N,
+                                              rows, VPQ_QMV_AUTO, activation);
+      if (st != VPQ_OK) { return st; }
+    }
+    return VPQ_OK;
   }
   return vpq_qmm_gated_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, 0, 0, activation);
 }
