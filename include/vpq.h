@@ -165,6 +165,24 @@ int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
                        const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
                        uint16_t* lora_t_ws);
 
+/* Split-K form of the fused kernel for GEMMs with few output tiles (M of a few
+ * hundred rows, or a narrow N, over a long K), where one workgroup per 256 x 128
+ * tile leaves most of the chip idle and each walks a long serial K loop: `splits`
+ * (2..16; 0 = chosen so that about one workgroup per CU results, at least 512 of K
+ * each; 1 = none) shares of K run as separate workgroups into fp32 planes
+ * [splits][M][N] in `ws`, and a fold adds the planes in order and rounds once.  The
+ * model is the reference's deep-K split (generative-models/shared/mma-splitk.h:
+ * 30-52, 66-140: f32 planes + fold, chosen by chunk width); results differ from the
+ * unsplit kernel only by the fp32 reassociation and are bit-reproducible.  No
+ * adapter, no gated store.  `ws`: vpq_qmm_workspace_bytes() bytes (0 where the
+ * automatic choice is not to split), 256-byte aligned, contents irrelevant; if it
+ * is also handed to the QMV split-K variant, zero it again first.
+ * VPQ_ERR_WORKSPACE if it is needed and missing or too small. */
+size_t vpq_qmm_workspace_bytes(int K, int N, int M);
+int vpq_qmm_splitk_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                              int K, int N, int M, int splits, void* ws, size_t ws_bytes);
+
 /* ---- a8: the dequant-once route -------------------------------------------
  * Replaces `gemm_mma_` (generative-models/minimax-h3/metal-minimax-h3-transformer.cc:
  * 2020-2160: `affine_dequant_w4g64` into a scratch, then a dense matrix-unit GEMM,
@@ -196,7 +214,9 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
  * to 64 rows run the QMV arithmetic in slabs of at most 16 rows (one launch per
  * slab), larger M the QMM arithmetic.  (The reference crosses over to the GEMM at
  * M = 8; here the 256-row GEMM tile does not pay below ~64 rows: measured 57 us at
- * 4096->4096 for any M <= 256 against ~10 us per slab.) */
+ * 4096->4096 for any M <= 256 against ~10 us per slab.)  Above 64 rows the GEMM
+ * splits K (vpq_qmm_splitk_w4g64_bf16) where that pays and `ws` has
+ * vpq_qmm_workspace_bytes() bytes. */
 int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y,
                           int K, int N, int M, void* ws, size_t ws_bytes);

@@ -170,3 +170,41 @@ def test_qmm_dense_route_matches_oracle(vpq, oracle, dev, D, M, N, K):
     # with the kept expansion: no expansion pass, same bits
     again = vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq, expand=False)
     assert torch.equal(again, out.view)
+
+
+@pytest.mark.parametrize("M,N,K,splits", [(100, 256, 2048, 0), (65, 128, 1024, 2), (300, 640, 4096, 0), (257, 129, 1536, 3),
+                                          (128, 4096, 4096, 0), (40, 96, 1088, 16)])
+def test_qmm_split_k(vpq, oracle, dev, D, M, N, K, splits):
+    # few output tiles over a long K: shares of K into fp32 planes, folded in order, rounded once
+    # (the reference's deep-K split, generative-models/shared/mma-splitk.h:30-52)
+    w, s, b = synth.make_weight(N, K, 3000 + N)
+    x = synth.make_act(M, K, 3100 + M)
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_splitk_w4g64(wd, sd, bd, xd, K, N, M, splits=splits, out=out.view)
+    torch.cuda.synchronize()
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    out.assert_intact()
+    again = vpq.qmm_splitk_w4g64(wd, sd, bd, xd, K, N, M, splits=splits)
+    assert torch.equal(again, out.view)                       # bit-reproducible
+    if splits > 1:
+        with pytest.raises(vpq.VpqError):
+            vpq.qmm_splitk_w4g64(wd, sd, bd, xd, K, N, M, splits=splits, ws=torch.empty(256, dtype=torch.uint8, device=dev))
+
+
+def test_linear_entrance_splits_k_when_given_the_room(vpq, oracle, dev, D):
+    M, N, K = 128, 512, 4096
+    w, s, b = synth.make_weight(N, K, 3200)
+    x = synth.make_act(M, K, 3201)
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    need = vpq.load().vpq_qmm_workspace_bytes(K, N, M)
+    assert need >= 2 * M * N * 4
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    split = vpq.linear_w4g64(wd, sd, bd, xd, K, N, M, ws=ws)
+    plain = vpq.linear_w4g64(wd, sd, bd, xd, K, N, M)
+    torch.cuda.synchronize()
+    parity.check_bf16(D.bits(split), y64, yb)
+    parity.check_bf16(D.bits(plain), y64, yb)
+    assert vpq.load().vpq_qmm_workspace_bytes(4096, 12288, 2048) == 0      # enough tiles: no split

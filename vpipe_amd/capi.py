@@ -32,6 +32,8 @@ SYMBOLS = [
     ("vpq_qmv_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _i]),
     ("vpq_qmv_workspace_bytes", _sz, [_i, _i, _i]),
     ("vpq_qmm_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _f, _vp]),
+    ("vpq_qmm_workspace_bytes", _sz, [_i, _i, _i]),
+    ("vpq_qmm_splitk_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz]),
     ("vpq_qmm_dense_route_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_lora_a_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f]),
     ("vpq_linear_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz]),
@@ -204,6 +206,20 @@ def linear_swiglu_w4g64(w, scales, biases, x, K, N, M, out=None, activation=VPQ_
         st = load().vpq_linear_gated_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
                                                 activation)
     _check(st, "vpq_linear_gated_w4g64_bf16")
+    return out
+
+
+def qmm_splitk_w4g64(w, scales, biases, x, K, N, M, splits=0, ws=None, out=None):
+    """Split-K QMM; ws: uint8 tensor of vpq_qmm_workspace_bytes (allocated here if None)."""
+    import torch
+    L = load()
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    if ws is None:
+        need = max(L.vpq_qmm_workspace_bytes(K, N, M), (splits if splits > 1 else 0) * M * N * 4, 256)
+        ws = torch.empty(need, dtype=torch.uint8, device=w.device)
+    _check(L.vpq_qmm_splitk_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M, splits,
+                                       _ptr(ws), ws.numel()), "vpq_qmm_splitk_w4g64_bf16")
     return out
 
 

@@ -258,6 +258,36 @@ int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
   return finish(vpq::launch_qmm_tile(hs, g));
 }
 
+size_t vpq_qmm_workspace_bytes(int K, int N, int M)
+{
+  if (K <= 0 || N <= 0 || M <= 0 || (K % 64) != 0) { return 0; }
+  if (ensure_init() != VPQ_OK) { return 0; }
+  return (vpq::qmm_splitk_workspace_bytes(K, N, M, g_dev.cu_count) + 255) / 256 * 256;
+}
+
+int vpq_qmm_splitk_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                              int splits, void* ws, size_t ws_bytes)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M <= 0 || splits < 0 || splits > 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16) || (ws != nullptr && !aligned(ws, 256))) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  if (splits == 0) { splits = vpq::qmm_choose_splits(K, N, M, g_dev.cu_count); }
+  if (splits > K / 64) { splits = K / 64; }
+  vpq::GemmArgs g{};
+  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
+  g.K = K; g.N = N; g.M = M;
+  g.cu_count = g_dev.cu_count;
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (splits <= 1) { return finish(vpq::launch_qmm_tile(hs, g)); }
+  if (ws == nullptr || ws_bytes < (size_t)splits * (size_t)M * (size_t)N * sizeof(float)) { return VPQ_ERR_WORKSPACE; }
+  return finish(vpq::launch_qmm_tile_splitk(hs, g, splits, static_cast<float*>(ws)));
+}
+
 int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                                    uint16_t* w_deq, int expand)
@@ -302,6 +332,13 @@ int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t
       if (st != VPQ_OK) { return st; }
     }
     return VPQ_OK;
+  }
+  // Few tiles and a long K: split K over more workgroups when the caller's workspace has the room.
+  if (ws != nullptr && aligned(ws, 256) && K > 0 && N > 0 && M > 0 && (K % 64) == 0 && ensure_init() == VPQ_OK) {
+    const int splits = vpq::qmm_choose_splits(K, N, M, g_dev.cu_count);
+    if (splits > 1 && ws_bytes >= (size_t)splits * (size_t)M * (size_t)N * sizeof(float)) {
+      return vpq_qmm_splitk_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, splits, ws, ws_bytes);
+    }
   }
   return vpq_qmm_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, nullptr, nullptr, 0, 0.0f, nullptr);
 }

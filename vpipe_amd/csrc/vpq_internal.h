@@ -108,6 +108,12 @@ hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, u
                          float alpha);
 // 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.
 hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a);
+// Split-K form of the same kernel (no adapter, no gated store): `splits` shares of the K steps,
+// fp32 planes [splits][M][N] in `plane`, then a fold.  qmm_choose_splits() returns 1 where the tiles
+// alone fill the chip.
+int qmm_choose_splits(int K, int N, int M, int cu_count);
+size_t qmm_splitk_workspace_bytes(int K, int N, int M, int cu_count);
+hipError_t launch_qmm_tile_splitk(hipStream_t st, const GemmArgs& a, int splits, float* plane);
 // y[M,N] = x[M,K] . b[N,K]^T on the vendor BLAS (bf16 in, fp32 accumulate, bf16 out).
 // 0, or -1 (rocBLAS unavailable) / -2 (the call failed) with *why set.
 int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,

@@ -67,6 +67,13 @@ struct TileParams {
   // SwiGLU store (gpu-kernels/metal/quant/affine_qmm_steel.metal:663-768): the pack is an
   // interleaved gate|up matrix and y[m * out_stride + out_off + g] = silu(gate_g) * up_g.
   int gate_act, out_stride, out_off;
+  // Split-K (ksplit > 1): workgroup blockIdx.x covers tile blockIdx.x % tiles and the K steps
+  // [ks * steps_per_split, ...) with ks = blockIdx.x / tiles; its fp32 accumulators go to
+  // plane[ks][M][N] and a fold kernel adds the planes in order and rounds once
+  // (generative-models/shared/mma-splitk.h:30-52: f32 planes, so the output is rounded once
+  // whatever the split count).
+  int ksplit, steps_per_split;
+  float* plane;
 };
 
 __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
@@ -142,11 +149,16 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   const bool producer = wave >= kConsumers;
 
   // Consecutive workgroups walk M first: they share one weight tile.
-  const int tile = blockIdx.x;
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int ks = p.ksplit > 1 ? (int)blockIdx.x / tiles : 0;
+  const int tile = (int)blockIdx.x - ks * tiles;
   const int tm = tile % p.tiles_m;
   const int tn = tile / p.tiles_m;
   const int m0 = tm * TM, n0 = tn * TN;
-  const int KT = p.K / TK;
+  // This workgroup's K steps: all of them, or its share of a split.
+  const int k_first = ks * p.steps_per_split;
+  const int KT = p.ksplit > 1 ? ((p.K / TK - k_first) < p.steps_per_split ? (p.K / TK - k_first) : p.steps_per_split)
+                              : p.K / TK;
 
   if (producer) {
     // ======================= producers =======================
@@ -154,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     const int pt = tid - kConsumers * 64; // 0..255
     // x tile: 32 direct-to-LDS loads per step, 8 per wavefront.  Load i of wave pw covers tile
     // rows (8 pw + i)*8 .. +8; lane l takes row l/8, LDS position l%8.
-    const uint8_t* xblk = reinterpret_cast<const uint8_t*>(p.x) + (size_t)m0 * p.K * 2;
+    const uint8_t* xblk = reinterpret_cast<const uint8_t*>(p.x) + (size_t)m0 * p.K * 2 + (size_t)k_first * (TK * 2);
     uint32_t a_off[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -166,9 +178,10 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     // W tile: thread pt dequantizes 32 codes of row pt/2 (k half pt%2) per step.
     const int qrow = pt >> 1, qhalf = pt & 1;
     const int qrg = (n0 + qrow < p.N) ? (n0 + qrow) : (p.N - 1);
-    const uint8_t* wrow = reinterpret_cast<const uint8_t*>(p.w) + (size_t)qrg * (p.K >> 1) + qhalf * 16;
-    const uint16_t* srow = p.scales + (size_t)qrg * (p.K >> 6);
-    const uint16_t* brow = p.biases + (size_t)qrg * (p.K >> 6);
+    const uint8_t* wrow = reinterpret_cast<const uint8_t*>(p.w) + (size_t)qrg * (p.K >> 1) + qhalf * 16 +
+                          (size_t)k_first * (TK / 2);
+    const uint16_t* srow = p.scales + (size_t)qrg * (p.K >> 6) + k_first;
+    const uint16_t* brow = p.biases + (size_t)qrg * (p.K >> 6) + k_first;
     int b_dst[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) { b_dst[i] = qrow * kRowB + swz(qrow, qhalf * 4 + i) * 16; }
@@ -352,6 +365,33 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   }
 
   // ---- store: lane holds, for x row m = lane%32 of each it, 4 consecutive n per register quad ----
+  if (p.ksplit > 1) {
+    const bool vec4 = (p.N & 3) == 0;
+#pragma unroll
+    for (int it = 0; it < kIT; ++it) {
+      const int m = m0 + wm * kWaveM + it * 32 + frow;
+      if (m >= p.M) { continue; }
+      float* prow = p.plane + ((size_t)ks * p.M + m) * p.N;
+#pragma unroll
+      for (int jt = 0; jt < 2; ++jt) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int n = n0 + wn * 64 + jt * 32 + rq * 8 + fkh * 4;
+          if (n >= p.N) { continue; }
+          if (vec4 && n + 3 < p.N) {
+            floatx4 v = {acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1], acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]};
+            *reinterpret_cast<floatx4*>(prow + n) = v;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (n + e < p.N) { prow[n + e] = acc[jt][it][rq * 4 + e]; }
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
   if (p.gate_act) {
     // A register quad is (gate, up, gate, up) of features n/2 and n/2 + 1 (n is a multiple of 4):
     // the activation is register-local and a quad becomes one dword of two bf16.
@@ -411,6 +451,72 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   }
 }
 
+// y[i] = bf16(plane[0][i] + plane[1][i] + ... ) in that order, i over M*N.
+__global__ __launch_bounds__(256) void splitk_fold_kernel(const float* __restrict__ plane, uint16_t* __restrict__ y,
+                                                          size_t count, int splits)
+{
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (size_t)gridDim.x * 256) {
+    float v = plane[i];
+    for (int s = 1; s < splits; ++s) { v += plane[(size_t)s * count + i]; }
+    y[i] = (uint16_t)f32_to_bf16_bits(v);
+  }
+}
+
+// Split count by a small cost model (microseconds, from measurements on MI355X): a workgroup costs
+// ~3 us to start and drain plus ~0.9 us per K step; workgroups run one per CU, so the grid takes
+// ceil(workgroups / CUs) rounds; the planes are written and read once more by the fold at ~4 TB/s.
+int qmm_choose_splits(int K, int N, int M, int cu_count)
+{
+  const int tiles = ((M + TM - 1) / TM) * ((N + TN - 1) / TN);
+  const int steps = K / TK;
+  const int cus = cu_count > 0 ? cu_count : 256;
+  if (tiles * 2 > cus) { return 1; }                   // the tiles alone fill at least half of the chip
+  auto cost = [&](int s) {
+    const int per = (steps + s - 1) / s;
+    const int rounds = (tiles * s + cus - 1) / cus;
+    double us = rounds * (3.0 + 0.9 * per);
+    if (s > 1) { us += 3.0 + (s + 0.5) * (double)M * (double)N * 4.0 / 4.0e6; }
+    return us;
+  };
+  int best = 1;
+  double best_us = cost(1);
+  for (int s = 2; s <= 16 && steps / s >= 4; ++s) {
+    const int per = (steps + s - 1) / s;
+    if ((steps + per - 1) / per != s) { continue; }    // shares would come out uneven: another count covers it
+    const double us = cost(s);
+    if (us < 0.9 * best_us) { best = s; best_us = us; }
+  }
+  return best;
+}
+
+size_t qmm_splitk_workspace_bytes(int K, int N, int M, int cu_count)
+{
+  const int s = qmm_choose_splits(K, N, M, cu_count);
+  return s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+
+hipError_t launch_qmm_tile_splitk(hipStream_t st, const GemmArgs& a, int splits, float* plane)
+{
+  TileParams p;
+  p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
+  p.lora_t = nullptr; p.lora_b = nullptr;
+  p.K = a.K; p.N = a.N; p.M = a.M; p.r = 0;
+  p.gate_act = 0; p.out_stride = a.N / 2; p.out_off = 0;
+  p.tiles_m = (a.M + TM - 1) / TM;
+  p.tiles_n = (a.N + TN - 1) / TN;
+  const int steps = a.K / TK;
+  p.steps_per_split = (steps + splits - 1) / splits;
+  p.ksplit = (steps + p.steps_per_split - 1) / p.steps_per_split;
+  p.plane = plane;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.ksplit)), block(kThreads);
+  hipError_t e = launch_kernel(qmm_tile_kernel<false>, grid, block, 0, st, p);
+  if (e != hipSuccess) { return e; }
+  const size_t count = (size_t)a.M * (size_t)a.N;
+  size_t blocks = (count + 255) / 256;
+  if (blocks > 65536) { blocks = 65536; }
+  return launch_kernel(splitk_fold_kernel, dim3((unsigned)blocks), dim3(256), 0, st, plane, a.y, count, p.ksplit);
+}
+
 hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a)
 {
   TileParams p;
@@ -422,6 +528,7 @@ hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a)
   p.out_off = a.out_off;
   p.tiles_m = (a.M + TM - 1) / TM;
   p.tiles_n = (a.N + TN - 1) / TN;
+  p.ksplit = 1; p.steps_per_split = a.K / TK; p.plane = nullptr;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
   return a.lora_t != nullptr ? launch_kernel(qmm_tile_kernel<true>, grid, block, 0, st, p)
                              : launch_kernel(qmm_tile_kernel<false>, grid, block, 0, st, p);
