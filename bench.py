@@ -469,6 +469,27 @@ def main():
             del w, s, b, wdeq
         out["dequant_w4g64"] = dq
 
+        # 8-bit twin, general kernel (one wavefront per row): 17/16 B per weight
+        w8 = {}
+        for K, N in ((4096, 4096), (5120, 151936)):
+            copies = max(2, min(8, int(600e6 // (N * K * 17 // 16))))
+            packs = []
+            for _ in range(copies):
+                w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 4), dtype=torch.int32, device=dev, generator=gen)
+                s = torch.empty((N, K // 64), dtype=torch.float32, device=dev).uniform_(0.0003, 0.0012, generator=gen).bfloat16()
+                packs.append((w, s, (-128.0 * s.float()).bfloat16()))
+            x = torch.randn((1, K), device=dev, generator=gen).bfloat16()
+            y = torch.empty((1, N), dtype=torch.bfloat16, device=dev)
+
+            def call8(i, x=x, y=y, K=K, N=N):
+                w, s, b = packs[i % copies]
+                vpipe_amd.qmv_w8g64(w, s, b, x, K, N, 1, out=y)
+            us = kernel_us(call8, 2 * copies)
+            nbytes = N * K * 17 // 16 + 2 * K + 2 * N
+            w8["%d->%d" % (K, N)] = {"us": round(us, 2), "GBps": round(nbytes / (us * 1e-6) / 1e9, 1)}
+            del packs
+        out["qmv_w8g64_m1"] = w8
+
     # ---- CPU baseline: the oracle's dequant + fp32 matmul on the host cores ------------
     if not args.no_cpu:
         from oracle import oracle

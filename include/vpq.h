@@ -304,6 +304,33 @@ int vpq_linear_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const ui
                                 const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                 int K, int N, int M, int activation);
 
+/* ---- 8-bit group-64 twins (w8g64) -------------------------------------------
+ * The same affine format with one BYTE per value: w uint32 [N, K/4],
+ * q[n, 4j+i] = (w[n,j] >> 8i) & 0xFF; scales, biases bf16 [N, K/64]
+ * (gpu-kernels/metal/quant/affine_dequant.metal:60-97).  A first, general path for
+ * the 8-bit checkpoints and the 8-bit linears of mixed-precision ones; not tuned
+ * like the 4-bit kernels:
+ *   vpq_dequant_w8g64_bf16           replaces `affine_dequant_w8g64` (:68-97), bit-exact.
+ *   vpq_qmv_w8g64_bf16 / _f32out     replace `affine_qmv_w8g64[_add]`
+ *                                    (affine_qmv.metal:3034-3050, 3122-3140): QMV arithmetic,
+ *                                    1 <= M <= 16, one wavefront per output row.
+ *   vpq_qmm_dense_route_w8g64_bf16   the dequant-once route for any M (replaces
+ *                                    `affine_qmm_steel_w8g64`, affine_qmm_steel.metal:1601-1672,
+ *                                    by the reference's own second route): expansion into
+ *                                    `w_deq` [N,K] bf16 + the vendor dense GEMM; arguments as
+ *                                    vpq_qmm_dense_route_w4g64_bf16.
+ * Requirements as for the 4-bit entries (K % 64 == 0; 16-byte aligned w, x). */
+int vpq_dequant_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                           const uint16_t* biases, uint16_t* w_deq, int K, int N);
+int vpq_qmv_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                       int K, int N, int M, const uint16_t* residual);
+int vpq_qmv_w8g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                         const uint16_t* biases, const uint16_t* x, float* y, int K, int N, int M);
+int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                                   int K, int N, int M, uint16_t* w_deq, int expand);
+
 /* ---- a12: the packer ------------------------------------------------------
  * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:
  * 243-301; slots 0:x 1:w 2:s 3:b 4:K 5:N 6:clip) driven by

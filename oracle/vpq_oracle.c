@@ -24,6 +24,8 @@
  *   swiglu / interleave    x*expit(x) of scipy, silu(v) - silu(-v) == v, limits;
  *                          numpy stacking; fused pack == silu(qmv(gate)) * qmv(up)
  *                          from two separate packs
+ *   w8g64                  numpy re-derivation from the byte view of the words, one-hot
+ *                          activations, float64 matmul
  *   quantize (packer)      exact recovery of on-grid data, the reference's
  *                          round-trip error bounds, numpy re-derivation
  * Parity that only an Apple-GPU run could pin -- the last-bit effect of the
@@ -431,6 +433,63 @@ void vpo_quantize_w4g64(const float* wsrc, uint32_t* codes, uint16_t* scales_f16
 /* Output byte sizes, generative-models/quantize/affine-quantizer.h:37-40. */
 size_t vpo_weight_bytes(int N, int K) { return (size_t)N * (size_t)(K * 4 / 32) * 4; }
 size_t vpo_scale_bytes(int N, int K) { return (size_t)N * (size_t)(K / VPO_GROUP) * 2; }
+
+/* ---- 8-bit twin (w8g64) ------------------------------------------------- */
+
+/* 8-bit affine weights hold one byte per value, four per u32 word, little-endian
+ * within the word: q[n, 4j+i] = (w[n,j] >> 8i) & 0xFF, a row is K/4 words
+ * (gpu-kernels/metal/quant/affine_dequant.metal:60-97, affine_qmv.metal:68-76,
+ * 168-172: qmv reads the row as raw bytes).  Scales and biases as for 4 bits,
+ * one pair per 64 values. */
+static inline unsigned code8(const uint32_t* w, size_t n, int Kw, int k)
+{
+  return (w[n * (size_t)Kw + (size_t)(k >> 2)] >> (8 * (k & 3))) & 0xffu;
+}
+
+/* affine_dequant_w8g64 (affine_dequant.metal:68-97): out = (elt)(s * (float)q + b);
+ * s*q is exact in fp32 (8-bit x 8-bit significands). */
+void vpo_dequant_w8g64_bf16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            uint16_t* out, int K, int N)
+{
+  const int Kw = K / 4, Kg = K / VPO_GROUP;
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)code8(w, n, Kw, k);
+      out[n * (size_t)K + k] = vpo_f32_to_bf16(sq + b);
+    }
+  }
+}
+
+/* QMV (affine_qmv_w8g64, affine_qmv.metal:3034-3050 = qmv_fast_impl<T,64,8>: the same
+ * factored sum scale*sum(x*q) + bias*sum(x), weight never rounded) when rounded == 0;
+ * the GEMM semantics (weight rounded to the element type first: affine_qmm_steel_w8g64,
+ * affine_qmm_steel.metal:1601-1624, and the dequant-once route) when rounded != 0.
+ * Double accumulation; y_bf16 (nullable) is the RNE cast. */
+void vpo_matmul_w8g64(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                      const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int M, int rounded)
+{
+  const int Kw = K / 4, Kg = K / VPO_GROUP;
+  float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)code8(w, n, Kw, k);
+      const float v = sq + b;
+      wrow[k] = rounded ? vpo_bf16_to_f32(vpo_f32_to_bf16(v)) : v;
+    }
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      double acc = 0.0;
+      const uint16_t* xr = x + m * (size_t)K;
+      for (int k = 0; k < K; ++k) { acc += (double)vpo_bf16_to_f32(xr[k]) * (double)wrow[k]; }
+      if (y64) { y64[m * (size_t)N + n] = acc; }
+      if (y_bf16) { y_bf16[m * (size_t)N + n] = vpo_f32_to_bf16((float)acc); }
+    }
+  }
+  free(wrow);
+}
 
 /* ---- timed CPU baseline ------------------------------------------------ */
 

@@ -417,3 +417,35 @@ def test_geglu_expression_against_torch_gelu_tanh(oracle):
     assert not np.allclose(o64, oracle.swiglu(y)[0], rtol=1e-2)
     assert np.array_equal(ob, oracle.f32_to_bf16(o64.astype(np.float32)))
 
+
+# ---- 8-bit twin (w8g64) ---------------------------------------------------------------
+
+def test_w8_oracle_against_numpy_from_the_byte_view(oracle):
+    # one byte per value, little-endian within the word (affine_dequant.metal:60-67): the byte view
+    # of the words IS the code matrix
+    N, K, M = 9, 192, 3
+    w, s, b = synth.make_weight8(N, K, 70)
+    q = w.view(np.uint8).reshape(N, K).astype(np.float64)
+    sf = synth.bf16_bits_to_f32(s).astype(np.float64).repeat(64, axis=1)
+    bf = synth.bf16_bits_to_f32(b).astype(np.float64).repeat(64, axis=1)
+    W = sf * q + bf                                    # exact in float64
+    got = oracle.dequant8_bf16(w, s, b, K, N)
+    assert np.array_equal(got, synth.f32_to_bf16_bits(W.astype(np.float32)))
+    x = synth.make_act(M, K, 71)
+    xf = synth.bf16_bits_to_f32(x).astype(np.float64)
+    y_qmv, _ = oracle.matmul8(w, s, b, x, K, N, M, rounded=False)
+    Wf32 = (sf.astype(np.float32) * q.astype(np.float32) + bf.astype(np.float32)).astype(np.float64)
+    assert np.allclose(y_qmv, xf @ Wf32.T, rtol=1e-12, atol=1e-12)
+    y_qmm, _ = oracle.matmul8(w, s, b, x, K, N, M, rounded=True)
+    Wb = synth.bf16_bits_to_f32(got).astype(np.float64)
+    assert np.allclose(y_qmm, xf @ Wb.T, rtol=1e-12, atol=1e-12)
+    # one-hot activation reads back one (rounded / unrounded) weight column
+    e = np.zeros((1, K), dtype=np.float32); e[0, 77] = 1.0
+    y1, _ = oracle.matmul8(w, s, b, synth.f32_to_bf16_bits(e), K, N, 1, rounded=True)
+    assert np.array_equal(y1[0], Wb[:, 77])
+    # byte order: code 0x04030201 is q = 1, 2, 3, 4
+    w1 = np.full((1, 16), 0x04030201, dtype=np.uint32)
+    one = synth.f32_to_bf16_bits(np.ones((1, 1), dtype=np.float32))
+    zero = np.zeros((1, 1), dtype=np.uint16)
+    assert list(synth.bf16_bits_to_f32(oracle.dequant8_bf16(w1, one, zero, 64, 1))[0, :4]) == [1.0, 2.0, 3.0, 4.0]
+

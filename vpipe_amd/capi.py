@@ -47,6 +47,10 @@ SYMBOLS = [
     ("vpq_qmv_gated_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     ("vpq_qmm_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
     ("vpq_linear_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_qmv_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    ("vpq_qmv_w8g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_qmm_dense_route_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_quantize_w4g64", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
     ("vpq_f16_to_bf16", _i, [_vp, _vp, _vp, _sz]),
     ("vpq_profile_enable", _i, [_i]),
@@ -220,6 +224,40 @@ def qmm_splitk_w4g64(w, scales, biases, x, K, N, M, splits=0, ws=None, out=None)
         ws = torch.empty(need, dtype=torch.uint8, device=w.device)
     _check(L.vpq_qmm_splitk_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M, splits,
                                        _ptr(ws), ws.numel()), "vpq_qmm_splitk_w4g64_bf16")
+    return out
+
+
+def dequant_w8g64(w, scales, biases, K, N, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((N, K), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_dequant_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out), K, N),
+           "vpq_dequant_w8g64_bf16")
+    return out
+
+
+def qmv_w8g64(w, scales, biases, x, K, N, M, out=None, residual=None, f32out=False):
+    import torch
+    L = load()
+    if f32out:
+        if out is None:
+            out = torch.empty((M, N), dtype=torch.float32, device=w.device)
+        _check(L.vpq_qmv_w8g64_f32out(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M),
+               "vpq_qmv_w8g64_f32out")
+        return out
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _check(L.vpq_qmv_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                _ptr(residual)), "vpq_qmv_w8g64_bf16")
+    return out
+
+
+def qmm_dense_route_w8g64(w, scales, biases, x, K, N, M, w_deq, expand=True, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_dense_route_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                                 K, N, M, _ptr(w_deq), 1 if expand else 0), "vpq_qmm_dense_route_w8g64_bf16")
     return out
 
 

@@ -45,6 +45,38 @@ hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* sca
                        biases, reinterpret_cast<uint4*>(out), Kw, total);
 }
 
+// 8-bit twin (gpu-kernels/metal/quant/affine_dequant.metal:60-97): one byte per value, four per word;
+// one thread per word, 8-byte stores.  s*q is exact in fp32 (8-bit x 8-bit significands).
+__global__ __launch_bounds__(256) void dequant_w8g64_kernel(
+    const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
+    const uint16_t* __restrict__ biases, uint2* __restrict__ out, int Kw, size_t total_words)
+{
+  const int Kg = Kw >> 4;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total_words; idx += (size_t)gridDim.x * 256) {
+    const size_t n = idx / (size_t)Kw;
+    const int j = (int)(idx - n * (size_t)Kw);
+    const size_t g = n * (size_t)Kg + (size_t)(j >> 4);
+    const float s = bf16_bits_to_f32(scales[g]);
+    const float b = bf16_bits_to_f32(biases[g]);
+    const uint32_t p = w[idx];
+    uint2 o;
+    o.x = pack_bf16x2(fmaf(s, (float)(p & 0xffu), b), fmaf(s, (float)((p >> 8) & 0xffu), b));
+    o.y = pack_bf16x2(fmaf(s, (float)((p >> 16) & 0xffu), b), fmaf(s, (float)(p >> 24), b));
+    out[idx] = o;
+  }
+}
+
+hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           uint16_t* out, int K, int N)
+{
+  const int Kw = K / 4;
+  const size_t total = (size_t)N * (size_t)Kw;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536 * 4) { blocks = 65536 * 4; }
+  return launch_kernel(dequant_w8g64_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, scales, biases,
+                       reinterpret_cast<uint2*>(out), Kw, total);
+}
+
 // Dequantizing embedding gather (gpu-kernels/metal/ops/llm_elementwise.metal:1676-1701): out row t
 // is the dense expansion of table row ids[t]; the arithmetic is the dequant kernel's, so a
 // gathered row is bit-identical to that row of the dense table.  One thread per packed word.

@@ -79,6 +79,10 @@ hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* sca
 hipError_t launch_embed_gather(hipStream_t st, const int* ids, const uint32_t* w, const uint16_t* scales,
                                const uint16_t* biases, uint16_t* out, int H, int T, int vocab);
 hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a);
+// The 8-bit twins (one byte per value, w is [N, K/4] words): dense expansion and the general QMV kernel.
+hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           uint16_t* out, int K, int N);
+hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a);
 // Returns hipErrorInvalidValue if the shape is outside what the MFMA kernel
 // handles (the caller then falls back to the simple kernel).
 bool qmv_mfma_supports(int K, int N, int M);

@@ -117,4 +117,84 @@ hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a)
 #undef VPQ_LAUNCH
 }
 
+// 8-bit twin (affine_qmv_w8g64, gpu-kernels/metal/quant/affine_qmv.metal:3034-3050): one byte per
+// value.  Each lane takes 16 consecutive k (one 128-bit load of codes, a quarter of a group) per
+// pass over the row; otherwise the kernel above: W = fma(s, q, b) in fp32, never rounded.
+template <int MT, bool F32OUT>
+__global__ __launch_bounds__(256) void qmv_simple8_kernel(
+    const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
+    const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x, void* __restrict__ y,
+    const uint16_t* __restrict__ residual, int K, int N, int M)
+{
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + wave;
+  if (n >= N) { return; }  // wave-uniform; no barrier in this kernel
+  const int Kw = K >> 2, Kg = K >> 6;
+  const uint32_t* wrow = w + (size_t)n * Kw;
+  const uint16_t* srow = scales + (size_t)n * Kg;
+  const uint16_t* brow = biases + (size_t)n * Kg;
+
+  for (int m0 = 0; m0 < M; m0 += MT) {
+    float acc[MT];
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) { acc[mm] = 0.0f; }
+    for (int k0 = lane * 16; k0 < K; k0 += kWave * 16) {
+      const uint4 c4 = *reinterpret_cast<const uint4*>(wrow + (k0 >> 2));
+      const uint32_t codes[4] = {c4.x, c4.y, c4.z, c4.w};
+      const float s = bf16_bits_to_f32(srow[k0 >> 6]);
+      const float b = bf16_bits_to_f32(brow[k0 >> 6]);
+      float wv[16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { wv[4 * i + j] = fmaf(s, (float)((codes[i] >> (8 * j)) & 0xffu), b); }
+      }
+#pragma unroll
+      for (int mm = 0; mm < MT; ++mm) {
+        const int row = (m0 + mm < M) ? (m0 + mm) : (M - 1);
+        const uint4* xp = reinterpret_cast<const uint4*>(x + (size_t)row * K + k0);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const uint4 x4 = xp[h];
+          const uint32_t xd[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            acc[mm] = fmaf(bf16_lo_to_f32(xd[j]), wv[8 * h + 2 * j], acc[mm]);
+            acc[mm] = fmaf(bf16_hi_to_f32(xd[j]), wv[8 * h + 2 * j + 1], acc[mm]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) {
+      const float total = wave_sum(acc[mm]);
+      const int row = m0 + mm;
+      if (lane == 0 && row < M) {
+        const size_t o = (size_t)row * N + n;
+        if (F32OUT) {
+          reinterpret_cast<float*>(y)[o] = total;
+        } else {
+          uint32_t v = f32_to_bf16_bits(total);
+          if (residual != nullptr) {
+            v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(residual[o]));
+          }
+          reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)v;
+        }
+      }
+    }
+  }
+}
+
+hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a)
+{
+  const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
+#define VPQ_LAUNCH8(MT, F32)                                                                    \
+  launch_kernel(qmv_simple8_kernel<MT, F32>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
+                a.residual, a.K, a.N, a.M)
+  if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH8(1, true) : VPQ_LAUNCH8(1, false); }
+  return a.y_f32 ? VPQ_LAUNCH8(4, true) : VPQ_LAUNCH8(4, false);
+#undef VPQ_LAUNCH8
+}
+
 }  // namespace vpq
