@@ -135,7 +135,9 @@ enum {
   VPQ_QMV_MFMA = 2,        /* LDS-staged codes, bf16 MFMA on the integer codes */
   VPQ_QMV_MFMA_SPLITK = 3, /* as 2, K split across workgroups through `ws` */
   VPQ_QMV_STREAM = 4,      /* M <= 4: persistent workgroups, x staged in LDS, prefetched items */
-  VPQ_QMV_RING = 5         /* x in registers across a workgroup's tiles, codes through a two-slot LDS ring per wavefront */
+  VPQ_QMV_RING = 5,        /* x in registers across a workgroup's tiles, codes through a two-slot LDS ring per wavefront */
+  VPQ_QMV_ROWS = 6         /* M <= 2, any K % 64: a wavefront streams whole rows with full-width loads, packed bf16
+                              dot products, no LDS; what AUTO takes for M <= 2 where K is not a multiple of 512 */
 };
 
 /* ---- a6/a7/a8 (+a10): QMM ----------------------------------------------
@@ -231,9 +233,10 @@ int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t
  * case w[1] = w[0] + q_rows*K/8 words (scales, biases alike); gate|up of an
  * MLP is count = 2.  Arithmetic and requirements are those of
  * vpq_qmv_w4g64_bf16 per pack (no residual); results are bit-identical to
- * `count` separate calls of its VPQ_QMV_MFMA kernel.  The pointer tables are
- * host arrays, read before the call returns.  Shapes the grouped kernel does
- * not take (K % 512 != 0) run as separate launches. */
+ * `count` separate calls of its VPQ_QMV_MFMA kernel where K % 512 == 0, of
+ * its VPQ_QMV_ROWS kernel for other K at M <= 2.  The pointer tables are
+ * host arrays, read before the call returns.  Shapes neither grouped kernel
+ * takes (K % 512 != 0 with M > 2) run as separate launches. */
 int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,
                              const uint16_t* const* scales, const uint16_t* const* biases,
                              const uint16_t* x, uint16_t* const* y, int K, const int* N, int M);

@@ -100,6 +100,32 @@ def test_qmv_small_shapes(vpq, oracle, dev, D, K, N, M, variant):
     assert not ws[:256].any().item()                # arrival counters are left zeroed
 
 
+ROWS_SHAPES = [
+    # K, N, M: K below, at and above one pass of 2048, not a multiple of it; N not a multiple of the rows per wavefront
+    (64, 5, 1), (512, 16, 2), (1024, 33, 1), (2048, 95, 2), (3840, 16, 1), (4096, 16 * 50 + 3, 1), (5120, 64, 2),
+    (12288, 160, 1), (17408, 33, 2),
+]
+
+
+@pytest.mark.parametrize("K,N,M", ROWS_SHAPES)
+def test_qmv_row_streaming_kernel(vpq, oracle, dev, D, K, N, M):
+    w, s, b = synth.make_weight(N, K, 8000 + K + N)
+    x = synth.make_act(M, K, 8100 + K + M)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=capi.VPQ_QMV_ROWS, f32out=True)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, variant=capi.VPQ_QMV_ROWS)
+    torch.cuda.synchronize()
+    parity.check_f32(f.cpu().numpy(), y64)
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    out.assert_intact()
+    res = synth.make_act(M, N, 8200 + N)
+    got = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, residual=D.bf16(res, dev), variant=capi.VPQ_QMV_ROWS))
+    want = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(D.bits(out.view)) + synth.bf16_bits_to_f32(res))
+    assert np.array_equal(got, want)
+
+
 STREAM_SHAPES = [
     # K, N, M: one and several slices per wavefront, ragged last tile, more tiles than
     # workgroups (each workgroup walks several tiles), every M the kernel takes
@@ -301,7 +327,8 @@ def test_linear_entrance_routes_by_rows(vpq, oracle, dev, D):
 
 
 @pytest.mark.parametrize("K,Ns,M", [(4096, (4096, 1024, 1024), 1), (4096, (12288, 12288), 1), (1024, (48, 33, 16, 95), 3),
-                                    (2048, (64,), 2), (12288, (160, 4096), 16), (3840, (64, 32), 1)])
+                                    (2048, (64,), 2), (12288, (160, 4096), 16), (3840, (64, 32), 1), (3840, (64, 160, 410), 2),
+                                    (1984, (240, 80), 5)])
 def test_qmv_grouped_launch_equals_separate_launches(vpq, oracle, dev, D, K, Ns, M):
     # q|k|v and gate|up in one launch (the reference's fused QKV GEMV, affine_qmv.metal:405-516):
     # bit-identical to separate launches, and within tolerance of the oracle

@@ -46,6 +46,28 @@ QMV_SHAPES = [
 ]
 
 
+@pytest.mark.parametrize("activation", [capi.VPQ_GATE_SWIGLU, capi.VPQ_GATE_GEGLU])
+@pytest.mark.parametrize("K,F,M", [(64, 5, 1), (1984, 17, 2), (2048, 24, 1), (3840, 33, 2), (5120, 80, 1)])
+def test_qmv_gated_row_streaming_kernel(vpq, oracle, dev, D, K, F, M, activation):
+    # the row-streaming kernel's register-local (gate, up) pairs; K not a multiple of 512 is also what
+    # the automatic choice sends there
+    _, _, pack = fused_pack(oracle, F, K, 520 + K + F)
+    x = synth.make_act(M, K, 620 + K + M)
+    y64, _ = oracle.qmv(*pack, x, K, 2 * F, M)
+    o64, ob = (oracle.swiglu if activation == capi.VPQ_GATE_SWIGLU else oracle.geglu)(y64)
+    wd, sd, bd, xd = stage(D, dev, pack, x)
+    f = vpq.qmv_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, variant=capi.VPQ_QMV_ROWS, f32out=True, activation=activation)
+    out = parity.Guarded((M, F), torch.bfloat16, dev)
+    vpq.qmv_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, out=out.view, variant=capi.VPQ_QMV_ROWS, activation=activation)
+    torch.cuda.synchronize()
+    parity.check_f32(f.cpu().numpy(), o64)
+    parity.check_bf16(D.bits(out.view), o64, ob, mismatch_over_all=activation == capi.VPQ_GATE_SWIGLU)
+    out.assert_intact()
+    if K % 512 != 0:
+        auto = vpq.qmv_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, variant=AUTO, activation=activation)
+        assert torch.equal(auto, out.view)
+
+
 @pytest.mark.parametrize("variant", [SIMPLE, MFMA, RING, AUTO])
 @pytest.mark.parametrize("K,F,M", QMV_SHAPES)
 def test_qmv_swiglu(vpq, oracle, dev, D, K, F, M, variant):

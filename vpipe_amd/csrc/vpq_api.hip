@@ -88,7 +88,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
   if (ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }
-  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_RING) { return VPQ_ERR_BAD_SHAPE; }
+  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_ROWS) { return VPQ_ERR_BAD_SHAPE; }
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
 
@@ -101,6 +101,10 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
 
   const bool mfma_ok = vpq::qmv_mfma_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
   if (variant == VPQ_QMV_SIMPLE) { return finish(vpq::launch_qmv_simple(hs, a)); }
+  if (variant == VPQ_QMV_ROWS) {
+    if (!vpq::qmv_rows_supports(K, N, M) || (gate_act != 0 && (N & 1) != 0)) { return VPQ_ERR_BAD_SHAPE; }
+    return finish(vpq::launch_qmv_rows(hs, a, 0));
+  }
   if (variant == VPQ_QMV_RING) {
     if (!mfma_ok || !vpq::qmv_ring_supports(K, N, M)) { return VPQ_ERR_BAD_SHAPE; }
     return finish(vpq::launch_qmv_ring(hs, a, 0, 0));
@@ -139,6 +143,9 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
     if (M >= 3 || even) { return finish(vpq::launch_qmv_ring(hs, a, 0, 0)); }
   }
   if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a, 1)); }
+  // K not a multiple of 512, or scales / biases off 16-byte alignment: the row-streaming kernel
+  // for up to two rows of x, the general one above.
+  if (vpq::qmv_rows_supports(K, N, M)) { return finish(vpq::launch_qmv_rows(hs, a, 0)); }
   return finish(vpq::launch_qmv_simple(hs, a));
 }
 
@@ -511,18 +518,19 @@ int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* con
 {
   if (w == nullptr || scales == nullptr || biases == nullptr || y == nullptr || N == nullptr) { return VPQ_ERR_NULL_POINTER; }
   if (count < 1 || count > 4) { return VPQ_ERR_BAD_SHAPE; }
-  bool grouped = vpq::qmv_mfma_supports(K, 1, M) && x != nullptr && aligned(x, 16);
+  // The tile kernel's grouped form where its shapes allow, else the row-streaming kernel's (M <= 2).
+  bool mfma_group = vpq::qmv_mfma_supports(K, 1, M);
   for (int i = 0; i < count; ++i) {
     int st = check_pack(w[i], scales[i], biases[i], K, N[i]);
     if (st != VPQ_OK) { return st; }
     if (y[i] == nullptr) { return VPQ_ERR_NULL_POINTER; }
     if (!aligned(y[i], 2)) { return VPQ_ERR_MISALIGNED; }
-    grouped = grouped && aligned(scales[i], 16) && aligned(biases[i], 16);
+    mfma_group = mfma_group && aligned(scales[i], 16) && aligned(biases[i], 16);
   }
   if (x == nullptr) { return VPQ_ERR_NULL_POINTER; }
   if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16)) { return VPQ_ERR_MISALIGNED; }
-  if (!grouped) {
+  if (!mfma_group && !vpq::qmv_rows_supports(K, 1, M)) {
     for (int i = 0; i < count; ++i) {
       const int st = vpq_qmv_w4g64_bf16(stream, w[i], scales[i], biases[i], x, y[i], K, N[i], M, nullptr, nullptr, 0,
                                         VPQ_QMV_AUTO);
@@ -537,6 +545,7 @@ int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* con
   vpq::QmvGroup g;
   g.count = count;
   for (int i = 0; i < count; ++i) { g.seg[i] = vpq::QmvSeg{w[i], scales[i], biases[i], y[i], N[i]}; }
+  if (!mfma_group) { return finish(vpq::launch_qmv_rows_group(reinterpret_cast<hipStream_t>(stream), a, g)); }
   return finish(vpq::launch_qmv_mfma_group(reinterpret_cast<hipStream_t>(stream), a, g));
 }
 

@@ -107,6 +107,10 @@ hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);
 bool qmv_ring_supports(int K, int N, int M);
 // tc_hint / nw_hint > 0 force the tiles / wavefronts per workgroup (measurement only).
 hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint);
+// Row-streaming kernel (M <= 2, any K % 64): rows_per_wave in {2, 4}, 0 = default.
+bool qmv_rows_supports(int K, int N, int M);
+hipError_t launch_qmv_rows(hipStream_t st, const QmvArgs& a, int rows_per_wave);
+hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g);
 // t[M,r] = bf16(alpha * bf16(x . A^T)), r in {32, 64, 96, 128}.
 hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
                          float alpha);

@@ -23,7 +23,6 @@
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
-#include <stdlib.h>
 
 namespace vpq {
 
