@@ -490,6 +490,38 @@ def main():
             del packs
         out["qmv_w8g64_m1"] = w8
 
+        # MoE decode block, pair-batched gathers (hidden 2048, expert inner 768, 128 experts, top-8,
+        # one token): 8 of the 128 gate|up slabs and 8 down slabs per step, a fresh random set of
+        # experts each launch over two layers' batches (679 MB, so the slabs come from HBM)
+        H, I, E, top_k = 2048, 768, 128, 8
+        batches = []
+        for _ in range(2):
+            gw = torch.randint(-2 ** 31, 2 ** 31 - 1, (E, 2 * I, H // 8), dtype=torch.int32, device=dev, generator=gen)
+            gs = torch.empty((E, 2 * I, H // 64), dtype=torch.float32, device=dev).uniform_(0.005, 0.02, generator=gen).bfloat16()
+            dw = torch.randint(-2 ** 31, 2 ** 31 - 1, (E, H, I // 8), dtype=torch.int32, device=dev, generator=gen)
+            ds = torch.empty((E, H, I // 64), dtype=torch.float32, device=dev).uniform_(0.005, 0.02, generator=gen).bfloat16()
+            batches.append((gw, gs, (-8.0 * gs.float()).bfloat16(), dw, ds, (-8.0 * ds.float()).bfloat16()))
+        ids = [torch.randperm(E, device=dev, generator=gen)[:top_k].to(torch.int32).contiguous() for _ in range(16)]
+        xm = torch.randn((1, H), device=dev, generator=gen).bfloat16()
+        actm = torch.empty((top_k, I), dtype=torch.bfloat16, device=dev)
+        partm = torch.empty((top_k, H), dtype=torch.bfloat16, device=dev)
+
+        def call_gu(i):
+            gw, gs, gb, _, _, _ = batches[i % 2]
+            vpipe_amd.gather_qmv_gated_w4g64(gw, gs, gb, xm, H, 2 * I, ids[i % 16], top_k, E, out=actm)
+
+        def call_dn(i):
+            _, _, _, dw, ds, db = batches[i % 2]
+            vpipe_amd.gather_down_qmv_w4g64(dw, ds, db, actm, I, H, ids[i % 16], E, out=partm)
+        us_gu = kernel_us(call_gu, 16)
+        us_dn = kernel_us(call_dn, 16)
+        b_gu = top_k * (2 * I * H * 9 // 16) + 2 * H + 2 * top_k * I
+        b_dn = top_k * (H * I * 9 // 16) + 2 * top_k * (I + H)
+        out["moe_gather_decode_top8_of_128"] = {
+            "gate|up+swiglu 2048->2x768": {"us": round(us_gu, 2), "GBps": round(b_gu / (us_gu * 1e-6) / 1e9, 1)},
+            "down 768->2048": {"us": round(us_dn, 2), "GBps": round(b_dn / (us_dn * 1e-6) / 1e9, 1)}}
+        del batches
+
     # ---- CPU baseline: the oracle's dequant + fp32 matmul on the host cores ------------
     if not args.no_cpu:
         from oracle import oracle

@@ -307,6 +307,36 @@ int vpq_linear_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const ui
                                 const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                 int K, int N, int M, int activation);
 
+/* ---- MoE: gathered expert projections (decode and pair-batched prefill) ----
+ * The router picks top_k of n_experts experts per token: npair = M*top_k
+ * (token, expert) pairs in the order token*top_k + slot, pair_eid[p] (device,
+ * int32) the expert of pair p.  An expert tensor is a BATCH of packs
+ * [n_experts, N, K/8] (scales, biases [n_experts, N, K/64]); one launch runs
+ * the QMV of every pair against its expert's slab
+ * (generative-models/qwen3/metal-qwen-model.cc:4190-4206).
+ *
+ * vpq_gather_qmv_gated_w4g64_bf16 replaces `affine_gather_qmv_swiglu_w4g64`
+ * (gpu-kernels/metal/quant/affine_qmv.metal:928-960; slots 0:w 1:scales
+ * 2:biases 3:x[M,K] 4:y[npair,N/2] 5:K 6:N=2*inner 7:pair_eid 8:top_k) and
+ * `affine_gather_qmv_geglu_w4g64` (:1494-1522): pair p contracts the
+ * interleaved gate|up slab of expert pair_eid[p] with x row p / top_k and
+ * stores act(gate)*up into y row p.
+ * vpq_gather_down_qmv_w4g64_bf16 replaces `affine_gather_down_qmv_w4g64`
+ * (:1265-1292; slots 0..6 the same with x[npair,K], y[npair,N], 7:pair_eid):
+ * pair p contracts the down slab with x row p into y row p, un-weighted (the
+ * routing weight is applied by the combine that follows).
+ * QMV arithmetic; a pair's result is bit-identical to the plain call
+ * (VPQ_QMV_ROWS) on that expert's slab and that row of x.  A pair whose id is
+ * outside [0, n_experts) gets zeros (the reference reads out of bounds there).
+ * Requires K % 64 == 0, 1 <= npair <= 65535, top_k >= 1, N even for the gated
+ * form; w, x 16-byte aligned. */
+int vpq_gather_qmv_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                    const int32_t* pair_eid, int npair, int top_k, int n_experts, int activation);
+int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                   const int32_t* pair_eid, int npair, int n_experts);
+
 /* ---- 8-bit group-64 twins (w8g64) -------------------------------------------
  * The same affine format with one BYTE per value: w uint32 [N, K/4],
  * q[n, 4j+i] = (w[n,j] >> 8i) & 0xFF; scales, biases bf16 [N, K/64]

@@ -407,3 +407,52 @@ def test_embedding_gather_call_site(enc, oracle, dev, D):
     assert ok, why
     assert np.array_equal(D.bits(out), oracle.embed_gather(ids, w, s, b, H, vocab))
 
+
+
+def test_moe_gathered_expert_call_sites(enc, oracle, dev, D):
+    # Qwen MoE block, pair-batched (generative-models/qwen3/metal-qwen-model.cc:4190-4206):
+    # gathered gate|up + SwiGLU -> act[np, I] (slots 0..4, 5:H 6:2*I 7:eid 8:top_k, grid {32, I/2, np}),
+    # then gathered down -> part[np, H] (5:I 6:H 7:eid, grid {32, H/4, np}); tg {32, 2, 1}
+    H, I, E, top_k, M = 1024, 128, 6, 3, 2
+    npair = M * top_k
+    gu = [synth.make_weight(2 * I, H, 900 + e) for e in range(E)]
+    dn = [synth.make_weight(H, I, 950 + e) for e in range(E)]
+    guw, gus, gub = (np.stack([p[i] for p in gu]) for i in range(3))
+    dw, ds, db = (np.stack([p[i] for p in dn]) for i in range(3))
+    x = synth.make_act(M, H, 990)
+    eid = np.array([4, 0, 5, 1, 4, 2], dtype=np.int32)
+    eidd = torch.from_numpy(eid).to(dev)
+    act = torch.zeros((npair, I), dtype=torch.bfloat16, device=dev)
+    part = torch.zeros((npair, H), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_qmv_bf16", "affine_gather_qmv_swiglu_w4g64") == 1
+    for i, t in enumerate((D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev), act)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, H)
+    enc.set_constant(6, 2 * I)
+    enc.set_buffer(7, eidd)
+    enc.set_constant(8, top_k)
+    enc.dispatch((32, I // 2, npair), (32, 2, 1))
+    assert enc.set_function("affine_qmv_bf16", "affine_gather_down_qmv_w4g64") == 1
+    for i, t in enumerate((D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), act, part)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, I)
+    enc.set_constant(6, H)
+    enc.set_buffer(7, eidd)
+    enc.dispatch((32, H // 4, npair), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    act_bits = D.bits(act)
+    a64 = np.empty((npair, I))
+    ab = np.empty((npair, I), dtype=np.uint16)
+    p64 = np.empty((npair, H))
+    pb = np.empty((npair, H), dtype=np.uint16)
+    for p in range(npair):
+        e, t = int(eid[p]), p // top_k
+        y64, _ = oracle.qmv(guw[e], gus[e], gub[e], x[t:t + 1], H, 2 * I, 1)
+        o64, ob = oracle.swiglu(y64)
+        a64[p], ab[p] = o64[0], ob[0]
+        # the down projection reads the activation the device produced
+        d64, dbits = oracle.qmv(dw[e], ds[e], db[e], act_bits[p:p + 1], I, H, 1)
+        p64[p], pb[p] = d64[0], dbits[0]
+    parity.check_bf16(act_bits, a64, ab)
+    parity.check_bf16(D.bits(part), p64, pb)

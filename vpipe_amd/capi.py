@@ -28,6 +28,8 @@ SYMBOLS = [
     ("vpq_device_cu_count", _i, []),
     ("vpq_dequant_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_embed_gather_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_gather_qmv_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
+    ("vpq_gather_down_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i]),
     ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
     ("vpq_qmv_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _i]),
     ("vpq_qmv_workspace_bytes", _sz, [_i, _i, _i]),
@@ -127,6 +129,29 @@ def embed_gather_w4g64(ids, w, scales, biases, H, vocab, out=None):
         out = torch.empty((T, H), dtype=torch.bfloat16, device=w.device)
     _check(load().vpq_embed_gather_w4g64_bf16(_stream(), _ptr(ids), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out),
                                               H, T, vocab), "vpq_embed_gather_w4g64_bf16")
+    return out
+
+
+def gather_qmv_gated_w4g64(w, scales, biases, x, K, N, pair_eid, top_k, n_experts, out=None, activation=VPQ_GATE_SWIGLU):
+    """Expert batch [E, N=2*inner, ...], x [M, K], pair_eid int32 [npair] -> bf16 [npair, N/2]."""
+    import torch
+    npair = pair_eid.numel()
+    if out is None:
+        out = torch.empty((npair, N // 2), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_gather_qmv_gated_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                  _ptr(pair_eid), npair, top_k, n_experts, activation),
+           "vpq_gather_qmv_gated_w4g64_bf16")
+    return out
+
+
+def gather_down_qmv_w4g64(w, scales, biases, x, K, N, pair_eid, n_experts, out=None):
+    """Expert batch [E, N, ...], x [npair, K], pair_eid int32 [npair] -> bf16 [npair, N]."""
+    import torch
+    npair = pair_eid.numel()
+    if out is None:
+        out = torch.empty((npair, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_gather_down_qmv_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                 _ptr(pair_eid), npair, n_experts), "vpq_gather_down_qmv_w4g64_bf16")
     return out
 
 

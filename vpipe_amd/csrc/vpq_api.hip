@@ -512,6 +512,45 @@ int vpq_linear_swiglu_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const u
   return vpq_linear_gated_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, VPQ_GATE_SWIGLU);
 }
 
+namespace {
+
+int gather_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                  const uint16_t* x, uint16_t* y, int K, int N, const int32_t* pair_eid, int npair, int x_div,
+                  int n_experts, int gate_act)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr || pair_eid == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (npair < 1 || npair > 65535 || x_div < 1 || n_experts < 1) { return VPQ_ERR_BAD_SHAPE; }
+  if (gate_act != 0 && (N & 1) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  // every slab and every row of x must keep the 16-byte alignment of the base
+  if (!aligned(x, 16) || !aligned(y, 2) || !aligned(pair_eid, 4)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y;
+  a.K = K; a.N = N; a.M = 1; a.y_f32 = false; a.cu_count = g_dev.cu_count;
+  a.gate_act = gate_act;
+  return finish(vpq::launch_qmv_rows_gather(reinterpret_cast<hipStream_t>(stream), a, pair_eid, npair, x_div, n_experts));
+}
+
+}  // namespace
+
+int vpq_gather_qmv_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                    const int32_t* pair_eid, int npair, int top_k, int n_experts, int activation)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return gather_common(stream, w, scales, biases, x, y, K, N, pair_eid, npair, top_k, n_experts, activation);
+}
+
+int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                   const int32_t* pair_eid, int npair, int n_experts)
+{
+  return gather_common(stream, w, scales, biases, x, y, K, N, pair_eid, npair, 1, n_experts, 0);
+}
+
 int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,
                              const uint16_t* const* scales, const uint16_t* const* biases,
                              const uint16_t* x, uint16_t* const* y, int K, const int* N, int M)

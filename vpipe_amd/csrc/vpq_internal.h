@@ -111,6 +111,11 @@ hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw
 bool qmv_rows_supports(int K, int N, int M);
 hipError_t launch_qmv_rows(hipStream_t st, const QmvArgs& a, int rows_per_wave);
 hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g);
+// Gathered (MoE) form, M = 1 per pair: a.w/scales/biases are batches [E, N, ...] of expert slabs,
+// pair p contracts slab pair_eid[p] with x row p / x_div into y row p (zeros for an id outside
+// [0, n_experts)); a.gate_act as in the plain form.
+hipError_t launch_qmv_rows_gather(hipStream_t st, const QmvArgs& a, const int* pair_eid, int pairs, int x_div,
+                                  int n_experts);
 // t[M,r] = bf16(alpha * bf16(x . A^T)), r in {32, 64, 96, 128}.
 hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
                          float alpha);

@@ -14,6 +14,14 @@
 // per row and pass, then one wave reduction per row.  The gated stores (SwiGLU / GEGLU over an
 // interleaved gate|up pack) are register-local: R is even, so a (gate, up) pair of rows belongs
 // to one wavefront.
+//
+// K <= 1024 leaves half of a 2048-wide pass idle, so there a row group takes 32 lanes and a
+// wavefront carries two of them (LPR = 32); the lanes past K hold zeros in the 64-lane form, so the
+// sums -- a butterfly from the widest step down -- are the same bits either way.
+//
+// Gathered form (MoE, gpu-kernels/metal/quant/affine_qmv.metal:908-962, 1262-1292): grid.y is a
+// (token, expert) pair p; the pack is a batch [E, N, K/8] of expert slabs and pair_eid[p] picks
+// the slab, x row p / x_div (gate|up: top_k pairs share a token's row) or p (down), y row p.
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -23,7 +31,6 @@ namespace {
 
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 
-constexpr int kPassK = kWave * 32;     // k-values a wavefront covers per pass (2048)
 
 __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c)
 {
@@ -46,10 +53,18 @@ struct RowsSegs {
   RowsSeg seg[4];
 };
 
-// R rows per wavefront, four wavefronts (4R rows) per workgroup, MT rows of x.
-template <int R, int MT, bool F32OUT>
+// Gathered launches: null pair_eid for the plain forms.
+struct RowsGather {
+  const int* pair_eid;
+  int x_div;        // x row of pair p is p / x_div
+  int n_experts;    // ids outside [0, n_experts) give zeros
+};
+
+// R rows per row group, 64 / LPR row groups per wavefront, four wavefronts per workgroup, MT rows of x.
+template <int R, int MT, bool F32OUT, int LPR>
 __global__ __launch_bounds__(256) void qmv_rows_kernel(
-    const RowsSegs g, const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, int K, int M, int gate_act)
+    const RowsSegs g, const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, int K, int M, int gate_act,
+    const RowsGather gather)
 {
   RowsSeg sg = g.seg[0];
 #pragma unroll
@@ -61,11 +76,27 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
   const uint16_t* __restrict__ biases = sg.biases;
   void* __restrict__ y = sg.y;
   const int N = sg.N;
+  constexpr int SUBS = kWave / LPR;      // row groups per wavefront
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int n0 = (((int)blockIdx.x - sg.first_block) * 4 + wave) * R;
-  if (n0 >= N) { return; }              // wave-uniform; the kernel has no barrier
+  const int sub = lane / LPR, ll = lane % LPR;
+  const int nw = (((int)blockIdx.x - sg.first_block) * 4 + wave) * SUBS * R;
+  if (nw >= N) { return; }              // wave-uniform; the kernel has no barrier
+  const int n0 = nw + sub * R;
   const int Kw = K >> 3, Kg = K >> 6;
+  bool expert_ok = true;
+  if (gather.pair_eid != nullptr) {
+    const int p = (int)blockIdx.y;
+    int e = gather.pair_eid[p];
+    expert_ok = e >= 0 && e < gather.n_experts;
+    e = expert_ok ? e : 0;
+    w += (size_t)e * (size_t)N * Kw;
+    scales += (size_t)e * (size_t)N * Kg;
+    biases += (size_t)e * (size_t)N * Kg;
+    x += (size_t)(p / gather.x_div) * K;
+    const size_t yo = (size_t)p * (size_t)(gate_act ? (N >> 1) : N);
+    y = F32OUT ? (void*)(reinterpret_cast<float*>(y) + yo) : (void*)(reinterpret_cast<uint16_t*>(y) + yo);
+  }
 
   uint32_t magic = 0x43004300u;         // bf16 128.0 in both halves
   uint32_t mask = 0x000f000fu;
@@ -150,10 +181,10 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
     }
   };
 
-  // The wavefront's passes: k0 = lane*32, then every 2048.  The next pass is fetched before the
+  // The row group's passes: k0 = ll*32, then every LPR*32.  The next pass is fetched before the
   // current one is contracted.
-  constexpr int kStep = kPassK;
-  int k0 = lane * 32;
+  constexpr int kStep = LPR * 32;
+  int k0 = ll * 32;
   if (k0 < K) {
     Pass cur;
     fetch(k0, cur);
@@ -176,9 +207,14 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) { total[m][r] = wave_sum(acc[r][m]); }
+    for (int r = 0; r < R; ++r) {
+      float v = acc[r][m];
+#pragma unroll
+      for (int off = LPR / 2; off >= 1; off >>= 1) { v += __shfl_xor(v, off, kWave); }
+      total[m][r] = expert_ok ? v : 0.0f;
+    }
   }
-  if (lane != 0) { return; }
+  if (ll != 0) { return; }
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
     if (m >= M) { continue; }
@@ -222,25 +258,29 @@ bool qmv_rows_supports(int K, int N, int M)
 
 namespace {
 
-hipError_t launch_rows_segments(hipStream_t st, RowsSegs& g, const QmvArgs& a, int rows_per_wave)
+hipError_t launch_rows_segments(hipStream_t st, RowsSegs& g, const QmvArgs& a, int rows_per_wave,
+                                const RowsGather& gather, int pairs)
 {
   double bytes = 0.0;
   for (int i = 0; i < g.count; ++i) { bytes += (double)g.seg[i].N * (double)a.K * 9.0 / 16.0; }
-  // Two rows per wavefront finish sooner on layer-sized packs (more, shorter wavefronts: 4096->4096
+  // Two rows per row group finish sooner on layer-sized packs (more, shorter wavefronts: 4096->4096
   // 4.3 vs 4.4 us, 5120->5120 6.6 vs 7.1, 17408->5120 14.7 vs 15.9); four on lm_head-sized ones,
   // where x is re-read half as often (5120->151936: 94 vs 100 us).
   const int R = rows_per_wave == 2 || rows_per_wave == 4 ? rows_per_wave : (bytes >= 150e6 ? 4 : 2);
+  const bool half = a.K <= 1024 && a.M == 1 && R == 2;      // 32 lanes per row group
+  const int rows_per_block = 4 * R * (half ? 2 : 1);
   int blocks = 0;
   for (int i = 0; i < g.count; ++i) {
     g.seg[i].first_block = blocks;
-    blocks += (g.seg[i].N + 4 * R - 1) / (4 * R);
+    blocks += (g.seg[i].N + rows_per_block - 1) / rows_per_block;
   }
-  const dim3 grid((unsigned)blocks), block(256);
-#define VPQ_ROWS(RR, MT, F32) \
-  launch_kernel(qmv_rows_kernel<RR, MT, F32>, grid, block, 0, st, g, a.x, a.residual, a.K, a.M, a.gate_act)
-#define VPQ_ROWS_M(RR)                                                               \
-  (a.M == 1 ? (a.y_f32 ? VPQ_ROWS(RR, 1, true) : VPQ_ROWS(RR, 1, false))             \
-            : (a.y_f32 ? VPQ_ROWS(RR, 2, true) : VPQ_ROWS(RR, 2, false)))
+  const dim3 grid((unsigned)blocks, (unsigned)pairs), block(256);
+#define VPQ_ROWS(RR, MT, F32, LPR) \
+  launch_kernel(qmv_rows_kernel<RR, MT, F32, LPR>, grid, block, 0, st, g, a.x, a.residual, a.K, a.M, a.gate_act, gather)
+#define VPQ_ROWS_M(RR)                                                                       \
+  (a.M == 1 ? (a.y_f32 ? VPQ_ROWS(RR, 1, true, 64) : VPQ_ROWS(RR, 1, false, 64))             \
+            : (a.y_f32 ? VPQ_ROWS(RR, 2, true, 64) : VPQ_ROWS(RR, 2, false, 64)))
+  if (half) { return a.y_f32 ? VPQ_ROWS(2, 1, true, 32) : VPQ_ROWS(2, 1, false, 32); }
   return R == 2 ? VPQ_ROWS_M(2) : VPQ_ROWS_M(4);
 #undef VPQ_ROWS_M
 #undef VPQ_ROWS
@@ -253,7 +293,7 @@ hipError_t launch_qmv_rows(hipStream_t st, const QmvArgs& a, int rows_per_wave)
   RowsSegs g{};
   g.count = 1;
   g.seg[0] = RowsSeg{a.w, a.scales, a.biases, a.y, a.N, 0};
-  return launch_rows_segments(st, g, a, rows_per_wave);
+  return launch_rows_segments(st, g, a, rows_per_wave, RowsGather{nullptr, 1, 0}, 1);
 }
 
 hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGroup& grp)
@@ -263,7 +303,16 @@ hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGrou
   for (int i = 0; i < grp.count; ++i) {
     g.seg[i] = RowsSeg{grp.seg[i].w, grp.seg[i].scales, grp.seg[i].biases, grp.seg[i].y, grp.seg[i].N, 0};
   }
-  return launch_rows_segments(st, g, a, 0);
+  return launch_rows_segments(st, g, a, 0, RowsGather{nullptr, 1, 0}, 1);
+}
+
+hipError_t launch_qmv_rows_gather(hipStream_t st, const QmvArgs& a, const int* pair_eid, int pairs, int x_div,
+                                  int n_experts)
+{
+  RowsSegs g{};
+  g.count = 1;
+  g.seg[0] = RowsSeg{a.w, a.scales, a.biases, a.y, a.N, 0};
+  return launch_rows_segments(st, g, a, 2, RowsGather{pair_eid, x_div, n_experts}, pairs);
 }
 
 }  // namespace vpq

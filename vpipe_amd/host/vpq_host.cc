@@ -90,6 +90,9 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_geglu_w4g64", QuantKernel::QmvGeglu},
     {"affine_qmm_steel_bf16", "affine_qmm_geglu_w4g64", QuantKernel::QmmGeglu},
     {"llm_elementwise_bf16", "dequant_embed_gather_f16", QuantKernel::EmbedGather},
+    {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w4g64", QuantKernel::GatherSwiglu},
+    {"affine_qmv_bf16", "affine_gather_qmv_geglu_w4g64", QuantKernel::GatherGeglu},
+    {"affine_qmv_bf16", "affine_gather_down_qmv_w4g64", QuantKernel::GatherDown},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm128", QuantKernel::QmmSwiglu},
@@ -410,7 +413,30 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
       const uint16_t* x = static_cast<const uint16_t*>(buf(3));
       uint16_t* y = static_cast<uint16_t*>(buf(4));
       const int K = ival(5), N = ival(6);
-      if (kind == QuantKernel::Qmm) {
+      if (kind == QuantKernel::GatherSwiglu || kind == QuantKernel::GatherGeglu || kind == QuantKernel::GatherDown) {
+        // gpu-kernels/metal/quant/affine_qmv.metal:928-960, 1265-1292, 1494-1522: slot 7 = pair_eid,
+        // 8 = top_k (gate|up only), one (token, expert) pair per grid.z
+        // (generative-models/qwen3/metal-qwen-model.cc:4190-4206).  The expert count is not a slot:
+        // it is the number of [N, K/8] slabs the bound code buffer holds.
+        const bool down = kind == QuantKernel::GatherDown;
+        if (!buf(7) || (!down && !has_int(8))) {
+          status = VPQ_ERR_NULL_POINTER;
+        } else if (K <= 0 || N <= 0 || K % 64 != 0) {
+          status = VPQ_ERR_BAD_SHAPE;
+        } else {
+          const std::size_t slab = static_cast<std::size_t>(N) * static_cast<std::size_t>(K / 2);
+          const std::size_t experts = _slots[0].bytes / slab;
+          const int E = experts > 0x7fffffffu ? 0x7fffffff : static_cast<int>(experts);
+          const int npair = static_cast<int>(grid.z);
+          const int32_t* eid = static_cast<const int32_t*>(buf(7));
+          if (down) {
+            status = vpq_gather_down_qmv_w4g64_bf16(st, w, sc, bi, x, y, K, N, eid, npair, E);
+          } else {
+            status = vpq_gather_qmv_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, eid, npair, ival(8), E,
+                                                     kind == QuantKernel::GatherGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
+          }
+        }
+      } else if (kind == QuantKernel::Qmm) {
         if (!has_int(7)) {
           status = VPQ_ERR_NULL_POINTER;
         } else {

@@ -81,6 +81,10 @@ enum class QuantKernel : std::uint8_t {
   QmmGeglu,       // affine_qmm_geglu_w4g64: as QmmSwiglu
   EmbedGather,    // dequant_embed_gather_f16: slots 0:ids 1:w 2:scales 3:biases 4:out 5:H; T = grid.y,
                   //   the vocabulary size is what the bound code buffer holds
+  GatherSwiglu,   // affine_gather_qmv_swiglu_w4g64: expert batch [E, 2*inner, ...], slot 7 = pair_eid buffer,
+                  //   8 = top_k; pairs = grid.z; the expert count is what the bound code buffer holds
+  GatherGeglu,    // affine_gather_qmv_geglu_w4g64: as GatherSwiglu
+  GatherDown,     // affine_gather_down_qmv_w4g64: x [npair, K], slot 7 = pair_eid buffer; pairs = grid.z
 };
 
 class QuantFunction {
