@@ -490,6 +490,13 @@ def main():
             del packs
         out["qmv_w8g64_m1"] = w8
 
+        # greedy tail: argmax over the lm_head's 151936 bf16 logits (both launches of the two-stage form)
+        lg = torch.randn((1, 151936), device=dev, generator=gen).bfloat16()
+        tok = torch.empty((1,), dtype=torch.int32, device=dev)
+        out["argmax_v151936"] = {
+            "two_stage_us": round(kernel_us(lambda i: vpipe_amd.argmax_bf16(lg, out=tok, two_stage=True), 16), 2),
+            "one_workgroup_us": round(kernel_us(lambda i: vpipe_amd.argmax_bf16(lg, out=tok, two_stage=False), 16), 2)}
+
         # MoE decode block, pair-batched gathers (hidden 2048, expert inner 768, 128 experts, top-8,
         # one token): 8 of the 128 gate|up slabs and 8 down slabs per step, a fresh random set of
         # experts each launch over two layers' batches (679 MB, so the slabs come from HBM)

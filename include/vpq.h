@@ -337,6 +337,27 @@ int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
                                    const int32_t* pair_eid, int npair, int n_experts);
 
+/* ---- greedy tail: argmax of the lm_head's logits on the device ------------------
+ * Replaces `argmax_f16` (gpu-kernels/metal/ops/llm_elementwise.metal:2906-2941;
+ * slots 0:logits 1:out_id 2:V), and the two-stage pair `argmax_partial_f16`
+ * (:2977-3028; 0:logits 1:partials 2:V 3:M) + `argmax_combine_f16` (:3030-3062;
+ * 0:partials 1:out_id 2:M), which keep the sampled token on the device: out_id
+ * is read back by the next step's embedding gather as its `ids`.
+ * out_id[r] = index of the largest of the V bf16 logits of row r, the LOWEST
+ * index among equal maxima (a left-to-right `v > best` scan), a NaN never
+ * wins; 0 for a row of nothing but NaNs.  Exact, whatever the reduction order.
+ *   vpq_argmax_bf16          logits [rows, V] -> out_id [rows].  With ws == NULL one
+ *                            workgroup scans a row; with vpq_argmax_workspace_bytes(V, rows)
+ *                            bytes of ws (4-byte aligned) a row is scanned by slabs and combined.
+ *   vpq_argmax_partial_bf16  one row: `parts` (1..65535) contiguous slabs -> partials, 2*parts
+ *                            4-byte slots (value as fp32, index as int32; opaque to the caller).
+ *   vpq_argmax_combine       partials of one row -> out_id[0]. */
+size_t vpq_argmax_workspace_bytes(int V, int rows);
+int vpq_argmax_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, int rows,
+                    void* ws, size_t ws_bytes);
+int vpq_argmax_partial_bf16(vpq_stream_t stream, const uint16_t* logits, float* partials, int V, int parts);
+int vpq_argmax_combine(vpq_stream_t stream, const float* partials, int32_t* out_id, int parts);
+
 /* ---- 8-bit group-64 twins (w8g64) -------------------------------------------
  * The same affine format with one BYTE per value: w uint32 [N, K/4],
  * q[n, 4j+i] = (w[n,j] >> 8i) & 0xFF; scales, biases bf16 [N, K/64]

@@ -117,6 +117,17 @@ def embed_gather(ids, w, s, b, H, vocab):
     return out
 
 
+def argmax(logits):
+    """bf16 bits [rows, V] -> int32 [rows]: lowest index of the largest non-NaN logit (0 if there is none)."""
+    logits = _c(logits, np.uint16)
+    if logits.ndim == 1:
+        logits = logits.reshape(1, -1)
+    rows, V = logits.shape
+    out = np.empty((rows,), dtype=np.int32)
+    lib().vpo_argmax_bf16(_p(logits, _u16p), out.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), V, rows)
+    return out
+
+
 def qmv(w, s, b, x, K, N, M, residual=None):
     """-> (y64 [M,N] float64, y_bf16 [M,N] uint16); un-rounded-weight semantics."""
     w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)

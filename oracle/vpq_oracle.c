@@ -202,6 +202,26 @@ void vpo_embed_gather_w4g64_bf16(const int32_t* ids, const uint32_t* w, const ui
   }
 }
 
+/* Greedy argmax of a row of logits, gpu-kernels/metal/ops/llm_elementwise.metal:2906-2941: the
+ * result of its strided scans and its lowest-index tie-break is the one of a left-to-right scan
+ * that takes an entry only when it is strictly greater -- the lowest index among the maxima; a
+ * NaN compares false and never wins; best starts at -inf with index 0.  An entry equal to -inf is
+ * taken over the initial index by the two-stage twin (:2995-3000: `val == best && i < bi`), which is
+ * what is restated here, so a leading NaN is never the answer while a finite or -inf entry exists. */
+void vpo_argmax_bf16(const uint16_t* logits, int32_t* out_id, int V, int rows)
+{
+  for (int r = 0; r < rows; ++r) {
+    const uint16_t* src = logits + (size_t)r * (size_t)V;
+    float best = -INFINITY;
+    int bi = -1;
+    for (int i = 0; i < V; ++i) {
+      const float v = vpo_bf16_to_f32(src[i]);
+      if (v > best || (bi < 0 && v == best)) { best = v; bi = i; }
+    }
+    out_id[r] = bi < 0 ? 0 : bi;
+  }
+}
+
 /* ---- a2/a3: QMV -------------------------------------------------------- */
 
 /* The CPU reference loop of the reference's own QMV test,

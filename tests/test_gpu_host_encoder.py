@@ -456,3 +456,33 @@ def test_moe_gathered_expert_call_sites(enc, oracle, dev, D):
         p64[p], pb[p] = d64[0], dbits[0]
     parity.check_bf16(act_bits, a64, ab)
     parity.check_bf16(D.bits(part), p64, pb)
+
+
+def test_argmax_call_sites_of_the_host_layer(enc, oracle, dev, D):
+    # the pipelined decode loop's tail (generative-models: argmax_partial_f16 + argmax_combine_f16 over the
+    # lm_head's logits, or the single-threadgroup argmax_f16); grids as the reference dispatches them
+    V, M = 151936, 64
+    bits = synth.f32_to_bf16_bits(np.random.default_rng(5200).integers(-30, 30, size=(1, V)).astype(np.float32) / 2.0)
+    logits = D.bf16(bits, dev)
+    want = int(oracle.argmax(bits)[0])
+    out = torch.full((2,), -1, dtype=torch.int32, device=dev)
+    partials = torch.zeros((2 * M,), dtype=torch.float32, device=dev)
+    assert enc.set_function("llm_elementwise_bf16", "argmax_f16") == 1
+    enc.set_buffer(0, logits)
+    enc.set_buffer(1, out)
+    enc.set_constant(2, V)
+    enc.dispatch((256, 1, 1), (256, 1, 1))
+    assert enc.set_function("llm_elementwise_bf16", "argmax_partial_f16") == 1
+    enc.set_buffer(0, logits)
+    enc.set_buffer(1, partials)
+    enc.set_constant(2, V)
+    enc.set_constant(3, M)
+    enc.dispatch((256 * M, 1, 1), (256, 1, 1))
+    assert enc.set_function("llm_elementwise_bf16", "argmax_combine_f16") == 1
+    enc.set_buffer(0, partials)
+    enc.set_buffer(1, out, 4)
+    enc.set_constant(2, M)
+    enc.dispatch((256, 1, 1), (256, 1, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert out.cpu().tolist() == [want, want]

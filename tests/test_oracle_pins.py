@@ -449,3 +449,24 @@ def test_w8_oracle_against_numpy_from_the_byte_view(oracle):
     zero = np.zeros((1, 1), dtype=np.uint16)
     assert list(synth.bf16_bits_to_f32(oracle.dequant8_bf16(w1, one, zero, 64, 1))[0, :4]) == [1.0, 2.0, 3.0, 4.0]
 
+
+
+def test_argmax_is_the_first_maximum(oracle):
+    # pinned against numpy's argmax (first occurrence of the maximum) on NaN-free rows with many
+    # ties, and against a plain left-to-right scan written out here for rows with NaN and -inf
+    rng = np.random.default_rng(77)
+    vals = rng.integers(-40, 40, size=(6, 5000)).astype(np.float32) / 4.0      # bf16-exact, heavy ties
+    bits = synth.f32_to_bf16_bits(vals)
+    assert np.array_equal(oracle.argmax(bits), np.argmax(synth.bf16_bits_to_f32(bits), axis=1).astype(np.int32))
+    nan, ninf, pinf = 0x7FC0, 0xFF80, 0x7F80
+    one, two = 0x3F80, 0x4000
+    cases = [([nan, one, two, two], 2), ([ninf, ninf, ninf], 0), ([nan, ninf, ninf], 1), ([nan, nan], 0),
+             ([two, nan, pinf, pinf], 2), ([one], 0), ([nan, 0x8000, 0x0000], 1)]      # -0.0 == +0.0: the first
+    for row, want in cases:
+        best, bi = -np.inf, -1
+        for i, h in enumerate(row):
+            v = float(synth.bf16_bits_to_f32(np.array([h], dtype=np.uint16))[0])
+            if v > best or (bi < 0 and v == best):
+                best, bi = v, i
+        assert max(bi, 0) == want
+        assert int(oracle.argmax(np.array(row, dtype=np.uint16))[0]) == want

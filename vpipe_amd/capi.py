@@ -28,6 +28,10 @@ SYMBOLS = [
     ("vpq_device_cu_count", _i, []),
     ("vpq_dequant_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_embed_gather_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_argmax_workspace_bytes", _sz, [_i, _i]),
+    ("vpq_argmax_bf16", _i, [_vp, _vp, _vp, _i, _i, _vp, _sz]),
+    ("vpq_argmax_partial_bf16", _i, [_vp, _vp, _vp, _i, _i]),
+    ("vpq_argmax_combine", _i, [_vp, _vp, _vp, _i]),
     ("vpq_gather_qmv_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
     ("vpq_gather_down_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i]),
     ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
@@ -129,6 +133,21 @@ def embed_gather_w4g64(ids, w, scales, biases, H, vocab, out=None):
         out = torch.empty((T, H), dtype=torch.bfloat16, device=w.device)
     _check(load().vpq_embed_gather_w4g64_bf16(_stream(), _ptr(ids), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out),
                                               H, T, vocab), "vpq_embed_gather_w4g64_bf16")
+    return out
+
+
+def argmax_bf16(logits, out=None, two_stage=True):
+    """bf16 [rows, V] (or [V]) -> int32 [rows]: lowest index of the largest logit of each row."""
+    import torch
+    L = load()
+    rows, V = (1, logits.numel()) if logits.dim() == 1 else logits.shape
+    if out is None:
+        out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    ws, ws_bytes = None, 0
+    if two_stage:
+        ws_bytes = L.vpq_argmax_workspace_bytes(V, rows)
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=logits.device)
+    _check(L.vpq_argmax_bf16(_stream(), _ptr(logits), _ptr(out), V, rows, _ptr(ws), ws_bytes), "vpq_argmax_bf16")
     return out
 
 

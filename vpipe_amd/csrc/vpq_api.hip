@@ -551,6 +551,49 @@ int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
   return gather_common(stream, w, scales, biases, x, y, K, N, pair_eid, npair, 1, n_experts, 0);
 }
 
+size_t vpq_argmax_workspace_bytes(int V, int rows)
+{
+  if (V <= 0 || rows <= 0) { return 0; }
+  return (size_t)rows * (size_t)vpq::argmax_parts(V) * 2 * sizeof(float);
+}
+
+int vpq_argmax_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, int rows, void* ws,
+                    size_t ws_bytes)
+{
+  if (logits == nullptr || out_id == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (V <= 0 || rows <= 0 || rows > 65535) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(logits, 2) || !aligned(out_id, 4) || (ws != nullptr && !aligned(ws, 4))) { return VPQ_ERR_MISALIGNED; }
+  if (ws != nullptr && ws_bytes < vpq_argmax_workspace_bytes(V, rows)) { return VPQ_ERR_WORKSPACE; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (ws == nullptr) { return finish(vpq::launch_argmax_row(hs, logits, out_id, V, rows)); }
+  const int parts = vpq::argmax_parts(V);
+  const int e = finish(vpq::launch_argmax_partial(hs, logits, static_cast<float*>(ws), V, rows, parts));
+  if (e != VPQ_OK) { return e; }
+  return finish(vpq::launch_argmax_combine(hs, static_cast<const float*>(ws), out_id, rows, parts));
+}
+
+int vpq_argmax_partial_bf16(vpq_stream_t stream, const uint16_t* logits, float* partials, int V, int parts)
+{
+  if (logits == nullptr || partials == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (V <= 0 || parts < 1 || parts > 65535) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(logits, 2) || !aligned(partials, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_argmax_partial(reinterpret_cast<hipStream_t>(stream), logits, partials, V, 1, parts));
+}
+
+int vpq_argmax_combine(vpq_stream_t stream, const float* partials, int32_t* out_id, int parts)
+{
+  if (partials == nullptr || out_id == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (parts < 1) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(partials, 4) || !aligned(out_id, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_argmax_combine(reinterpret_cast<hipStream_t>(stream), partials, out_id, 1, parts));
+}
+
 int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,
                              const uint16_t* const* scales, const uint16_t* const* biases,
                              const uint16_t* x, uint16_t* const* y, int K, const int* N, int M)

@@ -116,6 +116,13 @@ hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGrou
 // [0, n_experts)); a.gate_act as in the plain form.
 hipError_t launch_qmv_rows_gather(hipStream_t st, const QmvArgs& a, const int* pair_eid, int pairs, int x_div,
                                   int n_experts);
+// Greedy argmax of `rows` rows of V bf16 logits (lowest index among equal maxima, a NaN never
+// wins): one workgroup per row, or slabs into `partials` (two 4-byte slots per slab: value, index)
+// and a combine; argmax_parts(V) is the slab count the size-based entrance uses.
+int argmax_parts(int V);
+hipError_t launch_argmax_row(hipStream_t st, const uint16_t* logits, int* out_id, int V, int rows);
+hipError_t launch_argmax_partial(hipStream_t st, const uint16_t* logits, float* partials, int V, int rows, int parts);
+hipError_t launch_argmax_combine(hipStream_t st, const float* partials, int* out_id, int rows, int parts);
 // t[M,r] = bf16(alpha * bf16(x . A^T)), r in {32, 64, 96, 128}.
 hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
                          float alpha);

@@ -90,6 +90,9 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_geglu_w4g64", QuantKernel::QmvGeglu},
     {"affine_qmm_steel_bf16", "affine_qmm_geglu_w4g64", QuantKernel::QmmGeglu},
     {"llm_elementwise_bf16", "dequant_embed_gather_f16", QuantKernel::EmbedGather},
+    {"llm_elementwise_bf16", "argmax_f16", QuantKernel::Argmax},
+    {"llm_elementwise_bf16", "argmax_partial_f16", QuantKernel::ArgmaxPartial},
+    {"llm_elementwise_bf16", "argmax_combine_f16", QuantKernel::ArgmaxCombine},
     {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w4g64", QuantKernel::GatherSwiglu},
     {"affine_qmv_bf16", "affine_gather_qmv_geglu_w4g64", QuantKernel::GatherGeglu},
     {"affine_qmv_bf16", "affine_gather_down_qmv_w4g64", QuantKernel::GatherDown},
@@ -376,6 +379,24 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
       status = vpq_embed_gather_w4g64_bf16(st, static_cast<const int32_t*>(buf(0)), static_cast<const uint32_t*>(buf(1)),
                                            static_cast<const uint16_t*>(buf(2)), static_cast<const uint16_t*>(buf(3)),
                                            static_cast<uint16_t*>(buf(4)), H, static_cast<int>(grid.y), vocab);
+    }
+  } else if (kind == QuantKernel::Argmax || kind == QuantKernel::ArgmaxPartial || kind == QuantKernel::ArgmaxCombine) {
+    // gpu-kernels/metal/ops/llm_elementwise.metal:2906-2941, 2977-3028, 3030-3062.  The partials of the
+    // two-stage pair are two 4-byte slots per slab, as the reference's; only the pair reads them.
+    if (kind == QuantKernel::Argmax) {
+      status = (!buf(0) || !buf(1) || !has_int(2))
+                   ? VPQ_ERR_NULL_POINTER
+                   : vpq_argmax_bf16(st, static_cast<const uint16_t*>(buf(0)), static_cast<int32_t*>(buf(1)), ival(2), 1,
+                                     nullptr, 0);
+    } else if (kind == QuantKernel::ArgmaxPartial) {
+      status = (!buf(0) || !buf(1) || !has_int(2) || !has_int(3))
+                   ? VPQ_ERR_NULL_POINTER
+                   : vpq_argmax_partial_bf16(st, static_cast<const uint16_t*>(buf(0)), static_cast<float*>(buf(1)), ival(2),
+                                             ival(3));
+    } else {
+      status = (!buf(0) || !buf(1) || !has_int(2))
+                   ? VPQ_ERR_NULL_POINTER
+                   : vpq_argmax_combine(st, static_cast<const float*>(buf(0)), static_cast<int32_t*>(buf(1)), ival(2));
     }
   } else if (kind == QuantKernel::QmvQkv) {
     // gpu-kernels/metal/quant/affine_qmv.metal:497-516: slots 0:w 1:scales 2:biases 3:x 4:q_out
