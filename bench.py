@@ -490,6 +490,31 @@ def main():
             del packs
         out["qmv_w8g64_m1"] = w8
 
+        # group-32 twin (GGUF Q4_0 repacked), M=1: affine form (5/8 B per weight) and scale-only form
+        # (bias never read: 9/16 B per weight)
+        g32 = {}
+        for K, N in ((4096, 4096), (4096, 12288)):
+            copies = max(2, min(8, int(600e6 // (N * K * 5 // 8))))
+            packs = []
+            for _ in range(copies):
+                w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev, generator=gen)
+                s = torch.empty((N, K // 32), dtype=torch.float32, device=dev).uniform_(0.005, 0.02, generator=gen).bfloat16()
+                packs.append((w, s, (-8.0 * s.float()).bfloat16()))
+            x = torch.randn((1, K), device=dev, generator=gen).bfloat16()
+            y = torch.empty((1, N), dtype=torch.bfloat16, device=dev)
+
+            def call32(i, x=x, y=y, K=K, N=N, so=False):
+                w, s, b = packs[i % copies]
+                vpipe_amd.qmv_w4g32(w, s, None if so else b, x, K, N, 1, out=y, scale_only=so)
+            us_a = kernel_us(call32, 2 * copies)
+            us_q = kernel_us(lambda i: call32(i, so=True), 2 * copies)
+            g32["%d->%d" % (K, N)] = {
+                "affine": {"us": round(us_a, 2), "GBps": round((N * K * 5 // 8 + 2 * K + 2 * N) / (us_a * 1e-6) / 1e9, 1)},
+                "q40_scale_only": {"us": round(us_q, 2),
+                                   "GBps": round((N * K * 9 // 16 + 2 * K + 2 * N) / (us_q * 1e-6) / 1e9, 1)}}
+            del packs
+        out["qmv_w4g32_m1"] = g32
+
         # greedy tail: argmax over the lm_head's 151936 bf16 logits (both launches of the two-stage form)
         lg = torch.randn((1, 151936), device=dev, generator=gen).bfloat16()
         tok = torch.empty((1,), dtype=torch.int32, device=dev)

@@ -337,6 +337,36 @@ int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
                                    const int32_t* pair_eid, int npair, int n_experts);
 
+/* ---- 4-bit group-32 twins (w4g32; GGUF Q4_0 repacked to affine) ---------------
+ * The 4-bit pack with a scale and a bias per 32 values: w uint32 [N, K/8] as
+ * above, scales, biases bf16 [N, K/32].
+ *   vpq_dequant_w4g32_bf16           replaces `affine_dequant_w4g32`
+ *                                    (gpu-kernels/metal/quant/affine_dequant.metal:196-228), bit-exact.
+ *   vpq_qmv_w4g32_bf16 / _f32out     replace `affine_qmv_w4g32[_add]` (affine_qmv.metal:305-320,
+ *                                    367-384) and, with scale_only != 0, the Q4_0 forms
+ *                                    `affine_qmv_w4g32[_add]_q40` (:327-342, 387-403): the bias is
+ *                                    -8 * scale computed in registers and `biases` is never read
+ *                                    (may be NULL) -- bit-identical to the affine form on a pack
+ *                                    whose stored bias is -8 * scale, 10 % fewer bytes.
+ *                                    QMV arithmetic, 1 <= M <= 16.
+ *   vpq_qmv_gated_w4g32_bf16         replaces `affine_qmv_geglu_w4g32[_q40]` (:1451-1490) and the
+ *                                    SwiGLU twin over an interleaved gate|up pack; y [M, N/2].
+ *   vpq_qmm_dense_route_w4g32_bf16   GEMM by expansion into w_deq[N,K] + the vendor GEMM
+ *                                    (expand as in vpq_qmm_dense_route_w4g64_bf16).
+ * Requires K % 32 == 0; w, x 16-byte aligned. */
+int vpq_dequant_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                           const uint16_t* biases, uint16_t* w_deq, int K, int N);
+int vpq_qmv_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                       const uint16_t* x, uint16_t* y, int K, int N, int M, const uint16_t* residual,
+                       int scale_only);
+int vpq_qmv_w4g32_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                         const uint16_t* x, float* y, int K, int N, int M, int scale_only);
+int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int scale_only);
+int vpq_qmm_dense_route_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                   uint16_t* w_deq, int expand);
+
 /* ---- greedy tail: argmax of the lm_head's logits on the device ------------------
  * Replaces `argmax_f16` (gpu-kernels/metal/ops/llm_elementwise.metal:2906-2941;
  * slots 0:logits 1:out_id 2:V), and the two-stage pair `argmax_partial_f16`

@@ -139,6 +139,25 @@ def qmv(w, s, b, x, K, N, M, residual=None):
     return y64, yb
 
 
+def dequant_g32_bf16(w, s, b, K, N):
+    """w4g32: scales, biases [N, K/32] -> bf16 bits [N, K]."""
+    w, s, b = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16)
+    out = np.empty((N, K), dtype=np.uint16)
+    lib().vpo_dequant_w4g32_bf16(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(out, _u16p), K, N)
+    return out
+
+
+def qmv_g32(w, s, b, x, K, N, M, residual=None, scale_only=False):
+    """w4g32 QMV -> (y64, y_bf16); scale_only: the Q4_0 form, b = -8*s, `b` not read (may be None)."""
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    residual = _c(residual, np.uint16)
+    y64 = np.empty((M, N), dtype=np.float64)
+    yb = np.empty((M, N), dtype=np.uint16)
+    lib().vpo_qmv_w4g32(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y64, _f64p), _p(yb, _u16p),
+                        K, N, M, _p(residual, _u16p), 1 if scale_only else 0)
+    return y64, yb
+
+
 def qmv_factored(w, s, b, x, K, N, M):
     w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
     y64 = np.empty((M, N), dtype=np.float64)

@@ -179,6 +179,22 @@ void vpo_dequant_w4g64_bf16(const uint32_t* w, const uint16_t* scales, const uin
   }
 }
 
+/* group-32 twin, gpu-kernels/metal/quant/affine_dequant.metal:196-228 (GGUF Q4_0 repacked to
+ * affine): the same expression with a scale and a bias per 32 values, scales/biases [N, K/32]. */
+void vpo_dequant_w4g32_bf16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            uint16_t* out, int K, int N)
+{
+  const int Kw = K / 8, Kg = K / 32;
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / 32]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / 32]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      out[n * (size_t)K + k] = vpo_f32_to_bf16(sq + b);
+    }
+  }
+}
+
 /* Dequantizing embedding gather, gpu-kernels/metal/ops/llm_elementwise.metal:1676-1701:
  * out[t, h] = T(s * q + b) of table row ids[t] -- the dequant expression above applied
  * to the selected rows.  Rows with an id outside [0, vocab) are zero-filled here
@@ -244,6 +260,40 @@ void vpo_qmv_w4g64(const uint32_t* w, const uint16_t* scales, const uint16_t* bi
     for (int k = 0; k < K; ++k) {
       const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
       const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      wrow[k] = sq + b;
+    }
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      double acc = 0.0;
+      const uint16_t* xr = x + m * (size_t)K;
+      for (int k = 0; k < K; ++k) { acc += (double)vpo_bf16_to_f32(xr[k]) * (double)wrow[k]; }
+      if (y64) { y64[m * (size_t)N + n] = acc; }
+      if (y_bf16) {
+        uint16_t v = vpo_f32_to_bf16((float)acc);
+        if (residual) {
+          v = vpo_f32_to_bf16(vpo_bf16_to_f32(v) + vpo_bf16_to_f32(residual[m * (size_t)N + n]));
+        }
+        y_bf16[m * (size_t)N + n] = v;
+      }
+    }
+  }
+  free(wrow);
+}
+
+/* group-32 twins of the QMV, gpu-kernels/metal/quant/affine_qmv.metal:305-342 (`affine_qmv_w4g32`,
+ * `affine_qmv_w4g32_q40`) and their `_add` forms (:367-403): the loop above with a scale and a
+ * bias per 32 values.  scale_only != 0 is the Q4_0 form, which never reads `biases` (may be NULL)
+ * and uses b = -8 * s, exact in fp32 (affine_qmv.metal:252-256). */
+void vpo_qmv_w4g32(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, double* y64, uint16_t* y_bf16,
+                   int K, int N, int M, const uint16_t* residual, int scale_only)
+{
+  const int Kw = K / 8, Kg = K / 32;
+  float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / 32]);
+      const float b = scale_only ? -8.0f * s : vpo_bf16_to_f32(biases[n * Kg + k / 32]);
       const float sq = s * (float)nibble(w, n, Kw, k);
       wrow[k] = sq + b;
     }

@@ -486,3 +486,48 @@ def test_argmax_call_sites_of_the_host_layer(enc, oracle, dev, D):
     ok, why = enc.wait_ok()
     assert ok, why
     assert out.cpu().tolist() == [want, want]
+
+
+def test_eight_bit_and_group32_function_names(enc, oracle, dev, D):
+    # the twins keep the slot layout of the 4-bit group-64 functions; the Q4_0 names ignore slot 2
+    K, N = 1024, 96
+    x = synth.make_act(1, K, 1200)
+    xd = D.bf16(x, dev)
+    res = synth.make_act(1, N, 1201)
+
+    w8, s8, b8 = synth.make_weight8(N, K, 1202)
+    y8 = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_w8g64", D.u32(w8, dev), D.bf16(s8, dev), D.bf16(b8, dev), xd, y8,
+                  K, N, grid=(32, N // 4, 1))
+    wq, sq, bq = synth.make_weight_g32(N, K, 1203, q40=True)
+    wqd, sqd, bqd = D.u32(wq, dev), D.bf16(sq, dev), D.bf16(bq, dev)
+    ya = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    yq = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    yr = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    junk = torch.zeros((4,), dtype=torch.bfloat16, device=dev)          # slot 2 of a Q4_0 call: "pass anything"
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_w4g32", wqd, sqd, bqd, xd, ya, K, N, grid=(32, N // 4, 1))
+    encode_linear(enc, "affine_qmv_bf16", "affine_qmv_w4g32_q40", wqd, sqd, junk, xd, yq, K, N, grid=(32, N // 4, 1))
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_w4g32_add_q40") == 1
+    for i, t in enumerate((wqd, sqd, junk, xd, yr)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.set_buffer(7, D.bf16(res, dev))
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    dense = torch.zeros((N, K), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_dequant_bf16", "affine_dequant_w4g32") == 1
+    for i, t in enumerate((wqd, sqd, bqd, dense)):
+        enc.set_buffer(i, t)
+    enc.set_constant(4, K)
+    enc.set_constant(5, N)
+    enc.dispatch((K // 8, N, 1), (64, 1, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    y64, yb = oracle.matmul8(w8, s8, b8, x, K, N, 1, rounded=False)
+    parity.check_bf16(D.bits(y8), y64, yb)
+    y64, yb = oracle.qmv_g32(wq, sq, None, x, K, N, 1, scale_only=True)
+    parity.check_bf16(D.bits(yq), y64, yb)
+    assert torch.equal(ya, yq)
+    want = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(D.bits(yq)) + synth.bf16_bits_to_f32(res))
+    assert np.array_equal(D.bits(yr), want)
+    assert np.array_equal(D.bits(dense), oracle.dequant_g32_bf16(wq, sq, bq, K, N))

@@ -470,3 +470,36 @@ def test_argmax_is_the_first_maximum(oracle):
                 best, bi = v, i
         assert max(bi, 0) == want
         assert int(oracle.argmax(np.array(row, dtype=np.uint16))[0]) == want
+
+
+def test_group32_twins_against_closed_forms_and_the_group64_oracle(oracle):
+    # (1) a group-64 pack rewritten with every scale and bias repeated twice is a group-32 pack of
+    # the same weight: both oracles must give the same bits; (2) the dense expansion against the
+    # closed form in numpy; (3) the QMV against a float64 matmul of that expansion; (4) the Q4_0
+    # form (bias never read) equals the affine form whose stored bias is -8*scale.
+    N, K, M = 24, 256, 3
+    w, s64, b64 = synth.make_weight(N, K, 910)
+    x = synth.make_act(M, K, 911)
+    s32, b32 = np.repeat(s64, 2, axis=1), np.repeat(b64, 2, axis=1)
+    assert np.array_equal(oracle.dequant_g32_bf16(w, s32, b32, K, N), oracle.dequant_bf16(w, s64, b64, K, N))
+    y64a, yba = oracle.qmv_g32(w, s32, b32, x, K, N, M)
+    y64b, ybb = oracle.qmv(w, s64, b64, x, K, N, M)
+    assert np.array_equal(y64a, y64b) and np.array_equal(yba, ybb)
+
+    w, s, b = synth.make_weight_g32(N, K, 912)
+    q = synth.unpack_nibbles(w, K).astype(np.float32)
+    sf = np.repeat(synth.bf16_bits_to_f32(s), 32, axis=1)
+    bf = np.repeat(synth.bf16_bits_to_f32(b), 32, axis=1)
+    dense32 = (sf * q).astype(np.float32) + bf            # s*q exact in fp32, one rounding in the add
+    assert np.array_equal(oracle.dequant_g32_bf16(w, s, b, K, N), synth.f32_to_bf16_bits(dense32))
+    y64, _ = oracle.qmv_g32(w, s, b, x, K, N, M)
+    want = synth.bf16_bits_to_f32(x).astype(np.float64) @ dense32.astype(np.float64).T
+    assert np.allclose(y64, want, rtol=1e-12, atol=1e-9)
+
+    w, s, b = synth.make_weight_g32(N, K, 913, q40=True)
+    ya, yb_a = oracle.qmv_g32(w, s, b, x, K, N, M)
+    yq, yb_q = oracle.qmv_g32(w, s, None, x, K, N, M, scale_only=True)
+    assert np.array_equal(ya, yq) and np.array_equal(yb_a, yb_q)
+    res = synth.make_act(M, N, 914)
+    _, with_res = oracle.qmv_g32(w, s, None, x, K, N, M, residual=res, scale_only=True)
+    assert np.array_equal(with_res, synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(yb_q) + synth.bf16_bits_to_f32(res)))

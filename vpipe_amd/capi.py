@@ -28,6 +28,11 @@ SYMBOLS = [
     ("vpq_device_cu_count", _i, []),
     ("vpq_dequant_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_embed_gather_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_dequant_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_qmv_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
+    ("vpq_qmv_w4g32_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_qmv_gated_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
+    ("vpq_qmm_dense_route_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_argmax_workspace_bytes", _sz, [_i, _i]),
     ("vpq_argmax_bf16", _i, [_vp, _vp, _vp, _i, _i, _vp, _sz]),
     ("vpq_argmax_partial_bf16", _i, [_vp, _vp, _vp, _i, _i]),
@@ -133,6 +138,50 @@ def embed_gather_w4g64(ids, w, scales, biases, H, vocab, out=None):
         out = torch.empty((T, H), dtype=torch.bfloat16, device=w.device)
     _check(load().vpq_embed_gather_w4g64_bf16(_stream(), _ptr(ids), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out),
                                               H, T, vocab), "vpq_embed_gather_w4g64_bf16")
+    return out
+
+
+def dequant_w4g32(w, scales, biases, K, N, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((N, K), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_dequant_w4g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out), K, N),
+           "vpq_dequant_w4g32_bf16")
+    return out
+
+
+def qmv_w4g32(w, scales, biases, x, K, N, M, out=None, residual=None, f32out=False, scale_only=False, activation=0):
+    """group-32 QMV; biases may be None with scale_only; activation != 0: interleaved gate|up pack -> [M, N/2]."""
+    import torch
+    L = load()
+    so = 1 if scale_only else 0
+    if activation:
+        if out is None:
+            out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=w.device)
+        _check(L.vpq_qmv_gated_w4g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                          activation, so), "vpq_qmv_gated_w4g32_bf16")
+        return out
+    if f32out:
+        if out is None:
+            out = torch.empty((M, N), dtype=torch.float32, device=w.device)
+        _check(L.vpq_qmv_w4g32_f32out(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M, so),
+               "vpq_qmv_w4g32_f32out")
+        return out
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _check(L.vpq_qmv_w4g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                _ptr(residual), so), "vpq_qmv_w4g32_bf16")
+    return out
+
+
+def qmm_dense_route_w4g32(w, scales, biases, x, K, N, M, w_deq=None, expand=True, out=None):
+    import torch
+    if w_deq is None:
+        w_deq = torch.empty((N, K), dtype=torch.bfloat16, device=w.device)
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_dense_route_w4g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                                 _ptr(w_deq), 1 if expand else 0), "vpq_qmm_dense_route_w4g32_bf16")
     return out
 
 

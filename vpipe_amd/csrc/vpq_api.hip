@@ -551,6 +551,100 @@ int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
   return gather_common(stream, w, scales, biases, x, y, K, N, pair_eid, npair, 1, n_experts, 0);
 }
 
+namespace {
+
+int check_pack_g32(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, int K, int N, bool scale_only)
+{
+  if (w == nullptr || scales == nullptr || (!scale_only && biases == nullptr)) { return VPQ_ERR_NULL_POINTER; }
+  if (K <= 0 || N <= 0 || (K % 32) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(w, 16) || !aligned(scales, 2) || (!scale_only && !aligned(biases, 2))) { return VPQ_ERR_MISALIGNED; }
+  return VPQ_OK;
+}
+
+int qmv_g32_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, void* y, bool y_f32, int K, int N, int M, const uint16_t* residual,
+                   int gate_act, bool scale_only)
+{
+  int st = check_pack_g32(w, scales, biases, K, N, scale_only);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (gate_act != 0 && ((N & 1) != 0 || residual != nullptr)) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2) || (residual != nullptr && !aligned(residual, 2))) {
+    return VPQ_ERR_MISALIGNED;
+  }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y; a.residual = residual;
+  a.K = K; a.N = N; a.M = M; a.y_f32 = y_f32; a.cu_count = g_dev.cu_count;
+  a.gate_act = gate_act;
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  // up to two rows of x: the row-streaming kernel; more: one wavefront per weight row
+  if (M <= 2) { return finish(vpq::launch_qmv_rows_g32(hs, a, scale_only)); }
+  return finish(vpq::launch_qmv_simple_g32(hs, a, scale_only));
+}
+
+}  // namespace
+
+int vpq_dequant_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           uint16_t* w_deq, int K, int N)
+{
+  int st = check_pack_g32(w, scales, biases, K, N, false);
+  if (st != VPQ_OK) { return st; }
+  if (w_deq == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (!aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_dequant_g32(reinterpret_cast<hipStream_t>(stream), w, scales, biases, w_deq, K, N));
+}
+
+int vpq_qmv_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                       const uint16_t* x, uint16_t* y, int K, int N, int M, const uint16_t* residual, int scale_only)
+{
+  return qmv_g32_common(stream, w, scales, biases, x, y, false, K, N, M, residual, 0, scale_only != 0);
+}
+
+int vpq_qmv_w4g32_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                         const uint16_t* x, float* y, int K, int N, int M, int scale_only)
+{
+  return qmv_g32_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr, 0, scale_only != 0);
+}
+
+int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int scale_only)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return qmv_g32_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, activation, scale_only != 0);
+}
+
+int vpq_qmm_dense_route_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                   uint16_t* w_deq, int expand)
+{
+  int st = check_pack_g32(w, scales, biases, K, N, false);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (w_deq == nullptr) { return VPQ_ERR_WORKSPACE; }
+  if (M <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (expand != 0) {
+    st = finish(vpq::launch_dequant_g32(hs, w, scales, biases, w_deq, K, N));
+    if (st != VPQ_OK) { return st; }
+  }
+  std::string why;
+  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, &why);
+  if (rc != 0) {
+    strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
+    g_last_error[sizeof(g_last_error) - 1] = '\0';
+    return rc == -1 ? VPQ_ERR_UNSUPPORTED : VPQ_ERR_DEVICE;
+  }
+  return VPQ_OK;
+}
+
 size_t vpq_argmax_workspace_bytes(int V, int rows)
 {
   if (V <= 0 || rows <= 0) { return 0; }

@@ -9,16 +9,18 @@ namespace vpq {
 // stores.  out = bf16_rne(fp32(s*q + b)); s*q is exact in fp32 (8-bit x 4-bit
 // significands), so the fused multiply-add below equals the two-step form of
 // gpu-kernels/metal/quant/affine_dequant.metal:45-52 bit for bit.
-__global__ __launch_bounds__(256) void dequant_w4g64_kernel(
+// WS: log2 of the words per quantization group (3: group 64; 2: group 32, affine_dequant.metal:196-228).
+template <int WS>
+__global__ __launch_bounds__(256) void dequant_w4_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, uint4* __restrict__ out, int Kw, size_t total_words)
 {
-  const int Kg = Kw >> 3;
+  const int Kg = Kw >> WS;
   for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total_words;
        idx += (size_t)gridDim.x * 256) {
     const size_t n = idx / (size_t)Kw;
     const int j = (int)(idx - n * (size_t)Kw);
-    const size_t g = n * (size_t)Kg + (size_t)(j >> 3);
+    const size_t g = n * (size_t)Kg + (size_t)(j >> WS);
     const float s = bf16_bits_to_f32(scales[g]);
     const float b = bf16_bits_to_f32(biases[g]);
     const uint32_t p = w[idx];
@@ -41,7 +43,18 @@ hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* sca
   const size_t total = (size_t)N * (size_t)Kw;
   size_t blocks = (total + 255) / 256;
   if (blocks > 65536 * 4) { blocks = 65536 * 4; }
-  return launch_kernel(dequant_w4g64_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, scales,
+  return launch_kernel(dequant_w4_kernel<3>, dim3((unsigned)blocks), dim3(256), 0, st, w, scales,
+                       biases, reinterpret_cast<uint4*>(out), Kw, total);
+}
+
+hipError_t launch_dequant_g32(hipStream_t st, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, uint16_t* out, int K, int N)
+{
+  const int Kw = K / 8;
+  const size_t total = (size_t)N * (size_t)Kw;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536 * 4) { blocks = 65536 * 4; }
+  return launch_kernel(dequant_w4_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, st, w, scales,
                        biases, reinterpret_cast<uint4*>(out), Kw, total);
 }
 

@@ -79,6 +79,11 @@ hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* sca
 hipError_t launch_embed_gather(hipStream_t st, const int* ids, const uint32_t* w, const uint16_t* scales,
                                const uint16_t* biases, uint16_t* out, int H, int T, int vocab);
 hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a);
+// group-32 twins (scales, biases [N, K/32]; K % 32 == 0); scale_only: Q4_0 pack, bias = -8 * scale, a.biases unread.
+hipError_t launch_dequant_g32(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                              uint16_t* out, int K, int N);
+hipError_t launch_qmv_simple_g32(hipStream_t st, const QmvArgs& a, bool scale_only);
+hipError_t launch_qmv_rows_g32(hipStream_t st, const QmvArgs& a, bool scale_only);   // M <= 2
 // The 8-bit twins (one byte per value, w is [N, K/4] words): dense expansion and the general QMV kernel.
 hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                            uint16_t* out, int K, int N);

@@ -61,7 +61,10 @@ struct RowsGather {
 };
 
 // R rows per row group, 64 / LPR row groups per wavefront, four wavefronts per workgroup, MT rows of x.
-template <int R, int MT, bool F32OUT, int LPR>
+// GS: log2 of the quantization group (6: group 64; 5: group 32, a lane's 32 values are one group).
+// SO: scale-only (Q4_0) pack, the bias is -8 * scale and `biases` is never read
+// (gpu-kernels/metal/quant/affine_qmv.metal:252-256).
+template <int R, int MT, bool F32OUT, int LPR, int GS = 6, bool SO = false>
 __global__ __launch_bounds__(256) void qmv_rows_kernel(
     const RowsSegs g, const uint16_t* __restrict__ x, const uint16_t* __restrict__ residual, int K, int M, int gate_act,
     const RowsGather gather)
@@ -83,7 +86,7 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
   const int nw = (((int)blockIdx.x - sg.first_block) * 4 + wave) * SUBS * R;
   if (nw >= N) { return; }              // wave-uniform; the kernel has no barrier
   const int n0 = nw + sub * R;
-  const int Kw = K >> 3, Kg = K >> 6;
+  const int Kw = K >> 3, Kg = K >> GS;
   bool expert_ok = true;
   if (gather.pair_eid != nullptr) {
     const int p = (int)blockIdx.y;
@@ -130,8 +133,8 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       p.c[r] = *reinterpret_cast<const uint4*>(wrow[r] + (k0 >> 3));
-      p.sb[r] = srow[r][k0 >> 6];
-      p.bb[r] = brow[r][k0 >> 6];
+      p.sb[r] = srow[r][k0 >> GS];
+      p.bb[r] = SO ? 0u : brow[r][k0 >> GS];
     }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
@@ -166,7 +169,7 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
     for (int r = 0; r < R; ++r) {
       const uint32_t cw[4] = {p.c[r].x, p.c[r].y, p.c[r].z, p.c[r].w};
       const float s = bf16_bits_to_f32(p.sb[r]);
-      const float b = bf16_bits_to_f32(p.bb[r]);
+      const float b = SO ? -8.0f * s : bf16_bits_to_f32(p.bb[r]);
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         float d = 0.0f;
@@ -259,15 +262,15 @@ bool qmv_rows_supports(int K, int N, int M)
 namespace {
 
 hipError_t launch_rows_segments(hipStream_t st, RowsSegs& g, const QmvArgs& a, int rows_per_wave,
-                                const RowsGather& gather, int pairs)
+                                const RowsGather& gather, int pairs, int group = 64, bool scale_only = false)
 {
   double bytes = 0.0;
   for (int i = 0; i < g.count; ++i) { bytes += (double)g.seg[i].N * (double)a.K * 9.0 / 16.0; }
   // Two rows per row group finish sooner on layer-sized packs (more, shorter wavefronts: 4096->4096
   // 4.3 vs 4.4 us, 5120->5120 6.6 vs 7.1, 17408->5120 14.7 vs 15.9); four on lm_head-sized ones,
   // where x is re-read half as often (5120->151936: 94 vs 100 us).
-  const int R = rows_per_wave == 2 || rows_per_wave == 4 ? rows_per_wave : (bytes >= 150e6 ? 4 : 2);
-  const bool half = a.K <= 1024 && a.M == 1 && R == 2;      // 32 lanes per row group
+  const int R = group == 32 ? 2 : (rows_per_wave == 2 || rows_per_wave == 4 ? rows_per_wave : (bytes >= 150e6 ? 4 : 2));
+  const bool half = group == 64 && a.K <= 1024 && a.M == 1 && R == 2;      // 32 lanes per row group
   const int rows_per_block = 4 * R * (half ? 2 : 1);
   int blocks = 0;
   for (int i = 0; i < g.count; ++i) {
@@ -280,8 +283,16 @@ hipError_t launch_rows_segments(hipStream_t st, RowsSegs& g, const QmvArgs& a, i
 #define VPQ_ROWS_M(RR)                                                                       \
   (a.M == 1 ? (a.y_f32 ? VPQ_ROWS(RR, 1, true, 64) : VPQ_ROWS(RR, 1, false, 64))             \
             : (a.y_f32 ? VPQ_ROWS(RR, 2, true, 64) : VPQ_ROWS(RR, 2, false, 64)))
+#define VPQ_ROWS32(MT, F32, SO) \
+  launch_kernel(qmv_rows_kernel<2, MT, F32, 64, 5, SO>, grid, block, 0, st, g, a.x, a.residual, a.K, a.M, a.gate_act, gather)
+#define VPQ_ROWS32_M(SO)                                                             \
+  (a.M == 1 ? (a.y_f32 ? VPQ_ROWS32(1, true, SO) : VPQ_ROWS32(1, false, SO))         \
+            : (a.y_f32 ? VPQ_ROWS32(2, true, SO) : VPQ_ROWS32(2, false, SO)))
+  if (group == 32) { return scale_only ? VPQ_ROWS32_M(true) : VPQ_ROWS32_M(false); }
   if (half) { return a.y_f32 ? VPQ_ROWS(2, 1, true, 32) : VPQ_ROWS(2, 1, false, 32); }
   return R == 2 ? VPQ_ROWS_M(2) : VPQ_ROWS_M(4);
+#undef VPQ_ROWS32_M
+#undef VPQ_ROWS32
 #undef VPQ_ROWS_M
 #undef VPQ_ROWS
 }
@@ -313,6 +324,14 @@ hipError_t launch_qmv_rows_gather(hipStream_t st, const QmvArgs& a, const int* p
   g.count = 1;
   g.seg[0] = RowsSeg{a.w, a.scales, a.biases, a.y, a.N, 0};
   return launch_rows_segments(st, g, a, 2, RowsGather{pair_eid, x_div, n_experts}, pairs);
+}
+
+hipError_t launch_qmv_rows_g32(hipStream_t st, const QmvArgs& a, bool scale_only)
+{
+  RowsSegs g{};
+  g.count = 1;
+  g.seg[0] = RowsSeg{a.w, a.scales, a.biases, a.y, a.N, 0};
+  return launch_rows_segments(st, g, a, 2, RowsGather{nullptr, 1, 0}, 1, 32, scale_only);
 }
 
 }  // namespace vpq

@@ -14,7 +14,9 @@
 
 namespace vpq {
 
-template <int MT, bool F32OUT>
+// GS: log2 of the quantization group (6, or 5 for the group-32 packs); SO: scale-only (Q4_0) pack, the
+// bias is -8 * scale and `biases` is never read (affine_qmv.metal:305-342, 252-256).
+template <int MT, bool F32OUT, int GS = 6, bool SO = false>
 __global__ __launch_bounds__(256) void qmv_simple_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x, void* __restrict__ y,
@@ -26,21 +28,21 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
   const int n_raw = blockIdx.x * 4 + wave;
   const bool live = n_raw < N;            // wave-uniform
   const int n = live ? n_raw : N - 1;     // idle wavefronts redo the last row and store nothing
-  const int Kw = K >> 3, Kg = K >> 6;
+  const int Kw = K >> 3, Kg = K >> GS;
   const uint32_t* wrow = w + (size_t)n * Kw;
   const uint16_t* srow = scales + (size_t)n * Kg;
-  const uint16_t* brow = biases + (size_t)n * Kg;
+  const uint16_t* brow = SO ? nullptr : biases + (size_t)n * Kg;
 
   for (int m0 = 0; m0 < M; m0 += MT) {
     float acc[MT];
 #pragma unroll
     for (int mm = 0; mm < MT; ++mm) { acc[mm] = 0.0f; }
-    // Each lane takes 32 consecutive k (one 128-bit load of codes, half a group).
+    // Each lane takes 32 consecutive k (one 128-bit load of codes, half a group of 64).
     for (int k0 = lane * 32; k0 < K; k0 += kWave * 32) {
       const uint4 c4 = *reinterpret_cast<const uint4*>(wrow + (k0 >> 3));
       const uint32_t codes[4] = {c4.x, c4.y, c4.z, c4.w};
-      const float s = bf16_bits_to_f32(srow[k0 >> 6]);
-      const float b = bf16_bits_to_f32(brow[k0 >> 6]);
+      const float s = bf16_bits_to_f32(srow[k0 >> GS]);
+      const float b = SO ? -8.0f * s : bf16_bits_to_f32(brow[k0 >> GS]);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float wv[8];
@@ -114,6 +116,19 @@ hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a)
                 a.residual, a.K, a.N, a.M, a.gate_act)
   if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH(1, true) : VPQ_LAUNCH(1, false); }
   return a.y_f32 ? VPQ_LAUNCH(4, true) : VPQ_LAUNCH(4, false);
+#undef VPQ_LAUNCH
+}
+
+hipError_t launch_qmv_simple_g32(hipStream_t st, const QmvArgs& a, bool scale_only)
+{
+  const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
+#define VPQ_LAUNCH(MT, F32, SO)                                                                       \
+  launch_kernel(qmv_simple_kernel<MT, F32, 5, SO>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
+                a.residual, a.K, a.N, a.M, a.gate_act)
+#define VPQ_LAUNCH_SO(MT, F32) (scale_only ? VPQ_LAUNCH(MT, F32, true) : VPQ_LAUNCH(MT, F32, false))
+  if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH_SO(1, true) : VPQ_LAUNCH_SO(1, false); }
+  return a.y_f32 ? VPQ_LAUNCH_SO(4, true) : VPQ_LAUNCH_SO(4, false);
+#undef VPQ_LAUNCH_SO
 #undef VPQ_LAUNCH
 }
 

@@ -69,6 +69,7 @@ struct FnEntry {
   const char* library;
   const char* function;
   QuantKernel kind;
+  QuantFormat format = QuantFormat::W4G64;
 };
 
 // Function names of the reference's bf16 metallibs that this path serves.
@@ -100,6 +101,18 @@ const FnEntry kFunctions[] = {
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm128", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64_rs", QuantKernel::QmmSwiglu},
+    // 8-bit and group-32 twins (gpu-kernels/metal/quant/affine_dequant.metal:68-97, 196-228;
+    // affine_qmv.metal:305-403, 1451-1490, 3034-3050, 3122-3140; affine_qmm_steel.metal:1601-)
+    {"affine_dequant_bf16", "affine_dequant_w8g64", QuantKernel::Dequant, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_w8g64", QuantKernel::Qmv, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
+    {"affine_dequant_bf16", "affine_dequant_w4g32", QuantKernel::Dequant, QuantFormat::W4G32},
+    {"affine_qmv_bf16", "affine_qmv_w4g32", QuantKernel::Qmv, QuantFormat::W4G32},
+    {"affine_qmv_bf16", "affine_qmv_w4g32_add", QuantKernel::QmvAdd, QuantFormat::W4G32},
+    {"affine_qmv_bf16", "affine_qmv_w4g32_q40", QuantKernel::Qmv, QuantFormat::W4G32Q40},
+    {"affine_qmv_bf16", "affine_qmv_w4g32_add_q40", QuantKernel::QmvAdd, QuantFormat::W4G32Q40},
+    {"affine_qmv_bf16", "affine_qmv_geglu_w4g32", QuantKernel::QmvGeglu, QuantFormat::W4G32},
+    {"affine_qmv_bf16", "affine_qmv_geglu_w4g32_q40", QuantKernel::QmvGeglu, QuantFormat::W4G32Q40},
 };
 
 }  // namespace
@@ -119,6 +132,7 @@ QuantFunction QuantLibrary::function(const std::string& fn_name) const
   for (const FnEntry& e : kFunctions) {
     if (_name == e.library && fn_name == e.function) {
       fn._kind = e.kind;
+      fn._format = e.format;
       fn._name = fn_name;
       break;
     }
@@ -357,7 +371,41 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
 
   int status = VPQ_OK;
   const QuantKernel kind = _fn.kind();
-  if (kind == QuantKernel::Dequant) {
+  const QuantFormat fmt = _fn.format();
+  if (fmt != QuantFormat::W4G64) {
+    // The 8-bit and group-32 twins keep the slot layout of the 4-bit group-64 functions:
+    // dequant 0:w 1:scales 2:biases 3:w_deq 4:K 5:N; QMV 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N [7:residual],
+    // rows from grid.x.  The Q4_0 forms ignore slot 2.
+    const bool q40 = fmt == QuantFormat::W4G32Q40;
+    const uint32_t* w = static_cast<const uint32_t*>(buf(0));
+    const uint16_t* sc = static_cast<const uint16_t*>(buf(1));
+    const uint16_t* bi = static_cast<const uint16_t*>(buf(2));
+    if (kind == QuantKernel::Dequant) {
+      if (!w || !sc || !bi || !buf(3) || !has_int(4) || !has_int(5)) {
+        status = VPQ_ERR_NULL_POINTER;
+      } else if (fmt == QuantFormat::W8G64) {
+        status = vpq_dequant_w8g64_bf16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
+      } else {
+        status = vpq_dequant_w4g32_bf16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
+      }
+    } else if (!w || !sc || (!bi && !q40) || !buf(3) || !buf(4) || !has_int(5) || !has_int(6) ||
+               (kind == QuantKernel::QmvAdd && !buf(7))) {
+      status = VPQ_ERR_NULL_POINTER;
+    } else {
+      const uint16_t* x = static_cast<const uint16_t*>(buf(3));
+      uint16_t* y = static_cast<uint16_t*>(buf(4));
+      const int K = ival(5), N = ival(6);
+      const int M = grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1;
+      const uint16_t* residual = kind == QuantKernel::QmvAdd ? static_cast<const uint16_t*>(buf(7)) : nullptr;
+      if (fmt == QuantFormat::W8G64) {
+        status = vpq_qmv_w8g64_bf16(st, w, sc, bi, x, y, K, N, M, residual);
+      } else if (kind == QuantKernel::QmvGeglu) {
+        status = vpq_qmv_gated_w4g32_bf16(st, w, sc, q40 ? nullptr : bi, x, y, K, N, M, VPQ_GATE_GEGLU, q40 ? 1 : 0);
+      } else {
+        status = vpq_qmv_w4g32_bf16(st, w, sc, q40 ? nullptr : bi, x, y, K, N, M, residual, q40 ? 1 : 0);
+      }
+    }
+  } else if (kind == QuantKernel::Dequant) {
     // slots 0:w 1:scales 2:biases 3:w_deq 4:K 5:N
     if (!buf(0) || !buf(1) || !buf(2) || !buf(3) || !has_int(4) || !has_int(5)) {
       status = VPQ_ERR_NULL_POINTER;

@@ -90,16 +90,26 @@ enum class QuantKernel : std::uint8_t {
   ArgmaxCombine,  // argmax_combine_f16: slots 0:partials 1:out_id 2:M
 };
 
+// The packed format a function name ends in.
+enum class QuantFormat : std::uint8_t {
+  W4G64 = 0,      // _w4g64: 4-bit codes, a scale and a bias per 64 values
+  W8G64,          // _w8g64: one byte per value
+  W4G32,          // _w4g32: 4-bit codes, a scale and a bias per 32 values
+  W4G32Q40,       // _w4g32_q40 / _w4g32_add_q40: as W4G32 with the bias buffer never read (bias = -8 * scale)
+};
+
 class QuantFunction {
 public:
   QuantFunction() noexcept = default;
   bool valid() const noexcept { return _kind != QuantKernel::None; }
   QuantKernel kind() const noexcept { return _kind; }
+  QuantFormat format() const noexcept { return _format; }
   const std::string& name() const noexcept { return _name; }
 
 private:
   friend class QuantLibrary;
   QuantKernel _kind = QuantKernel::None;
+  QuantFormat _format = QuantFormat::W4G64;
   std::string _name;
 };
 

@@ -73,6 +73,21 @@ def make_weight8(N, K, seed):
     return w, s, f32_to_bf16_bits(b32)
 
 
+def make_weight_g32(N, K, seed, q40=False):
+    """group-32 twin: (w uint32 [N,K/8], scales, biases bf16 bits [N,K/32]); q40: biases = bf16(-8*scale) exactly,
+    the redundant bias of a Q4_0 pack."""
+    assert K % 32 == 0
+    rng = np.random.default_rng(seed)
+    w = rng.integers(0, 2**32, size=(N, K // 8), dtype=np.uint32)
+    s = f32_to_bf16_bits(rng.uniform(0.005, 0.02, size=(N, K // 32)).astype(np.float32))
+    if q40:
+        b32 = np.float32(-8.0) * bf16_bits_to_f32(s)        # exact: a power of two times a bf16
+    else:
+        z = rng.standard_normal(size=(N, K // 32)).astype(np.float32)
+        b32 = np.float32(-8.0) * bf16_bits_to_f32(s) * (np.float32(1.0) + np.float32(0.05) * z)
+    return w, s, f32_to_bf16_bits(b32)
+
+
 def make_act(M, K, seed, std=1.0):
     rng = np.random.default_rng(seed)
     return f32_to_bf16_bits((rng.standard_normal(size=(M, K)) * std).astype(np.float32))
