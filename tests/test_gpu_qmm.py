@@ -208,3 +208,60 @@ def test_linear_entrance_splits_k_when_given_the_room(vpq, oracle, dev, D):
     parity.check_bf16(D.bits(split), y64, yb)
     parity.check_bf16(D.bits(plain), y64, yb)
     assert vpq.load().vpq_qmm_workspace_bytes(4096, 12288, 2048) == 0      # enough tiles: no split
+
+
+# M, N, K: the minimal K (one block of 8 steps), ragged M and N in both tile widths, more than one
+# band of 8 rows of tiles (M > 2048), a single row
+BIG_TILE_SHAPES = [(300, 520, 512), (257, 193, 1024), (2300, 200, 512), (1, 8, 512), (640, 384, 1536)]
+
+
+@pytest.mark.parametrize("tile_n", [192, 256])
+@pytest.mark.parametrize("M,N,K", BIG_TILE_SHAPES)
+def test_qmm_large_tile_kernel(vpq, oracle, dev, D, M, N, K, tile_n):
+    # against the oracle, and bit for bit against the 256x128 tile kernel: same MFMA, same K order
+    w, s, b = synth.make_weight(N, K, 7100 + N + K)
+    x = synth.make_act(M, K, 7200 + M + K)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, tile_n=tile_n)
+    small = vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, tile_n=128)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    assert torch.equal(out.view, small)
+    rng = np.random.default_rng(M + N)
+    ms = np.unique(np.concatenate([np.arange(min(4, M)), np.arange(max(M - 4, 0), M), rng.integers(0, M, 24)]))
+    y64, yb = oracle.qmm(w, s, b, x[ms], K, N, len(ms))
+    parity.check_bf16(D.bits(out.view)[ms], y64, yb)
+
+
+@pytest.mark.parametrize("tile_n", [192, 256])
+@pytest.mark.parametrize("r", [32, 64, 96])
+def test_qmm_large_tile_kernel_with_lora(vpq, oracle, dev, D, r, tile_n):
+    M, N, K, alpha = 300, 450, 1024, 0.75
+    w, s, b = synth.make_weight(N, K, 7300 + r)
+    s[:] = synth.f32_to_bf16_bits(np.float32(0.0005))      # small base: the delta is a visible part of y
+    b[:] = synth.f32_to_bf16_bits(np.float32(-0.004))
+    x = synth.make_act(M, K, 7301)
+    A, B = synth.make_lora(N, K, r, 7302, std=0.05)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    Ad, Bd = D.bf16(A, dev), D.bf16(B, dev)
+    t_ws = torch.empty((M, r), dtype=torch.bfloat16, device=dev)
+    got = vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, lora_A=Ad, lora_B=Bd, r=r, alpha=alpha, t_ws=t_ws, tile_n=tile_n)
+    small = vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, lora_A=Ad, lora_B=Bd, r=r, alpha=alpha, tile_n=128)
+    assert torch.equal(got, small)
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M, t=D.bits(t_ws), B=B, r=r)
+    parity.check_bf16(D.bits(got), y64, yb)
+    base = vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, tile_n=tile_n)
+    assert not torch.equal(base, got)
+
+
+def test_qmm_large_tile_kernel_refuses_what_it_cannot_take(vpq, dev, D):
+    M, N, K = 64, 64, 576                                   # K not a multiple of 512
+    w, s, b = synth.make_weight(N, K, 1)
+    x = synth.make_act(M, K, 2)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    with pytest.raises(vpq.VpqError):
+        vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, tile_n=256)
+    with pytest.raises(vpq.VpqError):
+        vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, tile_n=64)
+    vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, tile_n=128)

@@ -43,6 +43,7 @@ SYMBOLS = [
     ("vpq_qmv_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _i]),
     ("vpq_qmv_workspace_bytes", _sz, [_i, _i, _i]),
     ("vpq_qmm_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _f, _vp]),
+    ("vpq_qmm_tiled_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _f, _vp, _i]),
     ("vpq_qmm_workspace_bytes", _sz, [_i, _i, _i]),
     ("vpq_qmm_splitk_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz]),
     ("vpq_qmm_dense_route_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
@@ -362,12 +363,18 @@ def lora_a(x, A, M, K, r, alpha, out=None):
     return out
 
 
-def qmm_w4g64(w, scales, biases, x, K, N, M, out=None, lora_A=None, lora_B=None, r=0, alpha=0.0, t_ws=None):
+def qmm_w4g64(w, scales, biases, x, K, N, M, out=None, lora_A=None, lora_B=None, r=0, alpha=0.0, t_ws=None, tile_n=0):
+    """tile_n: 0 = the library's choice; 128 the 256x128 tile kernel; 192 / 256 the large-tile kernel."""
     import torch
     if out is None:
         out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
     if lora_A is not None and t_ws is None:
         t_ws = torch.empty((M, r), dtype=torch.bfloat16, device=w.device)
+    if tile_n:
+        _check(load().vpq_qmm_tiled_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                               K, N, M, _ptr(lora_A), _ptr(lora_B), r, alpha, _ptr(t_ws), tile_n),
+               "vpq_qmm_tiled_w4g64_bf16")
+        return out
     _check(load().vpq_qmm_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
                                      K, N, M, _ptr(lora_A), _ptr(lora_B), r, alpha, _ptr(t_ws)),
            "vpq_qmm_w4g64_bf16")

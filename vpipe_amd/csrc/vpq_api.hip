@@ -300,10 +300,13 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
   return finish(vpq::launch_lora_a(reinterpret_cast<hipStream_t>(stream), x, lora_a, t, M, K, r, alpha));
 }
 
-int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
-                       const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
-                       const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
-                       uint16_t* lora_t_ws)
+namespace {
+
+// tile: 0 = by size, 128 = the 256 x 128 tile kernel, 192 / 256 = the large-tile kernel at that width
+int qmm_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+               const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+               const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
+               uint16_t* lora_t_ws, int tile)
 {
   int st = check_pack(w, scales, biases, K, N);
   if (st != VPQ_OK) { return st; }
@@ -331,7 +334,37 @@ int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
   g.lora_b = lora ? lora_b : nullptr;
   g.r = lora ? r : 0;
   g.cu_count = g_dev.cu_count;
+  if (tile == 192 || tile == 256) {
+    if (!vpq::qmm_big_supports(g)) { return VPQ_ERR_BAD_SHAPE; }
+    return finish(vpq::launch_qmm_big(hs, g, tile));
+  }
+  // The large-tile kernel once its tiles make at least two rounds over the CUs (measured at
+  // M = 16320: 0.98-1.07 against 0.75-0.89 PFLOP/s); below that the smaller tile fills the chip better.
+  if (tile == 0 && vpq::qmm_big_supports(g)) {
+    const int bn = vpq::qmm_big_tile_n(N, M, g_dev.cu_count);
+    const long tiles = (long)((M + 255) / 256) * (long)((N + bn - 1) / bn);
+    if (tiles >= 2L * (g_dev.cu_count > 0 ? g_dev.cu_count : 256)) { return finish(vpq::launch_qmm_big(hs, g, bn)); }
+  }
   return finish(vpq::launch_qmm_tile(hs, g));
+}
+
+}  // namespace
+
+int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                       const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
+                       uint16_t* lora_t_ws)
+{
+  return qmm_common(stream, w, scales, biases, x, y, K, N, M, lora_a, lora_b, r, alpha, lora_t_ws, 0);
+}
+
+int vpq_qmm_tiled_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                             const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
+                             uint16_t* lora_t_ws, int tile_n)
+{
+  if (tile_n != 128 && tile_n != 192 && tile_n != 256) { return VPQ_ERR_BAD_SHAPE; }
+  return qmm_common(stream, w, scales, biases, x, y, K, N, M, lora_a, lora_b, r, alpha, lora_t_ws, tile_n);
 }
 
 size_t vpq_qmm_workspace_bytes(int K, int N, int M)

@@ -133,6 +133,12 @@ hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, u
                          float alpha);
 // 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.
 hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a);
+// Large-tile kernel (256 x 256 or 256 x 192 per workgroup, four wavefronts that each load, dequantize
+// and multiply): K % 512 == 0, 16-byte aligned scales / biases, no gated store; same bits as the tile
+// kernel.  tile_n 0 = qmm_big_tile_n().
+bool qmm_big_supports(const GemmArgs& a);
+int qmm_big_tile_n(int N, int M, int cu_count);
+hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n);
 // Split-K form of the same kernel (no adapter, no gated store): `splits` shares of the K steps,
 // fp32 planes [splits][M][N] in `plane`, then a fold.  qmm_choose_splits() returns 1 where the tiles
 // alone fill the chip.

@@ -1,0 +1,453 @@
+// QMM, large-tile kernel: y[M,N] = x[M,K] . bf16(W)^T (+ t[M,r] . B[N,r]^T) for GEMMs with many
+// tiles (the video-DiT projections, M in the thousands).  Same arithmetic as the 256 x 128 tile
+// kernel -- W = bf16_rne(fp32(s*q+b)) (gpu-kernels/metal/quant/affine_qmm_steel.metal:78-96),
+// v_mfma_f32_32x32x16_bf16 over K in ascending order, fp32 accumulators, one rounding -- and the
+// same bits; what differs is who does what.
+//
+// A workgroup owns 256(M) x BN(N) of y, BN = 64 NT in {256, 192}, and has FOUR wavefronts, one per
+// SIMD, each with a 128 x (BN/2) block of accumulators (up to 256 registers, in the accumulation
+// file).  A wavefront's operand reads from LDS are then (4 + NT) fragments per 4 NT MFMAs -- half the
+// LDS bytes per MFMA of a 128 x 64 block -- which is what bounds the smaller tile: there the LDS
+// pipe is busy longer than the matrix pipe.  With one wavefront per SIMD nothing else can fill the
+// matrix pipe's shadow, so every wavefront does all three jobs and the instruction stream itself
+// interleaves them: after each MFMA comes one piece (<= 8 vector instructions) of the
+// dequantization of the NEXT step's weight row and, every other time, one fragment read for the
+// next quarter step, pinned in that order by scheduling barriers.
+//
+// Per 64-wide K step and workgroup, everything arrives by direct-to-LDS loads:
+//   x tile [256,64] bf16      8 loads per wavefront (8 rows x 128 contiguous bytes each);
+//   codes  [BN rows x 32 B]   2 loads per wavefront (32 rows x 32 bytes), into a two-slot ring;
+//   scales, biases            1 load each per wavefront and 8 steps (64 rows x 16 bytes), two slots.
+// A wavefront brings in the codes and scales of the rows its own threads dequantize (thread t =
+// tile row t), so only its own load counter stands between the load and the read.  The loads are
+// written out by hand: the compiler orders every later LDS read after a direct-to-LDS load it
+// knows about, whichever array that load fills, which would serialize the pipeline; hand-written,
+// the only waits in the loop are the explicit ones, counted exactly (requests retire in order).
+// Two LDS stages of x (2 x 32 KB) and of the dequantized W (2 x 32 KB) + the rings (2 x 8 + 2 x 8 KB)
+// are the whole 160 KB.
+//
+// Tiles are walked in bands of 8 rows of tiles, M first inside a band: workgroups go to the 8 XCDs
+// round-robin, so the workgroups an XCD receives while a band lasts read the same 256 rows of x.
+#include <type_traits>
+
+#include "vpq_device.h"
+#include "vpq_internal.h"
+
+namespace vpq {
+
+namespace {
+
+constexpr int BM = 256, BK = 64;
+constexpr int kBigThreads = 256;
+constexpr int kRow = BK * 2;                 // 128 bytes per LDS row
+constexpr int kXBytes = BM * kRow;           // 32 KB per stage
+constexpr int kWBytes = 256 * kRow;          // 32 KB per stage (BN <= 256)
+constexpr int kCodeBytes = 256 * 32;         // 8 KB: the 32 bytes of codes of one K step per row
+constexpr int kScaleBytes = 256 * 32;        // 8 KB: 8 scales | 8 biases (8 K steps) per row
+
+struct BigParams {
+  const uint32_t* w;
+  const uint16_t* scales;
+  const uint16_t* biases;
+  const uint16_t* x;
+  uint16_t* y;
+  const uint16_t* lora_t;   // [M,r] or nullptr
+  const uint16_t* lora_b;   // [N,r]
+  int K, N, M, r;
+  int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+
+// Byte I of a dword as fp32 (selects v_cvt_f32_ubyteI).
+template <int I>
+__device__ __forceinline__ float ubyte_f32(uint32_t v) { return (float)((v >> (8 * I)) & 0xffu); }
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>());
+    static_for<I + 1, N>(f);
+  }
+}
+
+// Workgroup barrier without a memory fence: the callers wait on the counters they need.
+__device__ __forceinline__ void wg_barrier()
+{
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+__device__ __forceinline__ uint32_t lds_addr(const uint8_t* q)
+{
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)q;
+}
+
+// 16 bytes per lane, global -> LDS at lds_dst + 16 * lane.  M0 is used by nothing else in this kernel.
+__device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* src)
+{
+  const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+}
+
+}  // namespace
+
+template <int NT, bool LORA>
+__global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
+{
+  constexpr int BN = 64 * NT;               // weight rows per workgroup
+  constexpr int MQ = 4 * NT;                // MFMAs per quarter step (16 of K)
+  // One array per stage and operand.
+  __shared__ __attribute__((aligned(16))) uint8_t x_lds0[kXBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t x_lds1[kXBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t w_lds0[kWBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t w_lds1[kWBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t c_lds[2 * kCodeBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t sb_lds[2 * kScaleBytes];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tile = (int)blockIdx.x;
+  const int band = tile / (8 * p.tiles_n);
+  const int in_band = tile - band * (8 * p.tiles_n);
+  const int band_h = (p.tiles_m - band * 8) < 8 ? (p.tiles_m - band * 8) : 8;
+  const int tm = band * 8 + in_band % band_h;
+  const int tn = in_band / band_h;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int KT = p.K / BK;                  // a multiple of 8 (K % 512 == 0)
+
+  // ---- x tile: 8 direct-to-LDS loads per wavefront and step.  Load i of wavefront w covers tile rows
+  // (8w + i)*8 .. +8; lane l takes row l/8 and lands at LDS position l%8 of it.
+  const uint8_t* xblk = reinterpret_cast<const uint8_t*>(p.x) + (size_t)m0 * p.K * 2;
+  uint32_t a_off[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = (wave * 8 + i) * 8 + (lane >> 3);
+    const int chunk = swz(row, lane & 7);
+    const int rg = (m0 + row < p.M) ? row : (p.M - 1 - m0);
+    a_off[i] = (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u;
+  }
+  auto issue_x = [&](int step, auto stage_c) {
+    const uint8_t* src = xblk + (size_t)step * (BK * 2);
+    const uint32_t dst = lds_addr(decltype(stage_c)::value ? x_lds1 : x_lds0) + wave * (64 * kRow);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { dma16(dst + i * (8 * kRow), src + a_off[i]); }
+  };
+  // ---- codes, scales, biases of the rows 64w .. 64w+63 (wavefronts past BN rows bring in nothing) ----
+  const bool dq_wave = wave * 64 < BN;      // wave-uniform
+  uint32_t c_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = wave * 64 + i * 32 + (lane >> 1);
+    const int rg = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
+    c_off[i] = (uint32_t)rg * (uint32_t)(p.K >> 1) + (uint32_t)(lane & 1) * 16u;
+  }
+  const uint8_t* wblk = reinterpret_cast<const uint8_t*>(p.w);
+  auto issue_codes = [&](int u) {
+    if (!dq_wave) { return; }
+    const uint8_t* src = wblk + (size_t)u * 32;
+    const uint32_t dst = lds_addr(c_lds) + (u & 1) * kCodeBytes + wave * (64 * 32);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) { dma16(dst + i * (32 * 32), src + c_off[i]); }
+  };
+  const int qrow = tid;                     // the tile row this thread dequantizes
+  const int qrg = (n0 + qrow < p.N) ? (n0 + qrow) : (p.N - 1);
+  const uint8_t* srow = reinterpret_cast<const uint8_t*>(p.scales) + (size_t)qrg * (p.K >> 5);   // K/64 entries of 2 bytes
+  const uint8_t* brow = reinterpret_cast<const uint8_t*>(p.biases) + (size_t)qrg * (p.K >> 5);
+  auto issue_scales = [&](int blk) {
+    if (!dq_wave) { return; }
+    const uint32_t dst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave * (64 * 16);
+    dma16(dst, srow + (size_t)blk * 16);
+    dma16(dst + 256 * 16, brow + (size_t)blk * 16);
+  };
+  int b_dst[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) { b_dst[i] = qrow * kRow + swz(qrow, i) * 16; }
+
+  // ---- multiplier side ----
+  const int wm = wave >> 1, wn = wave & 1;
+  floatx16 acc[NT][4];   // [jt: 32 weight rows][it: 32 x rows]
+#pragma unroll
+  for (int jt = 0; jt < NT; ++jt) {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) { acc[jt][it][e] = 0.0f; }
+    }
+  }
+  const int frow = lane & 31;      // row of a 32-row operand fragment
+  const int fkh = lane >> 5;       // which 8 of the 16 k
+  int w_rd[NT], x_rd[4];           // stage-relative operand rows
+#pragma unroll
+  for (int jt = 0; jt < NT; ++jt) { w_rd[jt] = (wn * (BN / 2) + jt * 32 + frow) * kRow; }
+#pragma unroll
+  for (int it = 0; it < 4; ++it) { x_rd[it] = (wm * 128 + it * 32 + frow) * kRow; }
+  const int f_sw = (frow >> 1) & 7;   // the fragment offsets are multiples of 16 rows: same swizzle for all
+
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+
+  // One K step: multiplies stage ST while -- with FILL -- the codes of step s+1 become the W tile of the
+  // other stage.  Piece P (0..63) of that dequantization is word P/8 of the row step at stage P%8 of
+  //   0: split the nibbles   1..4: two values each, fma(s, q, b)   5: pack to bf16   6: store   7: -
+  // and the pieces are dealt out evenly over the step's 4 MQ MFMAs.
+  auto compute = [&](auto stage_c, auto fill_c, int s, int ksteps) {
+    constexpr int ST = decltype(stage_c)::value;
+    constexpr bool FILL = decltype(fill_c)::value;
+    const uint8_t* xb = ST ? x_lds1 : x_lds0;
+    const uint8_t* wb = ST ? w_lds1 : w_lds0;
+    uint8_t* nb = ST ? w_lds0 : w_lds1;                  // W stage of step s+1
+    const int u = s + 1;
+    float sc = 0.0f, bi = 0.0f;
+    uint32_t cw[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (FILL) {
+      const uint8_t* sb = sb_lds + ((u >> 3) & 1) * kScaleBytes + qrow * 16 + (u & 7) * 2;
+      sc = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb));
+      bi = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
+      const uint4 c_lo = *reinterpret_cast<const uint4*>(c_lds + (u & 1) * kCodeBytes + qrow * 32);
+      const uint4 c_hi = *reinterpret_cast<const uint4*>(c_lds + (u & 1) * kCodeBytes + qrow * 32 + 16);
+      cw[0] = c_lo.x; cw[1] = c_lo.y; cw[2] = c_lo.z; cw[3] = c_lo.w;
+      cw[4] = c_hi.x; cw[5] = c_hi.y; cw[6] = c_hi.z; cw[7] = c_hi.w;
+    }
+    bf16x8 wf[2][NT], xf[2][4];                          // operand fragments of the current / the next quarter
+    auto frag = [&](int buf, int ks, int idx) {          // idx: 0 = w0, 1..4 = x0..x3, 5.. = w1..
+      const int c = ((2 * ks + fkh) ^ f_sw) * 16;
+      if (idx == 0) {
+        wf[buf][0] = *reinterpret_cast<const bf16x8*>(wb + w_rd[0] + c);
+      } else if (idx <= 4) {
+        xf[buf][idx - 1] = *reinterpret_cast<const bf16x8*>(xb + x_rd[idx - 1] + c);
+      } else {
+        wf[buf][idx - 4] = *reinterpret_cast<const bf16x8*>(wb + w_rd[idx - 4] + c);
+      }
+    };
+#pragma unroll
+    for (int i = 0; i < 4 + NT; ++i) { frag(0, 0, i); }
+    uint32_t lo = 0, hi = 0;
+    float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    uint4 o = make_uint4(0, 0, 0, 0);
+    auto piece = [&](auto pc) {
+      constexpr int P = decltype(pc)::value;
+      constexpr int W = P >> 3, S = P & 7;
+      if constexpr (S == 0) {
+        lo = cw[W] & 0x0f0f0f0fu;                        // q0 q2 q4 q6
+        hi = (cw[W] >> 4) & 0x0f0f0f0fu;                 // q1 q3 q5 q7
+      } else if constexpr (S == 1) {
+        v[0] = fmaf(sc, ubyte_f32<0>(lo), bi); v[1] = fmaf(sc, ubyte_f32<0>(hi), bi);
+      } else if constexpr (S == 2) {
+        v[2] = fmaf(sc, ubyte_f32<1>(lo), bi); v[3] = fmaf(sc, ubyte_f32<1>(hi), bi);
+      } else if constexpr (S == 3) {
+        v[4] = fmaf(sc, ubyte_f32<2>(lo), bi); v[5] = fmaf(sc, ubyte_f32<2>(hi), bi);
+      } else if constexpr (S == 4) {
+        v[6] = fmaf(sc, ubyte_f32<3>(lo), bi); v[7] = fmaf(sc, ubyte_f32<3>(hi), bi);
+      } else if constexpr (S == 5) {
+        o.x = pack_bf16x2(v[0], v[1]); o.y = pack_bf16x2(v[2], v[3]);
+        o.z = pack_bf16x2(v[4], v[5]); o.w = pack_bf16x2(v[6], v[7]);
+      } else if constexpr (S == 6) {
+        // unconditional: threads past BN rows fill rows of the stage that nobody reads (a condition
+        // here would pull the whole word's arithmetic under one branch, out of the MFMAs' shadow)
+        *reinterpret_cast<uint4*>(nb + b_dst[W]) = o;
+      }
+    };
+    static_for<0, 4>([&](auto qc) {
+      constexpr int Q = decltype(qc)::value;
+      constexpr int B = Q & 1;
+      if (Q < ksteps) {
+        static_for<0, MQ>([&](auto jc) {
+          constexpr int J = decltype(jc)::value;
+          constexpr int JT = J >> 2, IT = J & 3;
+          acc[JT][IT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[B][JT], xf[B][IT], acc[JT][IT], 0, 0, 0);
+          if constexpr (FILL) {
+            constexpr int G = Q * MQ + J;                // MFMA index within the step
+            static_for<(G * 64) / (4 * MQ), ((G + 1) * 64) / (4 * MQ)>(piece);
+          }
+          // the next quarter's fragments, one read after every MFMA until they are all requested
+          if constexpr (Q < 3 && J < 4 + NT) {
+            if (Q + 1 < ksteps) { frag(1 - B, Q + 1, J); }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      }
+    });
+  };
+
+  // ---- prologue: x(0), the codes of steps 0 and 1, the first block of scales; step 0's W tile ----
+  issue_scales(0);
+  issue_codes(0);
+  issue_codes(1);
+  issue_x(0, S0());
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  {
+    const uint8_t* sb = sb_lds + qrow * 16;
+    const float sc = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb));
+    const float bi = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
+    if (qrow < BN) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint4 c4 = *reinterpret_cast<const uint4*>(c_lds + qrow * 32 + h * 16);
+        const uint32_t c[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t lo = c[i] & 0x0f0f0f0fu, hi = (c[i] >> 4) & 0x0f0f0f0fu;
+          uint4 o;
+          o.x = pack_bf16x2(fmaf(sc, ubyte_f32<0>(lo), bi), fmaf(sc, ubyte_f32<0>(hi), bi));
+          o.y = pack_bf16x2(fmaf(sc, ubyte_f32<1>(lo), bi), fmaf(sc, ubyte_f32<1>(hi), bi));
+          o.z = pack_bf16x2(fmaf(sc, ubyte_f32<2>(lo), bi), fmaf(sc, ubyte_f32<2>(hi), bi));
+          o.w = pack_bf16x2(fmaf(sc, ubyte_f32<3>(lo), bi), fmaf(sc, ubyte_f32<3>(hi), bi));
+          *reinterpret_cast<uint4*>(w_lds0 + b_dst[h * 4 + i]) = o;
+        }
+      }
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  wg_barrier();
+
+  // ---- K loop.  Requests of step s, in issue order: x(s+1) [8], codes(s+2) [2] into the slot step s's
+  // codes have left; on steps 8b the scales and biases of block b+1 [2].  Before the barrier x(s+1) and
+  // codes(s+2) must have landed: only the two scale requests may stay in flight (wavefronts that
+  // request no codes or scales wait for everything, which is their x tile).
+  auto step = [&](auto stage_c, auto fill_c, int s) {
+    using St = decltype(stage_c);
+    using Nx = std::integral_constant<int, 1 - St::value>;
+    constexpr bool FILL = decltype(fill_c)::value;      // false for the last step only
+    bool scales_out = false;
+    if constexpr (FILL) { issue_x(s + 1, Nx()); }
+    if (s + 2 < KT) { issue_codes(s + 2); }
+    if (St::value == 0 && (s & 7) == 0 && s + 8 < KT && dq_wave) {
+      issue_scales((s >> 3) + 1);
+      scales_out = true;
+    }
+    compute(St(), fill_c, s, 4);
+    if (scales_out) {
+      asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    }
+    wg_barrier();
+  };
+  // No condition surrounds the arithmetic inside the loop; the last pair of steps is written out.
+  int s = 0;
+  for (; s + 2 < KT; s += 2) {
+    step(S0(), std::true_type(), s);
+    step(S1(), std::true_type(), s + 1);
+  }
+  step(S0(), std::true_type(), s);
+  step(S1(), std::false_type(), s + 1);
+
+  if (LORA) {
+    // r more values of K from t[M,r] and B[N,r], dense, through stage 0
+    // (gpu-kernels/metal/gemm/dense_gemm_mma.metal:297-348).
+    const int steps = (p.r + BK - 1) / BK;
+    for (int st = 0; st < steps; ++st) {
+      const int kleft = p.r - st * BK;                 // >= 32, a multiple of 32
+      const int chunks = kleft >= BK ? 8 : (kleft >> 3);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int row = (wave * 8 + i) * 8 + (lane >> 3);
+        const int chunk = swz(row, lane & 7);
+        const int rg = (m0 + row < p.M) ? (m0 + row) : (p.M - 1);
+        if (chunk < chunks) {
+          dma16(lds_addr(x_lds0) + wave * (64 * kRow) + i * (8 * kRow),
+                reinterpret_cast<const uint8_t*>(p.lora_t + (size_t)rg * p.r + st * BK + chunk * 8));
+        }
+      }
+      if (dq_wave) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int row = (wave * 8 + i) * 8 + (lane >> 3);
+          const int chunk = swz(row, lane & 7);
+          const int rg = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
+          if (chunk < chunks) {
+            dma16(lds_addr(w_lds0) + wave * (64 * kRow) + i * (8 * kRow),
+                  reinterpret_cast<const uint8_t*>(p.lora_b + (size_t)rg * p.r + st * BK + chunk * 8));
+          }
+        }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      wg_barrier();                                    // tiles ready
+      compute(S0(), std::false_type(), 0, chunks >> 1);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wg_barrier();                                    // everyone done with them
+    }
+  }
+
+  // ---- store: lane holds, for x row m = lane%32 of each it, 4 consecutive n per register quad ----
+  const bool vec_ok = (p.N & 3) == 0;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int m = m0 + wm * 128 + it * 32 + frow;
+    if (m >= p.M) { continue; }
+    uint16_t* yrow = p.y + (size_t)m * p.N;
+#pragma unroll
+    for (int jt = 0; jt < NT; ++jt) {
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int n = n0 + wn * (BN / 2) + jt * 32 + rq * 8 + fkh * 4;
+        if (n >= p.N) { continue; }
+        const float v0 = acc[jt][it][rq * 4 + 0], v1 = acc[jt][it][rq * 4 + 1];
+        const float v2 = acc[jt][it][rq * 4 + 2], v3 = acc[jt][it][rq * 4 + 3];
+        if (vec_ok && n + 3 < p.N) {
+          uint2 o;
+          o.x = pack_bf16x2(v0, v1);
+          o.y = pack_bf16x2(v2, v3);
+          *reinterpret_cast<uint2*>(yrow + n) = o;
+        } else {
+          const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (n + e < p.N) { yrow[n + e] = (uint16_t)f32_to_bf16_bits(v[e]); }
+          }
+        }
+      }
+    }
+  }
+}
+
+bool qmm_big_supports(const GemmArgs& a)
+{
+  // K in blocks of 8 steps (the scale ring) with 16-byte aligned rows of scales; 32-bit offsets
+  // inside the pack and inside a band of x; no gated store.
+  if (a.K % 512 != 0 || a.M < 1 || a.N < 1 || a.gate_act != 0) { return false; }
+  if ((reinterpret_cast<uintptr_t>(a.scales) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.biases) & 15) != 0) { return false; }
+  if ((double)a.N * (double)a.K / 2.0 >= 4.0e9 || (double)BM * (double)a.K * 2.0 >= 4.0e9) { return false; }
+  if (a.lora_t != nullptr && (a.r < 32 || a.r % 32 != 0)) { return false; }
+  return true;
+}
+
+// Tile width by the number of whole rounds of workgroups over the CUs: 256 unless 192 fills the
+// last round better (4096 -> 12288 at M = 2048: 384 tiles of 256 are one and a half rounds of 256
+// CUs, 512 tiles of 192 are two).
+int qmm_big_tile_n(int N, int M, int cu_count)
+{
+  const int cus = cu_count > 0 ? cu_count : 256;
+  const long tm = (M + BM - 1) / BM;
+  auto cost = [&](int bn) {
+    const long tiles = tm * ((N + bn - 1) / bn);
+    const long rounds = (tiles + cus - 1) / cus;
+    return (double)rounds * (double)bn;          // time of a round grows with the tile width
+  };
+  return cost(192) < cost(256) ? 192 : 256;
+}
+
+hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
+{
+  const int bn = tile_n == 192 || tile_n == 256 ? tile_n : qmm_big_tile_n(a.N, a.M, a.cu_count);
+  BigParams p;
+  p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
+  p.lora_t = a.lora_t; p.lora_b = a.lora_b;
+  p.K = a.K; p.N = a.N; p.M = a.M; p.r = a.r;
+  p.tiles_m = (a.M + BM - 1) / BM;
+  p.tiles_n = (a.N + bn - 1) / bn;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kBigThreads);
+  const bool lora = a.lora_t != nullptr;
+  if (bn == 192) {
+    return lora ? launch_kernel(qmm_big_kernel<3, true>, grid, block, 0, st, p)
+                : launch_kernel(qmm_big_kernel<3, false>, grid, block, 0, st, p);
+  }
+  return lora ? launch_kernel(qmm_big_kernel<4, true>, grid, block, 0, st, p)
+              : launch_kernel(qmm_big_kernel<4, false>, grid, block, 0, st, p);
+}
+
+}  // namespace vpq
