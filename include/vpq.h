@@ -229,7 +229,15 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
  * M = 8; here the 256-row GEMM tile does not pay below ~64 rows: measured 57 us at
  * 4096->4096 for any M <= 256 against ~10 us per slab.)  Above 64 rows the GEMM
  * splits K (vpq_qmm_splitk_w4g64_bf16) where that pays and `ws` has
- * vpq_qmm_workspace_bytes() bytes. */
+ * vpq_qmm_workspace_bytes() bytes.  From 1024 rows on, when `ws` holds the
+ * expanded weight (N*K*2 bytes), the GEMM runs by the dequant-once route
+ * (vpq_qmm_dense_route_w4g64_bf16: expansion + vendor GEMM, the reference's route
+ * for large M, minimax-h3/metal-minimax-h3-transformer.cc:2020-2160), which is the
+ * faster one there; without that room, or without the vendor BLAS, the fused kernels.
+ * vpq_linear_workspace_bytes() is the size that lets the entrance take its best
+ * route for the shape (0: none needed); `ws` is 256-byte aligned scratch whose
+ * contents are irrelevant and undefined afterwards. */
+size_t vpq_linear_workspace_bytes(int K, int N, int M);
 int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y,
                           int K, int N, int M, void* ws, size_t ws_bytes);

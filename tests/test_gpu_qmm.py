@@ -265,3 +265,28 @@ def test_qmm_large_tile_kernel_refuses_what_it_cannot_take(vpq, dev, D):
     with pytest.raises(vpq.VpqError):
         vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, tile_n=64)
     vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, tile_n=128)
+
+
+def test_linear_entrance_takes_the_dequant_once_route_when_given_the_room(vpq, oracle, dev, D):
+    M, N, K = 1100, 384, 512
+    w, s, b = synth.make_weight(N, K, 7400)
+    x = synth.make_act(M, K, 7401)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    need = vpq.load().vpq_linear_workspace_bytes(K, N, M)
+    assert need >= N * K * 2
+    assert vpq.load().vpq_linear_workspace_bytes(K, N, 512) == vpq.load().vpq_qmm_workspace_bytes(K, N, 512)
+    ws = torch.zeros((need,), dtype=torch.uint8, device=dev)
+    y = vpq.linear_w4g64(wd, sd, bd, xd, K, N, M, ws=ws)
+    torch.cuda.synchronize()
+    # the workspace now holds the expanded weight, bit-exact, and y is the dense route's result
+    dense = ws[:N * K * 2].view(torch.bfloat16).view(N, K)
+    assert np.array_equal(D.bits(dense), oracle.dequant_bf16(w, s, b, K, N))
+    wdeq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+    assert torch.equal(y, vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, wdeq))
+    rng = np.random.default_rng(5)
+    ms = np.unique(rng.integers(0, M, 48))
+    y64, yb = oracle.qmm(w, s, b, x[ms], K, N, len(ms))
+    parity.check_bf16(D.bits(y)[ms], y64, yb)
+    # too little room: the fused kernel, same numbers within the tolerance
+    small = vpq.linear_w4g64(wd, sd, bd, xd, K, N, M, ws=ws[:4096])
+    parity.check_bf16(D.bits(small)[ms], y64, yb)

@@ -33,6 +33,7 @@ SYMBOLS = [
     ("vpq_qmv_w4g32_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmv_gated_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     ("vpq_qmm_dense_route_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
+    ("vpq_linear_workspace_bytes", _sz, [_i, _i, _i]),
     ("vpq_argmax_workspace_bytes", _sz, [_i, _i]),
     ("vpq_argmax_bf16", _i, [_vp, _vp, _vp, _i, _i, _vp, _sz]),
     ("vpq_argmax_partial_bf16", _i, [_vp, _vp, _vp, _i, _i]),

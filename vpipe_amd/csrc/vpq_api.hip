@@ -75,6 +75,10 @@ int check_pack(const uint32_t* w, const uint16_t* scales, const uint16_t* biases
   return VPQ_OK;
 }
 
+// Rows from which the size-based entrance takes the dequant-once route when the workspace holds the
+// expanded weight: the expansion costs ~20 us per 28 MB pack, the vendor GEMM then runs ~1.4x faster.
+constexpr int kDenseRouteMinRows = 1024;
+
 int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                const uint16_t* biases, const uint16_t* x, void* y, bool y_f32, int K, int N, int M,
                const uint16_t* residual, void* ws, size_t ws_bytes, int variant, int gate_act = 0)
@@ -367,6 +371,13 @@ int vpq_qmm_tiled_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
   return qmm_common(stream, w, scales, biases, x, y, K, N, M, lora_a, lora_b, r, alpha, lora_t_ws, tile_n);
 }
 
+size_t vpq_linear_workspace_bytes(int K, int N, int M)
+{
+  if (K <= 0 || N <= 0 || M <= 0 || (K % 64) != 0) { return 0; }
+  if (M >= kDenseRouteMinRows) { return ((size_t)N * (size_t)K * 2 + 255) / 256 * 256; }
+  return vpq_qmm_workspace_bytes(K, N, M);
+}
+
 size_t vpq_qmm_workspace_bytes(int K, int N, int M)
 {
   if (K <= 0 || N <= 0 || M <= 0 || (K % 64) != 0) { return 0; }
@@ -441,6 +452,15 @@ int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t
       if (st != VPQ_OK) { return st; }
     }
     return VPQ_OK;
+  }
+  // Many rows: expanding the pack once into the workspace and running the vendor GEMM on it beats the
+  // fused kernels (measured: 0.98-1.07 against 0.81-0.88 PFLOP/s at M = 2048, 1.35-1.5 against 0.98-1.1
+  // at M = 16320, expansion included), the reference's own route for large M
+  // (generative-models/minimax-h3/metal-minimax-h3-transformer.cc:2020-2160).
+  if (ws != nullptr && aligned(ws, 256) && M >= kDenseRouteMinRows && K > 0 && N > 0 && (K % 64) == 0 &&
+      ws_bytes >= (size_t)N * (size_t)K * 2) {
+    const int st = vpq_qmm_dense_route_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, static_cast<uint16_t*>(ws), 1);
+    if (st != VPQ_ERR_UNSUPPORTED) { return st; }      // no vendor BLAS in this process: the fused kernels
   }
   // Few tiles and a long K: split K over more workgroups when the caller's workspace has the room.
   if (ws != nullptr && aligned(ws, 256) && K > 0 && N > 0 && M > 0 && (K % 64) == 0 && ensure_init() == VPQ_OK) {
