@@ -92,6 +92,14 @@ __device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* src)
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
 }
 
+// The same from a wave-uniform base (scalar registers) plus a 32-bit offset per lane: stepping along K
+// then costs scalar additions only.
+__device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* base, uint32_t lane_off)
+{
+  const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(m0v), "v"(lane_off), "s"(base) : "memory");
+}
+
 }  // namespace
 
 template <int NT, bool LORA>
@@ -134,7 +142,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     const uint8_t* src = xblk + (size_t)step * (BK * 2);
     const uint32_t dst = lds_addr(decltype(stage_c)::value ? x_lds1 : x_lds0) + wave * (64 * kRow);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { dma16(dst + i * (8 * kRow), src + a_off[i]); }
+    for (int i = 0; i < 8; ++i) { dma16(dst + i * (8 * kRow), src, a_off[i]); }
   };
   // ---- codes, scales, biases of the rows 64w .. 64w+63 (wavefronts past BN rows bring in nothing) ----
   const bool dq_wave = wave * 64 < BN;      // wave-uniform
@@ -151,7 +159,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     const uint8_t* src = wblk + (size_t)u * 32;
     const uint32_t dst = lds_addr(c_lds) + (u & 1) * kCodeBytes + wave * (64 * 32);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) { dma16(dst + i * (32 * 32), src + c_off[i]); }
+    for (int i = 0; i < 2; ++i) { dma16(dst + i * (32 * 32), src, c_off[i]); }
   };
   const int qrow = tid;                     // the tile row this thread dequantizes
   const int qrg = (n0 + qrow < p.N) ? (n0 + qrow) : (p.N - 1);
