@@ -18,9 +18,9 @@
 //   x tile [256,64] bf16      8 loads per wavefront (8 rows x 128 contiguous bytes each);
 //   codes  [BN rows x 32 B]   2 loads per wavefront (32 rows x 32 bytes), into a two-slot ring;
 //   scales, biases            1 load each per wavefront and 8 steps (64 rows x 16 bytes), two slots.
-// A wavefront brings in the codes and scales of the rows its own threads dequantize (thread t =
-// tile row t), so only its own load counter stands between the load and the read.  The loads are
-// written out by hand: the compiler orders every later LDS read after a direct-to-LDS load it
+// The BN x 8 words of a step's codes are dealt out evenly over the 256 threads for dequantization;
+// the step-end barrier, which follows every wavefront's wait for its own loads, stands between a
+// load and its readers.  The loads are written out by hand: the compiler orders every later LDS read after a direct-to-LDS load it
 // knows about, whichever array that load fills, which would serialize the pipeline; hand-written,
 // the only waits in the loop are the explicit ones, counted exactly (requests retire in order).
 // Two LDS stages of x (2 x 32 KB) and of the dequantized W (2 x 32 KB) + the rings (2 x 8 + 2 x 8 KB)
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
 #pragma unroll
     for (int i = 0; i < 8; ++i) { dma16(dst + i * (8 * kRow), src, a_off[i]); }
   };
-  // ---- codes, scales, biases of the rows 64w .. 64w+63 (wavefronts past BN rows bring in nothing) ----
+  // ---- codes, scales, biases: wavefront w brings in those of rows 64w .. 64w+63 (nothing past BN rows) ----
   const bool dq_wave = wave * 64 < BN;      // wave-uniform
   uint32_t c_off[2];
 #pragma unroll
@@ -171,9 +171,40 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     dma16(dst, srow + (size_t)blk * 16);
     dma16(dst + 256 * 16, brow + (size_t)blk * 16);
   };
-  int b_dst[8];
+  // ---- dequantization: the BN x 8 words of a step's codes are dealt out evenly, thread t takes the WPT
+  // consecutive words from t*WPT on (row-major: word j of row r is 8r + j).  BN = 256: its own row;
+  // BN = 192: six words that may straddle two rows.  d_row is the first row, d_w0 the first word in it.
+  constexpr int WPT = 2 * NT;
+  const int d_row = (tid * WPT) >> 3, d_w0 = (tid * WPT) & 7;
+  int b_dst[WPT];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) { b_dst[i] = qrow * kRow + swz(qrow, i) * 16; }
+  for (int j = 0; j < WPT; ++j) {
+    const int row = d_row + ((d_w0 + j) >> 3), word = (d_w0 + j) & 7;
+    b_dst[j] = row * kRow + swz(row, word) * 16;
+  }
+  // scale and bias of rows d_row and d_row + 1 for step u, the thread's codes of step u
+  auto load_row_params = [&](int u, float (&sc)[2], float (&bi)[2], uint32_t (&cw)[WPT]) {
+    const uint8_t* sb = sb_lds + ((u >> 3) & 1) * kScaleBytes + d_row * 16 + (u & 7) * 2;
+    sc[0] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb));
+    bi[0] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
+    sc[1] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 16));
+    bi[1] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 256 * 16 + 16));
+    const uint8_t* cp = c_lds + (u & 1) * kCodeBytes + tid * (WPT * 4);
+    if constexpr (WPT % 4 == 0) {
+#pragma unroll
+      for (int j = 0; j < WPT; j += 4) {
+        const uint4 c4 = *reinterpret_cast<const uint4*>(cp + j * 4);
+        cw[j] = c4.x; cw[j + 1] = c4.y; cw[j + 2] = c4.z; cw[j + 3] = c4.w;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < WPT; j += 2) {
+        const uint2 c2 = *reinterpret_cast<const uint2*>(cp + j * 4);
+        cw[j] = c2.x;
+        cw[j + 1] = c2.y;
+      }
+    }
+  };
 
   // ---- multiplier side ----
   const int wm = wave >> 1, wn = wave & 1;
@@ -209,17 +240,12 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     const uint8_t* wb = ST ? w_lds1 : w_lds0;
     uint8_t* nb = ST ? w_lds0 : w_lds1;                  // W stage of step s+1
     const int u = s + 1;
-    float sc = 0.0f, bi = 0.0f;
-    uint32_t cw[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (FILL) {
-      const uint8_t* sb = sb_lds + ((u >> 3) & 1) * kScaleBytes + qrow * 16 + (u & 7) * 2;
-      sc = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb));
-      bi = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
-      const uint4 c_lo = *reinterpret_cast<const uint4*>(c_lds + (u & 1) * kCodeBytes + qrow * 32);
-      const uint4 c_hi = *reinterpret_cast<const uint4*>(c_lds + (u & 1) * kCodeBytes + qrow * 32 + 16);
-      cw[0] = c_lo.x; cw[1] = c_lo.y; cw[2] = c_lo.z; cw[3] = c_lo.w;
-      cw[4] = c_hi.x; cw[5] = c_hi.y; cw[6] = c_hi.z; cw[7] = c_hi.w;
-    }
+    float sc2[2] = {0.0f, 0.0f}, bi2[2] = {0.0f, 0.0f};
+    uint32_t cw[WPT];
+#pragma unroll
+    for (int j = 0; j < WPT; ++j) { cw[j] = 0; }
+    if (FILL) { load_row_params(u, sc2, bi2, cw); }
+    float sc = 0.0f, bi = 0.0f;                          // of the word in work
     bf16x8 wf[2][NT], xf[2][4];                          // operand fragments of the current / the next quarter
     auto frag = [&](int buf, int ks, int idx) {          // idx: 0 = w0, 1..4 = x0..x3, 5.. = w1..
       const int c = ((2 * ks + fkh) ^ f_sw) * 16;
@@ -242,6 +268,13 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       if constexpr (S == 0) {
         lo = cw[W] & 0x0f0f0f0fu;                        // q0 q2 q4 q6
         hi = (cw[W] >> 4) & 0x0f0f0f0fu;                 // q1 q3 q5 q7
+        if constexpr (NT == 4) {                         // the thread's own row
+          sc = sc2[0]; bi = bi2[0];
+        } else {
+          const bool second = d_w0 + W >= 8;
+          sc = second ? sc2[1] : sc2[0];
+          bi = second ? bi2[1] : bi2[0];
+        }
       } else if constexpr (S == 1) {
         v[0] = fmaf(sc, ubyte_f32<0>(lo), bi); v[1] = fmaf(sc, ubyte_f32<0>(hi), bi);
       } else if constexpr (S == 2) {
@@ -254,8 +287,6 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
         o.x = pack_bf16x2(v[0], v[1]); o.y = pack_bf16x2(v[2], v[3]);
         o.z = pack_bf16x2(v[4], v[5]); o.w = pack_bf16x2(v[6], v[7]);
       } else if constexpr (S == 6) {
-        // unconditional: threads past BN rows fill rows of the stage that nobody reads (a condition
-        // here would pull the whole word's arithmetic under one branch, out of the MFMAs' shadow)
         *reinterpret_cast<uint4*>(nb + b_dst[W]) = o;
       }
     };
@@ -269,7 +300,8 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
           acc[JT][IT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[B][JT], xf[B][IT], acc[JT][IT], 0, 0, 0);
           if constexpr (FILL) {
             constexpr int G = Q * MQ + J;                // MFMA index within the step
-            static_for<(G * 64) / (4 * MQ), ((G + 1) * 64) / (4 * MQ)>(piece);
+            static_assert(WPT * 8 == 4 * MQ, "one piece per MFMA");
+            piece(std::integral_constant<int, G>());
           }
           // the next quarter's fragments, one read after every MFMA until they are all requested
           if constexpr (Q < 3 && J < 4 + NT) {
@@ -287,26 +319,22 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   issue_codes(1);
   issue_x(0, S0());
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  wg_barrier();                             // the codes and scales a thread reads were brought in by any wavefront
   {
-    const uint8_t* sb = sb_lds + qrow * 16;
-    const float sc = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb));
-    const float bi = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
-    if (qrow < BN) {
+    float sc2[2], bi2[2];
+    uint32_t cw[WPT];
+    load_row_params(0, sc2, bi2, cw);
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const uint4 c4 = *reinterpret_cast<const uint4*>(c_lds + qrow * 32 + h * 16);
-        const uint32_t c[4] = {c4.x, c4.y, c4.z, c4.w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t lo = c[i] & 0x0f0f0f0fu, hi = (c[i] >> 4) & 0x0f0f0f0fu;
-          uint4 o;
-          o.x = pack_bf16x2(fmaf(sc, ubyte_f32<0>(lo), bi), fmaf(sc, ubyte_f32<0>(hi), bi));
-          o.y = pack_bf16x2(fmaf(sc, ubyte_f32<1>(lo), bi), fmaf(sc, ubyte_f32<1>(hi), bi));
-          o.z = pack_bf16x2(fmaf(sc, ubyte_f32<2>(lo), bi), fmaf(sc, ubyte_f32<2>(hi), bi));
-          o.w = pack_bf16x2(fmaf(sc, ubyte_f32<3>(lo), bi), fmaf(sc, ubyte_f32<3>(hi), bi));
-          *reinterpret_cast<uint4*>(w_lds0 + b_dst[h * 4 + i]) = o;
-        }
-      }
+    for (int j = 0; j < WPT; ++j) {
+      const bool second = d_w0 + j >= 8;
+      const float sc = second ? sc2[1] : sc2[0], bi = second ? bi2[1] : bi2[0];
+      const uint32_t lo = cw[j] & 0x0f0f0f0fu, hi = (cw[j] >> 4) & 0x0f0f0f0fu;
+      uint4 o;
+      o.x = pack_bf16x2(fmaf(sc, ubyte_f32<0>(lo), bi), fmaf(sc, ubyte_f32<0>(hi), bi));
+      o.y = pack_bf16x2(fmaf(sc, ubyte_f32<1>(lo), bi), fmaf(sc, ubyte_f32<1>(hi), bi));
+      o.z = pack_bf16x2(fmaf(sc, ubyte_f32<2>(lo), bi), fmaf(sc, ubyte_f32<2>(hi), bi));
+      o.w = pack_bf16x2(fmaf(sc, ubyte_f32<3>(lo), bi), fmaf(sc, ubyte_f32<3>(hi), bi));
+      *reinterpret_cast<uint4*>(w_lds0 + b_dst[j]) = o;
     }
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
