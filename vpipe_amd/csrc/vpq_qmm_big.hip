@@ -268,6 +268,9 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       if constexpr (S == 0) {
         lo = cw[W] & 0x0f0f0f0fu;                        // q0 q2 q4 q6
         hi = (cw[W] >> 4) & 0x0f0f0f0fu;                 // q1 q3 q5 q7
+        // No instruction: keeps the masked words as they are, so that each value is one v_cvt_f32_ubyteN
+        // of them (otherwise the mask is folded into a bit-field extract per value, one instruction more).
+        asm volatile("" : "+v"(lo), "+v"(hi));
         if constexpr (NT == 4) {                         // the thread's own row
           sc = sc2[0]; bi = bi2[0];
         } else {
@@ -328,7 +331,8 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     for (int j = 0; j < WPT; ++j) {
       const bool second = d_w0 + j >= 8;
       const float sc = second ? sc2[1] : sc2[0], bi = second ? bi2[1] : bi2[0];
-      const uint32_t lo = cw[j] & 0x0f0f0f0fu, hi = (cw[j] >> 4) & 0x0f0f0f0fu;
+      uint32_t lo = cw[j] & 0x0f0f0f0fu, hi = (cw[j] >> 4) & 0x0f0f0f0fu;
+      asm volatile("" : "+v"(lo), "+v"(hi));
       uint4 o;
       o.x = pack_bf16x2(fmaf(sc, ubyte_f32<0>(lo), bi), fmaf(sc, ubyte_f32<0>(hi), bi));
       o.y = pack_bf16x2(fmaf(sc, ubyte_f32<1>(lo), bi), fmaf(sc, ubyte_f32<1>(hi), bi));

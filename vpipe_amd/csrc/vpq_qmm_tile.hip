@@ -85,8 +85,11 @@ __device__ __forceinline__ float ubyte_f32(uint32_t v) { return (float)((v >> (8
 // 8 nibbles of one word -> 8 bf16 of fma(s, q, b), as one 16-byte LDS chunk.
 __device__ __forceinline__ uint4 dequant_word(uint32_t word, float s, float b)
 {
-  const uint32_t lo = word & 0x0f0f0f0fu;          // q0 q2 q4 q6
-  const uint32_t hi = (word >> 4) & 0x0f0f0f0fu;   // q1 q3 q5 q7
+  uint32_t lo = word & 0x0f0f0f0fu;                // q0 q2 q4 q6
+  uint32_t hi = (word >> 4) & 0x0f0f0f0fu;         // q1 q3 q5 q7
+  // No instruction: keeps the masked words as they are, so that each value is one v_cvt_f32_ubyteN
+  // of them (otherwise the mask is folded into a bit-field extract per value, one instruction more).
+  asm volatile("" : "+v"(lo), "+v"(hi));
   const float v0 = fmaf(s, ubyte_f32<0>(lo), b);
   const float v1 = fmaf(s, ubyte_f32<0>(hi), b);
   const float v2 = fmaf(s, ubyte_f32<1>(lo), b);
