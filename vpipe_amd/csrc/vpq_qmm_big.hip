@@ -233,7 +233,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   // other stage.  Piece P (0..63) of that dequantization is word P/8 of the row step at stage P%8 of
   //   0: split the nibbles   1..4: two values each, fma(s, q, b)   5: pack to bf16   6: store   7: -
   // and the pieces are dealt out evenly over the step's 4 MQ MFMAs.
-  auto compute = [&](auto stage_c, auto fill_c, int s, int ksteps) {
+  auto compute = [&](auto stage_c, auto fill_c, int s, int ksteps, auto&& loads) {
     constexpr int ST = decltype(stage_c)::value;
     constexpr bool FILL = decltype(fill_c)::value;
     const uint8_t* xb = ST ? x_lds1 : x_lds0;
@@ -305,6 +305,8 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
             constexpr int G = Q * MQ + J;                // MFMA index within the step
             static_assert(WPT * 8 == 4 * MQ, "one piece per MFMA");
             piece(std::integral_constant<int, G>());
+            // the step's 12 load requests, one after every other MFMA of its first 24
+            if constexpr ((G & 1) == 1 && G < 24) { loads(std::integral_constant<int, (G >> 1)>()); }
           }
           // the next quarter's fragments, one read after every MFMA until they are all requested
           if constexpr (Q < 3 && J < 4 + NT) {
@@ -352,14 +354,28 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     using St = decltype(stage_c);
     using Nx = std::integral_constant<int, 1 - St::value>;
     constexpr bool FILL = decltype(fill_c)::value;      // false for the last step only
-    bool scales_out = false;
-    if constexpr (FILL) { issue_x(s + 1, Nx()); }
-    if (s + 2 < KT) { issue_codes(s + 2); }
-    if (St::value == 0 && (s & 7) == 0 && s + 8 < KT && dq_wave) {
-      issue_scales((s >> 3) + 1);
-      scales_out = true;
-    }
-    compute(St(), fill_c, s, 4);
+    const bool codes_out = s + 2 < KT && dq_wave;
+    const bool scales_out = St::value == 0 && (s & 7) == 0 && s + 8 < KT && dq_wave;
+    // The requests go out from inside the MFMA stream, in the order x [8], codes [2], scales [2].
+    const uint8_t* xsrc = xblk + (size_t)(s + 1) * (BK * 2);
+    const uint32_t xdst = lds_addr(Nx::value ? x_lds1 : x_lds0) + wave * (64 * kRow);
+    const uint8_t* csrc = wblk + (size_t)(s + 2) * 32;
+    const uint32_t cdst = lds_addr(c_lds) + (s & 1) * kCodeBytes + wave * (64 * 32);
+    const int blk = (s >> 3) + 1;
+    const uint32_t sdst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave * (64 * 16);
+    auto loads = [&](auto ic) {
+      constexpr int I = decltype(ic)::value;
+      if constexpr (I < 8) {
+        dma16(xdst + I * (8 * kRow), xsrc, a_off[I]);
+      } else if constexpr (I < 10) {
+        if (codes_out) { dma16(cdst + (I - 8) * (32 * 32), csrc, c_off[I - 8]); }
+      } else if constexpr (I == 10) {
+        if (scales_out) { dma16(sdst, srow + (size_t)blk * 16); }
+      } else {
+        if (scales_out) { dma16(sdst + 256 * 16, brow + (size_t)blk * 16); }
+      }
+    };
+    compute(St(), fill_c, s, 4, loads);
     if (scales_out) {
       asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
     } else {
@@ -407,7 +423,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       wg_barrier();                                    // tiles ready
-      compute(S0(), std::false_type(), 0, chunks >> 1);
+      compute(S0(), std::false_type(), 0, chunks >> 1, [](auto) {});
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       wg_barrier();                                    // everyone done with them
     }
