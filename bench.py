@@ -356,7 +356,7 @@ def main():
         out["qmm_m2048"] = qmm
         out["roofline_qmm"] = {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TF,
                                "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TF, 4), "traffic": None,
-                               "kernel": "qmm_big_kernel<3,false> (4096->12288: 256x192 tiles), qmm_tile_kernel<false> "
+                               "kernel": "qmm_big_kernel<3,false> (4096->12288: 256x192 tiles) and qmm_big_kernel<2,false> "
                                          "(12288->4096, 4096->4096: 256x128 tiles); flops of the three over their time",
                                "note": "vendor_dense_bf16_TFLOPs in qmm_m2048 = torch.matmul on the expanded "
                                        "weight, same operands: the dense-GEMM rate this box sustains on real data"}

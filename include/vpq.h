@@ -168,10 +168,10 @@ int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
                        uint16_t* lora_t_ws);
 
 /* The same with the kernel named: tile_n = 128 is the 256 x 128 tile kernel (any K % 64 == 0),
- * 192 / 256 the large-tile kernel (256 x tile_n per workgroup; needs K % 512 == 0 and 16-byte
+ * 192 / 256 / -128 the large-tile kernel at width 192 / 256 / 128 (needs K % 512 == 0 and 16-byte
  * aligned scales and biases, else VPQ_ERR_BAD_SHAPE), which vpq_qmm_w4g64_bf16 takes by itself once
- * its tiles make two rounds over the CUs (the video-DiT projections; 4096 -> 12288 at M = 2048 at
- * width 192).  Both kernels accumulate K in the same order with the same instruction: their
+ * its tiles fill the CUs (the prefill and video-DiT projections), at the width a small cost model
+ * picks.  Both kernels accumulate K in the same order with the same instruction: their
  * results are bit-identical.  For measurement and tests; no counterpart in the reference. */
 int vpq_qmm_tiled_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,

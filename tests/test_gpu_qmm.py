@@ -215,7 +215,7 @@ def test_linear_entrance_splits_k_when_given_the_room(vpq, oracle, dev, D):
 BIG_TILE_SHAPES = [(300, 520, 512), (257, 193, 1024), (2300, 200, 512), (1, 8, 512), (640, 384, 1536)]
 
 
-@pytest.mark.parametrize("tile_n", [192, 256])
+@pytest.mark.parametrize("tile_n", [-128, 192, 256])
 @pytest.mark.parametrize("M,N,K", BIG_TILE_SHAPES)
 def test_qmm_large_tile_kernel(vpq, oracle, dev, D, M, N, K, tile_n):
     # against the oracle, and bit for bit against the 256x128 tile kernel: same MFMA, same K order
@@ -234,7 +234,7 @@ def test_qmm_large_tile_kernel(vpq, oracle, dev, D, M, N, K, tile_n):
     parity.check_bf16(D.bits(out.view)[ms], y64, yb)
 
 
-@pytest.mark.parametrize("tile_n", [192, 256])
+@pytest.mark.parametrize("tile_n", [-128, 192, 256])
 @pytest.mark.parametrize("r", [32, 64, 96])
 def test_qmm_large_tile_kernel_with_lora(vpq, oracle, dev, D, r, tile_n):
     M, N, K, alpha = 300, 450, 1024, 0.75

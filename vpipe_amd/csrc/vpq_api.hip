@@ -306,7 +306,8 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
 
 namespace {
 
-// tile: 0 = by size, 128 = the 256 x 128 tile kernel, 192 / 256 = the large-tile kernel at that width
+// tile: 0 = by size, 128 = the 256 x 128 tile kernel, 192 / 256 = the large-tile kernel at that width,
+// -128 = the large-tile kernel at width 128
 int qmm_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
@@ -338,16 +339,18 @@ int qmm_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   g.lora_b = lora ? lora_b : nullptr;
   g.r = lora ? r : 0;
   g.cu_count = g_dev.cu_count;
-  if (tile == 192 || tile == 256) {
+  if (tile == 192 || tile == 256 || tile == -128) {
     if (!vpq::qmm_big_supports(g)) { return VPQ_ERR_BAD_SHAPE; }
-    return finish(vpq::launch_qmm_big(hs, g, tile));
+    return finish(vpq::launch_qmm_big(hs, g, tile < 0 ? -tile : tile));
   }
-  // The large-tile kernel once its tiles make at least two rounds over the CUs (measured at
-  // M = 16320: 0.98-1.07 against 0.75-0.89 PFLOP/s); below that the smaller tile fills the chip better.
+  // The large-tile kernel once its tiles fill the CUs at least once (measured: 1.02-1.16 against
+  // 0.83-0.91 PFLOP/s at M = 16320, 0.98 against 0.78 at 4096 -> 12288 and 0.94 against 0.91 at
+  // 12288 -> 4096 with M = 2048); with fewer tiles the two are equal and the tile kernel has the
+  // split-K form beside it.
   if (tile == 0 && vpq::qmm_big_supports(g)) {
     const int bn = vpq::qmm_big_tile_n(N, M, g_dev.cu_count);
     const long tiles = (long)((M + 255) / 256) * (long)((N + bn - 1) / bn);
-    if (tiles >= 2L * (g_dev.cu_count > 0 ? g_dev.cu_count : 256)) { return finish(vpq::launch_qmm_big(hs, g, bn)); }
+    if (tiles >= (long)(g_dev.cu_count > 0 ? g_dev.cu_count : 256)) { return finish(vpq::launch_qmm_big(hs, g, bn)); }
   }
   return finish(vpq::launch_qmm_tile(hs, g));
 }
@@ -367,7 +370,7 @@ int vpq_qmm_tiled_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
                              const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
                              uint16_t* lora_t_ws, int tile_n)
 {
-  if (tile_n != 128 && tile_n != 192 && tile_n != 256) { return VPQ_ERR_BAD_SHAPE; }
+  if (tile_n != 128 && tile_n != -128 && tile_n != 192 && tile_n != 256) { return VPQ_ERR_BAD_SHAPE; }
   return qmm_common(stream, w, scales, biases, x, y, K, N, M, lora_a, lora_b, r, alpha, lora_t_ws, tile_n);
 }
 

@@ -4,7 +4,7 @@
 // v_mfma_f32_32x32x16_bf16 over K in ascending order, fp32 accumulators, one rounding -- and the
 // same bits; what differs is who does what.
 //
-// A workgroup owns 256(M) x BN(N) of y, BN = 64 NT in {256, 192}, and has FOUR wavefronts, one per
+// A workgroup owns 256(M) x BN(N) of y, BN = 64 NT in {256, 192, 128}, and has FOUR wavefronts, one per
 // SIMD, each with a 128 x (BN/2) block of accumulators (up to 256 registers, in the accumulation
 // file).  A wavefront's operand reads from LDS are then (4 + NT) fragments per 4 NT MFMAs -- half the
 // LDS bytes per MFMA of a 128 x 64 block -- which is what bounds the smaller tile: there the LDS
@@ -472,24 +472,31 @@ bool qmm_big_supports(const GemmArgs& a)
   return true;
 }
 
-// Tile width by the number of whole rounds of workgroups over the CUs: 256 unless 192 fills the
-// last round better (4096 -> 12288 at M = 2048: 384 tiles of 256 are one and a half rounds of 256
-// CUs, 512 tiles of 192 are two).
+// Tile width by a small cost model: workgroups run one per CU, so a launch takes ceil(tiles / CUs)
+// rounds, and a round's time grows with the tile width (the MFMA work) over the width's efficiency
+// (measured with whole rounds: 256 wide 1.02, 192 wide 0.98, 128 wide 0.94 PFLOP/s).  4096 -> 12288 at
+// M = 2048: 384 tiles of 256 are one and a half rounds of 256 CUs, 512 tiles of 192 are two;
+// N = 4096 at M = 2048 is exactly one round of 128-wide tiles.
 int qmm_big_tile_n(int N, int M, int cu_count)
 {
   const int cus = cu_count > 0 ? cu_count : 256;
   const long tm = (M + BM - 1) / BM;
-  auto cost = [&](int bn) {
-    const long tiles = tm * ((N + bn - 1) / bn);
+  const int widths[3] = {256, 192, 128};
+  const double eff[3] = {1.0, 0.95, 0.90};
+  int best = 256;
+  double best_cost = 0.0;
+  for (int i = 0; i < 3; ++i) {
+    const long tiles = tm * ((N + widths[i] - 1) / widths[i]);
     const long rounds = (tiles + cus - 1) / cus;
-    return (double)rounds * (double)bn;          // time of a round grows with the tile width
-  };
-  return cost(192) < cost(256) ? 192 : 256;
+    const double cost = (double)rounds * (double)widths[i] / eff[i];
+    if (i == 0 || cost < best_cost) { best = widths[i]; best_cost = cost; }
+  }
+  return best;
 }
 
 hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
 {
-  const int bn = tile_n == 192 || tile_n == 256 ? tile_n : qmm_big_tile_n(a.N, a.M, a.cu_count);
+  const int bn = tile_n == 128 || tile_n == 192 || tile_n == 256 ? tile_n : qmm_big_tile_n(a.N, a.M, a.cu_count);
   BigParams p;
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
   p.lora_t = a.lora_t; p.lora_b = a.lora_b;
@@ -498,6 +505,10 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
   p.tiles_n = (a.N + bn - 1) / bn;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kBigThreads);
   const bool lora = a.lora_t != nullptr;
+  if (bn == 128) {
+    return lora ? launch_kernel(qmm_big_kernel<2, true>, grid, block, 0, st, p)
+                : launch_kernel(qmm_big_kernel<2, false>, grid, block, 0, st, p);
+  }
   if (bn == 192) {
     return lora ? launch_kernel(qmm_big_kernel<3, true>, grid, block, 0, st, p)
                 : launch_kernel(qmm_big_kernel<3, false>, grid, block, 0, st, p);
