@@ -257,3 +257,31 @@ def test_qmm_and_linear_geglu(vpq, oracle, dev, D, M, F, K):
     with pytest.raises(capi.VpqError):
         vpq.qmm_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, activation=3)
 
+
+
+# shapes whose tiles fill the CUs, so that the gated store of the large-tile GEMM kernel runs, at each of its
+# tile widths (the library picks 128, 256, 192 for these), ragged M, strided and offset output windows
+@pytest.mark.parametrize("activation", [capi.VPQ_GATE_SWIGLU, capi.VPQ_GATE_GEGLU])
+@pytest.mark.parametrize("M,F,K,stride,off", [(4100, 2048, 512, 0, 0), (4100, 3072, 512, 3200, 64), (2048, 6144, 512, 6145, 1)])
+def test_qmm_gated_store_of_the_large_tile_kernel(vpq, oracle, dev, D, M, F, K, stride, off, activation):
+    _, _, pack = fused_pack(oracle, F, K, 2100 + F)
+    x = synth.make_act(M, K, 2101 + M)
+    wd, sd, bd, xd = stage(D, dev, pack, x)
+    width = stride if stride > 0 else F
+    out = parity.Guarded((M, width), torch.bfloat16, dev)
+    out.view.fill_(7.0)
+    vpq.qmm_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, M, out=out.view, out_stride=stride, out_off=off, activation=activation)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    got_all = out.view
+    if stride > 0:      # nothing outside the window was touched
+        assert bool((got_all[:, :off] == 7.0).all()) and bool((got_all[:, off + F:] == 7.0).all())
+    rng = np.random.default_rng(F + M)
+    rows = np.unique(np.concatenate([[0, M - 1, 255, 256, 2047 % M], rng.choice(M, 16, replace=False)]))
+    feats = np.unique(np.concatenate([[0, F - 1, 63, 64, 95, 96, 127, 128], rng.choice(F, 64, replace=False)]))
+    sel = np.stack([2 * feats, 2 * feats + 1], 1).ravel()
+    w, s, b = pack
+    y64 = oracle.qmm(w[sel], s[sel], b[sel], x[rows], K, len(sel), len(rows))[0]
+    o64, ob = (oracle.swiglu if activation == capi.VPQ_GATE_SWIGLU else oracle.geglu)(y64)
+    got = D.bits(got_all[torch.from_numpy(rows).to(dev)][:, torch.from_numpy(off + feats).to(dev)])
+    parity.check_bf16(got, o64, ob, mismatch_over_all=activation == capi.VPQ_GATE_SWIGLU)

@@ -522,6 +522,14 @@ int vpq_qmm_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
   g.gate_act = activation;
   g.out_stride = out_stride;
   g.out_off = out_off;
+  // as vpq_qmm_w4g64_bf16: the large-tile kernel once its tiles fill the CUs (bit-identical results)
+  if (vpq::qmm_big_supports(g)) {
+    const int bn = vpq::qmm_big_tile_n(N, M, g_dev.cu_count);
+    const long tiles = (long)((M + 255) / 256) * (long)((N + bn - 1) / bn);
+    if (tiles >= (long)(g_dev.cu_count > 0 ? g_dev.cu_count : 256)) {
+      return finish(vpq::launch_qmm_big(reinterpret_cast<hipStream_t>(stream), g, bn));
+    }
+  }
   return finish(vpq::launch_qmm_tile(reinterpret_cast<hipStream_t>(stream), g));
 }
 

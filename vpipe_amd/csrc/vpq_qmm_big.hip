@@ -55,6 +55,9 @@ struct BigParams {
   const uint16_t* lora_b;   // [N,r]
   int K, N, M, r;
   int tiles_m, tiles_n;
+  // Gated store (1 SwiGLU, 2 GEGLU): the pack is an interleaved gate|up matrix and
+  // y[m * out_stride + out_off + g] = act(gate_g) * up_g (affine_qmm_steel.metal:663-768, 1460-1572).
+  int gate_act, out_stride, out_off;
 };
 
 __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
@@ -430,6 +433,34 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   }
 
   // ---- store: lane holds, for x row m = lane%32 of each it, 4 consecutive n per register quad ----
+  if (!LORA && p.gate_act) {                           // never together with an adapter
+    // A register quad is (gate, up, gate, up) of features n/2 and n/2 + 1 (n is a multiple of 4):
+    // the activation is register-local and a quad becomes one dword of two bf16.
+    const bool pair_ok = ((p.out_stride | p.out_off) & 1) == 0;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int m = m0 + wm * 128 + it * 32 + frow;
+      if (m >= p.M) { continue; }
+      uint16_t* yrow = p.y + (size_t)m * p.out_stride + p.out_off;
+#pragma unroll
+      for (int jt = 0; jt < NT; ++jt) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int n = n0 + wn * (BN / 2) + jt * 32 + rq * 8 + fkh * 4;
+          if (n >= p.N) { continue; }
+          const float f0 = gated_f32(p.gate_act, acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
+          const float f1 = gated_f32(p.gate_act, acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
+          if (pair_ok && n + 3 < p.N) {
+            *reinterpret_cast<uint32_t*>(yrow + (n >> 1)) = pack_bf16x2(f0, f1);
+          } else {
+            yrow[n >> 1] = (uint16_t)f32_to_bf16_bits(f0);
+            if (n + 3 < p.N) { yrow[(n >> 1) + 1] = (uint16_t)f32_to_bf16_bits(f1); }
+          }
+        }
+      }
+    }
+    return;
+  }
   const bool vec_ok = (p.N & 3) == 0;
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
@@ -464,8 +495,9 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
 bool qmm_big_supports(const GemmArgs& a)
 {
   // K in blocks of 8 steps (the scale ring) with 16-byte aligned rows of scales; 32-bit offsets
-  // inside the pack and inside a band of x; no gated store.
-  if (a.K % 512 != 0 || a.M < 1 || a.N < 1 || a.gate_act != 0) { return false; }
+  // inside the pack and inside a band of x.
+  if (a.K % 512 != 0 || a.M < 1 || a.N < 1) { return false; }
+  if (a.gate_act != 0 && (a.lora_t != nullptr || (a.N & 1) != 0)) { return false; }
   if ((reinterpret_cast<uintptr_t>(a.scales) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.biases) & 15) != 0) { return false; }
   if ((double)a.N * (double)a.K / 2.0 >= 4.0e9 || (double)BM * (double)a.K * 2.0 >= 4.0e9) { return false; }
   if (a.lora_t != nullptr && (a.r < 32 || a.r % 32 != 0)) { return false; }
@@ -503,6 +535,9 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
   p.K = a.K; p.N = a.N; p.M = a.M; p.r = a.r;
   p.tiles_m = (a.M + BM - 1) / BM;
   p.tiles_n = (a.N + bn - 1) / bn;
+  p.gate_act = a.gate_act;
+  p.out_stride = a.out_stride > 0 ? a.out_stride : a.N / 2;
+  p.out_off = a.out_off;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kBigThreads);
   const bool lora = a.lora_t != nullptr;
   if (bn == 128) {
