@@ -356,6 +356,57 @@ int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
                                    const int32_t* pair_eid, int npair, int n_experts);
 
+/* ---- MoE prefill: expert-sorted (grouped) GEMMs ---------------------------
+ * With many tokens the pairs are sorted by expert into blocks of
+ * vpq_qmm_grouped_block_rows() slots, each block owned by ONE expert, and two
+ * tiled GEMMs run over the sorted slots, reading every expert slab once per
+ * block instead of once per pair
+ * (generative-models/qwen3/metal-qwen-model.cc:4209-4264).
+ *
+ * vpq_moe_sort_pairs replaces the sort's four dispatches `moe_ifill_i32`,
+ * `moe_hist_i32`, `moe_sort_setup_i32`, `moe_scatter_i32`
+ * (gpu-kernels/metal/ops/llm_elementwise.metal:255-326) with the reference's
+ * sizing: max_tiles >= ceil(npair / block_rows) + min(n_experts, npair) blocks,
+ * npad = max_tiles * block_rows slots.  Outputs (device, int32):
+ * tile2e[max_tiles] expert per block (-1 unused), srow[npad] token row per slot
+ * (= pair / top_k; -1 padding), sdst[npad] pair per slot (-1 padding),
+ * ntiles[1] blocks in use.  Experts ascend; the order of the pairs inside an
+ * expert's share is unspecified, as in the reference.  A pair whose id is
+ * outside [0, n_experts) gets no slot.  ws: vpq_moe_sort_workspace_bytes()
+ * bytes of device memory, 4-byte aligned.  block_rows is any positive count
+ * (the GEMMs below need vpq_qmm_grouped_block_rows()).
+ *
+ * vpq_qmm_grouped_gated_w4g64_bf16 replaces `affine_qmm_grouped_swiglu_w4g64`
+ * and `affine_qmm_grouped_geglu_w4g64` (gpu-kernels/metal/quant/
+ * affine_qmm_steel.metal:1314-1339, 1266-1288; slots 0:w[E,N,K/8] 1:scales
+ * 2:biases 3:x[rows_x,K] 4:y[npad,N/2] 5:K 6:N=2*inner 7:npad 8:tile2e 9:srow):
+ * slot i contracts x row srow[i] with the interleaved gate|up slab of its
+ * block's expert and stores act(gate)*up into y row i; a padding slot
+ * (srow < 0, or >= rows_x) stores zeros, as the reference's zero-filled rows do;
+ * a block with tile2e < 0 (or >= n_experts) is left untouched.
+ * vpq_qmm_grouped_down_w4g64_bf16 replaces `affine_qmm_grouped_w4g64`
+ * (:1042-1066; 3:x[npad,K] sorted activations 4:y[rows_y,N] 9:sdst): slot i
+ * contracts x row i with the down slab and stores into y row sdst[i]
+ * (nothing for sdst < 0 or >= rows_y).
+ * QMM arithmetic (bf16-rounded weight, fp32 accumulation over K ascending, one
+ * rounding): a slot's result has the bits of vpq_qmm_tiled_w4g64_bf16 (tile
+ * 128) on that row and that expert's slab.  Requires K % 64 == 0, npad a
+ * positive multiple of vpq_qmm_grouped_block_rows(), N even for the gated form,
+ * rows * K * 2 < 4e9 for x; w, x 16-byte aligned. */
+int vpq_qmm_grouped_block_rows(void);
+size_t vpq_moe_sort_workspace_bytes(int n_experts);
+int vpq_moe_sort_pairs(vpq_stream_t stream, const int32_t* pair_eid, int npair, int top_k, int n_experts,
+                       int block_rows, int max_tiles, int32_t* tile2e, int32_t* srow, int32_t* sdst,
+                       int32_t* ntiles, void* ws, size_t ws_bytes);
+int vpq_qmm_grouped_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                     int npad, const int32_t* tile2e, const int32_t* srow, int n_experts,
+                                     int rows_x, int activation);
+int vpq_qmm_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                    int npad, const int32_t* tile2e, const int32_t* sdst, int n_experts,
+                                    int rows_y);
+
 /* ---- 4-bit group-32 twins (w4g32; GGUF Q4_0 repacked to affine) ---------------
  * The 4-bit pack with a scale and a bias per 32 values: w uint32 [N, K/8] as
  * above, scales, biases bf16 [N, K/32].

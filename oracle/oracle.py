@@ -185,6 +185,38 @@ def qmm(w, s, b, x, K, N, M, t=None, B=None, r=0):
     return y64, yb
 
 
+_i32p = ctypes.POINTER(ctypes.c_int32)
+
+
+def moe_sort_pairs(eid, top_k, E, block_rows, max_tiles):
+    """-> (tile2e [max_tiles], srow [npad], sdst [npad], blocks in use); pairs of an expert in ascending order."""
+    eid = _c(eid, np.int32)
+    npad = max_tiles * block_rows
+    t2e = np.empty(max_tiles, dtype=np.int32)
+    srow = np.empty(npad, dtype=np.int32)
+    sdst = np.empty(npad, dtype=np.int32)
+    lib().vpo_moe_sort_pairs.restype = ctypes.c_int
+    used = lib().vpo_moe_sort_pairs(_p(eid, _i32p), int(eid.size), top_k, E, block_rows, max_tiles,
+                                    _p(t2e, _i32p), _p(srow, _i32p), _p(sdst, _i32p))
+    return t2e, srow, sdst, used
+
+
+def qmm_grouped(w, s, b, x, K, N, block_rows, tile2e, srow=None, sdst=None, rows_y=None):
+    """Grouped expert GEMM over sorted slots -> (y64, y_bf16).  With srow (gate|up) the outputs are
+    [npad, N] in slot order; with sdst (down) they are [rows_y, N] in pair order (rows no slot
+    writes stay zero)."""
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    tile2e, srow, sdst = _c(tile2e, np.int32), _c(srow, np.int32), _c(sdst, np.int32)
+    npad = int(tile2e.size) * block_rows
+    rows = npad if sdst is None else rows_y
+    y64 = np.zeros((rows, N), dtype=np.float64)
+    yb = np.zeros((rows, N), dtype=np.uint16)
+    lib().vpo_qmm_grouped_w4g64(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y64, _f64p),
+                                _p(yb, _u16p), K, N, npad, block_rows, _p(tile2e, _i32p), _p(srow, _i32p),
+                                _p(sdst, _i32p))
+    return y64, yb
+
+
 def interleave(a, b):
     """Rows of a and b (same shape, same dtype) alternating: out[2g] = a[g], out[2g+1] = b[g]."""
     a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)

@@ -458,6 +458,100 @@ void vpo_geglu_pairs(const double* y, double* out64, uint16_t* out_bf16, int M, 
   }
 }
 
+/* ---- MoE prefill: the expert sort and the grouped GEMMs ------------------- */
+
+/* gpu-kernels/metal/ops/llm_elementwise.metal:255-326 (moe_ifill_i32, moe_hist_i32,
+ * moe_sort_setup_i32, moe_scatter_i32): a histogram of the pairs over the experts, every
+ * expert's share rounded up to whole blocks of block_rows slots, experts ascending;
+ * tile2e[t] the expert of block t (-1 unused), srow[slot] = pair / top_k, sdst[slot] = pair
+ * (-1 for padding slots).  The reference hands the slots of an expert out by an atomic
+ * counter (any order); this restatement takes the pairs in ascending order.  A pair with an
+ * id outside [0, E) is skipped (the reference would index out of bounds).  Returns the blocks
+ * in use. */
+int vpo_moe_sort_pairs(const int32_t* eid, int np, int top_k, int E, int block_rows, int max_tiles,
+                       int32_t* tile2e, int32_t* srow, int32_t* sdst)
+{
+  const int npad = max_tiles * block_rows;
+  int* hist = (int*)calloc((size_t)E, sizeof(int));
+  int* boff = (int*)calloc((size_t)E, sizeof(int));
+  int* cursor = (int*)calloc((size_t)E, sizeof(int));
+  for (int i = 0; i < npad; ++i) { srow[i] = -1; sdst[i] = -1; }
+  for (int t = 0; t < max_tiles; ++t) { tile2e[t] = -1; }
+  for (int p = 0; p < np; ++p) {
+    if (eid[p] >= 0 && eid[p] < E) { hist[eid[p]] += 1; }
+  }
+  int off = 0;
+  for (int e = 0; e < E; ++e) {
+    boff[e] = off;
+    const int nt = (hist[e] + block_rows - 1) / block_rows;
+    const int t0 = off / block_rows;
+    for (int t = 0; t < nt; ++t) {
+      if (t0 + t < max_tiles) { tile2e[t0 + t] = e; }
+    }
+    off += nt * block_rows;
+  }
+  for (int p = 0; p < np; ++p) {
+    const int e = eid[p];
+    if (e < 0 || e >= E) { continue; }
+    const int slot = boff[e] + cursor[e]++;
+    if (slot < npad) { srow[slot] = p / top_k; sdst[slot] = p; }
+  }
+  free(hist); free(boff); free(cursor);
+  return off / block_rows;
+}
+
+/* The grouped expert GEMMs over the sorted slots
+ * (gpu-kernels/metal/quant/affine_qmm_steel.metal:1092-1170 gate|up with the gathering
+ * loader :972-1020, :1367-1458 down with the scattering store): block t = slots
+ * [t*block_rows, ...) multiplies the slab of expert tile2e[t] of the batched pack
+ * [E, N, K/8] (a block with tile2e < 0 is skipped, its outputs untouched).
+ *   srow != NULL (gate|up): x row of slot i is x[srow[i]], zeros for srow[i] < 0; the sums
+ *     go to y64[i, :] (the caller applies the gated store);
+ *   sdst != NULL (down): x row of slot i is x[i]; the sums go to y64[sdst[i], :] and their
+ *     bf16 rounding to y_bf16[sdst[i], :] (slots with sdst < 0 write nothing).
+ * Arithmetic of vpo_qmm_w4g64: bf16-rounded weights, contraction in double. */
+void vpo_qmm_grouped_w4g64(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int npad,
+                           int block_rows, const int32_t* tile2e, const int32_t* srow,
+                           const int32_t* sdst)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
+  for (int t = 0; t < npad / block_rows; ++t) {
+    const int e = tile2e[t];
+    if (e < 0) { continue; }
+    const uint32_t* we = w + (size_t)e * N * Kw;
+    const uint16_t* se = scales + (size_t)e * N * Kg;
+    const uint16_t* be = biases + (size_t)e * N * Kg;
+    for (size_t n = 0; n < (size_t)N; ++n) {
+      for (int k = 0; k < K; ++k) {
+        const float s = vpo_bf16_to_f32(se[n * Kg + k / VPO_GROUP]);
+        const float b = vpo_bf16_to_f32(be[n * Kg + k / VPO_GROUP]);
+        const float sq = s * (float)nibble(we, n, Kw, k);
+        wrow[k] = vpo_bf16_to_f32(vpo_f32_to_bf16(sq + b));
+      }
+      for (int i = t * block_rows; i < (t + 1) * block_rows; ++i) {
+        double acc = 0.0;
+        long dst = i;
+        if (srow) {
+          if (srow[i] >= 0) {
+            const uint16_t* xr = x + (size_t)srow[i] * K;
+            for (int k = 0; k < K; ++k) { acc += (double)vpo_bf16_to_f32(xr[k]) * (double)wrow[k]; }
+          }
+        } else {
+          if (sdst[i] < 0) { continue; }
+          dst = sdst[i];
+          const uint16_t* xr = x + (size_t)i * K;
+          for (int k = 0; k < K; ++k) { acc += (double)vpo_bf16_to_f32(xr[k]) * (double)wrow[k]; }
+        }
+        if (y64) { y64[(size_t)dst * N + n] = acc; }
+        if (y_bf16) { y_bf16[(size_t)dst * N + n] = vpo_f32_to_bf16((float)acc); }
+      }
+    }
+  }
+  free(wrow);
+}
+
 /* ---- a12: the packer --------------------------------------------------- */
 
 /* gpu-kernels/metal/quant/affine_dequant.metal:243-285 (affine_quant_impl<4,64>):

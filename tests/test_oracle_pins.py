@@ -503,3 +503,62 @@ def test_group32_twins_against_closed_forms_and_the_group64_oracle(oracle):
     res = synth.make_act(M, N, 914)
     _, with_res = oracle.qmv_g32(w, s, None, x, K, N, M, residual=res, scale_only=True)
     assert np.array_equal(with_res, synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(yb_q) + synth.bf16_bits_to_f32(res)))
+
+
+def test_moe_sort_and_grouped_gemm_reduce_to_the_per_pair_statement(oracle):
+    """The expert sort against numpy's stable argsort (an independent statement of a counting sort) and
+    its invariants; the grouped GEMMs against the plain oracle GEMM of every pair on its expert's
+    slab (the reference's claim for them: "token-exact with the per-pair paths",
+    gpu-kernels/metal/quant/affine_qmm_steel.metal:1027-1031)."""
+    E, top_k, T, B = 5, 2, 9, 4
+    rng = np.random.default_rng(31)
+    eid = rng.integers(0, E, size=T * top_k, dtype=np.int32)
+    eid[3] = 4
+    eid[eid == 2] = 1                                   # expert 2 gets nothing
+    npair = eid.size
+    max_tiles = (npair + B - 1) // B + E
+    t2e, srow, sdst, used = oracle.moe_sort_pairs(eid, top_k, E, B, max_tiles)
+    hist = np.bincount(eid, minlength=E)
+    blocks = (hist + B - 1) // B
+    assert used == blocks.sum()
+    assert np.array_equal(t2e[:used], np.repeat(np.arange(E), blocks)) and (t2e[used:] == -1).all()
+    order = np.argsort(eid, kind="stable")              # pairs by expert, ascending inside an expert
+    first = np.concatenate([[0], np.cumsum(blocks)[:-1]]) * B
+    want_sdst = np.full(max_tiles * B, -1, dtype=np.int32)
+    pos = 0
+    for e in range(E):
+        want_sdst[first[e]:first[e] + hist[e]] = order[pos:pos + hist[e]]
+        pos += hist[e]
+    assert np.array_equal(sdst, want_sdst)
+    assert np.array_equal(srow, np.where(want_sdst >= 0, want_sdst // top_k, -1))
+    assert sorted(sdst[sdst >= 0].tolist()) == list(range(npair))
+
+    K, inner, H = 128, 6, 10
+    gu = [synth.make_weight(2 * inner, K, 700 + e) for e in range(E)]
+    dn = [synth.make_weight(H, K, 800 + e) for e in range(E)]
+    guw, gus, gub = (np.stack([p[i] for p in gu]) for i in range(3))
+    dw, ds, db = (np.stack([p[i] for p in dn]) for i in range(3))
+    x = synth.make_act(T, K, 900)
+    y64, yb = oracle.qmm_grouped(guw, gus, gub, x, K, 2 * inner, B, t2e, srow=srow)
+    for slot in range(max_tiles * B):
+        if t2e[slot // B] < 0:
+            continue
+        if srow[slot] < 0:
+            assert not y64[slot].any()                  # zero row in, zero sums out
+            continue
+        e = t2e[slot // B]
+        assert e == eid[sdst[slot]]
+        p64, pb = oracle.qmm(guw[e], gus[e], gub[e], x[srow[slot]:srow[slot] + 1], K, 2 * inner, 1)
+        assert np.array_equal(y64[slot], p64[0]) and np.array_equal(yb[slot], pb[0])
+    xs = synth.make_act(max_tiles * B, K, 901)
+    d64, dbits = oracle.qmm_grouped(dw, ds, db, xs, K, H, B, t2e, sdst=sdst, rows_y=npair)
+    for slot in range(max_tiles * B):
+        p = sdst[slot]
+        if p < 0:
+            continue
+        p64, pb = oracle.qmm(dw[eid[p]], ds[eid[p]], db[eid[p]], xs[slot:slot + 1], K, H, 1)
+        assert np.array_equal(d64[p], p64[0]) and np.array_equal(dbits[p], pb[0])
+    # ids outside [0, E) get no slot
+    bad = np.array([1, -1, E, 0], dtype=np.int32)
+    t2, sr, sd, u = oracle.moe_sort_pairs(bad, 1, E, B, 6)
+    assert sorted(sd[sd >= 0].tolist()) == [0, 3] and u == 2

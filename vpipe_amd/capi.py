@@ -40,6 +40,11 @@ SYMBOLS = [
     ("vpq_argmax_combine", _i, [_vp, _vp, _vp, _i]),
     ("vpq_gather_qmv_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
     ("vpq_gather_down_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i]),
+    ("vpq_qmm_grouped_block_rows", _i, []),
+    ("vpq_moe_sort_workspace_bytes", _sz, [_i]),
+    ("vpq_moe_sort_pairs", _i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz]),
+    ("vpq_qmm_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _i]),
+    ("vpq_qmm_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
     ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
     ("vpq_qmv_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _i]),
     ("vpq_qmv_workspace_bytes", _sz, [_i, _i, _i]),
@@ -222,6 +227,58 @@ def gather_down_qmv_w4g64(w, scales, biases, x, K, N, pair_eid, n_experts, out=N
         out = torch.empty((npair, N), dtype=torch.bfloat16, device=w.device)
     _check(load().vpq_gather_down_qmv_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
                                                  _ptr(pair_eid), npair, n_experts), "vpq_gather_down_qmv_w4g64_bf16")
+    return out
+
+
+def grouped_block_rows():
+    return int(load().vpq_qmm_grouped_block_rows())
+
+
+def moe_max_tiles(npair, n_experts, block_rows):
+    """Blocks to provide for npair pairs: every expert's share rounded up to whole blocks."""
+    return (npair + block_rows - 1) // block_rows + min(n_experts, npair)
+
+
+def moe_sort_pairs(pair_eid, top_k, n_experts, block_rows=None, max_tiles=None):
+    """pair_eid int32 [npair] -> (tile2e [max_tiles], srow [npad], sdst [npad], ntiles [1]), device int32."""
+    import torch
+    L = load()
+    npair = pair_eid.numel()
+    if block_rows is None:
+        block_rows = grouped_block_rows()
+    if max_tiles is None:
+        max_tiles = moe_max_tiles(npair, n_experts, block_rows)
+    dev = pair_eid.device
+    npad = max_tiles * block_rows
+    t2e = torch.empty(max_tiles, dtype=torch.int32, device=dev)
+    srow = torch.empty(npad, dtype=torch.int32, device=dev)
+    sdst = torch.empty(npad, dtype=torch.int32, device=dev)
+    ntiles = torch.empty(1, dtype=torch.int32, device=dev)
+    ws_bytes = int(L.vpq_moe_sort_workspace_bytes(n_experts))
+    ws = torch.empty(ws_bytes // 4, dtype=torch.int32, device=dev)
+    _check(L.vpq_moe_sort_pairs(_stream(), _ptr(pair_eid), npair, top_k, n_experts, block_rows, max_tiles, _ptr(t2e),
+                                _ptr(srow), _ptr(sdst), _ptr(ntiles), _ptr(ws), ws_bytes), "vpq_moe_sort_pairs")
+    return t2e, srow, sdst, ntiles
+
+
+def qmm_grouped_gated_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out=None, activation=VPQ_GATE_SWIGLU):
+    """Expert batch [E, N=2*inner, ...], x [rows_x, K], sorted slots -> bf16 [npad, N/2] in slot order."""
+    import torch
+    npad = srow.numel()
+    if out is None:
+        out = torch.empty((npad, N // 2), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_grouped_gated_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                   npad, _ptr(tile2e), _ptr(srow), n_experts, x.shape[0], activation),
+           "vpq_qmm_grouped_gated_w4g64_bf16")
+    return out
+
+
+def qmm_grouped_down_w4g64(w, scales, biases, x, K, N, tile2e, sdst, n_experts, out):
+    """Expert batch [E, N, ...], x [npad, K] in slot order -> rows of out [npair, N] in pair order."""
+    npad = sdst.numel()
+    _check(load().vpq_qmm_grouped_down_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                  npad, _ptr(tile2e), _ptr(sdst), n_experts, out.shape[0]),
+           "vpq_qmm_grouped_down_w4g64_bf16")
     return out
 
 

@@ -615,6 +615,96 @@ int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
   return gather_common(stream, w, scales, biases, x, y, K, N, pair_eid, npair, 1, n_experts, 0);
 }
 
+int vpq_qmm_grouped_block_rows(void) { return vpq::kGroupedBlockRows; }
+
+size_t vpq_moe_sort_workspace_bytes(int n_experts)
+{
+  return n_experts > 0 ? (size_t)3 * (size_t)n_experts * sizeof(int32_t) : 0;
+}
+
+int vpq_moe_sort_pairs(vpq_stream_t stream, const int32_t* pair_eid, int npair, int top_k, int n_experts,
+                       int block_rows, int max_tiles, int32_t* tile2e, int32_t* srow, int32_t* sdst,
+                       int32_t* ntiles, void* ws, size_t ws_bytes)
+{
+  if (pair_eid == nullptr || tile2e == nullptr || srow == nullptr || sdst == nullptr || ntiles == nullptr ||
+      ws == nullptr) {
+    return VPQ_ERR_NULL_POINTER;
+  }
+  if (npair < 1 || top_k < 1 || n_experts < 1 || block_rows < 1 || max_tiles < 1) { return VPQ_ERR_BAD_SHAPE; }
+  if (npair > (1 << 24) || n_experts > 65536) { return VPQ_ERR_BAD_SHAPE; }
+  // every expert's share rounded up to whole blocks must fit
+  const long long need = ((long long)npair + block_rows - 1) / block_rows + (n_experts < npair ? n_experts : npair);
+  if ((long long)max_tiles < need || (long long)max_tiles * block_rows > 0x7fffffffLL) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(pair_eid, 4) || !aligned(tile2e, 4) || !aligned(srow, 4) || !aligned(sdst, 4) || !aligned(ntiles, 4) ||
+      !aligned(ws, 4)) {
+    return VPQ_ERR_MISALIGNED;
+  }
+  if (ws_bytes < vpq_moe_sort_workspace_bytes(n_experts)) { return VPQ_ERR_WORKSPACE; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_moe_sort(reinterpret_cast<hipStream_t>(stream), pair_eid, npair, top_k, n_experts,
+                                     block_rows, max_tiles, tile2e, srow, sdst, ntiles, static_cast<int*>(ws)));
+}
+
+namespace {
+
+int grouped_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, uint16_t* y, int K, int N, int npad, const int32_t* tile2e,
+                   const int32_t* srow, const int32_t* sdst, int n_experts, int rows, int gate_act)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr || tile2e == nullptr || (srow == nullptr && sdst == nullptr)) {
+    return VPQ_ERR_NULL_POINTER;
+  }
+  if (npad < vpq::kGroupedBlockRows || (npad % vpq::kGroupedBlockRows) != 0 || n_experts < 1 || rows < 1) {
+    return VPQ_ERR_BAD_SHAPE;
+  }
+  if (gate_act != 0 && (N & 1) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  // the kernel addresses rows of x by 32-bit byte offsets
+  const long long xrows = srow != nullptr ? rows : npad;
+  if (xrows * (long long)K * 2 >= 4000000000LL) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 2) || !aligned(tile2e, 4) || (srow != nullptr && !aligned(srow, 4)) ||
+      (sdst != nullptr && !aligned(sdst, 4))) {
+    return VPQ_ERR_MISALIGNED;
+  }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::GemmArgs g{};
+  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
+  g.K = K; g.N = N; g.M = npad; g.lora_t = nullptr; g.lora_b = nullptr; g.r = 0;
+  g.cu_count = g_dev.cu_count;
+  g.gate_act = gate_act; g.out_stride = N / 2; g.out_off = 0;
+  vpq::GroupedArgs ga{};
+  ga.tile2e = tile2e; ga.srow = srow; ga.sdst = sdst;
+  ga.n_experts = n_experts;
+  ga.rows_x = srow != nullptr ? rows : npad;
+  ga.rows_y = sdst != nullptr ? rows : npad;
+  return finish(vpq::launch_qmm_grouped(reinterpret_cast<hipStream_t>(stream), g, ga));
+}
+
+}  // namespace
+
+int vpq_qmm_grouped_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                     int npad, const int32_t* tile2e, const int32_t* srow, int n_experts,
+                                     int rows_x, int activation)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (srow == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  return grouped_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, srow, nullptr, n_experts, rows_x,
+                        activation);
+}
+
+int vpq_qmm_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                    int npad, const int32_t* tile2e, const int32_t* sdst, int n_experts,
+                                    int rows_y)
+{
+  if (sdst == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  return grouped_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, nullptr, sdst, n_experts, rows_y, 0);
+}
+
 namespace {
 
 int check_pack_g32(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, int K, int N, bool scale_only)

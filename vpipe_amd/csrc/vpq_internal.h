@@ -133,6 +133,18 @@ hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, u
                          float alpha);
 // 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.
 hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a);
+// Grouped (expert-sorted) form of the tile kernel at 128 rows per block: a.w/scales/biases are the
+// batched pack [E, N, ...], a.M the padded slot count (a multiple of kGroupedBlockRows); see TileParams.
+constexpr int kGroupedBlockRows = 128;
+struct GroupedArgs {
+  const int* tile2e;   // [a.M / kGroupedBlockRows]
+  const int* srow;     // [a.M] or nullptr: x row per slot
+  const int* sdst;     // [a.M] or nullptr: y row per slot
+  int n_experts, rows_x, rows_y;
+};
+hipError_t launch_moe_sort(hipStream_t st, const int* pair_eid, int n_pairs, int top_k, int n_experts, int block_rows,
+                           int max_tiles, int* tile2e, int* srow, int* sdst, int* ntiles, int* ws);
+hipError_t launch_qmm_grouped(hipStream_t st, const GemmArgs& a, const GroupedArgs& g);
 // Large-tile kernel (256 x 256 or 256 x 192 per workgroup, four wavefronts that each load, dequantize
 // and multiply): K % 512 == 0, 16-byte aligned scales / biases, no gated store; same bits as the tile
 // kernel.  tile_n 0 = qmm_big_tile_n().

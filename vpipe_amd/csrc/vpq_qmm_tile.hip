@@ -47,11 +47,8 @@ constexpr int TM = 256, TN = 128, TK = 64;
 constexpr int kConsumers = 4;                        // consumer wavefronts: kConsumers/2 along M, 2 along N
 constexpr int kProducers = 4;
 constexpr int kThreads = (kConsumers + kProducers) * 64;
-constexpr int kWaveM = TM / (kConsumers / 2);       // x rows per consumer wavefront
-constexpr int kIT = kWaveM / 32;                    // 32-row x fragments per consumer wavefront
 constexpr int kStages = 3;
 constexpr int kRowB = TK * 2;                       // 128 bytes per LDS row
-constexpr int kXStage = TM * kRowB;                 // 32 KB
 constexpr int kWStage = TN * kRowB;                 // 16 KB
 
 struct TileParams {
@@ -74,6 +71,15 @@ struct TileParams {
   // whatever the split count).
   int ksplit, steps_per_split;
   float* plane;
+  // Grouped (expert-sorted) form, rows in blocks of the tile height that each belong to one expert
+  // (gpu-kernels/metal/quant/affine_qmm_steel.metal:1022-1040): tile2e[block] is the expert whose
+  // slab of the batched pack [E, N, ...] the block multiplies (< 0: nothing to do); with srow, x row
+  // of slot i is x[srow[i]] (< 0: a padding slot, whose output is zero); with sdst, the output row of
+  // slot i goes to y[sdst[i]] (< 0: not written).
+  const int* tile2e = nullptr;
+  const int* srow = nullptr;
+  const int* sdst = nullptr;
+  int n_experts = 0, rows_x = 0, rows_y = 0;
 };
 
 __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
@@ -140,9 +146,15 @@ __device__ __forceinline__ void wait_codes(CodeRegs& r)
 
 }  // namespace
 
-template <bool LORA>
+// TMK: rows of x per workgroup (256; 128 for the grouped form, whose blocks of rows are that tall).
+template <bool LORA, int TMK = TM, bool GROUPED = false>
 __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
 {
+  static_assert(TMK == 256 || (TMK == 128 && !LORA), "tile heights built");
+  constexpr int kWaveM = TMK / (kConsumers / 2);   // x rows per consumer wavefront
+  constexpr int kIT = kWaveM / 32;                 // 32-row x fragments per consumer wavefront
+  constexpr int kXStage = TMK * kRowB;             // 32 KB at 256 rows
+  constexpr int kXL = TMK / 32;                    // x-tile loads per producer wavefront and step
   __shared__ __attribute__((aligned(16))) uint8_t x_lds[kStages * kXStage];   // 96 KB
   __shared__ __attribute__((aligned(16))) uint8_t w_lds[kStages * kWStage];   // 48 KB
 
@@ -157,7 +169,17 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   const int tile = (int)blockIdx.x - ks * tiles;
   const int tm = tile % p.tiles_m;
   const int tn = tile / p.tiles_m;
-  const int m0 = tm * TM, n0 = tn * TN;
+  const int m0 = tm * TMK, n0 = tn * TN;
+  const uint32_t* pw_base = p.w;
+  const uint16_t* ps_base = p.scales;
+  const uint16_t* pb_base = p.biases;
+  if constexpr (GROUPED) {
+    const int e = p.tile2e[tm];
+    if (e < 0 || e >= p.n_experts) { return; }        // the whole workgroup, before any barrier
+    pw_base += (size_t)e * (size_t)p.N * (size_t)(p.K >> 3);
+    ps_base += (size_t)e * (size_t)p.N * (size_t)(p.K >> 6);
+    pb_base += (size_t)e * (size_t)p.N * (size_t)(p.K >> 6);
+  }
   // This workgroup's K steps: all of them, or its share of a split.
   const int k_first = ks * p.steps_per_split;
   const int KT = p.ksplit > 1 ? ((p.K / TK - k_first) < p.steps_per_split ? (p.K / TK - k_first) : p.steps_per_split)
@@ -169,31 +191,38 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     const int pt = tid - kConsumers * 64; // 0..255
     // x tile: 32 direct-to-LDS loads per step, 8 per wavefront.  Load i of wave pw covers tile
     // rows (8 pw + i)*8 .. +8; lane l takes row l/8, LDS position l%8.
-    const uint8_t* xblk = reinterpret_cast<const uint8_t*>(p.x) + (size_t)m0 * p.K * 2 + (size_t)k_first * (TK * 2);
-    uint32_t a_off[8];
+    const bool gathered = GROUPED && p.srow != nullptr;
+    const uint8_t* xblk = reinterpret_cast<const uint8_t*>(p.x) + (gathered ? (size_t)0 : (size_t)m0 * p.K * 2) +
+                          (size_t)k_first * (TK * 2);
+    uint32_t a_off[kXL];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = (pw * 8 + i) * 8 + (lane >> 3);
+    for (int i = 0; i < kXL; ++i) {
+      const int row = (pw * kXL + i) * 8 + (lane >> 3);
       const int chunk = swz(row, lane & 7);
-      const int rg = (m0 + row < p.M) ? row : (p.M - 1 - m0);
+      int rg = (m0 + row < p.M) ? row : (p.M - 1 - m0);
+      if (gathered) {
+        // A padding slot reads row 0 (any readable row): its output is written as zero.
+        const int src = p.srow[m0 + rg];
+        rg = (src >= 0 && src < p.rows_x) ? src : 0;
+      }
       a_off[i] = (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u;
     }
     // W tile: thread pt dequantizes 32 codes of row pt/2 (k half pt%2) per step.
     const int qrow = pt >> 1, qhalf = pt & 1;
     const int qrg = (n0 + qrow < p.N) ? (n0 + qrow) : (p.N - 1);
-    const uint8_t* wrow = reinterpret_cast<const uint8_t*>(p.w) + (size_t)qrg * (p.K >> 1) + qhalf * 16 +
+    const uint8_t* wrow = reinterpret_cast<const uint8_t*>(pw_base) + (size_t)qrg * (p.K >> 1) + qhalf * 16 +
                           (size_t)k_first * (TK / 2);
-    const uint16_t* srow = p.scales + (size_t)qrg * (p.K >> 6) + k_first;
-    const uint16_t* brow = p.biases + (size_t)qrg * (p.K >> 6) + k_first;
+    const uint16_t* srow = ps_base + (size_t)qrg * (p.K >> 6) + k_first;
+    const uint16_t* brow = pb_base + (size_t)qrg * (p.K >> 6) + k_first;
     int b_dst[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) { b_dst[i] = qrow * kRowB + swz(qrow, qhalf * 4 + i) * 16; }
 
     auto issue_x = [&](int step, int stage) {
       const uint8_t* src = xblk + (size_t)step * (TK * 2);
-      uint8_t* dst = x_lds + stage * kXStage + pw * (64 * kRowB);
+      uint8_t* dst = x_lds + stage * kXStage + pw * (kXL * 8 * kRowB);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kXL; ++i) {
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + a_off[i]),
                                          (__attribute__((address_space(3))) void*)(dst + i * (8 * kRowB)), 16, 0, 0);
       }
@@ -223,23 +252,24 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");   // all but the 6 code requests
     wg_barrier();
 
-    // Steady state, step s fills the stage of step t = s+2.  Requests in issue order:
-    //   ..., x(t-1) [8], codes(t+1) [3], x(t) [8], codes(t+2) [3]
+    // Steady state, step s fills the stage of step t = s+2.  Requests in issue order, with X = kXL
+    // (8 at 256 rows):
+    //   ..., x(t-1) [X], codes(t+1) [3], x(t) [X], codes(t+2) [3]
     // x(t) goes out first so that it has two whole steps to land.  codes(t) were requested two
-    // steps ago: 8 + 3 + 8 = 19 younger requests may stay in flight while they are awaited.
-    // Before the barrier x(t-1), the tile of step s+1, must have landed: 14 younger requests.
-    // The first fill follows the prologue, where only codes(3) [3] and x(2) [8] are younger.
+    // steps ago: X + 3 + X younger requests may stay in flight while they are awaited (19).
+    // Before the barrier x(t-1), the tile of step s+1, must have landed: 3 + X + 3 younger requests (14).
+    // The first fill follows the prologue, where only codes(3) [3] and x(2) [X] are younger (11).
     auto fill = [&](auto younger, int t, int stage, CodeRegs& r) {
       issue_x(t, stage);
       wait_codes<decltype(younger)::value>(r);
       dequant_to(stage, r);
       request(r, t + 2 < KT ? t + 2 : t);           // the last two requests are never used
-      asm volatile("s_waitcnt vmcnt(14) lgkmcnt(0)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kXL + 6) : "memory");
     };
     auto next_stage = [](int stage) { return stage == kStages - 1 ? 0 : stage + 1; };
     auto odd_fill = [&](int t, int stage) {
       if (t < KT) {
-        fill(std::integral_constant<int, 19>(), t, stage, rb);
+        fill(std::integral_constant<int, 2 * kXL + 3>(), t, stage, rb);
       } else {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       }
@@ -247,7 +277,7 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     int tstage = 2;                        // stage of step s+2
     int s = 0;
     if (KT > 2) {
-      fill(std::integral_constant<int, 11>(), 2, tstage, ra);
+      fill(std::integral_constant<int, kXL + 3>(), 2, tstage, ra);
       wg_barrier();
       tstage = next_stage(tstage);
       odd_fill(3, tstage);
@@ -256,7 +286,7 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
       s = 2;
     }
     for (; s + 2 < KT; s += 2) {
-      fill(std::integral_constant<int, 19>(), s + 2, tstage, ra);   // even step: codes in ra
+      fill(std::integral_constant<int, 2 * kXL + 3>(), s + 2, tstage, ra);   // even step: codes in ra
       wg_barrier();
       tstage = next_stage(tstage);
       odd_fill(s + 3, tstage);
@@ -404,14 +434,21 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
       const int m = m0 + wm * kWaveM + it * 32 + frow;
       if (m >= p.M) { continue; }
       uint16_t* yrow = p.y + (size_t)m * p.out_stride + p.out_off;
+      bool pad_slot = false;                 // a padding slot of the grouped form: x = 0, so act(0) * 0 = +0
+      if constexpr (GROUPED) {
+        if (p.srow != nullptr) {
+          const int src = p.srow[m];
+          pad_slot = src < 0 || src >= p.rows_x;
+        }
+      }
 #pragma unroll
       for (int jt = 0; jt < 2; ++jt) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           const int n = n0 + wn * 64 + jt * 32 + rq * 8 + fkh * 4;
           if (n >= p.N) { continue; }
-          const float f0 = gated_f32(p.gate_act, acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
-          const float f1 = gated_f32(p.gate_act, acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
+          const float f0 = pad_slot ? 0.0f : gated_f32(p.gate_act, acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
+          const float f1 = pad_slot ? 0.0f : gated_f32(p.gate_act, acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
           if (pair_ok && n + 3 < p.N) {
             *reinterpret_cast<uint32_t*>(yrow + (n >> 1)) = pack_bf16x2(f0, f1);
           } else {
@@ -428,7 +465,14 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   for (int it = 0; it < kIT; ++it) {
     const int m = m0 + wm * kWaveM + it * 32 + frow;
     if (m >= p.M) { continue; }
-    uint16_t* yrow = p.y + (size_t)m * p.N;
+    int mdst = m;
+    if constexpr (GROUPED) {
+      if (p.sdst != nullptr) {
+        mdst = p.sdst[m];
+        if (mdst < 0 || mdst >= p.rows_y) { continue; }
+      }
+    }
+    uint16_t* yrow = p.y + (size_t)mdst * p.N;
 #pragma unroll
     for (int jt = 0; jt < 2; ++jt) {
 #pragma unroll
@@ -535,6 +579,24 @@ hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a)
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
   return a.lora_t != nullptr ? launch_kernel(qmm_tile_kernel<true>, grid, block, 0, st, p)
                              : launch_kernel(qmm_tile_kernel<false>, grid, block, 0, st, p);
+}
+
+hipError_t launch_qmm_grouped(hipStream_t st, const GemmArgs& a, const GroupedArgs& g)
+{
+  TileParams p;
+  p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
+  p.lora_t = nullptr; p.lora_b = nullptr;
+  p.K = a.K; p.N = a.N; p.M = a.M; p.r = 0;
+  p.gate_act = a.gate_act;
+  p.out_stride = a.out_stride > 0 ? a.out_stride : a.N / 2;
+  p.out_off = a.out_off;
+  p.tiles_m = a.M / kGroupedBlockRows;       // a.M is a whole number of blocks
+  p.tiles_n = (a.N + TN - 1) / TN;
+  p.ksplit = 1; p.steps_per_split = a.K / TK; p.plane = nullptr;
+  p.tile2e = g.tile2e; p.srow = g.srow; p.sdst = g.sdst;
+  p.n_experts = g.n_experts; p.rows_x = g.rows_x; p.rows_y = g.rows_y;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
+  return launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, true>, grid, block, 0, st, p);
 }
 
 }  // namespace vpq
