@@ -553,6 +553,38 @@ def main():
         out["moe_gather_decode_top8_of_128"] = {
             "gate|up+swiglu 2048->2x768": {"us": round(us_gu, 2), "GBps": round(b_gu / (us_gu * 1e-6) / 1e9, 1)},
             "down 768->2048": {"us": round(us_dn, 2), "GBps": round(b_dn / (us_dn * 1e-6) / 1e9, 1)}}
+
+        # MoE prefill block of the same model, 2048 tokens (16384 pairs): the pair sort, then the two
+        # expert-sorted GEMMs; beside them the pair-batched gathers (one QMV per pair) on the same pairs.
+        # TFLOPs count the pairs' flops only, not the padding slots'.
+        T = 2048
+        eid = torch.randint(0, E, (T * top_k,), dtype=torch.int32, device=dev, generator=gen)
+        xt = torch.randn((T, H), device=dev, generator=gen).bfloat16()
+        gw, gs, gb, dw, ds, db = batches[0]
+        sorted_ = {}
+
+        def call_sort(i):
+            sorted_["v"] = vpipe_amd.moe_sort_pairs(eid, top_k, E)
+        us_sort = kernel_us(call_sort, 8)
+        t2e, srow, sdst, ntiles = sorted_["v"]
+        npad = srow.numel()
+        gact = torch.empty((npad, I), dtype=torch.bfloat16, device=dev)
+        partp = torch.empty((T * top_k, H), dtype=torch.bfloat16, device=dev)
+        us_ggu = kernel_us(lambda i: vpipe_amd.qmm_grouped_gated_w4g64(gw, gs, gb, xt, H, 2 * I, t2e, srow, E, out=gact), 8)
+        us_gdn = kernel_us(lambda i: vpipe_amd.qmm_grouped_down_w4g64(dw, ds, db, gact, I, H, t2e, sdst, E, out=partp), 8)
+        actp = torch.empty((T * top_k, I), dtype=torch.bfloat16, device=dev)
+        us_pgu = kernel_us(lambda i: vpipe_amd.gather_qmv_gated_w4g64(gw, gs, gb, xt, H, 2 * I, eid, top_k, E, out=actp), 4)
+        us_pdn = kernel_us(lambda i: vpipe_amd.gather_down_qmv_w4g64(dw, ds, db, actp, I, H, eid, E, out=partp), 4)
+        f_gu = 2.0 * T * top_k * 2 * I * H
+        f_dn = 2.0 * T * top_k * H * I
+        out["moe_grouped_prefill_t2048_top8_of_128"] = {
+            "blocks_in_use": int(ntiles.cpu()[0]), "slots": int(ntiles.cpu()[0]) * vpipe_amd.grouped_block_rows(),
+            "pairs": T * top_k,
+            "pair_sort_us": round(us_sort, 2),
+            "gate|up+swiglu 2048->2x768": {"us": round(us_ggu, 2), "TFLOPs": round(f_gu / (us_ggu * 1e-6) / 1e12, 1),
+                                           "pair_gather_qmv_us": round(us_pgu, 2)},
+            "down 768->2048": {"us": round(us_gdn, 2), "TFLOPs": round(f_dn / (us_gdn * 1e-6) / 1e12, 1),
+                               "pair_gather_qmv_us": round(us_pdn, 2)}}
         del batches
 
     # ---- CPU baseline: the oracle's dequant + fp32 matmul on the host cores ------------

@@ -409,6 +409,56 @@ def test_embedding_gather_call_site(enc, oracle, dev, D):
 
 
 
+def test_moe_grouped_expert_call_sites(vpq, enc, oracle, dev, D):
+    # Qwen MoE block at prefill, expert-sorted (generative-models/qwen3/metal-qwen-model.cc:4239-4264):
+    # gate|up + SwiGLU over the gathered hidden rows -> gact[npad, I] (slots 0..4, 5:H 6:2*I 7:npad
+    # 8:tile2e 9:srow), then down -> part[np, H] scattered to pair order (5:I 6:H 7:npad 8:tile2e 9:sdst)
+    H, I, E, top_k, T = 512, 128, 5, 2, 70
+    gu = [synth.make_weight(2 * I, H, 1900 + e) for e in range(E)]
+    dn = [synth.make_weight(H, I, 1950 + e) for e in range(E)]
+    guw, gus, gub = (np.stack([p[i] for p in gu]) for i in range(3))
+    dw, ds, db = (np.stack([p[i] for p in dn]) for i in range(3))
+    x = synth.make_act(T, H, 1990)
+    eid = np.random.default_rng(1991).integers(0, E, size=T * top_k, dtype=np.int32)
+    npair = eid.size
+    B = vpq.grouped_block_rows()
+    t2e_d, srow_d, sdst_d, _ = vpq.moe_sort_pairs(torch.from_numpy(eid).to(dev), top_k, E)
+    torch.cuda.synchronize()
+    t2e, srow, sdst = (o.cpu().numpy() for o in (t2e_d, srow_d, sdst_d))
+    npad = srow.size
+    gact = torch.zeros((npad, I), dtype=torch.bfloat16, device=dev)
+    part = torch.zeros((npair, H), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_qmm_steel_bf16", "affine_qmm_grouped_swiglu_w4g64") == 1
+    for i, t in enumerate((D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev), gact)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, H)
+    enc.set_constant(6, 2 * I)
+    enc.set_constant(7, npad)
+    enc.set_buffer(8, t2e_d)
+    enc.set_buffer(9, srow_d)
+    enc.dispatch((((2 * I + 31) // 32) * 32, ((npad + 31) // 32) * 2, 2), (32, 2, 2))
+    assert enc.set_function("affine_qmm_steel_bf16", "affine_qmm_grouped_w4g64") == 1
+    for i, t in enumerate((D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), gact, part)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, I)
+    enc.set_constant(6, H)
+    enc.set_constant(7, npad)
+    enc.set_buffer(8, t2e_d)
+    enc.set_buffer(9, sdst_d)
+    enc.dispatch((((H + 31) // 32) * 32, ((npad + 31) // 32) * 2, 2), (32, 2, 2))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    gact_bits = D.bits(gact)
+    y64, _ = oracle.qmm_grouped(guw, gus, gub, x, H, 2 * I, B, t2e, srow=srow)
+    a64, ab = oracle.swiglu(y64)
+    live = srow >= 0
+    parity.check_bf16(gact_bits[live], a64[live], ab[live])
+    assert not gact_bits[~live].any()
+    # the down projection reads the activation the device produced
+    d64, dbits = oracle.qmm_grouped(dw, ds, db, gact_bits, I, H, B, t2e, sdst=sdst, rows_y=npair)
+    parity.check_bf16(D.bits(part), d64, dbits)
+
+
 def test_moe_gathered_expert_call_sites(enc, oracle, dev, D):
     # Qwen MoE block, pair-batched (generative-models/qwen3/metal-qwen-model.cc:4190-4206):
     # gathered gate|up + SwiGLU -> act[np, I] (slots 0..4, 5:H 6:2*I 7:eid 8:top_k, grid {32, I/2, np}),

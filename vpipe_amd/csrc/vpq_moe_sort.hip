@@ -37,12 +37,32 @@ __global__ __launch_bounds__(256) void moe_sort_fill_kernel(int* tile2e, int max
   }
 }
 
+// Pairs per workgroup of the histogram and scatter kernels, and the expert count up to which a workgroup
+// counts in LDS first (one global atomic per expert and workgroup instead of one per pair).
+constexpr int kSortChunk = 1024;
+constexpr int kSortLdsExperts = 4096;
+
 __global__ __launch_bounds__(256) void moe_sort_hist_kernel(const int* __restrict__ eid, int n_pairs, int n_experts, int* hist)
 {
-  const int p = (int)blockIdx.x * 256 + (int)threadIdx.x;
-  if (p >= n_pairs) { return; }
-  const int e = eid[p];
-  if (e >= 0 && e < n_experts) { atomicAdd(hist + e, 1); }
+  __shared__ int local[kSortLdsExperts];
+  const int p0 = (int)blockIdx.x * kSortChunk;
+  const bool in_lds = n_experts <= kSortLdsExperts;
+  if (in_lds) {
+    for (int e = (int)threadIdx.x; e < n_experts; e += 256) { local[e] = 0; }
+    __syncthreads();
+  }
+  for (int i = (int)threadIdx.x; i < kSortChunk; i += 256) {
+    const int p = p0 + i;
+    if (p >= n_pairs) { break; }
+    const int e = eid[p];
+    if (e >= 0 && e < n_experts) { atomicAdd(in_lds ? local + e : hist + e, 1); }
+  }
+  if (in_lds) {
+    __syncthreads();
+    for (int e = (int)threadIdx.x; e < n_experts; e += 256) {
+      if (local[e] != 0) { atomicAdd(hist + e, local[e]); }
+    }
+  }
 }
 
 // One wavefront: lane l owns the experts [l * per, (l + 1) * per).
@@ -82,14 +102,38 @@ __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int* __rest
                                                                int* cursor, int* srow, int* sdst, int n_pairs, int top_k,
                                                                int n_experts, int npad)
 {
-  const int p = (int)blockIdx.x * 256 + (int)threadIdx.x;
-  if (p >= n_pairs) { return; }
-  const int e = eid[p];
-  if (e < 0 || e >= n_experts) { return; }
-  const int slot = boff[e] + atomicAdd(cursor + e, 1);
-  if (slot < npad) {
-    srow[slot] = p / top_k;
-    sdst[slot] = p;
+  __shared__ int local[kSortLdsExperts];     // pairs of this workgroup per expert, then their first ticket
+  const int p0 = (int)blockIdx.x * kSortChunk;
+  const bool in_lds = n_experts <= kSortLdsExperts;
+  int rank[kSortChunk / 256];
+  if (in_lds) {
+    for (int e = (int)threadIdx.x; e < n_experts; e += 256) { local[e] = 0; }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kSortChunk / 256; ++j) {
+      const int p = p0 + j * 256 + (int)threadIdx.x;
+      const int e = p < n_pairs ? eid[p] : -1;
+      rank[j] = (e >= 0 && e < n_experts) ? atomicAdd(local + e, 1) : 0;
+    }
+    __syncthreads();
+    for (int e = (int)threadIdx.x; e < n_experts; e += 256) {
+      const int c = local[e];
+      if (c != 0) { local[e] = atomicAdd(cursor + e, c); }     // a run of c tickets
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < kSortChunk / 256; ++j) {
+    const int p = p0 + j * 256 + (int)threadIdx.x;
+    if (p >= n_pairs) { continue; }
+    const int e = eid[p];
+    if (e < 0 || e >= n_experts) { continue; }
+    const int ticket = in_lds ? local[e] + rank[j] : atomicAdd(cursor + e, 1);
+    const int slot = boff[e] + ticket;
+    if (slot < npad) {
+      srow[slot] = p / top_k;
+      sdst[slot] = p;
+    }
   }
 }
 
@@ -108,7 +152,7 @@ hipError_t launch_moe_sort(hipStream_t st, const int* pair_eid, int n_pairs, int
   hipError_t e = launch_kernel(moe_sort_fill_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, st, tile2e, max_tiles, srow,
                                sdst, npad, hist, n_experts);
   if (e != hipSuccess) { return e; }
-  const dim3 pgrid((unsigned)((n_pairs + 255) / 256));
+  const dim3 pgrid((unsigned)((n_pairs + kSortChunk - 1) / kSortChunk));
   e = launch_kernel(moe_sort_hist_kernel, pgrid, dim3(256), 0, st, pair_eid, n_pairs, n_experts, hist);
   if (e != hipSuccess) { return e; }
   e = launch_kernel(moe_sort_setup_kernel, dim3(1), dim3(64), 0, st, (const int*)hist, boff, cursor, tile2e, ntiles,

@@ -97,6 +97,9 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w4g64", QuantKernel::GatherSwiglu},
     {"affine_qmv_bf16", "affine_gather_qmv_geglu_w4g64", QuantKernel::GatherGeglu},
     {"affine_qmv_bf16", "affine_gather_down_qmv_w4g64", QuantKernel::GatherDown},
+    {"affine_qmm_steel_bf16", "affine_qmm_grouped_swiglu_w4g64", QuantKernel::GroupedSwiglu},
+    {"affine_qmm_steel_bf16", "affine_qmm_grouped_geglu_w4g64", QuantKernel::GroupedGeglu},
+    {"affine_qmm_steel_bf16", "affine_qmm_grouped_w4g64", QuantKernel::GroupedDown},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm128", QuantKernel::QmmSwiglu},
@@ -503,6 +506,33 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
           } else {
             status = vpq_gather_qmv_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, eid, npair, ival(8), E,
                                                      kind == QuantKernel::GatherGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
+          }
+        }
+      } else if (kind == QuantKernel::GroupedSwiglu || kind == QuantKernel::GroupedGeglu ||
+                 kind == QuantKernel::GroupedDown) {
+        // gpu-kernels/metal/quant/affine_qmm_steel.metal:1042-1066, 1266-1339: slot 7 = npad (sorted slots,
+        // whole blocks of vpq_qmm_grouped_block_rows()), 8 = tile2e, 9 = srow (gate|up) or sdst (down)
+        // (generative-models/qwen3/metal-qwen-model.cc:4239-4264).  Expert count and the row counts the
+        // index buffers may name are what the bound buffers hold.
+        const bool down = kind == QuantKernel::GroupedDown;
+        if (!has_int(7) || !buf(8) || !buf(9)) {
+          status = VPQ_ERR_NULL_POINTER;
+        } else if (K <= 0 || N <= 0 || K % 64 != 0) {
+          status = VPQ_ERR_BAD_SHAPE;
+        } else {
+          const std::size_t slab = static_cast<std::size_t>(N) * static_cast<std::size_t>(K / 2);
+          const std::size_t experts = _slots[0].bytes / slab;
+          const int E = experts > 0x7fffffffu ? 0x7fffffff : static_cast<int>(experts);
+          const std::size_t rows = down ? _slots[4].bytes / (static_cast<std::size_t>(N) * 2)
+                                        : _slots[3].bytes / (static_cast<std::size_t>(K) * 2);
+          const int nrows = rows > 0x7fffffffu ? 0x7fffffff : static_cast<int>(rows);
+          const int32_t* t2e = static_cast<const int32_t*>(buf(8));
+          const int32_t* idx = static_cast<const int32_t*>(buf(9));
+          if (down) {
+            status = vpq_qmm_grouped_down_w4g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), t2e, idx, E, nrows);
+          } else {
+            status = vpq_qmm_grouped_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), t2e, idx, E, nrows,
+                                                      kind == QuantKernel::GroupedGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
           }
         }
       } else if (kind == QuantKernel::Qmm) {

@@ -85,6 +85,10 @@ enum class QuantKernel : std::uint8_t {
                   //   8 = top_k; pairs = grid.z; the expert count is what the bound code buffer holds
   GatherGeglu,    // affine_gather_qmv_geglu_w4g64: as GatherSwiglu
   GatherDown,     // affine_gather_down_qmv_w4g64: x [npair, K], slot 7 = pair_eid buffer; pairs = grid.z
+  GroupedSwiglu,  // affine_qmm_grouped_swiglu_w4g64: expert batch, x = hidden rows gathered through slot 9 = srow,
+                  //   slot 7 = npad, 8 = tile2e; y [npad, N/2] in slot order
+  GroupedGeglu,   // affine_qmm_grouped_geglu_w4g64: as GroupedSwiglu
+  GroupedDown,    // affine_qmm_grouped_w4g64: x [npad, K] in slot order, slot 9 = sdst, y rows in pair order
   Argmax,         // argmax_f16: slots 0:logits 1:out_id 2:V (one workgroup)
   ArgmaxPartial,  // argmax_partial_f16: slots 0:logits 1:partials 2:V 3:M slabs
   ArgmaxCombine,  // argmax_combine_f16: slots 0:partials 1:out_id 2:M
