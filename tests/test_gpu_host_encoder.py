@@ -423,13 +423,15 @@ def test_moe_grouped_expert_call_sites(vpq, enc, oracle, dev, D):
     npair = eid.size
     B = vpq.grouped_block_rows()
     t2e_d, srow_d, sdst_d, _ = vpq.moe_sort_pairs(torch.from_numpy(eid).to(dev), top_k, E)
-    torch.cuda.synchronize()
     t2e, srow, sdst = (o.cpu().numpy() for o in (t2e_d, srow_d, sdst_d))
     npad = srow.size
     gact = torch.zeros((npad, I), dtype=torch.bfloat16, device=dev)
     part = torch.zeros((npair, H), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()               # the encoder's stream is not ordered after torch's fills
     assert enc.set_function("affine_qmm_steel_bf16", "affine_qmm_grouped_swiglu_w4g64") == 1
-    for i, t in enumerate((D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev), gact)):
+    # staged tensors stay alive until the stream has run: a freed one may be handed to the next upload
+    gu_d = (D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev), gact)
+    for i, t in enumerate(gu_d):
         enc.set_buffer(i, t)
     enc.set_constant(5, H)
     enc.set_constant(6, 2 * I)
@@ -438,7 +440,8 @@ def test_moe_grouped_expert_call_sites(vpq, enc, oracle, dev, D):
     enc.set_buffer(9, srow_d)
     enc.dispatch((((2 * I + 31) // 32) * 32, ((npad + 31) // 32) * 2, 2), (32, 2, 2))
     assert enc.set_function("affine_qmm_steel_bf16", "affine_qmm_grouped_w4g64") == 1
-    for i, t in enumerate((D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), gact, part)):
+    dn_d = (D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), gact, part)
+    for i, t in enumerate(dn_d):
         enc.set_buffer(i, t)
     enc.set_constant(5, I)
     enc.set_constant(6, H)
@@ -475,7 +478,8 @@ def test_moe_gathered_expert_call_sites(enc, oracle, dev, D):
     act = torch.zeros((npair, I), dtype=torch.bfloat16, device=dev)
     part = torch.zeros((npair, H), dtype=torch.bfloat16, device=dev)
     assert enc.set_function("affine_qmv_bf16", "affine_gather_qmv_swiglu_w4g64") == 1
-    for i, t in enumerate((D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev), act)):
+    gu_d = (D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev), act)   # kept alive until the stream has run
+    for i, t in enumerate(gu_d):
         enc.set_buffer(i, t)
     enc.set_constant(5, H)
     enc.set_constant(6, 2 * I)
@@ -483,7 +487,8 @@ def test_moe_gathered_expert_call_sites(enc, oracle, dev, D):
     enc.set_constant(8, top_k)
     enc.dispatch((32, I // 2, npair), (32, 2, 1))
     assert enc.set_function("affine_qmv_bf16", "affine_gather_down_qmv_w4g64") == 1
-    for i, t in enumerate((D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), act, part)):
+    dn_d = (D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), act, part)
+    for i, t in enumerate(dn_d):
         enc.set_buffer(i, t)
     enc.set_constant(5, I)
     enc.set_constant(6, H)

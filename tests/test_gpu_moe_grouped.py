@@ -77,7 +77,7 @@ def test_pair_sort_skips_ids_out_of_range_and_rejects_bad_arguments(vpq, oracle,
 
 # K (hidden), inner, H (down out), E, T, top_k: the Qwen3-MoE block scaled down; K of the down GEMM = inner
 GROUPED_SHAPES = [(512, 128, 512, 6, 150, 2, False), (2048, 768, 2048, 16, 200, 4, True), (576, 96, 200, 3, 40, 1, False),
-                  (1024, 160, 1026, 9, 300, 3, True)]
+                  (1024, 160, 1026, 9, 300, 3, True), (512, 64, 100, 4, 90, 2, False)]      # last: one 128-wide tile of N
 
 
 @pytest.mark.parametrize("activation", [capi.VPQ_GATE_SWIGLU, capi.VPQ_GATE_GEGLU])
@@ -149,3 +149,39 @@ def test_grouped_gemms_reject_bad_arguments(vpq, dev):
     assert L.vpq_qmm_grouped_down_w4g64_bf16(None, p, p, p, p, p, 60, 8, 128, p, p, 1, 1) == -2           # K % 64
     assert L.vpq_qmm_grouped_down_w4g64_bf16(None, p, p, p, p, p, 64, 8, 128, p, p, 0, 1) == -2           # no expert
     assert L.vpq_qmm_grouped_down_w4g64_bf16(None, p, p, p, p, p, 64, 8, 128, None, p, 1, 1) == -1
+
+
+def test_grouped_gemms_take_the_slots_of_a_block_in_any_order(vpq, oracle, dev, D):
+    # padding slots need not trail: a permutation of the slots inside every block permutes the gate|up
+    # rows and leaves the down rows (pair order) as they were, bit for bit
+    K, inner, H, E, T, top_k = 512, 128, 300, 4, 50, 2
+    B = vpq.grouped_block_rows()
+    guw, gus, gub = expert_batch(E, 2 * inner, K, 5600)
+    dw, ds, db = expert_batch(E, H, inner, 5601)
+    x = synth.make_act(T, K, 5602)
+    eid = routed(E, T, top_k, 5603)
+    t2e, srow, sdst, _ = oracle.moe_sort_pairs(eid, top_k, E, B, vpq.moe_max_tiles(eid.size, E, B))
+    npad = srow.size
+    rng = np.random.default_rng(5604)
+    perm = np.concatenate([t * B + rng.permutation(B) for t in range(npad // B)])
+    xs = synth.make_act(npad, inner, 5605)
+    guwd, gusd, gubd, xd = D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev)
+    dwd, dsd, dbd = D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev)
+    t2e_d = torch.from_numpy(t2e).to(dev)
+
+    def run(srow_, sdst_, xs_):
+        act = vpq.qmm_grouped_gated_w4g64(guwd, gusd, gubd, xd, K, 2 * inner, t2e_d, torch.from_numpy(srow_).to(dev), E)
+        part = torch.zeros((eid.size, H), dtype=torch.bfloat16, device=dev)
+        vpq.qmm_grouped_down_w4g64(dwd, dsd, dbd, D.bf16(xs_, dev), inner, H, t2e_d, torch.from_numpy(sdst_).to(dev), E,
+                                   out=part)
+        return D.bits(act), D.bits(part)
+    act0, part0 = run(srow, sdst, xs)
+    act1, part1 = run(np.ascontiguousarray(srow[perm]), np.ascontiguousarray(sdst[perm]), np.ascontiguousarray(xs[perm]))
+    used = t2e >= 0
+    rows_used = np.repeat(used, B)
+    assert np.array_equal(act1[rows_used], act0[perm][rows_used])
+    assert np.array_equal(part1, part0)
+    y64, _ = oracle.qmm_grouped(guw, gus, gub, x, K, 2 * inner, B, t2e, srow=srow)
+    a64, ab = oracle.swiglu(y64)
+    live = srow >= 0
+    parity.check_bf16(act0[live], a64[live], ab[live])

@@ -49,7 +49,6 @@ constexpr int kProducers = 4;
 constexpr int kThreads = (kConsumers + kProducers) * 64;
 constexpr int kStages = 3;
 constexpr int kRowB = TK * 2;                       // 128 bytes per LDS row
-constexpr int kWStage = TN * kRowB;                 // 16 KB
 
 struct TileParams {
   const uint32_t* w;
@@ -144,13 +143,32 @@ __device__ __forceinline__ void wait_codes(CodeRegs& r)
   asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r.codes), "+v"(r.s_bits), "+v"(r.b_bits) : "n"(YOUNGER) : "memory");
 }
 
+// The same for the one or two register sets of a step (requests retire in order: YOUNGER counts
+// from the last of them).
+template <int YOUNGER>
+__device__ __forceinline__ void wait_codes(CodeRegs (&r)[1]) { wait_codes<YOUNGER>(r[0]); }
+
+template <int YOUNGER>
+__device__ __forceinline__ void wait_codes(CodeRegs (&r)[2])
+{
+  asm volatile("s_waitcnt vmcnt(%6)"
+               : "+v"(r[0].codes), "+v"(r[0].s_bits), "+v"(r[0].b_bits), "+v"(r[1].codes), "+v"(r[1].s_bits), "+v"(r[1].b_bits)
+               : "n"(YOUNGER)
+               : "memory");
+}
+
 }  // namespace
 
-// TMK: rows of x per workgroup (256; 128 for the grouped form, whose blocks of rows are that tall).
-template <bool LORA, int TMK = TM, bool GROUPED = false>
+// TMK x TNK: rows of x and weight rows per workgroup: 256 x 128, or 128 x {128, 256} for the grouped
+// form, whose blocks of rows are 128 tall (the wider tile gives a K step as much work as 256 x 128).
+template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false>
 __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
 {
-  static_assert(TMK == 256 || (TMK == 128 && !LORA), "tile heights built");
+  static_assert((TMK == 256 && TNK == 128) || (TMK == 128 && !LORA && (TNK == 128 || TNK == 256)), "tiles built");
+  constexpr int kWStage = TNK * kRowB;             // 16 KB at 128 weight rows
+  constexpr int kWH = TNK / 128;                   // weight rows (code requests) per producer thread and step
+  constexpr int kJT = TNK / 64;                    // 32-row W fragments per consumer wavefront
+  constexpr int kCR = 3 * kWH;                     // code, scale and bias requests per producer thread and step
   constexpr int kWaveM = TMK / (kConsumers / 2);   // x rows per consumer wavefront
   constexpr int kIT = kWaveM / 32;                 // 32-row x fragments per consumer wavefront
   constexpr int kXStage = TMK * kRowB;             // 32 KB at 256 rows
@@ -169,7 +187,7 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   const int tile = (int)blockIdx.x - ks * tiles;
   const int tm = tile % p.tiles_m;
   const int tn = tile / p.tiles_m;
-  const int m0 = tm * TMK, n0 = tn * TN;
+  const int m0 = tm * TMK, n0 = tn * TNK;
   const uint32_t* pw_base = p.w;
   const uint16_t* ps_base = p.scales;
   const uint16_t* pb_base = p.biases;
@@ -207,14 +225,21 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
       }
       a_off[i] = (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u;
     }
-    // W tile: thread pt dequantizes 32 codes of row pt/2 (k half pt%2) per step.
+    // W tile: thread pt dequantizes 32 codes of row pt/2 (k half pt%2) per step, and of row pt/2 + 128
+    // in a 256-row tile.
     const int qrow = pt >> 1, qhalf = pt & 1;
-    const int qrg = (n0 + qrow < p.N) ? (n0 + qrow) : (p.N - 1);
-    const uint8_t* wrow = reinterpret_cast<const uint8_t*>(pw_base) + (size_t)qrg * (p.K >> 1) + qhalf * 16 +
-                          (size_t)k_first * (TK / 2);
-    const uint16_t* srow = ps_base + (size_t)qrg * (p.K >> 6) + k_first;
-    const uint16_t* brow = pb_base + (size_t)qrg * (p.K >> 6) + k_first;
-    int b_dst[4];
+    const uint8_t* wrow[kWH];
+    const uint16_t* srow[kWH];
+    const uint16_t* brow[kWH];
+#pragma unroll
+    for (int h = 0; h < kWH; ++h) {
+      const int qrg = (n0 + qrow + 128 * h < p.N) ? (n0 + qrow + 128 * h) : (p.N - 1);
+      wrow[h] = reinterpret_cast<const uint8_t*>(pw_base) + (size_t)qrg * (p.K >> 1) + qhalf * 16 +
+                (size_t)k_first * (TK / 2);
+      srow[h] = ps_base + (size_t)qrg * (p.K >> 6) + k_first;
+      brow[h] = pb_base + (size_t)qrg * (p.K >> 6) + k_first;
+    }
+    int b_dst[4];                          // row + 128 has the same swizzle: + 128 rows of bytes
 #pragma unroll
     for (int i = 0; i < 4; ++i) { b_dst[i] = qrow * kRowB + swz(qrow, qhalf * 4 + i) * 16; }
 
@@ -227,18 +252,22 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
                                          (__attribute__((address_space(3))) void*)(dst + i * (8 * kRowB)), 16, 0, 0);
       }
     };
-    auto dequant_to = [&](int stage, const CodeRegs& r) {
-      const float sc = bf16_bits_to_f32(r.s_bits), bi = bf16_bits_to_f32(r.b_bits);
-      uint8_t* nb = w_lds + stage * kWStage;
+    auto dequant_to = [&](int stage, const CodeRegs (&r)[kWH]) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word(r.codes[i], sc, bi); }
+      for (int h = 0; h < kWH; ++h) {
+        const float sc = bf16_bits_to_f32(r[h].s_bits), bi = bf16_bits_to_f32(r[h].b_bits);
+        uint8_t* nb = w_lds + stage * kWStage + h * (128 * kRowB);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word(r[h].codes[i], sc, bi); }
+      }
     };
-    auto request = [&](CodeRegs& r, int step) {
-      request_codes(r, wrow + (size_t)step * (TK / 2), srow + step, brow + step);
+    auto request = [&](CodeRegs (&r)[kWH], int step) {
+#pragma unroll
+      for (int h = 0; h < kWH; ++h) { request_codes(r[h], wrow[h] + (size_t)step * (TK / 2), srow[h] + step, brow[h] + step); }
     };
 
     // Prologue: steps 0 and 1 complete in stages 0 and 1; codes of steps 2 and 3 requested.
-    CodeRegs ra, rb;                       // codes of even / odd steps
+    CodeRegs ra[kWH], rb[kWH];             // codes of even / odd steps
     request(ra, 0);
     request(rb, KT > 1 ? 1 : 0);
     issue_x(0, 0);
@@ -249,27 +278,27 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     if (KT > 1) { dequant_to(1, rb); }
     request(ra, KT > 2 ? 2 : 0);
     request(rb, KT > 3 ? 3 : 0);
-    asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");   // all but the 6 code requests
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(2 * kCR) : "memory");   // all but the code requests of steps 2, 3
     wg_barrier();
 
     // Steady state, step s fills the stage of step t = s+2.  Requests in issue order, with X = kXL
-    // (8 at 256 rows):
-    //   ..., x(t-1) [X], codes(t+1) [3], x(t) [X], codes(t+2) [3]
+    // (8 at 256 rows of x) and C = kCR (3 at 128 weight rows):
+    //   ..., x(t-1) [X], codes(t+1) [C], x(t) [X], codes(t+2) [C]
     // x(t) goes out first so that it has two whole steps to land.  codes(t) were requested two
-    // steps ago: X + 3 + X younger requests may stay in flight while they are awaited (19).
-    // Before the barrier x(t-1), the tile of step s+1, must have landed: 3 + X + 3 younger requests (14).
-    // The first fill follows the prologue, where only codes(3) [3] and x(2) [X] are younger (11).
-    auto fill = [&](auto younger, int t, int stage, CodeRegs& r) {
+    // steps ago: X + C + X younger requests may stay in flight while they are awaited (19).
+    // Before the barrier x(t-1), the tile of step s+1, must have landed: C + X + C younger requests (14).
+    // The first fill follows the prologue, where only codes(3) [C] and x(2) [X] are younger (11).
+    auto fill = [&](auto younger, int t, int stage, CodeRegs (&r)[kWH]) {
       issue_x(t, stage);
       wait_codes<decltype(younger)::value>(r);
       dequant_to(stage, r);
       request(r, t + 2 < KT ? t + 2 : t);           // the last two requests are never used
-      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kXL + 6) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kXL + 2 * kCR) : "memory");
     };
     auto next_stage = [](int stage) { return stage == kStages - 1 ? 0 : stage + 1; };
     auto odd_fill = [&](int t, int stage) {
       if (t < KT) {
-        fill(std::integral_constant<int, 2 * kXL + 3>(), t, stage, rb);
+        fill(std::integral_constant<int, 2 * kXL + kCR>(), t, stage, rb);
       } else {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       }
@@ -277,7 +306,7 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     int tstage = 2;                        // stage of step s+2
     int s = 0;
     if (KT > 2) {
-      fill(std::integral_constant<int, kXL + 3>(), 2, tstage, ra);
+      fill(std::integral_constant<int, kXL + kCR>(), 2, tstage, ra);
       wg_barrier();
       tstage = next_stage(tstage);
       odd_fill(3, tstage);
@@ -286,7 +315,7 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
       s = 2;
     }
     for (; s + 2 < KT; s += 2) {
-      fill(std::integral_constant<int, 2 * kXL + 3>(), s + 2, tstage, ra);   // even step: codes in ra
+      fill(std::integral_constant<int, 2 * kXL + kCR>(), s + 2, tstage, ra);   // even step: codes in ra
       wg_barrier();
       tstage = next_stage(tstage);
       odd_fill(s + 3, tstage);
@@ -336,9 +365,9 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
 
   // ======================= consumers =======================
   const int wm = wave >> 1, wn = wave & 1;
-  floatx16 acc[2][kIT];   // [jt: 32 weight rows][it: 32 x rows]
+  floatx16 acc[kJT][kIT];   // [jt: 32 weight rows][it: 32 x rows]
 #pragma unroll
-  for (int jt = 0; jt < 2; ++jt) {
+  for (int jt = 0; jt < kJT; ++jt) {
 #pragma unroll
     for (int it = 0; it < kIT; ++it) {
 #pragma unroll
@@ -347,12 +376,26 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
   }
   const int frow = lane & 31;      // row of a 32-row operand fragment
   const int fkh = lane >> 5;       // which 8 of the 16 k
-  int w_rd[2], x_rd[kIT];          // stage-relative operand rows
+  int w_rd[kJT], x_rd[kIT];        // stage-relative operand rows
 #pragma unroll
-  for (int jt = 0; jt < 2; ++jt) { w_rd[jt] = (wn * 64 + jt * 32 + frow) * kRowB; }
+  for (int jt = 0; jt < kJT; ++jt) { w_rd[jt] = (wn * (TNK / 2) + jt * 32 + frow) * kRowB; }
 #pragma unroll
   for (int it = 0; it < kIT; ++it) { x_rd[it] = (wm * kWaveM + it * 32 + frow) * kRowB; }
   const int f_sw = (frow >> 1) & 7;   // the tile offsets are multiples of 16 rows: same swizzle for all
+  // Grouped form: a 32-row fragment of x whose slots are all padding (the tail of an expert's last block)
+  // is neither read nor multiplied; its accumulators stay zero.
+  bool frag_live[kIT];
+#pragma unroll
+  for (int it = 0; it < kIT; ++it) { frag_live[it] = true; }
+  if constexpr (GROUPED) {
+    static_assert(!GROUPED || kWaveM == 64, "one index per lane covers the wavefront's rows");
+    const int* idx = p.srow != nullptr ? p.srow : p.sdst;
+    const int lim = p.srow != nullptr ? p.rows_x : p.rows_y;
+    const int v = idx[m0 + wm * kWaveM + lane];
+    const unsigned long long mask = __ballot(v >= 0 && v < lim);
+#pragma unroll
+    for (int it = 0; it < kIT; ++it) { frag_live[it] = ((mask >> (32 * it)) & 0xffffffffull) != 0; }
+  }
 
   auto mma_stage = [&](int stage, int ksteps) {
     const uint8_t* xb = x_lds + stage * kXStage;
@@ -361,16 +404,20 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     for (int ks = 0; ks < 4; ++ks) {
       if (ks < ksteps) {
         const int c = ((2 * ks + fkh) ^ f_sw) * 16;
-        bf16x8 wf[2], xf[kIT];
+        bf16x8 wf[kJT], xf[kIT];
 #pragma unroll
-        for (int jt = 0; jt < 2; ++jt) { wf[jt] = *reinterpret_cast<const bf16x8*>(wb + w_rd[jt] + c); }
+        for (int jt = 0; jt < kJT; ++jt) { wf[jt] = *reinterpret_cast<const bf16x8*>(wb + w_rd[jt] + c); }
 #pragma unroll
-        for (int it = 0; it < kIT; ++it) { xf[it] = *reinterpret_cast<const bf16x8*>(xb + x_rd[it] + c); }
+        for (int it = 0; it < kIT; ++it) {
+          if (!GROUPED || frag_live[it]) { xf[it] = *reinterpret_cast<const bf16x8*>(xb + x_rd[it] + c); }
+        }
 #pragma unroll
-        for (int jt = 0; jt < 2; ++jt) {
+        for (int jt = 0; jt < kJT; ++jt) {
 #pragma unroll
           for (int it = 0; it < kIT; ++it) {
-            acc[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[jt], xf[it], acc[jt][it], 0, 0, 0);
+            if (!GROUPED || frag_live[it]) {
+              acc[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[jt], xf[it], acc[jt][it], 0, 0, 0);
+            }
           }
         }
       }
@@ -406,10 +453,10 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
       if (m >= p.M) { continue; }
       float* prow = p.plane + ((size_t)ks * p.M + m) * p.N;
 #pragma unroll
-      for (int jt = 0; jt < 2; ++jt) {
+      for (int jt = 0; jt < kJT; ++jt) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-          const int n = n0 + wn * 64 + jt * 32 + rq * 8 + fkh * 4;
+          const int n = n0 + wn * (TNK / 2) + jt * 32 + rq * 8 + fkh * 4;
           if (n >= p.N) { continue; }
           if (vec4 && n + 3 < p.N) {
             floatx4 v = {acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1], acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]};
@@ -442,10 +489,10 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
         }
       }
 #pragma unroll
-      for (int jt = 0; jt < 2; ++jt) {
+      for (int jt = 0; jt < kJT; ++jt) {
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-          const int n = n0 + wn * 64 + jt * 32 + rq * 8 + fkh * 4;
+          const int n = n0 + wn * (TNK / 2) + jt * 32 + rq * 8 + fkh * 4;
           if (n >= p.N) { continue; }
           const float f0 = pad_slot ? 0.0f : gated_f32(p.gate_act, acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
           const float f1 = pad_slot ? 0.0f : gated_f32(p.gate_act, acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
@@ -474,10 +521,10 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
     }
     uint16_t* yrow = p.y + (size_t)mdst * p.N;
 #pragma unroll
-    for (int jt = 0; jt < 2; ++jt) {
+    for (int jt = 0; jt < kJT; ++jt) {
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        const int n = n0 + wn * 64 + jt * 32 + rq * 8 + fkh * 4;
+        const int n = n0 + wn * (TNK / 2) + jt * 32 + rq * 8 + fkh * 4;
         if (n >= p.N) { continue; }
         const float v0 = acc[jt][it][rq * 4 + 0], v1 = acc[jt][it][rq * 4 + 1];
         const float v2 = acc[jt][it][rq * 4 + 2], v3 = acc[jt][it][rq * 4 + 3];
@@ -591,12 +638,14 @@ hipError_t launch_qmm_grouped(hipStream_t st, const GemmArgs& a, const GroupedAr
   p.out_stride = a.out_stride > 0 ? a.out_stride : a.N / 2;
   p.out_off = a.out_off;
   p.tiles_m = a.M / kGroupedBlockRows;       // a.M is a whole number of blocks
-  p.tiles_n = (a.N + TN - 1) / TN;
+  const bool wide = a.N > TN;                // 128 x 256 tiles unless one 128-wide tile holds all of N
+  p.tiles_n = wide ? (a.N + 2 * TN - 1) / (2 * TN) : 1;
   p.ksplit = 1; p.steps_per_split = a.K / TK; p.plane = nullptr;
   p.tile2e = g.tile2e; p.srow = g.srow; p.sdst = g.sdst;
   p.n_experts = g.n_experts; p.rows_x = g.rows_x; p.rows_y = g.rows_y;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
-  return launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, true>, grid, block, 0, st, p);
+  return wide ? launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true>, grid, block, 0, st, p)
+              : launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, TN, true>, grid, block, 0, st, p);
 }
 
 }  // namespace vpq
