@@ -45,7 +45,7 @@ namespace {
 
 constexpr int TM = 256, TN = 128, TK = 64;
 constexpr int kConsumers = 4;                        // consumer wavefronts: kConsumers/2 along M, 2 along N
-constexpr int kProducers = 4;
+constexpr int kProducers = 4;                        // producer wavefronts (8 in the 128 x 256 grouped form)
 constexpr int kThreads = (kConsumers + kProducers) * 64;
 constexpr int kStages = 3;
 constexpr int kRowB = TK * 2;                       // 128 bytes per LDS row
@@ -161,18 +161,21 @@ __device__ __forceinline__ void wait_codes(CodeRegs (&r)[2])
 
 // TMK x TNK: rows of x and weight rows per workgroup: 256 x 128, or 128 x {128, 256} for the grouped
 // form, whose blocks of rows are 128 tall (the wider tile gives a K step as much work as 256 x 128).
-template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false>
-__global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
+// P: producer wavefronts.  Where the step is as long as a producer's chain (wait, dequantize, store,
+// wait, barrier) -- the 128-row forms, with half the MFMAs per weight -- 8 producers halve that chain.
+template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false, int P = kProducers>
+__global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const TileParams p)
 {
-  static_assert((TMK == 256 && TNK == 128) || (TMK == 128 && !LORA && (TNK == 128 || TNK == 256)), "tiles built");
+  static_assert((TMK == 256 && TNK == 128 && P == 4) || (TMK == 128 && !LORA && (TNK == 128 || TNK == 256)), "tiles built");
+  static_assert(TMK % (8 * P) == 0 && TNK % (32 * P) == 0, "whole loads per producer");
   constexpr int kWStage = TNK * kRowB;             // 16 KB at 128 weight rows
-  constexpr int kWH = TNK / 128;                   // weight rows (code requests) per producer thread and step
+  constexpr int kWH = TNK / (32 * P);              // weight rows (code requests) per producer thread and step
   constexpr int kJT = TNK / 64;                    // 32-row W fragments per consumer wavefront
   constexpr int kCR = 3 * kWH;                     // code, scale and bias requests per producer thread and step
   constexpr int kWaveM = TMK / (kConsumers / 2);   // x rows per consumer wavefront
   constexpr int kIT = kWaveM / 32;                 // 32-row x fragments per consumer wavefront
   constexpr int kXStage = TMK * kRowB;             // 32 KB at 256 rows
-  constexpr int kXL = TMK / 32;                    // x-tile loads per producer wavefront and step
+  constexpr int kXL = TMK / (8 * P);               // x-tile loads per producer wavefront and step
   __shared__ __attribute__((aligned(16))) uint8_t x_lds[kStages * kXStage];   // 96 KB
   __shared__ __attribute__((aligned(16))) uint8_t w_lds[kStages * kWStage];   // 48 KB
 
@@ -205,8 +208,8 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
 
   if (producer) {
     // ======================= producers =======================
-    const int pw = wave - kConsumers;     // 0..3
-    const int pt = tid - kConsumers * 64; // 0..255
+    const int pw = wave - kConsumers;     // 0..P-1
+    const int pt = tid - kConsumers * 64; // 0..64P-1
     // x tile: 32 direct-to-LDS loads per step, 8 per wavefront.  Load i of wave pw covers tile
     // rows (8 pw + i)*8 .. +8; lane l takes row l/8, LDS position l%8.
     const bool gathered = GROUPED && p.srow != nullptr;
@@ -225,21 +228,21 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
       }
       a_off[i] = (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u;
     }
-    // W tile: thread pt dequantizes 32 codes of row pt/2 (k half pt%2) per step, and of row pt/2 + 128
-    // in a 256-row tile.
+    // W tile: thread pt dequantizes 32 codes of row pt/2 (k half pt%2) per step, and with kWH = 2 those of
+    // row pt/2 + 32 P as well.
     const int qrow = pt >> 1, qhalf = pt & 1;
     const uint8_t* wrow[kWH];
     const uint16_t* srow[kWH];
     const uint16_t* brow[kWH];
 #pragma unroll
     for (int h = 0; h < kWH; ++h) {
-      const int qrg = (n0 + qrow + 128 * h < p.N) ? (n0 + qrow + 128 * h) : (p.N - 1);
+      const int qrg = (n0 + qrow + 32 * P * h < p.N) ? (n0 + qrow + 32 * P * h) : (p.N - 1);
       wrow[h] = reinterpret_cast<const uint8_t*>(pw_base) + (size_t)qrg * (p.K >> 1) + qhalf * 16 +
                 (size_t)k_first * (TK / 2);
       srow[h] = ps_base + (size_t)qrg * (p.K >> 6) + k_first;
       brow[h] = pb_base + (size_t)qrg * (p.K >> 6) + k_first;
     }
-    int b_dst[4];                          // row + 128 has the same swizzle: + 128 rows of bytes
+    int b_dst[4];                          // row + 32 P has the same swizzle: + 32 P rows of bytes
 #pragma unroll
     for (int i = 0; i < 4; ++i) { b_dst[i] = qrow * kRowB + swz(qrow, qhalf * 4 + i) * 16; }
 
@@ -256,7 +259,7 @@ __global__ __launch_bounds__(kThreads) void qmm_tile_kernel(const TileParams p)
 #pragma unroll
       for (int h = 0; h < kWH; ++h) {
         const float sc = bf16_bits_to_f32(r[h].s_bits), bi = bf16_bits_to_f32(r[h].b_bits);
-        uint8_t* nb = w_lds + stage * kWStage + h * (128 * kRowB);
+        uint8_t* nb = w_lds + stage * kWStage + h * (32 * P * kRowB);
 #pragma unroll
         for (int i = 0; i < 4; ++i) { *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word(r[h].codes[i], sc, bi); }
       }
@@ -644,8 +647,10 @@ hipError_t launch_qmm_grouped(hipStream_t st, const GemmArgs& a, const GroupedAr
   p.tile2e = g.tile2e; p.srow = g.srow; p.sdst = g.sdst;
   p.n_experts = g.n_experts; p.rows_x = g.rows_x; p.rows_y = g.rows_y;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
-  return wide ? launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true>, grid, block, 0, st, p)
-              : launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, TN, true>, grid, block, 0, st, p);
+  if (wide) {
+    return launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true, 8>, grid, dim3((kConsumers + 8) * 64), 0, st, p);
+  }
+  return launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, TN, true>, grid, block, 0, st, p);
 }
 
 }  // namespace vpq
