@@ -356,7 +356,6 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   auto step = [&](auto stage_c, auto fill_c, int s) {
     using St = decltype(stage_c);
     using Nx = std::integral_constant<int, 1 - St::value>;
-    constexpr bool FILL = decltype(fill_c)::value;      // false for the last step only
     const bool codes_out = s + 2 < KT && dq_wave;
     const bool scales_out = St::value == 0 && (s & 7) == 0 && s + 8 < KT && dq_wave;
     // The requests go out from inside the MFMA stream, in the order x [8], codes [2], scales [2].
