@@ -135,6 +135,33 @@ __device__ __forceinline__ void request_codes(CodeRegs& r, const uint8_t* codes,
   asm volatile("global_load_ushort %0, %1, off" : "=v"(r.b_bits) : "v"(b) : "memory");
 }
 
+// The codes alone (scale and bias come from the LDS ring, see SBR).
+__device__ __forceinline__ void request_codes_only(CodeRegs& r, const uint8_t* codes)
+{
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.codes) : "v"(codes) : "memory");
+}
+
+// Scale and bias of one row and step from the ring, as loads the compiler does not track (it would order
+// them after every direct-to-LDS load of the wavefront); the caller's LDS queue is empty before them.
+__device__ __forceinline__ void read_scale_bias(CodeRegs& r, uint32_t s_addr, uint32_t b_addr)
+{
+  asm volatile("ds_read_u16 %0, %1" : "=v"(r.s_bits) : "v"(s_addr) : "memory");
+  asm volatile("ds_read_u16 %0, %1" : "=v"(r.b_bits) : "v"(b_addr) : "memory");
+}
+
+__device__ __forceinline__ uint32_t lds_addr_of(const uint8_t* q)
+{
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)q;
+}
+
+// 16 bytes per lane, global -> LDS at lds_dst + 16 * lane, written out by hand for the same reason.
+// M0 is used by nothing else in the wavefronts that call this.
+__device__ __forceinline__ void dma16_raw(uint32_t lds_dst, const uint8_t* src)
+{
+  const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+}
+
 // Waits until at most YOUNGER vector-memory requests issued after r's are outstanding; the
 // registers pass through the statement so that no use of them can be moved above the wait.
 template <int YOUNGER>
@@ -163,7 +190,11 @@ __device__ __forceinline__ void wait_codes(CodeRegs (&r)[2])
 // form, whose blocks of rows are 128 tall (the wider tile gives a K step as much work as 256 x 128).
 // P: producer wavefronts.  Where the step is as long as a producer's chain (wait, dequantize, store,
 // wait, barrier) -- the 128-row forms, with half the MFMAs per weight -- 8 producers halve that chain.
-template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false, int P = kProducers>
+// SBR: scales and biases come through an LDS ring in windows of 8 K steps (16 bytes per row and array),
+// brought in by the CONSUMER wavefronts, whose load counter nothing else uses: a 2-byte load per row, array
+// and step costs a 32-byte sector each, twice the bytes of the codes.  Needs K % 512 == 0, 16-byte
+// aligned scales and biases and no split of K.
+template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false, int P = kProducers, bool SBR = false>
 __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const TileParams p)
 {
   static_assert((TMK == 256 && TNK == 128 && P == 4) || (TMK == 128 && !LORA && (TNK == 128 || TNK == 256)), "tiles built");
@@ -171,13 +202,16 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
   constexpr int kWStage = TNK * kRowB;             // 16 KB at 128 weight rows
   constexpr int kWH = TNK / (32 * P);              // weight rows (code requests) per producer thread and step
   constexpr int kJT = TNK / 64;                    // 32-row W fragments per consumer wavefront
-  constexpr int kCR = 3 * kWH;                     // code, scale and bias requests per producer thread and step
+  constexpr int kCR = (SBR ? 1 : 3) * kWH;         // code (, scale and bias) requests per producer thread and step
+  constexpr int kSbSlot = 2 * TNK * 16;            // one window of the ring: scales | biases, 16 bytes per row
+  static_assert(!SBR || kWH == 1, "one row per producer thread");
   constexpr int kWaveM = TMK / (kConsumers / 2);   // x rows per consumer wavefront
   constexpr int kIT = kWaveM / 32;                 // 32-row x fragments per consumer wavefront
   constexpr int kXStage = TMK * kRowB;             // 32 KB at 256 rows
   constexpr int kXL = TMK / (8 * P);               // x-tile loads per producer wavefront and step
   __shared__ __attribute__((aligned(16))) uint8_t x_lds[kStages * kXStage];   // 96 KB
   __shared__ __attribute__((aligned(16))) uint8_t w_lds[kStages * kWStage];   // 48 KB
+  __shared__ __attribute__((aligned(16))) uint8_t sb_ring[SBR ? 2 * kSbSlot : 16];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -266,7 +300,24 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
     };
     auto request = [&](CodeRegs (&r)[kWH], int step) {
 #pragma unroll
-      for (int h = 0; h < kWH; ++h) { request_codes(r[h], wrow[h] + (size_t)step * (TK / 2), srow[h] + step, brow[h] + step); }
+      for (int h = 0; h < kWH; ++h) {
+        if constexpr (SBR) {
+          request_codes_only(r[h], wrow[h] + (size_t)step * (TK / 2));
+        } else {
+          request_codes(r[h], wrow[h] + (size_t)step * (TK / 2), srow[h] + step, brow[h] + step);
+        }
+      }
+    };
+    // SBR: scale and bias of this thread's row for step t, from the window t / 8 of the ring.
+    const uint32_t sb_row = lds_addr_of(sb_ring) + (uint32_t)qrow * 16u;
+    auto fetch_sb = [&](CodeRegs (&r)[kWH], int t) {
+      if constexpr (SBR) {
+        const uint32_t a = sb_row + (uint32_t)((t >> 3) & 1) * kSbSlot + (uint32_t)(t & 7) * 2u;
+        read_scale_bias(r[0], a, a + TNK * 16);
+      }
+    };
+    auto settle_sb = [&](CodeRegs (&r)[kWH]) {
+      if constexpr (SBR) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0].s_bits), "+v"(r[0].b_bits) : : "memory"); }
     };
 
     // Prologue: steps 0 and 1 complete in stages 0 and 1; codes of steps 2 and 3 requested.
@@ -277,11 +328,20 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
     if (KT > 1) { issue_x(1, 1); }
     wait_codes<0>(ra);
     wait_codes<0>(rb);
+    if constexpr (SBR) {
+      wg_barrier();                        // the consumers have brought in the first two windows of the ring
+      fetch_sb(ra, 0);
+      fetch_sb(rb, KT > 1 ? 1 : 0);
+      settle_sb(ra);
+      settle_sb(rb);
+    }
     dequant_to(0, ra);
     if (KT > 1) { dequant_to(1, rb); }
     request(ra, KT > 2 ? 2 : 0);
     request(rb, KT > 3 ? 3 : 0);
+    fetch_sb(ra, 2);                       // step 2's scale and bias (window 0)
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(2 * kCR) : "memory");   // all but the code requests of steps 2, 3
+    settle_sb(ra);
     wg_barrier();
 
     // Steady state, step s fills the stage of step t = s+2.  Requests in issue order, with X = kXL
@@ -291,17 +351,21 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
     // steps ago: X + C + X younger requests may stay in flight while they are awaited (19).
     // Before the barrier x(t-1), the tile of step s+1, must have landed: C + X + C younger requests (14).
     // The first fill follows the prologue, where only codes(3) [C] and x(2) [X] are younger (11).
-    auto fill = [&](auto younger, int t, int stage, CodeRegs (&r)[kWH]) {
+    // rn: the other register set, which the next fill uses.  SBR: its scale and bias are read from the ring
+    // here, behind this step's work, and have landed by the wait at the end (not in the chain of the next fill).
+    auto fill = [&](auto younger, int t, int stage, CodeRegs (&r)[kWH], CodeRegs (&rn)[kWH]) {
       issue_x(t, stage);
       wait_codes<decltype(younger)::value>(r);
       dequant_to(stage, r);
       request(r, t + 2 < KT ? t + 2 : t);           // the last two requests are never used
+      fetch_sb(rn, t + 1);
       asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kXL + 2 * kCR) : "memory");
+      settle_sb(rn);
     };
     auto next_stage = [](int stage) { return stage == kStages - 1 ? 0 : stage + 1; };
     auto odd_fill = [&](int t, int stage) {
       if (t < KT) {
-        fill(std::integral_constant<int, 2 * kXL + kCR>(), t, stage, rb);
+        fill(std::integral_constant<int, 2 * kXL + kCR>(), t, stage, rb, ra);
       } else {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       }
@@ -309,7 +373,7 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
     int tstage = 2;                        // stage of step s+2
     int s = 0;
     if (KT > 2) {
-      fill(std::integral_constant<int, kXL + kCR>(), 2, tstage, ra);
+      fill(std::integral_constant<int, kXL + kCR>(), 2, tstage, ra, rb);
       wg_barrier();
       tstage = next_stage(tstage);
       odd_fill(3, tstage);
@@ -318,7 +382,7 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
       s = 2;
     }
     for (; s + 2 < KT; s += 2) {
-      fill(std::integral_constant<int, 2 * kXL + kCR>(), s + 2, tstage, ra);   // even step: codes in ra
+      fill(std::integral_constant<int, 2 * kXL + kCR>(), s + 2, tstage, ra, rb);   // even step: codes in ra
       wg_barrier();
       tstage = next_stage(tstage);
       odd_fill(s + 3, tstage);
@@ -427,13 +491,48 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
     }
   };
 
+  // SBR: window wdw of the scales and biases (K steps 8 wdw .. 8 wdw + 7) into its slot of the ring.  The
+  // 2 TNK (array, row) entries of a window are dealt out 64 to a load over the four consumer wavefronts.
+  auto issue_window = [&](int wdw) {
+    if constexpr (SBR) {
+      constexpr int kLoads = 2 * TNK / 64 / kConsumers;        // 1 at 128 rows, 2 at 256
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) {
+        const int e = (wave * kLoads + j) * 64 + lane;         // entry: array e / TNK, row e % TNK
+        const int arr = e / TNK, row = e % TNK;
+        const int rg = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
+        const uint16_t* src = (arr ? pb_base : ps_base) + (size_t)rg * (p.K >> 6) + (size_t)wdw * 8;
+        dma16_raw(lds_addr_of(sb_ring) + (uint32_t)(wdw & 1) * kSbSlot + (uint32_t)(wave * kLoads + j) * 1024u,
+                  reinterpret_cast<const uint8_t*>(src));
+      }
+    }
+  };
+  if constexpr (SBR) {
+    issue_window(0);
+    if (KT > 8) { issue_window(1); }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    wg_barrier();                        // the producers read the ring from here on
+  }
   wg_barrier();                          // stages 0 and 1 are ready
   int cstage = 0;
-  for (int s = 0; s < KT; ++s) {
-    mma_stage(cstage, 4);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // every operand read of this stage is done
-    wg_barrier();
-    cstage = (cstage == kStages - 1) ? 0 : cstage + 1;
+  if constexpr (SBR) {
+    // The producers fill two steps ahead: window s/8 + 1 is first read in step s + 5 and the slot it
+    // replaces (window s/8 - 1) was last read in step s - 4.  Landed before the barrier of step s + 3.
+    for (int s = 0; s < KT; ++s) {
+      if ((s & 7) == 0 && s > 0 && s + 8 < KT) { issue_window((s >> 3) + 1); }
+      mma_stage(cstage, 4);
+      if ((s & 7) == 3) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // every operand read of this stage is done
+      wg_barrier();
+      cstage = (cstage == kStages - 1) ? 0 : cstage + 1;
+    }
+  } else {
+    for (int s = 0; s < KT; ++s) {
+      mma_stage(cstage, 4);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // every operand read of this stage is done
+      wg_barrier();
+      cstage = (cstage == kStages - 1) ? 0 : cstage + 1;
+    }
   }
   if (LORA) {
     const int steps = (p.r + TK - 1) / TK;
@@ -592,6 +691,13 @@ size_t qmm_splitk_workspace_bytes(int K, int N, int M, int cu_count)
   return s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
+// The scale/bias ring's windows are 16-byte loads of 8 groups: whole windows in every row, aligned.
+static bool sb_ring_ok(const GemmArgs& a)
+{
+  return (a.K % 512) == 0 && (reinterpret_cast<uintptr_t>(a.scales) & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(a.biases) & 15) == 0;
+}
+
 hipError_t launch_qmm_tile_splitk(hipStream_t st, const GemmArgs& a, int splits, float* plane)
 {
   TileParams p;
@@ -648,7 +754,9 @@ hipError_t launch_qmm_grouped(hipStream_t st, const GemmArgs& a, const GroupedAr
   p.n_experts = g.n_experts; p.rows_x = g.rows_x; p.rows_y = g.rows_y;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
   if (wide) {
-    return launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true, 8>, grid, dim3((kConsumers + 8) * 64), 0, st, p);
+    const dim3 block12((kConsumers + 8) * 64);
+    return sb_ring_ok(a) ? launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true, 8, true>, grid, block12, 0, st, p)
+                         : launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true, 8>, grid, block12, 0, st, p);
   }
   return launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, TN, true>, grid, block, 0, st, p);
 }
