@@ -227,9 +227,9 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
  * to 64 rows run the QMV arithmetic in slabs of at most 16 rows (one launch per
  * slab), larger M the QMM arithmetic.  (The reference crosses over to the GEMM at
  * M = 8; here the 256-row GEMM tile does not pay below ~64 rows: measured 57 us at
- * 4096->4096 for any M <= 256 against ~10 us per slab.)  Above 64 rows the GEMM
+ * 4096->4096 for any M <= 256 against ~10 us per slab.)  Above 32 rows the GEMM
  * splits K (vpq_qmm_splitk_w4g64_bf16) where that pays and `ws` has
- * vpq_qmm_workspace_bytes() bytes.  From 1024 rows on, when `ws` holds the
+ * vpq_qmm_workspace_bytes() bytes (without that room, 33..64 rows stay slabs).  From 1024 rows on, when `ws` holds the
  * expanded weight (N*K*2 bytes), the GEMM runs by the dequant-once route
  * (vpq_qmm_dense_route_w4g64_bf16: expansion + vendor GEMM, the reference's route
  * for large M, minimax-h3/metal-minimax-h3-transformer.cc:2020-2160), which is the

@@ -210,6 +210,32 @@ def test_linear_entrance_splits_k_when_given_the_room(vpq, oracle, dev, D):
     assert vpq.load().vpq_qmm_workspace_bytes(4096, 12288, 2048) == 0      # enough tiles: no split
 
 
+@pytest.mark.parametrize("M", [33, 48, 64])
+def test_linear_entrance_at_three_or_four_slabs(vpq, oracle, dev, D, M):
+    # with the room to split K the GEMM (bf16-rounded weights), without it slabs of QMV (un-rounded
+    # weights): each within the tolerance of its own oracle, and not the same bits
+    N, K = 384, 4096
+    w, s, b = synth.make_weight(N, K, 3300 + M)
+    x = synth.make_act(M, K, 3301 + M)
+    y64, yb = oracle.qmm(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    need = vpq.load().vpq_linear_workspace_bytes(K, N, M)
+    assert need >= 2 * M * N * 4
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    split = vpq.linear_w4g64(wd, sd, bd, xd, K, N, M, ws=ws)
+    direct = vpq.qmm_splitk_w4g64(wd, sd, bd, xd, K, N, M, splits=0, ws=ws.clone())
+    slabs = vpq.linear_w4g64(wd, sd, bd, xd, K, N, M)
+    torch.cuda.synchronize()
+    assert torch.equal(split, direct)
+    assert not torch.equal(split, slabs)
+    parity.check_bf16(D.bits(split), y64, yb)
+    v64, vb = oracle.qmv(w, s, b, x, K, N, M)                 # the slabs' arithmetic: un-rounded weights
+    parity.check_bf16(D.bits(slabs), v64, vb)
+    # 32 rows and fewer stay slabs whatever the workspace
+    x32 = xd[:32].contiguous()
+    assert torch.equal(vpq.linear_w4g64(wd, sd, bd, x32, K, N, 32, ws=ws), vpq.linear_w4g64(wd, sd, bd, x32, K, N, 32))
+
+
 # M, N, K: the minimal K (one block of 8 steps), ragged M and N in both tile widths, more than one
 # band of 8 rows of tiles (M > 2048), a single row
 BIG_TILE_SHAPES = [(300, 520, 512), (257, 193, 1024), (2300, 200, 512), (1, 8, 512), (640, 384, 1536)]

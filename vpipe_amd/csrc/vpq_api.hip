@@ -442,19 +442,30 @@ int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
 // the 256-row GEMM tile: below it the tile kernel has one row of tiles and N/128 workgroups, and
 // its time is its K loop's latency (57 us at 4096->4096 for any M <= 256) against ~10 us per slab.
 constexpr int kSlabPlanMaxRows = 64;
+constexpr int kSlabPlanSplitRows = 32;   // above: the split-K GEMM instead, when the workspace has the room
 
 int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                           void* ws, size_t ws_bytes)
 {
   if (M >= 1 && M <= kSlabPlanMaxRows && x != nullptr && y != nullptr && K > 0 && N > 0) {
-    for (int m0 = 0; m0 < M; m0 += 16) {
-      const int rows = M - m0 < 16 ? M - m0 : 16;
-      const int st = vpq_qmv_w4g64_bf16(stream, w, scales, biases, x + (size_t)m0 * K, y + (size_t)m0 * N, K, N, rows,
-                                        nullptr, ws, ws_bytes, VPQ_QMV_AUTO);
-      if (st != VPQ_OK) { return st; }
+    // Three or four slabs: the GEMM with K split over the workgroups is faster where the workspace lets it
+    // split (measured at 64 rows: 40 / 34 / 21 us against 43 / 68 / 31 us for four slabs at
+    // 4096->12288 / 12288->4096 / 4096->4096; two slabs, 23 / 35 / 16 us, stay ahead of it).
+    bool split_gemm = false;
+    if (M > kSlabPlanSplitRows && ws != nullptr && aligned(ws, 256) && (K % 64) == 0 && ensure_init() == VPQ_OK) {
+      const int splits = vpq::qmm_choose_splits(K, N, M, g_dev.cu_count);
+      split_gemm = splits > 1 && ws_bytes >= (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
     }
-    return VPQ_OK;
+    if (!split_gemm) {
+      for (int m0 = 0; m0 < M; m0 += 16) {
+        const int rows = M - m0 < 16 ? M - m0 : 16;
+        const int st = vpq_qmv_w4g64_bf16(stream, w, scales, biases, x + (size_t)m0 * K, y + (size_t)m0 * N, K, N, rows,
+                                          nullptr, ws, ws_bytes, VPQ_QMV_AUTO);
+        if (st != VPQ_OK) { return st; }
+      }
+      return VPQ_OK;
+    }
   }
   // Many rows: expanding the pack once into the workspace and running the vendor GEMM on it beats the
   // fused kernels (measured: 0.98-1.07 against 0.81-0.88 PFLOP/s at M = 2048, 1.35-1.5 against 0.98-1.1
