@@ -473,7 +473,25 @@ int vpq_argmax_combine(vpq_stream_t stream, const float* partials, int32_t* out_
  *                                    by the reference's own second route): expansion into
  *                                    `w_deq` [N,K] bf16 + the vendor dense GEMM; arguments as
  *                                    vpq_qmm_dense_route_w4g64_bf16.
+ *   vpq_qmv_gated_w8g64_bf16         replaces `affine_qmv_swiglu_w8g64` and `affine_qmv_geglu_w8g64`
+ *                                    (affine_qmv.metal:3140-3178): interleaved gate|up pack
+ *                                    [N = 2*ffn, K/4], y [M, N/2] = act(gate) * up, 1 <= M <= 16.
+ *   vpq_gather_qmv_gated_w8g64_bf16  replaces `affine_gather_qmv_swiglu_w8g64` (:962-990) and
+ *                                    `affine_gather_qmv_geglu_w8g64` (:1524-1552);
+ *   vpq_gather_down_qmv_w8g64_bf16   replaces `affine_gather_down_qmv_w8g64` (:1295-1322): the MoE
+ *                                    gathers over a batched 8-bit pack [E, N, K/4], arguments and
+ *                                    conventions of the 4-bit vpq_gather_* entries; a pair is
+ *                                    bit-identical to the plain 8-bit call on that expert's slab.
  * Requirements as for the 4-bit entries (K % 64 == 0; 16-byte aligned w, x). */
+int vpq_qmv_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                             int activation);
+int vpq_gather_qmv_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                    const int32_t* pair_eid, int npair, int top_k, int n_experts, int activation);
+int vpq_gather_down_qmv_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                   const int32_t* pair_eid, int npair, int n_experts);
 int vpq_dequant_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                            const uint16_t* biases, uint16_t* w_deq, int K, int N);
 int vpq_qmv_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

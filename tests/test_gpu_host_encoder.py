@@ -586,3 +586,54 @@ def test_eight_bit_and_group32_function_names(enc, oracle, dev, D):
     want = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(D.bits(yq)) + synth.bf16_bits_to_f32(res))
     assert np.array_equal(D.bits(yr), want)
     assert np.array_equal(D.bits(dense), oracle.dequant_g32_bf16(wq, sq, bq, K, N))
+
+
+def test_eight_bit_gated_and_gathered_function_names(vpq, enc, dev, D):
+    # affine_qmv_swiglu_w8g64 / affine_qmv_geglu_w8g64 (slots 0..6, rows from grid.x) and the 8-bit MoE gathers
+    # (slot 7 = pair_eid, 8 = top_k, pairs = grid.z): the encoder's results are the C ABI's, bit for bit
+    K, inner, H, E, top_k, M = 512, 24, 72, 4, 2, 2
+    packs = []
+    for e in range(E):
+        g, u = synth.make_weight8(inner, K, 3000 + 2 * e), synth.make_weight8(inner, K, 3001 + 2 * e)
+        packs.append(tuple(np.stack([a, b], axis=1).reshape((2 * inner,) + a.shape[1:]) for a, b in zip(g, u)))
+    guw, gus, gub = (np.stack([p[i] for p in packs]) for i in range(3))
+    dn = [synth.make_weight8(H, 64, 3100 + e) for e in range(E)]
+    dw, ds, db = (np.stack([p[i] for p in dn]) for i in range(3))
+    x = synth.make_act(M, K, 3200)
+    xs = synth.make_act(M * top_k, 64, 3201)
+    eid = torch.tensor([3, 0, 1, 3], dtype=torch.int32, device=dev)
+    gu_d = (D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev))
+    dn_d = (D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), D.bf16(xs, dev))
+    y_sw = torch.zeros((M, inner), dtype=torch.bfloat16, device=dev)
+    y_ge = torch.zeros((M, inner), dtype=torch.bfloat16, device=dev)
+    act = torch.zeros((M * top_k, inner), dtype=torch.bfloat16, device=dev)
+    part = torch.zeros((M * top_k, H), dtype=torch.bfloat16, device=dev)
+    for name, y in (("affine_qmv_swiglu_w8g64", y_sw), ("affine_qmv_geglu_w8g64", y_ge)):
+        assert enc.set_function("affine_qmv_bf16", name) == 1
+        for i, t in enumerate((gu_d[0][1], gu_d[1][1], gu_d[2][1], gu_d[3], y)):      # expert 1's slab as a plain pack
+            enc.set_buffer(i, t)
+        enc.set_constant(5, K)
+        enc.set_constant(6, 2 * inner)
+        enc.dispatch((32 * M, inner // 2, 1), (32, 2, 1))
+    assert enc.set_function("affine_qmv_bf16", "affine_gather_qmv_swiglu_w8g64") == 1
+    for i, t in enumerate(gu_d + (act,)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, 2 * inner)
+    enc.set_buffer(7, eid)
+    enc.set_constant(8, top_k)
+    enc.dispatch((32, inner // 2, M * top_k), (32, 2, 1))
+    assert enc.set_function("affine_qmv_bf16", "affine_gather_down_qmv_w8g64") == 1
+    for i, t in enumerate(dn_d + (part,)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, 64)
+    enc.set_constant(6, H)
+    enc.set_buffer(7, eid)
+    enc.dispatch((32, H // 4, M * top_k), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert torch.equal(y_sw, vpq.qmv_gated_w8g64(gu_d[0][1], gu_d[1][1], gu_d[2][1], gu_d[3], K, 2 * inner, M, activation=1))
+    assert torch.equal(y_ge, vpq.qmv_gated_w8g64(gu_d[0][1], gu_d[1][1], gu_d[2][1], gu_d[3], K, 2 * inner, M, activation=2))
+    assert torch.equal(act, vpq.gather_qmv_gated_w8g64(*gu_d, K, 2 * inner, eid, top_k, E))
+    assert torch.equal(part, vpq.gather_down_qmv_w8g64(*dn_d, 64, H, eid, E))
+    assert y_sw.abs().sum() > 0 and not torch.equal(y_sw, y_ge)

@@ -69,3 +69,91 @@ def test_qmm_w8_dense_route(vpq, oracle, dev, D, M, N, K):
     parity.check_bf16(D.bits(y), y64, yb)
     y2 = vpq.qmm_dense_route_w8g64(wd, sd, bd, xd, K, N, M, wdeq, expand=False)
     assert torch.equal(y, y2)
+
+
+def interleaved8(ffn, K, seed):
+    """Gate and up 8-bit packs and their interleaved [2*ffn, ...] form (row 2g gate, 2g+1 up)."""
+    g = synth.make_weight8(ffn, K, seed)
+    u = synth.make_weight8(ffn, K, seed + 1)
+    return tuple(np.stack([a, b], axis=1).reshape((2 * ffn,) + a.shape[1:]) for a, b in zip(g, u))
+
+
+@pytest.mark.parametrize("activation", [1, 2])
+@pytest.mark.parametrize("K,ffn,M", [(64, 3, 1), (1024, 40, 2), (3840, 17, 1), (4096, 96, 16)])
+def test_qmv_w8_gated(vpq, oracle, dev, D, K, ffn, M, activation):
+    w, s, b = interleaved8(ffn, K, 2300 + K + ffn)
+    x = synth.make_act(M, K, 2400 + K + M)
+    y64, _ = oracle.matmul8(w, s, b, x, K, 2 * ffn, M, rounded=False)
+    want64, wantb = (oracle.swiglu if activation == 1 else oracle.geglu)(y64)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M, ffn), torch.bfloat16, dev)
+    vpq.qmv_gated_w8g64(wd, sd, bd, xd, K, 2 * ffn, M, out=out.view, activation=activation)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_bf16(D.bits(out.view), want64, wantb, mismatch_over_all=activation == 1)
+
+
+@pytest.mark.parametrize("activation", [1, 2])
+def test_gathered_expert_projections_w8(vpq, oracle, dev, D, activation):
+    # the MoE block of the 4-bit gather tests with 8-bit experts: every pair against the oracle on its
+    # expert's slab and bit for bit against the plain 8-bit calls on that slab
+    K, inner, H, E, top_k, M = 1024, 48, 200, 5, 3, 2
+    gu = [interleaved8(inner, K, 2500 + 7 * e) for e in range(E)]
+    dn = [synth.make_weight8(H, 64 * ((inner + 63) // 64), 2600 + e) for e in range(E)]
+    Kd = 64 * ((inner + 63) // 64)
+    guw, gus, gub = (np.stack([p[i] for p in gu]) for i in range(3))
+    dw, ds, db = (np.stack([p[i] for p in dn]) for i in range(3))
+    x = synth.make_act(M, K, 2700)
+    npair = M * top_k
+    eid = np.array([4, 0, 2, 1, 4, 3], dtype=np.int32)
+    eidd = torch.from_numpy(eid).to(dev)
+    guwd, gusd, gubd, xd = stage(D, dev, guw, gus, gub, x)
+    act = parity.Guarded((npair, inner), torch.bfloat16, dev)
+    vpq.gather_qmv_gated_w8g64(guwd, gusd, gubd, xd, K, 2 * inner, eidd, top_k, E, out=act.view, activation=activation)
+    torch.cuda.synchronize()
+    act.assert_intact()
+    got = D.bits(act.view)
+    fn = oracle.swiglu if activation == 1 else oracle.geglu
+    want64 = np.empty((npair, inner))
+    wantb = np.empty((npair, inner), dtype=np.uint16)
+    for p in range(npair):
+        e, t = int(eid[p]), p // top_k
+        y64, _ = oracle.matmul8(guw[e], gus[e], gub[e], x[t:t + 1], K, 2 * inner, 1, rounded=False)
+        want64[p], wantb[p] = (a[0] for a in fn(y64))
+        plain = vpq.qmv_gated_w8g64(guwd[e], gusd[e], gubd[e], xd[t:t + 1], K, 2 * inner, 1, activation=activation)
+        assert np.array_equal(got[p], D.bits(plain)[0])
+    parity.check_bf16(got, want64, wantb, mismatch_over_all=activation == 1)
+    # down: x [npair, Kd] in pair order
+    xs = synth.make_act(npair, Kd, 2701)
+    dwd, dsd, dbd, xsd = stage(D, dev, dw, ds, db, xs)
+    part = parity.Guarded((npair, H), torch.bfloat16, dev)
+    vpq.gather_down_qmv_w8g64(dwd, dsd, dbd, xsd, Kd, H, eidd, E, out=part.view)
+    torch.cuda.synchronize()
+    part.assert_intact()
+    gotd = D.bits(part.view)
+    d64 = np.empty((npair, H))
+    dbits = np.empty((npair, H), dtype=np.uint16)
+    for p in range(npair):
+        e = int(eid[p])
+        a64, ab = oracle.matmul8(dw[e], ds[e], db[e], xs[p:p + 1], Kd, H, 1, rounded=False)
+        d64[p], dbits[p] = a64[0], ab[0]
+        plain = vpq.qmv_w8g64(dwd[e], dsd[e], dbd[e], xsd[p:p + 1], Kd, H, 1)
+        assert np.array_equal(gotd[p], D.bits(plain)[0])
+    parity.check_bf16(gotd, d64, dbits)
+
+
+def test_w8_gather_ids_out_of_range_and_bad_arguments(vpq, dev, D):
+    K, inner, E = 256, 8, 3
+    w, s, b = (np.stack([p[i] for p in [interleaved8(inner, K, 2800 + e) for e in range(E)]]) for i in range(3))
+    x = synth.make_act(2, K, 2801)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    eid = torch.tensor([1, -1, E, 2], dtype=torch.int32, device=dev)
+    got = D.bits(vpq.gather_qmv_gated_w8g64(wd, sd, bd, xd, K, 2 * inner, eid, 2, E))
+    assert not got[1].any() and not got[2].any() and got[0].any() and got[3].any()
+    L = vpq.load()
+    p = wd.data_ptr()
+    assert L.vpq_qmv_gated_w8g64_bf16(None, p, p, p, p, p, 64, 7, 1, 1) == -2          # odd N
+    assert L.vpq_qmv_gated_w8g64_bf16(None, p, p, p, p, p, 64, 8, 17, 1) == -2         # rows
+    assert L.vpq_qmv_gated_w8g64_bf16(None, p, p, p, p, p, 64, 8, 1, 5) == -2          # activation
+    assert L.vpq_gather_down_qmv_w8g64_bf16(None, p, p, p, p, p, 64, 8, None, 1, 1) == -1
+    assert L.vpq_gather_qmv_gated_w8g64_bf16(None, p, p, p, p, p, 64, 8, p, 1, 0, 1, 1) == -2   # top_k 0

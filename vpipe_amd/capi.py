@@ -66,6 +66,9 @@ SYMBOLS = [
     ("vpq_qmm_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
     ("vpq_linear_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_gather_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
+    ("vpq_gather_down_qmv_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i]),
     ("vpq_qmv_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     ("vpq_qmv_w8g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     ("vpq_qmm_dense_route_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
@@ -376,6 +379,39 @@ def qmm_splitk_w4g64(w, scales, biases, x, K, N, M, splits=0, ws=None, out=None)
         ws = torch.empty(need, dtype=torch.uint8, device=w.device)
     _check(L.vpq_qmm_splitk_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M, splits,
                                        _ptr(ws), ws.numel()), "vpq_qmm_splitk_w4g64_bf16")
+    return out
+
+
+def qmv_gated_w8g64(w, scales, biases, x, K, N, M, out=None, activation=VPQ_GATE_SWIGLU):
+    """8-bit interleaved gate|up pack [N=2*ffn, K/4], x [M, K] -> bf16 [M, N/2]."""
+    import torch
+    if out is None:
+        out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmv_gated_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                           activation), "vpq_qmv_gated_w8g64_bf16")
+    return out
+
+
+def gather_qmv_gated_w8g64(w, scales, biases, x, K, N, pair_eid, top_k, n_experts, out=None, activation=VPQ_GATE_SWIGLU):
+    """8-bit expert batch [E, N=2*inner, K/4], x [M, K], pair_eid int32 [npair] -> bf16 [npair, N/2]."""
+    import torch
+    npair = pair_eid.numel()
+    if out is None:
+        out = torch.empty((npair, N // 2), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_gather_qmv_gated_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                  _ptr(pair_eid), npair, top_k, n_experts, activation),
+           "vpq_gather_qmv_gated_w8g64_bf16")
+    return out
+
+
+def gather_down_qmv_w8g64(w, scales, biases, x, K, N, pair_eid, n_experts, out=None):
+    """8-bit expert batch [E, N, K/4], x [npair, K], pair_eid int32 [npair] -> bf16 [npair, N]."""
+    import torch
+    npair = pair_eid.numel()
+    if out is None:
+        out = torch.empty((npair, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_gather_down_qmv_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                 _ptr(pair_eid), npair, n_experts), "vpq_gather_down_qmv_w8g64_bf16")
     return out
 
 

@@ -233,6 +233,49 @@ int vpq_qmv_w8g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t*
   return qmv8_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr);
 }
 
+static int rows8_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                        const uint16_t* x, uint16_t* y, int K, int N, int rows, int gate_act, const int32_t* pair_eid,
+                        bool gathered, int x_div, int n_experts)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr || (gathered && pair_eid == nullptr)) { return VPQ_ERR_NULL_POINTER; }
+  if (gate_act != 0 && gate_act != VPQ_GATE_SWIGLU && gate_act != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (rows < 1 || rows > 65535 || (gate_act != 0 && (N & 1) != 0)) { return VPQ_ERR_BAD_SHAPE; }
+  if (gathered ? (x_div < 1 || n_experts < 1) : rows > 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 2) || (gathered && !aligned(pair_eid, 4))) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y;
+  a.K = K; a.N = N; a.M = 1; a.y_f32 = false; a.cu_count = g_dev.cu_count;
+  a.gate_act = gate_act;
+  return finish(vpq::launch_qmv_rows8(reinterpret_cast<hipStream_t>(stream), a, rows, gathered ? pair_eid : nullptr, x_div,
+                                      n_experts));
+}
+
+int vpq_qmv_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return rows8_common(stream, w, scales, biases, x, y, K, N, M, activation, nullptr, false, 1, 1);
+}
+
+int vpq_gather_qmv_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                    const int32_t* pair_eid, int npair, int top_k, int n_experts, int activation)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return rows8_common(stream, w, scales, biases, x, y, K, N, npair, activation, pair_eid, true, top_k, n_experts);
+}
+
+int vpq_gather_down_qmv_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                   const int32_t* pair_eid, int npair, int n_experts)
+{
+  return rows8_common(stream, w, scales, biases, x, y, K, N, npair, 0, pair_eid, true, 1, n_experts);
+}
+
 int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                                    uint16_t* w_deq, int expand)

@@ -88,6 +88,9 @@ hipError_t launch_qmv_rows_g32(hipStream_t st, const QmvArgs& a, bool scale_only
 hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                            uint16_t* out, int K, int N);
 hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a);
+// 8-bit gated / gathered QMV, one wavefront per output and row (a.gate_act: interleaved gate|up pack);
+// rows = rows of x, or with pair_eid the (token, expert) pairs over a batched pack.
+hipError_t launch_qmv_rows8(hipStream_t st, const QmvArgs& a, int rows, const int* pair_eid, int x_div, int n_experts);
 // Returns hipErrorInvalidValue if the shape is outside what the MFMA kernel
 // handles (the caller then falls back to the simple kernel).
 bool qmv_mfma_supports(int K, int N, int M);

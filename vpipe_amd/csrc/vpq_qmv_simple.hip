@@ -201,6 +201,92 @@ __global__ __launch_bounds__(256) void qmv_simple8_kernel(
   }
 }
 
+// 8-bit gated and gathered forms (affine_qmv_swiglu_w8g64 / affine_qmv_geglu_w8g64,
+// gpu-kernels/metal/quant/affine_qmv.metal:3140-3178; affine_gather_qmv_swiglu_w8g64 :962-990,
+// affine_gather_qmv_geglu_w8g64 :1524-1552, affine_gather_down_qmv_w8g64 :1295-1322).  One wavefront
+// per output: a plain row, or (GATED) the gate and the up row of a feature of the interleaved pack,
+// whose two sums meet in that wavefront's registers.  blockIdx.y is the row of x, or with pair_eid
+// the (token, expert) pair: the pack is then the slab pair_eid[pair] of a batch [E, N, K/4], x row
+// pair / x_div, y row pair; an id outside [0, n_experts) gives zeros.
+template <bool GATED>
+__global__ __launch_bounds__(256) void qmv_rows8_kernel(
+    const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales, const uint16_t* __restrict__ biases,
+    const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int K, int N, int gate_act,
+    const int* __restrict__ pair_eid, int x_div, int n_experts)
+{
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int outs = GATED ? (N >> 1) : N;
+  const int o = blockIdx.x * 4 + wave;
+  if (o >= outs) { return; }  // wave-uniform; no barrier in this kernel
+  const int m = blockIdx.y;
+  const int Kw = K >> 2, Kg = K >> 6;
+  int xrow = m;
+  if (pair_eid != nullptr) {
+    const int e = pair_eid[m];
+    if (e < 0 || e >= n_experts) {
+      if (lane == 0) { y[(size_t)m * outs + o] = 0; }
+      return;
+    }
+    w += (size_t)e * (size_t)N * Kw;
+    scales += (size_t)e * (size_t)N * Kg;
+    biases += (size_t)e * (size_t)N * Kg;
+    xrow = m / x_div;
+  }
+  const uint16_t* xr = x + (size_t)xrow * K;
+  constexpr int R = GATED ? 2 : 1;
+  const int n0 = GATED ? 2 * o : o;
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) { acc[r] = 0.0f; }
+  for (int k0 = lane * 16; k0 < K; k0 += kWave * 16) {
+    const uint4* xp = reinterpret_cast<const uint4*>(xr + k0);
+    float xv[16];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint4 x4 = xp[h];
+      const uint32_t xd[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        xv[8 * h + 2 * j] = bf16_lo_to_f32(xd[j]);
+        xv[8 * h + 2 * j + 1] = bf16_hi_to_f32(xd[j]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const size_t n = (size_t)(n0 + r);
+      const uint4 c4 = *reinterpret_cast<const uint4*>(w + n * Kw + (k0 >> 2));
+      const uint32_t codes[4] = {c4.x, c4.y, c4.z, c4.w};
+      const float s = bf16_bits_to_f32(scales[n * Kg + (k0 >> 6)]);
+      const float b = bf16_bits_to_f32(biases[n * Kg + (k0 >> 6)]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[r] = fmaf(xv[4 * i + j], fmaf(s, (float)((codes[i] >> (8 * j)) & 0xffu), b), acc[r]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) { acc[r] = wave_sum(acc[r]); }
+  if (lane == 0) {
+    const float v = GATED ? gated_f32(gate_act, acc[0], acc[R - 1]) : acc[0];
+    y[(size_t)m * outs + o] = (uint16_t)f32_to_bf16_bits(v);
+  }
+}
+
+hipError_t launch_qmv_rows8(hipStream_t st, const QmvArgs& a, int rows, const int* pair_eid, int x_div, int n_experts)
+{
+  const int outs = a.gate_act ? a.N / 2 : a.N;
+  const dim3 grid((unsigned)((outs + 3) / 4), (unsigned)rows), block(256);
+  uint16_t* y = static_cast<uint16_t*>(a.y);
+  return a.gate_act ? launch_kernel(qmv_rows8_kernel<true>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, y, a.K, a.N,
+                                    a.gate_act, pair_eid, x_div, n_experts)
+                    : launch_kernel(qmv_rows8_kernel<false>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, y, a.K, a.N, 0,
+                                    pair_eid, x_div, n_experts);
+}
+
 hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a)
 {
   const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);

@@ -109,6 +109,11 @@ const FnEntry kFunctions[] = {
     {"affine_dequant_bf16", "affine_dequant_w8g64", QuantKernel::Dequant, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64", QuantKernel::Qmv, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_swiglu_w8g64", QuantKernel::QmvSwiglu, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_geglu_w8g64", QuantKernel::QmvGeglu, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w8g64", QuantKernel::GatherSwiglu, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_gather_qmv_geglu_w8g64", QuantKernel::GatherGeglu, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_gather_down_qmv_w8g64", QuantKernel::GatherDown, QuantFormat::W8G64},
     {"affine_dequant_bf16", "affine_dequant_w4g32", QuantKernel::Dequant, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_w4g32", QuantKernel::Qmv, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_w4g32_add", QuantKernel::QmvAdd, QuantFormat::W4G32},
@@ -400,7 +405,30 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
       const int K = ival(5), N = ival(6);
       const int M = grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1;
       const uint16_t* residual = kind == QuantKernel::QmvAdd ? static_cast<const uint16_t*>(buf(7)) : nullptr;
-      if (fmt == QuantFormat::W8G64) {
+      const bool gather = kind == QuantKernel::GatherSwiglu || kind == QuantKernel::GatherGeglu ||
+                          kind == QuantKernel::GatherDown;
+      if (fmt == QuantFormat::W8G64 && gather) {
+        // gpu-kernels/metal/quant/affine_qmv.metal:962-990, 1295-1322, 1524-1552: slot 7 = pair_eid, 8 = top_k
+        // (gate|up only), pairs = grid.z; the expert count is what the bound code buffer holds (K bytes a row)
+        const bool down = kind == QuantKernel::GatherDown;
+        if (!buf(7) || (!down && !has_int(8))) {
+          status = VPQ_ERR_NULL_POINTER;
+        } else if (K <= 0 || N <= 0 || K % 64 != 0) {
+          status = VPQ_ERR_BAD_SHAPE;
+        } else {
+          const std::size_t experts = _slots[0].bytes / (static_cast<std::size_t>(N) * static_cast<std::size_t>(K));
+          const int E = experts > 0x7fffffffu ? 0x7fffffff : static_cast<int>(experts);
+          const int32_t* eid = static_cast<const int32_t*>(buf(7));
+          const int npair = static_cast<int>(grid.z);
+          status = down ? vpq_gather_down_qmv_w8g64_bf16(st, w, sc, bi, x, y, K, N, eid, npair, E)
+                        : vpq_gather_qmv_gated_w8g64_bf16(st, w, sc, bi, x, y, K, N, eid, npair, ival(8), E,
+                                                          kind == QuantKernel::GatherGeglu ? VPQ_GATE_GEGLU
+                                                                                           : VPQ_GATE_SWIGLU);
+        }
+      } else if (fmt == QuantFormat::W8G64 && (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu)) {
+        status = vpq_qmv_gated_w8g64_bf16(st, w, sc, bi, x, y, K, N, M,
+                                          kind == QuantKernel::QmvGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
+      } else if (fmt == QuantFormat::W8G64) {
         status = vpq_qmv_w8g64_bf16(st, w, sc, bi, x, y, K, N, M, residual);
       } else if (kind == QuantKernel::QmvGeglu) {
         status = vpq_qmv_gated_w4g32_bf16(st, w, sc, q40 ? nullptr : bi, x, y, K, N, M, VPQ_GATE_GEGLU, q40 ? 1 : 0);
