@@ -503,6 +503,36 @@ int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                    int K, int N, int M, uint16_t* w_deq, int expand);
 
+/* ---- IEEE binary16 element type (f16) ------------------------------------
+ * The reference builds every kernel for two element types (VPIPE_ELT = bfloat
+ * and half: apple-silicon/metal-compute/CMakeLists.txt:71-72, 159-162; the
+ * metallibs without the `_bf16` suffix).  These entries are the f16 forms of
+ * the 4-bit group-64 functions: scales, biases, x, y, residual and w_deq are
+ * IEEE binary16 bit patterns, the packed codes are the same.  A first, general
+ * path (one wavefront per output row for the QMV, expansion + vendor GEMM for
+ * the QMM), not tuned like the bf16 kernels:
+ *   vpq_dequant_w4g64_f16         `affine_dequant_w4g64` (affine_dequant.metal:25-58), bit-exact:
+ *                                 f16_rne(fp32(s) * q + fp32(b)).
+ *   vpq_qmv_w4g64_f16 / _f32out   `affine_qmv_w4g64[_add]` (affine_qmv.metal:286-301, 347-363),
+ *                                 1 <= M <= 16, fp32 accumulation, un-rounded weights.
+ *   vpq_qmv_gated_w4g64_f16       `affine_qmv_swiglu_w4g64`, `affine_qmv_geglu_w4g64` (:891-906, 1432-1447).
+ *   vpq_qmm_dense_route_w4g64_f16 the dequant-once route (expansion into w_deq [N,K] f16 + vendor
+ *                                 GEMM), arguments as vpq_qmm_dense_route_w4g64_bf16.
+ * Requirements as for the bf16 entries. */
+int vpq_dequant_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                          const uint16_t* biases, uint16_t* w_deq, int K, int N);
+int vpq_qmv_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                      const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                      int K, int N, int M, const uint16_t* residual);
+int vpq_qmv_w4g64_f16_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, float* y, int K, int N, int M);
+int vpq_qmv_gated_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                            const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                            int activation);
+int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                  const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                                  int K, int N, int M, uint16_t* w_deq, int expand);
+
 /* ---- a12: the packer ------------------------------------------------------
  * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:
  * 243-301; slots 0:x 1:w 2:s 3:b 4:K 5:N 6:clip) driven by

@@ -185,6 +185,25 @@ def qmm(w, s, b, x, K, N, M, t=None, B=None, r=0):
     return y64, yb
 
 
+def dequant_f16(w, s, b, K, N):
+    """binary16 scales / biases -> binary16 bits [N, K]."""
+    w, s, b = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16)
+    out = np.empty((N, K), dtype=np.uint16)
+    lib().vpo_dequant_w4g64_f16(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(out, _u16p), K, N)
+    return out
+
+
+def matmul_f16(w, s, b, x, K, N, M, rounded, residual=None):
+    """binary16 elements -> (y64, y_f16 bits); rounded: the GEMM's binary16-rounded weights."""
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    residual = _c(residual, np.uint16)
+    y64 = np.empty((M, N), dtype=np.float64)
+    yh = np.empty((M, N), dtype=np.uint16)
+    lib().vpo_matmul_w4g64_f16(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y64, _f64p), _p(yh, _u16p),
+                               K, N, M, _p(residual, _u16p), 1 if rounded else 0)
+    return y64, yh
+
+
 _i32p = ctypes.POINTER(ctypes.c_int32)
 
 

@@ -458,6 +458,58 @@ void vpo_geglu_pairs(const double* y, double* out64, uint16_t* out_bf16, int M, 
   }
 }
 
+/* ---- IEEE binary16 element type ----------------------------------------- */
+
+/* The reference's kernels are templates over the element type T (VPIPE_ELT = bfloat or half,
+ * apple-silicon/metal-compute/CMakeLists.txt:71-72, 159-162); these are the restatements above
+ * with T = half: scales, biases, x, outputs and the residual are binary16, the arithmetic in
+ * between is the same fp32 (gpu-kernels/metal/quant/affine_dequant.metal:45-52,
+ * affine_qmv.metal:151-174, 264-266, affine_qmm_steel.metal:78-96). */
+void vpo_dequant_w4g64_f16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           uint16_t* out, int K, int N)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_f16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_f16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      out[n * (size_t)K + k] = vpo_f32_to_f16(sq + b);
+    }
+  }
+}
+
+/* rounded != 0: the GEMM's weights, rounded to binary16 before the contraction; 0: the GEMV's. */
+void vpo_matmul_w4g64_f16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                          const uint16_t* x, double* y64, uint16_t* y_f16,
+                          int K, int N, int M, const uint16_t* residual, int rounded)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_f16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_f16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      wrow[k] = rounded ? vpo_f16_to_f32(vpo_f32_to_f16(sq + b)) : sq + b;
+    }
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      double acc = 0.0;
+      const uint16_t* xr = x + m * (size_t)K;
+      for (int k = 0; k < K; ++k) { acc += (double)vpo_f16_to_f32(xr[k]) * (double)wrow[k]; }
+      if (y64) { y64[m * (size_t)N + n] = acc; }
+      if (y_f16) {
+        uint16_t v = vpo_f32_to_f16((float)acc);
+        if (residual) {
+          v = vpo_f32_to_f16(vpo_f16_to_f32(v) + vpo_f16_to_f32(residual[m * (size_t)N + n]));
+        }
+        y_f16[m * (size_t)N + n] = v;
+      }
+    }
+  }
+  free(wrow);
+}
+
 /* ---- MoE prefill: the expert sort and the grouped GEMMs ------------------- */
 
 /* gpu-kernels/metal/ops/llm_elementwise.metal:255-326 (moe_ifill_i32, moe_hist_i32,

@@ -1,0 +1,108 @@
+"""GPU parity of the IEEE binary16 element type (the reference's VPIPE_ELT = half build) for the 4-bit
+group-64 pack: dense expansion bit-exact, QMV (plain, residual, gated) and the dequant-once GEMM route
+against the CPU oracle's binary16 twins, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from tests import parity
+from tests.test_oracle_pins import f16_pack
+
+pytestmark = pytest.mark.gpu
+
+F16_TOL = 2e-3
+
+
+def dev16(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).to(dev).view(torch.float16)
+
+
+def bits16(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def check_f16(got_bits, ref64):
+    """|got - ref| <= 2e-3 * max(|ref|, 1e-2 rms) + one binary16 step at |ref| (one rounding)."""
+    got = got_bits.view(np.float16).astype(np.float64)
+    rms = np.sqrt((ref64 ** 2).mean())
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref64), 2.0 ** -14))) - 10)
+    allowed = F16_TOL * np.maximum(np.abs(ref64), 1e-2 * rms) + ulp
+    worst = (np.abs(got - ref64) / allowed).max()
+    assert worst <= 1.0, "binary16 output off by %.2f x the allowed error" % worst
+    assert parity.rel_l2(got, ref64) <= 2e-3 + 3e-4
+
+
+@pytest.mark.parametrize("N,K", [(1, 64), (33, 192), (257, 3840), (1024, 4096)])
+def test_dequant_f16_bit_exact(vpq, oracle, dev, D, N, K):
+    w, s, b = f16_pack(N, K, 100 + N)
+    out = vpq.dequant_w4g64_f16(D.u32(w, dev), dev16(s, dev), dev16(b, dev), K, N)
+    assert np.array_equal(bits16(out), oracle.dequant_f16(w, s, b, K, N))
+
+
+@pytest.mark.parametrize("K,N,M", [(64, 5, 1), (192, 33, 3), (3840, 16, 1), (4096, 95, 8), (2560, 64, 16), (4096, 4096, 1)])
+def test_qmv_f16(vpq, oracle, dev, D, K, N, M):
+    w, s, b = f16_pack(N, K, 200 + K + N)
+    x = np.random.default_rng(300 + K + M).standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    y64, _ = oracle.matmul_f16(w, s, b, x, K, N, M, rounded=False)
+    wd, sd, bd, xd = D.u32(w, dev), dev16(s, dev), dev16(b, dev), dev16(x, dev)
+    f = vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, f32out=True)
+    out = parity.Guarded((M, N), torch.float16, dev)
+    vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_f32(f.cpu().numpy(), y64)
+    check_f16(bits16(out.view), y64)
+    # the bf16 build of the same kernel on the same pack read as bf16 differs: the element type is live
+    assert not torch.equal(out.view.view(torch.int16), vpq.qmv_w4g64(wd, sd.view(torch.bfloat16), bd.view(torch.bfloat16),
+                                                                     xd.view(torch.bfloat16), K, N, M, variant=1).view(torch.int16))
+
+
+def test_qmv_f16_residual_and_gated(vpq, oracle, dev, D):
+    K, ffn, M = 1024, 40, 2
+    N = 2 * ffn
+    w, s, b = f16_pack(N, K, 401)
+    x = np.random.default_rng(402).standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    res = np.random.default_rng(403).standard_normal((M, N)).astype(np.float16).view(np.uint16)
+    y64, _ = oracle.matmul_f16(w, s, b, x, K, N, M, rounded=False)
+    _, want_add = oracle.matmul_f16(w, s, b, x, K, N, M, rounded=False, residual=res)
+    wd, sd, bd, xd = D.u32(w, dev), dev16(s, dev), dev16(b, dev), dev16(x, dev)
+    got_add = bits16(vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, residual=dev16(res, dev)))
+    plain = bits16(vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M))
+    redo = (plain.view(np.float16).astype(np.float32) + res.view(np.float16).astype(np.float32)).astype(np.float16)
+    assert np.array_equal(got_add, redo.view(np.uint16))          # rounded, then added in binary16
+    assert (np.abs(got_add.view(np.float16).astype(np.float64) - want_add.view(np.float16).astype(np.float64)) <=
+            2e-3 * np.abs(y64) + 4e-3).all()
+    for activation, fn in ((1, oracle.swiglu), (2, oracle.geglu)):
+        g64, _ = fn(y64)
+        got = bits16(vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, activation=activation))
+        check_f16(got, g64)
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (130, 320, 256), (257, 129, 512)])
+def test_qmm_f16_dense_route(vpq, oracle, dev, D, M, N, K):
+    w, s, b = f16_pack(N, K, 500 + M)
+    x = np.random.default_rng(501 + M).standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    y64, _ = oracle.matmul_f16(w, s, b, x, K, N, M, rounded=True)
+    wd, sd, bd, xd = D.u32(w, dev), dev16(s, dev), dev16(b, dev), dev16(x, dev)
+    w_deq = torch.empty((N, K), dtype=torch.float16, device=dev)
+    try:
+        got = vpq.qmm_dense_route_w4g64_f16(wd, sd, bd, xd, K, N, M, w_deq)
+    except vpq.VpqError as e:
+        if e.status == -6:
+            pytest.skip("no vendor BLAS in this process")
+        raise
+    torch.cuda.synchronize()
+    assert np.array_equal(bits16(w_deq), oracle.dequant_f16(w, s, b, K, N))
+    check_f16(bits16(got), y64)
+    kept = vpq.qmm_dense_route_w4g64_f16(wd, sd, bd, xd, K, N, M, w_deq, expand=False)
+    assert torch.equal(kept, got)
+
+
+def test_f16_entries_reject_bad_arguments(vpq, dev):
+    L = vpq.load()
+    p = torch.zeros(4096, dtype=torch.int32, device=dev).data_ptr()
+    assert L.vpq_dequant_w4g64_f16(None, p, p, p, None, 64, 8) == -1
+    assert L.vpq_qmv_w4g64_f16(None, p, p, p, p, p, 60, 8, 1, None) == -2
+    assert L.vpq_qmv_w4g64_f16(None, p, p, p, p, p, 64, 8, 17, None) == -2
+    assert L.vpq_qmv_gated_w4g64_f16(None, p, p, p, p, p, 64, 7, 1, 1) == -2
+    assert L.vpq_qmm_dense_route_w4g64_f16(None, p, p, p, p, p, 64, 8, 4, None, 1) == -4

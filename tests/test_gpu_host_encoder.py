@@ -637,3 +637,27 @@ def test_eight_bit_gated_and_gathered_function_names(vpq, enc, dev, D):
     assert torch.equal(act, vpq.gather_qmv_gated_w8g64(*gu_d, K, 2 * inner, eid, top_k, E))
     assert torch.equal(part, vpq.gather_down_qmv_w8g64(*dn_d, 64, H, eid, E))
     assert y_sw.abs().sum() > 0 and not torch.equal(y_sw, y_ge)
+
+
+def test_binary16_library_names(vpq, enc, oracle, dev, D):
+    # the metallibs without the `_bf16` suffix hold the IEEE binary16 build of the same function names
+    from tests.test_oracle_pins import f16_pack
+    K, N = 512, 48
+    w, s, b = f16_pack(N, K, 77)
+    x = np.random.default_rng(78).standard_normal((1, K)).astype(np.float16).view(np.uint16)
+    as16 = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).to(dev).view(torch.float16)
+    wd, sd, bd, xd = D.u32(w, dev), as16(s), as16(b), as16(x)
+    dense = torch.zeros((N, K), dtype=torch.float16, device=dev)
+    y = torch.zeros((1, N), dtype=torch.float16, device=dev)
+    assert enc.set_function("affine_dequant", "affine_dequant_w4g64") == 1
+    for i, t in enumerate((wd, sd, bd, dense)):
+        enc.set_buffer(i, t)
+    enc.set_constant(4, K)
+    enc.set_constant(5, N)
+    enc.dispatch((K // 8, N, 1), (64, 1, 1))
+    encode_linear(enc, "affine_qmv", "affine_qmv_w4g64", wd, sd, bd, xd, y, K, N, grid=(32, N // 4, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert np.array_equal(dense.view(torch.int16).cpu().numpy().view(np.uint16), oracle.dequant_f16(w, s, b, K, N))
+    assert torch.equal(y, vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, 1))
+    assert enc.set_function("affine_qmv", "affine_qmm_steel_w4g64") == 0       # not in that library

@@ -562,3 +562,40 @@ def test_moe_sort_and_grouped_gemm_reduce_to_the_per_pair_statement(oracle):
     bad = np.array([1, -1, E, 0], dtype=np.int32)
     t2, sr, sd, u = oracle.moe_sort_pairs(bad, 1, E, B, 6)
     assert sorted(sd[sd >= 0].tolist()) == [0, 3] and u == 2
+
+
+def f16_pack(N, K, seed):
+    """A 4-bit pack whose scales and biases are IEEE binary16 (the reference's VPIPE_ELT = half build)."""
+    rng = np.random.default_rng(seed)
+    w = rng.integers(0, 2**32, size=(N, K // 8), dtype=np.uint32)
+    s = rng.uniform(0.005, 0.02, size=(N, K // 64)).astype(np.float16)
+    b = (np.float32(-8.0) * s.astype(np.float32) * (1 + 0.05 * rng.standard_normal(s.shape))).astype(np.float16)
+    return w, s.view(np.uint16), b.view(np.uint16)
+
+
+def test_f16_element_twins_against_numpy_float16(oracle):
+    """binary16 twins: the dense expansion against numpy's own float16 arithmetic written from the layout
+    (shifts on the packed words, a float32 multiply-add, numpy's round-to-nearest-even cast), the two
+    contractions against a float64 matmul of that expansion, the residual add in binary16."""
+    N, K, M = 19, 256, 3
+    w, s, b = f16_pack(N, K, 41)
+    q = ((w[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF).reshape(N, K).astype(np.float32)
+    sf = np.repeat(s.view(np.float16).astype(np.float32), 64, axis=1)
+    bf = np.repeat(b.view(np.float16).astype(np.float32), 64, axis=1)
+    dense32 = sf * q + bf                                   # s*q is exact in fp32: no contraction issue
+    want = dense32.astype(np.float16)
+    assert np.array_equal(oracle.dequant_f16(w, s, b, K, N), want.view(np.uint16))
+    x = np.random.default_rng(42).standard_normal((M, K)).astype(np.float16)
+    xb = x.view(np.uint16)
+    y64, yh = oracle.matmul_f16(w, s, b, xb, K, N, M, rounded=False)
+    ref = x.astype(np.float64) @ dense32.astype(np.float64).T
+    assert np.allclose(y64, ref, rtol=0, atol=1e-12 * np.abs(ref).max() + 1e-12)
+    assert np.array_equal(yh, ref.astype(np.float32).astype(np.float16).view(np.uint16))
+    r64, _ = oracle.matmul_f16(w, s, b, xb, K, N, M, rounded=True)
+    refr = x.astype(np.float64) @ want.astype(np.float64).T
+    assert np.allclose(r64, refr, rtol=0, atol=1e-12 * np.abs(refr).max() + 1e-12)
+    assert not np.array_equal(r64, y64)                     # the rounding of the weights is visible
+    res = np.random.default_rng(43).standard_normal((M, N)).astype(np.float16)
+    _, ya = oracle.matmul_f16(w, s, b, xb, K, N, M, rounded=False, residual=res.view(np.uint16))
+    want_add = (yh.view(np.float16).astype(np.float32) + res.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(ya, want_add.view(np.uint16))

@@ -65,6 +65,11 @@ SYMBOLS = [
     ("vpq_qmv_gated_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     ("vpq_qmm_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
     ("vpq_linear_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_dequant_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_qmv_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    ("vpq_qmv_w4g64_f16_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_qmv_gated_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_qmm_dense_route_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_gather_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
@@ -412,6 +417,48 @@ def gather_down_qmv_w8g64(w, scales, biases, x, K, N, pair_eid, n_experts, out=N
         out = torch.empty((npair, N), dtype=torch.bfloat16, device=w.device)
     _check(load().vpq_gather_down_qmv_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
                                                  _ptr(pair_eid), npair, n_experts), "vpq_gather_down_qmv_w8g64_bf16")
+    return out
+
+
+def dequant_w4g64_f16(w, scales, biases, K, N, out=None):
+    """binary16 scales / biases (torch.float16) -> float16 [N, K]."""
+    import torch
+    if out is None:
+        out = torch.empty((N, K), dtype=torch.float16, device=w.device)
+    _check(load().vpq_dequant_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out), K, N),
+           "vpq_dequant_w4g64_f16")
+    return out
+
+
+def qmv_w4g64_f16(w, scales, biases, x, K, N, M, out=None, residual=None, f32out=False, activation=0):
+    """float16 elements; activation != 0: interleaved gate|up pack -> [M, N/2]."""
+    import torch
+    L = load()
+    if activation:
+        if out is None:
+            out = torch.empty((M, N // 2), dtype=torch.float16, device=w.device)
+        _check(L.vpq_qmv_gated_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                         activation), "vpq_qmv_gated_w4g64_f16")
+        return out
+    if f32out:
+        if out is None:
+            out = torch.empty((M, N), dtype=torch.float32, device=w.device)
+        _check(L.vpq_qmv_w4g64_f16_f32out(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M),
+               "vpq_qmv_w4g64_f16_f32out")
+        return out
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=w.device)
+    _check(L.vpq_qmv_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                               _ptr(residual)), "vpq_qmv_w4g64_f16")
+    return out
+
+
+def qmm_dense_route_w4g64_f16(w, scales, biases, x, K, N, M, w_deq, expand=True, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=w.device)
+    _check(load().vpq_qmm_dense_route_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                                _ptr(w_deq), 1 if expand else 0), "vpq_qmm_dense_route_w4g64_f16")
     return out
 
 

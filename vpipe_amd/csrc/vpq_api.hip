@@ -481,6 +481,87 @@ int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
   return VPQ_OK;
 }
 
+// ---- IEEE binary16 element type (VPIPE_ELT = half) ----
+
+int vpq_dequant_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                          uint16_t* w_deq, int K, int N)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (w_deq == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (!aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_dequant_f16(reinterpret_cast<hipStream_t>(stream), w, scales, biases, w_deq, K, N));
+}
+
+static int qmv_f16_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                          const uint16_t* x, void* y, bool y_f32, int K, int N, int M, const uint16_t* residual,
+                          int gate_act)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (gate_act != 0 && ((N & 1) != 0 || residual != nullptr)) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2) || (residual != nullptr && !aligned(residual, 2))) {
+    return VPQ_ERR_MISALIGNED;
+  }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y; a.residual = residual;
+  a.K = K; a.N = N; a.M = M; a.y_f32 = y_f32; a.cu_count = g_dev.cu_count;
+  a.gate_act = gate_act;
+  return finish(vpq::launch_qmv_simple_f16(reinterpret_cast<hipStream_t>(stream), a));
+}
+
+int vpq_qmv_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                      const uint16_t* x, uint16_t* y, int K, int N, int M, const uint16_t* residual)
+{
+  return qmv_f16_common(stream, w, scales, biases, x, y, false, K, N, M, residual, 0);
+}
+
+int vpq_qmv_w4g64_f16_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, float* y, int K, int N, int M)
+{
+  return qmv_f16_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr, 0);
+}
+
+int vpq_qmv_gated_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return qmv_f16_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, activation);
+}
+
+int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                  const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                  uint16_t* w_deq, int expand)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (w_deq == nullptr) { return VPQ_ERR_WORKSPACE; }
+  if (M <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (expand != 0) {
+    st = finish(vpq::launch_dequant_f16(hs, w, scales, biases, w_deq, K, N));
+    if (st != VPQ_OK) { return st; }
+  }
+  std::string why;
+  const int rc = vpq::dense_gemm_elt(hs, x, w_deq, y, M, N, K, true, &why);
+  if (rc != 0) {
+    strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
+    g_last_error[sizeof(g_last_error) - 1] = '\0';
+    return rc == -1 ? VPQ_ERR_UNSUPPORTED : VPQ_ERR_DEVICE;
+  }
+  return VPQ_OK;
+}
+
 // Rows up to which the size-based entrances run the GEMV arithmetic in slabs of 16 rows instead of
 // the 256-row GEMM tile: below it the tile kernel has one row of tiles and N/128 workgroups, and
 // its time is its K loop's latency (57 us at 4096->4096 for any M <= 256) against ~10 us per slab.

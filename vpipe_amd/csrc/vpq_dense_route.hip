@@ -22,7 +22,7 @@ namespace {
 // The few rocBLAS declarations this file needs (rocblas/internal/rocblas-types.h, -functions.h).
 typedef void* rb_handle;
 constexpr int kOpNone = 111, kOpTranspose = 112;
-constexpr int kBf16 = 168, kF32 = 151;
+constexpr int kBf16 = 168, kF16 = 150, kF32 = 151;
 typedef int (*rb_create_handle_t)(rb_handle*);
 typedef int (*rb_set_stream_t)(rb_handle, hipStream_t);
 typedef int (*rb_gemm_ex_t)(rb_handle, int, int, int, int, int, const void*, const void*, int, int, const void*, int,
@@ -81,6 +81,14 @@ bool open_locked(Rocblas& r)
 int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,
                     std::string* why)
 {
+  return dense_gemm_elt(st, x, b, y, M, N, K, false, why);
+}
+
+// The same with IEEE binary16 operands and result when f16 is set.
+int dense_gemm_elt(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, bool f16,
+                   std::string* why)
+{
+  const int dt = f16 ? kF16 : kBf16;
   Rocblas& r = rocblas();
   std::lock_guard<std::mutex> lock(r.mu);
   if (!open_locked(r)) {
@@ -91,8 +99,8 @@ int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16
   if (rc == 0) {
     // Column-major view: y^T (N x M, ld N) = b (as K x N, ld K)^T . x (as K x M, ld K).
     const float alpha = 1.0f, beta = 0.0f;
-    rc = r.gemm_ex(r.handle, kOpTranspose, kOpNone, N, M, K, &alpha, b, kBf16, K, x, kBf16, K, &beta, y, kBf16, N, y,
-                   kBf16, N, kF32, 0, 0, 0u);
+    rc = r.gemm_ex(r.handle, kOpTranspose, kOpNone, N, M, K, &alpha, b, dt, K, x, dt, K, &beta, y, dt, N, y, dt, N, kF32, 0,
+                   0, 0u);
   }
   if (rc != 0) {
     if (why) { *why = "rocBLAS status " + std::to_string(rc); }

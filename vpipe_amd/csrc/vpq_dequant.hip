@@ -10,7 +10,8 @@ namespace vpq {
 // significands), so the fused multiply-add below equals the two-step form of
 // gpu-kernels/metal/quant/affine_dequant.metal:45-52 bit for bit.
 // WS: log2 of the words per quantization group (3: group 64; 2: group 32, affine_dequant.metal:196-228).
-template <int WS>
+// F16: scales, biases and the output are IEEE binary16 (the reference's VPIPE_ELT = half build).
+template <int WS, bool F16 = false>
 __global__ __launch_bounds__(256) void dequant_w4_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, uint4* __restrict__ out, int Kw, size_t total_words)
@@ -21,17 +22,17 @@ __global__ __launch_bounds__(256) void dequant_w4_kernel(
     const size_t n = idx / (size_t)Kw;
     const int j = (int)(idx - n * (size_t)Kw);
     const size_t g = n * (size_t)Kg + (size_t)(j >> WS);
-    const float s = bf16_bits_to_f32(scales[g]);
-    const float b = bf16_bits_to_f32(biases[g]);
+    const float s = elt_bits_to_f32<F16>(scales[g]);
+    const float b = elt_bits_to_f32<F16>(biases[g]);
     const uint32_t p = w[idx];
     float v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) { v[i] = fmaf(s, (float)((p >> (4 * i)) & 0xfu), b); }
     uint4 o;
-    o.x = pack_bf16x2(v[0], v[1]);
-    o.y = pack_bf16x2(v[2], v[3]);
-    o.z = pack_bf16x2(v[4], v[5]);
-    o.w = pack_bf16x2(v[6], v[7]);
+    o.x = pack_elt2<F16>(v[0], v[1]);
+    o.y = pack_elt2<F16>(v[2], v[3]);
+    o.z = pack_elt2<F16>(v[4], v[5]);
+    o.w = pack_elt2<F16>(v[6], v[7]);
     out[idx] = o;
   }
 }
@@ -44,6 +45,17 @@ hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* sca
   size_t blocks = (total + 255) / 256;
   if (blocks > 65536 * 4) { blocks = 65536 * 4; }
   return launch_kernel(dequant_w4_kernel<3>, dim3((unsigned)blocks), dim3(256), 0, st, w, scales,
+                       biases, reinterpret_cast<uint4*>(out), Kw, total);
+}
+
+hipError_t launch_dequant_f16(hipStream_t st, const uint32_t* w, const uint16_t* scales,
+                              const uint16_t* biases, uint16_t* out, int K, int N)
+{
+  const int Kw = K / 8;
+  const size_t total = (size_t)N * (size_t)Kw;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536 * 4) { blocks = 65536 * 4; }
+  return launch_kernel(dequant_w4_kernel<3, true>, dim3((unsigned)blocks), dim3(256), 0, st, w, scales,
                        biases, reinterpret_cast<uint4*>(out), Kw, total);
 }
 

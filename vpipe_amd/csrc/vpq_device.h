@@ -57,6 +57,40 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
   return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
 
+// fp32 -> IEEE binary16 bits, round to nearest even (v_cvt_f16_f32).
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f)
+{
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// Element-type helpers of the kernels that exist for both element types of the reference
+// (VPIPE_ELT = bfloat or half): F16 = false bf16, true IEEE binary16.
+template <bool F16>
+__device__ __forceinline__ float elt_bits_to_f32(uint32_t bits16)
+{
+  return F16 ? f16_bits_to_f32(bits16) : bf16_bits_to_f32(bits16);
+}
+template <bool F16>
+__device__ __forceinline__ float elt_lo_to_f32(uint32_t packed)
+{
+  return F16 ? f16_bits_to_f32(packed & 0xffffu) : bf16_lo_to_f32(packed);
+}
+template <bool F16>
+__device__ __forceinline__ float elt_hi_to_f32(uint32_t packed)
+{
+  return F16 ? f16_bits_to_f32(packed >> 16) : bf16_hi_to_f32(packed);
+}
+template <bool F16>
+__device__ __forceinline__ uint32_t f32_to_elt_bits(float f)
+{
+  return F16 ? f32_to_f16_bits(f) : f32_to_bf16_bits(f);
+}
+template <bool F16>
+__device__ __forceinline__ uint32_t pack_elt2(float a, float b)
+{
+  return F16 ? (f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16)) : pack_bf16x2(a, b);
+}
+
 // Gated activation of one (gate, up) pair of fp32 sums, the store expressions of the fused
 // gate|up kernels:
 //   kGateSwiglu  silu(gate) * up, silu(g) = g / (1 + exp(-g))

@@ -164,6 +164,12 @@ hipError_t launch_qmm_tile_splitk(hipStream_t st, const GemmArgs& a, int splits,
 // 0, or -1 (rocBLAS unavailable) / -2 (the call failed) with *why set.
 int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,
                     std::string* why);
+int dense_gemm_elt(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, bool f16,
+                   std::string* why);
+// IEEE binary16 element type (the reference's VPIPE_ELT = half build): dense expansion and the general QMV.
+hipError_t launch_dequant_f16(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                              uint16_t* out, int K, int N);
+hipError_t launch_qmv_simple_f16(hipStream_t st, const QmvArgs& a);
 hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
                            uint16_t* b_f16, int K, int N, float clip);
 hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out, size_t count);

@@ -16,7 +16,7 @@ namespace vpq {
 
 // GS: log2 of the quantization group (6, or 5 for the group-32 packs); SO: scale-only (Q4_0) pack, the
 // bias is -8 * scale and `biases` is never read (affine_qmv.metal:305-342, 252-256).
-template <int MT, bool F32OUT, int GS = 6, bool SO = false>
+template <int MT, bool F32OUT, int GS = 6, bool SO = false, bool F16 = false>
 __global__ __launch_bounds__(256) void qmv_simple_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x, void* __restrict__ y,
@@ -41,8 +41,8 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
     for (int k0 = lane * 32; k0 < K; k0 += kWave * 32) {
       const uint4 c4 = *reinterpret_cast<const uint4*>(wrow + (k0 >> 3));
       const uint32_t codes[4] = {c4.x, c4.y, c4.z, c4.w};
-      const float s = bf16_bits_to_f32(srow[k0 >> GS]);
-      const float b = SO ? -8.0f * s : bf16_bits_to_f32(brow[k0 >> GS]);
+      const float s = elt_bits_to_f32<F16>(srow[k0 >> GS]);
+      const float b = SO ? -8.0f * s : elt_bits_to_f32<F16>(brow[k0 >> GS]);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         float wv[8];
@@ -55,8 +55,8 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
           const uint32_t xd[4] = {x4.x, x4.y, x4.z, x4.w};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            acc[mm] = fmaf(bf16_lo_to_f32(xd[j]), wv[2 * j], acc[mm]);
-            acc[mm] = fmaf(bf16_hi_to_f32(xd[j]), wv[2 * j + 1], acc[mm]);
+            acc[mm] = fmaf(elt_lo_to_f32<F16>(xd[j]), wv[2 * j], acc[mm]);
+            acc[mm] = fmaf(elt_hi_to_f32<F16>(xd[j]), wv[2 * j + 1], acc[mm]);
           }
         }
       }
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
             if (F32OUT) {
               reinterpret_cast<float*>(y)[o] = v;
             } else {
-              reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)f32_to_bf16_bits(v);
+              reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)f32_to_elt_bits<F16>(v);
             }
           }
         }
@@ -97,9 +97,9 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
         if (F32OUT) {
           reinterpret_cast<float*>(y)[o] = total;
         } else {
-          uint32_t v = f32_to_bf16_bits(total);
+          uint32_t v = f32_to_elt_bits<F16>(total);
           if (residual != nullptr) {
-            v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(residual[o]));
+            v = f32_to_elt_bits<F16>(elt_bits_to_f32<F16>(v) + elt_bits_to_f32<F16>(residual[o]));
           }
           reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)v;
         }
@@ -113,6 +113,19 @@ hipError_t launch_qmv_simple(hipStream_t st, const QmvArgs& a)
   const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
 #define VPQ_LAUNCH(MT, F32)                                                                    \
   launch_kernel(qmv_simple_kernel<MT, F32>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
+                a.residual, a.K, a.N, a.M, a.gate_act)
+  if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH(1, true) : VPQ_LAUNCH(1, false); }
+  return a.y_f32 ? VPQ_LAUNCH(4, true) : VPQ_LAUNCH(4, false);
+#undef VPQ_LAUNCH
+}
+
+// IEEE binary16 elements (x, scales, biases, y, residual): the reference's VPIPE_ELT = half build of
+// affine_qmv_w4g64[_add] and the gated forms.
+hipError_t launch_qmv_simple_f16(hipStream_t st, const QmvArgs& a)
+{
+  const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
+#define VPQ_LAUNCH(MT, F32)                                                                                   \
+  launch_kernel(qmv_simple_kernel<MT, F32, 6, false, true>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
                 a.residual, a.K, a.N, a.M, a.gate_act)
   if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH(1, true) : VPQ_LAUNCH(1, false); }
   return a.y_f32 ? VPQ_LAUNCH(4, true) : VPQ_LAUNCH(4, false);

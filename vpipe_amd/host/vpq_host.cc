@@ -114,6 +114,13 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w8g64", QuantKernel::GatherSwiglu, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_gather_qmv_geglu_w8g64", QuantKernel::GatherGeglu, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_gather_down_qmv_w8g64", QuantKernel::GatherDown, QuantFormat::W8G64},
+    // IEEE binary16 build (VPIPE_ELT = half; generative-models/qwen3/metal-qwen-model.cc:771-772: the library
+    // names without the suffix)
+    {"affine_dequant", "affine_dequant_w4g64", QuantKernel::Dequant, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_w4g64", QuantKernel::Qmv, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_w4g64_add", QuantKernel::QmvAdd, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_swiglu_w4g64", QuantKernel::QmvSwiglu, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_geglu_w4g64", QuantKernel::QmvGeglu, QuantFormat::W4G64F16},
     {"affine_dequant_bf16", "affine_dequant_w4g32", QuantKernel::Dequant, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_w4g32", QuantKernel::Qmv, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_w4g32_add", QuantKernel::QmvAdd, QuantFormat::W4G32},
@@ -391,6 +398,8 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
     if (kind == QuantKernel::Dequant) {
       if (!w || !sc || !bi || !buf(3) || !has_int(4) || !has_int(5)) {
         status = VPQ_ERR_NULL_POINTER;
+      } else if (fmt == QuantFormat::W4G64F16) {
+        status = vpq_dequant_w4g64_f16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
       } else if (fmt == QuantFormat::W8G64) {
         status = vpq_dequant_w8g64_bf16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
       } else {
@@ -407,7 +416,14 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
       const uint16_t* residual = kind == QuantKernel::QmvAdd ? static_cast<const uint16_t*>(buf(7)) : nullptr;
       const bool gather = kind == QuantKernel::GatherSwiglu || kind == QuantKernel::GatherGeglu ||
                           kind == QuantKernel::GatherDown;
-      if (fmt == QuantFormat::W8G64 && gather) {
+      if (fmt == QuantFormat::W4G64F16) {
+        if (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu) {
+          status = vpq_qmv_gated_w4g64_f16(st, w, sc, bi, x, y, K, N, M,
+                                           kind == QuantKernel::QmvGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
+        } else {
+          status = vpq_qmv_w4g64_f16(st, w, sc, bi, x, y, K, N, M, residual);
+        }
+      } else if (fmt == QuantFormat::W8G64 && gather) {
         // gpu-kernels/metal/quant/affine_qmv.metal:962-990, 1295-1322, 1524-1552: slot 7 = pair_eid, 8 = top_k
         // (gate|up only), pairs = grid.z; the expert count is what the bound code buffer holds (K bytes a row)
         const bool down = kind == QuantKernel::GatherDown;
