@@ -491,6 +491,49 @@ def main():
             del packs
         out["qmv_w8g64_m1"] = w8
 
+        # 8-bit fused gate|up + SwiGLU (interleaved pack 4096 -> 2 x 12288) and the 8-bit MoE gathers of the
+        # decode block below (hidden 2048, inner 768, 128 experts, top-8); IEEE binary16 elements on the
+        # general kernel (one wavefront per row)
+        w8g = {}
+        K, F = 4096, 12288
+        packs = []
+        for _ in range(3):
+            w = torch.randint(-2 ** 31, 2 ** 31 - 1, (2 * F, K // 4), dtype=torch.int32, device=dev, generator=gen)
+            s = torch.empty((2 * F, K // 64), dtype=torch.float32, device=dev).uniform_(0.0003, 0.0012, generator=gen).bfloat16()
+            packs.append((w, s, (-128.0 * s.float()).bfloat16()))
+        x = torch.randn((1, K), device=dev, generator=gen).bfloat16()
+        y = torch.empty((1, F), dtype=torch.bfloat16, device=dev)
+        us = kernel_us(lambda i: vpipe_amd.qmv_gated_w8g64(*packs[i % 3], x, K, 2 * F, 1, out=y), 6)
+        w8g["gate|up+swiglu 4096->2x12288"] = {"us": round(us, 2),
+                                               "GBps": round((2 * F * K * 17 // 16) / (us * 1e-6) / 1e9, 1)}
+        del packs
+        H8, I8, E8, k8 = 2048, 768, 128, 8
+        gw8 = torch.randint(-2 ** 31, 2 ** 31 - 1, (E8, 2 * I8, H8 // 4), dtype=torch.int32, device=dev, generator=gen)
+        gs8 = torch.empty((E8, 2 * I8, H8 // 64), dtype=torch.float32, device=dev).uniform_(0.0003, 0.0012, generator=gen).bfloat16()
+        gb8 = (-128.0 * gs8.float()).bfloat16()
+        ids8 = [torch.randperm(E8, device=dev, generator=gen)[:k8].to(torch.int32).contiguous() for _ in range(16)]
+        xm8 = torch.randn((1, H8), device=dev, generator=gen).bfloat16()
+        act8 = torch.empty((k8, I8), dtype=torch.bfloat16, device=dev)
+        us = kernel_us(lambda i: vpipe_amd.gather_qmv_gated_w8g64(gw8, gs8, gb8, xm8, H8, 2 * I8, ids8[i % 16], k8, E8, out=act8), 16)
+        w8g["moe gather gate|up+swiglu 2048->2x768, top-8 of 128"] = {
+            "us": round(us, 2), "GBps": round(k8 * (2 * I8 * H8 * 17 // 16) / (us * 1e-6) / 1e9, 1)}
+        del gw8, gs8, gb8
+        out["qmv_w8g64_gated_and_gathered"] = w8g
+
+        f16 = {}
+        for K, N in ((4096, 4096), (4096, 12288)):
+            packs = []
+            for _ in range(4):
+                w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev, generator=gen)
+                s = torch.empty((N, K // 64), dtype=torch.float32, device=dev).uniform_(0.005, 0.02, generator=gen).half()
+                packs.append((w, s, (-8.0 * s.float()).half()))
+            x = torch.randn((1, K), device=dev, generator=gen).half()
+            y = torch.empty((1, N), dtype=torch.float16, device=dev)
+            us = kernel_us(lambda i, x=x, y=y, K=K, N=N: vpipe_amd.qmv_w4g64_f16(*packs[i % 4], x, K, N, 1, out=y), 8)
+            f16["%d->%d" % (K, N)] = {"us": round(us, 2), "GBps": round((N * K * 9 // 16 + 2 * K + 2 * N) / (us * 1e-6) / 1e9, 1)}
+            del packs
+        out["qmv_f16_elements_m1"] = f16
+
         # group-32 twin (GGUF Q4_0 repacked), M=1: affine form (5/8 B per weight) and scale-only form
         # (bias never read: 9/16 B per weight)
         g32 = {}
