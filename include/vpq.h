@@ -482,7 +482,17 @@ int vpq_argmax_combine(vpq_stream_t stream, const float* partials, int32_t* out_
  *                                    gathers over a batched 8-bit pack [E, N, K/4], arguments and
  *                                    conventions of the 4-bit vpq_gather_* entries; a pair is
  *                                    bit-identical to the plain 8-bit call on that expert's slab.
+ *   vpq_gather_qmv_gated_split_bf16  replaces `affine_gather_qmv_swiglu_w4w8g64` and `_w8w4g64`
+ *                                    (:1198-1260; slots 0..2 gate pack, 3..5 up pack, 6:x 7:y 8:K
+ *                                    9:ffn 10:pair_eid 11:top_k): gate and up as SEPARATE batched
+ *                                    packs [E, ffn, ...] of gate_bits / up_bits in {4, 8} each (what a
+ *                                    per-tensor quantizer leaves), y [npair, ffn] = act(gate) * up.
+ *                                    pair_eid NULL: no experts, npair <= 16 rows of x.
  * Requirements as for the 4-bit entries (K % 64 == 0; 16-byte aligned w, x). */
+int vpq_gather_qmv_gated_split_bf16(vpq_stream_t stream, const uint32_t* wg, const uint16_t* sg, const uint16_t* bg,
+                                    int gate_bits, const uint32_t* wu, const uint16_t* su, const uint16_t* bu,
+                                    int up_bits, const uint16_t* x, uint16_t* y, int K, int ffn,
+                                    const int32_t* pair_eid, int npair, int top_k, int n_experts, int activation);
 int vpq_qmv_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                              int activation);

@@ -661,3 +661,28 @@ def test_binary16_library_names(vpq, enc, oracle, dev, D):
     assert np.array_equal(dense.view(torch.int16).cpu().numpy().view(np.uint16), oracle.dequant_f16(w, s, b, K, N))
     assert torch.equal(y, vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, 1))
     assert enc.set_function("affine_qmv", "affine_qmm_steel_w4g64") == 0       # not in that library
+
+
+def test_mixed_width_gather_function_names(vpq, enc, dev, D):
+    # affine_gather_qmv_swiglu_w4w8g64 / _w8w4g64: slots 0..2 gate pack, 3..5 up pack, 6:x 7:y 8:K 9:ffn 10:pair_eid 11:top_k
+    K, ffn, E, top_k, M = 512, 24, 3, 2, 2
+    g4 = [synth.make_weight(ffn, K, 3300 + e) for e in range(E)]
+    u8 = [synth.make_weight8(ffn, K, 3310 + e) for e in range(E)]
+    gd = tuple(f(np.stack([p[i] for p in g4]), dev) for i, f in enumerate((D.u32, D.bf16, D.bf16)))
+    ud = tuple(f(np.stack([p[i] for p in u8]), dev) for i, f in enumerate((D.u32, D.bf16, D.bf16)))
+    xd = D.bf16(synth.make_act(M, K, 3320), dev)
+    eid = torch.tensor([2, 0, 1, 2], dtype=torch.int32, device=dev)
+    for name, gate, up, gb, ub in (("affine_gather_qmv_swiglu_w4w8g64", gd, ud, 4, 8), ("affine_gather_qmv_swiglu_w8w4g64", ud, gd, 8, 4)):
+        y = torch.zeros((M * top_k, ffn), dtype=torch.bfloat16, device=dev)
+        assert enc.set_function("affine_qmv_bf16", name) == 1
+        for i, t in enumerate(gate + up + (xd, y)):
+            enc.set_buffer(i, t)
+        enc.set_constant(8, K)
+        enc.set_constant(9, ffn)
+        enc.set_buffer(10, eid)
+        enc.set_constant(11, top_k)
+        enc.dispatch((32, ffn // 4, M * top_k), (32, 2, 1))
+        ok, why = enc.wait_ok()
+        assert ok, why
+        assert torch.equal(y, vpq.gather_qmv_gated_split(gate, gb, up, ub, xd, K, ffn, eid, top_k, E))
+        assert y.abs().sum() > 0

@@ -157,3 +157,58 @@ def test_w8_gather_ids_out_of_range_and_bad_arguments(vpq, dev, D):
     assert L.vpq_qmv_gated_w8g64_bf16(None, p, p, p, p, p, 64, 8, 1, 5) == -2          # activation
     assert L.vpq_gather_down_qmv_w8g64_bf16(None, p, p, p, p, p, 64, 8, None, 1, 1) == -1
     assert L.vpq_gather_qmv_gated_w8g64_bf16(None, p, p, p, p, p, 64, 8, p, 1, 0, 1, 1) == -2   # top_k 0
+
+
+@pytest.mark.parametrize("activation", [1, 2])
+@pytest.mark.parametrize("gate_bits,up_bits", [(4, 8), (8, 4), (4, 4), (8, 8)])
+def test_gathered_gate_up_at_mixed_widths(vpq, oracle, dev, D, gate_bits, up_bits, activation):
+    # gate and up as separate batched packs, each at its own width: every pair against the oracle's sums of
+    # the two packs of its expert (4-bit: the QMV oracle, 8-bit: its byte twin) through the gated store
+    K, ffn, E, top_k, M = 1024, 40, 4, 2, 3
+    mk = {4: synth.make_weight, 8: synth.make_weight8}
+    gate = [mk[gate_bits](ffn, K, 2900 + 3 * e) for e in range(E)]
+    up = [mk[up_bits](ffn, K, 2950 + 3 * e) for e in range(E)]
+    gs = tuple(np.stack([p[i] for p in gate]) for i in range(3))
+    us = tuple(np.stack([p[i] for p in up]) for i in range(3))
+    x = synth.make_act(M, K, 2990)
+    eid = np.array([3, 0, 1, 1, 2, 3], dtype=np.int32)
+    npair = eid.size
+    gd, ud = stage(D, dev, *gs), stage(D, dev, *us)
+    xd = D.bf16(x, dev)
+    out = parity.Guarded((npair, ffn), torch.bfloat16, dev)
+    vpq.gather_qmv_gated_split(gd, gate_bits, ud, up_bits, xd, K, ffn, torch.from_numpy(eid).to(dev), top_k, E, out=out.view,
+                               activation=activation)
+    torch.cuda.synchronize()
+    out.assert_intact()
+
+    def sums(bits, pack, xr):
+        if bits == 4:
+            return oracle.qmv(pack[0], pack[1], pack[2], xr, K, ffn, 1)[0]
+        return oracle.matmul8(pack[0], pack[1], pack[2], xr, K, ffn, 1, rounded=False)[0]
+    fn = oracle.swiglu if activation == 1 else oracle.geglu
+    want64 = np.empty((npair, ffn))
+    wantb = np.empty((npair, ffn), dtype=np.uint16)
+    for p in range(npair):
+        e, t = int(eid[p]), p // top_k
+        y = np.empty((1, 2 * ffn))
+        y[0, 0::2] = sums(gate_bits, gate[e], x[t:t + 1])[0]
+        y[0, 1::2] = sums(up_bits, up[e], x[t:t + 1])[0]
+        want64[p], wantb[p] = (a[0] for a in fn(y))
+    parity.check_bf16(D.bits(out.view), want64, wantb, mismatch_over_all=activation == 1)
+    # without experts: rows of x against expert 0's packs
+    plain = vpq.gather_qmv_gated_split([t[0] for t in gd], gate_bits, [t[0] for t in ud], up_bits, xd, K, ffn, None, 1, 1,
+                                       activation=activation)
+    again = vpq.gather_qmv_gated_split(gd, gate_bits, ud, up_bits, xd, K, ffn, torch.zeros(M, dtype=torch.int32, device=dev), 1, E,
+                                       activation=activation)
+    assert torch.equal(plain, again)
+
+
+def test_mixed_width_gather_rejects_bad_arguments(vpq, dev):
+    L = vpq.load()
+    p = torch.zeros(4096, dtype=torch.int32, device=dev).data_ptr()
+    f = L.vpq_gather_qmv_gated_split_bf16
+    assert f(None, p, p, p, 4, p, p, p, 8, p, p, 64, 8, p, 1, 1, 1, 1) == 0
+    assert f(None, p, p, p, 5, p, p, p, 8, p, p, 64, 8, p, 1, 1, 1, 1) == -2     # width
+    assert f(None, p, p, p, 4, None, p, p, 8, p, p, 64, 8, p, 1, 1, 1, 1) == -1
+    assert f(None, p, p, p, 4, p, p, p, 8, p, p, 64, 8, None, 17, 1, 1, 1) == -2  # rows without experts
+    assert f(None, p, p, p, 4, p, p, p, 8, p, p, 64, 8, p, 1, 1, 1, 3) == -2     # activation

@@ -72,6 +72,7 @@ SYMBOLS = [
     ("vpq_qmm_dense_route_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_gather_qmv_gated_split_bf16", _i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
     ("vpq_gather_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
     ("vpq_gather_down_qmv_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i]),
     ("vpq_qmv_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -384,6 +385,20 @@ def qmm_splitk_w4g64(w, scales, biases, x, K, N, M, splits=0, ws=None, out=None)
         ws = torch.empty(need, dtype=torch.uint8, device=w.device)
     _check(L.vpq_qmm_splitk_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M, splits,
                                        _ptr(ws), ws.numel()), "vpq_qmm_splitk_w4g64_bf16")
+    return out
+
+
+def gather_qmv_gated_split(gate, gate_bits, up, up_bits, x, K, ffn, pair_eid, top_k, n_experts, out=None,
+                           activation=VPQ_GATE_SWIGLU):
+    """gate, up: (w, scales, biases) of separate (batched) packs at their own widths; pair_eid None: rows of x."""
+    import torch
+    rows = x.shape[0] if pair_eid is None else pair_eid.numel()
+    if out is None:
+        out = torch.empty((rows, ffn), dtype=torch.bfloat16, device=x.device)
+    _check(load().vpq_gather_qmv_gated_split_bf16(_stream(), _ptr(gate[0]), _ptr(gate[1]), _ptr(gate[2]), gate_bits,
+                                                  _ptr(up[0]), _ptr(up[1]), _ptr(up[2]), up_bits, _ptr(x), _ptr(out), K, ffn,
+                                                  _ptr(pair_eid), rows, top_k, n_experts, activation),
+           "vpq_gather_qmv_gated_split_bf16")
     return out
 
 

@@ -254,6 +254,33 @@ static int rows8_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* 
                                       n_experts));
 }
 
+int vpq_gather_qmv_gated_split_bf16(vpq_stream_t stream, const uint32_t* wg, const uint16_t* sg, const uint16_t* bg,
+                                    int gate_bits, const uint32_t* wu, const uint16_t* su, const uint16_t* bu, int up_bits,
+                                    const uint16_t* x, uint16_t* y, int K, int ffn, const int32_t* pair_eid, int npair,
+                                    int top_k, int n_experts, int activation)
+{
+  if (wg == nullptr || sg == nullptr || bg == nullptr || wu == nullptr || su == nullptr || bu == nullptr || x == nullptr ||
+      y == nullptr) {
+    return VPQ_ERR_NULL_POINTER;
+  }
+  if ((gate_bits != 4 && gate_bits != 8) || (up_bits != 4 && up_bits != 8)) { return VPQ_ERR_BAD_SHAPE; }
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (K <= 0 || (K % 64) != 0 || ffn < 1 || npair < 1 || npair > 65535) { return VPQ_ERR_BAD_SHAPE; }
+  if (pair_eid != nullptr ? (top_k < 1 || n_experts < 1) : npair > 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(wg, 16) || !aligned(wu, 16) || !aligned(x, 16) || !aligned(sg, 2) || !aligned(bg, 2) || !aligned(su, 2) ||
+      !aligned(bu, 2) || !aligned(y, 2) || (pair_eid != nullptr && !aligned(pair_eid, 4))) {
+    return VPQ_ERR_MISALIGNED;
+  }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::SplitGateUp a{};
+  a.wg = wg; a.sg = sg; a.bg = bg; a.gate_bits = gate_bits;
+  a.wu = wu; a.su = su; a.bu = bu; a.up_bits = up_bits;
+  a.x = x; a.y = y; a.K = K; a.F = ffn; a.rows = npair; a.gate_act = activation;
+  a.pair_eid = pair_eid; a.x_div = pair_eid != nullptr ? top_k : 1; a.n_experts = n_experts;
+  return finish(vpq::launch_qmv_split_gate_up(reinterpret_cast<hipStream_t>(stream), a));
+}
+
 int vpq_qmv_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                              const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
 {

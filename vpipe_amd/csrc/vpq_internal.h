@@ -88,6 +88,15 @@ hipError_t launch_qmv_rows_g32(hipStream_t st, const QmvArgs& a, bool scale_only
 hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                            uint16_t* out, int K, int N);
 hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a);
+// Mixed-width fused gate/up over separate packs (4 or 8 bits each); rows = pairs (pair_eid) or rows of x.
+struct SplitGateUp {
+  const uint32_t* wg; const uint16_t* sg; const uint16_t* bg; int gate_bits;
+  const uint32_t* wu; const uint16_t* su; const uint16_t* bu; int up_bits;
+  const uint16_t* x; uint16_t* y;
+  int K, F, rows, gate_act;
+  const int* pair_eid; int x_div, n_experts;
+};
+hipError_t launch_qmv_split_gate_up(hipStream_t st, const SplitGateUp& a);
 // 8-bit gated / gathered QMV, one wavefront per output and row (a.gate_act: interleaved gate|up pack);
 // rows = rows of x, or with pair_eid the (token, expert) pairs over a batched pack.
 hipError_t launch_qmv_rows8(hipStream_t st, const QmvArgs& a, int rows, const int* pair_eid, int x_div, int n_experts);

@@ -300,6 +300,90 @@ hipError_t launch_qmv_rows8(hipStream_t st, const QmvArgs& a, int rows, const in
                                     pair_eid, x_div, n_experts);
 }
 
+// Mixed-width fused gate/up (affine_gather_qmv_swiglu_w4w8g64 / _w8w4g64,
+// gpu-kernels/metal/quant/affine_qmv.metal:991-1260): gate and up are SEPARATE packs [E, ffn, ...], each at
+// its own width (4 or 8 bits) as a per-tensor quantizer left them; a wavefront contracts the gate row and
+// the up row of one feature with x and stores act(gate) * up.  Same bytes off DRAM as a uniform layer of
+// those widths, no widened copy.  blockIdx.y: the pair (pair_eid) or the row of x.
+template <int BITS>
+__device__ __forceinline__ float row_dot_wave(const uint32_t* __restrict__ wrow, const uint16_t* __restrict__ srow,
+                                              const uint16_t* __restrict__ brow, const uint16_t* __restrict__ xr, int K,
+                                              int lane)
+{
+  constexpr int VPL = BITS == 4 ? 32 : 16;        // values per lane and pass: one 128-bit load of codes
+  float acc = 0.0f;
+  for (int k0 = lane * VPL; k0 < K; k0 += kWave * VPL) {
+    const uint4 c4 = *reinterpret_cast<const uint4*>(wrow + (BITS == 4 ? (k0 >> 3) : (k0 >> 2)));
+    const uint32_t codes[4] = {c4.x, c4.y, c4.z, c4.w};
+    const float s = bf16_bits_to_f32(srow[k0 >> 6]);
+    const float b = bf16_bits_to_f32(brow[k0 >> 6]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      constexpr int PER = BITS == 4 ? 8 : 4;      // values per code word
+      const uint4* xp = reinterpret_cast<const uint4*>(xr + k0 + PER * i);
+      if (BITS == 4) {
+        const uint4 x4 = xp[0];
+        const uint32_t xd[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc = fmaf(bf16_lo_to_f32(xd[j]), fmaf(s, (float)((codes[i] >> (8 * j)) & 0xfu), b), acc);
+          acc = fmaf(bf16_hi_to_f32(xd[j]), fmaf(s, (float)((codes[i] >> (8 * j + 4)) & 0xfu), b), acc);
+        }
+      } else {
+        const uint2 x2 = *reinterpret_cast<const uint2*>(xr + k0 + 4 * i);
+        acc = fmaf(bf16_lo_to_f32(x2.x), fmaf(s, (float)(codes[i] & 0xffu), b), acc);
+        acc = fmaf(bf16_hi_to_f32(x2.x), fmaf(s, (float)((codes[i] >> 8) & 0xffu), b), acc);
+        acc = fmaf(bf16_lo_to_f32(x2.y), fmaf(s, (float)((codes[i] >> 16) & 0xffu), b), acc);
+        acc = fmaf(bf16_hi_to_f32(x2.y), fmaf(s, (float)(codes[i] >> 24), b), acc);
+      }
+    }
+  }
+  return wave_sum(acc);
+}
+
+template <int GB, int UB>
+__global__ __launch_bounds__(256) void qmv_split_gate_up_kernel(
+    const uint32_t* __restrict__ wg, const uint16_t* __restrict__ sg, const uint16_t* __restrict__ bg,
+    const uint32_t* __restrict__ wu, const uint16_t* __restrict__ su, const uint16_t* __restrict__ bu,
+    const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int K, int F, int gate_act,
+    const int* __restrict__ pair_eid, int x_div, int n_experts)
+{
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int f = blockIdx.x * 4 + wave;
+  if (f >= F) { return; }  // wave-uniform; no barrier in this kernel
+  const int m = blockIdx.y;
+  const int Kg = K >> 6;
+  const size_t gw = (size_t)(K >> (GB == 4 ? 3 : 2)), uw = (size_t)(K >> (UB == 4 ? 3 : 2));   // words per row
+  int xrow = m;
+  size_t e = 0;
+  if (pair_eid != nullptr) {
+    const int id = pair_eid[m];
+    if (id < 0 || id >= n_experts) {
+      if (lane == 0) { y[(size_t)m * F + f] = 0; }
+      return;
+    }
+    e = (size_t)id;
+    xrow = m / x_div;
+  }
+  const size_t row = e * (size_t)F + (size_t)f;
+  const uint16_t* xr = x + (size_t)xrow * K;
+  const float g = row_dot_wave<GB>(wg + row * gw, sg + row * Kg, bg + row * Kg, xr, K, lane);
+  const float u = row_dot_wave<UB>(wu + row * uw, su + row * Kg, bu + row * Kg, xr, K, lane);
+  if (lane == 0) { y[(size_t)m * F + f] = (uint16_t)f32_to_bf16_bits(gated_f32(gate_act, g, u)); }
+}
+
+hipError_t launch_qmv_split_gate_up(hipStream_t st, const SplitGateUp& a)
+{
+  const dim3 grid((unsigned)((a.F + 3) / 4), (unsigned)a.rows), block(256);
+#define VPQ_SPLIT(GB, UB)                                                                                       \
+  launch_kernel(qmv_split_gate_up_kernel<GB, UB>, grid, block, 0, st, a.wg, a.sg, a.bg, a.wu, a.su, a.bu, a.x, a.y, a.K, \
+                a.F, a.gate_act, a.pair_eid, a.x_div, a.n_experts)
+  if (a.gate_bits == 4) { return a.up_bits == 4 ? VPQ_SPLIT(4, 4) : VPQ_SPLIT(4, 8); }
+  return a.up_bits == 4 ? VPQ_SPLIT(8, 4) : VPQ_SPLIT(8, 8);
+#undef VPQ_SPLIT
+}
+
 hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a)
 {
   const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);

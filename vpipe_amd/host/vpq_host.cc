@@ -100,6 +100,8 @@ const FnEntry kFunctions[] = {
     {"affine_qmm_steel_bf16", "affine_qmm_grouped_swiglu_w4g64", QuantKernel::GroupedSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_grouped_geglu_w4g64", QuantKernel::GroupedGeglu},
     {"affine_qmm_steel_bf16", "affine_qmm_grouped_w4g64", QuantKernel::GroupedDown},
+    {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w4w8g64", QuantKernel::GatherSplit48},
+    {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w8w4g64", QuantKernel::GatherSplit84},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64", QuantKernel::QmmSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm128", QuantKernel::QmmSwiglu},
@@ -451,6 +453,26 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
       } else {
         status = vpq_qmv_w4g32_bf16(st, w, sc, q40 ? nullptr : bi, x, y, K, N, M, residual, q40 ? 1 : 0);
       }
+    }
+  } else if (kind == QuantKernel::GatherSplit48 || kind == QuantKernel::GatherSplit84) {
+    // gpu-kernels/metal/quant/affine_qmv.metal:1198-1260; the expert count is what the gate code buffer holds
+    bool have = has_int(8) && has_int(9) && has_int(11) && buf(10);
+    for (unsigned i = 0; i < 8; ++i) { have = have && buf(i); }
+    if (!have) {
+      status = VPQ_ERR_NULL_POINTER;
+    } else if (ival(8) <= 0 || ival(8) % 64 != 0 || ival(9) <= 0) {
+      status = VPQ_ERR_BAD_SHAPE;
+    } else {
+      const int K = ival(8), F = ival(9);
+      const int gbits = kind == QuantKernel::GatherSplit48 ? 4 : 8, ubits = 12 - gbits;
+      const std::size_t slab = static_cast<std::size_t>(F) * static_cast<std::size_t>(K) * gbits / 8;
+      const std::size_t experts = _slots[0].bytes / slab;
+      const int E = experts > 0x7fffffffu ? 0x7fffffff : static_cast<int>(experts);
+      status = vpq_gather_qmv_gated_split_bf16(
+          st, static_cast<const uint32_t*>(buf(0)), static_cast<const uint16_t*>(buf(1)), static_cast<const uint16_t*>(buf(2)),
+          gbits, static_cast<const uint32_t*>(buf(3)), static_cast<const uint16_t*>(buf(4)),
+          static_cast<const uint16_t*>(buf(5)), ubits, static_cast<const uint16_t*>(buf(6)), static_cast<uint16_t*>(buf(7)), K, F,
+          static_cast<const int32_t*>(buf(10)), static_cast<int>(grid.z), ival(11), E, VPQ_GATE_SWIGLU);
     }
   } else if (kind == QuantKernel::Dequant) {
     // slots 0:w 1:scales 2:biases 3:w_deq 4:K 5:N
