@@ -482,6 +482,14 @@ int vpq_argmax_combine(vpq_stream_t stream, const float* partials, int32_t* out_
  *                                    gathers over a batched 8-bit pack [E, N, K/4], arguments and
  *                                    conventions of the 4-bit vpq_gather_* entries; a pair is
  *                                    bit-identical to the plain 8-bit call on that expert's slab.
+ *   vpq_qmm_w8g64_bf16, vpq_qmm_gated_w8g64_bf16   the fused tile kernel with byte codes: replace
+ *                                    `affine_qmm_steel_w8g64[_bm64|_bm128]` (affine_qmm_steel.metal:1601-1672)
+ *                                    and `affine_qmm_swiglu_w8g64*` / `affine_qmm_geglu_w8g64` (:1700-1890);
+ *                                    arguments as vpq_qmm_w4g64_bf16 (no adapter) / vpq_qmm_gated_w4g64_bf16.
+ *   vpq_qmm_grouped_gated_w8g64_bf16, vpq_qmm_grouped_down_w8g64_bf16   the expert-sorted MoE GEMMs over a
+ *                                    batched 8-bit pack: replace `affine_qmm_grouped_swiglu_w8g64`,
+ *                                    `affine_qmm_grouped_geglu_w8g64`, `affine_qmm_grouped_w8g64` (:1069-1090,
+ *                                    1290-1312, 1341-1366); arguments as the 4-bit vpq_qmm_grouped_* entries.
  *   vpq_gather_qmv_gated_split_bf16  replaces `affine_gather_qmv_swiglu_w4w8g64` and `_w8w4g64`
  *                                    (:1198-1260; slots 0..2 gate pack, 3..5 up pack, 6:x 7:y 8:K
  *                                    9:ffn 10:pair_eid 11:top_k): gate and up as SEPARATE batched
@@ -493,6 +501,19 @@ int vpq_gather_qmv_gated_split_bf16(vpq_stream_t stream, const uint32_t* wg, con
                                     int gate_bits, const uint32_t* wu, const uint16_t* su, const uint16_t* bu,
                                     int up_bits, const uint16_t* x, uint16_t* y, int K, int ffn,
                                     const int32_t* pair_eid, int npair, int top_k, int n_experts, int activation);
+int vpq_qmm_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M);
+int vpq_qmm_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                             int out_stride, int out_off, int activation);
+int vpq_qmm_grouped_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                     int npad, const int32_t* tile2e, const int32_t* srow, int n_experts,
+                                     int rows_x, int activation);
+int vpq_qmm_grouped_down_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                    int npad, const int32_t* tile2e, const int32_t* sdst, int n_experts,
+                                    int rows_y);
 int vpq_qmv_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                              int activation);

@@ -220,7 +220,7 @@ def moe_sort_pairs(eid, top_k, E, block_rows, max_tiles):
     return t2e, srow, sdst, used
 
 
-def qmm_grouped(w, s, b, x, K, N, block_rows, tile2e, srow=None, sdst=None, rows_y=None):
+def qmm_grouped(w, s, b, x, K, N, block_rows, tile2e, srow=None, sdst=None, rows_y=None, bits=4):
     """Grouped expert GEMM over sorted slots -> (y64, y_bf16).  With srow (gate|up) the outputs are
     [npad, N] in slot order; with sdst (down) they are [rows_y, N] in pair order (rows no slot
     writes stay zero)."""
@@ -230,7 +230,7 @@ def qmm_grouped(w, s, b, x, K, N, block_rows, tile2e, srow=None, sdst=None, rows
     rows = npad if sdst is None else rows_y
     y64 = np.zeros((rows, N), dtype=np.float64)
     yb = np.zeros((rows, N), dtype=np.uint16)
-    lib().vpo_qmm_grouped_w4g64(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y64, _f64p),
+    (lib().vpo_qmm_grouped_w4g64 if bits == 4 else lib().vpo_qmm_grouped_w8g64)(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y64, _f64p),
                                 _p(yb, _u16p), K, N, npad, block_rows, _p(tile2e, _i32p), _p(srow, _i32p),
                                 _p(sdst, _i32p))
     return y64, yb

@@ -139,6 +139,7 @@ void vpo_f16_to_f32_array(const uint16_t* in, float* out, size_t n)
   for (size_t i = 0; i < n; ++i) { out[i] = vpo_f16_to_f32(in[i]); }
 }
 
+static inline unsigned code8(const uint32_t* w, size_t n, int Kw, int k);
 static inline unsigned nibble(const uint32_t* w, size_t n, int Kw, int k)
 {
   return (w[n * (size_t)Kw + (size_t)(k >> 3)] >> (4 * (k & 7))) & 0xfu;
@@ -562,12 +563,12 @@ int vpo_moe_sort_pairs(const int32_t* eid, int np, int top_k, int E, int block_r
  *   sdst != NULL (down): x row of slot i is x[i]; the sums go to y64[sdst[i], :] and their
  *     bf16 rounding to y_bf16[sdst[i], :] (slots with sdst < 0 write nothing).
  * Arithmetic of vpo_qmm_w4g64: bf16-rounded weights, contraction in double. */
-void vpo_qmm_grouped_w4g64(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                           const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int npad,
-                           int block_rows, const int32_t* tile2e, const int32_t* srow,
-                           const int32_t* sdst)
+static void qmm_grouped_bits(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int npad,
+                            int block_rows, const int32_t* tile2e, const int32_t* srow,
+                            const int32_t* sdst, int bits)
 {
-  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  const int Kw = bits == 4 ? K / 8 : K / 4, Kg = K / VPO_GROUP;
   float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
   for (int t = 0; t < npad / block_rows; ++t) {
     const int e = tile2e[t];
@@ -579,7 +580,7 @@ void vpo_qmm_grouped_w4g64(const uint32_t* w, const uint16_t* scales, const uint
       for (int k = 0; k < K; ++k) {
         const float s = vpo_bf16_to_f32(se[n * Kg + k / VPO_GROUP]);
         const float b = vpo_bf16_to_f32(be[n * Kg + k / VPO_GROUP]);
-        const float sq = s * (float)nibble(we, n, Kw, k);
+        const float sq = s * (float)(bits == 4 ? nibble(we, n, Kw, k) : code8(we, n, Kw, k));
         wrow[k] = vpo_bf16_to_f32(vpo_f32_to_bf16(sq + b));
       }
       for (int i = t * block_rows; i < (t + 1) * block_rows; ++i) {
@@ -602,6 +603,25 @@ void vpo_qmm_grouped_w4g64(const uint32_t* w, const uint16_t* scales, const uint
     }
   }
   free(wrow);
+}
+
+void vpo_qmm_grouped_w4g64(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int npad,
+                           int block_rows, const int32_t* tile2e, const int32_t* srow,
+                           const int32_t* sdst)
+{
+  qmm_grouped_bits(w, scales, biases, x, y64, y_bf16, K, N, npad, block_rows, tile2e, srow, sdst, 4);
+}
+
+/* 8-bit twins (affine_qmm_grouped_w8g64, affine_qmm_grouped_swiglu_w8g64, affine_qmm_grouped_geglu_w8g64,
+ * gpu-kernels/metal/quant/affine_qmm_steel.metal:1069-1090, 1290-1312, 1341-1366: "fully bit-parameterized"):
+ * one byte per value, the batched pack [E, N, K/4]. */
+void vpo_qmm_grouped_w8g64(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int npad,
+                           int block_rows, const int32_t* tile2e, const int32_t* srow,
+                           const int32_t* sdst)
+{
+  qmm_grouped_bits(w, scales, biases, x, y64, y_bf16, K, N, npad, block_rows, tile2e, srow, sdst, 8);
 }
 
 /* ---- a12: the packer --------------------------------------------------- */

@@ -686,3 +686,48 @@ def test_mixed_width_gather_function_names(vpq, enc, dev, D):
         assert ok, why
         assert torch.equal(y, vpq.gather_qmv_gated_split(gate, gb, up, ub, xd, K, ffn, eid, top_k, E))
         assert y.abs().sum() > 0
+
+
+def test_eight_bit_gemm_function_names(vpq, enc, dev, D):
+    # affine_qmm_steel_w8g64 (slot 7 = M), affine_qmm_swiglu_w8g64, and the 8-bit expert-sorted pair
+    # (slot 7 = npad, 8 = tile2e, 9 = srow / sdst): the encoder's results are the C ABI's
+    K, ffn, H, E, top_k, T = 512, 64, 96, 3, 2, 40
+    packs = []
+    for e in range(E):
+        g, u = synth.make_weight8(ffn, K, 3900 + 2 * e), synth.make_weight8(ffn, K, 3901 + 2 * e)
+        packs.append(tuple(np.stack([a, b], axis=1).reshape((2 * ffn,) + a.shape[1:]) for a, b in zip(g, u)))
+    gu_d = tuple(f(np.stack([p[i] for p in packs]), dev) for i, f in enumerate((D.u32, D.bf16, D.bf16)))
+    dn = [synth.make_weight8(H, ffn, 3950 + e) for e in range(E)]
+    dn_d = tuple(f(np.stack([p[i] for p in dn]), dev) for i, f in enumerate((D.u32, D.bf16, D.bf16)))
+    xd = D.bf16(synth.make_act(T, K, 3960), dev)
+    eid = torch.from_numpy(np.random.default_rng(3961).integers(0, E, size=T * top_k, dtype=np.int32)).to(dev)
+    t2e, srow, sdst, _ = vpq.moe_sort_pairs(eid, top_k, E)
+    npad = srow.numel()
+    y = torch.zeros((T, 2 * ffn), dtype=torch.bfloat16, device=dev)
+    yg = torch.zeros((T, ffn), dtype=torch.bfloat16, device=dev)
+    gact = torch.zeros((npad, ffn), dtype=torch.bfloat16, device=dev)
+    part = torch.zeros((T * top_k, H), dtype=torch.bfloat16, device=dev)
+    one = tuple(t[1] for t in gu_d)                       # expert 1's slab as a plain pack
+    encode_linear(enc, "affine_qmm_steel_bf16", "affine_qmm_steel_w8g64", *one, xd, y, K, 2 * ffn, M=T, grid=(2 * ffn, T, 2), tg=(32, 2, 2))
+    encode_linear(enc, "affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64", *one, xd, yg, K, 2 * ffn, M=T, grid=(2 * ffn, T, 2), tg=(32, 2, 2))
+    for name, pack, src, dst, kk, nn, idx in (("affine_qmm_grouped_swiglu_w8g64", gu_d, xd, gact, K, 2 * ffn, srow),
+                                               ("affine_qmm_grouped_w8g64", dn_d, gact, part, ffn, H, sdst)):
+        assert enc.set_function("affine_qmm_steel_bf16", name) == 1
+        for i, t in enumerate(pack + (src, dst)):
+            enc.set_buffer(i, t)
+        enc.set_constant(5, kk)
+        enc.set_constant(6, nn)
+        enc.set_constant(7, npad)
+        enc.set_buffer(8, t2e)
+        enc.set_buffer(9, idx)
+        enc.dispatch((((nn + 31) // 32) * 32, ((npad + 31) // 32) * 2, 2), (32, 2, 2))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert torch.equal(y, vpq.qmm_w8g64(*one, xd, K, 2 * ffn, T))
+    assert torch.equal(yg, vpq.qmm_w8g64(*one, xd, K, 2 * ffn, T, activation=1))
+    want_act = vpq.qmm_grouped_gated_w8g64(*gu_d, xd, K, 2 * ffn, t2e, srow, E)
+    live = (srow >= 0)
+    assert torch.equal(gact[live], want_act[live])
+    want_part = torch.zeros_like(part)
+    vpq.qmm_grouped_down_w8g64(*dn_d, gact, ffn, H, t2e, sdst, E, out=want_part)
+    assert torch.equal(part, want_part) and part.abs().sum() > 0

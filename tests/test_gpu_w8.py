@@ -212,3 +212,73 @@ def test_mixed_width_gather_rejects_bad_arguments(vpq, dev):
     assert f(None, p, p, p, 4, None, p, p, 8, p, p, 64, 8, p, 1, 1, 1, 1) == -1
     assert f(None, p, p, p, 4, p, p, p, 8, p, p, 64, 8, None, 17, 1, 1, 1) == -2  # rows without experts
     assert f(None, p, p, p, 4, p, p, p, 8, p, p, 64, 8, p, 1, 1, 1, 3) == -2     # activation
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (300, 200, 128), (257, 129, 512), (40, 384, 1024), (520, 260, 1536)])
+def test_qmm_w8_fused_tile_kernel(vpq, oracle, dev, D, M, N, K):
+    # byte codes through the fused tile kernel: the GEMM oracle (bf16-rounded weights), and the expansion the
+    # dequant-once route makes holds the same weights
+    w, s, b = synth.make_weight8(N, K, 3400 + M)
+    x = synth.make_act(M, K, 3401 + M)
+    y64, yb = oracle.matmul8(w, s, b, x, K, N, M, rounded=True)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_w8g64(wd, sd, bd, xd, K, N, M, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_bf16(D.bits(out.view), y64, yb)
+
+
+@pytest.mark.parametrize("activation", [1, 2])
+def test_qmm_w8_gated_store(vpq, oracle, dev, D, activation):
+    K, ffn, M = 512, 100, 270
+    w, s, b = interleaved8(ffn, K, 3500)
+    x = synth.make_act(M, K, 3501)
+    y64, _ = oracle.matmul8(w, s, b, x, K, 2 * ffn, M, rounded=True)
+    want64, wantb = (oracle.swiglu if activation == 1 else oracle.geglu)(y64)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    got = vpq.qmm_w8g64(wd, sd, bd, xd, K, 2 * ffn, M, activation=activation)
+    parity.check_bf16(D.bits(got), want64, wantb, mismatch_over_all=activation == 1)
+
+
+@pytest.mark.parametrize("K,inner,H,E,T,top_k", [(512, 128, 300, 5, 150, 2), (1024, 64, 100, 4, 90, 2), (576, 96, 512, 3, 60, 1)])
+def test_grouped_expert_gemms_w8(vpq, oracle, dev, D, K, inner, H, E, T, top_k):
+    # the expert-sorted prefill GEMMs over 8-bit experts (K = 576: the per-step scale loads, K % 512 == 0: the
+    # ring; N <= 128: the narrow tile), against the oracle on the same slots; a slot equals the plain fused
+    # 8-bit GEMM on its row and slab bit for bit
+    B = vpq.grouped_block_rows()
+    Kd = 64 * ((inner + 63) // 64)
+    gu = [interleaved8(inner, K, 3600 + 5 * e) for e in range(E)]
+    dn = [synth.make_weight8(H, Kd, 3700 + e) for e in range(E)]
+    guw, gus, gub = (np.stack([p[i] for p in gu]) for i in range(3))
+    dw, ds, db = (np.stack([p[i] for p in dn]) for i in range(3))
+    x = synth.make_act(T, K, 3800)
+    eid = np.random.default_rng(3801 + K).integers(0, E, size=T * top_k, dtype=np.int32)
+    npair = eid.size
+    t2e_d, srow_d, sdst_d, ntiles_d = vpq.moe_sort_pairs(torch.from_numpy(eid).to(dev), top_k, E)
+    t2e, srow, sdst = (o.cpu().numpy() for o in (t2e_d, srow_d, sdst_d))
+    npad, used = srow.size, int(ntiles_d.cpu()[0])
+    guwd, gusd, gubd, xd = stage(D, dev, guw, gus, gub, x)
+    act = parity.Guarded((npad, inner), torch.bfloat16, dev)
+    vpq.qmm_grouped_gated_w8g64(guwd, gusd, gubd, xd, K, 2 * inner, t2e_d, srow_d, E, out=act.view)
+    torch.cuda.synchronize()
+    act.assert_intact()
+    got = D.bits(act.view)
+    y64, _ = oracle.qmm_grouped(guw, gus, gub, x, K, 2 * inner, B, t2e, srow=srow, bits=8)
+    want64, wantb = oracle.swiglu(y64[:used * B])
+    live = srow[:used * B] >= 0
+    assert not got[:used * B][~live].any()
+    parity.check_bf16(got[:used * B][live], want64[live], wantb[live])
+    for e in np.unique(eid):
+        slots = np.nonzero((t2e[np.arange(npad) // B] == e) & (srow >= 0))[0]
+        rows = torch.from_numpy(srow[slots].astype(np.int64)).to(dev)
+        plain = vpq.qmm_w8g64(guwd[e], gusd[e], gubd[e], xd[rows].contiguous(), K, 2 * inner, len(slots), activation=1)
+        assert np.array_equal(got[slots], D.bits(plain)), "expert %d" % e
+    xs = synth.make_act(npad, Kd, 3802)
+    dwd, dsd, dbd, xsd = stage(D, dev, dw, ds, db, xs)
+    part = parity.Guarded((npair, H), torch.bfloat16, dev)
+    vpq.qmm_grouped_down_w8g64(dwd, dsd, dbd, xsd, Kd, H, t2e_d, sdst_d, E, out=part.view)
+    torch.cuda.synchronize()
+    part.assert_intact()
+    d64, dbits = oracle.qmm_grouped(dw, ds, db, xs, Kd, H, B, t2e, sdst=sdst, rows_y=npair, bits=8)
+    parity.check_bf16(D.bits(part.view), d64, dbits)

@@ -72,6 +72,10 @@ SYMBOLS = [
     ("vpq_qmm_dense_route_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_qmm_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_qmm_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
+    ("vpq_qmm_grouped_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _i]),
+    ("vpq_qmm_grouped_down_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
     ("vpq_gather_qmv_gated_split_bf16", _i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
     ("vpq_gather_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
     ("vpq_gather_down_qmv_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i]),
@@ -399,6 +403,35 @@ def gather_qmv_gated_split(gate, gate_bits, up, up_bits, x, K, ffn, pair_eid, to
                                                   _ptr(up[0]), _ptr(up[1]), _ptr(up[2]), up_bits, _ptr(x), _ptr(out), K, ffn,
                                                   _ptr(pair_eid), rows, top_k, n_experts, activation),
            "vpq_gather_qmv_gated_split_bf16")
+    return out
+
+
+def qmm_w8g64(w, scales, biases, x, K, N, M, out=None, activation=0, out_stride=0, out_off=0):
+    """Fused 8-bit GEMM on the tile kernel; activation != 0: interleaved gate|up pack -> [M, N/2]."""
+    import torch
+    if out is None:
+        out = torch.empty((M, N // 2 if activation else N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_gated_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                           out_stride, out_off, activation), "vpq_qmm_gated_w8g64_bf16")
+    return out
+
+
+def qmm_grouped_gated_w8g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out=None, activation=VPQ_GATE_SWIGLU):
+    import torch
+    npad = srow.numel()
+    if out is None:
+        out = torch.empty((npad, N // 2), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_grouped_gated_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                   npad, _ptr(tile2e), _ptr(srow), n_experts, x.shape[0], activation),
+           "vpq_qmm_grouped_gated_w8g64_bf16")
+    return out
+
+
+def qmm_grouped_down_w8g64(w, scales, biases, x, K, N, tile2e, sdst, n_experts, out):
+    npad = sdst.numel()
+    _check(load().vpq_qmm_grouped_down_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                  npad, _ptr(tile2e), _ptr(sdst), n_experts, out.shape[0]),
+           "vpq_qmm_grouped_down_w8g64_bf16")
     return out
 
 

@@ -812,7 +812,7 @@ namespace {
 
 int grouped_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                    const uint16_t* x, uint16_t* y, int K, int N, int npad, const int32_t* tile2e,
-                   const int32_t* srow, const int32_t* sdst, int n_experts, int rows, int gate_act)
+                   const int32_t* srow, const int32_t* sdst, int n_experts, int rows, int gate_act, int bits = 4)
 {
   int st = check_pack(w, scales, biases, K, N);
   if (st != VPQ_OK) { return st; }
@@ -837,6 +837,7 @@ int grouped_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scale
   g.K = K; g.N = N; g.M = npad; g.lora_t = nullptr; g.lora_b = nullptr; g.r = 0;
   g.cu_count = g_dev.cu_count;
   g.gate_act = gate_act; g.out_stride = N / 2; g.out_off = 0;
+  g.bits = bits;
   vpq::GroupedArgs ga{};
   ga.tile2e = tile2e; ga.srow = srow; ga.sdst = sdst;
   ga.n_experts = n_experts;
@@ -866,6 +867,59 @@ int vpq_qmm_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, cons
   if (sdst == nullptr) { return VPQ_ERR_NULL_POINTER; }
   return grouped_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, nullptr, sdst, n_experts, rows_y, 0);
 }
+
+// ---- 8-bit twins on the fused tile kernel ----
+
+int vpq_qmm_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int out_stride, int out_off, int activation)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (activation != 0 && activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (M <= 0 || out_off < 0 || (activation != 0 && (N & 1) != 0)) { return VPQ_ERR_BAD_SHAPE; }
+  if (activation == 0 && (out_stride != 0 || out_off != 0)) { return VPQ_ERR_BAD_SHAPE; }
+  if (out_stride > 0 && out_off + N / 2 > out_stride) { return VPQ_ERR_BAD_SHAPE; }
+  if (out_stride <= 0 && out_off != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if ((long long)M * (long long)K * 2 >= 4000000000LL) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::GemmArgs g{};
+  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
+  g.K = K; g.N = N; g.M = M; g.lora_t = nullptr; g.lora_b = nullptr; g.r = 0;
+  g.cu_count = g_dev.cu_count;
+  g.gate_act = activation; g.out_stride = out_stride; g.out_off = out_off;
+  g.bits = 8;
+  return finish(vpq::launch_qmm_tile(reinterpret_cast<hipStream_t>(stream), g));
+}
+
+int vpq_qmm_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                       const uint16_t* x, uint16_t* y, int K, int N, int M)
+{
+  return vpq_qmm_gated_w8g64_bf16(stream, w, scales, biases, x, y, K, N, M, 0, 0, 0);
+}
+
+int vpq_qmm_grouped_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                     int npad, const int32_t* tile2e, const int32_t* srow, int n_experts,
+                                     int rows_x, int activation)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (srow == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  return grouped_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, srow, nullptr, n_experts, rows_x,
+                        activation, 8);
+}
+
+int vpq_qmm_grouped_down_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                    int npad, const int32_t* tile2e, const int32_t* sdst, int n_experts,
+                                    int rows_y)
+{
+  if (sdst == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  return grouped_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, nullptr, sdst, n_experts, rows_y, 0, 8);
+}
+
 
 namespace {
 

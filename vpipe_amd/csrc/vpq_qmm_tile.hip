@@ -120,30 +120,51 @@ __device__ __forceinline__ void wg_barrier()
   asm volatile("" ::: "memory");
 }
 
-// One step's codes (32 nibbles), scale and bias of a producer thread, requested by load
-// instructions the compiler does not track: the owner waits for them with wait_codes().
-struct CodeRegs {
+// One step's codes (32 values: 16 bytes at 4 bits, 2 x 16 at 8 bits), scale and bias of a producer
+// thread, requested by load instructions the compiler does not track: the owner waits for them with
+// wait_codes().
+template <int BITS>
+struct CodeRegsT {
   u32x4 codes;
   uint32_t s_bits, b_bits;
 };
+template <>
+struct CodeRegsT<8> {
+  u32x4 codes, codes2;
+  uint32_t s_bits, b_bits;
+};
+using CodeRegs = CodeRegsT<4>;
 
-__device__ __forceinline__ void request_codes(CodeRegs& r, const uint8_t* codes, const uint16_t* s,
-                                              const uint16_t* b)
+__device__ __forceinline__ void request_code_words(CodeRegsT<4>& r, const uint8_t* codes)
 {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.codes) : "v"(codes) : "memory");
+}
+__device__ __forceinline__ void request_code_words(CodeRegsT<8>& r, const uint8_t* codes)
+{
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.codes) : "v"(codes) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(r.codes2) : "v"(codes) : "memory");
+}
+
+template <int BITS>
+__device__ __forceinline__ void request_codes(CodeRegsT<BITS>& r, const uint8_t* codes, const uint16_t* s,
+                                              const uint16_t* b)
+{
+  request_code_words(r, codes);
   asm volatile("global_load_ushort %0, %1, off" : "=v"(r.s_bits) : "v"(s) : "memory");
   asm volatile("global_load_ushort %0, %1, off" : "=v"(r.b_bits) : "v"(b) : "memory");
 }
 
 // The codes alone (scale and bias come from the LDS ring, see SBR).
-__device__ __forceinline__ void request_codes_only(CodeRegs& r, const uint8_t* codes)
+template <int BITS>
+__device__ __forceinline__ void request_codes_only(CodeRegsT<BITS>& r, const uint8_t* codes)
 {
-  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r.codes) : "v"(codes) : "memory");
+  request_code_words(r, codes);
 }
 
 // Scale and bias of one row and step from the ring, as loads the compiler does not track (it would order
 // them after every direct-to-LDS load of the wavefront); the caller's LDS queue is empty before them.
-__device__ __forceinline__ void read_scale_bias(CodeRegs& r, uint32_t s_addr, uint32_t b_addr)
+template <int BITS>
+__device__ __forceinline__ void read_scale_bias(CodeRegsT<BITS>& r, uint32_t s_addr, uint32_t b_addr)
 {
   asm volatile("ds_read_u16 %0, %1" : "=v"(r.s_bits) : "v"(s_addr) : "memory");
   asm volatile("ds_read_u16 %0, %1" : "=v"(r.b_bits) : "v"(b_addr) : "memory");
@@ -165,23 +186,29 @@ __device__ __forceinline__ void dma16_raw(uint32_t lds_dst, const uint8_t* src)
 // Waits until at most YOUNGER vector-memory requests issued after r's are outstanding; the
 // registers pass through the statement so that no use of them can be moved above the wait.
 template <int YOUNGER>
-__device__ __forceinline__ void wait_codes(CodeRegs& r)
+__device__ __forceinline__ void wait_codes(CodeRegsT<4>& r)
 {
   asm volatile("s_waitcnt vmcnt(%3)" : "+v"(r.codes), "+v"(r.s_bits), "+v"(r.b_bits) : "n"(YOUNGER) : "memory");
 }
-
-// The same for the one or two register sets of a step (requests retire in order: YOUNGER counts
-// from the last of them).
 template <int YOUNGER>
-__device__ __forceinline__ void wait_codes(CodeRegs (&r)[1]) { wait_codes<YOUNGER>(r[0]); }
-
-template <int YOUNGER>
-__device__ __forceinline__ void wait_codes(CodeRegs (&r)[2])
+__device__ __forceinline__ void wait_codes(CodeRegsT<8>& r)
 {
-  asm volatile("s_waitcnt vmcnt(%6)"
-               : "+v"(r[0].codes), "+v"(r[0].s_bits), "+v"(r[0].b_bits), "+v"(r[1].codes), "+v"(r[1].s_bits), "+v"(r[1].b_bits)
-               : "n"(YOUNGER)
-               : "memory");
+  asm volatile("s_waitcnt vmcnt(%4)" : "+v"(r.codes), "+v"(r.codes2), "+v"(r.s_bits), "+v"(r.b_bits) : "n"(YOUNGER) : "memory");
+}
+
+// The same for the register set of a step (one per producer thread in every form built).
+template <int YOUNGER, int BITS>
+__device__ __forceinline__ void wait_codes(CodeRegsT<BITS> (&r)[1]) { wait_codes<YOUNGER>(r[0]); }
+
+// 8 bytes of two packed words -> 8 bf16 of fma(s, q, b), as one 16-byte LDS chunk (the 8-bit pack).
+__device__ __forceinline__ uint4 dequant_bytes(uint32_t w0, uint32_t w1, float s, float b)
+{
+  uint4 o;
+  o.x = pack_bf16x2(fmaf(s, ubyte_f32<0>(w0), b), fmaf(s, ubyte_f32<1>(w0), b));
+  o.y = pack_bf16x2(fmaf(s, ubyte_f32<2>(w0), b), fmaf(s, ubyte_f32<3>(w0), b));
+  o.z = pack_bf16x2(fmaf(s, ubyte_f32<0>(w1), b), fmaf(s, ubyte_f32<1>(w1), b));
+  o.w = pack_bf16x2(fmaf(s, ubyte_f32<2>(w1), b), fmaf(s, ubyte_f32<3>(w1), b));
+  return o;
 }
 
 }  // namespace
@@ -194,7 +221,7 @@ __device__ __forceinline__ void wait_codes(CodeRegs (&r)[2])
 // brought in by the CONSUMER wavefronts, whose load counter nothing else uses: a 2-byte load per row, array
 // and step costs a 32-byte sector each, twice the bytes of the codes.  Needs K % 512 == 0, 16-byte
 // aligned scales and biases and no split of K.
-template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false, int P = kProducers, bool SBR = false>
+template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false, int P = kProducers, bool SBR = false, int BITS = 4>
 __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const TileParams p)
 {
   static_assert((TMK == 256 && TNK == 128 && P == 4) || (TMK == 128 && !LORA && (TNK == 128 || TNK == 256)), "tiles built");
@@ -202,7 +229,9 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
   constexpr int kWStage = TNK * kRowB;             // 16 KB at 128 weight rows
   constexpr int kWH = TNK / (32 * P);              // weight rows (code requests) per producer thread and step
   constexpr int kJT = TNK / 64;                    // 32-row W fragments per consumer wavefront
-  constexpr int kCR = (SBR ? 1 : 3) * kWH;         // code (, scale and bias) requests per producer thread and step
+  constexpr int kCR = ((SBR ? 0 : 2) + BITS / 4) * kWH;   // code (, scale and bias) requests per producer thread and step
+  static_assert(BITS == 4 || (BITS == 8 && kWH == 1 && !LORA), "widths built");
+  using CodeRegs = CodeRegsT<BITS>;                // BITS: 4, or 8 (one byte per value: gpu-kernels/metal/quant/affine_qmm_steel.metal:1601-1672)
   constexpr int kSbSlot = 2 * TNK * 16;            // one window of the ring: scales | biases, 16 bytes per row
   static_assert(!SBR || kWH == 1, "one row per producer thread");
   constexpr int kWaveM = TMK / (kConsumers / 2);   // x rows per consumer wavefront
@@ -231,7 +260,7 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
   if constexpr (GROUPED) {
     const int e = p.tile2e[tm];
     if (e < 0 || e >= p.n_experts) { return; }        // the whole workgroup, before any barrier
-    pw_base += (size_t)e * (size_t)p.N * (size_t)(p.K >> 3);
+    pw_base += (size_t)e * (size_t)p.N * (size_t)(p.K >> (BITS == 4 ? 3 : 2));
     ps_base += (size_t)e * (size_t)p.N * (size_t)(p.K >> 6);
     pb_base += (size_t)e * (size_t)p.N * (size_t)(p.K >> 6);
   }
@@ -271,8 +300,8 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
 #pragma unroll
     for (int h = 0; h < kWH; ++h) {
       const int qrg = (n0 + qrow + 32 * P * h < p.N) ? (n0 + qrow + 32 * P * h) : (p.N - 1);
-      wrow[h] = reinterpret_cast<const uint8_t*>(pw_base) + (size_t)qrg * (p.K >> 1) + qhalf * 16 +
-                (size_t)k_first * (TK / 2);
+      wrow[h] = reinterpret_cast<const uint8_t*>(pw_base) + (size_t)qrg * (p.K * BITS / 8) + qhalf * (4 * BITS) +
+                (size_t)k_first * (TK * BITS / 8);
       srow[h] = ps_base + (size_t)qrg * (p.K >> 6) + k_first;
       brow[h] = pb_base + (size_t)qrg * (p.K >> 6) + k_first;
     }
@@ -295,16 +324,23 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
         const float sc = bf16_bits_to_f32(r[h].s_bits), bi = bf16_bits_to_f32(r[h].b_bits);
         uint8_t* nb = w_lds + stage * kWStage + h * (32 * P * kRowB);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word(r[h].codes[i], sc, bi); }
+        for (int i = 0; i < 4; ++i) {
+          if constexpr (BITS == 4) {
+            *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word(r[h].codes[i], sc, bi);
+          } else {
+            const u32x4& cw = i < 2 ? r[h].codes : r[h].codes2;
+            *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_bytes(cw[2 * (i & 1)], cw[2 * (i & 1) + 1], sc, bi);
+          }
+        }
       }
     };
     auto request = [&](CodeRegs (&r)[kWH], int step) {
 #pragma unroll
       for (int h = 0; h < kWH; ++h) {
         if constexpr (SBR) {
-          request_codes_only(r[h], wrow[h] + (size_t)step * (TK / 2));
+          request_codes_only(r[h], wrow[h] + (size_t)step * (TK * BITS / 8));
         } else {
-          request_codes(r[h], wrow[h] + (size_t)step * (TK / 2), srow[h] + step, brow[h] + step);
+          request_codes(r[h], wrow[h] + (size_t)step * (TK * BITS / 8), srow[h] + step, brow[h] + step);
         }
       }
     };
@@ -733,6 +769,10 @@ hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a)
   p.tiles_n = (a.N + TN - 1) / TN;
   p.ksplit = 1; p.steps_per_split = a.K / TK; p.plane = nullptr;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
+  if (a.bits == 8) {
+    if (a.lora_t != nullptr) { return hipErrorInvalidValue; }     // no 8-bit form with the adapter
+    return launch_kernel(qmm_tile_kernel<false, TM, TN, false, kProducers, false, 8>, grid, block, 0, st, p);
+  }
   return a.lora_t != nullptr ? launch_kernel(qmm_tile_kernel<true>, grid, block, 0, st, p)
                              : launch_kernel(qmm_tile_kernel<false>, grid, block, 0, st, p);
 }
@@ -755,8 +795,16 @@ hipError_t launch_qmm_grouped(hipStream_t st, const GemmArgs& a, const GroupedAr
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
   if (wide) {
     const dim3 block12((kConsumers + 8) * 64);
+    if (a.bits == 8) {
+      return sb_ring_ok(a)
+                 ? launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true, 8, true, 8>, grid, block12, 0, st, p)
+                 : launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true, 8, false, 8>, grid, block12, 0, st, p);
+    }
     return sb_ring_ok(a) ? launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true, 8, true>, grid, block12, 0, st, p)
                          : launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, 2 * TN, true, 8>, grid, block12, 0, st, p);
+  }
+  if (a.bits == 8) {
+    return launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, TN, true, kProducers, false, 8>, grid, block, 0, st, p);
   }
   return launch_kernel(qmm_tile_kernel<false, kGroupedBlockRows, TN, true>, grid, block, 0, st, p);
 }

@@ -111,6 +111,17 @@ const FnEntry kFunctions[] = {
     {"affine_dequant_bf16", "affine_dequant_w8g64", QuantKernel::Dequant, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64", QuantKernel::Qmv, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64", QuantKernel::Qmm, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64_bm64", QuantKernel::Qmm, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64_bm128", QuantKernel::Qmm, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64", QuantKernel::QmmSwiglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_bm64", QuantKernel::QmmSwiglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_bm128", QuantKernel::QmmSwiglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_bm64_rs", QuantKernel::QmmSwiglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_geglu_w8g64", QuantKernel::QmmGeglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_grouped_swiglu_w8g64", QuantKernel::GroupedSwiglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_grouped_geglu_w8g64", QuantKernel::GroupedGeglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_grouped_w8g64", QuantKernel::GroupedDown, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_swiglu_w8g64", QuantKernel::QmvSwiglu, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_geglu_w8g64", QuantKernel::QmvGeglu, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w8g64", QuantKernel::GatherSwiglu, QuantFormat::W8G64},
@@ -418,7 +429,40 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
       const uint16_t* residual = kind == QuantKernel::QmvAdd ? static_cast<const uint16_t*>(buf(7)) : nullptr;
       const bool gather = kind == QuantKernel::GatherSwiglu || kind == QuantKernel::GatherGeglu ||
                           kind == QuantKernel::GatherDown;
-      if (fmt == QuantFormat::W4G64F16) {
+      const bool grouped = kind == QuantKernel::GroupedSwiglu || kind == QuantKernel::GroupedGeglu ||
+                           kind == QuantKernel::GroupedDown;
+      if (fmt == QuantFormat::W8G64 && (kind == QuantKernel::Qmm || kind == QuantKernel::QmmSwiglu ||
+                                        kind == QuantKernel::QmmGeglu)) {
+        // gpu-kernels/metal/quant/affine_qmm_steel.metal:1601-1890: the 4-bit GEMM slots (7 = M, 8 = out_stride,
+        // 9 = out_off for the strided gated form) over byte codes
+        if (!has_int(7)) {
+          status = VPQ_ERR_NULL_POINTER;
+        } else {
+          const int act = kind == QuantKernel::Qmm ? 0 : (kind == QuantKernel::QmmGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
+          status = vpq_qmm_gated_w8g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), act != 0 && has_int(8) ? ival(8) : 0,
+                                            act != 0 && has_int(9) ? ival(9) : 0, act);
+        }
+      } else if (fmt == QuantFormat::W8G64 && grouped) {
+        // :1069-1090, 1290-1366: slot 7 = npad, 8 = tile2e, 9 = srow / sdst, as the 4-bit grouped functions
+        const bool down = kind == QuantKernel::GroupedDown;
+        if (!has_int(7) || !buf(8) || !buf(9)) {
+          status = VPQ_ERR_NULL_POINTER;
+        } else if (K <= 0 || N <= 0 || K % 64 != 0) {
+          status = VPQ_ERR_BAD_SHAPE;
+        } else {
+          const std::size_t experts = _slots[0].bytes / (static_cast<std::size_t>(N) * static_cast<std::size_t>(K));
+          const int E = experts > 0x7fffffffu ? 0x7fffffff : static_cast<int>(experts);
+          const std::size_t rows = down ? _slots[4].bytes / (static_cast<std::size_t>(N) * 2)
+                                        : _slots[3].bytes / (static_cast<std::size_t>(K) * 2);
+          const int nrows = rows > 0x7fffffffu ? 0x7fffffff : static_cast<int>(rows);
+          const int32_t* t2e = static_cast<const int32_t*>(buf(8));
+          const int32_t* idx = static_cast<const int32_t*>(buf(9));
+          status = down ? vpq_qmm_grouped_down_w8g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), t2e, idx, E, nrows)
+                        : vpq_qmm_grouped_gated_w8g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), t2e, idx, E, nrows,
+                                                           kind == QuantKernel::GroupedGeglu ? VPQ_GATE_GEGLU
+                                                                                             : VPQ_GATE_SWIGLU);
+        }
+      } else if (fmt == QuantFormat::W4G64F16) {
         if (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu) {
           status = vpq_qmv_gated_w4g64_f16(st, w, sc, bi, x, y, K, N, M,
                                            kind == QuantKernel::QmvGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
