@@ -421,6 +421,10 @@ int vpq_qmm_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, cons
  *                                    QMV arithmetic, 1 <= M <= 16.
  *   vpq_qmv_gated_w4g32_bf16         replaces `affine_qmv_geglu_w4g32[_q40]` (:1451-1490) and the
  *                                    SwiGLU twin over an interleaved gate|up pack; y [M, N/2].
+ *   vpq_qmm_w4g32_bf16, vpq_qmm_gated_w4g32_bf16   the fused tile kernel with a scale and a bias per 32
+ *                                    values: replace `affine_qmm_steel_w4g32`
+ *                                    (affine_qmm_steel.metal:618-640) and `affine_qmm_geglu_w4g32`
+ *                                    (:1573-1596) plus the SwiGLU twin; K % 64 == 0, any M.
  *   vpq_qmm_dense_route_w4g32_bf16   GEMM by expansion into w_deq[N,K] + the vendor GEMM
  *                                    (expand as in vpq_qmm_dense_route_w4g64_bf16).
  * Requires K % 32 == 0; w, x 16-byte aligned. */
@@ -433,6 +437,10 @@ int vpq_qmv_w4g32_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t*
                          const uint16_t* x, float* y, int K, int N, int M, int scale_only);
 int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                              const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int scale_only);
+int vpq_qmm_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                       const uint16_t* x, uint16_t* y, int K, int N, int M);
+int vpq_qmm_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation);
 int vpq_qmm_dense_route_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                                    uint16_t* w_deq, int expand);

@@ -112,3 +112,40 @@ def test_g32_rejects_bad_arguments(vpq, dev):
     assert L.vpq_qmv_gated_w4g32_bf16(None, p, p, p, p, p, 32, 7, 1, capi.VPQ_GATE_SWIGLU, 0) == -2
     assert L.vpq_dequant_w4g32_bf16(None, p, p, p, None, 32, 8) == -1
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (300, 200, 128), (257, 129, 512), (520, 260, 1536)])
+def test_qmm_g32_fused_tile_kernel(vpq, oracle, dev, D, M, N, K):
+    # the fused kernel with a scale and a bias per 32 values: the GEMM on the oracle's bit-exact expansion
+    w, s, b = synth.make_weight_g32(N, K, 6900 + N)
+    x = synth.make_act(M, K, 6901 + M)
+    dense = oracle.dequant_g32_bf16(w, s, b, K, N)
+    y64 = synth.bf16_bits_to_f32(x).astype(np.float64) @ synth.bf16_bits_to_f32(dense).astype(np.float64).T
+    yb = synth.f32_to_bf16_bits(y64.astype(np.float32))
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_w4g32(wd, sd, bd, xd, K, N, M, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    # a group-64 pack with every scale and bias written twice is the same matrix: the group-64 kernel's bits
+    w64, s64, b64 = synth.make_weight(N, K, 6902 + N)
+    s2, b2 = np.repeat(s64, 2, axis=1), np.repeat(b64, 2, axis=1)
+    got32 = vpq.qmm_w4g32(D.u32(w64, dev), D.bf16(s2, dev), D.bf16(b2, dev), xd, K, N, M)
+    got64 = vpq.qmm_w4g64(D.u32(w64, dev), D.bf16(s64, dev), D.bf16(b64, dev), xd, K, N, M, tile_n=128)
+    assert torch.equal(got32, got64)
+
+
+@pytest.mark.parametrize("activation", [capi.VPQ_GATE_SWIGLU, capi.VPQ_GATE_GEGLU])
+def test_qmm_g32_gated_store(vpq, oracle, dev, D, activation):
+    K, F, M = 512, 70, 130
+    w, s, b = synth.make_weight_g32(2 * F, K, 6950)
+    x = synth.make_act(M, K, 6951)
+    dense = oracle.dequant_g32_bf16(w, s, b, K, 2 * F)
+    y64 = synth.bf16_bits_to_f32(x).astype(np.float64) @ synth.bf16_bits_to_f32(dense).astype(np.float64).T
+    want64, wantb = (oracle.swiglu if activation == capi.VPQ_GATE_SWIGLU else oracle.geglu)(y64)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    got = vpq.qmm_w4g32(wd, sd, bd, xd, K, 2 * F, M, activation=activation)
+    parity.check_bf16(D.bits(got), want64, wantb, mismatch_over_all=activation == capi.VPQ_GATE_SWIGLU)
+    assert vpq.load().vpq_qmm_w4g32_bf16(None, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), xd.data_ptr(), got.data_ptr(),
+                                         96, 8, 4) == -2            # K % 64

@@ -73,6 +73,8 @@ SYMBOLS = [
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_qmm_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_qmm_gated_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
     ("vpq_qmm_grouped_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _i]),
     ("vpq_qmm_grouped_down_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
@@ -403,6 +405,16 @@ def gather_qmv_gated_split(gate, gate_bits, up, up_bits, x, K, ffn, pair_eid, to
                                                   _ptr(up[0]), _ptr(up[1]), _ptr(up[2]), up_bits, _ptr(x), _ptr(out), K, ffn,
                                                   _ptr(pair_eid), rows, top_k, n_experts, activation),
            "vpq_gather_qmv_gated_split_bf16")
+    return out
+
+
+def qmm_w4g32(w, scales, biases, x, K, N, M, out=None, activation=0):
+    """Fused group-32 GEMM on the tile kernel; activation != 0: interleaved gate|up pack -> [M, N/2]."""
+    import torch
+    if out is None:
+        out = torch.empty((M, N // 2 if activation else N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_gated_w4g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                           activation), "vpq_qmm_gated_w4g32_bf16")
     return out
 
 

@@ -988,6 +988,33 @@ int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
   return qmv_g32_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, activation, scale_only != 0);
 }
 
+int vpq_qmm_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
+{
+  int st = check_pack_g32(w, scales, biases, K, N, false);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (activation != 0 && activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (M <= 0 || (K % 64) != 0 || (activation != 0 && (N & 1) != 0)) { return VPQ_ERR_BAD_SHAPE; }
+  if ((long long)M * (long long)K * 2 >= 4000000000LL) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::GemmArgs g{};
+  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
+  g.K = K; g.N = N; g.M = M; g.lora_t = nullptr; g.lora_b = nullptr; g.r = 0;
+  g.cu_count = g_dev.cu_count;
+  g.gate_act = activation; g.out_stride = 0; g.out_off = 0;
+  g.group = 32;
+  return finish(vpq::launch_qmm_tile(reinterpret_cast<hipStream_t>(stream), g));
+}
+
+int vpq_qmm_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                       const uint16_t* x, uint16_t* y, int K, int N, int M)
+{
+  return vpq_qmm_gated_w4g32_bf16(stream, w, scales, biases, x, y, K, N, M, 0);
+}
+
 int vpq_qmm_dense_route_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                                    uint16_t* w_deq, int expand)

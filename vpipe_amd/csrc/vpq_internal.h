@@ -72,6 +72,7 @@ struct GemmArgs {
   int out_stride = 0;
   int out_off = 0;
   int bits = 4;              // 8: one byte per value, w [N, K/4] (the tile kernel only)
+  int group = 64;            // 32: scales / biases [N, K/32] (the tile kernel only, 4-bit)
 };
 
 hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* scales,

@@ -221,7 +221,8 @@ __device__ __forceinline__ uint4 dequant_bytes(uint32_t w0, uint32_t w1, float s
 // brought in by the CONSUMER wavefronts, whose load counter nothing else uses: a 2-byte load per row, array
 // and step costs a 32-byte sector each, twice the bytes of the codes.  Needs K % 512 == 0, 16-byte
 // aligned scales and biases and no split of K.
-template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false, int P = kProducers, bool SBR = false, int BITS = 4>
+template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false, int P = kProducers, bool SBR = false, int BITS = 4,
+          int GROUP = 64>
 __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const TileParams p)
 {
   static_assert((TMK == 256 && TNK == 128 && P == 4) || (TMK == 128 && !LORA && (TNK == 128 || TNK == 256)), "tiles built");
@@ -231,6 +232,11 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
   constexpr int kJT = TNK / 64;                    // 32-row W fragments per consumer wavefront
   constexpr int kCR = ((SBR ? 0 : 2) + BITS / 4) * kWH;   // code (, scale and bias) requests per producer thread and step
   static_assert(BITS == 4 || (BITS == 8 && kWH == 1 && !LORA), "widths built");
+  // GROUP: values per scale and bias, 64 or 32 (affine_qmm_steel_w4g32, gpu-kernels/metal/quant/
+  // affine_qmm_steel.metal:618-640).  A producer thread's 32 values of a step are one group of 32: it reads
+  // the scale of its half.
+  static_assert(GROUP == 64 || (GROUP == 32 && !SBR && !GROUPED && !LORA && BITS == 4), "groups built");
+  constexpr int kGPS = TK / GROUP;                 // groups per K step
   using CodeRegs = CodeRegsT<BITS>;                // BITS: 4, or 8 (one byte per value: gpu-kernels/metal/quant/affine_qmm_steel.metal:1601-1672)
   constexpr int kSbSlot = 2 * TNK * 16;            // one window of the ring: scales | biases, 16 bytes per row
   static_assert(!SBR || kWH == 1, "one row per producer thread");
@@ -302,8 +308,8 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
       const int qrg = (n0 + qrow + 32 * P * h < p.N) ? (n0 + qrow + 32 * P * h) : (p.N - 1);
       wrow[h] = reinterpret_cast<const uint8_t*>(pw_base) + (size_t)qrg * (p.K * BITS / 8) + qhalf * (4 * BITS) +
                 (size_t)k_first * (TK * BITS / 8);
-      srow[h] = ps_base + (size_t)qrg * (p.K >> 6) + k_first;
-      brow[h] = pb_base + (size_t)qrg * (p.K >> 6) + k_first;
+      srow[h] = ps_base + (size_t)qrg * (p.K / GROUP) + (size_t)k_first * kGPS + (GROUP == 32 ? qhalf : 0);
+      brow[h] = pb_base + (size_t)qrg * (p.K / GROUP) + (size_t)k_first * kGPS + (GROUP == 32 ? qhalf : 0);
     }
     int b_dst[4];                          // row + 32 P has the same swizzle: + 32 P rows of bytes
 #pragma unroll
@@ -340,7 +346,7 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
         if constexpr (SBR) {
           request_codes_only(r[h], wrow[h] + (size_t)step * (TK * BITS / 8));
         } else {
-          request_codes(r[h], wrow[h] + (size_t)step * (TK * BITS / 8), srow[h] + step, brow[h] + step);
+          request_codes(r[h], wrow[h] + (size_t)step * (TK * BITS / 8), srow[h] + step * kGPS, brow[h] + step * kGPS);
         }
       }
     };
@@ -770,8 +776,12 @@ hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a)
   p.ksplit = 1; p.steps_per_split = a.K / TK; p.plane = nullptr;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
   if (a.bits == 8) {
-    if (a.lora_t != nullptr) { return hipErrorInvalidValue; }     // no 8-bit form with the adapter
+    if (a.lora_t != nullptr || a.group != 64) { return hipErrorInvalidValue; }     // no 8-bit form with the adapter
     return launch_kernel(qmm_tile_kernel<false, TM, TN, false, kProducers, false, 8>, grid, block, 0, st, p);
+  }
+  if (a.group == 32) {
+    if (a.lora_t != nullptr) { return hipErrorInvalidValue; }
+    return launch_kernel(qmm_tile_kernel<false, TM, TN, false, kProducers, false, 4, 32>, grid, block, 0, st, p);
   }
   return a.lora_t != nullptr ? launch_kernel(qmm_tile_kernel<true>, grid, block, 0, st, p)
                              : launch_kernel(qmm_tile_kernel<false>, grid, block, 0, st, p);

@@ -139,6 +139,8 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_w4g32_add", QuantKernel::QmvAdd, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_w4g32_q40", QuantKernel::Qmv, QuantFormat::W4G32Q40},
     {"affine_qmv_bf16", "affine_qmv_w4g32_add_q40", QuantKernel::QmvAdd, QuantFormat::W4G32Q40},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g32", QuantKernel::Qmm, QuantFormat::W4G32},
+    {"affine_qmm_steel_bf16", "affine_qmm_geglu_w4g32", QuantKernel::QmmGeglu, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_geglu_w4g32", QuantKernel::QmvGeglu, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_geglu_w4g32_q40", QuantKernel::QmvGeglu, QuantFormat::W4G32Q40},
 };
@@ -442,6 +444,11 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
           status = vpq_qmm_gated_w8g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), act != 0 && has_int(8) ? ival(8) : 0,
                                             act != 0 && has_int(9) ? ival(9) : 0, act);
         }
+      } else if (fmt == QuantFormat::W4G32 && (kind == QuantKernel::Qmm || kind == QuantKernel::QmmGeglu)) {
+        // gpu-kernels/metal/quant/affine_qmm_steel.metal:618-640, 1573-1596: slot 7 = M
+        status = !has_int(7) ? VPQ_ERR_NULL_POINTER
+                             : vpq_qmm_gated_w4g32_bf16(st, w, sc, bi, x, y, K, N, ival(7),
+                                                        kind == QuantKernel::QmmGeglu ? VPQ_GATE_GEGLU : 0);
       } else if (fmt == QuantFormat::W8G64 && grouped) {
         // :1069-1090, 1290-1366: slot 7 = npad, 8 = tile2e, 9 = srow / sdst, as the 4-bit grouped functions
         const bool down = kind == QuantKernel::GroupedDown;
