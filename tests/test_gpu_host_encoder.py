@@ -731,3 +731,18 @@ def test_eight_bit_gemm_function_names(vpq, enc, dev, D):
     want_part = torch.zeros_like(part)
     vpq.qmm_grouped_down_w8g64(*dn_d, gact, ffn, H, t2e, sdst, E, out=want_part)
     assert torch.equal(part, want_part) and part.abs().sum() > 0
+
+
+def test_group32_gemm_function_names(vpq, enc, dev, D):
+    K, N, M = 256, 72, 50
+    w, s, b = synth.make_weight_g32(N, K, 4000)
+    wd, sd, bd = D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev)
+    xd = D.bf16(synth.make_act(M, K, 4001), dev)
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    yg = torch.zeros((M, N // 2), dtype=torch.bfloat16, device=dev)
+    encode_linear(enc, "affine_qmm_steel_bf16", "affine_qmm_steel_w4g32", wd, sd, bd, xd, y, K, N, M=M, grid=(N, M, 2), tg=(32, 2, 2))
+    encode_linear(enc, "affine_qmm_steel_bf16", "affine_qmm_geglu_w4g32", wd, sd, bd, xd, yg, K, N, M=M, grid=(N, M, 2), tg=(32, 2, 2))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert torch.equal(y, vpq.qmm_w4g32(wd, sd, bd, xd, K, N, M))
+    assert torch.equal(yg, vpq.qmm_w4g32(wd, sd, bd, xd, K, N, M, activation=2))
