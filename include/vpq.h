@@ -439,6 +439,10 @@ int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
                              const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int scale_only);
 int vpq_qmm_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                        const uint16_t* x, uint16_t* y, int K, int N, int M);
+/* The size-based entrance over a group-32 pack: slabs of vpq_qmv_w4g32_bf16 up to 64 rows (at every M where
+ * K % 64 != 0), vpq_qmm_w4g32_bf16 above. */
+int vpq_linear_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                          const uint16_t* x, uint16_t* y, int K, int N, int M);
 int vpq_qmm_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                              const uint16_t* x, uint16_t* y, int K, int N, int M, int activation);
 int vpq_qmm_dense_route_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
@@ -511,6 +515,11 @@ int vpq_gather_qmv_gated_split_bf16(vpq_stream_t stream, const uint32_t* wg, con
                                     const int32_t* pair_eid, int npair, int top_k, int n_experts, int activation);
 int vpq_qmm_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                        const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M);
+/* The size-based entrance over an 8-bit pack (qmm_auto_'s ladder, generative-models/qwen3/
+ * metal-qwen-model.cc:3964-4033, which takes the width from the layer): slabs of vpq_qmv_w8g64_bf16 up to
+ * 64 rows, vpq_qmm_w8g64_bf16 above. */
+int vpq_linear_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                          const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M);
 int vpq_qmm_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                              int out_stride, int out_off, int activation);

@@ -282,3 +282,29 @@ def test_grouped_expert_gemms_w8(vpq, oracle, dev, D, K, inner, H, E, T, top_k):
     part.assert_intact()
     d64, dbits = oracle.qmm_grouped(dw, ds, db, xs, Kd, H, B, t2e, sdst=sdst, rows_y=npair, bits=8)
     parity.check_bf16(D.bits(part.view), d64, dbits)
+
+
+@pytest.mark.parametrize("M", [1, 16, 40, 64, 65, 300])
+def test_linear_entrances_of_the_format_twins(vpq, dev, D, M):
+    # up to 64 rows slabs of the GEMV, above the fused GEMM: the bits of the direct calls
+    K, N = 512, 136
+    x = synth.make_act(M, K, 4100 + M)
+    xd = D.bf16(x, dev)
+    w8 = stage(D, dev, *synth.make_weight8(N, K, 4101))
+    g32 = stage(D, dev, *synth.make_weight_g32(N, K, 4102))
+    got8 = vpq.linear_twin("w8g64", *w8, xd, K, N, M)
+    got32 = vpq.linear_twin("w4g32", *g32, xd, K, N, M)
+    if M <= 64:
+        want8 = torch.cat([vpq.qmv_w8g64(*w8, xd[m0:m0 + 16].contiguous(), K, N, min(16, M - m0)) for m0 in range(0, M, 16)])
+        want32 = torch.cat([vpq.qmv_w4g32(*g32, xd[m0:m0 + 16].contiguous(), K, N, min(16, M - m0)) for m0 in range(0, M, 16)])
+    else:
+        want8 = vpq.qmm_w8g64(*w8, xd, K, N, M)
+        want32 = vpq.qmm_w4g32(*g32, xd, K, N, M)
+    assert torch.equal(got8, want8) and torch.equal(got32, want32)
+    # a group-32 pack with K % 64 == 32 has no fused GEMM: slabs at every M
+    K2 = 480
+    g2 = stage(D, dev, *synth.make_weight_g32(N, K2, 4103))
+    x2 = D.bf16(synth.make_act(M, K2, 4104), dev)
+    got = vpq.linear_twin("w4g32", *g2, x2, K2, N, M)
+    want = torch.cat([vpq.qmv_w4g32(*g2, x2[m0:m0 + 16].contiguous(), K2, N, min(16, M - m0)) for m0 in range(0, M, 16)])
+    assert torch.equal(got, want)

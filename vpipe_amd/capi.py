@@ -73,6 +73,8 @@ SYMBOLS = [
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_linear_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    ("vpq_linear_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     ("vpq_qmm_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     ("vpq_qmm_gated_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
@@ -405,6 +407,16 @@ def gather_qmv_gated_split(gate, gate_bits, up, up_bits, x, K, ffn, pair_eid, to
                                                   _ptr(up[0]), _ptr(up[1]), _ptr(up[2]), up_bits, _ptr(x), _ptr(out), K, ffn,
                                                   _ptr(pair_eid), rows, top_k, n_experts, activation),
            "vpq_gather_qmv_gated_split_bf16")
+    return out
+
+
+def linear_twin(kind, w, scales, biases, x, K, N, M, out=None):
+    """kind: "w8g64" or "w4g32": the size-based entrance of that format."""
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    fn = getattr(load(), "vpq_linear_%s_bf16" % kind)
+    _check(fn(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M), "vpq_linear_%s_bf16" % kind)
     return out
 
 

@@ -900,6 +900,23 @@ int vpq_qmm_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
   return vpq_qmm_gated_w8g64_bf16(stream, w, scales, biases, x, y, K, N, M, 0, 0, 0);
 }
 
+// Size-based entrances of the format twins (the ladder of vpq_linear_w4g64_bf16 without a workspace: slabs of
+// the GEMV arithmetic up to 64 rows, the fused GEMM above).
+int vpq_linear_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                          const uint16_t* x, uint16_t* y, int K, int N, int M)
+{
+  if (M >= 1 && M <= kSlabPlanMaxRows && x != nullptr && y != nullptr && K > 0 && N > 0) {
+    for (int m0 = 0; m0 < M; m0 += 16) {
+      const int rows = M - m0 < 16 ? M - m0 : 16;
+      const int st = vpq_qmv_w8g64_bf16(stream, w, scales, biases, x + (size_t)m0 * K, y + (size_t)m0 * N, K, N, rows,
+                                        nullptr);
+      if (st != VPQ_OK) { return st; }
+    }
+    return VPQ_OK;
+  }
+  return vpq_qmm_w8g64_bf16(stream, w, scales, biases, x, y, K, N, M);
+}
+
 int vpq_qmm_grouped_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                      const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
                                      int npad, const int32_t* tile2e, const int32_t* srow, int n_experts,
@@ -1013,6 +1030,22 @@ int vpq_qmm_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
                        const uint16_t* x, uint16_t* y, int K, int N, int M)
 {
   return vpq_qmm_gated_w4g32_bf16(stream, w, scales, biases, x, y, K, N, M, 0);
+}
+
+int vpq_linear_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                          const uint16_t* x, uint16_t* y, int K, int N, int M)
+{
+  // K % 64 != 0 (a group-32 pack may have K % 64 == 32) has no fused GEMM: slabs at every M
+  if (M >= 1 && (M <= kSlabPlanMaxRows || (K % 64) != 0) && x != nullptr && y != nullptr && K > 0 && N > 0) {
+    for (int m0 = 0; m0 < M; m0 += 16) {
+      const int rows = M - m0 < 16 ? M - m0 : 16;
+      const int st = vpq_qmv_w4g32_bf16(stream, w, scales, biases, x + (size_t)m0 * K, y + (size_t)m0 * N, K, N, rows,
+                                        nullptr, 0);
+      if (st != VPQ_OK) { return st; }
+    }
+    return VPQ_OK;
+  }
+  return vpq_qmm_w4g32_bf16(stream, w, scales, biases, x, y, K, N, M);
 }
 
 int vpq_qmm_dense_route_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
