@@ -746,3 +746,44 @@ def test_group32_gemm_function_names(vpq, enc, dev, D):
     assert ok, why
     assert torch.equal(y, vpq.qmm_w4g32(wd, sd, bd, xd, K, N, M))
     assert torch.equal(yg, vpq.qmm_w4g32(wd, sd, bd, xd, K, N, M, activation=2))
+
+
+@pytest.mark.parametrize("M", [3, 100])
+def test_load_and_run_eight_bit_and_group32_packs(vpq, enc, dev, D, tmp_path, M):
+    # packs of the other two formats written with the format's own library, opened again, their width and
+    # group recovered from the shapes, loaded and run through quant_linear_forward: the bits of the C ABI's
+    # size-based entrances on the same tensors
+    L = enc.L
+    L.hr_open.restype = ctypes.c_void_p
+    L.hr_open.argtypes = [ctypes.c_char_p, ctypes.c_int]
+    L.hr_close.argtypes = [ctypes.c_void_p]
+    L.hr_why.restype = ctypes.c_char_p
+    L.hd_load_and_run.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_void_p,
+                                  ctypes.c_void_p, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]
+    K, N = 512, 72
+    w8, s8, b8 = synth.make_weight8(N, K, 4200)
+    w32, s32, b32 = synth.make_weight_g32(N, K, 4201)
+    as_bf16 = lambda a: torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).view(torch.bfloat16)
+    import safetensors.torch as sttorch
+    sttorch.save_file({"a.weight": torch.from_numpy(w8.view(np.int32)),
+                       "a.scales": as_bf16(s8), "a.biases": as_bf16(b8),
+                       "b.weight": torch.from_numpy(w32.view(np.int32)), "b.scales": as_bf16(s32), "b.biases": as_bf16(b32)},
+                      str(tmp_path / "model.safetensors"))
+    # the reader wants U32 weights: rewrite the header's dtype of the two code tensors (I32 -> U32, same bytes)
+    raw = (tmp_path / "model.safetensors").read_bytes()
+    hlen = int.from_bytes(raw[:8], "little")
+    header = raw[8:8 + hlen].replace(b'"I32"', b'"U32"')
+    assert len(header) == hlen
+    (tmp_path / "model.safetensors").write_bytes(raw[:8] + header + raw[8 + hlen:])
+    r = L.hr_open(str(tmp_path / "model.safetensors").encode(), 0)
+    assert r, L.hr_why()
+    xd = D.bf16(synth.make_act(M, K, 4202), dev)
+    kn = (ctypes.c_int * 2)()
+    for prefix, kind, pack in ((b"a", "w8g64", (w8, s8, b8)), (b"b", "w4g32", (w32, s32, b32))):
+        yd = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+        torch.cuda.synchronize()
+        assert L.hd_load_and_run(enc.h, r, prefix, K, xd.data_ptr(), yd.data_ptr(), M, kn) == 1, L.hr_why()
+        assert tuple(kn) == (K, N)
+        want = vpq.linear_twin(kind, D.u32(pack[0], dev), D.bf16(pack[1], dev), D.bf16(pack[2], dev), xd, K, N, M)
+        assert torch.equal(yd, want) and yd.abs().sum() > 0
+    L.hr_close(r)

@@ -725,7 +725,16 @@ void quant_linear_forward(CommandStream& stream, const Linear& lin, const Device
   int status;
   const bool with_lora = lora != nullptr && lora->a != nullptr && lora->b != nullptr && lora->rank > 0 &&
                          lora->strength != 0.f && !lora->a->empty() && !lora->b->empty();
-  if (with_lora) {
+  const bool w4g64 = lin.bits == 4 && lin.group == 64;
+  if (!w4g64) {
+    // The format twins: their own size-based entrances; no adapter on them.
+    if (with_lora || !((lin.bits == 8 && lin.group == 64) || (lin.bits == 4 && lin.group == 32))) {
+      stream.record_error(VPQ_ERR_BAD_SHAPE, "quant_linear_forward: pack format");
+      return;
+    }
+    status = lin.bits == 8 ? vpq_linear_w8g64_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M)
+                           : vpq_linear_w4g32_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M);
+  } else if (with_lora) {
     // An adapter always takes the GEMM route: its second factor is folded into the tile's accumulator.
     if (lora_t == nullptr || lora_t->size() < static_cast<std::size_t>(M) * lora->rank * 2) {
       stream.record_error(VPQ_ERR_WORKSPACE, "quant_linear_forward: lora_t scratch too small");

@@ -525,21 +525,27 @@ bool PackFile::load_linear(CommandStream& stream, const std::string& prefix, int
   }
   if (w->dtype != "U32" || w->shape.size() != 2 || s->shape.size() != 2 || b->shape != s->shape ||
       b->dtype != s->dtype || (s->dtype != "F16" && s->dtype != "BF16")) {
-    set_why(why, prefix + ": not a U32 [N, K/8] weight with F16 or BF16 [N, K/64] scales and biases");
+    set_why(why, prefix + ": not a U32 [N, K*bits/32] weight with F16 or BF16 [N, K/group] scales and biases");
     return false;
   }
   if (K <= 0) { K = (int)(w->shape[1] * 8); }
   const int N = (int)w->shape[0];
-  if (affine_bits(prefix, K) != 4 || affine_group(prefix, K) != 64 || K % 64 != 0 || w->shape[1] * 8 != K ||
-      s->shape[0] != N || s->shape[1] * 64 != K) {
-    set_why(why, prefix + ": " + std::to_string(affine_bits(prefix, K)) + "-bit group-" +
-                     std::to_string(affine_group(prefix, K)) + " pack; this path takes 4-bit group-64 only");
+  // Width and group from the shapes (generative-models/qwen3/metal-qwen-model.cc:653-676); served: 4-bit group-64,
+  // 8-bit group-64, 4-bit group-32.
+  const int bits = affine_bits(prefix, K), group = affine_group(prefix, K);
+  const bool served = (bits == 4 && group == 64) || (bits == 8 && group == 64) || (bits == 4 && group == 32);
+  if (!served || K % group != 0 || w->shape[1] * 32 != (long long)K * bits || s->shape[0] != N ||
+      s->shape[1] * group != K) {
+    set_why(why, prefix + ": " + std::to_string(bits) + "-bit group-" + std::to_string(group) +
+                     " pack; this path takes 4-bit group-64, 8-bit group-64 and 4-bit group-32");
     return false;
   }
   std::vector<std::uint8_t> host((std::size_t)std::max(w->nbytes, s->nbytes));
   LoadedLinear l;
   l.K = K;
   l.N = N;
+  l.bits = bits;
+  l.group = group;
   l.codes = DeviceBuffer::allocate((std::size_t)w->nbytes);
   l.scales = DeviceBuffer::allocate((std::size_t)s->nbytes);
   l.qbias = DeviceBuffer::allocate((std::size_t)b->nbytes);

@@ -42,11 +42,13 @@ struct TensorInfo {
 struct LoadedLinear {
   DeviceBuffer codes, scales, qbias;
   int K = 0, N = 0;
+  int bits = 4, group = 64;
   Linear view() const
   {
     Linear l;
     l.codes = &codes; l.scales = &scales; l.qbias = &qbias;
     l.K = K; l.N = N;
+    l.bits = bits; l.group = group;
     return l;
   }
 };
