@@ -599,3 +599,24 @@ def test_f16_element_twins_against_numpy_float16(oracle):
     _, ya = oracle.matmul_f16(w, s, b, xb, K, N, M, rounded=False, residual=res.view(np.uint16))
     want_add = (yh.view(np.float16).astype(np.float32) + res.astype(np.float32)).astype(np.float16)
     assert np.array_equal(ya, want_add.view(np.uint16))
+
+
+def test_grouped_gemm_oracle_with_byte_codes_reduces_to_the_plain_8bit_gemm(oracle):
+    """The 8-bit form of the grouped restatement: every live slot equals the plain 8-bit GEMM oracle
+    (bf16-rounded weights) of its row on its expert's slab."""
+    E, top_k, T, B, K, N = 3, 2, 7, 4, 128, 9
+    eid = np.random.default_rng(51).integers(0, E, size=T * top_k, dtype=np.int32)
+    t2e, srow, sdst, _ = oracle.moe_sort_pairs(eid, top_k, E, B, (eid.size + B - 1) // B + E)
+    packs = [synth.make_weight8(N, K, 600 + e) for e in range(E)]
+    w, s, b = (np.stack([p[i] for p in packs]) for i in range(3))
+    x = synth.make_act(T, K, 52)
+    y64, yb = oracle.qmm_grouped(w, s, b, x, K, N, B, t2e, srow=srow, bits=8)
+    seen = 0
+    for slot in range(srow.size):
+        if t2e[slot // B] < 0 or srow[slot] < 0:
+            continue
+        e = t2e[slot // B]
+        p64, pb = oracle.matmul8(w[e], s[e], b[e], x[srow[slot]:srow[slot] + 1], K, N, 1, rounded=True)
+        assert np.array_equal(y64[slot], p64[0]) and np.array_equal(yb[slot], pb[0])
+        seen += 1
+    assert seen == eid.size
