@@ -3,7 +3,8 @@ serving loop would run it): every replay, with new inputs written between replay
 own eager work and synchronizations in between, gives the bits of the same calls made eagerly.  Covers
 the QMV kernels (single, grouped, ring, split-K with its self-resetting counters, gated), the fused GEMM
 kernels (tile, large-tile, split-K fold, LoRA with its x.A^T launch), the MoE pair sort (its fill kernel,
-histogram and tickets) with the expert-sorted GEMMs, and the argmax tail -- nothing in them allocates,
+histogram and tickets) with the expert-sorted GEMMs (4-bit and 8-bit), the 8-bit and group-32 QMV and fused
+GEMMs, the mixed-width gate/up and the argmax tail -- nothing in them allocates,
 clears memory with a memset node or keeps state between calls."""
 import numpy as np
 import pytest
@@ -33,12 +34,18 @@ def test_graph_replays_match_eager_calls(vpq, dev, D):
     gud = stage(D, dev, *(np.stack([p[i] for p in gu]) for i in range(3)))
     dnd = stage(D, dev, *(np.stack([p[i] for p in dn]) for i in range(3)))
 
+    p8 = stage(D, dev, *synth.make_weight8(N2, K, 9007))
+    p8g = stage(D, dev, *synth.make_weight8(2 * N2, K, 9008))
+    p32 = stage(D, dev, *synth.make_weight_g32(N2, K, 9009))
+    gu8 = stage(D, dev, *(np.stack([synth.make_weight8(2 * inner, Kq, 9300 + e)[i] for e in range(E)]) for i in range(3)))
+
     # inputs that change between replays (written in place)
     x1 = torch.empty((1, K), dtype=torch.bfloat16, device=dev)
     x8 = torch.empty((8, K), dtype=torch.bfloat16, device=dev)
     xq = torch.empty((Mq, Kq), dtype=torch.bfloat16, device=dev)
     xb = torch.empty((256, 1024), dtype=torch.bfloat16, device=dev)
     xt = torch.empty((T, Kq), dtype=torch.bfloat16, device=dev)
+    xq8 = torch.empty((Mq, K), dtype=torch.bfloat16, device=dev)
     eid = torch.empty((T * top_k,), dtype=torch.int32, device=dev)
     logits = torch.empty((2, 5000), dtype=torch.bfloat16, device=dev)
     ws_qmv = vpq.qmv_workspace(K, N1, 1, dev)
@@ -62,7 +69,9 @@ def test_graph_replays_match_eager_calls(vpq, dev, D):
         return {"single": fresh((1, N1)), "splitk": fresh((1, N1)), "ga": fresh((1, N1)), "gb": fresh((1, N2)),
                 "ring": fresh((8, N2)), "gated": fresh((1, N2)), "tile": fresh((Mq, Nq)), "lora": fresh((Mq, Nq)),
                 "fold": fresh((64, Nq)), "big": fresh((256, 256)), "gact": fresh((npad, inner)),
-                "part": fresh((T * top_k, Kq)), "tok": fresh((2,), torch.int32)}
+                "part": fresh((T * top_k, Kq)), "tok": fresh((2,), torch.int32), "w8": fresh((8, N2)),
+                "w8gated": fresh((1, N2)), "w8gemm": fresh((Mq, N2)), "g32gemm": fresh((Mq, N2)), "g32": fresh((1, N2)),
+                "gact8": fresh((npad, inner)), "split": fresh((1, N2))}
 
     def layer(o):
         vpq.qmv_w4g64(*p1, x1, K, N1, 1, out=o["single"])
@@ -82,11 +91,18 @@ def test_graph_replays_match_eager_calls(vpq, dev, D):
         vpq.qmm_grouped_gated_w4g64(*gud, xt, Kq, 2 * inner, t2e, srow, E, out=o["gact"])
         vpq.qmm_grouped_down_w4g64(*dnd, o["gact"], inner, Kq, t2e, sdst, E, out=o["part"])
         vpq.argmax_bf16(logits, out=o["tok"], two_stage=False)
+        vpq.qmv_w8g64(*p8, x8, K, N2, 8, out=o["w8"])
+        vpq.qmv_gated_w8g64(*p8g, x1, K, 2 * N2, 1, out=o["w8gated"])
+        vpq.qmm_w8g64(*p8, xq8, K, N2, Mq, out=o["w8gemm"])
+        vpq.qmm_w4g32(*p32, xq8, K, N2, Mq, out=o["g32gemm"])
+        vpq.qmv_w4g32(*p32, x1, K, N2, 1, out=o["g32"])
+        vpq.qmm_grouped_gated_w8g64(*gu8, xt, Kq, 2 * inner, t2e, srow, E, out=o["gact8"])
+        vpq.gather_qmv_gated_split(p2, 4, p8, 8, x1, K, N2, None, 1, 1, out=o["split"])
 
     def new_inputs(seed):
         g = torch.Generator(device=dev)
         g.manual_seed(seed)
-        for t in (x1, x8, xq, xb, xt, logits):
+        for t in (x1, x8, xq, xb, xt, xq8, logits):
             t.copy_(torch.randn(t.shape, device=dev, generator=g).bfloat16())
         eid.copy_(torch.randint(0, E, eid.shape, dtype=torch.int32, device=dev, generator=g))
 
@@ -106,9 +122,10 @@ def test_graph_replays_match_eager_calls(vpq, dev, D):
         graph.replay()
         torch.cuda.synchronize()
         for name in eager:
-            if name == "gact":
+            if name in ("gact", "gact8"):
                 continue                          # slot order inside an expert may differ between two sorts
             assert torch.equal(eager[name], captured[name]), "%s differs on the replay with seed %d" % (name, seed)
         # the gate|up activations as a multiset of rows per replay: compare after undoing the slot order
-        assert torch.equal(torch.sort(eager["gact"].float().sum(dim=1)).values,
-                           torch.sort(captured["gact"].float().sum(dim=1)).values)
+        for name in ("gact", "gact8"):
+            assert torch.equal(torch.sort(eager[name].float().sum(dim=1)).values,
+                               torch.sort(captured[name].float().sum(dim=1)).values), name
