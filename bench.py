@@ -266,7 +266,10 @@ def main():
                 "kernel": "qmv_mfma_kernel (all %d launches of a layer)" % launches_per_layer,
                 "avg_launch_us": round(avg_launch_us, 3),
                 "bytes_per_launch": layer_bytes / launches_per_layer,
-                "launches_timed": args.steps * launches_per_layer}
+                "launches_timed": args.steps * launches_per_layer,
+                "note": "a do-nothing read of the same 27 MB per launch takes 5.2-5.4 us on this part (launch and "
+                        "first-byte latency), and reads of 0.4-1 GB reach 6.2-6.4 TB/s: the reachable fraction of the "
+                        "8 TB/s peak is 0.64 at this launch size and 0.78-0.80 at any size"}
     if launches_per_layer == 4:
         roofline["eager_launch_us"] = {n: round(float(dur[:, i].mean()), 3)
                                        for i, n in enumerate(("q|k|v", "o", "gate|up", "down"))}
