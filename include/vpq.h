@@ -136,8 +136,11 @@ enum {
   VPQ_QMV_MFMA_SPLITK = 3, /* as 2, K split across workgroups through `ws` */
   VPQ_QMV_STREAM = 4,      /* M <= 4: persistent workgroups, x staged in LDS, prefetched items */
   VPQ_QMV_RING = 5,        /* x in registers across a workgroup's tiles, codes through a two-slot LDS ring per wavefront */
-  VPQ_QMV_ROWS = 6         /* M <= 2, any K % 64: a wavefront streams whole rows with full-width loads, packed bf16
+  VPQ_QMV_ROWS = 6,        /* M <= 2, any K % 64: a wavefront streams whole rows with full-width loads, packed bf16
                               dot products, no LDS; what AUTO takes for M <= 2 where K is not a multiple of 512 */
+  VPQ_QMV_FLOW = 7         /* M = 1, K % 512 == 0, K >= 2048: one wavefront per (row set, K part), every load of the
+                              launch requested up front, x in registers, scales / biases staged in LDS; what AUTO
+                              takes for M = 1 below lm_head-sized packs */
 };
 
 /* ---- a6/a7/a8 (+a10): QMM ----------------------------------------------
@@ -252,7 +255,8 @@ int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t
  * case w[1] = w[0] + q_rows*K/8 words (scales, biases alike); gate|up of an
  * MLP is count = 2.  Arithmetic and requirements are those of
  * vpq_qmv_w4g64_bf16 per pack (no residual); results are bit-identical to
- * `count` separate calls of its VPQ_QMV_MFMA kernel where K % 512 == 0, of
+ * `count` separate calls of its VPQ_QMV_FLOW kernel at M = 1 (K % 512 == 0,
+ * K >= 2048), of its VPQ_QMV_MFMA kernel at other M where K % 512 == 0, of
  * its VPQ_QMV_ROWS kernel for other K at M <= 2.  The pointer tables are
  * host arrays, read before the call returns.  Shapes neither grouped kernel
  * takes (K % 512 != 0 with M > 2) run as separate launches. */

@@ -13,6 +13,7 @@ from vpipe_amd import capi, synth
 pytestmark = pytest.mark.gpu
 
 SIMPLE, MFMA, SPLITK, AUTO = capi.VPQ_QMV_SIMPLE, capi.VPQ_QMV_MFMA, capi.VPQ_QMV_MFMA_SPLITK, capi.VPQ_QMV_AUTO
+FLOW = capi.VPQ_QMV_FLOW
 
 
 def stage(D, dev, w, s, b, x=None):
@@ -124,6 +125,63 @@ def test_qmv_row_streaming_kernel(vpq, oracle, dev, D, K, N, M):
     got = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, residual=D.bf16(res, dev), variant=capi.VPQ_QMV_ROWS))
     want = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(D.bits(out.view)) + synth.bf16_bits_to_f32(res))
     assert np.array_equal(got, want)
+
+
+FLOW_SHAPES = [
+    # K, N: one to nine slices of 2048, K not a multiple of 2048 (idle lanes in the last slice), every plan of
+    # slices per wavefront x K parts (2560: 2x1, 4096: 2x1, 5120: 3x1, 8192: 4x1, 12288: 3x2, 14336: 4x2, 17408: 3x3),
+    # N not a multiple of the rows per wavefront / workgroup
+    (2048, 5), (2560, 33), (4096, 16 * 50 + 3), (5120, 64), (8192, 95), (12288, 161), (14336, 18), (17408, 33),
+    (24576, 7), (4096, 1),
+]
+
+
+@pytest.mark.parametrize("K,N", FLOW_SHAPES)
+def test_qmv_flow_kernel(vpq, oracle, dev, D, K, N):
+    M = 1
+    w, s, b = synth.make_weight(N, K, 8300 + K + N)
+    x = synth.make_act(M, K, 8400 + K)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=FLOW, f32out=True)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, variant=FLOW)
+    torch.cuda.synchronize()
+    parity.check_f32(f.cpu().numpy(), y64)
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    out.assert_intact()
+    # AUTO takes this kernel at M = 1 below lm_head-sized packs: same bits
+    assert np.array_equal(D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=AUTO)), D.bits(out.view))
+    res = synth.make_act(M, N, 8500 + N)
+    got = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, residual=D.bf16(res, dev), variant=FLOW))
+    want = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(D.bits(out.view)) + synth.bf16_bits_to_f32(res))
+    assert np.array_equal(got, want)
+
+
+def test_qmv_flow_kernel_refuses_what_it_does_not_take(vpq, dev, D):
+    w, s, b = synth.make_weight(16, 1024, 1)
+    wd, sd, bd = stage(D, dev, w, s, b)
+    x = D.bf16(synth.make_act(2, 1024, 2), dev)
+    with pytest.raises(capi.VpqError):
+        vpq.qmv_w4g64(wd, sd, bd, x[:1].contiguous(), 1024, 16, 1, variant=FLOW)      # K below one slice
+    w, s, b = synth.make_weight(16, 2048, 1)
+    wd, sd, bd = stage(D, dev, w, s, b)
+    x = D.bf16(synth.make_act(2, 2048, 2), dev)
+    with pytest.raises(capi.VpqError):
+        vpq.qmv_w4g64(wd, sd, bd, x, 2048, 16, 2, variant=FLOW)                        # two rows of x
+
+
+def test_qmv_flow_one_hot_reads_back_weights_exactly(vpq, oracle, dev, D):
+    # x = e_k: y[n] must be fp32(s*q+b) exactly (layout, nibble order, K parts, un-rounded weights)
+    K, N = 12288, 10
+    w, s, b = synth.make_weight(N, K, 6)
+    d32 = oracle.dequant_f32(w, s, b, K, N)
+    wd, sd, bd = stage(D, dev, w, s, b)
+    for k in [0, 1, 4, 7, 8, 31, 32, 63, 64, 2047, 2048, 6143, 6144, 6145, 9999, K - 1]:
+        x = np.zeros((1, K), dtype=np.float32)
+        x[0, k] = 1.0
+        y = vpq.qmv_w4g64(wd, sd, bd, D.bf16(synth.f32_to_bf16_bits(x), dev), K, N, 1, variant=FLOW, f32out=True)
+        assert np.array_equal(y.cpu().numpy()[0], d32[:, k]), k
 
 
 STREAM_SHAPES = [
@@ -342,7 +400,8 @@ def test_qmv_grouped_launch_equals_separate_launches(vpq, oracle, dev, D, K, Ns,
     outs = [parity.Guarded((M, N), torch.bfloat16, dev) for N in Ns]
     vpq.qmv_group_w4g64(packs, xd, K, M, outs=[o.view for o in outs])
     torch.cuda.synchronize()
-    variant = MFMA if K % 512 == 0 else AUTO
+    # the kernel a grouped launch shares its arithmetic with: the streaming one at M = 1, the tile one otherwise
+    variant = (FLOW if M == 1 and K >= 2048 else MFMA) if K % 512 == 0 else AUTO
     for (wd, sd, bd, N), (y64, yb), out in zip(packs, refs, outs):
         got = D.bits(out.view)
         parity.check_bf16(got, y64, yb)

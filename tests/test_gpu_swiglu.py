@@ -68,6 +68,24 @@ def test_qmv_gated_row_streaming_kernel(vpq, oracle, dev, D, K, F, M, activation
         assert torch.equal(auto, out.view)
 
 
+@pytest.mark.parametrize("activation", [capi.VPQ_GATE_SWIGLU, capi.VPQ_GATE_GEGLU])
+@pytest.mark.parametrize("K,F", [(2048, 3), (4096, 101), (12288, 37), (17408, 9)])
+def test_qmv_gated_flow_kernel(vpq, oracle, dev, D, K, F, activation):
+    # the streaming M = 1 kernel's register-local gated store (a gate/up pair of rows is one wavefront's)
+    _, _, pack = fused_pack(oracle, F, K, 520 + K + F)
+    x = synth.make_act(1, K, 620 + K)
+    y64, _ = oracle.qmv(*pack, x, K, 2 * F, 1)
+    o64, ob = oracle.swiglu(y64) if activation == capi.VPQ_GATE_SWIGLU else oracle.geglu(y64)
+    wd, sd, bd, xd = stage(D, dev, pack, x)
+    f = vpq.qmv_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, 1, variant=capi.VPQ_QMV_FLOW, f32out=True, activation=activation)
+    out = parity.Guarded((1, F), torch.bfloat16, dev)
+    vpq.qmv_swiglu_w4g64(wd, sd, bd, xd, K, 2 * F, 1, out=out.view, variant=capi.VPQ_QMV_FLOW, activation=activation)
+    torch.cuda.synchronize()
+    parity.check_f32(f.cpu().numpy(), o64)
+    parity.check_bf16(D.bits(out.view), o64, ob, mismatch_over_all=activation == capi.VPQ_GATE_SWIGLU)
+    out.assert_intact()
+
+
 @pytest.mark.parametrize("variant", [SIMPLE, MFMA, RING, AUTO])
 @pytest.mark.parametrize("K,F,M", QMV_SHAPES)
 def test_qmv_swiglu(vpq, oracle, dev, D, K, F, M, variant):

@@ -92,7 +92,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
   if (ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }
-  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_ROWS) { return VPQ_ERR_BAD_SHAPE; }
+  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_FLOW) { return VPQ_ERR_BAD_SHAPE; }
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
 
@@ -104,7 +104,12 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
 
   const bool mfma_ok = vpq::qmv_mfma_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
+  const bool flow_ok = vpq::qmv_flow_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
   if (variant == VPQ_QMV_SIMPLE) { return finish(vpq::launch_qmv_simple(hs, a)); }
+  if (variant == VPQ_QMV_FLOW) {
+    if (!flow_ok) { return VPQ_ERR_BAD_SHAPE; }
+    return finish(vpq::launch_qmv_flow(hs, a));
+  }
   if (variant == VPQ_QMV_ROWS) {
     if (!vpq::qmv_rows_supports(K, N, M) || (gate_act != 0 && (N & 1) != 0)) { return VPQ_ERR_BAD_SHAPE; }
     return finish(vpq::launch_qmv_rows(hs, a, 0));
@@ -136,6 +141,9 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   // one-item-per-wavefront kernel finishes sooner.
   const double pack_bytes = (double)N * (double)K * 9.0 / 16.0;
   if (stream_ok && pack_bytes >= 150e6) { return finish(vpq::launch_qmv_stream(hs, a)); }
+  // One row of x over a layer-sized pack: the streaming kernel that requests the whole pack up front
+  // (measured, HBM-cold: 4096->12288 6.6 us against 9.0 for the tile kernel, 4096->2x12288 10.9 against 15.6).
+  if (flow_ok) { return finish(vpq::launch_qmv_flow(hs, a)); }
   // Several rows of x: the ring kernel keeps a slice of x in registers for all the tiles of a
   // workgroup (one workgroup per CU, up to 16 / 8 tiles each at 5..8 / 9..16 rows), so x is
   // re-read from L2 once per slice and workgroup instead of once per item (measured at 16 rows:
@@ -1151,6 +1159,9 @@ int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* con
   vpq::QmvGroup g;
   g.count = count;
   for (int i = 0; i < count; ++i) { g.seg[i] = vpq::QmvSeg{w[i], scales[i], biases[i], y[i], N[i]}; }
+  if (mfma_group && vpq::qmv_flow_supports(K, 1, M)) {
+    return finish(vpq::launch_qmv_flow_group(reinterpret_cast<hipStream_t>(stream), a, g));
+  }
   if (!mfma_group) { return finish(vpq::launch_qmv_rows_group(reinterpret_cast<hipStream_t>(stream), a, g)); }
   return finish(vpq::launch_qmv_mfma_group(reinterpret_cast<hipStream_t>(stream), a, g));
 }

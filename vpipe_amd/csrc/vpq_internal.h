@@ -121,6 +121,11 @@ struct QmvGroup {
 };
 hipError_t launch_qmv_mfma_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g);
 size_t qmv_mfma_workspace_bytes(int K, int N, int M);
+// Streaming kernel for M = 1 (K % 512 == 0, K >= 2048, 16-byte aligned scales / biases): one wavefront per
+// (row set, K part), every load requested up front; also as one launch over up to four packs that share x.
+bool qmv_flow_supports(int K, int N, int M);
+hipError_t launch_qmv_flow(hipStream_t st, const QmvArgs& a);
+hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g);
 bool qmv_stream_supports(int K, int N, int M);
 hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);
 bool qmv_ring_supports(int K, int N, int M);
