@@ -10,11 +10,14 @@
 //
 // Order of requests (vector-memory results return in order, so what a multiply needs must have
 // been requested before the codes it goes with):
-//   1. scales and biases of the wavefront's rows and K range: 16-byte direct-to-LDS loads
-//      (1 KB per instruction, scales and biases in the same instruction where they fit);
-//   2. the lane's 32 values of x per slice (kept in registers for all rows, as packed pairs,
-//      with their fp32 sum);
-//   3. the codes, RB * SPW loads of 16 bytes per lane.
+//   1. x of the workgroup's K range, by direct-to-LDS loads shared between its wavefronts (a
+//      wavefront then keeps its lanes' 32 values per slice in registers for all rows, as packed
+//      pairs, with their fp32 sum);
+//   2. the codes, RB * SPW loads of 16 bytes per lane, as soon as their addresses are known:
+//      the time to the first code request is paid by every wavefront of the launch;
+//   3. scales and biases of the wavefront's rows and K range: 16-byte direct-to-LDS loads
+//      (1 KB per instruction, scales and biases in the same instruction where they fit).  They
+//      are applied to the per-(row, slice) dot products at the end.
 // The loads are inline assembly so that the only waits are the counted ones written here: the
 // compiler would otherwise wait for every outstanding load before the first LDS read.
 //
@@ -25,6 +28,7 @@
 //     y += s * dot + (b - 128 * s) * sx
 // per row and slice (a lane's 32 values lie in one quantization group), one wave reduction per
 // row at the end.
+#include <mutex>
 #include <type_traits>
 
 #include "vpq_device.h"
@@ -39,6 +43,7 @@ typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 
 constexpr int kSlice = 2048;          // values of K per slice (64 lanes x 32)
 constexpr int kMaxWavesPerWg = 8;
+constexpr int kMaxLdsBytes = 96 * 1024;   // x of the K range + the scale/bias windows; K <= 32768 fits
 
 __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c)
 {
@@ -111,45 +116,98 @@ struct FlowSeg {
   const uint16_t* biases;
   void* y;
   int N;
-  int first_block;
 };
 
-struct FlowParams {
-  int count;
-  FlowSeg seg[4];
+// Kernel arguments.  The single-pack form is 64 bytes, one cache line of the argument buffer: every wavefront of
+// the launch waits for its arguments before its first request, and each further line costs a quarter of a
+// microsecond on layer-sized packs.
+struct FlowHead {
   const uint16_t* x;
   const uint16_t* residual;
   int K;
-  int wk;          // wavefronts that share a row set (K parts)
-  int wr;          // row sets per workgroup
-  int gate_act;
+  // bits 0-23: 3 bits per wavefront of a workgroup, its row set (wavefront = row set * wk + K part);
+  // 24-25: wk - 1 (wavefronts that share a row set); 26-28: wr - 1 (row sets per workgroup); 29-30: gate_act
+  uint32_t shape;
 };
+// C packs that share x; pack i owns the workgroups from first_block[i] on (first_block[0] = 0).
+template <int C>
+struct FlowParams {
+  FlowHead h;
+  const uint32_t* w[C];
+  const uint16_t* scales[C];
+  const uint16_t* biases[C];
+  void* y[C];
+  int N[C];
+  int first_block[C];
+};
+static_assert(sizeof(FlowParams<1>) == 64, "single-pack arguments: one line");
+static_assert(sizeof(FlowParams<2>) <= 128, "two packs: two lines");
+
+// Forces a kernel argument into scalar registers here, so that all argument loads go out together at the
+// top of the kernel instead of one round trip per first use.
+template <typename T>
+__device__ __forceinline__ void pin_scalar(const T& v) { asm volatile("" : : "s"(v)); }
 
 }  // namespace
 
-template <int SPW, int RB, bool F32OUT>
-__global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const FlowParams p)
+
+// XM: how x reaches a wavefront's registers.
+//   kXOwn     each wavefront loads its own lanes' values (4 KB per slice and wavefront, from L2 after the first
+//             wavefront); scales and biases are requested first, x second, the codes last; no barrier.
+//   kXShared  the workgroup's K range of x is copied to LDS once by direct-to-LDS loads shared between its
+//             wavefronts (one barrier); the codes are requested right after the wavefront's share of x, scales and
+//             biases last.  Pays where a row set's x is large against its codes (long K).
+// Either way the scales and biases are applied to the per-(row, slice) dot products at the end, in the same order:
+// the two modes give the same bits.
+constexpr int kXOwn = 0, kXShared = 1;
+
+template <int SPW, int RB, bool F32OUT, int XM, int C>
+__global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const FlowParams<C> p)
 {
   constexpr int NL = RB * SPW;                 // code loads of a wavefront
   constexpr int PPR = SPW * 4;                 // 16-byte pieces of scales (or biases) per row and K part
   constexpr int P = RB * PPR;
   constexpr int NDMA = (2 * P + 63) / 64;
-  __shared__ __attribute__((aligned(16))) uint8_t sb_lds[kMaxWavesPerWg * NDMA * 1024];
-  __shared__ float red[kMaxWavesPerWg * RB];
+  // LDS: [kXShared: x of the workgroup's K range, wk * SPW slices of 4 KB,] one window of scales/biases per
+  // wavefront, the row sums of the K parts.
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-  FlowSeg sg = p.seg[0];
-#pragma unroll
-  for (int i = 1; i < 4; ++i) {
-    if (i < p.count && (int)blockIdx.x >= p.seg[i].first_block) { sg = p.seg[i]; }
-  }
+  // ---- arguments: everything in one batch of scalar loads, the segment chosen without branches
+  const uint16_t* xg = p.h.x;
+  const uint16_t* residual = p.h.residual;
+  const int K = p.h.K;
+  const uint32_t shape = p.h.shape;
+  pin_scalar(xg); pin_scalar(residual); pin_scalar(K); pin_scalar(shape);
+  const int blk = (int)blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rs = wave / p.wk, part = wave - rs * p.wk;
-  const int K = p.K, N = sg.N;
+  const uint32_t* w_[C]; const uint16_t* s_[C]; const uint16_t* b_[C]; void* y_[C]; int n_[C], fb_[C];
+#pragma unroll
+  for (int i = 0; i < C; ++i) {
+    w_[i] = p.w[i]; s_[i] = p.scales[i]; b_[i] = p.biases[i]; y_[i] = p.y[i]; n_[i] = p.N[i]; fb_[i] = p.first_block[i];
+    pin_scalar(w_[i]); pin_scalar(s_[i]); pin_scalar(b_[i]); pin_scalar(y_[i]); pin_scalar(n_[i]); pin_scalar(fb_[i]);
+  }
+  const uint32_t* wq = w_[0]; const uint16_t* sq = s_[0]; const uint16_t* bq = b_[0]; void* yq = y_[0];
+  int N = n_[0], first_block = 0;
+#pragma unroll
+  for (int i = 1; i < C; ++i) {
+    const bool take = blk >= fb_[i];
+    wq = take ? w_[i] : wq; sq = take ? s_[i] : sq; bq = take ? b_[i] : bq; yq = take ? y_[i] : yq;
+    N = take ? n_[i] : N; first_block = take ? fb_[i] : first_block;
+  }
+  const int wk = (int)((shape >> 24) & 3u) + 1, wr = (int)((shape >> 26) & 7u) + 1, gate_act = (int)((shape >> 29) & 3u);
+
+  const int rs = (int)((shape >> (3 * wave)) & 7u), part = wave - rs * wk;
+  const int W = wk * wr;
   const int Kg = K >> 6;
-  const int row_begin = (((int)blockIdx.x - sg.first_block) * p.wr + rs) * RB;
+  const int row_begin = ((blk - first_block) * wr + rs) * RB;
   const bool active = row_begin < N;           // wave-uniform
+  if (XM == kXOwn && wk == 1 && !active) { return; }
   const int slice0 = part * SPW;
+  const int x_bytes = XM == kXShared ? wk * SPW * (kSlice * 2) : 0;
+  uint8_t* sbl = lds + x_bytes + wave * (NDMA * 1024);
+  float* red = reinterpret_cast<float*>(lds + x_bytes + W * (NDMA * 1024));
+  const uint32_t lds_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds;
 
   uint32_t magic = 0x43004300u;                // bf16 128.0 in both halves
   uint32_t mask = 0x000f000fu;
@@ -157,26 +215,15 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
   asm volatile("" : "+s"(mask));               // that each pair costs one v_and_or_b32
   const uint32_t ones = 0x3f803f80u;           // bf16 1.0 twice
 
-  float tot[RB];
+  bool kvalid[SPW];
 #pragma unroll
-  for (int r = 0; r < RB; ++r) { tot[r] = 0.0f; }
+  for (int s = 0; s < SPW; ++s) { kvalid[s] = (slice0 + s) * kSlice + lane * 32 < K; }
 
-  if (active) {
-    bool kvalid[SPW];
-    uint32_t koff[SPW];                        // byte offset of the lane's 16 bytes in a row of codes
-#pragma unroll
-    for (int s = 0; s < SPW; ++s) {
-      const int k0 = (slice0 + s) * kSlice + lane * 32;
-      kvalid[s] = k0 < K;
-      koff[s] = kvalid[s] ? (uint32_t)(k0 >> 1) : 0u;
-    }
-
-    // 1. scales and biases -> this wavefront's LDS window: piece i < P is 16 bytes of scales of row
-    // i / PPR, P <= i < 2P the same of the biases; pieces past K re-read the first piece of the part
-    // (finite values; their lanes multiply them by zero).
-    uint8_t* sbl = sb_lds + wave * (NDMA * 1024);
-    const uint32_t sbl_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)sbl;
-    const int g0 = slice0 * 32;                // first group of the part (< Kg for an active part)
+  // Scales and biases -> this wavefront's LDS window: piece i < P is 16 bytes of scales of row i / PPR,
+  // P <= i < 2P the same of the biases; pieces past K re-read the first piece of the part (finite values; their
+  // lanes multiply them by zero).
+  auto request_scales_biases = [&]() {
+    const int g0 = slice0 * 32;                // first group of the part (< Kg: every part holds a slice)
 #pragma unroll
     for (int j = 0; j < NDMA; ++j) {
       int i = lane + 64 * j;
@@ -186,39 +233,73 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
       const int row = i / PPR, pc = i % PPR;
       const int n = (row_begin + row < N) ? (row_begin + row) : (N - 1);
       const int g = (g0 + pc * 8 < Kg) ? (g0 + pc * 8) : g0;
-      const uint16_t* src = (isb ? sg.biases : sg.scales) + (size_t)n * Kg + g;
-      dma16(sbl_a + j * 1024, src);
+      const uint16_t* src = (isb ? bq : sq) + (size_t)n * Kg + g;
+      dma16(lds_a + (uint32_t)(x_bytes + wave * (NDMA * 1024) + j * 1024), src);
     }
-    // 2. x
-    u32x4v xr[SPW][4];
+  };
+
+  u32x4v xr[XM == kXOwn ? SPW : 1][4];
+  if (XM == kXShared) {
+    // x of the workgroup's K range -> LDS, the wavefronts taking the 1 KB pieces round-robin.  Piece j is
+    // quarter t = j % 4 of slice j / 4: lane i brings the 16 bytes at values 32 i + 8 t of the slice, so that a
+    // lane's later reads (its 32 values, quarter by quarter) are one 16-byte word per lane at consecutive
+    // addresses.  Pieces past K re-read the start of x; their lanes use zeros instead.
+    for (int j = wave; j < 4 * wk * SPW; j += W) {
+      const int k = (j >> 2) * kSlice + lane * 32 + (j & 3) * 8;
+      dma16(lds_a + (uint32_t)(j * 1024), xg + (k < K ? k : 0));
+    }
+  } else if (active) {
+    request_scales_biases();
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
       const uint32_t xo = kvalid[s] ? (uint32_t)((slice0 + s) * (kSlice * 2) + lane * 64) : 0u;
 #pragma unroll
-      for (int t = 0; t < 4; ++t) { xr[s][t] = gload16(p.x, xo + t * 16); }
+      for (int t = 0; t < 4; ++t) { xr[s][t] = gload16(xg, xo + t * 16); }
     }
-    // 3. codes
-    u32x4v c[RB][SPW];
-    const uint8_t* wbase = reinterpret_cast<const uint8_t*>(sg.w) + (size_t)row_begin * (size_t)(K >> 1);
+  }
+
+  float tot[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) { tot[r] = 0.0f; }
+
+  // codes
+  constexpr int AFTER = XM == kXShared ? NDMA : 0;     // requests that follow the codes
+  u32x4v c[RB][SPW];
+  if (active) {
+    const uint8_t* wbase = reinterpret_cast<const uint8_t*>(wq) + (size_t)row_begin * (size_t)(K >> 1);
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       const int rr = (row_begin + r < N) ? r : (N - 1 - row_begin);
-      const uint8_t* wr = wbase + (size_t)rr * (size_t)(K >> 1);
+      const uint8_t* wrow = wbase + (size_t)rr * (size_t)(K >> 1);
 #pragma unroll
-      for (int s = 0; s < SPW; ++s) { c[r][s] = gload16(wr, koff[s]); }
+      for (int s = 0; s < SPW; ++s) {
+        const uint32_t koff = kvalid[s] ? (uint32_t)((slice0 + s) * (kSlice / 2) + lane * 16) : 0u;
+        c[r][s] = gload16(wrow, koff);
+      }
     }
+    if (XM == kXShared) { request_scales_biases(); }
+    wait_vm<NL + AFTER>();                       // x (this wavefront's values, or its share) has landed
+  } else if (XM == kXShared) {
+    wait_vm<0>();
+  }
+  if (XM == kXShared) { __syncthreads(); }       // ... and everybody else's share
 
-    wait_vm<NL>();                             // scales, biases and x have landed
-    uint32_t xp[SPW][16];
+  if (active) {
+    uint32_t xp[SPW][16];                        // pairs (x_i, x_{i+4}) of each run of eight
     float sx[SPW];
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
       float sum = 0.0f;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        touch(xr[s][t]);
-        u32x4v d = xr[s][t];
-        if (!kvalid[s]) { d = u32x4v{0u, 0u, 0u, 0u}; }
+        uint4 d;
+        if (XM == kXShared) {
+          d = *reinterpret_cast<const uint4*>(lds + (((slice0 + s) * 4 + t) * 64 + lane) * 16);
+        } else {
+          touch(xr[s][t]);
+          d = make_uint4(xr[s][t].x, xr[s][t].y, xr[s][t].z, xr[s][t].w);
+        }
+        if (!kvalid[s]) { d = make_uint4(0u, 0u, 0u, 0u); }
         xp[s][4 * t + 0] = __builtin_amdgcn_perm(d.z, d.x, 0x05040100u);   // x0,x4
         xp[s][4 * t + 1] = __builtin_amdgcn_perm(d.z, d.x, 0x07060302u);   // x1,x5
         xp[s][4 * t + 2] = __builtin_amdgcn_perm(d.w, d.y, 0x05040100u);   // x2,x6
@@ -230,25 +311,14 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
       }
       sx[s] = sum;
     }
-    uint32_t sraw[RB][SPW], braw[RB][SPW];
-#pragma unroll
-    for (int r = 0; r < RB; ++r) {
-#pragma unroll
-      for (int s = 0; s < SPW; ++s) {
-        const int o = r * (PPR * 16) + s * 64 + (lane >> 1) * 2;
-        sraw[r][s] = *reinterpret_cast<const uint16_t*>(sbl + o);
-        braw[r][s] = *reinterpret_cast<const uint16_t*>(sbl + P * 16 + o);
-      }
-    }
-
-    float acc[RB];
+    // The dot products of every (row, slice) as the codes arrive; scales and biases when everything has landed.
+    float dots[RB][SPW];
     float chain = sx[0];
     static_for<0, RB>([&](auto rc) {
       constexpr int r = decltype(rc)::value;
-      acc[r] = 0.0f;
       static_for<0, SPW>([&](auto sc_) {
         constexpr int s = decltype(sc_)::value;
-        wait_vm_after<NL - 1 - (r * SPW + s)>(chain);
+        wait_vm_after<AFTER + NL - 1 - (r * SPW + s)>(chain);
         touch(c[r][s]);
         const uint32_t cw[4] = {c[r][s].x, c[r][s].y, c[r][s].z, c[r][s].w};
         float d0 = 0.0f, d1 = 0.0f;
@@ -259,19 +329,30 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
           d0 = dot2(xp[s][4 * t + 2], ((cw[t] >> 8) & mask) | magic, d0);
           d1 = dot2(xp[s][4 * t + 3], ((cw[t] >> 12) & mask) | magic, d1);
         }
-        const float sc = bf16_bits_to_f32(sraw[r][s]);
-        const float bi = bf16_bits_to_f32(braw[r][s]);
-        acc[r] = fmaf(sc, d0 + d1, acc[r]);
-        acc[r] = fmaf(fmaf(-128.0f, sc, bi), sx[s], acc[r]);
-        chain = acc[r];
+        dots[r][s] = d0 + d1;                    // sum x * (128 + q)
+        chain = dots[r][s];
       });
     });
+    if (AFTER > 0) { wait_vm_after<0>(chain); }
+    float acc[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      acc[r] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < SPW; ++s) {
+        const int o = r * (PPR * 16) + s * 64 + (lane >> 1) * 2;
+        const float sc = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sbl + o));
+        const float bi = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sbl + P * 16 + o));
+        acc[r] = fmaf(sc, dots[r][s], acc[r]);
+        acc[r] = fmaf(fmaf(-128.0f, sc, bi), sx[s], acc[r]);
+      }
+    }
 #pragma unroll
     for (int r = 0; r < RB; ++r) { tot[r] = wave_total_l63(acc[r]); }
   }
 
   // Row sums of the K parts meet in LDS; the wavefront of part 0 adds them in part order.
-  if (p.wk > 1) {
+  if (wk > 1) {
     if (lane == 63) {
 #pragma unroll
       for (int r = 0; r < RB; ++r) { red[wave * RB + r] = tot[r]; }
@@ -282,25 +363,25 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
 #pragma unroll
       for (int r = 0; r < RB; ++r) {
         float v = tot[r];
-        for (int q = 1; q < p.wk; ++q) { v += red[(wave + q) * RB + r]; }
+        for (int q = 1; q < wk; ++q) { v += red[(wave + q) * RB + r]; }
         tot[r] = v;
       }
     }
   }
   if (!active || lane != 63) { return; }
 
-  if (p.gate_act) {
+  if (gate_act) {
     // rows 2g and 2g+1 are the gate and the up row of feature g; RB is even, so a pair is one wavefront's
 #pragma unroll
     for (int r = 0; r < RB; r += 2) {
       const int n = row_begin + r;
       if (n + 1 < N) {
-        const float v = gated_f32(p.gate_act, tot[r], tot[r + 1]);
+        const float v = gated_f32(gate_act, tot[r], tot[r + 1]);
         const size_t o = (size_t)(n >> 1);
         if (F32OUT) {
-          reinterpret_cast<float*>(sg.y)[o] = v;
+          reinterpret_cast<float*>(yq)[o] = v;
         } else {
-          reinterpret_cast<uint16_t*>(sg.y)[o] = (uint16_t)f32_to_bf16_bits(v);
+          reinterpret_cast<uint16_t*>(yq)[o] = (uint16_t)f32_to_bf16_bits(v);
         }
       }
     }
@@ -311,11 +392,11 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
     const int n = row_begin + r;
     if (n < N) {
       if (F32OUT) {
-        reinterpret_cast<float*>(sg.y)[n] = tot[r];
+        reinterpret_cast<float*>(yq)[n] = tot[r];
       } else {
         uint32_t v = f32_to_bf16_bits(tot[r]);
-        if (p.residual != nullptr) { v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(p.residual[n])); }
-        reinterpret_cast<uint16_t*>(sg.y)[n] = (uint16_t)v;
+        if (residual != nullptr) { v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(residual[n])); }
+        reinterpret_cast<uint16_t*>(yq)[n] = (uint16_t)v;
       }
     }
   }
@@ -325,103 +406,135 @@ namespace {
 
 struct FlowPlan {
   int spw, wk, wr, rb;
+  int xm;          // kXOwn or kXShared
 };
 
-// Slices per wavefront and K parts: the fewest idle slice slots, then the fewest parts.
+// Slices per wavefront and K parts, from measurements on MI355X with HBM-cold packs: up to three slices (K <= 6144)
+// a wavefront walks the whole K; longer rows are split between 2 to 4 wavefronts of the workgroup (12288->4096:
+// 7.5 us as 2 parts x 3 slices x 4 rows against 8.0 as one part of 6 slices).  Four wavefronts per workgroup; two
+// rows per wavefront on small packs (more, shorter wavefronts spread the pack over the CUs sooner), four on large
+// ones; x shared through LDS.
 FlowPlan flow_plan(int K, double pack_bytes)
 {
   const int slices = (K + kSlice - 1) / kSlice;
-  FlowPlan best{0, 0, 0, 0};
-  int best_waste = 1 << 30;
-  for (int spw = 4; spw >= 1; --spw) {
-    const int wk = (slices + spw - 1) / spw;
-    if (wk > kMaxWavesPerWg) { continue; }
-    const int waste = wk * spw - slices;
-    if (waste < best_waste) {
-      best_waste = waste;
-      best.spw = spw;
-      best.wk = wk;
-    }
-  }
-  if (best.spw == 0) { return best; }
-  int wr = 4 / best.wk;
-  if (wr < 1) { wr = 1; }
-  if (best.wk == 3) { wr = 2; }
-  best.wr = wr;
-  // Rows per wavefront: 8 to 12 code loads in flight per wavefront on layer-sized packs; fewer on small
-  // ones, where more wavefronts spread the pack over the CUs.
-  best.rb = (best.spw <= 2 && pack_bytes >= 12e6) ? 4 : 2;
-  return best;
+  FlowPlan pl{0, 0, 0, 0, kXShared};
+  pl.wk = slices <= 3 ? 1 : (slices + 3) / 4;
+  if (pl.wk == 1 && slices > 3) { pl.wk = 2; }
+  if (slices > 3 && slices <= 8) { pl.wk = 2; }
+  if (pl.wk > 4) { return pl; }
+  pl.spw = (slices + pl.wk - 1) / pl.wk;
+  pl.wr = pl.wk == 1 ? 4 : 2;
+  pl.rb = pl.wk == 1 ? ((pl.spw <= 2 && pack_bytes >= 40e6) ? 4 : 2) : (pack_bytes >= 20e6 ? 4 : 2);
+  return pl;
 }
 
-hipError_t launch_flow(hipStream_t st, FlowParams& p, const QmvArgs& a, double pack_bytes, const FlowPlan* forced)
+template <int S, int R, bool F32, int XM, int C>
+hipError_t launch_flow_kernel(dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st, const FlowParams<C>& p)
 {
-  const FlowPlan pl = forced != nullptr ? *forced : flow_plan(a.K, pack_bytes);
-  if (pl.spw == 0 || pl.wk * pl.wr > kMaxWavesPerWg || pl.wk * pl.spw * kSlice < a.K) { return hipErrorInvalidValue; }
-  p.x = a.x;
-  p.K = a.K;
-  p.wk = pl.wk;
-  p.wr = pl.wr;
-  const int rows_per_block = pl.wr * pl.rb;
+  const auto kern = qmv_flow_kernel<S, R, F32, XM, C>;
+  static std::once_flag once;          // one per instantiation
+  static hipError_t attr_status = hipSuccess;
+  std::call_once(once, [&] {
+    attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      kMaxLdsBytes);
+  });
+  if (attr_status != hipSuccess) { return attr_status; }
+  return launch_kernel(kern, grid, block, lds_bytes, st, p);
+}
+
+template <int C>
+hipError_t dispatch_flow(const FlowPlan& pl, bool y_f32, const FlowHead& h, const FlowSeg* segs, int rows_per_block,
+                         dim3 block, size_t lds_bytes, hipStream_t st)
+{
+  FlowParams<C> p;
+  p.h = h;
   int blocks = 0;
-  for (int i = 0; i < p.count; ++i) {
-    p.seg[i].first_block = blocks;
-    blocks += (p.seg[i].N + rows_per_block - 1) / rows_per_block;
+  for (int i = 0; i < C; ++i) {
+    p.w[i] = segs[i].w; p.scales[i] = segs[i].scales; p.biases[i] = segs[i].biases; p.y[i] = segs[i].y; p.N[i] = segs[i].N;
+    p.first_block[i] = blocks;
+    blocks += (segs[i].N + rows_per_block - 1) / rows_per_block;
   }
-  const dim3 grid((unsigned)blocks), block((unsigned)(64 * pl.wk * pl.wr));
-#define VPQ_FLOW(S, R)                                                                              \
-  if (pl.spw == S && pl.rb == R) {                                                                  \
-    return a.y_f32 ? launch_kernel(qmv_flow_kernel<S, R, true>, grid, block, 0, st, p)              \
-                   : launch_kernel(qmv_flow_kernel<S, R, false>, grid, block, 0, st, p);            \
+  const dim3 grid((unsigned)blocks);
+#define VPQ_FLOW(S, R)                                                                                          \
+  if (pl.spw == S && pl.rb == R) {                                                                              \
+    if (pl.xm == kXShared) {                                                                                    \
+      return y_f32 ? launch_flow_kernel<S, R, true, kXShared, C>(grid, block, lds_bytes, st, p)            \
+                   : launch_flow_kernel<S, R, false, kXShared, C>(grid, block, lds_bytes, st, p);          \
+    }                                                                                                           \
+    return y_f32 ? launch_flow_kernel<S, R, true, kXOwn, C>(grid, block, lds_bytes, st, p)                 \
+                 : launch_flow_kernel<S, R, false, kXOwn, C>(grid, block, lds_bytes, st, p);               \
   }
-  VPQ_FLOW(1, 2) VPQ_FLOW(2, 2) VPQ_FLOW(3, 2) VPQ_FLOW(4, 2) VPQ_FLOW(6, 2)
+  VPQ_FLOW(1, 2) VPQ_FLOW(2, 2) VPQ_FLOW(3, 2) VPQ_FLOW(4, 2) VPQ_FLOW(5, 2) VPQ_FLOW(6, 2)
   VPQ_FLOW(1, 4) VPQ_FLOW(2, 4) VPQ_FLOW(3, 4) VPQ_FLOW(4, 4)
 #undef VPQ_FLOW
   return hipErrorInvalidValue;
+}
+
+// segs[0 .. count): the packs; count == 1 takes the one-line argument form.
+hipError_t launch_flow(hipStream_t st, const FlowSeg* segs, int count, const QmvArgs& a, double pack_bytes,
+                       const FlowPlan* forced)
+{
+  const FlowPlan pl = forced != nullptr ? *forced : flow_plan(a.K, pack_bytes);
+  if (pl.spw == 0 || pl.wk < 1 || pl.wk > 4 || pl.wr < 1 || pl.wk * pl.wr > kMaxWavesPerWg ||
+      pl.wk * pl.spw * kSlice < a.K || (pl.xm != kXOwn && pl.xm != kXShared)) {
+    return hipErrorInvalidValue;
+  }
+  FlowHead h;
+  h.x = a.x;
+  h.residual = count == 1 ? a.residual : nullptr;
+  h.K = a.K;
+  h.shape = ((uint32_t)(pl.wk - 1) << 24) | ((uint32_t)(pl.wr - 1) << 26) | ((uint32_t)(count == 1 ? a.gate_act : 0) << 29);
+  for (int wv = 0; wv < pl.wk * pl.wr; ++wv) { h.shape |= (uint32_t)(wv / pl.wk) << (3 * wv); }
+  const int rows_per_block = pl.wr * pl.rb;
+  const int W = pl.wk * pl.wr;
+  const int ndma = (2 * pl.rb * pl.spw * 4 + 63) / 64;
+  const size_t lds_bytes = (pl.xm == kXShared ? (size_t)pl.wk * pl.spw * (kSlice * 2) : 0) + (size_t)W * ndma * 1024 +
+                           (size_t)W * pl.rb * sizeof(float);
+  if (lds_bytes > (size_t)kMaxLdsBytes) { return hipErrorInvalidValue; }
+  const dim3 block((unsigned)(64 * W));
+  switch (count) {
+    case 1: return dispatch_flow<1>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st);
+    case 2: return dispatch_flow<2>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st);
+    case 3: return dispatch_flow<3>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st);
+    case 4: return dispatch_flow<4>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 }  // namespace
 
 bool qmv_flow_supports(int K, int N, int M)
 {
-  return M == 1 && N >= 1 && K >= kSlice && K % 512 == 0 && (K + kSlice - 1) / kSlice <= 4 * kMaxWavesPerWg;
+  return M == 1 && N >= 1 && K >= kSlice && K % 512 == 0 && K <= 32768;
 }
 
 hipError_t launch_qmv_flow(hipStream_t st, const QmvArgs& a)
 {
-  FlowParams p{};
-  p.count = 1;
-  p.seg[0] = FlowSeg{a.w, a.scales, a.biases, a.y, a.N, 0};
-  p.residual = a.residual;
-  p.gate_act = a.gate_act;
-  return launch_flow(st, p, a, (double)a.N * (double)a.K * 9.0 / 16.0, nullptr);
+  const FlowSeg seg{a.w, a.scales, a.biases, a.y, a.N};
+  return launch_flow(st, &seg, 1, a, (double)a.N * (double)a.K * 9.0 / 16.0, nullptr);
 }
 
 // Measurement only: the single-pack launch with the plan given (slices per wavefront, K parts, row sets per
-// workgroup, rows per wavefront).
-hipError_t launch_qmv_flow_planned(hipStream_t st, const QmvArgs& a, int spw, int wk, int wr, int rb)
+// workgroup, rows per wavefront, x mode).
+hipError_t launch_qmv_flow_planned(hipStream_t st, const QmvArgs& a, int spw, int wk, int wr, int rb, int xm)
 {
-  FlowParams p{};
-  p.count = 1;
-  p.seg[0] = FlowSeg{a.w, a.scales, a.biases, a.y, a.N, 0};
-  p.residual = a.residual;
-  p.gate_act = a.gate_act;
-  const FlowPlan pl{spw, wk, wr, rb};
-  return launch_flow(st, p, a, 0.0, &pl);
+  const FlowSeg seg{a.w, a.scales, a.biases, a.y, a.N};
+  const FlowPlan pl{spw, wk, wr, rb, xm};
+  return launch_flow(st, &seg, 1, a, 0.0, &pl);
 }
 
 hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g)
 {
-  FlowParams p{};
-  p.count = g.count;
+  FlowSeg segs[4];
   double bytes = 0.0;
   for (int i = 0; i < g.count; ++i) {
-    p.seg[i] = FlowSeg{g.seg[i].w, g.seg[i].scales, g.seg[i].biases, g.seg[i].y, g.seg[i].N, 0};
+    segs[i] = FlowSeg{g.seg[i].w, g.seg[i].scales, g.seg[i].biases, g.seg[i].y, g.seg[i].N};
     bytes += (double)g.seg[i].N * (double)a.K * 9.0 / 16.0;
   }
-  p.residual = nullptr;
-  p.gate_act = 0;
-  return launch_flow(st, p, a, bytes, nullptr);
+  QmvArgs b = a;
+  b.residual = nullptr;
+  b.gate_act = 0;
+  return launch_flow(st, segs, g.count, b, bytes, nullptr);
 }
 
 }  // namespace vpq
