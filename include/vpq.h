@@ -472,6 +472,16 @@ size_t vpq_argmax_workspace_bytes(int V, int rows);
 int vpq_argmax_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, int rows,
                     void* ws, size_t ws_bytes);
 int vpq_argmax_partial_bf16(vpq_stream_t stream, const uint16_t* logits, float* partials, int V, int parts);
+/* The two-stage vpq_argmax_bf16 for callers that cannot allocate or pass a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The slab
+ * pairs go to a static device array of the library (128 KB per GPU, held until the process ends) instead of
+ * `ws`; the call allocates nothing and gives the bits of vpq_argmax_bf16 with a workspace.  rows is limited to
+ * VPQ_ARGMAX_STATIC_MAX_ROWS (more: VPQ_ERR_WORKSPACE, with the limit in vpq_last_device_error()); V is not.
+ * All calls on one GPU share the array: calls that overlap on a GPU (two streams, two threads) race; calls in
+ * stream order on one stream do not.  vpq_init() resolves the array's address for the current device; else the
+ * first call on a device does. */
+#define VPQ_ARGMAX_STATIC_MAX_ROWS 64
+int vpq_argmax_bf16_static(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, int rows);
 int vpq_argmax_combine(vpq_stream_t stream, const float* partials, int32_t* out_id, int parts);
 
 /* ---- 8-bit group-64 twins (w8g64) -------------------------------------------

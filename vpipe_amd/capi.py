@@ -36,6 +36,7 @@ SYMBOLS = [
     ("vpq_linear_workspace_bytes", _sz, [_i, _i, _i]),
     ("vpq_argmax_workspace_bytes", _sz, [_i, _i]),
     ("vpq_argmax_bf16", _i, [_vp, _vp, _vp, _i, _i, _vp, _sz]),
+    ("vpq_argmax_bf16_static", _i, [_vp, _vp, _vp, _i, _i]),
     ("vpq_argmax_partial_bf16", _i, [_vp, _vp, _vp, _i, _i]),
     ("vpq_argmax_combine", _i, [_vp, _vp, _vp, _i]),
     ("vpq_gather_qmv_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i]),
@@ -93,6 +94,10 @@ SYMBOLS = [
     ("vpq_weight_bytes", _sz, [_i, _i]),
     ("vpq_scale_bytes", _sz, [_i, _i]),
 ]
+
+
+VPQ_ERR_WORKSPACE = -4
+VPQ_ARGMAX_STATIC_MAX_ROWS = 64
 
 
 class VpqError(RuntimeError):
@@ -221,6 +226,14 @@ def argmax_bf16(logits, out=None, two_stage=True):
         ws_bytes = L.vpq_argmax_workspace_bytes(V, rows)
         ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=logits.device)
     _check(L.vpq_argmax_bf16(_stream(), _ptr(logits), _ptr(out), V, rows, _ptr(ws), ws_bytes), "vpq_argmax_bf16")
+    return out
+
+
+def argmax_bf16_static(logits, out):
+    """As argmax_bf16(two_stage=True) through the entry point that allocates nothing: `out` (int32 [rows]) is the
+    caller's, the slab pairs go to the library's static device scratch."""
+    rows, V = (1, logits.numel()) if logits.dim() == 1 else logits.shape
+    _check(load().vpq_argmax_bf16_static(_stream(), _ptr(logits), _ptr(out), V, rows), "vpq_argmax_bf16_static")
     return out
 
 

@@ -3,6 +3,7 @@
 #include "../../include/vpq.h"
 
 #include <hip/hip_runtime.h>
+#include <stdio.h>
 #include <string.h>
 
 #include <atomic>
@@ -183,7 +184,16 @@ const char* vpq_status_string(int status)
 
 const char* vpq_last_device_error(void) { return g_last_error; }
 
-int vpq_init(void) { return ensure_init(); }
+int vpq_init(void)
+{
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  // also resolves the static scratch of vpq_argmax_bf16_static for the current device, so that the entry
+  // point itself has no first-call work left
+  float* unused = nullptr;
+  const hipError_t e = vpq::argmax_static_scratch(&unused);
+  return e == hipSuccess ? VPQ_OK : device_error(e);
+}
 
 int vpq_device_cu_count(void) { return g_dev.status.load() == VPQ_OK ? g_dev.cu_count : 0; }
 
@@ -1104,6 +1114,30 @@ int vpq_argmax_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id
   const int e = finish(vpq::launch_argmax_partial(hs, logits, static_cast<float*>(ws), V, rows, parts));
   if (e != VPQ_OK) { return e; }
   return finish(vpq::launch_argmax_combine(hs, static_cast<const float*>(ws), out_id, rows, parts));
+}
+
+int vpq_argmax_bf16_static(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, int rows)
+{
+  if (logits == nullptr || out_id == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (V <= 0 || rows <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (rows > vpq::kArgmaxStaticRows) {
+    snprintf(g_last_error, sizeof(g_last_error), "vpq_argmax_bf16_static: %d rows, the static scratch holds %d", rows,
+             vpq::kArgmaxStaticRows);
+    return VPQ_ERR_WORKSPACE;
+  }
+  if (!aligned(logits, 2) || !aligned(out_id, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  float* partials = nullptr;
+  const hipError_t se = vpq::argmax_static_scratch(&partials);
+  if (se != hipSuccess) { return device_error(se); }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  // Every pair the combine reads is written by this call's first stage: nothing of an earlier call is read,
+  // so nothing has to be cleared.
+  const int parts = vpq::argmax_parts(V);
+  const int e = finish(vpq::launch_argmax_partial(hs, logits, partials, V, rows, parts));
+  if (e != VPQ_OK) { return e; }
+  return finish(vpq::launch_argmax_combine(hs, partials, out_id, rows, parts));
 }
 
 int vpq_argmax_partial_bf16(vpq_stream_t stream, const uint16_t* logits, float* partials, int V, int parts)

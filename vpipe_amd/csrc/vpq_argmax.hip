@@ -9,6 +9,8 @@
 // a contiguous slab of the row to a (value, index) pair, one workgroup per row combines the pairs.
 // Every comparison is "greater, or equal with a lower index", which makes the reduction order
 // irrelevant: the result is exact, not a matter of tolerance.
+#include <mutex>
+
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -17,6 +19,15 @@ namespace vpq {
 namespace {
 
 constexpr int kNoIndex = 0x7fffffff;
+
+// Scratch of the entry point that allocates nothing: (value, index) pairs of up to kArgmaxStaticRows rows x 256
+// slabs, 128 KB per GPU for the life of the process.  In host code this name only stands for the symbol: the
+// memory is reached through the address hipGetSymbolAddress returns for the current device.
+__device__ __align__(256) float scratch[kArgmaxStaticRows * 256 * 2];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
 
 __device__ __forceinline__ void take_better(float& best, int& bi, float v, int i)
 {
@@ -98,6 +109,24 @@ int argmax_parts(int V)
   // about 2048 entries per slab, at most 256 slabs (one combine pass of 256 threads)
   const int p = (V + 2047) / 2048;
   return p < 1 ? 1 : (p > 256 ? 256 : p);
+}
+
+hipError_t argmax_static_scratch(float** out)
+{
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { return e; }
+  if (dev < 0 || dev >= kMaxDevices) { return hipErrorInvalidDevice; }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));     // this device's copy of the array
+    if (e != hipSuccess) { return e; }
+    if (ptr == nullptr) { return hipErrorInvalidSymbol; }
+    g_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return hipSuccess;
 }
 
 hipError_t launch_argmax_row(hipStream_t st, const uint16_t* logits, int* out_id, int V, int rows)

@@ -144,6 +144,10 @@ hipError_t launch_qmv_rows_gather(hipStream_t st, const QmvArgs& a, const int* p
 // wins): one workgroup per row, or slabs into `partials` (two 4-byte slots per slab: value, index)
 // and a combine; argmax_parts(V) is the slab count the size-based entrance uses.
 int argmax_parts(int V);
+// Rows the static scratch of vpq_argmax_bf16_static holds, and its per-device address (resolved once per
+// device, with that device current; allocates nothing).
+constexpr int kArgmaxStaticRows = 64;
+hipError_t argmax_static_scratch(float** out);
 hipError_t launch_argmax_row(hipStream_t st, const uint16_t* logits, int* out_id, int V, int rows);
 hipError_t launch_argmax_partial(hipStream_t st, const uint16_t* logits, float* partials, int V, int rows, int parts);
 hipError_t launch_argmax_combine(hipStream_t st, const float* partials, int* out_id, int rows, int parts);
