@@ -32,11 +32,25 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16
-# HBM-side bytes per decode layer of the default workload (all its QMV launches together),
-# from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE per dispatch).  FETCH_SIZE reads half
-# the bytes of a 256 MiB device-to-device copy on this part, so it is scaled by 2.0; WRITE_SIZE
-# by 1.0.  109.68 MB fetched per layer, writes below the counter's resolution.
-TRAFFIC_PER_LAYER = 109.68e6
+# HBM-side bytes per decode layer of the default workload (all its QMV launches together) come from the
+# committed summary of two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE per dispatch, scaled by what the
+# same counters read for a device-to-device copy of known size); the file states the build it was taken from.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qmv_flow_kernel_decode_layer_m1_hbm_traffic_pmc.txt")
+
+
+def traffic_from_profile():
+    """(bytes per layer, text naming the profiled build) from the committed summary, or (None, None)."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, None
+    val, build = None, None
+    for line in text.splitlines():
+        if line.startswith("traffic_bytes_per_layer:"):
+            val = float(line.split(":", 1)[1])
+        if line.startswith("build:"):
+            build = line.split(":", 1)[1].strip()
+    return val, build
 
 DECODE_LAYER = [("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024), ("o", 4096, 4096),
                 ("gate", 4096, 12288), ("up", 4096, 12288), ("down", 12288, 4096)]
@@ -182,8 +196,9 @@ def main():
         main.wait_stream(side[0])
         project(li, 6)
 
-    def time_steps(layer_pass, steps, use_graph):
-        """ms per step of `steps` passes: one HIP graph replayed between two events (or eager)."""
+    def time_steps(layer_pass, steps, use_graph, repeats=7):
+        """ms per step of `steps` passes: one HIP graph replayed between two events (or eager), the median of
+        `repeats` such timings (and all of them, for the spread)."""
         graph = None
         if use_graph:
             graph = torch.cuda.CUDAGraph()
@@ -192,17 +207,20 @@ def main():
                     layer_pass(i % args.layers)
             graph.replay()                      # untimed: first replay uploads the graph
             torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        if graph is not None:
-            graph.replay()
-        else:
-            for i in range(steps):
-                layer_pass(i % args.layers)
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / steps
+        times = []
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            if graph is not None:
+                graph.replay()
+            else:
+                for i in range(steps):
+                    layer_pass(i % args.layers)
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) / steps)
+        return float(np.median(times)), times
 
     def kernel_durations(layer_pass, launches_per_pass):
         """Per-kernel durations (hipExtLaunchKernel events: kernel start -> end), us [pass, launch]."""
@@ -236,11 +254,70 @@ def main():
     torch.cuda.synchronize()
 
     # ---- timed region ---------------------------------------------------------------
-    ms_per_step = time_steps(layer_pass, args.steps, use_graph)
+    ms_per_step, ms_all = time_steps(layer_pass, args.steps, use_graph)
     value = layer_bytes / (ms_per_step * 1e-3) / 1e9
     launch = ("hipgraph, " if use_graph else "eager, ") + launch_text
     other = "separate" if args.launch != "separate" else "grouped"
-    ms_other = time_steps(modes[other][0], args.steps, use_graph) if args.variant == 0 and not args.only else None
+    ms_other = time_steps(modes[other][0], args.steps, use_graph)[0] if args.variant == 0 and not args.only else None
+
+    # ---- what this GPU gives to ANY kernel at these launch sizes, measured in this run the same way ----
+    # A kernel that only reads (the library's measurement aid: 16-byte loads, all requested up front) over the
+    # same byte counts per launch as the layer's launches, from a rotating buffer larger than the last-level
+    # cache, as the same kind of HIP graph; and a kernel that does nothing.
+    ceilings = None
+    if not args.only:
+        sink = torch.zeros((4,), dtype=torch.int32, device=dev)
+        if launches_per_layer == 4:
+            launch_bytes = [sum(alg_bytes(K, N, 1) for _, K, N in DECODE_LAYER[0:3]), alg_bytes(4096, 4096, 1),
+                            sum(alg_bytes(K, N, 1) for _, K, N in DECODE_LAYER[4:6]), alg_bytes(12288, 4096, 1)]
+        else:
+            launch_bytes = [alg_bytes(K, N, 1) for _, K, N in DECODE_LAYER]
+        launch_bytes = [(b + 15) // 16 * 16 for b in launch_bytes]
+        per_layer = sum(launch_bytes)
+        pool = torch.empty((args.layers * per_layer + 4096,), dtype=torch.uint8, device=dev).random_(generator=gen)
+        base = (pool.data_ptr() + 255) // 256 * 256
+
+        def pass_read(li):
+            off = base + li * per_layer
+            for nb in launch_bytes:
+                st_ = L.vpq_profile_read_kernel(vpipe_amd.capi._stream(), ctypes.c_void_p(off), nb, ctypes.c_void_p(sink.data_ptr()))
+                if st_ != 0:
+                    raise vpipe_amd.VpqError(st_, "vpq_profile_read_kernel")
+                off += nb
+
+        def pass_empty(li):
+            for _ in launch_bytes:
+                L.vpq_profile_empty_kernel(vpipe_amd.capi._stream(), ctypes.c_void_p(sink.data_ptr()))
+
+        for i in range(args.layers):
+            pass_read(i)
+            pass_empty(i)
+        torch.cuda.synchronize()
+        ms_read, _ = time_steps(pass_read, args.steps, use_graph)
+        ms_empty, _ = time_steps(pass_empty, args.steps, use_graph)
+        dur_read = kernel_durations(pass_read, len(launch_bytes))
+        dur_empty = kernel_durations(pass_empty, len(launch_bytes))
+        ceilings = {"read_only_kernel_us_per_layer": round(ms_read * 1e3, 3),
+                    "read_only_kernel_GBps": round(per_layer / (ms_read * 1e-3) / 1e9, 1),
+                    "empty_kernel_us_per_launch_in_graph": round(ms_empty * 1e3 / len(launch_bytes), 3),
+                    "read_only_eager_kernel_us": {"%.1f MB" % (nb / 1e6): round(float(dur_read[:, i].mean()), 3)
+                                                  for i, nb in enumerate(launch_bytes)},
+                    "empty_eager_kernel_us": round(float(dur_empty.mean()), 3),
+                    "bytes_per_launch": launch_bytes}
+        # the lm_head-sized launch (config 3's 5120 -> 151936): one read of 438 MB, eager kernel duration
+        big = alg_bytes(5120, 151936, 1) // 16 * 16
+        bigpool = torch.empty((2 * big + 256,), dtype=torch.uint8, device=dev).random_(generator=gen)
+        bbase = (bigpool.data_ptr() + 255) // 256 * 256
+        L.vpq_profile_enable(8)
+        for i in range(8):
+            L.vpq_profile_read_kernel(vpipe_amd.capi._stream(), ctypes.c_void_p(bbase + (i % 2) * big), big, ctypes.c_void_p(sink.data_ptr()))
+        kb = (ctypes.c_float * 8)()
+        n = L.vpq_profile_read(kb, 8)
+        L.vpq_profile_enable(0)
+        us_big = float(np.median(kb[2:n])) * 1e3
+        ceilings["read_only_eager_kernel_us"]["%.1f MB" % (big / 1e6)] = round(us_big, 2)
+        ceilings["read_only_GBps_at_438MB"] = round(big / (us_big * 1e-6) / 1e9, 1)
+        del pool, bigpool
 
     # ---- roofline of the dominant kernel ------------------------------------------------
     # Every launch of the timed region is the same kernel (qmv_mfma_kernel); its average launch
@@ -260,16 +337,20 @@ def main():
             per_shape[name] = {"K": K, "N": N, "us": round(us, 3),
                                "GBps": round(alg_bytes(K, N, 1) / (us * 1e-6) / 1e9, 1)}
     default_workload = args.variant == 0
+    traffic_layer, traffic_build = traffic_from_profile()
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": TRAFFIC_PER_LAYER / launches_per_layer if default_workload else None,
-                "kernel": "qmv_mfma_kernel (all %d launches of a layer)" % launches_per_layer,
+                "traffic": (traffic_layer / launches_per_layer) if (default_workload and traffic_layer and launches_per_layer == 4) else None,
+                "traffic_profile": ("profiles/" + os.path.basename(TRAFFIC_PROFILE) + " (" + str(traffic_build) + ")") if traffic_layer else None,
+                "kernel": "qmv_flow_kernel (all %d launches of a layer)" % launches_per_layer,
                 "avg_launch_us": round(avg_launch_us, 3),
                 "bytes_per_launch": layer_bytes / launches_per_layer,
                 "launches_timed": args.steps * launches_per_layer,
-                "note": "a do-nothing read of the same 27 MB per launch takes 5.2-5.4 us on this part (launch and "
-                        "first-byte latency), and reads of 0.4-1 GB reach 6.2-6.4 TB/s: the reachable fraction of the "
-                        "8 TB/s peak is 0.64 at this launch size and 0.78-0.80 at any size"}
+                "timing": "median of %d replays of one HIP graph of %d steps; all replays, us per layer: %s"
+                          % (len(ms_all), args.steps, [round(t * 1e3, 3) for t in ms_all])}
+    if ceilings is not None:
+        roofline["measured_ceilings"] = ceilings
+        roofline["frac_of_read_only_kernel"] = round(ceilings["read_only_kernel_us_per_layer"] / (ms_per_step * 1e3), 4)
     if launches_per_layer == 4:
         roofline["eager_launch_us"] = {n: round(float(dur[:, i].mean()), 3)
                                        for i, n in enumerate(("q|k|v", "o", "gate|up", "down"))}
@@ -440,7 +521,7 @@ def main():
         for i in range(args.layers):
             pass_fused_mlp(i)
         torch.cuda.synchronize()
-        ms_f = time_steps(pass_fused_mlp, args.steps, use_graph)
+        ms_f, _ = time_steps(pass_fused_mlp, args.steps, use_graph)
         fm = {"us_per_layer": round(ms_f * 1e3, 3), "GBps": round((layer_bytes - 2 * 12288) / (ms_f * 1e-3) / 1e9, 1),
               "launches_per_layer": 4}
         M = 2048
@@ -645,6 +726,10 @@ def main():
         del batches
 
     # ---- CPU baseline: the oracle's dequant + fp32 matmul on the host cores ------------
+    # The reference's CPU path (quantize-module expansion + plain fp32 dot, OpenMP over output rows) restated in
+    # oracle/vpq_oracle.c, timed here on this box's host cores.  `cpu_baseline` is the headline workload
+    # (config 2); `cpu_baseline_configs` holds configs 1 (the three forms timed separately), 3 (every shape and
+    # M, one call each) and 4-5 (a 64-row subsample of M, scaled linearly: extrapolated).
     if not args.no_cpu:
         from oracle import oracle
         host = []
@@ -665,13 +750,94 @@ def main():
             cpu_pass()
             n_pass += 1
             el = time.perf_counter() - t0
-            if el > 10.0 or n_pass >= 200:
+            if el > 6.0 or n_pass >= 200:
                 break
+        cpu_model = "unknown"
+        try:
+            for line in open("/proc/cpuinfo"):
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+        except OSError:
+            pass
         out["cpu_baseline"] = {"value": round(layer_bytes * n_pass / el / 1e9, 2), "unit": "GB/s",
                                "cores": oracle.num_threads(), "kind": "port",
                                "sample": "%d passes of the same decode-layer set (one layer's weights), "
                                          "dequant to fp32 [N,K] + fp32 dot, OpenMP over N" % n_pass,
-                               "ms_per_step": round(el / n_pass * 1e3, 3)}
+                               "ms_per_step": round(el / n_pass * 1e3, 3),
+                               "nproc": os.cpu_count(), "omp_max_threads": oracle.num_threads(), "cpu_model": cpu_model}
+
+        def timed(fn, min_s=0.25, max_calls=50):
+            fn()
+            t0 = time.perf_counter()
+            n = 0
+            while True:
+                fn()
+                n += 1
+                el = time.perf_counter() - t0
+                if el > min_s or n >= max_calls:
+                    return el / n
+
+        def host_pack(N, K, seed):
+            rng = np.random.default_rng(seed)
+            w = rng.integers(0, 2 ** 32, size=(N, K // 8), dtype=np.uint32)
+            sf = rng.uniform(0.005, 0.02, size=(N, K // 64)).astype(np.float32)
+            s = torch.from_numpy(sf).bfloat16().view(torch.int16).numpy().view(np.uint16)
+            bf = (-8.0 * sf * (1.0 + 0.05 * rng.standard_normal((N, K // 64)))).astype(np.float32)
+            b = torch.from_numpy(bf).bfloat16().view(torch.int16).numpy().view(np.uint16)
+            return w, s, b
+
+        def host_x(M, K, seed):
+            rng = np.random.default_rng(seed)
+            return torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32)).bfloat16().view(torch.int16).numpy().view(np.uint16)
+
+        cfg = {}
+        # config 1: one 4096 -> 4096 QMV, the three forms separately
+        K, N = 4096, 4096
+        w, s, b = host_pack(N, K, 1)
+        x = host_x(1, K, 2)
+        wdeq, xf = np.empty((N, K), dtype=np.float32), np.empty((1, K), dtype=np.float32)
+        t_dq = timed(lambda: oracle.cpu_dequant_f32(w, s, b, K, N, wdeq))
+        t_mv = timed(lambda: oracle.cpu_matmul_f32(wdeq, x, K, N, 1, xf=xf))
+        t_fu = timed(lambda: oracle.cpu_fused_qmv(w, s, b, x, K, N, 1, xf=xf))
+        ab = alg_bytes(K, N, 1)
+        cfg["config1_qmv_4096x4096_m1"] = {
+            "dequant_to_fp32_us": round(t_dq * 1e6, 1), "fp32_gemv_us": round(t_mv * 1e6, 1),
+            "fused_dequant_dot_us": round(t_fu * 1e6, 1),
+            "GBps_dequant_plus_gemv": round(ab / (t_dq + t_mv) / 1e9, 2), "GBps_fused": round(ab / t_fu / 1e9, 2)}
+        # config 3: every shape and M, one call each (the expansion dominates and does not depend on M)
+        c3 = {}
+        for K, N in SMALL_BATCH:
+            w, s, b = host_pack(N, K, 3 + N)
+            wdeq = np.empty((N, K), dtype=np.float32)
+            row = {}
+            for M in (1, 2, 4, 8, 16):
+                x = host_x(M, K, 4 + M)
+                xf = np.empty((M, K), dtype=np.float32)
+                big = N * K > 200e6
+                t = timed(lambda: oracle.cpu_dequant_matmul(w, s, b, x, K, N, M, wdeq=wdeq, xf=xf),
+                          min_s=0.0 if big else 0.1, max_calls=1 if big else 5)
+                row["M=%d" % M] = {"us": round(t * 1e6, 1), "GBps": round(alg_bytes(K, N, M) / t / 1e9, 2)}
+            c3["%d->%d" % (K, N)] = row
+            del w, s, b, wdeq
+        cfg["config3_small_batch"] = c3
+        # configs 4-5: 64 rows of x, scaled to M (extrapolated)
+        for name, shapes, M in (("config4_prefill_m2048", [(K, N) for _, K, N in PREFILL], 2048),
+                                ("config5_dit_m16320", DIT, 16320)):
+            res = {}
+            for K, N in shapes:
+                w, s, b = host_pack(N, K, 5 + N)
+                x = host_x(64, K, 6)
+                wdeq, xf = np.empty((N, K), dtype=np.float32), np.empty((64, K), dtype=np.float32)
+                t_dq = timed(lambda: oracle.cpu_dequant_f32(w, s, b, K, N, wdeq), min_s=0.0, max_calls=1)
+                t_mm = timed(lambda: oracle.cpu_matmul_f32(wdeq, x, K, N, 64, xf=xf), min_s=0.0, max_calls=1)
+                t_full = t_dq + t_mm * (M / 64.0)
+                res["%d->%d" % (K, N)] = {"extrapolated_ms": round(t_full * 1e3, 1),
+                                          "extrapolated_TFLOPs": round(2.0 * M * N * K / t_full / 1e12, 4),
+                                          "measured": "expansion %.1f ms + 64 rows of x %.1f ms, scaled by M/64" % (t_dq * 1e3, t_mm * 1e3)}
+                del w, s, b, wdeq
+            cfg[name] = res
+        out["cpu_baseline_configs"] = cfg
 
     if args.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(generator=gen)

@@ -621,6 +621,12 @@ int vpq_f16_to_bf16(vpq_stream_t stream, const uint16_t* in_f16, uint16_t* out_b
  * thread at a time. */
 int vpq_profile_enable(int max_launches);
 int vpq_profile_read(float* kernel_ms, int capacity);
+/* The yardsticks a benchmark times beside the product's kernels, in the same run and the same way: a kernel that
+ * does nothing (launch + completion), and a kernel that only reads the first `bytes` (>= 16, a multiple of 16 is
+ * read) of `src` with 16-byte loads, eight in flight per thread, all requested before the first is used.  `sink`
+ * (4 bytes of device memory) is never written. */
+int vpq_profile_empty_kernel(vpq_stream_t stream, void* sink);
+int vpq_profile_read_kernel(vpq_stream_t stream, const void* src, size_t bytes, void* sink);
 
 /* Output byte sizes of the packer (generative-models/quantize/affine-quantizer.h:37-40). */
 size_t vpq_weight_bytes(int N, int K);

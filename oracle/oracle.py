@@ -310,5 +310,33 @@ def cpu_dequant_matmul(w, s, b, x, K, N, M, wdeq=None, xf=None):
     return y
 
 
+def cpu_dequant_f32(w, s, b, K, N, wdeq):
+    """Stage 1 of the timed baseline alone: the pack expanded to fp32 [N,K]."""
+    w, s, b = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16)
+    lib().vpo_cpu_dequant_f32(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(wdeq, _f32p), K, N)
+    return wdeq
+
+
+def cpu_matmul_f32(wdeq, x, K, N, M, xf=None):
+    """Stage 2 alone: fp32 dot of every row of the expanded matrix with every row of x, bf16 out."""
+    x = _c(x, np.uint16)
+    if xf is None:
+        xf = np.empty((M, K), dtype=np.float32)
+    y = np.empty((M, N), dtype=np.uint16)
+    lib().vpo_cpu_matmul_f32(_p(wdeq, _f32p), _p(x, _u16p), _p(y, _u16p), _p(xf, _f32p), K, N, M)
+    return y
+
+
+def cpu_fused_qmv(w, s, b, x, K, N, M, xf=None):
+    """The fused form: each weight expanded in a register and multiplied at once."""
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    if xf is None:
+        xf = np.empty((M, K), dtype=np.float32)
+    y = np.empty((M, N), dtype=np.uint16)
+    lib().vpo_cpu_fused_qmv(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y, _u16p), _p(xf, _f32p),
+                            K, N, M)
+    return y
+
+
 def num_threads():
     return int(lib().vpo_num_threads())

@@ -767,6 +767,67 @@ void vpo_cpu_dequant_matmul(const uint32_t* w, const uint16_t* scales, const uin
   }
 }
 
+/* The two stages of the baseline on their own, and the fused form (each weight expanded in a register
+ * and multiplied at once, no fp32 matrix in memory): same expressions, same order of the sum. */
+void vpo_cpu_dequant_f32(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, float* wdeq,
+                         int K, int N)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+#pragma omp parallel for schedule(static)
+  for (long n = 0; n < (long)N; ++n) {
+    float* o = wdeq + (size_t)n * K;
+    for (int j = 0; j < Kw; ++j) {
+      const uint32_t p = w[(size_t)n * Kw + j];
+      const float s = vpo_bf16_to_f32(scales[(size_t)n * Kg + j / 8]);
+      const float b = vpo_bf16_to_f32(biases[(size_t)n * Kg + j / 8]);
+      for (int i = 0; i < 8; ++i) {
+        const float sq = s * (float)((p >> (4 * i)) & 0xfu);
+        o[j * 8 + i] = sq + b;
+      }
+    }
+  }
+}
+
+void vpo_cpu_matmul_f32(const float* wdeq, const uint16_t* x, uint16_t* y, float* xf, int K, int N, int M)
+{
+  for (size_t i = 0; i < (size_t)M * (size_t)K; ++i) { xf[i] = vpo_bf16_to_f32(x[i]); }
+#pragma omp parallel for schedule(static)
+  for (long n = 0; n < (long)N; ++n) {
+    const float* wr = wdeq + (size_t)n * K;
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      const float* xr = xf + m * (size_t)K;
+      float acc = 0.0f;
+#pragma omp simd reduction(+ : acc)
+      for (int k = 0; k < K; ++k) { acc += xr[k] * wr[k]; }
+      y[m * (size_t)N + (size_t)n] = vpo_f32_to_bf16(acc);
+    }
+  }
+}
+
+void vpo_cpu_fused_qmv(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, const uint16_t* x,
+                       uint16_t* y, float* xf, int K, int N, int M)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  for (size_t i = 0; i < (size_t)M * (size_t)K; ++i) { xf[i] = vpo_bf16_to_f32(x[i]); }
+#pragma omp parallel for schedule(static)
+  for (long n = 0; n < (long)N; ++n) {
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      const float* xr = xf + m * (size_t)K;
+      float acc = 0.0f;
+      for (int j = 0; j < Kw; ++j) {
+        const uint32_t p = w[(size_t)n * Kw + j];
+        const float s = vpo_bf16_to_f32(scales[(size_t)n * Kg + j / 8]);
+        const float b = vpo_bf16_to_f32(biases[(size_t)n * Kg + j / 8]);
+        for (int i = 0; i < 8; ++i) {
+          const float sq = s * (float)((p >> (4 * i)) & 0xfu);
+          acc += xr[j * 8 + i] * (sq + b);
+        }
+      }
+      y[m * (size_t)N + (size_t)n] = vpo_f32_to_bf16(acc);
+    }
+  }
+}
+
 #ifdef _OPENMP
 #include <omp.h>
 int vpo_num_threads(void) { return omp_get_max_threads(); }

@@ -9,15 +9,16 @@ Tolerances (written once, used by every GPU test):
     the fp32 and float64 sums may sit on either side of a rounding boundary);
     every element that is not tiny against the rms within one bf16 ulp of
     bf16_rne(oracle); at most 2% of elements differing from it at all; rel-L2
-    against the float64 oracle <= 2e-3 plus the noise of one bf16 store
-    (2^-9 / sqrt(3) ~ 1.1e-3).
+    against the float64 oracle <= 2e-3 on outputs of 256 elements or more (the
+    noise of one bf16 store alone is ~1.6e-3 rms; smaller outputs add the 2^-8
+    worst case of a single rounding).
 """
 import numpy as np
 
 from vpipe_amd import synth
 
 F32_TOL = 2e-3
-REL_L2_TOL = 2e-3 + 1.2e-3
+REL_L2_TOL = 2e-3
 
 
 def floor_rel_err(got, ref64):
@@ -77,7 +78,11 @@ def check_bf16(got_bits, ref64, ref_bits=None, mismatch_over_all=True):
     mismatch = float((counted != 0).mean()) if counted.size else 0.0
     assert mismatch <= 0.02, "bf16 output differs from bf16(oracle) on %.2f%% of elements" % (100 * mismatch)
     r = rel_l2(got, ref64)
-    assert r <= REL_L2_TOL, "rel-L2 %.3e" % r
+    # One bf16 store alone is worth ~1.6e-3 rms (up to 2^-8 on a single element), so below a few hundred
+    # elements the sample's own rounding noise can pass 2e-3: there the single-rounding worst case is added
+    # (the per-element bounds above are what binds on tiny outputs).
+    tol = REL_L2_TOL if got.size >= 256 else REL_L2_TOL + 2.0 ** -8
+    assert r <= tol, "rel-L2 %.3e" % r
     return mismatch, r
 
 

@@ -127,6 +127,55 @@ def test_qmv_row_streaming_kernel(vpq, oracle, dev, D, K, N, M):
     assert np.array_equal(got, want)
 
 
+def _packer_case(kind, N, K, seed):
+    """bf16-representable fp32 weights that exercise one corner of affine_quant_w4_g64
+    (gpu-kernels/metal/quant/affine_dequant.metal:243-285)."""
+    rng = np.random.default_rng(seed)
+    if kind == "gauss":
+        v = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    elif kind == "ties":
+        # mn = 0, mx = 15 in every group, so scale = 1 exactly and values at j + 0.5 sit on rounding ties:
+        # Metal's round() takes them away from zero
+        v = rng.integers(0, 31, size=(N, K)).astype(np.float32) * 0.5
+        v[:, 0::64] = 0.0
+        v[:, 1::64] = 15.0
+    elif kind == "constant":
+        # constant groups: scale 0, inv 0, every code 0; every other group is ordinary
+        v = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+        for g in range(0, K // 64, 2):
+            v[:, g * 64:(g + 1) * 64] = rng.standard_normal((N, 1)).astype(np.float32)
+    elif kind == "outliers":
+        v = (rng.standard_normal((N, K)) * 0.02).astype(np.float32)
+        v[rng.random((N, K)) < 0.01] *= 40.0
+    else:
+        raise ValueError(kind)
+    return synth.bf16_bits_to_f32(synth.f32_to_bf16_bits(v))
+
+
+@pytest.mark.parametrize("kind,N,K,clip", [
+    ("gauss", 96, 1024, 1.0), ("gauss", 4096, 4096, 1.0), ("gauss", 33, 320, 0.9), ("outliers", 257, 2048, 0.75),
+    ("ties", 64, 512, 1.0), ("constant", 48, 1024, 1.0), ("constant", 48, 1024, 0.8), ("gauss", 1, 64, 1.0),
+])
+def test_packer_matches_the_oracle_bit_for_bit(vpq, oracle, dev, D, kind, N, K, clip):
+    # codes, F16 scales and F16 zero points of the device packer == the CPU restatement, for clipped ranges,
+    # exact rounding ties, constant groups (scale 0) and a layer-sized matrix
+    v = _packer_case(kind, N, K, 600 + N + K)
+    codes, s16, b16 = oracle.quantize(v, K, N, clip=clip)
+    wd, sd, bd = vpq.quantize_w4g64(D.bf16(synth.f32_to_bf16_bits(v), dev), K, N, clip=clip)
+    torch.cuda.synchronize()
+    assert np.array_equal(wd.cpu().numpy().view(np.uint32), codes)
+    assert np.array_equal(sd.cpu().numpy().view(np.uint16), s16)
+    assert np.array_equal(bd.cpu().numpy().view(np.uint16), b16)
+    if kind == "ties":
+        # the known answer itself: scale 1, zero point 0, code = round-half-away(v)
+        q = (codes[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 15
+        assert np.array_equal(q.reshape(N, K), np.minimum(np.floor(v + 0.5), 15).astype(np.uint32))
+    if kind == "constant":
+        q = (codes[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 15
+        assert not q.reshape(N, K // 64, 64)[:, 0::2].any()
+        assert not s16.reshape(N, K // 64)[:, 0::2].any()
+
+
 FLOW_SHAPES = [
     # K, N: one to nine slices of 2048, K not a multiple of 2048 (idle lanes in the last slice), every plan of
     # slices per wavefront x K parts (2560: 2x1, 4096: 2x1, 5120: 3x1, 8192: 4x1, 12288: 3x2, 14336: 4x2, 17408: 3x3),
@@ -313,6 +362,27 @@ def test_qmv_batched_rows_are_independent(vpq, oracle, dev, D):
             assert np.array_equal(full[m], one[0]), (variant, m)
 
 
+def test_qmv_ring_rows_are_independent(vpq, oracle, dev, D):
+    # the same contract for the ring kernel, within each of its register forms (2..4, 5..8, 9..16 rows of x):
+    # a row's result depends on that row of x only -- not on its position, not on its neighbours
+    K, N = 2048, 80
+    w, s, b = synth.make_weight(N, K, 79)
+    wd, sd, bd = stage(D, dev, w, s, b)
+    for M in (3, 7, 12):
+        x = synth.make_act(M, K, 80 + M)
+        xd = D.bf16(x, dev)
+        full = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=capi.VPQ_QMV_RING))
+        perm = np.random.default_rng(M).permutation(M)
+        shuffled = D.bits(vpq.qmv_w4g64(wd, sd, bd, D.bf16(x[perm], dev), K, N, M, variant=capi.VPQ_QMV_RING))
+        assert np.array_equal(shuffled, full[perm]), M
+        fewer = D.bits(vpq.qmv_w4g64(wd, sd, bd, D.bf16(x[:M - 1], dev), K, N, M - 1, variant=capi.VPQ_QMV_RING))
+        assert np.array_equal(fewer, full[:M - 1]), M
+        other = x.copy()
+        other[1:] = synth.make_act(M - 1, K, 99 + M)
+        mixed = D.bits(vpq.qmv_w4g64(wd, sd, bd, D.bf16(other, dev), K, N, M, variant=capi.VPQ_QMV_RING))
+        assert np.array_equal(mixed[0], full[0]), M
+
+
 def test_qmv_residual_add(vpq, oracle, dev, D):
     K, N, M = 1024, 48, 2
     w, s, b = synth.make_weight(N, K, 61)
@@ -343,7 +413,7 @@ def test_qmv_decode_layer_shapes_full(vpq, oracle, dev, D, K, N):
 
 
 @pytest.mark.parametrize("K,N", [(5120, 5120), (5120, 17408), (17408, 5120), (5120, 151936)])
-@pytest.mark.parametrize("M", [1, 16])
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 16])
 def test_qmv_small_batch_shapes_row_sample(vpq, oracle, dev, D, K, N, M):
     # full-size launch; the oracle evaluates a sample of output rows (first and last
     # tiles included), since every output row depends on its own weight row only.

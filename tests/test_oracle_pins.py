@@ -620,3 +620,22 @@ def test_grouped_gemm_oracle_with_byte_codes_reduces_to_the_plain_8bit_gemm(orac
         assert np.array_equal(y64[slot], p64[0]) and np.array_equal(yb[slot], pb[0])
         seen += 1
     assert seen == eid.size
+
+
+def test_cpu_baseline_stages_agree_with_the_oracle(oracle):
+    # the timed baseline's pieces (expansion, fp32 dot, fused form) against the float64 oracle and each other
+    K, N, M = 1024, 33, 3
+    w, s, b = synth.make_weight(N, K, 1)
+    x = synth.make_act(M, K, 2)
+    wdeq = np.empty((N, K), dtype=np.float32)
+    oracle.cpu_dequant_f32(w, s, b, K, N, wdeq)
+    assert np.array_equal(wdeq, oracle.dequant_f32(w, s, b, K, N))
+    staged = oracle.cpu_matmul_f32(wdeq, x, K, N, M)
+    whole = oracle.cpu_dequant_matmul(w, s, b, x, K, N, M)
+    fused = oracle.cpu_fused_qmv(w, s, b, x, K, N, M)
+    assert np.array_equal(staged, whole)
+    y64, _ = oracle.qmv(w, s, b, x, K, N, M)
+    for got in (staged, fused):
+        g = synth.bf16_bits_to_f32(got).astype(np.float64)
+        rms = np.sqrt((y64 ** 2).mean())
+        assert (np.abs(g - y64) / np.maximum(np.abs(y64), 1e-2 * rms)).max() < 1e-2

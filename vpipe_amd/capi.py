@@ -91,6 +91,8 @@ SYMBOLS = [
     ("vpq_f16_to_bf16", _i, [_vp, _vp, _vp, _sz]),
     ("vpq_profile_enable", _i, [_i]),
     ("vpq_profile_read", _i, [_vp, _i]),
+    ("vpq_profile_empty_kernel", _i, [_vp, _vp]),
+    ("vpq_profile_read_kernel", _i, [_vp, _vp, _sz, _vp]),
     ("vpq_weight_bytes", _sz, [_i, _i]),
     ("vpq_scale_bytes", _sz, [_i, _i]),
 ]

@@ -137,14 +137,13 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
     if (!stream_ok) { return VPQ_ERR_BAD_SHAPE; }
     return finish(vpq::launch_qmv_stream(hs, a));
   }
-  // Measured on MI355X (HBM-cold weights): the streaming kernel wins once a wavefront can walk a
-  // tile's whole K and the launch is long (lm_head-sized packs); below that the
-  // one-item-per-wavefront kernel finishes sooner.
+  // One row of x: the streaming kernel that requests the whole pack up front (measured, HBM-cold: 4096->12288
+  // 6.8 us against 9.0 for the tile kernel, 4096->2x12288 11.5 against 15.6, the 5120->151936 lm_head 75.6 against
+  // 79.7 for the persistent kernel below).
+  if (flow_ok) { return finish(vpq::launch_qmv_flow(hs, a)); }
+  // Two to four rows over an lm_head-sized pack: persistent workgroups that walk a tile's whole K.
   const double pack_bytes = (double)N * (double)K * 9.0 / 16.0;
   if (stream_ok && pack_bytes >= 150e6) { return finish(vpq::launch_qmv_stream(hs, a)); }
-  // One row of x over a layer-sized pack: the streaming kernel that requests the whole pack up front
-  // (measured, HBM-cold: 4096->12288 6.6 us against 9.0 for the tile kernel, 4096->2x12288 10.9 against 15.6).
-  if (flow_ok) { return finish(vpq::launch_qmv_flow(hs, a)); }
   // Several rows of x: the ring kernel keeps a slice of x in registers for all the tiles of a
   // workgroup (one workgroup per CU, up to 16 / 8 tiles each at 5..8 / 9..16 rows), so x is
   // re-read from L2 once per slice and workgroup instead of once per item (measured at 16 rows:
@@ -1217,6 +1216,25 @@ int vpq_f16_to_bf16(vpq_stream_t stream, const uint16_t* in_f16, uint16_t* out_b
   const int st = ensure_init();
   if (st != VPQ_OK) { return st; }
   return finish(vpq::launch_f16_to_bf16(reinterpret_cast<hipStream_t>(stream), in_f16, out_bf16, count));
+}
+
+int vpq_profile_empty_kernel(vpq_stream_t stream, void* sink)
+{
+  if (sink == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (!aligned(sink, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_profile_empty(reinterpret_cast<hipStream_t>(stream), static_cast<uint32_t*>(sink)));
+}
+
+int vpq_profile_read_kernel(vpq_stream_t stream, const void* src, size_t bytes, void* sink)
+{
+  if (src == nullptr || sink == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (bytes < 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(src, 16) || !aligned(sink, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_profile_read(reinterpret_cast<hipStream_t>(stream), src, bytes, static_cast<uint32_t*>(sink)));
 }
 
 int vpq_profile_enable(int max_launches)

@@ -176,6 +176,9 @@ __global__ __launch_bounds__(64) void quantize_w4g64_kernel(
     mx = fmaxf(mx, v[i]);
   }
   if (clip < 1.0f) {
+    // every product rounded on its own (no fused multiply-add), as the expressions read; the CPU restatement
+    // is built the same way
+#pragma clang fp contract(off)
     const float mid = 0.5f * (mn + mx);
     mn = mid + (mn - mid) * clip;
     mx = mid + (mx - mid) * clip;

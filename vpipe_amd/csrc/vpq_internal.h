@@ -38,6 +38,10 @@ inline hipError_t launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds_byte
   return hipGetLastError();
 }
 
+// Measurement aids (vpq_profile.hip): a kernel that does nothing, a kernel that only reads `bytes` of src.
+hipError_t launch_profile_empty(hipStream_t st, uint32_t* sink);
+hipError_t launch_profile_read(hipStream_t st, const void* src, size_t bytes, uint32_t* sink);
+
 struct QmvArgs {
   const uint32_t* w;
   const uint16_t* scales;
