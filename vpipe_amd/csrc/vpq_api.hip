@@ -338,11 +338,11 @@ int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const
     if (st != VPQ_OK) { return st; }
   }
   std::string why;
-  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, &why);
+  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, g_dev.cu_count, &why);
   if (rc != 0) {
     strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
     g_last_error[sizeof(g_last_error) - 1] = '\0';
-    return rc == -1 ? VPQ_ERR_UNSUPPORTED : VPQ_ERR_DEVICE;
+    return VPQ_ERR_DEVICE;
   }
   return VPQ_OK;
 }
@@ -516,11 +516,11 @@ int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
     if (st != VPQ_OK) { return st; }
   }
   std::string why;
-  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, &why);
+  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, g_dev.cu_count, &why);
   if (rc != 0) {
     strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
     g_last_error[sizeof(g_last_error) - 1] = '\0';
-    return rc == -1 ? VPQ_ERR_UNSUPPORTED : VPQ_ERR_DEVICE;
+    return VPQ_ERR_DEVICE;
   }
   return VPQ_OK;
 }
@@ -597,11 +597,11 @@ int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const 
     if (st != VPQ_OK) { return st; }
   }
   std::string why;
-  const int rc = vpq::dense_gemm_elt(hs, x, w_deq, y, M, N, K, true, &why);
+  const int rc = vpq::dense_gemm_elt(hs, x, w_deq, y, M, N, K, true, g_dev.cu_count, &why);
   if (rc != 0) {
     strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
     g_last_error[sizeof(g_last_error) - 1] = '\0';
-    return rc == -1 ? VPQ_ERR_UNSUPPORTED : VPQ_ERR_DEVICE;
+    return VPQ_ERR_DEVICE;
   }
   return VPQ_OK;
 }
@@ -640,9 +640,8 @@ int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t
   // at M = 16320, expansion included), the reference's own route for large M
   // (generative-models/minimax-h3/metal-minimax-h3-transformer.cc:2020-2160).
   if (ws != nullptr && aligned(ws, 256) && M >= kDenseRouteMinRows && K > 0 && N > 0 && (K % 64) == 0 &&
-      ws_bytes >= (size_t)N * (size_t)K * 2) {
-    const int st = vpq_qmm_dense_route_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, static_cast<uint16_t*>(ws), 1);
-    if (st != VPQ_ERR_UNSUPPORTED) { return st; }      // no vendor BLAS in this process: the fused kernels
+      ws_bytes >= (size_t)N * (size_t)K * 2 && vpq::dense_gemm_supports(M, N, K)) {
+    return vpq_qmm_dense_route_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, static_cast<uint16_t*>(ws), 1);
   }
   // Few tiles and a long K: split K over more workgroups when the caller's workspace has the room.
   if (ws != nullptr && aligned(ws, 256) && K > 0 && N > 0 && M > 0 && (K % 64) == 0 && ensure_init() == VPQ_OK) {
@@ -1083,11 +1082,11 @@ int vpq_qmm_dense_route_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const
     if (st != VPQ_OK) { return st; }
   }
   std::string why;
-  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, &why);
+  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, g_dev.cu_count, &why);
   if (rc != 0) {
     strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
     g_last_error[sizeof(g_last_error) - 1] = '\0';
-    return rc == -1 ? VPQ_ERR_UNSUPPORTED : VPQ_ERR_DEVICE;
+    return VPQ_ERR_DEVICE;
   }
   return VPQ_OK;
 }

@@ -184,12 +184,15 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n);
 int qmm_choose_splits(int K, int N, int M, int cu_count);
 size_t qmm_splitk_workspace_bytes(int K, int N, int M, int cu_count);
 hipError_t launch_qmm_tile_splitk(hipStream_t st, const GemmArgs& a, int splits, float* plane);
-// y[M,N] = x[M,K] . b[N,K]^T on the vendor BLAS (bf16 in, fp32 accumulate, bf16 out).
-// 0, or -1 (rocBLAS unavailable) / -2 (the call failed) with *why set.
-int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,
+// y[M,N] = x[M,K] . b[N,K]^T on the large-tile kernel with dense 2-byte weights (bf16, or binary16 with f16;
+// fp32 accumulate, one rounding).  0, or -2 (shape outside the kernel / launch failed) with *why set.
+bool dense_gemm_supports(int M, int N, int K);
+hipError_t launch_dense_gemm(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,
+                             bool f16, int cu_count);
+int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, int cu_count,
                     std::string* why);
 int dense_gemm_elt(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, bool f16,
-                   std::string* why);
+                   int cu_count, std::string* why);
 // IEEE binary16 element type (the reference's VPIPE_ELT = half build): dense expansion and the general QMV.
 hipError_t launch_dequant_f16(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                               uint16_t* out, int K, int N);

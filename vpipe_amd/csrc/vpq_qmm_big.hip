@@ -105,9 +105,17 @@ __device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* base, uin
 
 }  // namespace
 
-template <int NT, bool LORA>
+// WSRC: where the weight tile comes from.  kPacked4: 4-bit codes + scales + biases, dequantized in the kernel (the
+// fused GEMM).  kDenseBf16 / kDenseF16: p.w is an expanded [N,K] matrix of 2-byte elements that goes to LDS as
+// the x tile does -- the dense matrix-unit GEMM of the dequant-once route
+// (gpu-kernels/metal/gemm/dense_gemm_mma.metal:44-93, 139-140, 195): same tiles, same MFMA stream, no
+// dequantization pieces; any K % 32 == 0.
+constexpr int kPacked4 = 0, kDenseBf16 = 1, kDenseF16 = 2;
+
+template <int NT, bool LORA, int WSRC = kPacked4>
 __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
 {
+  constexpr bool DENSE = WSRC != kPacked4;
   constexpr int BN = 64 * NT;               // weight rows per workgroup
   constexpr int MQ = 4 * NT;                // MFMAs per quarter step (16 of K)
   // One array per stage and operand.
@@ -128,24 +136,30 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   const int tm = band * 8 + in_band % band_h;
   const int tn = in_band / band_h;
   const int m0 = tm * BM, n0 = tn * BN;
-  const int KT = p.K / BK;                  // a multiple of 8 (K % 512 == 0)
+  const int KT = (p.K + BK - 1) / BK;       // packed: a multiple of 8 (K % 512 == 0); dense: the last step may hold 32
+  const int tail_chunks = (p.K & (BK - 1)) >> 3;   // 16-byte chunks of a row in a partial last step (0: none)
 
   // ---- x tile: 8 direct-to-LDS loads per wavefront and step.  Load i of wavefront w covers tile rows
   // (8w + i)*8 .. +8; lane l takes row l/8 and lands at LDS position l%8 of it.
   const uint8_t* xblk = reinterpret_cast<const uint8_t*>(p.x) + (size_t)m0 * p.K * 2;
   uint32_t a_off[8];
+  uint32_t tail_ok = 0;                     // bit i: this lane's chunk of load i exists in a partial last step
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int row = (wave * 8 + i) * 8 + (lane >> 3);
     const int chunk = swz(row, lane & 7);
     const int rg = (m0 + row < p.M) ? row : (p.M - 1 - m0);
     a_off[i] = (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u;
+    if (chunk < tail_chunks) { tail_ok |= 1u << i; }
   }
-  auto issue_x = [&](int step, auto stage_c) {
+  // partial: the step is the last one and holds fewer than 64 values of K (dense weights only)
+  auto issue_x = [&](int step, auto stage_c, bool partial = false) {
     const uint8_t* src = xblk + (size_t)step * (BK * 2);
     const uint32_t dst = lds_addr(decltype(stage_c)::value ? x_lds1 : x_lds0) + wave * (64 * kRow);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { dma16(dst + i * (8 * kRow), src, a_off[i]); }
+    for (int i = 0; i < 8; ++i) {
+      if (!partial || ((tail_ok >> i) & 1u)) { dma16(dst + i * (8 * kRow), src, a_off[i]); }
+    }
   };
   // ---- codes, scales, biases: wavefront w brings in those of rows 64w .. 64w+63 (nothing past BN rows) ----
   const bool dq_wave = wave * 64 < BN;      // wave-uniform
@@ -157,6 +171,24 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     c_off[i] = (uint32_t)rg * (uint32_t)(p.K >> 1) + (uint32_t)(lane & 1) * 16u;
   }
   const uint8_t* wblk = reinterpret_cast<const uint8_t*>(p.w);
+  // dense W tile: as the x tile, rows 64w .. 64w+63 of the tile by wavefront w
+  uint32_t wd_off[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = (wave * 8 + i) * 8 + (lane >> 3);
+    const int chunk = swz(row, lane & 7);
+    const int rg = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
+    wd_off[i] = DENSE ? (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u : 0u;
+  }
+  auto issue_wdense = [&](int step, auto stage_c, bool partial = false) {
+    if (!dq_wave) { return; }
+    const uint8_t* src = wblk + (size_t)step * (BK * 2);
+    const uint32_t dst = lds_addr(decltype(stage_c)::value ? w_lds1 : w_lds0) + wave * (64 * kRow);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (!partial || ((tail_ok >> i) & 1u)) { dma16(dst + i * (8 * kRow), src, wd_off[i]); }   // same rows' swizzle as x
+    }
+  };
   auto issue_codes = [&](int u) {
     if (!dq_wave) { return; }
     const uint8_t* src = wblk + (size_t)u * 32;
@@ -236,9 +268,19 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   // other stage.  Piece P (0..63) of that dequantization is word P/8 of the row step at stage P%8 of
   //   0: split the nibbles   1..4: two values each, fma(s, q, b)   5: pack to bf16   6: store   7: -
   // and the pieces are dealt out evenly over the step's 4 MQ MFMAs.
-  auto compute = [&](auto stage_c, auto fill_c, int s, int ksteps, auto&& loads) {
+  auto mfma = [](const bf16x8& a, const bf16x8& b, const floatx16& c) {
+    if constexpr (WSRC == kDenseF16) {
+      typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+      return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+    } else {
+      return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+  };
+  // NLD: load requests handed out from inside the step's MFMA stream (0: none), one after every other MFMA
+  auto compute = [&](auto stage_c, auto fill_c, auto nld_c, int s, int ksteps, auto&& loads) {
     constexpr int ST = decltype(stage_c)::value;
     constexpr bool FILL = decltype(fill_c)::value;
+    constexpr int NLD = decltype(nld_c)::value;
     const uint8_t* xb = ST ? x_lds1 : x_lds0;
     const uint8_t* wb = ST ? w_lds1 : w_lds0;
     uint8_t* nb = ST ? w_lds0 : w_lds1;                  // W stage of step s+1
@@ -303,14 +345,14 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
         static_for<0, MQ>([&](auto jc) {
           constexpr int J = decltype(jc)::value;
           constexpr int JT = J >> 2, IT = J & 3;
-          acc[JT][IT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[B][JT], xf[B][IT], acc[JT][IT], 0, 0, 0);
+          acc[JT][IT] = mfma(wf[B][JT], xf[B][IT], acc[JT][IT]);
+          constexpr int G = Q * MQ + J;                  // MFMA index within the step
           if constexpr (FILL) {
-            constexpr int G = Q * MQ + J;                // MFMA index within the step
             static_assert(WPT * 8 == 4 * MQ, "one piece per MFMA");
             piece(std::integral_constant<int, G>());
-            // the step's 12 load requests, one after every other MFMA of its first 24
-            if constexpr ((G & 1) == 1 && G < 24) { loads(std::integral_constant<int, (G >> 1)>()); }
           }
+          // the step's load requests, one after every other MFMA from its start
+          if constexpr ((G & 1) == 1 && G < 2 * NLD) { loads(std::integral_constant<int, (G >> 1)>()); }
           // the next quarter's fragments, one read after every MFMA until they are all requested
           if constexpr (Q < 3 && J < 4 + NT) {
             if (Q + 1 < ksteps) { frag(1 - B, Q + 1, J); }
@@ -322,32 +364,40 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   };
 
   // ---- prologue: x(0), the codes of steps 0 and 1, the first block of scales; step 0's W tile ----
-  issue_scales(0);
-  issue_codes(0);
-  issue_codes(1);
-  issue_x(0, S0());
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  wg_barrier();                             // the codes and scales a thread reads were brought in by any wavefront
-  {
-    float sc2[2], bi2[2];
-    uint32_t cw[WPT];
-    load_row_params(0, sc2, bi2, cw);
+  if constexpr (DENSE) {
+    const bool partial0 = KT == 1 && tail_chunks != 0;
+    issue_wdense(0, S0(), partial0);
+    issue_x(0, S0(), partial0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    wg_barrier();
+  } else {
+    issue_scales(0);
+    issue_codes(0);
+    issue_codes(1);
+    issue_x(0, S0());
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    wg_barrier();                             // the codes and scales a thread reads were brought in by any wavefront
+    {
+      float sc2[2], bi2[2];
+      uint32_t cw[WPT];
+      load_row_params(0, sc2, bi2, cw);
 #pragma unroll
-    for (int j = 0; j < WPT; ++j) {
-      const bool second = d_w0 + j >= 8;
-      const float sc = second ? sc2[1] : sc2[0], bi = second ? bi2[1] : bi2[0];
-      uint32_t lo = cw[j] & 0x0f0f0f0fu, hi = (cw[j] >> 4) & 0x0f0f0f0fu;
-      asm volatile("" : "+v"(lo), "+v"(hi));
-      uint4 o;
-      o.x = pack_bf16x2(fmaf(sc, ubyte_f32<0>(lo), bi), fmaf(sc, ubyte_f32<0>(hi), bi));
-      o.y = pack_bf16x2(fmaf(sc, ubyte_f32<1>(lo), bi), fmaf(sc, ubyte_f32<1>(hi), bi));
-      o.z = pack_bf16x2(fmaf(sc, ubyte_f32<2>(lo), bi), fmaf(sc, ubyte_f32<2>(hi), bi));
-      o.w = pack_bf16x2(fmaf(sc, ubyte_f32<3>(lo), bi), fmaf(sc, ubyte_f32<3>(hi), bi));
-      *reinterpret_cast<uint4*>(w_lds0 + b_dst[j]) = o;
+      for (int j = 0; j < WPT; ++j) {
+        const bool second = d_w0 + j >= 8;
+        const float sc = second ? sc2[1] : sc2[0], bi = second ? bi2[1] : bi2[0];
+        uint32_t lo = cw[j] & 0x0f0f0f0fu, hi = (cw[j] >> 4) & 0x0f0f0f0fu;
+        asm volatile("" : "+v"(lo), "+v"(hi));
+        uint4 o;
+        o.x = pack_bf16x2(fmaf(sc, ubyte_f32<0>(lo), bi), fmaf(sc, ubyte_f32<0>(hi), bi));
+        o.y = pack_bf16x2(fmaf(sc, ubyte_f32<1>(lo), bi), fmaf(sc, ubyte_f32<1>(hi), bi));
+        o.z = pack_bf16x2(fmaf(sc, ubyte_f32<2>(lo), bi), fmaf(sc, ubyte_f32<2>(hi), bi));
+        o.w = pack_bf16x2(fmaf(sc, ubyte_f32<3>(lo), bi), fmaf(sc, ubyte_f32<3>(hi), bi));
+        *reinterpret_cast<uint4*>(w_lds0 + b_dst[j]) = o;
+      }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wg_barrier();
   }
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  wg_barrier();
 
   // ---- K loop.  Requests of step s, in issue order: x(s+1) [8], codes(s+2) [2] into the slot step s's
   // codes have left; on steps 8b the scales and biases of block b+1 [2].  Before the barrier x(s+1) and
@@ -377,7 +427,11 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
         if (scales_out) { dma16(sdst + 256 * 16, brow + (size_t)blk * 16); }
       }
     };
-    compute(St(), fill_c, s, 4, loads);
+    if constexpr (decltype(fill_c)::value) {
+      compute(St(), fill_c, std::integral_constant<int, 12>(), s, 4, loads);
+    } else {
+      compute(St(), fill_c, std::integral_constant<int, 0>(), s, 4, loads);
+    }
     if (scales_out) {
       asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
     } else {
@@ -385,14 +439,55 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     }
     wg_barrier();
   };
-  // No condition surrounds the arithmetic inside the loop; the last pair of steps is written out.
-  int s = 0;
-  for (; s + 2 < KT; s += 2) {
+  // Dense weights: x(s+1) [8] and W(s+1) [8] go out from inside step s's MFMA stream; all of them have
+  // landed at the barrier.
+  auto dense_step = [&](auto stage_c, auto more_c, int s) {
+    using St = decltype(stage_c);
+    using Nx = std::integral_constant<int, 1 - St::value>;
+    const uint8_t* xsrc = xblk + (size_t)(s + 1) * (BK * 2);
+    const uint32_t xdst = lds_addr(Nx::value ? x_lds1 : x_lds0) + wave * (64 * kRow);
+    const uint8_t* wsrc = wblk + (size_t)(s + 1) * (BK * 2);
+    const uint32_t wdst = lds_addr(Nx::value ? w_lds1 : w_lds0) + wave * (64 * kRow);
+    const bool next_partial = s + 2 == KT && tail_chunks != 0;     // the step being fetched is a partial last one
+    auto loads = [&](auto ic) {
+      constexpr int I = decltype(ic)::value;
+      if constexpr (I < 8) {
+        if (!next_partial || ((tail_ok >> I) & 1u)) { dma16(xdst + I * (8 * kRow), xsrc, a_off[I]); }
+      } else {
+        if (dq_wave && (!next_partial || ((tail_ok >> (I - 8)) & 1u))) { dma16(wdst + (I - 8) * (8 * kRow), wsrc, wd_off[I - 8]); }
+      }
+    };
+    const int quarters = (s + 1 == KT && tail_chunks != 0) ? (tail_chunks >> 1) : 4;
+    if constexpr (decltype(more_c)::value) {
+      compute(St(), std::false_type(), std::integral_constant<int, 16>(), s, quarters, loads);
+    } else {
+      compute(St(), std::false_type(), std::integral_constant<int, 0>(), s, quarters, loads);
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    wg_barrier();
+  };
+  if constexpr (DENSE) {
+    int s = 0;
+    for (; s + 2 < KT; s += 2) {
+      dense_step(S0(), std::true_type(), s);
+      dense_step(S1(), std::true_type(), s + 1);
+    }
+    if (s + 2 == KT) {
+      dense_step(S0(), std::true_type(), s);
+      dense_step(S1(), std::false_type(), s + 1);
+    } else {
+      dense_step(S0(), std::false_type(), s);
+    }
+  } else {
+    // No condition surrounds the arithmetic inside the loop; the last pair of steps is written out.
+    int s = 0;
+    for (; s + 2 < KT; s += 2) {
+      step(S0(), std::true_type(), s);
+      step(S1(), std::true_type(), s + 1);
+    }
     step(S0(), std::true_type(), s);
-    step(S1(), std::true_type(), s + 1);
+    step(S1(), std::false_type(), s + 1);
   }
-  step(S0(), std::true_type(), s);
-  step(S1(), std::false_type(), s + 1);
 
   if (LORA) {
     // r more values of K from t[M,r] and B[N,r], dense, through stage 0
@@ -425,7 +520,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       wg_barrier();                                    // tiles ready
-      compute(S0(), std::false_type(), 0, chunks >> 1, [](auto) {});
+      compute(S0(), std::false_type(), std::integral_constant<int, 0>(), 0, chunks >> 1, [](auto) {});
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       wg_barrier();                                    // everyone done with them
     }
@@ -460,6 +555,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     }
     return;
   }
+  constexpr bool F16 = WSRC == kDenseF16;
   const bool vec_ok = (p.N & 3) == 0;
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
@@ -476,14 +572,14 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
         const float v2 = acc[jt][it][rq * 4 + 2], v3 = acc[jt][it][rq * 4 + 3];
         if (vec_ok && n + 3 < p.N) {
           uint2 o;
-          o.x = pack_bf16x2(v0, v1);
-          o.y = pack_bf16x2(v2, v3);
+          o.x = pack_elt2<F16>(v0, v1);
+          o.y = pack_elt2<F16>(v2, v3);
           *reinterpret_cast<uint2*>(yrow + n) = o;
         } else {
           const float v[4] = {v0, v1, v2, v3};
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if (n + e < p.N) { yrow[n + e] = (uint16_t)f32_to_bf16_bits(v[e]); }
+            if (n + e < p.N) { yrow[n + e] = (uint16_t)f32_to_elt_bits<F16>(v[e]); }
           }
         }
       }
@@ -549,6 +645,35 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
   }
   return lora ? launch_kernel(qmm_big_kernel<4, true>, grid, block, 0, st, p)
               : launch_kernel(qmm_big_kernel<4, false>, grid, block, 0, st, p);
+}
+
+// y[M,N] = x[M,K] . b[N,K]^T on the large-tile kernel with dense weights (2-byte elements, fp32 accumulation):
+// the contraction stage of the dequant-once route.  K % 32 == 0 (a last K step of 32), 16-byte aligned rows.
+bool dense_gemm_supports(int M, int N, int K)
+{
+  return M >= 1 && N >= 1 && K >= 32 && K % 32 == 0 && (double)N * (double)K * 2.0 < 4.0e9 &&
+         (double)BM * (double)K * 2.0 < 4.0e9;
+}
+
+hipError_t launch_dense_gemm(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,
+                             bool f16, int cu_count)
+{
+  if (!dense_gemm_supports(M, N, K)) { return hipErrorInvalidValue; }
+  const int bn = qmm_big_tile_n(N, M, cu_count);
+  BigParams p{};
+  p.w = reinterpret_cast<const uint32_t*>(b);
+  p.x = x; p.y = y;
+  p.K = K; p.N = N; p.M = M;
+  p.tiles_m = (M + BM - 1) / BM;
+  p.tiles_n = (N + bn - 1) / bn;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kBigThreads);
+#define VPQ_DENSE(NTV)                                                                      \
+  (f16 ? launch_kernel(qmm_big_kernel<NTV, false, kDenseF16>, grid, block, 0, st, p)       \
+       : launch_kernel(qmm_big_kernel<NTV, false, kDenseBf16>, grid, block, 0, st, p))
+  if (bn == 128) { return VPQ_DENSE(2); }
+  if (bn == 192) { return VPQ_DENSE(3); }
+  return VPQ_DENSE(4);
+#undef VPQ_DENSE
 }
 
 }  // namespace vpq
