@@ -373,39 +373,40 @@ def main():
     if ms_other is not None:
         out["us_per_layer_" + other] = round(ms_other * 1e3, 3)
 
-    def dense_gemm_us(w, s, b, x, y, K, N, iters=10):
-        """Yardstick, not product: the vendor library's dense bf16 GEMM (torch.matmul) on the SAME
-        operands with the weight expanded to bf16 beforehand -- what a GEMM with no dequantization
-        at all reaches on this box with these (non-trivial) values."""
-        wdeq = vpipe_amd.dequant_w4g64(w, s, b, K, N)
-        for _ in range(3):
-            torch.matmul(x, wdeq.t(), out=y)
-        torch.cuda.synchronize()
+    def steady_us(fn, iters, warm_ms=40.0):
+        """us per call of fn at the clocks the box settles at: the calls run back to back for warm_ms before the
+        timed ones (the first milliseconds after an idle spell run at lower clocks), then `iters` calls between
+        two events on the stream."""
         t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn()
+        torch.cuda.synchronize()
+        t0.record()
+        fn()
+        t1.record()
+        torch.cuda.synchronize()
+        n_warm = max(2, int(warm_ms / max(t0.elapsed_time(t1), 1e-3)))
+        for _ in range(n_warm):
+            fn()
         t0.record()
         for _ in range(iters):
-            torch.matmul(x, wdeq.t(), out=y)
+            fn()
         t1.record()
         torch.cuda.synchronize()
         return t0.elapsed_time(t1) * 1e3 / iters
 
+    def dense_gemm_us(w, s, b, x, y, K, N, iters=20):
+        """Yardstick, not product: the vendor library's dense bf16 GEMM (torch.matmul) on the SAME
+        operands with the weight expanded to bf16 beforehand -- what a GEMM with no dequantization
+        at all reaches on this box with these (non-trivial) values."""
+        wdeq = vpipe_amd.dequant_w4g64(w, s, b, K, N)
+        return steady_us(lambda: torch.matmul(x, wdeq.t(), out=y), iters)
+
     def dense_route_us(w, s, b, x, y, K, N, M, iters):
-        """The library's own dequant-once route: (expansion + vendor GEMM per call, vendor GEMM alone
+        """The library's own dequant-once route: (expansion + dense GEMM per call, dense GEMM alone
         when the expansion is kept), us per call from events on the stream."""
         wdeq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
-        res = []
-        for expand in (True, False):
-            for _ in range(2):
-                vpipe_amd.qmm_dense_route_w4g64(w, s, b, x, K, N, M, wdeq, expand=expand, out=y)
-            torch.cuda.synchronize()
-            t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            t0.record()
-            for _ in range(iters):
-                vpipe_amd.qmm_dense_route_w4g64(w, s, b, x, K, N, M, wdeq, expand=expand, out=y)
-            t1.record()
-            torch.cuda.synchronize()
-            res.append(t0.elapsed_time(t1) * 1e3 / iters)
-        return res
+        return [steady_us(lambda: vpipe_amd.qmm_dense_route_w4g64(w, s, b, x, K, N, M, wdeq, expand=expand, out=y), iters)
+                for expand in (True, False)]
 
     # ---- QMM at M = 2048 ---------------------------------------------------------------
     if not args.no_qmm:
@@ -416,21 +417,11 @@ def main():
             w, s, b = make_weight(torch, N, K, dev, gen)
             x = torch.randn((M, K), device=dev, generator=gen).bfloat16()
             y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
-            for _ in range(3):
-                vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y)
-            torch.cuda.synchronize()
-            iters = 10
-            L.vpq_profile_enable(iters)
-            for _ in range(iters):
-                vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y)
-            kb = (ctypes.c_float * iters)()
-            n = L.vpq_profile_read(kb, iters)
-            L.vpq_profile_enable(0)
-            us = float(np.mean(kb[:n])) * 1e3
+            us = steady_us(lambda: vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y), 20)
             flops = 2.0 * M * N * K
             qmm[name] = {"K": K, "N": N, "M": M, "us": round(us, 2), "TFLOPs": round(flops / (us * 1e-6) / 1e12, 1),
                          "vendor_dense_bf16_TFLOPs": round(flops / (dense_gemm_us(w, s, b, x, y, K, N) * 1e-6) / 1e12, 1)}
-            dr = dense_route_us(w, s, b, x, y, K, N, M, 10)
+            dr = dense_route_us(w, s, b, x, y, K, N, M, 20)
             qmm[name]["dense_route_TFLOPs"] = round(flops / (dr[0] * 1e-6) / 1e12, 1)
             qmm[name]["dense_route_kept_expansion_TFLOPs"] = round(flops / (dr[1] * 1e-6) / 1e12, 1)
             tot_flops += flops
@@ -442,8 +433,11 @@ def main():
                                "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TF, 4), "traffic": None,
                                "kernel": "qmm_big_kernel<3,false> (4096->12288: 256x192 tiles) and qmm_big_kernel<2,false> "
                                          "(12288->4096, 4096->4096: 256x128 tiles); flops of the three over their time",
+                               "timing": "us per call over 20 back-to-back calls after 40 ms of the same calls "
+                                         "(the clocks the box settles at), events on the stream",
                                "note": "vendor_dense_bf16_TFLOPs in qmm_m2048 = torch.matmul on the expanded "
-                                       "weight, same operands: the dense-GEMM rate this box sustains on real data"}
+                                       "weight, same operands, timed the same way: the dense-GEMM rate this box "
+                                       "sustains on real data"}
 
     # ---- the other configurations, as context (not part of `value`) -----------------------
     if not args.no_extras:
@@ -488,16 +482,16 @@ def main():
             A = (torch.randn((r, K), device=dev, generator=gen) * 0.02).bfloat16()
             B = (torch.randn((N, r), device=dev, generator=gen) * 0.02).bfloat16()
             t = torch.empty((M, r), dtype=torch.bfloat16, device=dev)
-            us0 = kernel_us(lambda i: vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y), 3)
-            us1 = kernel_us(lambda i: vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y, lora_A=A, lora_B=B, r=r,
-                                                         alpha=alpha, t_ws=t), 3)
+            us0 = steady_us(lambda: vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y), 5)
+            us1 = steady_us(lambda: vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y, lora_A=A, lora_B=B, r=r,
+                                                        alpha=alpha, t_ws=t), 5)
             flops = 2.0 * M * N * K
             dit["%d->%d" % (K, N)] = {"us": round(us0, 1), "TFLOPs": round(flops / (us0 * 1e-6) / 1e12, 1),
                                       "us_with_lora": round(us1, 1),
                                       "TFLOPs_with_lora": round(flops / (us1 * 1e-6) / 1e12, 1),
                                       "vendor_dense_bf16_TFLOPs": round(
-                                          flops / (dense_gemm_us(w, s, b, x, y, K, N, iters=3) * 1e-6) / 1e12, 1)}
-            dr = dense_route_us(w, s, b, x, y, K, N, M, 3)
+                                          flops / (dense_gemm_us(w, s, b, x, y, K, N, iters=5) * 1e-6) / 1e12, 1)}
+            dr = dense_route_us(w, s, b, x, y, K, N, M, 5)
             dit["%d->%d" % (K, N)]["dense_route_TFLOPs"] = round(flops / (dr[0] * 1e-6) / 1e12, 1)
             dit["%d->%d" % (K, N)]["dense_route_kept_expansion_TFLOPs"] = round(flops / (dr[1] * 1e-6) / 1e12, 1)
             del w, s, b, x, y, A, B, t
@@ -528,16 +522,7 @@ def main():
         w, s, b = fused[0]
         x = torch.randn((M, 4096), device=dev, generator=gen).bfloat16()
         y = torch.empty((M, 12288), dtype=torch.bfloat16, device=dev)
-        for _ in range(3):
-            vpipe_amd.qmm_swiglu_w4g64(w, s, b, x, 4096, 24576, M, out=y)
-        torch.cuda.synchronize()
-        L.vpq_profile_enable(10)
-        for _ in range(10):
-            vpipe_amd.qmm_swiglu_w4g64(w, s, b, x, 4096, 24576, M, out=y)
-        kb = (ctypes.c_float * 10)()
-        n = L.vpq_profile_read(kb, 10)
-        L.vpq_profile_enable(0)
-        us = float(np.mean(kb[:n])) * 1e3
+        us = steady_us(lambda: vpipe_amd.qmm_swiglu_w4g64(w, s, b, x, 4096, 24576, M, out=y), 20)
         fm["qmm_swiglu_m2048_4096->2x12288"] = {"us": round(us, 2),
                                                "TFLOPs": round(2.0 * M * 24576 * 4096 / (us * 1e-6) / 1e12, 1)}
         out["fused_mlp_swiglu"] = fm

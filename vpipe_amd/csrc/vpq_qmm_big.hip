@@ -66,6 +66,11 @@ __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >>
 template <int I>
 __device__ __forceinline__ float ubyte_f32(uint32_t v) { return (float)((v >> (8 * I)) & 0xffu); }
 
+// `when(c, f)`: f() if c -- decided at compile time for std::true_type / std::false_type, at run time for bool.
+template <typename F> __device__ __forceinline__ void when(std::true_type, F&& f) { f(); }
+template <typename F> __device__ __forceinline__ void when(std::false_type, F&&) {}
+template <typename F> __device__ __forceinline__ void when(bool c, F&& f) { if (c) { f(); } }
+
 template <int I, int N, typename F>
 __device__ __forceinline__ void static_for(F&& f)
 {
@@ -263,11 +268,9 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
 
   using S0 = std::integral_constant<int, 0>;
   using S1 = std::integral_constant<int, 1>;
+  using Yes = std::true_type;
+  using No = std::false_type;
 
-  // One K step: multiplies stage ST while -- with FILL -- the codes of step s+1 become the W tile of the
-  // other stage.  Piece P (0..63) of that dequantization is word P/8 of the row step at stage P%8 of
-  //   0: split the nibbles   1..4: two values each, fma(s, q, b)   5: pack to bf16   6: store   7: -
-  // and the pieces are dealt out evenly over the step's 4 MQ MFMAs.
   auto mfma = [](const bf16x8& a, const bf16x8& b, const floatx16& c) {
     if constexpr (WSRC == kDenseF16) {
       typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
@@ -276,94 +279,154 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
   };
-  // NLD: load requests handed out from inside the step's MFMA stream (0: none), one after every other MFMA
-  auto compute = [&](auto stage_c, auto fill_c, auto nld_c, int s, int ksteps, auto&& loads) {
+
+  // ---- the pipeline.  A step's barrier stands at its 3/4 point, after the MFMAs of quarters 0..2: by then a
+  // wavefront has every fragment of the step in registers and has waited for its own loads, so behind the barrier
+  // the step's stage may be overwritten and the other stage (step s+1: x loaded, W loaded or dequantized) may be
+  // read.  Quarter 3's MFMAs then cover the first fragment reads of step s+1, and the work of the window that
+  // lasts until the next barrier starts under them:
+  //   load requests  x(s+2) [8]; packed: codes(s+3) [2], on steps 8b the scales and biases of block b+1 [2];
+  //                  dense: W(s+2) [8] -- one request every SP MFMAs, all landed at the next barrier;
+  //   packed         the dequantization of W(s+2) into the step's own stage, one piece per MFMA: piece P is word
+  //                  P/8 of the thread's codes at stage P%8 of
+  //                    0: split the nibbles   1..4: two values each, fma(s, q, b)   5: pack to bf16   6: store   7: -
+  // The state of both (fragments, codes, the word in work) lives across steps.
+  constexpr int NLOADS = DENSE ? 16 : 12;
+  constexpr int SP = NT == 2 ? 1 : 2;
+  constexpr int NPRE = (MQ + SP - 1) / SP < NLOADS ? (MQ + SP - 1) / SP : NLOADS;   // requests made under quarter 3
+  bf16x8 wf[2][NT], xf[2][4];                          // operand fragments of the current / the next quarter
+  float sc2[2] = {0.0f, 0.0f}, bi2[2] = {0.0f, 0.0f};  // scale and bias of the thread's one or two rows
+  uint32_t cw[WPT];                                    // its codes of the step being dequantized
+#pragma unroll
+  for (int j = 0; j < WPT; ++j) { cw[j] = 0; }
+  float sc = 0.0f, bi = 0.0f;                          // of the word in work
+  uint32_t lo = 0, hi = 0;
+  float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  uint4 o = make_uint4(0, 0, 0, 0);
+  auto frag = [&](const uint8_t* xb, const uint8_t* wb, int buf, int ks, int idx) {   // idx: 0 = w0, 1..4 = x0..x3, 5.. = w1..
+    const int c = ((2 * ks + fkh) ^ f_sw) * 16;
+    if (idx == 0) {
+      wf[buf][0] = *reinterpret_cast<const bf16x8*>(wb + w_rd[0] + c);
+    } else if (idx <= 4) {
+      xf[buf][idx - 1] = *reinterpret_cast<const bf16x8*>(xb + x_rd[idx - 1] + c);
+    } else {
+      wf[buf][idx - 4] = *reinterpret_cast<const bf16x8*>(wb + w_rd[idx - 4] + c);
+    }
+  };
+  auto piece = [&](auto pc, uint8_t* nb) {
+    constexpr int P = decltype(pc)::value;
+    constexpr int W = P >> 3, S = P & 7;
+    if constexpr (S == 0) {
+      lo = cw[W] & 0x0f0f0f0fu;                        // q0 q2 q4 q6
+      hi = (cw[W] >> 4) & 0x0f0f0f0fu;                 // q1 q3 q5 q7
+      // No instruction: keeps the masked words as they are, so that each value is one v_cvt_f32_ubyteN
+      // of them (otherwise the mask is folded into a bit-field extract per value, one instruction more).
+      asm volatile("" : "+v"(lo), "+v"(hi));
+      if constexpr (NT == 4) {                         // the thread's own row
+        sc = sc2[0]; bi = bi2[0];
+      } else {
+        const bool second = d_w0 + W >= 8;
+        sc = second ? sc2[1] : sc2[0];
+        bi = second ? bi2[1] : bi2[0];
+      }
+    } else if constexpr (S == 1) {
+      v[0] = fmaf(sc, ubyte_f32<0>(lo), bi); v[1] = fmaf(sc, ubyte_f32<0>(hi), bi);
+    } else if constexpr (S == 2) {
+      v[2] = fmaf(sc, ubyte_f32<1>(lo), bi); v[3] = fmaf(sc, ubyte_f32<1>(hi), bi);
+    } else if constexpr (S == 3) {
+      v[4] = fmaf(sc, ubyte_f32<2>(lo), bi); v[5] = fmaf(sc, ubyte_f32<2>(hi), bi);
+    } else if constexpr (S == 4) {
+      v[6] = fmaf(sc, ubyte_f32<3>(lo), bi); v[7] = fmaf(sc, ubyte_f32<3>(hi), bi);
+    } else if constexpr (S == 5) {
+      o.x = pack_bf16x2(v[0], v[1]); o.y = pack_bf16x2(v[2], v[3]);
+      o.z = pack_bf16x2(v[4], v[5]); o.w = pack_bf16x2(v[6], v[7]);
+    } else if constexpr (S == 6) {
+      *reinterpret_cast<uint4*>(nb + b_dst[W]) = o;
+    }
+  };
+  // Request I of the window that opens behind the barrier of step `win`: x(win+2) goes to the stage of step win.
+  auto window_load = [&](auto ic, int win, auto stage_c) {
+    constexpr int I = decltype(ic)::value;
+    constexpr int STG = decltype(stage_c)::value;
+    const int step_to = win + 2;
+    const uint32_t xdst = lds_addr(STG ? x_lds1 : x_lds0) + wave * (64 * kRow);
+    const uint8_t* xsrc = xblk + (size_t)step_to * (BK * 2);
+    if constexpr (DENSE) {
+      const bool partial = tail_chunks != 0 && step_to + 1 == KT;
+      if constexpr (I < 8) {
+        const uint32_t wdst = lds_addr(STG ? w_lds1 : w_lds0) + wave * (64 * kRow);
+        if (dq_wave && (!partial || ((tail_ok >> I) & 1u))) {
+          dma16(wdst + I * (8 * kRow), wblk + (size_t)step_to * (BK * 2), wd_off[I]);
+        }
+      } else {
+        if (!partial || ((tail_ok >> (I - 8)) & 1u)) { dma16(xdst + (I - 8) * (8 * kRow), xsrc, a_off[I - 8]); }
+      }
+    } else {
+      if constexpr (I < 8) {
+        dma16(xdst + I * (8 * kRow), xsrc, a_off[I]);
+      } else if constexpr (I < 10) {                    // codes(win+3) into the slot codes(win+1) have left
+        if (win + 3 < KT && dq_wave) {
+          dma16(lds_addr(c_lds) + (1 - STG) * kCodeBytes + wave * (64 * 32) + (I - 8) * (32 * 32),
+                wblk + (size_t)(win + 3) * 32, c_off[I - 8]);
+        }
+      } else {
+        const int blk = (win >> 3) + 1;
+        if ((win & 7) == 0 && win + 8 < KT && dq_wave) {
+          const uint32_t sdst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave * (64 * 16);
+          if constexpr (I == 10) { dma16(sdst, srow + (size_t)blk * 16); }
+          else { dma16(sdst + 256 * 16, brow + (size_t)blk * 16); }
+        }
+      }
+    }
+  };
+  // Step s on stage ST.  m1: a step s+1 exists, m2: a step s+2 exists (std::true_type / std::false_type, or bool
+  // where the choice is left to run time); `quarters` < 4 only on a last step that holds fewer than 64 values of K
+  // (dense weights).
+  auto pstep = [&](auto stage_c, auto m1, auto m2, int s, int quarters) {
     constexpr int ST = decltype(stage_c)::value;
-    constexpr bool FILL = decltype(fill_c)::value;
-    constexpr int NLD = decltype(nld_c)::value;
+    using Nx = std::integral_constant<int, 1 - ST>;
     const uint8_t* xb = ST ? x_lds1 : x_lds0;
     const uint8_t* wb = ST ? w_lds1 : w_lds0;
-    uint8_t* nb = ST ? w_lds0 : w_lds1;                  // W stage of step s+1
-    const int u = s + 1;
-    float sc2[2] = {0.0f, 0.0f}, bi2[2] = {0.0f, 0.0f};
-    uint32_t cw[WPT];
-#pragma unroll
-    for (int j = 0; j < WPT; ++j) { cw[j] = 0; }
-    if (FILL) { load_row_params(u, sc2, bi2, cw); }
-    float sc = 0.0f, bi = 0.0f;                          // of the word in work
-    bf16x8 wf[2][NT], xf[2][4];                          // operand fragments of the current / the next quarter
-    auto frag = [&](int buf, int ks, int idx) {          // idx: 0 = w0, 1..4 = x0..x3, 5.. = w1..
-      const int c = ((2 * ks + fkh) ^ f_sw) * 16;
-      if (idx == 0) {
-        wf[buf][0] = *reinterpret_cast<const bf16x8*>(wb + w_rd[0] + c);
-      } else if (idx <= 4) {
-        xf[buf][idx - 1] = *reinterpret_cast<const bf16x8*>(xb + x_rd[idx - 1] + c);
-      } else {
-        wf[buf][idx - 4] = *reinterpret_cast<const bf16x8*>(wb + w_rd[idx - 4] + c);
-      }
-    };
-#pragma unroll
-    for (int i = 0; i < 4 + NT; ++i) { frag(0, 0, i); }
-    uint32_t lo = 0, hi = 0;
-    float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    uint4 o = make_uint4(0, 0, 0, 0);
-    auto piece = [&](auto pc) {
-      constexpr int P = decltype(pc)::value;
-      constexpr int W = P >> 3, S = P & 7;
-      if constexpr (S == 0) {
-        lo = cw[W] & 0x0f0f0f0fu;                        // q0 q2 q4 q6
-        hi = (cw[W] >> 4) & 0x0f0f0f0fu;                 // q1 q3 q5 q7
-        // No instruction: keeps the masked words as they are, so that each value is one v_cvt_f32_ubyteN
-        // of them (otherwise the mask is folded into a bit-field extract per value, one instruction more).
-        asm volatile("" : "+v"(lo), "+v"(hi));
-        if constexpr (NT == 4) {                         // the thread's own row
-          sc = sc2[0]; bi = bi2[0];
-        } else {
-          const bool second = d_w0 + W >= 8;
-          sc = second ? sc2[1] : sc2[0];
-          bi = second ? bi2[1] : bi2[0];
-        }
-      } else if constexpr (S == 1) {
-        v[0] = fmaf(sc, ubyte_f32<0>(lo), bi); v[1] = fmaf(sc, ubyte_f32<0>(hi), bi);
-      } else if constexpr (S == 2) {
-        v[2] = fmaf(sc, ubyte_f32<1>(lo), bi); v[3] = fmaf(sc, ubyte_f32<1>(hi), bi);
-      } else if constexpr (S == 3) {
-        v[4] = fmaf(sc, ubyte_f32<2>(lo), bi); v[5] = fmaf(sc, ubyte_f32<2>(hi), bi);
-      } else if constexpr (S == 4) {
-        v[6] = fmaf(sc, ubyte_f32<3>(lo), bi); v[7] = fmaf(sc, ubyte_f32<3>(hi), bi);
-      } else if constexpr (S == 5) {
-        o.x = pack_bf16x2(v[0], v[1]); o.y = pack_bf16x2(v[2], v[3]);
-        o.z = pack_bf16x2(v[4], v[5]); o.w = pack_bf16x2(v[6], v[7]);
-      } else if constexpr (S == 6) {
-        *reinterpret_cast<uint4*>(nb + b_dst[W]) = o;
-      }
-    };
+    const uint8_t* nxb = ST ? x_lds0 : x_lds1;
+    uint8_t* nwb = ST ? w_lds0 : w_lds1;
+    uint8_t* ownb = ST ? w_lds1 : w_lds0;
     static_for<0, 4>([&](auto qc) {
       constexpr int Q = decltype(qc)::value;
       constexpr int B = Q & 1;
-      if (Q < ksteps) {
+      if constexpr (Q == 3 && !DENSE) { when(m2, [&] { load_row_params(s + 2, sc2, bi2, cw); }); }
+      if (Q < quarters) {
         static_for<0, MQ>([&](auto jc) {
           constexpr int J = decltype(jc)::value;
           constexpr int JT = J >> 2, IT = J & 3;
           acc[JT][IT] = mfma(wf[B][JT], xf[B][IT], acc[JT][IT]);
-          constexpr int G = Q * MQ + J;                  // MFMA index within the step
-          if constexpr (FILL) {
-            static_assert(WPT * 8 == 4 * MQ, "one piece per MFMA");
-            piece(std::integral_constant<int, G>());
+          constexpr int GB = Q == 3 ? J : MQ * (Q + 1) + J;    // MFMA slot counted from the previous barrier
+          if constexpr (!DENSE) {
+            if constexpr (Q == 3) { when(m2, [&] { piece(std::integral_constant<int, GB>(), ownb); }); }
+            else { when(m1, [&] { piece(std::integral_constant<int, GB>(), nwb); }); }
           }
-          // the step's load requests, one after every other MFMA from its start
-          if constexpr ((G & 1) == 1 && G < 2 * NLD) { loads(std::integral_constant<int, (G >> 1)>()); }
+          if constexpr (GB % SP == 0 && GB / SP < NLOADS) {
+            if constexpr (Q == 3) { when(m2, [&] { window_load(std::integral_constant<int, GB / SP>(), s, stage_c); }); }
+            else { when(m1, [&] { window_load(std::integral_constant<int, GB / SP>(), s - 1, Nx()); }); }
+          }
           // the next quarter's fragments, one read after every MFMA until they are all requested
-          if constexpr (Q < 3 && J < 4 + NT) {
-            if (Q + 1 < ksteps) { frag(1 - B, Q + 1, J); }
+          if constexpr (J < 4 + NT) {
+            if constexpr (Q < 3) { if (Q + 1 < quarters) { frag(xb, wb, 1 - B, Q + 1, J); } }
+            else { when(m1, [&] { frag(nxb, nwb, 0, 0, J); }); }
           }
           __builtin_amdgcn_sched_barrier(0);
+        });
+      }
+      if constexpr (Q == 2) {
+        when(m1, [&] {
+          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          wg_barrier();
         });
       }
     });
   };
 
-  // ---- prologue: x(0), the codes of steps 0 and 1, the first block of scales; step 0's W tile ----
+  // ---- prologue: stage 0 complete (x(0); W(0) loaded or dequantized), the part of step 1's window that a
+  // quarter 3 before step 0 would have done, the first fragments ----
   if constexpr (DENSE) {
     const bool partial0 = KT == 1 && tail_chunks != 0;
     issue_wdense(0, S0(), partial0);
@@ -377,116 +440,33 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     issue_x(0, S0());
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     wg_barrier();                             // the codes and scales a thread reads were brought in by any wavefront
-    {
-      float sc2[2], bi2[2];
-      uint32_t cw[WPT];
-      load_row_params(0, sc2, bi2, cw);
-#pragma unroll
-      for (int j = 0; j < WPT; ++j) {
-        const bool second = d_w0 + j >= 8;
-        const float sc = second ? sc2[1] : sc2[0], bi = second ? bi2[1] : bi2[0];
-        uint32_t lo = cw[j] & 0x0f0f0f0fu, hi = (cw[j] >> 4) & 0x0f0f0f0fu;
-        asm volatile("" : "+v"(lo), "+v"(hi));
-        uint4 o;
-        o.x = pack_bf16x2(fmaf(sc, ubyte_f32<0>(lo), bi), fmaf(sc, ubyte_f32<0>(hi), bi));
-        o.y = pack_bf16x2(fmaf(sc, ubyte_f32<1>(lo), bi), fmaf(sc, ubyte_f32<1>(hi), bi));
-        o.z = pack_bf16x2(fmaf(sc, ubyte_f32<2>(lo), bi), fmaf(sc, ubyte_f32<2>(hi), bi));
-        o.w = pack_bf16x2(fmaf(sc, ubyte_f32<3>(lo), bi), fmaf(sc, ubyte_f32<3>(hi), bi));
-        *reinterpret_cast<uint4*>(w_lds0 + b_dst[j]) = o;
-      }
-    }
+    load_row_params(0, sc2, bi2, cw);
+    static_for<0, 4 * MQ>([&](auto pc) { piece(pc, w_lds0); });
+    load_row_params(1, sc2, bi2, cw);
+    static_for<0, MQ>([&](auto pc) { piece(pc, w_lds1); });
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     wg_barrier();
   }
+  if (KT > 1) { static_for<0, NPRE>([&](auto ic) { window_load(ic, -1, S1()); }); }
+#pragma unroll
+  for (int i = 0; i < 4 + NT; ++i) { frag(x_lds0, w_lds0, 0, 0, i); }
 
-  // ---- K loop.  Requests of step s, in issue order: x(s+1) [8], codes(s+2) [2] into the slot step s's
-  // codes have left; on steps 8b the scales and biases of block b+1 [2].  Before the barrier x(s+1) and
-  // codes(s+2) must have landed: only the two scale requests may stay in flight (wavefronts that
-  // request no codes or scales wait for everything, which is their x tile).
-  auto step = [&](auto stage_c, auto fill_c, int s) {
-    using St = decltype(stage_c);
-    using Nx = std::integral_constant<int, 1 - St::value>;
-    const bool codes_out = s + 2 < KT && dq_wave;
-    const bool scales_out = St::value == 0 && (s & 7) == 0 && s + 8 < KT && dq_wave;
-    // The requests go out from inside the MFMA stream, in the order x [8], codes [2], scales [2].
-    const uint8_t* xsrc = xblk + (size_t)(s + 1) * (BK * 2);
-    const uint32_t xdst = lds_addr(Nx::value ? x_lds1 : x_lds0) + wave * (64 * kRow);
-    const uint8_t* csrc = wblk + (size_t)(s + 2) * 32;
-    const uint32_t cdst = lds_addr(c_lds) + (s & 1) * kCodeBytes + wave * (64 * 32);
-    const int blk = (s >> 3) + 1;
-    const uint32_t sdst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave * (64 * 16);
-    auto loads = [&](auto ic) {
-      constexpr int I = decltype(ic)::value;
-      if constexpr (I < 8) {
-        dma16(xdst + I * (8 * kRow), xsrc, a_off[I]);
-      } else if constexpr (I < 10) {
-        if (codes_out) { dma16(cdst + (I - 8) * (32 * 32), csrc, c_off[I - 8]); }
-      } else if constexpr (I == 10) {
-        if (scales_out) { dma16(sdst, srow + (size_t)blk * 16); }
-      } else {
-        if (scales_out) { dma16(sdst + 256 * 16, brow + (size_t)blk * 16); }
-      }
-    };
-    if constexpr (decltype(fill_c)::value) {
-      compute(St(), fill_c, std::integral_constant<int, 12>(), s, 4, loads);
-    } else {
-      compute(St(), fill_c, std::integral_constant<int, 0>(), s, 4, loads);
-    }
-    if (scales_out) {
-      asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    }
-    wg_barrier();
-  };
-  // Dense weights: x(s+1) [8] and W(s+1) [8] go out from inside step s's MFMA stream; all of them have
-  // landed at the barrier.
-  auto dense_step = [&](auto stage_c, auto more_c, int s) {
-    using St = decltype(stage_c);
-    using Nx = std::integral_constant<int, 1 - St::value>;
-    const uint8_t* xsrc = xblk + (size_t)(s + 1) * (BK * 2);
-    const uint32_t xdst = lds_addr(Nx::value ? x_lds1 : x_lds0) + wave * (64 * kRow);
-    const uint8_t* wsrc = wblk + (size_t)(s + 1) * (BK * 2);
-    const uint32_t wdst = lds_addr(Nx::value ? w_lds1 : w_lds0) + wave * (64 * kRow);
-    const bool next_partial = s + 2 == KT && tail_chunks != 0;     // the step being fetched is a partial last one
-    auto loads = [&](auto ic) {
-      constexpr int I = decltype(ic)::value;
-      if constexpr (I < 8) {
-        if (!next_partial || ((tail_ok >> I) & 1u)) { dma16(xdst + I * (8 * kRow), xsrc, a_off[I]); }
-      } else {
-        if (dq_wave && (!next_partial || ((tail_ok >> (I - 8)) & 1u))) { dma16(wdst + (I - 8) * (8 * kRow), wsrc, wd_off[I - 8]); }
-      }
-    };
-    const int quarters = (s + 1 == KT && tail_chunks != 0) ? (tail_chunks >> 1) : 4;
-    if constexpr (decltype(more_c)::value) {
-      compute(St(), std::false_type(), std::integral_constant<int, 16>(), s, quarters, loads);
-    } else {
-      compute(St(), std::false_type(), std::integral_constant<int, 0>(), s, quarters, loads);
-    }
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    wg_barrier();
-  };
+  // ---- K loop.  Packed: no condition surrounds the arithmetic inside it, the last two steps are written out
+  // (K is a multiple of 512).  Dense: any number of steps, the conditions are wave-uniform branches. ----
   if constexpr (DENSE) {
-    int s = 0;
-    for (; s + 2 < KT; s += 2) {
-      dense_step(S0(), std::true_type(), s);
-      dense_step(S1(), std::true_type(), s + 1);
-    }
-    if (s + 2 == KT) {
-      dense_step(S0(), std::true_type(), s);
-      dense_step(S1(), std::false_type(), s + 1);
-    } else {
-      dense_step(S0(), std::false_type(), s);
+    const int last_quarters = tail_chunks != 0 ? (tail_chunks >> 1) : 4;
+    for (int s = 0; s < KT; s += 2) {
+      pstep(S0(), s + 1 < KT, s + 2 < KT, s, s + 1 == KT ? last_quarters : 4);
+      if (s + 1 < KT) { pstep(S1(), s + 2 < KT, s + 3 < KT, s + 1, s + 2 == KT ? last_quarters : 4); }
     }
   } else {
-    // No condition surrounds the arithmetic inside the loop; the last pair of steps is written out.
     int s = 0;
-    for (; s + 2 < KT; s += 2) {
-      step(S0(), std::true_type(), s);
-      step(S1(), std::true_type(), s + 1);
+    for (; s + 3 < KT; s += 2) {
+      pstep(S0(), Yes(), Yes(), s, 4);
+      pstep(S1(), Yes(), Yes(), s + 1, 4);
     }
-    step(S0(), std::true_type(), s);
-    step(S1(), std::false_type(), s + 1);
+    pstep(S0(), Yes(), No(), s, 4);
+    pstep(S1(), No(), No(), s + 1, 4);
   }
 
   if (LORA) {
@@ -494,6 +474,8 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     // (gpu-kernels/metal/gemm/dense_gemm_mma.metal:297-348).
     const int steps = (p.r + BK - 1) / BK;
     for (int st = 0; st < steps; ++st) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wg_barrier();                                    // everyone done with stage 0
       const int kleft = p.r - st * BK;                 // >= 32, a multiple of 32
       const int chunks = kleft >= BK ? 8 : (kleft >> 3);
 #pragma unroll
@@ -520,9 +502,9 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       wg_barrier();                                    // tiles ready
-      compute(S0(), std::false_type(), std::integral_constant<int, 0>(), 0, chunks >> 1, [](auto) {});
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      wg_barrier();                                    // everyone done with them
+#pragma unroll
+      for (int i = 0; i < 4 + NT; ++i) { frag(x_lds0, w_lds0, 0, 0, i); }
+      pstep(S0(), No(), No(), 0, chunks >> 1);
     }
   }
 
@@ -556,6 +538,46 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     return;
   }
   constexpr bool F16 = WSRC == kDenseF16;
+  if ((p.N & 7) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0) {
+    // Rows of y in whole 16-byte pieces: each wavefront turns its block round in an LDS region of its own, 32 x
+    // rows at a time -- written as the accumulators lie (lane = x row, 4 consecutive n per register quad), read back
+    // along the rows -- so that a store instruction covers runs of 64 NT bytes per row instead of 16-byte pieces of
+    // 32 rows.  The stages are free by now; one barrier, since other wavefronts may still be reading them.
+    constexpr int kRowBytes = 64 * NT;             // the wavefront's BN/2 columns
+    constexpr int kPitch = kRowBytes + 16;
+    constexpr int LPR = kRowBytes / 16;            // 16-byte pieces per row
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wg_barrier();
+    uint8_t* region = wave == 0 ? x_lds0 : wave == 1 ? x_lds1 : wave == 2 ? w_lds0 : w_lds1;
+    const int ncol0 = n0 + wn * (BN / 2);
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+#pragma unroll
+      for (int jt = 0; jt < NT; ++jt) {
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          uint2 o;
+          o.x = pack_elt2<F16>(acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
+          o.y = pack_elt2<F16>(acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
+          *reinterpret_cast<uint2*>(region + frow * kPitch + (jt * 32 + rq * 8 + fkh * 4) * 2) = o;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int idx0 = 0; idx0 < 32 * LPR; idx0 += 64) {
+        const int idx = idx0 + lane;
+        const int r = idx / LPR, c = idx - r * LPR;
+        const int m = m0 + wm * 128 + it * 32 + r;
+        const int n = ncol0 + c * 8;
+        if (idx < 32 * LPR && m < p.M && n < p.N) {
+          const uint4 q = *reinterpret_cast<const uint4*>(region + r * kPitch + c * 16);
+          *reinterpret_cast<uint4*>(p.y + (size_t)m * p.N + n) = q;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the region is rewritten by the next block
+    }
+    return;
+  }
   const bool vec_ok = (p.N & 3) == 0;
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
