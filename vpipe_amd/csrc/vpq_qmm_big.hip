@@ -11,23 +11,30 @@
 // pipe is busy longer than the matrix pipe.  With one wavefront per SIMD nothing else can fill the
 // matrix pipe's shadow, so every wavefront does all three jobs and the instruction stream itself
 // interleaves them: after each MFMA comes one piece (<= 8 vector instructions) of the
-// dequantization of the NEXT step's weight row and, every other time, one fragment read for the
-// next quarter step, pinned in that order by scheduling barriers.
+// dequantization of a coming step's weight row, one fragment read for the next quarter step and, every
+// SP-th time, one load request, pinned in that order by scheduling barriers.
 //
 // Per 64-wide K step and workgroup, everything arrives by direct-to-LDS loads:
 //   x tile [256,64] bf16      8 loads per wavefront (8 rows x 128 contiguous bytes each);
 //   codes  [BN rows x 32 B]   2 loads per wavefront (32 rows x 32 bytes), into a two-slot ring;
 //   scales, biases            1 load each per wavefront and 8 steps (64 rows x 16 bytes), two slots.
-// The BN x 8 words of a step's codes are dealt out evenly over the 256 threads for dequantization;
-// the step-end barrier, which follows every wavefront's wait for its own loads, stands between a
-// load and its readers.  The loads are written out by hand: the compiler orders every later LDS read after a direct-to-LDS load it
-// knows about, whichever array that load fills, which would serialize the pipeline; hand-written,
-// the only waits in the loop are the explicit ones, counted exactly (requests retire in order).
+// The BN x 8 words of a step's codes are dealt out evenly over the 256 threads for dequantization.
+// The loads are written out by hand: the compiler orders every later LDS read after a direct-to-LDS
+// load it knows about, whichever array that load fills, which would serialize the pipeline;
+// hand-written, the only waits in the loop are the explicit ones.
 // Two LDS stages of x (2 x 32 KB) and of the dequantized W (2 x 32 KB) + the rings (2 x 8 + 2 x 8 KB)
 // are the whole 160 KB.
 //
-// Tiles are walked in bands of 8 rows of tiles, M first inside a band: workgroups go to the 8 XCDs
-// round-robin, so the workgroups an XCD receives while a band lasts read the same 256 rows of x.
+// A step has ONE barrier, at its 3/4 point (after the MFMAs of quarters 0..2, when every fragment of
+// the step is in registers): see the pipeline's comment in the kernel.  Measured on 256 x 256 tiles
+// (cycles per step; 2048 are the MFMAs alone): barrier at the step's end with the first fragment reads
+// behind it 3080, this pipeline 2400-2500 with dense weights, 2900 with the dequantization; what is
+// left over the MFMAs is the issue of the load requests (10-25 cycles each, wherever they stand).
+//
+// Tile order: from two full rounds of the chip on, the 32 workgroups an XCD runs together form a block of
+// tiles (4 x 8, 8 x 4, ...) so that they share rows of x and weight tiles through that XCD's L2; below
+// that, bands of 8 rows of tiles, M first inside a band.  The store goes through LDS, a wavefront's
+// block turned round 32 rows at a time, so that a store instruction covers runs of 64 NT bytes per row.
 #include <type_traits>
 
 #include "vpq_device.h"
@@ -55,6 +62,7 @@ struct BigParams {
   const uint16_t* lora_b;   // [N,r]
   int K, N, M, r;
   int tiles_m, tiles_n;
+  int bmt, bnt, nbn;        // tile blocks per XCD (bmt = 0: bands of 8 rows of tiles), blocks along N
   // Gated store (1 SwiGLU, 2 GEGLU): the pack is an interleaved gate|up matrix and
   // y[m * out_stride + out_off + g] = act(gate_g) * up_g (affine_qmm_steel.metal:663-768, 1460-1572).
   int gate_act, out_stride, out_off;
@@ -134,15 +142,27 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int tile = (int)blockIdx.x;
-  const int band = tile / (8 * p.tiles_n);
-  const int in_band = tile - band * (8 * p.tiles_n);
-  const int band_h = (p.tiles_m - band * 8) < 8 ? (p.tiles_m - band * 8) : 8;
-  const int tm = band * 8 + in_band % band_h;
-  const int tn = in_band / band_h;
+  int tm, tn;
+  if (p.bmt != 0) {
+    // Workgroups go to the 8 XCDs round-robin, 32 at a time each: workgroup i is number (i / 8) % 32 of the
+    // (i / 256)-th set that XCD i % 8 runs.  A set is a block of bmt x bnt tiles, so that the workgroups an XCD
+    // runs together share rows of x (bnt of them each) and weight tiles (bmt each) through that XCD's L2.
+    const int wg = (int)blockIdx.x;
+    const int slot = (wg >> 3) & 31, blk = (wg >> 8) * 8 + (wg & 7);
+    tm = (blk / p.nbn) * p.bmt + slot / p.bnt;
+    tn = (blk % p.nbn) * p.bnt + slot % p.bnt;
+    if (tm >= p.tiles_m || tn >= p.tiles_n) { return; }
+  } else {
+    const int tile = (int)blockIdx.x;
+    const int band = tile / (8 * p.tiles_n);
+    const int in_band = tile - band * (8 * p.tiles_n);
+    const int band_h = (p.tiles_m - band * 8) < 8 ? (p.tiles_m - band * 8) : 8;
+    tm = band * 8 + in_band % band_h;
+    tn = in_band / band_h;
+  }
   const int m0 = tm * BM, n0 = tn * BN;
-  const int KT = (p.K + BK - 1) / BK;       // packed: a multiple of 8 (K % 512 == 0); dense: the last step may hold 32
-  const int tail_chunks = (p.K & (BK - 1)) >> 3;   // 16-byte chunks of a row in a partial last step (0: none)
+  const int KT = p.K / BK;                  // whole steps.  Packed: a multiple of 8 (K % 512 == 0)
+  const int tail_chunks = (p.K & (BK - 1)) >> 3;   // dense: 16-byte chunks of a row in the half step after them (0: none)
 
   // ---- x tile: 8 direct-to-LDS loads per wavefront and step.  Load i of wavefront w covers tile rows
   // (8w + i)*8 .. +8; lane l takes row l/8 and lands at LDS position l%8 of it.
@@ -157,14 +177,11 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     a_off[i] = (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u;
     if (chunk < tail_chunks) { tail_ok |= 1u << i; }
   }
-  // partial: the step is the last one and holds fewer than 64 values of K (dense weights only)
-  auto issue_x = [&](int step, auto stage_c, bool partial = false) {
+  auto issue_x = [&](int step, auto stage_c) {
     const uint8_t* src = xblk + (size_t)step * (BK * 2);
     const uint32_t dst = lds_addr(decltype(stage_c)::value ? x_lds1 : x_lds0) + wave * (64 * kRow);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (!partial || ((tail_ok >> i) & 1u)) { dma16(dst + i * (8 * kRow), src, a_off[i]); }
-    }
+    for (int i = 0; i < 8; ++i) { dma16(dst + i * (8 * kRow), src, a_off[i]); }
   };
   // ---- codes, scales, biases: wavefront w brings in those of rows 64w .. 64w+63 (nothing past BN rows) ----
   const bool dq_wave = wave * 64 < BN;      // wave-uniform
@@ -176,23 +193,23 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     c_off[i] = (uint32_t)rg * (uint32_t)(p.K >> 1) + (uint32_t)(lane & 1) * 16u;
   }
   const uint8_t* wblk = reinterpret_cast<const uint8_t*>(p.w);
-  // dense W tile: as the x tile, rows 64w .. 64w+63 of the tile by wavefront w
-  uint32_t wd_off[8];
+  // dense W tile: as the x tile; its BN rows are dealt out evenly, wavefront w brings in rows 16 NT w .. + 16 NT
+  constexpr int NWL = 2 * NT;               // loads per wavefront and step
+  uint32_t wd_off[NWL];
+  uint32_t wtail_ok = 0;                    // as tail_ok, for the W loads
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = (wave * 8 + i) * 8 + (lane >> 3);
+  for (int i = 0; i < NWL; ++i) {
+    const int row = (wave * NWL + i) * 8 + (lane >> 3);
     const int chunk = swz(row, lane & 7);
     const int rg = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
     wd_off[i] = DENSE ? (uint32_t)rg * (uint32_t)p.K * 2u + (uint32_t)chunk * 16u : 0u;
+    if (chunk < tail_chunks) { wtail_ok |= 1u << i; }
   }
-  auto issue_wdense = [&](int step, auto stage_c, bool partial = false) {
-    if (!dq_wave) { return; }
+  auto issue_wdense = [&](int step, auto stage_c) {
     const uint8_t* src = wblk + (size_t)step * (BK * 2);
-    const uint32_t dst = lds_addr(decltype(stage_c)::value ? w_lds1 : w_lds0) + wave * (64 * kRow);
+    const uint32_t dst = lds_addr(decltype(stage_c)::value ? w_lds1 : w_lds0) + wave * (NWL * 8 * kRow);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if (!partial || ((tail_ok >> i) & 1u)) { dma16(dst + i * (8 * kRow), src, wd_off[i]); }   // same rows' swizzle as x
-    }
+    for (int i = 0; i < NWL; ++i) { dma16(dst + i * (8 * kRow), src, wd_off[i]); }
   };
   auto issue_codes = [&](int u) {
     if (!dq_wave) { return; }
@@ -291,9 +308,9 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   //                  P/8 of the thread's codes at stage P%8 of
   //                    0: split the nibbles   1..4: two values each, fma(s, q, b)   5: pack to bf16   6: store   7: -
   // The state of both (fragments, codes, the word in work) lives across steps.
-  constexpr int NLOADS = DENSE ? 16 : 12;
+  constexpr int NLOADS = DENSE ? 8 + 2 * NT : 12;
   constexpr int SP = NT == 2 ? 1 : 2;
-  constexpr int NPRE = (MQ + SP - 1) / SP < NLOADS ? (MQ + SP - 1) / SP : NLOADS;   // requests made under quarter 3
+  constexpr int NPRE = MQ / SP < NLOADS ? MQ / SP : NLOADS;   // requests made under quarter 3 (slots SP-1, 2SP-1, ...)
   bf16x8 wf[2][NT], xf[2][4];                          // operand fragments of the current / the next quarter
   float sc2[2] = {0.0f, 0.0f}, bi2[2] = {0.0f, 0.0f};  // scale and bias of the thread's one or two rows
   uint32_t cw[WPT];                                    // its codes of the step being dequantized
@@ -352,14 +369,11 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     const uint32_t xdst = lds_addr(STG ? x_lds1 : x_lds0) + wave * (64 * kRow);
     const uint8_t* xsrc = xblk + (size_t)step_to * (BK * 2);
     if constexpr (DENSE) {
-      const bool partial = tail_chunks != 0 && step_to + 1 == KT;
-      if constexpr (I < 8) {
-        const uint32_t wdst = lds_addr(STG ? w_lds1 : w_lds0) + wave * (64 * kRow);
-        if (dq_wave && (!partial || ((tail_ok >> I) & 1u))) {
-          dma16(wdst + I * (8 * kRow), wblk + (size_t)step_to * (BK * 2), wd_off[I]);
-        }
+      if constexpr (I < NWL) {
+        const uint32_t wdst = lds_addr(STG ? w_lds1 : w_lds0) + wave * (NWL * 8 * kRow);
+        dma16(wdst + I * (8 * kRow), wblk + (size_t)step_to * (BK * 2), wd_off[I]);
       } else {
-        if (!partial || ((tail_ok >> (I - 8)) & 1u)) { dma16(xdst + (I - 8) * (8 * kRow), xsrc, a_off[I - 8]); }
+        dma16(xdst + (I - NWL) * (8 * kRow), xsrc, a_off[I - NWL]);
       }
     } else {
       if constexpr (I < 8) {
@@ -380,9 +394,8 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     }
   };
   // Step s on stage ST.  m1: a step s+1 exists, m2: a step s+2 exists (std::true_type / std::false_type, or bool
-  // where the choice is left to run time); `quarters` < 4 only on a last step that holds fewer than 64 values of K
-  // (dense weights).
-  auto pstep = [&](auto stage_c, auto m1, auto m2, int s, int quarters) {
+  // where the choice is left to run time).
+  auto pstep = [&](auto stage_c, auto m1, auto m2, int s) {
     constexpr int ST = decltype(stage_c)::value;
     using Nx = std::integral_constant<int, 1 - ST>;
     const uint8_t* xb = ST ? x_lds1 : x_lds0;
@@ -394,7 +407,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       constexpr int Q = decltype(qc)::value;
       constexpr int B = Q & 1;
       if constexpr (Q == 3 && !DENSE) { when(m2, [&] { load_row_params(s + 2, sc2, bi2, cw); }); }
-      if (Q < quarters) {
+      {
         static_for<0, MQ>([&](auto jc) {
           constexpr int J = decltype(jc)::value;
           constexpr int JT = J >> 2, IT = J & 3;
@@ -404,13 +417,13 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
             if constexpr (Q == 3) { when(m2, [&] { piece(std::integral_constant<int, GB>(), ownb); }); }
             else { when(m1, [&] { piece(std::integral_constant<int, GB>(), nwb); }); }
           }
-          if constexpr (GB % SP == 0 && GB / SP < NLOADS) {
+          if constexpr (GB % SP == SP - 1 && GB / SP < NLOADS) {
             if constexpr (Q == 3) { when(m2, [&] { window_load(std::integral_constant<int, GB / SP>(), s, stage_c); }); }
             else { when(m1, [&] { window_load(std::integral_constant<int, GB / SP>(), s - 1, Nx()); }); }
           }
           // the next quarter's fragments, one read after every MFMA until they are all requested
           if constexpr (J < 4 + NT) {
-            if constexpr (Q < 3) { if (Q + 1 < quarters) { frag(xb, wb, 1 - B, Q + 1, J); } }
+            if constexpr (Q < 3) { frag(xb, wb, 1 - B, Q + 1, J); }
             else { when(m1, [&] { frag(nxb, nwb, 0, 0, J); }); }
           }
           __builtin_amdgcn_sched_barrier(0);
@@ -425,48 +438,80 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     });
   };
 
-  // ---- prologue: stage 0 complete (x(0); W(0) loaded or dequantized), the part of step 1's window that a
-  // quarter 3 before step 0 would have done, the first fragments ----
-  if constexpr (DENSE) {
-    const bool partial0 = KT == 1 && tail_chunks != 0;
-    issue_wdense(0, S0(), partial0);
-    issue_x(0, S0(), partial0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    wg_barrier();
-  } else {
-    issue_scales(0);
-    issue_codes(0);
-    issue_codes(1);
-    issue_x(0, S0());
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    wg_barrier();                             // the codes and scales a thread reads were brought in by any wavefront
-    load_row_params(0, sc2, bi2, cw);
-    static_for<0, 4 * MQ>([&](auto pc) { piece(pc, w_lds0); });
-    load_row_params(1, sc2, bi2, cw);
-    static_for<0, MQ>([&](auto pc) { piece(pc, w_lds1); });
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    wg_barrier();
-  }
-  if (KT > 1) { static_for<0, NPRE>([&](auto ic) { window_load(ic, -1, S1()); }); }
+  // `nq` quarter steps (16 of K each) on the tiles in stage 0, nothing overlapped: for the short extra pieces of K
+  // (a dense half step, the adapter's rank).
+  auto plain_quarters = [&](int nq) {
+    for (int q = 0; q < nq; ++q) {
 #pragma unroll
-  for (int i = 0; i < 4 + NT; ++i) { frag(x_lds0, w_lds0, 0, 0, i); }
+      for (int i = 0; i < 4 + NT; ++i) { frag(x_lds0, w_lds0, 0, q, i); }
+#pragma unroll
+      for (int j = 0; j < MQ; ++j) { acc[j >> 2][j & 3] = mfma(wf[0][j >> 2], xf[0][j & 3], acc[j >> 2][j & 3]); }
+    }
+  };
 
-  // ---- K loop.  Packed: no condition surrounds the arithmetic inside it, the last two steps are written out
-  // (K is a multiple of 512).  Dense: any number of steps, the conditions are wave-uniform branches. ----
+  if (KT > 0) {
+    // ---- prologue: stage 0 complete (x(0); W(0) loaded or dequantized), the part of step 1's window that a
+    // quarter 3 before step 0 would have done, the first fragments ----
+    if constexpr (DENSE) {
+      issue_wdense(0, S0());
+      issue_x(0, S0());
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      wg_barrier();
+    } else {
+      issue_scales(0);
+      issue_codes(0);
+      issue_codes(1);
+      issue_x(0, S0());
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      wg_barrier();                             // the codes and scales a thread reads were brought in by any wavefront
+      load_row_params(0, sc2, bi2, cw);
+      static_for<0, 4 * MQ>([&](auto pc) { piece(pc, w_lds0); });
+      load_row_params(1, sc2, bi2, cw);
+      static_for<0, MQ>([&](auto pc) { piece(pc, w_lds1); });
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wg_barrier();
+    }
+    if (KT > 1) { static_for<0, NPRE>([&](auto ic) { window_load(ic, -1, S1()); }); }
+#pragma unroll
+    for (int i = 0; i < 4 + NT; ++i) { frag(x_lds0, w_lds0, 0, 0, i); }
+
+    // ---- K loop.  Packed: no condition surrounds the arithmetic inside it, the last two steps are written out
+    // (K is a multiple of 512).  Dense: any number of steps, the conditions are wave-uniform branches. ----
+    if constexpr (DENSE) {
+      for (int s = 0; s < KT; s += 2) {
+        pstep(S0(), s + 1 < KT, s + 2 < KT, s);
+        if (s + 1 < KT) { pstep(S1(), s + 2 < KT, s + 3 < KT, s + 1); }
+      }
+    } else {
+      int s = 0;
+      for (; s + 3 < KT; s += 2) {
+        pstep(S0(), Yes(), Yes(), s);
+        pstep(S1(), Yes(), Yes(), s + 1);
+      }
+      pstep(S0(), Yes(), No(), s);
+      pstep(S1(), No(), No(), s + 1);
+    }
+  }
+
   if constexpr (DENSE) {
-    const int last_quarters = tail_chunks != 0 ? (tail_chunks >> 1) : 4;
-    for (int s = 0; s < KT; s += 2) {
-      pstep(S0(), s + 1 < KT, s + 2 < KT, s, s + 1 == KT ? last_quarters : 4);
-      if (s + 1 < KT) { pstep(S1(), s + 2 < KT, s + 3 < KT, s + 1, s + 2 == KT ? last_quarters : 4); }
+    if (tail_chunks != 0) {
+      // the last 32 values of K: half rows into stage 0 (only the lanes whose chunk exists), two quarter steps
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wg_barrier();                                    // everyone done with stage 0
+      const uint8_t* xsrc = xblk + (size_t)KT * (BK * 2);
+      const uint8_t* wsrc = wblk + (size_t)KT * (BK * 2);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if ((tail_ok >> i) & 1u) { dma16(lds_addr(x_lds0) + wave * (64 * kRow) + i * (8 * kRow), xsrc, a_off[i]); }
+      }
+#pragma unroll
+      for (int i = 0; i < NWL; ++i) {
+        if ((wtail_ok >> i) & 1u) { dma16(lds_addr(w_lds0) + wave * (NWL * 8 * kRow) + i * (8 * kRow), wsrc, wd_off[i]); }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      wg_barrier();
+      plain_quarters(tail_chunks >> 1);
     }
-  } else {
-    int s = 0;
-    for (; s + 3 < KT; s += 2) {
-      pstep(S0(), Yes(), Yes(), s, 4);
-      pstep(S1(), Yes(), Yes(), s + 1, 4);
-    }
-    pstep(S0(), Yes(), No(), s, 4);
-    pstep(S1(), No(), No(), s + 1, 4);
   }
 
   if (LORA) {
@@ -502,9 +547,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       }
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       wg_barrier();                                    // tiles ready
-#pragma unroll
-      for (int i = 0; i < 4 + NT; ++i) { frag(x_lds0, w_lds0, 0, 0, i); }
-      pstep(S0(), No(), No(), 0, chunks >> 1);
+      plain_quarters(chunks >> 1);
     }
   }
 
@@ -643,6 +686,27 @@ int qmm_big_tile_n(int N, int M, int cu_count)
   return best;
 }
 
+namespace {
+
+// Tile order and grid size.  From two full rounds of the chip on: blocks of 32 tiles per XCD, in the shape that
+// leaves the fewest empty places (then the squarest); below that, bands of 8 rows of tiles.
+unsigned plan_tile_order(BigParams& p)
+{
+  p.bmt = 0; p.bnt = 0; p.nbn = 0;
+  const long tiles = (long)p.tiles_m * p.tiles_n;
+  if (tiles < 512) { return (unsigned)tiles; }
+  const int shapes[6][2] = {{4, 8}, {8, 4}, {2, 16}, {16, 2}, {1, 32}, {32, 1}};
+  long best_sets = 0;
+  for (int i = 0; i < 6; ++i) {
+    const long nbm = (p.tiles_m + shapes[i][0] - 1) / shapes[i][0], nbn = (p.tiles_n + shapes[i][1] - 1) / shapes[i][1];
+    const long sets = (nbm * nbn + 7) / 8;               // rounds of 8 XCDs x 32 workgroups
+    if (i == 0 || sets < best_sets) { best_sets = sets; p.bmt = shapes[i][0]; p.bnt = shapes[i][1]; p.nbn = (int)nbn; }
+  }
+  return (unsigned)(best_sets * 256);
+}
+
+}  // namespace
+
 hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
 {
   const int bn = tile_n == 128 || tile_n == 192 || tile_n == 256 ? tile_n : qmm_big_tile_n(a.N, a.M, a.cu_count);
@@ -655,7 +719,7 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
   p.gate_act = a.gate_act;
   p.out_stride = a.out_stride > 0 ? a.out_stride : a.N / 2;
   p.out_off = a.out_off;
-  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kBigThreads);
+  const dim3 grid(plan_tile_order(p)), block(kBigThreads);
   const bool lora = a.lora_t != nullptr;
   if (bn == 128) {
     return lora ? launch_kernel(qmm_big_kernel<2, true>, grid, block, 0, st, p)
@@ -688,7 +752,7 @@ hipError_t launch_dense_gemm(hipStream_t st, const uint16_t* x, const uint16_t* 
   p.K = K; p.N = N; p.M = M;
   p.tiles_m = (M + BM - 1) / BM;
   p.tiles_n = (N + bn - 1) / bn;
-  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kBigThreads);
+  const dim3 grid(plan_tile_order(p)), block(kBigThreads);
 #define VPQ_DENSE(NTV)                                                                      \
   (f16 ? launch_kernel(qmm_big_kernel<NTV, false, kDenseF16>, grid, block, 0, st, p)       \
        : launch_kernel(qmm_big_kernel<NTV, false, kDenseBf16>, grid, block, 0, st, p))
