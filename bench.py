@@ -120,19 +120,25 @@ def main():
             w, s, b = make_weight(torch, N, K, dev, gen)
             x = torch.randn((M, K), device=dev, generator=gen).bfloat16()
             y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
-            for _ in range(3):
+            for _ in range(150):                       # ~40 ms: the clocks settle
                 vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y)
             torch.cuda.synchronize()
             t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             t0.record()
-            for _ in range(10):
+            for _ in range(20):
                 vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y)
             t1.record()
             torch.cuda.synchronize()
-            us = t0.elapsed_time(t1) * 1e3 / 10
+            us = t0.elapsed_time(t1) * 1e3 / 20
             res[name] = {"K": K, "N": N, "M": M, "us": round(us, 2),
                          "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 1)}
-        print(json.dumps({"qmm_m2048_fused_kernel_only": res}))
+        if args.copy_calibration:
+            src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(generator=gen)
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+        print(json.dumps({"qmm_m2048_fused_kernel_only": res, "build": vpipe_amd.build_id()}))
         return
 
     # ---- inputs, resident in HBM ------------------------------------------------
@@ -355,6 +361,10 @@ def main():
         roofline["eager_launch_us"] = {n: round(float(dur[:, i].mean()), 3)
                                        for i, n in enumerate(("q|k|v", "o", "gate|up", "down"))}
 
+    build = vpipe_amd.build_id()
+    roofline["build"] = build
+    if traffic_layer:
+        roofline["traffic_profile_is_of_this_build"] = bool(traffic_build) and str(traffic_build).split()[0] == build
     out = {
         "metric": "4-bit QMV HBM GB/s at batch 1 (decode-layer projection set)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -114,6 +114,13 @@ def lib_path():
     return _SO
 
 
+def build_id():
+    """First 12 hex digits of the SHA-256 of the built library: names the build a measurement was taken on."""
+    import hashlib
+    with open(_SO, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:12]
+
+
 def load():
     """dlopen libvpq.so (built by `python -m vpipe_amd.build`); raises if absent."""
     global _lib
