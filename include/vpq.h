@@ -360,6 +360,32 @@ int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
                                    const int32_t* pair_eid, int npair, int n_experts);
 
+/* ---- MoE: expert-sorted GEMV, two slots per tile ---------------------------
+ * For a few rows per expert the reference sorts the (token, expert) pairs
+ * into per-expert tiles of MAXM = 2 slots and runs a GEMV that reads the
+ * expert's slab once per tile instead of once per pair
+ * (gpu-kernels/metal/quant/affine_qmv.metal:2551-2719).  vpq_moe_sort_pairs
+ * with block_rows = VPQ_QMV_GROUPED_SLOTS builds tile2e / srow for it.
+ *
+ * vpq_qmv_grouped_gated_w4g64_bf16 replaces `affine_grouped_swiglu_w4g64`
+ * (:2707; slots 0:w 1:scales 2:biases 3:x[rows,K] 4:y[npad,N/2] 5:K 6:N
+ * 7:srow 8:tile2e; grid.z = tile): slot s of tile t reads x row srow[s] and
+ * stores act(gate)*up of expert tile2e[t]'s interleaved gate|up slab into y
+ * row s.  vpq_qmv_grouped_down_w4g64_bf16 replaces `affine_grouped_down_w4g64`
+ * (:2708): x[npad,K] and y[npad,N] both in slot order.  A slot with
+ * srow[s] < 0 is padding and a tile with tile2e[t] < 0 (or an id >=
+ * n_experts) is unused: nothing is written for them.  A live slot's result is
+ * bit-identical to the plain call (VPQ_QMV_ROWS) on that slab and that row.
+ * Requires K % 64 == 0, npad a positive multiple of VPQ_QMV_GROUPED_SLOTS,
+ * npad / 2 <= 65535, N even for the gated form; w, x 16-byte aligned. */
+#define VPQ_QMV_GROUPED_SLOTS 2
+int vpq_qmv_grouped_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
+                                     const int32_t* tile2e, const int32_t* srow, int n_experts, int activation);
+int vpq_qmv_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
+                                    const int32_t* tile2e, const int32_t* srow, int n_experts);
+
 /* ---- MoE prefill: expert-sorted (grouped) GEMMs ---------------------------
  * With many tokens the pairs are sorted by expert into blocks of
  * vpq_qmm_grouped_block_rows() slots, each block owned by ONE expert, and two

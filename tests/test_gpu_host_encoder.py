@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from tests import parity
-from vpipe_amd import synth
+from vpipe_amd import capi, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -460,6 +460,57 @@ def test_moe_grouped_expert_call_sites(vpq, enc, oracle, dev, D):
     # the down projection reads the activation the device produced
     d64, dbits = oracle.qmm_grouped(dw, ds, db, gact_bits, I, H, B, t2e, sdst=sdst, rows_y=npair)
     parity.check_bf16(D.bits(part), d64, dbits)
+
+
+def test_moe_sorted_gemv_call_sites(vpq, enc, oracle, dev, D):
+    # a few rows per expert: tiles of two sorted slots (gpu-kernels/metal/quant/affine_qmv.metal:2682-2708; slots 0..4,
+    # 5:K 6:N 7:srow 8:tile2e, one tile per grid.z): gate|up + SwiGLU over the gathered hidden rows -> gact[npad, I],
+    # then down over gact in slot order -> part[npad, H]
+    H, I, E, top_k, T = 512, 128, 7, 2, 6
+    gu = [synth.make_weight(2 * I, H, 2900 + e) for e in range(E)]
+    dn = [synth.make_weight(H, I, 2950 + e) for e in range(E)]
+    guw, gus, gub = (np.stack([p[i] for p in gu]) for i in range(3))
+    dw, ds, db = (np.stack([p[i] for p in dn]) for i in range(3))
+    x = synth.make_act(T, H, 2990)
+    eid = np.random.default_rng(2991).integers(0, E, size=T * top_k, dtype=np.int32)
+    B = capi.VPQ_QMV_GROUPED_SLOTS
+    t2e_d, srow_d, _, _ = vpq.moe_sort_pairs(torch.from_numpy(eid).to(dev), top_k, E, block_rows=B)
+    t2e, srow = t2e_d.cpu().numpy(), srow_d.cpu().numpy()
+    npad = srow.size
+    gact = torch.zeros((npad, I), dtype=torch.bfloat16, device=dev)
+    part = torch.zeros((npad, H), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()               # the encoder's stream is not ordered after torch's fills
+    assert enc.set_function("affine_qmv_bf16", "affine_grouped_swiglu_w4g64") == 1
+    gu_d = (D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev), gact)
+    for i, t in enumerate(gu_d):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, H)
+    enc.set_constant(6, 2 * I)
+    enc.set_buffer(7, srow_d)
+    enc.set_buffer(8, t2e_d)
+    enc.dispatch((32, 2 * ((2 * I + 7) // 8), npad // B), (32, 2, 1))
+    assert enc.set_function("affine_qmv_bf16", "affine_grouped_down_w4g64") == 1
+    dn_d = (D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), gact, part)
+    for i, t in enumerate(dn_d):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, I)
+    enc.set_constant(6, H)
+    enc.set_buffer(7, srow_d)
+    enc.set_buffer(8, t2e_d)
+    enc.dispatch((32, 2 * ((H + 7) // 8), npad // B), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    live = np.nonzero(srow >= 0)[0]
+    gact_bits = D.bits(gact)
+    y64 = np.concatenate([oracle.qmv(guw[t2e[s // B]], gus[t2e[s // B]], gub[t2e[s // B]], x[srow[s]:srow[s] + 1], H, 2 * I, 1)[0]
+                          for s in live])
+    a64, ab = oracle.swiglu(y64)
+    parity.check_bf16(gact_bits[live], a64, ab)
+    assert not gact_bits[srow < 0].any()
+    # the down projection reads the activation the device produced
+    pairs = [oracle.qmv(dw[t2e[s // B]], ds[t2e[s // B]], db[t2e[s // B]], gact_bits[s:s + 1], I, H, 1) for s in live]
+    parity.check_bf16(D.bits(part)[live], np.concatenate([p[0] for p in pairs]), np.concatenate([p[1] for p in pairs]))
+    assert not D.bits(part)[srow < 0].any()
 
 
 def test_moe_gathered_expert_call_sites(enc, oracle, dev, D):

@@ -185,3 +185,80 @@ def test_grouped_gemms_take_the_slots_of_a_block_in_any_order(vpq, oracle, dev, 
     a64, ab = oracle.swiglu(y64)
     live = srow >= 0
     parity.check_bf16(act0[live], a64[live], ab[live])
+
+
+# K (hidden), inner, H (down out), E, T, top_k: a few rows per expert, the case the two-slot tiles are for
+SORTED_QMV_SHAPES = [(512, 128, 512, 6, 9, 2, False), (2048, 768, 2048, 16, 20, 4, True), (576, 96, 200, 3, 5, 1, False),
+                     (1024, 160, 1026, 40, 16, 8, True)]
+
+
+@pytest.mark.parametrize("activation", [capi.VPQ_GATE_SWIGLU, capi.VPQ_GATE_GEGLU])
+@pytest.mark.parametrize("K,inner,H,E,T,top_k,skew", SORTED_QMV_SHAPES)
+def test_sorted_expert_gemv_two_slots_per_tile(vpq, oracle, dev, D, K, inner, H, E, T, top_k, skew, activation):
+    """gpu-kernels/metal/quant/affine_qmv.metal:2551-2719 (`affine_grouped_swiglu_w4g64`, `affine_grouped_down_w4g64`,
+    MAXM = 2): QMV arithmetic (weight never rounded) over pairs sorted into per-expert tiles of two slots; padding
+    slots and unused tiles are left untouched; a live slot is bit for bit the plain row-streaming QMV."""
+    B = capi.VPQ_QMV_GROUPED_SLOTS
+    Kd = ((inner + 63) // 64) * 64
+    guw, gus, gub = expert_batch(E, 2 * inner, K, 6100 + K)
+    dw, ds, db = expert_batch(E, H, Kd, 6200 + K)
+    x = synth.make_act(T, K, 6300 + K)
+    eid = routed(E, T, top_k, 6400 + K, skew)
+    t2e_d, srow_d, sdst_d, ntiles_d = vpq.moe_sort_pairs(torch.from_numpy(eid).to(dev), top_k, E, block_rows=B)
+    t2e, srow, sdst = (o.cpu().numpy() for o in (t2e_d, srow_d, sdst_d))
+    check_sort(eid, top_k, E, B, t2e, srow, sdst, ntiles_d.cpu().numpy(), oracle)
+    npad = srow.size
+    live = srow >= 0
+    seven = D.bits(torch.full((1,), 7.0, dtype=torch.bfloat16))[0]
+
+    # ---- gate|up + activation, x rows gathered through srow ----
+    guwd, gusd, gubd, xd = D.u32(guw, dev), D.bf16(gus, dev), D.bf16(gub, dev), D.bf16(x, dev)
+    act_out = parity.Guarded((npad, inner), torch.bfloat16, dev)
+    act_out.view.fill_(7.0)
+    vpq.qmv_grouped_gated_w4g64(guwd, gusd, gubd, xd, K, 2 * inner, t2e_d, srow_d, E, out=act_out.view, activation=activation)
+    torch.cuda.synchronize()
+    act_out.assert_intact()
+    got = D.bits(act_out.view)
+    assert (got[~live] == seven).all()                   # padding slots and unused tiles: untouched
+    act = oracle.swiglu if activation == capi.VPQ_GATE_SWIGLU else oracle.geglu
+    slots = np.nonzero(live)[0]
+    y64 = np.concatenate([oracle.qmv(guw[t2e[s // B]], gus[t2e[s // B]], gub[t2e[s // B]], x[srow[s]:srow[s] + 1], K, 2 * inner, 1)[0]
+                          for s in slots])
+    want64, wantb = act(y64)
+    parity.check_bf16(got[slots], want64, wantb, mismatch_over_all=activation == capi.VPQ_GATE_SWIGLU)
+    for s in slots:
+        e = int(t2e[s // B])
+        plain = vpq.qmv_swiglu_w4g64(guwd[e], gusd[e], gubd[e], xd[int(srow[s]):int(srow[s]) + 1].contiguous(), K, 2 * inner, 1,
+                                     variant=capi.VPQ_QMV_ROWS, activation=activation)
+        assert np.array_equal(got[s], D.bits(plain)[0]), "slot %d" % s
+
+    # ---- down over the sorted activations, y in slot order ----
+    xs = synth.make_act(npad, Kd, 6500 + K)
+    dwd, dsd, dbd, xsd = D.u32(dw, dev), D.bf16(ds, dev), D.bf16(db, dev), D.bf16(xs, dev)
+    down = parity.Guarded((npad, H), torch.bfloat16, dev)
+    down.view.fill_(7.0)
+    vpq.qmv_grouped_down_w4g64(dwd, dsd, dbd, xsd, Kd, H, t2e_d, srow_d, E, out=down.view)
+    torch.cuda.synchronize()
+    down.assert_intact()
+    gotd = D.bits(down.view)
+    assert (gotd[~live] == seven).all()
+    pairs = [oracle.qmv(dw[t2e[s // B]], ds[t2e[s // B]], db[t2e[s // B]], xs[s:s + 1], Kd, H, 1) for s in slots]
+    parity.check_bf16(gotd[slots], np.concatenate([p[0] for p in pairs]), np.concatenate([p[1] for p in pairs]))
+    for s in slots:
+        e = int(t2e[s // B])
+        plain = vpq.qmv_w4g64(dwd[e], dsd[e], dbd[e], xsd[int(s):int(s) + 1].contiguous(), Kd, H, 1, variant=capi.VPQ_QMV_ROWS)
+        assert np.array_equal(gotd[s], D.bits(plain)[0]), "slot %d" % s
+
+
+def test_sorted_expert_gemv_rejects_bad_arguments(vpq, dev):
+    L = vpq.load()
+    buf = torch.zeros(1 << 16, dtype=torch.int32, device=dev)
+    p = buf.data_ptr()
+    act = capi.VPQ_GATE_SWIGLU
+    assert L.vpq_qmv_grouped_gated_w4g64_bf16(None, p, p, p, p, p, 64, 8, 2, p, None, 1, act) == -1
+    assert L.vpq_qmv_grouped_gated_w4g64_bf16(None, p, p, p, p, p, 64, 8, 3, p, p, 1, act) == -2      # not whole tiles
+    assert L.vpq_qmv_grouped_gated_w4g64_bf16(None, p, p, p, p, p, 64, 7, 2, p, p, 1, act) == -2      # odd N
+    assert L.vpq_qmv_grouped_gated_w4g64_bf16(None, p, p, p, p, p, 64, 8, 2, p, p, 1, 9) == -2        # activation
+    assert L.vpq_qmv_grouped_down_w4g64_bf16(None, p, p, p, p, p, 60, 8, 2, p, p, 1) == -2            # K % 64
+    assert L.vpq_qmv_grouped_down_w4g64_bf16(None, p, p, p, p, p, 64, 8, 2, p, p, 0) == -2            # no expert
+    assert L.vpq_qmv_grouped_down_w4g64_bf16(None, p, p, p, p, p, 64, 8, 2, None, p, 1) == -1

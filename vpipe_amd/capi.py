@@ -46,6 +46,8 @@ SYMBOLS = [
     ("vpq_moe_sort_pairs", _i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz]),
     ("vpq_qmm_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _i]),
     ("vpq_qmm_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
+    ("vpq_qmv_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
+    ("vpq_qmv_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i]),
     ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
     ("vpq_qmv_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _i]),
     ("vpq_qmv_workspace_bytes", _sz, [_i, _i, _i]),
@@ -318,6 +320,27 @@ def qmm_grouped_down_w4g64(w, scales, biases, x, K, N, tile2e, sdst, n_experts, 
     _check(load().vpq_qmm_grouped_down_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
                                                   npad, _ptr(tile2e), _ptr(sdst), n_experts, out.shape[0]),
            "vpq_qmm_grouped_down_w4g64_bf16")
+    return out
+
+
+VPQ_QMV_GROUPED_SLOTS = 2
+
+
+def qmv_grouped_gated_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out, activation=VPQ_GATE_SWIGLU):
+    """Expert batch [E, N=2*inner, ...], x [rows_x, K], tiles of two sorted slots -> live rows of out [npad, N/2]."""
+    npad = srow.numel()
+    _check(load().vpq_qmv_grouped_gated_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                   npad, _ptr(tile2e), _ptr(srow), n_experts, activation),
+           "vpq_qmv_grouped_gated_w4g64_bf16")
+    return out
+
+
+def qmv_grouped_down_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out):
+    """Expert batch [E, N, ...], x [npad, K] in slot order -> live rows of out [npad, N] in slot order."""
+    npad = srow.numel()
+    _check(load().vpq_qmv_grouped_down_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                  npad, _ptr(tile2e), _ptr(srow), n_experts),
+           "vpq_qmv_grouped_down_w4g64_bf16")
     return out
 
 

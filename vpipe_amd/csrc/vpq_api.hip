@@ -793,6 +793,49 @@ int vpq_gather_down_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
   return gather_common(stream, w, scales, biases, x, y, K, N, pair_eid, npair, 1, n_experts, 0);
 }
 
+namespace {
+
+int sorted_qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                      const uint16_t* x, uint16_t* y, int K, int N, int npad, const int32_t* tile2e, const int32_t* srow,
+                      int n_experts, int gate_act, bool x_from_srow)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr || tile2e == nullptr || srow == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (npad < VPQ_QMV_GROUPED_SLOTS || (npad % VPQ_QMV_GROUPED_SLOTS) != 0 || npad / VPQ_QMV_GROUPED_SLOTS > 65535 ||
+      n_experts < 1) {
+    return VPQ_ERR_BAD_SHAPE;
+  }
+  if (gate_act != 0 && gate_act != VPQ_GATE_SWIGLU && gate_act != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (gate_act != 0 && (N & 1) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 2) || !aligned(tile2e, 4) || !aligned(srow, 4)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y;
+  a.K = K; a.N = N; a.M = VPQ_QMV_GROUPED_SLOTS; a.y_f32 = false; a.cu_count = g_dev.cu_count;
+  a.gate_act = gate_act;
+  return finish(vpq::launch_qmv_rows_sorted(reinterpret_cast<hipStream_t>(stream), a, tile2e, srow,
+                                            npad / VPQ_QMV_GROUPED_SLOTS, x_from_srow, n_experts));
+}
+
+}  // namespace
+
+int vpq_qmv_grouped_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
+                                     const int32_t* tile2e, const int32_t* srow, int n_experts, int activation)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return sorted_qmv_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, srow, n_experts, activation, true);
+}
+
+int vpq_qmv_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
+                                    const int32_t* tile2e, const int32_t* srow, int n_experts)
+{
+  return sorted_qmv_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, srow, n_experts, 0, false);
+}
+
 int vpq_qmm_grouped_block_rows(void) { return vpq::kGroupedBlockRows; }
 
 size_t vpq_moe_sort_workspace_bytes(int n_experts)

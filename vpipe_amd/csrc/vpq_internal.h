@@ -144,6 +144,9 @@ hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGrou
 // [0, n_experts)); a.gate_act as in the plain form.
 hipError_t launch_qmv_rows_gather(hipStream_t st, const QmvArgs& a, const int* pair_eid, int pairs, int x_div,
                                   int n_experts);
+// Sorted pairs, two slots per tile (a.M = 2): expert tile2e[tile], x row srow[slot] (x_from_srow) or the slot.
+hipError_t launch_qmv_rows_sorted(hipStream_t st, const QmvArgs& a, const int* tile2e, const int* srow, int tiles,
+                                  bool x_from_srow, int n_experts);
 // Greedy argmax of `rows` rows of V bf16 logits (lowest index among equal maxima, a NaN never
 // wins): one workgroup per row, or slabs into `partials` (two 4-byte slots per slab: value, index)
 // and a combine; argmax_parts(V) is the slab count the size-based entrance uses.

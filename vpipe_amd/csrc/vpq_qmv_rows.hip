@@ -22,6 +22,10 @@
 // Gathered form (MoE, gpu-kernels/metal/quant/affine_qmv.metal:908-962, 1262-1292): grid.y is a
 // (token, expert) pair p; the pack is a batch [E, N, K/8] of expert slabs and pair_eid[p] picks
 // the slab, x row p / x_div (gate|up: top_k pairs share a token's row) or p (down), y row p.
+//
+// Sorted form (MoE prefill with few rows per expert, gpu-kernels/metal/quant/affine_qmv.metal:2551-2719, MAXM = 2):
+// the pairs have been sorted into per-expert tiles of two slots; grid.y is a tile, its expert's slab is read once
+// for both slots.  Per-row arithmetic is that of the plain kernel.
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -58,6 +62,11 @@ struct RowsGather {
   const int* pair_eid;
   int x_div;        // x row of pair p is p / x_div
   int n_experts;    // ids outside [0, n_experts) give zeros
+  // Sorted (grouped) form: grid.y is a tile of two slots owned by expert tile2e[tile] (< 0: unused tile, nothing
+  // is written); slot s is live where srow[s] >= 0 and reads x row srow[s] (x_from_srow) or row s, writes y row s.
+  const int* tile2e = nullptr;
+  const int* srow = nullptr;
+  int x_from_srow = 0;
 };
 
 // R rows per row group, 64 / LPR row groups per wavefront, four wavefronts per workgroup, MT rows of x.
@@ -88,7 +97,30 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
   const int n0 = nw + sub * R;
   const int Kw = K >> 3, Kg = K >> GS;
   bool expert_ok = true;
-  if (gather.pair_eid != nullptr) {
+  const uint16_t* xrow[MT];
+  bool live[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    xrow[m] = x + (size_t)(m < M ? m : M - 1) * K;
+    live[m] = m < M;
+  }
+  if (gather.tile2e != nullptr) {
+    const int t = (int)blockIdx.y;
+    const int e = gather.tile2e[t];
+    if (e < 0 || e >= gather.n_experts) { return; }      // block-uniform; the kernel has no barrier
+    w += (size_t)e * (size_t)N * Kw;
+    scales += (size_t)e * (size_t)N * Kg;
+    biases += (size_t)e * (size_t)N * Kg;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const int slot = t * MT + m;
+      const int rr = gather.srow[slot];
+      live[m] = rr >= 0;
+      xrow[m] = x + (size_t)(gather.x_from_srow ? (rr >= 0 ? rr : 0) : slot) * K;
+    }
+    const size_t yo = (size_t)t * MT * (size_t)(gate_act ? (N >> 1) : N);
+    y = F32OUT ? (void*)(reinterpret_cast<float*>(y) + yo) : (void*)(reinterpret_cast<uint16_t*>(y) + yo);
+  } else if (gather.pair_eid != nullptr) {
     const int p = (int)blockIdx.y;
     int e = gather.pair_eid[p];
     expert_ok = e >= 0 && e < gather.n_experts;
@@ -96,7 +128,7 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
     w += (size_t)e * (size_t)N * Kw;
     scales += (size_t)e * (size_t)N * Kg;
     biases += (size_t)e * (size_t)N * Kg;
-    x += (size_t)(p / gather.x_div) * K;
+    xrow[0] = x + (size_t)(p / gather.x_div) * K;
     const size_t yo = (size_t)p * (size_t)(gate_act ? (N >> 1) : N);
     y = F32OUT ? (void*)(reinterpret_cast<float*>(y) + yo) : (void*)(reinterpret_cast<uint16_t*>(y) + yo);
   }
@@ -138,8 +170,7 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
     }
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-      const int row = m < M ? m : M - 1;
-      const uint4* xs = reinterpret_cast<const uint4*>(x + (size_t)row * K + k0);
+      const uint4* xs = reinterpret_cast<const uint4*>(xrow[m] + k0);
 #pragma unroll
       for (int t = 0; t < 4; ++t) { p.xd[m][t] = xs[t]; }
     }
@@ -220,7 +251,7 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(
   if (ll != 0) { return; }
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
-    if (m >= M) { continue; }
+    if (!live[m]) { continue; }
     if (gate_act) {
 #pragma unroll
       for (int r = 0; r < R; r += 2) {
@@ -324,6 +355,20 @@ hipError_t launch_qmv_rows_gather(hipStream_t st, const QmvArgs& a, const int* p
   g.count = 1;
   g.seg[0] = RowsSeg{a.w, a.scales, a.biases, a.y, a.N, 0};
   return launch_rows_segments(st, g, a, 2, RowsGather{pair_eid, x_div, n_experts}, pairs);
+}
+
+// a.M = 2 (slots per tile); a.x is the hidden [rows, K] (x_from_srow) or the sorted activations [2 tiles, K].
+hipError_t launch_qmv_rows_sorted(hipStream_t st, const QmvArgs& a, const int* tile2e, const int* srow, int tiles,
+                                  bool x_from_srow, int n_experts)
+{
+  RowsSegs g{};
+  g.count = 1;
+  g.seg[0] = RowsSeg{a.w, a.scales, a.biases, a.y, a.N, 0};
+  RowsGather ga{nullptr, 1, n_experts};
+  ga.tile2e = tile2e;
+  ga.srow = srow;
+  ga.x_from_srow = x_from_srow ? 1 : 0;
+  return launch_rows_segments(st, g, a, 2, ga, tiles);
 }
 
 hipError_t launch_qmv_rows_g32(hipStream_t st, const QmvArgs& a, bool scale_only)

@@ -100,6 +100,8 @@ const FnEntry kFunctions[] = {
     {"affine_qmm_steel_bf16", "affine_qmm_grouped_swiglu_w4g64", QuantKernel::GroupedSwiglu},
     {"affine_qmm_steel_bf16", "affine_qmm_grouped_geglu_w4g64", QuantKernel::GroupedGeglu},
     {"affine_qmm_steel_bf16", "affine_qmm_grouped_w4g64", QuantKernel::GroupedDown},
+    {"affine_qmv_bf16", "affine_grouped_swiglu_w4g64", QuantKernel::SortedSwiglu},
+    {"affine_qmv_bf16", "affine_grouped_down_w4g64", QuantKernel::SortedDown},
     {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w4w8g64", QuantKernel::GatherSplit48},
     {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w8w4g64", QuantKernel::GatherSplit84},
     {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64", QuantKernel::QmmSwiglu},
@@ -624,6 +626,24 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
             status = vpq_gather_qmv_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, eid, npair, ival(8), E,
                                                      kind == QuantKernel::GatherGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
           }
+        }
+      } else if (kind == QuantKernel::SortedSwiglu || kind == QuantKernel::SortedDown) {
+        // gpu-kernels/metal/quant/affine_qmv.metal:2682-2708: slot 7 = srow, 8 = tile2e, one tile of two sorted
+        // slots per grid.z.  The expert count is the number of [N, K/8] slabs the bound code buffer holds.
+        if (!buf(7) || !buf(8)) {
+          status = VPQ_ERR_NULL_POINTER;
+        } else if (K <= 0 || N <= 0 || K % 64 != 0) {
+          status = VPQ_ERR_BAD_SHAPE;
+        } else {
+          const std::size_t slab = static_cast<std::size_t>(N) * static_cast<std::size_t>(K / 2);
+          const std::size_t experts = _slots[0].bytes / slab;
+          const int E = experts > 0x7fffffffu ? 0x7fffffff : static_cast<int>(experts);
+          const int npad = static_cast<int>(grid.z) * VPQ_QMV_GROUPED_SLOTS;
+          const int32_t* srow = static_cast<const int32_t*>(buf(7));
+          const int32_t* t2e = static_cast<const int32_t*>(buf(8));
+          status = kind == QuantKernel::SortedDown
+                       ? vpq_qmv_grouped_down_w4g64_bf16(st, w, sc, bi, x, y, K, N, npad, t2e, srow, E)
+                       : vpq_qmv_grouped_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, npad, t2e, srow, E, VPQ_GATE_SWIGLU);
         }
       } else if (kind == QuantKernel::GroupedSwiglu || kind == QuantKernel::GroupedGeglu ||
                  kind == QuantKernel::GroupedDown) {

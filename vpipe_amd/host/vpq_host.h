@@ -89,6 +89,9 @@ enum class QuantKernel : std::uint8_t {
                   //   slot 7 = npad, 8 = tile2e; y [npad, N/2] in slot order
   GroupedGeglu,   // affine_qmm_grouped_geglu_w4g64: as GroupedSwiglu
   GroupedDown,    // affine_qmm_grouped_w4g64: x [npad, K] in slot order, slot 9 = sdst, y rows in pair order
+  SortedSwiglu,   // affine_grouped_swiglu_w4g64: expert batch, tiles of two sorted slots (tile = grid.z), slot 7 = srow
+                  //   (x row per slot, < 0 padding), 8 = tile2e; y [npad, N/2] in slot order
+  SortedDown,     // affine_grouped_down_w4g64: x [npad, K] and y [npad, N] in slot order, slots 7, 8 as SortedSwiglu
   GatherSplit48,  // affine_gather_qmv_swiglu_w4w8g64: slots 0..2 gate pack (4-bit), 3..5 up pack (8-bit), 6:x 7:y 8:K
                   //   9:ffn 10:pair_eid 11:top_k; pairs = grid.z
   GatherSplit84,  // affine_gather_qmv_swiglu_w8w4g64: gate 8-bit, up 4-bit
