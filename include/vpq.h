@@ -204,16 +204,17 @@ int vpq_qmm_splitk_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint
  * 2020-2160: `affine_dequant_w4g64` into a scratch, then a dense matrix-unit GEMM,
  * gpu-kernels/metal/gemm/dense_gemm_mma.metal:44-93): the pack is expanded into
  * `w_deq` (bf16 [N,K], caller-owned, 2*N*K bytes, 16-byte aligned) and
- * y = bf16( x . w_deq^T ) is computed by the vendor BLAS (rocBLAS gemm_ex, bf16
- * operands, fp32 accumulation).  Same arithmetic as vpq_qmm_w4g64_bf16 up to the
- * order of the fp32 additions.  `expand` != 0 runs the expansion first; 0 says
- * that `w_deq` already holds this pack's expansion (a weight is immutable after
- * load, so a caller with the room expands each Linear once).  No adapter on this
- * route.  rocBLAS is opened at first use (that call allocates its handle);
- * VPQ_ERR_UNSUPPORTED with the reason in vpq_last_device_error() if it is not
- * there.  On MI355X this route is the faster one where M is large (measured
- * 1.5 PFLOP/s at M = 16320 against 0.9 fused) and the fused kernel where the
- * 2*N*K bytes are not available. */
+ * y = bf16( x . w_deq^T ) is computed by the library's own dense GEMM (the
+ * large-tile MFMA kernel with the weight tile loaded instead of dequantized:
+ * bf16 operands, fp32 accumulation over K in ascending order, one rounding).
+ * Same arithmetic as vpq_qmm_w4g64_bf16.  `expand` != 0 runs the expansion
+ * first; 0 says that `w_deq` already holds this pack's expansion (a weight is
+ * immutable after load, so a caller with the room expands each Linear once).
+ * No adapter on this route; nothing is allocated and no other library is
+ * loaded.  Requires K % 32 == 0 (K % 64 == 0 for the 64-wide groups of this
+ * entry point anyway).  On MI355X this route is the faster one where M is very
+ * large (measured at M = 16320: 1.3 PFLOP/s against 1.2 fused) and the fused
+ * kernel elsewhere or where the 2*N*K bytes are not available. */
 int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                    int K, int N, int M, uint16_t* w_deq, int expand);
@@ -232,11 +233,11 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
  * M = 8; here the 256-row GEMM tile does not pay below ~64 rows: measured 57 us at
  * 4096->4096 for any M <= 256 against ~10 us per slab.)  Above 32 rows the GEMM
  * splits K (vpq_qmm_splitk_w4g64_bf16) where that pays and `ws` has
- * vpq_qmm_workspace_bytes() bytes (without that room, 33..64 rows stay slabs).  From 1024 rows on, when `ws` holds the
+ * vpq_qmm_workspace_bytes() bytes (without that room, 33..64 rows stay slabs).  From 8192 rows on, when `ws` holds the
  * expanded weight (N*K*2 bytes), the GEMM runs by the dequant-once route
- * (vpq_qmm_dense_route_w4g64_bf16: expansion + vendor GEMM, the reference's route
+ * (vpq_qmm_dense_route_w4g64_bf16: expansion + dense GEMM, the reference's route
  * for large M, minimax-h3/metal-minimax-h3-transformer.cc:2020-2160), which is the
- * faster one there; without that room, or without the vendor BLAS, the fused kernels.
+ * faster one there; below that, or without that room, the fused kernels.
  * vpq_linear_workspace_bytes() is the size that lets the entrance take its best
  * route for the shape (0: none needed); `ws` is 256-byte aligned scratch whose
  * contents are irrelevant and undefined afterwards. */
@@ -455,7 +456,7 @@ int vpq_qmm_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, cons
  *                                    values: replace `affine_qmm_steel_w4g32`
  *                                    (affine_qmm_steel.metal:618-640) and `affine_qmm_geglu_w4g32`
  *                                    (:1573-1596) plus the SwiGLU twin; K % 64 == 0, any M.
- *   vpq_qmm_dense_route_w4g32_bf16   GEMM by expansion into w_deq[N,K] + the vendor GEMM
+ *   vpq_qmm_dense_route_w4g32_bf16   GEMM by expansion into w_deq[N,K] + the library's dense GEMM
  *                                    (expand as in vpq_qmm_dense_route_w4g64_bf16).
  * Requires K % 32 == 0; w, x 16-byte aligned. */
 int vpq_dequant_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
@@ -523,7 +524,7 @@ int vpq_argmax_combine(vpq_stream_t stream, const float* partials, int32_t* out_
  *   vpq_qmm_dense_route_w8g64_bf16   the dequant-once route for any M (replaces
  *                                    `affine_qmm_steel_w8g64`, affine_qmm_steel.metal:1601-1672,
  *                                    by the reference's own second route): expansion into
- *                                    `w_deq` [N,K] bf16 + the vendor dense GEMM; arguments as
+ *                                    `w_deq` [N,K] bf16 + the library's dense GEMM; arguments as
  *                                    vpq_qmm_dense_route_w4g64_bf16.
  *   vpq_qmv_gated_w8g64_bf16         replaces `affine_qmv_swiglu_w8g64` and `affine_qmv_geglu_w8g64`
  *                                    (affine_qmv.metal:3140-3178): interleaved gate|up pack
@@ -597,14 +598,14 @@ int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const
  * metallibs without the `_bf16` suffix).  These entries are the f16 forms of
  * the 4-bit group-64 functions: scales, biases, x, y, residual and w_deq are
  * IEEE binary16 bit patterns, the packed codes are the same.  A first, general
- * path (one wavefront per output row for the QMV, expansion + vendor GEMM for
+ * path (one wavefront per output row for the QMV, expansion + the dense GEMM for
  * the QMM), not tuned like the bf16 kernels:
  *   vpq_dequant_w4g64_f16         `affine_dequant_w4g64` (affine_dequant.metal:25-58), bit-exact:
  *                                 f16_rne(fp32(s) * q + fp32(b)).
  *   vpq_qmv_w4g64_f16 / _f32out   `affine_qmv_w4g64[_add]` (affine_qmv.metal:286-301, 347-363),
  *                                 1 <= M <= 16, fp32 accumulation, un-rounded weights.
  *   vpq_qmv_gated_w4g64_f16       `affine_qmv_swiglu_w4g64`, `affine_qmv_geglu_w4g64` (:891-906, 1432-1447).
- *   vpq_qmm_dense_route_w4g64_f16 the dequant-once route (expansion into w_deq [N,K] f16 + vendor
+ *   vpq_qmm_dense_route_w4g64_f16 the dequant-once route (expansion into w_deq [N,K] f16 + the dense
  *                                 GEMM), arguments as vpq_qmm_dense_route_w4g64_bf16.
  * Requirements as for the bf16 entries. */
 int vpq_dequant_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

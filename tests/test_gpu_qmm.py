@@ -155,7 +155,7 @@ def test_qmm_video_dit_shapes_with_lora(vpq, oracle, dev, D, K, N):
 
 @pytest.mark.parametrize("M,N,K", [(64, 64, 64), (130, 320, 256), (33, 33, 128), (257, 129, 512), (1, 8, 64)])
 def test_qmm_dense_route_matches_oracle(vpq, oracle, dev, D, M, N, K):
-    # the dequant-once route (expansion + vendor dense GEMM): same arithmetic as the fused kernel
+    # the dequant-once route (expansion + the library's dense GEMM): same arithmetic as the fused kernel
     w, s, b = synth.make_weight(N, K, 4200 + N + K)
     x = synth.make_act(M, K, 4300 + M)
     y64, yb = oracle.qmm(w, s, b, x, K, N, M)
@@ -170,6 +170,9 @@ def test_qmm_dense_route_matches_oracle(vpq, oracle, dev, D, M, N, K):
     # with the kept expansion: no expansion pass, same bits
     again = vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq, expand=False)
     assert torch.equal(again, out.view)
+    # and the bits of the fused large-tile kernel: the dense GEMM is that kernel with the weight tile loaded
+    if K % 512 == 0:
+        assert torch.equal(vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, tile_n=256), out.view)
 
 
 @pytest.mark.parametrize("M,N,K,splits", [(100, 256, 2048, 0), (65, 128, 1024, 2), (300, 640, 4096, 0), (257, 129, 1536, 3),
@@ -294,7 +297,7 @@ def test_qmm_large_tile_kernel_refuses_what_it_cannot_take(vpq, dev, D):
 
 
 def test_linear_entrance_takes_the_dequant_once_route_when_given_the_room(vpq, oracle, dev, D):
-    M, N, K = 1100, 384, 512
+    M, N, K = 8200, 384, 512
     w, s, b = synth.make_weight(N, K, 7400)
     x = synth.make_act(M, K, 7401)
     wd, sd, bd, xd = stage(D, dev, w, s, b, x)
@@ -313,6 +316,7 @@ def test_linear_entrance_takes_the_dequant_once_route_when_given_the_room(vpq, o
     ms = np.unique(rng.integers(0, M, 48))
     y64, yb = oracle.qmm(w, s, b, x[ms], K, N, len(ms))
     parity.check_bf16(D.bits(y)[ms], y64, yb)
-    # too little room: the fused kernel, same numbers within the tolerance
+    # too little room: the fused kernel -- the same arithmetic in the same order, so the same bits
     small = vpq.linear_w4g64(wd, sd, bd, xd, K, N, M, ws=ws[:4096])
     parity.check_bf16(D.bits(small)[ms], y64, yb)
+    assert torch.equal(small, y)

@@ -77,8 +77,10 @@ int check_pack(const uint32_t* w, const uint16_t* scales, const uint16_t* biases
 }
 
 // Rows from which the size-based entrance takes the dequant-once route when the workspace holds the
-// expanded weight: the expansion costs ~20 us per 28 MB pack, the vendor GEMM then runs ~1.4x faster.
-constexpr int kDenseRouteMinRows = 1024;
+// expanded weight: the expansion costs ~20 us per 28 MB pack, the dense GEMM then runs ~1.1x faster than the
+// fused kernel where the tiles are many (measured at M = 16320: 1.3 against 1.2 PFLOP/s; at M = 2048 the two
+// are even on 4096->12288 and the fused kernel is ahead on the N = 4096 shapes).
+constexpr int kDenseRouteMinRows = 8192;
 
 int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                const uint16_t* biases, const uint16_t* x, void* y, bool y_f32, int K, int N, int M,
@@ -635,9 +637,8 @@ int vpq_linear_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t
       return VPQ_OK;
     }
   }
-  // Many rows: expanding the pack once into the workspace and running the vendor GEMM on it beats the
-  // fused kernels (measured: 0.98-1.07 against 0.81-0.88 PFLOP/s at M = 2048, 1.35-1.5 against 0.98-1.1
-  // at M = 16320, expansion included), the reference's own route for large M
+  // Very many rows: expanding the pack once into the workspace and running the dense GEMM on it beats the
+  // fused kernels, the reference's own route for large M
   // (generative-models/minimax-h3/metal-minimax-h3-transformer.cc:2020-2160).
   if (ws != nullptr && aligned(ws, 256) && M >= kDenseRouteMinRows && K > 0 && N > 0 && (K % 64) == 0 &&
       ws_bytes >= (size_t)N * (size_t)K * 2 && vpq::dense_gemm_supports(M, N, K)) {
