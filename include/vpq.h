@@ -644,8 +644,9 @@ int vpq_f16_to_bf16(vpq_stream_t stream, const uint16_t* in_f16, uint16_t* out_b
  * n launches; n <= 0 switches it off.  vpq_profile_read() waits for the recorded
  * launches, writes each kernel's duration in milliseconds, in launch order, to
  * kernel_ms[0..capacity) and returns how many launches were recorded (or a
- * negative status), then starts over.  Not for use under graph capture; one
- * thread at a time. */
+ * negative status), then starts over.  Not for use under graph capture.  The
+ * recording state is shared and unsynchronised: while it is on, only one thread
+ * may call into the library. */
 int vpq_profile_enable(int max_launches);
 int vpq_profile_read(float* kernel_ms, int capacity);
 /* The yardsticks a benchmark times beside the product's kernels, in the same run and the same way: a kernel that

@@ -837,4 +837,13 @@ def test_load_and_run_eight_bit_and_group32_packs(vpq, enc, dev, D, tmp_path, M)
         assert tuple(kn) == (K, N)
         want = vpq.linear_twin(kind, D.u32(pack[0], dev), D.bf16(pack[1], dev), D.bf16(pack[2], dev), xd, K, N, M)
         assert torch.equal(yd, want) and yd.abs().sum() > 0
+    # without K: the 8-bit group-64 pack is the one pair of served formats its two shapes agree on; the 4-bit
+    # group-32 shapes fit no group-64 format and the loader asks for K instead of guessing
+    yd = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+    assert L.hd_load_and_run(enc.h, r, b"a", 0, xd.data_ptr(), yd.data_ptr(), M, kn) == 1, L.hr_why()
+    assert tuple(kn) == (K, N)
+    assert torch.equal(yd, vpq.linear_twin("w8g64", D.u32(w8, dev), D.bf16(s8, dev), D.bf16(b8, dev), xd, K, N, M))
+    assert L.hd_load_and_run(enc.h, r, b"b", 0, xd.data_ptr(), yd.data_ptr(), M, kn) == 0
+    assert b"pass K" in L.hr_why()
     L.hr_close(r)

@@ -94,7 +94,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (gate_act != 0 && ((N & 1) != 0 || residual != nullptr || variant == VPQ_QMV_STREAM)) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
-  if (ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }
+  if (variant == VPQ_QMV_MFMA_SPLITK && ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }   // the only user of ws
   if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_FLOW) { return VPQ_ERR_BAD_SHAPE; }
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
@@ -886,7 +886,8 @@ int grouped_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scale
   // the kernel addresses rows of x by 32-bit byte offsets
   const long long xrows = srow != nullptr ? rows : npad;
   if (xrows * (long long)K * 2 >= 4000000000LL) { return VPQ_ERR_BAD_SHAPE; }
-  if (!aligned(x, 16) || !aligned(y, 2) || !aligned(tile2e, 4) || (srow != nullptr && !aligned(srow, 4)) ||
+  // y rows are stored in 4- and 8-byte pieces
+  if (!aligned(x, 16) || !aligned(y, 8) || !aligned(tile2e, 4) || (srow != nullptr && !aligned(srow, 4)) ||
       (sdst != nullptr && !aligned(sdst, 4))) {
     return VPQ_ERR_MISALIGNED;
   }

@@ -101,11 +101,12 @@ __device__ __forceinline__ uint32_t lds_addr(const uint8_t* q)
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)q;
 }
 
-// 16 bytes per lane, global -> LDS at lds_dst + 16 * lane.  M0 is used by nothing else in this kernel.
+// 16 bytes per lane, global -> LDS at lds_dst + 16 * lane.  The LDS base travels in M0, bound as an operand: the
+// compiler writes it and knows its value (the s_nop is the wait state between that write and the load).
 __device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* src)
 {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "{m0}"(m0v) : "memory");
 }
 
 // The same from a wave-uniform base (scalar registers) plus a 32-bit offset per lane: stepping along K
@@ -113,7 +114,7 @@ __device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* src)
 __device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* base, uint32_t lane_off)
 {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(m0v), "v"(lane_off), "s"(base) : "memory");
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_off), "s"(base), "{m0}"(m0v) : "memory");
 }
 
 }  // namespace

@@ -176,11 +176,12 @@ __device__ __forceinline__ uint32_t lds_addr_of(const uint8_t* q)
 }
 
 // 16 bytes per lane, global -> LDS at lds_dst + 16 * lane, written out by hand for the same reason.
-// M0 is used by nothing else in the wavefronts that call this.
+// The LDS base travels in M0, bound as an operand: the compiler writes it and knows its value, as for the
+// builtin form used elsewhere in this kernel (the s_nop is the wait state between that write and the load).
 __device__ __forceinline__ void dma16_raw(uint32_t lds_dst, const uint8_t* src)
 {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "{m0}"(m0v) : "memory");
 }
 
 // Waits until at most YOUNGER vector-memory requests issued after r's are outstanding; the

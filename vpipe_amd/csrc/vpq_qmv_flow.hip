@@ -68,11 +68,12 @@ __device__ __forceinline__ u32x4v gload16(const void* base, uint32_t voff)
   return r;
 }
 
-// 16 bytes per lane, global -> LDS at lds_dst + 16 * lane.  M0 is used by nothing else here.
+// 16 bytes per lane, global -> LDS at lds_dst + 16 * lane.  The LDS base travels in M0, bound as an operand: the
+// compiler writes it and knows its value (the s_nop is the wait state between that write and the load).
 __device__ __forceinline__ void dma16(uint32_t lds_dst, const void* src)
 {
   const uint32_t m0v = __builtin_amdgcn_readfirstlane(lds_dst);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0v), "v"(src) : "memory");
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "{m0}"(m0v) : "memory");
 }
 
 template <int N>

@@ -34,6 +34,8 @@
 // hazard recogniser cannot see what such a statement writes, and a register an
 // MFMA in flight still reads can be overwritten.  Everything here is plain C
 // and builtins.
+#include <atomic>
+
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -419,13 +421,15 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   const size_t lds_bytes = (size_t)nw * p.wave_lds_bytes + (size_t)nw * mr * kWave * sizeof(float);
   const dim3 grid((unsigned)((a.N + kTileN - 1) / kTileN), (unsigned)split), block((unsigned)(nw * kWave));
 
-  static bool attr_done[8] = {false, false, false, false, false, false, false, false};
+  // the attribute is set once per kernel, whichever thread comes first (atomic flags: two threads may both set
+  // it, which is harmless; neither launches before its own call has returned)
+  static std::atomic<bool> attr_done[8];
   auto launch = [&](auto kern, int slot) -> hipError_t {
-    if (!attr_done[slot]) {
+    if (!attr_done[slot].load(std::memory_order_acquire)) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
       if (e != hipSuccess) { return e; }
-      attr_done[slot] = true;
+      attr_done[slot].store(true, std::memory_order_release);
     }
     return launch_kernel(kern, grid, block, lds_bytes, st, p);
   };
@@ -474,13 +478,13 @@ hipError_t launch_qmv_mfma_group(hipStream_t st, const QmvArgs& a, const QmvGrou
   p.wave_lds_bytes = kItemBytes + (xlds ? a.M * kXRowBytes + kXsumBytes : 0);
   const size_t lds_bytes = (size_t)nw * p.wave_lds_bytes + (size_t)nw * mr * kWave * sizeof(float);
   const dim3 grid((unsigned)tiles, 1u), block((unsigned)(nw * kWave));
-  static bool attr_done[3] = {false, false, false};
+  static std::atomic<bool> attr_done[3];
   auto launch = [&](auto kern, int slot) -> hipError_t {
-    if (!attr_done[slot]) {
+    if (!attr_done[slot].load(std::memory_order_acquire)) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsBytes);
       if (e != hipSuccess) { return e; }
-      attr_done[slot] = true;
+      attr_done[slot].store(true, std::memory_order_release);
     }
     return launch_kernel(kern, grid, block, lds_bytes, st, p);
   };

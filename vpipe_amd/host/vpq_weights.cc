@@ -368,6 +368,11 @@ bool PackFile::add_shard(const std::string& path, std::string* why)
         return false;
       }
       ti.shape.push_back(d.inum);
+      // keeps the element count below 2^56, so that count * element size cannot wrap
+      if (d.inum != 0 && count > ((std::uint64_t)1 << 56) / (std::uint64_t)d.inum) {
+        set_why(why, path + ": shape of '" + m.first + "' too large");
+        return false;
+      }
       count *= (std::uint64_t)d.inum;
     }
     const Json& b0 = off->items[0];
@@ -528,7 +533,26 @@ bool PackFile::load_linear(CommandStream& stream, const std::string& prefix, int
     set_why(why, prefix + ": not a U32 [N, K*bits/32] weight with F16 or BF16 [N, K/group] scales and biases");
     return false;
   }
-  if (K <= 0) { K = (int)(w->shape[1] * 8); }
+  if (K <= 0) {
+    // No K given: the (width, group) pair that both shapes agree on, among the served ones; K from it.  The shapes
+    // alone cannot tell 4-bit group-32 from 8-bit group-64 (same words and same scales per row), so a caller with
+    // such packs passes K.
+    const long long words = w->shape[1], groups = s->shape[1];
+    int found = 0;
+    const int cand[2][2] = {{4, 64}, {8, 64}};
+    for (const auto& c : cand) {
+      const long long k = words * 32 / c[0];
+      if (words * 32 % c[0] == 0 && k % c[1] == 0 && k / c[1] == groups && k <= 0x7fffffffLL) {
+        K = (int)k;
+        ++found;
+      }
+    }
+    if (found != 1) {
+      set_why(why, prefix + ": cannot tell the width and group from a [N, " + std::to_string(words) + "] weight with [N, " +
+                       std::to_string(groups) + "] scales; pass K");
+      return false;
+    }
+  }
   const int N = (int)w->shape[0];
   // Width and group from the shapes (generative-models/qwen3/metal-qwen-model.cc:653-676); served: 4-bit group-64,
   // 8-bit group-64, 4-bit group-32.
