@@ -36,17 +36,18 @@ MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16
 # committed summary of two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE per dispatch, scaled by what the
 # same counters read for a device-to-device copy of known size); the file states the build it was taken from.
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qmv_flow_kernel_decode_layer_m1_hbm_traffic_pmc.txt")
+QMM_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qmm_big_kernel_m2048_mfma_lds_traffic_pmc.txt")
 
 
-def traffic_from_profile():
-    """(bytes per layer, text naming the profiled build) from the committed summary, or (None, None)."""
+def traffic_from_profile(path=TRAFFIC_PROFILE, key="traffic_bytes_per_layer:"):
+    """(bytes under `key`, text naming the profiled build) from a committed summary, or (None, None)."""
     try:
-        text = open(TRAFFIC_PROFILE).read()
+        text = open(path).read()
     except OSError:
         return None, None
     val, build = None, None
     for line in text.splitlines():
-        if line.startswith("traffic_bytes_per_layer:"):
+        if line.startswith(key):
             val = float(line.split(":", 1)[1])
         if line.startswith("build:"):
             build = line.split(":", 1)[1].strip()
@@ -439,9 +440,14 @@ def main():
             del w, s, b, x, y
         ach = tot_flops / (tot_us * 1e-6) / 1e12
         out["qmm_m2048"] = qmm
+        qmm_traffic, qmm_traffic_build = traffic_from_profile(QMM_TRAFFIC_PROFILE, "traffic_bytes_4096x12288_m2048:")
         out["roofline_qmm"] = {"bound": "mfma", "achieved": round(ach, 1), "peak": MFMA_BF16_PEAK_TF,
-                               "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TF, 4), "traffic": None,
-                               "kernel": "qmm_big_kernel<3,false> (4096->12288: 256x192 tiles) and qmm_big_kernel<2,false> "
+                               "unit": "TFLOP/s", "frac": round(ach / MFMA_BF16_PEAK_TF, 4), "traffic": qmm_traffic,
+                               "traffic_of": "one 4096->12288 launch at M = 2048 (fetched + written; algorithmic 95.4 MB), "
+                                             "profiles/" + os.path.basename(QMM_TRAFFIC_PROFILE) + " (" + str(qmm_traffic_build) + ")",
+                               "traffic_profile_is_of_this_build": bool(qmm_traffic_build) and
+                                                                   str(qmm_traffic_build).split()[0] == vpipe_amd.build_id(),
+                               "kernel": "qmm_big_kernel<3,false,0> (4096->12288: 256x192 tiles) and qmm_big_kernel<2,false,0> "
                                          "(12288->4096, 4096->4096: 256x128 tiles); flops of the three over their time",
                                "timing": "us per call over 20 back-to-back calls after 40 ms of the same calls "
                                          "(the clocks the box settles at), events on the stream",
