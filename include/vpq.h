@@ -423,7 +423,8 @@ int vpq_qmv_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, cons
  * rounding): a slot's result has the bits of vpq_qmm_tiled_w4g64_bf16 (tile
  * 128) on that row and that expert's slab.  Requires K % 64 == 0, npad a
  * positive multiple of vpq_qmm_grouped_block_rows(), N even for the gated form,
- * rows * K * 2 < 4e9 for x; w, x 16-byte aligned. */
+ * rows * K * 2 < 4e9 for x; w, x 16-byte aligned, y 8-byte aligned (its rows are
+ * stored in 4- and 8-byte pieces). */
 int vpq_qmm_grouped_block_rows(void);
 size_t vpq_moe_sort_workspace_bytes(int n_experts);
 int vpq_moe_sort_pairs(vpq_stream_t stream, const int32_t* pair_eid, int npair, int top_k, int n_experts,
