@@ -661,6 +661,12 @@ def main():
         out["argmax_v151936"] = {
             "two_stage_us": round(kernel_us(lambda i: vpipe_amd.argmax_bf16(lg, out=tok, two_stage=True), 16), 2),
             "one_workgroup_us": round(kernel_us(lambda i: vpipe_amd.argmax_bf16(lg, out=tok, two_stage=False), 16), 2)}
+        # stochastic tail: the one-workgroup sampler (top-k 50, top-p 0.9, 24 bisection steps each) over the same logits
+        seen_b = torch.zeros((151936,), dtype=torch.uint8, device=dev)
+        ws_b = torch.empty((151936,), dtype=torch.bfloat16, device=dev)
+        out["sample_topp_v151936"] = {
+            "one_workgroup_us": round(kernel_us(lambda i: vpipe_amd.sample_topp_bf16(lg.view(-1), seen_b, 0.8, 0.9, 1000 + i,
+                                                                                      ws=ws_b, out=tok, top_k=50), 8), 1)}
 
         # MoE decode block, pair-batched gathers (hidden 2048, expert inner 768, 128 experts, top-8,
         # one token): 8 of the 128 gate|up slabs and 8 down slabs per step, a fresh random set of

@@ -637,6 +637,28 @@ int vpq_quantize_w4g64(vpq_stream_t stream, const uint16_t* src, uint32_t* w,
  * (docs/PLUGINS.md:210-213). */
 int vpq_f16_to_bf16(vpq_stream_t stream, const uint16_t* in_f16, uint16_t* out_bf16, size_t count);
 
+/* ---- the stochastic sampler tail ------------------------------------------
+ * vpq_sample_topp_bf16 replaces `sample_topp_f16`
+ * (gpu-kernels/metal/ops/llm_elementwise.metal:3116-3262; slots 0:logits
+ * 1:out_id 2:V 3:temp 4:top_p 5:seed 6:ws 7:n_iter 8:rep_penalty
+ * 9:presence_penalty 10:top_k 11:min_p 12:seen; one threadgroup): the whole
+ * sampler over one row of bf16 logits on the device, in the host sampler's
+ * order -- repetition and presence penalty on the tokens marked in `seen`
+ * ([V] bytes, in/out: the drawn token is marked), temperature, softmax weights
+ * (cached in `ws`, [V] bf16 scratch), top-k (0 or >= V: off), min-p, top-p as
+ * weight thresholds found by n_iter bisection steps each, then a Gumbel-max
+ * draw over the kept set with a hash of (seed, index), lowest index on ties;
+ * token 0 if nothing is kept.  The draw is an exact function of its inputs:
+ * exp, log and the reduction order are fixed (see vpq_sample.hip), so the
+ * same (logits, seen, parameters, seed) give the same token on every run.
+ * The reference's multi-threadgroup histogram variant (:3318-3574), which
+ * loosens the thresholds to bin edges, is not built.
+ * Requires V >= 1, n_iter >= 0, rep != 0; all pointers non-NULL, logits and ws
+ * 2-byte, out_id 4-byte aligned. */
+int vpq_sample_topp_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, float temp,
+                         float top_p, uint32_t seed, uint16_t* ws, int n_iter, float rep_penalty,
+                         float presence_penalty, int top_k, float min_p, uint8_t* seen);
+
 /* ---- measurement aid (no counterpart in the reference's kernels; the
  * reference times command buffers with Fence::gpu_times(),
  * apple-silicon/metal-compute/command-stream.h:119-126) -----------------------

@@ -128,6 +128,42 @@ def argmax(logits):
     return out
 
 
+def sample_exp(x):
+    L = lib()
+    L.vpo_sample_exp.restype = ctypes.c_float
+    L.vpo_sample_exp.argtypes = [ctypes.c_float]
+    return np.array([L.vpo_sample_exp(float(v)) for v in np.asarray(x, dtype=np.float32).ravel()], dtype=np.float32)
+
+
+def sample_log(x):
+    L = lib()
+    L.vpo_sample_log.restype = ctypes.c_float
+    L.vpo_sample_log.argtypes = [ctypes.c_float]
+    return np.array([L.vpo_sample_log(float(v)) for v in np.asarray(x, dtype=np.float32).ravel()], dtype=np.float32)
+
+
+def sample_hash_u01(x):
+    L = lib()
+    L.vpo_sample_hash_u01.restype = ctypes.c_float
+    L.vpo_sample_hash_u01.argtypes = [ctypes.c_uint32]
+    return np.array([L.vpo_sample_hash_u01(int(v)) for v in np.asarray(x, dtype=np.uint32).ravel()], dtype=np.float32)
+
+
+def sample_topp(logits, seen, temp, top_p, seed, n_iter=24, rep=1.0, pres=0.0, top_k=0, min_p=0.0):
+    """bf16 bits [V], uint8 [V] -> (token, cached weights bf16 bits [V], seen after the draw)."""
+    L = lib()
+    L.vpo_sample_topp_bf16.restype = ctypes.c_int32
+    L.vpo_sample_topp_bf16.argtypes = [_u16p, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_uint32, _u16p,
+                                       ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_float,
+                                       ctypes.POINTER(ctypes.c_uint8)]
+    logits = _c(logits, np.uint16)
+    seen = np.array(seen, dtype=np.uint8, copy=True)
+    ws = np.empty(logits.shape, dtype=np.uint16)
+    tok = L.vpo_sample_topp_bf16(_p(logits, _u16p), logits.size, temp, top_p, seed, _p(ws, _u16p), n_iter, rep, pres, top_k,
+                                 min_p, seen.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)))
+    return int(tok), ws, seen
+
+
 def qmv(w, s, b, x, K, N, M, residual=None):
     """-> (y64 [M,N] float64, y_bf16 [M,N] uint16); un-rounded-weight semantics."""
     w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)

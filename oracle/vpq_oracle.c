@@ -239,6 +239,179 @@ void vpo_argmax_bf16(const uint16_t* logits, int32_t* out_id, int V, int rows)
   }
 }
 
+/* ---- the stochastic sampler tail ------------------------------------------
+ * gpu-kernels/metal/ops/llm_elementwise.metal:3063-3298 (`sample_topp_f16`): repetition and presence penalty ->
+ * temperature -> softmax weights (cached in the element type) -> top-k, min-p, top-p as weight thresholds found by
+ * bisection -> Gumbel-max draw over the kept set with a hash of (seed, index), lowest index on ties; 0 if nothing
+ * is kept; the drawn token is marked seen.  The reference leaves the last bits of exp, log and of its reduction
+ * order to Metal; they are pinned here to explicit fp32 operations (this file is compiled without contraction):
+ *   exp, log    the Cephes single-precision polynomials, written out;
+ *   reductions  thread t of 1024 takes the indices t, t + 1024, ... in ascending order, the 1024 partial results
+ *               meet in a halving tree a[t] op= a[t + s], s = 512 .. 1 (the reference's own loop, :3141-3146). */
+#define VPO_SAMPLE_THREADS 1024
+
+float vpo_sample_exp(float x)
+{
+  if (!(x >= -87.0f)) { return 0.0f; }
+  const float n = rintf(x * 1.44269504088896341f);
+  float r = x - n * 0.693359375f;
+  r = r - n * -2.12194440e-4f;
+  float p = 1.9875691500e-4f;
+  p = p * r + 1.3981999507e-3f;
+  p = p * r + 8.3334519073e-3f;
+  p = p * r + 4.1665795894e-2f;
+  p = p * r + 1.6666665459e-1f;
+  p = p * r + 5.0000001201e-1f;
+  p = p * (r * r) + r;
+  p = p + 1.0f;
+  union { uint32_t u; float f; } sc;
+  sc.u = (uint32_t)((int)n + 127) << 23;
+  return p * sc.f;
+}
+
+float vpo_sample_log(float x)
+{
+  union { uint32_t u; float f; } v;
+  v.f = x;
+  int e = (int)(v.u >> 23) - 126;
+  v.u = (v.u & 0x007fffffu) | 0x3f000000u;
+  float m = v.f;
+  if (m < 0.707106781186547524f) {
+    e -= 1;
+    m = m + m - 1.0f;
+  } else {
+    m = m - 1.0f;
+  }
+  const float z = m * m;
+  float y = 7.0376836292e-2f;
+  y = y * m + -1.1514610310e-1f;
+  y = y * m + 1.1676998740e-1f;
+  y = y * m + -1.2420140846e-1f;
+  y = y * m + 1.4249322787e-1f;
+  y = y * m + -1.6668057665e-1f;
+  y = y * m + 2.0000714765e-1f;
+  y = y * m + -2.4999993993e-1f;
+  y = y * m + 3.3333331174e-1f;
+  y = y * m * z;
+  const float fe = (float)e;
+  y = y + fe * -2.12194440e-4f;
+  y = y - 0.5f * z;
+  float r = m + y;
+  r = r + fe * 0.693359375f;
+  return r;
+}
+
+/* llm_elementwise.metal:3096-3104 */
+float vpo_sample_hash_u01(uint32_t x)
+{
+  x ^= x >> 16; x *= 0x7feb352dU;
+  x ^= x >> 15; x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return ((float)x + 0.5f) * (1.0f / 4294967296.0f);
+}
+
+/* llm_elementwise.metal:3106-3113 */
+static float vpo_sample_eff(float v, int seen, float rep, float pres)
+{
+  if (seen) {
+    v = (v >= 0.0f) ? (v / rep) : (v * rep);
+    v -= pres;
+  }
+  return v;
+}
+
+static float vpo_tree_f(float* a, int is_max)
+{
+  for (int s = VPO_SAMPLE_THREADS >> 1; s > 0; s >>= 1) {
+    for (int t = 0; t < s; ++t) { a[t] = is_max ? (a[t] > a[t + s] ? a[t] : a[t + s]) : (a[t] + a[t + s]); }
+  }
+  return a[0];
+}
+
+/* ws [V] receives the cached weights (element type), seen [V] is read and the drawn token set; returns the token. */
+int32_t vpo_sample_topp_bf16(const uint16_t* logits, int V, float temp, float top_p, uint32_t seed, uint16_t* ws,
+                             int n_iter, float rep, float pres, int top_k, float min_p, uint8_t* seen)
+{
+  const int T = VPO_SAMPLE_THREADS;
+  float tg[VPO_SAMPLE_THREADS];
+  int tgi[VPO_SAMPLE_THREADS];
+  const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
+  for (int t = 0; t < T; ++t) {
+    float m = -INFINITY;
+    for (int i = t; i < V; i += T) {
+      const float e = vpo_sample_eff(vpo_bf16_to_f32(logits[i]), seen[i] != 0, rep, pres);
+      m = e > m ? e : m;
+    }
+    tg[t] = m;
+  }
+  const float maxl = vpo_tree_f(tg, 1);
+  for (int t = 0; t < T; ++t) {
+    float z = 0.0f;
+    for (int i = t; i < V; i += T) {
+      const float e = vpo_sample_eff(vpo_bf16_to_f32(logits[i]), seen[i] != 0, rep, pres);
+      const float w = vpo_sample_exp((e - maxl) * inv_t);
+      ws[i] = vpo_f32_to_bf16(w);
+      z = z + w;
+    }
+    tg[t] = z;
+  }
+  const float Z = vpo_tree_f(tg, 0);
+  const float target = top_p * Z;
+  float t_k = 0.0f;
+  if (top_k > 0 && top_k < V) {
+    float lo = 0.0f, hi = 1.0f;
+    for (int it = 0; it < n_iter; ++it) {
+      const float mid = 0.5f * (lo + hi);
+      long C = 0;
+      for (int i = 0; i < V; ++i) { C += vpo_bf16_to_f32(ws[i]) >= mid; }      /* integer: the order is irrelevant */
+      if (C >= top_k) { lo = mid; } else { hi = mid; }
+    }
+    t_k = lo;
+  }
+  const float t_mp = fmaxf(min_p, 0.0f);
+  const float t_floor = fmaxf(t_k, t_mp);
+  float lo = t_floor, hi = 1.0f;
+  for (int it = 0; it < n_iter; ++it) {
+    const float mid = 0.5f * (lo + hi);
+    for (int t = 0; t < T; ++t) {
+      float mass = 0.0f;
+      for (int i = t; i < V; i += T) {
+        const float w = vpo_bf16_to_f32(ws[i]);
+        if (w >= mid) { mass = mass + w; }
+      }
+      tg[t] = mass;
+    }
+    const float M = vpo_tree_f(tg, 0);
+    if (M >= target) { lo = mid; } else { hi = mid; }
+  }
+  const float wt = fmaxf(lo, t_floor);
+  for (int t = 0; t < T; ++t) {
+    float best = -INFINITY;
+    int bi = -1;
+    for (int i = t; i < V; i += T) {
+      if (vpo_bf16_to_f32(ws[i]) >= wt) {
+        const float e = vpo_sample_eff(vpo_bf16_to_f32(logits[i]), seen[i] != 0, rep, pres);
+        const float u = vpo_sample_hash_u01(seed ^ ((uint32_t)i * 2654435761u + 1u));
+        const float a = 0.0f - vpo_sample_log(u + 1e-20f) + 1e-20f;
+        const float g = 0.0f - vpo_sample_log(a);
+        const float score = e * inv_t + g;
+        if (score > best) { best = score; bi = i; }
+      }
+    }
+    tg[t] = best;
+    tgi[t] = bi;
+  }
+  for (int s = T >> 1; s > 0; s >>= 1) {
+    for (int t = 0; t < s; ++t) {
+      const int take = tg[t + s] > tg[t] || (tg[t + s] == tg[t] && tgi[t + s] >= 0 && (tgi[t] < 0 || tgi[t + s] < tgi[t]));
+      if (take) { tg[t] = tg[t + s]; tgi[t] = tgi[t + s]; }
+    }
+  }
+  const int pick = tgi[0] >= 0 ? tgi[0] : 0;
+  seen[pick] = 1;
+  return pick;
+}
+
 /* ---- a2/a3: QMV -------------------------------------------------------- */
 
 /* The CPU reference loop of the reference's own QMV test,

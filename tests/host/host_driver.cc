@@ -66,6 +66,11 @@ void hd_set_constant_i32(void* h, unsigned index, int value)
   static_cast<Session*>(h)->enc.set_constant(index, value);
 }
 
+void hd_set_constant_f32(void* h, unsigned index, float value)
+{
+  static_cast<Session*>(h)->enc.set_constant(index, value);
+}
+
 void hd_dispatch(void* h, unsigned gx, unsigned gy, unsigned gz, unsigned tx, unsigned ty, unsigned tz)
 {
   static_cast<Session*>(h)->enc.dispatch(LaunchDims{gx, gy, gz}, LaunchDims{tx, ty, tz});

@@ -59,6 +59,10 @@ class Driver:
     def set_constant(self, index, v):
         self.L.hd_set_constant_i32(self.h, index, int(v))
 
+    def set_constant_f32(self, index, v):
+        self.L.hd_set_constant_f32.argtypes = [ctypes.c_void_p, ctypes.c_uint, ctypes.c_float]
+        self.L.hd_set_constant_f32(self.h, index, float(v))
+
     def dispatch(self, grid, tg):
         torch.cuda.synchronize()   # the tests stage their tensors on torch's stream
         self.L.hd_dispatch(self.h, *grid, *tg)
@@ -592,6 +596,38 @@ def test_argmax_call_sites_of_the_host_layer(enc, oracle, dev, D):
     ok, why = enc.wait_ok()
     assert ok, why
     assert out.cpu().tolist() == [want, want]
+
+
+def test_sampler_call_site_of_the_host_layer(enc, oracle, dev, D):
+    # llm::Sampler on the device (gpu-kernels/metal/ops/llm_elementwise.metal:3116-3130): one threadgroup, thirteen slots
+    V = 6000
+    bits = synth.f32_to_bf16_bits((np.random.default_rng(2300).standard_normal(V) * 3).astype(np.float32))
+    seen = np.zeros(V, dtype=np.uint8)
+    seen[::7] = 1
+    want, ws_want, seen_want = oracle.sample_topp(bits, seen, 0.8, 0.9, 4242, n_iter=20, rep=1.3, pres=0.2, top_k=64, min_p=0.01)
+    ld, out = D.bf16(bits, dev), torch.zeros((1,), dtype=torch.int32, device=dev)
+    ws = torch.zeros((V,), dtype=torch.bfloat16, device=dev)
+    seen_d = torch.from_numpy(seen.copy()).to(dev)
+    torch.cuda.synchronize()
+    assert enc.set_function("llm_elementwise_bf16", "sample_topp_f16") == 1
+    enc.set_buffer(0, ld)
+    enc.set_buffer(1, out)
+    enc.set_constant(2, V)
+    enc.set_constant_f32(3, 0.8)
+    enc.set_constant_f32(4, 0.9)
+    enc.set_constant(5, 4242)
+    enc.set_buffer(6, ws)
+    enc.set_constant(7, 20)
+    enc.set_constant_f32(8, 1.3)
+    enc.set_constant_f32(9, 0.2)
+    enc.set_constant(10, 64)
+    enc.set_constant_f32(11, 0.01)
+    enc.set_buffer(12, seen_d)
+    enc.dispatch((1, 1, 1), (256, 1, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert int(out.cpu()[0]) == want
+    assert np.array_equal(D.bits(ws), ws_want) and np.array_equal(seen_d.cpu().numpy(), seen_want)
 
 
 def test_eight_bit_and_group32_function_names(enc, oracle, dev, D):

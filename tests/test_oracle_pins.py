@@ -639,3 +639,103 @@ def test_cpu_baseline_stages_agree_with_the_oracle(oracle):
         g = synth.bf16_bits_to_f32(got).astype(np.float64)
         rms = np.sqrt((y64 ** 2).mean())
         assert (np.abs(g - y64) / np.maximum(np.abs(y64), 1e-2 * rms)).max() < 1e-2
+
+
+# ---- the sampler tail (llm_elementwise.metal:3063-3298) ---------------------------------------------
+
+def _sampler_kept_set_f64(logits_f, seen, temp, top_p, rep, pres, top_k, min_p):
+    """The host sampler's pipeline in float64 with a sort (no bisection): the set of tokens that survive, and their
+    probabilities.  Independent of the oracle's thresholds; equal to them wherever no weight sits at a threshold."""
+    v = logits_f.astype(np.float64)
+    pen = np.where(v >= 0, v / rep, v * rep) - pres
+    eff = np.where(seen != 0, pen, v)
+    w = np.exp((eff - eff.max()) / max(temp, 1e-6))
+    keep = np.ones(w.shape, dtype=bool)
+    if 0 < top_k < w.size:
+        keep &= w >= np.sort(w)[::-1][top_k - 1]
+    keep &= w >= max(min_p, 0.0)
+    order = np.argsort(-w * keep, kind="stable")
+    csum = np.cumsum((w * keep)[order])
+    n_nucleus = int(np.searchsorted(csum, top_p * w.sum(), side="left")) + 1
+    nucleus = np.zeros_like(keep)
+    nucleus[order[:n_nucleus]] = True
+    keep &= nucleus
+    p = w * keep
+    return keep, p / p.sum(), eff
+
+
+def test_sampler_exp_log_and_hash_are_what_they_say(oracle):
+    x = np.concatenate([np.linspace(-87, 0, 4001), -np.geomspace(1e-8, 80, 500)]).astype(np.float32)
+    e = oracle.sample_exp(x).astype(np.float64)
+    assert np.max(np.abs(e - np.exp(x.astype(np.float64))) / np.exp(x.astype(np.float64))) < 2e-7
+    assert oracle.sample_exp([-88.0, -1e9, -np.inf])[0] == 0 and not oracle.sample_exp([-1e9, -np.inf, np.nan]).any()
+    assert oracle.sample_exp([0.0])[0] == 1.0
+    u = np.concatenate([np.geomspace(1e-20, 1, 3000), np.linspace(0.5, 2, 701), [46.0, 3.4e38]]).astype(np.float32)
+    l = oracle.sample_log(u).astype(np.float64)
+    ref = np.log(u.astype(np.float64))
+    assert np.max(np.abs(l - ref) / np.maximum(np.abs(ref), 1e-3)) < 2e-7
+    assert oracle.sample_log([1.0])[0] == 0.0
+    # the hash, re-stated with Python integers (llm_elementwise.metal:3096-3104)
+    def h(x):
+        x ^= x >> 16; x = (x * 0x7feb352d) & 0xffffffff
+        x ^= x >> 15; x = (x * 0x846ca68b) & 0xffffffff
+        x ^= x >> 16
+        return np.float32((np.float32(x) + np.float32(0.5)) * np.float32(1.0 / 4294967296.0))
+    xs = [0, 1, 2, 12345, 0x80000000, 0xffffffff, 2654435761]
+    assert np.array_equal(oracle.sample_hash_u01(xs), np.array([h(v) for v in xs], dtype=np.float32))
+    us = oracle.sample_hash_u01(np.arange(200000, dtype=np.uint32))
+    assert 0 < us.min() and us.max() <= 1.0 and abs(us.mean() - 0.5) < 5e-3
+
+
+def test_sampler_degenerate_settings_reduce_to_argmax(oracle):
+    rng = np.random.default_rng(31)
+    V = 5000
+    bits = synth.f32_to_bf16_bits((rng.standard_normal(V) * 4).astype(np.float32))
+    seen = np.zeros(V, dtype=np.uint8)
+    top = int(oracle.argmax(bits)[0])
+    for seed in range(5):
+        assert oracle.sample_topp(bits, seen, 1.0, 1.0, seed, top_k=1)[0] == top          # only the best survives
+        assert oracle.sample_topp(bits, seen, 1.0, 1e-6, seed)[0] == top                  # a nucleus of one
+        assert oracle.sample_topp(bits, seen, 1.0, 1.0, seed, min_p=1.0)[0] == top        # floor at the largest weight
+        assert oracle.sample_topp(bits, seen, 1e-4, 1.0, seed)[0] == top                  # temperature -> 0
+    tok, ws, seen_after = oracle.sample_topp(bits, seen, 0.8, 0.9, 7)
+    assert seen_after[tok] == 1 and seen_after.sum() == 1 and not seen.any()
+    assert synth.bf16_bits_to_f32(ws).max() == 1.0                                        # the largest weight is exactly 1
+    # a repetition penalty that pushes the favourite below the runner-up changes the greedy answer
+    vals = np.full(V, -5.0, dtype=np.float32); vals[10] = 4.0; vals[20] = 3.5
+    bits2 = synth.f32_to_bf16_bits(vals)
+    seen2 = np.zeros(V, dtype=np.uint8); seen2[10] = 1
+    assert oracle.sample_topp(bits2, seen2, 1.0, 1.0, 0, top_k=1)[0] == 10                # 4.0 / 1.0 still first
+    assert oracle.sample_topp(bits2, seen2, 1.0, 1.0, 0, top_k=1, rep=1.5)[0] == 20       # 4 / 1.5 < 3.5
+    assert oracle.sample_topp(bits2, seen2, 1.0, 1.0, 0, top_k=1, pres=1.0)[0] == 20      # 4 - 1 < 3.5
+    vals[10] = -1.0; vals[20] = -1.2                                                      # negative logits are multiplied
+    assert oracle.sample_topp(synth.f32_to_bf16_bits(vals), seen2, 1.0, 1.0, 0, top_k=1, rep=1.5)[0] == 20
+
+
+@pytest.mark.parametrize("temp,top_p,top_k,min_p,rep,pres", [(1.0, 1.0, 0, 0.0, 1.0, 0.0), (0.7, 0.9, 0, 0.0, 1.0, 0.0),
+                                                            (1.3, 1.0, 12, 0.0, 1.0, 0.0), (1.0, 0.95, 40, 0.02, 1.2, 0.3)])
+def test_sampler_draws_from_the_filtered_distribution(oracle, temp, top_p, top_k, min_p, rep, pres):
+    """Over many seeds the drawn tokens lie in the kept set of an independent float64 restatement of the pipeline
+    (sorted, no bisection) and follow its renormalised probabilities (chi-square)."""
+    rng = np.random.default_rng(41)
+    V = 300
+    vals = (rng.standard_normal(V) * 2.0).astype(np.float32)
+    bits = synth.f32_to_bf16_bits(vals)
+    seen = (rng.random(V) < 0.2).astype(np.uint8)
+    keep, prob, _ = _sampler_kept_set_f64(synth.bf16_bits_to_f32(bits), seen, temp, top_p, rep, pres, top_k, min_p)
+    draws = 6000
+    counts = np.zeros(V)
+    for seed in range(draws):
+        tok, ws, _ = oracle.sample_topp(bits, seen, temp, top_p, seed * 2654435761 % (1 << 32), n_iter=30, rep=rep, pres=pres,
+                                        top_k=top_k, min_p=min_p)
+        counts[tok] += 1
+    # thresholds sit between weights (bf16-cached), so the kept set may differ from the float64 one by tokens whose
+    # weight is within bf16 rounding of a threshold: allow those, nothing else
+    w = synth.bf16_bits_to_f32(ws).astype(np.float64)
+    outside = np.nonzero((counts > 0) & ~keep)[0]
+    edge = w[keep].min() if keep.any() else 0.0
+    assert all(abs(w[i] - edge) <= edge * 2.0 ** -7 for i in outside), outside
+    big = keep & (prob * draws >= 8)
+    chi2 = (((counts[big] - prob[big] * draws) ** 2) / (prob[big] * draws)).sum()
+    dof = int(big.sum())
+    assert chi2 < dof + 6 * np.sqrt(2 * dof) + 10, (chi2, dof)

@@ -46,6 +46,7 @@ SYMBOLS = [
     ("vpq_moe_sort_pairs", _i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _sz]),
     ("vpq_qmm_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _i]),
     ("vpq_qmm_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
+    ("vpq_sample_topp_bf16", _i, [_vp, _vp, _vp, _i, _f, _f, ctypes.c_uint32, _vp, _i, _f, _f, _i, _f, _vp]),
     ("vpq_qmv_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
     ("vpq_qmv_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i]),
     ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
@@ -237,6 +238,19 @@ def argmax_bf16(logits, out=None, two_stage=True):
         ws_bytes = L.vpq_argmax_workspace_bytes(V, rows)
         ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=logits.device)
     _check(L.vpq_argmax_bf16(_stream(), _ptr(logits), _ptr(out), V, rows, _ptr(ws), ws_bytes), "vpq_argmax_bf16")
+    return out
+
+
+def sample_topp_bf16(logits, seen, temp, top_p, seed, ws=None, out=None, n_iter=24, rep=1.0, pres=0.0, top_k=0, min_p=0.0):
+    """One row of bf16 logits [V] and its seen flags (uint8 [V], updated in place) -> int32 [1] with the drawn token."""
+    import torch
+    V = logits.numel()
+    if ws is None:
+        ws = torch.empty((V,), dtype=torch.bfloat16, device=logits.device)
+    if out is None:
+        out = torch.empty((1,), dtype=torch.int32, device=logits.device)
+    _check(load().vpq_sample_topp_bf16(_stream(), _ptr(logits), _ptr(out), V, temp, top_p, seed, _ptr(ws), n_iter, rep, pres,
+                                       top_k, min_p, _ptr(seen)), "vpq_sample_topp_bf16")
     return out
 
 

@@ -837,6 +837,19 @@ int vpq_qmv_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, cons
   return sorted_qmv_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, srow, n_experts, 0, false);
 }
 
+int vpq_sample_topp_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, float temp,
+                         float top_p, uint32_t seed, uint16_t* ws, int n_iter, float rep_penalty,
+                         float presence_penalty, int top_k, float min_p, uint8_t* seen)
+{
+  if (logits == nullptr || out_id == nullptr || ws == nullptr || seen == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (V < 1 || n_iter < 0 || rep_penalty == 0.0f) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(logits, 2) || !aligned(ws, 2) || !aligned(out_id, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_sample_topp(reinterpret_cast<hipStream_t>(stream), logits, out_id, V, temp, top_p, seed, ws,
+                                        n_iter, rep_penalty, presence_penalty, top_k, min_p, seen));
+}
+
 int vpq_qmm_grouped_block_rows(void) { return vpq::kGroupedBlockRows; }
 
 size_t vpq_moe_sort_workspace_bytes(int n_experts)

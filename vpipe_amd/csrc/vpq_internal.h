@@ -207,4 +207,9 @@ hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out,
 hipError_t launch_interleave_rows(hipStream_t st, const void* a, const void* b, void* out, size_t row_bytes,
                                   size_t rows);
 
+// The sampler tail (vpq_sample.hip): one workgroup over one row of logits.
+hipError_t launch_sample_topp(hipStream_t st, const uint16_t* logits, int32_t* out_id, int V, float temp, float top_p,
+                              uint32_t seed, uint16_t* ws, int n_iter, float rep, float pres, int top_k, float min_p,
+                              uint8_t* seen);
+
 }  // namespace vpq

@@ -94,6 +94,7 @@ const FnEntry kFunctions[] = {
     {"llm_elementwise_bf16", "argmax_f16", QuantKernel::Argmax},
     {"llm_elementwise_bf16", "argmax_partial_f16", QuantKernel::ArgmaxPartial},
     {"llm_elementwise_bf16", "argmax_combine_f16", QuantKernel::ArgmaxCombine},
+    {"llm_elementwise_bf16", "sample_topp_f16", QuantKernel::SampleTopp},
     {"affine_qmv_bf16", "affine_gather_qmv_swiglu_w4g64", QuantKernel::GatherSwiglu},
     {"affine_qmv_bf16", "affine_gather_qmv_geglu_w4g64", QuantKernel::GatherGeglu},
     {"affine_qmv_bf16", "affine_gather_down_qmv_w4g64", QuantKernel::GatherDown},
@@ -568,6 +569,16 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
                    ? VPQ_ERR_NULL_POINTER
                    : vpq_argmax_combine(st, static_cast<const float*>(buf(0)), static_cast<int32_t*>(buf(1)), ival(2));
     }
+  } else if (kind == QuantKernel::SampleTopp) {
+    // gpu-kernels/metal/ops/llm_elementwise.metal:3116-3130: 0:logits 1:out_id 2:V 3:temp 4:top_p 5:seed 6:ws 7:n_iter
+    // 8:rep 9:pres 10:top_k 11:min_p 12:seen
+    bool have = buf(0) && buf(1) && buf(6) && buf(12);
+    for (unsigned i : {2u, 3u, 4u, 5u, 7u, 8u, 9u, 10u, 11u}) { have = have && has_int(i); }
+    auto fval = [&](unsigned i) { return _slots[i].fvalue; };
+    status = !have ? VPQ_ERR_NULL_POINTER
+                   : vpq_sample_topp_bf16(st, static_cast<const uint16_t*>(buf(0)), static_cast<int32_t*>(buf(1)), ival(2),
+                                          fval(3), fval(4), static_cast<uint32_t>(_slots[5].ivalue), static_cast<uint16_t*>(buf(6)),
+                                          ival(7), fval(8), fval(9), ival(10), fval(11), static_cast<uint8_t*>(buf(12)));
   } else if (kind == QuantKernel::QmvQkv) {
     // gpu-kernels/metal/quant/affine_qmv.metal:497-516: slots 0:w 1:scales 2:biases 3:x 4:q_out
     // 5:k_out 6:v_out 7:K 8:q_rows 9:k_rows 10:v_rows; the pack is the row-concatenated q|k|v.

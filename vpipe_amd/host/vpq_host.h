@@ -98,6 +98,8 @@ enum class QuantKernel : std::uint8_t {
   Argmax,         // argmax_f16: slots 0:logits 1:out_id 2:V (one workgroup)
   ArgmaxPartial,  // argmax_partial_f16: slots 0:logits 1:partials 2:V 3:M slabs
   ArgmaxCombine,  // argmax_combine_f16: slots 0:partials 1:out_id 2:M
+  SampleTopp,     // sample_topp_f16: slots 0:logits 1:out_id 2:V 3:temp 4:top_p 5:seed 6:ws 7:n_iter 8:rep 9:pres
+                  //   10:top_k 11:min_p 12:seen (one workgroup); float constants are 4-byte constants
 };
 
 // The packed format a function name ends in.
@@ -197,7 +199,7 @@ public:
 private:
   friend class CommandStream;
   explicit ComputeEncoder(CommandStream* s) noexcept : _stream(s) {}
-  static constexpr unsigned kSlots = 12;
+  static constexpr unsigned kSlots = 16;
   struct Slot {
     void* ptr = nullptr;
     std::size_t bytes = 0;       // bytes from ptr to the end of the bound buffer
