@@ -598,9 +598,11 @@ int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const
  * and half: apple-silicon/metal-compute/CMakeLists.txt:71-72, 159-162; the
  * metallibs without the `_bf16` suffix).  These entries are the f16 forms of
  * the 4-bit group-64 functions: scales, biases, x, y, residual and w_deq are
- * IEEE binary16 bit patterns, the packed codes are the same.  A first, general
- * path (one wavefront per output row for the QMV, expansion + the dense GEMM for
- * the QMM), not tuned like the bf16 kernels:
+ * IEEE binary16 bit patterns, the packed codes are the same.  One row of x on
+ * K % 512 == 0, K >= 2048 with 16-byte aligned scales and biases takes the
+ * streaming decode kernel of the bf16 entry on binary16 arithmetic (same
+ * speed); every other QMV shape takes a general path (one wavefront per
+ * output row); the QMM is expansion + the dense GEMM:
  *   vpq_dequant_w4g64_f16         `affine_dequant_w4g64` (affine_dequant.metal:25-58), bit-exact:
  *                                 f16_rne(fp32(s) * q + fp32(b)).
  *   vpq_qmv_w4g64_f16 / _f32out   `affine_qmv_w4g64[_add]` (affine_qmv.metal:286-301, 347-363),

@@ -78,6 +78,34 @@ def test_qmv_f16_residual_and_gated(vpq, oracle, dev, D):
         check_f16(got, g64)
 
 
+@pytest.mark.parametrize("K,N", [(2048, 38), (2560, 250), (5120, 1030), (17408, 66)])
+def test_qmv_f16_one_row_streaming_kernel(vpq, oracle, dev, D, K, N):
+    """One row of x on K % 512 == 0 takes the streaming decode kernel on binary16 arithmetic: plain, fp32 out,
+    residual and both gated forms, ragged N, guard bands intact."""
+    M = 1
+    w, s, b = f16_pack(N, K, 600 + K + N)
+    x = np.random.default_rng(601 + K).standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    res = np.random.default_rng(602 + K).standard_normal((M, N)).astype(np.float16).view(np.uint16)
+    y64, _ = oracle.matmul_f16(w, s, b, x, K, N, M, rounded=False)
+    wd, sd, bd, xd = D.u32(w, dev), dev16(s, dev), dev16(b, dev), dev16(x, dev)
+    parity.check_f32(vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, f32out=True).cpu().numpy(), y64)
+    out = parity.Guarded((M, N), torch.float16, dev)
+    vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    plain = bits16(out.view)
+    check_f16(plain, y64)
+    got_add = bits16(vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, residual=dev16(res, dev)))
+    redo = (plain.view(np.float16).astype(np.float32) + res.view(np.float16).astype(np.float32)).astype(np.float16)
+    assert np.array_equal(got_add, redo.view(np.uint16))
+    for activation, fn in ((1, oracle.swiglu), (2, oracle.geglu)):
+        g64, _ = fn(y64)
+        check_f16(bits16(vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, activation=activation)), g64)
+    # a pack whose scales sit off 16 bytes takes the general kernel: same values to the tolerance
+    so = torch.empty(sd.numel() + 1, dtype=torch.float16, device=dev)[1:].view(sd.shape).copy_(sd)
+    check_f16(bits16(vpq.qmv_w4g64_f16(wd, so, bd, xd, K, N, M)), y64)
+
+
 @pytest.mark.parametrize("M,N,K", [(64, 64, 64), (130, 320, 256), (257, 129, 512)])
 def test_qmm_f16_dense_route(vpq, oracle, dev, D, M, N, K):
     w, s, b = f16_pack(N, K, 500 + M)

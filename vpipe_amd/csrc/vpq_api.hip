@@ -559,6 +559,10 @@ static int qmv_f16_common(vpq_stream_t stream, const uint32_t* w, const uint16_t
   a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y; a.residual = residual;
   a.K = K; a.N = N; a.M = M; a.y_f32 = y_f32; a.cu_count = g_dev.cu_count;
   a.gate_act = gate_act;
+  // one row of x on a K the streaming kernel takes: the same kernel as for bf16, on binary16 arithmetic
+  if (vpq::qmv_flow_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16)) {
+    return finish(vpq::launch_qmv_flow_f16(reinterpret_cast<hipStream_t>(stream), a));
+  }
   return finish(vpq::launch_qmv_simple_f16(reinterpret_cast<hipStream_t>(stream), a));
 }
 

@@ -45,9 +45,17 @@ constexpr int kSlice = 2048;          // values of K per slice (64 lanes x 32)
 constexpr int kMaxWavesPerWg = 8;
 constexpr int kMaxLdsBytes = 96 * 1024;   // x of the K range + the scale/bias windows; K <= 32768 fits
 
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+
+// a.lo * b.lo + a.hi * b.hi + c on pairs of bf16 (F16 = false) or IEEE binary16 (true), fp32 accumulation
+template <bool F16 = false>
 __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c)
 {
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+  if constexpr (F16) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2, a), __builtin_bit_cast(halfx2, b), c, false);
+  } else {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+  }
 }
 
 template <int I, int N, typename F>
@@ -162,7 +170,10 @@ __device__ __forceinline__ void pin_scalar(const T& v) { asm volatile("" : : "s"
 // the two modes give the same bits.
 constexpr int kXOwn = 0, kXShared = 1;
 
-template <int SPW, int RB, bool F32OUT, int XM, int C>
+// F16: the elements (x, scales, biases, y, residual) are IEEE binary16 instead of bf16 (the reference's
+// VPIPE_ELT = half build).  The codes then become binary16 pairs 16 + q (the code shifted to mantissa bits 6..9,
+// exact; 1024 + q with the code left in bits 0..3 would cost eight times bf16's cancellation noise).
+template <int SPW, int RB, bool F32OUT, int XM, int C, bool F16 = false>
 __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const FlowParams<C> p)
 {
   constexpr int NL = RB * SPW;                 // code loads of a wavefront
@@ -210,11 +221,12 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
   float* red = reinterpret_cast<float*>(lds + x_bytes + W * (NDMA * 1024));
   const uint32_t lds_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds;
 
-  uint32_t magic = 0x43004300u;                // bf16 128.0 in both halves
-  uint32_t mask = 0x000f000fu;
+  uint32_t magic = F16 ? 0x4c004c00u : 0x43004300u;   // 16.0 (binary16) or 128.0 (bf16) in both halves
+  uint32_t mask = F16 ? 0x03c003c0u : 0x000f000fu;
   asm volatile("" : "+v"(magic));              // no instruction: hides the constants from folding, so
   asm volatile("" : "+s"(mask));               // that each pair costs one v_and_or_b32
-  const uint32_t ones = 0x3f803f80u;           // bf16 1.0 twice
+  const uint32_t ones = F16 ? 0x3c003c00u : 0x3f803f80u;   // 1.0 twice
+  constexpr float kOffset = F16 ? -16.0f : -128.0f;
 
   bool kvalid[SPW];
 #pragma unroll
@@ -305,10 +317,10 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
         xp[s][4 * t + 1] = __builtin_amdgcn_perm(d.z, d.x, 0x07060302u);   // x1,x5
         xp[s][4 * t + 2] = __builtin_amdgcn_perm(d.w, d.y, 0x05040100u);   // x2,x6
         xp[s][4 * t + 3] = __builtin_amdgcn_perm(d.w, d.y, 0x07060302u);   // x3,x7
-        sum = dot2(d.x, ones, sum);
-        sum = dot2(d.y, ones, sum);
-        sum = dot2(d.z, ones, sum);
-        sum = dot2(d.w, ones, sum);
+        sum = dot2<F16>(d.x, ones, sum);
+        sum = dot2<F16>(d.y, ones, sum);
+        sum = dot2<F16>(d.z, ones, sum);
+        sum = dot2<F16>(d.w, ones, sum);
       }
       sx[s] = sum;
     }
@@ -325,12 +337,20 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
         float d0 = 0.0f, d1 = 0.0f;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          d0 = dot2(xp[s][4 * t + 0], ((cw[t] >> 0) & mask) | magic, d0);
-          d1 = dot2(xp[s][4 * t + 1], ((cw[t] >> 4) & mask) | magic, d1);
-          d0 = dot2(xp[s][4 * t + 2], ((cw[t] >> 8) & mask) | magic, d0);
-          d1 = dot2(xp[s][4 * t + 3], ((cw[t] >> 12) & mask) | magic, d1);
+          if constexpr (F16) {
+            // the code goes to mantissa bits 6..9 of 16.0: 16 + q, exact (a step of 1/64 there)
+            d0 = dot2<true>(xp[s][4 * t + 0], ((cw[t] << 6) & mask) | magic, d0);
+            d1 = dot2<true>(xp[s][4 * t + 1], ((cw[t] << 2) & mask) | magic, d1);
+            d0 = dot2<true>(xp[s][4 * t + 2], ((cw[t] >> 2) & mask) | magic, d0);
+            d1 = dot2<true>(xp[s][4 * t + 3], ((cw[t] >> 6) & mask) | magic, d1);
+          } else {
+            d0 = dot2(xp[s][4 * t + 0], ((cw[t] >> 0) & mask) | magic, d0);
+            d1 = dot2(xp[s][4 * t + 1], ((cw[t] >> 4) & mask) | magic, d1);
+            d0 = dot2(xp[s][4 * t + 2], ((cw[t] >> 8) & mask) | magic, d0);
+            d1 = dot2(xp[s][4 * t + 3], ((cw[t] >> 12) & mask) | magic, d1);
+          }
         }
-        dots[r][s] = d0 + d1;                    // sum x * (128 + q)
+        dots[r][s] = d0 + d1;                    // sum x * (128 + q), binary16: sum x * (16 + q)
         chain = dots[r][s];
       });
     });
@@ -342,10 +362,10 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
 #pragma unroll
       for (int s = 0; s < SPW; ++s) {
         const int o = r * (PPR * 16) + s * 64 + (lane >> 1) * 2;
-        const float sc = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sbl + o));
-        const float bi = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sbl + P * 16 + o));
+        const float sc = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sbl + o));
+        const float bi = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sbl + P * 16 + o));
         acc[r] = fmaf(sc, dots[r][s], acc[r]);
-        acc[r] = fmaf(fmaf(-128.0f, sc, bi), sx[s], acc[r]);
+        acc[r] = fmaf(fmaf(kOffset, sc, bi), sx[s], acc[r]);
       }
     }
 #pragma unroll
@@ -382,7 +402,7 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
         if (F32OUT) {
           reinterpret_cast<float*>(yq)[o] = v;
         } else {
-          reinterpret_cast<uint16_t*>(yq)[o] = (uint16_t)f32_to_bf16_bits(v);
+          reinterpret_cast<uint16_t*>(yq)[o] = (uint16_t)f32_to_elt_bits<F16>(v);
         }
       }
     }
@@ -395,8 +415,8 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
       if (F32OUT) {
         reinterpret_cast<float*>(yq)[n] = tot[r];
       } else {
-        uint32_t v = f32_to_bf16_bits(tot[r]);
-        if (residual != nullptr) { v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(residual[n])); }
+        uint32_t v = f32_to_elt_bits<F16>(tot[r]);
+        if (residual != nullptr) { v = f32_to_elt_bits<F16>(elt_bits_to_f32<F16>(v) + elt_bits_to_f32<F16>(residual[n])); }
         reinterpret_cast<uint16_t*>(yq)[n] = (uint16_t)v;
       }
     }
@@ -429,10 +449,10 @@ FlowPlan flow_plan(int K, double pack_bytes)
   return pl;
 }
 
-template <int S, int R, bool F32, int XM, int C>
+template <int S, int R, bool F32, int XM, int C, bool F16 = false>
 hipError_t launch_flow_kernel(dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st, const FlowParams<C>& p)
 {
-  const auto kern = qmv_flow_kernel<S, R, F32, XM, C>;
+  const auto kern = qmv_flow_kernel<S, R, F32, XM, C, F16>;
   static std::once_flag once;          // one per instantiation
   static hipError_t attr_status = hipSuccess;
   std::call_once(once, [&] {
@@ -445,7 +465,7 @@ hipError_t launch_flow_kernel(dim3 grid, dim3 block, size_t lds_bytes, hipStream
 
 template <int C>
 hipError_t dispatch_flow(const FlowPlan& pl, bool y_f32, const FlowHead& h, const FlowSeg* segs, int rows_per_block,
-                         dim3 block, size_t lds_bytes, hipStream_t st)
+                         dim3 block, size_t lds_bytes, hipStream_t st, bool f16)
 {
   FlowParams<C> p;
   p.h = h;
@@ -456,6 +476,21 @@ hipError_t dispatch_flow(const FlowPlan& pl, bool y_f32, const FlowHead& h, cons
     blocks += (segs[i].N + rows_per_block - 1) / rows_per_block;
   }
   const dim3 grid((unsigned)blocks);
+  if (f16) {
+    // binary16 elements: single packs, x shared through LDS
+    if constexpr (C == 1) {
+      if (pl.xm != kXShared) { return hipErrorInvalidValue; }
+#define VPQ_FLOW16(S, R)                                                                                        \
+  if (pl.spw == S && pl.rb == R) {                                                                              \
+    return y_f32 ? launch_flow_kernel<S, R, true, kXShared, 1, true>(grid, block, lds_bytes, st, p)        \
+                 : launch_flow_kernel<S, R, false, kXShared, 1, true>(grid, block, lds_bytes, st, p);      \
+  }
+      VPQ_FLOW16(1, 2) VPQ_FLOW16(2, 2) VPQ_FLOW16(3, 2) VPQ_FLOW16(4, 2) VPQ_FLOW16(5, 2) VPQ_FLOW16(6, 2)
+      VPQ_FLOW16(1, 4) VPQ_FLOW16(2, 4) VPQ_FLOW16(3, 4) VPQ_FLOW16(4, 4)
+#undef VPQ_FLOW16
+    }
+    return hipErrorInvalidValue;
+  }
 #define VPQ_FLOW(S, R)                                                                                          \
   if (pl.spw == S && pl.rb == R) {                                                                              \
     if (pl.xm == kXShared) {                                                                                    \
@@ -473,7 +508,7 @@ hipError_t dispatch_flow(const FlowPlan& pl, bool y_f32, const FlowHead& h, cons
 
 // segs[0 .. count): the packs; count == 1 takes the one-line argument form.
 hipError_t launch_flow(hipStream_t st, const FlowSeg* segs, int count, const QmvArgs& a, double pack_bytes,
-                       const FlowPlan* forced)
+                       const FlowPlan* forced, bool f16 = false)
 {
   const FlowPlan pl = forced != nullptr ? *forced : flow_plan(a.K, pack_bytes);
   if (pl.spw == 0 || pl.wk < 1 || pl.wk > 4 || pl.wr < 1 || pl.wk * pl.wr > kMaxWavesPerWg ||
@@ -494,10 +529,10 @@ hipError_t launch_flow(hipStream_t st, const FlowSeg* segs, int count, const Qmv
   if (lds_bytes > (size_t)kMaxLdsBytes) { return hipErrorInvalidValue; }
   const dim3 block((unsigned)(64 * W));
   switch (count) {
-    case 1: return dispatch_flow<1>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st);
-    case 2: return dispatch_flow<2>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st);
-    case 3: return dispatch_flow<3>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st);
-    case 4: return dispatch_flow<4>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st);
+    case 1: return dispatch_flow<1>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st, f16);
+    case 2: return dispatch_flow<2>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st, f16);
+    case 3: return dispatch_flow<3>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st, f16);
+    case 4: return dispatch_flow<4>(pl, a.y_f32, h, segs, rows_per_block, block, lds_bytes, st, f16);
     default: return hipErrorInvalidValue;
   }
 }
@@ -513,6 +548,13 @@ hipError_t launch_qmv_flow(hipStream_t st, const QmvArgs& a)
 {
   const FlowSeg seg{a.w, a.scales, a.biases, a.y, a.N};
   return launch_flow(st, &seg, 1, a, (double)a.N * (double)a.K * 9.0 / 16.0, nullptr);
+}
+
+// The same kernel over IEEE binary16 elements (x, scales, biases, y, residual).
+hipError_t launch_qmv_flow_f16(hipStream_t st, const QmvArgs& a)
+{
+  const FlowSeg seg{a.w, a.scales, a.biases, a.y, a.N};
+  return launch_flow(st, &seg, 1, a, (double)a.N * (double)a.K * 9.0 / 16.0, nullptr, true);
 }
 
 // Measurement only: the single-pack launch with the plan given (slices per wavefront, K parts, row sets per
