@@ -630,6 +630,18 @@ def main():
             del packs
         out["qmv_f16_elements_m1"] = f16
 
+        # the fused GEMM on binary16 elements (the large-tile kernel with the f16 MFMA), clocks settled
+        K, N, M16 = 4096, 12288, 2048
+        w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev, generator=gen)
+        s = torch.empty((N, K // 64), dtype=torch.float32, device=dev).uniform_(0.005, 0.02, generator=gen).half()
+        b = (-8.0 * s.float()).half()
+        x = torch.randn((M16, K), device=dev, generator=gen).half()
+        y = torch.empty((M16, N), dtype=torch.float16, device=dev)
+        us = steady_us(lambda: vpipe_amd.qmm_w4g64_f16(w, s, b, x, K, N, M16, out=y), 10)
+        out["qmm_f16_elements_m2048_4096->12288"] = {"us": round(us, 2),
+                                                     "TFLOPs": round(2.0 * M16 * N * K / (us * 1e-6) / 1e12, 1)}
+        del w, s, b, x, y
+
         # group-32 twin (GGUF Q4_0 repacked), M=1: affine form (5/8 B per weight) and scale-only form
         # (bias never read: 9/16 B per weight)
         g32 = {}

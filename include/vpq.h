@@ -610,6 +610,15 @@ int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const
  *   vpq_qmv_gated_w4g64_f16       `affine_qmv_swiglu_w4g64`, `affine_qmv_geglu_w4g64` (:891-906, 1432-1447).
  *   vpq_qmm_dense_route_w4g64_f16 the dequant-once route (expansion into w_deq [N,K] f16 + the dense
  *                                 GEMM), arguments as vpq_qmm_dense_route_w4g64_bf16.
+ *   vpq_qmm_w4g64_f16             the fused GEMM `affine_qmm_steel_w4g64[_bm64|_bm128]` (affine_qmm_steel.metal:
+ *                                 470-560) and, with activation VPQ_GATE_SWIGLU / VPQ_GATE_GEGLU, the gated
+ *                                 `affine_qmm_swiglu_w4g64*`, `affine_qmm_geglu_w4g64` (y [M,N/2], N even) on
+ *                                 binary16 elements: weight tile = f16_rne(fp32(s*q+b)), f16 MFMA, fp32
+ *                                 accumulation, one rounding -- the large-tile kernel of the bf16 entry, so it
+ *                                 needs K % 512 == 0 and 16-byte aligned scales / biases (VPQ_ERR_BAD_SHAPE
+ *                                 otherwise: take the dequant-once route); x and y 16-byte aligned.  Its
+ *                                 results have the bits of the dequant-once route where that picks the same
+ *                                 tile width.
  * Requirements as for the bf16 entries. */
 int vpq_dequant_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, uint16_t* w_deq, int K, int N);
@@ -621,6 +630,9 @@ int vpq_qmv_w4g64_f16_f32out(vpq_stream_t stream, const uint32_t* w, const uint1
 int vpq_qmv_gated_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                             const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                             int activation);
+int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                      const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                      int K, int N, int M, int activation);
 int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                   const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                   int K, int N, int M, uint16_t* w_deq, int expand);

@@ -121,6 +121,44 @@ def test_qmm_f16_dense_route(vpq, oracle, dev, D, M, N, K):
     assert torch.equal(kept, got)
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 64, 512), (130, 328, 1024), (257, 136, 512), (300, 520, 1536)])
+def test_qmm_f16_fused(vpq, oracle, dev, D, M, N, K):
+    """The fused GEMM on binary16 elements (weight tile = f16(s q + b), f16 MFMA, fp32 accumulation): against
+    the oracle's rounded-weight twin, bit for bit against the dequant-once route (same tiles, same order of
+    accumulation), gated stores against the oracle's activations, guard bands intact."""
+    w, s, b = f16_pack(N, K, 700 + M)
+    x = np.random.default_rng(701 + M).standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    y64, _ = oracle.matmul_f16(w, s, b, x, K, N, M, rounded=True)
+    wd, sd, bd, xd = D.u32(w, dev), dev16(s, dev), dev16(b, dev), dev16(x, dev)
+    out = parity.Guarded((M, N), torch.float16, dev)
+    vpq.qmm_w4g64_f16(wd, sd, bd, xd, K, N, M, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    check_f16(bits16(out.view), y64)
+    w_deq = torch.empty((N, K), dtype=torch.float16, device=dev)
+    assert torch.equal(out.view, vpq.qmm_dense_route_w4g64_f16(wd, sd, bd, xd, K, N, M, w_deq))
+    # the element type is live: the bf16 kernel on the same bits gives something else
+    assert not torch.equal(out.view.view(torch.int16),
+                           vpq.qmm_w4g64(wd, sd.view(torch.bfloat16), bd.view(torch.bfloat16), xd.view(torch.bfloat16),
+                                         K, N, M).view(torch.int16))
+    for activation, fn in ((1, oracle.swiglu), (2, oracle.geglu)):
+        g64, _ = fn(y64)
+        og = parity.Guarded((M, N // 2), torch.float16, dev)
+        vpq.qmm_w4g64_f16(wd, sd, bd, xd, K, N, M, activation=activation, out=og.view)
+        torch.cuda.synchronize()
+        og.assert_intact()
+        check_f16(bits16(og.view), g64)
+
+
+def test_qmm_f16_fused_rejects(vpq, dev):
+    L = vpq.load()
+    p = torch.zeros(1 << 16, dtype=torch.int32, device=dev).data_ptr()
+    assert L.vpq_qmm_w4g64_f16(None, p, p, p, p, p, 448, 8, 4, 0) == -2         # K % 512 != 0: the dequant-once route
+    assert L.vpq_qmm_w4g64_f16(None, p, p, p, p, p, 512, 7, 4, 1) == -2         # gated needs an even N
+    assert L.vpq_qmm_w4g64_f16(None, p, p, p, p, p, 512, 8, 4, 3) == -2
+    assert L.vpq_qmm_w4g64_f16(None, p, p, p, None, p, 512, 8, 4, 0) == -1
+
+
 def test_f16_entries_reject_bad_arguments(vpq, dev):
     L = vpq.load()
     p = torch.zeros(4096, dtype=torch.int32, device=dev).data_ptr()

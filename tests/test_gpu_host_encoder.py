@@ -748,6 +748,18 @@ def test_binary16_library_names(vpq, enc, oracle, dev, D):
     assert np.array_equal(dense.view(torch.int16).cpu().numpy().view(np.uint16), oracle.dequant_f16(w, s, b, K, N))
     assert torch.equal(y, vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, 1))
     assert enc.set_function("affine_qmv", "affine_qmm_steel_w4g64") == 0       # not in that library
+    # the fused GEMM of the binary16 build, plain and gated, under its function names (slot 7 = M)
+    M = 70
+    xm = as16(np.random.default_rng(79).standard_normal((M, K)).astype(np.float16).view(np.uint16))
+    ym = torch.zeros((M, N), dtype=torch.float16, device=dev)
+    yg = torch.zeros((M, N // 2), dtype=torch.float16, device=dev)
+    encode_linear(enc, "affine_qmm_steel", "affine_qmm_steel_w4g64_bm64", wd, sd, bd, xm, ym, K, N, M=M, grid=(1, 2, 1))
+    encode_linear(enc, "affine_qmm_steel", "affine_qmm_swiglu_w4g64", wd, sd, bd, xm, yg, K, N, M=M, grid=(1, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert torch.equal(ym, vpq.qmm_w4g64_f16(wd, sd, bd, xm, K, N, M))
+    assert torch.equal(yg, vpq.qmm_w4g64_f16(wd, sd, bd, xm, K, N, M, activation=1))
+    assert ym.abs().sum() > 0 and yg.abs().sum() > 0
 
 
 def test_mixed_width_gather_function_names(vpq, enc, dev, D):

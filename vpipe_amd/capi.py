@@ -74,6 +74,7 @@ SYMBOLS = [
     ("vpq_qmv_w4g64_f16_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     ("vpq_qmv_gated_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_dense_route_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
+    ("vpq_qmm_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
@@ -590,6 +591,17 @@ def qmm_dense_route_w4g64_f16(w, scales, biases, x, K, N, M, w_deq, expand=True,
         out = torch.empty((M, N), dtype=torch.float16, device=w.device)
     _check(load().vpq_qmm_dense_route_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
                                                 _ptr(w_deq), 1 if expand else 0), "vpq_qmm_dense_route_w4g64_f16")
+    return out
+
+
+def qmm_w4g64_f16(w, scales, biases, x, K, N, M, activation=0, out=None):
+    """The fused GEMM on IEEE binary16 elements (the large-tile kernel: K % 512 == 0); activation 1 / 2 gives
+    the SwiGLU / GEGLU store of an interleaved gate|up pack, y [M, N/2]."""
+    import torch
+    if out is None:
+        out = torch.empty((M, N // 2 if activation else N), dtype=torch.float16, device=w.device)
+    _check(load().vpq_qmm_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                    activation), "vpq_qmm_w4g64_f16")
     return out
 
 

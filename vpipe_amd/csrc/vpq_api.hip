@@ -585,6 +585,29 @@ int vpq_qmv_gated_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16
   return qmv_f16_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, activation);
 }
 
+// The fused GEMM on binary16 elements: the large-tile kernel only (K % 512 == 0, 16-byte aligned scales and
+// biases); activation 0 = plain y [M,N], else the gated store of an interleaved gate|up pack, y [M,N/2].
+int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                      const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
+{
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (activation != 0 && activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (M <= 0 || (activation != 0 && (N & 1) != 0)) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::GemmArgs g{};
+  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
+  g.K = K; g.N = N; g.M = M;
+  g.cu_count = g_dev.cu_count;
+  g.gate_act = activation;
+  g.f16 = true;
+  if (!vpq::qmm_big_supports(g)) { return VPQ_ERR_BAD_SHAPE; }
+  return finish(vpq::launch_qmm_big(reinterpret_cast<hipStream_t>(stream), g, 0));
+}
+
 int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                                   uint16_t* w_deq, int expand)

@@ -88,7 +88,15 @@ __device__ __forceinline__ uint32_t f32_to_elt_bits(float f)
 template <bool F16>
 __device__ __forceinline__ uint32_t pack_elt2(float a, float b)
 {
-  return F16 ? (f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16)) : pack_bf16x2(a, b);
+  if constexpr (F16) {
+    // one v_cvt_pk_f16_f32 (round to nearest even)
+    typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    const floatx2 f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, halfx2));
+  } else {
+    return pack_bf16x2(a, b);
+  }
 }
 
 // Gated activation of one (gate, up) pair of fp32 sums, the store expressions of the fused

@@ -77,6 +77,7 @@ struct GemmArgs {
   int out_off = 0;
   int bits = 4;              // 8: one byte per value, w [N, K/4] (the tile kernel only)
   int group = 64;            // 32: scales / biases [N, K/32] (the tile kernel only, 4-bit)
+  bool f16 = false;          // elements are IEEE binary16 (the large-tile kernel only, no adapter)
 };
 
 hipError_t launch_dequant(hipStream_t st, const uint32_t* w, const uint16_t* scales,

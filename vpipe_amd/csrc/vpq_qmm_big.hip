@@ -124,12 +124,13 @@ __device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* base, uin
 // the x tile does -- the dense matrix-unit GEMM of the dequant-once route
 // (gpu-kernels/metal/gemm/dense_gemm_mma.metal:44-93, 139-140, 195): same tiles, same MFMA stream, no
 // dequantization pieces; any K % 32 == 0.
-constexpr int kPacked4 = 0, kDenseBf16 = 1, kDenseF16 = 2;
+constexpr int kPacked4 = 0, kDenseBf16 = 1, kDenseF16 = 2, kPacked4F16 = 3;
 
 template <int NT, bool LORA, int WSRC = kPacked4>
 __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
 {
-  constexpr bool DENSE = WSRC != kPacked4;
+  constexpr bool DENSE = WSRC == kDenseBf16 || WSRC == kDenseF16;
+  constexpr bool F16 = WSRC == kDenseF16 || WSRC == kPacked4F16;    // elements are IEEE binary16, not bf16
   constexpr int BN = 64 * NT;               // weight rows per workgroup
   constexpr int MQ = 4 * NT;                // MFMAs per quarter step (16 of K)
   // One array per stage and operand.
@@ -243,10 +244,10 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   // scale and bias of rows d_row and d_row + 1 for step u, the thread's codes of step u
   auto load_row_params = [&](int u, float (&sc)[2], float (&bi)[2], uint32_t (&cw)[WPT]) {
     const uint8_t* sb = sb_lds + ((u >> 3) & 1) * kScaleBytes + d_row * 16 + (u & 7) * 2;
-    sc[0] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb));
-    bi[0] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
-    sc[1] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 16));
-    bi[1] = bf16_bits_to_f32(*reinterpret_cast<const uint16_t*>(sb + 256 * 16 + 16));
+    sc[0] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb));
+    bi[0] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
+    sc[1] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 16));
+    bi[1] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 256 * 16 + 16));
     const uint8_t* cp = c_lds + (u & 1) * kCodeBytes + tid * (WPT * 4);
     if constexpr (WPT % 4 == 0) {
 #pragma unroll
@@ -290,7 +291,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   using No = std::false_type;
 
   auto mfma = [](const bf16x8& a, const bf16x8& b, const floatx16& c) {
-    if constexpr (WSRC == kDenseF16) {
+    if constexpr (F16) {
       typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
       return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
     } else {
@@ -356,8 +357,8 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     } else if constexpr (S == 4) {
       v[6] = fmaf(sc, ubyte_f32<3>(lo), bi); v[7] = fmaf(sc, ubyte_f32<3>(hi), bi);
     } else if constexpr (S == 5) {
-      o.x = pack_bf16x2(v[0], v[1]); o.y = pack_bf16x2(v[2], v[3]);
-      o.z = pack_bf16x2(v[4], v[5]); o.w = pack_bf16x2(v[6], v[7]);
+      o.x = pack_elt2<F16>(v[0], v[1]); o.y = pack_elt2<F16>(v[2], v[3]);
+      o.z = pack_elt2<F16>(v[4], v[5]); o.w = pack_elt2<F16>(v[6], v[7]);
     } else if constexpr (S == 6) {
       *reinterpret_cast<uint4*>(nb + b_dst[W]) = o;
     }
@@ -571,17 +572,16 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
           const float f0 = gated_f32(p.gate_act, acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
           const float f1 = gated_f32(p.gate_act, acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
           if (pair_ok && n + 3 < p.N) {
-            *reinterpret_cast<uint32_t*>(yrow + (n >> 1)) = pack_bf16x2(f0, f1);
+            *reinterpret_cast<uint32_t*>(yrow + (n >> 1)) = pack_elt2<F16>(f0, f1);
           } else {
-            yrow[n >> 1] = (uint16_t)f32_to_bf16_bits(f0);
-            if (n + 3 < p.N) { yrow[(n >> 1) + 1] = (uint16_t)f32_to_bf16_bits(f1); }
+            yrow[n >> 1] = (uint16_t)f32_to_elt_bits<F16>(f0);
+            if (n + 3 < p.N) { yrow[(n >> 1) + 1] = (uint16_t)f32_to_elt_bits<F16>(f1); }
           }
         }
       }
     }
     return;
   }
-  constexpr bool F16 = WSRC == kDenseF16;
   if ((p.N & 7) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0) {
     // Rows of y in whole 16-byte pieces: each wavefront turns its block round in an LDS region of its own, 32 x
     // rows at a time -- written as the accumulators lie (lane = x row, 4 consecutive n per register quad), read back
@@ -722,6 +722,13 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
   p.out_off = a.out_off;
   const dim3 grid(plan_tile_order(p)), block(kBigThreads);
   const bool lora = a.lora_t != nullptr;
+  if (a.f16) {
+    // IEEE binary16 elements: the plain and the gated GEMM (no adapter path)
+    if (lora) { return hipErrorInvalidValue; }
+    if (bn == 128) { return launch_kernel(qmm_big_kernel<2, false, kPacked4F16>, grid, block, 0, st, p); }
+    if (bn == 192) { return launch_kernel(qmm_big_kernel<3, false, kPacked4F16>, grid, block, 0, st, p); }
+    return launch_kernel(qmm_big_kernel<4, false, kPacked4F16>, grid, block, 0, st, p);
+  }
   if (bn == 128) {
     return lora ? launch_kernel(qmm_big_kernel<2, true>, grid, block, 0, st, p)
                 : launch_kernel(qmm_big_kernel<2, false>, grid, block, 0, st, p);

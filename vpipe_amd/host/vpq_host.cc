@@ -137,6 +137,11 @@ const FnEntry kFunctions[] = {
     {"affine_qmv", "affine_qmv_w4g64_add", QuantKernel::QmvAdd, QuantFormat::W4G64F16},
     {"affine_qmv", "affine_qmv_swiglu_w4g64", QuantKernel::QmvSwiglu, QuantFormat::W4G64F16},
     {"affine_qmv", "affine_qmv_geglu_w4g64", QuantKernel::QmvGeglu, QuantFormat::W4G64F16},
+    {"affine_qmm_steel", "affine_qmm_steel_w4g64", QuantKernel::Qmm, QuantFormat::W4G64F16},
+    {"affine_qmm_steel", "affine_qmm_steel_w4g64_bm64", QuantKernel::Qmm, QuantFormat::W4G64F16},
+    {"affine_qmm_steel", "affine_qmm_steel_w4g64_bm128", QuantKernel::Qmm, QuantFormat::W4G64F16},
+    {"affine_qmm_steel", "affine_qmm_swiglu_w4g64", QuantKernel::QmmSwiglu, QuantFormat::W4G64F16},
+    {"affine_qmm_steel", "affine_qmm_geglu_w4g64", QuantKernel::QmmGeglu, QuantFormat::W4G64F16},
     {"affine_dequant_bf16", "affine_dequant_w4g32", QuantKernel::Dequant, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_w4g32", QuantKernel::Qmv, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_w4g32_add", QuantKernel::QmvAdd, QuantFormat::W4G32},
@@ -447,6 +452,11 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
           status = vpq_qmm_gated_w8g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), act != 0 && has_int(8) ? ival(8) : 0,
                                             act != 0 && has_int(9) ? ival(9) : 0, act);
         }
+      } else if (fmt == QuantFormat::W4G64F16 && (kind == QuantKernel::Qmm || kind == QuantKernel::QmmSwiglu ||
+                                                  kind == QuantKernel::QmmGeglu)) {
+        // the fused GEMM of the binary16 build: slot 7 = M
+        const int act = kind == QuantKernel::Qmm ? 0 : (kind == QuantKernel::QmmGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
+        status = !has_int(7) ? VPQ_ERR_NULL_POINTER : vpq_qmm_w4g64_f16(st, w, sc, bi, x, y, K, N, ival(7), act);
       } else if (fmt == QuantFormat::W4G32 && (kind == QuantKernel::Qmm || kind == QuantKernel::QmmGeglu)) {
         // gpu-kernels/metal/quant/affine_qmm_steel.metal:618-640, 1573-1596: slot 7 = M
         status = !has_int(7) ? VPQ_ERR_NULL_POINTER
