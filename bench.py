@@ -605,15 +605,26 @@ def main():
         del gw8, gs8, gb8
         out["qmv_w8g64_gated_and_gathered"] = w8g
 
-        # fused 8-bit GEMM (the tile kernel with byte codes) at M = 2048, beside the 8-bit dequant-once route
+        # fused 8-bit GEMM at M = 2048 (the large-tile kernel with byte codes; the tile kernel beside it), clocks settled
         K, N, M8 = 4096, 12288, 2048
         w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 4), dtype=torch.int32, device=dev, generator=gen)
         s = torch.empty((N, K // 64), dtype=torch.float32, device=dev).uniform_(0.0003, 0.0012, generator=gen).bfloat16()
         b = (-128.0 * s.float()).bfloat16()
         x = torch.randn((M8, K), device=dev, generator=gen).bfloat16()
         y = torch.empty((M8, N), dtype=torch.bfloat16, device=dev)
-        us = kernel_us(lambda i: vpipe_amd.qmm_w8g64(w, s, b, x, K, N, M8, out=y), 5)
-        out["qmm_w8g64_m2048_4096->12288"] = {"us": round(us, 2), "TFLOPs": round(2.0 * M8 * N * K / (us * 1e-6) / 1e12, 1)}
+        us = steady_us(lambda: vpipe_amd.qmm_w8g64(w, s, b, x, K, N, M8, out=y), 10)
+        us_t = steady_us(lambda: vpipe_amd.qmm_w8g64(w, s, b, x, K, N, M8, out=y, tile_n=128), 10)
+        out["qmm_w8g64_m2048_4096->12288"] = {"us": round(us, 2), "TFLOPs": round(2.0 * M8 * N * K / (us * 1e-6) / 1e12, 1),
+                                              "tile_kernel_TFLOPs": round(2.0 * M8 * N * K / (us_t * 1e-6) / 1e12, 1)}
+        del w, s, b
+        # the group-32 pack on the same shape
+        w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev, generator=gen)
+        s = torch.empty((N, K // 32), dtype=torch.float32, device=dev).uniform_(0.005, 0.02, generator=gen).bfloat16()
+        b = (-8.0 * s.float()).bfloat16()
+        us = steady_us(lambda: vpipe_amd.qmm_w4g32(w, s, b, x, K, N, M8, out=y), 10)
+        us_t = steady_us(lambda: vpipe_amd.qmm_w4g32(w, s, b, x, K, N, M8, out=y, tile_n=128), 10)
+        out["qmm_w4g32_m2048_4096->12288"] = {"us": round(us, 2), "TFLOPs": round(2.0 * M8 * N * K / (us * 1e-6) / 1e12, 1),
+                                              "tile_kernel_TFLOPs": round(2.0 * M8 * N * K / (us_t * 1e-6) / 1e12, 1)}
         del w, s, b, x, y
 
         f16 = {}

@@ -453,10 +453,13 @@ int vpq_qmm_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, cons
  *                                    QMV arithmetic, 1 <= M <= 16.
  *   vpq_qmv_gated_w4g32_bf16         replaces `affine_qmv_geglu_w4g32[_q40]` (:1451-1490) and the
  *                                    SwiGLU twin over an interleaved gate|up pack; y [M, N/2].
- *   vpq_qmm_w4g32_bf16, vpq_qmm_gated_w4g32_bf16   the fused tile kernel with a scale and a bias per 32
+ *   vpq_qmm_w4g32_bf16, vpq_qmm_gated_w4g32_bf16   the fused kernels with a scale and a bias per 32
  *                                    values: replace `affine_qmm_steel_w4g32`
  *                                    (affine_qmm_steel.metal:618-640) and `affine_qmm_geglu_w4g32`
- *                                    (:1573-1596) plus the SwiGLU twin; K % 64 == 0, any M.
+ *                                    (:1573-1596) plus the SwiGLU twin; K % 64 == 0, any M.  Chosen by size as
+ *                                    for the group-64 pack: the large-tile kernel once its tiles fill the CUs
+ *                                    (K % 512 == 0, 16-byte aligned scales / biases), else the 256 x 128 tile
+ *                                    kernel; the two give the same bits.
  *   vpq_qmm_dense_route_w4g32_bf16   GEMM by expansion into w_deq[N,K] + the library's dense GEMM
  *                                    (expand as in vpq_qmm_dense_route_w4g64_bf16).
  * Requires K % 32 == 0; w, x 16-byte aligned. */
@@ -471,6 +474,10 @@ int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
                              const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int scale_only);
 int vpq_qmm_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                        const uint16_t* x, uint16_t* y, int K, int N, int M);
+/* As vpq_qmm_tiled_w8g64_bf16 for the group-32 pack (tile_n 128, -128, 192, 256). */
+int vpq_qmm_tiled_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                             int K, int N, int M, int activation, int tile_n);
 /* The size-based entrance over a group-32 pack: slabs of vpq_qmv_w4g32_bf16 up to 64 rows (at every M where
  * K % 64 != 0), vpq_qmm_w4g32_bf16 above. */
 int vpq_linear_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
@@ -536,7 +543,8 @@ int vpq_argmax_combine(vpq_stream_t stream, const float* partials, int32_t* out_
  *                                    gathers over a batched 8-bit pack [E, N, K/4], arguments and
  *                                    conventions of the 4-bit vpq_gather_* entries; a pair is
  *                                    bit-identical to the plain 8-bit call on that expert's slab.
- *   vpq_qmm_w8g64_bf16, vpq_qmm_gated_w8g64_bf16   the fused tile kernel with byte codes: replace
+ *   vpq_qmm_w8g64_bf16, vpq_qmm_gated_w8g64_bf16   the fused kernels with byte codes (the large-tile kernel
+ *                                    once its tiles fill the CUs, else the 256 x 128 tile kernel; same bits): replace
  *                                    `affine_qmm_steel_w8g64[_bm64|_bm128]` (affine_qmm_steel.metal:1601-1672)
  *                                    and `affine_qmm_swiglu_w8g64*` / `affine_qmm_geglu_w8g64` (:1700-1890);
  *                                    arguments as vpq_qmm_w4g64_bf16 (no adapter) / vpq_qmm_gated_w4g64_bf16.
@@ -557,6 +565,15 @@ int vpq_gather_qmv_gated_split_bf16(vpq_stream_t stream, const uint32_t* wg, con
                                     const int32_t* pair_eid, int npair, int top_k, int n_experts, int activation);
 int vpq_qmm_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                        const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M);
+/* Names the kernel of the fused 8-bit GEMM (measurement and tests), as vpq_qmm_tiled_w4g64_bf16 does for the
+ * 4-bit pack: tile_n 128 = the 256 x 128 tile kernel, 192 = the large-tile kernel (K % 512 == 0, 16-byte
+ * aligned scales / biases; byte codes take weight tiles of up to 192 rows), -128 = the large-tile kernel at
+ * width 128.  activation 0 = plain y [M,N], else the gated store y [M,N/2].  VPQ_ERR_BAD_SHAPE where the
+ * named kernel does not take the shape.  vpq_qmm_w8g64_bf16 / vpq_qmm_gated_w8g64_bf16 choose by size: the
+ * large-tile kernel once its tiles fill the CUs. */
+int vpq_qmm_tiled_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                             const uint16_t* biases, const uint16_t* x, uint16_t* y,
+                             int K, int N, int M, int activation, int tile_n);
 /* The size-based entrance over an 8-bit pack (qmm_auto_'s ladder, generative-models/qwen3/
  * metal-qwen-model.cc:3964-4033, which takes the width from the layer): slabs of vpq_qmv_w8g64_bf16 up to
  * 64 rows, vpq_qmm_w8g64_bf16 above. */

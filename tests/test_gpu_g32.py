@@ -136,6 +136,38 @@ def test_qmm_g32_fused_tile_kernel(vpq, oracle, dev, D, M, N, K):
     assert torch.equal(got32, got64)
 
 
+@pytest.mark.parametrize("tile_n", [256, 192, -128])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 512), (300, 200, 1024), (257, 136, 512), (520, 392, 1536)])
+def test_qmm_g32_large_tile_kernel(vpq, oracle, dev, D, M, N, K, tile_n):
+    """Groups of 32 through the large-tile kernel at its three tile widths: the GEMM on the oracle's bit-exact
+    expansion, the bits of the 256 x 128 tile kernel, the gated stores, and on a group-64 pack with doubled scales
+    the bits of the group-64 large-tile kernel."""
+    w, s, b = synth.make_weight_g32(N, K, 7100 + N)
+    x = synth.make_act(M, K, 7101 + M)
+    dense = oracle.dequant_g32_bf16(w, s, b, K, N)
+    y64 = synth.bf16_bits_to_f32(x).astype(np.float64) @ synth.bf16_bits_to_f32(dense).astype(np.float64).T
+    yb = synth.f32_to_bf16_bits(y64.astype(np.float32))
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_w4g32(wd, sd, bd, xd, K, N, M, out=out.view, tile_n=tile_n)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    assert torch.equal(out.view, vpq.qmm_w4g32(wd, sd, bd, xd, K, N, M, tile_n=128))
+    for activation, fn in ((capi.VPQ_GATE_SWIGLU, oracle.swiglu), (capi.VPQ_GATE_GEGLU, oracle.geglu)):
+        want64, wantb = fn(y64)
+        og = parity.Guarded((M, N // 2), torch.bfloat16, dev)
+        vpq.qmm_w4g32(wd, sd, bd, xd, K, N, M, out=og.view, activation=activation, tile_n=tile_n)
+        torch.cuda.synchronize()
+        og.assert_intact()
+        parity.check_bf16(D.bits(og.view), want64, wantb, mismatch_over_all=activation == capi.VPQ_GATE_SWIGLU)
+    w64, s64, b64 = synth.make_weight(N, K, 7102 + N)
+    s2, b2 = np.repeat(s64, 2, axis=1), np.repeat(b64, 2, axis=1)
+    got32 = vpq.qmm_w4g32(D.u32(w64, dev), D.bf16(s2, dev), D.bf16(b2, dev), xd, K, N, M, tile_n=tile_n)
+    got64 = vpq.qmm_w4g64(D.u32(w64, dev), D.bf16(s64, dev), D.bf16(b64, dev), xd, K, N, M, tile_n=tile_n)
+    assert torch.equal(got32, got64)
+
+
 @pytest.mark.parametrize("activation", [capi.VPQ_GATE_SWIGLU, capi.VPQ_GATE_GEGLU])
 def test_qmm_g32_gated_store(vpq, oracle, dev, D, activation):
     K, F, M = 512, 70, 130

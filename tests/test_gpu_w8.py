@@ -229,6 +229,39 @@ def test_qmm_w8_fused_tile_kernel(vpq, oracle, dev, D, M, N, K):
     parity.check_bf16(D.bits(out.view), y64, yb)
 
 
+@pytest.mark.parametrize("tile_n", [192, -128])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 512), (300, 200, 1024), (257, 136, 512), (520, 392, 1536)])
+def test_qmm_w8_large_tile_kernel(vpq, oracle, dev, D, M, N, K, tile_n):
+    """Byte codes through the large-tile kernel (tiles of 192 and 128 weight rows): the GEMM oracle, the bits of
+    the 256 x 128 tile kernel (same weights, same order of accumulation along K), both gated stores."""
+    w, s, b = synth.make_weight8(N, K, 3600 + M)
+    x = synth.make_act(M, K, 3601 + M)
+    y64, yb = oracle.matmul8(w, s, b, x, K, N, M, rounded=True)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_w8g64(wd, sd, bd, xd, K, N, M, out=out.view, tile_n=tile_n)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    assert torch.equal(out.view, vpq.qmm_w8g64(wd, sd, bd, xd, K, N, M, tile_n=128))
+    for activation, fn in ((1, oracle.swiglu), (2, oracle.geglu)):
+        want64, wantb = fn(y64)
+        og = parity.Guarded((M, N // 2), torch.bfloat16, dev)
+        vpq.qmm_w8g64(wd, sd, bd, xd, K, N, M, out=og.view, activation=activation, tile_n=tile_n)
+        torch.cuda.synchronize()
+        og.assert_intact()
+        parity.check_bf16(D.bits(og.view), want64, wantb, mismatch_over_all=activation == 1)
+        assert torch.equal(og.view, vpq.qmm_w8g64(wd, sd, bd, xd, K, N, M, activation=activation, tile_n=128))
+
+
+def test_qmm_w8_kernel_names_reject(vpq, dev):
+    L = vpq.load()
+    p = torch.zeros(1 << 16, dtype=torch.int32, device=dev).data_ptr()
+    assert L.vpq_qmm_tiled_w8g64_bf16(None, p, p, p, p, p, 512, 8, 4, 0, 256) == -2      # byte codes: up to 192 rows
+    assert L.vpq_qmm_tiled_w8g64_bf16(None, p, p, p, p, p, 448, 8, 4, 0, 192) == -2      # K % 512
+    assert L.vpq_qmm_tiled_w8g64_bf16(None, p, p, p, p, p, 512, 7, 4, 1, 192) == -2      # gated: even N
+
+
 @pytest.mark.parametrize("activation", [1, 2])
 def test_qmm_w8_gated_store(vpq, oracle, dev, D, activation):
     K, ffn, M = 512, 100, 270

@@ -75,6 +75,8 @@ SYMBOLS = [
     ("vpq_qmv_gated_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_dense_route_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_qmm_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_qmm_tiled_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
+    ("vpq_qmm_tiled_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmv_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
@@ -480,21 +482,31 @@ def linear_twin(kind, w, scales, biases, x, K, N, M, out=None):
     return out
 
 
-def qmm_w4g32(w, scales, biases, x, K, N, M, out=None, activation=0):
-    """Fused group-32 GEMM on the tile kernel; activation != 0: interleaved gate|up pack -> [M, N/2]."""
+def qmm_w4g32(w, scales, biases, x, K, N, M, out=None, activation=0, tile_n=0):
+    """Fused group-32 GEMM; activation != 0: interleaved gate|up pack -> [M, N/2].  tile_n: 0 = the library's
+    choice; 128 the 256x128 tile kernel; -128 / 192 / 256 the large-tile kernel at that width."""
     import torch
     if out is None:
         out = torch.empty((M, N // 2 if activation else N), dtype=torch.bfloat16, device=w.device)
+    if tile_n:
+        _check(load().vpq_qmm_tiled_w4g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                               activation, tile_n), "vpq_qmm_tiled_w4g32_bf16")
+        return out
     _check(load().vpq_qmm_gated_w4g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
                                            activation), "vpq_qmm_gated_w4g32_bf16")
     return out
 
 
-def qmm_w8g64(w, scales, biases, x, K, N, M, out=None, activation=0, out_stride=0, out_off=0):
-    """Fused 8-bit GEMM on the tile kernel; activation != 0: interleaved gate|up pack -> [M, N/2]."""
+def qmm_w8g64(w, scales, biases, x, K, N, M, out=None, activation=0, out_stride=0, out_off=0, tile_n=0):
+    """Fused 8-bit GEMM; activation != 0: interleaved gate|up pack -> [M, N/2].  tile_n: 0 = the library's choice;
+    128 the 256x128 tile kernel; -128 / 192 the large-tile kernel at that width."""
     import torch
     if out is None:
         out = torch.empty((M, N // 2 if activation else N), dtype=torch.bfloat16, device=w.device)
+    if tile_n:
+        _check(load().vpq_qmm_tiled_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                               activation, tile_n), "vpq_qmm_tiled_w8g64_bf16")
+        return out
     _check(load().vpq_qmm_gated_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
                                            out_stride, out_off, activation), "vpq_qmm_gated_w8g64_bf16")
     return out

@@ -969,7 +969,29 @@ int vpq_qmm_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, cons
   return grouped_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, nullptr, sdst, n_experts, rows_y, 0);
 }
 
-// ---- 8-bit twins on the fused tile kernel ----
+// ---- 8-bit twins on the fused kernels ----
+
+namespace {
+
+// The fused GEMM of a format twin (byte codes, groups of 32).  tile: 0 = by size, as for the 4-bit group-64 pack
+// (the large-tile kernel once its tiles fill the CUs), 128 = the 256 x 128 tile kernel, 192 / 256 = the large-tile
+// kernel at that width, -128 = the large-tile kernel at width 128.
+int twin_gemm_launch(vpq_stream_t stream, const vpq::GemmArgs& g, int tile)
+{
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (tile == 192 || tile == 256 || tile == -128) {
+    if (!vpq::qmm_big_supports(g) || (tile == 256 && g.bits == 8)) { return VPQ_ERR_BAD_SHAPE; }
+    return finish(vpq::launch_qmm_big(hs, g, tile < 0 ? -tile : tile));
+  }
+  if (tile == 0 && vpq::qmm_big_supports(g)) {
+    const int bn = vpq::qmm_big_tile_n(g.N, g.M, g_dev.cu_count, g.bits == 8 ? 192 : 256);
+    const long tiles = (long)((g.M + 255) / 256) * (long)((g.N + bn - 1) / bn);
+    if (tiles >= (long)(g_dev.cu_count > 0 ? g_dev.cu_count : 256)) { return finish(vpq::launch_qmm_big(hs, g, bn)); }
+  }
+  return finish(vpq::launch_qmm_tile(hs, g));
+}
+
+}  // namespace
 
 int vpq_qmm_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                              const uint16_t* x, uint16_t* y, int K, int N, int M, int out_stride, int out_off, int activation)
@@ -992,7 +1014,29 @@ int vpq_qmm_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
   g.cu_count = g_dev.cu_count;
   g.gate_act = activation; g.out_stride = out_stride; g.out_off = out_off;
   g.bits = 8;
-  return finish(vpq::launch_qmm_tile(reinterpret_cast<hipStream_t>(stream), g));
+  return twin_gemm_launch(stream, g, 0);
+}
+
+int vpq_qmm_tiled_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int tile_n)
+{
+  if (tile_n != 128 && tile_n != -128 && tile_n != 192) { return VPQ_ERR_BAD_SHAPE; }
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (activation != 0 && activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  if (M <= 0 || (activation != 0 && (N & 1) != 0)) { return VPQ_ERR_BAD_SHAPE; }
+  if ((long long)M * (long long)K * 2 >= 4000000000LL) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::GemmArgs g{};
+  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
+  g.K = K; g.N = N; g.M = M;
+  g.cu_count = g_dev.cu_count;
+  g.gate_act = activation;
+  g.bits = 8;
+  return twin_gemm_launch(stream, g, tile_n);
 }
 
 int vpq_qmm_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
@@ -1106,8 +1150,10 @@ int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
   return qmv_g32_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, activation, scale_only != 0);
 }
 
-int vpq_qmm_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
+namespace {
+
+int qmm_g32_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int tile_n)
 {
   int st = check_pack_g32(w, scales, biases, K, N, false);
   if (st != VPQ_OK) { return st; }
@@ -1124,7 +1170,22 @@ int vpq_qmm_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
   g.cu_count = g_dev.cu_count;
   g.gate_act = activation; g.out_stride = 0; g.out_off = 0;
   g.group = 32;
-  return finish(vpq::launch_qmm_tile(reinterpret_cast<hipStream_t>(stream), g));
+  return twin_gemm_launch(stream, g, tile_n);
+}
+
+}  // namespace
+
+int vpq_qmm_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
+{
+  return qmm_g32_common(stream, w, scales, biases, x, y, K, N, M, activation, 0);
+}
+
+int vpq_qmm_tiled_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                             const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int tile_n)
+{
+  if (tile_n != 128 && tile_n != -128 && tile_n != 192 && tile_n != 256) { return VPQ_ERR_BAD_SHAPE; }
+  return qmm_g32_common(stream, w, scales, biases, x, y, K, N, M, activation, tile_n);
 }
 
 int vpq_qmm_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,

@@ -90,10 +90,9 @@ __device__ __forceinline__ uint32_t pack_elt2(float a, float b)
 {
   if constexpr (F16) {
     // one v_cvt_pk_f16_f32 (round to nearest even)
-    typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
-    typedef float floatx2 __attribute__((ext_vector_type(2)));
-    const floatx2 f = {a, b};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, halfx2));
+    uint32_t r;
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
   } else {
     return pack_bf16x2(a, b);
   }

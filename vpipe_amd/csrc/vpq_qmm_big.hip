@@ -124,21 +124,29 @@ __device__ __forceinline__ void dma16(uint32_t lds_dst, const uint8_t* base, uin
 // the x tile does -- the dense matrix-unit GEMM of the dequant-once route
 // (gpu-kernels/metal/gemm/dense_gemm_mma.metal:44-93, 139-140, 195): same tiles, same MFMA stream, no
 // dequantization pieces; any K % 32 == 0.
-constexpr int kPacked4 = 0, kDenseBf16 = 1, kDenseF16 = 2, kPacked4F16 = 3;
+constexpr int kPacked4 = 0, kDenseBf16 = 1, kDenseF16 = 2, kPacked4F16 = 3, kPacked8 = 4, kPacked4G32 = 5;
 
 template <int NT, bool LORA, int WSRC = kPacked4>
 __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
 {
   constexpr bool DENSE = WSRC == kDenseBf16 || WSRC == kDenseF16;
   constexpr bool F16 = WSRC == kDenseF16 || WSRC == kPacked4F16;    // elements are IEEE binary16, not bf16
+  constexpr bool W8 = WSRC == kPacked8;     // one byte per code: 64 bytes per row and step, w [N, K/4] words
+  constexpr bool G32 = WSRC == kPacked4G32; // groups of 32: two scales and biases per row and step
+  static_assert(!(W8 && NT == 4), "byte codes: the doubled code ring fits LDS up to 192-row weight tiles");
+  constexpr int CRB = W8 ? 64 : 32;         // bytes of codes per row and step
+  constexpr int NC = W8 ? 4 : 2;            // code loads per wavefront and step (1 KB each)
+  constexpr int kCodeSlot = W8 ? 64 * NT * 64 : kCodeBytes;
+  constexpr int kWStage = W8 ? 64 * NT * kRow : kWBytes;
+  constexpr int SBLK = G32 ? 4 : 8;         // steps per 16-byte block of a row's scales
   constexpr int BN = 64 * NT;               // weight rows per workgroup
   constexpr int MQ = 4 * NT;                // MFMAs per quarter step (16 of K)
   // One array per stage and operand.
   __shared__ __attribute__((aligned(16))) uint8_t x_lds0[kXBytes];
   __shared__ __attribute__((aligned(16))) uint8_t x_lds1[kXBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t w_lds0[kWBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t w_lds1[kWBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t c_lds[2 * kCodeBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t w_lds0[kWStage];
+  __shared__ __attribute__((aligned(16))) uint8_t w_lds1[kWStage];
+  __shared__ __attribute__((aligned(16))) uint8_t c_lds[2 * kCodeSlot];
   __shared__ __attribute__((aligned(16))) uint8_t sb_lds[2 * kScaleBytes];
 
   const int tid = threadIdx.x;
@@ -187,12 +195,14 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   };
   // ---- codes, scales, biases: wavefront w brings in those of rows 64w .. 64w+63 (nothing past BN rows) ----
   const bool dq_wave = wave * 64 < BN;      // wave-uniform
-  uint32_t c_off[2];
+  uint32_t c_off[NC];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int row = wave * 64 + i * 32 + (lane >> 1);
+  for (int i = 0; i < NC; ++i) {
+    // a load covers 1 KB: 32 rows of 32 bytes (two lanes a row), or 16 rows of 64 bytes (four lanes a row)
+    const int row = W8 ? wave * 64 + i * 16 + (lane >> 2) : wave * 64 + i * 32 + (lane >> 1);
     const int rg = (n0 + row < p.N) ? (n0 + row) : (p.N - 1);
-    c_off[i] = (uint32_t)rg * (uint32_t)(p.K >> 1) + (uint32_t)(lane & 1) * 16u;
+    c_off[i] = W8 ? (uint32_t)rg * (uint32_t)p.K + (uint32_t)(lane & 3) * 16u
+                  : (uint32_t)rg * (uint32_t)(p.K >> 1) + (uint32_t)(lane & 1) * 16u;
   }
   const uint8_t* wblk = reinterpret_cast<const uint8_t*>(p.w);
   // dense W tile: as the x tile; its BN rows are dealt out evenly, wavefront w brings in rows 16 NT w .. + 16 NT
@@ -215,15 +225,16 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   };
   auto issue_codes = [&](int u) {
     if (!dq_wave) { return; }
-    const uint8_t* src = wblk + (size_t)u * 32;
-    const uint32_t dst = lds_addr(c_lds) + (u & 1) * kCodeBytes + wave * (64 * 32);
+    const uint8_t* src = wblk + (size_t)u * CRB;
+    const uint32_t dst = lds_addr(c_lds) + (u & 1) * kCodeSlot + wave * (64 * CRB);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) { dma16(dst + i * (32 * 32), src, c_off[i]); }
+    for (int i = 0; i < NC; ++i) { dma16(dst + i * 1024, src, c_off[i]); }
   };
   const int qrow = tid;                     // the tile row this thread dequantizes
   const int qrg = (n0 + qrow < p.N) ? (n0 + qrow) : (p.N - 1);
-  const uint8_t* srow = reinterpret_cast<const uint8_t*>(p.scales) + (size_t)qrg * (p.K >> 5);   // K/64 entries of 2 bytes
-  const uint8_t* brow = reinterpret_cast<const uint8_t*>(p.biases) + (size_t)qrg * (p.K >> 5);
+  const int sb_row_bytes = G32 ? (p.K >> 4) : (p.K >> 5);     // K/32 or K/64 entries of 2 bytes
+  const uint8_t* srow = reinterpret_cast<const uint8_t*>(p.scales) + (size_t)qrg * sb_row_bytes;
+  const uint8_t* brow = reinterpret_cast<const uint8_t*>(p.biases) + (size_t)qrg * sb_row_bytes;
   auto issue_scales = [&](int blk) {
     if (!dq_wave) { return; }
     const uint32_t dst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave * (64 * 16);
@@ -233,7 +244,9 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   // ---- dequantization: the BN x 8 words of a step's codes are dealt out evenly, thread t takes the WPT
   // consecutive words from t*WPT on (row-major: word j of row r is 8r + j).  BN = 256: its own row;
   // BN = 192: six words that may straddle two rows.  d_row is the first row, d_w0 the first word in it.
+  // (Byte codes: a 16-byte piece of the tile, 8 values, is two words; "word" below then means such a pair.)
   constexpr int WPT = 2 * NT;
+  constexpr int NCW = W8 ? 2 * WPT : WPT;   // 32-bit words of codes per thread and step
   const int d_row = (tid * WPT) >> 3, d_w0 = (tid * WPT) & 7;
   int b_dst[WPT];
 #pragma unroll
@@ -242,22 +255,39 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     b_dst[j] = row * kRow + swz(row, word) * 16;
   }
   // scale and bias of rows d_row and d_row + 1 for step u, the thread's codes of step u
-  auto load_row_params = [&](int u, float (&sc)[2], float (&bi)[2], uint32_t (&cw)[WPT]) {
-    const uint8_t* sb = sb_lds + ((u >> 3) & 1) * kScaleBytes + d_row * 16 + (u & 7) * 2;
-    sc[0] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb));
-    bi[0] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
-    sc[1] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 16));
-    bi[1] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 256 * 16 + 16));
-    const uint8_t* cp = c_lds + (u & 1) * kCodeBytes + tid * (WPT * 4);
-    if constexpr (WPT % 4 == 0) {
+  // sc / bi [0], [1]: of the thread's pieces before and from piece `sw_at` on.  Group 64: rows d_row and
+  // d_row + 1.  Groups of 32: a thread's pieces lie in at most two (row, half of the step) groups, and the change
+  // is where the position in the row passes a multiple of 4: [0] = (d_row, the half d_w0 lies in), [1] = the
+  // upper half of d_row if d_w0 lies in the lower one, else the lower half of d_row + 1.
+  const bool starts_upper = d_w0 >= 4;
+  const int sw_at = G32 ? 4 - (d_w0 & 3) : 8 - d_w0;
+  auto load_row_params = [&](int u, float (&sc)[2], float (&bi)[2], uint32_t (&cw)[NCW]) {
+    if constexpr (G32) {
+      const uint8_t* sb = sb_lds + ((u >> 2) & 1) * kScaleBytes + d_row * 16 + (u & 3) * 4;
+      const uint32_t s0 = *reinterpret_cast<const uint32_t*>(sb), s1 = *reinterpret_cast<const uint32_t*>(sb + 16);
+      const uint32_t b0 = *reinterpret_cast<const uint32_t*>(sb + 256 * 16), b1 = *reinterpret_cast<const uint32_t*>(sb + 256 * 16 + 16);
+      const float s0l = bf16_lo_to_f32(s0), s0h = bf16_hi_to_f32(s0), b0l = bf16_lo_to_f32(b0), b0h = bf16_hi_to_f32(b0);
+      sc[0] = starts_upper ? s0h : s0l;
+      bi[0] = starts_upper ? b0h : b0l;
+      sc[1] = starts_upper ? bf16_lo_to_f32(s1) : s0h;
+      bi[1] = starts_upper ? bf16_lo_to_f32(b1) : b0h;
+    } else {
+      const uint8_t* sb = sb_lds + ((u >> 3) & 1) * kScaleBytes + d_row * 16 + (u & 7) * 2;
+      sc[0] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb));
+      bi[0] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
+      sc[1] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 16));
+      bi[1] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 256 * 16 + 16));
+    }
+    const uint8_t* cp = c_lds + (u & 1) * kCodeSlot + tid * (NCW * 4);
+    if constexpr (NCW % 4 == 0) {
 #pragma unroll
-      for (int j = 0; j < WPT; j += 4) {
+      for (int j = 0; j < NCW; j += 4) {
         const uint4 c4 = *reinterpret_cast<const uint4*>(cp + j * 4);
         cw[j] = c4.x; cw[j + 1] = c4.y; cw[j + 2] = c4.z; cw[j + 3] = c4.w;
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < WPT; j += 2) {
+      for (int j = 0; j < NCW; j += 2) {
         const uint2 c2 = *reinterpret_cast<const uint2*>(cp + j * 4);
         cw[j] = c2.x;
         cw[j + 1] = c2.y;
@@ -310,14 +340,14 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   //                  P/8 of the thread's codes at stage P%8 of
   //                    0: split the nibbles   1..4: two values each, fma(s, q, b)   5: pack to bf16   6: store   7: -
   // The state of both (fragments, codes, the word in work) lives across steps.
-  constexpr int NLOADS = DENSE ? 8 + 2 * NT : 12;
+  constexpr int NLOADS = DENSE ? 8 + 2 * NT : 10 + NC;
   constexpr int SP = NT == 2 ? 1 : 2;
   constexpr int NPRE = MQ / SP < NLOADS ? MQ / SP : NLOADS;   // requests made under quarter 3 (slots SP-1, 2SP-1, ...)
   bf16x8 wf[2][NT], xf[2][4];                          // operand fragments of the current / the next quarter
-  float sc2[2] = {0.0f, 0.0f}, bi2[2] = {0.0f, 0.0f};  // scale and bias of the thread's one or two rows
-  uint32_t cw[WPT];                                    // its codes of the step being dequantized
+  float sc2[2] = {0.0f, 0.0f}, bi2[2] = {0.0f, 0.0f};  // scale and bias of the thread's one or two groups
+  uint32_t cw[NCW];                                    // its codes of the step being dequantized
 #pragma unroll
-  for (int j = 0; j < WPT; ++j) { cw[j] = 0; }
+  for (int j = 0; j < NCW; ++j) { cw[j] = 0; }
   float sc = 0.0f, bi = 0.0f;                          // of the word in work
   uint32_t lo = 0, hi = 0;
   float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -336,18 +366,28 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     constexpr int P = decltype(pc)::value;
     constexpr int W = P >> 3, S = P & 7;
     if constexpr (S == 0) {
-      lo = cw[W] & 0x0f0f0f0fu;                        // q0 q2 q4 q6
-      hi = (cw[W] >> 4) & 0x0f0f0f0fu;                 // q1 q3 q5 q7
-      // No instruction: keeps the masked words as they are, so that each value is one v_cvt_f32_ubyteN
-      // of them (otherwise the mask is folded into a bit-field extract per value, one instruction more).
-      asm volatile("" : "+v"(lo), "+v"(hi));
-      if constexpr (NT == 4) {                         // the thread's own row
-        sc = sc2[0]; bi = bi2[0];
+      if constexpr (W8) {
+        lo = cw[2 * W];                                // q0 q1 q2 q3
+        hi = cw[2 * W + 1];                            // q4 q5 q6 q7
       } else {
-        const bool second = d_w0 + W >= 8;
+        lo = cw[W] & 0x0f0f0f0fu;                      // q0 q2 q4 q6
+        hi = (cw[W] >> 4) & 0x0f0f0f0fu;               // q1 q3 q5 q7
+        // No instruction: keeps the masked words as they are, so that each value is one v_cvt_f32_ubyteN
+        // of them (otherwise the mask is folded into a bit-field extract per value, one instruction more).
+        asm volatile("" : "+v"(lo), "+v"(hi));
+      }
+      if constexpr (NT == 4) {                         // the thread's own row; groups of 32: pieces 4-7 second group
+        sc = sc2[G32 ? (W >> 2) : 0]; bi = bi2[G32 ? (W >> 2) : 0];
+      } else {
+        const bool second = W >= sw_at;
         sc = second ? sc2[1] : sc2[0];
         bi = second ? bi2[1] : bi2[0];
       }
+    } else if constexpr (W8 && S >= 1 && S <= 4) {
+      if constexpr (S == 1) { v[0] = fmaf(sc, ubyte_f32<0>(lo), bi); v[4] = fmaf(sc, ubyte_f32<0>(hi), bi); }
+      if constexpr (S == 2) { v[1] = fmaf(sc, ubyte_f32<1>(lo), bi); v[5] = fmaf(sc, ubyte_f32<1>(hi), bi); }
+      if constexpr (S == 3) { v[2] = fmaf(sc, ubyte_f32<2>(lo), bi); v[6] = fmaf(sc, ubyte_f32<2>(hi), bi); }
+      if constexpr (S == 4) { v[3] = fmaf(sc, ubyte_f32<3>(lo), bi); v[7] = fmaf(sc, ubyte_f32<3>(hi), bi); }
     } else if constexpr (S == 1) {
       v[0] = fmaf(sc, ubyte_f32<0>(lo), bi); v[1] = fmaf(sc, ubyte_f32<0>(hi), bi);
     } else if constexpr (S == 2) {
@@ -380,16 +420,16 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     } else {
       if constexpr (I < 8) {
         dma16(xdst + I * (8 * kRow), xsrc, a_off[I]);
-      } else if constexpr (I < 10) {                    // codes(win+3) into the slot codes(win+1) have left
+      } else if constexpr (I < 8 + NC) {                // codes(win+3) into the slot codes(win+1) have left
         if (win + 3 < KT && dq_wave) {
-          dma16(lds_addr(c_lds) + (1 - STG) * kCodeBytes + wave * (64 * 32) + (I - 8) * (32 * 32),
-                wblk + (size_t)(win + 3) * 32, c_off[I - 8]);
+          dma16(lds_addr(c_lds) + (1 - STG) * kCodeSlot + wave * (64 * CRB) + (I - 8) * 1024,
+                wblk + (size_t)(win + 3) * CRB, c_off[I - 8]);
         }
       } else {
-        const int blk = (win >> 3) + 1;
-        if ((win & 7) == 0 && win + 8 < KT && dq_wave) {
+        const int blk = (win >> (G32 ? 2 : 3)) + 1;
+        if ((win & (SBLK - 1)) == 0 && win + SBLK < KT && dq_wave) {
           const uint32_t sdst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave * (64 * 16);
-          if constexpr (I == 10) { dma16(sdst, srow + (size_t)blk * 16); }
+          if constexpr (I == 8 + NC) { dma16(sdst, srow + (size_t)blk * 16); }
           else { dma16(sdst + 256 * 16, brow + (size_t)blk * 16); }
         }
       }
@@ -660,8 +700,12 @@ bool qmm_big_supports(const GemmArgs& a)
   if (a.K % 512 != 0 || a.M < 1 || a.N < 1) { return false; }
   if (a.gate_act != 0 && (a.lora_t != nullptr || (a.N & 1) != 0)) { return false; }
   if ((reinterpret_cast<uintptr_t>(a.scales) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.biases) & 15) != 0) { return false; }
-  if ((double)a.N * (double)a.K / 2.0 >= 4.0e9 || (double)BM * (double)a.K * 2.0 >= 4.0e9) { return false; }
+  if ((double)a.N * (double)a.K / (a.bits == 8 ? 1.0 : 2.0) >= 4.0e9 || (double)BM * (double)a.K * 2.0 >= 4.0e9) { return false; }
   if (a.lora_t != nullptr && (a.r < 32 || a.r % 32 != 0)) { return false; }
+  // the other formats and the binary16 elements come without the adapter path, and not combined
+  const int modes = (a.bits == 8) + (a.group == 32) + (a.f16 ? 1 : 0);
+  if (modes > 1 || (modes == 1 && a.lora_t != nullptr)) { return false; }
+  if ((a.bits != 4 && a.bits != 8) || (a.group != 64 && a.group != 32)) { return false; }
   return true;
 }
 
@@ -670,19 +714,20 @@ bool qmm_big_supports(const GemmArgs& a)
 // (measured with whole rounds: 256 wide 1.02, 192 wide 0.98, 128 wide 0.94 PFLOP/s).  4096 -> 12288 at
 // M = 2048: 384 tiles of 256 are one and a half rounds of 256 CUs, 512 tiles of 192 are two;
 // N = 4096 at M = 2048 is exactly one round of 128-wide tiles.
-int qmm_big_tile_n(int N, int M, int cu_count)
+int qmm_big_tile_n(int N, int M, int cu_count, int max_width)
 {
   const int cus = cu_count > 0 ? cu_count : 256;
   const long tm = (M + BM - 1) / BM;
   const int widths[3] = {256, 192, 128};
   const double eff[3] = {1.0, 0.95, 0.90};
-  int best = 256;
+  const int first = max_width >= 256 ? 0 : 1;          // byte codes: tiles up to 192 rows of weights
+  int best = widths[first];
   double best_cost = 0.0;
-  for (int i = 0; i < 3; ++i) {
+  for (int i = first; i < 3; ++i) {
     const long tiles = tm * ((N + widths[i] - 1) / widths[i]);
     const long rounds = (tiles + cus - 1) / cus;
     const double cost = (double)rounds * (double)widths[i] / eff[i];
-    if (i == 0 || cost < best_cost) { best = widths[i]; best_cost = cost; }
+    if (i == first || cost < best_cost) { best = widths[i]; best_cost = cost; }
   }
   return best;
 }
@@ -710,7 +755,9 @@ unsigned plan_tile_order(BigParams& p)
 
 hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
 {
-  const int bn = tile_n == 128 || tile_n == 192 || tile_n == 256 ? tile_n : qmm_big_tile_n(a.N, a.M, a.cu_count);
+  const int widest = a.bits == 8 ? 192 : 256;
+  const int bn = tile_n == 128 || tile_n == 192 || (tile_n == 256 && widest == 256) ? tile_n
+                                                                                  : qmm_big_tile_n(a.N, a.M, a.cu_count, widest);
   BigParams p;
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
   p.lora_t = a.lora_t; p.lora_b = a.lora_b;
@@ -722,6 +769,17 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
   p.out_off = a.out_off;
   const dim3 grid(plan_tile_order(p)), block(kBigThreads);
   const bool lora = a.lora_t != nullptr;
+  if (a.bits == 8) {
+    if (lora || a.f16 || a.group != 64) { return hipErrorInvalidValue; }
+    if (bn == 128) { return launch_kernel(qmm_big_kernel<2, false, kPacked8>, grid, block, 0, st, p); }
+    return launch_kernel(qmm_big_kernel<3, false, kPacked8>, grid, block, 0, st, p);
+  }
+  if (a.group == 32) {
+    if (lora || a.f16) { return hipErrorInvalidValue; }
+    if (bn == 128) { return launch_kernel(qmm_big_kernel<2, false, kPacked4G32>, grid, block, 0, st, p); }
+    if (bn == 192) { return launch_kernel(qmm_big_kernel<3, false, kPacked4G32>, grid, block, 0, st, p); }
+    return launch_kernel(qmm_big_kernel<4, false, kPacked4G32>, grid, block, 0, st, p);
+  }
   if (a.f16) {
     // IEEE binary16 elements: the plain and the gated GEMM (no adapter path)
     if (lora) { return hipErrorInvalidValue; }
