@@ -386,6 +386,15 @@ int vpq_qmv_grouped_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, con
 int vpq_qmv_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
                                     const int32_t* tile2e, const int32_t* srow, int n_experts);
+/* The same over a batched 8-bit pack [E, N, K/4]: `affine_grouped_swiglu_w8g64`, `affine_grouped_down_w8g64`
+ * (affine_qmv.metal:2718-2719).  A live slot is bit-identical to the pair-gathered 8-bit call
+ * (vpq_gather_qmv_gated_w8g64_bf16 / vpq_gather_down_qmv_w8g64_bf16) of that expert on that row. */
+int vpq_qmv_grouped_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
+                                     const int32_t* tile2e, const int32_t* srow, int n_experts, int activation);
+int vpq_qmv_grouped_down_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
+                                    const int32_t* tile2e, const int32_t* srow, int n_experts);
 
 /* ---- MoE prefill: expert-sorted (grouped) GEMMs ---------------------------
  * With many tokens the pairs are sorted by expert into blocks of

@@ -517,6 +517,47 @@ def test_moe_sorted_gemv_call_sites(vpq, enc, oracle, dev, D):
     assert not D.bits(part)[srow < 0].any()
 
 
+def test_moe_sorted_gemv_w8_call_sites(vpq, enc, dev, D):
+    # the 8-bit twins under their function names (affine_qmv.metal:2718-2719): same slots as the 4-bit functions
+    H, I, E, top_k, T = 256, 64, 5, 2, 5
+    gu = [synth.make_weight8(2 * I, H, 2800 + e) for e in range(E)]
+    dn = [synth.make_weight8(H, I, 2850 + e) for e in range(E)]
+    gu_d = tuple(f(np.stack([p[i] for p in gu]), dev) for i, f in enumerate((D.u32, D.bf16, D.bf16)))
+    dn_d = tuple(f(np.stack([p[i] for p in dn]), dev) for i, f in enumerate((D.u32, D.bf16, D.bf16)))
+    xd = D.bf16(synth.make_act(T, H, 2890), dev)
+    eid = np.random.default_rng(2891).integers(0, E, size=T * top_k, dtype=np.int32)
+    B = capi.VPQ_QMV_GROUPED_SLOTS
+    t2e_d, srow_d, _, _ = vpq.moe_sort_pairs(torch.from_numpy(eid).to(dev), top_k, E, block_rows=B)
+    npad = srow_d.numel()
+    gact = torch.zeros((npad, I), dtype=torch.bfloat16, device=dev)
+    part = torch.zeros((npad, H), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+    assert enc.set_function("affine_qmv_bf16", "affine_grouped_swiglu_w8g64") == 1
+    for i, t in enumerate(gu_d + (xd, gact)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, H)
+    enc.set_constant(6, 2 * I)
+    enc.set_buffer(7, srow_d)
+    enc.set_buffer(8, t2e_d)
+    enc.dispatch((32, 2 * ((2 * I + 7) // 8), npad // B), (32, 2, 1))
+    assert enc.set_function("affine_qmv_bf16", "affine_grouped_down_w8g64") == 1
+    for i, t in enumerate(dn_d + (gact, part)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, I)
+    enc.set_constant(6, H)
+    enc.set_buffer(7, srow_d)
+    enc.set_buffer(8, t2e_d)
+    enc.dispatch((32, 2 * ((H + 7) // 8), npad // B), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    want_act = torch.zeros_like(gact)
+    vpq.qmv_grouped_gated_w8g64(*gu_d, xd, H, 2 * I, t2e_d, srow_d, E, out=want_act)
+    want_part = torch.zeros_like(part)
+    vpq.qmv_grouped_down_w8g64(*dn_d, want_act, I, H, t2e_d, srow_d, E, out=want_part)
+    assert torch.equal(gact, want_act) and torch.equal(part, want_part)
+    assert gact.abs().sum() > 0 and part.abs().sum() > 0
+
+
 def test_moe_gathered_expert_call_sites(enc, oracle, dev, D):
     # Qwen MoE block, pair-batched (generative-models/qwen3/metal-qwen-model.cc:4190-4206):
     # gathered gate|up + SwiGLU -> act[np, I] (slots 0..4, 5:H 6:2*I 7:eid 8:top_k, grid {32, I/2, np}),

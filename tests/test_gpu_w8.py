@@ -274,6 +274,65 @@ def test_qmm_w8_gated_store(vpq, oracle, dev, D, activation):
     parity.check_bf16(D.bits(got), want64, wantb, mismatch_over_all=activation == 1)
 
 
+@pytest.mark.parametrize("activation", [1, 2])
+@pytest.mark.parametrize("K,inner,H,E,T,top_k", [(512, 96, 200, 5, 9, 2), (1024, 40, 130, 16, 5, 3), (192, 64, 64, 3, 20, 1)])
+def test_sorted_expert_gemv_w8_two_slots_per_tile(vpq, oracle, dev, D, K, inner, H, E, T, top_k, activation):
+    """gpu-kernels/metal/quant/affine_qmv.metal:2718-2719 (`affine_grouped_swiglu_w8g64`, `affine_grouped_down_w8g64`,
+    MAXM = 2) over 8-bit experts: QMV arithmetic against the oracle on every live slot, padding slots and unused
+    tiles untouched, a live slot bit for bit the pair-gathered 8-bit call of its expert on its row."""
+    from vpipe_amd import capi
+    B = capi.VPQ_QMV_GROUPED_SLOTS
+    Kd = 64 * ((inner + 63) // 64)
+    gu = [interleaved8(inner, K, 3900 + 5 * e) for e in range(E)]
+    dn = [synth.make_weight8(H, Kd, 3950 + e) for e in range(E)]
+    guw, gus, gub = (np.stack([p[i] for p in gu]) for i in range(3))
+    dw, ds, db = (np.stack([p[i] for p in dn]) for i in range(3))
+    x = synth.make_act(T, K, 3990 + K)
+    eid = np.random.default_rng(3991 + K).integers(0, E, size=T * top_k, dtype=np.int32)
+    eid_d = torch.from_numpy(eid).to(dev)
+    t2e_d, srow_d, sdst_d, _ = vpq.moe_sort_pairs(eid_d, top_k, E, block_rows=B)
+    t2e, srow, sdst = (o.cpu().numpy() for o in (t2e_d, srow_d, sdst_d))
+    npad = srow.size
+    live = srow >= 0
+    slots = np.nonzero(live)[0]
+    assert slots.size == eid.size
+    seven = D.bits(torch.full((1,), 7.0, dtype=torch.bfloat16))[0]
+
+    guwd, gusd, gubd, xd = stage(D, dev, guw, gus, gub, x)
+    act_out = parity.Guarded((npad, inner), torch.bfloat16, dev)
+    act_out.view.fill_(7.0)
+    vpq.qmv_grouped_gated_w8g64(guwd, gusd, gubd, xd, K, 2 * inner, t2e_d, srow_d, E, out=act_out.view, activation=activation)
+    torch.cuda.synchronize()
+    act_out.assert_intact()
+    got = D.bits(act_out.view)
+    assert (got[~live] == seven).all()
+    y64 = np.concatenate([oracle.matmul8(guw[t2e[s // B]], gus[t2e[s // B]], gub[t2e[s // B]], x[srow[s]:srow[s] + 1], K, 2 * inner, 1,
+                                         rounded=False)[0] for s in slots])
+    want64, wantb = (oracle.swiglu if activation == 1 else oracle.geglu)(y64)
+    parity.check_bf16(got[slots], want64, wantb, mismatch_over_all=activation == 1)
+    pairwise = D.bits(vpq.gather_qmv_gated_w8g64(guwd, gusd, gubd, xd, K, 2 * inner, eid_d, top_k, E, activation=activation))
+    assert np.array_equal(got[slots], pairwise[sdst[slots]])
+
+    xs = synth.make_act(npad, Kd, 3995 + K)
+    dwd, dsd, dbd, xsd = stage(D, dev, dw, ds, db, xs)
+    down = parity.Guarded((npad, H), torch.bfloat16, dev)
+    down.view.fill_(7.0)
+    vpq.qmv_grouped_down_w8g64(dwd, dsd, dbd, xsd, Kd, H, t2e_d, srow_d, E, out=down.view)
+    torch.cuda.synchronize()
+    down.assert_intact()
+    gotd = D.bits(down.view)
+    assert (gotd[~live] == seven).all()
+    pairs = [oracle.matmul8(dw[t2e[s // B]], ds[t2e[s // B]], db[t2e[s // B]], xs[s:s + 1], Kd, H, 1, rounded=False) for s in slots]
+    parity.check_bf16(gotd[slots], np.concatenate([p[0] for p in pairs]), np.concatenate([p[1] for p in pairs]))
+    slot_eid = torch.from_numpy(np.ascontiguousarray(t2e[slots // B]).astype(np.int32)).to(dev)
+    pairwise = D.bits(vpq.gather_down_qmv_w8g64(dwd, dsd, dbd, xsd[torch.from_numpy(slots).to(dev)].contiguous(), Kd, H, slot_eid, E))
+    assert np.array_equal(gotd[slots], pairwise)
+    L = vpq.load()
+    p = xsd.data_ptr()
+    assert L.vpq_qmv_grouped_gated_w8g64_bf16(None, p, p, p, p, p, 64, 8, 3, p, p, 1, 1) == -2      # not whole tiles
+    assert L.vpq_qmv_grouped_down_w8g64_bf16(None, p, p, p, p, p, 60, 8, 2, p, p, 1) == -2          # K % 64
+
+
 @pytest.mark.parametrize("K,inner,H,E,T,top_k", [(512, 128, 300, 5, 150, 2), (1024, 64, 100, 4, 90, 2), (576, 96, 512, 3, 60, 1)])
 def test_grouped_expert_gemms_w8(vpq, oracle, dev, D, K, inner, H, E, T, top_k):
     # the expert-sorted prefill GEMMs over 8-bit experts (K = 576: the per-step scale loads, K % 512 == 0: the

@@ -49,6 +49,8 @@ SYMBOLS = [
     ("vpq_sample_topp_bf16", _i, [_vp, _vp, _vp, _i, _f, _f, ctypes.c_uint32, _vp, _i, _f, _f, _i, _f, _vp]),
     ("vpq_qmv_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
     ("vpq_qmv_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i]),
+    ("vpq_qmv_grouped_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
+    ("vpq_qmv_grouped_down_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i]),
     ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
     ("vpq_qmv_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _i]),
     ("vpq_qmv_workspace_bytes", _sz, [_i, _i, _i]),
@@ -343,22 +345,30 @@ def qmm_grouped_down_w4g64(w, scales, biases, x, K, N, tile2e, sdst, n_experts, 
 VPQ_QMV_GROUPED_SLOTS = 2
 
 
-def qmv_grouped_gated_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out, activation=VPQ_GATE_SWIGLU):
+def qmv_grouped_gated_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out, activation=VPQ_GATE_SWIGLU, bits=4):
     """Expert batch [E, N=2*inner, ...], x [rows_x, K], tiles of two sorted slots -> live rows of out [npad, N/2]."""
     npad = srow.numel()
-    _check(load().vpq_qmv_grouped_gated_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
-                                                   npad, _ptr(tile2e), _ptr(srow), n_experts, activation),
-           "vpq_qmv_grouped_gated_w4g64_bf16")
+    name = "vpq_qmv_grouped_gated_w%dg64_bf16" % bits
+    _check(getattr(load(), name)(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                 npad, _ptr(tile2e), _ptr(srow), n_experts, activation), name)
     return out
 
 
-def qmv_grouped_down_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out):
+def qmv_grouped_down_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out, bits=4):
     """Expert batch [E, N, ...], x [npad, K] in slot order -> live rows of out [npad, N] in slot order."""
     npad = srow.numel()
-    _check(load().vpq_qmv_grouped_down_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
-                                                  npad, _ptr(tile2e), _ptr(srow), n_experts),
-           "vpq_qmv_grouped_down_w4g64_bf16")
+    name = "vpq_qmv_grouped_down_w%dg64_bf16" % bits
+    _check(getattr(load(), name)(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                 npad, _ptr(tile2e), _ptr(srow), n_experts), name)
     return out
+
+
+def qmv_grouped_gated_w8g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out, activation=VPQ_GATE_SWIGLU):
+    return qmv_grouped_gated_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out, activation, bits=8)
+
+
+def qmv_grouped_down_w8g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out):
+    return qmv_grouped_down_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, out, bits=8)
 
 
 def qmv_w4g64(w, scales, biases, x, K, N, M, out=None, residual=None, ws=None, variant=0, f32out=False):

@@ -825,7 +825,7 @@ namespace {
 
 int sorted_qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                       const uint16_t* x, uint16_t* y, int K, int N, int npad, const int32_t* tile2e, const int32_t* srow,
-                      int n_experts, int gate_act, bool x_from_srow)
+                      int n_experts, int gate_act, bool x_from_srow, int bits = 4)
 {
   int st = check_pack(w, scales, biases, K, N);
   if (st != VPQ_OK) { return st; }
@@ -843,6 +843,10 @@ int sorted_qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* sc
   a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y;
   a.K = K; a.N = N; a.M = VPQ_QMV_GROUPED_SLOTS; a.y_f32 = false; a.cu_count = g_dev.cu_count;
   a.gate_act = gate_act;
+  if (bits == 8) {
+    return finish(vpq::launch_qmv_rows8_sorted(reinterpret_cast<hipStream_t>(stream), a, tile2e, srow,
+                                               npad / VPQ_QMV_GROUPED_SLOTS, n_experts));
+  }
   return finish(vpq::launch_qmv_rows_sorted(reinterpret_cast<hipStream_t>(stream), a, tile2e, srow,
                                             npad / VPQ_QMV_GROUPED_SLOTS, x_from_srow, n_experts));
 }
@@ -862,6 +866,21 @@ int vpq_qmv_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, cons
                                     const int32_t* tile2e, const int32_t* srow, int n_experts)
 {
   return sorted_qmv_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, srow, n_experts, 0, false);
+}
+
+int vpq_qmv_grouped_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
+                                     const int32_t* tile2e, const int32_t* srow, int n_experts, int activation)
+{
+  if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
+  return sorted_qmv_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, srow, n_experts, activation, true, 8);
+}
+
+int vpq_qmv_grouped_down_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
+                                    const int32_t* tile2e, const int32_t* srow, int n_experts)
+{
+  return sorted_qmv_common(stream, w, scales, biases, x, y, K, N, npad, tile2e, srow, n_experts, 0, false, 8);
 }
 
 int vpq_sample_topp_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, float temp,

@@ -107,6 +107,9 @@ hipError_t launch_qmv_split_gate_up(hipStream_t st, const SplitGateUp& a);
 // 8-bit gated / gathered QMV, one wavefront per output and row (a.gate_act: interleaved gate|up pack);
 // rows = rows of x, or with pair_eid the (token, expert) pairs over a batched pack.
 hipError_t launch_qmv_rows8(hipStream_t st, const QmvArgs& a, int rows, const int* pair_eid, int x_div, int n_experts);
+// Two-slot expert-sorted GEMV over a batched 8-bit pack (a.gate_act != 0: x rows gathered through srow).
+hipError_t launch_qmv_rows8_sorted(hipStream_t st, const QmvArgs& a, const int* tile2e, const int* srow, int tiles,
+                                   int n_experts);
 // Returns hipErrorInvalidValue if the shape is outside what the MFMA kernel
 // handles (the caller then falls back to the simple kernel).
 bool qmv_mfma_supports(int K, int N, int M);

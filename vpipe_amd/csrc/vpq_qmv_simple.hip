@@ -300,6 +300,110 @@ hipError_t launch_qmv_rows8(hipStream_t st, const QmvArgs& a, int rows, const in
                                     pair_eid, x_div, n_experts);
 }
 
+// Expert-sorted form for a few rows per expert (gpu-kernels/metal/quant/affine_qmv.metal:2551-2719,
+// `affine_grouped_swiglu_w8g64`, `affine_grouped_down_w8g64`, MAXM = 2): blockIdx.y is a tile of two slots owned by
+// expert tile2e[tile] (outside [0, n_experts): unused tile, nothing written); slot s is live where srow[s] >= 0 and
+// reads x row srow[s] (X_FROM_SROW: the gate|up projection gathers the hidden rows) or row s (the down projection
+// reads the sorted activations), and writes y row s.  A wavefront reads its row (or gate and up rows) of the
+// expert's slab once for both slots; per slot the arithmetic is qmv_rows8_kernel's, term for term.
+template <bool GATED, bool X_FROM_SROW>
+__global__ __launch_bounds__(256) void qmv_rows8_sorted_kernel(
+    const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales, const uint16_t* __restrict__ biases,
+    const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int K, int N, int gate_act,
+    const int* __restrict__ tile2e, const int* __restrict__ srow, int n_experts)
+{
+  constexpr int MT = 2;                       // slots per tile
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int outs = GATED ? (N >> 1) : N;
+  const int o = blockIdx.x * 4 + wave;
+  if (o >= outs) { return; }  // wave-uniform; no barrier in this kernel
+  const int t = blockIdx.y;
+  const int e = tile2e[t];
+  if (e < 0 || e >= n_experts) { return; }
+  const int Kw = K >> 2, Kg = K >> 6;
+  w += (size_t)e * (size_t)N * Kw;
+  scales += (size_t)e * (size_t)N * Kg;
+  biases += (size_t)e * (size_t)N * Kg;
+  const uint16_t* xr[MT];
+  bool live[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const int slot = t * MT + m;
+    const int rr = srow[slot];
+    live[m] = rr >= 0;
+    xr[m] = x + (size_t)(X_FROM_SROW ? (rr >= 0 ? rr : 0) : slot) * K;
+  }
+  constexpr int R = GATED ? 2 : 1;
+  const int n0 = GATED ? 2 * o : o;
+  float acc[MT][R];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) { acc[m][r] = 0.0f; }
+  }
+  for (int k0 = lane * 16; k0 < K; k0 += kWave * 16) {
+    float xv[MT][16];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const uint4* xp = reinterpret_cast<const uint4*>(xr[m] + k0);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint4 x4 = xp[h];
+        const uint32_t xd[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          xv[m][8 * h + 2 * j] = bf16_lo_to_f32(xd[j]);
+          xv[m][8 * h + 2 * j + 1] = bf16_hi_to_f32(xd[j]);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const size_t n = (size_t)(n0 + r);
+      const uint4 c4 = *reinterpret_cast<const uint4*>(w + n * Kw + (k0 >> 2));
+      const uint32_t codes[4] = {c4.x, c4.y, c4.z, c4.w};
+      const float s = bf16_bits_to_f32(scales[n * Kg + (k0 >> 6)]);
+      const float b = bf16_bits_to_f32(biases[n * Kg + (k0 >> 6)]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float wv = fmaf(s, (float)((codes[i] >> (8 * j)) & 0xffu), b);
+#pragma unroll
+          for (int m = 0; m < MT; ++m) { acc[m][r] = fmaf(xv[m][4 * i + j], wv, acc[m][r]); }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) { acc[m][r] = wave_sum(acc[m][r]); }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      if (!live[m]) { continue; }
+      const float v = GATED ? gated_f32(gate_act, acc[m][0], acc[m][R - 1]) : acc[m][0];
+      y[(size_t)(t * MT + m) * outs + o] = (uint16_t)f32_to_bf16_bits(v);
+    }
+  }
+}
+
+// a.gate_act != 0: the gate|up projection (x rows through srow); else the down projection (x in slot order).
+hipError_t launch_qmv_rows8_sorted(hipStream_t st, const QmvArgs& a, const int* tile2e, const int* srow, int tiles,
+                                   int n_experts)
+{
+  const int outs = a.gate_act ? a.N / 2 : a.N;
+  const dim3 grid((unsigned)((outs + 3) / 4), (unsigned)tiles), block(256);
+  uint16_t* y = static_cast<uint16_t*>(a.y);
+  return a.gate_act ? launch_kernel(qmv_rows8_sorted_kernel<true, true>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, y,
+                                    a.K, a.N, a.gate_act, tile2e, srow, n_experts)
+                    : launch_kernel(qmv_rows8_sorted_kernel<false, false>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, y,
+                                    a.K, a.N, 0, tile2e, srow, n_experts);
+}
+
 // Mixed-width fused gate/up (affine_gather_qmv_swiglu_w4w8g64 / _w8w4g64,
 // gpu-kernels/metal/quant/affine_qmv.metal:991-1260): gate and up are SEPARATE packs [E, ffn, ...], each at
 // its own width (4 or 8 bits) as a per-tensor quantizer left them; a wavefront contracts the gate row and

@@ -114,6 +114,8 @@ const FnEntry kFunctions[] = {
     {"affine_dequant_bf16", "affine_dequant_w8g64", QuantKernel::Dequant, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64", QuantKernel::Qmv, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_grouped_swiglu_w8g64", QuantKernel::SortedSwiglu, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_grouped_down_w8g64", QuantKernel::SortedDown, QuantFormat::W8G64},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64", QuantKernel::Qmm, QuantFormat::W8G64},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64_bm64", QuantKernel::Qmm, QuantFormat::W8G64},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64_bm128", QuantKernel::Qmm, QuantFormat::W8G64},
@@ -462,6 +464,23 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
         status = !has_int(7) ? VPQ_ERR_NULL_POINTER
                              : vpq_qmm_gated_w4g32_bf16(st, w, sc, bi, x, y, K, N, ival(7),
                                                         kind == QuantKernel::QmmGeglu ? VPQ_GATE_GEGLU : 0);
+      } else if (fmt == QuantFormat::W8G64 && (kind == QuantKernel::SortedSwiglu || kind == QuantKernel::SortedDown)) {
+        // gpu-kernels/metal/quant/affine_qmv.metal:2682-2719: slot 7 = srow, 8 = tile2e, one tile of two sorted
+        // slots per grid.z; the expert count is the number of [N, K] byte slabs the bound code buffer holds
+        if (!buf(7) || !buf(8)) {
+          status = VPQ_ERR_NULL_POINTER;
+        } else if (K <= 0 || N <= 0 || K % 64 != 0) {
+          status = VPQ_ERR_BAD_SHAPE;
+        } else {
+          const std::size_t experts = _slots[0].bytes / (static_cast<std::size_t>(N) * static_cast<std::size_t>(K));
+          const int E = experts > 0x7fffffffu ? 0x7fffffff : static_cast<int>(experts);
+          const int npad = static_cast<int>(grid.z) * VPQ_QMV_GROUPED_SLOTS;
+          const int32_t* srow = static_cast<const int32_t*>(buf(7));
+          const int32_t* t2e = static_cast<const int32_t*>(buf(8));
+          status = kind == QuantKernel::SortedDown
+                       ? vpq_qmv_grouped_down_w8g64_bf16(st, w, sc, bi, x, y, K, N, npad, t2e, srow, E)
+                       : vpq_qmv_grouped_gated_w8g64_bf16(st, w, sc, bi, x, y, K, N, npad, t2e, srow, E, VPQ_GATE_SWIGLU);
+        }
       } else if (fmt == QuantFormat::W8G64 && grouped) {
         // :1069-1090, 1290-1366: slot 7 = npad, 8 = tile2e, 9 = srow / sdst, as the 4-bit grouped functions
         const bool down = kind == QuantKernel::GroupedDown;
