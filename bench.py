@@ -461,13 +461,13 @@ def main():
             for _ in range(2):
                 fn(0)
             torch.cuda.synchronize()
-            L.vpq_profile_enable(4 * iters)
+            L.vpq_profile_enable(8 * iters)
             for i in range(iters):
                 fn(i)
-            kb = (ctypes.c_float * (4 * iters))()
-            n = L.vpq_profile_read(kb, 4 * iters)
+            kb = (ctypes.c_float * (8 * iters))()
+            n = L.vpq_profile_read(kb, 8 * iters)
             L.vpq_profile_enable(0)
-            return float(np.sum(kb[:n])) * 1e3 / iters     # all kernels of a call (LoRA: two)
+            return float(np.sum(kb[:n])) * 1e3 / iters     # all kernels of a call (LoRA: two, the sampler: five)
 
         # small-batch QMV of a 5120-hidden model, weights rotated so that they come from HBM
         small = {}
@@ -687,9 +687,16 @@ def main():
         # stochastic tail: the one-workgroup sampler (top-k 50, top-p 0.9, 24 bisection steps each) over the same logits
         seen_b = torch.zeros((151936,), dtype=torch.uint8, device=dev)
         ws_b = torch.empty((151936,), dtype=torch.bfloat16, device=dev)
+        n_slabs = vpipe_amd.sample_hist_slabs(151936)
+        work_b = torch.empty((int(L.vpq_sample_hist_workspace_bytes(n_slabs)) // 4,), dtype=torch.float32, device=dev)
         out["sample_topp_v151936"] = {
             "one_workgroup_us": round(kernel_us(lambda i: vpipe_amd.sample_topp_bf16(lg.view(-1), seen_b, 0.8, 0.9, 1000 + i,
-                                                                                      ws=ws_b, out=tok, top_k=50), 8), 1)}
+                                                                                      ws=ws_b, out=tok, top_k=50), 8), 1),
+            # the same draw over n_slabs workgroups with histogram thresholds: all five launches of a call
+            "histogram_slabs": n_slabs,
+            "histogram_us": round(kernel_us(lambda i: vpipe_amd.sample_hist_bf16(lg.view(-1), seen_b, 0.8, 0.9, 1000 + i,
+                                                                                 ws=ws_b, out=tok, work=work_b, n_slabs=n_slabs,
+                                                                                 top_k=50), 8), 1)}
 
         # MoE decode block, pair-batched gathers (hidden 2048, expert inner 768, 128 experts, top-8,
         # one token): 8 of the 128 gate|up slabs and 8 down slabs per step, a fresh random set of

@@ -691,13 +691,34 @@ int vpq_f16_to_bf16(vpq_stream_t stream, const uint16_t* in_f16, uint16_t* out_b
  * token 0 if nothing is kept.  The draw is an exact function of its inputs:
  * exp, log and the reduction order are fixed (see vpq_sample.hip), so the
  * same (logits, seen, parameters, seed) give the same token on every run.
- * The reference's multi-threadgroup histogram variant (:3318-3574), which
- * loosens the thresholds to bin edges, is not built.
+ * One workgroup: ~0.5-0.9 ms at 151936 logits; see vpq_sample_hist_bf16.
  * Requires V >= 1, n_iter >= 0, rep != 0; all pointers non-NULL, logits and ws
  * 2-byte, out_id 4-byte aligned. */
 int vpq_sample_topp_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, float temp,
                          float top_p, uint32_t seed, uint16_t* ws, int n_iter, float rep_penalty,
                          float presence_penalty, int top_k, float min_p, uint8_t* seen);
+
+/* vpq_sample_hist_bf16 replaces the reference's multi-threadgroup sampler
+ * `sample_max_partial_f16`, `sample_max_combine_f16`, `sample_zhist_partial_f16`,
+ * `sample_zhist_combine_f16`, `sample_thresh_f16`, `sample_pick_partial_f16`,
+ * `sample_pick_combine_f16` (llm_elementwise.metal:3255-3640; its M is n_slabs
+ * here) -- seven dispatches there, one call (five launches) here.  Same
+ * pipeline and arguments as vpq_sample_topp_bf16 without n_iter: the
+ * vocabulary is cut into n_slabs contiguous slabs of ceil(V / n_slabs) indices,
+ * one workgroup each, and top-k / top-p become the low edge of a bin of a
+ * histogram of the weights (1024 bins uniform in -log w over [0, 40)), so the
+ * kept set is the exact sampler's plus at most one bin (weights within a
+ * factor e^(40/1024) = 1.04 below the exact threshold); min-p stays exact.
+ * The draw is an exact function of (logits, seen, parameters, seed, n_slabs).
+ * `work`: vpq_sample_hist_workspace_bytes(n_slabs) bytes of device scratch
+ * (slab maxima, per-slab histograms, their sum, the threshold, per-slab
+ * picks), 4-byte aligned; nothing in it needs to be cleared.
+ * Requires V >= 1, rep != 0, 1 <= n_slabs <= 1024, ceil(V / n_slabs) <= 65535
+ * (the per-slab fixed-point masses); other requirements as above. */
+size_t vpq_sample_hist_workspace_bytes(int n_slabs);
+int vpq_sample_hist_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, float temp,
+                         float top_p, uint32_t seed, uint16_t* ws, float rep_penalty, float presence_penalty,
+                         int top_k, float min_p, uint8_t* seen, int n_slabs, void* work, size_t work_bytes);
 
 /* ---- measurement aid (no counterpart in the reference's kernels; the
  * reference times command buffers with Fence::gpu_times(),

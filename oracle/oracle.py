@@ -164,6 +164,23 @@ def sample_topp(logits, seen, temp, top_p, seed, n_iter=24, rep=1.0, pres=0.0, t
     return int(tok), ws, seen
 
 
+def sample_hist(logits, seen, temp, top_p, seed, n_slabs, rep=1.0, pres=0.0, top_k=0, min_p=0.0):
+    """The sampler over n_slabs slabs with histogram thresholds: bf16 bits [V], uint8 [V] ->
+    (token, cached weights bf16 bits [V], seen after the draw, weight threshold)."""
+    L = lib()
+    L.vpo_sample_hist_bf16.restype = ctypes.c_int32
+    L.vpo_sample_hist_bf16.argtypes = [_u16p, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_uint32, _u16p,
+                                       ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_float,
+                                       ctypes.POINTER(ctypes.c_uint8), ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+    logits = _c(logits, np.uint16)
+    seen = np.array(seen, dtype=np.uint8, copy=True)
+    ws = np.empty(logits.shape, dtype=np.uint16)
+    wt = ctypes.c_float(0.0)
+    tok = L.vpo_sample_hist_bf16(_p(logits, _u16p), logits.size, temp, top_p, seed, _p(ws, _u16p), rep, pres, top_k, min_p,
+                                 seen.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), n_slabs, ctypes.byref(wt))
+    return int(tok), ws, seen, float(wt.value)
+
+
 def qmv(w, s, b, x, K, N, M, residual=None):
     """-> (y64 [M,N] float64, y_bf16 [M,N] uint16); un-rounded-weight semantics."""
     w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)

@@ -412,6 +412,152 @@ int32_t vpo_sample_topp_bf16(const uint16_t* logits, int V, float temp, float to
   return pick;
 }
 
+/* ---- the sampler over many workgroups, thresholds from a histogram ----------
+ * gpu-kernels/metal/ops/llm_elementwise.metal:3255-3640 (`sample_max_partial_f16` .. `sample_pick_combine_f16`): the
+ * same pipeline as above with the vocabulary cut into n_slabs contiguous slabs (slab = ceil(V / n_slabs) indices),
+ * and the top-k / top-p thresholds read off a histogram of the weights instead of bisected:
+ *   bins     1024, uniform in -log(w) over [0, 40): bin(w) = clamp(int(-log(max(w, 1e-30)) / (40/1024)), 0, 1023)
+ *            (:3305-3314), bin 0 the largest weights; per bin a count and a mass, the mass summed per slab in
+ *            fixed point (uint32 of w * 2^16, truncated; :3293-3303, 3398-3400) and then as fp32;
+ *   combine  counts, masses and Z of the slabs are added in slab order 0, 1, ... (:3432-3452);
+ *   thresh   a scan from bin 0 down: t_k = low edge exp(-(b+1) * 40/1024) of the bin where the running count first
+ *            reaches top_k (0 < top_k < V), t_p that of the bin where the running mass first reaches top_p * Z;
+ *            wt = max(t_k, max(min_p, 0), t_p); a target never reached leaves its threshold 0 (:3461-3497).  The
+ *            running sums are formed in two levels (chunks of 32 bins), see below;
+ *   pick     Gumbel-max over {ws_i >= wt} per slab, lowest index on ties, then over the slabs (:3499-3600).
+ * Fixed here as above: exp / log are the written-out polynomials; inside a slab a thread t of 256 takes the indices
+ * lo + t, lo + t + 256, ... in ascending order and the 256 partial sums meet in a halving tree.  wt_out (nullable)
+ * receives the threshold. */
+#define VPO_HIST_THREADS 256
+#define VPO_HIST_BINS 1024
+
+static int vpo_sample_bin(float w)
+{
+  const float lw = 0.0f - vpo_sample_log(w > 1e-30f ? w : 1e-30f);
+  int b = (int)(lw / (40.0f / 1024.0f));
+  if (b < 0) { b = 0; }
+  if (b >= VPO_HIST_BINS) { b = VPO_HIST_BINS - 1; }
+  return b;
+}
+
+int32_t vpo_sample_hist_bf16(const uint16_t* logits, int V, float temp, float top_p, uint32_t seed, uint16_t* ws,
+                             float rep, float pres, int top_k, float min_p, uint8_t* seen, int n_slabs, float* wt_out)
+{
+  const int T = VPO_HIST_THREADS, B = VPO_HIST_BINS;
+  const int slab = (V + n_slabs - 1) / n_slabs;
+  const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
+  const float binw = 40.0f / 1024.0f;
+  float tg[VPO_HIST_THREADS];
+  int tgi[VPO_HIST_THREADS];
+  /* pass A: the largest penalised logit (a maximum: no order) */
+  float maxl = -INFINITY;
+  for (int i = 0; i < V; ++i) {
+    const float e = vpo_sample_eff(vpo_bf16_to_f32(logits[i]), seen[i] != 0, rep, pres);
+    maxl = e > maxl ? e : maxl;
+  }
+  /* pass B: weights, per slab a partial Z and a histogram; combined in slab order */
+  float* hist = (float*)calloc((size_t)(2 * B), sizeof(float));
+  uint32_t* cnt = (uint32_t*)malloc((size_t)B * sizeof(uint32_t));
+  uint32_t* mass = (uint32_t*)malloc((size_t)B * sizeof(uint32_t));
+  float Z = 0.0f;
+  for (int g = 0; g < n_slabs; ++g) {
+    const int lo = g * slab;
+    const int hi = lo + slab < V ? lo + slab : V;
+    memset(cnt, 0, (size_t)B * sizeof(uint32_t));
+    memset(mass, 0, (size_t)B * sizeof(uint32_t));
+    for (int t = 0; t < T; ++t) {
+      float z = 0.0f;
+      for (int i = lo + t; i < hi; i += T) {
+        const float e = vpo_sample_eff(vpo_bf16_to_f32(logits[i]), seen[i] != 0, rep, pres);
+        const float w = vpo_sample_exp((e - maxl) * inv_t);
+        ws[i] = vpo_f32_to_bf16(w);
+        z = z + w;
+        const int b = vpo_sample_bin(w);
+        cnt[b] += 1u;
+        mass[b] += (uint32_t)(w * 65536.0f);
+      }
+      tg[t] = z;
+    }
+    for (int s = T >> 1; s > 0; s >>= 1) {
+      for (int t = 0; t < s; ++t) { tg[t] = tg[t] + tg[t + s]; }
+    }
+    Z = Z + tg[0];
+    for (int b = 0; b < B; ++b) {
+      hist[b] = hist[b] + (float)cnt[b];
+      hist[B + b] = hist[B + b] + (float)mass[b] * (1.0f / 65536.0f);
+    }
+  }
+  /* thresholds: the running sum at a bin is (the totals of the 32-bin chunks before its chunk) + (its chunk up to
+   * it), each sum in ascending order from 0 -- the reference's single scan (:3476-3489) up to the association of
+   * the fp32 additions of the masses (the counts are integers) */
+  const float target = top_p * Z;
+  float t_k = 0.0f, t_p = 0.0f, before_cnt = 0.0f, before_mass = 0.0f;
+  int have_k = 0, have_p = 0;
+  const int do_k = top_k > 0 && top_k < V;
+  for (int j = 0; j < B / 32; ++j) {
+    float tot_cnt = 0.0f, tot_mass = 0.0f;
+    for (int b = 32 * j; b < 32 * j + 32; ++b) { tot_cnt = tot_cnt + hist[b]; tot_mass = tot_mass + hist[B + b]; }
+    if (do_k && !have_k && before_cnt + tot_cnt >= (float)top_k) {
+      float in_chunk = 0.0f;
+      for (int b = 32 * j; b < 32 * j + 32; ++b) {
+        in_chunk = in_chunk + hist[b];
+        if (before_cnt + in_chunk >= (float)top_k) { t_k = vpo_sample_exp(0.0f - (float)(b + 1) * binw); break; }
+      }
+      have_k = 1;
+    }
+    if (!have_p && before_mass + tot_mass >= target) {
+      float in_chunk = 0.0f;
+      for (int b = 32 * j; b < 32 * j + 32; ++b) {
+        in_chunk = in_chunk + hist[B + b];
+        if (before_mass + in_chunk >= target) { t_p = vpo_sample_exp(0.0f - (float)(b + 1) * binw); break; }
+      }
+      have_p = 1;
+    }
+    if ((!do_k || have_k) && have_p) { break; }
+    before_cnt = before_cnt + tot_cnt;
+    before_mass = before_mass + tot_mass;
+  }
+  free(hist); free(cnt); free(mass);
+  const float wt = fmaxf(fmaxf(t_k, fmaxf(min_p, 0.0f)), t_p);
+  if (wt_out) { *wt_out = wt; }
+  /* pass C: Gumbel-max per slab, then over the slabs */
+  float best_all = -INFINITY;
+  int bi_all = -1;
+  for (int g = 0; g < n_slabs; ++g) {
+    const int lo = g * slab;
+    const int hi = lo + slab < V ? lo + slab : V;
+    for (int t = 0; t < T; ++t) {
+      float best = -INFINITY;
+      int bi = -1;
+      for (int i = lo + t; i < hi; i += T) {
+        if (vpo_bf16_to_f32(ws[i]) >= wt) {
+          const float e = vpo_sample_eff(vpo_bf16_to_f32(logits[i]), seen[i] != 0, rep, pres);
+          const float u = vpo_sample_hash_u01(seed ^ ((uint32_t)i * 2654435761u + 1u));
+          const float a = 0.0f - vpo_sample_log(u + 1e-20f) + 1e-20f;
+          const float gum = 0.0f - vpo_sample_log(a);
+          const float score = e * inv_t + gum;
+          if (score > best) { best = score; bi = i; }
+        }
+      }
+      tg[t] = best;
+      tgi[t] = bi;
+    }
+    for (int s = T >> 1; s > 0; s >>= 1) {
+      for (int t = 0; t < s; ++t) {
+        const int take = tg[t + s] > tg[t] || (tg[t + s] == tg[t] && tgi[t + s] >= 0 && (tgi[t] < 0 || tgi[t + s] < tgi[t]));
+        if (take) { tg[t] = tg[t + s]; tgi[t] = tgi[t + s]; }
+      }
+    }
+    if (tgi[0] >= 0 && (tg[0] > best_all || (tg[0] == best_all && (bi_all < 0 || tgi[0] < bi_all)))) {
+      best_all = tg[0];
+      bi_all = tgi[0];
+    }
+  }
+  const int pick = bi_all >= 0 ? bi_all : 0;
+  seen[pick] = 1;
+  return pick;
+}
+
 /* ---- a2/a3: QMV -------------------------------------------------------- */
 
 /* The CPU reference loop of the reference's own QMV test,

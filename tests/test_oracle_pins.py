@@ -739,3 +739,77 @@ def test_sampler_draws_from_the_filtered_distribution(oracle, temp, top_p, top_k
     chi2 = (((counts[big] - prob[big] * draws) ** 2) / (prob[big] * draws)).sum()
     dof = int(big.sum())
     assert chi2 < dof + 6 * np.sqrt(2 * dof) + 10, (chi2, dof)
+
+
+def test_histogram_sampler_with_the_filters_off_is_the_exact_sampler(oracle):
+    """No top-k, no top-p: nothing depends on the histogram, so the token (and the cached weights) are those of the
+    one-workgroup sampler, which is pinned above; with min-p alone the threshold is min_p itself in both."""
+    rng = np.random.default_rng(51)
+    for V, n_slabs in ((1, 1), (300, 1), (300, 7), (5000, 3), (5000, 64)):
+        bits = synth.f32_to_bf16_bits((rng.standard_normal(V) * 3).astype(np.float32))
+        seen = (rng.random(V) < 0.15).astype(np.uint8)
+        for seed in range(12):
+            for min_p in (0.0, 0.03):
+                a = oracle.sample_topp(bits, seen, 0.9, 1.0, seed, rep=1.3, pres=0.2, min_p=min_p)
+                b = oracle.sample_hist(bits, seen, 0.9, 1.0, seed, n_slabs, rep=1.3, pres=0.2, min_p=min_p)
+                assert a[0] == b[0] and np.array_equal(a[1], b[1]) and np.array_equal(a[2], b[2])
+                w = synth.bf16_bits_to_f32(b[1])
+                assert np.array_equal(w >= b[3], w >= np.float32(min_p))      # the threshold keeps what min_p keeps
+
+
+@pytest.mark.parametrize("temp,top_p,top_k,min_p", [(1.0, 0.9, 0, 0.0), (0.7, 1.0, 25, 0.0), (1.2, 0.8, 60, 0.0),
+                                                    (1.0, 0.95, 40, 0.01), (1.0, 0.5, 3, 0.0)])
+def test_histogram_sampler_threshold_is_the_low_edge_of_the_boundary_bin(oracle, temp, top_p, top_k, min_p):
+    """The threshold against a float64 sort: for top-k it is the low edge of the bin holding the k-th largest weight,
+    for top-p that of the bin holding the last weight of the smallest nucleus -- at most the exact threshold, and
+    more than it divided by one bin's width (two where the truncated fixed-point masses may push the nucleus one bin
+    on); the three thresholds combine by their maximum."""
+    rng = np.random.default_rng(61)
+    binw = 40.0 / 1024.0
+    for V, n_slabs in ((400, 1), (6000, 5), (6000, 64)):
+        vals = synth.bf16_bits_to_f32(synth.f32_to_bf16_bits((rng.standard_normal(V) * 2.5).astype(np.float32)))
+        bits = synth.f32_to_bf16_bits(vals)
+        seen = np.zeros(V, dtype=np.uint8)
+        _, _, _, wt = oracle.sample_hist(bits, seen, temp, top_p, 3, n_slabs, top_k=top_k, min_p=min_p)
+        w = np.exp((vals.astype(np.float64) - vals.max()) / temp)
+        sw = np.sort(w)[::-1]
+        lo, hi = [], []
+        if 0 < top_k < V:
+            lo.append(sw[top_k - 1] * np.exp(-binw)); hi.append(sw[top_k - 1])
+        n = int(np.searchsorted(np.cumsum(sw), top_p * w.sum(), side="left"))
+        if n < V:
+            lo.append(sw[n] * np.exp(-2 * binw)); hi.append(sw[n])
+        lo.append(min_p); hi.append(min_p)
+        assert max(lo) * (1 - 1e-5) < wt <= max(hi) * (1 + 1e-5), (V, n_slabs, wt, lo, hi)
+        # and it is a bin edge (or min_p): -log(wt) / binw is an integer
+        if wt > min_p:
+            r = -np.log(float(wt)) / binw
+            assert abs(r - round(r)) < 1e-3 and round(r) >= 1
+
+
+def test_histogram_sampler_draws_from_the_kept_set(oracle):
+    """Draws over many seeds stay inside {w >= threshold} and follow the renormalised float64 probabilities of that
+    set (chi-square); the drawn token is marked seen."""
+    rng = np.random.default_rng(71)
+    V, n_slabs, temp, top_p, top_k = 300, 4, 0.9, 0.92, 35
+    bits = synth.f32_to_bf16_bits((rng.standard_normal(V) * 2.0).astype(np.float32))
+    seen = (rng.random(V) < 0.2).astype(np.uint8)
+    rep, pres = 1.2, 0.3
+    _, _, eff = _sampler_kept_set_f64(synth.bf16_bits_to_f32(bits), seen, temp, 1.0, rep, pres, 0, 0.0)
+    draws = 6000
+    counts = np.zeros(V)
+    for seed in range(draws):
+        tok, ws, seen_after, wt = oracle.sample_hist(bits, seen, temp, top_p, seed * 2654435761 % (1 << 32), n_slabs, rep=rep,
+                                                     pres=pres, top_k=top_k)
+        counts[tok] += 1
+        assert seen_after[tok] == 1
+    w = synth.bf16_bits_to_f32(ws).astype(np.float64)
+    keep = w >= wt
+    assert not counts[~keep].any()
+    assert top_k <= keep.sum() < V // 2                       # looser than top-k by at most a bin, far from everything
+    p64 = np.exp((eff - eff.max()) / temp) * keep
+    p64 /= p64.sum()
+    big = keep & (p64 * draws >= 8)
+    chi2 = (((counts[big] - p64[big] * draws) ** 2) / (p64[big] * draws)).sum()
+    dof = int(big.sum())
+    assert chi2 < dof + 6 * np.sqrt(2 * dof) + 10, (chi2, dof)

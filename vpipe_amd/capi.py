@@ -47,6 +47,8 @@ SYMBOLS = [
     ("vpq_qmm_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _i]),
     ("vpq_qmm_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
     ("vpq_sample_topp_bf16", _i, [_vp, _vp, _vp, _i, _f, _f, ctypes.c_uint32, _vp, _i, _f, _f, _i, _f, _vp]),
+    ("vpq_sample_hist_workspace_bytes", _sz, [_i]),
+    ("vpq_sample_hist_bf16", _i, [_vp, _vp, _vp, _i, _f, _f, ctypes.c_uint32, _vp, _f, _f, _i, _f, _vp, _i, _vp, _sz]),
     ("vpq_qmv_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
     ("vpq_qmv_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i]),
     ("vpq_qmv_grouped_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
@@ -256,6 +258,32 @@ def sample_topp_bf16(logits, seen, temp, top_p, seed, ws=None, out=None, n_iter=
         out = torch.empty((1,), dtype=torch.int32, device=logits.device)
     _check(load().vpq_sample_topp_bf16(_stream(), _ptr(logits), _ptr(out), V, temp, top_p, seed, _ptr(ws), n_iter, rep, pres,
                                        top_k, min_p, _ptr(seen)), "vpq_sample_topp_bf16")
+    return out
+
+
+def sample_hist_slabs(V):
+    """A slab count for vpq_sample_hist_bf16: about 4096 logits per workgroup, at most 64 workgroups."""
+    return max(1, min(64, (V + 4095) // 4096), (V + 65534) // 65535)
+
+
+def sample_hist_bf16(logits, seen, temp, top_p, seed, ws=None, out=None, work=None, n_slabs=0, rep=1.0, pres=0.0, top_k=0,
+                     min_p=0.0):
+    """As sample_topp_bf16 over n_slabs workgroups with the thresholds read off a histogram of the weights."""
+    import torch
+    V = logits.numel()
+    if n_slabs <= 0:
+        n_slabs = sample_hist_slabs(V)
+    L = load()
+    if ws is None:
+        ws = torch.empty((V,), dtype=torch.bfloat16, device=logits.device)
+    if out is None:
+        out = torch.empty((1,), dtype=torch.int32, device=logits.device)
+    need = int(L.vpq_sample_hist_workspace_bytes(n_slabs))
+    if work is None:
+        work = torch.empty((max(need, 4) // 4,), dtype=torch.float32, device=logits.device)
+    _check(L.vpq_sample_hist_bf16(_stream(), _ptr(logits), _ptr(out), V, temp, top_p, seed, _ptr(ws), rep, pres, top_k, min_p,
+                                  _ptr(seen), n_slabs, _ptr(work), work.numel() * work.element_size()),
+           "vpq_sample_hist_bf16")
     return out
 
 

@@ -896,6 +896,28 @@ int vpq_sample_topp_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* o
                                         n_iter, rep_penalty, presence_penalty, top_k, min_p, seen));
 }
 
+size_t vpq_sample_hist_workspace_bytes(int n_slabs)
+{
+  return n_slabs >= 1 && n_slabs <= 1024 ? vpq::sample_hist_work_words(n_slabs) * sizeof(float) : 0;
+}
+
+int vpq_sample_hist_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, float temp,
+                         float top_p, uint32_t seed, uint16_t* ws, float rep_penalty, float presence_penalty,
+                         int top_k, float min_p, uint8_t* seen, int n_slabs, void* work, size_t work_bytes)
+{
+  if (logits == nullptr || out_id == nullptr || ws == nullptr || seen == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (V < 1 || rep_penalty == 0.0f || n_slabs < 1 || n_slabs > 1024) { return VPQ_ERR_BAD_SHAPE; }
+  // a slab's fixed-point mass of one bin stays below 2^32
+  if (((long long)V + n_slabs - 1) / n_slabs > 65535) { return VPQ_ERR_BAD_SHAPE; }
+  if (work == nullptr || work_bytes < vpq_sample_hist_workspace_bytes(n_slabs)) { return VPQ_ERR_WORKSPACE; }
+  if (!aligned(logits, 2) || !aligned(ws, 2) || !aligned(out_id, 4) || !aligned(work, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_sample_hist(reinterpret_cast<hipStream_t>(stream), logits, out_id, V, temp, top_p, seed, ws,
+                                        rep_penalty, presence_penalty, top_k, min_p, seen, n_slabs,
+                                        static_cast<float*>(work)));
+}
+
 int vpq_qmm_grouped_block_rows(void) { return vpq::kGroupedBlockRows; }
 
 size_t vpq_moe_sort_workspace_bytes(int n_experts)

@@ -216,5 +216,10 @@ hipError_t launch_interleave_rows(hipStream_t st, const void* a, const void* b, 
 hipError_t launch_sample_topp(hipStream_t st, const uint16_t* logits, int32_t* out_id, int V, float temp, float top_p,
                               uint32_t seed, uint16_t* ws, int n_iter, float rep, float pres, int top_k, float min_p,
                               uint8_t* seen);
+// The sampler over n_slabs workgroups with histogram thresholds; work holds sample_hist_work_words(n_slabs) fp32 words.
+size_t sample_hist_work_words(int n_slabs);
+hipError_t launch_sample_hist(hipStream_t st, const uint16_t* logits, int32_t* out_id, int V, float temp, float top_p,
+                              uint32_t seed, uint16_t* ws, float rep, float pres, int top_k, float min_p, uint8_t* seen,
+                              int n_slabs, float* work);
 
 }  // namespace vpq

@@ -208,7 +208,267 @@ __global__ __launch_bounds__(kSampleThreads) void sample_topp_kernel(
   }
 }
 
+// ---- the sampler over many workgroups, thresholds from a histogram ----------------------------------------------
+// (llm_elementwise.metal:3255-3640: `sample_max_partial_f16`, `sample_max_combine_f16`, `sample_zhist_partial_f16`,
+// `sample_zhist_combine_f16`, `sample_thresh_f16`, `sample_pick_partial_f16`, `sample_pick_combine_f16`.)  The
+// vocabulary is cut into n_slabs contiguous slabs, one workgroup of 256 threads each; top-k and top-p become the low
+// edge of a histogram bin (1024 bins uniform in -log w over [0, 40), bin 0 the largest weights), so the kept set is
+// the exact sampler's plus at most one bin's worth of weights.  Five launches instead of the reference's seven: the
+// combine of the maxima is the prologue of the weight pass (every workgroup reduces the n_slabs maxima itself), and
+// the combine of the histograms and the threshold scan are one workgroup.
+//   work (fp32 words): [0, S) slab maxima | S x (2 B + 1): per slab counts, masses, Z | 2 B + 1: their sums |
+//   1: the weight threshold | 2 S: per slab (best score, its index)
+// Exactness as above: a thread takes lo + t, lo + t + 256, ... in ascending order, partial sums meet in a halving
+// tree, slabs are added in slab order; counts and the fixed-point masses of a slab are integer sums.
+constexpr int kHistThreads = 256;
+constexpr int kHistBins = 1024;
+constexpr float kHistBinWidth = 40.0f / 1024.0f;
+
+__device__ __forceinline__ int sample_bin(float w)
+{
+  const float lw = 0.0f - sample_log(w > 1e-30f ? w : 1e-30f);
+  int b = (int)(lw / kHistBinWidth);
+  if (b < 0) { b = 0; }
+  if (b >= kHistBins) { b = kHistBins - 1; }
+  return b;
+}
+
+template <typename T, typename Op>
+__device__ __forceinline__ T tree256(T* a, T mine, Op op)
+{
+  const int t = threadIdx.x;
+  a[t] = mine;
+  __syncthreads();
+  for (int s = kHistThreads >> 1; s > 0; s >>= 1) {
+    if (t < s) { a[t] = op(a[t], a[t + s]); }
+    __syncthreads();
+  }
+  const T r = a[0];
+  __syncthreads();
+  return r;
+}
+
+__global__ __launch_bounds__(kHistThreads) void sample_hist_max_kernel(
+    const uint16_t* __restrict__ logits, float* __restrict__ slab_max, int V, int slab, float rep, float pres,
+    const uint8_t* __restrict__ seen)
+{
+  __shared__ float tg[kHistThreads];
+  const int lo = blockIdx.x * slab;
+  const int hi = lo + slab < V ? lo + slab : V;
+  float m = -INFINITY;
+  for (int i = lo + threadIdx.x; i < hi; i += kHistThreads) {
+    const float e = sample_eff(bf16_bits_to_f32(logits[i]), seen[i] != 0, rep, pres);
+    m = e > m ? e : m;
+  }
+  const float r = tree256(tg, m, [](float a, float b) { return a > b ? a : b; });
+  if (threadIdx.x == 0) { slab_max[blockIdx.x] = r; }
+}
+
+__global__ __launch_bounds__(kHistThreads) void sample_hist_weights_kernel(
+    const uint16_t* __restrict__ logits, uint16_t* __restrict__ ws, const float* __restrict__ slab_max,
+    float* __restrict__ partials, int V, int slab, int n_slabs, float temp, float rep, float pres,
+    const uint8_t* __restrict__ seen)
+{
+  __shared__ float tg[kHistThreads];
+  __shared__ uint32_t h_cnt[kHistBins];
+  __shared__ uint32_t h_mass[kHistBins];
+  const int t = threadIdx.x;
+  auto fmax_op = [](float a, float b) { return a > b ? a : b; };
+  float m = -INFINITY;
+  for (int p = t; p < n_slabs; p += kHistThreads) { m = fmax_op(m, slab_max[p]); }
+  const float maxl = tree256(tg, m, fmax_op);
+  for (int b = t; b < kHistBins; b += kHistThreads) { h_cnt[b] = 0u; h_mass[b] = 0u; }
+  __syncthreads();
+  const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
+  const int lo = blockIdx.x * slab;
+  const int hi = lo + slab < V ? lo + slab : V;
+  float z = 0.0f;
+  for (int i = lo + t; i < hi; i += kHistThreads) {
+    const float e = sample_eff(bf16_bits_to_f32(logits[i]), seen[i] != 0, rep, pres);
+    const float w = sample_exp((e - maxl) * inv_t);
+    ws[i] = (uint16_t)f32_to_bf16_bits(w);
+    z = z + w;
+    const int b = sample_bin(w);
+    atomicAdd(&h_cnt[b], 1u);
+    atomicAdd(&h_mass[b], (uint32_t)(w * 65536.0f));
+  }
+  const float Zs = tree256(tg, z, [](float a, float b) { return a + b; });     // its barriers also close the histogram
+  float* P = partials + (size_t)blockIdx.x * (size_t)(2 * kHistBins + 1);
+  for (int b = t; b < kHistBins; b += kHistThreads) {
+    P[b] = (float)h_cnt[b];
+    P[kHistBins + b] = (float)h_mass[b] * (1.0f / 65536.0f);
+  }
+  if (t == 0) { P[2 * kHistBins] = Zs; }
+}
+
+// One workgroup of 1024 threads: the slabs' histograms and Z added in slab order (a thread owns a cell; its loads
+// are issued sixteen at a time, the additions stay in slab order), then the scan for the two bins where the running
+// count reaches top_k and the running mass reaches top_p Z -- in two levels so that no thread walks more than 32
+// bins at a stretch: 32 chunks of 32 bins are summed by 64 threads, one thread walks the chunk totals and then the
+// bins of the chunk that crosses.  The running sum at a bin is (sum of the chunk totals before its chunk) + (sum of
+// its chunk up to it), every sum taken in ascending order from 0.
+__global__ __launch_bounds__(kSampleThreads) void sample_hist_thresh_kernel(
+    const float* __restrict__ partials, float* __restrict__ hist_out, float* __restrict__ wt_out, int n_slabs, int V,
+    float top_p, int top_k, float min_p)
+{
+  constexpr int kChunk = 32, kChunks = kHistBins / kChunk;
+  __shared__ float hist[2 * kHistBins + 1];
+  __shared__ float chunk_tot[2 * kChunks];          // counts, then masses
+  const int stride = 2 * kHistBins + 1;
+  for (int c = threadIdx.x; c < stride; c += kSampleThreads) {
+    float acc = 0.0f;
+    for (int p0 = 0; p0 < n_slabs; p0 += 16) {
+      float v[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) { v[q] = p0 + q < n_slabs ? partials[(size_t)(p0 + q) * stride + c] : 0.0f; }
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        if (p0 + q < n_slabs) { acc = acc + v[q]; }
+      }
+    }
+    hist[c] = acc;
+    hist_out[c] = acc;
+  }
+  __syncthreads();
+  if (threadIdx.x < 2 * kChunks) {
+    const float* h = hist + threadIdx.x * kChunk;   // chunks of the counts, then of the masses
+    float sum = 0.0f;
+    for (int b = 0; b < kChunk; ++b) { sum = sum + h[b]; }
+    chunk_tot[threadIdx.x] = sum;
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) { return; }
+  const float target = top_p * hist[2 * kHistBins];
+  float t_k = 0.0f, t_p = 0.0f, before_cnt = 0.0f, before_mass = 0.0f;
+  bool have_k = false, have_p = false;
+  const bool do_k = top_k > 0 && top_k < V;
+  for (int j = 0; j < kChunks; ++j) {
+    if (do_k && !have_k && before_cnt + chunk_tot[j] >= (float)top_k) {
+      float in_chunk = 0.0f;
+      for (int b = j * kChunk; b < (j + 1) * kChunk; ++b) {
+        in_chunk = in_chunk + hist[b];
+        if (before_cnt + in_chunk >= (float)top_k) { t_k = sample_exp(0.0f - (float)(b + 1) * kHistBinWidth); break; }
+      }
+      have_k = true;
+    }
+    if (!have_p && before_mass + chunk_tot[kChunks + j] >= target) {
+      float in_chunk = 0.0f;
+      for (int b = j * kChunk; b < (j + 1) * kChunk; ++b) {
+        in_chunk = in_chunk + hist[kHistBins + b];
+        if (before_mass + in_chunk >= target) { t_p = sample_exp(0.0f - (float)(b + 1) * kHistBinWidth); break; }
+      }
+      have_p = true;
+    }
+    if ((!do_k || have_k) && have_p) { break; }
+    before_cnt = before_cnt + chunk_tot[j];
+    before_mass = before_mass + chunk_tot[kChunks + j];
+  }
+  wt_out[0] = fmaxf(fmaxf(t_k, fmaxf(min_p, 0.0f)), t_p);
+}
+
+__global__ __launch_bounds__(kHistThreads) void sample_hist_pick_kernel(
+    const uint16_t* __restrict__ logits, const uint16_t* __restrict__ ws, const float* __restrict__ wt_in,
+    float* __restrict__ pick_score, int32_t* __restrict__ pick_idx, int V, int slab, float temp, uint32_t seed, float rep,
+    float pres, const uint8_t* __restrict__ seen)
+{
+  __shared__ float tg[kHistThreads];
+  __shared__ int tgi[kHistThreads];
+  const int t = threadIdx.x;
+  const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
+  const float wt = wt_in[0];
+  const int lo = blockIdx.x * slab;
+  const int hi = lo + slab < V ? lo + slab : V;
+  float best = -INFINITY;
+  int bi = -1;
+  for (int i = lo + t; i < hi; i += kHistThreads) {
+    if (bf16_bits_to_f32(ws[i]) >= wt) {
+      const float e = sample_eff(bf16_bits_to_f32(logits[i]), seen[i] != 0, rep, pres);
+      const float u = sample_hash_u01(seed ^ ((uint32_t)i * 2654435761u + 1u));
+      const float a = 0.0f - sample_log(u + 1e-20f) + 1e-20f;
+      const float g = 0.0f - sample_log(a);
+      const float score = e * inv_t + g;
+      if (score > best) { best = score; bi = i; }
+    }
+  }
+  tg[t] = best;
+  tgi[t] = bi;
+  __syncthreads();
+  for (int s = kHistThreads >> 1; s > 0; s >>= 1) {
+    if (t < s) {
+      const bool take = tg[t + s] > tg[t] || (tg[t + s] == tg[t] && tgi[t + s] >= 0 && (tgi[t] < 0 || tgi[t + s] < tgi[t]));
+      if (take) { tg[t] = tg[t + s]; tgi[t] = tgi[t + s]; }
+    }
+    __syncthreads();
+  }
+  if (t == 0) { pick_score[blockIdx.x] = tg[0]; pick_idx[blockIdx.x] = tgi[0]; }
+}
+
+__global__ __launch_bounds__(kHistThreads) void sample_hist_pick_combine_kernel(
+    const float* __restrict__ pick_score, const int32_t* __restrict__ pick_idx, int n_slabs, int32_t* __restrict__ out_id,
+    uint8_t* __restrict__ seen)
+{
+  __shared__ float tg[kHistThreads];
+  __shared__ int tgi[kHistThreads];
+  const int t = threadIdx.x;
+  float best = -INFINITY;
+  int bi = -1;
+  for (int p = t; p < n_slabs; p += kHistThreads) {
+    const float sc = pick_score[p];
+    const int id = pick_idx[p];
+    if (id < 0) { continue; }
+    if (sc > best || (sc == best && (bi < 0 || id < bi))) { best = sc; bi = id; }
+  }
+  tg[t] = best;
+  tgi[t] = bi;
+  __syncthreads();
+  for (int s = kHistThreads >> 1; s > 0; s >>= 1) {
+    if (t < s) {
+      const bool take = tgi[t + s] >= 0 && (tgi[t] < 0 || tg[t + s] > tg[t] || (tg[t + s] == tg[t] && tgi[t + s] < tgi[t]));
+      if (take) { tg[t] = tg[t + s]; tgi[t] = tgi[t + s]; }
+    }
+    __syncthreads();
+  }
+  if (t == 0) {
+    const int pick = tgi[0] >= 0 ? tgi[0] : 0;
+    out_id[0] = pick;
+    seen[pick] = 1;
+  }
+}
+
 }  // namespace
+
+size_t sample_hist_work_words(int n_slabs)
+{
+  return (size_t)n_slabs + (size_t)n_slabs * (2 * kHistBins + 1) + (2 * kHistBins + 1) + 1 + 2 * (size_t)n_slabs;
+}
+
+hipError_t launch_sample_hist(hipStream_t st, const uint16_t* logits, int32_t* out_id, int V, float temp, float top_p,
+                              uint32_t seed, uint16_t* ws, float rep, float pres, int top_k, float min_p, uint8_t* seen,
+                              int n_slabs, float* work)
+{
+  const int slab = (V + n_slabs - 1) / n_slabs;
+  float* slab_max = work;
+  float* partials = slab_max + n_slabs;
+  float* hist = partials + (size_t)n_slabs * (2 * kHistBins + 1);
+  float* wt = hist + (2 * kHistBins + 1);
+  float* pick_score = wt + 1;
+  int32_t* pick_idx = reinterpret_cast<int32_t*>(pick_score + n_slabs);
+  const dim3 slabs((unsigned)n_slabs), one(1), block(kHistThreads);
+  hipError_t e = launch_kernel(sample_hist_max_kernel, slabs, block, 0, st, logits, slab_max, V, slab, rep, pres,
+                               (const uint8_t*)seen);
+  if (e != hipSuccess) { return e; }
+  e = launch_kernel(sample_hist_weights_kernel, slabs, block, 0, st, logits, ws, (const float*)slab_max, partials, V, slab,
+                    n_slabs, temp, rep, pres, (const uint8_t*)seen);
+  if (e != hipSuccess) { return e; }
+  e = launch_kernel(sample_hist_thresh_kernel, one, dim3(kSampleThreads), 0, st, (const float*)partials, hist, wt, n_slabs, V,
+                    top_p, top_k, min_p);
+  if (e != hipSuccess) { return e; }
+  e = launch_kernel(sample_hist_pick_kernel, slabs, block, 0, st, logits, (const uint16_t*)ws, (const float*)wt, pick_score,
+                    pick_idx, V, slab, temp, seed, rep, pres, (const uint8_t*)seen);
+  if (e != hipSuccess) { return e; }
+  return launch_kernel(sample_hist_pick_combine_kernel, one, block, 0, st, (const float*)pick_score,
+                       (const int32_t*)pick_idx, n_slabs, out_id, seen);
+}
 
 hipError_t launch_sample_topp(hipStream_t st, const uint16_t* logits, int32_t* out_id, int V, float temp, float top_p,
                               uint32_t seed, uint16_t* ws, int n_iter, float rep, float pres, int top_k, float min_p,
