@@ -659,6 +659,12 @@ int vpq_qmv_gated_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16
 int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                       const uint16_t* biases, const uint16_t* x, uint16_t* y,
                       int K, int N, int M, int activation);
+/* The grouped launch on binary16 elements (`affine_qmv_qkv_w4g64` of the half build, affine_qmv.metal:497-516):
+ * arguments and results as vpq_qmv_group_w4g64_bf16 -- bit-identical to `count` calls of vpq_qmv_w4g64_f16; one
+ * launch at M = 1 on K % 512 == 0, K >= 2048 with 16-byte aligned scales / biases, separate calls otherwise. */
+int vpq_qmv_group_w4g64_f16(vpq_stream_t stream, int count, const uint32_t* const* w,
+                            const uint16_t* const* scales, const uint16_t* const* biases,
+                            const uint16_t* x, uint16_t* const* y, int K, const int* N, int M);
 int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                   const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                   int K, int N, int M, uint16_t* w_deq, int expand);
@@ -713,7 +719,7 @@ int vpq_sample_topp_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* o
  * `work`: vpq_sample_hist_workspace_bytes(n_slabs) bytes of device scratch
  * (slab maxima, per-slab histograms, their sum, the threshold, per-slab
  * picks), 4-byte aligned; nothing in it needs to be cleared.
- * Requires V >= 1, rep != 0, 1 <= n_slabs <= 1024, ceil(V / n_slabs) <= 65535
+ * Requires 1 <= V <= 2^24, rep != 0, 1 <= n_slabs <= 1024, ceil(V / n_slabs) <= 65535
  * (the per-slab fixed-point masses); other requirements as above. */
 size_t vpq_sample_hist_workspace_bytes(int n_slabs);
 int vpq_sample_hist_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* out_id, int V, float temp,

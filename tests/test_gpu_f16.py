@@ -106,6 +106,29 @@ def test_qmv_f16_one_row_streaming_kernel(vpq, oracle, dev, D, K, N):
     check_f16(bits16(vpq.qmv_w4g64_f16(wd, so, bd, xd, K, N, M)), y64)
 
 
+@pytest.mark.parametrize("K,rows,M", [(2048, (64, 16, 16), 1), (4096, (520, 136), 1), (4096, (96, 40, 40, 8), 1), (1024, (48, 16, 16), 1),
+                                      (2048, (64, 16), 3)])
+def test_qmv_f16_grouped_launch(vpq, oracle, dev, D, K, rows, M):
+    """Several packs sharing x (q|k|v, gate|up) on binary16 elements: each output has the bits of its own
+    vpq_qmv_w4g64_f16 call (one launch where the streaming kernel takes the shape, separate calls otherwise)."""
+    x = np.random.default_rng(801 + K).standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    xd = dev16(x, dev)
+    packs, singles = [], []
+    for i, n in enumerate(rows):
+        w, s, b = f16_pack(n, K, 810 + 7 * i + K)
+        wd, sd, bd = D.u32(w, dev), dev16(s, dev), dev16(b, dev)
+        packs.append((wd, sd, bd, n))
+        singles.append(vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, n, M))
+        y64, _ = oracle.matmul_f16(w, s, b, x, K, n, M, rounded=False)
+        check_f16(bits16(singles[-1]), y64)
+    outs = [parity.Guarded((M, n), torch.float16, dev) for n in rows]
+    vpq.qmv_group_w4g64_f16(packs, xd, K, M, outs=[o.view for o in outs])
+    torch.cuda.synchronize()
+    for o, single in zip(outs, singles):
+        o.assert_intact()
+        assert torch.equal(o.view, single)
+
+
 @pytest.mark.parametrize("M,N,K", [(64, 64, 64), (130, 320, 256), (257, 129, 512)])
 def test_qmm_f16_dense_route(vpq, oracle, dev, D, M, N, K):
     w, s, b = f16_pack(N, K, 500 + M)

@@ -789,6 +789,19 @@ def test_binary16_library_names(vpq, enc, oracle, dev, D):
     assert np.array_equal(dense.view(torch.int16).cpu().numpy().view(np.uint16), oracle.dequant_f16(w, s, b, K, N))
     assert torch.equal(y, vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, 1))
     assert enc.set_function("affine_qmv", "affine_qmm_steel_w4g64") == 0       # not in that library
+    # the fused q|k|v GEMV of the binary16 build (slots 4..6 the three outputs, 7:K 8..10 the row counts)
+    rows = (24, 16, 8)
+    qo, ko, vo = (torch.zeros((1, r), dtype=torch.float16, device=dev) for r in rows)
+    assert enc.set_function("affine_qmv", "affine_qmv_qkv_w4g64") == 1
+    for i, t in enumerate((wd, sd, bd, xd, qo, ko, vo)):
+        enc.set_buffer(i, t)
+    enc.set_constant(7, K)
+    for i, r in enumerate(rows):
+        enc.set_constant(8 + i, r)
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert torch.equal(torch.cat((qo, ko, vo), dim=1), y)
     # the fused GEMM of the binary16 build, plain and gated, under its function names (slot 7 = M)
     M = 70
     xm = as16(np.random.default_rng(79).standard_normal((M, K)).astype(np.float16).view(np.uint16))

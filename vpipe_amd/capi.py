@@ -64,6 +64,7 @@ SYMBOLS = [
     ("vpq_lora_a_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f]),
     ("vpq_linear_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz]),
     ("vpq_qmv_group_w4g64_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
+    ("vpq_qmv_group_w4g64_f16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
     ("vpq_interleave_rows", _i, [_vp, _vp, _vp, _vp, _sz, _sz]),
     ("vpq_qmv_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmv_swiglu_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
@@ -740,7 +741,8 @@ class QmvGroup:
     """The pointer tables of a grouped launch, built once for a fixed set of tensors so that a
     launch costs one foreign call (a decode loop launches the same groups every token)."""
 
-    def __init__(self, packs, x, K, M, outs):
+    def __init__(self, packs, x, K, M, outs, f16=False):
+        self.entry = "vpq_qmv_group_w4g64_f16" if f16 else "vpq_qmv_group_w4g64_bf16"
         n = len(packs)
         PA = ctypes.c_void_p * n
         self.keep = (packs, x, outs)       # the tables hold raw pointers: keep the tensors alive
@@ -754,8 +756,8 @@ class QmvGroup:
         self.outs = outs
 
     def launch(self):
-        _check(load().vpq_qmv_group_w4g64_bf16(_stream(), self.n, self.w, self.s, self.b, self.x, self.y, self.K,
-                                               self.N, self.M), "vpq_qmv_group_w4g64_bf16")
+        _check(getattr(load(), self.entry)(_stream(), self.n, self.w, self.s, self.b, self.x, self.y, self.K,
+                                           self.N, self.M), self.entry)
         return self.outs
 
 
@@ -765,6 +767,14 @@ def qmv_group_w4g64(packs, x, K, M, outs=None):
     if outs is None:
         outs = [torch.empty((M, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
     return QmvGroup(packs, x, K, M, outs).launch()
+
+
+def qmv_group_w4g64_f16(packs, x, K, M, outs=None):
+    """As qmv_group_w4g64 on IEEE binary16 elements."""
+    import torch
+    if outs is None:
+        outs = [torch.empty((M, p[3]), dtype=torch.float16, device=x.device) for p in packs]
+    return QmvGroup(packs, x, K, M, outs, f16=True).launch()
 
 
 def quantize_w4g64(src, K, N, clip=1.0):

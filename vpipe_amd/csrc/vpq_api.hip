@@ -906,7 +906,8 @@ int vpq_sample_hist_bf16(vpq_stream_t stream, const uint16_t* logits, int32_t* o
                          int top_k, float min_p, uint8_t* seen, int n_slabs, void* work, size_t work_bytes)
 {
   if (logits == nullptr || out_id == nullptr || ws == nullptr || seen == nullptr) { return VPQ_ERR_NULL_POINTER; }
-  if (V < 1 || rep_penalty == 0.0f || n_slabs < 1 || n_slabs > 1024) { return VPQ_ERR_BAD_SHAPE; }
+  // counts travel as fp32: exact up to 2^24 logits
+  if (V < 1 || V > (1 << 24) || rep_penalty == 0.0f || n_slabs < 1 || n_slabs > 1024) { return VPQ_ERR_BAD_SHAPE; }
   // a slab's fixed-point mass of one bin stays below 2^32
   if (((long long)V + n_slabs - 1) / n_slabs > 65535) { return VPQ_ERR_BAD_SHAPE; }
   if (work == nullptr || work_bytes < vpq_sample_hist_workspace_bytes(n_slabs)) { return VPQ_ERR_WORKSPACE; }
@@ -1383,6 +1384,40 @@ int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* con
   }
   if (!mfma_group) { return finish(vpq::launch_qmv_rows_group(reinterpret_cast<hipStream_t>(stream), a, g)); }
   return finish(vpq::launch_qmv_mfma_group(reinterpret_cast<hipStream_t>(stream), a, g));
+}
+
+int vpq_qmv_group_w4g64_f16(vpq_stream_t stream, int count, const uint32_t* const* w,
+                            const uint16_t* const* scales, const uint16_t* const* biases,
+                            const uint16_t* x, uint16_t* const* y, int K, const int* N, int M)
+{
+  if (w == nullptr || scales == nullptr || biases == nullptr || y == nullptr || N == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (count < 1 || count > 4) { return VPQ_ERR_BAD_SHAPE; }
+  bool one_launch = vpq::qmv_flow_supports(K, 1, M);
+  for (int i = 0; i < count; ++i) {
+    int st = check_pack(w[i], scales[i], biases[i], K, N[i]);
+    if (st != VPQ_OK) { return st; }
+    if (y[i] == nullptr) { return VPQ_ERR_NULL_POINTER; }
+    if (!aligned(y[i], 2)) { return VPQ_ERR_MISALIGNED; }
+    one_launch = one_launch && aligned(scales[i], 16) && aligned(biases[i], 16);
+  }
+  if (x == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16)) { return VPQ_ERR_MISALIGNED; }
+  if (!one_launch) {
+    for (int i = 0; i < count; ++i) {
+      const int st = vpq_qmv_w4g64_f16(stream, w[i], scales[i], biases[i], x, y[i], K, N[i], M, nullptr);
+      if (st != VPQ_OK) { return st; }
+    }
+    return VPQ_OK;
+  }
+  int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.x = x; a.K = K; a.M = M; a.y_f32 = false; a.cu_count = g_dev.cu_count;
+  vpq::QmvGroup g;
+  g.count = count;
+  for (int i = 0; i < count; ++i) { g.seg[i] = vpq::QmvSeg{w[i], scales[i], biases[i], y[i], N[i]}; }
+  return finish(vpq::launch_qmv_flow_group(reinterpret_cast<hipStream_t>(stream), a, g, true));
 }
 
 int vpq_quantize_w4g64(vpq_stream_t stream, const uint16_t* src, uint32_t* w, uint16_t* scales_f16,

@@ -134,7 +134,7 @@ size_t qmv_mfma_workspace_bytes(int K, int N, int M);
 bool qmv_flow_supports(int K, int N, int M);
 hipError_t launch_qmv_flow(hipStream_t st, const QmvArgs& a);
 hipError_t launch_qmv_flow_f16(hipStream_t st, const QmvArgs& a);    // IEEE binary16 elements
-hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g);
+hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g, bool f16 = false);
 bool qmv_stream_supports(int K, int N, int M);
 hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);
 bool qmv_ring_supports(int K, int N, int M);

@@ -477,18 +477,18 @@ hipError_t dispatch_flow(const FlowPlan& pl, bool y_f32, const FlowHead& h, cons
   }
   const dim3 grid((unsigned)blocks);
   if (f16) {
-    // binary16 elements: single packs, x shared through LDS
-    if constexpr (C == 1) {
-      if (pl.xm != kXShared) { return hipErrorInvalidValue; }
+    // binary16 elements: x shared through LDS; grouped launches store the element type
+    if (pl.xm != kXShared || (C > 1 && y_f32)) { return hipErrorInvalidValue; }
 #define VPQ_FLOW16(S, R)                                                                                        \
   if (pl.spw == S && pl.rb == R) {                                                                              \
-    return y_f32 ? launch_flow_kernel<S, R, true, kXShared, 1, true>(grid, block, lds_bytes, st, p)        \
-                 : launch_flow_kernel<S, R, false, kXShared, 1, true>(grid, block, lds_bytes, st, p);      \
+    if constexpr (C == 1) {                                                                                     \
+      if (y_f32) { return launch_flow_kernel<S, R, true, kXShared, 1, true>(grid, block, lds_bytes, st, p); }   \
+    }                                                                                                           \
+    return launch_flow_kernel<S, R, false, kXShared, C, true>(grid, block, lds_bytes, st, p);                   \
   }
-      VPQ_FLOW16(1, 2) VPQ_FLOW16(2, 2) VPQ_FLOW16(3, 2) VPQ_FLOW16(4, 2) VPQ_FLOW16(5, 2) VPQ_FLOW16(6, 2)
-      VPQ_FLOW16(1, 4) VPQ_FLOW16(2, 4) VPQ_FLOW16(3, 4) VPQ_FLOW16(4, 4)
+    VPQ_FLOW16(1, 2) VPQ_FLOW16(2, 2) VPQ_FLOW16(3, 2) VPQ_FLOW16(4, 2) VPQ_FLOW16(5, 2) VPQ_FLOW16(6, 2)
+    VPQ_FLOW16(1, 4) VPQ_FLOW16(2, 4) VPQ_FLOW16(3, 4) VPQ_FLOW16(4, 4)
 #undef VPQ_FLOW16
-    }
     return hipErrorInvalidValue;
   }
 #define VPQ_FLOW(S, R)                                                                                          \
@@ -566,7 +566,7 @@ hipError_t launch_qmv_flow_planned(hipStream_t st, const QmvArgs& a, int spw, in
   return launch_flow(st, &seg, 1, a, 0.0, &pl);
 }
 
-hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g)
+hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g, bool f16)
 {
   FlowSeg segs[4];
   double bytes = 0.0;
@@ -577,7 +577,7 @@ hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGrou
   QmvArgs b = a;
   b.residual = nullptr;
   b.gate_act = 0;
-  return launch_flow(st, segs, g.count, b, bytes, nullptr);
+  return launch_flow(st, segs, g.count, b, bytes, nullptr, f16);
 }
 
 }  // namespace vpq

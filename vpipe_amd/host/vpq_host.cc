@@ -139,6 +139,7 @@ const FnEntry kFunctions[] = {
     {"affine_qmv", "affine_qmv_w4g64_add", QuantKernel::QmvAdd, QuantFormat::W4G64F16},
     {"affine_qmv", "affine_qmv_swiglu_w4g64", QuantKernel::QmvSwiglu, QuantFormat::W4G64F16},
     {"affine_qmv", "affine_qmv_geglu_w4g64", QuantKernel::QmvGeglu, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_qkv_w4g64", QuantKernel::QmvQkv, QuantFormat::W4G64F16},
     {"affine_qmm_steel", "affine_qmm_steel_w4g64", QuantKernel::Qmm, QuantFormat::W4G64F16},
     {"affine_qmm_steel", "affine_qmm_steel_w4g64_bm64", QuantKernel::Qmm, QuantFormat::W4G64F16},
     {"affine_qmm_steel", "affine_qmm_steel_w4g64_bm128", QuantKernel::Qmm, QuantFormat::W4G64F16},
@@ -412,7 +413,7 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
   int status = VPQ_OK;
   const QuantKernel kind = _fn.kind();
   const QuantFormat fmt = _fn.format();
-  if (fmt != QuantFormat::W4G64) {
+  if (fmt != QuantFormat::W4G64 && kind != QuantKernel::QmvQkv) {
     // The 8-bit and group-32 twins keep the slot layout of the 4-bit group-64 functions:
     // dequant 0:w 1:scales 2:biases 3:w_deq 4:K 5:N; QMV 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N [7:residual],
     // rows from grid.x.  The Q4_0 forms ignore slot 2.
@@ -630,8 +631,10 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
         bi[i] = static_cast<const uint16_t*>(buf(2)) + r0 * (size_t)(K / 64);
         r0 += (size_t)rows[i];
       }
-      status = vpq_qmv_group_w4g64_bf16(st, rows[2] > 0 ? 3 : 2, w, sc, bi, static_cast<const uint16_t*>(buf(3)), y, K,
-                                        rows, 1);
+      status = fmt == QuantFormat::W4G64F16
+                   ? vpq_qmv_group_w4g64_f16(st, rows[2] > 0 ? 3 : 2, w, sc, bi, static_cast<const uint16_t*>(buf(3)), y, K, rows, 1)
+                   : vpq_qmv_group_w4g64_bf16(st, rows[2] > 0 ? 3 : 2, w, sc, bi, static_cast<const uint16_t*>(buf(3)), y, K, rows,
+                                              1);
     }
   } else {
     // slots 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N, 7: residual | m_total | M
