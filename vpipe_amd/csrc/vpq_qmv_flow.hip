@@ -508,9 +508,9 @@ hipError_t dispatch_flow(const FlowPlan& pl, bool y_f32, const FlowHead& h, cons
 
 // segs[0 .. count): the packs; count == 1 takes the one-line argument form.
 hipError_t launch_flow(hipStream_t st, const FlowSeg* segs, int count, const QmvArgs& a, double pack_bytes,
-                       const FlowPlan* forced, bool f16 = false)
+                       bool f16 = false)
 {
-  const FlowPlan pl = forced != nullptr ? *forced : flow_plan(a.K, pack_bytes);
+  const FlowPlan pl = flow_plan(a.K, pack_bytes);
   if (pl.spw == 0 || pl.wk < 1 || pl.wk > 4 || pl.wr < 1 || pl.wk * pl.wr > kMaxWavesPerWg ||
       pl.wk * pl.spw * kSlice < a.K || (pl.xm != kXOwn && pl.xm != kXShared)) {
     return hipErrorInvalidValue;
@@ -547,23 +547,14 @@ bool qmv_flow_supports(int K, int N, int M)
 hipError_t launch_qmv_flow(hipStream_t st, const QmvArgs& a)
 {
   const FlowSeg seg{a.w, a.scales, a.biases, a.y, a.N};
-  return launch_flow(st, &seg, 1, a, (double)a.N * (double)a.K * 9.0 / 16.0, nullptr);
+  return launch_flow(st, &seg, 1, a, (double)a.N * (double)a.K * 9.0 / 16.0);
 }
 
 // The same kernel over IEEE binary16 elements (x, scales, biases, y, residual).
 hipError_t launch_qmv_flow_f16(hipStream_t st, const QmvArgs& a)
 {
   const FlowSeg seg{a.w, a.scales, a.biases, a.y, a.N};
-  return launch_flow(st, &seg, 1, a, (double)a.N * (double)a.K * 9.0 / 16.0, nullptr, true);
-}
-
-// Measurement only: the single-pack launch with the plan given (slices per wavefront, K parts, row sets per
-// workgroup, rows per wavefront, x mode).
-hipError_t launch_qmv_flow_planned(hipStream_t st, const QmvArgs& a, int spw, int wk, int wr, int rb, int xm)
-{
-  const FlowSeg seg{a.w, a.scales, a.biases, a.y, a.N};
-  const FlowPlan pl{spw, wk, wr, rb, xm};
-  return launch_flow(st, &seg, 1, a, 0.0, &pl);
+  return launch_flow(st, &seg, 1, a, (double)a.N * (double)a.K * 9.0 / 16.0, true);
 }
 
 hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g, bool f16)
@@ -577,7 +568,7 @@ hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGrou
   QmvArgs b = a;
   b.residual = nullptr;
   b.gate_act = 0;
-  return launch_flow(st, segs, g.count, b, bytes, nullptr, f16);
+  return launch_flow(st, segs, g.count, b, bytes, f16);
 }
 
 }  // namespace vpq
