@@ -386,6 +386,12 @@ int vpq_qmv_grouped_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, con
 int vpq_qmv_grouped_down_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                     const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int npad,
                                     const int32_t* tile2e, const int32_t* srow, int n_experts);
+/* Rows of the sorted down projection back to pair order: replaces `moe_scatter_back_f16`
+ * (gpu-kernels/metal/ops/llm_elementwise.metal:328-342; slots 0:dsorted[npad,H] 1:sdst[npad] 2:partials[npair,H] 3:H):
+ * partials[sdst[s], :] = dsorted[s, :] for every slot with 0 <= sdst[s] < npair (padding slots are skipped; the
+ * reference does not check the upper bound).  A copy of 2-byte elements: serves both element types. */
+int vpq_moe_scatter_back_bf16(vpq_stream_t stream, const uint16_t* dsorted, const int32_t* sdst,
+                              uint16_t* partials, int npad, int H, int npair);
 /* The same over a batched 8-bit pack [E, N, K/4]: `affine_grouped_swiglu_w8g64`, `affine_grouped_down_w8g64`
  * (affine_qmv.metal:2718-2719).  A live slot is bit-identical to the pair-gathered 8-bit call
  * (vpq_gather_qmv_gated_w8g64_bf16 / vpq_gather_down_qmv_w8g64_bf16) of that expert on that row. */

@@ -250,6 +250,43 @@ def test_sorted_expert_gemv_two_slots_per_tile(vpq, oracle, dev, D, K, inner, H,
         assert np.array_equal(gotd[s], D.bits(plain)[0]), "slot %d" % s
 
 
+@pytest.mark.parametrize("H", [64, 100, 2048])
+def test_scatter_back_to_pair_order(vpq, dev, D, H):
+    """llm_elementwise.metal:328-342: rows in slot order go to the pair each slot names; padding slots and names
+    outside [0, npair) write nothing; rows no slot names keep what they held."""
+    E, T, top_k, B = 6, 11, 2, capi.VPQ_QMV_GROUPED_SLOTS
+    eid = np.random.default_rng(6600 + H).integers(0, E, size=T * top_k, dtype=np.int32)
+    eid[3] = -1                                            # a pair without a slot
+    _, _, sdst_d, _ = vpq.moe_sort_pairs(torch.from_numpy(eid).to(dev), top_k, E, block_rows=B)
+    sdst = sdst_d.cpu().numpy()
+    npad, npair = sdst.size, eid.size
+    rows = synth.make_act(npad, H, 6601 + H)
+    rows_d = D.bf16(rows, dev)
+    out = parity.Guarded((npair, H), torch.bfloat16, dev)
+    out.view.fill_(7.0)
+    vpq.moe_scatter_back(rows_d, sdst_d, npair, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    seven = D.bits(torch.full((1,), 7.0, dtype=torch.bfloat16))[0]
+    want = np.full((npair, H), seven, dtype=np.uint16)
+    for s_, p_ in enumerate(sdst):
+        if p_ >= 0:
+            want[p_] = rows[s_]
+    assert np.array_equal(D.bits(out.view), want)
+    assert (want[3] == seven).all() and (want[eid >= 0] != seven).any()
+    # a name past the pairs is skipped, not followed
+    bad = sdst.copy()
+    bad[np.nonzero(bad >= 0)[0][0]] = npair + 5
+    out.view.fill_(7.0)
+    vpq.moe_scatter_back(rows_d, torch.from_numpy(bad).to(dev), npair, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    L = vpq.load()
+    p = rows_d.data_ptr()
+    assert L.vpq_moe_scatter_back_bf16(None, p, sdst_d.data_ptr(), None, npad, H, npair) == -1
+    assert L.vpq_moe_scatter_back_bf16(None, p, sdst_d.data_ptr(), p, 0, H, npair) == -2
+
+
 def test_sorted_expert_gemv_rejects_bad_arguments(vpq, dev):
     L = vpq.load()
     buf = torch.zeros(1 << 16, dtype=torch.int32, device=dev)

@@ -51,6 +51,7 @@ SYMBOLS = [
     ("vpq_sample_hist_bf16", _i, [_vp, _vp, _vp, _i, _f, _f, ctypes.c_uint32, _vp, _f, _f, _i, _f, _vp, _i, _vp, _sz]),
     ("vpq_qmv_grouped_gated_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
     ("vpq_qmv_grouped_down_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i]),
+    ("vpq_moe_scatter_back_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     ("vpq_qmv_grouped_gated_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i]),
     ("vpq_qmv_grouped_down_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i]),
     ("vpq_qmv_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, _i]),
@@ -389,6 +390,17 @@ def qmv_grouped_down_w4g64(w, scales, biases, x, K, N, tile2e, srow, n_experts, 
     name = "vpq_qmv_grouped_down_w%dg64_bf16" % bits
     _check(getattr(load(), name)(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
                                  npad, _ptr(tile2e), _ptr(srow), n_experts), name)
+    return out
+
+
+def moe_scatter_back(dsorted, sdst, npair, out=None):
+    """Sorted rows [npad, H] -> pair order [npair, H] (rows no slot points at are left as they are)."""
+    import torch
+    npad, H = dsorted.shape
+    if out is None:
+        out = torch.zeros((npair, H), dtype=dsorted.dtype, device=dsorted.device)
+    _check(load().vpq_moe_scatter_back_bf16(_stream(), _ptr(dsorted), _ptr(sdst), _ptr(out), npad, H, npair),
+           "vpq_moe_scatter_back_bf16")
     return out
 
 

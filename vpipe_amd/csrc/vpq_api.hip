@@ -950,6 +950,19 @@ int vpq_moe_sort_pairs(vpq_stream_t stream, const int32_t* pair_eid, int npair, 
                                      block_rows, max_tiles, tile2e, srow, sdst, ntiles, static_cast<int*>(ws)));
 }
 
+int vpq_moe_scatter_back_bf16(vpq_stream_t stream, const uint16_t* dsorted, const int32_t* sdst, uint16_t* partials,
+                              int npad, int H, int npair)
+{
+  if (dsorted == nullptr || sdst == nullptr || partials == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (npad < 1 || H < 1 || npair < 1 || (long long)npad * (long long)H > 0x3fffffffffLL) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(dsorted, 2) || !aligned(partials, 2) || !aligned(sdst, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  const bool wide = (H % 8) == 0 && aligned(dsorted, 16) && aligned(partials, 16);
+  return finish(vpq::launch_moe_scatter_back(reinterpret_cast<hipStream_t>(stream), dsorted, sdst, partials, npad, H, npair,
+                                             wide));
+}
+
 namespace {
 
 int grouped_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,

@@ -177,6 +177,8 @@ struct GroupedArgs {
   const int* sdst;     // [a.M] or nullptr: y row per slot
   int n_experts, rows_x, rows_y;
 };
+hipError_t launch_moe_scatter_back(hipStream_t st, const uint16_t* dsorted, const int* sdst, uint16_t* partials, int npad,
+                                   int H, int n_pairs, bool wide);
 hipError_t launch_moe_sort(hipStream_t st, const int* pair_eid, int n_pairs, int top_k, int n_experts, int block_rows,
                            int max_tiles, int* tile2e, int* srow, int* sdst, int* ntiles, int* ws);
 hipError_t launch_qmm_grouped(hipStream_t st, const GemmArgs& a, const GroupedArgs& g);

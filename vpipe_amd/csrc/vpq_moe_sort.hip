@@ -137,7 +137,36 @@ __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const int* __rest
   }
 }
 
+// `moe_scatter_back_f16` (gpu-kernels/metal/ops/llm_elementwise.metal:328-342): rows of the sorted down
+// projection back to pair order, partials[sdst[slot]] = dsorted[slot]; padding slots (sdst < 0) and destinations
+// outside [0, n_pairs) are skipped.  16 bytes per thread where the rows allow, else 2.
+template <typename V>
+__global__ __launch_bounds__(256) void moe_scatter_back_kernel(const V* __restrict__ dsorted, const int* __restrict__ sdst,
+                                                              V* __restrict__ partials, int npad, int row_vecs, int n_pairs)
+{
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (size_t)npad * (size_t)row_vecs) { return; }
+  const int slot = (int)(i / (size_t)row_vecs);
+  const int v = (int)(i - (size_t)slot * (size_t)row_vecs);
+  const int p = sdst[slot];
+  if (p < 0 || p >= n_pairs) { return; }
+  partials[(size_t)p * row_vecs + v] = dsorted[(size_t)slot * row_vecs + v];
+}
+
 }  // namespace
+
+hipError_t launch_moe_scatter_back(hipStream_t st, const uint16_t* dsorted, const int* sdst, uint16_t* partials, int npad,
+                                   int H, int n_pairs, bool wide)
+{
+  if (wide) {
+    const size_t n = (size_t)npad * (size_t)(H / 8);
+    return launch_kernel(moe_scatter_back_kernel<uint4>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                         reinterpret_cast<const uint4*>(dsorted), sdst, reinterpret_cast<uint4*>(partials), npad, H / 8, n_pairs);
+  }
+  const size_t n = (size_t)npad * (size_t)H;
+  return launch_kernel(moe_scatter_back_kernel<uint16_t>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, dsorted, sdst,
+                       partials, npad, H, n_pairs);
+}
 
 hipError_t launch_moe_sort(hipStream_t st, const int* pair_eid, int n_pairs, int top_k, int n_experts, int block_rows,
                            int max_tiles, int* tile2e, int* srow, int* sdst, int* ntiles, int* ws)
