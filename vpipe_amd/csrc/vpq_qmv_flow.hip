@@ -173,8 +173,10 @@ constexpr int kXOwn = 0, kXShared = 1;
 // F16: the elements (x, scales, biases, y, residual) are IEEE binary16 instead of bf16 (the reference's
 // VPIPE_ELT = half build).  The codes then become binary16 pairs 16 + q (the code shifted to mantissa bits 6..9,
 // exact; 1024 + q with the code left in bits 0..3 would cost eight times bf16's cancellation noise).
-template <int SPW, int RB, bool F32OUT, int XM, int C, bool F16 = false>
-__global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const FlowParams<C> p)
+// PRELOADED: the arguments are already in scalar registers (nothing to batch; the residual is left to be loaded
+// when the store needs it).
+template <int SPW, int RB, bool F32OUT, int XM, int C, bool F16 = false, bool PRELOADED = false>
+__device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
 {
   constexpr int NL = RB * SPW;                 // code loads of a wavefront
   constexpr int PPR = SPW * 4;                 // 16-byte pieces of scales (or biases) per row and K part
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
   const uint16_t* residual = p.h.residual;
   const int K = p.h.K;
   const uint32_t shape = p.h.shape;
-  pin_scalar(xg); pin_scalar(residual); pin_scalar(K); pin_scalar(shape);
+  if constexpr (!PRELOADED) { pin_scalar(xg); pin_scalar(residual); pin_scalar(K); pin_scalar(shape); }
   const int blk = (int)blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -197,15 +199,32 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
 #pragma unroll
   for (int i = 0; i < C; ++i) {
     w_[i] = p.w[i]; s_[i] = p.scales[i]; b_[i] = p.biases[i]; y_[i] = p.y[i]; n_[i] = p.N[i]; fb_[i] = p.first_block[i];
-    pin_scalar(w_[i]); pin_scalar(s_[i]); pin_scalar(b_[i]); pin_scalar(y_[i]); pin_scalar(n_[i]); pin_scalar(fb_[i]);
+    if constexpr (!PRELOADED) {
+      pin_scalar(w_[i]); pin_scalar(s_[i]); pin_scalar(b_[i]); pin_scalar(y_[i]); pin_scalar(n_[i]); pin_scalar(fb_[i]);
+    }
   }
   const uint32_t* wq = w_[0]; const uint16_t* sq = s_[0]; const uint16_t* bq = b_[0]; void* yq = y_[0];
   int N = n_[0], first_block = 0;
+  if constexpr (PRELOADED && C > 1) {
+    // The first pack's arguments are in registers already, the others' are still on their way from the argument
+    // buffer: a branch, so that the workgroups of the first pack (which come first) do not wait for them.
+    if (blk >= fb_[1]) {
+      wq = w_[1]; sq = s_[1]; bq = b_[1]; yq = y_[1]; N = n_[1]; first_block = fb_[1];
 #pragma unroll
-  for (int i = 1; i < C; ++i) {
-    const bool take = blk >= fb_[i];
-    wq = take ? w_[i] : wq; sq = take ? s_[i] : sq; bq = take ? b_[i] : bq; yq = take ? y_[i] : yq;
-    N = take ? n_[i] : N; first_block = take ? fb_[i] : first_block;
+      for (int i = 2; i < C; ++i) {
+        const bool take = blk >= fb_[i];
+        wq = take ? w_[i] : wq; sq = take ? s_[i] : sq; bq = take ? b_[i] : bq; yq = take ? y_[i] : yq;
+        N = take ? n_[i] : N; first_block = take ? fb_[i] : first_block;
+      }
+      asm volatile("" : "+s"(wq), "+s"(sq), "+s"(bq), "+s"(N), "+s"(first_block));   // keeps this a branch
+    }
+  } else {
+#pragma unroll
+    for (int i = 1; i < C; ++i) {
+      const bool take = blk >= fb_[i];
+      wq = take ? w_[i] : wq; sq = take ? s_[i] : sq; bq = take ? b_[i] : bq; yq = take ? y_[i] : yq;
+      N = take ? n_[i] : N; first_block = take ? fb_[i] : first_block;
+    }
   }
   const int wk = (int)((shape >> 24) & 3u) + 1, wr = (int)((shape >> 26) & 7u) + 1, gate_act = (int)((shape >> 29) & 3u);
 
@@ -423,6 +442,59 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const Flo
   }
 }
 
+template <int SPW, int RB, bool F32OUT, int XM, int C, bool F16 = false>
+__global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const FlowParams<C> p)
+{
+  qmv_flow_body<SPW, RB, F32OUT, XM, C, F16>(p);
+}
+
+// The single-pack form with its sixteen argument words as separate kernel arguments: this file is compiled with
+// kernel-argument preloading, which delivers the first sixteen words in scalar registers when a wavefront starts,
+// so a wavefront's first requests do not wait for a load of the argument buffer (an aggregate argument is not
+// preloaded).
+template <int SPW, int RB, bool F32OUT, int XM, bool F16 = false>
+__global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel_1(
+    const uint16_t* x, const uint32_t* w, const uint16_t* scales, const uint16_t* biases, void* y, int K, uint32_t shape,
+    int N, const uint16_t* residual)
+{
+  // Fourteen words arrive preloaded: everything a wavefront needs for its requests.  The residual (read at the
+  // store) follows them and is loaded from the argument buffer in the usual way.
+  FlowParams<1> p;
+  p.h.x = x; p.h.residual = residual; p.h.K = K; p.h.shape = shape;
+  p.w[0] = w; p.scales[0] = scales; p.biases[0] = biases; p.y[0] = y; p.N[0] = N; p.first_block[0] = 0;
+  qmv_flow_body<SPW, RB, F32OUT, XM, 1, F16, true>(p);
+}
+
+// The grouped form (2..4 packs sharing x) with preloaded arguments: the fourteen preloaded words hold what every
+// workgroup needs (x, K, the shape word, where each pack's workgroups start) and the first pack; the other packs
+// and the first pack's y follow as an aggregate, which is read from the argument buffer.
+template <int C>
+struct FlowRest {
+  void* y0;
+  const uint32_t* w[C - 1];
+  const uint16_t* scales[C - 1];
+  const uint16_t* biases[C - 1];
+  void* y[C - 1];
+  int N[C - 1];
+};
+
+template <int SPW, int RB, bool F32OUT, int XM, int C, bool F16 = false>
+__global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel_g(
+    const uint16_t* x, int K, uint32_t shape, int N0, int fb1, int fb2, int fb3, const uint32_t* w0,
+    const uint16_t* scales0, const uint16_t* biases0, const FlowRest<C> rest)
+{
+  FlowParams<C> p;
+  p.h.x = x; p.h.residual = nullptr; p.h.K = K; p.h.shape = shape;
+  p.w[0] = w0; p.scales[0] = scales0; p.biases[0] = biases0; p.y[0] = rest.y0; p.N[0] = N0; p.first_block[0] = 0;
+  const int fb[3] = {fb1, fb2, fb3};
+#pragma unroll
+  for (int i = 1; i < C; ++i) {
+    p.w[i] = rest.w[i - 1]; p.scales[i] = rest.scales[i - 1]; p.biases[i] = rest.biases[i - 1]; p.y[i] = rest.y[i - 1];
+    p.N[i] = rest.N[i - 1]; p.first_block[i] = fb[i - 1];
+  }
+  qmv_flow_body<SPW, RB, F32OUT, XM, C, F16, true>(p);
+}
+
 namespace {
 
 struct FlowPlan {
@@ -452,15 +524,37 @@ FlowPlan flow_plan(int K, double pack_bytes)
 template <int S, int R, bool F32, int XM, int C, bool F16 = false>
 hipError_t launch_flow_kernel(dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st, const FlowParams<C>& p)
 {
-  const auto kern = qmv_flow_kernel<S, R, F32, XM, C, F16>;
   static std::once_flag once;          // one per instantiation
   static hipError_t attr_status = hipSuccess;
-  std::call_once(once, [&] {
-    attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      kMaxLdsBytes);
-  });
-  if (attr_status != hipSuccess) { return attr_status; }
-  return launch_kernel(kern, grid, block, lds_bytes, st, p);
+  if constexpr (C == 1) {
+    const auto kern = qmv_flow_kernel_1<S, R, F32, XM, F16>;
+    std::call_once(once, [&] {
+      attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        kMaxLdsBytes);
+    });
+    if (attr_status != hipSuccess) { return attr_status; }
+    return launch_kernel(kern, grid, block, lds_bytes, st, p.h.x, p.w[0], p.scales[0], p.biases[0], p.y[0], p.h.K,
+                         p.h.shape, p.N[0], p.h.residual);
+  } else {
+    // a grouped launch has no residual
+    const auto kern = qmv_flow_kernel_g<S, R, F32, XM, C, F16>;
+    std::call_once(once, [&] {
+      attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        kMaxLdsBytes);
+    });
+    if (attr_status != hipSuccess) { return attr_status; }
+    if (p.h.residual != nullptr) { return hipErrorInvalidValue; }
+    FlowRest<C> rest;
+    rest.y0 = p.y[0];
+    int fb[3] = {0x7fffffff, 0x7fffffff, 0x7fffffff};
+    for (int i = 1; i < C; ++i) {
+      rest.w[i - 1] = p.w[i]; rest.scales[i - 1] = p.scales[i]; rest.biases[i - 1] = p.biases[i]; rest.y[i - 1] = p.y[i];
+      rest.N[i - 1] = p.N[i];
+      fb[i - 1] = p.first_block[i];
+    }
+    return launch_kernel(kern, grid, block, lds_bytes, st, p.h.x, p.h.K, p.h.shape, p.N[0], fb[0], fb[1], fb[2], p.w[0],
+                         p.scales[0], p.biases[0], rest);
+  }
 }
 
 template <int C>
