@@ -18,18 +18,15 @@ SOURCES = ["vpq_api.hip", "vpq_dequant.hip", "vpq_qmv_simple.hip", "vpq_qmv_mfma
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed fp32 VALU ops are switched off for every kernel (device pass only; the
 # host pass prints a harmless "not a recognized feature" note).
+# Kernel-argument preloading: the first words of a kernel's scalar arguments arrive in scalar registers when a
+# wavefront starts (see VPQ_PRELOADED_WORDS in vpq_internal.h).
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-
-
-# Per-file additions.  The streaming decode kernel takes its sixteen argument words preloaded into scalar registers
-# (device pass option; it only affects kernels whose leading arguments are scalars or pointers).
-EXTRA_FLAGS = {"vpq_qmv_flow.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"]}
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 
 def _compile(src):
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

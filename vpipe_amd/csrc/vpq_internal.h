@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include <string>
+#include <cstring>
 #include <vector>
 
 namespace vpq {
@@ -36,6 +37,45 @@ inline hipError_t launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds_byte
     hipLaunchKernelGGL(kernel, grid, block, lds_bytes, st, args...);
   }
   return hipGetLastError();
+}
+
+// Kernel arguments in registers at wavefront start.  The library is compiled with kernel-argument preloading: the
+// first fourteen 32-bit words of a kernel's arguments arrive in scalar registers with the wavefront instead of
+// being loaded from the argument buffer (a round trip of most of a microsecond before the first request can go
+// out) -- but only if they are scalar arguments; an aggregate argument is always read from the buffer.  A kernel
+// that takes a parameter struct P therefore takes its first 56 bytes as fourteen words (VPQ_PRELOADED_WORDS) and the
+// rest as PreloadTail<P>, and puts P together again with preload_assemble; launch_preloaded splits P on the host.
+// Order the fields of P so that what the first requests need comes first and what only the store needs comes last.
+constexpr int kPreloadWords = 14;
+template <typename P>
+struct PreloadTail {
+  static_assert(sizeof(P) > kPreloadWords * 4 && sizeof(P) % 4 == 0, "parameter struct of whole words, longer than the preloaded part");
+  uint32_t w[(sizeof(P) - kPreloadWords * 4) / 4];
+};
+#define VPQ_PRELOADED_WORDS                                                                                          \
+  uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, uint32_t a4, uint32_t a5, uint32_t a6, uint32_t a7, uint32_t a8, \
+      uint32_t a9, uint32_t a10, uint32_t a11, uint32_t a12, uint32_t a13
+#define VPQ_PRELOADED_WORD_LIST a0, a1, a2, a3, a4, a5, a6, a7, a8, a9, a10, a11, a12, a13
+
+template <typename P>
+__device__ __forceinline__ P preload_assemble(VPQ_PRELOADED_WORDS, const PreloadTail<P>& tail)
+{
+  const uint32_t head[kPreloadWords] = {VPQ_PRELOADED_WORD_LIST};
+  P p;
+  __builtin_memcpy(&p, head, sizeof(head));
+  __builtin_memcpy(reinterpret_cast<char*>(&p) + sizeof(head), tail.w, sizeof(tail.w));
+  return p;
+}
+
+template <typename F, typename P>
+inline hipError_t launch_preloaded(F kernel, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st, const P& p)
+{
+  uint32_t h[kPreloadWords];
+  PreloadTail<P> tail;
+  std::memcpy(h, &p, sizeof(h));
+  std::memcpy(tail.w, reinterpret_cast<const char*>(&p) + sizeof(h), sizeof(tail.w));
+  return launch_kernel(kernel, grid, block, lds_bytes, st, h[0], h[1], h[2], h[3], h[4], h[5], h[6], h[7], h[8], h[9], h[10],
+                       h[11], h[12], h[13], tail);
 }
 
 // Measurement aids (vpq_profile.hip): a kernel that does nothing, a kernel that only reads `bytes` of src.

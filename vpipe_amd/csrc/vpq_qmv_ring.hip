@@ -34,6 +34,7 @@
 //
 // No inline-assembly VALU instruction may sit near the MFMAs (the compiler's hazard
 // recogniser cannot see what such a statement writes); the asm here is loads and waits only.
+#include <cstddef>
 #include <type_traits>
 
 #include "vpq_device.h"
@@ -56,19 +57,23 @@ constexpr int kXBytes = kXLoads * 1024;  // staged rows of one slice of x
 // 64 KB where x lives in registers (more tiles per workgroup = fewer reloads of x).
 constexpr int max_tc_mr(int mr) { return mr == 1 ? 4 : 32; }
 
+// The first fourteen words arrive preloaded (everything the requests need); y, residual and gate_act, which only
+// the store reads, follow.
 struct RingParams {
   const uint32_t* w;
   const uint16_t* scales;
   const uint16_t* biases;
   const uint16_t* x;
-  void* y;
-  const uint16_t* residual;
   int K, N, M;
   int slices;   // K / 512
   int tiles;    // ceil(N / 16)
   int tc;       // tiles per workgroup
+  void* y;
+  const uint16_t* residual;
   int gate_act; // rows are interleaved gate|up; y is [M, N/2] = act(gate) * up (1 SwiGLU, 2 GEGLU)
+  int pad_;
 };
+static_assert(offsetof(RingParams, y) == kPreloadWords * 4, "y starts the part that is not preloaded");
 
 // Eight nibbles of one packed word -> eight bf16 values 128+q, element order
 // [k0,k4,k1,k5,k2,k6,k3,k7].  `mask` and `magic` arrive as opaque register values so that
@@ -138,8 +143,9 @@ struct Taken {
 // MR: accumulator registers per lane = ceil(M/4).  Row m of x sits in MFMA row 4*(m%4) + m/4,
 // so that output row m is register m/4 of lane group m%4.  MR == 1 (M <= 4) stages x through LDS.
 template <int NW, int MR, bool F32OUT>
-__global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(const RingParams p)
+__global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, const PreloadTail<RingParams> tail)
 {
+  const RingParams p = preload_assemble<RingParams>(VPQ_PRELOADED_WORD_LIST, tail);
   constexpr bool XDMA = (MR == 1);
   __shared__ __attribute__((aligned(16))) uint8_t ring0[NW * kSlotBytes];
   __shared__ __attribute__((aligned(16))) uint8_t ring1[NW * kSlotBytes];
@@ -201,7 +207,9 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(const RingParams p)
     }
     // Lanes 0-15: the 8 scales of rows 0-15; lanes 16-31: their biases; lanes 32-63 repeat.
     const int srow = (n0 + fr < p.N) ? (n0 + fr) : (p.N - 1);
-    const uint16_t* sb = ((lane & 16) ? p.biases : p.scales) + (size_t)srow * Kg + (size_t)sl * kG;
+    const uint16_t* const scales_v = p.scales;       // values, not a choice between two fields' addresses
+    const uint16_t* const biases_v = p.biases;
+    const uint16_t* sb = ((lane & 16) ? biases_v : scales_v) + (size_t)srow * Kg + (size_t)sl * kG;
     load_to_lds(sb, slot + kCodeBytes);
   };
 
@@ -412,13 +420,13 @@ hipError_t launch_nw(hipStream_t st, const RingParams& p, int mr, bool f32)
 {
   const dim3 grid((unsigned)((p.tiles + p.tc - 1) / p.tc)), block((unsigned)(NW * kWave));
   if (f32) {
-    if (mr == 1) { return launch_kernel(qmv_ring_kernel<NW, 1, true>, grid, block, 0, st, p); }
-    if (mr == 2) { return launch_kernel(qmv_ring_kernel<NW, 2, true>, grid, block, 0, st, p); }
-    return launch_kernel(qmv_ring_kernel<NW, 4, true>, grid, block, 0, st, p);
+    if (mr == 1) { return launch_preloaded(qmv_ring_kernel<NW, 1, true>, grid, block, 0, st, p); }
+    if (mr == 2) { return launch_preloaded(qmv_ring_kernel<NW, 2, true>, grid, block, 0, st, p); }
+    return launch_preloaded(qmv_ring_kernel<NW, 4, true>, grid, block, 0, st, p);
   }
-  if (mr == 1) { return launch_kernel(qmv_ring_kernel<NW, 1, false>, grid, block, 0, st, p); }
-  if (mr == 2) { return launch_kernel(qmv_ring_kernel<NW, 2, false>, grid, block, 0, st, p); }
-  return launch_kernel(qmv_ring_kernel<NW, 4, false>, grid, block, 0, st, p);
+  if (mr == 1) { return launch_preloaded(qmv_ring_kernel<NW, 1, false>, grid, block, 0, st, p); }
+  if (mr == 2) { return launch_preloaded(qmv_ring_kernel<NW, 2, false>, grid, block, 0, st, p); }
+  return launch_preloaded(qmv_ring_kernel<NW, 4, false>, grid, block, 0, st, p);
 }
 
 }  // namespace

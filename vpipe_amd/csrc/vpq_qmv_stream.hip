@@ -20,6 +20,8 @@
 // The LDS regions are separate static arrays on purpose: the compiler orders a
 // ds_read after an outstanding direct-to-LDS load only when the two may alias,
 // and reads of staged x must not wait for the next item's codes.
+#include <cstddef>
+
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -36,20 +38,21 @@ constexpr int kItemBytes = kTileN * kRowBytes;   // 4096
 constexpr int kXPad = 16;                        // bytes of padding per staged 512-value slice row
 constexpr int kSliceStride = kKS * 2 + kXPad;    // LDS bytes of one staged slice of one x row
 
+// The first fourteen words arrive preloaded (what the requests need); the store's y and residual follow.
 struct StreamParams {
   const uint32_t* w;
   const uint16_t* scales;
   const uint16_t* biases;
   const uint16_t* x;
-  void* y;
-  const uint16_t* residual;
   int K, N, M;
   int slices;       // K / 512
   int tiles;        // ceil(N / 16)
-  int R;            // K slices per wavefront
-  int wpt;          // wavefronts per tile = ceil(slices / R)
-  int tpb;          // tiles per workgroup
+  // bits 0-15: R, the K slices per wavefront; 16-23: wavefronts per tile = ceil(slices / R); 24-31: tiles per workgroup
+  int plan;
+  void* y;
+  const uint16_t* residual;
 };
+static_assert(offsetof(StreamParams, y) == kPreloadWords * 4, "y starts the part that is not preloaded");
 
 __device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t word, uint32_t mask, uint32_t magic)
 {
@@ -76,8 +79,10 @@ __device__ __forceinline__ uint4 permute_x(uint4 d)
 // NWMAX: wavefronts the static LDS is sized for (the launch may use fewer).
 // XBYTES: bytes of LDS for the staged x of the whole K range, all M rows.
 template <int NWMAX, int XBYTES, bool F32OUT>
-__global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(const StreamParams p)
+__global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(VPQ_PRELOADED_WORDS, const PreloadTail<StreamParams> tail)
 {
+  const StreamParams p = preload_assemble<StreamParams>(VPQ_PRELOADED_WORD_LIST, tail);
+  const int plan_R = p.plan & 0xffff, plan_wpt = (p.plan >> 16) & 0xff, plan_tpb = (p.plan >> 24) & 0xff;
   // Capacity of the per-(row, group) -128*sum(x) table: XBYTES holds M*K/512 slices of 1040
   // bytes, each with 8 groups.
   constexpr int GROUPS = XBYTES / 128 + 8;
@@ -94,12 +99,12 @@ __global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(const StreamPara
   const uint32_t row_bytes_total = (uint32_t)p.K >> 1;
 
   // ---- this wavefront's unit: one tile, slices [sl0, sl1) ----
-  const int tile_local = wave / p.wpt;
-  const int kr = wave - tile_local * p.wpt;
-  const int tile = blockIdx.x * p.tpb + tile_local;
+  const int tile_local = wave / plan_wpt;
+  const int kr = wave - tile_local * plan_wpt;
+  const int tile = blockIdx.x * plan_tpb + tile_local;
   const bool active = tile < p.tiles;
-  const int sl0 = kr * p.R;
-  int sl1 = sl0 + p.R;
+  const int sl0 = kr * plan_R;
+  int sl1 = sl0 + plan_R;
   if (sl1 > p.slices) { sl1 = p.slices; }
 
   // ---- per-lane offsets.  Rows past N (ragged last tile) re-read the last real row; their
@@ -232,11 +237,11 @@ __global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(const StreamPara
 
   // acc of lane l is this wavefront's part of y[m = l/16][tile*16 + l%16].
   float total = acc;
-  if (p.wpt > 1) {
+  if (plan_wpt > 1) {
     red_lds[wave * kWave + lane] = acc;
     __syncthreads();
     if (kr != 0) { return; }
-    for (int i = 1; i < p.wpt; ++i) { total += red_lds[(wave + i) * kWave + lane]; }
+    for (int i = 1; i < plan_wpt; ++i) { total += red_lds[(wave + i) * kWave + lane]; }
   }
   const int n = tile * kTileN + fr;
   if (active && g < p.M && n < p.N) {
@@ -278,16 +283,17 @@ hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a)
   while (wpt < 8 && wpt < p.slices && (long)p.tiles * wpt < want_units) { wpt *= 2; }
   if (wpt > p.slices) { wpt = p.slices; }
   if (wpt > 8) { wpt = 8; }
-  p.R = (p.slices + wpt - 1) / wpt;
-  p.wpt = (p.slices + p.R - 1) / p.R;
-  p.tpb = 8 / p.wpt;
-  if (p.tpb > p.tiles) { p.tpb = p.tiles; }
-  const int nw = p.tpb * p.wpt;
-  const dim3 grid((unsigned)((p.tiles + p.tpb - 1) / p.tpb)), block((unsigned)(nw * kWave));
+  const int R = (p.slices + wpt - 1) / wpt;
+  wpt = (p.slices + R - 1) / R;
+  int tpb = 8 / wpt;
+  if (tpb > p.tiles) { tpb = p.tiles; }
+  p.plan = R | (wpt << 16) | (tpb << 24);
+  const int nw = tpb * wpt;
+  const dim3 grid((unsigned)((p.tiles + tpb - 1) / tpb)), block((unsigned)(nw * kWave));
 
 #define VPQ_STREAM(XB)                                                                 \
-  (a.y_f32 ? launch_kernel(qmv_stream_kernel<8, XB, true>, grid, block, 0, st, p)      \
-           : launch_kernel(qmv_stream_kernel<8, XB, false>, grid, block, 0, st, p))
+  (a.y_f32 ? launch_preloaded(qmv_stream_kernel<8, XB, true>, grid, block, 0, st, p)      \
+           : launch_preloaded(qmv_stream_kernel<8, XB, false>, grid, block, 0, st, p))
   if (xbytes <= 13 * 1024) { return VPQ_STREAM(13 * 1024); }
   if (xbytes <= 26 * 1024) { return VPQ_STREAM(26 * 1024); }
   if (xbytes <= 40 * 1024) { return VPQ_STREAM(40 * 1024); }
