@@ -147,15 +147,12 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   const double pack_bytes = (double)N * (double)K * 9.0 / 16.0;
   if (stream_ok && pack_bytes >= 150e6) { return finish(vpq::launch_qmv_stream(hs, a)); }
   // Several rows of x: the ring kernel keeps a slice of x in registers for all the tiles of a
-  // workgroup (one workgroup per CU, up to 16 / 8 tiles each at 5..8 / 9..16 rows), so x is
-  // re-read from L2 once per slice and workgroup instead of once per item (measured at 16 rows:
-  // 117 vs 284 us at 5120->151936, 17.6 vs 39.9 us at 5120->17408; at 4 rows 8.8 vs 12.0 us at
-  // 4096->12288).  Its workgroups have 8 wavefronts: with 2 rows it only pays where the
-  // k-slices fill them evenly.
-  if (mfma_ok && vpq::qmv_ring_supports(K, N, M) && M >= 2) {
-    const bool even = ((K / 512) % 8) == 0;
-    if (M >= 3 || even) { return finish(vpq::launch_qmv_ring(hs, a, 0, 0)); }
-  }
+  // workgroup (one workgroup per CU; it chooses its tiles per workgroup so that the launch runs in
+  // few, full generations of workgroups), so x is re-read from L2 once per slice and workgroup instead
+  // of once per item (measured at 16 rows: 117 vs 284 us at 5120->151936, 17.6 vs 39.9 us at
+  // 5120->17408; at 4 rows 8.8 vs 12.0 us at 4096->12288; at 2 rows 15.1 vs 17.1 us at 5120->17408,
+  // 16.0 vs 17.5 at 17408->5120).
+  if (mfma_ok && vpq::qmv_ring_supports(K, N, M) && M >= 2) { return finish(vpq::launch_qmv_ring(hs, a, 0, 0)); }
   if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a, 1)); }
   // K not a multiple of 512, or scales / biases off 16-byte alignment: the row-streaming kernel
   // for up to two rows of x, the general one above.

@@ -444,16 +444,31 @@ hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw
   p.tiles = (a.N + kTileN - 1) / kTileN;
   int mr = (a.M + 3) / 4;
   if (mr == 3) { mr = 4; }
-  // Enough tiles per workgroup that one workgroup per CU covers the matrix in one pass.
   const int cus = a.cu_count > 0 ? a.cu_count : 256;
-  int tc = (p.tiles + cus - 1) / cus;
-  // 3 or 4 rows over a wide matrix: the two-register form takes more tiles per workgroup than
-  // the staged-x form has room for, which is worth more than its idle accumulator register.
-  if (mr == 1 && a.M >= 3 && tc > max_tc_mr(1)) { mr = 2; }
+  // Tiles per workgroup.  One workgroup is resident per CU, so the launch runs in generations of `cus`
+  // workgroups, each lasting about as long as a workgroup's bytes: its tiles' codes, scales and biases plus
+  // all of x once.  The count that minimises generations x bytes per workgroup wins; the largest count
+  // often does not (9496 tiles at 16 per workgroup: 594 workgroups, a third generation for 82 of them).
+  const double tile_bytes = 16.0 * (double)a.K * 9.0 / 16.0, x_bytes = (double)a.M * (double)a.K * 2.0;
+  auto plan = [&](int regs, int& tc_out) {
+    double best = 0.0;
+    for (int t = 1; t <= max_tc_mr(regs) / regs; ++t) {
+      const int wgs = (p.tiles + t - 1) / t;
+      const double cost = (double)((wgs + cus - 1) / cus) * ((double)t * tile_bytes + x_bytes);
+      if (t == 1 || cost <= best) { best = cost; tc_out = t; }
+    }
+    return best;
+  };
+  int tc = 1;
+  const double cost = plan(mr, tc);
+  // Up to 4 rows: the staged-x form has room for 4 tiles per workgroup; where that costs a generation the
+  // two-register form (up to 16 tiles) is worth more than its idle accumulator register.
+  if (mr == 1 && a.M >= 2) {
+    int tc2 = 1;
+    if (plan(2, tc2) * 1.05 < cost) { mr = 2; tc = tc2; }
+  }
   const int tc_max = max_tc_mr(mr) / mr;
-  if (tc_hint > 0) { tc = tc_hint; }
-  if (tc > tc_max) { tc = tc_max; }
-  if (tc < 1) { tc = 1; }
+  if (tc_hint > 0) { tc = tc_hint < tc_max ? tc_hint : tc_max; }
   p.tc = tc;
   return launch_nw<8>(st, p, mr, a.y_f32);
 }
