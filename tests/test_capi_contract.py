@@ -84,3 +84,19 @@ def test_host_layer_and_its_test_driver_load():
     for name in ("hd_open", "hd_close", "hd_set_function", "hd_set_buffer", "hd_set_constant_i32", "hd_dispatch",
                  "hd_scope_begin", "hd_scope_end", "hd_dispatch_count", "hd_wait_ok", "hd_reason", "hd_quant_linear"):
         assert hasattr(D, name), name
+
+
+def test_build_refuses_kernels_that_spill():
+    """The build reads the compiler's per-kernel resource remarks and fails on scratch use (a spilled destination
+    register of an asynchronous load is a fault waiting to happen); one named kernel is exempt."""
+    from vpipe_amd import build
+    def remark(name, scratch):
+        return ("x.hip:1:1: remark: Function Name: %s [-Rpass-analysis=kernel-resource-usage]\n"
+                "x.hip:1:1: remark:     VGPRs: 64 [-Rpass-analysis=kernel-resource-usage]\n"
+                "x.hip:1:1: remark:     ScratchSize [bytes/lane]: %d [-Rpass-analysis=kernel-resource-usage]\n"
+                % (name, scratch))
+    build._check_no_scratch("x.hip", remark("_ZN3vpq15qmv_ring_kernelILi8ELi2ELb1EEEv", 0))
+    build._check_no_scratch("x.hip", remark("_ZN3vpq14qmm_big_kernelILi4ELb0ELi3EEEvNS_9BigParamsE", 60))
+    with pytest.raises(RuntimeError, match="spill"):
+        build._check_no_scratch("x.hip", remark("_ZN3vpq15qmv_ring_kernelILi8ELi2ELb1EEEv", 276) +
+                                remark("_ZN3vpq15qmv_flow_kernel_1ILi2ELi2EEEv", 0))

@@ -7,6 +7,7 @@ into one shared library that exports the C ABI declared in include/vpq.h.
 """
 import concurrent.futures
 import os
+import re
 import subprocess
 import sys
 
@@ -24,13 +25,36 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-u
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 
+# No kernel may spill registers to scratch memory.  Several kernels issue loads from inline assembly and wait for
+# them later with counted waits: the compiler takes the destination registers as written at once, and a spill of
+# one of them saves garbage and frees the register for other use while the load is still on its way to it (seen
+# once: a later address came out of such a register and the launch faulted).  The build fails instead.  The one
+# exception spills in its epilogue only, after its last load has landed (the binary16 256 x 256 GEMM tile).
+SCRATCH_ALLOWED = re.compile(r"qmm_big_kernelILi4ELb0ELi3E")
+
+
+def _check_no_scratch(src, remarks):
+    bad = []
+    for block in re.split(r"remark: [^\n]*Function Name: ", remarks)[1:]:
+        name = block.split()[0]
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", block)
+        if m and int(m.group(1)) > 0 and not SCRATCH_ALLOWED.search(name):
+            bad.append("%s: %s bytes per lane" % (name, m.group(1)))
+    if bad:
+        raise RuntimeError("%s: kernels that spill to scratch memory (not allowed, see build.py):\n  %s"
+                           % (src, "\n  ".join(bad)))
+
+
 def _compile(src):
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC] + FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
-    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
+        err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "remark:" not in l)
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
+    _check_no_scratch(src, r.stderr)
+    err = "\n".join(l for l in r.stderr.splitlines()
+                    if "packed-fp32-ops" not in l and "remark:" not in l and "-Rpass-analysis" not in l)
     return obj, err
 
 
