@@ -350,11 +350,20 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
     auto step = [&](int i, uint8_t* slot) {
       take(slot, x_behind > 0, it);
       if (x_behind > 0) { --x_behind; }
-      request(i + 2, slot);
-      if (fresh) {
+      if (!XDMA && fresh) {
+        // x in registers: the loads of the new slice drain the queue.  Issued before the slot is re-requested they
+        // wait for the one item in flight (requested an item ago) and for themselves (L2), not for a request
+        // to HBM made a moment earlier.
         fetch_x(r, std::integral_constant<int, kItemLoads>());
         fresh = false;
-        if (XDMA && r + 1 < rounds) { request_x(r + 1); x_behind = 2; }
+        request(i + 2, slot);
+      } else {
+        request(i + 2, slot);
+        if (fresh) {
+          fetch_x(r, std::integral_constant<int, kItemLoads>());
+          fresh = false;
+          if (r + 1 < rounds) { request_x(r + 1); x_behind = 2; }
+        }
       }
       compute(i, it);
       if (--left == 0) { ++r; left = TC; fresh = true; }

@@ -296,7 +296,9 @@ hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a)
            : launch_preloaded(qmv_stream_kernel<8, XB, false>, grid, block, 0, st, p))
   if (xbytes <= 13 * 1024) { return VPQ_STREAM(13 * 1024); }
   if (xbytes <= 26 * 1024) { return VPQ_STREAM(26 * 1024); }
-  if (xbytes <= 40 * 1024) { return VPQ_STREAM(40 * 1024); }
+  // 42 KB: four rows of K = 5120 (41600 bytes) still leave room for two workgroups per CU; the next size does not
+  // (lm_head at 4 rows: 98 us with one workgroup per CU).
+  if (xbytes <= 42 * 1024) { return VPQ_STREAM(42 * 1024); }
   return VPQ_STREAM(72 * 1024);
 #undef VPQ_STREAM
 }
