@@ -85,11 +85,12 @@ __global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(VPQ_PRELOADED_WO
   const int plan_R = p.plan & 0xffff, plan_wpt = (p.plan >> 16) & 0xff, plan_tpb = (p.plan >> 24) & 0xff;
   // Capacity of the per-(row, group) -128*sum(x) table: XBYTES holds M*K/512 slices of 1040
   // bytes, each with 8 groups.
-  constexpr int GROUPS = XBYTES / 128 + 8;
+  constexpr int GROUPS = XBYTES / kSliceStride * kG;
   __shared__ __attribute__((aligned(16))) uint8_t codes_lds[NWMAX * kItemBytes];
   __shared__ __attribute__((aligned(16))) uint8_t x_lds[XBYTES];
   __shared__ __attribute__((aligned(16))) float xneg_lds[GROUPS];
-  __shared__ float red_lds[NWMAX * kWave];
+  // The partial sums of wavefronts that share a tile meet in the code buffers once nobody reads codes any more.
+  float* red_lds = reinterpret_cast<float*>(codes_lds);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -238,6 +239,7 @@ __global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(VPQ_PRELOADED_WO
   // acc of lane l is this wavefront's part of y[m = l/16][tile*16 + l%16].
   float total = acc;
   if (plan_wpt > 1) {
+    __syncthreads();                         // every wavefront has taken its last item out of its buffer
     red_lds[wave * kWave + lane] = acc;
     __syncthreads();
     if (kr != 0) { return; }
