@@ -250,6 +250,8 @@ RING_SHAPES = STREAM_SHAPES + [
     (1024, 16 * 3000, 6), (512, 16 * 2100 + 5, 12),
     # 3 and 4 rows over a wide matrix take the two-register form
     (1024, 16 * 1400 + 2, 3), (512, 16 * 1300, 4),
+    # ... and so do 2 rows where that saves a generation of workgroups (1300 tiles: 6 per workgroup, one generation)
+    (512, 16 * 1300, 2), (1536, 16 * 1088 + 7, 2),
 ]
 
 
