@@ -57,6 +57,25 @@ def test_qmv_f16(vpq, oracle, dev, D, K, N, M):
                                                                      xd.view(torch.bfloat16), K, N, M, variant=1).view(torch.int16))
 
 
+@pytest.mark.parametrize("K,N,M", [(512, 16, 2), (1024, 37, 4), (5120, 530, 3), (5120, 1029, 5), (4608, 250, 8),
+                                   (2560, 64, 12), (8192, 100, 16), (512, 16 * 1300, 2), (17408, 66, 9)])
+def test_qmv_f16_several_rows_ring_kernel(vpq, oracle, dev, D, K, N, M):
+    """2..16 rows of x on K % 512 == 0 run on the ring kernel's binary16 mode: x through LDS (up to 4 rows) and in
+    registers, one and several slices per wavefront, ragged last tile, the two-register form at 2 rows."""
+    w, s, b = f16_pack(N, K, 900 + K + N)
+    x = np.random.default_rng(950 + K + M).standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    y64, _ = oracle.matmul_f16(w, s, b, x, K, N, M, rounded=False)
+    wd, sd, bd, xd = D.u32(w, dev), dev16(s, dev), dev16(b, dev), dev16(x, dev)
+    f = vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, f32out=True)
+    out = parity.Guarded((M, N), torch.float16, dev)
+    vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_f32(f.cpu().numpy(), y64)
+    check_f16(bits16(out.view), y64)
+    assert torch.equal(f, vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, f32out=True))     # bit-reproducible
+
+
 def test_qmv_f16_residual_and_gated(vpq, oracle, dev, D):
     K, ffn, M = 1024, 40, 2
     N = 2 * ffn

@@ -560,6 +560,11 @@ static int qmv_f16_common(vpq_stream_t stream, const uint32_t* w, const uint16_t
   if (vpq::qmv_flow_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16)) {
     return finish(vpq::launch_qmv_flow_f16(reinterpret_cast<hipStream_t>(stream), a));
   }
+  // several rows: the ring kernel on binary16 arithmetic (K % 512 == 0)
+  if (M >= 2 && vpq::qmv_mfma_supports(K, N, M) && vpq::qmv_ring_supports(K, N, M) && aligned(scales, 16) &&
+      aligned(biases, 16)) {
+    return finish(vpq::launch_qmv_ring(reinterpret_cast<hipStream_t>(stream), a, 0, 0, true));
+  }
   return finish(vpq::launch_qmv_simple_f16(reinterpret_cast<hipStream_t>(stream), a));
 }
 

@@ -77,18 +77,39 @@ static_assert(offsetof(RingParams, y) == kPreloadWords * 4, "y starts the part t
 
 // Eight nibbles of one packed word -> eight bf16 values 128+q, element order
 // [k0,k4,k1,k5,k2,k6,k3,k7].  `mask` and `magic` arrive as opaque register values so that
-// each pair costs a single v_and_or_b32.
-__device__ __forceinline__ bf16x8 ring_codes_to_bf16(uint32_t word, uint32_t mask, uint32_t magic)
+// each pair costs a single v_and_or_b32.  F16: binary16 values 16+q instead (the code shifted to
+// mantissa bits 6..9, where a step is 1/64 of 16.0's exponent: exact).
+template <bool F16>
+__device__ __forceinline__ u32x4 ring_codes_to_elts(uint32_t word, uint32_t mask, uint32_t magic)
 {
   u32x4 v;
-  v[0] = (word & mask) | magic;
-  v[1] = ((word >> 4) & mask) | magic;
-  v[2] = ((word >> 8) & mask) | magic;
-  v[3] = ((word >> 12) & mask) | magic;
-  return __builtin_bit_cast(bf16x8, v);
+  if constexpr (F16) {
+    v[0] = ((word << 6) & mask) | magic;
+    v[1] = ((word << 2) & mask) | magic;
+    v[2] = ((word >> 2) & mask) | magic;
+    v[3] = ((word >> 6) & mask) | magic;
+  } else {
+    v[0] = (word & mask) | magic;
+    v[1] = ((word >> 4) & mask) | magic;
+    v[2] = ((word >> 8) & mask) | magic;
+    v[3] = ((word >> 12) & mask) | magic;
+  }
+  return v;
 }
 
-// Eight consecutive bf16 of x -> the element order ring_codes_to_bf16 produces.
+// D = A (16 x 32) * B (32 x 16) + C on bf16 or binary16 operands, fp32 accumulation.
+template <bool F16>
+__device__ __forceinline__ floatx4 ring_mfma(u32x4 a, u32x4 b, floatx4 c)
+{
+  if constexpr (F16) {
+    typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+}
+
+// Eight consecutive elements of x -> the element order ring_codes_to_elts produces.
 __device__ __forceinline__ u32x4 ring_permute_x(u32x4 d)
 {
   u32x4 v;
@@ -142,7 +163,9 @@ struct Taken {
 
 // MR: accumulator registers per lane = ceil(M/4).  Row m of x sits in MFMA row 4*(m%4) + m/4,
 // so that output row m is register m/4 of lane group m%4.  MR == 1 (M <= 4) stages x through LDS.
-template <int NW, int MR, bool F32OUT>
+// F16: x, scales, biases, y and the residual are IEEE binary16 (the reference's VPIPE_ELT = half build); the codes
+// become 16+q and the offset -16*sum(x).
+template <int NW, int MR, bool F32OUT, bool F16 = false>
 __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, const PreloadTail<RingParams> tail)
 {
   const RingParams p = preload_assemble<RingParams>(VPQ_PRELOADED_WORD_LIST, tail);
@@ -174,13 +197,13 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
   const int ld_row = lane >> 4;
   const int ld_pos = lane & 15;
 
-  uint32_t magic = 0x43004300u;             // bf16 128.0 in both halves
-  uint32_t mask = 0x000f000fu;
+  uint32_t magic = F16 ? 0x4c004c00u : 0x43004300u;   // 16.0 (binary16) or 128.0 (bf16) in both halves
+  uint32_t mask = F16 ? 0x03c003c0u : 0x000f000fu;
   asm volatile("" : "+v"(magic));           // no instruction: only hides the constants
   asm volatile("" : "+s"(mask));            // from constant folding
-  u32x4 m128;
-  m128[0] = m128[1] = m128[2] = m128[3] = 0xc300c300u;  // bf16 -128.0
-  const bf16x8 neg128 = __builtin_bit_cast(bf16x8, m128);
+  u32x4 neg128;                             // the offset of the codes, negated: -128.0 (bf16) or -16.0 (binary16)
+  neg128[0] = neg128[1] = neg128[2] = neg128[3] = F16 ? 0xcc00cc00u : 0xc300c300u;
+  constexpr float kBiasOverOffset = F16 ? -0.0625f : -0.0078125f;
 
   // This wavefront's items: slices wave, wave+NW, ... (rounds) x the workgroup's tiles.
   const int rounds = (p.slices - wave + NW - 1) / NW;     // <= 0 for an idle wavefront
@@ -287,8 +310,8 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
 #pragma unroll
     for (int grp = 0; grp < kG; ++grp) {
       floatx4 xn = {0.f, 0.f, 0.f, 0.f};
-      xn = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xq[2 * grp]), neg128, xn, 0, 0, 0);
-      xn = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xq[2 * grp + 1]), neg128, xn, 0, 0, 0);
+      xn = ring_mfma<F16>(xq[2 * grp], neg128, xn);
+      xn = ring_mfma<F16>(xq[2 * grp + 1], neg128, xn);
 #pragma unroll
       for (int q = 0; q < MR; ++q) { xneg[grp][q] = xn[q]; }
     }
@@ -309,13 +332,11 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
       floatx4 s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int q = 0; q < MR; ++q) { s4[q] = xneg[grp][q]; }
-      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xq[2 * grp]),
-                                                    ring_codes_to_bf16(cw[0], mask, magic), s4, 0, 0, 0);
-      s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xq[2 * grp + 1]),
-                                                    ring_codes_to_bf16(cw[1], mask, magic), s4, 0, 0, 0);
-      const float s = (grp & 1) ? bf16_hi_to_f32(sd[grp >> 1]) : bf16_lo_to_f32(sd[grp >> 1]);
-      const float b = (grp & 1) ? bf16_hi_to_f32(bd[grp >> 1]) : bf16_lo_to_f32(bd[grp >> 1]);
-      const float b2 = b * -0.0078125f;              // bias * sum(x) = (bias / -128) * xneg
+      s4 = ring_mfma<F16>(xq[2 * grp], ring_codes_to_elts<F16>(cw[0], mask, magic), s4);
+      s4 = ring_mfma<F16>(xq[2 * grp + 1], ring_codes_to_elts<F16>(cw[1], mask, magic), s4);
+      const float s = (grp & 1) ? elt_hi_to_f32<F16>(sd[grp >> 1]) : elt_lo_to_f32<F16>(sd[grp >> 1]);
+      const float b = (grp & 1) ? elt_hi_to_f32<F16>(bd[grp >> 1]) : elt_lo_to_f32<F16>(bd[grp >> 1]);
+      const float b2 = b * kBiasOverOffset;          // bias * sum(x) = (bias / -offset) * xneg
 #pragma unroll
       for (int q = 0; q < MR; ++q) {
         acc[q] = fmaf(s, s4[q], acc[q]);
@@ -399,7 +420,7 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
         if (F32OUT) {
           reinterpret_cast<float*>(p.y)[o] = v;
         } else {
-          reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)f32_to_bf16_bits(v);
+          reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)f32_to_elt_bits<F16>(v);
         }
       }
     } else if (tile < p.tiles && m < p.M && n < p.N) {
@@ -407,9 +428,9 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
       if (F32OUT) {
         reinterpret_cast<float*>(p.y)[o] = total;
       } else {
-        uint32_t v = f32_to_bf16_bits(total);
+        uint32_t v = f32_to_elt_bits<F16>(total);
         if (p.residual != nullptr) {
-          v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(p.residual[o]));
+          v = f32_to_elt_bits<F16>(elt_bits_to_f32<F16>(v) + elt_bits_to_f32<F16>(p.residual[o]));
         }
         reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)v;
       }
@@ -424,24 +445,24 @@ bool qmv_ring_supports(int K, int N, int M)
 
 namespace {
 
-template <int NW>
+template <int NW, bool F16>
 hipError_t launch_nw(hipStream_t st, const RingParams& p, int mr, bool f32)
 {
   const dim3 grid((unsigned)((p.tiles + p.tc - 1) / p.tc)), block((unsigned)(NW * kWave));
   if (f32) {
-    if (mr == 1) { return launch_preloaded(qmv_ring_kernel<NW, 1, true>, grid, block, 0, st, p); }
-    if (mr == 2) { return launch_preloaded(qmv_ring_kernel<NW, 2, true>, grid, block, 0, st, p); }
-    return launch_preloaded(qmv_ring_kernel<NW, 4, true>, grid, block, 0, st, p);
+    if (mr == 1) { return launch_preloaded(qmv_ring_kernel<NW, 1, true, F16>, grid, block, 0, st, p); }
+    if (mr == 2) { return launch_preloaded(qmv_ring_kernel<NW, 2, true, F16>, grid, block, 0, st, p); }
+    return launch_preloaded(qmv_ring_kernel<NW, 4, true, F16>, grid, block, 0, st, p);
   }
-  if (mr == 1) { return launch_preloaded(qmv_ring_kernel<NW, 1, false>, grid, block, 0, st, p); }
-  if (mr == 2) { return launch_preloaded(qmv_ring_kernel<NW, 2, false>, grid, block, 0, st, p); }
-  return launch_preloaded(qmv_ring_kernel<NW, 4, false>, grid, block, 0, st, p);
+  if (mr == 1) { return launch_preloaded(qmv_ring_kernel<NW, 1, false, F16>, grid, block, 0, st, p); }
+  if (mr == 2) { return launch_preloaded(qmv_ring_kernel<NW, 2, false, F16>, grid, block, 0, st, p); }
+  return launch_preloaded(qmv_ring_kernel<NW, 4, false, F16>, grid, block, 0, st, p);
 }
 
 }  // namespace
 
 // tc_hint > 0 forces the tiles per workgroup (measurement).
-hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint)
+hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint, bool f16)
 {
   (void)nw_hint;
   RingParams p;
@@ -479,7 +500,7 @@ hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw
   const int tc_max = max_tc_mr(mr) / mr;
   if (tc_hint > 0) { tc = tc_hint < tc_max ? tc_hint : tc_max; }
   p.tc = tc;
-  return launch_nw<8>(st, p, mr, a.y_f32);
+  return f16 ? launch_nw<8, true>(st, p, mr, a.y_f32) : launch_nw<8, false>(st, p, mr, a.y_f32);
 }
 
 }  // namespace vpq
