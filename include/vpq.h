@@ -633,8 +633,9 @@ int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const
  * IEEE binary16 bit patterns, the packed codes are the same.  One row of x on
  * K % 512 == 0, K >= 2048 with 16-byte aligned scales and biases takes the
  * streaming decode kernel of the bf16 entry on binary16 arithmetic (same
- * speed), 2..16 rows on K % 512 == 0 the ring kernel (VPQ_QMV_RING) on binary16
- * arithmetic; every other QMV shape takes a general path (one wavefront per
+ * speed), 2..16 rows on K % 512 == 0 the ring kernel (VPQ_QMV_RING) or, for 2..4
+ * rows over 150 MB of codes and more, the streaming kernel (VPQ_QMV_STREAM) on
+ * binary16 arithmetic; every other QMV shape takes a general path (one wavefront per
  * output row); the QMM is expansion + the dense GEMM:
  *   vpq_dequant_w4g64_f16         `affine_dequant_w4g64` (affine_dequant.metal:25-58), bit-exact:
  *                                 f16_rne(fp32(s) * q + fp32(b)).

@@ -76,6 +76,25 @@ def test_qmv_f16_several_rows_ring_kernel(vpq, oracle, dev, D, K, N, M):
     assert torch.equal(f, vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, f32out=True))     # bit-reproducible
 
 
+@pytest.mark.parametrize("M", [2, 3, 4])
+def test_qmv_f16_lm_head_rows_streaming_kernel(vpq, oracle, dev, D, M):
+    """2..4 rows over an lm_head-sized pack (>= 150 MB of codes) run on the streaming MFMA kernel's binary16 mode.
+    Full-size launch; the oracle evaluates a sample of output rows (first and last tiles included)."""
+    K, N = 5120, 151936
+    w, s, b = f16_pack(N, K, 1200 + M)
+    x = np.random.default_rng(1250 + M).standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    rng = np.random.default_rng(N + M)
+    rows = np.unique(np.concatenate([np.arange(16), np.arange(N - 16, N), rng.integers(0, N, 224)]))
+    y64, _ = oracle.matmul_f16(w[rows], s[rows], b[rows], x, K, len(rows), M, rounded=False)
+    wd, sd, bd, xd = D.u32(w, dev), dev16(s, dev), dev16(b, dev), dev16(x, dev)
+    f = vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M, f32out=True).cpu().numpy()
+    y = bits16(vpq.qmv_w4g64_f16(wd, sd, bd, xd, K, N, M))
+    parity.check_f32(f[:, rows], y64)
+    check_f16(y[:, rows], y64)
+    z = vpq.qmv_w4g64_f16(wd, sd, bd, torch.zeros_like(xd), K, N, M, f32out=True)
+    assert not z.any().item()                                  # all rows: zero activations give exactly zero
+
+
 def test_qmv_f16_residual_and_gated(vpq, oracle, dev, D):
     K, ffn, M = 1024, 40, 2
     N = 2 * ffn

@@ -560,9 +560,13 @@ static int qmv_f16_common(vpq_stream_t stream, const uint32_t* w, const uint16_t
   if (vpq::qmv_flow_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16)) {
     return finish(vpq::launch_qmv_flow_f16(reinterpret_cast<hipStream_t>(stream), a));
   }
-  // several rows: the ring kernel on binary16 arithmetic (K % 512 == 0)
-  if (M >= 2 && vpq::qmv_mfma_supports(K, N, M) && vpq::qmv_ring_supports(K, N, M) && aligned(scales, 16) &&
-      aligned(biases, 16)) {
+  // several rows (K % 512 == 0): the kernels of the bf16 entry on binary16 arithmetic -- two to four rows over an
+  // lm_head-sized pack the streaming kernel, otherwise the ring kernel
+  const bool tuned = M >= 2 && vpq::qmv_mfma_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
+  if (tuned && gate_act == 0 && vpq::qmv_stream_supports(K, N, M) && (double)N * (double)K * 9.0 / 16.0 >= 150e6) {
+    return finish(vpq::launch_qmv_stream(reinterpret_cast<hipStream_t>(stream), a, true));
+  }
+  if (tuned && vpq::qmv_ring_supports(K, N, M)) {
     return finish(vpq::launch_qmv_ring(reinterpret_cast<hipStream_t>(stream), a, 0, 0, true));
   }
   return finish(vpq::launch_qmv_simple_f16(reinterpret_cast<hipStream_t>(stream), a));

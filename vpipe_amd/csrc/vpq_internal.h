@@ -176,7 +176,7 @@ hipError_t launch_qmv_flow(hipStream_t st, const QmvArgs& a);
 hipError_t launch_qmv_flow_f16(hipStream_t st, const QmvArgs& a);    // IEEE binary16 elements
 hipError_t launch_qmv_flow_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g, bool f16 = false);
 bool qmv_stream_supports(int K, int N, int M);
-hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a);
+hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a, bool f16 = false);
 bool qmv_ring_supports(int K, int N, int M);
 // tc_hint / nw_hint > 0 force the tiles / wavefronts per workgroup (measurement only).
 hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint, bool f16 = false);

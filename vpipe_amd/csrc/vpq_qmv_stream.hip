@@ -54,14 +54,35 @@ struct StreamParams {
 };
 static_assert(offsetof(StreamParams, y) == kPreloadWords * 4, "y starts the part that is not preloaded");
 
-__device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t word, uint32_t mask, uint32_t magic)
+// Eight nibbles of a packed word -> eight elements 128+q (bf16) or 16+q (binary16: the code shifted to mantissa
+// bits 6..9), element order [k0,k4,k1,k5,k2,k6,k3,k7]; one v_and_or_b32 per pair.
+template <bool F16>
+__device__ __forceinline__ u32x4 codes_to_elts(uint32_t word, uint32_t mask, uint32_t magic)
 {
   u32x4 v;
-  v[0] = (word & mask) | magic;
-  v[1] = ((word >> 4) & mask) | magic;
-  v[2] = ((word >> 8) & mask) | magic;
-  v[3] = ((word >> 12) & mask) | magic;
-  return __builtin_bit_cast(bf16x8, v);
+  if constexpr (F16) {
+    v[0] = ((word << 6) & mask) | magic;
+    v[1] = ((word << 2) & mask) | magic;
+    v[2] = ((word >> 2) & mask) | magic;
+    v[3] = ((word >> 6) & mask) | magic;
+  } else {
+    v[0] = (word & mask) | magic;
+    v[1] = ((word >> 4) & mask) | magic;
+    v[2] = ((word >> 8) & mask) | magic;
+    v[3] = ((word >> 12) & mask) | magic;
+  }
+  return v;
+}
+
+template <bool F16>
+__device__ __forceinline__ floatx4 stream_mfma(u32x4 a, u32x4 b, floatx4 c)
+{
+  if constexpr (F16) {
+    typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
 }
 
 __device__ __forceinline__ uint4 permute_x(uint4 d)
@@ -78,7 +99,8 @@ __device__ __forceinline__ uint4 permute_x(uint4 d)
 
 // NWMAX: wavefronts the static LDS is sized for (the launch may use fewer).
 // XBYTES: bytes of LDS for the staged x of the whole K range, all M rows.
-template <int NWMAX, int XBYTES, bool F32OUT>
+// F16: x, scales, biases, y and the residual are IEEE binary16; the offset of the codes is 16 instead of 128.
+template <int NWMAX, int XBYTES, bool F32OUT, bool F16 = false>
 __global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(VPQ_PRELOADED_WORDS, const PreloadTail<StreamParams> tail)
 {
   const StreamParams p = preload_assemble<StreamParams>(VPQ_PRELOADED_WORD_LIST, tail);
@@ -165,18 +187,18 @@ __global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(VPQ_PRELOADED_WO
       const int j = i - m * pieces_per_row;                 // 16-byte piece within the row
       const uint4 d = *reinterpret_cast<const uint4*>(p.x + (size_t)m * p.K + (size_t)j * 8);
       *reinterpret_cast<uint4*>(x_lds + m * xrow_stride + (j >> 6) * kSliceStride + (j & 63) * 16) = permute_x(d);
-      float sum = ((bf16_lo_to_f32(d.x) + bf16_hi_to_f32(d.x)) + (bf16_lo_to_f32(d.y) + bf16_hi_to_f32(d.y))) +
-                  ((bf16_lo_to_f32(d.z) + bf16_hi_to_f32(d.z)) + (bf16_lo_to_f32(d.w) + bf16_hi_to_f32(d.w)));
+      float sum = ((elt_lo_to_f32<F16>(d.x) + elt_hi_to_f32<F16>(d.x)) + (elt_lo_to_f32<F16>(d.y) + elt_hi_to_f32<F16>(d.y))) +
+                  ((elt_lo_to_f32<F16>(d.z) + elt_hi_to_f32<F16>(d.z)) + (elt_lo_to_f32<F16>(d.w) + elt_hi_to_f32<F16>(d.w)));
       sum += __shfl_xor(sum, 1, kWave);
       sum += __shfl_xor(sum, 2, kWave);
       sum += __shfl_xor(sum, 4, kWave);
-      if ((lane & 7) == 0) { xneg_lds[m * Kg + (j >> 3)] = -128.0f * sum; }
+      if ((lane & 7) == 0) { xneg_lds[m * Kg + (j >> 3)] = (F16 ? -16.0f : -128.0f) * sum; }
     }
   }
   __syncthreads();
 
-  uint32_t magic = 0x43004300u;             // bf16 128.0 in both halves
-  uint32_t mask = 0x000f000fu;
+  uint32_t magic = F16 ? 0x4c004c00u : 0x43004300u;   // 16.0 (binary16) or 128.0 (bf16) in both halves
+  uint32_t mask = F16 ? 0x03c003c0u : 0x000f000fu;
   asm volatile("" : "+v"(magic));           // no instruction: hides the constants from folding
   asm volatile("" : "+s"(mask));
 
@@ -222,16 +244,16 @@ __global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(VPQ_PRELOADED_WO
       const uint32_t bd[4] = {bv.x, bv.y, bv.z, bv.w};
 #pragma unroll
       for (int grp = 0; grp < kG; ++grp) {
-        const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(xs + grp * 128);
-        const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(xs + grp * 128 + 16);
+        const u32x4 a0 = *reinterpret_cast<const u32x4*>(xs + grp * 128);
+        const u32x4 a1 = *reinterpret_cast<const u32x4*>(xs + grp * 128 + 16);
         floatx4 s4 = {0.f, 0.f, 0.f, 0.f};
-        s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, codes_to_bf16(cw[grp].x, mask, magic), s4, 0, 0, 0);
-        s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, codes_to_bf16(cw[grp].y, mask, magic), s4, 0, 0, 0);
-        const float sc = (grp & 1) ? bf16_hi_to_f32(sd[grp >> 1]) : bf16_lo_to_f32(sd[grp >> 1]);
-        const float bi = (grp & 1) ? bf16_hi_to_f32(bd[grp >> 1]) : bf16_lo_to_f32(bd[grp >> 1]);
+        s4 = stream_mfma<F16>(a0, codes_to_elts<F16>(cw[grp].x, mask, magic), s4);
+        s4 = stream_mfma<F16>(a1, codes_to_elts<F16>(cw[grp].y, mask, magic), s4);
+        const float sc = (grp & 1) ? elt_hi_to_f32<F16>(sd[grp >> 1]) : elt_lo_to_f32<F16>(sd[grp >> 1]);
+        const float bi = (grp & 1) ? elt_hi_to_f32<F16>(bd[grp >> 1]) : elt_lo_to_f32<F16>(bd[grp >> 1]);
         const float sxq = s4[0] + xneg[grp];               // sum(x*(128+q)) - 128*sum(x)
         acc = fmaf(sc, sxq, acc);
-        acc = fmaf(bi * -0.0078125f, xneg[grp], acc);      // bias * sum(x)
+        acc = fmaf(bi * (F16 ? -0.0625f : -0.0078125f), xneg[grp], acc);      // bias * sum(x)
       }
     }
   }
@@ -251,9 +273,9 @@ __global__ __launch_bounds__(NWMAX * 64) void qmv_stream_kernel(VPQ_PRELOADED_WO
     if (F32OUT) {
       reinterpret_cast<float*>(p.y)[o] = total;
     } else {
-      uint32_t v = f32_to_bf16_bits(total);
+      uint32_t v = f32_to_elt_bits<F16>(total);
       if (p.residual != nullptr) {
-        v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(p.residual[o]));
+        v = f32_to_elt_bits<F16>(elt_bits_to_f32<F16>(v) + elt_bits_to_f32<F16>(p.residual[o]));
       }
       reinterpret_cast<uint16_t*>(p.y)[o] = (uint16_t)v;
     }
@@ -268,7 +290,7 @@ bool qmv_stream_supports(int K, int N, int M)
   return xbytes <= 72 * 1024;
 }
 
-hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a)
+hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a, bool f16)
 {
   StreamParams p;
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y; p.residual = a.residual;
@@ -293,9 +315,11 @@ hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a)
   const int nw = tpb * wpt;
   const dim3 grid((unsigned)((p.tiles + tpb - 1) / tpb)), block((unsigned)(nw * kWave));
 
-#define VPQ_STREAM(XB)                                                                 \
-  (a.y_f32 ? launch_preloaded(qmv_stream_kernel<8, XB, true>, grid, block, 0, st, p)      \
-           : launch_preloaded(qmv_stream_kernel<8, XB, false>, grid, block, 0, st, p))
+#define VPQ_STREAM(XB)                                                                                   \
+  (f16 ? (a.y_f32 ? launch_preloaded(qmv_stream_kernel<8, XB, true, true>, grid, block, 0, st, p)          \
+                  : launch_preloaded(qmv_stream_kernel<8, XB, false, true>, grid, block, 0, st, p))        \
+       : (a.y_f32 ? launch_preloaded(qmv_stream_kernel<8, XB, true>, grid, block, 0, st, p)                \
+                  : launch_preloaded(qmv_stream_kernel<8, XB, false>, grid, block, 0, st, p)))
   if (xbytes <= 13 * 1024) { return VPQ_STREAM(13 * 1024); }
   if (xbytes <= 26 * 1024) { return VPQ_STREAM(26 * 1024); }
   // 42 KB: four rows of K = 5120 (41600 bytes) still leave room for two workgroups per CU; the next size does not
