@@ -489,7 +489,8 @@ int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
                              const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, int scale_only);
 int vpq_qmm_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                        const uint16_t* x, uint16_t* y, int K, int N, int M);
-/* As vpq_qmm_tiled_w8g64_bf16 for the group-32 pack (tile_n 128, -128, 192, 256). */
+/* As vpq_qmm_tiled_w8g64_bf16 for the group-32 pack (tile_n 128, -128, 256; the large-tile kernel has no 192-wide
+ * form for groups of 32: VPQ_ERR_BAD_SHAPE). */
 int vpq_qmm_tiled_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                              const uint16_t* biases, const uint16_t* x, uint16_t* y,
                              int K, int N, int M, int activation, int tile_n);

@@ -1041,11 +1041,12 @@ int twin_gemm_launch(vpq_stream_t stream, const vpq::GemmArgs& g, int tile)
 {
   hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
   if (tile == 192 || tile == 256 || tile == -128) {
-    if (!vpq::qmm_big_supports(g) || (tile == 256 && g.bits == 8)) { return VPQ_ERR_BAD_SHAPE; }
+    // byte codes: up to 192 wide; groups of 32: 256 or 128 wide
+    if (!vpq::qmm_big_supports(g) || (tile == 256 && g.bits == 8) || (tile == 192 && g.group == 32)) { return VPQ_ERR_BAD_SHAPE; }
     return finish(vpq::launch_qmm_big(hs, g, tile < 0 ? -tile : tile));
   }
   if (tile == 0 && vpq::qmm_big_supports(g)) {
-    const int bn = vpq::qmm_big_tile_n(g.N, g.M, g_dev.cu_count, g.bits == 8 ? 192 : 256);
+    const int bn = vpq::qmm_big_tile_n(g.N, g.M, g_dev.cu_count, g.bits == 8 ? 192 : 256, g.group != 32);
     const long tiles = (long)((g.M + 255) / 256) * (long)((g.N + bn - 1) / bn);
     if (tiles >= (long)(g_dev.cu_count > 0 ? g_dev.cu_count : 256)) { return finish(vpq::launch_qmm_big(hs, g, bn)); }
   }

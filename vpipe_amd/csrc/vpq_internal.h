@@ -226,7 +226,7 @@ hipError_t launch_qmm_grouped(hipStream_t st, const GemmArgs& a, const GroupedAr
 // and multiply): K % 512 == 0, 16-byte aligned scales / biases, no gated store; same bits as the tile
 // kernel.  tile_n 0 = qmm_big_tile_n().
 bool qmm_big_supports(const GemmArgs& a);
-int qmm_big_tile_n(int N, int M, int cu_count, int max_width = 256);
+int qmm_big_tile_n(int N, int M, int cu_count, int max_width = 256, bool with_192 = true);
 hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n);
 // Split-K form of the same kernel (no adapter, no gated store): `splits` shares of the K steps,
 // fp32 planes [splits][M][N] in `plane`, then a fold.  qmm_choose_splits() returns 1 where the tiles

@@ -134,18 +134,24 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   constexpr bool W8 = WSRC == kPacked8;     // one byte per code: 64 bytes per row and step, w [N, K/4] words
   constexpr bool G32 = WSRC == kPacked4G32; // groups of 32: two scales and biases per row and step
   static_assert(!(W8 && NT == 4), "byte codes: the doubled code ring fits LDS up to 192-row weight tiles");
+  static_assert(!(G32 && NT == 3), "groups of 32: 256- and 128-row weight tiles only");
   constexpr int CRB = W8 ? 64 : 32;         // bytes of codes per row and step
   constexpr int NC = W8 ? 4 : 2;            // code loads per wavefront and step (1 KB each)
   constexpr int kCodeSlot = W8 ? 64 * NT * 64 : kCodeBytes;
-  constexpr int kWStage = W8 ? 64 * NT * kRow : kWBytes;
+  constexpr int kWStage = 64 * NT * kRow;   // BN rows of 128 bytes
+  // Stages of x.  Two where the window between two barriers (4 NT MFMAs per quarter) is long enough for a request
+  // to L2 to come back; the 128-row tile's window is 32 MFMAs, about the latency itself, so there x is requested a
+  // step further ahead into a third stage (its weight stages are half as large, which is where the room comes from).
+  constexpr int NX = (NT == 2 && !DENSE) ? 3 : 2;
   constexpr int SBLK = G32 ? 4 : 8;         // steps per 16-byte block of a row's scales
   constexpr int BN = 64 * NT;               // weight rows per workgroup
   constexpr int MQ = 4 * NT;                // MFMAs per quarter step (16 of K)
-  // One array per stage and operand.
-  __shared__ __attribute__((aligned(16))) uint8_t x_lds0[kXBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t x_lds1[kXBytes];
-  __shared__ __attribute__((aligned(16))) uint8_t w_lds0[kWStage];
-  __shared__ __attribute__((aligned(16))) uint8_t w_lds1[kWStage];
+  __shared__ __attribute__((aligned(16))) uint8_t x_lds[NX * kXBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t w_lds[2 * kWStage];
+  uint8_t* const x_lds0 = x_lds;
+  uint8_t* const x_lds1 = x_lds + kXBytes;
+  uint8_t* const w_lds0 = w_lds;
+  uint8_t* const w_lds1 = w_lds + kWStage;
   __shared__ __attribute__((aligned(16))) uint8_t c_lds[2 * kCodeSlot];
   __shared__ __attribute__((aligned(16))) uint8_t sb_lds[2 * kScaleBytes];
 
@@ -195,6 +201,10 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   };
   // ---- codes, scales, biases: wavefront w brings in those of rows 64w .. 64w+63 (nothing past BN rows) ----
   const bool dq_wave = wave * 64 < BN;      // wave-uniform
+  // The wavefront's offsets inside the LDS arrays, held in scalar registers for the whole kernel (the empty asm
+  // keeps the compiler from recomputing them from the thread index before every request).
+  uint32_t wave_x = wave * (64 * kRow), wave_c = wave * (64 * CRB), wave_s = wave * (64 * 16), wave_wd = wave * (2 * NT * 8 * kRow);
+  asm volatile("" : "+s"(wave_x), "+s"(wave_c), "+s"(wave_s), "+s"(wave_wd));
   uint32_t c_off[NC];
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
@@ -235,16 +245,18 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   const int sb_row_bytes = G32 ? (p.K >> 4) : (p.K >> 5);     // K/32 or K/64 entries of 2 bytes
   const uint8_t* srow = reinterpret_cast<const uint8_t*>(p.scales) + (size_t)qrg * sb_row_bytes;
   const uint8_t* brow = reinterpret_cast<const uint8_t*>(p.biases) + (size_t)qrg * sb_row_bytes;
+  const uint32_t sb_off = (uint32_t)qrg * (uint32_t)sb_row_bytes;   // the thread's row inside the scales / biases array
+  int sb_due = SBLK < KT ? 0 : 0x7fffffff;  // the window in which the next block of scales and biases is requested
   auto issue_scales = [&](int blk) {
     if (!dq_wave) { return; }
     const uint32_t dst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave * (64 * 16);
     dma16(dst, srow + (size_t)blk * 16);
     dma16(dst + 256 * 16, brow + (size_t)blk * 16);
   };
-  // ---- dequantization: the BN x 8 words of a step's codes are dealt out evenly, thread t takes the WPT
-  // consecutive words from t*WPT on (row-major: word j of row r is 8r + j).  BN = 256: its own row;
-  // BN = 192: six words that may straddle two rows.  d_row is the first row, d_w0 the first word in it.
-  // (Byte codes: a 16-byte piece of the tile, 8 values, is two words; "word" below then means such a pair.)
+  // ---- dequantization: the BN x 8 pieces of a step's weight tile (a piece = 8 values of a row = one 16-byte
+  // store; 4-bit codes: one word of codes, byte codes: two) are dealt out evenly, thread t takes the WPT
+  // consecutive pieces from t*WPT on (row-major: piece j of row r is 8r + j).  BN = 256: its own row; BN = 128:
+  // half a row; BN = 192: six pieces that may straddle two rows.  d_row is the first row, d_w0 the first piece in it.
   constexpr int WPT = 2 * NT;
   constexpr int NCW = W8 ? 2 * WPT : WPT;   // 32-bit words of codes per thread and step
   const int d_row = (tid * WPT) >> 3, d_w0 = (tid * WPT) & 7;
@@ -254,47 +266,13 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     const int row = d_row + ((d_w0 + j) >> 3), word = (d_w0 + j) & 7;
     b_dst[j] = row * kRow + swz(row, word) * 16;
   }
-  // scale and bias of rows d_row and d_row + 1 for step u, the thread's codes of step u
-  // sc / bi [0], [1]: of the thread's pieces before and from piece `sw_at` on.  Group 64: rows d_row and
-  // d_row + 1.  Groups of 32: a thread's pieces lie in at most two (row, half of the step) groups, and the change
-  // is where the position in the row passes a multiple of 4: [0] = (d_row, the half d_w0 lies in), [1] = the
-  // upper half of d_row if d_w0 lies in the lower one, else the lower half of d_row + 1.
+  // A thread's pieces lie in at most two (row, group) sets of scale and bias, A before piece `sw_at` and B from it
+  // on.  Group 64: rows d_row and d_row + 1 (only the 192-row tile reaches B).  Groups of 32: the change is where
+  // the position in the row passes a multiple of 4: A = (d_row, the half d_w0 lies in), B = the upper half of
+  // d_row if d_w0 lies in the lower one, else the lower half of d_row + 1.
   const bool starts_upper = d_w0 >= 4;
   const int sw_at = G32 ? 4 - (d_w0 & 3) : 8 - d_w0;
-  auto load_row_params = [&](int u, float (&sc)[2], float (&bi)[2], uint32_t (&cw)[NCW]) {
-    if constexpr (G32) {
-      const uint8_t* sb = sb_lds + ((u >> 2) & 1) * kScaleBytes + d_row * 16 + (u & 3) * 4;
-      const uint32_t s0 = *reinterpret_cast<const uint32_t*>(sb), s1 = *reinterpret_cast<const uint32_t*>(sb + 16);
-      const uint32_t b0 = *reinterpret_cast<const uint32_t*>(sb + 256 * 16), b1 = *reinterpret_cast<const uint32_t*>(sb + 256 * 16 + 16);
-      const float s0l = bf16_lo_to_f32(s0), s0h = bf16_hi_to_f32(s0), b0l = bf16_lo_to_f32(b0), b0h = bf16_hi_to_f32(b0);
-      sc[0] = starts_upper ? s0h : s0l;
-      bi[0] = starts_upper ? b0h : b0l;
-      sc[1] = starts_upper ? bf16_lo_to_f32(s1) : s0h;
-      bi[1] = starts_upper ? bf16_lo_to_f32(b1) : b0h;
-    } else {
-      const uint8_t* sb = sb_lds + ((u >> 3) & 1) * kScaleBytes + d_row * 16 + (u & 7) * 2;
-      sc[0] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb));
-      bi[0] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 256 * 16));
-      sc[1] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 16));
-      bi[1] = elt_bits_to_f32<F16>(*reinterpret_cast<const uint16_t*>(sb + 256 * 16 + 16));
-    }
-    const uint8_t* cp = c_lds + (u & 1) * kCodeSlot + tid * (NCW * 4);
-    if constexpr (NCW % 4 == 0) {
-#pragma unroll
-      for (int j = 0; j < NCW; j += 4) {
-        const uint4 c4 = *reinterpret_cast<const uint4*>(cp + j * 4);
-        cw[j] = c4.x; cw[j + 1] = c4.y; cw[j + 2] = c4.z; cw[j + 3] = c4.w;
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < NCW; j += 2) {
-        const uint2 c2 = *reinterpret_cast<const uint2*>(cp + j * 4);
-        cw[j] = c2.x;
-        cw[j + 1] = c2.y;
-      }
-    }
-  };
-
+  constexpr bool TWO_SETS = NT == 3 || (G32 && NT == 4);   // the thread's pieces of a step can lie in two sets
   // ---- multiplier side ----
   const int wm = wave >> 1, wn = wave & 1;
   floatx16 acc[NT][4];   // [jt: 32 weight rows][it: 32 x rows]
@@ -335,149 +313,347 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   // read.  Quarter 3's MFMAs then cover the first fragment reads of step s+1, and the work of the window that
   // lasts until the next barrier starts under them:
   //   load requests  x(s+2) [8]; packed: codes(s+3) [2], on steps 8b the scales and biases of block b+1 [2];
-  //                  dense: W(s+2) [8] -- one request every SP MFMAs, all landed at the next barrier;
-  //   packed         the dequantization of W(s+2) into the step's own stage, one piece per MFMA: piece P is word
-  //                  P/8 of the thread's codes at stage P%8 of
-  //                    0: split the nibbles   1..4: two values each, fma(s, q, b)   5: pack to bf16   6: store   7: -
-  // The state of both (fragments, codes, the word in work) lives across steps.
-  constexpr int NLOADS = DENSE ? 8 + 2 * NT : 10 + NC;
-  constexpr int SP = NT == 2 ? 1 : 2;
-  constexpr int NPRE = MQ / SP < NLOADS ? MQ / SP : NLOADS;   // requests made under quarter 3 (slots SP-1, 2SP-1, ...)
+  //                  dense: W(s+2) [2 NT] -- one request every second MFMA, all landed at the next barrier;
+  //   packed         the dequantization of W(s+2) into the step's own stage, a few instructions per MFMA.
+  // The state of both (fragments, codes, the piece in work) lives across steps.
+  //
+  // What a slot may hold.  With one wavefront per SIMD the instructions between two MFMAs issue in that MFMA's
+  // shadow only up to a point: measured on this part (a loop of v_mfma_f32_32x32x16_bf16 with n other instructions
+  // after each, four wavefronts), the MFMA's 32 cycles hold up to 4 further instructions of any kind at +0.5 cycles
+  // each; the fifth and sixth cost 8 cycles each (4 vector instructions + 1 LDS read: 41 against 37), s_nop and
+  // s_waitcnt are free, a 16-byte LDS store of a wavefront occupies the LDS write path for 16-18 cycles, and a
+  // direct-to-LDS load every second slot is free while one in every slot doubles the slot (the same write path).
+  // So the work of a window is cut into single instructions (ops) and dealt out so that no slot holds more than
+  // 4: a fragment read counts 1, a load request 2 (the M0 write and the load; its s_nop is free), and the ops of
+  // the dequantization fill what is left, in order.
+  constexpr int NLOADS = DENSE ? 8 + 2 * NT : 9 + NC;           // packed: codes, one pair of scales and biases, x
+  constexpr int NSLOT = 4 * MQ;                                // slots of a window (barrier to barrier)
+  constexpr int LSTRIDE = 2;                                   // a load request every LSTRIDE-th slot, from slot 1 on
+  // ---- the ops of a window's dequantization (of W(s+2)): NP ops that fetch the thread's codes, scales and biases
+  // from the rings and convert them, then OPW ops per piece:
+  //   4-bit   0 choose set A or B | 1 t = c >> 8 | 2-5 the four nibble pairs in place: c & 000f000f (q0,q4),
+  //           c & 00f000f0 (q1,q5), t & 000f000f (q2,q6), t & 00f000f0 (q3,q7) | 6-13 one v_fma_mix_f32 per value |
+  //           14-17 pack to bf16 pairs | 18 store
+  //   bytes   0 choose | 1-2 t0 = c0 >> 8, t1 = c1 >> 8 | 3-6 c0, t0, c1, t1 & 00ff00ff | 7-14 | 15-18 | 19
+  // A masked code in one half of a register, read as binary16, is the denormal q * 2^-24 (16 q * 2^-24 for the
+  // nibbles left at bits 4-7), which v_fma_mix_f32 widens exactly: fma(q 2^-24, s 2^24, b) has the same exact
+  // product and sum as fma(s, q, b), so the rounded weight has the same bits
+  // (gpu-kernels/metal/quant/affine_qmm_steel.metal:78-96) for every |s| < 2^104 -- with 18 instructions per 8
+  // weights instead of 24 (convert + fma per value).
+  constexpr int RDW = NCW % 4 == 0 ? 4 : 2;                    // words per LDS read of the thread's codes (their alignment)
+  constexpr int NRD = NCW / RDW;
+  constexpr int NP = DENSE ? 0 : NRD + 4;                      // + raw reads A, raw reads B, convert A, convert B
+  constexpr int OPW = W8 ? 20 : 19;
+  constexpr int NOPS = DENSE ? 0 : NP + WPT * OPW;
+  struct Plan {
+    int load_of[NSLOT];        // the request made in a slot, or -1
+    int op_begin[NSLOT + 1];   // the slot's ops are [op_begin[g], op_begin[g + 1])
+  };
+  constexpr auto make_plan = []() constexpr {
+    Plan pl{};
+    int next_load = 0;
+    for (int g = 0; g < NSLOT; ++g) {
+      pl.load_of[g] = (g % LSTRIDE == LSTRIDE - 1 && next_load < NLOADS) ? next_load++ : -1;
+    }
+    int u = 0;
+    for (int g = 0; g < NSLOT; ++g) {
+      pl.op_begin[g] = u;
+      int room = 4 - ((g % MQ) < 4 + NT ? 1 : 0) - (pl.load_of[g] >= 0 ? 2 : 0);
+      while (u < NOPS) {
+        int wgt = 1;
+        if (u < NP) {
+          const int k = u - NRD;                               // 0, 1 raw reads; 2, 3 conversions
+          if (k == 0) { wgt = 2; }
+          if (k == 1) { wgt = (NT == 3) ? 2 : 0; }
+          if (k == 2) { wgt = (W8 ? 2 : 3) + (G32 ? 1 : 0); }
+          if (k == 3) { wgt = TWO_SETS ? (W8 ? 2 : 3) + (G32 ? 1 : 0) : 0; }
+        } else {
+          const int pc = (u - NP) / OPW, op = (u - NP) % OPW;
+          if (op == 0) { wgt = (NT == 3 && pc >= 2) ? (W8 ? 2 : 3) : 0; }
+        }
+        if (wgt > room && room < 4) { break; }                 // does not fit beside what the slot already holds
+        room -= wgt;
+        ++u;
+        if (room <= 0) { break; }
+      }
+    }
+    pl.op_begin[NSLOT] = NOPS;                                 // what did not fit goes to the last slot
+    return pl;
+  };
+  static constexpr Plan plan = make_plan();
+
   bf16x8 wf[2][NT], xf[2][4];                          // operand fragments of the current / the next quarter
-  float sc2[2] = {0.0f, 0.0f}, bi2[2] = {0.0f, 0.0f};  // scale and bias of the thread's one or two groups
-  uint32_t cw[NCW];                                    // its codes of the step being dequantized
+  struct RowSet { float s24, s20, b; };                // scale * 2^24, scale * 2^20, bias
+  RowSet set_a{0.0f, 0.0f, 0.0f}, set_b{0.0f, 0.0f, 0.0f}, cur{0.0f, 0.0f, 0.0f};
+  uint32_t raw_a[2] = {0, 0}, raw_b[2] = {0, 0};       // scale and bias as read from the ring
+  uint32_t cw[NCW];                                    // the thread's codes of the step being dequantized
 #pragma unroll
   for (int j = 0; j < NCW; ++j) { cw[j] = 0; }
-  float sc = 0.0f, bi = 0.0f;                          // of the word in work
-  uint32_t lo = 0, hi = 0;
+  uint32_t t0 = 0, t1 = 0, mk[4] = {0, 0, 0, 0};
   float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   uint4 o = make_uint4(0, 0, 0, 0);
+  // Three stages of x: the stage of a step is a run-time offset (xo_*), and the fragment reads of quarter ks go
+  // through xa[ks], the LDS address of the lane's piece of x fragment 0 in the stage that quarter is read from next.
+  uint32_t xo_prev = 2 * kXBytes, xo_cur = 0, xo_next = kXBytes;   // stages of steps s-1, s, s+1 (bytes into x_lds)
+  uint32_t xa_base[4], xa[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    xa_base[ks] = lds_addr(x_lds) + (uint32_t)x_rd[0] + (uint32_t)(((2 * ks + fkh) ^ f_sw) * 16);
+    xa[ks] = xa_base[ks];
+  }
   auto frag = [&](const uint8_t* xb, const uint8_t* wb, int buf, int ks, int idx) {   // idx: 0 = w0, 1..4 = x0..x3, 5.. = w1..
     const int c = ((2 * ks + fkh) ^ f_sw) * 16;
     if (idx == 0) {
       wf[buf][0] = *reinterpret_cast<const bf16x8*>(wb + w_rd[0] + c);
     } else if (idx <= 4) {
+      if constexpr (NX == 3) {
+        if (xb == nullptr) {     // (decided at compile time: every call passes a literal) read through xa[ks]
+          xf[buf][idx - 1] = *(__attribute__((address_space(3))) const bf16x8*)(uintptr_t)(xa[ks] + (uint32_t)(idx - 1) * (32 * kRow));
+          return;
+        }
+      }
       xf[buf][idx - 1] = *reinterpret_cast<const bf16x8*>(xb + x_rd[idx - 1] + c);
     } else {
       wf[buf][idx - 4] = *reinterpret_cast<const bf16x8*>(wb + w_rd[idx - 4] + c);
     }
   };
-  auto piece = [&](auto pc, uint8_t* nb) {
-    constexpr int P = decltype(pc)::value;
-    constexpr int W = P >> 3, S = P & 7;
-    if constexpr (S == 0) {
-      if constexpr (W8) {
-        lo = cw[2 * W];                                // q0 q1 q2 q3
-        hi = cw[2 * W + 1];                            // q4 q5 q6 q7
+  // Single instructions of the dequantization, as volatile asm so that each stays in the slot it is written in (the
+  // scheduling barriers pin machine instructions, but the compiler would still sink plain arithmetic to its first
+  // use before they apply).  fma(binary16 half HI of `code` widened, scale, bias):
+  auto mix = [](auto hi_c, uint32_t code, float scale, float bias) {
+    float r;
+    if constexpr (decltype(hi_c)::value) {
+      asm volatile("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(code), "v"(scale), "v"(bias));
+    } else {
+      asm volatile("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(code), "v"(scale), "v"(bias));
+    }
+    return r;
+  };
+  auto shr8 = [](uint32_t c) { uint32_t r; asm volatile("v_lshrrev_b32 %0, 8, %1" : "=v"(r) : "v"(c)); return r; };
+  auto andm = [](uint32_t c, uint32_t m) { uint32_t r; asm volatile("v_and_b32 %0, %1, %2" : "=v"(r) : "s"(m), "v"(c)); return r; };
+  auto pk2 = [](float a, float b) {
+    uint32_t r;
+    if constexpr (F16) { asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b)); }
+    else { asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b)); }
+    return r;
+  };
+  auto pick = [](float a, float b, uint64_t second) {   // second ? b : a, per lane
+    float r;
+    asm volatile("v_cndmask_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "s"(second));
+    return r;
+  };
+  uint32_t mask_lo = W8 ? 0x00ff00ffu : 0x000f000fu, mask_hi = 0x00f000f0u;
+  asm volatile("" : "+s"(mask_lo), "+s"(mask_hi));       // in scalar registers: no literal in every instruction
+  auto to_set = [](uint32_t sbits, uint32_t bbits) {
+    const float sc = elt_bits_to_f32<F16>(sbits);
+    return RowSet{sc * 16777216.0f, sc * 1048576.0f, elt_bits_to_f32<F16>(bbits)};
+  };
+  // Op U of the window that dequantizes W(u) into the stage `nb`.
+  auto dq_op = [&](auto uc, int u, uint8_t* nb) {
+    constexpr int U = decltype(uc)::value;
+    if constexpr (U < NRD) {
+      const uint8_t* cp = c_lds + (u & 1) * kCodeSlot + tid * (NCW * 4) + U * (RDW * 4);
+      if constexpr (RDW == 4) {
+        const uint4 c4 = *reinterpret_cast<const uint4*>(cp);
+        cw[4 * U] = c4.x; cw[4 * U + 1] = c4.y; cw[4 * U + 2] = c4.z; cw[4 * U + 3] = c4.w;
       } else {
-        lo = cw[W] & 0x0f0f0f0fu;                      // q0 q2 q4 q6
-        hi = (cw[W] >> 4) & 0x0f0f0f0fu;               // q1 q3 q5 q7
-        // No instruction: keeps the masked words as they are, so that each value is one v_cvt_f32_ubyteN
-        // of them (otherwise the mask is folded into a bit-field extract per value, one instruction more).
-        asm volatile("" : "+v"(lo), "+v"(hi));
+        const uint2 c2 = *reinterpret_cast<const uint2*>(cp);
+        cw[2 * U] = c2.x; cw[2 * U + 1] = c2.y;
       }
-      if constexpr (NT == 4) {                         // the thread's own row; groups of 32: pieces 4-7 second group
-        sc = sc2[G32 ? (W >> 2) : 0]; bi = bi2[G32 ? (W >> 2) : 0];
+    } else if constexpr (U < NP) {
+      constexpr int k = U - NRD;
+      // group 64: 2-byte entries, 8 steps per 16-byte block of a row; groups of 32: a dword of two entries per step
+      const uint8_t* sb = G32 ? sb_lds + ((u >> 2) & 1) * kScaleBytes + d_row * 16 + (u & 3) * 4
+                              : sb_lds + ((u >> 3) & 1) * kScaleBytes + d_row * 16 + (u & 7) * 2;
+      if constexpr (k == 0) {
+        if constexpr (G32) {
+          raw_a[0] = *reinterpret_cast<const uint32_t*>(sb); raw_a[1] = *reinterpret_cast<const uint32_t*>(sb + 256 * 16);
+        } else {
+          raw_a[0] = *reinterpret_cast<const uint16_t*>(sb); raw_a[1] = *reinterpret_cast<const uint16_t*>(sb + 256 * 16);
+        }
+      } else if constexpr (k == 1) {
+        if constexpr (NT == 3) {                               // the next row's
+          if constexpr (G32) {
+            raw_b[0] = *reinterpret_cast<const uint32_t*>(sb + 16); raw_b[1] = *reinterpret_cast<const uint32_t*>(sb + 256 * 16 + 16);
+          } else {
+            raw_b[0] = *reinterpret_cast<const uint16_t*>(sb + 16); raw_b[1] = *reinterpret_cast<const uint16_t*>(sb + 256 * 16 + 16);
+          }
+        }
+      } else if constexpr (k == 2) {
+        if constexpr (G32) {
+          const uint32_t sh = (NT == 4 || !starts_upper) ? 0u : 16u;   // NT == 4: set A is the lower half of the row's step
+          if constexpr (NT == 4) { set_a = to_set(raw_a[0] & 0xffffu, raw_a[1] & 0xffffu); }
+          else { set_a = to_set((raw_a[0] >> sh) & 0xffffu, (raw_a[1] >> sh) & 0xffffu); }
+        } else {
+          set_a = to_set(raw_a[0], raw_a[1]);
+        }
       } else {
-        const bool second = W >= sw_at;
-        sc = second ? sc2[1] : sc2[0];
-        bi = second ? bi2[1] : bi2[0];
+        if constexpr (G32 && NT == 4) { set_b = to_set(raw_a[0] >> 16, raw_a[1] >> 16); }
+        else if constexpr (G32 && NT == 3) {
+          // the lower half of the next row, or the upper half of this one: choose the bits, convert once
+          const uint32_t sbits = starts_upper ? (raw_b[0] & 0xffffu) : (raw_a[0] >> 16);
+          const uint32_t bbits = starts_upper ? (raw_b[1] & 0xffffu) : (raw_a[1] >> 16);
+          set_b = to_set(sbits, bbits);
+        } else if constexpr (NT == 3) { set_b = to_set(raw_b[0], raw_b[1]); }
       }
-    } else if constexpr (W8 && S >= 1 && S <= 4) {
-      if constexpr (S == 1) { v[0] = fmaf(sc, ubyte_f32<0>(lo), bi); v[4] = fmaf(sc, ubyte_f32<0>(hi), bi); }
-      if constexpr (S == 2) { v[1] = fmaf(sc, ubyte_f32<1>(lo), bi); v[5] = fmaf(sc, ubyte_f32<1>(hi), bi); }
-      if constexpr (S == 3) { v[2] = fmaf(sc, ubyte_f32<2>(lo), bi); v[6] = fmaf(sc, ubyte_f32<2>(hi), bi); }
-      if constexpr (S == 4) { v[3] = fmaf(sc, ubyte_f32<3>(lo), bi); v[7] = fmaf(sc, ubyte_f32<3>(hi), bi); }
-    } else if constexpr (S == 1) {
-      v[0] = fmaf(sc, ubyte_f32<0>(lo), bi); v[1] = fmaf(sc, ubyte_f32<0>(hi), bi);
-    } else if constexpr (S == 2) {
-      v[2] = fmaf(sc, ubyte_f32<1>(lo), bi); v[3] = fmaf(sc, ubyte_f32<1>(hi), bi);
-    } else if constexpr (S == 3) {
-      v[4] = fmaf(sc, ubyte_f32<2>(lo), bi); v[5] = fmaf(sc, ubyte_f32<2>(hi), bi);
-    } else if constexpr (S == 4) {
-      v[6] = fmaf(sc, ubyte_f32<3>(lo), bi); v[7] = fmaf(sc, ubyte_f32<3>(hi), bi);
-    } else if constexpr (S == 5) {
-      o.x = pack_elt2<F16>(v[0], v[1]); o.y = pack_elt2<F16>(v[2], v[3]);
-      o.z = pack_elt2<F16>(v[4], v[5]); o.w = pack_elt2<F16>(v[6], v[7]);
-    } else if constexpr (S == 6) {
-      *reinterpret_cast<uint4*>(nb + b_dst[W]) = o;
+    } else {
+      constexpr int PC = (U - NP) / OPW, OP = (U - NP) % OPW;
+      if constexpr (OP == 0) {
+        if constexpr (NT == 3 && PC >= 2) {
+          const uint64_t second = __builtin_amdgcn_ballot_w64(PC >= sw_at);
+          cur.s24 = pick(set_a.s24, set_b.s24, second);
+          if constexpr (!W8) { cur.s20 = pick(set_a.s20, set_b.s20, second); }
+          cur.b = pick(set_a.b, set_b.b, second);
+        } else if constexpr (G32 && NT == 4 && PC == 4) {
+          cur = set_b;                                         // no instruction: the second half of the row's step
+        } else if constexpr (PC == 0) {
+          cur = set_a;
+        }
+      } else if constexpr (W8) {
+        const uint32_t c0 = cw[2 * PC], c1 = cw[2 * PC + 1];   // q0 q1 q2 q3 | q4 q5 q6 q7, a byte each
+        if constexpr (OP == 1) { t0 = shr8(c0); }
+        if constexpr (OP == 2) { t1 = shr8(c1); }
+        if constexpr (OP == 3) { mk[0] = andm(c0, mask_lo); }  // q0, q2
+        if constexpr (OP == 4) { mk[1] = andm(t0, mask_lo); }  // q1, q3
+        if constexpr (OP == 5) { mk[2] = andm(c1, mask_lo); }  // q4, q6
+        if constexpr (OP == 6) { mk[3] = andm(t1, mask_lo); }  // q5, q7
+        if constexpr (OP == 7) { v[0] = mix(No(), mk[0], cur.s24, cur.b); }
+        if constexpr (OP == 8) { v[1] = mix(No(), mk[1], cur.s24, cur.b); }
+        if constexpr (OP == 9) { v[2] = mix(Yes(), mk[0], cur.s24, cur.b); }
+        if constexpr (OP == 10) { v[3] = mix(Yes(), mk[1], cur.s24, cur.b); }
+        if constexpr (OP == 11) { v[4] = mix(No(), mk[2], cur.s24, cur.b); }
+        if constexpr (OP == 12) { v[5] = mix(No(), mk[3], cur.s24, cur.b); }
+        if constexpr (OP == 13) { v[6] = mix(Yes(), mk[2], cur.s24, cur.b); }
+        if constexpr (OP == 14) { v[7] = mix(Yes(), mk[3], cur.s24, cur.b); }
+        if constexpr (OP >= 15 && OP <= 18) {
+          const uint32_t pk = pk2(v[2 * (OP - 15)], v[2 * (OP - 15) + 1]);
+          if constexpr (OP == 15) { o.x = pk; } else if constexpr (OP == 16) { o.y = pk; }
+          else if constexpr (OP == 17) { o.z = pk; } else { o.w = pk; }
+        }
+        if constexpr (OP == 19) { *reinterpret_cast<uint4*>(nb + b_dst[PC]) = o; }
+      } else {
+        const uint32_t c = cw[PC];
+        if constexpr (OP == 1) { t0 = shr8(c); }
+        if constexpr (OP == 2) { mk[0] = andm(c, mask_lo); }   // q0, q4
+        if constexpr (OP == 3) { mk[1] = andm(c, mask_hi); }   // 16 q1, 16 q5
+        if constexpr (OP == 4) { mk[2] = andm(t0, mask_lo); }  // q2, q6
+        if constexpr (OP == 5) { mk[3] = andm(t0, mask_hi); }  // 16 q3, 16 q7
+        if constexpr (OP == 6) { v[0] = mix(No(), mk[0], cur.s24, cur.b); }
+        if constexpr (OP == 7) { v[1] = mix(No(), mk[1], cur.s20, cur.b); }
+        if constexpr (OP == 8) { v[2] = mix(No(), mk[2], cur.s24, cur.b); }
+        if constexpr (OP == 9) { v[3] = mix(No(), mk[3], cur.s20, cur.b); }
+        if constexpr (OP == 10) { v[4] = mix(Yes(), mk[0], cur.s24, cur.b); }
+        if constexpr (OP == 11) { v[5] = mix(Yes(), mk[1], cur.s20, cur.b); }
+        if constexpr (OP == 12) { v[6] = mix(Yes(), mk[2], cur.s24, cur.b); }
+        if constexpr (OP == 13) { v[7] = mix(Yes(), mk[3], cur.s20, cur.b); }
+        if constexpr (OP >= 14 && OP <= 17) {
+          const uint32_t pk = pk2(v[2 * (OP - 14)], v[2 * (OP - 14) + 1]);
+          if constexpr (OP == 14) { o.x = pk; } else if constexpr (OP == 15) { o.y = pk; }
+          else if constexpr (OP == 16) { o.z = pk; } else { o.w = pk; }
+        }
+        if constexpr (OP == 18) { *reinterpret_cast<uint4*>(nb + b_dst[PC]) = o; }
+      }
     }
   };
-  // Request I of the window that opens behind the barrier of step `win`: x(win+2) goes to the stage of step win.
-  auto window_load = [&](auto ic, int win, auto stage_c) {
+  // Request I of the window that opens behind the barrier of step `win`: x(win + NX) goes to the stage of step win
+  // (`xo_win` where there are three).  Packed: the codes and the scales come first and x last, so that with three
+  // stages the window's barrier can leave the x requests in flight (they are not needed before the one after).
+  auto window_load = [&](auto ic, int win, auto stage_c, uint32_t xo_win) {
     constexpr int I = decltype(ic)::value;
     constexpr int STG = decltype(stage_c)::value;
     const int step_to = win + 2;
-    const uint32_t xdst = lds_addr(STG ? x_lds1 : x_lds0) + wave * (64 * kRow);
-    const uint8_t* xsrc = xblk + (size_t)step_to * (BK * 2);
     if constexpr (DENSE) {
+      const uint32_t xdst = lds_addr(STG ? x_lds1 : x_lds0) + wave_x;
       if constexpr (I < NWL) {
-        const uint32_t wdst = lds_addr(STG ? w_lds1 : w_lds0) + wave * (NWL * 8 * kRow);
+        const uint32_t wdst = lds_addr(STG ? w_lds1 : w_lds0) + wave_wd;
         dma16(wdst + I * (8 * kRow), wblk + (size_t)step_to * (BK * 2), wd_off[I]);
       } else {
-        dma16(xdst + (I - NWL) * (8 * kRow), xsrc, a_off[I - NWL]);
+        dma16(xdst + (I - NWL) * (8 * kRow), xblk + (size_t)step_to * (BK * 2), a_off[I - NWL]);
       }
     } else {
-      if constexpr (I < 8) {
-        dma16(xdst + I * (8 * kRow), xsrc, a_off[I]);
-      } else if constexpr (I < 8 + NC) {                // codes(win+3) into the slot codes(win+1) have left
-        if (win + 3 < KT && dq_wave) {
-          dma16(lds_addr(c_lds) + (1 - STG) * kCodeSlot + wave * (64 * CRB) + (I - 8) * 1024,
-                wblk + (size_t)(win + 3) * CRB, c_off[I - 8]);
+      if constexpr (I < NC) {
+        // codes(win+3) into the slot codes(win+1) have left.  Past the last step the last step's codes are read
+        // again (nobody uses them) rather than branching round the request; 4-bit codes: every wavefront brings in
+        // 64 rows of the 256-row slot, tile rows or not.
+        const int cstep = win + 3 < KT ? win + 3 : KT - 1;
+        if (!W8 || dq_wave) {
+          dma16(lds_addr(c_lds) + (1 - STG) * kCodeSlot + wave_c + I * 1024, wblk + (size_t)cstep * CRB, c_off[I]);
+        }
+      } else if constexpr (I == NC) {
+        // scales and biases of the next block of steps, both in this slot, when the window's step starts a block
+        if (win == sb_due) {
+          const int blk = (win >> (G32 ? 2 : 3)) + 1;
+          const uint32_t sdst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave_s;
+          dma16(sdst, reinterpret_cast<const uint8_t*>(p.scales) + (size_t)blk * 16, sb_off);
+          dma16(sdst + 256 * 16, reinterpret_cast<const uint8_t*>(p.biases) + (size_t)blk * 16, sb_off);
+          sb_due = win + 2 * SBLK < KT ? win + SBLK : 0x7fffffff;
         }
       } else {
-        const int blk = (win >> (G32 ? 2 : 3)) + 1;
-        if ((win & (SBLK - 1)) == 0 && win + SBLK < KT && dq_wave) {
-          const uint32_t sdst = lds_addr(sb_lds) + (blk & 1) * kScaleBytes + wave * (64 * 16);
-          if constexpr (I == 8 + NC) { dma16(sdst, srow + (size_t)blk * 16); }
-          else { dma16(sdst + 256 * 16, brow + (size_t)blk * 16); }
+        constexpr int X = I - NC - 1;
+        if constexpr (NX == 3) {
+          // past the last step the last step's tile is read again, into a stage nobody reads any more
+          const int xstep = win + 3 < KT ? win + 3 : KT - 1;
+          dma16(lds_addr(x_lds) + xo_win + wave_x + X * (8 * kRow), xblk + (size_t)xstep * (BK * 2), a_off[X]);
+        } else {
+          dma16(lds_addr(STG ? x_lds1 : x_lds0) + wave_x + X * (8 * kRow), xblk + (size_t)step_to * (BK * 2), a_off[X]);
         }
       }
     }
   };
-  // Step s on stage ST.  m1: a step s+1 exists, m2: a step s+2 exists (std::true_type / std::false_type, or bool
-  // where the choice is left to run time).
+  // Slot G of the window behind the barrier of step `win`: its request, its ops (they dequantize W(win+2) into `nb`).
+  auto window_slot = [&](auto gc, int win, auto stage_c, uint32_t xo_win, uint8_t* nb) {
+    constexpr int G = decltype(gc)::value;
+    if constexpr (plan.load_of[G] >= 0) { window_load(std::integral_constant<int, plan.load_of[G]>(), win, stage_c, xo_win); }
+    if constexpr (!DENSE) {
+      static_for<plan.op_begin[G], plan.op_begin[G + 1]>([&](auto uc) { dq_op(uc, win + 2, nb); });
+    }
+  };
+  // Step s on stage ST.  m1: a step s+1 exists, m2: a step s+2 exists (std::true_type / std::false_type).
   auto pstep = [&](auto stage_c, auto m1, auto m2, int s) {
     constexpr int ST = decltype(stage_c)::value;
     using Nx = std::integral_constant<int, 1 - ST>;
-    const uint8_t* xb = ST ? x_lds1 : x_lds0;
+    const uint8_t* xb = NX == 3 ? nullptr : (ST ? x_lds1 : x_lds0);
     const uint8_t* wb = ST ? w_lds1 : w_lds0;
-    const uint8_t* nxb = ST ? x_lds0 : x_lds1;
+    const uint8_t* nxb = NX == 3 ? nullptr : (ST ? x_lds0 : x_lds1);
     uint8_t* nwb = ST ? w_lds0 : w_lds1;
     uint8_t* ownb = ST ? w_lds1 : w_lds0;
     static_for<0, 4>([&](auto qc) {
       constexpr int Q = decltype(qc)::value;
       constexpr int B = Q & 1;
-      if constexpr (Q == 3 && !DENSE) { when(m2, [&] { load_row_params(s + 2, sc2, bi2, cw); }); }
-      {
-        static_for<0, MQ>([&](auto jc) {
-          constexpr int J = decltype(jc)::value;
-          constexpr int JT = J >> 2, IT = J & 3;
-          acc[JT][IT] = mfma(wf[B][JT], xf[B][IT], acc[JT][IT]);
-          constexpr int GB = Q == 3 ? J : MQ * (Q + 1) + J;    // MFMA slot counted from the previous barrier
-          if constexpr (!DENSE) {
-            if constexpr (Q == 3) { when(m2, [&] { piece(std::integral_constant<int, GB>(), ownb); }); }
-            else { when(m1, [&] { piece(std::integral_constant<int, GB>(), nwb); }); }
-          }
-          if constexpr (GB % SP == SP - 1 && GB / SP < NLOADS) {
-            if constexpr (Q == 3) { when(m2, [&] { window_load(std::integral_constant<int, GB / SP>(), s, stage_c); }); }
-            else { when(m1, [&] { window_load(std::integral_constant<int, GB / SP>(), s - 1, Nx()); }); }
-          }
-          // the next quarter's fragments, one read after every MFMA until they are all requested
-          if constexpr (J < 4 + NT) {
-            if constexpr (Q < 3) { frag(xb, wb, 1 - B, Q + 1, J); }
-            else { when(m1, [&] { frag(nxb, nwb, 0, 0, J); }); }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      }
+      static_for<0, MQ>([&](auto jc) {
+        constexpr int J = decltype(jc)::value;
+        constexpr int JT = J >> 2, IT = J & 3;
+        acc[JT][IT] = mfma(wf[B][JT], xf[B][IT], acc[JT][IT]);
+        constexpr int GB = Q == 3 ? J : MQ * (Q + 1) + J;    // slot counted from the previous barrier
+        if constexpr (Q == 3) { when(m2, [&] { window_slot(std::integral_constant<int, GB>(), s, stage_c, xo_cur, ownb); }); }
+        else { when(m1, [&] { window_slot(std::integral_constant<int, GB>(), s - 1, Nx(), xo_prev, nwb); }); }
+        // the next quarter's fragments, one read after every MFMA until they are all requested
+        if constexpr (J < 4 + NT) {
+          if constexpr (Q < 3) { frag(xb, wb, 1 - B, Q + 1, J); }
+          else { when(m1, [&] { frag(nxb, nwb, 0, 0, J); }); }
+        }
+        if constexpr (NX == 3) {
+          // quarter Q's reads (of k slice Q + 1) are out: that slice's address moves on to the next step's stage;
+          // slice 0, read under quarter 3, moves before it
+          if constexpr (J == 4 + NT && Q < 3) { xa[Q + 1] = xa_base[Q + 1] + xo_next; }
+          if constexpr (J == 4 + NT + 1 && Q == 2) { xa[0] = xa_base[0] + xo_next; }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
       if constexpr (Q == 2) {
         when(m1, [&] {
-          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          // everything this wavefront asked for has landed -- with three stages of x all but the window's own 8
+          // requests for x, which came last and are read two barriers on
+          if constexpr (NX == 3) { asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory"); }
+          else { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
           wg_barrier();
         });
       }
     });
+    if constexpr (NX == 3) {
+      const uint32_t t = xo_prev;
+      xo_prev = xo_cur; xo_cur = xo_next; xo_next = t;
+    }
   };
 
   // `nq` quarter steps (16 of K each) on the tiles in stage 0, nothing overlapped: for the short extra pieces of K
@@ -492,47 +668,61 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   };
 
   if (KT > 0) {
-    // ---- prologue: stage 0 complete (x(0); W(0) loaded or dequantized), the part of step 1's window that a
-    // quarter 3 before step 0 would have done, the first fragments ----
-    if constexpr (DENSE) {
-      issue_wdense(0, S0());
-      issue_x(0, S0());
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      wg_barrier();
-    } else {
-      issue_scales(0);
-      issue_codes(0);
-      issue_codes(1);
-      issue_x(0, S0());
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      wg_barrier();                             // the codes and scales a thread reads were brought in by any wavefront
-      load_row_params(0, sc2, bi2, cw);
-      static_for<0, 4 * MQ>([&](auto pc) { piece(pc, w_lds0); });
-      load_row_params(1, sc2, bi2, cw);
-      static_for<0, MQ>([&](auto pc) { piece(pc, w_lds1); });
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      wg_barrier();
-    }
-    if (KT > 1) { static_for<0, NPRE>([&](auto ic) { window_load(ic, -1, S1()); }); }
+    // Steps alternate between the two stages and the last step runs on stage 1, so that the written-out last steps
+    // are the same for every K: an odd number of steps (dense weights only) starts on stage 1, as if a step on
+    // stage 0 had gone before.
+    const bool odd = DENSE && (KT & 1) != 0;
+    // ---- prologue: the first step's stage complete (x(0); W(0) loaded or dequantized), the part of step 1's
+    // window that a quarter 3 before step 0 would have done, the first fragments ----
+    auto prologue = [&](auto first_c) {
+      constexpr int P0 = decltype(first_c)::value;
+      using Other = std::integral_constant<int, 1 - P0>;
+      if constexpr (DENSE) {
+        issue_wdense(0, first_c);
+        issue_x(0, first_c);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wg_barrier();
+      } else {
+        issue_scales(0);
+        issue_codes(0);
+        issue_codes(1);
+        issue_x(0, first_c);
+        if constexpr (NX == 3) { issue_x(1, S1()); }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wg_barrier();                           // the codes and scales a thread reads were brought in by any wavefront
+        static_for<0, NOPS>([&](auto uc) { dq_op(uc, 0, w_lds0); });
+        static_for<0, plan.op_begin[MQ]>([&](auto uc) { dq_op(uc, 1, w_lds1); });
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wg_barrier();
+      }
+      if (KT > 1) {
+        static_for<0, MQ>([&](auto gc) {
+          if constexpr (plan.load_of[decltype(gc)::value] >= 0) {
+            window_load(std::integral_constant<int, plan.load_of[decltype(gc)::value]>(), -1, Other(), xo_prev);
+          }
+        });
+      }
 #pragma unroll
-    for (int i = 0; i < 4 + NT; ++i) { frag(x_lds0, w_lds0, 0, 0, i); }
-
-    // ---- K loop.  Packed: no condition surrounds the arithmetic inside it, the last two steps are written out
-    // (K is a multiple of 512).  Dense: any number of steps, the conditions are wave-uniform branches. ----
+      for (int i = 0; i < 4 + NT; ++i) { frag(P0 ? x_lds1 : x_lds0, P0 ? w_lds1 : w_lds0, 0, 0, i); }
+      if constexpr (NX == 3) { xa[0] = xa_base[0] + xo_next; }   // as a quarter 2 before step 0 would have left it
+    };
     if constexpr (DENSE) {
-      for (int s = 0; s < KT; s += 2) {
-        pstep(S0(), s + 1 < KT, s + 2 < KT, s);
-        if (s + 1 < KT) { pstep(S1(), s + 2 < KT, s + 3 < KT, s + 1); }
-      }
+      if (odd) { prologue(S1()); } else { prologue(S0()); }
     } else {
-      int s = 0;
-      for (; s + 3 < KT; s += 2) {
-        pstep(S0(), Yes(), Yes(), s);
-        pstep(S1(), Yes(), Yes(), s + 1);
-      }
-      pstep(S0(), Yes(), No(), s);
-      pstep(S1(), No(), No(), s + 1);
+      prologue(S0());
     }
+
+    // ---- K loop.  No condition surrounds the arithmetic inside a step: the last two steps are written out.  With
+    // an odd number of steps the count runs from -1 and the step on stage 0 that would be step -1 is skipped. ----
+    int s = DENSE ? -(KT & 1) : 0;
+    if constexpr (DENSE) { asm volatile("" : "+s"(s)); }   // stays in a scalar register (it feeds the request addresses)
+    for (; s + 3 < KT; s += 2) {
+      if (s >= 0) { pstep(S0(), Yes(), Yes(), s); }
+      pstep(S1(), Yes(), Yes(), s + 1);
+    }
+    if (s >= 0) { pstep(S0(), Yes(), No(), s); }
+    pstep(S1(), No(), No(), s + 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // three stages: the repeated last requests, before LDS is reused
   }
 
   if constexpr (DENSE) {
@@ -714,7 +904,7 @@ bool qmm_big_supports(const GemmArgs& a)
 // (measured with whole rounds: 256 wide 1.02, 192 wide 0.98, 128 wide 0.94 PFLOP/s).  4096 -> 12288 at
 // M = 2048: 384 tiles of 256 are one and a half rounds of 256 CUs, 512 tiles of 192 are two;
 // N = 4096 at M = 2048 is exactly one round of 128-wide tiles.
-int qmm_big_tile_n(int N, int M, int cu_count, int max_width)
+int qmm_big_tile_n(int N, int M, int cu_count, int max_width, bool with_192)
 {
   const int cus = cu_count > 0 ? cu_count : 256;
   const long tm = (M + BM - 1) / BM;
@@ -724,6 +914,7 @@ int qmm_big_tile_n(int N, int M, int cu_count, int max_width)
   int best = widths[first];
   double best_cost = 0.0;
   for (int i = first; i < 3; ++i) {
+    if (widths[i] == 192 && !with_192) { continue; }     // groups of 32: 256 and 128 wide only
     const long tiles = tm * ((N + widths[i] - 1) / widths[i]);
     const long rounds = (tiles + cus - 1) / cus;
     const double cost = (double)rounds * (double)widths[i] / eff[i];
@@ -756,8 +947,9 @@ unsigned plan_tile_order(BigParams& p)
 hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
 {
   const int widest = a.bits == 8 ? 192 : 256;
-  const int bn = tile_n == 128 || tile_n == 192 || (tile_n == 256 && widest == 256) ? tile_n
-                                                                                  : qmm_big_tile_n(a.N, a.M, a.cu_count, widest);
+  const bool with_192 = a.group != 32;
+  const int bn = tile_n == 128 || (tile_n == 192 && with_192) || (tile_n == 256 && widest == 256)
+                     ? tile_n : qmm_big_tile_n(a.N, a.M, a.cu_count, widest, with_192);
   BigParams p;
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
   p.lora_t = a.lora_t; p.lora_b = a.lora_b;
@@ -776,8 +968,9 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
   }
   if (a.group == 32) {
     if (lora || a.f16) { return hipErrorInvalidValue; }
+    // 256 and 128 wide only: the 192-wide tile, whose threads' pieces change between two (row, half step) sets at a
+    // place that differs from thread to thread, does not fit the registers beside the accumulators
     if (bn == 128) { return launch_kernel(qmm_big_kernel<2, false, kPacked4G32>, grid, block, 0, st, p); }
-    if (bn == 192) { return launch_kernel(qmm_big_kernel<3, false, kPacked4G32>, grid, block, 0, st, p); }
     return launch_kernel(qmm_big_kernel<4, false, kPacked4G32>, grid, block, 0, st, p);
   }
   if (a.f16) {

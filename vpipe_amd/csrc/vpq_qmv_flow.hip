@@ -160,30 +160,24 @@ __device__ __forceinline__ void pin_scalar(const T& v) { asm volatile("" : : "s"
 }  // namespace
 
 
-// XM: how x reaches a wavefront's registers.
-//   kXOwn     each wavefront loads its own lanes' values (4 KB per slice and wavefront, from L2 after the first
-//             wavefront); scales and biases are requested first, x second, the codes last; no barrier.
-//   kXShared  the workgroup's K range of x is copied to LDS once by direct-to-LDS loads shared between its
-//             wavefronts (one barrier); the codes are requested right after the wavefront's share of x, scales and
-//             biases last.  Pays where a row set's x is large against its codes (long K).
-// Either way the scales and biases are applied to the per-(row, slice) dot products at the end, in the same order:
-// the two modes give the same bits.
-constexpr int kXOwn = 0, kXShared = 1;
-
+// x reaches a wavefront through LDS: the workgroup's K range of x is copied there once by direct-to-LDS loads
+// shared between its wavefronts (one barrier); the codes are requested right after the wavefront's share of x,
+// scales and biases last, and they are applied to the per-(row, slice) dot products at the end.
+//
 // F16: the elements (x, scales, biases, y, residual) are IEEE binary16 instead of bf16 (the reference's
 // VPIPE_ELT = half build).  The codes then become binary16 pairs 16 + q (the code shifted to mantissa bits 6..9,
 // exact; 1024 + q with the code left in bits 0..3 would cost eight times bf16's cancellation noise).
 // PRELOADED: the arguments are already in scalar registers (nothing to batch; the residual is left to be loaded
 // when the store needs it).
-template <int SPW, int RB, bool F32OUT, int XM, int C, bool F16 = false, bool PRELOADED = false>
+template <int SPW, int RB, bool F32OUT, int C, bool F16 = false, bool PRELOADED = false>
 __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
 {
   constexpr int NL = RB * SPW;                 // code loads of a wavefront
   constexpr int PPR = SPW * 4;                 // 16-byte pieces of scales (or biases) per row and K part
   constexpr int P = RB * PPR;
   constexpr int NDMA = (2 * P + 63) / 64;
-  // LDS: [kXShared: x of the workgroup's K range, wk * SPW slices of 4 KB,] one window of scales/biases per
-  // wavefront, the row sums of the K parts.
+  // LDS: x of the workgroup's K range (wk * SPW slices of 4 KB), one window of scales/biases per wavefront, the
+  // row sums of the K parts.
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   // ---- arguments: everything in one batch of scalar loads, the segment chosen without branches
@@ -233,9 +227,8 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
   const int Kg = K >> 6;
   const int row_begin = ((blk - first_block) * wr + rs) * RB;
   const bool active = row_begin < N;           // wave-uniform
-  if (XM == kXOwn && wk == 1 && !active) { return; }
   const int slice0 = part * SPW;
-  const int x_bytes = XM == kXShared ? wk * SPW * (kSlice * 2) : 0;
+  const int x_bytes = wk * SPW * (kSlice * 2);
   uint8_t* sbl = lds + x_bytes + wave * (NDMA * 1024);
   float* red = reinterpret_cast<float*>(lds + x_bytes + W * (NDMA * 1024));
   const uint32_t lds_a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)lds;
@@ -270,8 +263,7 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
     }
   };
 
-  u32x4v xr[XM == kXOwn ? SPW : 1][4];
-  if (XM == kXShared) {
+  {
     // x of the workgroup's K range -> LDS, the wavefronts taking the 1 KB pieces round-robin.  Piece j is
     // quarter t = j % 4 of slice j / 4: lane i brings the 16 bytes at values 32 i + 8 t of the slice, so that a
     // lane's later reads (its 32 values, quarter by quarter) are one 16-byte word per lane at consecutive
@@ -280,14 +272,6 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
       const int k = (j >> 2) * kSlice + lane * 32 + (j & 3) * 8;
       dma16(lds_a + (uint32_t)(j * 1024), xg + (k < K ? k : 0));
     }
-  } else if (active) {
-    request_scales_biases();
-#pragma unroll
-    for (int s = 0; s < SPW; ++s) {
-      const uint32_t xo = kvalid[s] ? (uint32_t)((slice0 + s) * (kSlice * 2) + lane * 64) : 0u;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) { xr[s][t] = gload16(xg, xo + t * 16); }
-    }
   }
 
   float tot[RB];
@@ -295,7 +279,7 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
   for (int r = 0; r < RB; ++r) { tot[r] = 0.0f; }
 
   // codes
-  constexpr int AFTER = XM == kXShared ? NDMA : 0;     // requests that follow the codes
+  constexpr int AFTER = NDMA;                  // requests that follow the codes
   u32x4v c[RB][SPW];
   if (active) {
     const uint8_t* wbase = reinterpret_cast<const uint8_t*>(wq) + (size_t)row_begin * (size_t)(K >> 1);
@@ -309,12 +293,12 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
         c[r][s] = gload16(wrow, koff);
       }
     }
-    if (XM == kXShared) { request_scales_biases(); }
-    wait_vm<NL + AFTER>();                       // x (this wavefront's values, or its share) has landed
-  } else if (XM == kXShared) {
+    request_scales_biases();
+    wait_vm<NL + AFTER>();                       // this wavefront's share of x has landed
+  } else {
     wait_vm<0>();
   }
-  if (XM == kXShared) { __syncthreads(); }       // ... and everybody else's share
+  __syncthreads();                               // ... and everybody else's share
 
   if (active) {
     uint32_t xp[SPW][16];                        // pairs (x_i, x_{i+4}) of each run of eight
@@ -324,13 +308,7 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
       float sum = 0.0f;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        uint4 d;
-        if (XM == kXShared) {
-          d = *reinterpret_cast<const uint4*>(lds + (((slice0 + s) * 4 + t) * 64 + lane) * 16);
-        } else {
-          touch(xr[s][t]);
-          d = make_uint4(xr[s][t].x, xr[s][t].y, xr[s][t].z, xr[s][t].w);
-        }
+        uint4 d = *reinterpret_cast<const uint4*>(lds + (((slice0 + s) * 4 + t) * 64 + lane) * 16);
         if (!kvalid[s]) { d = make_uint4(0u, 0u, 0u, 0u); }
         xp[s][4 * t + 0] = __builtin_amdgcn_perm(d.z, d.x, 0x05040100u);   // x0,x4
         xp[s][4 * t + 1] = __builtin_amdgcn_perm(d.z, d.x, 0x07060302u);   // x1,x5
@@ -373,7 +351,7 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
         chain = dots[r][s];
       });
     });
-    if (AFTER > 0) { wait_vm_after<0>(chain); }
+    wait_vm_after<0>(chain);
     float acc[RB];
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
@@ -442,17 +420,11 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
   }
 }
 
-template <int SPW, int RB, bool F32OUT, int XM, int C, bool F16 = false>
-__global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel(const FlowParams<C> p)
-{
-  qmv_flow_body<SPW, RB, F32OUT, XM, C, F16>(p);
-}
-
 // The single-pack form with its sixteen argument words as separate kernel arguments: this file is compiled with
 // kernel-argument preloading, which delivers the first sixteen words in scalar registers when a wavefront starts,
 // so a wavefront's first requests do not wait for a load of the argument buffer (an aggregate argument is not
 // preloaded).
-template <int SPW, int RB, bool F32OUT, int XM, bool F16 = false>
+template <int SPW, int RB, bool F32OUT, bool F16 = false>
 __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel_1(
     const uint16_t* x, const uint32_t* w, const uint16_t* scales, const uint16_t* biases, void* y, int K, uint32_t shape,
     int N, const uint16_t* residual)
@@ -462,7 +434,7 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel_1(
   FlowParams<1> p;
   p.h.x = x; p.h.residual = residual; p.h.K = K; p.h.shape = shape;
   p.w[0] = w; p.scales[0] = scales; p.biases[0] = biases; p.y[0] = y; p.N[0] = N; p.first_block[0] = 0;
-  qmv_flow_body<SPW, RB, F32OUT, XM, 1, F16, true>(p);
+  qmv_flow_body<SPW, RB, F32OUT, 1, F16, true>(p);
 }
 
 // The grouped form (2..4 packs sharing x) with preloaded arguments: the fourteen preloaded words hold what every
@@ -478,7 +450,7 @@ struct FlowRest {
   int N[C - 1];
 };
 
-template <int SPW, int RB, bool F32OUT, int XM, int C, bool F16 = false>
+template <int SPW, int RB, bool F32OUT, int C, bool F16 = false>
 __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel_g(
     const uint16_t* x, int K, uint32_t shape, int N0, int fb1, int fb2, int fb3, const uint32_t* w0,
     const uint16_t* scales0, const uint16_t* biases0, const FlowRest<C> rest)
@@ -492,14 +464,13 @@ __global__ __launch_bounds__(64 * kMaxWavesPerWg) void qmv_flow_kernel_g(
     p.w[i] = rest.w[i - 1]; p.scales[i] = rest.scales[i - 1]; p.biases[i] = rest.biases[i - 1]; p.y[i] = rest.y[i - 1];
     p.N[i] = rest.N[i - 1]; p.first_block[i] = fb[i - 1];
   }
-  qmv_flow_body<SPW, RB, F32OUT, XM, C, F16, true>(p);
+  qmv_flow_body<SPW, RB, F32OUT, C, F16, true>(p);
 }
 
 namespace {
 
 struct FlowPlan {
   int spw, wk, wr, rb;
-  int xm;          // kXOwn or kXShared
 };
 
 // Slices per wavefront and K parts, from measurements on MI355X with HBM-cold packs: up to three slices (K <= 6144)
@@ -510,7 +481,7 @@ struct FlowPlan {
 FlowPlan flow_plan(int K, double pack_bytes)
 {
   const int slices = (K + kSlice - 1) / kSlice;
-  FlowPlan pl{0, 0, 0, 0, kXShared};
+  FlowPlan pl{0, 0, 0, 0};
   pl.wk = slices <= 3 ? 1 : (slices + 3) / 4;
   if (pl.wk == 1 && slices > 3) { pl.wk = 2; }
   if (slices > 3 && slices <= 8) { pl.wk = 2; }
@@ -521,13 +492,13 @@ FlowPlan flow_plan(int K, double pack_bytes)
   return pl;
 }
 
-template <int S, int R, bool F32, int XM, int C, bool F16 = false>
+template <int S, int R, bool F32, int C, bool F16 = false>
 hipError_t launch_flow_kernel(dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st, const FlowParams<C>& p)
 {
   static std::once_flag once;          // one per instantiation
   static hipError_t attr_status = hipSuccess;
   if constexpr (C == 1) {
-    const auto kern = qmv_flow_kernel_1<S, R, F32, XM, F16>;
+    const auto kern = qmv_flow_kernel_1<S, R, F32, F16>;
     std::call_once(once, [&] {
       attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         kMaxLdsBytes);
@@ -537,7 +508,7 @@ hipError_t launch_flow_kernel(dim3 grid, dim3 block, size_t lds_bytes, hipStream
                          p.h.shape, p.N[0], p.h.residual);
   } else {
     // a grouped launch has no residual
-    const auto kern = qmv_flow_kernel_g<S, R, F32, XM, C, F16>;
+    const auto kern = qmv_flow_kernel_g<S, R, F32, C, F16>;
     std::call_once(once, [&] {
       attr_status = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         kMaxLdsBytes);
@@ -570,31 +541,21 @@ hipError_t dispatch_flow(const FlowPlan& pl, bool y_f32, const FlowHead& h, cons
     blocks += (segs[i].N + rows_per_block - 1) / rows_per_block;
   }
   const dim3 grid((unsigned)blocks);
-  if (f16) {
-    // binary16 elements: x shared through LDS; grouped launches store the element type
-    if (pl.xm != kXShared || (C > 1 && y_f32)) { return hipErrorInvalidValue; }
-#define VPQ_FLOW16(S, R)                                                                                        \
-  if (pl.spw == S && pl.rb == R) {                                                                              \
-    if constexpr (C == 1) {                                                                                     \
-      if (y_f32) { return launch_flow_kernel<S, R, true, kXShared, 1, true>(grid, block, lds_bytes, st, p); }   \
-    }                                                                                                           \
-    return launch_flow_kernel<S, R, false, kXShared, C, true>(grid, block, lds_bytes, st, p);                   \
+  // grouped launches store the element type
+  if (C > 1 && y_f32) { return hipErrorInvalidValue; }
+#define VPQ_FLOW(S, R)                                                                                    \
+  if (pl.spw == S && pl.rb == R) {                                                                        \
+    if constexpr (C == 1) {                                                                               \
+      if (y_f32) {                                                                                        \
+        return f16 ? launch_flow_kernel<S, R, true, 1, true>(grid, block, lds_bytes, st, p)               \
+                   : launch_flow_kernel<S, R, true, 1, false>(grid, block, lds_bytes, st, p);             \
+      }                                                                                                   \
+    }                                                                                                     \
+    return f16 ? launch_flow_kernel<S, R, false, C, true>(grid, block, lds_bytes, st, p)                  \
+               : launch_flow_kernel<S, R, false, C, false>(grid, block, lds_bytes, st, p);                \
   }
-    VPQ_FLOW16(1, 2) VPQ_FLOW16(2, 2) VPQ_FLOW16(3, 2) VPQ_FLOW16(4, 2) VPQ_FLOW16(5, 2) VPQ_FLOW16(6, 2)
-    VPQ_FLOW16(1, 4) VPQ_FLOW16(2, 4) VPQ_FLOW16(3, 4) VPQ_FLOW16(4, 4)
-#undef VPQ_FLOW16
-    return hipErrorInvalidValue;
-  }
-#define VPQ_FLOW(S, R)                                                                                          \
-  if (pl.spw == S && pl.rb == R) {                                                                              \
-    if (pl.xm == kXShared) {                                                                                    \
-      return y_f32 ? launch_flow_kernel<S, R, true, kXShared, C>(grid, block, lds_bytes, st, p)            \
-                   : launch_flow_kernel<S, R, false, kXShared, C>(grid, block, lds_bytes, st, p);          \
-    }                                                                                                           \
-    return y_f32 ? launch_flow_kernel<S, R, true, kXOwn, C>(grid, block, lds_bytes, st, p)                 \
-                 : launch_flow_kernel<S, R, false, kXOwn, C>(grid, block, lds_bytes, st, p);               \
-  }
-  VPQ_FLOW(1, 2) VPQ_FLOW(2, 2) VPQ_FLOW(3, 2) VPQ_FLOW(4, 2) VPQ_FLOW(5, 2) VPQ_FLOW(6, 2)
+  // every (slices per wavefront, rows per wavefront) that flow_plan can return
+  VPQ_FLOW(1, 2) VPQ_FLOW(2, 2) VPQ_FLOW(3, 2) VPQ_FLOW(4, 2)
   VPQ_FLOW(1, 4) VPQ_FLOW(2, 4) VPQ_FLOW(3, 4) VPQ_FLOW(4, 4)
 #undef VPQ_FLOW
   return hipErrorInvalidValue;
@@ -606,7 +567,7 @@ hipError_t launch_flow(hipStream_t st, const FlowSeg* segs, int count, const Qmv
 {
   const FlowPlan pl = flow_plan(a.K, pack_bytes);
   if (pl.spw == 0 || pl.wk < 1 || pl.wk > 4 || pl.wr < 1 || pl.wk * pl.wr > kMaxWavesPerWg ||
-      pl.wk * pl.spw * kSlice < a.K || (pl.xm != kXOwn && pl.xm != kXShared)) {
+      pl.wk * pl.spw * kSlice < a.K) {
     return hipErrorInvalidValue;
   }
   FlowHead h;
@@ -618,7 +579,7 @@ hipError_t launch_flow(hipStream_t st, const FlowSeg* segs, int count, const Qmv
   const int rows_per_block = pl.wr * pl.rb;
   const int W = pl.wk * pl.wr;
   const int ndma = (2 * pl.rb * pl.spw * 4 + 63) / 64;
-  const size_t lds_bytes = (pl.xm == kXShared ? (size_t)pl.wk * pl.spw * (kSlice * 2) : 0) + (size_t)W * ndma * 1024 +
+  const size_t lds_bytes = (size_t)pl.wk * pl.spw * (kSlice * 2) + (size_t)W * ndma * 1024 +
                            (size_t)W * pl.rb * sizeof(float);
   if (lds_bytes > (size_t)kMaxLdsBytes) { return hipErrorInvalidValue; }
   const dim3 block((unsigned)(64 * W));
