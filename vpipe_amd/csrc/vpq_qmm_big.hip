@@ -48,7 +48,6 @@ constexpr int BM = 256, BK = 64;
 constexpr int kBigThreads = 256;
 constexpr int kRow = BK * 2;                 // 128 bytes per LDS row
 constexpr int kXBytes = BM * kRow;           // 32 KB per stage
-constexpr int kWBytes = 256 * kRow;          // 32 KB per stage (BN <= 256)
 constexpr int kCodeBytes = 256 * 32;         // 8 KB: the 32 bytes of codes of one K step per row
 constexpr int kScaleBytes = 256 * 32;        // 8 KB: 8 scales | 8 biases (8 K steps) per row
 
@@ -139,14 +138,10 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   constexpr int NC = W8 ? 4 : 2;            // code loads per wavefront and step (1 KB each)
   constexpr int kCodeSlot = W8 ? 64 * NT * 64 : kCodeBytes;
   constexpr int kWStage = 64 * NT * kRow;   // BN rows of 128 bytes
-  // Stages of x.  Two where the window between two barriers (4 NT MFMAs per quarter) is long enough for a request
-  // to L2 to come back; the 128-row tile's window is 32 MFMAs, about the latency itself, so there x is requested a
-  // step further ahead into a third stage (its weight stages are half as large, which is where the room comes from).
-  constexpr int NX = (NT == 2 && !DENSE) ? 3 : 2;
   constexpr int SBLK = G32 ? 4 : 8;         // steps per 16-byte block of a row's scales
   constexpr int BN = 64 * NT;               // weight rows per workgroup
   constexpr int MQ = 4 * NT;                // MFMAs per quarter step (16 of K)
-  __shared__ __attribute__((aligned(16))) uint8_t x_lds[NX * kXBytes];
+  __shared__ __attribute__((aligned(16))) uint8_t x_lds[2 * kXBytes];
   __shared__ __attribute__((aligned(16))) uint8_t w_lds[2 * kWStage];
   uint8_t* const x_lds0 = x_lds;
   uint8_t* const x_lds1 = x_lds + kXBytes;
@@ -326,7 +321,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   // So the work of a window is cut into single instructions (ops) and dealt out so that no slot holds more than
   // 4: a fragment read counts 1, a load request 2 (the M0 write and the load; its s_nop is free), and the ops of
   // the dequantization fill what is left, in order.
-  constexpr int NLOADS = DENSE ? 8 + 2 * NT : 9 + NC;           // packed: codes, one pair of scales and biases, x
+  constexpr int NLOADS = DENSE ? 8 + 2 * NT : 9 + NC;           // packed: x, codes, one pair of scales and biases
   constexpr int NSLOT = 4 * MQ;                                // slots of a window (barrier to barrier)
   constexpr int LSTRIDE = 2;                                   // a load request every LSTRIDE-th slot, from slot 1 on
   // ---- the ops of a window's dequantization (of W(s+2)): NP ops that fetch the thread's codes, scales and biases
@@ -392,26 +387,11 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   uint32_t t0 = 0, t1 = 0, mk[4] = {0, 0, 0, 0};
   float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   uint4 o = make_uint4(0, 0, 0, 0);
-  // Three stages of x: the stage of a step is a run-time offset (xo_*), and the fragment reads of quarter ks go
-  // through xa[ks], the LDS address of the lane's piece of x fragment 0 in the stage that quarter is read from next.
-  uint32_t xo_prev = 2 * kXBytes, xo_cur = 0, xo_next = kXBytes;   // stages of steps s-1, s, s+1 (bytes into x_lds)
-  uint32_t xa_base[4], xa[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    xa_base[ks] = lds_addr(x_lds) + (uint32_t)x_rd[0] + (uint32_t)(((2 * ks + fkh) ^ f_sw) * 16);
-    xa[ks] = xa_base[ks];
-  }
   auto frag = [&](const uint8_t* xb, const uint8_t* wb, int buf, int ks, int idx) {   // idx: 0 = w0, 1..4 = x0..x3, 5.. = w1..
     const int c = ((2 * ks + fkh) ^ f_sw) * 16;
     if (idx == 0) {
       wf[buf][0] = *reinterpret_cast<const bf16x8*>(wb + w_rd[0] + c);
     } else if (idx <= 4) {
-      if constexpr (NX == 3) {
-        if (xb == nullptr) {     // (decided at compile time: every call passes a literal) read through xa[ks]
-          xf[buf][idx - 1] = *(__attribute__((address_space(3))) const bf16x8*)(uintptr_t)(xa[ks] + (uint32_t)(idx - 1) * (32 * kRow));
-          return;
-        }
-      }
       xf[buf][idx - 1] = *reinterpret_cast<const bf16x8*>(xb + x_rd[idx - 1] + c);
     } else {
       wf[buf][idx - 4] = *reinterpret_cast<const bf16x8*>(wb + w_rd[idx - 4] + c);
@@ -555,31 +535,32 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       }
     }
   };
-  // Request I of the window that opens behind the barrier of step `win`: x(win + NX) goes to the stage of step win
-  // (`xo_win` where there are three).  Packed: the codes and the scales come first and x last, so that with three
-  // stages the window's barrier can leave the x requests in flight (they are not needed before the one after).
-  auto window_load = [&](auto ic, int win, auto stage_c, uint32_t xo_win) {
+  // Request I of the window that opens behind the barrier of step `win`: x(win+2) goes to the stage of step win.
+  auto window_load = [&](auto ic, int win, auto stage_c) {
     constexpr int I = decltype(ic)::value;
     constexpr int STG = decltype(stage_c)::value;
     const int step_to = win + 2;
+    const uint32_t xdst = lds_addr(STG ? x_lds1 : x_lds0) + wave_x;
+    const uint8_t* xsrc = xblk + (size_t)step_to * (BK * 2);
     if constexpr (DENSE) {
-      const uint32_t xdst = lds_addr(STG ? x_lds1 : x_lds0) + wave_x;
       if constexpr (I < NWL) {
         const uint32_t wdst = lds_addr(STG ? w_lds1 : w_lds0) + wave_wd;
         dma16(wdst + I * (8 * kRow), wblk + (size_t)step_to * (BK * 2), wd_off[I]);
       } else {
-        dma16(xdst + (I - NWL) * (8 * kRow), xblk + (size_t)step_to * (BK * 2), a_off[I - NWL]);
+        dma16(xdst + (I - NWL) * (8 * kRow), xsrc, a_off[I - NWL]);
       }
     } else {
-      if constexpr (I < NC) {
+      if constexpr (I < 8) {
+        dma16(xdst + I * (8 * kRow), xsrc, a_off[I]);
+      } else if constexpr (I < 8 + NC) {
         // codes(win+3) into the slot codes(win+1) have left.  Past the last step the last step's codes are read
         // again (nobody uses them) rather than branching round the request; 4-bit codes: every wavefront brings in
         // 64 rows of the 256-row slot, tile rows or not.
         const int cstep = win + 3 < KT ? win + 3 : KT - 1;
         if (!W8 || dq_wave) {
-          dma16(lds_addr(c_lds) + (1 - STG) * kCodeSlot + wave_c + I * 1024, wblk + (size_t)cstep * CRB, c_off[I]);
+          dma16(lds_addr(c_lds) + (1 - STG) * kCodeSlot + wave_c + (I - 8) * 1024, wblk + (size_t)cstep * CRB, c_off[I - 8]);
         }
-      } else if constexpr (I == NC) {
+      } else {
         // scales and biases of the next block of steps, both in this slot, when the window's step starts a block
         if (win == sb_due) {
           const int blk = (win >> (G32 ? 2 : 3)) + 1;
@@ -588,22 +569,13 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
           dma16(sdst + 256 * 16, reinterpret_cast<const uint8_t*>(p.biases) + (size_t)blk * 16, sb_off);
           sb_due = win + 2 * SBLK < KT ? win + SBLK : 0x7fffffff;
         }
-      } else {
-        constexpr int X = I - NC - 1;
-        if constexpr (NX == 3) {
-          // past the last step the last step's tile is read again, into a stage nobody reads any more
-          const int xstep = win + 3 < KT ? win + 3 : KT - 1;
-          dma16(lds_addr(x_lds) + xo_win + wave_x + X * (8 * kRow), xblk + (size_t)xstep * (BK * 2), a_off[X]);
-        } else {
-          dma16(lds_addr(STG ? x_lds1 : x_lds0) + wave_x + X * (8 * kRow), xblk + (size_t)step_to * (BK * 2), a_off[X]);
-        }
       }
     }
   };
   // Slot G of the window behind the barrier of step `win`: its request, its ops (they dequantize W(win+2) into `nb`).
-  auto window_slot = [&](auto gc, int win, auto stage_c, uint32_t xo_win, uint8_t* nb) {
+  auto window_slot = [&](auto gc, int win, auto stage_c, uint8_t* nb) {
     constexpr int G = decltype(gc)::value;
-    if constexpr (plan.load_of[G] >= 0) { window_load(std::integral_constant<int, plan.load_of[G]>(), win, stage_c, xo_win); }
+    if constexpr (plan.load_of[G] >= 0) { window_load(std::integral_constant<int, plan.load_of[G]>(), win, stage_c); }
     if constexpr (!DENSE) {
       static_for<plan.op_begin[G], plan.op_begin[G + 1]>([&](auto uc) { dq_op(uc, win + 2, nb); });
     }
@@ -612,9 +584,9 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
   auto pstep = [&](auto stage_c, auto m1, auto m2, int s) {
     constexpr int ST = decltype(stage_c)::value;
     using Nx = std::integral_constant<int, 1 - ST>;
-    const uint8_t* xb = NX == 3 ? nullptr : (ST ? x_lds1 : x_lds0);
+    const uint8_t* xb = ST ? x_lds1 : x_lds0;
     const uint8_t* wb = ST ? w_lds1 : w_lds0;
-    const uint8_t* nxb = NX == 3 ? nullptr : (ST ? x_lds0 : x_lds1);
+    const uint8_t* nxb = ST ? x_lds0 : x_lds1;
     uint8_t* nwb = ST ? w_lds0 : w_lds1;
     uint8_t* ownb = ST ? w_lds1 : w_lds0;
     static_for<0, 4>([&](auto qc) {
@@ -625,35 +597,22 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
         constexpr int JT = J >> 2, IT = J & 3;
         acc[JT][IT] = mfma(wf[B][JT], xf[B][IT], acc[JT][IT]);
         constexpr int GB = Q == 3 ? J : MQ * (Q + 1) + J;    // slot counted from the previous barrier
-        if constexpr (Q == 3) { when(m2, [&] { window_slot(std::integral_constant<int, GB>(), s, stage_c, xo_cur, ownb); }); }
-        else { when(m1, [&] { window_slot(std::integral_constant<int, GB>(), s - 1, Nx(), xo_prev, nwb); }); }
+        if constexpr (Q == 3) { when(m2, [&] { window_slot(std::integral_constant<int, GB>(), s, stage_c, ownb); }); }
+        else { when(m1, [&] { window_slot(std::integral_constant<int, GB>(), s - 1, Nx(), nwb); }); }
         // the next quarter's fragments, one read after every MFMA until they are all requested
         if constexpr (J < 4 + NT) {
           if constexpr (Q < 3) { frag(xb, wb, 1 - B, Q + 1, J); }
           else { when(m1, [&] { frag(nxb, nwb, 0, 0, J); }); }
         }
-        if constexpr (NX == 3) {
-          // quarter Q's reads (of k slice Q + 1) are out: that slice's address moves on to the next step's stage;
-          // slice 0, read under quarter 3, moves before it
-          if constexpr (J == 4 + NT && Q < 3) { xa[Q + 1] = xa_base[Q + 1] + xo_next; }
-          if constexpr (J == 4 + NT + 1 && Q == 2) { xa[0] = xa_base[0] + xo_next; }
-        }
         __builtin_amdgcn_sched_barrier(0);
       });
       if constexpr (Q == 2) {
         when(m1, [&] {
-          // everything this wavefront asked for has landed -- with three stages of x all but the window's own 8
-          // requests for x, which came last and are read two barriers on
-          if constexpr (NX == 3) { asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory"); }
-          else { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
           wg_barrier();
         });
       }
     });
-    if constexpr (NX == 3) {
-      const uint32_t t = xo_prev;
-      xo_prev = xo_cur; xo_cur = xo_next; xo_next = t;
-    }
   };
 
   // `nq` quarter steps (16 of K each) on the tiles in stage 0, nothing overlapped: for the short extra pieces of K
@@ -687,7 +646,6 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
         issue_codes(0);
         issue_codes(1);
         issue_x(0, first_c);
-        if constexpr (NX == 3) { issue_x(1, S1()); }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         wg_barrier();                           // the codes and scales a thread reads were brought in by any wavefront
         static_for<0, NOPS>([&](auto uc) { dq_op(uc, 0, w_lds0); });
@@ -698,13 +656,12 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
       if (KT > 1) {
         static_for<0, MQ>([&](auto gc) {
           if constexpr (plan.load_of[decltype(gc)::value] >= 0) {
-            window_load(std::integral_constant<int, plan.load_of[decltype(gc)::value]>(), -1, Other(), xo_prev);
+            window_load(std::integral_constant<int, plan.load_of[decltype(gc)::value]>(), -1, Other());
           }
         });
       }
 #pragma unroll
       for (int i = 0; i < 4 + NT; ++i) { frag(P0 ? x_lds1 : x_lds0, P0 ? w_lds1 : w_lds0, 0, 0, i); }
-      if constexpr (NX == 3) { xa[0] = xa_base[0] + xo_next; }   // as a quarter 2 before step 0 would have left it
     };
     if constexpr (DENSE) {
       if (odd) { prologue(S1()); } else { prologue(S0()); }
@@ -722,7 +679,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     }
     if (s >= 0) { pstep(S0(), Yes(), No(), s); }
     pstep(S1(), No(), No(), s + 1);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // three stages: the repeated last requests, before LDS is reused
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the repeated last requests for codes, before LDS is reused
   }
 
   if constexpr (DENSE) {
