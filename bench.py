@@ -87,6 +87,12 @@ def main():
     ap.add_argument("--only-qmm", action="store_true",
                     help="run nothing but the fused QMM kernel on the three M=2048 projections and print their "
                          "timings (for a profiler: every qmm_tile_kernel dispatch then belongs to that workload)")
+    ap.add_argument("--only-small", type=int, default=0, metavar="M",
+                    help="run nothing but the small-batch QMV set (BASELINE config 3: four shapes) at M rows, weights "
+                         "rotated through HBM (for a profiler: every QMV dispatch then belongs to that workload)")
+    ap.add_argument("--only-dit", action="store_true",
+                    help="run nothing but the video-DiT QMM set (BASELINE config 5: three shapes at M = 16320) with "
+                         "the rank-32 adapter (for a profiler)")
     ap.add_argument("--no-extras", action="store_true", help="skip the small-batch QMV and video-DiT QMM sections")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -140,6 +146,38 @@ def main():
                 dst.copy_(src)
             torch.cuda.synchronize()
         print(json.dumps({"qmm_m2048_fused_kernel_only": res, "build": vpipe_amd.build_id()}))
+        return
+
+    if args.only_small:
+        M, res = args.only_small, {}
+        for K, N in SMALL_BATCH:
+            copies = max(2, min(8, int(600e6 // (N * K * 9 // 16))))
+            packs = [make_weight(torch, N, K, dev, gen) for _ in range(copies)]
+            x = torch.randn((M, K), device=dev, generator=gen).bfloat16()
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            for i in range(4 * copies):
+                w, s, b = packs[i % copies]
+                vpipe_amd.qmv_w4g64(w, s, b, x, K, N, M, out=y)
+            torch.cuda.synchronize()
+            res["%d->%d" % (K, N)] = {"launches": 4 * copies, "algorithmic_bytes": alg_bytes(K, N, M)}
+            del packs
+        print(json.dumps({"qmv_small_batch_only": res, "M": M, "build": vpipe_amd.build_id()}))
+        return
+    if args.only_dit:
+        M, r, res = 16320, 32, {}
+        for K, N in DIT:
+            w, s, b = make_weight(torch, N, K, dev, gen)
+            x = torch.randn((M, K), device=dev, generator=gen).bfloat16()
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            A = (torch.randn((r, K), device=dev, generator=gen) * 0.02).bfloat16()
+            B = (torch.randn((N, r), device=dev, generator=gen) * 0.02).bfloat16()
+            t = torch.empty((M, r), dtype=torch.bfloat16, device=dev)
+            for _ in range(6):
+                vpipe_amd.qmm_w4g64(w, s, b, x, K, N, M, out=y, lora_A=A, lora_B=B, r=r, alpha=1.0, t_ws=t)
+            torch.cuda.synchronize()
+            res["%d->%d" % (K, N)] = {"launches": 6, "flops": 2.0 * M * N * K, "lora_flops": 2.0 * M * r * (K + N)}
+            del w, s, b, x, y, A, B, t
+        print(json.dumps({"qmm_dit_only": res, "M": M, "r": r, "build": vpipe_amd.build_id()}))
         return
 
     # ---- inputs, resident in HBM ------------------------------------------------
@@ -470,7 +508,7 @@ def main():
             return float(np.sum(kb[:n])) * 1e3 / iters     # all kernels of a call (LoRA: two, the sampler: five)
 
         # small-batch QMV of a 5120-hidden model, weights rotated so that they come from HBM
-        small = {}
+        small, small_bytes, small_us = {}, 0.0, 0.0
         for K, N in SMALL_BATCH:
             copies = max(2, min(8, int(600e6 // (N * K * 9 // 16))))
             packs = [make_weight(torch, N, K, dev, gen) for _ in range(copies)]
@@ -482,11 +520,30 @@ def main():
                 def call(i, x=x, y=y, M=M):
                     w, s, b = packs[i % copies]
                     vpipe_amd.qmv_w4g64(w, s, b, x, K, N, M, out=y)
-                us = kernel_us(call, 2 * copies)
-                row["M=%d" % M] = {"us": round(us, 2), "GBps": round(alg_bytes(K, N, M) / (us * 1e-6) / 1e9, 1)}
+                # as the headline is timed: one HIP graph of back-to-back calls over the rotating packs between two
+                # events, median of 5 replays (launch gaps included, 1.6-1.7 us per launch in a graph); beside it
+                # the kernel's own duration from events around each eager launch (their floor is ~4 us)
+                n_calls = 8 * copies
+                saved_layers, args.layers = args.layers, n_calls
+                ms, _ = time_steps(call, n_calls, use_graph, repeats=5)
+                args.layers = saved_layers
+                us = ms * 1e3
+                us_ev = kernel_us(call, 2 * copies)
+                row["M=%d" % M] = {"us": round(us, 2), "GBps": round(alg_bytes(K, N, M) / (us * 1e-6) / 1e9, 1),
+                                   "eager_event_us": round(us_ev, 2)}
+                small_bytes += alg_bytes(K, N, M)
+                small_us += us
             small["%d->%d" % (K, N)] = row
             del packs
         out["qmv_small_batch"] = small
+        out["roofline_small_batch"] = {
+            "bound": "hbm", "achieved": round(small_bytes / (small_us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(small_bytes / (small_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": "qmv_flow_kernel_1 (M = 1), qmv_ring_kernel (2..16 rows), qmv_stream_kernel (2..4 rows over "
+                      "5120->151936): the 20 (shape, M) cases of BASELINE config 3, algorithmic bytes of all over "
+                      "the time of all",
+            "timing": "per case one HIP graph of 8 x (packs in rotation) calls, median of 5 replays",
+            "profile": "profiles/qmv_small_batch_m1_m4_m16.txt (rocprofv3 kernel trace + FETCH_SIZE / WRITE_SIZE)"}
 
         # video-DiT QMM with the fused rank-32 LoRA (flops of the base contraction only)
         M, r, alpha = 16320, 32, 1.0
@@ -512,6 +569,17 @@ def main():
             dit["%d->%d" % (K, N)]["dense_route_kept_expansion_TFLOPs"] = round(flops / (dr[1] * 1e-6) / 1e12, 1)
             del w, s, b, x, y, A, B, t
         out["qmm_dit_m16320_lora_r32"] = dit
+        dit_flops = sum(2.0 * M * N * K for K, N in DIT)
+        dit_us = sum(v["us"] for v in dit.values())
+        dit_us_lora = sum(v["us_with_lora"] for v in dit.values())
+        out["roofline_qmm_dit"] = {
+            "bound": "mfma", "achieved": round(dit_flops / (dit_us * 1e-6) / 1e12, 1), "peak": MFMA_BF16_PEAK_TF,
+            "unit": "TFLOP/s", "frac": round(dit_flops / (dit_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TF, 4), "traffic": None,
+            "achieved_with_lora_r32": round(dit_flops / (dit_us_lora * 1e-6) / 1e12, 1),
+            "kernel": "qmm_big_kernel<4,*,0> (256 x 256 tiles) + lora_a_kernel<1>; flops of the three base "
+                      "contractions (2 M N K) over their time, the adapter's flops not counted",
+            "timing": "us per call over 5 back-to-back calls after 40 ms of the same calls, events on the stream",
+            "profile": "profiles/qmm_big_kernel_dit_m16320_lora_r32.txt (rocprofv3 kernel trace + MFMA busy)"}
 
     # ---- fused gate|up + SwiGLU (interleaved pack), as context ------------------------------
     if not args.no_extras:

@@ -161,8 +161,9 @@ enum {
  * dense_gemm_mma.metal:297-348).  lora_a == NULL or alpha == 0 means no adapter,
  * and the output is then bit-identical to the call without one
  * (metal-minimax-h3-transformer.cc:2211-2219).
- * Requires K % 64 == 0, M, N > 0, r % 32 == 0 and 0 < r <= 128 when a LoRA is
- * given; x, y rows may be of any length (K, N) but the base pointers must be
+ * Requires K % 64 == 0, M, N > 0, and with a LoRA r % 16 == 0, 16 <= r <= VPQ_LORA_MAX_RANK (the reference's
+ * LoraFactors.rank is unconstrained, metal-minimax-h3-transformer.h:923-931; it runs rank 16 adapters, .h:365-367,
+ * and measures rank 384, .cc:1126-1132); x, y rows may be of any length (K, N) but the base pointers must be
  * 16-byte aligned. */
 int vpq_qmm_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                        const uint16_t* biases, const uint16_t* x, uint16_t* y,
@@ -219,8 +220,9 @@ int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                    int K, int N, int M, uint16_t* w_deq, int expand);
 
-/* The adapter's first GEMM alone: t[M,r] = bf16(alpha * bf16(x . A^T)).
+/* The adapter's first GEMM alone: t[M,r] = bf16(alpha * bf16(x . A^T)), r % 16 == 0, 16 <= r <= VPQ_LORA_MAX_RANK.
  * Replaces `lora_gemm_a_` (metal-minimax-h3-transformer.cc:1030-1067). */
+#define VPQ_LORA_MAX_RANK 512
 int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t,
                     int M, int K, int r, float alpha);
 

@@ -422,8 +422,7 @@ int32_t vpo_sample_topp_bf16(const uint16_t* logits, int V, float temp, float to
  *   combine  counts, masses and Z of the slabs are added in slab order 0, 1, ... (:3432-3452);
  *   thresh   a scan from bin 0 down: t_k = low edge exp(-(b+1) * 40/1024) of the bin where the running count first
  *            reaches top_k (0 < top_k < V), t_p that of the bin where the running mass first reaches top_p * Z;
- *            wt = max(t_k, max(min_p, 0), t_p); a target never reached leaves its threshold 0 (:3461-3497).  The
- *            running sums are formed in two levels (chunks of 32 bins), see below;
+ *            wt = max(t_k, max(min_p, 0), t_p); a target never reached leaves its threshold 0 (:3461-3497);
  *   pick     Gumbel-max over {ws_i >= wt} per slab, lowest index on ties, then over the slabs (:3499-3600).
  * Fixed here as above: exp / log are the written-out polynomials; inside a slab a thread t of 256 takes the indices
  * lo + t, lo + t + 256, ... in ascending order and the 256 partial sums meet in a halving tree.  wt_out (nullable)
@@ -487,35 +486,17 @@ int32_t vpo_sample_hist_bf16(const uint16_t* logits, int V, float temp, float to
       hist[B + b] = hist[B + b] + (float)mass[b] * (1.0f / 65536.0f);
     }
   }
-  /* thresholds: the running sum at a bin is (the totals of the 32-bin chunks before its chunk) + (its chunk up to
-   * it), each sum in ascending order from 0 -- the reference's single scan (:3476-3489) up to the association of
-   * the fp32 additions of the masses (the counts are integers) */
+  /* thresholds: the reference's single scan from bin 0 (:3476-3489), one running count and one running mass */
   const float target = top_p * Z;
-  float t_k = 0.0f, t_p = 0.0f, before_cnt = 0.0f, before_mass = 0.0f;
+  float t_k = 0.0f, t_p = 0.0f, cum_cnt = 0.0f, cum_mass = 0.0f;
   int have_k = 0, have_p = 0;
   const int do_k = top_k > 0 && top_k < V;
-  for (int j = 0; j < B / 32; ++j) {
-    float tot_cnt = 0.0f, tot_mass = 0.0f;
-    for (int b = 32 * j; b < 32 * j + 32; ++b) { tot_cnt = tot_cnt + hist[b]; tot_mass = tot_mass + hist[B + b]; }
-    if (do_k && !have_k && before_cnt + tot_cnt >= (float)top_k) {
-      float in_chunk = 0.0f;
-      for (int b = 32 * j; b < 32 * j + 32; ++b) {
-        in_chunk = in_chunk + hist[b];
-        if (before_cnt + in_chunk >= (float)top_k) { t_k = vpo_sample_exp(0.0f - (float)(b + 1) * binw); break; }
-      }
-      have_k = 1;
-    }
-    if (!have_p && before_mass + tot_mass >= target) {
-      float in_chunk = 0.0f;
-      for (int b = 32 * j; b < 32 * j + 32; ++b) {
-        in_chunk = in_chunk + hist[B + b];
-        if (before_mass + in_chunk >= target) { t_p = vpo_sample_exp(0.0f - (float)(b + 1) * binw); break; }
-      }
-      have_p = 1;
-    }
+  for (int b = 0; b < B; ++b) {
+    cum_cnt = cum_cnt + hist[b];
+    cum_mass = cum_mass + hist[B + b];
+    if (do_k && !have_k && cum_cnt >= (float)top_k) { t_k = vpo_sample_exp(0.0f - (float)(b + 1) * binw); have_k = 1; }
+    if (!have_p && cum_mass >= target) { t_p = vpo_sample_exp(0.0f - (float)(b + 1) * binw); have_p = 1; }
     if ((!do_k || have_k) && have_p) { break; }
-    before_cnt = before_cnt + tot_cnt;
-    before_mass = before_mass + tot_mass;
   }
   free(hist); free(cnt); free(mass);
   const float wt = fmaxf(fmaxf(t_k, fmaxf(min_p, 0.0f)), t_p);

@@ -72,7 +72,7 @@ def test_qmm_reference_lcg_inputs(vpq, oracle, dev, D):
     parity.check_bf16(got, y64, yb)
 
 
-@pytest.mark.parametrize("r,alpha", [(32, 1.0), (64, 0.625), (128, 2.0)])
+@pytest.mark.parametrize("r,alpha", [(16, 1.5), (32, 1.0), (48, 0.75), (64, 0.625), (128, 2.0), (256, 0.5), (384, 0.25)])
 def test_qmm_lora_fused(vpq, oracle, dev, D, r, alpha):
     M, N, K = 96, 160, 512
     w, s, b = synth.make_weight(N, K, 23)
@@ -264,7 +264,7 @@ def test_qmm_large_tile_kernel(vpq, oracle, dev, D, M, N, K, tile_n):
 
 
 @pytest.mark.parametrize("tile_n", [-128, 192, 256])
-@pytest.mark.parametrize("r", [32, 64, 96])
+@pytest.mark.parametrize("r", [16, 32, 48, 64, 96, 256, 384])
 def test_qmm_large_tile_kernel_with_lora(vpq, oracle, dev, D, r, tile_n):
     M, N, K, alpha = 300, 450, 1024, 0.75
     w, s, b = synth.make_weight(N, K, 7300 + r)

@@ -19,17 +19,44 @@ def _rows(V, rows, seed):
 def test_static_scratch_argmax_equals_the_workspace_form(vpq, oracle, dev, D):
     # two calls in a row on one stream, the second smaller (fewer rows, fewer slabs): the stale pairs of the
     # first call must not be read
-    free_before = torch.cuda.mem_get_info()[0]
+    assert vpq.load().vpq_init() == 0          # resolves the static array's address for this device
     for V, rows, seed in ((151936, 7, 1), (5000, 2, 2), (600001, 64, 3), (1, 1, 4)):
         bits = _rows(V, rows, seed)
         logits = D.bf16(bits, dev)
         want = vpq.argmax_bf16(logits, two_stage=True)
         out = torch.full((rows,), -7, dtype=torch.int32, device=dev)
-        got = vpq.argmax_bf16_static(logits, out)
         torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        got = vpq.argmax_bf16_static(logits, out)          # inputs and outputs exist: the call itself allocates nothing
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] >= free_before, "device memory was allocated by the static entry point"
         assert torch.equal(got, want), (V, rows)
         assert np.array_equal(got.cpu().numpy(), oracle.argmax(bits)), (V, rows)
-    assert torch.cuda.mem_get_info()[0] <= free_before + (64 << 20)   # (sanity: nothing large appeared)
+
+
+def test_static_scratch_argmax_under_graph_capture(vpq, oracle, dev, D):
+    """The callers the entry point is for cannot allocate: recorded into a HIP graph (an allocation or a symbol
+    lookup inside the call would fail the capture), replayed on fresh logits with eager work between the replays,
+    every replay checked."""
+    assert vpq.load().vpq_init() == 0
+    V, rows = 151936, 5
+    logits = D.bf16(_rows(V, rows, 20), dev)
+    out = torch.full((rows,), -7, dtype=torch.int32, device=dev)
+    vpq.argmax_bf16_static(logits, out)                    # (first call on this device done outside the capture)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        vpq.argmax_bf16_static(logits, out)
+    for rep in range(4):
+        bits = _rows(V, rows, 21 + rep)
+        logits.copy_(D.bf16(bits, dev))
+        out.fill_(-7)
+        other = vpq.argmax_bf16(D.bf16(_rows(999, 3, 40 + rep), dev), two_stage=True)   # eager work of the same kernels
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), oracle.argmax(bits)), rep
+        assert other.shape[0] == 3
 
 
 def test_static_scratch_argmax_rejects_what_its_array_cannot_hold(vpq, dev, D):

@@ -186,11 +186,12 @@ int vpq_init(void)
 {
   const int st = ensure_init();
   if (st != VPQ_OK) { return st; }
-  // also resolves the static scratch of vpq_argmax_bf16_static for the current device, so that the entry
-  // point itself has no first-call work left
+  // Also resolves the static scratch of vpq_argmax_bf16_static for the current device, so that the entry point
+  // itself has no first-call work left.  Best effort: a failure here concerns that one entry point only, which
+  // tries again on its first call and reports it there.
   float* unused = nullptr;
-  const hipError_t e = vpq::argmax_static_scratch(&unused);
-  return e == hipSuccess ? VPQ_OK : device_error(e);
+  (void)vpq::argmax_static_scratch(&unused);
+  return VPQ_OK;
 }
 
 int vpq_device_cu_count(void) { return g_dev.status.load() == VPQ_OK ? g_dev.cu_count : 0; }
@@ -383,7 +384,7 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
                     int M, int K, int r, float alpha)
 {
   if (x == nullptr || lora_a == nullptr || t == nullptr) { return VPQ_ERR_NULL_POINTER; }
-  if (M <= 0 || K <= 0 || (K % 64) != 0 || r <= 0 || r > 128 || (r % 32) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (M <= 0 || K <= 0 || (K % 64) != 0 || r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(lora_a, 16) || !aligned(t, 16)) { return VPQ_ERR_MISALIGNED; }
   const int st = ensure_init();
   if (st != VPQ_OK) { return st; }
@@ -408,7 +409,7 @@ int qmm_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (lora) {
     if (lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
     if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
-    if (r <= 0 || r > 128 || (r % 32) != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
     if (!aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) { return VPQ_ERR_MISALIGNED; }
   }
   st = ensure_init();

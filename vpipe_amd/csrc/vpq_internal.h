@@ -204,6 +204,8 @@ hipError_t launch_argmax_row(hipStream_t st, const uint16_t* logits, int* out_id
 hipError_t launch_argmax_partial(hipStream_t st, const uint16_t* logits, float* partials, int V, int rows, int parts);
 hipError_t launch_argmax_combine(hipStream_t st, const float* partials, int* out_id, int rows, int parts);
 // t[M,r] = bf16(alpha * bf16(x . A^T)), r in {32, 64, 96, 128}.
+// Adapter ranks: multiples of 16 up to this (the reference runs 16 and measures 384).
+constexpr int kLoraMaxRank = 512;
 hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
                          float alpha);
 // 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.

@@ -1,6 +1,7 @@
-// The adapter's first factor: t[M,r] = bf16(alpha * bf16(x[M,K] . A[r,K]^T)), r in {32,64,96,128}
-// (the SCALED tile of gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273, driven by lora_gemm_a_,
-// generative-models/minimax-h3/metal-minimax-h3-transformer.cc:1030-1067).
+// The adapter's first factor: t[M,r] = bf16(alpha * bf16(x[M,K] . A[r,K]^T)), any rank that is a multiple of 16
+// up to kLoraMaxRank (the SCALED tile of gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273, driven by
+// lora_gemm_a_, generative-models/minimax-h3/metal-minimax-h3-transformer.cc:1030-1067; the reference runs rank 16
+// adapters and measures rank 384, metal-minimax-h3-transformer.h:365-367, .cc:1126-1132).
 //
 // r is tiny against K, so this is a bandwidth kernel on x: every row of x is read once, A (r x K,
 // at most a few MB) stays in cache.  A workgroup owns 32 rows of x; its 8 wavefronts split K in
@@ -9,7 +10,9 @@
 // fixed tree and wavefront 0 rounds and stores.  Within a chunk the four MFMAs take
 // k = 32*half + 8*j + i (half = lane/32, j = MFMA, i < 8), so that a lane's operands for the
 // whole chunk are 64 contiguous bytes of its row: two lanes cover a row's 128-byte line, for x
-// and for A alike.
+// and for A alike.  Ranks above 128 run as blocks of 128 columns of t on grid.y (x is read once per
+// block; its 32 rows stay in L2 between the blocks of a workgroup's neighbours); a rank that is not a
+// multiple of 32 leaves the upper half of its last tile unused (rows of A clamped, nothing stored).
 #include "vpq_device.h"
 #include "vpq_internal.h"
 
@@ -41,9 +44,9 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p
   const int col = lane & 31;             // row of x (A operand) / row of the adapter (B operand)
   const int half = lane >> 5;
   const int m0 = blockIdx.x * kRows;
+  const int r0 = blockIdx.y * 128;       // first column of t of this block
   const int xrow = (m0 + col < p.M) ? (m0 + col) : (p.M - 1);
   const uint16_t* xp = p.x + (size_t)xrow * p.K + half * 32;
-  const uint16_t* ap = p.a + (size_t)col * p.K + half * 32;
 
   floatx16 acc[NT];
 #pragma unroll
@@ -60,7 +63,8 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p
     for (int j = 0; j < 4; ++j) { xa[j] = *reinterpret_cast<const bf16x8*>(xc + 8 * j); }
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
-      const uint16_t* ac = ap + (size_t)n * 32 * p.K + (size_t)c * kChunk;
+      const int arow = (r0 + n * 32 + col < p.r) ? (r0 + n * 32 + col) : (p.r - 1);
+      const uint16_t* ac = p.a + (size_t)arow * p.K + half * 32 + (size_t)c * kChunk;
       bf16x8 ab[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) { ab[j] = *reinterpret_cast<const bf16x8*>(ac + 8 * j); }
@@ -99,9 +103,9 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + 8 * (e >> 2) + 4 * half + (e & 3);
-        if (m < p.M) {
+        if (m < p.M && r0 + n * 32 + col < p.r) {
           const float v = bf16_bits_to_f32(f32_to_bf16_bits(acc[n][e]));
-          p.t[(size_t)m * p.r + n * 32 + col] = (uint16_t)f32_to_bf16_bits(p.alpha * v);
+          p.t[(size_t)m * p.r + r0 + n * 32 + col] = (uint16_t)f32_to_bf16_bits(p.alpha * v);
         }
       }
     }
@@ -111,9 +115,10 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p
 hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
                          float alpha)
 {
+  if (r < 16 || r % 16 != 0 || r > kLoraMaxRank) { return hipErrorInvalidValue; }
   LoraAParams p{x, a, t, M, K, r, alpha};
-  const dim3 grid((unsigned)((M + kRows - 1) / kRows)), block(kWaves * 64);
-  switch (r / 32) {
+  const dim3 grid((unsigned)((M + kRows - 1) / kRows), (unsigned)((r + 127) / 128)), block(kWaves * 64);
+  switch (r > 128 ? 4 : (r + 31) / 32) {   // tiles of 32 columns per block
     case 1: return launch_kernel(lora_a_kernel<1>, grid, block, 0, st, p);
     case 2: return launch_kernel(lora_a_kernel<2>, grid, block, 0, st, p);
     case 3: return launch_kernel(lora_a_kernel<3>, grid, block, 0, st, p);

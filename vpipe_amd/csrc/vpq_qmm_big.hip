@@ -710,7 +710,7 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     for (int st = 0; st < steps; ++st) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       wg_barrier();                                    // everyone done with stage 0
-      const int kleft = p.r - st * BK;                 // >= 32, a multiple of 32
+      const int kleft = p.r - st * BK;                 // >= 16, a multiple of 16
       const int chunks = kleft >= BK ? 8 : (kleft >> 3);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -848,7 +848,7 @@ bool qmm_big_supports(const GemmArgs& a)
   if (a.gate_act != 0 && (a.lora_t != nullptr || (a.N & 1) != 0)) { return false; }
   if ((reinterpret_cast<uintptr_t>(a.scales) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.biases) & 15) != 0) { return false; }
   if ((double)a.N * (double)a.K / (a.bits == 8 ? 1.0 : 2.0) >= 4.0e9 || (double)BM * (double)a.K * 2.0 >= 4.0e9) { return false; }
-  if (a.lora_t != nullptr && (a.r < 32 || a.r % 32 != 0)) { return false; }
+  if (a.lora_t != nullptr && (a.r < 16 || a.r % 16 != 0)) { return false; }
   // the other formats and the binary16 elements come without the adapter path, and not combined
   const int modes = (a.bits == 8) + (a.group == 32) + (a.f16 ? 1 : 0);
   if (modes > 1 || (modes == 1 && a.lora_t != nullptr)) { return false; }

@@ -440,7 +440,7 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
     if (LORA) {
       const int steps = (p.r + TK - 1) / TK;
       for (int st = 0; st < steps; ++st) {
-        const int kleft = p.r - st * TK;                 // >= 32, a multiple of 32
+        const int kleft = p.r - st * TK;                 // >= 16, a multiple of 16
         const int chunks = kleft >= TK ? 8 : (kleft >> 3);
         // t tile: 256 rows, as the x tile; B tile: 128 rows, 4 loads per wavefront.  Stage 0.
 #pragma unroll

@@ -302,18 +302,16 @@ __global__ __launch_bounds__(kHistThreads) void sample_hist_weights_kernel(
 }
 
 // One workgroup of 1024 threads: the slabs' histograms and Z added in slab order (a thread owns a cell; its loads
-// are issued sixteen at a time, the additions stay in slab order), then the scan for the two bins where the running
-// count reaches top_k and the running mass reaches top_p Z -- in two levels so that no thread walks more than 32
-// bins at a stretch: 32 chunks of 32 bins are summed by 64 threads, one thread walks the chunk totals and then the
-// bins of the chunk that crosses.  The running sum at a bin is (sum of the chunk totals before its chunk) + (sum of
-// its chunk up to it), every sum taken in ascending order from 0.
+// are issued sixteen at a time, the additions stay in slab order), then the reference's scan
+// (gpu-kernels/metal/ops/llm_elementwise.metal:3476-3497): one thread walks the bins from 0 with one running count
+// and one running mass -- the same additions in the same order, so that a crossing at a knife edge falls into the
+// same bin -- and stops at the bin where both targets are met (the bins are read eight at a time ahead of the
+// additions; a full walk of 1024 bins, no filter ever met, is a few microseconds).
 __global__ __launch_bounds__(kSampleThreads) void sample_hist_thresh_kernel(
     const float* __restrict__ partials, float* __restrict__ hist_out, float* __restrict__ wt_out, int n_slabs, int V,
     float top_p, int top_k, float min_p)
 {
-  constexpr int kChunk = 32, kChunks = kHistBins / kChunk;
   __shared__ float hist[2 * kHistBins + 1];
-  __shared__ float chunk_tot[2 * kChunks];          // counts, then masses
   const int stride = 2 * kHistBins + 1;
   for (int c = threadIdx.x; c < stride; c += kSampleThreads) {
     float acc = 0.0f;
@@ -330,38 +328,25 @@ __global__ __launch_bounds__(kSampleThreads) void sample_hist_thresh_kernel(
     hist_out[c] = acc;
   }
   __syncthreads();
-  if (threadIdx.x < 2 * kChunks) {
-    const float* h = hist + threadIdx.x * kChunk;   // chunks of the counts, then of the masses
-    float sum = 0.0f;
-    for (int b = 0; b < kChunk; ++b) { sum = sum + h[b]; }
-    chunk_tot[threadIdx.x] = sum;
-  }
-  __syncthreads();
   if (threadIdx.x != 0) { return; }
   const float target = top_p * hist[2 * kHistBins];
-  float t_k = 0.0f, t_p = 0.0f, before_cnt = 0.0f, before_mass = 0.0f;
-  bool have_k = false, have_p = false;
+  float t_k = 0.0f, t_p = 0.0f, cum_cnt = 0.0f, cum_mass = 0.0f;
+  bool have_k = false, have_p = false, done = false;
   const bool do_k = top_k > 0 && top_k < V;
-  for (int j = 0; j < kChunks; ++j) {
-    if (do_k && !have_k && before_cnt + chunk_tot[j] >= (float)top_k) {
-      float in_chunk = 0.0f;
-      for (int b = j * kChunk; b < (j + 1) * kChunk; ++b) {
-        in_chunk = in_chunk + hist[b];
-        if (before_cnt + in_chunk >= (float)top_k) { t_k = sample_exp(0.0f - (float)(b + 1) * kHistBinWidth); break; }
+  for (int b0 = 0; b0 < kHistBins && !done; b0 += 8) {
+    float c8[8], m8[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) { c8[q] = hist[b0 + q]; m8[q] = hist[kHistBins + b0 + q]; }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      if (!done) {
+        cum_cnt = cum_cnt + c8[q];
+        cum_mass = cum_mass + m8[q];
+        if (do_k && !have_k && cum_cnt >= (float)top_k) { t_k = sample_exp(0.0f - (float)(b0 + q + 1) * kHistBinWidth); have_k = true; }
+        if (!have_p && cum_mass >= target) { t_p = sample_exp(0.0f - (float)(b0 + q + 1) * kHistBinWidth); have_p = true; }
+        done = (!do_k || have_k) && have_p;
       }
-      have_k = true;
     }
-    if (!have_p && before_mass + chunk_tot[kChunks + j] >= target) {
-      float in_chunk = 0.0f;
-      for (int b = j * kChunk; b < (j + 1) * kChunk; ++b) {
-        in_chunk = in_chunk + hist[kHistBins + b];
-        if (before_mass + in_chunk >= target) { t_p = sample_exp(0.0f - (float)(b + 1) * kHistBinWidth); break; }
-      }
-      have_p = true;
-    }
-    if ((!do_k || have_k) && have_p) { break; }
-    before_cnt = before_cnt + chunk_tot[j];
-    before_mass = before_mass + chunk_tot[kChunks + j];
   }
   wt_out[0] = fmaxf(fmaxf(t_k, fmaxf(min_p, 0.0f)), t_p);
 }
