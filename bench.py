@@ -121,6 +121,14 @@ def main():
     if st != 0:
         raise vpipe_amd.VpqError(st, "vpq_init")
 
+    def copy_calibration():
+        """Three 256 MiB device-to-device copies: a kernel of known traffic beside the profiled ones."""
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(generator=gen)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
     if args.only_qmm:
         M, res = 2048, {}
         for name, K, N in PREFILL:
@@ -140,11 +148,7 @@ def main():
             res[name] = {"K": K, "N": N, "M": M, "us": round(us, 2),
                          "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 1)}
         if args.copy_calibration:
-            src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(generator=gen)
-            dst = torch.empty_like(src)
-            for _ in range(3):
-                dst.copy_(src)
-            torch.cuda.synchronize()
+            copy_calibration()
         print(json.dumps({"qmm_m2048_fused_kernel_only": res, "build": vpipe_amd.build_id()}))
         return
 
@@ -161,6 +165,8 @@ def main():
             torch.cuda.synchronize()
             res["%d->%d" % (K, N)] = {"launches": 4 * copies, "algorithmic_bytes": alg_bytes(K, N, M)}
             del packs
+        if args.copy_calibration:
+            copy_calibration()
         print(json.dumps({"qmv_small_batch_only": res, "M": M, "build": vpipe_amd.build_id()}))
         return
     if args.only_dit:
@@ -177,6 +183,8 @@ def main():
             torch.cuda.synchronize()
             res["%d->%d" % (K, N)] = {"launches": 6, "flops": 2.0 * M * N * K, "lora_flops": 2.0 * M * r * (K + N)}
             del w, s, b, x, y, A, B, t
+        if args.copy_calibration:
+            copy_calibration()
         print(json.dumps({"qmm_dit_only": res, "M": M, "r": r, "build": vpipe_amd.build_id()}))
         return
 
@@ -945,11 +953,7 @@ def main():
         out["cpu_baseline_configs"] = cfg
 
     if args.copy_calibration:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(generator=gen)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
+        copy_calibration()
         out["copy_calibration"] = {"bytes_read": 256 << 20, "bytes_written": 256 << 20, "copies": 3}
 
     print(json.dumps(out))
