@@ -138,9 +138,13 @@ enum {
   VPQ_QMV_RING = 5,        /* x in registers across a workgroup's tiles, codes through a two-slot LDS ring per wavefront */
   VPQ_QMV_ROWS = 6,        /* M <= 2, any K % 64: a wavefront streams whole rows with full-width loads, packed bf16
                               dot products, no LDS; what AUTO takes for M <= 2 where K is not a multiple of 512 */
-  VPQ_QMV_FLOW = 7         /* M = 1, K % 512 == 0, K >= 2048: one wavefront per (row set, K part), every load of the
+  VPQ_QMV_FLOW = 7,        /* M = 1, K % 512 == 0, K >= 2048: one wavefront per (row set, K part), every load of the
                               launch requested up front, x in registers, scales / biases staged in LDS; what AUTO
                               takes for M = 1 below lm_head-sized packs */
+  VPQ_QMV_RING_SPLITK = 8  /* as 5 with K split across workgroups (up to 4 parts, K >= 1024): fp32 planes in `ws`, added
+                              in part order by a fold launch that rounds once -- the deep-K split of
+                              generative-models/shared/mma-splitk.h:30-52.  AUTO takes it by itself for 2..16 rows when
+                              `ws` is given and its cost model says it pays (many rows of x, deep K, narrow N) */
 };
 
 /* ---- a6/a7/a8 (+a10): QMM ----------------------------------------------

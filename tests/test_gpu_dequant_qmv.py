@@ -314,6 +314,44 @@ def test_qmv_split_k_matches_oracle_and_is_deterministic(vpq, oracle, dev, D, K,
     parity.check_f32(f.cpu().numpy(), y64)
 
 
+@pytest.mark.parametrize("K,N,M", [(1024, 33, 16), (4096, 64, 5), (8192, 48, 2), (17408, 200, 16), (2560, 16, 9)])
+def test_qmv_ring_split_k_matches_oracle_and_is_deterministic(vpq, oracle, dev, D, K, N, M):
+    """The ring kernel with K split across workgroups (fp32 planes + fold launch): oracle parity with and without a
+    residual, the fp32 result before the store, the same bits run to run, and the planes' guard bytes intact."""
+    w, s, b = synth.make_weight(N, K, 41 + K)
+    x = synth.make_act(M, K, 42 + K)
+    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    ws = parity.Guarded((vpq.load().vpq_qmv_workspace_bytes(K, N, M) // 4,), torch.float32, dev)
+    ws.view.zero_()                                 # (the arrival counters at its start belong to the other split-K kernel)
+    runs = []
+    for _ in range(3):
+        out = parity.Guarded((M, N), torch.bfloat16, dev)
+        vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, ws=ws.view, variant=capi.VPQ_QMV_RING_SPLITK)
+        torch.cuda.synchronize()
+        out.assert_intact()
+        ws.assert_intact()
+        runs.append(D.bits(out.view).copy())
+    parity.check_bf16(runs[0], y64, yb)
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, ws=ws.view, variant=capi.VPQ_QMV_RING_SPLITK, f32out=True)
+    parity.check_f32(f.cpu().numpy(), y64)
+    # the unsplit kernel agrees to accumulation-order noise
+    f1 = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, variant=capi.VPQ_QMV_RING, f32out=True)
+    rms = float(np.sqrt((y64 ** 2).mean()))
+    assert (f - f1).abs().max().item() <= 1e-5 * rms + 1e-6
+    # residual: added to the rounded product, rounded again (affine_qmv.metal:347-363)
+    res = synth.make_act(M, N, 43 + K)
+    got = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, residual=D.bf16(res, dev), ws=ws.view, variant=capi.VPQ_QMV_RING_SPLITK)
+    want = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(runs[0]) + synth.bf16_bits_to_f32(res))
+    assert np.array_equal(D.bits(got), want)
+    # a workspace too small for the planes is refused
+    with pytest.raises(capi.VpqError) as e:
+        vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, ws=ws.view[: M * N], variant=capi.VPQ_QMV_RING_SPLITK)
+    assert e.value.status == capi.VPQ_ERR_WORKSPACE
+    assert not ws.view[:64].any().item()            # the counters' region was left alone
+
+
 def test_qmv_one_hot_reads_back_weights_exactly(vpq, oracle, dev, D):
     # x = e_k: y[n] must be bf16(fp32(s*q+b)) EXACTLY for every kernel -- layout,
     # nibble order and the un-rounded-weight arithmetic in one known answer.

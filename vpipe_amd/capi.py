@@ -17,6 +17,7 @@ _lib = None
 
 VPQ_GATE_SWIGLU, VPQ_GATE_GEGLU = 1, 2
 VPQ_QMV_AUTO, VPQ_QMV_SIMPLE, VPQ_QMV_MFMA, VPQ_QMV_MFMA_SPLITK, VPQ_QMV_STREAM, VPQ_QMV_RING, VPQ_QMV_ROWS, VPQ_QMV_FLOW = 0, 1, 2, 3, 4, 5, 6, 7
+VPQ_QMV_RING_SPLITK = 8
 
 # Every symbol include/vpq.h declares: (name, restype, argtypes).
 _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t

@@ -95,7 +95,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
   if (variant == VPQ_QMV_MFMA_SPLITK && ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }   // the only user of ws
-  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_FLOW) { return VPQ_ERR_BAD_SHAPE; }
+  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_RING_SPLITK) { return VPQ_ERR_BAD_SHAPE; }
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
 
@@ -119,7 +119,14 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   }
   if (variant == VPQ_QMV_RING) {
     if (!mfma_ok || !vpq::qmv_ring_supports(K, N, M)) { return VPQ_ERR_BAD_SHAPE; }
-    return finish(vpq::launch_qmv_ring(hs, a, 0, 0));
+    return finish(vpq::launch_qmv_ring(hs, a, 0, 1));
+  }
+  if (variant == VPQ_QMV_RING_SPLITK) {
+    if (!mfma_ok || !vpq::qmv_ring_supports(K, N, M) || K < 1024) { return VPQ_ERR_BAD_SHAPE; }
+    if (ws == nullptr || !aligned(ws, 16)) { return ws == nullptr ? VPQ_ERR_WORKSPACE : VPQ_ERR_MISALIGNED; }
+    const int parts = K / 512 < 4 ? K / 512 : 4;
+    if (ws_bytes < vpq::qmv_ring_workspace_bytes(K, N, M)) { return VPQ_ERR_WORKSPACE; }
+    return finish(vpq::launch_qmv_ring(hs, a, 0, parts));
   }
   if (variant == VPQ_QMV_STREAM) {
     // handled below, after the shape check of the streaming kernel
@@ -152,7 +159,12 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   // of once per item (measured at 16 rows: 117 vs 284 us at 5120->151936, 17.6 vs 39.9 us at
   // 5120->17408; at 4 rows 8.8 vs 12.0 us at 4096->12288; at 2 rows 15.1 vs 17.1 us at 5120->17408,
   // 16.0 vs 17.5 at 17408->5120).
-  if (mfma_ok && vpq::qmv_ring_supports(K, N, M) && M >= 2) { return finish(vpq::launch_qmv_ring(hs, a, 0, 0)); }
+  // (with a workspace the ring kernel splits K across workgroups where its cost model says that pays: many rows
+  // over a deep K and a narrow N)
+  if (mfma_ok && vpq::qmv_ring_supports(K, N, M) && M >= 2) {
+    if (a.ws != nullptr && !aligned(a.ws, 16)) { a.ws = nullptr; a.ws_bytes = 0; }
+    return finish(vpq::launch_qmv_ring(hs, a, 0, 0));
+  }
   if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a, 1)); }
   // K not a multiple of 512, or scales / biases off 16-byte alignment: the row-streaming kernel
   // for up to two rows of x, the general one above.

@@ -179,7 +179,8 @@ bool qmv_stream_supports(int K, int N, int M);
 hipError_t launch_qmv_stream(hipStream_t st, const QmvArgs& a, bool f16 = false);
 bool qmv_ring_supports(int K, int N, int M);
 // tc_hint / nw_hint > 0 force the tiles / wavefronts per workgroup (measurement only).
-hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint, bool f16 = false);
+hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int splits_hint, bool f16 = false);
+size_t qmv_ring_workspace_bytes(int K, int N, int M);   // planes of the widest K split the ring kernel takes
 // Row-streaming kernel (M <= 2, any K % 64): rows_per_wave in {2, 4}, 0 = default.
 bool qmv_rows_supports(int K, int N, int M);
 hipError_t launch_qmv_rows(hipStream_t st, const QmvArgs& a, int rows_per_wave);

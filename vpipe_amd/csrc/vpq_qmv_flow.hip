@@ -28,6 +28,8 @@
 //     y += s * dot + (b - 128 * s) * sx
 // per row and slice (a lane's 32 values lie in one quantization group), one wave reduction per
 // row at the end.
+#include <cstdio>
+#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 
@@ -475,19 +477,28 @@ struct FlowPlan {
 
 // Slices per wavefront and K parts, from measurements on MI355X with HBM-cold packs: up to three slices (K <= 6144)
 // a wavefront walks the whole K; longer rows are split between 2 to 4 wavefronts of the workgroup (12288->4096:
-// 7.5 us as 2 parts x 3 slices x 4 rows against 8.0 as one part of 6 slices).  Four wavefronts per workgroup; two
+// 7.5 us as 2 parts x 3 slices x 4 rows against 8.0 as one part of 6 slices; 17408->5120: 14.2 us with one row set
+// of 3 parts per workgroup against 15.9 with two, while 12288->4096 prefers two row sets of 2 parts: 8.0 against
+// 9.2; eight rows per wavefront measured slower everywhere).  Four wavefronts per workgroup up to two parts; two
 // rows per wavefront on small packs (more, shorter wavefronts spread the pack over the CUs sooner), four on large
 // ones; x shared through LDS.
 FlowPlan flow_plan(int K, double pack_bytes)
 {
   const int slices = (K + kSlice - 1) / kSlice;
   FlowPlan pl{0, 0, 0, 0};
+  // A forced plan for measurements, "spw,wk,wr,rb" in VPQ_FLOW_PLAN (the counterpart of the reference's forced GEMM
+  // route, metal-minimax-h3-transformer.cc:1912-1967); taken only if it covers K, checked again by the caller.
+  static const char* forced = getenv("VPQ_FLOW_PLAN");
+  if (forced != nullptr) {
+    FlowPlan f{0, 0, 0, 0};
+    if (sscanf(forced, "%d,%d,%d,%d", &f.spw, &f.wk, &f.wr, &f.rb) == 4 && f.spw * f.wk >= slices) { return f; }
+  }
   pl.wk = slices <= 3 ? 1 : (slices + 3) / 4;
   if (pl.wk == 1 && slices > 3) { pl.wk = 2; }
   if (slices > 3 && slices <= 8) { pl.wk = 2; }
   if (pl.wk > 4) { return pl; }
   pl.spw = (slices + pl.wk - 1) / pl.wk;
-  pl.wr = pl.wk == 1 ? 4 : 2;
+  pl.wr = pl.wk == 1 ? 4 : (pl.wk == 2 ? 2 : 1);
   pl.rb = pl.wk == 1 ? ((pl.spw <= 2 && pack_bytes >= 40e6) ? 4 : 2) : (pack_bytes >= 20e6 ? 4 : 2);
   return pl;
 }

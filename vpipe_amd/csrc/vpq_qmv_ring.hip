@@ -31,6 +31,14 @@
 //           table (added to what an earlier slice left there); after the last item one
 //           barrier, and the first TC*MR*64 threads add the rows in wavefront order and
 //           store y.  The order is fixed, so results are bit-reproducible.
+//   split   K split across workgroups (the deep-K split of generative-models/shared/mma-splitk.h:30-52: fp32
+//           planes, then a fold that adds them in order and rounds once): a workgroup re-reads all M rows of x
+//           over its K range, which on a narrow N (few tiles per workgroup) and many rows is several times its
+//           share of the pack -- 17408 -> 5120 at 16 rows: 557 KB of x for 78 KB of codes.  With `kparts` > 1
+//           grid.y is the part: the workgroup walks the slices of its part only (x over that range, `kparts` times
+//           the tiles for the same number of workgroups) and writes its fp32 sums to plane [part][M][N] of the
+//           caller's workspace; qmv_ring_fold_kernel adds the planes in part order and applies the store's
+//           residual and rounding (plain stores only: the gated entry points take no workspace).  No atomics, no fences: a second launch.
 //
 // No inline-assembly VALU instruction may sit near the MFMAs (the compiler's hazard
 // recogniser cannot see what such a statement writes); the asm here is loads and waits only.
@@ -71,6 +79,9 @@ struct RingParams {
   void* y;
   const uint16_t* residual;
   int gate_act; // rows are interleaved gate|up; y is [M, N/2] = act(gate) * up (1 SwiGLU, 2 GEGLU)
+  int kparts;   // workgroups along K (grid.y); > 1: fp32 sums go to `plane`, the fold kernel stores y
+  float* plane; // [kparts][M][N]
+  int part_slices;   // slices per part
   int pad_;
 };
 static_assert(offsetof(RingParams, y) == kPreloadWords * 4, "y starts the part that is not preloaded");
@@ -205,8 +216,11 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
   neg128[0] = neg128[1] = neg128[2] = neg128[3] = F16 ? 0xcc00cc00u : 0xc300c300u;
   constexpr float kBiasOverOffset = F16 ? -0.0625f : -0.0078125f;
 
-  // This wavefront's items: slices wave, wave+NW, ... (rounds) x the workgroup's tiles.
-  const int rounds = (p.slices - wave + NW - 1) / NW;     // <= 0 for an idle wavefront
+  // This wavefront's items: slices s_begin + wave, + NW, ... (rounds) of the workgroup's K part x its tiles.
+  const int part = (int)blockIdx.y;
+  const int s_begin = part * p.part_slices;
+  const int s_count = (p.slices - s_begin) < p.part_slices ? (p.slices - s_begin) : p.part_slices;
+  const int rounds = (s_count - wave + NW - 1) / NW;      // <= 0 for an idle wavefront
   const int n_items = rounds > 0 ? rounds * TC : 0;
 
   // Requests item i into a slot (i is clamped to the last item, so that the loop can request
@@ -216,7 +230,7 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
     const int ii = i < n_items ? i : n_items - 1;
     const int r = ii / TC;
     const int t = ii - r * TC;
-    const int sl = wave + r * NW;
+    const int sl = s_begin + wave + r * NW;
     int tile = tile0 + t;
     if (tile >= p.tiles) { tile = p.tiles - 1; }
     const int n0 = tile * kTileN;
@@ -263,7 +277,7 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
 
   // M <= 4: requests slice r of x, rows 0..3 (rows beyond M repeat the last one), 1 KB each.
   auto request_x = [&](int r) {
-    const int sl = wave + r * NW;
+    const int sl = s_begin + wave + r * NW;
 #pragma unroll
     for (int m = 0; m < kXLoads; ++m) {
       const int mm = m < p.M ? m : p.M - 1;
@@ -289,7 +303,7 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
                    :
                    : "memory");
     } else {
-      const int sl = wave + r * NW;
+      const int sl = s_begin + wave + r * NW;
       const uint16_t* xp = p.x + (size_t)x_row * p.K + (size_t)sl * kKS + g * 16;
 #pragma unroll
       for (int grp = 0; grp < kG; ++grp) {
@@ -405,13 +419,15 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
     const int t = o_idx / (MR * kWave);
     const int q = (o_idx / kWave) % MR;
     const int l = o_idx & 63;
-    const int live = p.slices < NW ? p.slices : NW;
+    const int live = s_count < NW ? s_count : NW;
     float total = 0.0f;
     for (int wv = 0; wv < live; ++wv) { total += sums[((t * NW + wv) * MR + q) * kWave + l]; }
     const int m = 4 * q + (l >> 4);
     const int tile = tile0 + t;
     const int n = tile * kTileN + (l & 15);
-    if (p.gate_act) {
+    if (p.kparts > 1) {
+      if (tile < p.tiles && m < p.M && n < p.N) { p.plane[((size_t)part * p.M + m) * p.N + n] = total; }
+    } else if (p.gate_act) {
       // Lanes 2j and 2j+1 hold the gate and the up sum of one feature (N is even).
       const float up = from_neighbour_lane(total);
       if (tile < p.tiles && m < p.M && n < p.N && (l & 1) == 0) {
@@ -438,9 +454,36 @@ __global__ __launch_bounds__(NW * 64) void qmv_ring_kernel(VPQ_PRELOADED_WORDS, 
   }
 }
 
+// y = store(plane[0] + plane[1] + ...), the parts added in order: one thread per output element.
+template <bool F32OUT, bool F16>
+__global__ __launch_bounds__(256) void qmv_ring_fold_kernel(const float* __restrict__ plane, void* __restrict__ y,
+                                                            const uint16_t* __restrict__ residual, int M, int N, int kparts)
+{
+  const size_t MN = (size_t)M * N;
+  const size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= MN) { return; }
+  float total = 0.0f;
+  for (int k = 0; k < kparts; ++k) { total += plane[k * MN + o]; }
+  if (F32OUT) {
+    reinterpret_cast<float*>(y)[o] = total;
+  } else {
+    uint32_t v = f32_to_elt_bits<F16>(total);
+    if (residual != nullptr) { v = f32_to_elt_bits<F16>(elt_bits_to_f32<F16>(v) + elt_bits_to_f32<F16>(residual[o])); }
+    reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)v;
+  }
+}
+
 bool qmv_ring_supports(int K, int N, int M)
 {
   return K % kKS == 0 && N >= 1 && M >= 1 && M <= 16;
+}
+
+size_t qmv_ring_workspace_bytes(int K, int N, int M)
+{
+  if (!qmv_ring_supports(K, N, M) || K / kKS < 2) { return 0; }
+  const int parts = K / kKS < 4 ? K / kKS : 4;
+  const size_t header = ((size_t)((N + kTileN - 1) / kTileN) * sizeof(unsigned) + 255) / 256 * 256;
+  return header + (size_t)parts * (size_t)M * (size_t)N * sizeof(float);
 }
 
 namespace {
@@ -448,7 +491,7 @@ namespace {
 template <int NW, bool F16>
 hipError_t launch_nw(hipStream_t st, const RingParams& p, int mr, bool f32)
 {
-  const dim3 grid((unsigned)((p.tiles + p.tc - 1) / p.tc)), block((unsigned)(NW * kWave));
+  const dim3 grid((unsigned)((p.tiles + p.tc - 1) / p.tc), (unsigned)p.kparts), block((unsigned)(NW * kWave));
   if (f32) {
     if (mr == 1) { return launch_preloaded(qmv_ring_kernel<NW, 1, true, F16>, grid, block, 0, st, p); }
     if (mr == 2) { return launch_preloaded(qmv_ring_kernel<NW, 2, true, F16>, grid, block, 0, st, p); }
@@ -461,10 +504,10 @@ hipError_t launch_nw(hipStream_t st, const RingParams& p, int mr, bool f32)
 
 }  // namespace
 
-// tc_hint > 0 forces the tiles per workgroup (measurement).
-hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw_hint, bool f16)
+// tc_hint > 0 forces the tiles per workgroup (measurement).  splits_hint: 0 = K across workgroups where a.ws has
+// the room and the cost model says it pays, 1 = never, n > 1 = n parts (if a.ws has the room).
+hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int splits_hint, bool f16)
 {
-  (void)nw_hint;
   RingParams p;
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
   p.residual = a.residual;
@@ -480,26 +523,64 @@ hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int nw
   // all of x once.  The count that minimises generations x bytes per workgroup wins; the largest count
   // often does not (9496 tiles at 16 per workgroup: 594 workgroups, a third generation for 82 of them).
   const double tile_bytes = 16.0 * (double)a.K * 9.0 / 16.0, x_bytes = (double)a.M * (double)a.K * 2.0;
-  auto plan = [&](int regs, int& tc_out) {
+  // cost of a launch with t tiles per workgroup and K in `parts` parts, in bytes a workgroup moves per generation
+  auto plan = [&](int regs, int parts, int& tc_out) {
     double best = 0.0;
     for (int t = 1; t <= max_tc_mr(regs) / regs; ++t) {
-      const int wgs = (p.tiles + t - 1) / t;
-      const double cost = (double)((wgs + cus - 1) / cus) * ((double)t * tile_bytes + x_bytes);
+      const int wgs = ((p.tiles + t - 1) / t) * parts;
+      const double cost = (double)((wgs + cus - 1) / cus) * ((double)t * tile_bytes + x_bytes) / (double)parts;
       if (t == 1 || cost <= best) { best = cost; tc_out = t; }
     }
     return best;
   };
   int tc = 1;
-  const double cost = plan(mr, tc);
+  double cost = plan(mr, 1, tc);
   // Up to 4 rows: the staged-x form has room for 4 tiles per workgroup; where that costs a generation the
   // two-register form (up to 16 tiles) is worth more than its idle accumulator register.
   if (mr == 1 && a.M >= 2) {
     int tc2 = 1;
-    if (plan(2, tc2) * 1.05 < cost) { mr = 2; tc = tc2; }
+    const double c2 = plan(2, 1, tc2);
+    if (c2 * 1.05 < cost) { mr = 2; tc = tc2; cost = c2; }
+  }
+  // K across workgroups where the caller's workspace holds the planes and it pays.  Measured (kernel + fold, us,
+  // unsplit / 4 parts): 17408 -> 5120 at 16 rows 26.3 / 23.5, at 8 rows 21.4 / 20.5, at 4 rows 17.2 / 22.5;
+  // 5120 -> 5120 at 16 rows 11.7 / 14.8; 5120 -> 17408 at 16 rows 19.4 / 31.1; 5120 -> 151936 123.8 / 202.2: the
+  // fold's launch and the shorter K walks cost more than the re-read x except for many rows over a deep K with few
+  // tiles per CU.  The planes start behind the arrival counters of the other split-K kernel, which must stay zero.
+  p.kparts = 1;
+  p.part_slices = p.slices;
+  p.plane = nullptr;
+  const size_t ws_header = ((size_t)p.tiles * sizeof(unsigned) + 255) / 256 * 256;
+  if (splits_hint != 1 && a.ws != nullptr && p.slices >= 2 && a.gate_act == 0) {     // (the gated entry points take no workspace)
+    int parts = splits_hint > 1 ? splits_hint : ((a.M >= 8 && p.slices >= 24 && p.tiles <= 2 * cus) ? 4 : 1);
+    if (parts > p.slices) { parts = p.slices; }
+    if (parts > 1 && ws_header + (size_t)parts * (size_t)a.M * (size_t)a.N * sizeof(float) <= a.ws_bytes) {
+      p.part_slices = (p.slices + parts - 1) / parts;
+      p.kparts = (p.slices + p.part_slices - 1) / p.part_slices;      // no empty part
+      p.plane = reinterpret_cast<float*>(static_cast<uint8_t*>(a.ws) + ws_header);
+      int tcp = 1;
+      plan(mr, p.kparts, tcp);
+      tc = tcp;
+    } else if (splits_hint > 1) {
+      return hipErrorInvalidValue;
+    }
   }
   const int tc_max = max_tc_mr(mr) / mr;
   if (tc_hint > 0) { tc = tc_hint < tc_max ? tc_hint : tc_max; }
   p.tc = tc;
+  p.pad_ = 0;
+  if (p.kparts > 1) {
+    const hipError_t e = f16 ? launch_nw<8, true>(st, p, mr, a.y_f32) : launch_nw<8, false>(st, p, mr, a.y_f32);
+    if (e != hipSuccess) { return e; }
+    const size_t outs = (size_t)a.M * a.N;
+    const dim3 fgrid((unsigned)((outs + 255) / 256)), fblock(256);
+    if (a.y_f32) {
+      return f16 ? launch_kernel(qmv_ring_fold_kernel<true, true>, fgrid, fblock, 0, st, (const float*)p.plane, a.y, a.residual, a.M, a.N, p.kparts)
+                 : launch_kernel(qmv_ring_fold_kernel<true, false>, fgrid, fblock, 0, st, (const float*)p.plane, a.y, a.residual, a.M, a.N, p.kparts);
+    }
+    return f16 ? launch_kernel(qmv_ring_fold_kernel<false, true>, fgrid, fblock, 0, st, (const float*)p.plane, a.y, a.residual, a.M, a.N, p.kparts)
+               : launch_kernel(qmv_ring_fold_kernel<false, false>, fgrid, fblock, 0, st, (const float*)p.plane, a.y, a.residual, a.M, a.N, p.kparts);
+  }
   return f16 ? launch_nw<8, true>(st, p, mr, a.y_f32) : launch_nw<8, false>(st, p, mr, a.y_f32);
 }
 
