@@ -35,6 +35,7 @@
 // tiles (4 x 8, 8 x 4, ...) so that they share rows of x and weight tiles through that XCD's L2; below
 // that, bands of 8 rows of tiles, M first inside a band.  The store goes through LDS, a wavefront's
 // block turned round 32 rows at a time, so that a store instruction covers runs of 64 NT bytes per row.
+#include <string>
 #include <type_traits>
 
 #include "vpq_device.h"
@@ -976,6 +977,32 @@ hipError_t launch_dense_gemm(hipStream_t st, const uint16_t* x, const uint16_t* 
   if (bn == 192) { return VPQ_DENSE(3); }
   return VPQ_DENSE(4);
 #undef VPQ_DENSE
+}
+
+// The contraction of the dequant-once route (the reference's `gemm_mma_`,
+// generative-models/minimax-h3/metal-minimax-h3-transformer.cc:2020-2160: affine_dequant into a scratch, then the
+// dense matrix-unit GEMM of gpu-kernels/metal/gemm/dense_gemm_mma.metal).  There the expansion costs 2*N*K bytes
+// of traffic per call; here the caller may keep the expansion of an immutable weight.  0, or -2 with *why set
+// when the shape is outside the kernel or the launch failed.
+int dense_gemm_elt(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, bool f16,
+                   int cu_count, std::string* why)
+{
+  if (!dense_gemm_supports(M, N, K)) {
+    if (why) { *why = "dense GEMM: K must be a multiple of 32 and the matrices below 4 GB"; }
+    return -2;
+  }
+  const hipError_t e = launch_dense_gemm(st, x, b, y, M, N, K, f16, cu_count);
+  if (e != hipSuccess) {
+    if (why) { *why = hipGetErrorString(e); }
+    return -2;
+  }
+  return 0;
+}
+
+int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, int cu_count,
+                    std::string* why)
+{
+  return dense_gemm_elt(st, x, b, y, M, N, K, false, cu_count, why);
 }
 
 }  // namespace vpq
