@@ -109,3 +109,41 @@ def test_build_refuses_kernels_that_spill():
                 remark(ring, vgprs=250)):                       # no headroom left
         with pytest.raises(RuntimeError, match="register allocation not allowed"):
             build._check_registers("x.hip", bad)
+
+
+def test_build_refuses_use_of_a_load_register_before_its_wait():
+    """The build walks the assembly of the kernels with asm loads into registers: from the load to the counted wait
+    that guarantees its arrival no instruction may name a destination register, on any static path."""
+    from vpipe_amd import build
+    name = "_ZN3vpq17qmv_flow_kernel_1ILi1ELi2ELb1ELb0EEEvPKtPKjS2_S2_PvijiS2_"
+
+    def kernel(body):
+        return "\t.text\n%s:\n%s\n\ts_endpgm\n.Lfunc_end0:\n" % (name, "\n".join("\t" + l for l in body))
+
+    ok = ["global_load_dwordx4 v[4:7], v1, s[2:3]",       # A
+          "global_load_dwordx4 v[8:11], v1, s[4:5]",      # B
+          "global_load_lds_dwordx4 v[2:3], off",          # to LDS: no register destination, but counted
+          "v_add_u32_e32 v1, 16, v1",                     # other registers are free
+          "s_waitcnt vmcnt(2)",                           # A has two younger operations: complete
+          "v_mov_b32_e32 v20, v4",
+          "s_waitcnt vmcnt(1)",
+          "v_mov_b32_e32 v21, v8"]
+    build._check_inflight("x.hip", kernel(ok))
+    # kernels outside the list are not walked
+    build._check_inflight("x.hip", kernel(ok[:2] + ["v_mov_b32_e32 v20, v4"]).replace("qmv_flow_kernel", "other_kernel"))
+    bad_cases = [
+        ok[:4] + ["v_mov_b32_e32 v20, v5"],                                  # a copy before any wait
+        ok[:4] + ["s_waitcnt vmcnt(2)", "v_mov_b32_e32 v20, v9"],            # B has one younger operation only
+        ok[:2] + ["v_mov_b32_e32 v6, 0"],                                    # overwritten while the load is on its way
+        ok[:2] + ["s_waitcnt lgkmcnt(0)", "ds_write_b128 v30, v[4:7]"],      # a wait on the other counter
+        # in flight on one of two joining paths
+        ["s_cbranch_scc1 .LBB0_2"] + ok[:1] + [".LBB0_2:", "v_mov_b32_e32 v20, v4"],
+        # around a loop: the load of one trip is read at the top of the next
+        [".LBB0_1:", "v_mov_b32_e32 v20, v4"] + ok[:1] + ["s_cbranch_scc1 .LBB0_1"],
+    ]
+    for body in bad_cases:
+        with pytest.raises(RuntimeError, match="used before its wait"):
+            build._check_inflight("x.hip", kernel(body))
+    # the same join is fine once both paths have waited
+    build._check_inflight("x.hip", kernel(["s_cbranch_scc1 .LBB0_2"] + ok[:1] + ["s_waitcnt vmcnt(0)", ".LBB0_2:",
+                                                                                  "v_mov_b32_e32 v20, v4"]))

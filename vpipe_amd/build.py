@@ -44,6 +44,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-u
 SCRATCH_ALLOWED = {"_ZN3vpq14qmm_big_kernelILi4ELb0ELi3EEE": 68}    # mangled-name prefix -> bytes per lane
 ASM_LOAD_KERNELS = re.compile(r"qmv_flow_kernel|qmv_ring_kernel")
 ASM_LOAD_VGPR_BUDGET = 224
+ASM_LOAD_SOURCES = ("vpq_qmv_flow.hip", "vpq_qmv_ring.hip")    # their assembly is walked by _check_inflight
 
 
 def _check_registers(src, remarks):
@@ -70,6 +71,109 @@ def _check_registers(src, remarks):
         raise RuntimeError("%s: register allocation not allowed (see build.py):\n  %s" % (src, "\n  ".join(bad)))
 
 
+# The registers of an asm load in flight, checked on the compiler's own assembly output of the kernels that have
+# such loads: from a `global_load_* vN, ...` with a register destination until the `s_waitcnt vmcnt(n)` that
+# guarantees its arrival (vector-memory operations retire in issue order, so a load with k younger operations is
+# complete after a wait for n <= k), no instruction may name one of its destination registers.  That is the whole
+# contract of gload16 / touch, and it covers what the resource checks above cannot see: a copy of the register made
+# by live-range splitting, a spill into another register, a reuse.  The walk is a forward data-flow over the basic
+# blocks (in-flight register -> fewest younger operations on any path, merged by union / minimum), so it does not
+# depend on how the compiler lays the blocks out.  It follows every static path, feasible or
+# not, so the kernels keep a wavefront that issues no such load on a path of its own.
+_VMEM = re.compile(r"^(global|buffer|flat|scratch)_(load|store|atomic)")
+_VREG = re.compile(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]")
+_LABEL = re.compile(r"^([.\w$]+):")
+
+
+def _vregs(text):
+    regs = set()
+    for m in _VREG.finditer(text):
+        if m.group(1) is not None:
+            regs.add(int(m.group(1)))
+        else:
+            regs.update(range(int(m.group(2)), int(m.group(3)) + 1))
+    return regs
+
+
+def _check_inflight(src, asm):
+    """Raises if an instruction of a kernel in `asm` touches the destination of a load that may still be in flight."""
+    bad = []
+    lines = asm.splitlines()
+    i = 0
+    while i < len(lines):
+        m = _LABEL.match(lines[i])
+        if not (m and lines[i].startswith("_Z") and ASM_LOAD_KERNELS.search(m.group(1))):
+            i += 1
+            continue
+        kernel = m.group(1)
+        # basic blocks of this function: [label, instructions]; ends at .Lfunc_end
+        blocks, cur = [], [kernel, []]
+        i += 1
+        while i < len(lines) and not lines[i].startswith(".Lfunc_end"):
+            t = lines[i].split(";")[0].strip()
+            i += 1
+            if not t:
+                continue
+            lm = _LABEL.match(t)
+            if lm:
+                blocks.append(cur)
+                cur = [lm.group(1), []]
+            elif not t.startswith("."):
+                cur[1].append(t)
+                if t.startswith(("s_branch", "s_cbranch", "s_endpgm", "s_setpc")):
+                    blocks.append(cur)
+                    cur = [None, []]
+        blocks.append(cur)
+        index = {b[0]: n for n, b in enumerate(blocks) if b[0]}
+        state_in = [None] * len(blocks)       # {register: fewest younger vector-memory operations}
+        state_in[0] = {}
+        work = [0]
+        seen_bad = set()
+        while work:
+            n = work.pop()
+            st = dict(state_in[n])
+            succ = [n + 1] if n + 1 < len(blocks) else []
+            for t in blocks[n][1]:
+                op = t.split()[0]
+                args = t[len(op):]
+                if op == "s_waitcnt":
+                    w = re.search(r"vmcnt\((\d+)\)", t)
+                    if w:
+                        st = {r: y for r, y in st.items() if y < int(w.group(1))}
+                    continue
+                hit = _vregs(args) & set(st)
+                if hit and (kernel, t) not in seen_bad:
+                    seen_bad.add((kernel, t))
+                    bad.append("%s: `%s` names v%d while a load into it may be in flight" % (kernel[:60], t, min(hit)))
+                if _VMEM.match(op):
+                    st = {r: min(y + 1, 64) for r, y in st.items()}
+                    if "_load" in op and "_lds_" not in op and not op.startswith("scratch"):
+                        for r in _vregs(args.split(",")[0]):
+                            st[r] = 0
+                if op == "s_branch":
+                    succ = []
+                if op in ("s_endpgm", "s_setpc_b64"):
+                    succ = []
+                if op.startswith(("s_branch", "s_cbranch")):
+                    tgt = t.split()[-1]
+                    if tgt in index:
+                        succ = succ + [index[tgt]]
+            for sn in succ:
+                old = state_in[sn]
+                if old is None:
+                    merged = dict(st)
+                else:
+                    merged = dict(old)
+                    for r, y in st.items():
+                        merged[r] = min(y, merged.get(r, y))
+                if merged != old:
+                    state_in[sn] = merged
+                    work.append(sn)
+    if bad:
+        raise RuntimeError("%s: register of an asm load used before its wait (see build.py):\n  %s"
+                           % (src, "\n  ".join(bad[:20])))
+
+
 def _compile(src):
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
     cmd = [HIPCC] + FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c", os.path.join(CSRC, src), "-o", obj]
@@ -78,6 +182,12 @@ def _compile(src):
         err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "remark:" not in l)
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
     _check_registers(src, r.stderr)
+    if src in ASM_LOAD_SOURCES:
+        a = subprocess.run([HIPCC] + FLAGS + ["-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", "-"],
+                           capture_output=True, text=True)
+        if a.returncode != 0:
+            raise RuntimeError("hipcc -S failed for %s:\n%s" % (src, a.stderr[-2000:]))
+        _check_inflight(src, a.stdout)
     err = "\n".join(l for l in r.stderr.splitlines()
                     if "packed-fp32-ops" not in l and "remark:" not in l and "-Rpass-analysis" not in l)
     return obj, err

@@ -276,14 +276,22 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
     }
   }
 
+  // A wavefront without rows (past N in the last workgroup) only brings its share of x and meets the barriers.  It
+  // leaves here, on a path of its own, so that no path on which code loads are in flight joins one on which they
+  // were never issued: the build checks the registers of those loads along every static path.
+  if (!active) {
+    wait_vm<0>();
+    __syncthreads();
+    if (wk > 1) { __syncthreads(); }
+    return;
+  }
+
   float tot[RB];
-#pragma unroll
-  for (int r = 0; r < RB; ++r) { tot[r] = 0.0f; }
 
   // codes
   constexpr int AFTER = NDMA;                  // requests that follow the codes
   u32x4v c[RB][SPW];
-  if (active) {
+  {
     const uint8_t* wbase = reinterpret_cast<const uint8_t*>(wq) + (size_t)row_begin * (size_t)(K >> 1);
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
@@ -297,12 +305,10 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
     }
     request_scales_biases();
     wait_vm<NL + AFTER>();                       // this wavefront's share of x has landed
-  } else {
-    wait_vm<0>();
   }
   __syncthreads();                               // ... and everybody else's share
 
-  if (active) {
+  {
     uint32_t xp[SPW][16];                        // pairs (x_i, x_{i+4}) of each run of eight
     float sx[SPW];
 #pragma unroll
@@ -388,7 +394,7 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
       }
     }
   }
-  if (!active || lane != 63) { return; }
+  if (lane != 63) { return; }
 
   if (gate_act) {
     // rows 2g and 2g+1 are the gate and the up row of feature g; RB is even, so a pair is one wavefront's
