@@ -10,9 +10,10 @@
 // LDS bytes per MFMA of a 128 x 64 block -- which is what bounds the smaller tile: there the LDS
 // pipe is busy longer than the matrix pipe.  With one wavefront per SIMD nothing else can fill the
 // matrix pipe's shadow, so every wavefront does all three jobs and the instruction stream itself
-// interleaves them: after each MFMA comes one piece (<= 8 vector instructions) of the
-// dequantization of a coming step's weight row, one fragment read for the next quarter step and, every
-// SP-th time, one load request, pinned in that order by scheduling barriers.
+// interleaves them: the work of a K step is cut into single instructions and dealt out over the step's MFMAs
+// by a plan made at compile time, at most four issue units behind each MFMA (a fragment read for the next
+// quarter step, every second time a load request, instructions of the dequantization of a coming step's
+// weight tile), written as asm statements and pinned in that order by scheduling barriers.
 //
 // Per 64-wide K step and workgroup, everything arrives by direct-to-LDS loads:
 //   x tile [256,64] bf16      8 loads per wavefront (8 rows x 128 contiguous bytes each);
@@ -28,8 +29,9 @@
 // A step has ONE barrier, at its 3/4 point (after the MFMAs of quarters 0..2, when every fragment of
 // the step is in registers): see the pipeline's comment in the kernel.  Measured on 256 x 256 tiles
 // (cycles per step; 2048 are the MFMAs alone): barrier at the step's end with the first fragment reads
-// behind it 3080, this pipeline 2400-2500 with dense weights, 2900 with the dequantization; what is
-// left over the MFMAs is the issue of the load requests (10-25 cycles each, wherever they stand).
+// behind it 3080; this pipeline with the slot plan 2200-2250 with dense weights, 2450-2550 with the
+// dequantization.  The shader clock falls as the cycles do (the part is power-limited under this load), so a
+// tenth fewer cycles has been worth 1-4 % in time.
 //
 // Tile order: from two full rounds of the chip on, the 32 workgroups an XCD runs together form a block of
 // tiles (4 x 8, 8 x 4, ...) so that they share rows of x and weight tiles through that XCD's L2; below
