@@ -107,11 +107,10 @@ int vpq_embed_gather_w4g64_bf16(vpq_stream_t stream, const int32_t* ids, const u
  * rounded result is added to it in fp32 and rounded again, as `_add` does
  * (:264-266).
  * Requires K % 64 == 0, N > 0, 1 <= M <= 16.
- * `ws` is scratch for the split-K variant: vpq_qmv_workspace_bytes() bytes,
- * 256-byte aligned, ZERO-FILLED ONCE by the caller before its first use (it
- * starts with arrival counters, which every call returns to zero; the rest
- * holds fp32 partials); it may be NULL, in which case shapes that would have
- * used split-K run unsplit.
+ * `ws` is scratch for the split of K across workgroups (fp32 planes):
+ * vpq_qmv_workspace_bytes() bytes, 16-byte aligned, no initial content
+ * needed; it may be NULL, in which case shapes that would have split K run
+ * unsplit.
  * `variant`: 0 = automatic; other values select a specific kernel for
  * measurement (see VPQ_QMV_* below). */
 int vpq_qmv_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
@@ -133,7 +132,7 @@ enum {
   VPQ_QMV_AUTO = 0,
   VPQ_QMV_SIMPLE = 1,      /* one wavefront per output row, fp32 VALU */
   VPQ_QMV_MFMA = 2,        /* LDS-staged codes, bf16 MFMA on the integer codes */
-  VPQ_QMV_MFMA_SPLITK = 3, /* as 2, K split across workgroups through `ws` */
+  /* 3 is unassigned */
   VPQ_QMV_STREAM = 4,      /* M <= 4: persistent workgroups, x staged in LDS, prefetched items */
   VPQ_QMV_RING = 5,        /* x in registers across a workgroup's tiles, codes through a two-slot LDS ring per wavefront */
   VPQ_QMV_ROWS = 6,        /* M <= 2, any K % 64: a wavefront streams whole rows with full-width loads, packed bf16
@@ -196,8 +195,7 @@ int vpq_qmm_tiled_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
  * 30-52, 66-140: f32 planes + fold, chosen by chunk width); results differ from the
  * unsplit kernel only by the fp32 reassociation and are bit-reproducible.  No
  * adapter, no gated store.  `ws`: vpq_qmm_workspace_bytes() bytes (0 where the
- * automatic choice is not to split), 256-byte aligned, contents irrelevant; if it
- * is also handed to the QMV split-K variant, zero it again first.
+ * automatic choice is not to split), 256-byte aligned, contents irrelevant.
  * VPQ_ERR_WORKSPACE if it is needed and missing or too small. */
 size_t vpq_qmm_workspace_bytes(int K, int N, int M);
 int vpq_qmm_splitk_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

@@ -12,7 +12,7 @@ from vpipe_amd import capi, synth
 
 pytestmark = pytest.mark.gpu
 
-SIMPLE, MFMA, SPLITK, AUTO = capi.VPQ_QMV_SIMPLE, capi.VPQ_QMV_MFMA, capi.VPQ_QMV_MFMA_SPLITK, capi.VPQ_QMV_AUTO
+SIMPLE, MFMA, AUTO = capi.VPQ_QMV_SIMPLE, capi.VPQ_QMV_MFMA, capi.VPQ_QMV_AUTO
 FLOW = capi.VPQ_QMV_FLOW
 
 
@@ -293,27 +293,6 @@ def test_qmv_streaming_kernel(vpq, oracle, dev, D, K, N, M):
     assert (f - f2).abs().max().item() <= 1e-5 * rms + 1e-6
 
 
-@pytest.mark.parametrize("K,N,M", [(2048, 16, 1), (4096, 64, 4), (1024, 33, 16), (8192, 48, 2)])
-def test_qmv_split_k_matches_oracle_and_is_deterministic(vpq, oracle, dev, D, K, N, M):
-    w, s, b = synth.make_weight(N, K, 31 + K)
-    x = synth.make_act(M, K, 32 + K)
-    y64, yb = oracle.qmv(w, s, b, x, K, N, M)
-    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
-    ws = vpq.qmv_workspace(K, N, M)
-    runs = []
-    for _ in range(3):
-        out = parity.Guarded((M, N), torch.bfloat16, dev)
-        vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, out=out.view, ws=ws, variant=SPLITK)
-        torch.cuda.synchronize()
-        out.assert_intact()
-        runs.append(D.bits(out.view).copy())
-        assert not ws[:256].any().item()            # arrival counters back to zero
-    parity.check_bf16(runs[0], y64, yb)
-    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
-    f = vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, ws=ws, variant=SPLITK, f32out=True)
-    parity.check_f32(f.cpu().numpy(), y64)
-
-
 @pytest.mark.parametrize("K,N,M", [(1024, 33, 16), (4096, 64, 5), (8192, 48, 2), (17408, 200, 16), (2560, 16, 9)])
 def test_qmv_ring_split_k_matches_oracle_and_is_deterministic(vpq, oracle, dev, D, K, N, M):
     """The ring kernel with K split across workgroups (fp32 planes + fold launch): oracle parity with and without a
@@ -323,7 +302,7 @@ def test_qmv_ring_split_k_matches_oracle_and_is_deterministic(vpq, oracle, dev, 
     y64, yb = oracle.qmv(w, s, b, x, K, N, M)
     wd, sd, bd, xd = stage(D, dev, w, s, b, x)
     ws = parity.Guarded((vpq.load().vpq_qmv_workspace_bytes(K, N, M) // 4,), torch.float32, dev)
-    ws.view.zero_()                                 # (the arrival counters at its start belong to the other split-K kernel)
+    ws.view.fill_(float("nan"))                     # the planes need no initial content
     runs = []
     for _ in range(3):
         out = parity.Guarded((M, N), torch.bfloat16, dev)
@@ -349,7 +328,6 @@ def test_qmv_ring_split_k_matches_oracle_and_is_deterministic(vpq, oracle, dev, 
     with pytest.raises(capi.VpqError) as e:
         vpq.qmv_w4g64(wd, sd, bd, xd, K, N, M, ws=ws.view[: M * N], variant=capi.VPQ_QMV_RING_SPLITK)
     assert e.value.status == capi.VPQ_ERR_WORKSPACE
-    assert not ws.view[:64].any().item()            # the counters' region was left alone
 
 
 def test_qmv_one_hot_reads_back_weights_exactly(vpq, oracle, dev, D):

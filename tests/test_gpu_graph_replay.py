@@ -75,7 +75,7 @@ def test_graph_replays_match_eager_calls(vpq, dev, D):
 
     def layer(o):
         vpq.qmv_w4g64(*p1, x1, K, N1, 1, out=o["single"])
-        vpq.qmv_w4g64(*p1, x1, K, N1, 1, out=o["splitk"], ws=ws_qmv, variant=capi.VPQ_QMV_MFMA_SPLITK)
+        vpq.qmv_w4g64(*p1, x1, K, N1, 1, out=o["splitk"], ws=ws_qmv, variant=capi.VPQ_QMV_RING_SPLITK)
         vpq.qmv_group_w4g64([p1 + (N1,), p2 + (N2,)], x1, K, 1, outs=[o["ga"], o["gb"]])
         vpq.qmv_w4g64(*p2, x8, K, N2, 8, out=o["ring"])
         vpq.qmv_swiglu_w4g64(*pg, x1, K, 2 * N2, 1, out=o["gated"])

@@ -11,7 +11,7 @@ from vpipe_amd import capi, synth
 
 pytestmark = pytest.mark.gpu
 
-SIMPLE, MFMA, SPLITK, RING, AUTO = (capi.VPQ_QMV_SIMPLE, capi.VPQ_QMV_MFMA, capi.VPQ_QMV_MFMA_SPLITK,
+SIMPLE, MFMA, SPLITK, RING, AUTO = (capi.VPQ_QMV_SIMPLE, capi.VPQ_QMV_MFMA, capi.VPQ_QMV_RING_SPLITK,
                                     capi.VPQ_QMV_RING, capi.VPQ_QMV_AUTO)
 
 

@@ -16,7 +16,7 @@ _SO = os.path.join(_HERE, "libvpq.so")
 _lib = None
 
 VPQ_GATE_SWIGLU, VPQ_GATE_GEGLU = 1, 2
-VPQ_QMV_AUTO, VPQ_QMV_SIMPLE, VPQ_QMV_MFMA, VPQ_QMV_MFMA_SPLITK, VPQ_QMV_STREAM, VPQ_QMV_RING, VPQ_QMV_ROWS, VPQ_QMV_FLOW = 0, 1, 2, 3, 4, 5, 6, 7
+VPQ_QMV_AUTO, VPQ_QMV_SIMPLE, VPQ_QMV_MFMA, VPQ_QMV_STREAM, VPQ_QMV_RING, VPQ_QMV_ROWS, VPQ_QMV_FLOW = 0, 1, 2, 4, 5, 6, 7
 VPQ_QMV_RING_SPLITK = 8
 
 # Every symbol include/vpq.h declares: (name, restype, argtypes).
@@ -166,7 +166,7 @@ def _check(st, where):
 
 
 def qmv_workspace(K, N, M, device="cuda"):
-    """Zero-filled split-K scratch for qmv_w4g64 (reusable across calls on one stream)."""
+    """Scratch for the split of K across workgroups in qmv_w4g64 (reusable across calls on one stream)."""
     import torch
     nbytes = load().vpq_qmv_workspace_bytes(K, N, M)
     return torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)

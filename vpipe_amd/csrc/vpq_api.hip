@@ -94,8 +94,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (gate_act != 0 && ((N & 1) != 0 || residual != nullptr || variant == VPQ_QMV_STREAM)) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
-  if (variant == VPQ_QMV_MFMA_SPLITK && ws != nullptr && !aligned(ws, 256)) { return VPQ_ERR_MISALIGNED; }   // the only user of ws
-  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_RING_SPLITK) { return VPQ_ERR_BAD_SHAPE; }
+  if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_RING_SPLITK || variant == 3) { return VPQ_ERR_BAD_SHAPE; }   // (3 is unassigned)
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
 
@@ -130,16 +129,9 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   }
   if (variant == VPQ_QMV_STREAM) {
     // handled below, after the shape check of the streaming kernel
-  } else if (variant == VPQ_QMV_MFMA || variant == VPQ_QMV_MFMA_SPLITK) {
+  } else if (variant == VPQ_QMV_MFMA) {
     if (!mfma_ok) { return VPQ_ERR_BAD_SHAPE; }
-    if (variant == VPQ_QMV_MFMA_SPLITK) {
-      if (ws == nullptr) { return VPQ_ERR_WORKSPACE; }
-      int splits = K / 512 < 4 ? K / 512 : 4;
-      if (splits < 2) { return VPQ_ERR_BAD_SHAPE; }
-      if (ws_bytes < vpq::qmv_mfma_workspace_bytes(K, N, M)) { return VPQ_ERR_WORKSPACE; }
-      return finish(vpq::launch_qmv_mfma(hs, a, splits));
-    }
-    return finish(vpq::launch_qmv_mfma(hs, a, 1));
+    return finish(vpq::launch_qmv_mfma(hs, a));
   }
   const bool stream_ok = mfma_ok && gate_act == 0 && vpq::qmv_stream_supports(K, N, M);
   if (variant == VPQ_QMV_STREAM) {
@@ -165,7 +157,7 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
     if (a.ws != nullptr && !aligned(a.ws, 16)) { a.ws = nullptr; a.ws_bytes = 0; }
     return finish(vpq::launch_qmv_ring(hs, a, 0, 0));
   }
-  if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a, 1)); }
+  if (mfma_ok) { return finish(vpq::launch_qmv_mfma(hs, a)); }
   // K not a multiple of 512, or scales / biases off 16-byte alignment: the row-streaming kernel
   // for up to two rows of x, the general one above.
   if (vpq::qmv_rows_supports(K, N, M)) { return finish(vpq::launch_qmv_rows(hs, a, 0)); }
@@ -389,7 +381,7 @@ int vpq_qmv_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t*
 size_t vpq_qmv_workspace_bytes(int K, int N, int M)
 {
   if (K <= 0 || N <= 0 || M < 1 || M > 16) { return 0; }
-  return vpq::qmv_mfma_workspace_bytes(K, N, M);
+  return (vpq::qmv_ring_workspace_bytes(K, N, M) + 255) / 256 * 256;
 }
 
 int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t,

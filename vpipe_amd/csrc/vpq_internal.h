@@ -153,7 +153,7 @@ hipError_t launch_qmv_rows8_sorted(hipStream_t st, const QmvArgs& a, const int* 
 // Returns hipErrorInvalidValue if the shape is outside what the MFMA kernel
 // handles (the caller then falls back to the simple kernel).
 bool qmv_mfma_supports(int K, int N, int M);
-hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits);
+hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a);
 // Up to four projections that share x, K and M in ONE launch (q|k|v, gate|up): a.w/scales/
 // biases/y/N/residual/ws are ignored, the segments give them.
 struct QmvSeg {
@@ -168,7 +168,6 @@ struct QmvGroup {
   QmvSeg seg[4];
 };
 hipError_t launch_qmv_mfma_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g);
-size_t qmv_mfma_workspace_bytes(int K, int N, int M);
 // Streaming kernel for M = 1 (K % 512 == 0, K >= 2048, 16-byte aligned scales / biases): one wavefront per
 // (row set, K part), every load requested up front; also as one launch over up to four packs that share x.
 bool qmv_flow_supports(int K, int N, int M);

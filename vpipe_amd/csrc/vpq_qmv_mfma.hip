@@ -4,9 +4,7 @@
 // k-values (8 quantization groups, 4 KB of codes).  A workgroup owns one 16-row
 // tile of N and a K range; its wavefronts take the items of that range
 // round-robin and their partial sums are added through LDS at the end (split-K
-// inside the workgroup).  With split_k > 1 several workgroups share a tile
-// through fp32 partials in a caller-provided workspace and the last one to
-// arrive folds them in a fixed order.
+// inside the workgroup).
 //
 // Per item and wavefront:
 //   codes   16 rows x 256 bytes, fetched with 128-bit direct-to-LDS loads in
@@ -59,12 +57,8 @@ struct QmvParams {
   const uint16_t* x;
   void* y;
   const uint16_t* residual;
-  float* partial;        // [split_k][M][N] fp32 (split_k > 1)
-  unsigned* counters;    // [tiles_n] arrival counters, zero between calls
   int K, N, M;
   int slices;            // K / 512
-  int slices_per_block;  // items of one workgroup's K range
-  int split_k;
   int wave_lds_bytes;    // codes buffer + staged x rows of one wavefront
   // Grouped launch (nseg > 1): workgroup blockIdx.x belongs to the segment whose tile range
   // holds it; each segment is its own [N_i, K] pack and output.
@@ -190,11 +184,7 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
 #pragma unroll
   for (int r = 0; r < MR; ++r) { acc[r] = 0.0f; }
 
-  const int sl_begin = blockIdx.y * p.slices_per_block;
-  int sl_end = sl_begin + p.slices_per_block;
-  if (sl_end > p.slices) { sl_end = p.slices; }
-
-  for (int sl = sl_begin + wave; sl < sl_end; sl += NW) {
+  for (int sl = wave; sl < p.slices; sl += NW) {
     // 1. codes: global -> LDS, no registers in between.
     const uint8_t* wbase = wtile + (size_t)sl * kRowBytes;
 #pragma unroll
@@ -294,26 +284,6 @@ __global__ __launch_bounds__(1024) void qmv_mfma_kernel(const QmvParams p)
   }
   const bool valid = owner && m < p.M && n < N_;
 
-  if (p.split_k > 1) {
-    // Publish this workgroup's partial, then let the last arrival fold all of
-    // them in index order (deterministic whatever the arrival order).
-    if (valid) { p.partial[((size_t)blockIdx.y * p.M + m) * p.N + n] = total; }
-    __threadfence();
-    __syncthreads();
-    __shared__ unsigned arrived;
-    if (t == 0) { arrived = atomicAdd(&p.counters[blockIdx.x], 1u); }
-    __syncthreads();
-    if (arrived != (unsigned)(p.split_k - 1)) { return; }
-    __threadfence();
-    if (valid) {
-      total = 0.0f;
-      for (int sk = 0; sk < p.split_k; ++sk) {
-        total += __builtin_nontemporal_load(&p.partial[((size_t)sk * p.M + m) * p.N + n]);
-      }
-    }
-    if (t == 0) { p.counters[blockIdx.x] = 0u; }
-  }
-
   if (p.gate_act) {
     // Lanes 2j and 2j+1 hold the gate and the up sum of feature (n0 + 2j) / 2; N is even, so both
     // are valid or neither.
@@ -350,23 +320,6 @@ namespace {
 // LDS, so this stays below the 160 KB of a CU.
 constexpr int kMaxLdsBytes = kMaxWaves * (kItemBytes + 4 * kXRowBytes + kXsumBytes) + kMaxWaves * 4 * kWave * 4;
 
-// Number of K ranges (workgroups per 16-row tile) for a shape: split only when
-// the tiles alone leave most of the chip idle.
-int choose_split(int K, int N, int cu_count)
-{
-  const int tiles = (N + kTileN - 1) / kTileN;
-  const int slices = K / kKS;
-  int split = 1;
-  while (tiles * split < cu_count && split * 2 <= slices && split < 8) { split *= 2; }
-  return split;
-}
-
-size_t counters_bytes(int N)
-{
-  const size_t tiles = (size_t)(N + kTileN - 1) / kTileN;
-  return (tiles * sizeof(unsigned) + 255) / 256 * 256;
-}
-
 }  // namespace
 
 bool qmv_mfma_supports(int K, int N, int M)
@@ -374,14 +327,7 @@ bool qmv_mfma_supports(int K, int N, int M)
   return K % kKS == 0 && N >= 1 && M >= 1 && M <= 16;
 }
 
-size_t qmv_mfma_workspace_bytes(int K, int N, int M)
-{
-  (void)K;
-  const size_t part = (size_t)8 * (size_t)M * (size_t)N * sizeof(float);
-  return counters_bytes(N) + (part + 255) / 256 * 256;
-}
-
-hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
+hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a)
 {
   QmvParams p;
   p.w = a.w; p.scales = a.scales; p.biases = a.biases; p.x = a.x; p.y = a.y;
@@ -391,26 +337,10 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   p.nseg = 1;
   p.slices = a.K / kKS;
 
-  int split = force_splits > 0 ? force_splits : choose_split(a.K, a.N, a.cu_count);
-  if (split > p.slices) { split = p.slices; }
-  if (split > 8) { split = 8; }
-  const size_t need = counters_bytes(a.N) + (size_t)split * a.M * a.N * sizeof(float);
-  if (split > 1 && (a.ws == nullptr || a.ws_bytes < need)) {
-    if (force_splits > 1) { return hipErrorInvalidValue; }
-    split = 1;
-  }
-  p.slices_per_block = (p.slices + split - 1) / split;
-  split = (p.slices + p.slices_per_block - 1) / p.slices_per_block;
-  p.split_k = split;
-  p.counters = reinterpret_cast<unsigned*>(a.ws);
-  p.partial = (a.ws != nullptr)
-                  ? reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.ws) + counters_bytes(a.N))
-                  : nullptr;
-
   // Wavefronts per workgroup: every wavefront gets the same number of items
   // where the slice count allows it.
-  const int per_wave = (p.slices_per_block + kMaxWaves - 1) / kMaxWaves;
-  int nw = (p.slices_per_block + per_wave - 1) / per_wave;
+  const int per_wave = (p.slices + kMaxWaves - 1) / kMaxWaves;
+  int nw = (p.slices + per_wave - 1) / per_wave;
   int mr = (a.M + 3) / 4;
   if (mr == 3) { mr = 4; }
   // The final reduction is done by mr*64 threads.
@@ -419,7 +349,7 @@ hipError_t launch_qmv_mfma(hipStream_t st, const QmvArgs& a, int force_splits)
   const bool xlds = a.M <= 4;
   p.wave_lds_bytes = kItemBytes + (xlds ? a.M * kXRowBytes + kXsumBytes : 0);
   const size_t lds_bytes = (size_t)nw * p.wave_lds_bytes + (size_t)nw * mr * kWave * sizeof(float);
-  const dim3 grid((unsigned)((a.N + kTileN - 1) / kTileN), (unsigned)split), block((unsigned)(nw * kWave));
+  const dim3 grid((unsigned)((a.N + kTileN - 1) / kTileN)), block((unsigned)(nw * kWave));
 
   // the attribute is set once per kernel, whichever thread comes first (atomic flags: two threads may both set
   // it, which is harmless; neither launches before its own call has returned)
@@ -451,10 +381,6 @@ hipError_t launch_qmv_mfma_group(hipStream_t st, const QmvArgs& a, const QmvGrou
   p.K = a.K; p.N = 0; p.M = a.M;
   p.gate_act = 0;
   p.slices = a.K / kKS;
-  p.slices_per_block = p.slices;
-  p.split_k = 1;
-  p.counters = nullptr;
-  p.partial = nullptr;
   p.nseg = g.count;
   int tiles = 0;
   for (int i = 0; i < 4; ++i) {

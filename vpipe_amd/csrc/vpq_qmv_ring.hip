@@ -482,8 +482,7 @@ size_t qmv_ring_workspace_bytes(int K, int N, int M)
 {
   if (!qmv_ring_supports(K, N, M) || K / kKS < 2) { return 0; }
   const int parts = K / kKS < 4 ? K / kKS : 4;
-  const size_t header = ((size_t)((N + kTileN - 1) / kTileN) * sizeof(unsigned) + 255) / 256 * 256;
-  return header + (size_t)parts * (size_t)M * (size_t)N * sizeof(float);
+  return (size_t)parts * (size_t)M * (size_t)N * sizeof(float);
 }
 
 namespace {
@@ -546,18 +545,18 @@ hipError_t launch_qmv_ring(hipStream_t st, const QmvArgs& a, int tc_hint, int sp
   // unsplit / 4 parts): 17408 -> 5120 at 16 rows 26.3 / 23.5, at 8 rows 21.4 / 20.5, at 4 rows 17.2 / 22.5;
   // 5120 -> 5120 at 16 rows 11.7 / 14.8; 5120 -> 17408 at 16 rows 19.4 / 31.1; 5120 -> 151936 123.8 / 202.2: the
   // fold's launch and the shorter K walks cost more than the re-read x except for many rows over a deep K with few
-  // tiles per CU.  The planes start behind the arrival counters of the other split-K kernel, which must stay zero.
+  // tiles per CU.  Every element of a plane is written by exactly one workgroup before the fold reads it, so the
+  // workspace needs no clearing.
   p.kparts = 1;
   p.part_slices = p.slices;
   p.plane = nullptr;
-  const size_t ws_header = ((size_t)p.tiles * sizeof(unsigned) + 255) / 256 * 256;
   if (splits_hint != 1 && a.ws != nullptr && p.slices >= 2 && a.gate_act == 0) {     // (the gated entry points take no workspace)
     int parts = splits_hint > 1 ? splits_hint : ((a.M >= 8 && p.slices >= 24 && p.tiles <= 2 * cus) ? 4 : 1);
     if (parts > p.slices) { parts = p.slices; }
-    if (parts > 1 && ws_header + (size_t)parts * (size_t)a.M * (size_t)a.N * sizeof(float) <= a.ws_bytes) {
+    if (parts > 1 && (size_t)parts * (size_t)a.M * (size_t)a.N * sizeof(float) <= a.ws_bytes) {
       p.part_slices = (p.slices + parts - 1) / parts;
       p.kparts = (p.slices + p.part_slices - 1) / p.part_slices;      // no empty part
-      p.plane = reinterpret_cast<float*>(static_cast<uint8_t*>(a.ws) + ws_header);
+      p.plane = static_cast<float*>(a.ws);
       int tcp = 1;
       plan(mr, p.kparts, tcp);
       tc = tcp;
