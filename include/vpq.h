@@ -672,6 +672,17 @@ int vpq_qmv_gated_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16
 int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                       const uint16_t* biases, const uint16_t* x, uint16_t* y,
                       int K, int N, int M, int activation);
+/* The runtime adapter on binary16 elements (the half build of `lora_gemm_a_` / the SCALED and the fused tile of
+ * gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273, 297-348, whose element type is VPIPE_ELT, :28-33):
+ * vpq_lora_a_f16 is t[M,r] = f16(alpha * f16(x . A^T)); vpq_qmm_lora_w4g64_f16 is vpq_qmm_w4g64_f16 (no
+ * activation) with y += t . B^T in the same accumulators before the one rounding.  A [r,K], B [N,r], t scratch
+ * [M,r], all binary16; r % 16 == 0, 16 <= r <= VPQ_LORA_MAX_RANK; lora_a == NULL or alpha == 0: no adapter. */
+int vpq_lora_a_f16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t,
+                   int M, int K, int r, float alpha);
+int vpq_qmm_lora_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                           const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                           const uint16_t* lora_a, const uint16_t* lora_b, int r, float alpha,
+                           uint16_t* lora_t_ws);
 /* The grouped launch on binary16 elements (`affine_qmv_qkv_w4g64` of the half build, affine_qmv.metal:497-516):
  * arguments and results as vpq_qmv_group_w4g64_bf16 -- bit-identical to `count` calls of vpq_qmv_w4g64_f16; one
  * launch at M = 1 on K % 512 == 0, K >= 2048 with 16-byte aligned scales / biases, separate calls otherwise. */

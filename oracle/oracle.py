@@ -257,6 +257,25 @@ def matmul_f16(w, s, b, x, K, N, M, rounded, residual=None):
     return y64, yh
 
 
+def lora_t_f16(x, A, M, K, r, alpha):
+    """binary16 x [M,K], A [r,K] -> t [M,r] binary16 bits, two roundings."""
+    x, A = _c(x, np.uint16), _c(A, np.uint16)
+    t = np.empty((M, r), dtype=np.uint16)
+    lib().vpo_lora_t_f16(_p(x, _u16p), _p(A, _u16p), _p(t, _u16p), M, K, r, ctypes.c_float(alpha))
+    return t
+
+
+def qmm_lora_f16(w, s, b, x, K, N, M, t, B, r):
+    """binary16 elements, rounded weights, the adapter's t . B^T in the same accumulator -> (y64, y_f16 bits)."""
+    w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
+    t, B = _c(t, np.uint16), _c(B, np.uint16)
+    y64 = np.empty((M, N), dtype=np.float64)
+    yh = np.empty((M, N), dtype=np.uint16)
+    lib().vpo_qmm_lora_w4g64_f16(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y64, _f64p), _p(yh, _u16p),
+                                 K, N, M, _p(t, _u16p), _p(B, _u16p), r)
+    return y64, yh
+
+
 _i32p = ctypes.POINTER(ctypes.c_int32)
 
 

@@ -811,6 +811,52 @@ void vpo_matmul_w4g64_f16(const uint32_t* w, const uint16_t* scales, const uint1
   free(wrow);
 }
 
+/* The adapter on binary16 elements: gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273 with VPIPE_ELT = half
+ * (:28-33) -- t[M,r] = f16((float)f16(x . A^T) * alpha), two roundings, the contraction in double. */
+void vpo_lora_t_f16(const uint16_t* x, const uint16_t* A, uint16_t* t, int M, int K, int r, float alpha)
+{
+  for (size_t m = 0; m < (size_t)M; ++m) {
+    for (int j = 0; j < r; ++j) {
+      double acc = 0.0;
+      for (int k = 0; k < K; ++k) {
+        acc += (double)vpo_f16_to_f32(x[m * (size_t)K + k]) * (double)vpo_f16_to_f32(A[(size_t)j * K + k]);
+      }
+      const float once = vpo_f16_to_f32(vpo_f32_to_f16((float)acc));
+      t[m * (size_t)r + j] = vpo_f32_to_f16(once * alpha);
+    }
+  }
+}
+
+/* The fused GEMM on binary16 elements with the adapter's second factor in the same accumulator before the one
+ * store (dense_gemm_mma.metal:297-348): y = f16(x . f16(s q + b)^T + t . B^T), B [N,r], t from vpo_lora_t_f16;
+ * contraction in double. */
+void vpo_qmm_lora_w4g64_f16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, const uint16_t* x,
+                            double* y64, uint16_t* y_f16, int K, int N, int M, const uint16_t* t, const uint16_t* B,
+                            int r)
+{
+  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_f16_to_f32(scales[n * Kg + k / VPO_GROUP]);
+      const float b = vpo_f16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float sq = s * (float)nibble(w, n, Kw, k);
+      wrow[k] = vpo_f16_to_f32(vpo_f32_to_f16(sq + b));
+    }
+    for (size_t m = 0; m < (size_t)M; ++m) {
+      double acc = 0.0;
+      const uint16_t* xr = x + m * (size_t)K;
+      for (int k = 0; k < K; ++k) { acc += (double)vpo_f16_to_f32(xr[k]) * (double)wrow[k]; }
+      for (int j = 0; j < r; ++j) {
+        acc += (double)vpo_f16_to_f32(t[m * (size_t)r + j]) * (double)vpo_f16_to_f32(B[n * (size_t)r + j]);
+      }
+      if (y64) { y64[m * (size_t)N + n] = acc; }
+      if (y_f16) { y_f16[m * (size_t)N + n] = vpo_f32_to_f16((float)acc); }
+    }
+  }
+  free(wrow);
+}
+
 /* ---- MoE prefill: the expert sort and the grouped GEMMs ------------------- */
 
 /* gpu-kernels/metal/ops/llm_elementwise.metal:255-326 (moe_ifill_i32, moe_hist_i32,

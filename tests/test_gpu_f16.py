@@ -211,6 +211,50 @@ def test_qmm_f16_fused(vpq, oracle, dev, D, M, N, K):
         check_f16(bits16(og.view), g64)
 
 
+@pytest.mark.parametrize("M,N,K,r", [(64, 64, 512, 16), (130, 328, 1024, 32), (300, 520, 1536, 48), (257, 136, 512, 128),
+                                     (96, 200, 1024, 384)])
+def test_qmm_f16_fused_with_adapter(vpq, oracle, dev, D, M, N, K, r):
+    """The adapter on binary16 elements: t bit for bit against the oracle where the fp32 sum is not at a rounding
+    boundary (at most a handful of elements one step off), the fused GEMM against the oracle's twin, alpha = 0 the
+    plain GEMM's bits, guard bands intact."""
+    w, s, b = f16_pack(N, K, 800 + M)
+    rng = np.random.default_rng(801 + M)
+    x = rng.standard_normal((M, K)).astype(np.float16).view(np.uint16)
+    A = (0.05 * rng.standard_normal((r, K))).astype(np.float16).view(np.uint16)
+    B = (0.05 * rng.standard_normal((N, r))).astype(np.float16).view(np.uint16)
+    alpha = 0.75
+    wd, sd, bd, xd, Ad, Bd = D.u32(w, dev), dev16(s, dev), dev16(b, dev), dev16(x, dev), dev16(A, dev), dev16(B, dev)
+    t_want = oracle.lora_t_f16(x, A, M, K, r, alpha)
+    t_got = parity.Guarded((M, r), torch.float16, dev)
+    vpq.lora_a_f16(xd, Ad, M, K, r, alpha, out=t_got.view)
+    torch.cuda.synchronize()
+    t_got.assert_intact()
+    tg = bits16(t_got.view)
+    off = tg != t_want
+    assert off.mean() <= 0.01
+    assert np.abs(tg.view(np.float16).astype(np.float64) - t_want.view(np.float16).astype(np.float64)).max() <= \
+        2.0 ** -10 * np.abs(t_want.view(np.float16).astype(np.float64)).max()
+    # the GEMM against the oracle fed with the t the device produced (its own rounding-boundary cases included)
+    y64, _ = oracle.qmm_lora_f16(w, s, b, x, K, N, M, tg, B, r)
+    out = parity.Guarded((M, N), torch.float16, dev)
+    t_ws = parity.Guarded((M, r), torch.float16, dev)
+    vpq.qmm_lora_w4g64_f16(wd, sd, bd, xd, K, N, M, Ad, Bd, r, alpha, out=out.view, t_ws=t_ws.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    t_ws.assert_intact()
+    assert torch.equal(t_ws.view, t_got.view)
+    check_f16(bits16(out.view), y64)
+    base64, _ = oracle.matmul_f16(w, s, b, x, K, N, M, rounded=True)
+    assert np.sqrt(((y64 - base64) ** 2).sum() / (y64 ** 2).sum()) > 1e-3          # the adapter is live
+    plain = vpq.qmm_w4g64_f16(wd, sd, bd, xd, K, N, M)
+    assert torch.equal(vpq.qmm_lora_w4g64_f16(wd, sd, bd, xd, K, N, M, Ad, Bd, r, 0.0), plain)
+    L = vpq.load()
+    p = out.view.data_ptr()
+    assert L.vpq_qmm_lora_w4g64_f16(None, p, p, p, p, p, K, N, M, p, p, 40, 1.0, p) == -2
+    assert L.vpq_qmm_lora_w4g64_f16(None, p, p, p, p, p, K, N, M, p, p, r, 1.0, None) == -4
+    assert L.vpq_lora_a_f16(None, p, p, p, M, K, 528, 1.0) == -2
+
+
 def test_qmm_f16_fused_rejects(vpq, dev):
     L = vpq.load()
     p = torch.zeros(1 << 16, dtype=torch.int32, device=dev).data_ptr()

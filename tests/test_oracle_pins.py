@@ -601,6 +601,34 @@ def test_f16_element_twins_against_numpy_float16(oracle):
     assert np.array_equal(ya, want_add.view(np.uint16))
 
 
+def test_f16_adapter_against_numpy_float16(oracle):
+    """The adapter on binary16 elements, written independently in numpy: t = f16(alpha * f16(x . A^T)) with the
+    contraction in float64 and numpy's own float16 casts, then y = f16(x . f16(W)^T + t . B^T); an adapter whose t is
+    zero leaves the base GEMM's bits; the delta is a visible part of the output."""
+    N, K, M, R = 21, 256, 5, 48
+    alpha = 0.625
+    w, s, b = f16_pack(N, K, 61)
+    rng = np.random.default_rng(62)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    A = (0.05 * rng.standard_normal((R, K))).astype(np.float16)
+    B = (0.05 * rng.standard_normal((N, R))).astype(np.float16)
+    t = oracle.lora_t_f16(x.view(np.uint16), A.view(np.uint16), M, K, R, alpha)
+    tt = (x.astype(np.float64) @ A.astype(np.float64).T).astype(np.float32).astype(np.float16)
+    want_t = (tt.astype(np.float32) * np.float32(alpha)).astype(np.float16)
+    assert np.array_equal(t, want_t.view(np.uint16))
+    y64, yh = oracle.qmm_lora_f16(w, s, b, x.view(np.uint16), K, N, M, t, B.view(np.uint16), R)
+    Wh = oracle.dequant_f16(w, s, b, K, N).view(np.float16).astype(np.float64)      # pinned above against numpy
+    base = x.astype(np.float64) @ Wh.T
+    delta = want_t.astype(np.float64) @ B.astype(np.float64).T
+    ref = base + delta
+    assert np.allclose(y64, ref, rtol=0, atol=1e-12 * np.abs(ref).max() + 1e-12)
+    assert np.array_equal(yh, ref.astype(np.float32).astype(np.float16).view(np.uint16))
+    assert np.sqrt((delta ** 2).sum() / (ref ** 2).sum()) > 0.01
+    b64, bh = oracle.matmul_f16(w, s, b, x.view(np.uint16), K, N, M, rounded=True)
+    z64, zh = oracle.qmm_lora_f16(w, s, b, x.view(np.uint16), K, N, M, np.zeros_like(t), B.view(np.uint16), R)
+    assert np.array_equal(z64, b64) and np.array_equal(zh, bh)
+
+
 def test_grouped_gemm_oracle_with_byte_codes_reduces_to_the_plain_8bit_gemm(oracle):
     """The 8-bit form of the grouped restatement: every live slot equals the plain 8-bit GEMM oracle
     (bf16-rounded weights) of its row on its expert's slab."""

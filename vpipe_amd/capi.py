@@ -82,6 +82,8 @@ SYMBOLS = [
     ("vpq_qmv_gated_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmm_dense_route_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_qmm_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    ("vpq_lora_a_f16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f]),
+    ("vpq_qmm_lora_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _f, _vp]),
     ("vpq_qmm_tiled_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     ("vpq_qmm_tiled_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     ("vpq_dequant_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
@@ -666,6 +668,26 @@ def qmm_w4g64_f16(w, scales, biases, x, K, N, M, activation=0, out=None):
         out = torch.empty((M, N // 2 if activation else N), dtype=torch.float16, device=w.device)
     _check(load().vpq_qmm_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
                                     activation), "vpq_qmm_w4g64_f16")
+    return out
+
+
+def lora_a_f16(x, A, M, K, r, alpha, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, r), dtype=torch.float16, device=x.device)
+    _check(load().vpq_lora_a_f16(_stream(), _ptr(x), _ptr(A), _ptr(out), M, K, r, alpha), "vpq_lora_a_f16")
+    return out
+
+
+def qmm_lora_w4g64_f16(w, scales, biases, x, K, N, M, lora_A, lora_B, r, alpha, out=None, t_ws=None):
+    """The fused binary16 GEMM with a runtime adapter (A [r,K], B [N,r], binary16)."""
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=w.device)
+    if t_ws is None:
+        t_ws = torch.empty((M, r), dtype=torch.float16, device=w.device)
+    _check(load().vpq_qmm_lora_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                         _ptr(lora_A), _ptr(lora_B), r, alpha, _ptr(t_ws)), "vpq_qmm_lora_w4g64_f16")
     return out
 
 

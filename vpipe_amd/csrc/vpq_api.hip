@@ -619,6 +619,48 @@ int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* sc
   return finish(vpq::launch_qmm_big(reinterpret_cast<hipStream_t>(stream), g, 0));
 }
 
+int vpq_lora_a_f16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t, int M, int K, int r,
+                   float alpha)
+{
+  if (x == nullptr || lora_a == nullptr || t == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M <= 0 || K <= 0 || (K % 64) != 0 || r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(lora_a, 16) || !aligned(t, 16)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_lora_a(reinterpret_cast<hipStream_t>(stream), x, lora_a, t, M, K, r, alpha, true));
+}
+
+// The fused GEMM on binary16 elements with a runtime adapter: the pre-pass t = f16(alpha * f16(x . A^T)), then the
+// large-tile kernel with r more values of K from t and B in the same accumulators.  alpha == 0 or lora_a == NULL: no
+// adapter.
+int vpq_qmm_lora_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           const uint16_t* x, uint16_t* y, int K, int N, int M, const uint16_t* lora_a,
+                           const uint16_t* lora_b, int r, float alpha, uint16_t* lora_t_ws)
+{
+  const bool lora = lora_a != nullptr && alpha != 0.0f;
+  if (!lora) { return vpq_qmm_w4g64_f16(stream, w, scales, biases, x, y, K, N, M, 0); }
+  int st = check_pack(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr || lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
+  if (M <= 0 || r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) {
+    return VPQ_ERR_MISALIGNED;
+  }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::GemmArgs g{};
+  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
+  g.K = K; g.N = N; g.M = M;
+  g.lora_t = lora_t_ws; g.lora_b = lora_b; g.r = r;
+  g.cu_count = g_dev.cu_count;
+  g.f16 = true;
+  if (!vpq::qmm_big_supports(g)) { return VPQ_ERR_BAD_SHAPE; }
+  st = vpq_lora_a_f16(stream, x, lora_a, lora_t_ws, M, K, r, alpha);
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_qmm_big(reinterpret_cast<hipStream_t>(stream), g, 0));
+}
+
 int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                                   uint16_t* w_deq, int expand)

@@ -207,7 +207,7 @@ hipError_t launch_argmax_combine(hipStream_t st, const float* partials, int* out
 // Adapter ranks: multiples of 16 up to this (the reference runs 16 and measures 384).
 constexpr int kLoraMaxRank = 512;
 hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
-                         float alpha);
+                         float alpha, bool f16 = false);
 // 256x128-tile quantized GEMM (+ fused LoRA second factor); a.w must be non-null.
 hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a);
 // Grouped (expert-sorted) form of the tile kernel at 128 rows per block: a.w/scales/biases are the

@@ -1,4 +1,5 @@
-// The adapter's first factor: t[M,r] = bf16(alpha * bf16(x[M,K] . A[r,K]^T)), any rank that is a multiple of 16
+// The adapter's first factor: t[M,r] = elt(alpha * elt(x[M,K] . A[r,K]^T)), elt = bf16 or IEEE binary16 (the
+// reference's VPIPE_ELT, gpu-kernels/metal/gemm/dense_gemm_mma.metal:28-33), any rank that is a multiple of 16
 // up to kLoraMaxRank (the SCALED tile of gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273, driven by
 // lora_gemm_a_, generative-models/minimax-h3/metal-minimax-h3-transformer.cc:1030-1067; the reference runs rank 16
 // adapters and measures rank 384, metal-minimax-h3-transformer.h:365-367, .cc:1126-1132).
@@ -34,7 +35,7 @@ struct LoraAParams {
 
 }  // namespace
 
-template <int NT>
+template <int NT, bool F16 = false>
 __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p)
 {
   __shared__ float part[(kWaves / 2) * NT * 16 * 64];   // four wavefronts' tiles at a time
@@ -69,7 +70,15 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p
 #pragma unroll
       for (int j = 0; j < 4; ++j) { ab[j] = *reinterpret_cast<const bf16x8*>(ac + 8 * j); }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) { acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[j], ab[j], acc[n], 0, 0, 0); }
+      for (int j = 0; j < 4; ++j) {
+        if constexpr (F16) {
+          typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+          acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, xa[j]), __builtin_bit_cast(halfx8, ab[j]),
+                                                          acc[n], 0, 0, 0);
+        } else {
+          acc[n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[j], ab[j], acc[n], 0, 0, 0);
+        }
+      }
     }
   }
 
@@ -104,8 +113,8 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + 8 * (e >> 2) + 4 * half + (e & 3);
         if (m < p.M && r0 + n * 32 + col < p.r) {
-          const float v = bf16_bits_to_f32(f32_to_bf16_bits(acc[n][e]));
-          p.t[(size_t)m * p.r + r0 + n * 32 + col] = (uint16_t)f32_to_bf16_bits(p.alpha * v);
+          const float v = elt_bits_to_f32<F16>(f32_to_elt_bits<F16>(acc[n][e]));
+          p.t[(size_t)m * p.r + r0 + n * 32 + col] = (uint16_t)f32_to_elt_bits<F16>(p.alpha * v);
         }
       }
     }
@@ -113,12 +122,21 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p
 }
 
 hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
-                         float alpha)
+                         float alpha, bool f16)
 {
   if (r < 16 || r % 16 != 0 || r > kLoraMaxRank) { return hipErrorInvalidValue; }
   LoraAParams p{x, a, t, M, K, r, alpha};
   const dim3 grid((unsigned)((M + kRows - 1) / kRows), (unsigned)((r + 127) / 128)), block(kWaves * 64);
-  switch (r > 128 ? 4 : (r + 31) / 32) {   // tiles of 32 columns per block
+  const int nt = r > 128 ? 4 : (r + 31) / 32;   // tiles of 32 columns per block
+  if (f16) {
+    switch (nt) {
+      case 1: return launch_kernel(lora_a_kernel<1, true>, grid, block, 0, st, p);
+      case 2: return launch_kernel(lora_a_kernel<2, true>, grid, block, 0, st, p);
+      case 3: return launch_kernel(lora_a_kernel<3, true>, grid, block, 0, st, p);
+      default: return launch_kernel(lora_a_kernel<4, true>, grid, block, 0, st, p);
+    }
+  }
+  switch (nt) {
     case 1: return launch_kernel(lora_a_kernel<1>, grid, block, 0, st, p);
     case 2: return launch_kernel(lora_a_kernel<2>, grid, block, 0, st, p);
     case 3: return launch_kernel(lora_a_kernel<3>, grid, block, 0, st, p);

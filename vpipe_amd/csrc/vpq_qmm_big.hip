@@ -852,9 +852,9 @@ bool qmm_big_supports(const GemmArgs& a)
   if ((reinterpret_cast<uintptr_t>(a.scales) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.biases) & 15) != 0) { return false; }
   if ((double)a.N * (double)a.K / (a.bits == 8 ? 1.0 : 2.0) >= 4.0e9 || (double)BM * (double)a.K * 2.0 >= 4.0e9) { return false; }
   if (a.lora_t != nullptr && (a.r < 16 || a.r % 16 != 0)) { return false; }
-  // the other formats and the binary16 elements come without the adapter path, and not combined
+  // the other code formats come without the adapter path; formats and element types are not combined
   const int modes = (a.bits == 8) + (a.group == 32) + (a.f16 ? 1 : 0);
-  if (modes > 1 || (modes == 1 && a.lora_t != nullptr)) { return false; }
+  if (modes > 1 || (modes == 1 && !a.f16 && a.lora_t != nullptr)) { return false; }
   if ((a.bits != 4 && a.bits != 8) || (a.group != 64 && a.group != 32)) { return false; }
   return true;
 }
@@ -934,11 +934,17 @@ hipError_t launch_qmm_big(hipStream_t st, const GemmArgs& a, int tile_n)
     return launch_kernel(qmm_big_kernel<4, false, kPacked4G32>, grid, block, 0, st, p);
   }
   if (a.f16) {
-    // IEEE binary16 elements: the plain and the gated GEMM (no adapter path)
-    if (lora) { return hipErrorInvalidValue; }
-    if (bn == 128) { return launch_kernel(qmm_big_kernel<2, false, kPacked4F16>, grid, block, 0, st, p); }
-    if (bn == 192) { return launch_kernel(qmm_big_kernel<3, false, kPacked4F16>, grid, block, 0, st, p); }
-    return launch_kernel(qmm_big_kernel<4, false, kPacked4F16>, grid, block, 0, st, p);
+    // IEEE binary16 elements
+    if (bn == 128) {
+      return lora ? launch_kernel(qmm_big_kernel<2, true, kPacked4F16>, grid, block, 0, st, p)
+                  : launch_kernel(qmm_big_kernel<2, false, kPacked4F16>, grid, block, 0, st, p);
+    }
+    if (bn == 192) {
+      return lora ? launch_kernel(qmm_big_kernel<3, true, kPacked4F16>, grid, block, 0, st, p)
+                  : launch_kernel(qmm_big_kernel<3, false, kPacked4F16>, grid, block, 0, st, p);
+    }
+    return lora ? launch_kernel(qmm_big_kernel<4, true, kPacked4F16>, grid, block, 0, st, p)
+                : launch_kernel(qmm_big_kernel<4, false, kPacked4F16>, grid, block, 0, st, p);
   }
   if (bn == 128) {
     return lora ? launch_kernel(qmm_big_kernel<2, true>, grid, block, 0, st, p)
