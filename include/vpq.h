@@ -653,11 +653,10 @@ int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const
  *                                 470-560) and, with activation VPQ_GATE_SWIGLU / VPQ_GATE_GEGLU, the gated
  *                                 `affine_qmm_swiglu_w4g64*`, `affine_qmm_geglu_w4g64` (y [M,N/2], N even) on
  *                                 binary16 elements: weight tile = f16_rne(fp32(s*q+b)), f16 MFMA, fp32
- *                                 accumulation, one rounding -- the large-tile kernel of the bf16 entry, so it
- *                                 needs K % 512 == 0 and 16-byte aligned scales / biases (VPQ_ERR_BAD_SHAPE
- *                                 otherwise: take the dequant-once route); x and y 16-byte aligned.  Its
- *                                 results have the bits of the dequant-once route where that picks the same
- *                                 tile width.
+ *                                 accumulation, one rounding -- the kernels of the bf16 entry (the large-tile
+ *                                 kernel once its tiles fill the CUs, K % 512 == 0 and 16-byte aligned scales /
+ *                                 biases; the 256 x 128 tile kernel otherwise, any K % 64 == 0); x and y
+ *                                 16-byte aligned.  Its results have the bits of the dequant-once route.
  * Requirements as for the bf16 entries. */
 int vpq_dequant_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, uint16_t* w_deq, int K, int N);

@@ -596,10 +596,14 @@ int vpq_qmv_gated_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16
   return qmv_f16_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, activation);
 }
 
-// The fused GEMM on binary16 elements: the large-tile kernel only (K % 512 == 0, 16-byte aligned scales and
-// biases); activation 0 = plain y [M,N], else the gated store of an interleaved gate|up pack, y [M,N/2].
-int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
-                      const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
+namespace {
+
+// The fused GEMM on binary16 elements: the large-tile kernel once its tiles fill the CUs (K % 512 == 0, 16-byte
+// aligned scales and biases), the 256 x 128 tile kernel otherwise -- same MFMA, same K order, same bits.
+// activation 0 = plain y [M,N], else the gated store of an interleaved gate|up pack, y [M,N/2] (no adapter then).
+int qmm_f16_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, uint16_t* y, int K, int N, int M, int activation, const uint16_t* lora_a,
+                   const uint16_t* lora_b, int r, float alpha, uint16_t* lora_t_ws)
 {
   int st = check_pack(w, scales, biases, K, N);
   if (st != VPQ_OK) { return st; }
@@ -607,16 +611,44 @@ int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* sc
   if (activation != 0 && activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
   if (M <= 0 || (activation != 0 && (N & 1) != 0)) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(y, 16)) { return VPQ_ERR_MISALIGNED; }
+  const bool lora = lora_a != nullptr && alpha != 0.0f;
+  if (lora) {
+    if (activation != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
+    if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
+    if (r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (!aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) { return VPQ_ERR_MISALIGNED; }
+  }
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (lora) {
+    st = finish(vpq::launch_lora_a(hs, x, lora_a, lora_t_ws, M, K, r, alpha, true));
+    if (st != VPQ_OK) { return st; }
+  }
   vpq::GemmArgs g{};
   g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
   g.K = K; g.N = N; g.M = M;
+  g.lora_t = lora ? lora_t_ws : nullptr;
+  g.lora_b = lora ? lora_b : nullptr;
+  g.r = lora ? r : 0;
   g.cu_count = g_dev.cu_count;
   g.gate_act = activation;
   g.f16 = true;
-  if (!vpq::qmm_big_supports(g)) { return VPQ_ERR_BAD_SHAPE; }
-  return finish(vpq::launch_qmm_big(reinterpret_cast<hipStream_t>(stream), g, 0));
+  if (vpq::qmm_big_supports(g)) {
+    const int bn = vpq::qmm_big_tile_n(N, M, g_dev.cu_count);
+    const long tiles = (long)((M + 255) / 256) * (long)((N + bn - 1) / bn);
+    if (tiles >= (long)(g_dev.cu_count > 0 ? g_dev.cu_count : 256)) { return finish(vpq::launch_qmm_big(hs, g, bn)); }
+  }
+  return finish(vpq::launch_qmm_tile(hs, g));
+}
+
+}  // namespace
+
+int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                      const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M, int activation)
+{
+  return qmm_f16_common(stream, w, scales, biases, x, y, K, N, M, activation, nullptr, nullptr, 0, 0.0f, nullptr);
 }
 
 int vpq_lora_a_f16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t, int M, int K, int r,
@@ -630,35 +662,13 @@ int vpq_lora_a_f16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_
   return finish(vpq::launch_lora_a(reinterpret_cast<hipStream_t>(stream), x, lora_a, t, M, K, r, alpha, true));
 }
 
-// The fused GEMM on binary16 elements with a runtime adapter: the pre-pass t = f16(alpha * f16(x . A^T)), then the
-// large-tile kernel with r more values of K from t and B in the same accumulators.  alpha == 0 or lora_a == NULL: no
-// adapter.
+// The same with a runtime adapter: the pre-pass t = f16(alpha * f16(x . A^T)), then r more values of K from t and B
+// in the GEMM's accumulators.  alpha == 0 or lora_a == NULL: no adapter.
 int vpq_qmm_lora_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                            const uint16_t* x, uint16_t* y, int K, int N, int M, const uint16_t* lora_a,
                            const uint16_t* lora_b, int r, float alpha, uint16_t* lora_t_ws)
 {
-  const bool lora = lora_a != nullptr && alpha != 0.0f;
-  if (!lora) { return vpq_qmm_w4g64_f16(stream, w, scales, biases, x, y, K, N, M, 0); }
-  int st = check_pack(w, scales, biases, K, N);
-  if (st != VPQ_OK) { return st; }
-  if (x == nullptr || y == nullptr || lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
-  if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
-  if (M <= 0 || r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
-  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) {
-    return VPQ_ERR_MISALIGNED;
-  }
-  st = ensure_init();
-  if (st != VPQ_OK) { return st; }
-  vpq::GemmArgs g{};
-  g.w = w; g.scales = scales; g.biases = biases; g.x = x; g.y = y;
-  g.K = K; g.N = N; g.M = M;
-  g.lora_t = lora_t_ws; g.lora_b = lora_b; g.r = r;
-  g.cu_count = g_dev.cu_count;
-  g.f16 = true;
-  if (!vpq::qmm_big_supports(g)) { return VPQ_ERR_BAD_SHAPE; }
-  st = vpq_lora_a_f16(stream, x, lora_a, lora_t_ws, M, K, r, alpha);
-  if (st != VPQ_OK) { return st; }
-  return finish(vpq::launch_qmm_big(reinterpret_cast<hipStream_t>(stream), g, 0));
+  return qmm_f16_common(stream, w, scales, biases, x, y, K, N, M, 0, lora_a, lora_b, r, alpha, lora_t_ws);
 }
 
 int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

@@ -87,7 +87,8 @@ __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >>
 template <int I>
 __device__ __forceinline__ float ubyte_f32(uint32_t v) { return (float)((v >> (8 * I)) & 0xffu); }
 
-// 8 nibbles of one word -> 8 bf16 of fma(s, q, b), as one 16-byte LDS chunk.
+// 8 nibbles of one word -> 8 bf16 (F16: IEEE binary16) of fma(s, q, b), as one 16-byte LDS chunk.
+template <bool F16 = false>
 __device__ __forceinline__ uint4 dequant_word(uint32_t word, float s, float b)
 {
   uint32_t lo = word & 0x0f0f0f0fu;                // q0 q2 q4 q6
@@ -104,10 +105,10 @@ __device__ __forceinline__ uint4 dequant_word(uint32_t word, float s, float b)
   const float v6 = fmaf(s, ubyte_f32<3>(lo), b);
   const float v7 = fmaf(s, ubyte_f32<3>(hi), b);
   uint4 o;
-  o.x = pack_bf16x2(v0, v1);
-  o.y = pack_bf16x2(v2, v3);
-  o.z = pack_bf16x2(v4, v5);
-  o.w = pack_bf16x2(v6, v7);
+  o.x = pack_elt2<F16>(v0, v1);
+  o.y = pack_elt2<F16>(v2, v3);
+  o.z = pack_elt2<F16>(v4, v5);
+  o.w = pack_elt2<F16>(v6, v7);
   return o;
 }
 
@@ -222,10 +223,13 @@ __device__ __forceinline__ uint4 dequant_bytes(uint32_t w0, uint32_t w1, float s
 // brought in by the CONSUMER wavefronts, whose load counter nothing else uses: a 2-byte load per row, array
 // and step costs a 32-byte sector each, twice the bytes of the codes.  Needs K % 512 == 0, 16-byte
 // aligned scales and biases and no split of K.
+// F16: x, scales, biases, the adapter's factors and y are IEEE binary16 (the reference's VPIPE_ELT = half build): the
+// weight tile is f16_rne(fp32(s*q+b)), the MFMA v_mfma_f32_32x32x16_f16; everything else is the same byte traffic.
 template <bool LORA, int TMK = TM, int TNK = TN, bool GROUPED = false, int P = kProducers, bool SBR = false, int BITS = 4,
-          int GROUP = 64>
+          int GROUP = 64, bool F16 = false>
 __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const TileParams p)
 {
+  static_assert(!F16 || (BITS == 4 && GROUP == 64 && !GROUPED && !SBR), "binary16 elements: the plain 4-bit group-64 tile");
   static_assert((TMK == 256 && TNK == 128 && P == 4) || (TMK == 128 && !LORA && (TNK == 128 || TNK == 256)), "tiles built");
   static_assert(TMK % (8 * P) == 0 && TNK % (32 * P) == 0, "whole loads per producer");
   constexpr int kWStage = TNK * kRowB;             // 16 KB at 128 weight rows
@@ -328,12 +332,12 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
     auto dequant_to = [&](int stage, const CodeRegs (&r)[kWH]) {
 #pragma unroll
       for (int h = 0; h < kWH; ++h) {
-        const float sc = bf16_bits_to_f32(r[h].s_bits), bi = bf16_bits_to_f32(r[h].b_bits);
+        const float sc = elt_bits_to_f32<F16>(r[h].s_bits), bi = elt_bits_to_f32<F16>(r[h].b_bits);
         uint8_t* nb = w_lds + stage * kWStage + h * (32 * P * kRowB);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           if constexpr (BITS == 4) {
-            *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word(r[h].codes[i], sc, bi);
+            *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_word<F16>(r[h].codes[i], sc, bi);
           } else {
             const u32x4& cw = i < 2 ? r[h].codes : r[h].codes2;
             *reinterpret_cast<uint4*>(nb + b_dst[i]) = dequant_bytes(cw[2 * (i & 1)], cw[2 * (i & 1) + 1], sc, bi);
@@ -526,7 +530,13 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
 #pragma unroll
           for (int it = 0; it < kIT; ++it) {
             if (!GROUPED || frag_live[it]) {
-              acc[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[jt], xf[it], acc[jt][it], 0, 0, 0);
+              if constexpr (F16) {
+                typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+                acc[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, wf[jt]),
+                                                                     __builtin_bit_cast(halfx8, xf[it]), acc[jt][it], 0, 0, 0);
+              } else {
+                acc[jt][it] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[jt], xf[it], acc[jt][it], 0, 0, 0);
+              }
             }
           }
         }
@@ -642,10 +652,10 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
           const float f0 = pad_slot ? 0.0f : gated_f32(p.gate_act, acc[jt][it][rq * 4 + 0], acc[jt][it][rq * 4 + 1]);
           const float f1 = pad_slot ? 0.0f : gated_f32(p.gate_act, acc[jt][it][rq * 4 + 2], acc[jt][it][rq * 4 + 3]);
           if (pair_ok && n + 3 < p.N) {
-            *reinterpret_cast<uint32_t*>(yrow + (n >> 1)) = pack_bf16x2(f0, f1);
+            *reinterpret_cast<uint32_t*>(yrow + (n >> 1)) = pack_elt2<F16>(f0, f1);
           } else {
-            yrow[n >> 1] = (uint16_t)f32_to_bf16_bits(f0);
-            if (n + 3 < p.N) { yrow[(n >> 1) + 1] = (uint16_t)f32_to_bf16_bits(f1); }
+            yrow[n >> 1] = (uint16_t)f32_to_elt_bits<F16>(f0);
+            if (n + 3 < p.N) { yrow[(n >> 1) + 1] = (uint16_t)f32_to_elt_bits<F16>(f1); }
           }
         }
       }
@@ -675,14 +685,14 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
         const float v2 = acc[jt][it][rq * 4 + 2], v3 = acc[jt][it][rq * 4 + 3];
         if (vec_ok && n + 3 < p.N) {
           uint2 o;
-          o.x = pack_bf16x2(v0, v1);
-          o.y = pack_bf16x2(v2, v3);
+          o.x = pack_elt2<F16>(v0, v1);
+          o.y = pack_elt2<F16>(v2, v3);
           *reinterpret_cast<uint2*>(yrow + n) = o;
         } else {
           const float v[4] = {v0, v1, v2, v3};
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if (n + e < p.N) { yrow[n + e] = (uint16_t)f32_to_bf16_bits(v[e]); }
+            if (n + e < p.N) { yrow[n + e] = (uint16_t)f32_to_elt_bits<F16>(v[e]); }
           }
         }
       }
@@ -777,12 +787,17 @@ hipError_t launch_qmm_tile(hipStream_t st, const GemmArgs& a)
   p.ksplit = 1; p.steps_per_split = a.K / TK; p.plane = nullptr;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n)), block(kThreads);
   if (a.bits == 8) {
-    if (a.lora_t != nullptr || a.group != 64) { return hipErrorInvalidValue; }     // no 8-bit form with the adapter
+    if (a.lora_t != nullptr || a.group != 64 || a.f16) { return hipErrorInvalidValue; }     // no 8-bit form with the adapter
     return launch_kernel(qmm_tile_kernel<false, TM, TN, false, kProducers, false, 8>, grid, block, 0, st, p);
   }
   if (a.group == 32) {
-    if (a.lora_t != nullptr) { return hipErrorInvalidValue; }
+    if (a.lora_t != nullptr || a.f16) { return hipErrorInvalidValue; }
     return launch_kernel(qmm_tile_kernel<false, TM, TN, false, kProducers, false, 4, 32>, grid, block, 0, st, p);
+  }
+  if (a.f16) {
+    return a.lora_t != nullptr
+               ? launch_kernel(qmm_tile_kernel<true, TM, TN, false, kProducers, false, 4, 64, true>, grid, block, 0, st, p)
+               : launch_kernel(qmm_tile_kernel<false, TM, TN, false, kProducers, false, 4, 64, true>, grid, block, 0, st, p);
   }
   return a.lora_t != nullptr ? launch_kernel(qmm_tile_kernel<true>, grid, block, 0, st, p)
                              : launch_kernel(qmm_tile_kernel<false>, grid, block, 0, st, p);
