@@ -325,6 +325,12 @@ enum { VPQ_GATE_SWIGLU = 1, VPQ_GATE_GEGLU = 2 };
 int vpq_qmv_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                              const uint16_t* biases, const uint16_t* x, uint16_t* y,
                              int K, int N, int M, int variant, int activation);
+/* `affine_qmv_gelu_mul_w4g64` (affine_qmv.metal:751-768, the store :268-279): the per-layer-input gate GEMV,
+ * y[n] = bf16(gelu_tanh(v) * mul[n]) with v the GEMV's result already rounded to bf16 (so the output equals the
+ * unfused GEMV + activation that reads y back); one row of x, mul bf16 [N].  Requirements of vpq_qmv_w4g64_bf16. */
+int vpq_qmv_gelu_mul_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                const uint16_t* mul);
 int vpq_qmv_gated_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                const uint16_t* biases, const uint16_t* x, float* y,
                                int K, int N, int M, int variant, int activation);
@@ -599,6 +605,10 @@ int vpq_qmm_tiled_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
  * 64 rows, vpq_qmm_w8g64_bf16 above. */
 int vpq_linear_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M);
+/* `affine_moe_gate_w8g64` (affine_qmv.metal:1323-1349): the shared-expert gate, gate[m] = bf16(sigmoid(W[1,K] . x[m]))
+ * for M rows of x (1 <= M <= 65535) over a one-row 8-bit pack (w uint32 [K/4], scales / biases bf16 [K/64]). */
+int vpq_moe_gate_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                            const uint16_t* biases, const uint16_t* x, uint16_t* gate, int K, int M);
 int vpq_qmm_gated_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                              const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                              int out_stride, int out_off, int activation);

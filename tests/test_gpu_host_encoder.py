@@ -949,3 +949,36 @@ def test_load_and_run_eight_bit_and_group32_packs(vpq, enc, dev, D, tmp_path, M)
     assert L.hd_load_and_run(enc.h, r, b"b", 0, xd.data_ptr(), yd.data_ptr(), M, kn) == 0
     assert b"pass K" in L.hr_why()
     L.hr_close(r)
+
+
+def test_gelu_mul_and_shared_expert_gate_function_names(vpq, enc, dev, D):
+    # affine_qmv_gelu_mul_w4g64 (slots 0..6 as the GEMV, 7 = the multiplier) and affine_moe_gate_w8g64 (0:w 1:scales
+    # 2:biases 3:x 4:gate 5:K, rows of x = grid.y): the encoder's results are the C ABI's, bit for bit
+    K, N, M = 2048, 96, 5
+    w, s, b = synth.make_weight(N, K, 4100)
+    x1 = synth.make_act(1, K, 4101)
+    mul = synth.make_act(1, N, 4102)
+    pd = (D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), D.bf16(x1, dev))
+    muld = D.bf16(mul, dev)
+    y = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_gelu_mul_w4g64") == 1
+    for i, t in enumerate(pd + (y,)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.set_buffer(7, muld)
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    w8, s8, b8 = synth.make_weight8(1, K, 4103)
+    xm = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(synth.make_act(M, K, 4104)) * np.float32(0.05))
+    gd = (D.u32(w8, dev), D.bf16(s8, dev), D.bf16(b8, dev), D.bf16(xm, dev))
+    gate = torch.zeros((M,), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_qmv_bf16", "affine_moe_gate_w8g64") == 1
+    for i, t in enumerate(gd + (gate,)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.dispatch((32, M, 1), (32, 1, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert torch.equal(y, vpq.qmv_gelu_mul_w4g64(*pd, K, N, muld))
+    assert torch.equal(gate, vpq.moe_gate_w8g64(*gd, K, M))
+    assert y.abs().sum() > 0 and gate.float().std() > 0

@@ -303,3 +303,36 @@ def test_qmm_gated_store_of_the_large_tile_kernel(vpq, oracle, dev, D, M, F, K, 
     o64, ob = (oracle.swiglu if activation == capi.VPQ_GATE_SWIGLU else oracle.geglu)(y64)
     got = D.bits(got_all[torch.from_numpy(rows).to(dev)][:, torch.from_numpy(off + feats).to(dev)])
     parity.check_bf16(got, o64, ob, mismatch_over_all=activation == capi.VPQ_GATE_SWIGLU)
+
+
+@pytest.mark.parametrize("K,N", [(4096, 300), (2048, 64), (12288, 512), (192, 10), (1024, 33)])
+def test_qmv_gelu_mul(vpq, oracle, dev, D, K, N):
+    """affine_qmv_gelu_mul_w4g64 (gpu-kernels/metal/quant/affine_qmv.metal:751-768, store :268-279): the GEMV's
+    bf16-rounded result goes through gelu_tanh and is multiplied by mul[n].  The store is checked on the device's own
+    GEMV output (whose parity other tests hold), so what is compared is the fused store against the oracle's
+    gelu_tanh(v) * mul; and the whole against the oracle's GEMV by rel-L2."""
+    w, s, b = synth.make_weight(N, K, 3100 + K + N)
+    x = synth.make_act(1, K, 3200 + K)
+    mul = synth.make_act(1, N, 3300 + N)
+    wd, sd, bd, xd = stage(D, dev, (w, s, b), x)
+    v_bits = D.bits(vpq.qmv_w4g64(wd, sd, bd, xd, K, N, 1))
+    pairs = np.stack([synth.bf16_bits_to_f32(v_bits[0]).astype(np.float64),
+                      synth.bf16_bits_to_f32(mul[0]).astype(np.float64)], axis=1).reshape(1, 2 * N)
+    o64, ob = oracle.geglu(pairs)
+    out = parity.Guarded((1, N), torch.bfloat16, dev)
+    vpq.qmv_gelu_mul_w4g64(wd, sd, bd, xd, K, N, D.bf16(mul, dev), out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    got = D.bits(out.view)
+    # (1 + tanh cancels in fp32 for strongly negative v, as in the reference: the tolerance of the GEGLU stores)
+    parity.check_bf16(got, o64, ob, mismatch_over_all=False)
+    # end to end against the oracle's GEMV (a 1-ulp difference in v moves the output by about as much)
+    _, yb = oracle.qmv(w, s, b, x, K, N, 1)
+    p2 = np.stack([synth.bf16_bits_to_f32(yb[0]).astype(np.float64),
+                   synth.bf16_bits_to_f32(mul[0]).astype(np.float64)], axis=1).reshape(1, 2 * N)
+    e64, _ = oracle.geglu(p2)
+    assert parity.rel_l2(synth.bf16_bits_to_f32(got).astype(np.float64), e64) <= 4e-3
+    L = vpq.load()
+    p = out.view.data_ptr()
+    assert L.vpq_qmv_gelu_mul_w4g64_bf16(None, p, p, p, p, p, K, N, None) == -1
+    assert L.vpq_qmv_gelu_mul_w4g64_bf16(None, p, p, p, p, p, K + 8, N, p) == -2

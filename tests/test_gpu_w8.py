@@ -400,3 +400,27 @@ def test_linear_entrances_of_the_format_twins(vpq, dev, D, M):
     got = vpq.linear_twin("w4g32", *g2, x2, K2, N, M)
     want = torch.cat([vpq.qmv_w4g32(*g2, x2[m0:m0 + 16].contiguous(), K2, N, min(16, M - m0)) for m0 in range(0, M, 16)])
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("K,M", [(64, 1), (2048, 1), (2048, 37), (4096, 300)])
+def test_moe_shared_expert_gate_w8(vpq, oracle, dev, D, K, M):
+    """affine_moe_gate_w8g64 (gpu-kernels/metal/quant/affine_qmv.metal:1323-1349): gate[m] = sigmoid(W[1,K] . x[m]) over
+    a one-row 8-bit pack, against the 8-bit GEMV oracle's float64 logits through numpy's logistic."""
+    w, s, b = synth.make_weight8(1, K, 5000 + K)
+    # logits of order 1: shrink the activations, otherwise every gate saturates
+    x = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(synth.make_act(M, K, 5100 + K + M)) * np.float32(2.0 / np.sqrt(K)))
+    y64, _ = oracle.matmul8(w, s, b, x, K, 1, M, rounded=False)
+    want = 1.0 / (1.0 + np.exp(-y64[:, 0]))
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    out = parity.Guarded((M,), torch.bfloat16, dev)
+    vpq.moe_gate_w8g64(wd, sd, bd, xd, K, M, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    got = synth.bf16_bits_to_f32(D.bits(out.view)).astype(np.float64)
+    assert 0.05 < want.min() or M == 1 or want.std() > 0.01        # the case is not degenerate
+    assert np.abs(got - want).max() <= 2e-3 * np.abs(want).max() + 2.0 ** -9
+    L = vpq.load()
+    p = out.view.data_ptr()
+    assert L.vpq_moe_gate_w8g64_bf16(None, p, p, p, p, None, K, M) == -1
+    assert L.vpq_moe_gate_w8g64_bf16(None, p, p, p, p, p, K, 0) == -2
+    assert L.vpq_moe_gate_w8g64_bf16(None, p, p, p, p, p, K + 4, M) == -2

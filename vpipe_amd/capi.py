@@ -83,6 +83,8 @@ SYMBOLS = [
     ("vpq_qmm_dense_route_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_qmm_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_lora_a_f16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f]),
+    ("vpq_qmv_gelu_mul_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    ("vpq_moe_gate_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmm_lora_w4g64_f16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _f, _vp]),
     ("vpq_qmm_tiled_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     ("vpq_qmm_tiled_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
@@ -668,6 +670,26 @@ def qmm_w4g64_f16(w, scales, biases, x, K, N, M, activation=0, out=None):
         out = torch.empty((M, N // 2 if activation else N), dtype=torch.float16, device=w.device)
     _check(load().vpq_qmm_w4g64_f16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
                                     activation), "vpq_qmm_w4g64_f16")
+    return out
+
+
+def qmv_gelu_mul_w4g64(w, scales, biases, x, K, N, mul, out=None):
+    """y[n] = bf16(gelu_tanh(bf16(W x)[n]) * mul[n]) for one row of x."""
+    import torch
+    if out is None:
+        out = torch.empty((1, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmv_gelu_mul_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                              _ptr(mul)), "vpq_qmv_gelu_mul_w4g64_bf16")
+    return out
+
+
+def moe_gate_w8g64(w, scales, biases, x, K, M, out=None):
+    """gate[m] = bf16(sigmoid(W[1,K] . x[m])) over a one-row 8-bit pack."""
+    import torch
+    if out is None:
+        out = torch.empty((M,), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_moe_gate_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, M),
+           "vpq_moe_gate_w8g64_bf16")
     return out
 
 

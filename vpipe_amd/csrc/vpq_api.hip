@@ -90,8 +90,10 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (st != VPQ_OK) { return st; }
   if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
   if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
-  if (gate_act != 0 && gate_act != VPQ_GATE_SWIGLU && gate_act != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
-  if (gate_act != 0 && ((N & 1) != 0 || residual != nullptr || variant == VPQ_QMV_STREAM)) { return VPQ_ERR_BAD_SHAPE; }
+  const bool gelu_mul = gate_act == vpq::kStoreGeluMul;       // `residual` is the multiplier [N]; bf16 store only
+  if (gate_act != 0 && gate_act != VPQ_GATE_SWIGLU && gate_act != VPQ_GATE_GEGLU && !gelu_mul) { return VPQ_ERR_BAD_SHAPE; }
+  if (gelu_mul && (residual == nullptr || y_f32 || variant != VPQ_QMV_AUTO)) { return residual == nullptr ? VPQ_ERR_NULL_POINTER : VPQ_ERR_BAD_SHAPE; }
+  if (gate_act != 0 && !gelu_mul && ((N & 1) != 0 || residual != nullptr || variant == VPQ_QMV_STREAM)) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2)) { return VPQ_ERR_MISALIGNED; }
   if (residual != nullptr && !aligned(residual, 2)) { return VPQ_ERR_MISALIGNED; }
   if (variant < VPQ_QMV_AUTO || variant > VPQ_QMV_RING_SPLITK || variant == 3) { return VPQ_ERR_BAD_SHAPE; }   // (3 is unassigned)
@@ -107,6 +109,9 @@ int qmv_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
 
   const bool mfma_ok = vpq::qmv_mfma_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
   const bool flow_ok = vpq::qmv_flow_supports(K, N, M) && aligned(scales, 16) && aligned(biases, 16);
+  if (gelu_mul) {        // the two kernels that have this store: the streaming one and the general one
+    return finish(flow_ok ? vpq::launch_qmv_flow(hs, a) : vpq::launch_qmv_simple(hs, a));
+  }
   if (variant == VPQ_QMV_SIMPLE) { return finish(vpq::launch_qmv_simple(hs, a)); }
   if (variant == VPQ_QMV_FLOW) {
     if (!flow_ok) { return VPQ_ERR_BAD_SHAPE; }
@@ -252,6 +257,23 @@ int vpq_qmv_w8g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t*
                          const uint16_t* x, float* y, int K, int N, int M)
 {
   return qmv8_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr);
+}
+
+int vpq_moe_gate_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            const uint16_t* x, uint16_t* gate, int K, int M)
+{
+  int st = check_pack(w, scales, biases, K, 1);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || gate == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M < 1 || M > 65535) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(gate, 2)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = gate;
+  a.K = K; a.N = 1; a.M = 1; a.y_f32 = false; a.cu_count = g_dev.cu_count;
+  a.gate_act = vpq::kStoreSigmoid;
+  return finish(vpq::launch_qmv_rows8(reinterpret_cast<hipStream_t>(stream), a, M, nullptr, 1, 1));
 }
 
 static int rows8_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
@@ -760,6 +782,13 @@ int vpq_qmv_gated_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
 {
   if (activation != VPQ_GATE_SWIGLU && activation != VPQ_GATE_GEGLU) { return VPQ_ERR_BAD_SHAPE; }
   return qmv_common(stream, w, scales, biases, x, y, false, K, N, M, nullptr, nullptr, 0, variant, activation);
+}
+
+int vpq_qmv_gelu_mul_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                const uint16_t* mul)
+{
+  return qmv_common(stream, w, scales, biases, x, y, false, K, N, 1, mul, nullptr, 0, VPQ_QMV_AUTO, vpq::kStoreGeluMul);
 }
 
 int vpq_qmv_gated_w4g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

@@ -105,6 +105,13 @@ __device__ __forceinline__ uint32_t pack_elt2(float a, float b)
 //   kGateGeglu   gelu_tanh(gate) * up = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * up
 //                (affine_qmv.metal:1423-1429, affine_qmm_steel.metal:1541-1544)
 constexpr int kGateNone = 0, kGateSwiglu = 1, kGateGeglu = 2;
+// The store of kStoreGeluMul: gelu_tanh(v) * mul on the GEMV's result already rounded to the element type
+// (gpu-kernels/metal/quant/affine_qmv.metal:268-279).
+__device__ __forceinline__ float gelu_mul_f32(float v, float mul)
+{
+  const float t = tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v));
+  return 0.5f * v * (1.0f + t) * mul;
+}
 __device__ __forceinline__ float gated_f32(int act, float gate, float up)
 {
   if (act == kGateGeglu) {

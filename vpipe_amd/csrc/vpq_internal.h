@@ -82,6 +82,14 @@ inline hipError_t launch_preloaded(F kernel, dim3 grid, dim3 block, size_t lds_b
 hipError_t launch_profile_empty(hipStream_t st, uint32_t* sink);
 hipError_t launch_profile_read(hipStream_t st, const void* src, size_t bytes, uint32_t* sink);
 
+// QmvArgs::gate_act beyond the pair activations (1 SwiGLU, 2 GEGLU): y[n] = elt(gelu_tanh(elt(sum[n])) * mul[n]),
+// the fused per-layer-input gate `affine_qmv_gelu_mul_w4g64` (gpu-kernels/metal/quant/affine_qmv.metal:751-768); the
+// multiplier [N] travels in `residual`.  One row of x, element-typed store only.
+constexpr int kStoreGeluMul = 3;
+// qmv_rows8_kernel, ungated: y = elt(sigmoid(sum)), the shared-expert gate `affine_moe_gate_w8g64`
+// (gpu-kernels/metal/quant/affine_qmv.metal:1323-1349).
+constexpr int kStoreSigmoid = 4;
+
 struct QmvArgs {
   const uint32_t* w;
   const uint16_t* scales;

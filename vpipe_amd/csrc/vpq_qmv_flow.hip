@@ -396,7 +396,7 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
   }
   if (lane != 63) { return; }
 
-  if (gate_act) {
+  if (gate_act == kGateSwiglu || gate_act == kGateGeglu) {
     // rows 2g and 2g+1 are the gate and the up row of feature g; RB is even, so a pair is one wavefront's
 #pragma unroll
     for (int r = 0; r < RB; r += 2) {
@@ -421,7 +421,11 @@ __device__ __forceinline__ void qmv_flow_body(const FlowParams<C>& p)
         reinterpret_cast<float*>(yq)[n] = tot[r];
       } else {
         uint32_t v = f32_to_elt_bits<F16>(tot[r]);
-        if (residual != nullptr) { v = f32_to_elt_bits<F16>(elt_bits_to_f32<F16>(v) + elt_bits_to_f32<F16>(residual[n])); }
+        if (gate_act == kStoreGeluMul) {
+          v = f32_to_elt_bits<F16>(gelu_mul_f32(elt_bits_to_f32<F16>(v), elt_bits_to_f32<F16>(residual[n])));
+        } else if (residual != nullptr) {
+          v = f32_to_elt_bits<F16>(elt_bits_to_f32<F16>(v) + elt_bits_to_f32<F16>(residual[n]));
+        }
         reinterpret_cast<uint16_t*>(yq)[n] = (uint16_t)v;
       }
     }

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
         }
       }
     }
-    if (gate_act) {
+    if (gate_act == kGateSwiglu || gate_act == kGateGeglu) {
       float total[MT];
 #pragma unroll
       for (int mm = 0; mm < MT; ++mm) { total[mm] = wave_sum(acc[mm]); }
@@ -98,7 +98,9 @@ __global__ __launch_bounds__(256) void qmv_simple_kernel(
           reinterpret_cast<float*>(y)[o] = total;
         } else {
           uint32_t v = f32_to_elt_bits<F16>(total);
-          if (residual != nullptr) {
+          if (gate_act == kStoreGeluMul) {          // `residual` is the multiplier, one value per output feature
+            v = f32_to_elt_bits<F16>(gelu_mul_f32(elt_bits_to_f32<F16>(v), elt_bits_to_f32<F16>(residual[n])));
+          } else if (residual != nullptr) {
             v = f32_to_elt_bits<F16>(elt_bits_to_f32<F16>(v) + elt_bits_to_f32<F16>(residual[o]));
           }
           reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)v;
@@ -284,16 +286,22 @@ __global__ __launch_bounds__(256) void qmv_rows8_kernel(
 #pragma unroll
   for (int r = 0; r < R; ++r) { acc[r] = wave_sum(acc[r]); }
   if (lane == 0) {
-    const float v = GATED ? gated_f32(gate_act, acc[0], acc[R - 1]) : acc[0];
+    const float v = GATED ? gated_f32(gate_act, acc[0], acc[R - 1])
+                          : (gate_act == kStoreSigmoid ? 1.0f / (1.0f + __expf(-acc[0])) : acc[0]);
     y[(size_t)m * outs + o] = (uint16_t)f32_to_bf16_bits(v);
   }
 }
 
 hipError_t launch_qmv_rows8(hipStream_t st, const QmvArgs& a, int rows, const int* pair_eid, int x_div, int n_experts)
 {
-  const int outs = a.gate_act ? a.N / 2 : a.N;
+  const bool gated = a.gate_act == kGateSwiglu || a.gate_act == kGateGeglu;
+  const int outs = gated ? a.N / 2 : a.N;
   const dim3 grid((unsigned)((outs + 3) / 4), (unsigned)rows), block(256);
   uint16_t* y = static_cast<uint16_t*>(a.y);
+  if (a.gate_act == kStoreSigmoid) {
+    return launch_kernel(qmv_rows8_kernel<false>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, y, a.K, a.N, a.gate_act,
+                         pair_eid, x_div, n_experts);
+  }
   return a.gate_act ? launch_kernel(qmv_rows8_kernel<true>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, y, a.K, a.N,
                                     a.gate_act, pair_eid, x_div, n_experts)
                     : launch_kernel(qmv_rows8_kernel<false>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, y, a.K, a.N, 0,

@@ -89,6 +89,7 @@ const FnEntry kFunctions[] = {
     {"affine_qmm_mma_bf16", "affine_qmm_mma_w4g64", QuantKernel::Qmm},
     {"affine_qmv_bf16", "affine_qmv_swiglu_w4g64", QuantKernel::QmvSwiglu},
     {"affine_qmv_bf16", "affine_qmv_geglu_w4g64", QuantKernel::QmvGeglu},
+    {"affine_qmv_bf16", "affine_qmv_gelu_mul_w4g64", QuantKernel::QmvGeluMul},
     {"affine_qmm_steel_bf16", "affine_qmm_geglu_w4g64", QuantKernel::QmmGeglu},
     {"llm_elementwise_bf16", "dequant_embed_gather_f16", QuantKernel::EmbedGather},
     {"llm_elementwise_bf16", "argmax_f16", QuantKernel::Argmax},
@@ -114,6 +115,7 @@ const FnEntry kFunctions[] = {
     {"affine_dequant_bf16", "affine_dequant_w8g64", QuantKernel::Dequant, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64", QuantKernel::Qmv, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_moe_gate_w8g64", QuantKernel::MoeGate, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_grouped_swiglu_w8g64", QuantKernel::SortedSwiglu, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_grouped_down_w8g64", QuantKernel::SortedDown, QuantFormat::W8G64},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64", QuantKernel::Qmm, QuantFormat::W8G64},
@@ -421,7 +423,13 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
     const uint32_t* w = static_cast<const uint32_t*>(buf(0));
     const uint16_t* sc = static_cast<const uint16_t*>(buf(1));
     const uint16_t* bi = static_cast<const uint16_t*>(buf(2));
-    if (kind == QuantKernel::Dequant) {
+    if (kind == QuantKernel::MoeGate) {
+      // gpu-kernels/metal/quant/affine_qmv.metal:1327-1349: grid {32, M, 1}
+      status = (!w || !sc || !bi || !buf(3) || !buf(4) || !has_int(5))
+                   ? VPQ_ERR_NULL_POINTER
+                   : vpq_moe_gate_w8g64_bf16(st, w, sc, bi, static_cast<const uint16_t*>(buf(3)),
+                                             static_cast<uint16_t*>(buf(4)), ival(5), static_cast<int>(grid.y));
+    } else if (kind == QuantKernel::Dequant) {
       if (!w || !sc || !bi || !buf(3) || !has_int(4) || !has_int(5)) {
         status = VPQ_ERR_NULL_POINTER;
       } else if (fmt == QuantFormat::W4G64F16) {
@@ -732,6 +740,10 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
           status = vpq_qmm_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, ival(7), stride, off,
                                             kind == QuantKernel::QmmGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
         }
+      } else if (kind == QuantKernel::QmvGeluMul) {
+        // gpu-kernels/metal/quant/affine_qmv.metal:751-768: slot 7 = the multiplier
+        const uint16_t* mul = static_cast<const uint16_t*>(buf(7));
+        status = mul == nullptr ? VPQ_ERR_NULL_POINTER : vpq_qmv_gelu_mul_w4g64_bf16(st, w, sc, bi, x, y, K, N, mul);
       } else if (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu) {
         // gpu-kernels/metal/quant/affine_qmv.metal:891-906: N = 2*ffn, rows from grid.x
         const int M = grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1;
