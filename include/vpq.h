@@ -701,6 +701,16 @@ int vpq_qmv_group_w4g64_f16(vpq_stream_t stream, int count, const uint32_t* cons
 int vpq_qmm_dense_route_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                   const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                   int K, int N, int M, uint16_t* w_deq, int expand);
+/* The grouped launch of the format twins (`affine_qmv_qkv_w4g32`, `affine_qmv_qkv_w8g64`, affine_qmv.metal:518-559):
+ * arguments as vpq_qmv_group_w4g64_bf16 (w uint32 [N_i, K/8] with scales / biases [N_i, K/32], resp. w uint32
+ * [N_i, K/4] with [N_i, K/64]); bit-identical to `count` calls of vpq_qmv_w4g32_bf16 / vpq_qmv_w8g64_bf16.  Group-32
+ * packs at M <= 2 run as one launch; the other cases are separate launches behind one call. */
+int vpq_qmv_group_w4g32_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,
+                             const uint16_t* const* scales, const uint16_t* const* biases,
+                             const uint16_t* x, uint16_t* const* y, int K, const int* N, int M, int scale_only);
+int vpq_qmv_group_w8g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,
+                             const uint16_t* const* scales, const uint16_t* const* biases,
+                             const uint16_t* x, uint16_t* const* y, int K, const int* N, int M);
 
 /* ---- a12: the packer ------------------------------------------------------
  * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:

@@ -181,3 +181,26 @@ def test_qmm_g32_gated_store(vpq, oracle, dev, D, activation):
     parity.check_bf16(D.bits(got), want64, wantb, mismatch_over_all=activation == capi.VPQ_GATE_SWIGLU)
     assert vpq.load().vpq_qmm_w4g32_bf16(None, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), xd.data_ptr(), got.data_ptr(),
                                          96, 8, 4) == -2            # K % 64
+
+
+@pytest.mark.parametrize("K,M,rows", [(4096, 1, (256, 64, 64)), (96, 2, (33, 7)), (2560, 5, (48, 16, 16)), (1024, 1, (40,))])
+def test_qmv_group_g32_is_the_separate_calls(vpq, dev, D, K, M, rows):
+    """affine_qmv_qkv_w4g32 (gpu-kernels/metal/quant/affine_qmv.metal:518-538): the row-concatenated q|k|v pack as one
+    call; every output has the bits of its own vpq_qmv_w4g32_bf16 call (whose parity test_qmv_g32 holds), guard bands
+    intact.  M <= 2 is one launch of the row-streaming kernel, more rows are separate launches."""
+    N = sum(rows)
+    w, s, b = synth.make_weight_g32(N, K, 6800 + K + N)
+    x = synth.make_act(M, K, 6900 + K + M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    packs, r0 = [], 0
+    for n in rows:
+        packs.append((wd[r0:r0 + n], sd[r0:r0 + n], bd[r0:r0 + n], n))
+        r0 += n
+    outs = [parity.Guarded((M, n), torch.bfloat16, dev) for n in rows]
+    vpq.qmv_group_w4g32(packs, xd, K, M, outs=[o.view for o in outs])
+    torch.cuda.synchronize()
+    for o, p in zip(outs, packs):
+        o.assert_intact()
+        assert torch.equal(o.view, vpq.qmv_w4g32(p[0], p[1], p[2], xd, K, p[3], M))
+    L = vpq.load()
+    assert L.vpq_qmv_group_w4g32_bf16(None, 5, None, None, None, None, None, K, None, M, 0) == -1

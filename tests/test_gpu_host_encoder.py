@@ -982,3 +982,28 @@ def test_gelu_mul_and_shared_expert_gate_function_names(vpq, enc, dev, D):
     assert torch.equal(y, vpq.qmv_gelu_mul_w4g64(*pd, K, N, muld))
     assert torch.equal(gate, vpq.moe_gate_w8g64(*gd, K, M))
     assert y.abs().sum() > 0 and gate.float().std() > 0
+
+
+@pytest.mark.parametrize("name", ["affine_qmv_qkv_w8g64", "affine_qmv_qkv_w4g32"])
+def test_fused_qkv_call_sites_of_the_format_twins(vpq, enc, dev, D, name):
+    # gpu-kernels/metal/quant/affine_qmv.metal:518-559: the slots of affine_qmv_qkv_w4g64 over the 8-bit and the
+    # group-32 pack; the three outputs are the C ABI's plain QMV over the whole pack, bit for bit
+    K, rows = 1024, (256, 64, 64)
+    N = sum(rows)
+    eight = name.endswith("w8g64")
+    w, s, b = synth.make_weight8(N, K, 60) if eight else synth.make_weight_g32(N, K, 61)
+    x = synth.make_act(1, K, 62)
+    wd, sd, bd, xd = D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), D.bf16(x, dev)
+    outs = [torch.zeros((1, r), dtype=torch.bfloat16, device=dev) for r in rows]
+    assert enc.set_function("affine_qmv_bf16", name) == 1
+    for i, t in enumerate((wd, sd, bd, xd, outs[0], outs[1], outs[2])):
+        enc.set_buffer(i, t)
+    enc.set_constant(7, K)
+    for i, r in enumerate(rows):
+        enc.set_constant(8 + i, r)
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    whole = vpq.qmv_w8g64(wd, sd, bd, xd, K, N, 1) if eight else vpq.qmv_w4g32(wd, sd, bd, xd, K, N, 1)
+    assert torch.equal(torch.cat(outs, dim=1), whole)
+    assert whole.abs().sum() > 0

@@ -424,3 +424,23 @@ def test_moe_shared_expert_gate_w8(vpq, oracle, dev, D, K, M):
     assert L.vpq_moe_gate_w8g64_bf16(None, p, p, p, p, None, K, M) == -1
     assert L.vpq_moe_gate_w8g64_bf16(None, p, p, p, p, p, K, 0) == -2
     assert L.vpq_moe_gate_w8g64_bf16(None, p, p, p, p, p, K + 4, M) == -2
+
+
+@pytest.mark.parametrize("K,M,rows", [(4096, 1, (256, 64, 64)), (192, 3, (33, 7)), (2048, 16, (48, 16, 16))])
+def test_qmv_group_w8_is_the_separate_calls(vpq, dev, D, K, M, rows):
+    """affine_qmv_qkv_w8g64 (gpu-kernels/metal/quant/affine_qmv.metal:540-559): the row-concatenated q|k|v pack behind
+    one call; every output has the bits of its own vpq_qmv_w8g64_bf16 call, guard bands intact."""
+    N = sum(rows)
+    w, s, b = synth.make_weight8(N, K, 5400 + K + N)
+    x = synth.make_act(M, K, 5500 + K + M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    packs, r0 = [], 0
+    for n in rows:
+        packs.append((wd[r0:r0 + n], sd[r0:r0 + n], bd[r0:r0 + n], n))
+        r0 += n
+    outs = [parity.Guarded((M, n), torch.bfloat16, dev) for n in rows]
+    vpq.qmv_group_w8g64(packs, xd, K, M, outs=[o.view for o in outs])
+    torch.cuda.synchronize()
+    for o, p in zip(outs, packs):
+        o.assert_intact()
+        assert torch.equal(o.view, vpq.qmv_w8g64(p[0], p[1], p[2], xd, K, p[3], M))

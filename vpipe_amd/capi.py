@@ -67,6 +67,8 @@ SYMBOLS = [
     ("vpq_linear_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz]),
     ("vpq_qmv_group_w4g64_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
     ("vpq_qmv_group_w4g64_f16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
+    ("vpq_qmv_group_w4g32_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i]),
+    ("vpq_qmv_group_w8g64_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
     ("vpq_interleave_rows", _i, [_vp, _vp, _vp, _vp, _sz, _sz]),
     ("vpq_qmv_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmv_swiglu_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
@@ -798,8 +800,9 @@ class QmvGroup:
     """The pointer tables of a grouped launch, built once for a fixed set of tensors so that a
     launch costs one foreign call (a decode loop launches the same groups every token)."""
 
-    def __init__(self, packs, x, K, M, outs, f16=False):
-        self.entry = "vpq_qmv_group_w4g64_f16" if f16 else "vpq_qmv_group_w4g64_bf16"
+    def __init__(self, packs, x, K, M, outs, f16=False, entry=None, extra=()):
+        self.entry = entry or ("vpq_qmv_group_w4g64_f16" if f16 else "vpq_qmv_group_w4g64_bf16")
+        self.extra = tuple(extra)
         n = len(packs)
         PA = ctypes.c_void_p * n
         self.keep = (packs, x, outs)       # the tables hold raw pointers: keep the tensors alive
@@ -814,7 +817,7 @@ class QmvGroup:
 
     def launch(self):
         _check(getattr(load(), self.entry)(_stream(), self.n, self.w, self.s, self.b, self.x, self.y, self.K,
-                                           self.N, self.M), self.entry)
+                                           self.N, self.M, *self.extra), self.entry)
         return self.outs
 
 
@@ -824,6 +827,22 @@ def qmv_group_w4g64(packs, x, K, M, outs=None):
     if outs is None:
         outs = [torch.empty((M, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
     return QmvGroup(packs, x, K, M, outs).launch()
+
+
+def qmv_group_w4g32(packs, x, K, M, outs=None, scale_only=False):
+    """The grouped launch over 4-bit group-32 packs (scales / biases [N, K/32])."""
+    import torch
+    if outs is None:
+        outs = [torch.empty((M, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
+    return QmvGroup(packs, x, K, M, outs, entry="vpq_qmv_group_w4g32_bf16", extra=(1 if scale_only else 0,)).launch()
+
+
+def qmv_group_w8g64(packs, x, K, M, outs=None):
+    """The grouped call over 8-bit group-64 packs (w uint32 [N, K/4])."""
+    import torch
+    if outs is None:
+        outs = [torch.empty((M, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
+    return QmvGroup(packs, x, K, M, outs, entry="vpq_qmv_group_w8g64_bf16").launch()
 
 
 def qmv_group_w4g64_f16(packs, x, K, M, outs=None):

@@ -1492,6 +1492,57 @@ int vpq_qmv_group_w4g64_bf16(vpq_stream_t stream, int count, const uint32_t* con
   return finish(vpq::launch_qmv_mfma_group(reinterpret_cast<hipStream_t>(stream), a, g));
 }
 
+// The fused-QKV GEMV of the format twins (`affine_qmv_qkv_w4g32`, `affine_qmv_qkv_w8g64`,
+// gpu-kernels/metal/quant/affine_qmv.metal:518-559): 1..4 packs that share x.  Group-32 packs at up to two rows of x
+// run as one launch of the row-streaming kernel; otherwise the packs are separate calls, with the same bits.
+int vpq_qmv_group_w4g32_bf16(vpq_stream_t stream, int count, const uint32_t* const* w, const uint16_t* const* scales,
+                             const uint16_t* const* biases, const uint16_t* x, uint16_t* const* y, int K, const int* N,
+                             int M, int scale_only)
+{
+  if (w == nullptr || scales == nullptr || y == nullptr || N == nullptr || (biases == nullptr && scale_only == 0)) {
+    return VPQ_ERR_NULL_POINTER;
+  }
+  if (count < 1 || count > 4) { return VPQ_ERR_BAD_SHAPE; }
+  if (x == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
+  for (int i = 0; i < count; ++i) {
+    const int st = check_pack_g32(w[i], scales[i], scale_only ? nullptr : biases[i], K, N[i], scale_only != 0);
+    if (st != VPQ_OK) { return st; }
+    if (y[i] == nullptr) { return VPQ_ERR_NULL_POINTER; }
+    if (!aligned(y[i], 2)) { return VPQ_ERR_MISALIGNED; }
+  }
+  if (!aligned(x, 16)) { return VPQ_ERR_MISALIGNED; }
+  if (M > 2) {
+    for (int i = 0; i < count; ++i) {
+      const int st = vpq_qmv_w4g32_bf16(stream, w[i], scales[i], scale_only ? nullptr : biases[i], x, y[i], K, N[i], M,
+                                        nullptr, scale_only);
+      if (st != VPQ_OK) { return st; }
+    }
+    return VPQ_OK;
+  }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.x = x; a.K = K; a.M = M; a.y_f32 = false; a.cu_count = g_dev.cu_count;
+  vpq::QmvGroup g;
+  g.count = count;
+  for (int i = 0; i < count; ++i) { g.seg[i] = vpq::QmvSeg{w[i], scales[i], scale_only ? nullptr : biases[i], y[i], N[i]}; }
+  return finish(vpq::launch_qmv_rows_group(reinterpret_cast<hipStream_t>(stream), a, g, 32, scale_only != 0));
+}
+
+int vpq_qmv_group_w8g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w, const uint16_t* const* scales,
+                             const uint16_t* const* biases, const uint16_t* x, uint16_t* const* y, int K, const int* N,
+                             int M)
+{
+  if (w == nullptr || scales == nullptr || biases == nullptr || y == nullptr || N == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (count < 1 || count > 4) { return VPQ_ERR_BAD_SHAPE; }
+  for (int i = 0; i < count; ++i) {
+    const int st = vpq_qmv_w8g64_bf16(stream, w[i], scales[i], biases[i], x, y[i], K, N[i], M, nullptr);
+    if (st != VPQ_OK) { return st; }
+  }
+  return VPQ_OK;
+}
+
 int vpq_qmv_group_w4g64_f16(vpq_stream_t stream, int count, const uint32_t* const* w,
                             const uint16_t* const* scales, const uint16_t* const* biases,
                             const uint16_t* x, uint16_t* const* y, int K, const int* N, int M)

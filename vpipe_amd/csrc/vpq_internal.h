@@ -191,7 +191,8 @@ size_t qmv_ring_workspace_bytes(int K, int N, int M);   // planes of the widest 
 // Row-streaming kernel (M <= 2, any K % 64): rows_per_wave in {2, 4}, 0 = default.
 bool qmv_rows_supports(int K, int N, int M);
 hipError_t launch_qmv_rows(hipStream_t st, const QmvArgs& a, int rows_per_wave);
-hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g);
+hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g, int group = 64,
+                                 bool scale_only = false);
 // Gathered (MoE) form, M = 1 per pair: a.w/scales/biases are batches [E, N, ...] of expert slabs,
 // pair p contracts slab pair_eid[p] with x row p / x_div into y row p (zeros for an id outside
 // [0, n_experts)); a.gate_act as in the plain form.

@@ -338,14 +338,14 @@ hipError_t launch_qmv_rows(hipStream_t st, const QmvArgs& a, int rows_per_wave)
   return launch_rows_segments(st, g, a, rows_per_wave, RowsGather{nullptr, 1, 0}, 1);
 }
 
-hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGroup& grp)
+hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGroup& grp, int group, bool scale_only)
 {
   RowsSegs g{};
   g.count = grp.count;
   for (int i = 0; i < grp.count; ++i) {
     g.seg[i] = RowsSeg{grp.seg[i].w, grp.seg[i].scales, grp.seg[i].biases, grp.seg[i].y, grp.seg[i].N, 0};
   }
-  return launch_rows_segments(st, g, a, 0, RowsGather{nullptr, 1, 0}, 1);
+  return launch_rows_segments(st, g, a, group == 32 ? 2 : 0, RowsGather{nullptr, 1, 0}, 1, group, scale_only);
 }
 
 hipError_t launch_qmv_rows_gather(hipStream_t st, const QmvArgs& a, const int* pair_eid, int pairs, int x_div,

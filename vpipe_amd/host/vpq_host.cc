@@ -116,6 +116,8 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_w8g64", QuantKernel::Qmv, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_moe_gate_w8g64", QuantKernel::MoeGate, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_qkv_w8g64", QuantKernel::QmvQkv, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_qkv_w4g32", QuantKernel::QmvQkv, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_grouped_swiglu_w8g64", QuantKernel::SortedSwiglu, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_grouped_down_w8g64", QuantKernel::SortedDown, QuantFormat::W8G64},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64", QuantKernel::Qmm, QuantFormat::W8G64},
@@ -632,17 +634,27 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
       const uint16_t* sc[3];
       const uint16_t* bi[3];
       uint16_t* y[3] = {static_cast<uint16_t*>(buf(4)), static_cast<uint16_t*>(buf(5)), static_cast<uint16_t*>(buf(6))};
+      // words of codes and groups per row of the format (:518-559: the 8-bit and the group-32 twins)
+      const size_t row_words = (size_t)(fmt == QuantFormat::W8G64 ? K / 4 : K / 8);
+      const size_t row_groups = (size_t)(fmt == QuantFormat::W4G32 ? K / 32 : K / 64);
       size_t r0 = 0;
       for (int i = 0; i < 3; ++i) {
-        w[i] = static_cast<const uint32_t*>(buf(0)) + r0 * (size_t)(K / 8);
-        sc[i] = static_cast<const uint16_t*>(buf(1)) + r0 * (size_t)(K / 64);
-        bi[i] = static_cast<const uint16_t*>(buf(2)) + r0 * (size_t)(K / 64);
+        w[i] = static_cast<const uint32_t*>(buf(0)) + r0 * row_words;
+        sc[i] = static_cast<const uint16_t*>(buf(1)) + r0 * row_groups;
+        bi[i] = static_cast<const uint16_t*>(buf(2)) + r0 * row_groups;
         r0 += (size_t)rows[i];
       }
-      status = fmt == QuantFormat::W4G64F16
-                   ? vpq_qmv_group_w4g64_f16(st, rows[2] > 0 ? 3 : 2, w, sc, bi, static_cast<const uint16_t*>(buf(3)), y, K, rows, 1)
-                   : vpq_qmv_group_w4g64_bf16(st, rows[2] > 0 ? 3 : 2, w, sc, bi, static_cast<const uint16_t*>(buf(3)), y, K, rows,
-                                              1);
+      const int count = rows[2] > 0 ? 3 : 2;
+      const uint16_t* x = static_cast<const uint16_t*>(buf(3));
+      if (fmt == QuantFormat::W4G64F16) {
+        status = vpq_qmv_group_w4g64_f16(st, count, w, sc, bi, x, y, K, rows, 1);
+      } else if (fmt == QuantFormat::W8G64) {
+        status = vpq_qmv_group_w8g64_bf16(st, count, w, sc, bi, x, y, K, rows, 1);
+      } else if (fmt == QuantFormat::W4G32) {
+        status = vpq_qmv_group_w4g32_bf16(st, count, w, sc, bi, x, y, K, rows, 1, 0);
+      } else {
+        status = vpq_qmv_group_w4g64_bf16(st, count, w, sc, bi, x, y, K, rows, 1);
+      }
     }
   } else {
     // slots 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N, 7: residual | m_total | M
