@@ -711,6 +711,19 @@ int vpq_qmv_group_w4g32_bf16(vpq_stream_t stream, int count, const uint32_t* con
 int vpq_qmv_group_w8g64_bf16(vpq_stream_t stream, int count, const uint32_t* const* w,
                              const uint16_t* const* scales, const uint16_t* const* biases,
                              const uint16_t* x, uint16_t* const* y, int K, const int* N, int M);
+/* `affine_qmv_qkv_rms_w4g64` / `_w4g32` / `_w8g64` (affine_qmv.metal:561-740): RMSNorm of the input row and the
+ * fused-QKV GEMV over it.  vpq_rmsnorm_bf16 is the norm alone, out[m,k] = bf16(float(x[m,k]) * inv_m * float(norm_w[k])),
+ * inv_m = rsqrt(sum_k x[m,k]^2 / K + eps) in fp32 (:601-616; norm_w holds Gemma's 1 + w already), 1 <= M <= 65535.
+ * vpq_qmv_qkv_rms_bf16 runs it on the one row x [K] into `x_norm_ws` (K elements of caller scratch, 16-byte aligned:
+ * the reference keeps the normalized row in threadgroup memory) and then the grouped GEMV of `format` (VPQ_FORMAT_*)
+ * over that row: two launches, the values of the fused kernel. */
+enum { VPQ_FORMAT_W4G64 = 0, VPQ_FORMAT_W4G32 = 1, VPQ_FORMAT_W8G64 = 2 };
+int vpq_rmsnorm_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* norm_w, uint16_t* out,
+                     int K, int M, float eps);
+int vpq_qmv_qkv_rms_bf16(vpq_stream_t stream, int format, int count, const uint32_t* const* w,
+                         const uint16_t* const* scales, const uint16_t* const* biases, const uint16_t* x,
+                         const uint16_t* norm_w, uint16_t* const* y, int K, const int* N, float eps,
+                         uint16_t* x_norm_ws);
 
 /* ---- a12: the packer ------------------------------------------------------
  * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:

@@ -257,6 +257,14 @@ def matmul_f16(w, s, b, x, K, N, M, rounded, residual=None):
     return y64, yh
 
 
+def rmsnorm(x, norm_w, K, M, eps):
+    """bf16 bits x [M,K], norm_w [K] -> bf16 bits [M,K]: x * rsqrt(mean(x^2) + eps) * norm_w."""
+    x, norm_w = _c(x, np.uint16), _c(norm_w, np.uint16)
+    out = np.empty((M, K), dtype=np.uint16)
+    lib().vpo_rmsnorm_bf16(_p(x, _u16p), _p(norm_w, _u16p), _p(out, _u16p), K, M, ctypes.c_float(eps))
+    return out
+
+
 def lora_t_f16(x, A, M, K, r, alpha):
     """binary16 x [M,K], A [r,K] -> t [M,r] binary16 bits, two roundings."""
     x, A = _c(x, np.uint16), _c(A, np.uint16)

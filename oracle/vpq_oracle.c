@@ -811,6 +811,25 @@ void vpo_matmul_w4g64_f16(const uint32_t* w, const uint16_t* scales, const uint1
   free(wrow);
 }
 
+/* RMSNorm ahead of the fused-QKV GEMV, gpu-kernels/metal/quant/affine_qmv.metal:601-616: the sum of squares, the
+ * mean and the reciprocal root in double here (the kernel: fp32), then the reference's product order in fp32,
+ * T(float(x[k]) * inv * float(norm_w[k])), one rounding. */
+void vpo_rmsnorm_bf16(const uint16_t* x, const uint16_t* norm_w, uint16_t* out, int K, int M, float eps)
+{
+  for (size_t m = 0; m < (size_t)M; ++m) {
+    double sq = 0.0;
+    for (int k = 0; k < K; ++k) {
+      const double v = (double)vpo_bf16_to_f32(x[m * (size_t)K + k]);
+      sq += v * v;
+    }
+    const float inv = (float)(1.0 / sqrt(sq / (double)K + (double)eps));
+    for (int k = 0; k < K; ++k) {
+      const float v = vpo_bf16_to_f32(x[m * (size_t)K + k]) * inv;
+      out[m * (size_t)K + k] = vpo_f32_to_bf16(v * vpo_bf16_to_f32(norm_w[k]));
+    }
+  }
+}
+
 /* The adapter on binary16 elements: gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273 with VPIPE_ELT = half
  * (:28-33) -- t[M,r] = f16((float)f16(x . A^T) * alpha), two roundings, the contraction in double. */
 void vpo_lora_t_f16(const uint16_t* x, const uint16_t* A, uint16_t* t, int M, int K, int r, float alpha)

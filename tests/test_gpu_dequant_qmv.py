@@ -513,3 +513,58 @@ def test_qmv_grouped_row_concatenated_qkv(vpq, oracle, dev, D):
     y64, yb = oracle.qmv(w, s, b, x, K, N, M)
     got = np.concatenate([D.bits(o) for o in outs], axis=1)
     parity.check_bf16(got, y64, yb)
+
+
+@pytest.mark.parametrize("K,M", [(64, 1), (1536, 3), (4096, 1), (5120, 40)])
+def test_rmsnorm_rows(vpq, oracle, dev, D, K, M):
+    """vpq_rmsnorm_bf16 (gpu-kernels/metal/quant/affine_qmv.metal:601-616): against the oracle to one bf16 step (fp32
+    against float64 sums move a few elements across a rounding boundary), the same bits run to run, guard bands."""
+    x = synth.make_act(M, K, 7100 + K)
+    nw = synth.f32_to_bf16_bits((1.0 + 0.1 * np.random.default_rng(7200 + K).standard_normal(K)).astype(np.float32))
+    want = oracle.rmsnorm(x, nw, K, M, 1e-6)
+    out = parity.Guarded((M, K), torch.bfloat16, dev)
+    vpq.rmsnorm_bf16(D.bf16(x, dev), D.bf16(nw, dev), K, M, 1e-6, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    got = D.bits(out.view)
+    assert (got != want).mean() <= 0.02
+    assert parity.bf16_ulp_distance(got, want).max() <= 1
+    assert torch.equal(out.view, vpq.rmsnorm_bf16(D.bf16(x, dev), D.bf16(nw, dev), K, M, 1e-6))
+
+
+@pytest.mark.parametrize("fmt", [0, 1, 2])
+@pytest.mark.parametrize("K,rows", [(4096, (256, 64, 64)), (1536, (96, 32))])
+def test_qmv_qkv_rms(vpq, oracle, dev, D, fmt, K, rows):
+    """affine_qmv_qkv_rms_w4g64 / _w4g32 / _w8g64 (affine_qmv.metal:561-740): the normalized row lands in the scratch
+    with the bits of vpq_rmsnorm_bf16, the outputs have the bits of the format's grouped GEMV over that row, and the
+    whole agrees with the oracle's GEMV over the oracle's normalized row."""
+    N = sum(rows)
+    make = (synth.make_weight, synth.make_weight_g32, synth.make_weight8)[fmt]
+    w, s, b = make(N, K, 7300 + K + fmt)
+    x = synth.make_act(1, K, 7400 + K)
+    nw = synth.f32_to_bf16_bits((1.0 + 0.1 * np.random.default_rng(7500 + K).standard_normal(K)).astype(np.float32))
+    wd, sd, bd, xd, nwd = D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), D.bf16(x, dev), D.bf16(nw, dev)
+    packs, r0 = [], 0
+    for n in rows:
+        packs.append((wd[r0:r0 + n], sd[r0:r0 + n], bd[r0:r0 + n], n))
+        r0 += n
+    ws = parity.Guarded((1, K), torch.bfloat16, dev)
+    outs = [parity.Guarded((1, n), torch.bfloat16, dev) for n in rows]
+    vpq.qmv_qkv_rms(fmt, packs, xd, nwd, K, 1e-6, outs=[o.view for o in outs], x_norm_ws=ws.view)
+    torch.cuda.synchronize()
+    ws.assert_intact()
+    xn = vpq.rmsnorm_bf16(xd, nwd, K, 1, 1e-6)
+    assert torch.equal(ws.view, xn)
+    group = (vpq.qmv_group_w4g64, vpq.qmv_group_w4g32, vpq.qmv_group_w8g64)[fmt]
+    for o, ref in zip(outs, group(packs, xn, K, 1)):
+        o.assert_intact()
+        assert torch.equal(o.view, ref)
+    xo = oracle.rmsnorm(x, nw, K, 1, 1e-6)
+    y64 = (oracle.qmv(w, s, b, xo, K, N, 1)[0], oracle.qmv_g32(w, s, b, xo, K, N, 1)[0],
+           oracle.matmul8(w, s, b, xo, K, N, 1, rounded=False)[0])[fmt]
+    got = synth.bf16_bits_to_f32(np.concatenate([D.bits(o.view) for o in outs], axis=1)).astype(np.float64)
+    assert parity.rel_l2(got, y64) <= 4e-3
+    L = vpq.load()
+    p = ws.view.data_ptr()
+    assert L.vpq_qmv_qkv_rms_bf16(None, 3, 1, None, None, None, p, p, None, K, None, 1e-6, p) == -2
+    assert L.vpq_qmv_qkv_rms_bf16(None, 0, 1, None, None, None, p, p, None, K, None, 1e-6, None) == -4

@@ -1007,3 +1007,34 @@ def test_fused_qkv_call_sites_of_the_format_twins(vpq, enc, dev, D, name):
     whole = vpq.qmv_w8g64(wd, sd, bd, xd, K, N, 1) if eight else vpq.qmv_w4g32(wd, sd, bd, xd, K, N, 1)
     assert torch.equal(torch.cat(outs, dim=1), whole)
     assert whole.abs().sum() > 0
+
+
+@pytest.mark.parametrize("name,fmt", [("affine_qmv_qkv_rms_w4g64", 0), ("affine_qmv_qkv_rms_w4g32", 1),
+                                      ("affine_qmv_qkv_rms_w8g64", 2)])
+def test_rmsnorm_fused_qkv_call_sites(vpq, enc, dev, D, name, fmt):
+    # gpu-kernels/metal/quant/affine_qmv.metal:671-740: slots 0:w 1:scales 2:biases 3:x 4:norm_w 5:q 6:k 7:v 8:K
+    # 9..11 rows 12:eps; the outputs are the C ABI's composed call, bit for bit
+    K, rows, eps = 1024, (256, 64, 64), 1e-6
+    N = sum(rows)
+    w, s, b = (synth.make_weight, synth.make_weight_g32, synth.make_weight8)[fmt](N, K, 70 + fmt)
+    x = synth.make_act(1, K, 73)
+    nw = synth.f32_to_bf16_bits((1.0 + 0.1 * np.random.default_rng(74).standard_normal(K)).astype(np.float32))
+    wd, sd, bd, xd, nwd = D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), D.bf16(x, dev), D.bf16(nw, dev)
+    outs = [torch.zeros((1, r), dtype=torch.bfloat16, device=dev) for r in rows]
+    assert enc.set_function("affine_qmv_bf16", name) == 1
+    for i, t in enumerate((wd, sd, bd, xd, nwd, outs[0], outs[1], outs[2])):
+        enc.set_buffer(i, t)
+    enc.set_constant(8, K)
+    for i, r in enumerate(rows):
+        enc.set_constant(9 + i, r)
+    enc.set_constant_f32(12, eps)
+    enc.dispatch((32, N // 8, 1), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    packs, r0 = [], 0
+    for n in rows:
+        packs.append((wd[r0:r0 + n], sd[r0:r0 + n], bd[r0:r0 + n], n))
+        r0 += n
+    for o, ref in zip(outs, vpq.qmv_qkv_rms(fmt, packs, xd, nwd, K, eps)):
+        assert torch.equal(o, ref)
+    assert outs[0].abs().sum() > 0

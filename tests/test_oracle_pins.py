@@ -629,6 +629,36 @@ def test_f16_adapter_against_numpy_float16(oracle):
     assert np.array_equal(z64, b64) and np.array_equal(zh, bh)
 
 
+def test_rmsnorm_against_torch_and_closed_forms(oracle):
+    """The RMSNorm ahead of the fused-QKV GEMV: against torch.nn.functional.rms_norm in float64 (an independent
+    routine) to one bf16 step with almost every element equal; a row of ones gives norm_w / sqrt(1 + eps); a row of
+    +-c with eps = 0 gives +-norm_w exactly, whatever c (scale invariance); rows are independent."""
+    import torch
+    K, M, eps = 1536, 3, 1e-6
+    x = synth.make_act(M, K, 71)
+    nw = synth.f32_to_bf16_bits((1.0 + 0.1 * np.random.default_rng(72).standard_normal(K)).astype(np.float32))
+    got = oracle.rmsnorm(x, nw, K, M, eps)
+    xt = torch.from_numpy(synth.bf16_bits_to_f32(x).astype(np.float64))
+    wt = torch.from_numpy(synth.bf16_bits_to_f32(nw).astype(np.float64))
+    ref = torch.nn.functional.rms_norm(xt, (K,), weight=wt, eps=eps).numpy()
+    want = synth.f32_to_bf16_bits(ref.astype(np.float32))
+    assert (got != want).mean() < 0.01 and parity_ulp(got, want) <= 1
+    assert np.array_equal(oracle.rmsnorm(x[1:2], nw, K, 1, eps), got[1:2])
+    ones = synth.f32_to_bf16_bits(np.ones((1, K), dtype=np.float32))
+    w1 = synth.bf16_bits_to_f32(nw).astype(np.float64) / np.sqrt(1.0 + 0.25)
+    g1 = oracle.rmsnorm(ones, nw, K, 1, 0.25)
+    assert parity_ulp(g1[0], synth.f32_to_bf16_bits(w1.astype(np.float32))) <= 1
+    sign = np.where(np.arange(K) % 3 == 0, -1.0, 1.0).astype(np.float32)
+    for c in (0.5, 8.0, 96.0):
+        gc = oracle.rmsnorm(synth.f32_to_bf16_bits((c * sign)[None, :]), nw, K, 1, 0.0)
+        assert np.array_equal(gc[0], synth.f32_to_bf16_bits(sign * synth.bf16_bits_to_f32(nw)))
+
+
+def parity_ulp(a, b):
+    from tests import parity
+    return int(parity.bf16_ulp_distance(a, b).max())
+
+
 def test_grouped_gemm_oracle_with_byte_codes_reduces_to_the_plain_8bit_gemm(oracle):
     """The 8-bit form of the grouped restatement: every live slot equals the plain 8-bit GEMM oracle
     (bf16-rounded weights) of its row on its expert's slab."""

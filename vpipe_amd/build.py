@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libvpq.so")
 SOURCES = ["vpq_api.hip", "vpq_dequant.hip", "vpq_qmv_simple.hip", "vpq_qmv_mfma.hip", "vpq_qmv_stream.hip", "vpq_qmv_ring.hip", "vpq_qmv_rows.hip", "vpq_qmv_flow.hip", "vpq_profile.hip", "vpq_argmax.hip", "vpq_sample.hip", "vpq_moe_sort.hip",
-           "vpq_lora_a.hip", "vpq_qmm_tile.hip", "vpq_qmm_big.hip"]
+           "vpq_lora_a.hip", "vpq_qmm_tile.hip", "vpq_qmm_big.hip", "vpq_norm.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed fp32 VALU ops are switched off for every kernel (device pass only; the
 # host pass prints a harmless "not a recognized feature" note).

@@ -69,6 +69,8 @@ SYMBOLS = [
     ("vpq_qmv_group_w4g64_f16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
     ("vpq_qmv_group_w4g32_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i]),
     ("vpq_qmv_group_w8g64_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
+    ("vpq_rmsnorm_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
+    ("vpq_qmv_qkv_rms_bf16", _i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _f, _vp]),
     ("vpq_interleave_rows", _i, [_vp, _vp, _vp, _vp, _sz, _sz]),
     ("vpq_qmv_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmv_swiglu_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
@@ -843,6 +845,34 @@ def qmv_group_w8g64(packs, x, K, M, outs=None):
     if outs is None:
         outs = [torch.empty((M, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
     return QmvGroup(packs, x, K, M, outs, entry="vpq_qmv_group_w8g64_bf16").launch()
+
+
+def rmsnorm_bf16(x, norm_w, K, M, eps, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
+    _check(load().vpq_rmsnorm_bf16(_stream(), _ptr(x), _ptr(norm_w), _ptr(out), K, M, eps), "vpq_rmsnorm_bf16")
+    return out
+
+
+VPQ_FORMAT_W4G64, VPQ_FORMAT_W4G32, VPQ_FORMAT_W8G64 = 0, 1, 2
+
+
+def qmv_qkv_rms(fmt, packs, x, norm_w, K, eps, outs=None, x_norm_ws=None):
+    """RMSNorm of the row x [1,K], then the grouped GEMV of the format over it; packs as qmv_group_w4g64."""
+    import torch
+    if outs is None:
+        outs = [torch.empty((1, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
+    if x_norm_ws is None:
+        x_norm_ws = torch.empty((1, K), dtype=torch.bfloat16, device=x.device)
+    n = len(packs)
+    PA = ctypes.c_void_p * n
+    wt, st, bt = (PA(*[p[i].data_ptr() for p in packs]) for i in range(3))
+    yt = PA(*[o.data_ptr() for o in outs])
+    Nt = (ctypes.c_int * n)(*[int(p[3]) for p in packs])
+    _check(load().vpq_qmv_qkv_rms_bf16(_stream(), fmt, n, wt, st, bt, _ptr(x), _ptr(norm_w), yt, K, Nt, eps, _ptr(x_norm_ws)),
+           "vpq_qmv_qkv_rms_bf16")
+    return outs
 
 
 def qmv_group_w4g64_f16(packs, x, K, M, outs=None):

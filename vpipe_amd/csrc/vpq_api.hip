@@ -1543,6 +1543,37 @@ int vpq_qmv_group_w8g64_bf16(vpq_stream_t stream, int count, const uint32_t* con
   return VPQ_OK;
 }
 
+int vpq_rmsnorm_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* norm_w, uint16_t* out, int K, int M, float eps)
+{
+  if (x == nullptr || norm_w == nullptr || out == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (K < 1 || M < 1 || M > 65535 || !(eps >= 0.0f)) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 2) || !aligned(norm_w, 2) || !aligned(out, 2)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_rmsnorm(reinterpret_cast<hipStream_t>(stream), x, norm_w, out, K, M, eps));
+}
+
+// `affine_qmv_qkv_rms_w4g64` / `_w4g32` / `_w8g64` (gpu-kernels/metal/quant/affine_qmv.metal:671-740): RMSNorm of the
+// one row of x, then the fused-QKV GEMV over the normalized row.  format: 0 = 4-bit group-64, 1 = 4-bit group-32,
+// 2 = 8-bit group-64.  x_norm_ws: K elements of scratch that receive the normalized row.
+int vpq_qmv_qkv_rms_bf16(vpq_stream_t stream, int format, int count, const uint32_t* const* w, const uint16_t* const* scales,
+                         const uint16_t* const* biases, const uint16_t* x, const uint16_t* norm_w, uint16_t* const* y,
+                         int K, const int* N, float eps, uint16_t* x_norm_ws)
+{
+  if (format < 0 || format > 2) { return VPQ_ERR_BAD_SHAPE; }
+  if (x_norm_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
+  if (!aligned(x_norm_ws, 16)) { return VPQ_ERR_MISALIGNED; }
+  // the packs are checked before anything runs, by the format's own entry point on a count of zero rows ...
+  if (w == nullptr || scales == nullptr || biases == nullptr || y == nullptr || N == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (count < 1 || count > 4) { return VPQ_ERR_BAD_SHAPE; }
+  if (K <= 0 || (K % (format == 1 ? 32 : 64)) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  int st = vpq_rmsnorm_bf16(stream, x, norm_w, x_norm_ws, K, 1, eps);
+  if (st != VPQ_OK) { return st; }
+  if (format == 1) { return vpq_qmv_group_w4g32_bf16(stream, count, w, scales, biases, x_norm_ws, y, K, N, 1, 0); }
+  if (format == 2) { return vpq_qmv_group_w8g64_bf16(stream, count, w, scales, biases, x_norm_ws, y, K, N, 1); }
+  return vpq_qmv_group_w4g64_bf16(stream, count, w, scales, biases, x_norm_ws, y, K, N, 1);
+}
+
 int vpq_qmv_group_w4g64_f16(vpq_stream_t stream, int count, const uint32_t* const* w,
                             const uint16_t* const* scales, const uint16_t* const* biases,
                             const uint16_t* x, uint16_t* const* y, int K, const int* N, int M)

@@ -191,6 +191,8 @@ size_t qmv_ring_workspace_bytes(int K, int N, int M);   // planes of the widest 
 // Row-streaming kernel (M <= 2, any K % 64): rows_per_wave in {2, 4}, 0 = default.
 bool qmv_rows_supports(int K, int N, int M);
 hipError_t launch_qmv_rows(hipStream_t st, const QmvArgs& a, int rows_per_wave);
+// out[m, k] = bf16(x[m, k] * rsqrt(mean(x[m, :]^2) + eps) * norm_w[k]): the RMSNorm ahead of the fused-QKV GEMV.
+hipError_t launch_rmsnorm(hipStream_t st, const uint16_t* x, const uint16_t* norm_w, uint16_t* out, int K, int M, float eps);
 hipError_t launch_qmv_rows_group(hipStream_t st, const QmvArgs& a, const QmvGroup& g, int group = 64,
                                  bool scale_only = false);
 // Gathered (MoE) form, M = 1 per pair: a.w/scales/biases are batches [E, N, ...] of expert slabs,

@@ -117,6 +117,9 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_moe_gate_w8g64", QuantKernel::MoeGate, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_qkv_w8g64", QuantKernel::QmvQkv, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_qkv_rms_w4g64", QuantKernel::QmvQkvRms},
+    {"affine_qmv_bf16", "affine_qmv_qkv_rms_w4g32", QuantKernel::QmvQkvRms, QuantFormat::W4G32},
+    {"affine_qmv_bf16", "affine_qmv_qkv_rms_w8g64", QuantKernel::QmvQkvRms, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_qkv_w4g32", QuantKernel::QmvQkv, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_grouped_swiglu_w8g64", QuantKernel::SortedSwiglu, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_grouped_down_w8g64", QuantKernel::SortedDown, QuantFormat::W8G64},
@@ -417,7 +420,7 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
   int status = VPQ_OK;
   const QuantKernel kind = _fn.kind();
   const QuantFormat fmt = _fn.format();
-  if (fmt != QuantFormat::W4G64 && kind != QuantKernel::QmvQkv) {
+  if (fmt != QuantFormat::W4G64 && kind != QuantKernel::QmvQkv && kind != QuantKernel::QmvQkvRms) {
     // The 8-bit and group-32 twins keep the slot layout of the 4-bit group-64 functions:
     // dequant 0:w 1:scales 2:biases 3:w_deq 4:K 5:N; QMV 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N [7:residual],
     // rows from grid.x.  The Q4_0 forms ignore slot 2.
@@ -619,6 +622,37 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
                    : vpq_sample_topp_bf16(st, static_cast<const uint16_t*>(buf(0)), static_cast<int32_t*>(buf(1)), ival(2),
                                           fval(3), fval(4), static_cast<uint32_t>(_slots[5].ivalue), static_cast<uint16_t*>(buf(6)),
                                           ival(7), fval(8), fval(9), ival(10), fval(11), static_cast<uint8_t*>(buf(12)));
+  } else if (kind == QuantKernel::QmvQkvRms) {
+    // gpu-kernels/metal/quant/affine_qmv.metal:671-740: slots 0:w 1:scales 2:biases 3:x 4:norm_w 5:q_out 6:k_out 7:v_out
+    // 8:K 9:q_rows 10:k_rows 11:v_rows 12:eps; the pack is the row-concatenated q|k|v
+    if (!buf(0) || !buf(1) || !buf(2) || !buf(3) || !buf(4) || !buf(5) || !buf(6) || !has_int(8) || !has_int(9) ||
+        !has_int(10) || !has_int(11) || !has_int(12) || (ival(11) > 0 && !buf(7))) {
+      status = VPQ_ERR_NULL_POINTER;
+    } else if (ival(8) <= 0 || ival(8) % 64 != 0 || ival(9) <= 0 || ival(10) <= 0 || ival(11) < 0) {
+      status = VPQ_ERR_BAD_SHAPE;
+    } else {
+      const int K = ival(8);
+      const int rows[3] = {ival(9), ival(10), ival(11)};
+      const uint32_t* w[3];
+      const uint16_t* sc[3];
+      const uint16_t* bi[3];
+      uint16_t* y[3] = {static_cast<uint16_t*>(buf(5)), static_cast<uint16_t*>(buf(6)), static_cast<uint16_t*>(buf(7))};
+      const size_t row_words = (size_t)(fmt == QuantFormat::W8G64 ? K / 4 : K / 8);
+      const size_t row_groups = (size_t)(fmt == QuantFormat::W4G32 ? K / 32 : K / 64);
+      size_t r0 = 0;
+      for (int i = 0; i < 3; ++i) {
+        w[i] = static_cast<const uint32_t*>(buf(0)) + r0 * row_words;
+        sc[i] = static_cast<const uint16_t*>(buf(1)) + r0 * row_groups;
+        bi[i] = static_cast<const uint16_t*>(buf(2)) + r0 * row_groups;
+        r0 += (size_t)rows[i];
+      }
+      // the normalized row: scratch of the stream (shared, so not inside a concurrent scope)
+      uint16_t* xn = in_scope ? nullptr : static_cast<uint16_t*>(s->qmv_workspace((size_t)K * 2));
+      const int format = fmt == QuantFormat::W8G64 ? VPQ_FORMAT_W8G64 : (fmt == QuantFormat::W4G32 ? VPQ_FORMAT_W4G32 : VPQ_FORMAT_W4G64);
+      status = xn == nullptr ? VPQ_ERR_WORKSPACE
+                             : vpq_qmv_qkv_rms_bf16(st, format, rows[2] > 0 ? 3 : 2, w, sc, bi, static_cast<const uint16_t*>(buf(3)),
+                                                    static_cast<const uint16_t*>(buf(4)), y, K, rows, _slots[12].fvalue, xn);
+    }
   } else if (kind == QuantKernel::QmvQkv) {
     // gpu-kernels/metal/quant/affine_qmv.metal:497-516: slots 0:w 1:scales 2:biases 3:x 4:q_out
     // 5:k_out 6:v_out 7:K 8:q_rows 9:k_rows 10:v_rows; the pack is the row-concatenated q|k|v.

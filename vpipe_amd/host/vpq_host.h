@@ -79,6 +79,8 @@ enum class QuantKernel : std::uint8_t {
   QmmSwiglu,      // affine_qmm_swiglu_w4g64[_bm64|_bm128|_bm64_rs]: slot 7 = M, 8 = out_stride, 9 = out_off (_rs)
   QmvGeglu,       // affine_qmv_geglu_w4g64: as QmvSwiglu with gelu_tanh(gate) * up
   QmvGeluMul,     // affine_qmv_gelu_mul_w4g64: one row of x, slot 7 = mul buffer [N]; y = gelu_tanh(W x) * mul
+  QmvQkvRms,      // affine_qmv_qkv_rms_w4g64 / _w4g32 / _w8g64: slots 0:w 1:scales 2:biases 3:x 4:norm_w 5:q 6:k 7:v 8:K
+                  //   9,10,11 = q_rows, k_rows, v_rows, 12 = eps (float); the normalized row goes through stream scratch
   MoeGate,        // affine_moe_gate_w8g64: slots 0:w 1:scales 2:biases 3:x 4:gate 5:K; rows of x = grid.y
   QmmGeglu,       // affine_qmm_geglu_w4g64: as QmmSwiglu
   EmbedGather,    // dequant_embed_gather_f16: slots 0:ids 1:w 2:scales 3:biases 4:out 5:H; T = grid.y,
