@@ -605,6 +605,19 @@ int vpq_qmm_tiled_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
  * 64 rows, vpq_qmm_w8g64_bf16 above. */
 int vpq_linear_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M);
+/* 8-bit codes in groups of 32 (GGUF q8 repacked to affine; the codec's int8 path): w uint32 [N, K/4], scales / biases
+ * bf16 [N, K/32], K % 32 == 0.  vpq_dequant_w8g32_bf16 replaces `affine_dequant_w8g32` (affine_dequant.metal:99-131),
+ * bit-exact; vpq_qmv_w8g32_bf16 replaces `affine_qmv_w8g32` (affine_qmv.metal:3053-3069), QMV arithmetic, 1 <= M <= 16;
+ * vpq_qmm_dense_route_w8g32_bf16 serves `affine_qmm_steel_w8g32` (affine_qmm_steel.metal:1674-1698) by the
+ * dequant-once route the reference's codec itself takes (arguments as vpq_qmm_dense_route_w4g64_bf16). */
+int vpq_dequant_w8g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                           const uint16_t* biases, uint16_t* w_deq, int K, int N);
+int vpq_qmv_w8g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                       const uint16_t* residual);
+int vpq_qmm_dense_route_w8g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                   uint16_t* w_deq, int expand);
 /* `affine_moe_gate_w8g64` (affine_qmv.metal:1323-1349): the shared-expert gate, gate[m] = bf16(sigmoid(W[1,K] . x[m]))
  * for M rows of x (1 <= M <= 65535) over a one-row 8-bit pack (w uint32 [K/4], scales / biases bf16 [K/64]). */
 int vpq_moe_gate_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

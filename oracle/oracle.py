@@ -356,14 +356,22 @@ def dequant8_bf16(w, s, b, K, N):
     return out
 
 
-def matmul8(w, s, b, x, K, N, M, rounded):
-    """w8g64 y = x . W^T -> (y64, y_bf16); rounded=False: QMV semantics, True: GEMM semantics."""
+def matmul8(w, s, b, x, K, N, M, rounded, group=64):
+    """8-bit codes, y = x . W^T -> (y64, y_bf16); rounded=False: QMV semantics, True: GEMM semantics."""
     w, s, b, x = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16), _c(x, np.uint16)
     y64 = np.empty((M, N), dtype=np.float64)
     yb = np.empty((M, N), dtype=np.uint16)
-    lib().vpo_matmul_w8g64(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y64, _f64p), _p(yb, _u16p),
-                           K, N, M, 1 if rounded else 0)
+    lib().vpo_matmul_w8(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(x, _u16p), _p(y64, _f64p), _p(yb, _u16p),
+                        K, N, M, 1 if rounded else 0, group)
     return y64, yb
+
+
+def dequant8_g32(w, s, b, K, N):
+    """w8g32: w uint32 [N, K/4], scales / biases [N, K/32] -> bf16 bits [N, K]."""
+    w, s, b = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16)
+    out = np.empty((N, K), dtype=np.uint16)
+    lib().vpo_dequant_w8_bf16(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(out, _u16p), K, N, 32)
+    return out
 
 
 def quantize(wsrc, K, N, clip=1.0):

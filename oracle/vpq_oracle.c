@@ -1049,18 +1049,24 @@ static inline unsigned code8(const uint32_t* w, size_t n, int Kw, int k)
 
 /* affine_dequant_w8g64 (affine_dequant.metal:68-97): out = (elt)(s * (float)q + b);
  * s*q is exact in fp32 (8-bit x 8-bit significands). */
-void vpo_dequant_w8g64_bf16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                            uint16_t* out, int K, int N)
+void vpo_dequant_w8_bf16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                         uint16_t* out, int K, int N, int group)
 {
-  const int Kw = K / 4, Kg = K / VPO_GROUP;
+  const int Kw = K / 4, Kg = K / group;
   for (size_t n = 0; n < (size_t)N; ++n) {
     for (int k = 0; k < K; ++k) {
-      const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
-      const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / group]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / group]);
       const float sq = s * (float)code8(w, n, Kw, k);
       out[n * (size_t)K + k] = vpo_f32_to_bf16(sq + b);
     }
   }
+}
+
+void vpo_dequant_w8g64_bf16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                            uint16_t* out, int K, int N)
+{
+  vpo_dequant_w8_bf16(w, scales, biases, out, K, N, VPO_GROUP);
 }
 
 /* QMV (affine_qmv_w8g64, affine_qmv.metal:3034-3050 = qmv_fast_impl<T,64,8>: the same
@@ -1068,15 +1074,25 @@ void vpo_dequant_w8g64_bf16(const uint32_t* w, const uint16_t* scales, const uin
  * the GEMM semantics (weight rounded to the element type first: affine_qmm_steel_w8g64,
  * affine_qmm_steel.metal:1601-1624, and the dequant-once route) when rounded != 0.
  * Double accumulation; y_bf16 (nullable) is the RNE cast. */
+/* The group is a parameter: 64, or 32 for the twins of affine_dequant.metal:99-131, affine_qmv.metal:3053-3069,
+ * affine_qmm_steel.metal:1674-1698, in which only the stride of the scales changes. */
+void vpo_matmul_w8(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int M, int rounded, int group);
 void vpo_matmul_w8g64(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                       const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int M, int rounded)
 {
-  const int Kw = K / 4, Kg = K / VPO_GROUP;
+  vpo_matmul_w8(w, scales, biases, x, y64, y_bf16, K, N, M, rounded, VPO_GROUP);
+}
+
+void vpo_matmul_w8(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                   const uint16_t* x, double* y64, uint16_t* y_bf16, int K, int N, int M, int rounded, int group)
+{
+  const int Kw = K / 4, Kg = K / group;
   float* wrow = (float*)malloc(sizeof(float) * (size_t)K);
   for (size_t n = 0; n < (size_t)N; ++n) {
     for (int k = 0; k < K; ++k) {
-      const float s = vpo_bf16_to_f32(scales[n * Kg + k / VPO_GROUP]);
-      const float b = vpo_bf16_to_f32(biases[n * Kg + k / VPO_GROUP]);
+      const float s = vpo_bf16_to_f32(scales[n * Kg + k / group]);
+      const float b = vpo_bf16_to_f32(biases[n * Kg + k / group]);
       const float sq = s * (float)code8(w, n, Kw, k);
       const float v = sq + b;
       wrow[k] = rounded ? vpo_bf16_to_f32(vpo_f32_to_bf16(v)) : v;

@@ -949,6 +949,25 @@ def test_load_and_run_eight_bit_and_group32_packs(vpq, enc, dev, D, tmp_path, M)
     assert L.hd_load_and_run(enc.h, r, b"b", 0, xd.data_ptr(), yd.data_ptr(), M, kn) == 0
     assert b"pass K" in L.hr_why()
     L.hr_close(r)
+    # 8-bit codes in groups of 32: the GEMV in slabs up to 64 rows, the dequant-once route above
+    w3, s3, b3 = synth.make_weight8(N, K, 4203, group=32)
+    sttorch.save_file({"c.weight": torch.from_numpy(w3.view(np.int32)), "c.scales": as_bf16(s3), "c.biases": as_bf16(b3)},
+                      str(tmp_path / "c.safetensors"))
+    raw = (tmp_path / "c.safetensors").read_bytes()
+    hlen = int.from_bytes(raw[:8], "little")
+    (tmp_path / "c.safetensors").write_bytes(raw[:8] + raw[8:8 + hlen].replace(b'"I32"', b'"U32"') + raw[8 + hlen:])
+    r = L.hr_open(str(tmp_path / "c.safetensors").encode(), 0)
+    assert r, L.hr_why()
+    yd = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+    assert L.hd_load_and_run(enc.h, r, b"c", K, xd.data_ptr(), yd.data_ptr(), M, kn) == 1, L.hr_why()
+    p3 = (D.u32(w3, dev), D.bf16(s3, dev), D.bf16(b3, dev))
+    if M <= 64:
+        want = torch.cat([vpq.qmv_w8g32(*p3, xd[m0:m0 + 16], K, N, min(16, M - m0)) for m0 in range(0, M, 16)])
+    else:
+        want = vpq.qmm_dense_route_w8g32(*p3, xd, K, N, M, torch.empty((N, K), dtype=torch.bfloat16, device=dev))
+    assert torch.equal(yd, want) and yd.abs().sum() > 0
+    L.hr_close(r)
 
 
 def test_gelu_mul_and_shared_expert_gate_function_names(vpq, enc, dev, D):
@@ -1038,3 +1057,41 @@ def test_rmsnorm_fused_qkv_call_sites(vpq, enc, dev, D, name, fmt):
     for o, ref in zip(outs, vpq.qmv_qkv_rms(fmt, packs, xd, nwd, K, eps)):
         assert torch.equal(o, ref)
     assert outs[0].abs().sum() > 0
+
+
+def test_eight_bit_group32_function_names(vpq, enc, dev, D):
+    # affine_dequant_w8g32, affine_qmv_w8g32, affine_qmm_steel_w8g32 (slots of the 4-bit functions; the GEMM's
+    # expansion goes through scratch of the stream): the encoder's results are the C ABI's, bit for bit
+    K, N, M, Mq = 512, 40, 2, 70
+    w, s, b = synth.make_weight8(N, K, 90, group=32)
+    x, xq = synth.make_act(M, K, 91), synth.make_act(Mq, K, 92)
+    wd, sd, bd, xd, xqd = D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), D.bf16(x, dev), D.bf16(xq, dev)
+    dq = torch.zeros((N, K), dtype=torch.bfloat16, device=dev)
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    yq = torch.zeros((Mq, N), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_dequant_bf16", "affine_dequant_w8g32") == 1
+    for i, t in enumerate((wd, sd, bd, dq)):
+        enc.set_buffer(i, t)
+    enc.set_constant(4, K)
+    enc.set_constant(5, N)
+    enc.dispatch((K // 4, N, 1), (32, 1, 1))
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_w8g32") == 1
+    for i, t in enumerate((wd, sd, bd, xd, y)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.dispatch((32 * M, N // 4, 1), (32, 2, 1))
+    assert enc.set_function("affine_qmm_steel_bf16", "affine_qmm_steel_w8g32") == 1
+    for i, t in enumerate((wd, sd, bd, xqd, yq)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.set_constant(7, Mq)
+    enc.dispatch(((N + 31) // 32, (Mq + 31) // 32, 1), (32, 2, 2))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert torch.equal(dq, vpq.dequant_w8g32(wd, sd, bd, K, N))
+    assert torch.equal(y, vpq.qmv_w8g32(wd, sd, bd, xd, K, N, M))
+    scratch = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+    assert torch.equal(yq, vpq.qmm_dense_route_w8g32(wd, sd, bd, xqd, K, N, Mq, scratch))
+    assert y.abs().sum() > 0 and yq.abs().sum() > 0

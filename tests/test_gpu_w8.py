@@ -444,3 +444,36 @@ def test_qmv_group_w8_is_the_separate_calls(vpq, dev, D, K, M, rows):
     for o, p in zip(outs, packs):
         o.assert_intact()
         assert torch.equal(o.view, vpq.qmv_w8g64(p[0], p[1], p[2], xd, K, p[3], M))
+
+
+@pytest.mark.parametrize("K,N,M", [(32, 5, 1), (96, 33, 3), (1024, 48, 2), (4096, 95, 8), (2560, 64, 16), (5120, 1024, 1)])
+def test_w8g32_dequant_qmv_and_dense_route(vpq, oracle, dev, D, K, N, M):
+    """affine_dequant_w8g32 (bit-exact), affine_qmv_w8g32 (QMV arithmetic, residual add) and affine_qmm_steel_w8g32 by the
+    dequant-once route, against the oracle's group-32 8-bit twins."""
+    w, s, b = synth.make_weight8(N, K, 5600 + K + N, group=32)
+    x = synth.make_act(M, K, 5700 + K + M)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    dq = parity.Guarded((N, K), torch.bfloat16, dev)
+    vpq.dequant_w8g32(wd, sd, bd, K, N, out=dq.view)
+    torch.cuda.synchronize()
+    dq.assert_intact()
+    assert np.array_equal(D.bits(dq.view), oracle.dequant8_g32(w, s, b, K, N))
+    y64, yb = oracle.matmul8(w, s, b, x, K, N, M, rounded=False, group=32)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmv_w8g32(wd, sd, bd, xd, K, N, M, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_bf16(D.bits(out.view), y64, yb)
+    res = synth.make_act(M, N, 5800 + N)
+    got = D.bits(vpq.qmv_w8g32(wd, sd, bd, xd, K, N, M, residual=D.bf16(res, dev)))
+    want = synth.f32_to_bf16_bits(synth.bf16_bits_to_f32(D.bits(out.view)) + synth.bf16_bits_to_f32(res))
+    assert np.array_equal(got, want)
+    r64, rb = oracle.matmul8(w, s, b, x, K, N, M, rounded=True, group=32)
+    w_deq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+    gemm = vpq.qmm_dense_route_w8g32(wd, sd, bd, xd, K, N, M, w_deq)
+    parity.check_bf16(D.bits(gemm), r64, rb)
+    assert torch.equal(w_deq, dq.view)
+    L = vpq.load()
+    p = out.view.data_ptr()
+    assert L.vpq_qmv_w8g32_bf16(None, p, p, p, p, p, K + 8, N, M, None) == -2
+    assert L.vpq_qmm_dense_route_w8g32_bf16(None, p, p, p, p, p, K, N, M, None, 1) == -4

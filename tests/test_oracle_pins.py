@@ -659,6 +659,34 @@ def parity_ulp(a, b):
     return int(parity.bf16_ulp_distance(a, b).max())
 
 
+def test_w8g32_twins_against_numpy_and_the_group64_oracle(oracle):
+    """8-bit codes in groups of 32: the dense expansion against numpy written from the byte view of the words, both
+    contractions against a float64 matmul of it, and a group-64 pack whose scales and biases are each stored twice
+    gives the group-64 oracle's bits."""
+    N, K, M = 11, 192, 3
+    w, s, b = synth.make_weight8(N, K, 81, group=32)
+    q = w.view(np.uint8).reshape(N, K).astype(np.float32)          # little-endian bytes = values in k order
+    sf = np.repeat(synth.bf16_bits_to_f32(s), 32, axis=1)
+    bf = np.repeat(synth.bf16_bits_to_f32(b), 32, axis=1)
+    dense32 = sf * q + bf                                          # s*q exact in fp32 (8 x 8 bit significands)
+    assert np.array_equal(oracle.dequant8_g32(w, s, b, K, N), synth.f32_to_bf16_bits(dense32))
+    x = synth.make_act(M, K, 82)
+    xf = synth.bf16_bits_to_f32(x).astype(np.float64)
+    y64, yb = oracle.matmul8(w, s, b, x, K, N, M, rounded=False, group=32)
+    ref = xf @ dense32.astype(np.float64).T
+    assert np.allclose(y64, ref, rtol=0, atol=1e-12 * np.abs(ref).max() + 1e-12)
+    assert np.array_equal(yb, synth.f32_to_bf16_bits(ref.astype(np.float32)))
+    r64, _ = oracle.matmul8(w, s, b, x, K, N, M, rounded=True, group=32)
+    refr = xf @ synth.bf16_bits_to_f32(synth.f32_to_bf16_bits(dense32)).astype(np.float64).T
+    assert np.allclose(r64, refr, rtol=0, atol=1e-12 * np.abs(refr).max() + 1e-12)
+    w6, s6, b6 = synth.make_weight8(N, K, 83)
+    s2, b2 = np.repeat(s6, 2, axis=1), np.repeat(b6, 2, axis=1)
+    assert np.array_equal(oracle.dequant8_g32(w6, s2, b2, K, N), oracle.dequant8_bf16(w6, s6, b6, K, N))
+    a64, ab = oracle.matmul8(w6, s2, b2, x, K, N, M, rounded=False, group=32)
+    c64, cb = oracle.matmul8(w6, s6, b6, x, K, N, M, rounded=False)
+    assert np.array_equal(a64, c64) and np.array_equal(ab, cb)
+
+
 def test_grouped_gemm_oracle_with_byte_codes_reduces_to_the_plain_8bit_gemm(oracle):
     """The 8-bit form of the grouped restatement: every live slot equals the plain 8-bit GEMM oracle
     (bf16-rounded weights) of its row on its expert's slab."""

@@ -70,6 +70,9 @@ SYMBOLS = [
     ("vpq_qmv_group_w4g32_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i]),
     ("vpq_qmv_group_w8g64_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
     ("vpq_rmsnorm_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
+    ("vpq_dequant_w8g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_qmv_w8g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    ("vpq_qmm_dense_route_w8g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_qmv_qkv_rms_bf16", _i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _f, _vp]),
     ("vpq_interleave_rows", _i, [_vp, _vp, _vp, _vp, _sz, _sz]),
     ("vpq_qmv_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
@@ -845,6 +848,33 @@ def qmv_group_w8g64(packs, x, K, M, outs=None):
     if outs is None:
         outs = [torch.empty((M, p[3]), dtype=torch.bfloat16, device=x.device) for p in packs]
     return QmvGroup(packs, x, K, M, outs, entry="vpq_qmv_group_w8g64_bf16").launch()
+
+
+def dequant_w8g32(w, scales, biases, K, N, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((N, K), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_dequant_w8g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out), K, N),
+           "vpq_dequant_w8g32_bf16")
+    return out
+
+
+def qmv_w8g32(w, scales, biases, x, K, N, M, out=None, residual=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmv_w8g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                     _ptr(residual)), "vpq_qmv_w8g32_bf16")
+    return out
+
+
+def qmm_dense_route_w8g32(w, scales, biases, x, K, N, M, w_deq, expand=True, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_dense_route_w8g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                                 _ptr(w_deq), 1 if expand else 0), "vpq_qmm_dense_route_w8g32_bf16")
+    return out
 
 
 def rmsnorm_bf16(x, norm_w, K, M, eps, out=None):

@@ -373,6 +373,76 @@ int vpq_qmm_dense_route_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const
   return VPQ_OK;
 }
 
+// ---- 8-bit codes in groups of 32 (GGUF q8 repacked; the codec's int8 path): `affine_dequant_w8g32`
+// (affine_dequant.metal:99-131), `affine_qmv_w8g32` (affine_qmv.metal:3053-3069), `affine_qmm_steel_w8g32`
+// (affine_qmm_steel.metal:1674-1698) by the dequant-once route, which is how the reference's codec runs it.
+namespace {
+
+int check_pack_w8g32(const uint32_t* w, const uint16_t* scales, const uint16_t* biases, int K, int N)
+{
+  if (w == nullptr || scales == nullptr || biases == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (K <= 0 || N <= 0 || (K % 32) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(w, 16) || !aligned(scales, 2) || !aligned(biases, 2)) { return VPQ_ERR_MISALIGNED; }
+  return VPQ_OK;
+}
+
+}  // namespace
+
+int vpq_dequant_w8g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                           uint16_t* w_deq, int K, int N)
+{
+  int st = check_pack_w8g32(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (w_deq == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (!aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_dequant8(reinterpret_cast<hipStream_t>(stream), w, scales, biases, w_deq, K, N, 32));
+}
+
+int vpq_qmv_w8g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                       const uint16_t* x, uint16_t* y, int K, int N, int M, const uint16_t* residual)
+{
+  int st = check_pack_w8g32(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (M < 1 || M > 16 || (K % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 2) || (residual != nullptr && !aligned(residual, 2))) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  vpq::QmvArgs a{};
+  a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y; a.residual = residual;
+  a.K = K; a.N = N; a.M = M; a.y_f32 = false; a.cu_count = g_dev.cu_count;
+  return finish(vpq::launch_qmv_simple8(reinterpret_cast<hipStream_t>(stream), a, 32));
+}
+
+int vpq_qmm_dense_route_w8g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                   const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                   uint16_t* w_deq, int expand)
+{
+  int st = check_pack_w8g32(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (w_deq == nullptr) { return VPQ_ERR_WORKSPACE; }
+  if (M <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (expand != 0) {
+    st = finish(vpq::launch_dequant8(hs, w, scales, biases, w_deq, K, N, 32));
+    if (st != VPQ_OK) { return st; }
+  }
+  std::string why;
+  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, g_dev.cu_count, &why);
+  if (rc != 0) {
+    strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
+    g_last_error[sizeof(g_last_error) - 1] = '\0';
+    return VPQ_ERR_DEVICE;
+  }
+  return VPQ_OK;
+}
+
 int vpq_embed_gather_w4g64_bf16(vpq_stream_t stream, const int32_t* ids, const uint32_t* w, const uint16_t* scales,
                                 const uint16_t* biases, uint16_t* out, int H, int T, int vocab)
 {

@@ -71,16 +71,18 @@ hipError_t launch_dequant_g32(hipStream_t st, const uint32_t* w, const uint16_t*
 }
 
 // 8-bit twin (gpu-kernels/metal/quant/affine_dequant.metal:60-97): one byte per value, four per word;
-// one thread per word, 8-byte stores.  s*q is exact in fp32 (8-bit x 8-bit significands).
-__global__ __launch_bounds__(256) void dequant_w8g64_kernel(
+// one thread per word, 8-byte stores.  s*q is exact in fp32 (8-bit x 8-bit significands).  WS: log2 of the words
+// per quantization group (4: group 64; 3: group 32, affine_dequant_w8g32, :99-131).
+template <int WS>
+__global__ __launch_bounds__(256) void dequant_w8_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, uint2* __restrict__ out, int Kw, size_t total_words)
 {
-  const int Kg = Kw >> 4;
+  const int Kg = Kw >> WS;
   for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total_words; idx += (size_t)gridDim.x * 256) {
     const size_t n = idx / (size_t)Kw;
     const int j = (int)(idx - n * (size_t)Kw);
-    const size_t g = n * (size_t)Kg + (size_t)(j >> 4);
+    const size_t g = n * (size_t)Kg + (size_t)(j >> WS);
     const float s = bf16_bits_to_f32(scales[g]);
     const float b = bf16_bits_to_f32(biases[g]);
     const uint32_t p = w[idx];
@@ -92,13 +94,17 @@ __global__ __launch_bounds__(256) void dequant_w8g64_kernel(
 }
 
 hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                           uint16_t* out, int K, int N)
+                           uint16_t* out, int K, int N, int group)
 {
   const int Kw = K / 4;
   const size_t total = (size_t)N * (size_t)Kw;
   size_t blocks = (total + 255) / 256;
   if (blocks > 65536 * 4) { blocks = 65536 * 4; }
-  return launch_kernel(dequant_w8g64_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w, scales, biases,
+  if (group == 32) {
+    return launch_kernel(dequant_w8_kernel<3>, dim3((unsigned)blocks), dim3(256), 0, st, w, scales, biases,
+                         reinterpret_cast<uint2*>(out), Kw, total);
+  }
+  return launch_kernel(dequant_w8_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, st, w, scales, biases,
                        reinterpret_cast<uint2*>(out), Kw, total);
 }
 

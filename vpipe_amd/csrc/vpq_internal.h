@@ -141,8 +141,8 @@ hipError_t launch_qmv_simple_g32(hipStream_t st, const QmvArgs& a, bool scale_on
 hipError_t launch_qmv_rows_g32(hipStream_t st, const QmvArgs& a, bool scale_only);   // M <= 2
 // The 8-bit twins (one byte per value, w is [N, K/4] words): dense expansion and the general QMV kernel.
 hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                           uint16_t* out, int K, int N);
-hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a);
+                           uint16_t* out, int K, int N, int group = 64);
+hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a, int group = 64);
 // Mixed-width fused gate/up over separate packs (4 or 8 bits each); rows = pairs (pair_eid) or rows of x.
 struct SplitGateUp {
   const uint32_t* wg; const uint16_t* sg; const uint16_t* bg; int gate_bits;

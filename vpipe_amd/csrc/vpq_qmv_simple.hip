@@ -149,8 +149,9 @@ hipError_t launch_qmv_simple_g32(hipStream_t st, const QmvArgs& a, bool scale_on
 
 // 8-bit twin (affine_qmv_w8g64, gpu-kernels/metal/quant/affine_qmv.metal:3034-3050): one byte per
 // value.  Each lane takes 16 consecutive k (one 128-bit load of codes, a quarter of a group) per
-// pass over the row; otherwise the kernel above: W = fma(s, q, b) in fp32, never rounded.
-template <int MT, bool F32OUT>
+// pass over the row; otherwise the kernel above: W = fma(s, q, b) in fp32, never rounded.  GS: log2 of the group
+// (6, or 5 for affine_qmv_w8g32, :3053-3069).
+template <int MT, bool F32OUT, int GS = 6>
 __global__ __launch_bounds__(256) void qmv_simple8_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x, void* __restrict__ y,
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(256) void qmv_simple8_kernel(
   const int lane = threadIdx.x & 63;
   const int n = blockIdx.x * 4 + wave;
   if (n >= N) { return; }  // wave-uniform; no barrier in this kernel
-  const int Kw = K >> 2, Kg = K >> 6;
+  const int Kw = K >> 2, Kg = K >> GS;
   const uint32_t* wrow = w + (size_t)n * Kw;
   const uint16_t* srow = scales + (size_t)n * Kg;
   const uint16_t* brow = biases + (size_t)n * Kg;
@@ -172,8 +173,8 @@ __global__ __launch_bounds__(256) void qmv_simple8_kernel(
     for (int k0 = lane * 16; k0 < K; k0 += kWave * 16) {
       const uint4 c4 = *reinterpret_cast<const uint4*>(wrow + (k0 >> 2));
       const uint32_t codes[4] = {c4.x, c4.y, c4.z, c4.w};
-      const float s = bf16_bits_to_f32(srow[k0 >> 6]);
-      const float b = bf16_bits_to_f32(brow[k0 >> 6]);
+      const float s = bf16_bits_to_f32(srow[k0 >> GS]);
+      const float b = bf16_bits_to_f32(brow[k0 >> GS]);
       float wv[16];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -496,14 +497,18 @@ hipError_t launch_qmv_split_gate_up(hipStream_t st, const SplitGateUp& a)
 #undef VPQ_SPLIT
 }
 
-hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a)
+hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a, int group)
 {
   const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
-#define VPQ_LAUNCH8(MT, F32)                                                                    \
-  launch_kernel(qmv_simple8_kernel<MT, F32>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
+#define VPQ_LAUNCH8(MT, F32, GS)                                                                    \
+  launch_kernel(qmv_simple8_kernel<MT, F32, GS>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
                 a.residual, a.K, a.N, a.M)
-  if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH8(1, true) : VPQ_LAUNCH8(1, false); }
-  return a.y_f32 ? VPQ_LAUNCH8(4, true) : VPQ_LAUNCH8(4, false);
+  if (group == 32) {
+    if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH8(1, true, 5) : VPQ_LAUNCH8(1, false, 5); }
+    return a.y_f32 ? VPQ_LAUNCH8(4, true, 5) : VPQ_LAUNCH8(4, false, 5);
+  }
+  if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH8(1, true, 6) : VPQ_LAUNCH8(1, false, 6); }
+  return a.y_f32 ? VPQ_LAUNCH8(4, true, 6) : VPQ_LAUNCH8(4, false, 6);
 #undef VPQ_LAUNCH8
 }
 

@@ -116,6 +116,9 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_w8g64", QuantKernel::Qmv, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_moe_gate_w8g64", QuantKernel::MoeGate, QuantFormat::W8G64},
+    {"affine_dequant_bf16", "affine_dequant_w8g32", QuantKernel::Dequant, QuantFormat::W8G32},
+    {"affine_qmv_bf16", "affine_qmv_w8g32", QuantKernel::Qmv, QuantFormat::W8G32},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g32", QuantKernel::Qmm, QuantFormat::W8G32},
     {"affine_qmv_bf16", "affine_qmv_qkv_w8g64", QuantKernel::QmvQkv, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_qkv_rms_w4g64", QuantKernel::QmvQkvRms},
     {"affine_qmv_bf16", "affine_qmv_qkv_rms_w4g32", QuantKernel::QmvQkvRms, QuantFormat::W4G32},
@@ -441,6 +444,8 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
         status = vpq_dequant_w4g64_f16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
       } else if (fmt == QuantFormat::W8G64) {
         status = vpq_dequant_w8g64_bf16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
+      } else if (fmt == QuantFormat::W8G32) {
+        status = vpq_dequant_w8g32_bf16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
       } else {
         status = vpq_dequant_w4g32_bf16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
       }
@@ -545,6 +550,17 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
                                           kind == QuantKernel::QmvGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
       } else if (fmt == QuantFormat::W8G64) {
         status = vpq_qmv_w8g64_bf16(st, w, sc, bi, x, y, K, N, M, residual);
+      } else if (fmt == QuantFormat::W8G32 && kind == QuantKernel::Qmm) {
+        // gpu-kernels/metal/quant/affine_qmm_steel.metal:1674-1698, slot 7 = M: the dequant-once route, the
+        // expansion in scratch of the stream (shared, so not inside a concurrent scope)
+        uint16_t* w_deq = (in_scope || K <= 0 || N <= 0)
+                              ? nullptr
+                              : static_cast<uint16_t*>(s->qmv_workspace(static_cast<std::size_t>(N) * static_cast<std::size_t>(K) * 2));
+        status = !has_int(7) ? VPQ_ERR_NULL_POINTER
+                             : (w_deq == nullptr ? VPQ_ERR_WORKSPACE
+                                                 : vpq_qmm_dense_route_w8g32_bf16(st, w, sc, bi, x, y, K, N, ival(7), w_deq, 1));
+      } else if (fmt == QuantFormat::W8G32) {
+        status = vpq_qmv_w8g32_bf16(st, w, sc, bi, x, y, K, N, M, residual);
       } else if (kind == QuantKernel::QmvGeglu) {
         status = vpq_qmv_gated_w4g32_bf16(st, w, sc, q40 ? nullptr : bi, x, y, K, N, M, VPQ_GATE_GEGLU, q40 ? 1 : 0);
       } else {
@@ -849,12 +865,28 @@ void quant_linear_forward(CommandStream& stream, const Linear& lin, const Device
   const bool w4g64 = lin.bits == 4 && lin.group == 64;
   if (!w4g64) {
     // The format twins: their own size-based entrances; no adapter on them.
-    if (with_lora || !((lin.bits == 8 && lin.group == 64) || (lin.bits == 4 && lin.group == 32))) {
+    if (with_lora || !((lin.bits == 8 || lin.bits == 4) && (lin.group == 64 || lin.group == 32))) {
       stream.record_error(VPQ_ERR_BAD_SHAPE, "quant_linear_forward: pack format");
       return;
     }
-    status = lin.bits == 8 ? vpq_linear_w8g64_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M)
-                           : vpq_linear_w4g32_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M);
+    if (lin.bits == 8 && lin.group == 32) {
+      // 8-bit codes in groups of 32: the GEMV in slabs of 16 rows up to 64 rows, the dequant-once route above (its
+      // expansion in scratch of the stream), which is the route the reference's codec takes for this format
+      status = VPQ_OK;
+      if (M <= 64) {
+        for (int m0 = 0; m0 < M && status == VPQ_OK; m0 += 16) {
+          const int rows = M - m0 < 16 ? M - m0 : 16;
+          status = vpq_qmv_w8g32_bf16(st, w, sc, bi, xp + (size_t)m0 * lin.K, yp + (size_t)m0 * lin.N, lin.K, lin.N, rows, nullptr);
+        }
+      } else {
+        uint16_t* w_deq = static_cast<uint16_t*>(stream.qmv_workspace((size_t)lin.N * (size_t)lin.K * 2));
+        status = w_deq == nullptr ? VPQ_ERR_WORKSPACE
+                                  : vpq_qmm_dense_route_w8g32_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M, w_deq, 1);
+      }
+    } else {
+      status = lin.bits == 8 ? vpq_linear_w8g64_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M)
+                             : vpq_linear_w4g32_bf16(st, w, sc, bi, xp, yp, lin.K, lin.N, M);
+    }
   } else if (with_lora) {
     // An adapter always takes the GEMM route: its second factor is folded into the tile's accumulator.
     if (lora_t == nullptr || lora_t->size() < static_cast<std::size_t>(M) * lora->rank * 2) {

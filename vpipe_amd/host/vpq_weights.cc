@@ -555,13 +555,13 @@ bool PackFile::load_linear(CommandStream& stream, const std::string& prefix, int
   }
   const int N = (int)w->shape[0];
   // Width and group from the shapes (generative-models/qwen3/metal-qwen-model.cc:653-676); served: 4-bit group-64,
-  // 8-bit group-64, 4-bit group-32.
+  // 8-bit group-64, 4-bit group-32, 8-bit group-32.
   const int bits = affine_bits(prefix, K), group = affine_group(prefix, K);
-  const bool served = (bits == 4 && group == 64) || (bits == 8 && group == 64) || (bits == 4 && group == 32);
+  const bool served = (bits == 4 || bits == 8) && (group == 64 || group == 32);
   if (!served || K % group != 0 || w->shape[1] * 32 != (long long)K * bits || s->shape[0] != N ||
       s->shape[1] * group != K) {
     set_why(why, prefix + ": " + std::to_string(bits) + "-bit group-" + std::to_string(group) +
-                     " pack; this path takes 4-bit group-64, 8-bit group-64 and 4-bit group-32");
+                     " pack; this path takes 4- and 8-bit codes in groups of 64 and 32");
     return false;
   }
   std::vector<std::uint8_t> host((std::size_t)std::max(w->nbytes, s->nbytes));

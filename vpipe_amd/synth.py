@@ -61,14 +61,14 @@ def make_weight(N, K, seed):
     return w, s, b
 
 
-def make_weight8(N, K, seed):
-    """8-bit twin: (w uint32 [N,K/4], one byte per value; scales, biases bf16 bits [N,K/64])."""
-    assert K % GROUP == 0
+def make_weight8(N, K, seed, group=GROUP):
+    """8-bit twin: (w uint32 [N,K/4], one byte per value; scales, biases bf16 bits [N,K/group], group 64 or 32)."""
+    assert K % group == 0
     rng = np.random.default_rng(seed)
     w = rng.integers(0, 2**32, size=(N, K // 4), dtype=np.uint32)  # uniform bytes
-    s32 = rng.uniform(0.0003, 0.0012, size=(N, K // GROUP)).astype(np.float32)
+    s32 = rng.uniform(0.0003, 0.0012, size=(N, K // group)).astype(np.float32)
     s = f32_to_bf16_bits(s32)
-    z = rng.standard_normal(size=(N, K // GROUP)).astype(np.float32)
+    z = rng.standard_normal(size=(N, K // group)).astype(np.float32)
     b32 = np.float32(-128.0) * bf16_bits_to_f32(s) * (np.float32(1.0) + np.float32(0.05) * z)
     return w, s, f32_to_bf16_bits(b32)
 
