@@ -578,7 +578,15 @@ def main():
             dr = dense_route_us(w, s, b, x, y, K, N, M, 5)
             dit["%d->%d" % (K, N)]["dense_route_TFLOPs"] = round(flops / (dr[0] * 1e-6) / 1e12, 1)
             dit["%d->%d" % (K, N)]["dense_route_kept_expansion_TFLOPs"] = round(flops / (dr[1] * 1e-6) / 1e12, 1)
-            del w, s, b, x, y, A, B, t
+            # the same route with the adapter in the dense GEMM's accumulators (the bits of the fused call)
+            wdeq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+            drl = [steady_us(lambda: vpipe_amd.qmm_dense_route_w4g64(w, s, b, x, K, N, M, wdeq, expand=e, out=y, lora_A=A,
+                                                                     lora_B=B, r=r, alpha=alpha, t_ws=t), 5)
+                   for e in (True, False)]
+            dit["%d->%d" % (K, N)]["dense_route_with_lora_TFLOPs"] = round(flops / (drl[0] * 1e-6) / 1e12, 1)
+            dit["%d->%d" % (K, N)]["dense_route_kept_expansion_with_lora_TFLOPs"] = round(flops / (drl[1] * 1e-6) / 1e12, 1)
+            dit["%d->%d" % (K, N)]["us_dense_route_with_lora"] = round(drl[0], 1)
+            del w, s, b, x, y, A, B, t, wdeq
         out["qmm_dit_m16320_lora_r32"] = dit
         dit_flops = sum(2.0 * M * N * K for K, N in DIT)
         dit_us = sum(v["us"] for v in dit.values())
@@ -587,7 +595,9 @@ def main():
             "bound": "mfma", "achieved": round(dit_flops / (dit_us * 1e-6) / 1e12, 1), "peak": MFMA_BF16_PEAK_TF,
             "unit": "TFLOP/s", "frac": round(dit_flops / (dit_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TF, 4), "traffic": None,
             "achieved_with_lora_r32": round(dit_flops / (dit_us_lora * 1e-6) / 1e12, 1),
-            "kernel": "qmm_big_kernel<4,*,0> (256 x 256 tiles) + lora_a_kernel<1>; flops of the three base "
+            "achieved_with_lora_r32_dense_route": round(
+                dit_flops / (sum(v["us_dense_route_with_lora"] for v in dit.values()) * 1e-6) / 1e12, 1),
+            "kernel": "qmm_big_kernel<4,*,0> (256 x 256 tiles) + lora_a_dma_kernel; flops of the three base "
                       "contractions (2 M N K) over their time, the adapter's flops not counted",
             "timing": "us per call over 5 back-to-back calls after 40 ms of the same calls, events on the stream",
             "profile": "profiles/qmm_big_kernel_dit_m16320_lora_r32.txt (rocprofv3 kernel trace + MFMA busy)"}

@@ -221,6 +221,13 @@ int vpq_qmm_splitk_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint
 int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y,
                                    int K, int N, int M, uint16_t* w_deq, int expand);
+/* The same route with the runtime adapter of vpq_qmm_w4g64_bf16 (arguments and requirements of both): the pre-pass,
+ * the expansion (expand != 0) or the kept one, the dense GEMM with t . B^T in the same accumulators; the result has
+ * the bits of vpq_qmm_w4g64_bf16 with that adapter.  Worth it where the tiles are many (M in the thousands). */
+int vpq_qmm_dense_route_lora_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                        const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                        uint16_t* w_deq, int expand, const uint16_t* lora_a, const uint16_t* lora_b,
+                                        int r, float alpha, uint16_t* lora_t_ws);
 
 /* The adapter's first GEMM alone: t[M,r] = bf16(alpha * bf16(x . A^T)), r % 16 == 0, 16 <= r <= VPQ_LORA_MAX_RANK.
  * Replaces `lora_gemm_a_` (metal-minimax-h3-transformer.cc:1030-1067). */

@@ -284,6 +284,41 @@ def test_qmm_large_tile_kernel_with_lora(vpq, oracle, dev, D, r, tile_n):
     assert not torch.equal(base, got)
 
 
+@pytest.mark.parametrize("M,N,K,r", [(300, 450, 1024, 32), (64, 40, 192, 16), (2304, 4096, 512, 48), (130, 328, 1536, 384)])
+def test_dense_route_with_lora_is_the_fused_gemm(vpq, oracle, dev, D, M, N, K, r):
+    """The dequant-once route with the runtime adapter: the bits of the fused GEMM with the same adapter (whose
+    parity test_qmm_lora_fused holds) where the fused kernel runs the same tiles, the oracle's tolerance everywhere,
+    the kept expansion the same bits, the scratch the adapter's t, guard bands intact."""
+    alpha = 0.75
+    w, s, b = synth.make_weight(N, K, 7600 + r)
+    s[:] = synth.f32_to_bf16_bits(np.float32(0.0005))
+    b[:] = synth.f32_to_bf16_bits(np.float32(-0.004))
+    x = synth.make_act(M, K, 7601)
+    A, B = synth.make_lora(N, K, r, 7602, std=0.05)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    Ad, Bd = D.bf16(A, dev), D.bf16(B, dev)
+    w_deq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+    t_ws = parity.Guarded((M, r), torch.bfloat16, dev)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq, out=out.view, lora_A=Ad, lora_B=Bd, r=r, alpha=alpha, t_ws=t_ws.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    t_ws.assert_intact()
+    assert torch.equal(t_ws.view, vpq.lora_a(xd, Ad, M, K, r, alpha))
+    rows = np.arange(M) if M * N * K < 2e9 else np.r_[0:40, 1000:1024, M - 40:M]
+    y64, yb = oracle.qmm(w, s, b, x[rows], K, N, len(rows), t=D.bits(t_ws.view)[rows], B=B, r=r)
+    parity.check_bf16(D.bits(out.view)[rows], y64, yb)
+    if K % 512 == 0:
+        assert torch.equal(out.view, vpq.qmm_w4g64(wd, sd, bd, xd, K, N, M, lora_A=Ad, lora_B=Bd, r=r, alpha=alpha))
+    kept = vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq, expand=False, lora_A=Ad, lora_B=Bd, r=r, alpha=alpha)
+    assert torch.equal(kept, out.view)
+    assert not torch.equal(out.view, vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq))
+    L = vpq.load()
+    p = out.view.data_ptr()
+    assert L.vpq_qmm_dense_route_lora_w4g64_bf16(None, p, p, p, p, p, K, N, M, p, 1, p, p, 40, 1.0, p) == -2
+    assert L.vpq_qmm_dense_route_lora_w4g64_bf16(None, p, p, p, p, p, K, N, M, p, 1, p, p, r, 1.0, None) == -4
+
+
 def test_qmm_large_tile_kernel_refuses_what_it_cannot_take(vpq, dev, D):
     M, N, K = 64, 64, 576                                   # K not a multiple of 512
     w, s, b = synth.make_weight(N, K, 1)

@@ -63,6 +63,7 @@ SYMBOLS = [
     ("vpq_qmm_workspace_bytes", _sz, [_i, _i, _i]),
     ("vpq_qmm_splitk_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz]),
     ("vpq_qmm_dense_route_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
+    ("vpq_qmm_dense_route_lora_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _f, _vp]),
     ("vpq_lora_a_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _i, _f]),
     ("vpq_linear_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _sz]),
     ("vpq_qmv_group_w4g64_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i]),
@@ -780,14 +781,23 @@ def qmm_w4g64(w, scales, biases, x, K, N, M, out=None, lora_A=None, lora_B=None,
     return out
 
 
-def qmm_dense_route_w4g64(w, scales, biases, x, K, N, M, w_deq, expand=True, out=None):
-    """Dequant-once route: w_deq is bf16 [N,K] scratch (or the kept expansion when expand=False)."""
+def qmm_dense_route_w4g64(w, scales, biases, x, K, N, M, w_deq, expand=True, out=None, lora_A=None, lora_B=None, r=0,
+                          alpha=0.0, t_ws=None):
+    """Dequant-once route: w_deq is bf16 [N,K] scratch (or the kept expansion when expand=False); with lora_A / lora_B
+    the runtime adapter of qmm_w4g64 in the dense GEMM's accumulators."""
     import torch
     if out is None:
         out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
-    _check(load().vpq_qmm_dense_route_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
-                                                 K, N, M, _ptr(w_deq), 1 if expand else 0),
-           "vpq_qmm_dense_route_w4g64_bf16")
+    if lora_A is None:
+        _check(load().vpq_qmm_dense_route_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                                     K, N, M, _ptr(w_deq), 1 if expand else 0),
+               "vpq_qmm_dense_route_w4g64_bf16")
+        return out
+    if t_ws is None:
+        t_ws = torch.empty((M, r), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_dense_route_lora_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out),
+                                                      K, N, M, _ptr(w_deq), 1 if expand else 0, _ptr(lora_A), _ptr(lora_B),
+                                                      r, alpha, _ptr(t_ws)), "vpq_qmm_dense_route_lora_w4g64_bf16")
     return out
 
 

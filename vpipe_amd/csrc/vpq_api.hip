@@ -598,21 +598,45 @@ int vpq_qmm_dense_route_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const
                                    const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
                                    uint16_t* w_deq, int expand)
 {
+  return vpq_qmm_dense_route_lora_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, w_deq, expand, nullptr, nullptr, 0,
+                                             0.0f, nullptr);
+}
+
+// The dequant-once route with the runtime adapter: the pre-pass t = bf16(alpha * bf16(x . A^T)), the expansion (or the
+// kept one), then the dense GEMM with t . B^T in the same accumulators -- the bits of vpq_qmm_w4g64_bf16 with the
+// same adapter.
+int vpq_qmm_dense_route_lora_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                        const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                        uint16_t* w_deq, int expand, const uint16_t* lora_a, const uint16_t* lora_b,
+                                        int r, float alpha, uint16_t* lora_t_ws)
+{
   int st = check_pack(w, scales, biases, K, N);
   if (st != VPQ_OK) { return st; }
   if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
   if (w_deq == nullptr) { return VPQ_ERR_WORKSPACE; }
   if (M <= 0) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(y, 16) || !aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  const bool lora = lora_a != nullptr && alpha != 0.0f;
+  if (lora) {
+    if (lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
+    if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
+    if (r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (!aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) { return VPQ_ERR_MISALIGNED; }
+  }
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
   hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (lora) {
+    st = finish(vpq::launch_lora_a(hs, x, lora_a, lora_t_ws, M, K, r, alpha));
+    if (st != VPQ_OK) { return st; }
+  }
   if (expand != 0) {
     st = finish(vpq::launch_dequant(hs, w, scales, biases, w_deq, K, N));
     if (st != VPQ_OK) { return st; }
   }
   std::string why;
-  const int rc = vpq::dense_gemm_bf16(hs, x, w_deq, y, M, N, K, g_dev.cu_count, &why);
+  const int rc = vpq::dense_gemm_elt(hs, x, w_deq, y, M, N, K, false, g_dev.cu_count, &why, lora ? lora_t_ws : nullptr,
+                                     lora ? lora_b : nullptr, lora ? r : 0);
   if (rc != 0) {
     strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
     g_last_error[sizeof(g_last_error) - 1] = '\0';

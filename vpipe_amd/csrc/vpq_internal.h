@@ -251,11 +251,13 @@ hipError_t launch_qmm_tile_splitk(hipStream_t st, const GemmArgs& a, int splits,
 // fp32 accumulate, one rounding).  0, or -2 (shape outside the kernel / launch failed) with *why set.
 bool dense_gemm_supports(int M, int N, int K);
 hipError_t launch_dense_gemm(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,
-                             bool f16, int cu_count);
+                             bool f16, int cu_count, const uint16_t* lora_t = nullptr, const uint16_t* lora_b = nullptr,
+                             int r = 0);
 int dense_gemm_bf16(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, int cu_count,
                     std::string* why);
 int dense_gemm_elt(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, bool f16,
-                   int cu_count, std::string* why);
+                   int cu_count, std::string* why, const uint16_t* lora_t = nullptr, const uint16_t* lora_b = nullptr,
+                   int r = 0);
 // IEEE binary16 element type (the reference's VPIPE_ELT = half build): dense expansion and the general QMV.
 hipError_t launch_dequant_f16(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                               uint16_t* out, int K, int N);

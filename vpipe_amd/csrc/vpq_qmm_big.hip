@@ -966,21 +966,27 @@ bool dense_gemm_supports(int M, int N, int K)
          (double)BM * (double)K * 2.0 < 4.0e9;
 }
 
+// lora_t [M,r] / lora_b [N,r] (nullable together, bf16 only): the adapter's second factor in the same accumulators, as in
+// the fused kernel.
 hipError_t launch_dense_gemm(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K,
-                             bool f16, int cu_count)
+                             bool f16, int cu_count, const uint16_t* lora_t, const uint16_t* lora_b, int r)
 {
   if (!dense_gemm_supports(M, N, K)) { return hipErrorInvalidValue; }
+  const bool lora = lora_t != nullptr;
+  if (lora && (f16 || lora_b == nullptr || r < 16 || r % 16 != 0)) { return hipErrorInvalidValue; }
   const int bn = qmm_big_tile_n(N, M, cu_count);
   BigParams p{};
   p.w = reinterpret_cast<const uint32_t*>(b);
   p.x = x; p.y = y;
+  p.lora_t = lora_t; p.lora_b = lora_b; p.r = lora ? r : 0;
   p.K = K; p.N = N; p.M = M;
   p.tiles_m = (M + BM - 1) / BM;
   p.tiles_n = (N + bn - 1) / bn;
   const dim3 grid(plan_tile_order(p)), block(kBigThreads);
 #define VPQ_DENSE(NTV)                                                                      \
   (f16 ? launch_kernel(qmm_big_kernel<NTV, false, kDenseF16>, grid, block, 0, st, p)       \
-       : launch_kernel(qmm_big_kernel<NTV, false, kDenseBf16>, grid, block, 0, st, p))
+       : (lora ? launch_kernel(qmm_big_kernel<NTV, true, kDenseBf16>, grid, block, 0, st, p) \
+               : launch_kernel(qmm_big_kernel<NTV, false, kDenseBf16>, grid, block, 0, st, p)))
   if (bn == 128) { return VPQ_DENSE(2); }
   if (bn == 192) { return VPQ_DENSE(3); }
   return VPQ_DENSE(4);
@@ -993,13 +999,13 @@ hipError_t launch_dense_gemm(hipStream_t st, const uint16_t* x, const uint16_t* 
 // of traffic per call; here the caller may keep the expansion of an immutable weight.  0, or -2 with *why set
 // when the shape is outside the kernel or the launch failed.
 int dense_gemm_elt(hipStream_t st, const uint16_t* x, const uint16_t* b, uint16_t* y, int M, int N, int K, bool f16,
-                   int cu_count, std::string* why)
+                   int cu_count, std::string* why, const uint16_t* lora_t, const uint16_t* lora_b, int r)
 {
   if (!dense_gemm_supports(M, N, K)) {
     if (why) { *why = "dense GEMM: K must be a multiple of 32 and the matrices below 4 GB"; }
     return -2;
   }
-  const hipError_t e = launch_dense_gemm(st, x, b, y, M, N, K, f16, cu_count);
+  const hipError_t e = launch_dense_gemm(st, x, b, y, M, N, K, f16, cu_count, lora_t, lora_b, r);
   if (e != hipSuccess) {
     if (why) { *why = hipGetErrorString(e); }
     return -2;
