@@ -612,6 +612,21 @@ int vpq_qmm_tiled_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint1
  * 64 rows, vpq_qmm_w8g64_bf16 above. */
 int vpq_linear_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
                           const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M);
+/* `affine_requant_w8_to_w4_g64` (affine_dequant.metal:134-186): the half-width copy of an 8-bit pack (the draft
+ * lm_head of speculative decoding).  Per group of 64: v = s8 q8 + b8 in fp32, scale = (max - min) / 15, bias = min,
+ * q4 = round-half-away((v - min) / scale) clamped to 0..15 (a constant group: scale 0, codes 0); s4 / b4 are the bf16
+ * roundings, the codes use the unrounded fp32 scale.  w8 uint32 [N, K/4], s8 / b8 bf16 [N, K/64] in; w4 uint32
+ * [N, K/8], s4 / b4 bf16 [N, K/64] out; K % 64 == 0, w8 and w4 16-byte aligned.  Bit-exact with IEEE division. */
+int vpq_requant_w8_to_w4_g64_bf16(vpq_stream_t stream, const uint32_t* w8, const uint16_t* s8, const uint16_t* b8,
+                                  uint32_t* w4, uint16_t* s4, uint16_t* b4, int K, int N);
+/* The 8-bit and group-32 twins of vpq_qmv_gelu_mul_w4g64_bf16: `affine_qmv_gelu_mul_w8g64` (affine_qmv.metal:788-805)
+ * and `affine_qmv_gelu_mul_w4g32` (:769-786; scale_only as in vpq_qmv_w4g32_bf16). */
+int vpq_qmv_gelu_mul_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                const uint16_t* mul);
+int vpq_qmv_gelu_mul_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
+                                const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N,
+                                const uint16_t* mul, int scale_only);
 /* 8-bit codes in groups of 32 (GGUF q8 repacked to affine; the codec's int8 path): w uint32 [N, K/4], scales / biases
  * bf16 [N, K/32], K % 32 == 0.  vpq_dequant_w8g32_bf16 replaces `affine_dequant_w8g32` (affine_dequant.metal:99-131),
  * bit-exact; vpq_qmv_w8g32_bf16 replaces `affine_qmv_w8g32` (affine_qmv.metal:3053-3069), QMV arithmetic, 1 <= M <= 16;

@@ -374,6 +374,17 @@ def dequant8_g32(w, s, b, K, N):
     return out
 
 
+def requant_w8_to_w4(w8, s8, b8, K, N):
+    """8-bit group-64 pack -> 4-bit group-64 pack (codes u32 [N, K/8], scales, biases bf16 bits [N, K/64])."""
+    w8, s8, b8 = _c(w8, np.uint32), _c(s8, np.uint16), _c(b8, np.uint16)
+    w4 = np.empty((N, K // 8), dtype=np.uint32)
+    s4 = np.empty((N, K // 64), dtype=np.uint16)
+    b4 = np.empty((N, K // 64), dtype=np.uint16)
+    lib().vpo_requant_w8_to_w4_g64(_p(w8, _u32p), _p(s8, _u16p), _p(b8, _u16p), _p(w4, _u32p), _p(s4, _u16p),
+                                   _p(b4, _u16p), K, N)
+    return w4, s4, b4
+
+
 def quantize(wsrc, K, N, clip=1.0):
     """fp32 [N,K] -> (codes u32 [N,K/8], scales f16 bits [N,K/64], biases f16 bits)."""
     wsrc = _c(wsrc, np.float32)

@@ -28,6 +28,10 @@
  *                          activations, float64 matmul
  *   quantize (packer)      exact recovery of on-grid data, the reference's
  *                          round-trip error bounds, numpy re-derivation
+ *   requantizer (8 -> 4)   bytes 17 c requantize to the nibbles c in k order (byte / nibble
+ *                          order, word layout), constant group, codes 0 and 15 used in every
+ *                          group, half-step reconstruction bound, vectorized numpy statement
+ *                          (the last bit of Metal's fast division is not pinned)
  * Parity that only an Apple-GPU run could pin -- the last-bit effect of the
  * Metal kernels' summation order (simd_sum tree, steel BlockMMA K order,
  * matmul2d) -- is NOT pinned: the oracle accumulates in double instead, and
@@ -1059,6 +1063,46 @@ void vpo_dequant_w8_bf16(const uint32_t* w, const uint16_t* scales, const uint16
       const float b = vpo_bf16_to_f32(biases[n * Kg + k / group]);
       const float sq = s * (float)code8(w, n, Kw, k);
       out[n * (size_t)K + k] = vpo_f32_to_bf16(sq + b);
+    }
+  }
+}
+
+/* affine_requant_w8_to_w4_g64 (affine_dequant.metal:134-186): per group of 64, expand the 8-bit codes to fp32
+ * (v = s8 * q8 + b8, the product exact), take min and max, and quantize again to 4 bits with
+ * scale = (max - min) / 15, bias = min, q4 = round((v - min) * (1 / scale)) (halves away from zero, as Metal's
+ * round) clamped to 0..15; a constant group gives scale 0 and all codes 0.  The stored scale and bias are the
+ * element-type roundings; the codes are computed with the unrounded fp32 scale.  Divisions are IEEE here (Metal's
+ * default fast division may differ in the last bit: only an Apple-GPU run could pin that bit). */
+void vpo_requant_w8_to_w4_g64(const uint32_t* w8, const uint16_t* s8, const uint16_t* b8,
+                              uint32_t* w4, uint16_t* s4, uint16_t* b4, int K, int N)
+{
+  const int Kw8 = K / 4, Kw4 = K / 8, Kg = K / VPO_GROUP;
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int g = 0; g < Kg; ++g) {
+      const float s = vpo_bf16_to_f32(s8[n * Kg + g]);
+      const float b = vpo_bf16_to_f32(b8[n * Kg + g]);
+      float v[VPO_GROUP];
+      float mn = INFINITY, mx = -INFINITY;
+      for (int i = 0; i < VPO_GROUP; ++i) {
+        const float sq = s * (float)code8(w8, n, Kw8, g * VPO_GROUP + i);
+        v[i] = sq + b;
+        mn = v[i] < mn ? v[i] : mn;
+        mx = v[i] > mx ? v[i] : mx;
+      }
+      const float scale = (mx - mn) / 15.0f;
+      const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+      s4[n * Kg + g] = vpo_f32_to_bf16(scale);
+      b4[n * Kg + g] = vpo_f32_to_bf16(mn);
+      for (int wi = 0; wi < VPO_GROUP / 8; ++wi) {
+        uint32_t packed = 0;
+        for (int i = 0; i < 8; ++i) {
+          const float d = v[wi * 8 + i] - mn;
+          int q = (int)roundf(d * inv);
+          q = q < 0 ? 0 : (q > 15 ? 15 : q);
+          packed |= (uint32_t)q << (4 * i);
+        }
+        w4[n * Kw4 + (size_t)g * (VPO_GROUP / 8) + wi] = packed;
+      }
     }
   }
 }

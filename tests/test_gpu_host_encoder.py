@@ -1003,6 +1003,69 @@ def test_gelu_mul_and_shared_expert_gate_function_names(vpq, enc, dev, D):
     assert y.abs().sum() > 0 and gate.float().std() > 0
 
 
+def test_requantizer_gelu_mul_twins_and_variant_names(vpq, enc, dev, D):
+    # affine_requant_w8_to_w4_g64 (0:w8 1:s8 2:b8 3:w4 4:s4 5:b4 6:K 7:N), the gelu-mul twins (the slots of the
+    # group-64 4-bit form), and the names the reference keeps for tiling / accumulator variants of the same
+    # mathematics: all are the C ABI's results, bit for bit
+    K, N = 1024, 48
+    w8, s8, b8 = synth.make_weight8(N, K, 4200)
+    wd, sd, bd = D.u32(w8, dev), D.bf16(s8, dev), D.bf16(b8, dev)
+    w4 = torch.zeros((N, K // 8), dtype=torch.int32, device=dev)
+    s4 = torch.zeros((N, K // 64), dtype=torch.bfloat16, device=dev)
+    b4 = torch.zeros((N, K // 64), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_dequant_bf16", "affine_requant_w8_to_w4_g64") == 1
+    for i, t in enumerate((wd, sd, bd, w4, s4, b4)):
+        enc.set_buffer(i, t)
+    enc.set_constant(6, K)
+    enc.set_constant(7, N)
+    enc.dispatch((K // 64, N, 1), (K // 64, 1, 1))
+    x = D.bf16(synth.make_act(1, K, 4201), dev)
+    mul = D.bf16(synth.make_act(1, N, 4202), dev)
+    y8 = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_gelu_mul_w8g64") == 1
+    for i, t in enumerate((wd, sd, bd, x, y8)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.set_buffer(7, mul)
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    g = synth.make_weight_g32(N, K, 4203)
+    gd = (D.u32(g[0], dev), D.bf16(g[1], dev), D.bf16(g[2], dev))
+    y32 = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_gelu_mul_w4g32") == 1
+    for i, t in enumerate(gd + (x, y32)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.set_buffer(7, mul)
+    enc.dispatch((32, N // 4, 1), (32, 2, 1))
+    yv = torch.zeros((1, N), dtype=torch.bfloat16, device=dev)
+    assert enc.set_function("affine_qmv_bf16", "affine_qmv_w8g64_r8p2") == 1
+    for i, t in enumerate((wd, sd, bd, x, yv)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.dispatch((1, N // 16, 1), (32, 2, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    want = vpq.requant_w8_to_w4(wd, sd, bd, K, N)
+    assert torch.equal(w4, want[0]) and torch.equal(s4, want[1]) and torch.equal(b4, want[2])
+    assert torch.equal(y8, vpq.qmv_gelu_mul_w8g64(wd, sd, bd, x, K, N, mul))
+    assert torch.equal(y32, vpq.qmv_gelu_mul_w4g32(*gd, x, K, N, mul))
+    assert torch.equal(yv, vpq.qmv_w8g64(wd, sd, bd, x, K, N, 1))
+    assert w4.abs().sum() > 0 and y8.abs().sum() > 0 and y32.abs().sum() > 0
+    for lib, name in [("affine_qmv_bf16", "affine_qmv_w4g64_r8p2"), ("affine_qmm", "affine_qmm_w4g64"),
+                      ("affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm64_acc16"),
+                      ("affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_acc16"),
+                      ("affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64_acc16"),
+                      ("affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64_rs_acc16"),
+                      ("affine_qmm_steel_bf16", "affine_qmm_steel_w8g64_bm64_acc16"),
+                      ("affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_acc16"),
+                      ("affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_bm64_acc16"),
+                      ("affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_bm64_rs_acc16")]:
+        assert enc.set_function(lib, name) == 1, name
+
+
 @pytest.mark.parametrize("name", ["affine_qmv_qkv_w8g64", "affine_qmv_qkv_w4g32"])
 def test_fused_qkv_call_sites_of_the_format_twins(vpq, enc, dev, D, name):
     # gpu-kernels/metal/quant/affine_qmv.metal:518-559: the slots of affine_qmv_qkv_w4g64 over the 8-bit and the

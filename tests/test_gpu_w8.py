@@ -477,3 +477,59 @@ def test_w8g32_dequant_qmv_and_dense_route(vpq, oracle, dev, D, K, N, M):
     p = out.view.data_ptr()
     assert L.vpq_qmv_w8g32_bf16(None, p, p, p, p, p, K + 8, N, M, None) == -2
     assert L.vpq_qmm_dense_route_w8g32_bf16(None, p, p, p, p, p, K, N, M, None, 1) == -4
+
+
+@pytest.mark.parametrize("N,K", [(1, 64), (37, 320), (512, 4096), (1000, 2048)])
+def test_requant_w8_to_w4_bit_exact(vpq, oracle, dev, D, N, K):
+    """affine_requant_w8_to_w4_g64 (gpu-kernels/metal/quant/affine_dequant.metal:134-186): codes, scales and biases of
+    the 4-bit copy, bit for bit against the oracle; one group of the pack is made constant (scale 0, codes 0)."""
+    w8, s8, b8 = synth.make_weight8(N, K, 5200 + N + K)
+    w8[N // 2, :16] = 0x3C3C3C3C
+    want = oracle.requant_w8_to_w4(w8, s8, b8, K, N)
+    wd, sd, bd = stage(D, dev, w8, s8, b8)
+    w4, s4, b4 = vpq.requant_w8_to_w4(wd, sd, bd, K, N)
+    torch.cuda.synchronize()
+    assert np.array_equal(w4.cpu().numpy().view(np.uint32), want[0])
+    assert np.array_equal(D.bits(s4), want[1]) and np.array_equal(D.bits(b4), want[2])
+    assert want[1][N // 2, 0] == 0 and not want[0][N // 2, :8].any()
+    # the copy is a pack of the 4-bit kernels: its expansion stays within half a step (+ the roundings of the stored
+    # scale and bias and of both expansions) of the 8-bit one
+    d8 = synth.bf16_bits_to_f32(D.bits(vpq.dequant_w8g64(wd, sd, bd, K, N))).astype(np.float64)
+    d4 = synth.bf16_bits_to_f32(D.bits(vpq.dequant_w4g64(w4, s4, b4, K, N))).astype(np.float64)
+    step = np.repeat(synth.bf16_bits_to_f32(want[1]).astype(np.float64), 64, axis=1)
+    assert (np.abs(d4 - d8) <= 0.5 * step + 2.0 ** -7 * (np.abs(d8) + 15 * step)).all()
+    L = vpq.load()
+    p = wd.data_ptr()
+    assert L.vpq_requant_w8_to_w4_g64_bf16(None, p, p, p, p, p, None, K, N) == -1
+    assert L.vpq_requant_w8_to_w4_g64_bf16(None, p, p, p, p, p, p, K + 32, N) == -2
+    assert L.vpq_requant_w8_to_w4_g64_bf16(None, p, p, p, p + 4, p, p, K, N) == -3
+
+
+@pytest.mark.parametrize("K,N", [(4096, 300), (192, 10), (1024, 33)])
+@pytest.mark.parametrize("fmt", ["w8g64", "w4g32"])
+def test_qmv_gelu_mul_twins(vpq, oracle, dev, D, K, N, fmt):
+    """affine_qmv_gelu_mul_w8g64 / affine_qmv_gelu_mul_w4g32 (gpu-kernels/metal/quant/affine_qmv.metal:769-805): the
+    store of the group-64 4-bit form on the twins' GEMV.  The fused store against the oracle's gelu_tanh(v) * mul on
+    the device's own GEMV output v (whose parity other tests hold)."""
+    w, s, b = synth.make_weight8(N, K, 5300 + K + N) if fmt == "w8g64" else synth.make_weight_g32(N, K, 5301 + K + N)
+    x = synth.make_act(1, K, 5302 + K)
+    mul = synth.make_act(1, N, 5303 + N)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    plain = vpq.qmv_w8g64 if fmt == "w8g64" else vpq.qmv_w4g32
+    fused = vpq.qmv_gelu_mul_w8g64 if fmt == "w8g64" else vpq.qmv_gelu_mul_w4g32
+    v_bits = D.bits(plain(wd, sd, bd, xd, K, N, 1))
+    pairs = np.stack([synth.bf16_bits_to_f32(v_bits[0]).astype(np.float64),
+                      synth.bf16_bits_to_f32(mul[0]).astype(np.float64)], axis=1).reshape(1, 2 * N)
+    o64, ob = oracle.geglu(pairs)
+    out = parity.Guarded((1, N), torch.bfloat16, dev)
+    fused(wd, sd, bd, xd, K, N, D.bf16(mul, dev), out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    parity.check_bf16(D.bits(out.view), o64, ob, mismatch_over_all=False)
+    assert np.abs(o64).max() > 0
+    L = vpq.load()
+    p = out.view.data_ptr()
+    if fmt == "w8g64":
+        assert L.vpq_qmv_gelu_mul_w8g64_bf16(None, p, p, p, p, p, K, N, None) == -1
+    else:
+        assert L.vpq_qmv_gelu_mul_w4g32_bf16(None, p, p, p, p, p, K, N, None, 0) == -1

@@ -687,6 +687,56 @@ def test_w8g32_twins_against_numpy_and_the_group64_oracle(oracle):
     assert np.array_equal(a64, c64) and np.array_equal(ab, cb)
 
 
+def test_requantizer_known_answers_invariants_and_numpy(oracle):
+    """affine_requant_w8_to_w4_g64 (gpu-kernels/metal/quant/affine_dequant.metal:134-186).  (a) A pack whose bytes are
+    17 c (c a nibble, 0 and 15 both present in every group) with power-of-two scale requantizes to exactly the nibbles
+    c in k order, scale 17 s and the same bias: pins the byte -> nibble order and the word layout.  (b) A constant
+    group: scale 0, codes 0, bias = the value.  (c) On a random pack: every group uses code 0 and code 15, the
+    reconstruction with the unrounded scale is within half a step, and the whole agrees with a vectorized numpy
+    statement written from the layout."""
+    rng = np.random.default_rng(91)
+    N, K = 5, 256
+    c = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    c.reshape(N, K // 64, 64)[:, :, 3] = 0
+    c.reshape(N, K // 64, 64)[:, :, 40] = 15
+    w8 = (c * 17).astype(np.uint8).view(np.uint32).reshape(N, K // 4)
+    s8 = synth.f32_to_bf16_bits(np.full((N, K // 64), 2.0 ** -6, np.float32))
+    b8 = synth.f32_to_bf16_bits(np.full((N, K // 64), -1.0, np.float32))
+    w4, s4, b4 = oracle.requant_w8_to_w4(w8, s8, b8, K, N)
+    nib = ((w4[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF).reshape(N, K).astype(np.uint8)
+    assert np.array_equal(nib, c)
+    assert np.array_equal(s4, synth.f32_to_bf16_bits(np.full((N, K // 64), 17.0 * 2.0 ** -6, np.float32)))
+    assert np.array_equal(b4, b8)
+    # (b)
+    w8c = np.full((1, 16), 0x5A5A5A5A, np.uint32)
+    s1 = synth.f32_to_bf16_bits(np.array([[0.25]], np.float32))
+    b1 = synth.f32_to_bf16_bits(np.array([[-3.0]], np.float32))
+    w4c, s4c, b4c = oracle.requant_w8_to_w4(w8c, s1, b1, 64, 1)
+    assert not w4c.any() and s4c[0, 0] == 0
+    assert b4c[0, 0] == synth.f32_to_bf16_bits(np.array([0.25 * 0x5A - 3.0], np.float32))[0]
+    # (c)
+    N, K = 13, 320
+    w8, s8, b8 = synth.make_weight8(N, K, 92)
+    w4, s4, b4 = oracle.requant_w8_to_w4(w8, s8, b8, K, N)
+    q8 = w8.view(np.uint8).reshape(N, K // 64, 64).astype(np.float32)
+    v = synth.bf16_bits_to_f32(s8)[:, :, None] * q8 + synth.bf16_bits_to_f32(b8)[:, :, None]
+    assert v.dtype == np.float32
+    mn, mx = v.min(axis=2, keepdims=True), v.max(axis=2, keepdims=True)
+    scale = (mx - mn) / np.float32(15.0)
+    inv = np.float32(1.0) / scale
+    t = (v - mn) * inv
+    fl = np.floor(t)
+    q4 = np.clip(np.where(t - fl >= np.float32(0.5), fl + 1, fl), 0, 15).astype(np.uint32)   # halves away from zero (t >= 0); t - fl is exact
+    assert (t - fl == np.float32(0.5)).any()                       # exact halves occur, so the tie rule is exercised
+    nib = ((w4[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF).reshape(N, K // 64, 64)
+    assert np.array_equal(nib, q4)
+    assert np.array_equal(s4, synth.f32_to_bf16_bits(scale[:, :, 0]))
+    assert np.array_equal(b4, synth.f32_to_bf16_bits(mn[:, :, 0]))
+    assert (nib.min(axis=2) == 0).all() and (nib.max(axis=2) == 15).all()
+    recon = mn.astype(np.float64) + scale.astype(np.float64) * nib
+    assert (np.abs(recon - v) <= 0.5 * scale * (1 + 1e-5)).all()
+
+
 def test_grouped_gemm_oracle_with_byte_codes_reduces_to_the_plain_8bit_gemm(oracle):
     """The 8-bit form of the grouped restatement: every live slot equals the plain 8-bit GEMM oracle
     (bf16-rounded weights) of its row on its expert's slab."""

@@ -73,6 +73,9 @@ SYMBOLS = [
     ("vpq_rmsnorm_bf16", _i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
     ("vpq_dequant_w8g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i]),
     ("vpq_qmv_w8g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    ("vpq_requant_w8_to_w4_g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_qmv_gelu_mul_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    ("vpq_qmv_gelu_mul_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i]),
     ("vpq_qmm_dense_route_w8g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_qmv_qkv_rms_bf16", _i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _f, _vp]),
     ("vpq_interleave_rows", _i, [_vp, _vp, _vp, _vp, _sz, _sz]),
@@ -689,6 +692,38 @@ def qmv_gelu_mul_w4g64(w, scales, biases, x, K, N, mul, out=None):
     _check(load().vpq_qmv_gelu_mul_w4g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
                                               _ptr(mul)), "vpq_qmv_gelu_mul_w4g64_bf16")
     return out
+
+
+def qmv_gelu_mul_w8g64(w, scales, biases, x, K, N, mul, out=None):
+    """The 8-bit twin of qmv_gelu_mul_w4g64."""
+    import torch
+    if out is None:
+        out = torch.empty((1, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmv_gelu_mul_w8g64_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                              _ptr(mul)), "vpq_qmv_gelu_mul_w8g64_bf16")
+    return out
+
+
+def qmv_gelu_mul_w4g32(w, scales, biases, x, K, N, mul, out=None, scale_only=False):
+    """The group-32 twin of qmv_gelu_mul_w4g64."""
+    import torch
+    if out is None:
+        out = torch.empty((1, N), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmv_gelu_mul_w4g32_bf16(_stream(), _ptr(w), _ptr(scales), _ptr(biases) if biases is not None else None,
+                                              _ptr(x), _ptr(out), K, N, _ptr(mul), int(scale_only)),
+           "vpq_qmv_gelu_mul_w4g32_bf16")
+    return out
+
+
+def requant_w8_to_w4(w8, s8, b8, K, N):
+    """8-bit group-64 pack -> (w4 uint32 [N, K/8] viewed as int32, s4, b4 bf16 [N, K/64])."""
+    import torch
+    w4 = torch.empty((N, K // 8), dtype=torch.int32, device=w8.device)
+    s4 = torch.empty((N, K // 64), dtype=torch.bfloat16, device=w8.device)
+    b4 = torch.empty((N, K // 64), dtype=torch.bfloat16, device=w8.device)
+    _check(load().vpq_requant_w8_to_w4_g64_bf16(_stream(), _ptr(w8), _ptr(s8), _ptr(b8), _ptr(w4), _ptr(s4), _ptr(b4),
+                                                K, N), "vpq_requant_w8_to_w4_g64_bf16")
+    return w4, s4, b4
 
 
 def moe_gate_w8g64(w, scales, biases, x, K, M, out=None):

@@ -230,11 +230,12 @@ int vpq_dequant_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_
 }
 
 static int qmv8_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                       const uint16_t* x, void* y, bool y_f32, int K, int N, int M, const uint16_t* residual)
+                       const uint16_t* x, void* y, bool y_f32, int K, int N, int M, const uint16_t* residual,
+                       int store = 0)
 {
   int st = check_pack(w, scales, biases, K, N);
   if (st != VPQ_OK) { return st; }
-  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (x == nullptr || y == nullptr || (store == vpq::kStoreGeluMul && residual == nullptr)) { return VPQ_ERR_NULL_POINTER; }
   if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2) || (residual != nullptr && !aligned(residual, 2))) {
     return VPQ_ERR_MISALIGNED;
@@ -244,6 +245,7 @@ static int qmv8_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* s
   vpq::QmvArgs a{};
   a.w = w; a.scales = scales; a.biases = biases; a.x = x; a.y = y; a.residual = residual;
   a.K = K; a.N = N; a.M = M; a.y_f32 = y_f32; a.cu_count = g_dev.cu_count;
+  a.gate_act = store;
   return finish(vpq::launch_qmv_simple8(reinterpret_cast<hipStream_t>(stream), a));
 }
 
@@ -257,6 +259,12 @@ int vpq_qmv_w8g64_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t*
                          const uint16_t* x, float* y, int K, int N, int M)
 {
   return qmv8_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr);
+}
+
+int vpq_qmv_gelu_mul_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                                const uint16_t* x, uint16_t* y, int K, int N, const uint16_t* mul)
+{
+  return qmv8_common(stream, w, scales, biases, x, y, false, K, N, 1, mul, vpq::kStoreGeluMul);
 }
 
 int vpq_moe_gate_w8g64_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
@@ -398,6 +406,18 @@ int vpq_dequant_w8g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_
   st = ensure_init();
   if (st != VPQ_OK) { return st; }
   return finish(vpq::launch_dequant8(reinterpret_cast<hipStream_t>(stream), w, scales, biases, w_deq, K, N, 32));
+}
+
+int vpq_requant_w8_to_w4_g64_bf16(vpq_stream_t stream, const uint32_t* w8, const uint16_t* s8, const uint16_t* b8,
+                                  uint32_t* w4, uint16_t* s4, uint16_t* b4, int K, int N)
+{
+  int st = check_pack(w8, s8, b8, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (w4 == nullptr || s4 == nullptr || b4 == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (!aligned(w4, 16) || !aligned(s4, 2) || !aligned(b4, 2)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_requant_w8_to_w4(reinterpret_cast<hipStream_t>(stream), w8, s8, b8, w4, s4, b4, K, N));
 }
 
 int vpq_qmv_w8g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
@@ -1343,7 +1363,9 @@ int qmv_g32_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scale
   if (st != VPQ_OK) { return st; }
   if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
   if (M < 1 || M > 16) { return VPQ_ERR_BAD_SHAPE; }
-  if (gate_act != 0 && ((N & 1) != 0 || residual != nullptr)) { return VPQ_ERR_BAD_SHAPE; }
+  const bool gelu_mul = gate_act == vpq::kStoreGeluMul;       // `residual` is the multiplier [N]
+  if (gelu_mul && residual == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (gate_act != 0 && !gelu_mul && ((N & 1) != 0 || residual != nullptr)) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(y, y_f32 ? 4 : 2) || (residual != nullptr && !aligned(residual, 2))) {
     return VPQ_ERR_MISALIGNED;
   }
@@ -1354,6 +1376,7 @@ int qmv_g32_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scale
   a.K = K; a.N = N; a.M = M; a.y_f32 = y_f32; a.cu_count = g_dev.cu_count;
   a.gate_act = gate_act;
   hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (gelu_mul) { return finish(vpq::launch_qmv_simple_g32(hs, a, scale_only)); }    // the kernel that has this store
   // up to two rows of x: the row-streaming kernel; more: one wavefront per weight row
   if (M <= 2) { return finish(vpq::launch_qmv_rows_g32(hs, a, scale_only)); }
   return finish(vpq::launch_qmv_simple_g32(hs, a, scale_only));
@@ -1383,6 +1406,12 @@ int vpq_qmv_w4g32_f32out(vpq_stream_t stream, const uint32_t* w, const uint16_t*
                          const uint16_t* x, float* y, int K, int N, int M, int scale_only)
 {
   return qmv_g32_common(stream, w, scales, biases, x, y, true, K, N, M, nullptr, 0, scale_only != 0);
+}
+
+int vpq_qmv_gelu_mul_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                                const uint16_t* x, uint16_t* y, int K, int N, const uint16_t* mul, int scale_only)
+{
+  return qmv_g32_common(stream, w, scales, biases, x, y, false, K, N, 1, mul, vpq::kStoreGeluMul, scale_only != 0);
 }
 
 int vpq_qmv_gated_w4g32_bf16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,

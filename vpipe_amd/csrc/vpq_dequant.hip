@@ -108,6 +108,70 @@ hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* sc
                        reinterpret_cast<uint2*>(out), Kw, total);
 }
 
+// 8-bit -> 4-bit requantizer (affine_requant_w8_to_w4_g64, gpu-kernels/metal/quant/affine_dequant.metal:134-186): one
+// thread per group of 64.  The group's 64 bytes come in as four 128-bit loads requested together; values are
+// v = s8 * q8 + b8 in fp32 (the product is exact), scale = (max - min) / 15 and 1 / scale by IEEE division,
+// q4 = round-half-away((v - min) / scale) clamped to 0..15, a constant group gives scale 0 and codes 0.  Stored
+// scale / bias: bf16 roundings of scale and min.  A load-time kernel (it builds the half-width copy of an lm_head),
+// bound by the 64 + 4 bytes read and 32 + 4 written per group.
+__global__ __launch_bounds__(256) void requant_w8_to_w4_kernel(
+    const uint4* __restrict__ w8, const uint16_t* __restrict__ s8, const uint16_t* __restrict__ b8,
+    uint4* __restrict__ w4, uint16_t* __restrict__ s4, uint16_t* __restrict__ b4, size_t groups)
+{
+  for (size_t g = (size_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (size_t)gridDim.x * 256) {
+    uint4 c[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { c[i] = w8[g * 4 + i]; }
+    const float s = bf16_bits_to_f32(s8[g]);
+    const float b = bf16_bits_to_f32(b8[g]);
+    float v[64];
+    float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t words[4] = {c[i].x, c[i].y, c[i].z, c[i].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float val = fmaf(s, (float)((words[j] >> (8 * k)) & 0xffu), b);
+          v[16 * i + 4 * j + k] = val;
+          mn = fminf(mn, val);
+          mx = fmaxf(mx, val);
+        }
+      }
+    }
+    const float scale = (mx - mn) / 15.0f;
+    const float inv = scale > 0.0f ? 1.0f / scale : 0.0f;
+    s4[g] = (uint16_t)f32_to_bf16_bits(scale);
+    b4[g] = (uint16_t)f32_to_bf16_bits(mn);
+    uint32_t out[8];
+#pragma unroll
+    for (int wi = 0; wi < 8; ++wi) {
+      uint32_t packed = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float d = v[wi * 8 + i] - mn;
+        int q = (int)roundf(d * inv);
+        q = q < 0 ? 0 : (q > 15 ? 15 : q);
+        packed |= (uint32_t)q << (4 * i);
+      }
+      out[wi] = packed;
+    }
+    w4[g * 2] = make_uint4(out[0], out[1], out[2], out[3]);
+    w4[g * 2 + 1] = make_uint4(out[4], out[5], out[6], out[7]);
+  }
+}
+
+hipError_t launch_requant_w8_to_w4(hipStream_t st, const uint32_t* w8, const uint16_t* s8, const uint16_t* b8,
+                                   uint32_t* w4, uint16_t* s4, uint16_t* b4, int K, int N)
+{
+  const size_t groups = (size_t)N * (size_t)(K / 64);
+  size_t blocks = (groups + 255) / 256;
+  if (blocks > 65536 * 4) { blocks = 65536 * 4; }
+  return launch_kernel(requant_w8_to_w4_kernel, dim3((unsigned)blocks), dim3(256), 0, st,
+                       reinterpret_cast<const uint4*>(w8), s8, b8, reinterpret_cast<uint4*>(w4), s4, b4, groups);
+}
+
 // Dequantizing embedding gather (gpu-kernels/metal/ops/llm_elementwise.metal:1676-1701): out row t
 // is the dense expansion of table row ids[t]; the arithmetic is the dequant kernel's, so a
 // gathered row is bit-identical to that row of the dense table.  One thread per packed word.

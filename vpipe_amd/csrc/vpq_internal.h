@@ -143,6 +143,9 @@ hipError_t launch_qmv_rows_g32(hipStream_t st, const QmvArgs& a, bool scale_only
 hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                            uint16_t* out, int K, int N, int group = 64);
 hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a, int group = 64);
+// 8-bit group-64 pack -> 4-bit group-64 pack of the same shape (one thread per group).
+hipError_t launch_requant_w8_to_w4(hipStream_t st, const uint32_t* w8, const uint16_t* s8, const uint16_t* b8,
+                                   uint32_t* w4, uint16_t* s4, uint16_t* b4, int K, int N);
 // Mixed-width fused gate/up over separate packs (4 or 8 bits each); rows = pairs (pair_eid) or rows of x.
 struct SplitGateUp {
   const uint32_t* wg; const uint16_t* sg; const uint16_t* bg; int gate_bits;

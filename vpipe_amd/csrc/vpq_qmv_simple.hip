@@ -150,12 +150,13 @@ hipError_t launch_qmv_simple_g32(hipStream_t st, const QmvArgs& a, bool scale_on
 // 8-bit twin (affine_qmv_w8g64, gpu-kernels/metal/quant/affine_qmv.metal:3034-3050): one byte per
 // value.  Each lane takes 16 consecutive k (one 128-bit load of codes, a quarter of a group) per
 // pass over the row; otherwise the kernel above: W = fma(s, q, b) in fp32, never rounded.  GS: log2 of the group
-// (6, or 5 for affine_qmv_w8g32, :3053-3069).
+// (6, or 5 for affine_qmv_w8g32, :3053-3069).  store == kStoreGeluMul: affine_qmv_gelu_mul_w8g64 (:789-805),
+// `residual` is then the multiplier [N].
 template <int MT, bool F32OUT, int GS = 6>
 __global__ __launch_bounds__(256) void qmv_simple8_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ x, void* __restrict__ y,
-    const uint16_t* __restrict__ residual, int K, int N, int M)
+    const uint16_t* __restrict__ residual, int K, int N, int M, int store)
 {
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -207,7 +208,9 @@ __global__ __launch_bounds__(256) void qmv_simple8_kernel(
           reinterpret_cast<float*>(y)[o] = total;
         } else {
           uint32_t v = f32_to_bf16_bits(total);
-          if (residual != nullptr) {
+          if (store == kStoreGeluMul) {          // `residual` is the multiplier, one value per output feature
+            v = f32_to_bf16_bits(gelu_mul_f32(bf16_bits_to_f32(v), bf16_bits_to_f32(residual[n])));
+          } else if (residual != nullptr) {
             v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(residual[o]));
           }
           reinterpret_cast<uint16_t*>(y)[o] = (uint16_t)v;
@@ -502,7 +505,7 @@ hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a, int group)
   const dim3 grid((unsigned)((a.N + 3) / 4)), block(256);
 #define VPQ_LAUNCH8(MT, F32, GS)                                                                    \
   launch_kernel(qmv_simple8_kernel<MT, F32, GS>, grid, block, 0, st, a.w, a.scales, a.biases, a.x, a.y, \
-                a.residual, a.K, a.N, a.M)
+                a.residual, a.K, a.N, a.M, a.gate_act)
   if (group == 32) {
     if (a.M == 1) { return a.y_f32 ? VPQ_LAUNCH8(1, true, 5) : VPQ_LAUNCH8(1, false, 5); }
     return a.y_f32 ? VPQ_LAUNCH8(4, true, 5) : VPQ_LAUNCH8(4, false, 5);

@@ -116,6 +116,25 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_w8g64", QuantKernel::Qmv, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_w8g64_add", QuantKernel::QmvAdd, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_moe_gate_w8g64", QuantKernel::MoeGate, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_gelu_mul_w8g64", QuantKernel::QmvGeluMul, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_gelu_mul_w4g32", QuantKernel::QmvGeluMul, QuantFormat::W4G32},
+    {"affine_dequant_bf16", "affine_requant_w8_to_w4_g64", QuantKernel::Requant84, QuantFormat::W8G64},
+    // Tiling variants the reference keeps beside its defaults (affine_qmv.metal:3072-3118: rows per simdgroup / packs
+    // per thread of the same GEMV) and its plain QMM (affine_qmm.metal:64-174): the same mathematics, served by the
+    // same kernels (the plain QMM exists in the binary16 build only).  The `_acc16` GEMMs accumulate in fp32 in the
+    // bf16 library (affine_qmm_steel.metal:50-56), so there they are the base functions under another name; the
+    // binary16 library's half accumulation is not served.
+    {"affine_qmv_bf16", "affine_qmv_w4g64_r8p2", QuantKernel::Qmv},
+    {"affine_qmv_bf16", "affine_qmv_w8g64_r8p2", QuantKernel::Qmv, QuantFormat::W8G64},
+    {"affine_qmm", "affine_qmm_w4g64", QuantKernel::Qmm, QuantFormat::W4G64F16},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm64_acc16", QuantKernel::Qmm},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_acc16", QuantKernel::QmmSwiglu},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64_acc16", QuantKernel::QmmSwiglu},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w4g64_bm64_rs_acc16", QuantKernel::QmmSwiglu},
+    {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g64_bm64_acc16", QuantKernel::Qmm, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_acc16", QuantKernel::QmmSwiglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_bm64_acc16", QuantKernel::QmmSwiglu, QuantFormat::W8G64},
+    {"affine_qmm_steel_bf16", "affine_qmm_swiglu_w8g64_bm64_rs_acc16", QuantKernel::QmmSwiglu, QuantFormat::W8G64},
     {"affine_dequant_bf16", "affine_dequant_w8g32", QuantKernel::Dequant, QuantFormat::W8G32},
     {"affine_qmv_bf16", "affine_qmv_w8g32", QuantKernel::Qmv, QuantFormat::W8G32},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w8g32", QuantKernel::Qmm, QuantFormat::W8G32},
@@ -437,6 +456,26 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
                    ? VPQ_ERR_NULL_POINTER
                    : vpq_moe_gate_w8g64_bf16(st, w, sc, bi, static_cast<const uint16_t*>(buf(3)),
                                              static_cast<uint16_t*>(buf(4)), ival(5), static_cast<int>(grid.y));
+    } else if (kind == QuantKernel::Requant84) {
+      // gpu-kernels/metal/quant/affine_dequant.metal:134-186: 0:w8 1:s8 2:b8 3:w4 4:s4 5:b4 6:K 7:N
+      status = (!w || !sc || !bi || !buf(3) || !buf(4) || !buf(5) || !has_int(6) || !has_int(7))
+                   ? VPQ_ERR_NULL_POINTER
+                   : vpq_requant_w8_to_w4_g64_bf16(st, w, sc, bi, static_cast<uint32_t*>(buf(3)),
+                                                   static_cast<uint16_t*>(buf(4)), static_cast<uint16_t*>(buf(5)), ival(6),
+                                                   ival(7));
+    } else if (kind == QuantKernel::QmvGeluMul) {
+      // gpu-kernels/metal/quant/affine_qmv.metal:769-805: the slots of the group-64 4-bit form, 7 = the multiplier
+      if (!w || !sc || !bi || !buf(3) || !buf(4) || !has_int(5) || !has_int(6) || !buf(7)) {
+        status = VPQ_ERR_NULL_POINTER;
+      } else if (fmt == QuantFormat::W8G64) {
+        status = vpq_qmv_gelu_mul_w8g64_bf16(st, w, sc, bi, static_cast<const uint16_t*>(buf(3)),
+                                             static_cast<uint16_t*>(buf(4)), ival(5), ival(6),
+                                             static_cast<const uint16_t*>(buf(7)));
+      } else {
+        status = vpq_qmv_gelu_mul_w4g32_bf16(st, w, sc, bi, static_cast<const uint16_t*>(buf(3)),
+                                             static_cast<uint16_t*>(buf(4)), ival(5), ival(6),
+                                             static_cast<const uint16_t*>(buf(7)), 0);
+      }
     } else if (kind == QuantKernel::Dequant) {
       if (!w || !sc || !bi || !buf(3) || !has_int(4) || !has_int(5)) {
         status = VPQ_ERR_NULL_POINTER;

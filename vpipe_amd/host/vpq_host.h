@@ -78,6 +78,7 @@ enum class QuantKernel : std::uint8_t {
   QmvSwiglu,      // affine_qmv_swiglu_w4g64: interleaved gate|up pack, N = 2*ffn, y [M, ffn]; M from grid.x / 32
   QmmSwiglu,      // affine_qmm_swiglu_w4g64[_bm64|_bm128|_bm64_rs]: slot 7 = M, 8 = out_stride, 9 = out_off (_rs)
   QmvGeglu,       // affine_qmv_geglu_w4g64: as QmvSwiglu with gelu_tanh(gate) * up
+  Requant84,      // affine_requant_w8_to_w4_g64: 0:w8 1:s8 2:b8 3:w4 4:s4 5:b4 6:K 7:N
   QmvGeluMul,     // affine_qmv_gelu_mul_w4g64: one row of x, slot 7 = mul buffer [N]; y = gelu_tanh(W x) * mul
   QmvQkvRms,      // affine_qmv_qkv_rms_w4g64 / _w4g32 / _w8g64: slots 0:w 1:scales 2:biases 3:x 4:norm_w 5:q 6:k 7:v 8:K
                   //   9,10,11 = q_rows, k_rows, v_rows, 12 = eps (float); the normalized row goes through stream scratch
