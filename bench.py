@@ -37,6 +37,7 @@ MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16
 # same counters read for a device-to-device copy of known size); the file states the build it was taken from.
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qmv_flow_kernel_decode_layer_m1_hbm_traffic_pmc.txt")
 QMM_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qmm_big_kernel_m2048_mfma_lds_traffic_pmc.txt")
+DIT_TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "qmm_big_kernel_dit_m16320_lora_r32.txt")
 
 
 def traffic_from_profile(path=TRAFFIC_PROFILE, key="traffic_bytes_per_layer:"):
@@ -591,9 +592,18 @@ def main():
         dit_flops = sum(2.0 * M * N * K for K, N in DIT)
         dit_us = sum(v["us"] for v in dit.values())
         dit_us_lora = sum(v["us_with_lora"] for v in dit.values())
+        dit_traffic, dit_traffic_build = traffic_from_profile(DIT_TRAFFIC_PROFILE,
+                                                              "traffic_bytes_per_launch_mean_of_the_three_shapes:")
+        dit_alg = sum(2.0 * M * K + N * K * 9 / 16.0 + 2.0 * M * N for K, N in DIT) / len(DIT)
         out["roofline_qmm_dit"] = {
             "bound": "mfma", "achieved": round(dit_flops / (dit_us * 1e-6) / 1e12, 1), "peak": MFMA_BF16_PEAK_TF,
-            "unit": "TFLOP/s", "frac": round(dit_flops / (dit_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TF, 4), "traffic": None,
+            "unit": "TFLOP/s", "frac": round(dit_flops / (dit_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TF, 4),
+            "traffic": dit_traffic,
+            "traffic_of": "mean over the three shapes of one qmm_big_kernel<4,true,0> launch with the rank-32 adapter "
+                          "(fetched + written; algorithmic mean %.1f MB: x, the pack and y once), profiles/%s (%s)"
+                          % (dit_alg / 1e6, os.path.basename(DIT_TRAFFIC_PROFILE), dit_traffic_build),
+            "traffic_profile_is_of_this_build": bool(dit_traffic_build) and
+                                                str(dit_traffic_build).split()[0] == vpipe_amd.build_id(),
             "achieved_with_lora_r32": round(dit_flops / (dit_us_lora * 1e-6) / 1e12, 1),
             "achieved_with_lora_r32_dense_route": round(
                 dit_flops / (sum(v["us_dense_route_with_lora"] for v in dit.values()) * 1e-6) / 1e12, 1),
