@@ -115,8 +115,9 @@ def test_qmm_lora_scale_zero_is_exactly_off(vpq, dev, D):
     assert np.array_equal(base, off)
 
 
-def _sampled_check(vpq, oracle, dev, D, M, N, K, seed, lora_r=0, alpha=1.0):
-    """Full-size launch; oracle on a sample of rows of x and rows of W (tile edges included)."""
+def _sampled_check(vpq, oracle, dev, D, M, N, K, seed, lora_r=0, alpha=1.0, dense_route_too=False):
+    """Full-size launch; oracle on a sample of rows of x and rows of W (tile edges included).  dense_route_too: the
+    dequant-once route with the same adapter gives the same bits over the whole output."""
     w, s, b = synth.make_weight(N, K, seed)
     x = synth.make_act(M, K, seed + 1)
     rng = np.random.default_rng(seed + 2)
@@ -139,6 +140,11 @@ def _sampled_check(vpq, oracle, dev, D, M, N, K, seed, lora_r=0, alpha=1.0):
         t_bits, B = t_all[ms], B[ns]
     y64, yb = oracle.qmm(w[ns], s[ns], b[ns], x[ms], K, len(ns), len(ms), t=t_bits, B=B, r=lora_r)
     parity.check_bf16(got, y64, yb)
+    if dense_route_too:
+        w_deq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+        y2 = vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(y2, y)
     return y
 
 
@@ -150,7 +156,7 @@ def test_qmm_prefill_shapes(vpq, oracle, dev, D, K, N):
 @pytest.mark.parametrize("K,N", [(5120, 5120), (5120, 20480), (20480, 5120)])
 def test_qmm_video_dit_shapes_with_lora(vpq, oracle, dev, D, K, N):
     # M = 16320 = 127*128 + 64: an M tail; y of 5120->20480 is 668 MB: 64-bit addressing
-    _sampled_check(vpq, oracle, dev, D, 16320, N, K, 0x5EED0005 + N, lora_r=32, alpha=1.0)
+    _sampled_check(vpq, oracle, dev, D, 16320, N, K, 0x5EED0005 + N, lora_r=32, alpha=1.0, dense_route_too=True)
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 64, 64), (130, 320, 256), (33, 33, 128), (257, 129, 512), (1, 8, 64)])
