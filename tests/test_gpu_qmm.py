@@ -102,6 +102,32 @@ def test_qmm_lora_fused(vpq, oracle, dev, D, r, alpha):
     assert np.sqrt((d ** 2).sum() / (want ** 2).sum()) > 0.05
 
 
+@pytest.mark.parametrize("M,K,r", [(1, 64, 16), (33, 192, 32), (257, 4096, 16), (1000, 5120, 32), (31, 1024, 48), (600, 2048, 128)])
+def test_lora_pre_pass_alone(vpq, oracle, dev, D, M, K, r):
+    """t = bf16(alpha * bf16(x . A^T)) (lora_gemm_a_, minimax-h3/metal-minimax-h3-transformer.cc:1030-1067) on ragged
+    M, a K of one chunk, K with fewer chunks than wavefronts, and both kernels (ranks up to 32 / above), against the
+    oracle within one ulp of the inner rounding bf16(x . A^T) (fp32 sums in another order than the oracle's double);
+    alpha = 2 scales that exactly, alpha = 0.875 can carry the one ulp across a binade (two ulps of the smaller one);
+    the scratch's guard bands stay intact."""
+    alpha = 2.0 if (M + r) % 3 else 0.875
+    x = synth.make_act(M, K, 8800 + M)
+    A, _ = synth.make_lora(8, K, r, 8801 + r, std=0.05)
+    t_ref = oracle.lora_t(x, A, M, K, r, alpha)
+    out = parity.Guarded((M, r), torch.bfloat16, dev)
+    vpq.lora_a(D.bf16(x, dev), D.bf16(A, dev), M, K, r, alpha, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    got = synth.bf16_bits_to_f32(D.bits(out.view)).astype(np.float64)
+    ref = synth.bf16_bits_to_f32(t_ref).astype(np.float64)
+    # one ulp of the inner rounding (2^-7 relative; 2^-6 of the result where alpha carries it across a binade), and
+    # where the sum cancels, the fp32 accumulation's own error against the oracle's double
+    mag = np.abs(synth.bf16_bits_to_f32(x).astype(np.float64)) @ np.abs(synth.bf16_bits_to_f32(A).astype(np.float64)).T
+    allowed = (2.0 ** -7 if alpha == 2.0 else 2.0 ** -6) * np.abs(ref) + alpha * 64 * 2.0 ** -24 * mag
+    assert (np.abs(got - ref) <= allowed).all()
+    assert (D.bits(out.view) != t_ref).mean() < 0.02
+    assert np.abs(synth.bf16_bits_to_f32(t_ref)).max() > 0
+
+
 def test_qmm_lora_scale_zero_is_exactly_off(vpq, dev, D):
     # minimax_h3_lora: strength 0 == no adapter, bit for bit (metal-minimax-h3-transformer.cc:2211-2219)
     M, N, K, r = 70, 130, 256, 32
