@@ -1686,7 +1686,8 @@ int vpq_qmv_qkv_rms_bf16(vpq_stream_t stream, int format, int count, const uint3
   if (format < 0 || format > 2) { return VPQ_ERR_BAD_SHAPE; }
   if (x_norm_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
   if (!aligned(x_norm_ws, 16)) { return VPQ_ERR_MISALIGNED; }
-  // the packs are checked before anything runs, by the format's own entry point on a count of zero rows ...
+  // (the packs themselves are checked by the format's own grouped entry point below: a refusal there has written the
+  // scratch and nothing else)
   if (w == nullptr || scales == nullptr || biases == nullptr || y == nullptr || N == nullptr) { return VPQ_ERR_NULL_POINTER; }
   if (count < 1 || count > 4) { return VPQ_ERR_BAD_SHAPE; }
   if (K <= 0 || (K % (format == 1 ? 32 : 64)) != 0) { return VPQ_ERR_BAD_SHAPE; }
