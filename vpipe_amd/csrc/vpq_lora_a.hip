@@ -124,7 +124,7 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_kernel(const LoraAParams p
 // Ranks up to 32 (one tile of 32 columns; what the video-DiT adapters and the reference's rank-16 adapters run): the
 // same decomposition with x AND A brought in by 128-bit direct-to-LDS loads -- one instruction covers 8 rows x 128
 // contiguous bytes (whole cache lines) instead of 16-byte pieces of 32 rows, which is what held the kernel above to a
-// third of the HBM rate (16320 x 5120: 58 -> see the profile; x is read once either way).  Every wavefront owns a
+// third of the HBM rate (16320 x 5120 at rank 32: 58 -> 34 us; x is read once either way).  Every wavefront owns a
 // ring of two 8 KB slots (32 rows of x and 32 rows of A, 64 values of K each, the 16-byte pieces of a row XOR-swizzled
 // by the row so that the operand reads do not collide on banks) and walks its chunks with two in flight; the waits
 // are counted by hand and the LDS reads are asm so that the compiler adds none of its own.  Within a chunk MFMA j
