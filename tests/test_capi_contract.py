@@ -147,3 +147,14 @@ def test_build_refuses_use_of_a_load_register_before_its_wait():
     # the same join is fine once both paths have waited
     build._check_inflight("x.hip", kernel(["s_cbranch_scc1 .LBB0_2"] + ok[:1] + ["s_waitcnt vmcnt(0)", ".LBB0_2:",
                                                                                   "v_mov_b32_e32 v20, v4"]))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # one GPU only: no collectives, no sharding; the benchmark says so instead of starting ranks
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stderr + r.stdout)
