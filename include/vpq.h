@@ -164,7 +164,7 @@ enum {
  * dense_gemm_mma.metal:297-348).  lora_a == NULL or alpha == 0 means no adapter,
  * and the output is then bit-identical to the call without one
  * (metal-minimax-h3-transformer.cc:2211-2219).
- * Requires K % 64 == 0, M, N > 0, and with a LoRA r % 16 == 0, 16 <= r <= VPQ_LORA_MAX_RANK (the reference's
+ * Requires K % 64 == 0, M, N > 0, and with a LoRA r % 8 == 0, 8 <= r <= VPQ_LORA_MAX_RANK (the reference's
  * LoraFactors.rank is unconstrained, metal-minimax-h3-transformer.h:923-931; it runs rank 16 adapters, .h:365-367,
  * and measures rank 384, .cc:1126-1132); x, y rows may be of any length (K, N) but the base pointers must be
  * 16-byte aligned. */
@@ -229,7 +229,7 @@ int vpq_qmm_dense_route_lora_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, 
                                         uint16_t* w_deq, int expand, const uint16_t* lora_a, const uint16_t* lora_b,
                                         int r, float alpha, uint16_t* lora_t_ws);
 
-/* The adapter's first GEMM alone: t[M,r] = bf16(alpha * bf16(x . A^T)), r % 16 == 0, 16 <= r <= VPQ_LORA_MAX_RANK.
+/* The adapter's first GEMM alone: t[M,r] = bf16(alpha * bf16(x . A^T)), r % 8 == 0, 8 <= r <= VPQ_LORA_MAX_RANK.
  * Replaces `lora_gemm_a_` (metal-minimax-h3-transformer.cc:1030-1067). */
 #define VPQ_LORA_MAX_RANK 512
 int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t,
@@ -720,7 +720,7 @@ int vpq_qmm_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* sc
  * gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273, 297-348, whose element type is VPIPE_ELT, :28-33):
  * vpq_lora_a_f16 is t[M,r] = f16(alpha * f16(x . A^T)); vpq_qmm_lora_w4g64_f16 is vpq_qmm_w4g64_f16 (no
  * activation) with y += t . B^T in the same accumulators before the one rounding.  A [r,K], B [N,r], t scratch
- * [M,r], all binary16; r % 16 == 0, 16 <= r <= VPQ_LORA_MAX_RANK; lora_a == NULL or alpha == 0: no adapter. */
+ * [M,r], all binary16; r % 8 == 0, 8 <= r <= VPQ_LORA_MAX_RANK; lora_a == NULL or alpha == 0: no adapter. */
 int vpq_lora_a_f16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_a, uint16_t* t,
                    int M, int K, int r, float alpha);
 int vpq_qmm_lora_w4g64_f16(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,

@@ -53,7 +53,7 @@ def test_host_side_validation_and_sizes():
     assert L.vpq_qmv_w4g64_bf16(null, one, one, one, one, one, 64, 8, 17, null, null, 0, 0) == -2
     assert L.vpq_qmv_w4g64_bf16(null, one, one, one, one, one, 64, 8, 0, null, null, 0, 0) == -2
     assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 0, null, null, 0, 0.0, null) == -2
-    assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, one, one, 40, 1.0, one) == -2      # rank not a multiple of 16
+    assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, one, one, 36, 1.0, one) == -2      # rank not a multiple of 8
     assert L.vpq_qmm_w4g64_bf16(null, one, one, one, one, one, 64, 8, 4, one, one, 528, 1.0, one) == -2     # above VPQ_LORA_MAX_RANK
     # misaligned codes / x
     assert L.vpq_dequant_w4g64_bf16(null, ctypes.c_void_p(4100), one, one, one, 64, 1) == -3

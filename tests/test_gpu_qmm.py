@@ -72,7 +72,8 @@ def test_qmm_reference_lcg_inputs(vpq, oracle, dev, D):
     parity.check_bf16(got, y64, yb)
 
 
-@pytest.mark.parametrize("r,alpha", [(16, 1.5), (32, 1.0), (48, 0.75), (64, 0.625), (128, 2.0), (256, 0.5), (384, 0.25)])
+@pytest.mark.parametrize("r,alpha", [(8, 1.0), (16, 1.5), (24, 0.5), (32, 1.0), (40, 1.25), (48, 0.75), (64, 0.625), (72, 1.0), (128, 2.0),
+                                     (256, 0.5), (384, 0.25)])
 def test_qmm_lora_fused(vpq, oracle, dev, D, r, alpha):
     M, N, K = 96, 160, 512
     w, s, b = synth.make_weight(N, K, 23)
@@ -102,7 +103,8 @@ def test_qmm_lora_fused(vpq, oracle, dev, D, r, alpha):
     assert np.sqrt((d ** 2).sum() / (want ** 2).sum()) > 0.05
 
 
-@pytest.mark.parametrize("M,K,r", [(1, 64, 16), (33, 192, 32), (257, 4096, 16), (1000, 5120, 32), (31, 1024, 48), (600, 2048, 128)])
+@pytest.mark.parametrize("M,K,r", [(1, 64, 16), (33, 192, 32), (257, 4096, 16), (1000, 5120, 32), (31, 1024, 48), (600, 2048, 128),
+                                   (50, 512, 8), (100, 1024, 24), (64, 2048, 40)])
 def test_lora_pre_pass_alone(vpq, oracle, dev, D, M, K, r):
     """t = bf16(alpha * bf16(x . A^T)) (lora_gemm_a_, minimax-h3/metal-minimax-h3-transformer.cc:1030-1067) on ragged
     M, a K of one chunk, K with fewer chunks than wavefronts, and both kernels (ranks up to 32 / above), against the
@@ -296,7 +298,7 @@ def test_qmm_large_tile_kernel(vpq, oracle, dev, D, M, N, K, tile_n):
 
 
 @pytest.mark.parametrize("tile_n", [-128, 192, 256])
-@pytest.mark.parametrize("r", [16, 32, 48, 64, 96, 256, 384])
+@pytest.mark.parametrize("r", [8, 16, 24, 32, 48, 64, 88, 96, 256, 384])
 def test_qmm_large_tile_kernel_with_lora(vpq, oracle, dev, D, r, tile_n):
     M, N, K, alpha = 300, 450, 1024, 0.75
     w, s, b = synth.make_weight(N, K, 7300 + r)
@@ -316,7 +318,8 @@ def test_qmm_large_tile_kernel_with_lora(vpq, oracle, dev, D, r, tile_n):
     assert not torch.equal(base, got)
 
 
-@pytest.mark.parametrize("M,N,K,r", [(300, 450, 1024, 32), (64, 40, 192, 16), (2304, 4096, 512, 48), (130, 328, 1536, 384)])
+@pytest.mark.parametrize("M,N,K,r", [(300, 450, 1024, 32), (64, 40, 192, 16), (2304, 4096, 512, 48), (130, 328, 1536, 384),
+                                     (200, 264, 512, 8), (90, 136, 640, 24)])
 def test_dense_route_with_lora_is_the_fused_gemm(vpq, oracle, dev, D, M, N, K, r):
     """The dequant-once route with the runtime adapter: the bits of the fused GEMM with the same adapter (whose
     parity test_qmm_lora_fused holds) where the fused kernel runs the same tiles, the oracle's tolerance everywhere,
@@ -347,7 +350,7 @@ def test_dense_route_with_lora_is_the_fused_gemm(vpq, oracle, dev, D, M, N, K, r
     assert not torch.equal(out.view, vpq.qmm_dense_route_w4g64(wd, sd, bd, xd, K, N, M, w_deq))
     L = vpq.load()
     p = out.view.data_ptr()
-    assert L.vpq_qmm_dense_route_lora_w4g64_bf16(None, p, p, p, p, p, K, N, M, p, 1, p, p, 40, 1.0, p) == -2
+    assert L.vpq_qmm_dense_route_lora_w4g64_bf16(None, p, p, p, p, p, K, N, M, p, 1, p, p, 36, 1.0, p) == -2
     assert L.vpq_qmm_dense_route_lora_w4g64_bf16(None, p, p, p, p, p, K, N, M, p, 1, p, p, r, 1.0, None) == -4
 
 

@@ -500,7 +500,7 @@ int vpq_lora_a_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora
                     int M, int K, int r, float alpha)
 {
   if (x == nullptr || lora_a == nullptr || t == nullptr) { return VPQ_ERR_NULL_POINTER; }
-  if (M <= 0 || K <= 0 || (K % 64) != 0 || r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (M <= 0 || K <= 0 || (K % 64) != 0 || r < 8 || r > vpq::kLoraMaxRank || (r % 8) != 0) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(lora_a, 16) || !aligned(t, 16)) { return VPQ_ERR_MISALIGNED; }
   const int st = ensure_init();
   if (st != VPQ_OK) { return st; }
@@ -525,7 +525,7 @@ int qmm_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scales,
   if (lora) {
     if (lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
     if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
-    if (r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (r < 8 || r > vpq::kLoraMaxRank || (r % 8) != 0) { return VPQ_ERR_BAD_SHAPE; }
     if (!aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) { return VPQ_ERR_MISALIGNED; }
   }
   st = ensure_init();
@@ -640,7 +640,7 @@ int vpq_qmm_dense_route_lora_w4g64_bf16(vpq_stream_t stream, const uint32_t* w, 
   if (lora) {
     if (lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
     if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
-    if (r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (r < 8 || r > vpq::kLoraMaxRank || (r % 8) != 0) { return VPQ_ERR_BAD_SHAPE; }
     if (!aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) { return VPQ_ERR_MISALIGNED; }
   }
   st = ensure_init();
@@ -752,7 +752,7 @@ int qmm_f16_common(vpq_stream_t stream, const uint32_t* w, const uint16_t* scale
     if (activation != 0) { return VPQ_ERR_BAD_SHAPE; }
     if (lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
     if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
-    if (r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (r < 8 || r > vpq::kLoraMaxRank || (r % 8) != 0) { return VPQ_ERR_BAD_SHAPE; }
     if (!aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) { return VPQ_ERR_MISALIGNED; }
   }
   st = ensure_init();
@@ -791,7 +791,7 @@ int vpq_lora_a_f16(vpq_stream_t stream, const uint16_t* x, const uint16_t* lora_
                    float alpha)
 {
   if (x == nullptr || lora_a == nullptr || t == nullptr) { return VPQ_ERR_NULL_POINTER; }
-  if (M <= 0 || K <= 0 || (K % 64) != 0 || r < 16 || r > vpq::kLoraMaxRank || (r % 16) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (M <= 0 || K <= 0 || (K % 64) != 0 || r < 8 || r > vpq::kLoraMaxRank || (r % 8) != 0) { return VPQ_ERR_BAD_SHAPE; }
   if (!aligned(x, 16) || !aligned(lora_a, 16) || !aligned(t, 16)) { return VPQ_ERR_MISALIGNED; }
   const int st = ensure_init();
   if (st != VPQ_OK) { return st; }

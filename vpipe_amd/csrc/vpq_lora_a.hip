@@ -1,5 +1,5 @@
 // The adapter's first factor: t[M,r] = elt(alpha * elt(x[M,K] . A[r,K]^T)), elt = bf16 or IEEE binary16 (the
-// reference's VPIPE_ELT, gpu-kernels/metal/gemm/dense_gemm_mma.metal:28-33), any rank that is a multiple of 16
+// reference's VPIPE_ELT, gpu-kernels/metal/gemm/dense_gemm_mma.metal:28-33), any rank that is a multiple of 8
 // up to kLoraMaxRank (the SCALED tile of gpu-kernels/metal/gemm/dense_gemm_mma.metal:227-273, driven by
 // lora_gemm_a_, generative-models/minimax-h3/metal-minimax-h3-transformer.cc:1030-1067; the reference runs rank 16
 // adapters and measures rank 384, metal-minimax-h3-transformer.h:365-367, .cc:1126-1132).
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(kWaves * 64) void lora_a_dma_kernel(const LoraAPara
 hipError_t launch_lora_a(hipStream_t st, const uint16_t* x, const uint16_t* a, uint16_t* t, int M, int K, int r,
                          float alpha, bool f16)
 {
-  if (r < 16 || r % 16 != 0 || r > kLoraMaxRank) { return hipErrorInvalidValue; }
+  if (r < 8 || r % 8 != 0 || r > kLoraMaxRank) { return hipErrorInvalidValue; }
   LoraAParams p{x, a, t, M, K, r, alpha};
   const dim3 grid((unsigned)((M + kRows - 1) / kRows), (unsigned)((r + 127) / 128)), block(kWaves * 64);
   if (r <= 32) {

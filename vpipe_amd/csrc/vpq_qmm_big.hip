@@ -713,8 +713,11 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
     for (int st = 0; st < steps; ++st) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       wg_barrier();                                    // everyone done with stage 0
-      const int kleft = p.r - st * BK;                 // >= 16, a multiple of 16
+      const int kleft = p.r - st * BK;                 // >= 8, a multiple of 8
       const int chunks = kleft >= BK ? 8 : (kleft >> 3);
+      // An odd number of 8-value pieces (a rank of 8 mod 16): the quarter step's other half is zeros, in both tiles
+      // (what lies in the stage from the K loop may be anything, a NaN pattern included).
+      const int zero_chunk = (chunks & 1) ? chunks : -1;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int row = (wave * 8 + i) * 8 + (lane >> 3);
@@ -723,6 +726,8 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
         if (chunk < chunks) {
           dma16(lds_addr(x_lds0) + wave * (64 * kRow) + i * (8 * kRow),
                 reinterpret_cast<const uint8_t*>(p.lora_t + (size_t)rg * p.r + st * BK + chunk * 8));
+        } else if (chunk == zero_chunk) {
+          *reinterpret_cast<uint4*>(x_lds0 + wave * (64 * kRow) + i * (8 * kRow) + lane * 16) = make_uint4(0, 0, 0, 0);
         }
       }
       if (dq_wave) {
@@ -734,12 +739,14 @@ __global__ __launch_bounds__(kBigThreads) void qmm_big_kernel(const BigParams p)
           if (chunk < chunks) {
             dma16(lds_addr(w_lds0) + wave * (64 * kRow) + i * (8 * kRow),
                   reinterpret_cast<const uint8_t*>(p.lora_b + (size_t)rg * p.r + st * BK + chunk * 8));
+          } else if (chunk == zero_chunk) {
+            *reinterpret_cast<uint4*>(w_lds0 + wave * (64 * kRow) + i * (8 * kRow) + lane * 16) = make_uint4(0, 0, 0, 0);
           }
         }
       }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       wg_barrier();                                    // tiles ready
-      plain_quarters(chunks >> 1);
+      plain_quarters((chunks + 1) >> 1);
     }
   }
 
@@ -851,7 +858,7 @@ bool qmm_big_supports(const GemmArgs& a)
   if (a.gate_act != 0 && (a.lora_t != nullptr || (a.N & 1) != 0)) { return false; }
   if ((reinterpret_cast<uintptr_t>(a.scales) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.biases) & 15) != 0) { return false; }
   if ((double)a.N * (double)a.K / (a.bits == 8 ? 1.0 : 2.0) >= 4.0e9 || (double)BM * (double)a.K * 2.0 >= 4.0e9) { return false; }
-  if (a.lora_t != nullptr && (a.r < 16 || a.r % 16 != 0)) { return false; }
+  if (a.lora_t != nullptr && (a.r < 8 || a.r % 8 != 0)) { return false; }
   // the other code formats come without the adapter path; formats and element types are not combined
   const int modes = (a.bits == 8) + (a.group == 32) + (a.f16 ? 1 : 0);
   if (modes > 1 || (modes == 1 && !a.f16 && a.lora_t != nullptr)) { return false; }
@@ -973,7 +980,7 @@ hipError_t launch_dense_gemm(hipStream_t st, const uint16_t* x, const uint16_t* 
 {
   if (!dense_gemm_supports(M, N, K)) { return hipErrorInvalidValue; }
   const bool lora = lora_t != nullptr;
-  if (lora && (f16 || lora_b == nullptr || r < 16 || r % 16 != 0)) { return hipErrorInvalidValue; }
+  if (lora && (f16 || lora_b == nullptr || r < 8 || r % 8 != 0)) { return hipErrorInvalidValue; }
   const int bn = qmm_big_tile_n(N, M, cu_count);
   BigParams p{};
   p.w = reinterpret_cast<const uint32_t*>(b);

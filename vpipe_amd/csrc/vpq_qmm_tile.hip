@@ -444,8 +444,10 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
     if (LORA) {
       const int steps = (p.r + TK - 1) / TK;
       for (int st = 0; st < steps; ++st) {
-        const int kleft = p.r - st * TK;                 // >= 16, a multiple of 16
+        const int kleft = p.r - st * TK;                 // >= 8, a multiple of 8
         const int chunks = kleft >= TK ? 8 : (kleft >> 3);
+        // an odd number of 8-value pieces (a rank of 8 mod 16): the quarter step's other half is zeros in both tiles
+        const int zero_chunk = (chunks & 1) ? chunks : -1;
         // t tile: 256 rows, as the x tile; B tile: 128 rows, 4 loads per wavefront.  Stage 0.
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -456,6 +458,8 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)(p.lora_t + (size_t)rg * p.r + st * TK + chunk * 8),
                 (__attribute__((address_space(3))) void*)(x_lds + pw * (64 * kRowB) + i * (8 * kRowB)), 16, 0, 0);
+          } else if (chunk == zero_chunk) {
+            *reinterpret_cast<uint4*>(x_lds + pw * (64 * kRowB) + i * (8 * kRowB) + lane * 16) = make_uint4(0, 0, 0, 0);
           }
         }
 #pragma unroll
@@ -467,9 +471,11 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)(p.lora_b + (size_t)rg * p.r + st * TK + chunk * 8),
                 (__attribute__((address_space(3))) void*)(w_lds + pw * (32 * kRowB) + i * (8 * kRowB)), 16, 0, 0);
+          } else if (chunk == zero_chunk) {
+            *reinterpret_cast<uint4*>(w_lds + pw * (32 * kRowB) + i * (8 * kRowB) + lane * 16) = make_uint4(0, 0, 0, 0);
           }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         wg_barrier();                                    // tiles ready
         wg_barrier();                                    // consumers done with them
       }
@@ -593,7 +599,7 @@ __global__ __launch_bounds__((kConsumers + P) * 64) void qmm_tile_kernel(const T
       const int kleft = p.r - st * TK;
       const int chunks = kleft >= TK ? 8 : (kleft >> 3);
       wg_barrier();
-      mma_stage(0, chunks >> 1);
+      mma_stage(0, (chunks + 1) >> 1);
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       wg_barrier();
     }
