@@ -752,13 +752,23 @@ int vpq_qmv_group_w8g64_bf16(vpq_stream_t stream, int count, const uint32_t* con
  * vpq_qmv_qkv_rms_bf16 runs it on the one row x [K] into `x_norm_ws` (K elements of caller scratch, 16-byte aligned:
  * the reference keeps the normalized row in threadgroup memory) and then the grouped GEMV of `format` (VPQ_FORMAT_*)
  * over that row: two launches, the values of the fused kernel. */
-enum { VPQ_FORMAT_W4G64 = 0, VPQ_FORMAT_W4G32 = 1, VPQ_FORMAT_W8G64 = 2 };
+enum { VPQ_FORMAT_W4G64 = 0, VPQ_FORMAT_W4G32 = 1, VPQ_FORMAT_W8G64 = 2, VPQ_FORMAT_W8G32 = 3 };
 int vpq_rmsnorm_bf16(vpq_stream_t stream, const uint16_t* x, const uint16_t* norm_w, uint16_t* out,
                      int K, int M, float eps);
 int vpq_qmv_qkv_rms_bf16(vpq_stream_t stream, int format, int count, const uint32_t* const* w,
                          const uint16_t* const* scales, const uint16_t* const* biases, const uint16_t* x,
                          const uint16_t* norm_w, uint16_t* const* y, int K, const int* N, float eps,
                          uint16_t* x_norm_ws);
+/* The dequant-once route with the runtime adapter over a pack of any format (VPQ_FORMAT_*: the 4-bit group-64 form is
+ * vpq_qmm_dense_route_lora_w4g64_bf16, whose arguments these are): the adapter's pre-pass into lora_t_ws, the format's
+ * expansion into w_deq (expand != 0) or the kept one, then the dense GEMM with t . B^T in the same accumulators -- the
+ * reference's route for an adapter over a quantized Linear of any width (`gemm_`, metal-minimax-h3-transformer.cc:
+ * 2205-2259, with Linear.bits 4 or 8).  The fused kernels of the 8-bit and group-32 packs take no adapter; this is
+ * their adapter path.  With an adapter K % 64 == 0. */
+int vpq_qmm_dense_route_lora_bf16(vpq_stream_t stream, int format, const uint32_t* w, const uint16_t* scales,
+                                  const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                  uint16_t* w_deq, int expand, const uint16_t* lora_a, const uint16_t* lora_b,
+                                  int r, float alpha, uint16_t* lora_t_ws);
 
 /* ---- a12: the packer ------------------------------------------------------
  * Replaces `affine_quant_w4_g64` (gpu-kernels/metal/quant/affine_dequant.metal:

@@ -122,6 +122,23 @@ void hd_quant_linear(void* h, void* codes, void* scales, void* qbias, int K, int
   }
 }
 
+// The same over a pack of another width / group (bits 4 or 8, group 64 or 32), with an adapter.
+void hd_quant_linear_fmt(void* h, void* codes, void* scales, void* qbias, int bits, int group, int K, int N, void* x, void* y,
+                         int M, void* lora_a, void* lora_b, int rank, float strength, void* lora_t)
+{
+  Session* s = static_cast<Session*>(h);
+  const size_t kb = (size_t)N * K * bits / 8, sb = (size_t)N * (K / group) * 2;
+  DeviceBuffer bc = DeviceBuffer::wrap(codes, kb), bs = DeviceBuffer::wrap(scales, sb), bq = DeviceBuffer::wrap(qbias, sb);
+  DeviceBuffer bx = DeviceBuffer::wrap(x, (size_t)M * K * 2), by = DeviceBuffer::wrap(y, (size_t)M * N * 2);
+  Linear lin;
+  lin.codes = &bc; lin.scales = &bs; lin.qbias = &bq; lin.K = K; lin.N = N; lin.bits = bits; lin.group = group;
+  DeviceBuffer la = DeviceBuffer::wrap(lora_a, (size_t)rank * K * 2), lb = DeviceBuffer::wrap(lora_b, (size_t)N * rank * 2);
+  DeviceBuffer lt = DeviceBuffer::wrap(lora_t, (size_t)M * rank * 2);
+  LoraFactors lf;
+  lf.a = &la; lf.b = &lb; lf.rank = rank; lf.strength = strength;
+  quant_linear_forward(s->stream, lin, bx, 0, by, 0, M, &lf, &lt);
+}
+
 // ---- checkpoint container (vpq_weights.h) ---------------------------------------------------
 
 void* hw_open(const char* dir, unsigned long long shard_max_bytes)

@@ -277,6 +277,37 @@ def test_quant_linear_forward_with_lora(enc, oracle, dev, D):
     parity.check_bf16(D.bits(yd), y64, yb)
 
 
+@pytest.mark.parametrize("bits,group,fmt", [(8, 64, 2), (4, 32, 1), (8, 32, 3)])
+def test_quant_linear_forward_with_lora_over_the_format_twins(vpq, enc, dev, D, bits, group, fmt):
+    # `gemm_` with an adapter over a Linear of another width or group (minimax-h3/metal-minimax-h3-transformer.cc:
+    # 2205-2259): the host takes the dequant-once route with the expansion in scratch of the stream; the bits of the
+    # C ABI's call
+    K, N, M, r, strength = 512, 136, 70, 24, 0.5
+    if bits == 8:
+        w, s, b = synth.make_weight8(N, K, 4300, group=group)
+    else:
+        w, s, b = synth.make_weight_g32(N, K, 4301)
+    x = synth.make_act(M, K, 4302)
+    A, B = synth.make_lora(N, K, r, 4303, std=0.05)
+    wd, sd, bd, xd = D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev), D.bf16(x, dev)
+    Ad, Bd = D.bf16(A, dev), D.bf16(B, dev)
+    td = torch.zeros((M, r), dtype=torch.bfloat16, device=dev)
+    yd = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    torch.cuda.synchronize()
+    L = enc.L
+    L.hd_quant_linear_fmt.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                      ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                      ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_void_p]
+    L.hd_quant_linear_fmt(enc.h, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), bits, group, K, N, xd.data_ptr(), yd.data_ptr(), M,
+                          Ad.data_ptr(), Bd.data_ptr(), r, strength, td.data_ptr())
+    ok, why = enc.wait_ok()
+    assert ok, why
+    w_deq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+    want = vpq.qmm_dense_route_lora(fmt, wd, sd, bd, xd, K, N, M, w_deq, Ad, Bd, r, strength)
+    assert torch.equal(yd, want)
+    assert yd.abs().sum() > 0
+
+
 def test_fused_qkv_call_site(enc, oracle, dev, D):
     # llama decode: one dispatch over the row-concatenated q|k|v pack, three output buffers
     # (gpu-kernels/metal/quant/affine_qmv.metal:405-516)

@@ -533,3 +533,52 @@ def test_qmv_gelu_mul_twins(vpq, oracle, dev, D, K, N, fmt):
         assert L.vpq_qmv_gelu_mul_w8g64_bf16(None, p, p, p, p, p, K, N, None) == -1
     else:
         assert L.vpq_qmv_gelu_mul_w4g32_bf16(None, p, p, p, p, p, K, N, None, 0) == -1
+
+
+@pytest.mark.parametrize("M,N,K,r", [(130, 264, 512, 16), (300, 136, 1024, 8), (64, 72, 192, 40)])
+@pytest.mark.parametrize("fmt", [1, 2, 3])
+def test_dense_route_with_adapter_over_the_format_twins(vpq, oracle, dev, D, fmt, M, N, K, r):
+    """vpq_qmm_dense_route_lora_bf16: the adapter over 4-bit group-32, 8-bit group-64 and 8-bit group-32 packs by the
+    dequant-once route (`gemm_` with Linear.bits 4 or 8, minimax-h3/metal-minimax-h3-transformer.cc:2205-2259).  t is
+    the pre-pass's (pinned by its own tests); y against float64 of x . W^T + t . B^T with W the oracle's expansion of
+    the pack; alpha = 0 and the kept expansion give the bits of the plain route."""
+    alpha = 0.75
+    if fmt == 1:
+        w, s, b = synth.make_weight_g32(N, K, 9100 + r)
+        dense = oracle.dequant_g32_bf16(w, s, b, K, N)
+        plain = vpq.qmm_dense_route_w4g32
+    elif fmt == 2:
+        w, s, b = synth.make_weight8(N, K, 9101 + r)
+        dense = oracle.dequant8_bf16(w, s, b, K, N)
+        plain = vpq.qmm_dense_route_w8g64
+    else:
+        w, s, b = synth.make_weight8(N, K, 9102 + r, group=32)
+        dense = oracle.dequant8_g32(w, s, b, K, N)
+        plain = vpq.qmm_dense_route_w8g32
+    x = synth.make_act(M, K, 9103)
+    A, B = synth.make_lora(N, K, r, 9104, std=0.05)
+    wd, sd, bd, xd = stage(D, dev, w, s, b, x)
+    Ad, Bd = D.bf16(A, dev), D.bf16(B, dev)
+    w_deq = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+    t_ws = parity.Guarded((M, r), torch.bfloat16, dev)
+    out = parity.Guarded((M, N), torch.bfloat16, dev)
+    vpq.qmm_dense_route_lora(fmt, wd, sd, bd, xd, K, N, M, w_deq, Ad, Bd, r, alpha, out=out.view, t_ws=t_ws.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    t_ws.assert_intact()
+    assert np.array_equal(D.bits(w_deq), dense)
+    assert torch.equal(t_ws.view, vpq.lora_a(xd, Ad, M, K, r, alpha))
+    f64 = lambda bits: synth.bf16_bits_to_f32(bits).astype(np.float64)
+    want = f64(x) @ f64(dense).T + f64(D.bits(t_ws.view)) @ f64(B).T
+    parity.check_bf16(D.bits(out.view), want, synth.f32_to_bf16_bits(want.astype(np.float32)))
+    base = plain(wd, sd, bd, xd, K, N, M, w_deq)
+    assert not torch.equal(base, out.view)
+    kept = vpq.qmm_dense_route_lora(fmt, wd, sd, bd, xd, K, N, M, w_deq, Ad, Bd, r, alpha, expand=False)
+    assert torch.equal(kept, out.view)
+    off = vpq.qmm_dense_route_lora(fmt, wd, sd, bd, xd, K, N, M, w_deq, Ad, Bd, r, 0.0)
+    assert torch.equal(off, base)
+    L = vpq.load()
+    p = out.view.data_ptr()
+    assert L.vpq_qmm_dense_route_lora_bf16(None, 7, p, p, p, p, p, K, N, M, p, 1, p, p, r, 1.0, p) == -2
+    assert L.vpq_qmm_dense_route_lora_bf16(None, fmt, p, p, p, p, p, K, N, M, p, 1, p, p, 12, 1.0, p) == -2
+    assert L.vpq_qmm_dense_route_lora_bf16(None, fmt, p, p, p, p, p, K, N, M, p, 1, p, None, r, 1.0, p) == -1

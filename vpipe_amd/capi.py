@@ -78,6 +78,7 @@ SYMBOLS = [
     ("vpq_qmv_gelu_mul_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i]),
     ("vpq_qmm_dense_route_w8g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_qmv_qkv_rms_bf16", _i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _f, _vp]),
+    ("vpq_qmm_dense_route_lora_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _f, _vp]),
     ("vpq_interleave_rows", _i, [_vp, _vp, _vp, _vp, _sz, _sz]),
     ("vpq_qmv_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     ("vpq_qmv_swiglu_w4g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
@@ -930,7 +931,7 @@ def rmsnorm_bf16(x, norm_w, K, M, eps, out=None):
     return out
 
 
-VPQ_FORMAT_W4G64, VPQ_FORMAT_W4G32, VPQ_FORMAT_W8G64 = 0, 1, 2
+VPQ_FORMAT_W4G64, VPQ_FORMAT_W4G32, VPQ_FORMAT_W8G64, VPQ_FORMAT_W8G32 = 0, 1, 2, 3
 
 
 def qmv_qkv_rms(fmt, packs, x, norm_w, K, eps, outs=None, x_norm_ws=None):
@@ -973,4 +974,18 @@ def f16_to_bf16(t):
     import torch
     out = torch.empty(t.shape, dtype=torch.int16, device=t.device)
     _check(load().vpq_f16_to_bf16(_stream(), _ptr(t), _ptr(out), t.numel()), "vpq_f16_to_bf16")
+    return out
+
+
+def qmm_dense_route_lora(fmt, w, scales, biases, x, K, N, M, w_deq, lora_A, lora_B, r, alpha, expand=True, out=None,
+                         t_ws=None):
+    """The dequant-once route with the runtime adapter over a pack of format fmt (VPQ_FORMAT_*)."""
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=w.device)
+    if t_ws is None:
+        t_ws = torch.empty((M, r), dtype=torch.bfloat16, device=w.device)
+    _check(load().vpq_qmm_dense_route_lora_bf16(_stream(), fmt, _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
+                                                M, _ptr(w_deq), 1 if expand else 0, _ptr(lora_A), _ptr(lora_B), r, alpha,
+                                                _ptr(t_ws)), "vpq_qmm_dense_route_lora_bf16")
     return out

@@ -1806,6 +1806,58 @@ int vpq_profile_read(float* kernel_ms, int capacity)
   return n;
 }
 
+// The dequant-once route with the runtime adapter for any of the pack formats: the adapter's pre-pass, the format's
+// expansion (or the kept one), the dense GEMM with t . B^T in the same accumulators.
+int vpq_qmm_dense_route_lora_bf16(vpq_stream_t stream, int format, const uint32_t* w, const uint16_t* scales,
+                                  const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                                  uint16_t* w_deq, int expand, const uint16_t* lora_a, const uint16_t* lora_b, int r,
+                                  float alpha, uint16_t* lora_t_ws)
+{
+  if (format == VPQ_FORMAT_W4G64) {
+    return vpq_qmm_dense_route_lora_w4g64_bf16(stream, w, scales, biases, x, y, K, N, M, w_deq, expand, lora_a, lora_b, r,
+                                               alpha, lora_t_ws);
+  }
+  int st = format == VPQ_FORMAT_W4G32   ? check_pack_g32(w, scales, biases, K, N, false)
+           : format == VPQ_FORMAT_W8G64 ? check_pack(w, scales, biases, K, N)
+           : format == VPQ_FORMAT_W8G32 ? check_pack_w8g32(w, scales, biases, K, N)
+                                        : VPQ_ERR_BAD_SHAPE;
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (w_deq == nullptr) { return VPQ_ERR_WORKSPACE; }
+  if (M <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  const bool lora = lora_a != nullptr && alpha != 0.0f;
+  if (lora) {
+    if (lora_b == nullptr) { return VPQ_ERR_NULL_POINTER; }
+    if (lora_t_ws == nullptr) { return VPQ_ERR_WORKSPACE; }
+    // the pre-pass walks K in chunks of 64
+    if (r < 8 || r > vpq::kLoraMaxRank || (r % 8) != 0 || (K % 64) != 0) { return VPQ_ERR_BAD_SHAPE; }
+    if (!aligned(lora_a, 16) || !aligned(lora_b, 16) || !aligned(lora_t_ws, 16)) { return VPQ_ERR_MISALIGNED; }
+  }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (lora) {
+    st = finish(vpq::launch_lora_a(hs, x, lora_a, lora_t_ws, M, K, r, alpha));
+    if (st != VPQ_OK) { return st; }
+  }
+  if (expand != 0) {
+    st = finish(format == VPQ_FORMAT_W4G32   ? vpq::launch_dequant_g32(hs, w, scales, biases, w_deq, K, N)
+                : format == VPQ_FORMAT_W8G64 ? vpq::launch_dequant8(hs, w, scales, biases, w_deq, K, N)
+                                             : vpq::launch_dequant8(hs, w, scales, biases, w_deq, K, N, 32));
+    if (st != VPQ_OK) { return st; }
+  }
+  std::string why;
+  const int rc = vpq::dense_gemm_elt(hs, x, w_deq, y, M, N, K, false, g_dev.cu_count, &why, lora ? lora_t_ws : nullptr,
+                                     lora ? lora_b : nullptr, lora ? r : 0);
+  if (rc != 0) {
+    strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
+    g_last_error[sizeof(g_last_error) - 1] = '\0';
+    return VPQ_ERR_DEVICE;
+  }
+  return VPQ_OK;
+}
+
 size_t vpq_weight_bytes(int N, int K) { return (size_t)N * (size_t)(K * 4 / 32) * 4; }
 size_t vpq_scale_bytes(int N, int K) { return (size_t)N * (size_t)(K / 64) * 2; }
 

@@ -903,12 +903,26 @@ void quant_linear_forward(CommandStream& stream, const Linear& lin, const Device
                          lora->strength != 0.f && !lora->a->empty() && !lora->b->empty();
   const bool w4g64 = lin.bits == 4 && lin.group == 64;
   if (!w4g64) {
-    // The format twins: their own size-based entrances; no adapter on them.
-    if (with_lora || !((lin.bits == 8 || lin.bits == 4) && (lin.group == 64 || lin.group == 32))) {
+    // The format twins: their own size-based entrances; an adapter goes by the dequant-once route (their fused
+    // kernels take none), the expansion in scratch of the stream.
+    if (!((lin.bits == 8 || lin.bits == 4) && (lin.group == 64 || lin.group == 32))) {
       stream.record_error(VPQ_ERR_BAD_SHAPE, "quant_linear_forward: pack format");
       return;
     }
-    if (lin.bits == 8 && lin.group == 32) {
+    if (with_lora) {
+      if (lora_t == nullptr || lora_t->size() < static_cast<std::size_t>(M) * lora->rank * 2) {
+        stream.record_error(VPQ_ERR_WORKSPACE, "quant_linear_forward: lora_t scratch too small");
+        return;
+      }
+      const int format = lin.bits == 8 ? (lin.group == 64 ? VPQ_FORMAT_W8G64 : VPQ_FORMAT_W8G32) : VPQ_FORMAT_W4G32;
+      uint16_t* w_deq = static_cast<uint16_t*>(stream.qmv_workspace((size_t)lin.N * (size_t)lin.K * 2));
+      status = w_deq == nullptr
+                   ? VPQ_ERR_WORKSPACE
+                   : vpq_qmm_dense_route_lora_bf16(st, format, w, sc, bi, xp, yp, lin.K, lin.N, M, w_deq, 1,
+                                                   static_cast<const uint16_t*>(lora->a->data()),
+                                                   static_cast<const uint16_t*>(lora->b->data()), lora->rank,
+                                                   lora->strength, static_cast<uint16_t*>(lora_t->data()));
+    } else if (lin.bits == 8 && lin.group == 32) {
       // 8-bit codes in groups of 32: the GEMV in slabs of 16 rows up to 64 rows, the dequant-once route above (its
       // expansion in scratch of the stream), which is the route the reference's codec takes for this format
       status = VPQ_OK;

@@ -273,7 +273,7 @@ struct Linear {
   const DeviceBuffer* qbias = nullptr;
   std::size_t codes_off = 0, scales_off = 0, qbias_off = 0;
   int K = 0, N = 0;
-  int bits = 4, group = 64;          // (4, 64), (8, 64) or (4, 32): the pack formats the library serves
+  int bits = 4, group = 64;          // (4, 64), (8, 64), (4, 32) or (8, 32): the pack formats the library serves
 };
 
 struct LoraFactors {
