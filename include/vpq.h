@@ -759,6 +759,16 @@ int vpq_qmv_qkv_rms_bf16(vpq_stream_t stream, int format, int count, const uint3
                          const uint16_t* const* scales, const uint16_t* const* biases, const uint16_t* x,
                          const uint16_t* norm_w, uint16_t* const* y, int K, const int* N, float eps,
                          uint16_t* x_norm_ws);
+/* 8-bit codes on IEEE binary16 elements -- the half build of `affine_dequant_w8g64` / `affine_dequant_w8g32`
+ * (affine_dequant.metal:60-131) and of `affine_qmm_steel_w8g64` / `_w8g32` (affine_qmm_steel.metal:1601-1698), which is
+ * what the reference's codec runs (moss/metal-moss-codec.cc:181-183, 579-581): scales, biases, x, y and w_deq are
+ * binary16, group is 64 or 32.  The expansion is bit-exact (f16(fp32(s q + b)), the product exact); the GEMM goes by the
+ * dequant-once route on the binary16 dense GEMM (arguments of vpq_qmm_dense_route_w4g64_f16). */
+int vpq_dequant_w8_f16(vpq_stream_t stream, int group, const uint32_t* w, const uint16_t* scales,
+                       const uint16_t* biases, uint16_t* w_deq, int K, int N);
+int vpq_qmm_dense_route_w8_f16(vpq_stream_t stream, int group, const uint32_t* w, const uint16_t* scales,
+                               const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                               uint16_t* w_deq, int expand);
 /* The dequant-once route with the runtime adapter over a pack of any format (VPQ_FORMAT_*: the 4-bit group-64 form is
  * vpq_qmm_dense_route_lora_w4g64_bf16, whose arguments these are): the adapter's pre-pass into lora_t_ws, the format's
  * expansion into w_deq (expand != 0) or the kept one, then the dense GEMM with t . B^T in the same accumulators -- the

@@ -374,6 +374,14 @@ def dequant8_g32(w, s, b, K, N):
     return out
 
 
+def dequant8_f16(w, s, b, K, N, group=64):
+    """8-bit codes, binary16 scales / biases [N, K/group] -> binary16 bits [N, K]."""
+    w, s, b = _c(w, np.uint32), _c(s, np.uint16), _c(b, np.uint16)
+    out = np.empty((N, K), dtype=np.uint16)
+    lib().vpo_dequant_w8_f16(_p(w, _u32p), _p(s, _u16p), _p(b, _u16p), _p(out, _u16p), K, N, group)
+    return out
+
+
 def requant_w8_to_w4(w8, s8, b8, K, N):
     """8-bit group-64 pack -> 4-bit group-64 pack (codes u32 [N, K/8], scales, biases bf16 bits [N, K/64])."""
     w8, s8, b8 = _c(w8, np.uint32), _c(s8, np.uint16), _c(b8, np.uint16)

@@ -784,6 +784,23 @@ void vpo_dequant_w4g64_f16(const uint32_t* w, const uint16_t* scales, const uint
   }
 }
 
+/* The half build of affine_dequant_w8g64 / _w8g32 (affine_dequant.metal:60-131 with VPIPE_ELT = half): one byte per
+ * value, binary16 scales and biases, out = f16(fp32(s * q + b)); the product is exact (11 x 8 bit significands). */
+void vpo_dequant_w8_f16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                        uint16_t* out, int K, int N, int group)
+{
+  const int Kw = K / 4, Kg = K / group;
+  for (size_t n = 0; n < (size_t)N; ++n) {
+    for (int k = 0; k < K; ++k) {
+      const float s = vpo_f16_to_f32(scales[n * Kg + k / group]);
+      const float b = vpo_f16_to_f32(biases[n * Kg + k / group]);
+      const uint32_t q = (w[n * Kw + k / 4] >> (8 * (k & 3))) & 0xffu;
+      const float sq = s * (float)q;
+      out[n * (size_t)K + k] = vpo_f32_to_f16(sq + b);
+    }
+  }
+}
+
 /* rounded != 0: the GEMM's weights, rounded to binary16 before the contraction; 0: the GEMV's. */
 void vpo_matmul_w4g64_f16(const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
                           const uint16_t* x, double* y64, uint16_t* y_f16,

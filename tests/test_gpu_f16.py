@@ -276,3 +276,40 @@ def test_f16_entries_reject_bad_arguments(vpq, dev):
     assert L.vpq_qmv_w4g64_f16(None, p, p, p, p, p, 64, 8, 17, None) == -2
     assert L.vpq_qmv_gated_w4g64_f16(None, p, p, p, p, p, 64, 7, 1, 1) == -2
     assert L.vpq_qmm_dense_route_w4g64_f16(None, p, p, p, p, p, 64, 8, 4, None, 1) == -4
+
+
+@pytest.mark.parametrize("group", [64, 32])
+@pytest.mark.parametrize("M,N,K", [(1, 8, 64), (70, 136, 320), (300, 264, 1024)])
+def test_w8_on_binary16_elements_expansion_and_dense_route(vpq, oracle, dev, D, group, M, N, K):
+    """The half build's affine_dequant_w8g64 / _w8g32 and affine_qmm_steel_w8g64 / _w8g32 (what the reference's codec
+    runs, moss/metal-moss-codec.cc:181-183, 579-581): the expansion bit for bit against the oracle, the GEMM by the
+    dequant-once route against float64 of x . W^T with W that expansion, the kept expansion the same bits."""
+    rng = np.random.default_rng(9300 + M + group)
+    w = rng.integers(0, 2**32, size=(N, K // 4), dtype=np.uint32)
+    s = rng.uniform(0.0003, 0.0012, size=(N, K // group)).astype(np.float16)
+    b = (-128.0 * s.astype(np.float32) * rng.uniform(0.9, 1.1, size=s.shape)).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    dense = oracle.dequant8_f16(w, s.view(np.uint16), b.view(np.uint16), K, N, group=group)
+    wd = torch.from_numpy(w.view(np.int32)).to(dev)
+    sd, bd, xd = torch.from_numpy(s).to(dev), torch.from_numpy(b).to(dev), torch.from_numpy(x).to(dev)
+    got = vpq.dequant_w8_f16(wd, sd, bd, K, N, group=group)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), dense)
+    w_deq = torch.empty((N, K), dtype=torch.float16, device=dev)
+    out = parity.Guarded((M, N), torch.float16, dev)
+    vpq.qmm_dense_route_w8_f16(wd, sd, bd, xd, K, N, M, w_deq, group=group, out=out.view)
+    torch.cuda.synchronize()
+    out.assert_intact()
+    assert np.array_equal(w_deq.cpu().numpy().view(np.uint16), dense)
+    want = x.astype(np.float64) @ dense.view(np.float16).astype(np.float64).T
+    y = out.view.cpu().numpy().astype(np.float64)
+    # one binary16 rounding of an fp32 sum: 2^-11 relative, plus the sum's own error where it cancels
+    mag = np.abs(x.astype(np.float64)) @ np.abs(dense.view(np.float16).astype(np.float64)).T
+    assert (np.abs(y - want) <= 2.0 ** -11 * np.abs(want) + 64 * 2.0 ** -24 * mag + 2.0 ** -24).all()
+    kept = vpq.qmm_dense_route_w8_f16(wd, sd, bd, xd, K, N, M, w_deq, group=group, expand=False)
+    assert torch.equal(kept, out.view)
+    L = vpq.load()
+    p = out.view.data_ptr()
+    assert L.vpq_dequant_w8_f16(None, 48, p, p, p, p, K, N) == -2
+    assert L.vpq_qmm_dense_route_w8_f16(None, group, p, p, p, p, p, K, N, M, None, 1) == -4
+    assert L.vpq_qmm_dense_route_w8_f16(None, group, p, p, p, p, p, K + 8, N, M, p, 1) == -2

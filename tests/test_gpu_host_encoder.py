@@ -308,6 +308,42 @@ def test_quant_linear_forward_with_lora_over_the_format_twins(vpq, enc, dev, D, 
     assert yd.abs().sum() > 0
 
 
+@pytest.mark.parametrize("group", [64, 32])
+def test_eight_bit_functions_of_the_binary16_libraries(vpq, enc, dev, D, group):
+    # the codec's call sites (generative-models/moss/metal-moss-codec.cc:181-183, 579-581): affine_dequant_w8g32 of
+    # library "affine_dequant" (0:w 1:scales 2:biases 3:w_deq 4:K 5:N) and affine_qmm_steel_w8g32 of "affine_qmm_steel"
+    # (the GEMM slots, 7 = M), and their group-64 twins: the C ABI's results, bit for bit
+    K, N, M = 512, 72, 90
+    rng = np.random.default_rng(4400 + group)
+    w = rng.integers(0, 2**32, size=(N, K // 4), dtype=np.uint32)
+    s = rng.uniform(0.0003, 0.0012, size=(N, K // group)).astype(np.float16)
+    b = (-128.0 * s.astype(np.float32)).astype(np.float16)
+    x = rng.standard_normal((M, K)).astype(np.float16)
+    wd = torch.from_numpy(w.view(np.int32)).to(dev)
+    sd, bd, xd = torch.from_numpy(s).to(dev), torch.from_numpy(b).to(dev), torch.from_numpy(x).to(dev)
+    dq = torch.zeros((N, K), dtype=torch.float16, device=dev)
+    y = torch.zeros((M, N), dtype=torch.float16, device=dev)
+    assert enc.set_function("affine_dequant", "affine_dequant_w8g%d" % group) == 1
+    for i, t in enumerate((wd, sd, bd, dq)):
+        enc.set_buffer(i, t)
+    enc.set_constant(4, K)
+    enc.set_constant(5, N)
+    enc.dispatch((K // 4, N, 1), (64, 1, 1))
+    assert enc.set_function("affine_qmm_steel", "affine_qmm_steel_w8g%d" % group) == 1
+    for i, t in enumerate((wd, sd, bd, xd, y)):
+        enc.set_buffer(i, t)
+    enc.set_constant(5, K)
+    enc.set_constant(6, N)
+    enc.set_constant(7, M)
+    enc.dispatch((N, M, 2), (32, 2, 2))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    assert torch.equal(dq, vpq.dequant_w8_f16(wd, sd, bd, K, N, group=group))
+    w_deq = torch.empty((N, K), dtype=torch.float16, device=dev)
+    assert torch.equal(y, vpq.qmm_dense_route_w8_f16(wd, sd, bd, xd, K, N, M, w_deq, group=group))
+    assert dq.abs().sum() > 0 and y.abs().sum() > 0
+
+
 def test_fused_qkv_call_site(enc, oracle, dev, D):
     # llama decode: one dispatch over the row-concatenated q|k|v pack, three output buffers
     # (gpu-kernels/metal/quant/affine_qmv.metal:405-516)

@@ -601,6 +601,22 @@ def test_f16_element_twins_against_numpy_float16(oracle):
     assert np.array_equal(ya, want_add.view(np.uint16))
 
 
+def test_w8_expansion_on_binary16_elements_against_numpy_float16(oracle):
+    """The half build's 8-bit expansion (groups of 64 and of 32): numpy's float16 arithmetic from the byte view of the
+    words -- a float32 multiply-add whose product is exact, numpy's round-to-nearest-even cast."""
+    rng = np.random.default_rng(44)
+    for group in (64, 32):
+        N, K = 13, 256
+        w = rng.integers(0, 2**32, size=(N, K // 4), dtype=np.uint32)
+        s = rng.uniform(0.0003, 0.0012, size=(N, K // group)).astype(np.float16)
+        b = (-128.0 * s.astype(np.float32) * rng.uniform(0.9, 1.1, size=s.shape)).astype(np.float16)
+        q = w.view(np.uint8).reshape(N, K).astype(np.float32)          # little-endian bytes = values in k order
+        dense32 = np.repeat(s.astype(np.float32), group, axis=1) * q + np.repeat(b.astype(np.float32), group, axis=1)
+        got = oracle.dequant8_f16(w, s.view(np.uint16), b.view(np.uint16), K, N, group=group)
+        assert np.array_equal(got, dense32.astype(np.float16).view(np.uint16))
+        assert np.abs(dense32).max() > 0
+
+
 def test_f16_adapter_against_numpy_float16(oracle):
     """The adapter on binary16 elements, written independently in numpy: t = f16(alpha * f16(x . A^T)) with the
     contraction in float64 and numpy's own float16 casts, then y = f16(x . f16(W)^T + t . B^T); an adapter whose t is

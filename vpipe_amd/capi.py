@@ -78,6 +78,8 @@ SYMBOLS = [
     ("vpq_qmv_gelu_mul_w4g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _i]),
     ("vpq_qmm_dense_route_w8g32_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_qmv_qkv_rms_bf16", _i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _f, _vp]),
+    ("vpq_dequant_w8_f16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i]),
+    ("vpq_qmm_dense_route_w8_f16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_qmm_dense_route_lora_bf16", _i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _f, _vp]),
     ("vpq_interleave_rows", _i, [_vp, _vp, _vp, _vp, _sz, _sz]),
     ("vpq_qmv_swiglu_w4g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
@@ -988,4 +990,23 @@ def qmm_dense_route_lora(fmt, w, scales, biases, x, K, N, M, w_deq, lora_A, lora
     _check(load().vpq_qmm_dense_route_lora_bf16(_stream(), fmt, _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N,
                                                 M, _ptr(w_deq), 1 if expand else 0, _ptr(lora_A), _ptr(lora_B), r, alpha,
                                                 _ptr(t_ws)), "vpq_qmm_dense_route_lora_bf16")
+    return out
+
+
+def dequant_w8_f16(w, scales, biases, K, N, group=64, out=None):
+    """8-bit codes, binary16 scales / biases -> binary16 [N, K]."""
+    import torch
+    if out is None:
+        out = torch.empty((N, K), dtype=torch.float16, device=w.device)
+    _check(load().vpq_dequant_w8_f16(_stream(), group, _ptr(w), _ptr(scales), _ptr(biases), _ptr(out), K, N),
+           "vpq_dequant_w8_f16")
+    return out
+
+
+def qmm_dense_route_w8_f16(w, scales, biases, x, K, N, M, w_deq, group=64, expand=True, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=w.device)
+    _check(load().vpq_qmm_dense_route_w8_f16(_stream(), group, _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
+                                             _ptr(w_deq), 1 if expand else 0), "vpq_qmm_dense_route_w8_f16")
     return out

@@ -1806,6 +1806,49 @@ int vpq_profile_read(float* kernel_ms, int capacity)
   return n;
 }
 
+// 8-bit codes on IEEE binary16 elements (the half build's affine_dequant_w8g64 / _w8g32 and affine_qmm_steel_w8g64 /
+// _w8g32): the expansion, and the GEMM by the dequant-once route on the binary16 dense GEMM.
+int vpq_dequant_w8_f16(vpq_stream_t stream, int group, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
+                       uint16_t* w_deq, int K, int N)
+{
+  if (group != 64 && group != 32) { return VPQ_ERR_BAD_SHAPE; }
+  int st = group == 64 ? check_pack(w, scales, biases, K, N) : check_pack_w8g32(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (w_deq == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (!aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_dequant8(reinterpret_cast<hipStream_t>(stream), w, scales, biases, w_deq, K, N, group, true));
+}
+
+int vpq_qmm_dense_route_w8_f16(vpq_stream_t stream, int group, const uint32_t* w, const uint16_t* scales,
+                               const uint16_t* biases, const uint16_t* x, uint16_t* y, int K, int N, int M,
+                               uint16_t* w_deq, int expand)
+{
+  if (group != 64 && group != 32) { return VPQ_ERR_BAD_SHAPE; }
+  int st = group == 64 ? check_pack(w, scales, biases, K, N) : check_pack_w8g32(w, scales, biases, K, N);
+  if (st != VPQ_OK) { return st; }
+  if (x == nullptr || y == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if (w_deq == nullptr) { return VPQ_ERR_WORKSPACE; }
+  if (M <= 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(w_deq, 16)) { return VPQ_ERR_MISALIGNED; }
+  st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  if (expand != 0) {
+    st = finish(vpq::launch_dequant8(hs, w, scales, biases, w_deq, K, N, group, true));
+    if (st != VPQ_OK) { return st; }
+  }
+  std::string why;
+  const int rc = vpq::dense_gemm_elt(hs, x, w_deq, y, M, N, K, true, g_dev.cu_count, &why);
+  if (rc != 0) {
+    strncpy(g_last_error, why.c_str(), sizeof(g_last_error) - 1);
+    g_last_error[sizeof(g_last_error) - 1] = '\0';
+    return VPQ_ERR_DEVICE;
+  }
+  return VPQ_OK;
+}
+
 // The dequant-once route with the runtime adapter for any of the pack formats: the adapter's pre-pass, the format's
 // expansion (or the kept one), the dense GEMM with t . B^T in the same accumulators.
 int vpq_qmm_dense_route_lora_bf16(vpq_stream_t stream, int format, const uint32_t* w, const uint16_t* scales,

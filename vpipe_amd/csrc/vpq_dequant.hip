@@ -73,7 +73,9 @@ hipError_t launch_dequant_g32(hipStream_t st, const uint32_t* w, const uint16_t*
 // 8-bit twin (gpu-kernels/metal/quant/affine_dequant.metal:60-97): one byte per value, four per word;
 // one thread per word, 8-byte stores.  s*q is exact in fp32 (8-bit x 8-bit significands).  WS: log2 of the words
 // per quantization group (4: group 64; 3: group 32, affine_dequant_w8g32, :99-131).
-template <int WS>
+// F16: scales, biases and the output are IEEE binary16 (the reference's VPIPE_ELT = half build, which is what its
+// codec runs this expansion in); s*q stays exact in fp32 (11-bit x 8-bit significands).
+template <int WS, bool F16 = false>
 __global__ __launch_bounds__(256) void dequant_w8_kernel(
     const uint32_t* __restrict__ w, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, uint2* __restrict__ out, int Kw, size_t total_words)
@@ -83,29 +85,31 @@ __global__ __launch_bounds__(256) void dequant_w8_kernel(
     const size_t n = idx / (size_t)Kw;
     const int j = (int)(idx - n * (size_t)Kw);
     const size_t g = n * (size_t)Kg + (size_t)(j >> WS);
-    const float s = bf16_bits_to_f32(scales[g]);
-    const float b = bf16_bits_to_f32(biases[g]);
+    const float s = elt_bits_to_f32<F16>(scales[g]);
+    const float b = elt_bits_to_f32<F16>(biases[g]);
     const uint32_t p = w[idx];
     uint2 o;
-    o.x = pack_bf16x2(fmaf(s, (float)(p & 0xffu), b), fmaf(s, (float)((p >> 8) & 0xffu), b));
-    o.y = pack_bf16x2(fmaf(s, (float)((p >> 16) & 0xffu), b), fmaf(s, (float)(p >> 24), b));
+    o.x = pack_elt2<F16>(fmaf(s, (float)(p & 0xffu), b), fmaf(s, (float)((p >> 8) & 0xffu), b));
+    o.y = pack_elt2<F16>(fmaf(s, (float)((p >> 16) & 0xffu), b), fmaf(s, (float)(p >> 24), b));
     out[idx] = o;
   }
 }
 
 hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                           uint16_t* out, int K, int N, int group)
+                           uint16_t* out, int K, int N, int group, bool f16)
 {
   const int Kw = K / 4;
   const size_t total = (size_t)N * (size_t)Kw;
   size_t blocks = (total + 255) / 256;
   if (blocks > 65536 * 4) { blocks = 65536 * 4; }
+  const dim3 grid((unsigned)blocks), block(256);
+  uint2* o = reinterpret_cast<uint2*>(out);
   if (group == 32) {
-    return launch_kernel(dequant_w8_kernel<3>, dim3((unsigned)blocks), dim3(256), 0, st, w, scales, biases,
-                         reinterpret_cast<uint2*>(out), Kw, total);
+    return f16 ? launch_kernel(dequant_w8_kernel<3, true>, grid, block, 0, st, w, scales, biases, o, Kw, total)
+               : launch_kernel(dequant_w8_kernel<3>, grid, block, 0, st, w, scales, biases, o, Kw, total);
   }
-  return launch_kernel(dequant_w8_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, st, w, scales, biases,
-                       reinterpret_cast<uint2*>(out), Kw, total);
+  return f16 ? launch_kernel(dequant_w8_kernel<4, true>, grid, block, 0, st, w, scales, biases, o, Kw, total)
+             : launch_kernel(dequant_w8_kernel<4>, grid, block, 0, st, w, scales, biases, o, Kw, total);
 }
 
 // 8-bit -> 4-bit requantizer (affine_requant_w8_to_w4_g64, gpu-kernels/metal/quant/affine_dequant.metal:134-186): one

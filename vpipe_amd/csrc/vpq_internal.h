@@ -141,7 +141,7 @@ hipError_t launch_qmv_simple_g32(hipStream_t st, const QmvArgs& a, bool scale_on
 hipError_t launch_qmv_rows_g32(hipStream_t st, const QmvArgs& a, bool scale_only);   // M <= 2
 // The 8-bit twins (one byte per value, w is [N, K/4] words): dense expansion and the general QMV kernel.
 hipError_t launch_dequant8(hipStream_t st, const uint32_t* w, const uint16_t* scales, const uint16_t* biases,
-                           uint16_t* out, int K, int N, int group = 64);
+                           uint16_t* out, int K, int N, int group = 64, bool f16 = false);
 hipError_t launch_qmv_simple8(hipStream_t st, const QmvArgs& a, int group = 64);
 // 8-bit group-64 pack -> 4-bit group-64 pack of the same shape (one thread per group).
 hipError_t launch_requant_w8_to_w4(hipStream_t st, const uint32_t* w8, const uint16_t* s8, const uint16_t* b8,

@@ -164,6 +164,11 @@ const FnEntry kFunctions[] = {
     // IEEE binary16 build (VPIPE_ELT = half; generative-models/qwen3/metal-qwen-model.cc:771-772: the library
     // names without the suffix)
     {"affine_dequant", "affine_dequant_w4g64", QuantKernel::Dequant, QuantFormat::W4G64F16},
+    // the 8-bit functions of the binary16 build (the codec's: generative-models/moss/metal-moss-codec.cc:181-183, 579-581)
+    {"affine_dequant", "affine_dequant_w8g64", QuantKernel::Dequant, QuantFormat::W8G64F16},
+    {"affine_dequant", "affine_dequant_w8g32", QuantKernel::Dequant, QuantFormat::W8G32F16},
+    {"affine_qmm_steel", "affine_qmm_steel_w8g64", QuantKernel::Qmm, QuantFormat::W8G64F16},
+    {"affine_qmm_steel", "affine_qmm_steel_w8g32", QuantKernel::Qmm, QuantFormat::W8G32F16},
     {"affine_qmv", "affine_qmv_w4g64", QuantKernel::Qmv, QuantFormat::W4G64F16},
     {"affine_qmv", "affine_qmv_w4g64_add", QuantKernel::QmvAdd, QuantFormat::W4G64F16},
     {"affine_qmv", "affine_qmv_swiglu_w4g64", QuantKernel::QmvSwiglu, QuantFormat::W4G64F16},
@@ -481,6 +486,9 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
         status = VPQ_ERR_NULL_POINTER;
       } else if (fmt == QuantFormat::W4G64F16) {
         status = vpq_dequant_w4g64_f16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
+      } else if (fmt == QuantFormat::W8G64F16 || fmt == QuantFormat::W8G32F16) {
+        status = vpq_dequant_w8_f16(st, fmt == QuantFormat::W8G64F16 ? 64 : 32, w, sc, bi, static_cast<uint16_t*>(buf(3)),
+                                    ival(4), ival(5));
       } else if (fmt == QuantFormat::W8G64) {
         status = vpq_dequant_w8g64_bf16(st, w, sc, bi, static_cast<uint16_t*>(buf(3)), ival(4), ival(5));
       } else if (fmt == QuantFormat::W8G32) {
@@ -589,6 +597,15 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
                                           kind == QuantKernel::QmvGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
       } else if (fmt == QuantFormat::W8G64) {
         status = vpq_qmv_w8g64_bf16(st, w, sc, bi, x, y, K, N, M, residual);
+      } else if ((fmt == QuantFormat::W8G64F16 || fmt == QuantFormat::W8G32F16) && kind == QuantKernel::Qmm) {
+        // the binary16 build's 8-bit GEMM, slot 7 = M: the dequant-once route on the binary16 dense GEMM
+        uint16_t* w_deq = (in_scope || K <= 0 || N <= 0)
+                              ? nullptr
+                              : static_cast<uint16_t*>(s->qmv_workspace(static_cast<std::size_t>(N) * static_cast<std::size_t>(K) * 2));
+        status = !has_int(7) ? VPQ_ERR_NULL_POINTER
+                             : (w_deq == nullptr ? VPQ_ERR_WORKSPACE
+                                                 : vpq_qmm_dense_route_w8_f16(st, fmt == QuantFormat::W8G64F16 ? 64 : 32, w, sc, bi, x,
+                                                                              y, K, N, ival(7), w_deq, 1));
       } else if (fmt == QuantFormat::W8G32 && kind == QuantKernel::Qmm) {
         // gpu-kernels/metal/quant/affine_qmm_steel.metal:1674-1698, slot 7 = M: the dequant-once route, the
         // expansion in scratch of the stream (shared, so not inside a concurrent scope)

@@ -115,6 +115,8 @@ enum class QuantFormat : std::uint8_t {
   W4G32Q40,       // _w4g32_q40 / _w4g32_add_q40: as W4G32 with the bias buffer never read (bias = -8 * scale)
   W8G32,          // _w8g32: one byte per value, a scale and a bias per 32 values
   W4G64F16,       // the metallibs without the `_bf16` suffix ("affine_qmv", "affine_dequant"): IEEE binary16 elements
+  W8G64F16,       // ... their 8-bit functions (expansion and GEMM)
+  W8G32F16,
 };
 
 class QuantFunction {
