@@ -789,6 +789,12 @@ int vpq_qmm_dense_route_lora_bf16(vpq_stream_t stream, int format, const uint32_
  * F16 bit patterns, the on-disk format.  `src` is bf16 [N,K]. */
 int vpq_quantize_w4g64(vpq_stream_t stream, const uint16_t* src, uint32_t* w,
                        uint16_t* scales_f16, uint16_t* biases_f16, int K, int N, float clip);
+/* The same packer for every width and group of the reference (`affine_quant_w4_g64`, `_w4_g32`, `_w8_g64`, `_w8_g32`,
+ * affine_dequant.metal:243-301): bits 4 or 8, group 64 or 32, scale = (max - min) / (2^bits - 1); w is
+ * [N, K * bits / 32] words, scales / biases F16 [N, K / group]; K % group == 0.  src_f16 != 0: `src` is IEEE binary16
+ * (the build the reference's quantizer runs, generative-models/quantize/affine-quantizer.cc:25), else bf16. */
+int vpq_quantize(vpq_stream_t stream, int bits, int group, int src_f16, const uint16_t* src, uint32_t* w,
+                 uint16_t* scales_f16, uint16_t* biases_f16, int K, int N, float clip);
 
 /* F16 -> bf16 conversion of scales / biases a bf16 model does once at load
  * (docs/PLUGINS.md:210-213). */

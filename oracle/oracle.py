@@ -393,14 +393,14 @@ def requant_w8_to_w4(w8, s8, b8, K, N):
     return w4, s4, b4
 
 
-def quantize(wsrc, K, N, clip=1.0):
-    """fp32 [N,K] -> (codes u32 [N,K/8], scales f16 bits [N,K/64], biases f16 bits)."""
+def quantize(wsrc, K, N, clip=1.0, bits=4, group=64):
+    """fp32 [N,K] -> (codes u32 [N, K*bits/32], scales f16 bits [N, K/group], biases f16 bits)."""
     wsrc = _c(wsrc, np.float32)
-    codes = np.empty((N, K // 8), dtype=np.uint32)
-    s = np.empty((N, K // 64), dtype=np.uint16)
-    b = np.empty((N, K // 64), dtype=np.uint16)
-    lib().vpo_quantize_w4g64(_p(wsrc, _f32p), _p(codes, _u32p), _p(s, _u16p), _p(b, _u16p),
-                             K, N, ctypes.c_float(clip))
+    codes = np.empty((N, K * bits // 32), dtype=np.uint32)
+    s = np.empty((N, K // group), dtype=np.uint16)
+    b = np.empty((N, K // group), dtype=np.uint16)
+    lib().vpo_quantize(_p(wsrc, _f32p), _p(codes, _u32p), _p(s, _u16p), _p(b, _u16p),
+                       K, N, ctypes.c_float(clip), bits, group)
     return codes, s, b
 
 

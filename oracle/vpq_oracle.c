@@ -1018,15 +1018,17 @@ void vpo_qmm_grouped_w8g64(const uint32_t* w, const uint16_t* scales, const uint
  * round() = half away from zero (C roundf), scale and mn emitted as F16.
  * Host twin: generative-models/quantize/model-quantizer.cc:240-264 (lround).
  * Input is fp32 here (the kernel widens its f16/bf16 input to float first). */
-void vpo_quantize_w4g64(const float* wsrc, uint32_t* codes, uint16_t* scales_f16,
-                        uint16_t* biases_f16, int K, int N, float clip)
+/* Every width and group (affine_quant_impl<BITS, GROUP>, :243-301: bits 4 or 8, group 64 or 32). */
+void vpo_quantize(const float* wsrc, uint32_t* codes, uint16_t* scales_f16, uint16_t* biases_f16, int K, int N,
+                  float clip, int bits, int group)
 {
-  const int Kw = K / 8, Kg = K / VPO_GROUP;
+  const int vpw = 32 / bits, wpg = group / vpw, qmax = (1 << bits) - 1;
+  const int Kw = K / vpw, Kg = K / group;
   for (size_t n = 0; n < (size_t)N; ++n) {
     for (int g = 0; g < Kg; ++g) {
-      const float* xp = wsrc + n * (size_t)K + (size_t)g * VPO_GROUP;
+      const float* xp = wsrc + n * (size_t)K + (size_t)g * group;
       float mn = INFINITY, mx = -INFINITY;
-      for (int i = 0; i < VPO_GROUP; ++i) {
+      for (int i = 0; i < group; ++i) {
         mn = fminf(mn, xp[i]);
         mx = fmaxf(mx, xp[i]);
       }
@@ -1035,21 +1037,27 @@ void vpo_quantize_w4g64(const float* wsrc, uint32_t* codes, uint16_t* scales_f16
         mn = mid + (mn - mid) * clip;
         mx = mid + (mx - mid) * clip;
       }
-      const float scale = (mx - mn) / 15.0f;
+      const float scale = (mx - mn) / (float)qmax;
       const float inv = (scale > 0.0f) ? 1.0f / scale : 0.0f;
       scales_f16[n * Kg + g] = vpo_f32_to_f16(scale);
       biases_f16[n * Kg + g] = vpo_f32_to_f16(mn);
-      for (int wi = 0; wi < VPO_GROUP / 8; ++wi) {
+      for (int wi = 0; wi < wpg; ++wi) {
         uint32_t packed = 0;
-        for (int i = 0; i < 8; ++i) {
-          int q = (int)roundf((xp[wi * 8 + i] - mn) * inv);
-          q = q < 0 ? 0 : (q > 15 ? 15 : q);
-          packed |= (uint32_t)q << (4 * i);
+        for (int i = 0; i < vpw; ++i) {
+          int q = (int)roundf((xp[wi * vpw + i] - mn) * inv);
+          q = q < 0 ? 0 : (q > qmax ? qmax : q);
+          packed |= (uint32_t)q << (bits * i);
         }
-        codes[n * (size_t)Kw + (size_t)g * (VPO_GROUP / 8) + wi] = packed;
+        codes[n * (size_t)Kw + (size_t)g * wpg + wi] = packed;
       }
     }
   }
+}
+
+void vpo_quantize_w4g64(const float* wsrc, uint32_t* codes, uint16_t* scales_f16,
+                        uint16_t* biases_f16, int K, int N, float clip)
+{
+  vpo_quantize(wsrc, codes, scales_f16, biases_f16, K, N, clip, 4, VPO_GROUP);
 }
 
 /* Output byte sizes, generative-models/quantize/affine-quantizer.h:37-40. */

@@ -176,6 +176,32 @@ def test_packer_matches_the_oracle_bit_for_bit(vpq, oracle, dev, D, kind, N, K, 
         assert not s16.reshape(N, K // 64)[:, 0::2].any()
 
 
+@pytest.mark.parametrize("bits,group", [(4, 64), (4, 32), (8, 64), (8, 32)])
+@pytest.mark.parametrize("kind,N,K,clip,f16", [("gauss", 96, 1024, 1.0, False), ("gauss", 33, 320, 0.9, True),
+                                               ("outliers", 257, 2048, 0.75, False), ("constant", 48, 1024, 1.0, True)])
+def test_packer_at_every_width_and_group(vpq, oracle, dev, D, bits, group, kind, N, K, clip, f16):
+    # affine_quant_w4_g64 / _w4_g32 / _w8_g64 / _w8_g32 (gpu-kernels/metal/quant/affine_dequant.metal:243-301) over a
+    # bf16 or a binary16 source: codes, F16 scales and F16 zero points bit for bit against the oracle
+    v = _packer_case(kind, N, K, 700 + N + K + bits + group)
+    if f16:
+        v = v.astype(np.float16).astype(np.float32)
+        src = torch.from_numpy(v.astype(np.float16)).to(dev)
+    else:
+        src = D.bf16(synth.f32_to_bf16_bits(v), dev)
+    codes, s16, b16 = oracle.quantize(v, K, N, clip=clip, bits=bits, group=group)
+    wd, sd, bd = vpq.quantize(src, K, N, bits=bits, group=group, clip=clip)
+    torch.cuda.synchronize()
+    assert np.array_equal(wd.cpu().numpy().view(np.uint32), codes)
+    assert np.array_equal(sd.cpu().numpy().view(np.uint16), s16)
+    assert np.array_equal(bd.cpu().numpy().view(np.uint16), b16)
+    assert codes.any() or kind == "constant"
+    L = vpq.load()
+    p = src.data_ptr()
+    assert L.vpq_quantize(None, 5, group, 0, p, p, p, p, K, N, 1.0) == -2
+    assert L.vpq_quantize(None, bits, 48, 0, p, p, p, p, K, N, 1.0) == -2
+    assert L.vpq_quantize(None, bits, group, 0, p, p, p, p, K + 8, N, 1.0) == -2
+
+
 FLOW_SHAPES = [
     # K, N: one to nine slices of 2048, K not a multiple of 2048 (idle lanes in the last slice), every plan of
     # slices per wavefront x K parts (2560: 2x1, 4096: 2x1, 5120: 3x1, 8192: 4x1, 12288: 3x2, 14336: 4x2, 17408: 3x3),

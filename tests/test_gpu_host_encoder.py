@@ -344,6 +344,75 @@ def test_eight_bit_functions_of_the_binary16_libraries(vpq, enc, dev, D, group):
     assert dq.abs().sum() > 0 and y.abs().sum() > 0
 
 
+def test_batched_gemv_names_of_every_tiling_and_format(vpq, enc, dev, D):
+    # gpu-kernels/metal/quant/affine_qmv.metal:1674-2549, 2725-2745, 2854-2872, 3003-3026: the batched GEMVs (rows =
+    # m_total in slot 7, grid {32, N/4, ceil(m_total / MAXM)}) in their tilings, gated forms and pack formats are the
+    # C ABI's QMV over m_total rows, bit for bit
+    K, N = 1024, 96
+    w, s, b = synth.make_weight(N, K, 4500)
+    w8, s8, b8 = synth.make_weight8(N, K, 4501)
+    wg, sg, bg = synth.make_weight_g32(N, K, 4502)
+    p4 = (D.u32(w, dev), D.bf16(s, dev), D.bf16(b, dev))
+    p8 = (D.u32(w8, dev), D.bf16(s8, dev), D.bf16(b8, dev))
+    pg = (D.u32(wg, dev), D.bf16(sg, dev), D.bf16(bg, dev))
+    cases = [("affine_qmv_batch8_xh16_w4g64", p4, 8, 0), ("affine_qmv_batch8_tg4_w4g64", p4, 5, 0),
+             ("affine_qmv_batch4_swiglu_w4g64", p4, 3, 1), ("affine_qmv_batch8_xp2_swiglu_w4g64", p4, 7, 1),
+             ("affine_qmv_batch_geglu_w4g64", p4, 2, 2), ("affine_qmv_batch_w8g64", p8, 2, 0),
+             ("affine_qmv_batch8_xd_w8g64", p8, 6, 0), ("affine_qmv_batch_w4g32", pg, 2, 0),
+             ("affine_qmv_batch_geglu_w4g32", pg, 2, 2)]
+    outs = []
+    for name, pack, M, act in cases:
+        x = D.bf16(synth.make_act(M, K, 4510 + M), dev)
+        y = torch.zeros((M, N // 2 if act else N), dtype=torch.bfloat16, device=dev)
+        assert enc.set_function("affine_qmv_bf16", name) == 1, name
+        for i, t in enumerate(pack + (x, y)):
+            enc.set_buffer(i, t)
+        enc.set_constant(5, K)
+        enc.set_constant(6, N)
+        enc.set_constant(7, M)
+        enc.dispatch((32, N // 4, (M + 1) // 2), (32, 2, 1))
+        outs.append((name, pack, M, act, x, y))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    for name, pack, M, act, x, y in outs:
+        if pack is p4:
+            want = vpq.qmv_swiglu_w4g64(*pack, x, K, N, M, activation=act) if act else vpq.qmv_w4g64(*pack, x, K, N, M)
+        elif pack is p8:
+            want = vpq.qmv_w8g64(*pack, x, K, N, M)
+        else:
+            want = vpq.qmv_w4g32(*pack, x, K, N, M, activation=act)
+        assert torch.equal(y, want), name
+        assert y.abs().sum() > 0
+
+
+@pytest.mark.parametrize("lib,name,bits,group", [("affine_dequant_bf16", "affine_quant_w4_g64", 4, 64),
+                                                 ("affine_dequant", "affine_quant_w8_g32", 8, 32),
+                                                 ("affine_dequant", "affine_quant_w4_g32", 4, 32),
+                                                 ("affine_dequant_bf16", "affine_quant_w8_g64", 8, 64)])
+def test_packer_function_names(vpq, enc, dev, D, lib, name, bits, group):
+    # AffineQuantizer::quantize_linear's dispatch (generative-models/quantize/affine-quantizer.cc:52-84): 0:x 1:w
+    # 2:scales 3:biases 4:K 5:N 6:clip, grid {K / group, N, 1}; the binary16 library takes a binary16 source
+    K, N, clip = 512, 40, 0.9
+    v = np.random.default_rng(4600 + bits + group).standard_normal((N, K)).astype(np.float32) * 0.05
+    src = torch.from_numpy(v.astype(np.float16)).to(dev) if lib == "affine_dequant" else D.bf16(synth.f32_to_bf16_bits(v), dev)
+    w = torch.zeros((N, K * bits // 32), dtype=torch.int32, device=dev)
+    s = torch.zeros((N, K // group), dtype=torch.float16, device=dev)
+    b = torch.zeros((N, K // group), dtype=torch.float16, device=dev)
+    assert enc.set_function(lib, name) == 1
+    for i, t in enumerate((src, w, s, b)):
+        enc.set_buffer(i, t)
+    enc.set_constant(4, K)
+    enc.set_constant(5, N)
+    enc.L.hd_set_constant_f32.argtypes = [ctypes.c_void_p, ctypes.c_uint, ctypes.c_float]
+    enc.L.hd_set_constant_f32(enc.h, 6, clip)
+    enc.dispatch((K // group, N, 1), (K // group, 1, 1))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    want = vpq.quantize(src, K, N, bits=bits, group=group, clip=clip)
+    assert torch.equal(w, want[0]) and torch.equal(s, want[1]) and torch.equal(b, want[2])
+    assert w.abs().sum() > 0
+
+
 def test_fused_qkv_call_site(enc, oracle, dev, D):
     # llama decode: one dispatch over the row-concatenated q|k|v pack, three output buffers
     # (gpu-kernels/metal/quant/affine_qmv.metal:405-516)

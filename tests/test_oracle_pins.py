@@ -332,6 +332,49 @@ def test_quantize_roundtrip_bounds_of_the_reference(oracle):
     assert np.array_equal(sf16, sc.astype(np.float16).view(np.uint16).reshape(N, K // G))
 
 
+@pytest.mark.parametrize("bits,group", [(4, 32), (8, 64), (8, 32)])
+def test_quantize_other_widths_and_groups(oracle, bits, group):
+    """affine_quant_impl<BITS, GROUP> (gpu-kernels/metal/quant/affine_dequant.metal:243-301) at the other three formats:
+    on-grid weights (every group spanning 0..2^bits - 1, f16-exact scale and bias) come back with their codes, scale
+    and bias -- which pins the word layout (values per word, words per group and row); a smooth source against a numpy
+    re-derivation with the tie rule written out; and the format's expansion of the result stays within half a step."""
+    qmax = (1 << bits) - 1
+    vpw = 32 // bits
+    N, K = 5, 256
+    rng = np.random.default_rng(70 + bits + group)
+    q = rng.integers(0, qmax + 1, size=(N, K), dtype=np.uint32)
+    q.reshape(N, K // group, group)[:, :, 0] = 0
+    q.reshape(N, K // group, group)[:, :, 1] = qmax
+    s = (rng.integers(1, 16, size=(N, K // group)) / 1024.0).astype(np.float32)
+    b = (-rng.integers(0, 256, size=(N, K // group)) / 256.0).astype(np.float32)
+    W = (np.repeat(s, group, axis=1) * q + np.repeat(b, group, axis=1)).astype(np.float32)
+    codes, sf16, bf16_ = oracle.quantize(W, K, N, bits=bits, group=group)
+    assert codes.shape == (N, K // vpw)
+    got = ((codes[:, :, None] >> (bits * np.arange(vpw, dtype=np.uint32))) & qmax).reshape(N, K)
+    assert np.array_equal(got, q)
+    assert np.array_equal(sf16.view(np.float16).astype(np.float32), s)
+    assert np.array_equal(bf16_.view(np.float16).astype(np.float32), b)
+    # smooth source, numpy re-derivation
+    N, K = 24, 256
+    n = np.arange(N)[:, None]
+    k = np.arange(K)[None, :]
+    src = (0.4 * np.sin(0.05 * k + 0.3 * n) + 0.1 * np.cos(0.7 * k) + 0.002 * (k - K / 2)).astype(np.float16).astype(np.float32)
+    codes, sf16, bf16_ = oracle.quantize(src, K, N, bits=bits, group=group)
+    g = src.reshape(N, K // group, group)
+    mn, mx = g.min(axis=2, keepdims=True), g.max(axis=2, keepdims=True)
+    sc = ((mx - mn) / np.float32(qmax)).astype(np.float32)
+    inv = np.where(sc > 0, np.float32(1.0) / sc, np.float32(0.0)).astype(np.float32)
+    t = ((g - mn) * inv).astype(np.float32)
+    fl = np.floor(t)
+    qn = np.clip(np.where(t - fl >= np.float32(0.5), fl + 1, fl), 0, qmax).astype(np.uint32).reshape(N, K)
+    got = ((codes[:, :, None] >> (bits * np.arange(vpw, dtype=np.uint32))) & qmax).reshape(N, K)
+    assert np.array_equal(got, qn)
+    assert np.array_equal(sf16, sc.astype(np.float16).view(np.uint16).reshape(N, K // group))
+    assert np.array_equal(bf16_, mn.astype(np.float16).view(np.uint16).reshape(N, K // group))
+    recon = mn + sc * qn.reshape(N, K // group, group)
+    assert (np.abs(recon - g) <= 0.5 * sc * (1 + 1e-5) + 1e-7).all()
+
+
 def test_cpu_baseline_is_the_same_algorithm(oracle):
     K, N, M = 512, 40, 3
     w, s, b = synth.make_weight(N, K, 51)

@@ -119,6 +119,7 @@ SYMBOLS = [
     ("vpq_qmv_w8g64_f32out", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     ("vpq_qmm_dense_route_w8g64_bf16", _i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i]),
     ("vpq_quantize_w4g64", _i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
+    ("vpq_quantize", _i, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _f]),
     ("vpq_f16_to_bf16", _i, [_vp, _vp, _vp, _sz]),
     ("vpq_profile_enable", _i, [_i]),
     ("vpq_profile_read", _i, [_vp, _i]),
@@ -1010,3 +1011,15 @@ def qmm_dense_route_w8_f16(w, scales, biases, x, K, N, M, w_deq, group=64, expan
     _check(load().vpq_qmm_dense_route_w8_f16(_stream(), group, _ptr(w), _ptr(scales), _ptr(biases), _ptr(x), _ptr(out), K, N, M,
                                              _ptr(w_deq), 1 if expand else 0), "vpq_qmm_dense_route_w8_f16")
     return out
+
+
+def quantize(src, K, N, bits=4, group=64, clip=1.0):
+    """The packer at any width and group: src bf16 or float16 [N, K] -> (w int32 [N, K*bits/32], scales, biases float16
+    [N, K/group])."""
+    import torch
+    w = torch.empty((N, K * bits // 32), dtype=torch.int32, device=src.device)
+    s = torch.empty((N, K // group), dtype=torch.float16, device=src.device)
+    b = torch.empty((N, K // group), dtype=torch.float16, device=src.device)
+    _check(load().vpq_quantize(_stream(), bits, group, 1 if src.dtype == torch.float16 else 0, _ptr(src), _ptr(w), _ptr(s),
+                               _ptr(b), K, N, clip), "vpq_quantize")
+    return w, s, b

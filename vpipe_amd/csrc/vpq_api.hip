@@ -1743,6 +1743,19 @@ int vpq_quantize_w4g64(vpq_stream_t stream, const uint16_t* src, uint32_t* w, ui
   return finish(vpq::launch_quantize(reinterpret_cast<hipStream_t>(stream), src, w, scales_f16, biases_f16, K, N, clip));
 }
 
+int vpq_quantize(vpq_stream_t stream, int bits, int group, int src_f16, const uint16_t* src, uint32_t* w,
+                 uint16_t* scales_f16, uint16_t* biases_f16, int K, int N, float clip)
+{
+  if (src == nullptr || w == nullptr || scales_f16 == nullptr || biases_f16 == nullptr) { return VPQ_ERR_NULL_POINTER; }
+  if ((bits != 4 && bits != 8) || (group != 64 && group != 32)) { return VPQ_ERR_BAD_SHAPE; }
+  if (K <= 0 || N <= 0 || (K % group) != 0) { return VPQ_ERR_BAD_SHAPE; }
+  if (!aligned(src, 16) || !aligned(w, 4)) { return VPQ_ERR_MISALIGNED; }
+  const int st = ensure_init();
+  if (st != VPQ_OK) { return st; }
+  return finish(vpq::launch_quantize(reinterpret_cast<hipStream_t>(stream), src, w, scales_f16, biases_f16, K, N, clip, bits,
+                                     group, src_f16 != 0));
+}
+
 int vpq_f16_to_bf16(vpq_stream_t stream, const uint16_t* in_f16, uint16_t* out_bf16, size_t count)
 {
   if (in_f16 == nullptr || out_bf16 == nullptr) { return VPQ_ERR_NULL_POINTER; }

@@ -219,33 +219,38 @@ hipError_t launch_embed_gather(hipStream_t st, const int* ids, const uint32_t* w
                        reinterpret_cast<uint4*>(out), Hw, vocab, total);
 }
 
-// One thread per 64-wide group, as the reference's packer
-// (gpu-kernels/metal/quant/affine_dequant.metal:243-285): min/max, optional
-// clip toward the midpoint, scale = (mx-mn)/15, q = clamp(round((v-mn)/scale)),
-// round half away from zero, scale and min emitted as IEEE F16.
-__global__ __launch_bounds__(64) void quantize_w4g64_kernel(
+// One thread per group, as the reference's packer (affine_quant_impl<BITS, GROUP>,
+// gpu-kernels/metal/quant/affine_dequant.metal:243-301: 4 or 8 bits, groups of 64 or 32): min/max, optional
+// clip toward the midpoint, scale = (mx-mn)/(2^BITS - 1), q = clamp(round((v-mn)/scale)),
+// round half away from zero, scale and min emitted as IEEE F16.  F16SRC: the source matrix is binary16 (the
+// reference's quantizer runs the VPIPE_ELT = half build, generative-models/quantize/affine-quantizer.cc:25), else bf16.
+template <int BITS, int GROUP, bool F16SRC>
+__global__ __launch_bounds__(64) void quantize_kernel(
     const uint16_t* __restrict__ src, uint32_t* __restrict__ w, uint16_t* __restrict__ s_f16,
     uint16_t* __restrict__ b_f16, int K, int N, float clip)
 {
-  const int Kg = K / kGroup;
+  constexpr int VPW = 32 / BITS;             // values per word
+  constexpr int WPG = GROUP / VPW;           // words per group
+  constexpr int QMAX = (1 << BITS) - 1;
+  const int Kg = K / GROUP;
   const int grp = blockIdx.x * 64 + threadIdx.x;
   const int n = blockIdx.y;
   if (grp >= Kg || n >= N) { return; }
-  const uint16_t* xp = src + (size_t)n * K + (size_t)grp * kGroup;
-  float v[kGroup];
+  const uint16_t* xp = src + (size_t)n * K + (size_t)grp * GROUP;
+  float v[GROUP];
   float mn = INFINITY, mx = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < kGroup / 8; ++i) {
+  for (int i = 0; i < GROUP / 8; ++i) {
     const uint4 d = reinterpret_cast<const uint4*>(xp)[i];
     const uint32_t dd[4] = {d.x, d.y, d.z, d.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      v[i * 8 + 2 * j] = bf16_lo_to_f32(dd[j]);
-      v[i * 8 + 2 * j + 1] = bf16_hi_to_f32(dd[j]);
+      v[i * 8 + 2 * j] = elt_lo_to_f32<F16SRC>(dd[j]);
+      v[i * 8 + 2 * j + 1] = elt_hi_to_f32<F16SRC>(dd[j]);
     }
   }
 #pragma unroll
-  for (int i = 0; i < kGroup; ++i) {
+  for (int i = 0; i < GROUP; ++i) {
     mn = fminf(mn, v[i]);
     mx = fmaxf(mx, v[i]);
   }
@@ -257,35 +262,46 @@ __global__ __launch_bounds__(64) void quantize_w4g64_kernel(
     mn = mid + (mn - mid) * clip;
     mx = mid + (mx - mid) * clip;
   }
-  const float scale = (mx - mn) / 15.0f;
+  const float scale = (mx - mn) / (float)QMAX;
   const float inv = (scale > 0.0f) ? 1.0f / scale : 0.0f;
   s_f16[(size_t)n * Kg + grp] = __builtin_bit_cast(uint16_t, (_Float16)scale);
   b_f16[(size_t)n * Kg + grp] = __builtin_bit_cast(uint16_t, (_Float16)mn);
-  uint32_t* wp = w + (size_t)n * (K / 8) + (size_t)grp * (kGroup / 8);
+  uint32_t* wp = w + (size_t)n * (K / VPW) + (size_t)grp * WPG;
 #pragma unroll
-  for (int wi = 0; wi < kGroup / 8; ++wi) {
+  for (int wi = 0; wi < WPG; ++wi) {
     uint32_t packed = 0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      int q = (int)roundf((v[wi * 8 + i] - mn) * inv);
-      q = q < 0 ? 0 : (q > 15 ? 15 : q);
-      packed |= (uint32_t)q << (4 * i);
+    for (int i = 0; i < VPW; ++i) {
+      int q = (int)roundf((v[wi * VPW + i] - mn) * inv);
+      q = q < 0 ? 0 : (q > QMAX ? QMAX : q);
+      packed |= (uint32_t)q << (BITS * i);
     }
     wp[wi] = packed;
   }
 }
 
 hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
-                           uint16_t* b_f16, int K, int N, float clip)
+                           uint16_t* b_f16, int K, int N, float clip, int bits, int group, bool f16_src)
 {
-  const int Kg = K / kGroup;
+  const int Kg = K / group;
+  const int wpr = K * bits / 32;                 // words per row
   // grid.y carries N; rows beyond 65535 are covered by launching in bands.
   for (int n0 = 0; n0 < N; n0 += 65535) {
     const int rows = (N - n0 < 65535) ? (N - n0) : 65535;
-    const hipError_t e = launch_kernel(
-        quantize_w4g64_kernel, dim3((unsigned)((Kg + 63) / 64), (unsigned)rows), dim3(64), 0, st,
-        src + (size_t)n0 * K, w + (size_t)n0 * (K / 8), s_f16 + (size_t)n0 * Kg,
-        b_f16 + (size_t)n0 * Kg, K, rows, clip);
+    const dim3 grid((unsigned)((Kg + 63) / 64), (unsigned)rows), block(64);
+    const uint16_t* sp = src + (size_t)n0 * K;
+    uint32_t* wp = w + (size_t)n0 * wpr;
+    uint16_t* ss = s_f16 + (size_t)n0 * Kg;
+    uint16_t* bb = b_f16 + (size_t)n0 * Kg;
+    hipError_t e = hipErrorInvalidValue;
+#define VPQ_QUANT(B, G)                                                                              \
+  (f16_src ? launch_kernel(quantize_kernel<B, G, true>, grid, block, 0, st, sp, wp, ss, bb, K, rows, clip) \
+           : launch_kernel(quantize_kernel<B, G, false>, grid, block, 0, st, sp, wp, ss, bb, K, rows, clip))
+    if (bits == 4 && group == 64) { e = VPQ_QUANT(4, 64); }
+    else if (bits == 4 && group == 32) { e = VPQ_QUANT(4, 32); }
+    else if (bits == 8 && group == 64) { e = VPQ_QUANT(8, 64); }
+    else if (bits == 8 && group == 32) { e = VPQ_QUANT(8, 32); }
+#undef VPQ_QUANT
     if (e != hipSuccess) { return e; }
   }
   return hipSuccess;

@@ -266,7 +266,7 @@ hipError_t launch_dequant_f16(hipStream_t st, const uint32_t* w, const uint16_t*
                               uint16_t* out, int K, int N);
 hipError_t launch_qmv_simple_f16(hipStream_t st, const QmvArgs& a);
 hipError_t launch_quantize(hipStream_t st, const uint16_t* src, uint32_t* w, uint16_t* s_f16,
-                           uint16_t* b_f16, int K, int N, float clip);
+                           uint16_t* b_f16, int K, int N, float clip, int bits = 4, int group = 64, bool f16_src = false);
 hipError_t launch_f16_to_bf16(hipStream_t st, const uint16_t* in, uint16_t* out, size_t count);
 // out row 2i = a row i, out row 2i+1 = b row i; rows of row_bytes (a multiple of 2) bytes.
 hipError_t launch_interleave_rows(hipStream_t st, const void* a, const void* b, void* out, size_t row_bytes,

@@ -82,6 +82,29 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_batch4_xp_w4g64", QuantKernel::QmvBatch},
     {"affine_qmv_bf16", "affine_qmv_batch8_xp_w4g64", QuantKernel::QmvBatch},
     {"affine_qmv_bf16", "affine_qmv_batch8_xp2_w4g64", QuantKernel::QmvBatch},
+    // the other tilings of the same batched GEMV (gpu-kernels/metal/quant/affine_qmv.metal:1911-2549: threadgroup-
+    // staged x, hoisted nibbles, weight packs in registers; `xh16` multiplies in half there and in fp32 here)
+    {"affine_qmv_bf16", "affine_qmv_batch8_xp1_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch8_tg_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch8_tg4_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch8_xd_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch8_xh_w4g64", QuantKernel::QmvBatch},
+    {"affine_qmv_bf16", "affine_qmv_batch8_xh16_w4g64", QuantKernel::QmvBatch},
+    // batched gated GEMVs (:2336-2354, 2854-2872, 3003): slot 7 = m_total
+    {"affine_qmv_bf16", "affine_qmv_batch_swiglu_w4g64", QuantKernel::QmvBatchSwiglu},
+    {"affine_qmv_bf16", "affine_qmv_batch4_swiglu_w4g64", QuantKernel::QmvBatchSwiglu},
+    {"affine_qmv_bf16", "affine_qmv_batch4_xp_swiglu_w4g64", QuantKernel::QmvBatchSwiglu},
+    {"affine_qmv_bf16", "affine_qmv_batch8_xp2_swiglu_w4g64", QuantKernel::QmvBatchSwiglu},
+    {"affine_qmv_bf16", "affine_qmv_batch_geglu_w4g64", QuantKernel::QmvBatchGeglu},
+    // batched GEMVs of the twins (:1718-1736, 2328-2334, 2725-2745, 3026)
+    {"affine_qmv_bf16", "affine_qmv_batch_w8g64", QuantKernel::QmvBatch, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_batch4_w8g64", QuantKernel::QmvBatch, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_batch4_xp_w8g64", QuantKernel::QmvBatch, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_batch8_xp2_w8g64", QuantKernel::QmvBatch, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_batch8_tg4_w8g64", QuantKernel::QmvBatch, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_batch8_xd_w8g64", QuantKernel::QmvBatch, QuantFormat::W8G64},
+    {"affine_qmv_bf16", "affine_qmv_batch_w4g32", QuantKernel::QmvBatch, QuantFormat::W4G32},
+    {"affine_qmv_bf16", "affine_qmv_batch_geglu_w4g32", QuantKernel::QmvBatchGeglu, QuantFormat::W4G32},
     {"affine_qmv_bf16", "affine_qmv_qkv_w4g64", QuantKernel::QmvQkv},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64", QuantKernel::Qmm},
     {"affine_qmm_steel_bf16", "affine_qmm_steel_w4g64_bm64", QuantKernel::Qmm},
@@ -119,6 +142,16 @@ const FnEntry kFunctions[] = {
     {"affine_qmv_bf16", "affine_qmv_gelu_mul_w8g64", QuantKernel::QmvGeluMul, QuantFormat::W8G64},
     {"affine_qmv_bf16", "affine_qmv_gelu_mul_w4g32", QuantKernel::QmvGeluMul, QuantFormat::W4G32},
     {"affine_dequant_bf16", "affine_requant_w8_to_w4_g64", QuantKernel::Requant84, QuantFormat::W8G64},
+    // the packer at every width and group (gpu-kernels/metal/quant/affine_dequant.metal:243-301); the reference's
+    // quantizer loads it from the binary16 library (generative-models/quantize/affine-quantizer.cc:25)
+    {"affine_dequant_bf16", "affine_quant_w4_g64", QuantKernel::QuantizeBf16, QuantFormat::W4G64},
+    {"affine_dequant_bf16", "affine_quant_w4_g32", QuantKernel::QuantizeBf16, QuantFormat::W4G32},
+    {"affine_dequant_bf16", "affine_quant_w8_g64", QuantKernel::QuantizeBf16, QuantFormat::W8G64},
+    {"affine_dequant_bf16", "affine_quant_w8_g32", QuantKernel::QuantizeBf16, QuantFormat::W8G32},
+    {"affine_dequant", "affine_quant_w4_g64", QuantKernel::QuantizeF16, QuantFormat::W4G64},
+    {"affine_dequant", "affine_quant_w4_g32", QuantKernel::QuantizeF16, QuantFormat::W4G32},
+    {"affine_dequant", "affine_quant_w8_g64", QuantKernel::QuantizeF16, QuantFormat::W8G64},
+    {"affine_dequant", "affine_quant_w8_g32", QuantKernel::QuantizeF16, QuantFormat::W8G32},
     // Tiling variants the reference keeps beside its defaults (affine_qmv.metal:3072-3118: rows per simdgroup / packs
     // per thread of the same GEMV) and its plain QMM (affine_qmm.metal:64-174): the same mathematics, served by the
     // same kernels (the plain QMM exists in the binary16 build only).  The `_acc16` GEMMs accumulate in fp32 in the
@@ -447,7 +480,16 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
   int status = VPQ_OK;
   const QuantKernel kind = _fn.kind();
   const QuantFormat fmt = _fn.format();
-  if (fmt != QuantFormat::W4G64 && kind != QuantKernel::QmvQkv && kind != QuantKernel::QmvQkvRms) {
+  if (kind == QuantKernel::QuantizeBf16 || kind == QuantKernel::QuantizeF16) {
+    // gpu-kernels/metal/quant/affine_dequant.metal:287-301: 0:x 1:w 2:scales 3:biases 4:K 5:N 6:clip
+    const int bits = (fmt == QuantFormat::W8G64 || fmt == QuantFormat::W8G32) ? 8 : 4;
+    const int group = (fmt == QuantFormat::W4G32 || fmt == QuantFormat::W8G32) ? 32 : 64;
+    status = (!buf(0) || !buf(1) || !buf(2) || !buf(3) || !has_int(4) || !has_int(5))
+                 ? VPQ_ERR_NULL_POINTER
+                 : vpq_quantize(st, bits, group, kind == QuantKernel::QuantizeF16 ? 1 : 0, static_cast<const uint16_t*>(buf(0)),
+                                static_cast<uint32_t*>(buf(1)), static_cast<uint16_t*>(buf(2)), static_cast<uint16_t*>(buf(3)),
+                                ival(4), ival(5), _slots[6].is_const ? _slots[6].fvalue : 1.0f);
+  } else if (fmt != QuantFormat::W4G64 && kind != QuantKernel::QmvQkv && kind != QuantKernel::QmvQkvRms) {
     // The 8-bit and group-32 twins keep the slot layout of the 4-bit group-64 functions:
     // dequant 0:w 1:scales 2:biases 3:w_deq 4:K 5:N; QMV 0:w 1:scales 2:biases 3:x 4:y 5:K 6:N [7:residual],
     // rows from grid.x.  The Q4_0 forms ignore slot 2.
@@ -503,7 +545,9 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
       const uint16_t* x = static_cast<const uint16_t*>(buf(3));
       uint16_t* y = static_cast<uint16_t*>(buf(4));
       const int K = ival(5), N = ival(6);
-      const int M = grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1;
+      const bool batched = kind == QuantKernel::QmvBatch || kind == QuantKernel::QmvBatchSwiglu ||
+                           kind == QuantKernel::QmvBatchGeglu;          // rows = m_total in slot 7 (a missing one: 0 rows, refused)
+      const int M = batched ? (has_int(7) ? ival(7) : 0) : (grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1);
       const uint16_t* residual = kind == QuantKernel::QmvAdd ? static_cast<const uint16_t*>(buf(7)) : nullptr;
       const bool gather = kind == QuantKernel::GatherSwiglu || kind == QuantKernel::GatherGeglu ||
                           kind == QuantKernel::GatherDown;
@@ -617,7 +661,7 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
                                                  : vpq_qmm_dense_route_w8g32_bf16(st, w, sc, bi, x, y, K, N, ival(7), w_deq, 1));
       } else if (fmt == QuantFormat::W8G32) {
         status = vpq_qmv_w8g32_bf16(st, w, sc, bi, x, y, K, N, M, residual);
-      } else if (kind == QuantKernel::QmvGeglu) {
+      } else if (kind == QuantKernel::QmvGeglu || kind == QuantKernel::QmvBatchGeglu) {
         status = vpq_qmv_gated_w4g32_bf16(st, w, sc, q40 ? nullptr : bi, x, y, K, N, M, VPQ_GATE_GEGLU, q40 ? 1 : 0);
       } else {
         status = vpq_qmv_w4g32_bf16(st, w, sc, q40 ? nullptr : bi, x, y, K, N, M, residual, q40 ? 1 : 0);
@@ -862,11 +906,14 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
         // gpu-kernels/metal/quant/affine_qmv.metal:751-768: slot 7 = the multiplier
         const uint16_t* mul = static_cast<const uint16_t*>(buf(7));
         status = mul == nullptr ? VPQ_ERR_NULL_POINTER : vpq_qmv_gelu_mul_w4g64_bf16(st, w, sc, bi, x, y, K, N, mul);
-      } else if (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu) {
-        // gpu-kernels/metal/quant/affine_qmv.metal:891-906: N = 2*ffn, rows from grid.x
-        const int M = grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1;
-        status = vpq_qmv_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, M, VPQ_QMV_AUTO,
-                                          kind == QuantKernel::QmvGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
+      } else if (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu || kind == QuantKernel::QmvBatchSwiglu ||
+                 kind == QuantKernel::QmvBatchGeglu) {
+        // gpu-kernels/metal/quant/affine_qmv.metal:891-906: N = 2*ffn, rows from grid.x; the batched forms
+        // (:2336-2354, 2854-2872, 3003) carry m_total in slot 7
+        const bool batched = kind == QuantKernel::QmvBatchSwiglu || kind == QuantKernel::QmvBatchGeglu;
+        const int M = batched ? (has_int(7) ? ival(7) : 0) : (grid.x >= 32 ? static_cast<int>(grid.x / 32) : 1);
+        const bool geglu = kind == QuantKernel::QmvGeglu || kind == QuantKernel::QmvBatchGeglu;
+        status = vpq_qmv_gated_w4g64_bf16(st, w, sc, bi, x, y, K, N, M, VPQ_QMV_AUTO, geglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
       } else {
         int M = 1;
         const uint16_t* residual = nullptr;

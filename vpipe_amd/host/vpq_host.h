@@ -72,6 +72,8 @@ enum class QuantKernel : std::uint8_t {
   Qmv,            // affine_qmv_w4g64              M from grid.x / 32
   QmvAdd,         // affine_qmv_w4g64_add          slot 7 = residual buffer
   QmvBatch,       // affine_qmv_batch*_w4g64       slot 7 = m_total
+  QmvBatchSwiglu, // affine_qmv_batch*_swiglu_w4g64: the gated GEMV over m_total rows (slot 7), N = 2 * ffn
+  QmvBatchGeglu,  // affine_qmv_batch_geglu_w4g64 / _w4g32
   Qmm,            // affine_qmm_steel_w4g64[_bm64|_bm128], affine_qmm_mma_w4g64    slot 7 = M
   QmvQkv,         // affine_qmv_qkv_w4g64: row-concatenated q|k|v pack, slots 4,5,6 = q,k,v outputs,
                   //   7 = K, 8,9,10 = q_rows, k_rows, v_rows (v_rows == 0: q|k only); one launch
@@ -79,6 +81,8 @@ enum class QuantKernel : std::uint8_t {
   QmmSwiglu,      // affine_qmm_swiglu_w4g64[_bm64|_bm128|_bm64_rs]: slot 7 = M, 8 = out_stride, 9 = out_off (_rs)
   QmvGeglu,       // affine_qmv_geglu_w4g64: as QmvSwiglu with gelu_tanh(gate) * up
   Requant84,      // affine_requant_w8_to_w4_g64: 0:w8 1:s8 2:b8 3:w4 4:s4 5:b4 6:K 7:N
+  QuantizeBf16,   // affine_quant_w{4,8}_g{64,32} of the bf16 library: 0:x 1:w 2:scales(F16) 3:biases(F16) 4:K 5:N 6:clip (float)
+  QuantizeF16,    // ... of the binary16 library (the source matrix is binary16)
   QmvGeluMul,     // affine_qmv_gelu_mul_w4g64: one row of x, slot 7 = mul buffer [N]; y = gelu_tanh(W x) * mul
   QmvQkvRms,      // affine_qmv_qkv_rms_w4g64 / _w4g32 / _w8g64: slots 0:w 1:scales 2:biases 3:x 4:norm_w 5:q 6:k 7:v 8:K
                   //   9,10,11 = q_rows, k_rows, v_rows, 12 = eps (float); the normalized row goes through stream scratch
