@@ -413,6 +413,36 @@ def test_packer_function_names(vpq, enc, dev, D, lib, name, bits, group):
     assert w.abs().sum() > 0
 
 
+def test_batched_gemv_names_of_the_binary16_library(vpq, enc, dev, D):
+    # the half build's batched GEMVs (library "affine_qmv", rows = m_total in slot 7): the C ABI's binary16 QMV
+    K, N = 1024, 64
+    rng = np.random.default_rng(4700)
+    w = rng.integers(0, 2**32, size=(N, K // 8), dtype=np.uint32)
+    s = rng.uniform(0.005, 0.02, size=(N, K // 64)).astype(np.float16)
+    b = (-8.0 * s.astype(np.float32)).astype(np.float16)
+    wd = torch.from_numpy(w.view(np.int32)).to(dev)
+    sd, bd = torch.from_numpy(s).to(dev), torch.from_numpy(b).to(dev)
+    outs = []
+    for name, M, act in (("affine_qmv_batch4_w4g64", 3, 0), ("affine_qmv_batch8_xp2_w4g64", 8, 0),
+                         ("affine_qmv_batch_swiglu_w4g64", 2, 1), ("affine_qmv_batch_geglu_w4g64", 2, 2)):
+        x = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float16)).to(dev)
+        y = torch.zeros((M, N // 2 if act else N), dtype=torch.float16, device=dev)
+        assert enc.set_function("affine_qmv", name) == 1, name
+        for i, t in enumerate((wd, sd, bd, x, y)):
+            enc.set_buffer(i, t)
+        enc.set_constant(5, K)
+        enc.set_constant(6, N)
+        enc.set_constant(7, M)
+        enc.dispatch((32, N // 4, (M + 1) // 2), (32, 2, 1))
+        outs.append((name, M, act, x, y))
+    ok, why = enc.wait_ok()
+    assert ok, why
+    for name, M, act, x, y in outs:
+        want = vpq.qmv_w4g64_f16(wd, sd, bd, x, K, N, M, activation=act) if act else vpq.qmv_w4g64_f16(wd, sd, bd, x, K, N, M)
+        assert torch.equal(y, want), name
+        assert y.abs().sum() > 0
+
+
 def test_fused_qkv_call_site(enc, oracle, dev, D):
     # llama decode: one dispatch over the row-concatenated q|k|v pack, three output buffers
     # (gpu-kernels/metal/quant/affine_qmv.metal:405-516)

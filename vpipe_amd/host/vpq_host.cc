@@ -207,6 +207,23 @@ const FnEntry kFunctions[] = {
     {"affine_qmv", "affine_qmv_swiglu_w4g64", QuantKernel::QmvSwiglu, QuantFormat::W4G64F16},
     {"affine_qmv", "affine_qmv_geglu_w4g64", QuantKernel::QmvGeglu, QuantFormat::W4G64F16},
     {"affine_qmv", "affine_qmv_qkv_w4g64", QuantKernel::QmvQkv, QuantFormat::W4G64F16},
+    // the batched GEMVs of the binary16 build (rows = m_total in slot 7)
+    {"affine_qmv", "affine_qmv_batch_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch4_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch4_xp_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_xp_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_xp2_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_xp1_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_tg_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_tg4_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_xd_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_xh_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_xh16_w4g64", QuantKernel::QmvBatch, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch_swiglu_w4g64", QuantKernel::QmvBatchSwiglu, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch4_swiglu_w4g64", QuantKernel::QmvBatchSwiglu, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch4_xp_swiglu_w4g64", QuantKernel::QmvBatchSwiglu, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch8_xp2_swiglu_w4g64", QuantKernel::QmvBatchSwiglu, QuantFormat::W4G64F16},
+    {"affine_qmv", "affine_qmv_batch_geglu_w4g64", QuantKernel::QmvBatchGeglu, QuantFormat::W4G64F16},
     {"affine_qmm_steel", "affine_qmm_steel_w4g64", QuantKernel::Qmm, QuantFormat::W4G64F16},
     {"affine_qmm_steel", "affine_qmm_steel_w4g64_bm64", QuantKernel::Qmm, QuantFormat::W4G64F16},
     {"affine_qmm_steel", "affine_qmm_steel_w4g64_bm128", QuantKernel::Qmm, QuantFormat::W4G64F16},
@@ -612,9 +629,10 @@ void ComputeEncoder::dispatch(LaunchDims grid, LaunchDims /*threads_per_threadgr
                                                                                              : VPQ_GATE_SWIGLU);
         }
       } else if (fmt == QuantFormat::W4G64F16) {
-        if (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu) {
-          status = vpq_qmv_gated_w4g64_f16(st, w, sc, bi, x, y, K, N, M,
-                                           kind == QuantKernel::QmvGeglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
+        if (kind == QuantKernel::QmvSwiglu || kind == QuantKernel::QmvGeglu || kind == QuantKernel::QmvBatchSwiglu ||
+            kind == QuantKernel::QmvBatchGeglu) {
+          const bool geglu = kind == QuantKernel::QmvGeglu || kind == QuantKernel::QmvBatchGeglu;
+          status = vpq_qmv_gated_w4g64_f16(st, w, sc, bi, x, y, K, N, M, geglu ? VPQ_GATE_GEGLU : VPQ_GATE_SWIGLU);
         } else {
           status = vpq_qmv_w4g64_f16(st, w, sc, bi, x, y, K, N, M, residual);
         }
